@@ -1,0 +1,154 @@
+"""ctypes binding of the C ABI in include/bf_hip.h (blackforge_amd/lib/libbf_hip.so).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+``BF_ERR_INVALID_ARGUMENT`` maps to ``ValueError`` (the reference throws std::invalid_argument),
+everything else to ``RuntimeError`` (std::runtime_error).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libbf_hip.so")
+
+OK, ERR_INVALID_ARGUMENT, ERR_RUNTIME, ERR_UNSUPPORTED = 0, 1, 2, 3
+ACT_SILU, ACT_GELU, ACT_RELU = 0, 1, 2
+
+c_size = ctypes.c_size_t
+c_ptr = ctypes.c_void_p
+c_int = ctypes.c_int
+c_float = ctypes.c_float
+c_ll = ctypes.c_longlong
+
+
+class DeviceProps(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 128), ("arch", ctypes.c_char * 32), ("compute_units", c_int),
+                ("clock_khz", c_int), ("wavefront_size", c_int), ("lds_bytes_per_block", c_int),
+                ("total_memory", c_size)]
+
+
+class PoolStats(ctypes.Structure):
+    _fields_ = [("bytes_from_driver", c_size), ("bytes_in_use", c_size), ("driver_allocations", c_size),
+                ("acquires", c_size)]
+
+
+P = c_ptr  # device pointer
+S = c_ptr  # stream
+
+# name -> argument types (every function returns int status unless listed in _SPECIAL)
+SIGNATURES = {
+    "bf_hip_device_count": [ctypes.POINTER(c_int)],
+    "bf_hip_device_props": [c_int, ctypes.POINTER(DeviceProps)],
+    "bf_hip_set_device": [c_int],
+    "bf_hip_get_device": [ctypes.POINTER(c_int)],
+    "bf_hip_synchronize": [],
+    "bf_hip_stream_create": [ctypes.POINTER(c_ptr)],
+    "bf_hip_stream_destroy": [S],
+    "bf_hip_stream_synchronize": [S],
+    "bf_hip_event_create": [ctypes.POINTER(c_ptr)],
+    "bf_hip_event_destroy": [c_ptr],
+    "bf_hip_event_record": [c_ptr, S],
+    "bf_hip_event_synchronize": [c_ptr],
+    "bf_hip_event_elapsed_ms": [c_ptr, c_ptr, ctypes.POINTER(c_float)],
+    "bf_hip_pool_acquire": [c_size, ctypes.POINTER(c_ptr)],
+    "bf_hip_pool_release": [P, c_size],
+    "bf_hip_pool_stats": [ctypes.POINTER(PoolStats)],
+    "bf_hip_pool_trim": [],
+    "bf_hip_memcpy_h2d": [P, c_ptr, c_size],
+    "bf_hip_memcpy_d2h": [c_ptr, P, c_size],
+    "bf_hip_memcpy_d2d": [P, P, c_size, S],
+    "bf_hip_fill_zero": [P, c_size, S],
+    "bf_hip_add": [P, P, P, c_size, S],
+    "bf_hip_scale": [P, c_float, P, c_size, S],
+    "bf_hip_add_bias": [P, P, P, c_size, c_size, S],
+    "bf_hip_add_bias_act": [P, P, P, c_size, c_size, c_int, S],
+    "bf_hip_add_bias_residual": [P, P, P, P, c_size, c_size, S],
+    "bf_hip_act_forward": [P, P, c_size, c_int, S],
+    "bf_hip_act_backward": [P, P, P, c_size, c_int, S],
+    "bf_hip_add_bias_act_backward": [P, P, P, P, P, c_size, c_size, c_int, S],
+    "bf_hip_accumulate": [P, P, c_size, S],
+    "bf_hip_zero_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_size), c_size, S],
+    "bf_hip_rmsnorm": [P, P, c_size, c_size, S],
+    "bf_hip_rmsnorm_backward": [P, P, P, c_size, c_size, S],
+    "bf_hip_softmax": [P, P, c_size, c_size, S],
+    "bf_hip_softmax_backward": [P, P, P, c_size, c_size, S],
+    "bf_hip_bias_grad": [P, P, c_size, c_size, S],
+    "bf_hip_count_out_of_range": [P, c_size, c_size, ctypes.POINTER(c_size), ctypes.POINTER(c_ll), S],
+    "bf_hip_embedding_forward": [P, P, P, c_size, c_size, c_size, S],
+    "bf_hip_embedding_backward": [P, P, P, c_size, c_size, c_size, S],
+    "bf_hip_positional_forward": [P, P, P, c_size, c_size, c_size, c_size, c_size, S],
+    "bf_hip_positional_backward": [P, P, c_size, c_size, c_size, c_size, S],
+    "bf_hip_concat_seq": [P, P, P, c_size, c_size, c_size, c_size, S],
+    "bf_hip_argmax_last_position": [P, c_size, c_size, ctypes.POINTER(c_ll), S],
+    "bf_hip_gemm_f32": [c_int, c_int, P, P, P, c_size, c_size, c_size, S],
+    "bf_hip_cvt_f32_bf16": [P, P, c_size, S],
+    "bf_hip_cvt_f32_bf16_transpose": [P, P, c_size, c_size, S],
+    "bf_hip_gemm_bf16_nt": [P, P, P, c_size, c_size, c_size, S],
+    "bf_hip_matmul_bf16": [P, P, P, c_size, c_size, c_size, c_int, S],
+    "bf_hip_matmul_bf16_backward": [P, P, P, P, P, c_size, c_size, c_size, c_int, S],
+    "bf_hip_invalidate_bf16_weight_cache": [],
+    "bf_hip_attention_forward": [P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
+    "bf_hip_attention_dot_o_do": [P, P, P, c_size, c_size, c_size, c_size, S],
+    "bf_hip_attention_backward": [P, P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float,
+                                  c_size, S],
+    "bf_hip_mse": [P, P, P, P, c_size, c_int, S],
+    "bf_hip_cross_entropy": [P, P, P, P, c_size, c_size, c_int, S],
+    "bf_hip_cross_entropy_sparse": [P, P, P, P, c_size, c_size, c_int, S],
+    "bf_hip_sgd_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_size), c_size, c_float, S],
+    "bf_hip_adamw_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr),
+                           ctypes.POINTER(c_size), c_size, c_ll, c_float, c_float, c_float, c_float, c_float, S],
+}
+_SPECIAL = {"bf_hip_last_error": ctypes.c_char_p, "bf_hip_version": ctypes.c_char_p}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the shipped library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                           "(there is no CPU fallback for the HIP operator library)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if a declared entry point is not exported
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    for name, restype in _SPECIAL.items():
+        fn = getattr(lib, name)
+        fn.argtypes = []
+        fn.restype = restype
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().bf_hip_last_error().decode(errors="replace")
+
+
+def check(status: int, name: str = "") -> None:
+    if status == OK:
+        return
+    message = last_error() or f"{name} failed with status {status}"
+    if status == ERR_INVALID_ARGUMENT:
+        raise ValueError(message)
+    raise RuntimeError(message)
+
+
+def call(name: str, *args) -> None:
+    check(getattr(load(), name)(*args), name)
+
+
+def device_count() -> int:
+    n = c_int(0)
+    call("bf_hip_device_count", ctypes.byref(n))
+    return n.value
+
+
+def device_props(index: int = 0) -> DeviceProps:
+    props = DeviceProps()
+    call("bf_hip_device_props", index, ctypes.byref(props))
+    return props

@@ -1,0 +1,635 @@
+// Fused causal attention, forward and backward, fp32 on the fp32 MFMA pipe (v_mfma_f32_32x32x2_f32).
+//
+// Layout: q [batch,newLen,dim], k/v [batch,totalLen,dim], heads contiguous in dim.  Query row i
+// (absolute position oldLen+i) attends to keys j <= oldLen+i.
+//
+// Three MFMA kernels, all with 256-thread workgroups (4 wavefronts, one per SIMD), 32 rows per wave:
+//   forward : a workgroup owns 128 query rows, streams K/V tiles through LDS, online softmax.
+//   dQ      : same ownership; recomputes P from the saved statistics, accumulates dQ in registers.
+//   dK/dV   : a workgroup owns 128 keys (K, V and both accumulators live in registers), streams
+//             Q/dO tiles through LDS, writes dK and dV once.  No atomics anywhere, so gradients are
+//             bit-reproducible; the price is that S and dP are recomputed in both backward kernels.
+//
+// Orientation trick (what makes the softmax cheap on 64-wide waves).  With the 32x32x2 MFMA
+//   A: lane l holds A[i = l%32][k = l/32]      B: lane l holds B[k = l/32][j = l%32]
+//   D: lane l, reg r holds D[i = 8*(r/4) + 4*(l/32) + r%4][j = l%32]
+// the query-owner kernels compute S^T = K * Q^T (M = keys, N = queries).  A lane then holds 16 keys of
+// ONE query column, so row max / row sum are 16 in-register operations plus one exchange with lane^32,
+// and P^T in D layout is already in B-operand layout for O^T = V^T * P^T (the k index of step r is the
+// key held in register r), so P never leaves registers.  The key-owner kernel computes S = Q * K^T
+// (M = queries, N = keys), whose D layout is the A-operand layout of dV = P^T * dO and dK = dS^T * Q.
+// Because a dot product does not care about the order of its terms, the k index of MFMA step t is
+// taken as (t, HD/2 + t) for the two lane halves, which makes every LDS operand read a contiguous
+// ds_read_b128.
+//
+// Head dims are padded in registers/LDS to HDP in {32, 64, 128, 256}; any headDim <= 256 and any
+// newLen/totalLen/oldLen are accepted (tiles are zero-filled and masked).
+#include "common.hpp"
+
+#include <cmath>
+
+namespace bf {
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct AttnParams {
+    const float* q; const float* k; const float* v; const float* o; const float* dO;
+    const float* lse2;   // [batch, heads, newLen]: m*log2(e) + log2(l)
+    const float* dvec;   // [batch, heads, newLen]: dot(O, dO)
+    float* out; float* m; float* l;
+    float* dQ; float* dK; float* dV;
+    int batch, heads, newLen, totalLen, dim, hd, oldLen;
+    float scale;
+    int numTiles;        // query tiles (forward, dQ) or key tiles (dK/dV) per (batch, head)
+};
+
+__device__ __forceinline__ float fastExp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Workgroup -> (batch*head, tile).  Workgroups are dealt round-robin to the 8 XCDs, each with its own
+// L2; this mapping gives every XCD a contiguous range of (batch, head) pairs so that the tiles that
+// share K/V (or Q/dO) hit the same L2.  Within a pair the heaviest tile comes first.
+__device__ __forceinline__ void decodeBlock(int numTiles, int totalBlocks, bool heavyIsLast, int& bh, int& tile) {
+    int id = blockIdx.x;
+    constexpr int kXcds = 8;
+    if (totalBlocks % kXcds == 0) id = (id % kXcds) * (totalBlocks / kXcds) + id / kXcds;
+    bh = id / numTiles;
+    int t = id - bh * numTiles;
+    tile = heavyIsLast ? numTiles - 1 - t : t;
+}
+
+// Cooperative copy of ROWS rows of one head ([row][hd] slices of a [.., dim] tensor) into LDS as
+// [ROWS][HDP+4], zero-filling rows >= rowLimit and columns >= hd.
+template <int HDP, int ROWS, bool VEC4>
+__device__ __forceinline__ void loadHeadTile(float* __restrict__ lds, const float* __restrict__ base, int dim, int row0,
+                                             int rowLimit, int hd, int tid) {
+    constexpr int LDSW = HDP + 4;
+    constexpr int V4 = HDP / 4;              // float4 slots per row
+    constexpr int SLOTS = ROWS * V4;
+#pragma unroll
+    for (int s = tid; s < SLOTS; s += 256) {
+        int r = s / V4, c = (s % V4) * 4;
+        int row = row0 + r;
+        float4v val = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (row < rowLimit && c < hd) {
+            const float* src = base + size_t(row) * dim + c;
+            if constexpr (VEC4) {
+                val = loadf4(src);
+            } else {
+                val.x = src[0];
+                if (c + 1 < hd) val.y = src[1];
+                if (c + 2 < hd) val.z = src[2];
+                if (c + 3 < hd) val.w = src[3];
+            }
+        }
+        storef4(lds + r * LDSW + c, val);
+    }
+}
+
+// Loads this lane's half of one head row as MFMA operand registers: reg[t] = row[half*HDP/2 + t] * mul.
+template <int HDP, bool VEC4>
+__device__ __forceinline__ void loadRowOperand(float (&reg)[HDP / 2], const float* __restrict__ row, bool valid, int hd,
+                                               int half, float mul) {
+    constexpr int HALF = HDP / 2;
+#pragma unroll
+    for (int t = 0; t < HALF; t += 4) {
+        int d = half * HALF + t;
+        float4v val = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (valid && d < hd) {
+            if constexpr (VEC4) {
+                val = loadf4(row + d);
+            } else {
+                val.x = row[d];
+                if (d + 1 < hd) val.y = row[d + 1];
+                if (d + 2 < hd) val.z = row[d + 2];
+                if (d + 3 < hd) val.w = row[d + 3];
+            }
+        }
+        reg[t] = val.x * mul; reg[t + 1] = val.y * mul; reg[t + 2] = val.z * mul; reg[t + 3] = val.w * mul;
+    }
+}
+
+// acc (32x32) += A * B with A rows read from LDS (row `ldsRow`, this lane's half, ds_read_b128) and B
+// from operand registers: the contraction over the head dimension.
+template <int HDP>
+__device__ __forceinline__ float16v headDot(const float* __restrict__ ldsRow, const float (&breg)[HDP / 2], float16v acc) {
+#pragma unroll
+    for (int t = 0; t < HDP / 2; t += 4) {
+        float4v a = loadf4(ldsRow + t);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, breg[t], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, breg[t + 1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, breg[t + 2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, breg[t + 3], acc, 0, 0, 0);
+    }
+    return acc;
+}
+// Same contraction with the register operand on the A side (key-owner kernel).
+template <int HDP>
+__device__ __forceinline__ float16v headDotB(const float* __restrict__ ldsRow, const float (&areg)[HDP / 2], float16v acc) {
+#pragma unroll
+    for (int t = 0; t < HDP / 2; t += 4) {
+        float4v a = loadf4(ldsRow + t);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, areg[t], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, areg[t + 1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, areg[t + 2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, areg[t + 3], acc, 0, 0, 0);
+    }
+    return acc;
+}
+
+// Row index inside a 32-row MFMA block held by register r of a lane in half `half`.
+__device__ __forceinline__ int dRow(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }
+
+// Stores a transposed accumulator (rows = head-dim index, column = this lane's query/key row) to
+// row `dst` of a [.., dim] tensor: element d = dt*32 + dRow(r, half).
+template <int HDP, bool VEC4>
+__device__ __forceinline__ void storeTransposed(float* __restrict__ dst, const float16v (&acc)[HDP / 32], int hd, int half,
+                                                float mul) {
+#pragma unroll
+    for (int dt = 0; dt < HDP / 32; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            int d = dt * 32 + 8 * g + 4 * half;
+            if (d < hd) {
+                float4v val = {acc[dt][4 * g] * mul, acc[dt][4 * g + 1] * mul, acc[dt][4 * g + 2] * mul, acc[dt][4 * g + 3] * mul};
+                if constexpr (VEC4) {
+                    storef4(dst + d, val);
+                } else {
+                    dst[d] = val.x;
+                    if (d + 1 < hd) dst[d + 1] = val.y;
+                    if (d + 2 < hd) dst[d + 2] = val.z;
+                    if (d + 3 < hd) dst[d + 3] = val.w;
+                }
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------------------
+template <int HDP, int BC, bool VEC4>
+__global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
+    constexpr int LDSW = HDP + 4, DT = HDP / 32;
+    extern __shared__ float smem[];
+    float* ks = smem;
+    float* vs = smem + BC * LDSW;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, qt;
+    decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const float* qb = p.q + size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const float* vb = p.v + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+
+    const int waveQ0 = qt * 128 + wave * 32;
+    const int i = waveQ0 + li;                    // this lane's query row
+    const bool rowValid = i < p.newLen;
+    float qreg[HDP / 2];
+    loadRowOperand<HDP, VEC4>(qreg, qb + size_t(i) * dim, rowValid, hd, half, p.scale * kLog2e);
+
+    float16v acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
+    float mrow = -INFINITY, lrow = 0.0f;
+
+    const int lastQuery = min(p.newLen, qt * 128 + 128) - 1;
+    const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);   // keys >= this are invisible to the tile
+    const int waveKeyEnd = p.oldLen + waveQ0 + 32;                       // keys >= this are invisible to the wave
+    const int myLimit = p.oldLen + i;                                    // last visible key of this lane's row
+
+    for (int kt0 = 0; kt0 < blockKeyEnd; kt0 += BC) {
+        loadHeadTile<HDP, BC, VEC4>(ks, kb, dim, kt0, p.totalLen, hd, tid);
+        loadHeadTile<HDP, BC, VEC4>(vs, vb, dim, kt0, p.totalLen, hd, tid);
+        __syncthreads();
+#pragma unroll
+        for (int sb = 0; sb < BC / 32; ++sb) {
+            const int key0 = kt0 + sb * 32;
+            if (key0 < waveKeyEnd && key0 < p.totalLen) {   // wave-uniform
+                float16v s;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+                s = headDot<HDP>(ks + (sb * 32 + li) * LDSW + half * (HDP / 2), qreg, s);
+                // s[r] = log2-scaled score of (key = key0 + dRow(r), query = i)
+                const bool needMask = (key0 + 31 > p.oldLen + waveQ0) || (key0 + 32 > p.totalLen);
+                if (needMask) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        int key = key0 + dRow(r, half);
+                        if (key > myLimit || key >= p.totalLen) s[r] = -INFINITY;
+                    }
+                }
+                float mx = s[0];
+#pragma unroll
+                for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const float mnew = fmaxf(mrow, mx);
+                const float corr = fastExp2(mrow - mnew);
+                float psum = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { s[r] = fastExp2(s[r] - mnew); psum += s[r]; }
+                lrow = lrow * corr + psum;
+                mrow = mnew;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+                // O^T += V^T * P^T : step r contracts over key dRow(r, half)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float* vrow = vs + (sb * 32 + dRow(r, half)) * LDSW + li;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+                        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[dt * 32], s[r], acc[dt], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    lrow += __shfl_xor(lrow, 32, 64);
+    if (rowValid) {
+        storeTransposed<HDP, VEC4>(p.out + (size_t(b) * p.newLen + i) * dim + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
+        if (half == 0) {
+            size_t idx = (size_t(b) * p.heads + h) * p.newLen + i;
+            p.m[idx] = mrow * kLn2;
+            p.l[idx] = lrow;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward, part 0: D = dot(O, dO) per (batch, head, row), and optionally the log2-domain
+// log-sum-exp lse2 = m*log2(e) + log2(l).  16 lanes per (row, head); HBM-bound.
+// ---------------------------------------------------------------------------------------------
+template <bool VEC4>
+__global__ void __launch_bounds__(256) attnDotKernel(const float* __restrict__ o, const float* __restrict__ dO,
+                                                      const float* __restrict__ m, const float* __restrict__ l,
+                                                      float* __restrict__ dvec, float* __restrict__ lse2, int batch, int heads,
+                                                      int newLen, int dim, int hd) {
+    const size_t groups = size_t(batch) * newLen * heads;    // (b, i, h) with h fastest: contiguous memory
+    const size_t group = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) / 16;
+    const int sub = threadIdx.x & 15;
+    if (group >= groups) return;
+    const size_t bi = group / heads;
+    const int h = int(group - bi * heads);
+    const float* po = o + bi * dim + size_t(h) * hd;
+    const float* pg = dO + bi * dim + size_t(h) * hd;
+    float acc = 0.0f;
+    if constexpr (VEC4) {
+        for (int d = sub * 4; d < hd; d += 64) {
+            float4v a = loadf4(po + d), g = loadf4(pg + d);
+            acc += a.x * g.x + a.y * g.y + a.z * g.z + a.w * g.w;
+        }
+    } else {
+        for (int d = sub; d < hd; d += 16) acc += po[d] * pg[d];
+    }
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (sub == 0) {
+        const size_t b = bi / newLen, i = bi - b * newLen;
+        const size_t idx = (b * heads + h) * newLen + i;
+        dvec[idx] = acc;
+        if (lse2) lse2[idx] = m[idx] * kLog2e + log2f(l[idx]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward, part 1: dQ (query-tile owner).  Same streaming structure as the forward.
+// ---------------------------------------------------------------------------------------------
+template <int HDP, int BC, bool VEC4>
+__global__ void __launch_bounds__(256) attnBackwardDqKernel(AttnParams p) {
+    constexpr int LDSW = HDP + 4, DT = HDP / 32;
+    extern __shared__ float smem[];
+    float* ks = smem;
+    float* vs = smem + BC * LDSW;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, qt;
+    decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const size_t qOff = size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const float* vb = p.v + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+
+    const int waveQ0 = qt * 128 + wave * 32;
+    const int i = waveQ0 + li;
+    const bool rowValid = i < p.newLen;
+    float qreg[HDP / 2], greg[HDP / 2];
+    loadRowOperand<HDP, VEC4>(qreg, p.q + qOff + size_t(i) * dim, rowValid, hd, half, p.scale * kLog2e);
+    loadRowOperand<HDP, VEC4>(greg, p.dO + qOff + size_t(i) * dim, rowValid, hd, half, 1.0f);
+    const size_t statIdx = (size_t(b) * p.heads + h) * p.newLen + i;
+    const float lse = rowValid ? p.lse2[statIdx] : INFINITY;   // padding rows: exp2(s - inf) = 0
+    const float dval = rowValid ? p.dvec[statIdx] : 0.0f;
+
+    float16v acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
+
+    const int lastQuery = min(p.newLen, qt * 128 + 128) - 1;
+    const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);
+    const int waveKeyEnd = p.oldLen + waveQ0 + 32;
+    const int myLimit = p.oldLen + i;
+
+    for (int kt0 = 0; kt0 < blockKeyEnd; kt0 += BC) {
+        loadHeadTile<HDP, BC, VEC4>(ks, kb, dim, kt0, p.totalLen, hd, tid);
+        loadHeadTile<HDP, BC, VEC4>(vs, vb, dim, kt0, p.totalLen, hd, tid);
+        __syncthreads();
+#pragma unroll
+        for (int sb = 0; sb < BC / 32; ++sb) {
+            const int key0 = kt0 + sb * 32;
+            if (key0 < waveKeyEnd && key0 < p.totalLen) {
+                float16v s, dp;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { s[r] = 0.0f; dp[r] = 0.0f; }
+                s = headDot<HDP>(ks + (sb * 32 + li) * LDSW + half * (HDP / 2), qreg, s);     // S^T  = K  * Q^T
+                dp = headDot<HDP>(vs + (sb * 32 + li) * LDSW + half * (HDP / 2), greg, dp);   // dP^T = V  * dO^T
+                const bool needMask = (key0 + 31 > p.oldLen + waveQ0) || (key0 + 32 > p.totalLen);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float prob = fastExp2(s[r] - lse);
+                    if (needMask) {
+                        int key = key0 + dRow(r, half);
+                        if (key > myLimit || key >= p.totalLen) prob = 0.0f;
+                    }
+                    s[r] = prob * (dp[r] - dval);   // dS^T (without the scale factor)
+                }
+                // dQ^T += K^T * dS^T : step r contracts over key dRow(r, half)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float* krow = ks + (sb * 32 + dRow(r, half)) * LDSW + li;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+                        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[dt * 32], s[r], acc[dt], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (rowValid) storeTransposed<HDP, VEC4>(p.dQ + qOff + size_t(i) * dim, acc, hd, half, p.scale);
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward, part 2: dK, dV (key-tile owner).  K and V of the wave's 32 keys stay in registers as MFMA
+// B operands; Q/dO tiles and the per-row statistics are streamed through LDS.
+// ---------------------------------------------------------------------------------------------
+template <int HDP, int BQ, bool VEC4>
+__global__ void __launch_bounds__(256) attnBackwardDkvKernel(AttnParams p) {
+    constexpr int LDSW = HDP + 4, DT = HDP / 32;
+    extern __shared__ float smem[];
+    float* qs = smem;
+    float* gs = smem + BQ * LDSW;
+    float* lses = gs + BQ * LDSW;   // [BQ]
+    float* dvs = lses + BQ;         // [BQ]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, kt;
+    decodeBlock(p.numTiles, gridDim.x, false, bh, kt);   // the first key tile is seen by every query: heaviest
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const size_t qOff = size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const size_t kOff = size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const size_t statOff = (size_t(b) * p.heads + h) * p.newLen;
+
+    const int waveK0 = kt * 128 + wave * 32;
+    const int key = waveK0 + li;                       // this lane's key (as B-operand column)
+    const bool keyValid = key < p.totalLen;
+    float kreg[HDP / 2], vreg[HDP / 2];
+    loadRowOperand<HDP, VEC4>(kreg, p.k + kOff + size_t(key) * dim, keyValid, hd, half, p.scale * kLog2e);
+    loadRowOperand<HDP, VEC4>(vreg, p.v + kOff + size_t(key) * dim, keyValid, hd, half, 1.0f);
+
+    float16v dk[DT], dv[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.0f; dv[dt][r] = 0.0f; }
+
+    // first query that can see any key of this workgroup's tile: oldLen + i >= kt*128
+    int firstQuery = kt * 128 - p.oldLen;
+    if (firstQuery < 0) firstQuery = 0;
+    const int q0Start = (firstQuery / BQ) * BQ;
+
+    for (int qt0 = q0Start; qt0 < p.newLen; qt0 += BQ) {
+        loadHeadTile<HDP, BQ, VEC4>(qs, p.q + qOff, dim, qt0, p.newLen, hd, tid);
+        loadHeadTile<HDP, BQ, VEC4>(gs, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+        if (tid < BQ) {
+            int qi = qt0 + tid;
+            lses[tid] = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
+            dvs[tid] = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int sb = 0; sb < BQ / 32; ++sb) {
+            const int q0 = qt0 + sb * 32;
+            // the wave's keys [waveK0, waveK0+32) are visible to some query of [q0, q0+32)?
+            if (q0 < p.newLen && p.oldLen + q0 + 31 >= waveK0 && waveK0 < p.totalLen) {
+                float16v s, dp;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { s[r] = 0.0f; dp[r] = 0.0f; }
+                s = headDotB<HDP>(qs + (sb * 32 + li) * LDSW + half * (HDP / 2), kreg, s);    // S  = Q  * K^T
+                dp = headDotB<HDP>(gs + (sb * 32 + li) * LDSW + half * (HDP / 2), vreg, dp);  // dP = dO * V^T
+                // register r: query = q0 + dRow(r, half), key = this lane's key
+                const bool needMask = (waveK0 + 31 > p.oldLen + q0) || (waveK0 + 32 > p.totalLen);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float4v lse4 = loadf4(lses + sb * 32 + 8 * g + 4 * half);
+                    float4v d4 = loadf4(dvs + sb * 32 + 8 * g + 4 * half);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int r = 4 * g + c;
+                        float prob = fastExp2(s[r] - lse4[c]);
+                        if (needMask) {
+                            int qi = q0 + dRow(r, half);
+                            if (key > p.oldLen + qi || !keyValid) prob = 0.0f;
+                        }
+                        s[r] = prob;                        // P
+                        dp[r] = prob * (dp[r] - d4[c]);     // dS (without the scale factor)
+                    }
+                }
+                // dV += P^T * dO, dK += dS^T * Q : step r contracts over query dRow(r, half)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float* grow = gs + (sb * 32 + dRow(r, half)) * LDSW + li;
+                    const float* qrow = qs + (sb * 32 + dRow(r, half)) * LDSW + li;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        dv[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(s[r], grow[dt * 32], dv[dt], 0, 0, 0);
+                        dk[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(dp[r], qrow[dt * 32], dk[dt], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // dk/dv[dt][r]: key = waveK0 + dRow(r, half), d = dt*32 + li  -> 128-byte coalesced rows
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const int d = dt * 32 + li;
+        if (d < hd) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int kk = waveK0 + dRow(r, half);
+                if (kk < p.totalLen) {
+                    p.dK[kOff + size_t(kk) * dim + d] = dk[dt][r] * p.scale;
+                    p.dV[kOff + size_t(kk) * dim + d] = dv[dt][r];
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------
+int paddedHeadDim(int hd) { return hd <= 32 ? 32 : hd <= 64 ? 64 : hd <= 128 ? 128 : 256; }
+
+template <typename K>
+int launchAttn(K kernel, size_t smemBytes, unsigned grid, const AttnParams& p, hipStream_t s) {
+    if (smemBytes > 48 * 1024)
+        BF_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       int(smemBytes)));
+    kernel<<<grid, 256, smemBytes, s>>>(p);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+bool vec4Ok(const AttnParams& p, std::initializer_list<const void*> ptrs) {
+    if (p.hd % 4 != 0 || p.dim % 4 != 0) return false;
+    for (const void* q : ptrs)
+        if (q && (reinterpret_cast<uintptr_t>(q) & 15u)) return false;
+    return true;
+}
+
+// KIND 0 forward, 1 dQ, 2 dK/dV
+template <int KIND, int HDP, int TILE>
+int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
+    constexpr size_t tileBytes = size_t(2) * TILE * (HDP + 4) * sizeof(float);
+    constexpr size_t smem = KIND == 2 ? tileBytes + 2 * TILE * sizeof(float) : tileBytes;
+    if constexpr (KIND == 0) {
+        return vec4 ? launchAttn(attnForwardKernel<HDP, TILE, true>, smem, grid, p, s)
+                    : launchAttn(attnForwardKernel<HDP, TILE, false>, smem, grid, p, s);
+    } else if constexpr (KIND == 1) {
+        return vec4 ? launchAttn(attnBackwardDqKernel<HDP, TILE, true>, smem, grid, p, s)
+                    : launchAttn(attnBackwardDqKernel<HDP, TILE, false>, smem, grid, p, s);
+    } else {
+        return vec4 ? launchAttn(attnBackwardDkvKernel<HDP, TILE, true>, smem, grid, p, s)
+                    : launchAttn(attnBackwardDkvKernel<HDP, TILE, false>, smem, grid, p, s);
+    }
+}
+
+template <int KIND>
+int dispatch(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
+    switch (paddedHeadDim(p.hd)) {
+        case 32: return dispatchVec<KIND, 32, 64>(p, vec4, grid, s);
+        case 64: return dispatchVec<KIND, 64, 64>(p, vec4, grid, s);
+        case 128: return dispatchVec<KIND, 128, 32>(p, vec4, grid, s);
+        default: return dispatchVec<KIND, 256, 32>(p, vec4, grid, s);
+    }
+}
+
+int checkShapes(const char* fn, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, size_t oldLen) {
+    if (heads == 0 || dim % heads != 0)
+        return failInvalid(fn, "numHeads (" + std::to_string(heads) + ") must divide dim (" + std::to_string(dim) + ")");
+    size_t hd = dim / heads;
+    if (hd > 256)
+        return failInvalid(fn, "headDim (" + std::to_string(hd) + ") exceeds the supported limit of the fused kernel (256)");
+    if (newLen > 0 && batch > 0 && totalLen == 0) return failInvalid(fn, "totalLen is 0");
+    if (batch * heads * ((newLen + 127) / 128 + (totalLen + 127) / 128) >= (size_t(1) << 31) || totalLen + oldLen + newLen >= (size_t(1) << 30) ||
+        dim >= (size_t(1) << 24))
+        return failInvalid(fn, "shape too large");
+    return BF_OK;
+}
+
+}  // namespace
+}  // namespace bf
+
+using namespace bf;
+
+extern "C" {
+
+int bf_hip_attention_forward(const float* q, const float* k, const float* v, float* out, float* m, float* l,
+                             size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
+                             size_t oldLen, bf_stream_t stream) {
+    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+    if (st != BF_OK) return st;
+    if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(q && k && v && out && m && l, "NULL pointer");
+    AttnParams p{};
+    p.q = q; p.k = k; p.v = v; p.out = out; p.m = m; p.l = l;
+    p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(totalLen);
+    p.dim = int(dim); p.hd = int(dim / heads); p.oldLen = int(oldLen); p.scale = scale;
+    p.numTiles = int((newLen + 127) / 128);
+    unsigned grid = unsigned(batch * heads * size_t(p.numTiles));
+    return dispatch<0>(p, vec4Ok(p, {q, k, v, out}), grid, asStream(stream));
+}
+
+int bf_hip_attention_dot_o_do(const float* out, const float* dOut, float* D, size_t batch, size_t heads, size_t newLen,
+                              size_t dim, bf_stream_t stream) {
+    BF_REQUIRE(heads != 0 && dim % heads == 0, "numHeads must divide dim");
+    if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(out && dOut && D, "NULL pointer");
+    size_t groups = batch * newLen * heads;
+    int hd = int(dim / heads);
+    bool vec4 = hd % 4 == 0 && dim % 4 == 0 && ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dOut)) & 15u) == 0;
+    unsigned grid = gridFor(groups * 16, 256, 1u << 30);
+    if (vec4) attnDotKernel<true><<<grid, 256, 0, asStream(stream)>>>(out, dOut, nullptr, nullptr, D, nullptr, int(batch), int(heads), int(newLen), int(dim), hd);
+    else attnDotKernel<false><<<grid, 256, 0, asStream(stream)>>>(out, dOut, nullptr, nullptr, D, nullptr, int(batch), int(heads), int(newLen), int(dim), hd);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_attention_backward(const float* dOut, const float* q, const float* k, const float* v, const float* out,
+                              const float* m, const float* l, float* dQ, float* dK, float* dV, size_t batch,
+                              size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
+                              bf_stream_t stream) {
+    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+    if (st != BF_OK) return st;
+    if (batch == 0 || dim == 0) return BF_OK;
+    hipStream_t s = asStream(stream);
+    if (newLen == 0) {   // no query: key/value gradients are zero
+        if (totalLen) {
+            BF_REQUIRE(dK && dV, "NULL pointer");
+            st = bf_hip_fill_zero(dK, batch * totalLen * dim * sizeof(float), stream);
+            if (st != BF_OK) return st;
+            return bf_hip_fill_zero(dV, batch * totalLen * dim * sizeof(float), stream);
+        }
+        return BF_OK;
+    }
+    BF_REQUIRE(dOut && q && k && v && out && m && l && dQ && dK && dV, "NULL pointer");
+    AttnParams p{};
+    p.q = q; p.k = k; p.v = v; p.o = out; p.dO = dOut; p.dQ = dQ; p.dK = dK; p.dV = dV;
+    p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(totalLen);
+    p.dim = int(dim); p.hd = int(dim / heads); p.oldLen = int(oldLen); p.scale = scale;
+
+    // workspace: lse2 | D, each [batch, heads, newLen]
+    size_t stats = batch * heads * newLen;
+    Scratch work(2 * stats * sizeof(float));
+    if (work.status != BF_OK) return work.status;
+    float* lse2 = work.as<float>();
+    float* dvec = lse2 + stats;
+    {
+        bool vec4 = p.hd % 4 == 0 && dim % 4 == 0 && ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dOut)) & 15u) == 0;
+        unsigned grid = gridFor(stats * 16, 256, 1u << 30);
+        if (vec4) attnDotKernel<true><<<grid, 256, 0, s>>>(out, dOut, m, l, dvec, lse2, p.batch, p.heads, p.newLen, p.dim, p.hd);
+        else attnDotKernel<false><<<grid, 256, 0, s>>>(out, dOut, m, l, dvec, lse2, p.batch, p.heads, p.newLen, p.dim, p.hd);
+        BF_LAUNCH_CHECK();
+    }
+    p.lse2 = lse2;
+    p.dvec = dvec;
+
+    p.numTiles = int((totalLen + 127) / 128);
+    st = dispatch<2>(p, vec4Ok(p, {q, k, v, dOut}), unsigned(batch * heads * size_t(p.numTiles)), s);
+    if (st != BF_OK) return st;
+    p.numTiles = int((newLen + 127) / 128);
+    return dispatch<1>(p, vec4Ok(p, {q, k, v, dOut, dQ}), unsigned(batch * heads * size_t(p.numTiles)), s);
+}
+
+}  // extern "C"

@@ -1,0 +1,146 @@
+// Shared host/device helpers for the gfx950 operator library (internal; not part of the C ABI).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "bf_hip.h"
+
+namespace bf {
+
+// ---- error reporting ---------------------------------------------------------------------------
+void setLastError(const std::string& message);
+int failInvalid(const char* function, const std::string& message);
+int failRuntime(const char* function, hipError_t error, const char* file, int line);
+
+#define BF_REQUIRE(cond, msg)                                       \
+    do {                                                            \
+        if (!(cond)) return ::bf::failInvalid(__func__, (msg));     \
+    } while (0)
+
+#define BF_HIP_TRY(expr)                                                            \
+    do {                                                                            \
+        hipError_t bf_err_ = (expr);                                                \
+        if (bf_err_ != hipSuccess) return ::bf::failRuntime(__func__, bf_err_, __FILE__, __LINE__); \
+    } while (0)
+
+#define BF_LAUNCH_CHECK() BF_HIP_TRY(hipGetLastError())
+
+inline hipStream_t asStream(bf_stream_t s) { return static_cast<hipStream_t>(s); }
+
+// ---- launch geometry ---------------------------------------------------------------------------
+constexpr int kWave = 64;            // CDNA wavefront
+constexpr int kBlock = 256;          // 4 waves: one per SIMD of a CU
+constexpr unsigned kMaxGridX = 1u << 20;
+
+inline unsigned gridFor(size_t work, size_t perBlock, unsigned cap = kMaxGridX) {
+    size_t blocks = (work + perBlock - 1) / perBlock;
+    if (blocks < 1) blocks = 1;
+    if (blocks > cap) blocks = cap;
+    return static_cast<unsigned>(blocks);
+}
+
+// Number of compute units of the current device (cached); used to size persistent grids.
+int computeUnits();
+
+// Scratch memory from the per-device pool, returned on scope exit.  The release only puts the block
+// back on the pool's free list; kernels already enqueued on a stream keep using it safely because
+// every later user of the block is enqueued behind them on the same stream or is ordered by the
+// caller (single host thread, one stream at a time per device, like the reference).
+struct Scratch {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    int status = BF_OK;
+    explicit Scratch(size_t n) : bytes(n) { status = bf_hip_pool_acquire(n, &ptr); }
+    ~Scratch() { if (ptr) bf_hip_pool_release(ptr, bytes); }
+    Scratch(const Scratch&) = delete;
+    Scratch& operator=(const Scratch&) = delete;
+    template <typename T> T* as() const { return static_cast<T*>(ptr); }
+};
+
+// A small table of descriptors (pointers, counts, chunk lists) that a multi-tensor kernel reads from
+// device memory.  The same table is needed step after step, so the device copy is kept per (device,
+// slot) and re-uploaded only when the host bytes change; an unchanged table costs no copy and no
+// host synchronisation.  `slot` separates users (zero, sgd, adamw).
+enum { kSlotZero = 0, kSlotSgd = 1, kSlotAdamW = 2, kSlotCount = 3 };
+int uploadDescriptorTable(int slot, const void* hostBytes, size_t bytes, hipStream_t stream, const void** devicePtr);
+
+// ---- device helpers ----------------------------------------------------------------------------
+#if defined(__HIPCC__)
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float waveSum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ double waveSumD(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float waveMax(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Block-wide reductions for blocks of up to 1024 threads (16 waves).  `scratch` must hold 16 values.
+template <typename T, typename Op>
+__device__ __forceinline__ T blockReduce(T v, T identity, Op op, T* scratch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = (blockDim.x + 63) >> 6;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, 64));
+    __syncthreads();  // protect scratch from a previous reduction still being read
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    T r = identity;
+    for (int w = 0; w < waves; ++w) r = op(r, scratch[w]);  // same order in every thread
+    return r;
+}
+struct OpSum { template <typename T> __device__ T operator()(T a, T b) const { return a + b; } };
+struct OpMaxF { __device__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+
+__device__ __forceinline__ float4v loadf4(const float* p) { return *reinterpret_cast<const float4v*>(p); }
+__device__ __forceinline__ void storef4(float* p, float4v v) { *reinterpret_cast<float4v*>(p) = v; }
+
+// Accurate activations: the formulas of the reference CPU backend, evaluated with the accurate
+// libm-style device functions (no fast-math approximations), so results stay within 1e-6 relative.
+__device__ __forceinline__ float siluF(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float reluF(float x) { return x > 0.0f ? x : 0.0f; }
+__device__ __forceinline__ float geluF(float x) {
+    float inner = 0.7978845608f * (x + 0.044715f * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(inner));
+}
+__device__ __forceinline__ float siluD(float x) {
+    float s = 1.0f / (1.0f + expf(-x));
+    return s * (1.0f + x * (1.0f - s));
+}
+__device__ __forceinline__ float reluD(float x) { return x > 0.0f ? 1.0f : 0.0f; }
+__device__ __forceinline__ float geluD(float x) {
+    float inner = 0.7978845608f * (x + 0.044715f * x * x * x);
+    float t = tanhf(inner);
+    float dInner = 0.7978845608f * (1.0f + 3.0f * 0.044715f * x * x);
+    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * dInner;
+}
+template <int ACT> __device__ __forceinline__ float actF(float x) {
+    if constexpr (ACT == BF_ACT_SILU) return siluF(x);
+    else if constexpr (ACT == BF_ACT_GELU) return geluF(x);
+    else return reluF(x);
+}
+template <int ACT> __device__ __forceinline__ float actD(float x) {
+    if constexpr (ACT == BF_ACT_SILU) return siluD(x);
+    else if constexpr (ACT == BF_ACT_GELU) return geluD(x);
+    else return reluD(x);
+}
+
+#endif  // __HIPCC__
+
+}  // namespace bf

@@ -1,0 +1,371 @@
+// Elementwise family: add, scale, bias (+activation, +residual), activations and their
+// derivatives, gradient accumulate, multi-tensor zero.
+//
+// All of these are HBM-bound (8-12 algorithmic bytes per element), so each kernel moves 16 bytes
+// per lane per access (dwordx4), keeps a few thousand wavefronts in flight with a grid-stride
+// loop, and the bias kernels use a 2-D thread layout (column fixed per thread, rows strided) so that
+// no integer division sits on the memory path and the bias vector is read once per thread.
+#include "common.hpp"
+
+#include <vector>
+
+namespace bf {
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- flat kernels -----------------------------------------------------------------------------
+template <typename F>
+__global__ void __launch_bounds__(kBlock) flat4Kernel(size_t n4, F f) {
+    size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) f.vec(i);
+}
+template <typename F>
+__global__ void __launch_bounds__(kBlock) flat1Kernel(size_t begin, size_t n, F f) {
+    size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = begin + size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) f.one(i);
+}
+
+// Runs f.vec(i) over groups of four elements when every pointer is 16-byte aligned, then f.one(i) over
+// the tail (or over everything otherwise).
+template <typename F>
+int launchFlat(size_t n, bool canVectorise, F f, hipStream_t stream) {
+    if (n == 0) return BF_OK;
+    const unsigned cap = unsigned(computeUnits()) * 16;
+    size_t done = 0;
+    if (canVectorise && n >= 4) {
+        size_t n4 = n / 4;
+        flat4Kernel<<<gridFor(n4, kBlock, cap), kBlock, 0, stream>>>(n4, f);
+        BF_LAUNCH_CHECK();
+        done = n4 * 4;
+    }
+    if (done < n) {
+        flat1Kernel<<<gridFor(n - done, kBlock, cap), kBlock, 0, stream>>>(done, n, f);
+        BF_LAUNCH_CHECK();
+    }
+    return BF_OK;
+}
+
+struct AddOp {
+    const float* a; const float* b; float* out;
+    __device__ void vec(size_t i) const { storef4(out + 4 * i, loadf4(a + 4 * i) + loadf4(b + 4 * i)); }
+    __device__ void one(size_t i) const { out[i] = a[i] + b[i]; }
+};
+struct ScaleOp {
+    const float* x; float* out; float factor;
+    __device__ void vec(size_t i) const { storef4(out + 4 * i, loadf4(x + 4 * i) * factor); }
+    __device__ void one(size_t i) const { out[i] = x[i] * factor; }
+};
+struct AccumulateOp {
+    float* target; const float* delta;
+    __device__ void vec(size_t i) const { storef4(target + 4 * i, loadf4(target + 4 * i) + loadf4(delta + 4 * i)); }
+    __device__ void one(size_t i) const { target[i] += delta[i]; }
+};
+template <int ACT>
+struct ActForwardOp {
+    const float* x; float* out;
+    __device__ void vec(size_t i) const {
+        float4v v = loadf4(x + 4 * i);
+        v.x = actF<ACT>(v.x); v.y = actF<ACT>(v.y); v.z = actF<ACT>(v.z); v.w = actF<ACT>(v.w);
+        storef4(out + 4 * i, v);
+    }
+    __device__ void one(size_t i) const { out[i] = actF<ACT>(x[i]); }
+};
+template <int ACT>
+struct ActBackwardOp {
+    const float* x; const float* g; float* out;
+    __device__ void vec(size_t i) const {
+        float4v v = loadf4(x + 4 * i), gv = loadf4(g + 4 * i);
+        v.x = gv.x * actD<ACT>(v.x); v.y = gv.y * actD<ACT>(v.y); v.z = gv.z * actD<ACT>(v.z); v.w = gv.w * actD<ACT>(v.w);
+        storef4(out + 4 * i, v);
+    }
+    __device__ void one(size_t i) const { out[i] = g[i] * actD<ACT>(x[i]); }
+};
+
+// ---- row/column kernels (bias family) ---------------------------------------------------------
+// Thread layout: blockDim = (bx, by); a thread owns column group (blockIdx.x*bx + tx) and walks rows
+// blockIdx.y*by + ty, stepping gridDim.y*by.
+struct RowGeom {
+    dim3 grid, block;
+    int vec;
+};
+
+RowGeom rowGeometry(size_t rows, size_t features, bool canVectorise, unsigned maxRowBlocks = 0) {
+    RowGeom g;
+    g.vec = (canVectorise && features % 4 == 0) ? 4 : 1;
+    size_t cols = features / g.vec;
+    unsigned bx = 1;
+    while (bx < 256 && bx < cols) bx <<= 1;
+    unsigned by = 256 / bx;
+    unsigned gx = unsigned((cols + bx - 1) / bx);
+    size_t rowBlocks = (rows + by - 1) / by;
+    size_t want = size_t(computeUnits()) * 16 / (gx ? gx : 1);
+    if (want < 1) want = 1;
+    if (rowBlocks > want) rowBlocks = want;
+    if (maxRowBlocks && rowBlocks > maxRowBlocks) rowBlocks = maxRowBlocks;
+    if (rowBlocks > 65535) rowBlocks = 65535;
+    if (rowBlocks < 1) rowBlocks = 1;
+    g.block = dim3(bx, by);
+    g.grid = dim3(gx, unsigned(rowBlocks));
+    return g;
+}
+
+template <int VEC> struct Pack;
+template <> struct Pack<4> {
+    using T = float4v;
+    static __device__ T load(const float* p) { return loadf4(p); }
+    static __device__ void store(float* p, T v) { storef4(p, v); }
+};
+template <> struct Pack<1> {
+    using T = float;
+    static __device__ T load(const float* p) { return *p; }
+    static __device__ void store(float* p, T v) { *p = v; }
+};
+template <int ACT> __device__ float4v actF4(float4v v) {
+    v.x = actF<ACT>(v.x); v.y = actF<ACT>(v.y); v.z = actF<ACT>(v.z); v.w = actF<ACT>(v.w); return v;
+}
+template <int ACT> __device__ float actF4(float v) { return actF<ACT>(v); }
+template <int ACT> __device__ float4v actD4(float4v v) {
+    v.x = actD<ACT>(v.x); v.y = actD<ACT>(v.y); v.z = actD<ACT>(v.z); v.w = actD<ACT>(v.w); return v;
+}
+template <int ACT> __device__ float actD4(float v) { return actD<ACT>(v); }
+
+// MODE 0: x + bias; 1: act(x + bias); 2: x + bias + residual
+template <int VEC, int MODE, int ACT>
+__global__ void __launch_bounds__(256) biasKernel(const float* __restrict__ x, const float* __restrict__ bias,
+                                                   const float* __restrict__ residual, float* __restrict__ out,
+                                                   size_t rows, size_t features) {
+    size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
+    if (col >= features) return;
+    typename Pack<VEC>::T b = Pack<VEC>::load(bias + col);
+    size_t rowStep = size_t(gridDim.y) * blockDim.y;
+    for (size_t r = size_t(blockIdx.y) * blockDim.y + threadIdx.y; r < rows; r += rowStep) {
+        size_t idx = r * features + col;
+        typename Pack<VEC>::T v = Pack<VEC>::load(x + idx) + b;
+        if constexpr (MODE == 1) v = actF4<ACT>(v);
+        if constexpr (MODE == 2) v = v + Pack<VEC>::load(residual + idx);
+        Pack<VEC>::store(out + idx, v);
+    }
+}
+
+// Column sums, optionally fused with dGemm = dHidden * act'(gemm + bias) (FUSED = 1).
+// Each block reduces its rows per column in registers, then over threadIdx.y through LDS, and writes
+// one partial row per blockIdx.y; columnFinishKernel adds the partial rows in a fixed order.
+template <int VEC, int FUSED, int ACT>
+__global__ void __launch_bounds__(256) columnSumKernel(const float* __restrict__ src, const float* __restrict__ bias,
+                                                        const float* __restrict__ dHidden, float* __restrict__ dGemm,
+                                                        float* __restrict__ partial, size_t rows, size_t features) {
+    __shared__ float lds[256 * 4];
+    size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
+    bool active = col < features;
+    typename Pack<VEC>::T acc = {};
+    if (active) {
+        typename Pack<VEC>::T b = {};
+        if constexpr (FUSED) b = Pack<VEC>::load(bias + col);
+        size_t rowStep = size_t(gridDim.y) * blockDim.y;
+        for (size_t r = size_t(blockIdx.y) * blockDim.y + threadIdx.y; r < rows; r += rowStep) {
+            size_t idx = r * features + col;
+            typename Pack<VEC>::T v = Pack<VEC>::load(src + idx);
+            if constexpr (FUSED) {
+                v = Pack<VEC>::load(dHidden + idx) * actD4<ACT>(v + b);
+                Pack<VEC>::store(dGemm + idx, v);
+            }
+            acc = acc + v;
+        }
+    }
+    if (partial == nullptr) return;
+    // reduce over threadIdx.y (fixed order), result in the ty == 0 threads
+    int slot = (threadIdx.y * blockDim.x + threadIdx.x) * VEC;
+    if constexpr (VEC == 4) { lds[slot] = acc.x; lds[slot + 1] = acc.y; lds[slot + 2] = acc.z; lds[slot + 3] = acc.w; }
+    else lds[slot] = acc;
+    __syncthreads();
+    if (threadIdx.y == 0 && active) {
+        for (int j = 0; j < VEC; ++j) {
+            float s = 0.0f;
+            for (unsigned ty = 0; ty < blockDim.y; ++ty) s += lds[(ty * blockDim.x + threadIdx.x) * VEC + j];
+            partial[size_t(blockIdx.y) * features + col + j] = s;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kBlock) columnFinishKernel(const float* __restrict__ partial, float* __restrict__ out,
+                                                             size_t parts, size_t features) {
+    size_t c = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= features) return;
+    float s = 0.0f;
+    for (size_t p = 0; p < parts; ++p) s += partial[p * features + c];
+    out[c] = s;
+}
+
+template <int FUSED, int ACT>
+int launchColumnSum(const float* src, const float* bias, const float* dHidden, float* dGemm, float* dBias,
+                    size_t rows, size_t features, hipStream_t stream) {
+    if (features == 0) return BF_OK;
+    if (rows == 0) {
+        if (dBias) return bf_hip_fill_zero(dBias, features * sizeof(float), stream);
+        return BF_OK;
+    }
+    bool vec = aligned16(src) && (!FUSED || (aligned16(bias) && aligned16(dHidden) && aligned16(dGemm)));
+    RowGeom g = rowGeometry(rows, features, vec, 128);
+    size_t parts = g.grid.y;
+    Scratch scratch(dBias ? parts * features * sizeof(float) : 0);
+    if (scratch.status != BF_OK) return scratch.status;
+    float* partial = dBias ? scratch.as<float>() : nullptr;
+    if (g.vec == 4)
+        columnSumKernel<4, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
+    else
+        columnSumKernel<1, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
+    BF_LAUNCH_CHECK();
+    if (dBias) {
+        columnFinishKernel<<<gridFor(features, kBlock), kBlock, 0, stream>>>(partial, dBias, parts, features);
+        BF_LAUNCH_CHECK();
+    }
+    return BF_OK;
+}
+
+struct ZeroTarget {
+    float* ptr;
+    size_t count;
+};
+
+// One block per chunk of one tensor; chunk table built on the host so that every block has work.
+struct ZeroChunk {
+    float* ptr;
+    unsigned count;
+};
+__global__ void __launch_bounds__(kBlock) zeroMultiKernel(const ZeroChunk* chunks) {
+    ZeroChunk c = chunks[blockIdx.x];
+    for (unsigned i = threadIdx.x; i < c.count; i += blockDim.x) c.ptr[i] = 0.0f;
+}
+
+}  // namespace
+}  // namespace bf
+
+using namespace bf;
+
+extern "C" {
+
+int bf_hip_add(const float* a, const float* b, float* out, size_t n, bf_stream_t stream) {
+    if (n == 0) return BF_OK;
+    BF_REQUIRE(a && b && out, "NULL pointer");
+    return launchFlat(n, aligned16(a) && aligned16(b) && aligned16(out), AddOp{a, b, out}, asStream(stream));
+}
+
+int bf_hip_scale(const float* x, float factor, float* out, size_t n, bf_stream_t stream) {
+    if (n == 0) return BF_OK;
+    BF_REQUIRE(x && out, "NULL pointer");
+    return launchFlat(n, aligned16(x) && aligned16(out), ScaleOp{x, out, factor}, asStream(stream));
+}
+
+int bf_hip_accumulate(float* target, const float* delta, size_t n, bf_stream_t stream) {
+    if (n == 0) return BF_OK;
+    BF_REQUIRE(target && delta, "NULL pointer");
+    return launchFlat(n, aligned16(target) && aligned16(delta), AccumulateOp{target, delta}, asStream(stream));
+}
+
+int bf_hip_act_forward(const float* x, float* out, size_t n, int act, bf_stream_t stream) {
+    if (n == 0) return BF_OK;
+    BF_REQUIRE(x && out, "NULL pointer");
+    bool vec = aligned16(x) && aligned16(out);
+    switch (act) {
+        case BF_ACT_SILU: return launchFlat(n, vec, ActForwardOp<BF_ACT_SILU>{x, out}, asStream(stream));
+        case BF_ACT_GELU: return launchFlat(n, vec, ActForwardOp<BF_ACT_GELU>{x, out}, asStream(stream));
+        case BF_ACT_RELU: return launchFlat(n, vec, ActForwardOp<BF_ACT_RELU>{x, out}, asStream(stream));
+        default: return failInvalid(__func__, "unknown activation " + std::to_string(act));
+    }
+}
+
+int bf_hip_act_backward(const float* x, const float* g, float* out, size_t n, int act, bf_stream_t stream) {
+    if (n == 0) return BF_OK;
+    BF_REQUIRE(x && g && out, "NULL pointer");
+    bool vec = aligned16(x) && aligned16(g) && aligned16(out);
+    switch (act) {
+        case BF_ACT_SILU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_SILU>{x, g, out}, asStream(stream));
+        case BF_ACT_GELU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_GELU>{x, g, out}, asStream(stream));
+        case BF_ACT_RELU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_RELU>{x, g, out}, asStream(stream));
+        default: return failInvalid(__func__, "unknown activation " + std::to_string(act));
+    }
+}
+
+#define BF_BIAS_LAUNCH(MODE, ACT)                                                                               \
+    do {                                                                                                        \
+        if (g.vec == 4)                                                                                         \
+            biasKernel<4, MODE, ACT><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
+        else                                                                                                    \
+            biasKernel<1, MODE, ACT><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
+    } while (0)
+
+int bf_hip_add_bias(const float* x, const float* bias, float* out, size_t rows, size_t features, bf_stream_t stream) {
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && bias && out, "NULL pointer");
+    const float* residual = nullptr;
+    RowGeom g = rowGeometry(rows, features, aligned16(x) && aligned16(bias) && aligned16(out));
+    BF_BIAS_LAUNCH(0, 0);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_add_bias_act(const float* x, const float* bias, float* out, size_t rows, size_t features, int act,
+                        bf_stream_t stream) {
+    BF_REQUIRE(act == BF_ACT_SILU || act == BF_ACT_GELU || act == BF_ACT_RELU, "unknown activation " + std::to_string(act));
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && bias && out, "NULL pointer");
+    const float* residual = nullptr;
+    RowGeom g = rowGeometry(rows, features, aligned16(x) && aligned16(bias) && aligned16(out));
+    if (act == BF_ACT_SILU) BF_BIAS_LAUNCH(1, BF_ACT_SILU);
+    else if (act == BF_ACT_GELU) BF_BIAS_LAUNCH(1, BF_ACT_GELU);
+    else BF_BIAS_LAUNCH(1, BF_ACT_RELU);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_add_bias_residual(const float* x, const float* bias, const float* residual, float* out, size_t rows,
+                             size_t features, bf_stream_t stream) {
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && bias && residual && out, "NULL pointer");
+    RowGeom g = rowGeometry(rows, features, aligned16(x) && aligned16(bias) && aligned16(out) && aligned16(residual));
+    BF_BIAS_LAUNCH(2, 0);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_bias_grad(const float* g, float* dBias, size_t rows, size_t features, bf_stream_t stream) {
+    if (features == 0) return BF_OK;
+    BF_REQUIRE(dBias && (g || rows == 0), "NULL pointer");
+    return launchColumnSum<0, 0>(g, nullptr, nullptr, nullptr, dBias, rows, features, asStream(stream));
+}
+
+int bf_hip_add_bias_act_backward(const float* gemm, const float* bias, const float* dHidden, float* dGemm,
+                                 float* dBias, size_t rows, size_t features, int act, bf_stream_t stream) {
+    BF_REQUIRE(act == BF_ACT_SILU || act == BF_ACT_GELU || act == BF_ACT_RELU, "unknown activation " + std::to_string(act));
+    if (features == 0) return BF_OK;
+    BF_REQUIRE((gemm && dHidden && dGemm) || rows == 0, "NULL pointer");
+    BF_REQUIRE(bias != nullptr, "NULL bias");
+    hipStream_t s = asStream(stream);
+    if (act == BF_ACT_SILU) return launchColumnSum<1, BF_ACT_SILU>(gemm, bias, dHidden, dGemm, dBias, rows, features, s);
+    if (act == BF_ACT_GELU) return launchColumnSum<1, BF_ACT_GELU>(gemm, bias, dHidden, dGemm, dBias, rows, features, s);
+    return launchColumnSum<1, BF_ACT_RELU>(gemm, bias, dHidden, dGemm, dBias, rows, features, s);
+}
+
+int bf_hip_zero_multi(float* const* ptrs, const size_t* counts, size_t numTensors, bf_stream_t stream) {
+    if (numTensors == 0) return BF_OK;
+    BF_REQUIRE(ptrs && counts, "NULL pointer");
+    constexpr size_t kChunk = size_t(kBlock) * 32;  // 8192 floats = 32 KiB per block
+    std::vector<ZeroChunk> chunks;
+    for (size_t t = 0; t < numTensors; ++t) {
+        BF_REQUIRE(ptrs[t] != nullptr || counts[t] == 0, "NULL tensor pointer");
+        for (size_t off = 0; off < counts[t]; off += kChunk) {
+            size_t c = counts[t] - off < kChunk ? counts[t] - off : kChunk;
+            chunks.push_back(ZeroChunk{ptrs[t] + off, unsigned(c)});
+        }
+    }
+    if (chunks.empty()) return BF_OK;
+    const void* table = nullptr;
+    int status = uploadDescriptorTable(kSlotZero, chunks.data(), chunks.size() * sizeof(ZeroChunk), asStream(stream), &table);
+    if (status != BF_OK) return status;
+    zeroMultiKernel<<<unsigned(chunks.size()), kBlock, 0, asStream(stream)>>>(static_cast<const ZeroChunk*>(table));
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,266 @@
+// Row-wise ops: rmsnorm, softmax and their backward passes.
+//
+// HBM-bound: 8 algorithmic bytes per element forward, 12 backward.  Each row is read once into
+// registers (see rowcache.hpp), reduced with wavefront shuffles (rows up to 1024 features: one
+// 64-lane wavefront per row, four rows per block) or one LDS exchange per reduction (longer rows),
+// and written once.
+#include "rowcache.hpp"
+
+namespace bf {
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr float kRmsNormEps = 1e-6f;
+
+// Visits the row either from the register cache or (CACHED == false) from global memory.
+template <int G, int MAXE, int VEC, bool CACHED>
+struct Row {
+    RowCache<G, MAXE, VEC> c;
+    const float* p;
+    size_t n;
+    int t;
+    __device__ void open(const float* row, size_t features, int thread, float fill) {
+        p = row; n = features; t = thread;
+        if constexpr (CACHED) c.load(row, features, thread, fill);
+    }
+    // f(value) over every element including padding (padding holds `fill`): for reductions
+    template <typename F> __device__ void reduce(F&& f) const {
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int i = 0; i < MAXE; ++i) f(c.r[i]);
+        } else {
+            for (size_t e = t; e < n; e += G) f(p[e]);
+        }
+    }
+    // f(value, element index) over valid elements only
+    template <typename F> __device__ void each(F&& f) const {
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int it = 0; it < MAXE / VEC; ++it)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    size_t e = RowCache<G, MAXE, VEC>::index(it, t, j);
+                    if (e < n) f(c.r[it * VEC + j], e);
+                }
+        } else {
+            for (size_t e = t; e < n; e += G) f(p[e], e);
+        }
+    }
+    // out[e] = f(value, e), vectorised when cached
+    template <typename F> __device__ void map(float* __restrict__ out, F&& f) {
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int it = 0; it < MAXE / VEC; ++it)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    size_t e = RowCache<G, MAXE, VEC>::index(it, t, j);
+                    c.r[it * VEC + j] = f(c.r[it * VEC + j], e);
+                }
+            c.store(out, n, t);
+        } else {
+            for (size_t e = t; e < n; e += G) out[e] = f(p[e], e);
+        }
+    }
+};
+
+#define BF_ROW_PROLOGUE()                                                            \
+    __shared__ float lds[16];                                                        \
+    __shared__ double ldsD[16];                                                      \
+    (void)lds; (void)ldsD;                                                           \
+    const int t = threadIdx.x % G;                                                   \
+    const size_t rowsPerBlock = blockDim.x / G;                                      \
+    const size_t rowStep = size_t(gridDim.x) * rowsPerBlock;                         \
+    const size_t firstRow = size_t(blockIdx.x) * rowsPerBlock + threadIdx.x / G;
+
+// When a whole block shares a row (G > 64) every thread must take part in the LDS reductions, so
+// the row loop is uniform across the block: rowsPerBlock == 1 there.
+
+template <int G, int MAXE, int VEC, bool CACHED>
+__global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormKernel(const float* __restrict__ x, float* __restrict__ out,
+                                                                    size_t rows, size_t features) {
+    BF_ROW_PROLOGUE();
+    for (size_t row = firstRow; row < rows; row += rowStep) {
+        Row<G, MAXE, VEC, CACHED> rx;
+        rx.open(x + row * features, features, t, 0.0f);
+        float ss = 0.0f;
+        rx.reduce([&](float v) { ss += v * v; });
+        ss = groupSum<G>(ss, lds);
+        float inv = 1.0f / sqrtf(ss / float(features) + kRmsNormEps);
+        rx.map(out + row * features, [&](float v, size_t) { return v * inv; });
+    }
+}
+
+template <int G, int MAXE, int VEC, bool CACHED>
+__global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const float* __restrict__ x, const float* __restrict__ g,
+                                                                            float* __restrict__ out, size_t rows, size_t features) {
+    BF_ROW_PROLOGUE();
+    for (size_t row = firstRow; row < rows; row += rowStep) {
+        Row<G, MAXE, VEC, CACHED> rx, rg;
+        rx.open(x + row * features, features, t, 0.0f);
+        rg.open(g + row * features, features, t, 0.0f);
+        float ss = 0.0f, gx = 0.0f;
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int i = 0; i < MAXE; ++i) { ss += rx.c.r[i] * rx.c.r[i]; gx += rg.c.r[i] * rx.c.r[i]; }
+        } else {
+            for (size_t e = t; e < features; e += G) { float xv = rx.p[e]; ss += xv * xv; gx += rg.p[e] * xv; }
+        }
+        ss = groupSum<G>(ss, lds);
+        gx = groupSum<G>(gx, lds);
+        float r = sqrtf(ss / float(features) + kRmsNormEps);
+        float invR = 1.0f / r;
+        float k = gx / (float(features) * r * r * r);
+        float* o = out + row * features;
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int i = 0; i < MAXE; ++i) rg.c.r[i] = rg.c.r[i] * invR - rx.c.r[i] * k;
+            rg.c.store(o, features, t);
+        } else {
+            for (size_t e = t; e < features; e += G) o[e] = rg.p[e] * invR - rx.p[e] * k;
+        }
+    }
+}
+
+template <int G, int MAXE, int VEC, bool CACHED>
+__global__ void __launch_bounds__(G > 256 ? G : 256) softmaxKernel(const float* __restrict__ x, float* __restrict__ out,
+                                                                    size_t rows, size_t features) {
+    BF_ROW_PROLOGUE();
+    for (size_t row = firstRow; row < rows; row += rowStep) {
+        Row<G, MAXE, VEC, CACHED> rx;
+        rx.open(x + row * features, features, t, -INFINITY);
+        float mx = -INFINITY;
+        rx.reduce([&](float v) { mx = fmaxf(mx, v); });
+        mx = groupMax<G>(mx, lds);
+        float sum = 0.0f;
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int i = 0; i < MAXE; ++i) { rx.c.r[i] = expf(rx.c.r[i] - mx); sum += rx.c.r[i]; }
+        } else {
+            for (size_t e = t; e < features; e += G) sum += expf(rx.p[e] - mx);
+        }
+        sum = groupSum<G>(sum, lds);
+        float inv = 1.0f / sum;
+        float* o = out + row * features;
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int i = 0; i < MAXE; ++i) rx.c.r[i] *= inv;
+            rx.c.store(o, features, t);
+        } else {
+            for (size_t e = t; e < features; e += G) o[e] = expf(rx.p[e] - mx) * inv;
+        }
+    }
+}
+
+// dx = y * (g - sum(g*y)) with y = softmax(x) recomputed in registers.
+template <int G, int MAXE, int VEC, bool CACHED>
+__global__ void __launch_bounds__(G > 256 ? G : 256) softmaxBackwardKernel(const float* __restrict__ x, const float* __restrict__ g,
+                                                                            float* __restrict__ out, size_t rows, size_t features) {
+    BF_ROW_PROLOGUE();
+    for (size_t row = firstRow; row < rows; row += rowStep) {
+        Row<G, MAXE, VEC, CACHED> rx, rg;
+        rx.open(x + row * features, features, t, -INFINITY);
+        rg.open(g + row * features, features, t, 0.0f);
+        float mx = -INFINITY;
+        rx.reduce([&](float v) { mx = fmaxf(mx, v); });
+        mx = groupMax<G>(mx, lds);
+        float sum = 0.0f, gy = 0.0f;
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int i = 0; i < MAXE; ++i) { rx.c.r[i] = expf(rx.c.r[i] - mx); sum += rx.c.r[i]; gy += rg.c.r[i] * rx.c.r[i]; }
+        } else {
+            for (size_t e = t; e < features; e += G) { float ev = expf(rx.p[e] - mx); sum += ev; gy += rg.p[e] * ev; }
+        }
+        sum = groupSum<G>(sum, lds);
+        gy = groupSum<G>(gy, lds);
+        float inv = 1.0f / sum;
+        float dot = gy * inv;  // sum_j g_j y_j
+        float* o = out + row * features;
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int i = 0; i < MAXE; ++i) rg.c.r[i] = rx.c.r[i] * inv * (rg.c.r[i] - dot);
+            rg.c.store(o, features, t);
+        } else {
+            for (size_t e = t; e < features; e += G) o[e] = expf(rx.p[e] - mx) * inv * (rg.p[e] - dot);
+        }
+    }
+}
+
+// Picks the instantiation for a row length.  ONE_INPUT kernels keep up to 16/32/64 elements per
+// thread, two-input kernels half of that for the 1024-thread group (register budget of 16 waves/CU).
+#define BF_ROW_LAUNCH(KERNEL, TWO_INPUTS, vecOk, rows, features, stream, ...)                                      \
+    do {                                                                                                           \
+        const bool vec4 = (vecOk) && (features) % 4 == 0;                                                          \
+        const int big = (TWO_INPUTS) ? 32 : 64;                                                                    \
+        const unsigned cap = unsigned(computeUnits()) * 8;                                                         \
+        if ((features) <= 64 * 16) {                                                                               \
+            unsigned grid = gridFor(rows, 4, cap);                                                                 \
+            if (vec4) KERNEL<64, 16, 4, true><<<grid, 256, 0, stream>>>(__VA_ARGS__);                              \
+            else KERNEL<64, 16, 1, true><<<grid, 256, 0, stream>>>(__VA_ARGS__);                                   \
+        } else if ((features) <= 256 * 32) {                                                                       \
+            unsigned grid = gridFor(rows, 1, cap);                                                                 \
+            if (vec4) KERNEL<256, 32, 4, true><<<grid, 256, 0, stream>>>(__VA_ARGS__);                             \
+            else KERNEL<256, 32, 1, true><<<grid, 256, 0, stream>>>(__VA_ARGS__);                                  \
+        } else if ((features) <= size_t(1024) * big) {                                                             \
+            unsigned grid = gridFor(rows, 1, cap);                                                                 \
+            if (TWO_INPUTS) {                                                                                      \
+                if (vec4) KERNEL<1024, 32, 4, true><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                       \
+                else KERNEL<1024, 32, 1, true><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                            \
+            } else {                                                                                               \
+                if (vec4) KERNEL<1024, 64, 4, true><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                       \
+                else KERNEL<1024, 64, 1, true><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                            \
+            }                                                                                                      \
+        } else {                                                                                                   \
+            unsigned grid = gridFor(rows, 1, cap);                                                                 \
+            KERNEL<1024, 4, 1, false><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                                     \
+        }                                                                                                          \
+    } while (0)
+
+}  // namespace
+}  // namespace bf
+
+using namespace bf;
+
+extern "C" {
+
+int bf_hip_rmsnorm(const float* x, float* out, size_t rows, size_t features, bf_stream_t stream) {
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && out, "NULL pointer");
+    hipStream_t s = asStream(stream);
+    BF_ROW_LAUNCH(rmsnormKernel, false, aligned16(x) && aligned16(out), rows, features, s, x, out, rows, features);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_rmsnorm_backward(const float* x, const float* g, float* out, size_t rows, size_t features,
+                            bf_stream_t stream) {
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && g && out, "NULL pointer");
+    hipStream_t s = asStream(stream);
+    BF_ROW_LAUNCH(rmsnormBackwardKernel, true, aligned16(x) && aligned16(g) && aligned16(out), rows, features, s, x, g,
+                  out, rows, features);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_softmax(const float* x, float* out, size_t rows, size_t features, bf_stream_t stream) {
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && out, "NULL pointer");
+    hipStream_t s = asStream(stream);
+    BF_ROW_LAUNCH(softmaxKernel, false, aligned16(x) && aligned16(out), rows, features, s, x, out, rows, features);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_softmax_backward(const float* x, const float* g, float* out, size_t rows, size_t features,
+                            bf_stream_t stream) {
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && g && out, "NULL pointer");
+    hipStream_t s = asStream(stream);
+    BF_ROW_LAUNCH(softmaxBackwardKernel, true, aligned16(x) && aligned16(g) && aligned16(out), rows, features, s, x, g,
+                  out, rows, features);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+}  // extern "C"

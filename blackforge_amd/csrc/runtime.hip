@@ -1,0 +1,308 @@
+// Devices, streams, events and the per-device memory pool.
+//
+// The pool replaces the reference's exact-byte-size free lists (device_pool.cu:29-65) with size
+// classes: requests are rounded up to a class (four classes per power of two, 512 B minimum, 2 MiB
+// granularity above 64 MiB) so that tensors of nearby sizes share blocks and a 288 GB card is not
+// fragmented by one free list per distinct shape.  As in the reference, released blocks stay cached
+// for the life of the process unless bf_hip_pool_trim() is called.
+#include "common.hpp"
+
+#include <algorithm>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+namespace bf {
+
+namespace {
+thread_local std::string g_lastError;
+}
+
+void setLastError(const std::string& message) { g_lastError = message; }
+
+int failInvalid(const char* function, const std::string& message) {
+    g_lastError = std::string(function) + ": " + message;
+    return BF_ERR_INVALID_ARGUMENT;
+}
+
+int failRuntime(const char* function, hipError_t error, const char* file, int line) {
+    g_lastError = std::string(file) + ":" + std::to_string(line) + ": " + function + ": HIP error: " +
+                  hipGetErrorString(error);
+    return BF_ERR_RUNTIME;
+}
+
+int computeUnits() {
+    static std::unordered_map<int, int> cache;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    auto it = cache.find(dev);
+    if (it != cache.end()) return it->second;
+    int cus = 256;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 256;
+    cache[dev] = cus;
+    return cus;
+}
+
+namespace {
+struct DescriptorTable {
+    std::vector<unsigned char> host;
+    void* device = nullptr;
+    size_t capacity = 0;
+};
+std::map<std::pair<int, int>, DescriptorTable>& descriptorTables() {
+    static std::map<std::pair<int, int>, DescriptorTable> tables;
+    return tables;
+}
+}  // namespace
+
+int uploadDescriptorTable(int slot, const void* hostBytes, size_t bytes, hipStream_t stream, const void** devicePtr) {
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    DescriptorTable& t = descriptorTables()[{dev, slot}];
+    const auto* src = static_cast<const unsigned char*>(hostBytes);
+    bool same = t.device != nullptr && t.host.size() == bytes && std::equal(src, src + bytes, t.host.begin());
+    if (!same) {
+        // kernels still reading the old table must finish before it is overwritten or freed
+        BF_HIP_TRY(hipStreamSynchronize(stream));
+        if (bytes > t.capacity) {
+            if (t.device) BF_HIP_TRY(hipFree(t.device));
+            t.device = nullptr;
+            size_t cap = bytes < 4096 ? 4096 : bytes * 2;
+            BF_HIP_TRY(hipMalloc(&t.device, cap));
+            t.capacity = cap;
+        }
+        BF_HIP_TRY(hipMemcpy(t.device, hostBytes, bytes, hipMemcpyHostToDevice));
+        t.host.assign(src, src + bytes);
+    }
+    *devicePtr = t.device;
+    return BF_OK;
+}
+
+namespace {
+
+size_t sizeClass(size_t bytes) {
+    constexpr size_t kMin = 512;
+    constexpr size_t kLarge = size_t(64) << 20;
+    constexpr size_t kLargeStep = size_t(2) << 20;
+    if (bytes <= kMin) return kMin;
+    if (bytes > kLarge) return (bytes + kLargeStep - 1) / kLargeStep * kLargeStep;
+    size_t pow2 = kMin;
+    while (pow2 < bytes) pow2 <<= 1;   // smallest power of two >= bytes
+    size_t quarter = pow2 >> 3;        // classes at 5/8, 6/8, 7/8, 8/8 of pow2
+    for (size_t c = (pow2 >> 1) + quarter; c < pow2; c += quarter)
+        if (bytes <= c) return c;
+    return pow2;
+}
+
+struct DevicePool {
+    std::unordered_map<size_t, std::vector<void*>> freeLists;
+    bf_pool_stats stats{};
+};
+
+std::unordered_map<int, DevicePool>& pools() {
+    static std::unordered_map<int, DevicePool> registry;
+    return registry;
+}
+
+__global__ void fillZeroKernel(uint32_t* dst, size_t words) {
+    size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < words; i += stride) dst[i] = 0u;
+}
+__global__ void fillZeroBytesKernel(unsigned char* dst, size_t bytes) {
+    size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < bytes) dst[i] = 0;
+}
+
+}  // namespace
+}  // namespace bf
+
+using namespace bf;
+
+extern "C" {
+
+const char* bf_hip_last_error(void) { return g_lastError.c_str(); }
+const char* bf_hip_version(void) { return "blackforge-hip 0.1 (gfx950)"; }
+
+int bf_hip_device_count(int* count) {
+    BF_REQUIRE(count != nullptr, "count is NULL");
+    int n = 0;
+    hipError_t err = hipGetDeviceCount(&n);
+    if (err != hipSuccess) {  // no driver / no device: the reference returns an empty list
+        (void)hipGetLastError();
+        n = 0;
+    }
+    *count = n;
+    return BF_OK;
+}
+
+int bf_hip_device_props(int index, bf_device_props* props) {
+    BF_REQUIRE(props != nullptr, "props is NULL");
+    hipDeviceProp_t p;
+    BF_HIP_TRY(hipGetDeviceProperties(&p, index));
+    snprintf(props->name, sizeof(props->name), "%s", p.name);
+    snprintf(props->arch, sizeof(props->arch), "%s", p.gcnArchName);
+    props->compute_units = p.multiProcessorCount;
+    props->clock_khz = p.clockRate;
+    props->wavefront_size = p.warpSize;
+    props->lds_bytes_per_block = static_cast<int>(p.sharedMemPerBlock);
+    props->total_memory = p.totalGlobalMem;
+    return BF_OK;
+}
+
+int bf_hip_set_device(int index) {
+    int n = 0;
+    bf_hip_device_count(&n);
+    BF_REQUIRE(index >= 0 && index < n, "device index " + std::to_string(index) + " out of range (" +
+                                            std::to_string(n) + " devices)");
+    BF_HIP_TRY(hipSetDevice(index));
+    return BF_OK;
+}
+
+int bf_hip_get_device(int* index) {
+    BF_REQUIRE(index != nullptr, "index is NULL");
+    BF_HIP_TRY(hipGetDevice(index));
+    return BF_OK;
+}
+
+int bf_hip_synchronize(void) {
+    BF_HIP_TRY(hipDeviceSynchronize());
+    return BF_OK;
+}
+
+int bf_hip_stream_create(bf_stream_t* stream) {
+    BF_REQUIRE(stream != nullptr, "stream is NULL");
+    hipStream_t s;
+    // blocking with respect to the default stream, so the synchronous copies of fromHost/toHost stay
+    // ordered with work enqueued on this stream
+    BF_HIP_TRY(hipStreamCreate(&s));
+    *stream = s;
+    return BF_OK;
+}
+int bf_hip_stream_destroy(bf_stream_t stream) {
+    if (stream) BF_HIP_TRY(hipStreamDestroy(asStream(stream)));
+    return BF_OK;
+}
+int bf_hip_stream_synchronize(bf_stream_t stream) {
+    BF_HIP_TRY(hipStreamSynchronize(asStream(stream)));
+    return BF_OK;
+}
+int bf_hip_event_create(bf_event_t* event) {
+    BF_REQUIRE(event != nullptr, "event is NULL");
+    hipEvent_t e;
+    BF_HIP_TRY(hipEventCreate(&e));
+    *event = e;
+    return BF_OK;
+}
+int bf_hip_event_destroy(bf_event_t event) {
+    if (event) BF_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return BF_OK;
+}
+int bf_hip_event_record(bf_event_t event, bf_stream_t stream) {
+    BF_HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(event), asStream(stream)));
+    return BF_OK;
+}
+int bf_hip_event_synchronize(bf_event_t event) {
+    BF_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+    return BF_OK;
+}
+int bf_hip_event_elapsed_ms(bf_event_t start, bf_event_t stop, float* ms) {
+    BF_REQUIRE(ms != nullptr, "ms is NULL");
+    BF_HIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+    return BF_OK;
+}
+
+int bf_hip_pool_acquire(size_t bytes, void** ptr) {
+    BF_REQUIRE(ptr != nullptr, "ptr is NULL");
+    *ptr = nullptr;
+    if (bytes == 0) return BF_OK;
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    DevicePool& pool = pools()[dev];
+    size_t cls = sizeClass(bytes);
+    std::vector<void*>& list = pool.freeLists[cls];
+    if (!list.empty()) {
+        *ptr = list.back();
+        list.pop_back();
+    } else {
+        BF_HIP_TRY(hipMalloc(ptr, cls));
+        pool.stats.bytes_from_driver += cls;
+        pool.stats.driver_allocations += 1;
+    }
+    pool.stats.bytes_in_use += cls;
+    pool.stats.acquires += 1;
+    return BF_OK;
+}
+
+int bf_hip_pool_release(void* ptr, size_t bytes) {
+    if (ptr == nullptr) return BF_OK;
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    DevicePool& pool = pools()[dev];
+    size_t cls = sizeClass(bytes);
+    pool.freeLists[cls].push_back(ptr);
+    pool.stats.bytes_in_use -= cls < pool.stats.bytes_in_use ? cls : pool.stats.bytes_in_use;
+    return BF_OK;
+}
+
+int bf_hip_pool_stats(bf_pool_stats* stats) {
+    BF_REQUIRE(stats != nullptr, "stats is NULL");
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    *stats = pools()[dev].stats;
+    return BF_OK;
+}
+
+int bf_hip_pool_trim(void) {
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    BF_HIP_TRY(hipDeviceSynchronize());
+    DevicePool& pool = pools()[dev];
+    for (auto& entry : pool.freeLists) {
+        for (void* p : entry.second) {
+            BF_HIP_TRY(hipFree(p));
+            pool.stats.bytes_from_driver -= entry.first;
+        }
+        entry.second.clear();
+    }
+    return BF_OK;
+}
+
+int bf_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    if (bytes == 0) return BF_OK;
+    BF_REQUIRE(dst && src, "NULL pointer");
+    BF_HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return BF_OK;
+}
+int bf_hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    if (bytes == 0) return BF_OK;
+    BF_REQUIRE(dst && src, "NULL pointer");
+    BF_HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return BF_OK;
+}
+int bf_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, bf_stream_t stream) {
+    if (bytes == 0) return BF_OK;
+    BF_REQUIRE(dst && src, "NULL pointer");
+    BF_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, asStream(stream)));
+    return BF_OK;
+}
+
+int bf_hip_fill_zero(void* dst, size_t bytes, bf_stream_t stream) {
+    if (bytes == 0) return BF_OK;
+    BF_REQUIRE(dst != nullptr, "NULL pointer");
+    BF_REQUIRE((reinterpret_cast<uintptr_t>(dst) & 3u) == 0, "dst must be 4-byte aligned");
+    size_t words = bytes / 4;
+    if (words) {
+        unsigned grid = gridFor(words, size_t(kBlock) * 8, unsigned(computeUnits()) * 8);
+        fillZeroKernel<<<grid, kBlock, 0, asStream(stream)>>>(static_cast<uint32_t*>(dst), words);
+        BF_LAUNCH_CHECK();
+    }
+    size_t tail = bytes - words * 4;
+    if (tail) {
+        fillZeroBytesKernel<<<1, 64, 0, asStream(stream)>>>(static_cast<unsigned char*>(dst) + words * 4, tail);
+        BF_LAUNCH_CHECK();
+    }
+    return BF_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,693 @@
+"""Python mirror of the reference GPU operator interface, on top of the C ABI.
+
+Function names, argument order and error behaviour follow the free functions of
+``blackforge::backend::cuda`` (reference ``include/blackforge/backend/cuda/{ops,autodiff,
+fused_attention,loss,optimizer}.hpp``): ops take ``DeviceTensor`` and return fresh ``DeviceTensor``
+objects, shape errors raise ``ValueError`` (std::invalid_argument in the reference) before anything is
+launched.  Every computation is done by ``libbf_hip.so``; this file only validates shapes, allocates
+results from the pool and sequences the composite blocks.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+from . import capi
+from .capi import ACT_GELU, ACT_RELU, ACT_SILU
+from .tensor import DeviceTensor
+
+_call = capi.call
+
+
+def _rows(t: DeviceTensor):
+    features = t.shape[-1]
+    return (t.elementCount() // features if features else 0), features
+
+
+def _require(cond: bool, message: str):
+    if not cond:
+        raise ValueError(message)
+
+
+# ------------------------------------------------------------------------------------------------
+# elementwise (ops.hpp:8-30, 82-84)
+# ------------------------------------------------------------------------------------------------
+def add(a: DeviceTensor, b: DeviceTensor) -> DeviceTensor:
+    _require(a.shape == b.shape, f"add: incompatible shapes {a.shape} and {b.shape}")
+    out = DeviceTensor(a.shape)
+    _call("bf_hip_add", a.ptr, b.ptr, out.ptr, a.elementCount(), None)
+    return out
+
+
+def scale(x: DeviceTensor, factor: float) -> DeviceTensor:
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_scale", x.ptr, factor, out.ptr, x.elementCount(), None)
+    return out
+
+
+def _check_bias(name, x, bias):
+    _require(x.rank() >= 2 and bias.rank() == 1 and x.shape[-1] == bias.shape[0],
+             f"{name}: expected input [..., features] and bias [features], got {x.shape} and {bias.shape}")
+
+
+def addBias(x: DeviceTensor, bias: DeviceTensor) -> DeviceTensor:
+    _check_bias("addBias", x, bias)
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_add_bias", x.ptr, bias.ptr, out.ptr, *_rows(x), None)
+    return out
+
+
+def addBiasAct(gemm: DeviceTensor, bias: DeviceTensor, act: int) -> DeviceTensor:
+    _check_bias("addBiasAct", gemm, bias)
+    out = DeviceTensor(gemm.shape)
+    _call("bf_hip_add_bias_act", gemm.ptr, bias.ptr, out.ptr, *_rows(gemm), act, None)
+    return out
+
+
+def addBiasSilu(gemm: DeviceTensor, bias: DeviceTensor) -> DeviceTensor:
+    return addBiasAct(gemm, bias, ACT_SILU)
+
+
+def addBiasResidual(gemm: DeviceTensor, bias: DeviceTensor, residual: DeviceTensor) -> DeviceTensor:
+    _check_bias("addBiasResidual", gemm, bias)
+    _require(gemm.shape == residual.shape, "addBiasResidual: residual shape differs")
+    out = DeviceTensor(gemm.shape)
+    _call("bf_hip_add_bias_residual", gemm.ptr, bias.ptr, residual.ptr, out.ptr, *_rows(gemm), None)
+    return out
+
+
+def _act(x, act):
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_act_forward", x.ptr, out.ptr, x.elementCount(), act, None)
+    return out
+
+
+def silu(x): return _act(x, ACT_SILU)
+def relu(x): return _act(x, ACT_RELU)
+def gelu(x): return _act(x, ACT_GELU)
+
+
+def _act_bwd(name, x, g, act):
+    _require(x.shape == g.shape, f"{name}: incompatible shapes")
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_act_backward", x.ptr, g.ptr, out.ptr, x.elementCount(), act, None)
+    return out
+
+
+def siluBackward(x, g): return _act_bwd("siluBackward", x, g, ACT_SILU)
+def reluBackward(x, g): return _act_bwd("reluBackward", x, g, ACT_RELU)
+def geluBackward(x, g): return _act_bwd("geluBackward", x, g, ACT_GELU)
+
+
+def accumulate(target: DeviceTensor, delta: DeviceTensor) -> None:
+    _call("bf_hip_accumulate", target.ptr, delta.ptr, target.elementCount(), None)
+
+
+def zeroFused(tensors: List[DeviceTensor]) -> None:
+    n = len(tensors)
+    if n == 0:
+        return
+    ptrs = (ctypes.c_void_p * n)(*[t.ptr.value if t.ptr else None for t in tensors])
+    counts = (ctypes.c_size_t * n)(*[t.elementCount() for t in tensors])
+    _call("bf_hip_zero_multi", ptrs, counts, n, None)
+
+
+# ------------------------------------------------------------------------------------------------
+# rows (ops.hpp:92-98, autodiff.hpp:52-84)
+# ------------------------------------------------------------------------------------------------
+def rmsnorm(x: DeviceTensor) -> DeviceTensor:
+    _require(x.rank() >= 2, "rmsnorm: needs a tensor of rank >= 2")
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_rmsnorm", x.ptr, out.ptr, *_rows(x), None)
+    return out
+
+
+def rmsnormBackward(x: DeviceTensor, g: DeviceTensor) -> DeviceTensor:
+    _require(x.shape == g.shape, "rmsnormBackward: incompatible shapes")
+    _require(x.rank() >= 2, "rmsnormBackward: needs a tensor of rank >= 2")
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_rmsnorm_backward", x.ptr, g.ptr, out.ptr, *_rows(x), None)
+    return out
+
+
+def softmax(x: DeviceTensor) -> DeviceTensor:
+    _require(x.rank() >= 2, "softmax: needs a tensor of rank >= 2")
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_softmax", x.ptr, out.ptr, *_rows(x), None)
+    return out
+
+
+def softmaxBackward(x: DeviceTensor, g: DeviceTensor) -> DeviceTensor:
+    _require(x.shape == g.shape, "softmaxBackward: incompatible shapes")
+    _require(x.rank() >= 2, "softmaxBackward: needs a tensor of rank >= 2")
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_softmax_backward", x.ptr, g.ptr, out.ptr, *_rows(x), None)
+    return out
+
+
+def biasGradientOnly(g: DeviceTensor) -> DeviceTensor:
+    _require(g.rank() >= 2, "biasGradientOnly: needs a gradient of rank >= 2")
+    out = DeviceTensor((g.shape[-1],))
+    _call("bf_hip_bias_grad", g.ptr, out.ptr, *_rows(g), None)
+    return out
+
+
+def addBiasBackward(g: DeviceTensor):
+    """Returns (dInput, dBias); dInput is a copy of g, as in the reference."""
+    _require(g.rank() >= 2, "addBiasBackward: needs a gradient of rank >= 2")
+    return g.clone(), biasGradientOnly(g)
+
+
+def addBiasActBackward(gemm: DeviceTensor, bias: DeviceTensor, dHidden: DeviceTensor, act: int):
+    _require(gemm.shape == dHidden.shape and bias.rank() == 1 and gemm.shape[-1] == bias.shape[0],
+             "addBiasSiluBackward: incompatible shapes")
+    dGemm = DeviceTensor(gemm.shape)
+    dBias = DeviceTensor(bias.shape)
+    _call("bf_hip_add_bias_act_backward", gemm.ptr, bias.ptr, dHidden.ptr, dGemm.ptr, dBias.ptr, *_rows(gemm), act,
+          None)
+    return dGemm, dBias
+
+
+def addBiasSiluBackward(gemm, bias, dHidden):
+    return addBiasActBackward(gemm, bias, dHidden, ACT_SILU)
+
+
+# ------------------------------------------------------------------------------------------------
+# gather / scatter (ops.hpp:104-122, autodiff.hpp:90-106)
+# ------------------------------------------------------------------------------------------------
+def _validate_ids(name: str, ids: DeviceTensor, limit: int, what: str):
+    bad, first = ctypes.c_size_t(), ctypes.c_longlong()
+    _call("bf_hip_count_out_of_range", ids.ptr, ids.elementCount(), limit, ctypes.byref(bad), ctypes.byref(first), None)
+    _require(bad.value == 0, f"{name}: {what} {first.value} outside [0, {limit})")
+
+
+def embeddingLookupPreValidated(ids: DeviceTensor, table: DeviceTensor) -> DeviceTensor:
+    _require(ids.rank() == 2, "embeddingLookup: token ids must have rank 2 [batch, seq]")
+    _require(table.rank() == 2, "embeddingLookup: table must have rank 2 [vocabSize, dim]")
+    out = DeviceTensor(ids.shape + (table.shape[1],))
+    _call("bf_hip_embedding_forward", ids.ptr, table.ptr, out.ptr, ids.elementCount(), table.shape[0], table.shape[1],
+          None)
+    return out
+
+
+def embeddingLookup(ids: DeviceTensor, table: DeviceTensor) -> DeviceTensor:
+    _require(ids.rank() == 2, "embeddingLookup: token ids must have rank 2 [batch, seq]")
+    _require(table.rank() == 2, "embeddingLookup: table must have rank 2 [vocabSize, dim]")
+    _validate_ids("embeddingLookup", ids, table.shape[0], "token id")
+    return embeddingLookupPreValidated(ids, table)
+
+
+def embeddingLookupBackwardPreValidated(ids: DeviceTensor, g: DeviceTensor, vocabSize: int) -> DeviceTensor:
+    _require(ids.rank() == 2 and g.rank() == 3 and ids.shape == g.shape[:2],
+             "embeddingLookupBackward: incompatible shapes")
+    out = DeviceTensor((vocabSize, g.shape[2]))
+    _call("bf_hip_embedding_backward", ids.ptr, g.ptr, out.ptr, ids.elementCount(), vocabSize, g.shape[2], None)
+    return out
+
+
+def embeddingLookupBackward(ids: DeviceTensor, g: DeviceTensor, vocabSize: int) -> DeviceTensor:
+    _require(ids.rank() == 2 and g.rank() == 3 and ids.shape == g.shape[:2],
+             "embeddingLookupBackward: incompatible shapes")
+    _validate_ids("embeddingLookupBackward", ids, vocabSize, "token id")
+    return embeddingLookupBackwardPreValidated(ids, g, vocabSize)
+
+
+def addPositionalEmbeddingAt(x: DeviceTensor, table: DeviceTensor, offset: int) -> DeviceTensor:
+    _require(x.rank() == 3, "addPositionalEmbedding: needs an input of rank 3 [batch, seq, dim]")
+    _require(table.rank() == 2 and table.shape[1] == x.shape[2], "addPositionalEmbedding: table [maxSeqLen, dim] mismatch")
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_positional_forward", x.ptr, table.ptr, out.ptr, x.shape[0], x.shape[1], x.shape[2], table.shape[0],
+          offset, None)
+    return out
+
+
+def addPositionalEmbedding(x, table):
+    return addPositionalEmbeddingAt(x, table, 0)
+
+
+def addPositionalEmbeddingBackward(g: DeviceTensor, maxSeqLen: int):
+    """Returns (dInput, dTable)."""
+    _require(g.rank() == 3, "addPositionalEmbeddingBackward: needs a gradient of rank 3")
+    dTable = DeviceTensor((maxSeqLen, g.shape[2]))
+    _call("bf_hip_positional_backward", g.ptr, dTable.ptr, g.shape[0], g.shape[1], g.shape[2], maxSeqLen, None)
+    return g.clone(), dTable
+
+
+def concatSeq(a: DeviceTensor, b: DeviceTensor) -> DeviceTensor:
+    out = DeviceTensor((a.shape[0], a.shape[1] + b.shape[1], a.shape[2]))
+    _call("bf_hip_concat_seq", a.ptr, b.ptr, out.ptr, a.shape[0], a.shape[1], b.shape[1], a.shape[2], None)
+    return out
+
+
+def argmaxLastPosition(logits: DeviceTensor) -> int:
+    """Greedy next-token choice over [1, seq, vocab] (or [seq, vocab]) logits, computed on the device."""
+    seq, vocab = logits.shape[-2], logits.shape[-1]
+    idx = ctypes.c_longlong()
+    _call("bf_hip_argmax_last_position", logits.ptr, seq, vocab, ctypes.byref(idx), None)
+    return idx.value
+
+
+# ------------------------------------------------------------------------------------------------
+# GEMM (ops.hpp:35-80,247-258; autodiff.hpp:23-44)
+# ------------------------------------------------------------------------------------------------
+def _gemm(ta, tb, a, b, m, n, k):
+    out = DeviceTensor((m, n))
+    _call("bf_hip_gemm_f32", ta, tb, a.ptr, b.ptr, out.ptr, m, n, k, None)
+    return out
+
+
+def matmul(a: DeviceTensor, b: DeviceTensor) -> DeviceTensor:
+    _require(a.rank() == 2 and b.rank() == 2 and a.shape[1] == b.shape[0], f"matmul: incompatible shapes {a.shape} x {b.shape}")
+    return _gemm(0, 0, a, b, a.shape[0], b.shape[1], a.shape[1])
+
+
+def matmulTransposeB(a: DeviceTensor, b: DeviceTensor) -> DeviceTensor:
+    _require(a.rank() == 2 and b.rank() == 2 and a.shape[1] == b.shape[1], "matmulTransposeB: incompatible shapes")
+    return _gemm(0, 1, a, b, a.shape[0], b.shape[0], a.shape[1])
+
+
+def _check_mm_bwd(name, a, b, g):
+    _require(a.rank() == 2 and b.rank() == 2 and g.rank() == 2 and a.shape[1] == b.shape[0]
+             and g.shape == (a.shape[0], b.shape[1]), f"{name}: incompatible shapes")
+
+
+def matmulBackward(a, b, g):
+    """Returns (dA, dB) of c = a @ b."""
+    _check_mm_bwd("matmulBackward", a, b, g)
+    m, k, n = a.shape[0], a.shape[1], b.shape[1]
+    return _gemm(0, 1, g, b, m, k, n), _gemm(1, 0, a, g, k, n, m)
+
+
+def matmulTransposeBBackward(a, b, g):
+    """Returns (dA, dB) of c = a @ b^T with a:[m,k], b:[n,k]."""
+    _require(a.rank() == 2 and b.rank() == 2 and g.rank() == 2 and a.shape[1] == b.shape[1]
+             and g.shape == (a.shape[0], b.shape[0]), "matmulTransposeBBackward: incompatible shapes")
+    m, k, n = a.shape[0], a.shape[1], b.shape[0]
+    return _gemm(0, 0, g, b, m, k, n), _gemm(1, 0, g, a, n, k, m)
+
+
+def _matmul_bf16(name, a, b, cache):
+    _require(a.rank() == 2 and b.rank() == 2 and a.shape[1] == b.shape[0], f"{name}: incompatible shapes")
+    out = DeviceTensor((a.shape[0], b.shape[1]))
+    _call("bf_hip_matmul_bf16", a.ptr, b.ptr, out.ptr, a.shape[0], a.shape[1], b.shape[1], cache, None)
+    return out
+
+
+def matmulBf16(a, b): return _matmul_bf16("matmulBf16", a, b, 0)
+def matmulBf16CachedWeight(a, b): return _matmul_bf16("matmulBf16CachedWeight", a, b, 1)
+
+
+def invalidateBf16WeightCache() -> None:
+    _call("bf_hip_invalidate_bf16_weight_cache")
+
+
+def _matmul_bf16_bwd(name, a, b, g, cache):
+    _check_mm_bwd(name, a, b, g)
+    dA, dB = DeviceTensor(a.shape), DeviceTensor(b.shape)
+    _call("bf_hip_matmul_bf16_backward", a.ptr, b.ptr, g.ptr, dA.ptr, dB.ptr, a.shape[0], a.shape[1], b.shape[1], cache,
+          None)
+    return dA, dB
+
+
+def matmulBf16Backward(a, b, g): return _matmul_bf16_bwd("matmulBf16Backward", a, b, g, 0)
+def matmulBf16BackwardCachedWeight(a, b, g): return _matmul_bf16_bwd("matmulBf16BackwardCachedWeight", a, b, g, 1)
+
+
+def _flat2d(t: DeviceTensor):
+    """A [rows, features] view descriptor (no copy): a non-owning alias used only inside one op."""
+    v = DeviceTensor.__new__(DeviceTensor)
+    rows, f = _rows(t)
+    v.shape, v.itemsize, v._bytes, v.ptr = (rows, f), t.itemsize, 0, t.ptr  # _bytes = 0: never released
+    return v
+
+
+def _linear(name, x, w, bias, mm):
+    _require(x.rank() >= 2, f"{name}: needs a tensor of rank >= 2")
+    _require(w.rank() == 2 and x.shape[-1] == w.shape[0], f"{name}: incompatible shapes {x.shape} x {w.shape}")
+    _require(bias.rank() == 1 and bias.shape[0] == w.shape[1], f"{name}: bias {bias.shape} does not match {w.shape}")
+    prod = mm(_flat2d(x), w)
+    out = DeviceTensor(x.shape[:-1] + (w.shape[1],))
+    _call("bf_hip_add_bias", prod.ptr, bias.ptr, out.ptr, prod.shape[0], prod.shape[1], None)
+    return out
+
+
+def linear(x, w, bias): return _linear("linear", x, w, bias, matmul)
+def linearBf16(x, w, bias): return _linear("linearBf16", x, w, bias, matmulBf16)
+def linearBf16CachedWeight(x, w, bias): return _linear("linearBf16CachedWeight", x, w, bias, matmulBf16CachedWeight)
+
+
+# ------------------------------------------------------------------------------------------------
+# fused attention (fused_attention.hpp:55,73)
+# ------------------------------------------------------------------------------------------------
+@dataclass
+class FusedAttentionForwardResult:
+    output: DeviceTensor
+    m: DeviceTensor
+    l: DeviceTensor
+
+
+@dataclass
+class FusedAttentionGrad:
+    dQ: DeviceTensor
+    dK: DeviceTensor
+    dV: DeviceTensor
+
+
+def fusedAttentionForward(q, k, v, numHeads: int, scaleFactor: float, oldLen: int) -> FusedAttentionForwardResult:
+    batch, newLen, dim = q.shape
+    totalLen = k.shape[1]
+    out = DeviceTensor((batch, newLen, dim))
+    m = DeviceTensor((batch, numHeads, newLen))
+    l = DeviceTensor((batch, numHeads, newLen))
+    _call("bf_hip_attention_forward", q.ptr, k.ptr, v.ptr, out.ptr, m.ptr, l.ptr, batch, numHeads, newLen, totalLen, dim,
+          scaleFactor, oldLen, None)
+    return FusedAttentionForwardResult(out, m, l)
+
+
+def fusedAttentionBackward(dOutput, q, k, v, output, m, l, numHeads: int, scaleFactor: float, oldLen: int) -> FusedAttentionGrad:
+    batch, newLen, dim = q.shape
+    totalLen = k.shape[1]
+    dQ, dK, dV = DeviceTensor(q.shape), DeviceTensor(k.shape), DeviceTensor(v.shape)
+    _call("bf_hip_attention_backward", dOutput.ptr, q.ptr, k.ptr, v.ptr, output.ptr, m.ptr, l.ptr, dQ.ptr, dK.ptr, dV.ptr,
+          batch, numHeads, newLen, totalLen, dim, scaleFactor, oldLen, None)
+    return FusedAttentionGrad(dQ, dK, dV)
+
+
+# ------------------------------------------------------------------------------------------------
+# composite blocks (ops.hpp:127-245, autodiff.hpp:117-177).  `act` selects the feed-forward
+# activation: ACT_SILU is the reference block, ACT_GELU the same block with gelu substituted.
+# ------------------------------------------------------------------------------------------------
+@dataclass
+class FeedForwardCache:
+    normed: Optional[DeviceTensor] = None
+    gemm1: Optional[DeviceTensor] = None
+    hidden: Optional[DeviceTensor] = None
+
+
+@dataclass
+class SelfAttentionCache:
+    normedFlat: Optional[DeviceTensor] = None
+    q: Optional[DeviceTensor] = None
+    k: Optional[DeviceTensor] = None
+    v: Optional[DeviceTensor] = None
+    attnOutput: Optional[DeviceTensor] = None
+    attnM: Optional[DeviceTensor] = None
+    attnL: Optional[DeviceTensor] = None
+
+
+@dataclass
+class KVCache:
+    k: Optional[DeviceTensor] = None
+    v: Optional[DeviceTensor] = None
+    length: int = 0
+
+
+def _mm(useBf16, cached):
+    if not useBf16:
+        return matmul
+    return matmulBf16CachedWeight if cached else matmulBf16
+
+
+def _mm_bwd(useBf16, cached):
+    if not useBf16:
+        return matmulBackward
+    return matmulBf16BackwardCachedWeight if cached else matmulBf16Backward
+
+
+def feedForwardForwardCached(x, w1, b1, w2, b2, useBf16: bool, cache: FeedForwardCache, act: int = ACT_SILU):
+    cache.normed = rmsnorm(x)
+    mm = _mm(useBf16, True)
+    hiddenShape = x.shape[:-1] + (w1.shape[1],)
+    cache.gemm1 = mm(_flat2d(cache.normed), w1).reshaped(hiddenShape)
+    cache.hidden = addBiasAct(cache.gemm1, b1, act)
+    gemm2 = mm(_flat2d(cache.hidden), w2).reshaped(x.shape[:-1] + (w2.shape[1],))
+    return addBiasResidual(gemm2, b2, x)
+
+
+def feedForward(x, w1, b1, w2, b2, act: int = ACT_SILU, useBf16: bool = False):
+    normed = rmsnorm(x)
+    lin = linearBf16 if useBf16 else linear
+    hidden = _act(lin(normed, w1, b1), act)
+    return add(x, lin(hidden, w2, b2))
+
+
+def feedForwardBf16(x, w1, b1, w2, b2, act: int = ACT_SILU):
+    return feedForward(x, w1, b1, w2, b2, act, True)
+
+
+@dataclass
+class FeedForwardGrad:
+    dInput: DeviceTensor
+    dW1: DeviceTensor
+    dB1: DeviceTensor
+    dW2: DeviceTensor
+    dB2: DeviceTensor
+
+
+def feedForwardBackwardCached(x, w1, b1, w2, b2, cache: FeedForwardCache, g, useBf16: bool, act: int = ACT_SILU) -> FeedForwardGrad:
+    bwd = _mm_bwd(useBf16, True)
+    dB2 = biasGradientOnly(g)
+    dHiddenFlat, dW2 = bwd(_flat2d(cache.hidden), w2, _flat2d(g))
+    dHidden = dHiddenFlat.reshaped(cache.hidden.shape)
+    dGemm1, dB1 = addBiasActBackward(cache.gemm1, b1, dHidden, act)
+    dNormedFlat, dW1 = bwd(_flat2d(cache.normed), w1, _flat2d(dGemm1))
+    dNormed = dNormedFlat.reshaped(cache.normed.shape)
+    dInput = add(g, rmsnormBackward(x, dNormed))
+    return FeedForwardGrad(dInput, dW1, dB1, dW2, dB2)
+
+
+def feedForwardBackward(x, w1, b1, w2, b2, g, act: int = ACT_SILU, useBf16: bool = False) -> FeedForwardGrad:
+    """Stateless variant: recomputes the forward, like autodiff.cu:624-652."""
+    cache = FeedForwardCache()
+    cache.normed = rmsnorm(x)
+    mm = _mm(useBf16, False)
+    cache.gemm1 = mm(_flat2d(cache.normed), w1).reshaped(x.shape[:-1] + (w1.shape[1],))
+    cache.hidden = addBiasAct(cache.gemm1, b1, act)
+    bwd = _mm_bwd(useBf16, False)
+    dB2 = biasGradientOnly(g)
+    dHiddenFlat, dW2 = bwd(_flat2d(cache.hidden), w2, _flat2d(g))
+    dGemm1, dB1 = addBiasActBackward(cache.gemm1, b1, dHiddenFlat.reshaped(cache.hidden.shape), act)
+    dNormedFlat, dW1 = bwd(_flat2d(cache.normed), w1, _flat2d(dGemm1))
+    dInput = add(g, rmsnormBackward(x, dNormedFlat.reshaped(x.shape)))
+    return FeedForwardGrad(dInput, dW1, dB1, dW2, dB2)
+
+
+def feedForwardBf16Backward(x, w1, b1, w2, b2, g, act: int = ACT_SILU):
+    return feedForwardBackward(x, w1, b1, w2, b2, g, act, True)
+
+
+def _check_attention(name, x, numHeads):
+    _require(x.rank() == 3, f"{name}: needs an input of rank 3 [batch, seq, dim]")
+    _require(numHeads != 0 and x.shape[2] % numHeads == 0, f"{name}: numHeads must divide dim exactly")
+
+
+def selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads: int, useBf16: bool, cache: SelfAttentionCache,
+                               cachedWeights: bool = True):
+    _check_attention("selfAttention", x, numHeads)
+    batch, seq, dim = x.shape
+    scaleFactor = 1.0 / math.sqrt(dim // numHeads)
+    mm = _mm(useBf16, cachedWeights)
+    cache.normedFlat = rmsnorm(x).reshaped((batch * seq, dim))
+    cache.q = mm(cache.normedFlat, wq).reshaped((batch, seq, dim))
+    cache.k = mm(cache.normedFlat, wk).reshaped((batch, seq, dim))
+    cache.v = mm(cache.normedFlat, wv).reshaped((batch, seq, dim))
+    attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, 0)
+    cache.attnOutput, cache.attnM, cache.attnL = attn.output, attn.m, attn.l
+    projected = mm(_flat2d(cache.attnOutput), wout).reshaped((batch, seq, dim))
+    return add(x, projected)
+
+
+def selfAttention(x, wq, wk, wv, wout, numHeads: int):
+    return selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, False, SelfAttentionCache(), False)
+
+
+def selfAttentionBf16(x, wq, wk, wv, wout, numHeads: int):
+    return selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, True, SelfAttentionCache(), False)
+
+
+@dataclass
+class SelfAttentionGrad:
+    dInput: DeviceTensor
+    dWq: DeviceTensor
+    dWk: DeviceTensor
+    dWv: DeviceTensor
+    dWout: DeviceTensor
+
+
+def selfAttentionBackwardCached(x, wq, wk, wv, wout, numHeads: int, cache: SelfAttentionCache, g, useBf16: bool,
+                                cachedWeights: bool = True) -> SelfAttentionGrad:
+    batch, seq, dim = x.shape
+    scaleFactor = 1.0 / math.sqrt(dim // numHeads)
+    bwd = _mm_bwd(useBf16, cachedWeights)
+    dOutFlat, dWout = bwd(_flat2d(cache.attnOutput), wout, _flat2d(g))
+    dOutput = dOutFlat.reshaped((batch, seq, dim))
+    ag = fusedAttentionBackward(dOutput, cache.q, cache.k, cache.v, cache.attnOutput, cache.attnM, cache.attnL, numHeads,
+                                scaleFactor, 0)
+    dNq, dWq = bwd(cache.normedFlat, wq, _flat2d(ag.dQ))
+    dNk, dWk = bwd(cache.normedFlat, wk, _flat2d(ag.dK))
+    dNv, dWv = bwd(cache.normedFlat, wv, _flat2d(ag.dV))
+    dNormed = add(add(dNq, dNk), dNv).reshaped((batch, seq, dim))
+    dInput = add(g, rmsnormBackward(x, dNormed))
+    return SelfAttentionGrad(dInput, dWq, dWk, dWv, dWout)
+
+
+def selfAttentionBackward(x, wq, wk, wv, wout, numHeads: int, g, useBf16: bool = False) -> SelfAttentionGrad:
+    """Stateless variant: recomputes the forward, like autodiff.cu:654-700."""
+    cache = SelfAttentionCache()
+    selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, useBf16, cache, False)
+    return selfAttentionBackwardCached(x, wq, wk, wv, wout, numHeads, cache, g, useBf16, False)
+
+
+def selfAttentionBf16Backward(x, wq, wk, wv, wout, numHeads: int, g):
+    return selfAttentionBackward(x, wq, wk, wv, wout, numHeads, g, True)
+
+
+def selfAttentionIncremental(xNew, wq, wk, wv, wout, numHeads: int, cache: KVCache, useBf16: bool = False):
+    _check_attention("selfAttentionIncremental", xNew, numHeads)
+    batch, newLen, dim = xNew.shape
+    mm = _mm(useBf16, False)
+    normedFlat = rmsnorm(xNew).reshaped((batch * newLen, dim))
+    qNew = mm(normedFlat, wq).reshaped((batch, newLen, dim))
+    kNew = mm(normedFlat, wk).reshaped((batch, newLen, dim))
+    vNew = mm(normedFlat, wv).reshaped((batch, newLen, dim))
+    oldLen = cache.length
+    if oldLen == 0:
+        cache.k, cache.v = kNew, vNew
+    else:
+        cache.k, cache.v = concatSeq(cache.k, kNew), concatSeq(cache.v, vNew)
+    cache.length = oldLen + newLen
+    scaleFactor = 1.0 / math.sqrt(dim // numHeads)
+    attn = fusedAttentionForward(qNew, cache.k, cache.v, numHeads, scaleFactor, oldLen)
+    projected = mm(_flat2d(attn.output), wout).reshaped((batch, newLen, dim))
+    return add(xNew, projected)
+
+
+def selfAttentionIncrementalBf16(xNew, wq, wk, wv, wout, numHeads: int, cache: KVCache):
+    return selfAttentionIncremental(xNew, wq, wk, wv, wout, numHeads, cache, True)
+
+
+# ------------------------------------------------------------------------------------------------
+# losses (loss.hpp:20-70)
+# ------------------------------------------------------------------------------------------------
+@dataclass
+class LossResult:
+    value: float
+    grad: DeviceTensor
+
+
+def _read_scalar(t: DeviceTensor) -> float:
+    return float(t.toHost().reshape(-1)[0])
+
+
+def meanSquaredErrorAccumulate(pred, target, lossAccumulator: DeviceTensor) -> DeviceTensor:
+    _require(pred.shape == target.shape, "meanSquaredError: incompatible shapes")
+    grad = DeviceTensor(pred.shape)
+    _call("bf_hip_mse", pred.ptr, target.ptr, grad.ptr, lossAccumulator.ptr, pred.elementCount(), 1, None)
+    return grad
+
+
+def meanSquaredError(pred, target) -> LossResult:
+    _require(pred.shape == target.shape, "meanSquaredError: incompatible shapes")
+    grad, total = DeviceTensor(pred.shape), DeviceTensor((1,))
+    n = pred.elementCount()
+    _call("bf_hip_mse", pred.ptr, target.ptr, grad.ptr, total.ptr, n, 0, None)
+    return LossResult(_read_scalar(total) / n if n else 0.0, grad)
+
+
+def _check_ce(name, logits, target):
+    _require(logits.shape == target.shape, f"{name}: incompatible shapes")
+    _require(logits.rank() >= 2, f"{name}: needs a tensor of rank >= 2")
+
+
+def softmaxCrossEntropyAccumulate(logits, target, lossAccumulator: DeviceTensor) -> DeviceTensor:
+    _check_ce("softmaxCrossEntropyAccumulate", logits, target)
+    grad = DeviceTensor(logits.shape)
+    _call("bf_hip_cross_entropy", logits.ptr, target.ptr, grad.ptr, lossAccumulator.ptr, *_rows(logits), 1, None)
+    return grad
+
+
+def softmaxCrossEntropy(logits, target) -> LossResult:
+    _check_ce("softmaxCrossEntropy", logits, target)
+    grad, total = DeviceTensor(logits.shape), DeviceTensor((1,))
+    rows, classes = _rows(logits)
+    _call("bf_hip_cross_entropy", logits.ptr, target.ptr, grad.ptr, total.ptr, rows, classes, 0, None)
+    return LossResult(_read_scalar(total) / rows if rows else 0.0, grad)
+
+
+def _check_sparse(name, logits, idx):
+    _require(logits.rank() >= 2, f"{name}: needs logits of rank >= 2")
+    _require(idx.elementCount() == _rows(logits)[0], f"{name}: targetIndices count does not match the logits rows")
+
+
+def softmaxCrossEntropySparseAccumulate(logits, targetIndices, lossAccumulator: DeviceTensor) -> DeviceTensor:
+    """Indices are the caller's precondition here (loss.hpp:59-70): no range check, no host sync."""
+    _check_sparse("softmaxCrossEntropySparseAccumulate", logits, targetIndices)
+    grad = DeviceTensor(logits.shape)
+    _call("bf_hip_cross_entropy_sparse", logits.ptr, targetIndices.ptr, grad.ptr, lossAccumulator.ptr, *_rows(logits), 1,
+          None)
+    return grad
+
+
+def softmaxCrossEntropySparse(logits, targetIndices) -> LossResult:
+    _check_sparse("softmaxCrossEntropySparse", logits, targetIndices)
+    rows, classes = _rows(logits)
+    if rows:
+        _validate_ids("softmaxCrossEntropySparse", targetIndices, classes, "class index")
+    grad, total = DeviceTensor(logits.shape), DeviceTensor((1,))
+    _call("bf_hip_cross_entropy_sparse", logits.ptr, targetIndices.ptr, grad.ptr, total.ptr, rows, classes, 0, None)
+    return LossResult(_read_scalar(total) / rows if rows else 0.0, grad)
+
+
+# ------------------------------------------------------------------------------------------------
+# optimizers (optimizer.hpp:17-66)
+# ------------------------------------------------------------------------------------------------
+@dataclass
+class Parameter:
+    name: str
+    value: DeviceTensor
+    grad: DeviceTensor
+
+
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.ptr.value if t.ptr else None for t in tensors])
+
+
+class SGD:
+    def __init__(self, learningRate: float):
+        self.learningRate = learningRate
+
+    def setLearningRate(self, learningRate: float):
+        self.learningRate = learningRate
+
+    def step(self, parameters: List[Parameter]):
+        n = len(parameters)
+        if n == 0:
+            return
+        counts = (ctypes.c_size_t * n)(*[p.value.elementCount() for p in parameters])
+        _call("bf_hip_sgd_multi", _ptr_array([p.value for p in parameters]), _ptr_array([p.grad for p in parameters]),
+              counts, n, self.learningRate, None)
+
+
+class AdamW:
+    def __init__(self, learningRate=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weightDecay=0.01):
+        self.learningRate, self.beta1, self.beta2, self.eps, self.weightDecay = learningRate, beta1, beta2, eps, weightDecay
+        self.stepCount = 0
+        self.state: Dict[str, tuple] = {}
+
+    def setLearningRate(self, learningRate: float):
+        self.learningRate = learningRate
+
+    def step(self, parameters: List[Parameter]):
+        self.stepCount += 1
+        n = len(parameters)
+        if n == 0:
+            return
+        for p in parameters:
+            if p.name not in self.state:
+                self.state[p.name] = (DeviceTensor.zeros(p.value.shape), DeviceTensor.zeros(p.value.shape))
+        counts = (ctypes.c_size_t * n)(*[p.value.elementCount() for p in parameters])
+        _call("bf_hip_adamw_multi", _ptr_array([p.value for p in parameters]), _ptr_array([p.grad for p in parameters]),
+              _ptr_array([self.state[p.name][0] for p in parameters]), _ptr_array([self.state[p.name][1] for p in parameters]),
+              counts, n, self.stepCount, self.learningRate, self.beta1, self.beta2, self.eps, self.weightDecay, None)

@@ -1,0 +1,259 @@
+/*
+ * bf_hip.h -- C ABI of the MI355X (gfx950) operator backend for BlackForge.
+ *
+ * This is the drop-in boundary: plain pointers and sizes, no C++ types.  Each entry point is what
+ * the host-side operator of the reference GPU backend (namespace blackforge::backend::cuda, headers
+ * under include/blackforge/backend/cuda/ of the reference) would call instead of launching its own
+ * kernels; the reference declaration each one serves is cited beside it.  The C++ operator layer with
+ * the reference's signatures (blackforge::backend::hip, include/blackforge/backend/hip/) is written
+ * on top of these functions only.
+ *
+ * Conventions
+ *   - Every tensor is dense row-major float32 in device memory (reference: device_tensor.hpp:19-75).
+ *     Token ids and class indices are floats holding integers, rounded to nearest (lroundf), as in the
+ *     reference (ops_elementwise.cu:305-326, loss.cu:134-192).
+ *   - Every function returns BF_OK or an error code; bf_hip_last_error() gives the message of the last
+ *     failure on the calling thread.  BF_ERR_INVALID_ARGUMENT corresponds to the reference throwing
+ *     std::invalid_argument, BF_ERR_RUNTIME to std::runtime_error from its CUDA check macros
+ *     (cuda_check.hpp:14-53).
+ *   - `stream` is a hipStream_t passed as void*; NULL is the default stream.  Kernels are enqueued
+ *     and not waited for, as in the reference; only the *_h2d / *_d2h copies and the functions
+ *     documented as synchronous block the host.
+ *   - Outputs never alias inputs unless a parameter says "in/out".  Zero-sized tensors are accepted
+ *     and launch nothing (reference: device_pool.cu:30-32).
+ *   - One host thread at a time per device, like the reference (device_pool.hpp:39-40).
+ */
+#ifndef BF_HIP_H
+#define BF_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BF_OK 0
+#define BF_ERR_INVALID_ARGUMENT 1
+#define BF_ERR_RUNTIME 2
+#define BF_ERR_UNSUPPORTED 3
+
+typedef void* bf_stream_t;
+typedef void* bf_event_t;
+
+/* Activation selector for the fused bias+activation entry points. */
+enum { BF_ACT_SILU = 0, BF_ACT_GELU = 1, BF_ACT_RELU = 2 };
+
+const char* bf_hip_last_error(void);
+const char* bf_hip_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Devices, streams, events          (reference: device_query.hpp:21,33; device_query.cu:9-40)
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+    char name[128];
+    char arch[32];            /* e.g. "gfx950" */
+    int compute_units;
+    int clock_khz;            /* peak engine clock */
+    int wavefront_size;
+    int lds_bytes_per_block;  /* max LDS a workgroup may use */
+    size_t total_memory;      /* bytes of HBM */
+} bf_device_props;
+
+int bf_hip_device_count(int* count);                 /* enumerateDevices(): 0 devices is not an error */
+int bf_hip_device_props(int index, bf_device_props* props);
+int bf_hip_set_device(int index);                    /* setActiveDevice() */
+int bf_hip_get_device(int* index);
+int bf_hip_synchronize(void);                        /* hipDeviceSynchronize */
+
+int bf_hip_stream_create(bf_stream_t* stream);       /* default priority; ordered with the default stream */
+int bf_hip_stream_destroy(bf_stream_t stream);
+int bf_hip_stream_synchronize(bf_stream_t stream);
+int bf_hip_event_create(bf_event_t* event);
+int bf_hip_event_destroy(bf_event_t event);
+int bf_hip_event_record(bf_event_t event, bf_stream_t stream);
+int bf_hip_event_synchronize(bf_event_t event);
+int bf_hip_event_elapsed_ms(bf_event_t start, bf_event_t stop, float* ms);
+
+/* ---------------------------------------------------------------------------------------------
+ * Device memory: per-device size-class pool over hipMalloc   (reference: device_pool.hpp:47-54,
+ * device_pool.cu:29-65; DeviceTensor::fromHost/toHost/zeros/clone device_tensor.cu:68-117)
+ * ------------------------------------------------------------------------------------------- */
+int bf_hip_pool_acquire(size_t bytes, void** ptr);   /* devicePoolAcquire; bytes == 0 -> *ptr = NULL */
+int bf_hip_pool_release(void* ptr, size_t bytes);    /* devicePoolRelease; same `bytes` as acquired */
+typedef struct {
+    size_t bytes_from_driver;   /* total hipMalloc'd by the pool on the current device */
+    size_t bytes_in_use;        /* handed out and not yet released */
+    size_t driver_allocations;  /* number of hipMalloc calls */
+    size_t acquires;            /* number of acquire calls served */
+} bf_pool_stats;
+int bf_hip_pool_stats(bf_pool_stats* stats);
+int bf_hip_pool_trim(void);                          /* hipFree every cached block of the current device */
+
+int bf_hip_memcpy_h2d(void* dst, const void* src, size_t bytes);   /* synchronous (fromHost) */
+int bf_hip_memcpy_d2h(void* dst, const void* src, size_t bytes);   /* synchronous (toHost)   */
+int bf_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, bf_stream_t stream);  /* clone() */
+int bf_hip_fill_zero(void* dst, size_t bytes, bf_stream_t stream); /* zeros(); a fill kernel, not a memset node */
+
+/* ---------------------------------------------------------------------------------------------
+ * Elementwise family                                             (reference: ops_elementwise.cu)
+ * ------------------------------------------------------------------------------------------- */
+/* add: ops.hpp:8 */
+int bf_hip_add(const float* a, const float* b, float* out, size_t n, bf_stream_t stream);
+/* scale(x, factor): backend::cpu::scale, used by the reference's gradient averaging
+ * (multi_gpu_train_runner.cu:282-297) */
+int bf_hip_scale(const float* x, float factor, float* out, size_t n, bf_stream_t stream);
+/* addBias: ops.hpp:14   out[r,c] = x[r,c] + bias[c] */
+int bf_hip_add_bias(const float* x, const float* bias, float* out, size_t rows, size_t features,
+                    bf_stream_t stream);
+/* addBiasSilu: ops.hpp:23 (act = BF_ACT_SILU); BF_ACT_GELU / BF_ACT_RELU give the same fusion with
+ * the reference's gelu / relu formulas.  out = act(gemm + bias) */
+int bf_hip_add_bias_act(const float* gemm, const float* bias, float* out, size_t rows, size_t features, int act,
+                        bf_stream_t stream);
+/* addBiasResidual: ops.hpp:30   out = gemm + bias + residual */
+int bf_hip_add_bias_residual(const float* gemm, const float* bias, const float* residual, float* out, size_t rows,
+                             size_t features, bf_stream_t stream);
+/* silu / relu / gelu: ops.hpp:82-84 */
+int bf_hip_act_forward(const float* x, float* out, size_t n, int act, bf_stream_t stream);
+/* siluBackward / reluBackward / geluBackward: autodiff.hpp:74-76   out = g * act'(x) */
+int bf_hip_act_backward(const float* x, const float* g, float* out, size_t n, int act, bf_stream_t stream);
+/* addBiasSiluBackward: autodiff.hpp:71.  dGemm = dHidden * act'(gemm + bias); dBias = column sums of
+ * dGemm (dBias may be NULL to skip it). */
+int bf_hip_add_bias_act_backward(const float* gemm, const float* bias, const float* dHidden, float* dGemm,
+                                 float* dBias, size_t rows, size_t features, int act, bf_stream_t stream);
+/* accumulate: model.cu:40-46   target += delta (in/out) */
+int bf_hip_accumulate(float* target, const float* delta, size_t n, bf_stream_t stream);
+/* zeroFused: model.cu:84-105.  `ptrs`/`counts` are HOST arrays of numTensors device pointers / element
+ * counts; one launch zeroes them all. */
+int bf_hip_zero_multi(float* const* ptrs, const size_t* counts, size_t numTensors, bf_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Row-wise ops                                     (reference: ops_elementwise.cu, autodiff.cu)
+ * ------------------------------------------------------------------------------------------- */
+/* rmsnorm: ops.hpp:92   y = x / sqrt(mean(x^2) + 1e-6), no gain */
+int bf_hip_rmsnorm(const float* x, float* out, size_t rows, size_t features, bf_stream_t stream);
+/* rmsnormBackward: autodiff.hpp:79 */
+int bf_hip_rmsnorm_backward(const float* x, const float* g, float* out, size_t rows, size_t features,
+                            bf_stream_t stream);
+/* softmax: ops.hpp:98 */
+int bf_hip_softmax(const float* x, float* out, size_t rows, size_t features, bf_stream_t stream);
+/* softmaxBackward: autodiff.hpp:84 (takes the forward INPUT, recomputes y) */
+int bf_hip_softmax_backward(const float* x, const float* g, float* out, size_t rows, size_t features,
+                            bf_stream_t stream);
+/* biasGradientOnly / addBiasBackward's dBias: autodiff.hpp:52,59   dBias[c] = sum_r g[r,c] */
+int bf_hip_bias_grad(const float* g, float* dBias, size_t rows, size_t features, bf_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Gather / scatter                                 (reference: ops_elementwise.cu, autodiff.cu)
+ * ------------------------------------------------------------------------------------------- */
+/* Range check used by the validating variants (embeddingLookup ops.hpp:104,
+ * embeddingLookupBackward autodiff.hpp:90, softmaxCrossEntropySparse loss.hpp:37): counts entries of
+ * `ids` whose rounded value is outside [0, limit).  Synchronous; *firstBad receives one offending
+ * rounded value when the count is non-zero. */
+int bf_hip_count_out_of_range(const float* ids, size_t count, size_t limit, size_t* numBad, long long* firstBad,
+                              bf_stream_t stream);
+/* embeddingLookupPreValidated: ops.hpp:110   out[t,:] = table[lround(ids[t]),:]  (bit-exact copy) */
+int bf_hip_embedding_forward(const float* ids, const float* table, float* out, size_t tokens, size_t vocab,
+                             size_t dim, bf_stream_t stream);
+/* embeddingLookupBackwardPreValidated: autodiff.hpp:98.  Writes every element of dTable[vocab,dim]
+ * once: rows are summed over their tokens in token order (deterministic, no atomics). */
+int bf_hip_embedding_backward(const float* ids, const float* g, float* dTable, size_t tokens, size_t vocab,
+                              size_t dim, bf_stream_t stream);
+/* addPositionalEmbedding / addPositionalEmbeddingAt: ops.hpp:115,122   out[b,s,:] = x[b,s,:] + table[offset+s,:] */
+int bf_hip_positional_forward(const float* x, const float* table, float* out, size_t batch, size_t seq, size_t dim,
+                              size_t maxSeq, size_t offset, bf_stream_t stream);
+/* addPositionalEmbeddingBackward: autodiff.hpp:106   dTable[s,:] = sum_b g[b,s,:]; rows >= seq are zero */
+int bf_hip_positional_backward(const float* g, float* dTable, size_t batch, size_t seq, size_t dim, size_t maxSeq,
+                               bf_stream_t stream);
+/* concatSeq (KV-cache growth): ops_transformer.cu:22-58   [batch,seqA,dim] ++ [batch,seqB,dim] */
+int bf_hip_concat_seq(const float* a, const float* b, float* out, size_t batch, size_t seqA, size_t seqB, size_t dim,
+                      bf_stream_t stream);
+/* argmaxLastPosition: main.cpp:504-518, moved to the device.  logits: [seq, vocab]; *index (HOST) gets
+ * the lowest index of the maximum of the last row.  Synchronous. */
+int bf_hip_argmax_last_position(const float* logits, size_t seq, size_t vocab, long long* index, bf_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * GEMM                                      (reference: ops_gemm.cu, ops_tensorcore.cu, autodiff.cu)
+ * ------------------------------------------------------------------------------------------- */
+/* C[M,N] = op(A) * op(B) in fp32 on fp32 MFMA.  op(A) is M x K: A is [M,K] (transA = 0) or [K,M]
+ * (transA = 1); op(B) is K x N: B is [K,N] (transB = 0) or [N,K] (transB = 1).
+ * matmul ops.hpp:35 (0,0); matmulTransposeB ops.hpp:40 (0,1); matmulBackward autodiff.hpp:23 (dA: 0,1 on
+ * G,B; dB: 1,0 on A,G); matmulTransposeBBackward autodiff.hpp:44 (dA: 0,0 on G,B; dB: 1,0 on G,A). */
+int bf_hip_gemm_f32(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K,
+                    bf_stream_t stream);
+/* floatToBf16 (round to nearest even): ops_tensorcore.cu:21-26,80-87.  `out` holds n bf16 values. */
+int bf_hip_cvt_f32_bf16(const float* x, uint16_t* out, size_t n, bf_stream_t stream);
+/* Same rounding, writing out[c,r] = bf16(x[r,c]) for x:[rows,cols]. */
+int bf_hip_cvt_f32_bf16_transpose(const float* x, uint16_t* out, size_t rows, size_t cols, bf_stream_t stream);
+/* C[M,N] (fp32) = A[M,K] * Bt[N,K]^T with bf16 operands, fp32 accumulate, on bf16 MFMA
+ * (the cublasLtMatmul call, ops_tensorcore.cu:293-304). */
+int bf_hip_gemm_bf16_nt(const uint16_t* A, const uint16_t* Bt, float* C, size_t M, size_t N, size_t K,
+                        bf_stream_t stream);
+/* matmulBf16 ops.hpp:53 (cacheWeight = 0) / matmulBf16CachedWeight ops.hpp:72 (cacheWeight = 1):
+ * c[m,n] = bf16(a[m,k]) * bf16(b[k,n]), fp32 accumulate.  With cacheWeight the bf16 image of `b` is kept
+ * per (device, pointer) until bf_hip_invalidate_bf16_weight_cache(). */
+int bf_hip_matmul_bf16(const float* a, const float* b, float* c, size_t m, size_t k, size_t n, int cacheWeight,
+                       bf_stream_t stream);
+/* matmulBf16Backward autodiff.hpp:29 / matmulBf16BackwardCachedWeight autodiff.hpp:36:
+ * dA[m,k] = bf16(g) * bf16(b)^T, dB[k,n] = bf16(a)^T * bf16(g).  Either output may be NULL. */
+int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, float* dA, float* dB, size_t m,
+                                size_t k, size_t n, int cacheWeight, bf_stream_t stream);
+/* invalidateBf16WeightCache: ops.hpp:80 */
+int bf_hip_invalidate_bf16_weight_cache(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Fused causal attention                                  (reference: fused_attention.hpp:55,73)
+ * q:[batch,newLen,dim]  k,v:[batch,totalLen,dim]  heads contiguous in dim, headDim = dim/heads <= 256.
+ * Query row i (absolute position oldLen+i) attends to keys j <= oldLen+i.
+ * ------------------------------------------------------------------------------------------- */
+/* fusedAttentionForward: out:[batch,newLen,dim]; m,l:[batch,heads,newLen] = row max of the scaled
+ * scores and sum of exp(score - m) (the statistics the backward reuses). */
+int bf_hip_attention_forward(const float* q, const float* k, const float* v, float* out, float* m, float* l,
+                             size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
+                             size_t oldLen, bf_stream_t stream);
+/* computeDKernel: fused_attention.cu:166-190   D[b,h,i] = dot(out[b,i,h,:], dOut[b,i,h,:]) */
+int bf_hip_attention_dot_o_do(const float* out, const float* dOut, float* D, size_t batch, size_t heads,
+                              size_t newLen, size_t dim, bf_stream_t stream);
+/* fusedAttentionBackward: dQ:[batch,newLen,dim], dK,dV:[batch,totalLen,dim].  dK/dV are accumulated
+ * by the workgroup that owns a key tile and written once; dQ by the workgroup that owns a query
+ * tile.  No atomics: results are bit-reproducible run to run. */
+int bf_hip_attention_backward(const float* dOut, const float* q, const float* k, const float* v, const float* out,
+                              const float* m, const float* l, float* dQ, float* dK, float* dV, size_t batch,
+                              size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
+                              bf_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Losses                                                      (reference: loss.hpp:20-70, loss.cu)
+ * Each writes grad (same shape as the prediction) and the SUM over the batch of the per-row (per-
+ * element for MSE) loss terms into lossSum[0] (device): overwritten when accumulate == 0, added to when
+ * accumulate != 0 (the *Accumulate variants, loss.hpp:54-70).  The mean is lossSum / rows (/ n).
+ * ------------------------------------------------------------------------------------------- */
+/* meanSquaredError[Accumulate]: grad = 2 (p - t) / n, lossSum = sum (p - t)^2 */
+int bf_hip_mse(const float* pred, const float* target, float* grad, float* lossSum, size_t n, int accumulate,
+               bf_stream_t stream);
+/* softmaxCrossEntropy[Accumulate]: dense targets */
+int bf_hip_cross_entropy(const float* logits, const float* target, float* grad, float* lossSum, size_t rows,
+                         size_t classes, int accumulate, bf_stream_t stream);
+/* softmaxCrossEntropySparse[Accumulate]: target class index per row; indices must already be in range */
+int bf_hip_cross_entropy_sparse(const float* logits, const float* targetIdx, float* grad, float* lossSum,
+                                size_t rows, size_t classes, int accumulate, bf_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Optimizers                                              (reference: optimizer.hpp:28-66, optimizer.cu)
+ * `params`, `grads`, `m`, `v`, `counts` are HOST arrays with one entry per tensor; one launch updates
+ * every tensor in place.
+ * ------------------------------------------------------------------------------------------- */
+/* SGD::step: p -= lr * g */
+int bf_hip_sgd_multi(float* const* params, const float* const* grads, const size_t* counts, size_t numTensors,
+                     float lr, bf_stream_t stream);
+/* AdamW::step with `step` the 1-based count after increment (optimizer.cu:103-107):
+ * m = b1 m + (1-b1) g; v = b2 v + (1-b2) g^2; p -= lr (m/(1-b1^t) / (sqrt(v/(1-b2^t)) + eps) + wd p) */
+int bf_hip_adamw_multi(float* const* params, const float* const* grads, float* const* m, float* const* v,
+                       const size_t* counts, size_t numTensors, long long step, float lr, float beta1, float beta2,
+                       float eps, float weightDecay, bf_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* BF_HIP_H */

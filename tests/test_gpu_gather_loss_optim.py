@@ -1,0 +1,169 @@
+"""GPU parity: embedding / positional / concat / argmax (bit-exact), losses, optimizers."""
+import numpy as np
+import pytest
+
+from parity import assert_bits_equal, assert_close
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+def r(rng, *s, scale=1.0):
+    return (rng.standard_normal(s) * scale).astype(f32)
+
+
+@pytest.mark.parametrize("batch,seq,vocab,dim", [(1, 3, 3, 2), (2, 5, 11, 6), (8, 64, 256, 128), (3, 33, 1000, 770), (2, 17, 50257, 8)])
+def test_embedding_gather_and_scatter_are_bit_exact(hip, oracle, rng, batch, seq, vocab, dim):
+    D, ops = hip.DeviceTensor, hip.ops
+    ids = rng.integers(0, vocab, (batch, seq)).astype(f32)
+    ids[0, 0] = vocab - 1
+    ids.flat[-1] = ids.flat[0]  # a repeated id
+    table, g = r(rng, vocab, dim), r(rng, batch, seq, dim)
+    assert_bits_equal(ops.embeddingLookup(D.fromHost(ids), D.fromHost(table)).toHost(), oracle.embeddingLookup(ids, table))
+    # gradient rows are summed in token order, like the CPU loop: identical bits
+    assert_bits_equal(ops.embeddingLookupBackward(D.fromHost(ids), D.fromHost(g), vocab).toHost(),
+                      oracle.embeddingLookupBackward(ids, g, vocab))
+
+
+def test_embedding_reference_literals_and_range_errors(hip):
+    """tests/backend/cpu/ops_tests.cpp:238-262, autodiff_tests.cpp:180-199, cuda/ops_tests.cu:300-306."""
+    D, ops = hip.DeviceTensor, hip.ops
+    table = D.fromHost(np.array([10, 11, 20, 21, 30, 31], f32).reshape(3, 2))
+    out = ops.embeddingLookup(D.fromHost(np.array([[0, 2, 1]], f32)), table).toHost()
+    np.testing.assert_array_equal(out.ravel(), [10, 11, 30, 31, 20, 21])
+    for bad in (3.0, -1.0):
+        with pytest.raises(ValueError):
+            ops.embeddingLookup(D.fromHost(np.array([[bad]], f32)), table)
+        with pytest.raises(ValueError):
+            ops.embeddingLookupBackward(D.fromHost(np.array([[bad]], f32)), D.zeros((1, 1, 2)), 3)
+    dt = ops.embeddingLookupBackward(D.fromHost(np.array([[0, 1, 0]], f32)),
+                                     D.fromHost(np.array([1, 2, 10, 20, 3, 4], f32).reshape(1, 3, 2)), 3).toHost()
+    np.testing.assert_array_equal(dt.ravel(), [4, 6, 10, 20, 0, 0])
+    # rounding of float ids: 1.4 -> 1, 1.6 -> 2 (lround)
+    out = ops.embeddingLookup(D.fromHost(np.array([[1.4, 1.6]], f32)), table).toHost()
+    np.testing.assert_array_equal(out.ravel(), [20, 21, 30, 31])
+
+
+@pytest.mark.parametrize("batch,seq,dim,max_seq", [(2, 2, 2, 2), (3, 5, 7, 9), (8, 64, 128, 64), (2, 100, 772, 128)])
+def test_positional_embedding(hip, oracle, rng, batch, seq, dim, max_seq):
+    D, ops = hip.DeviceTensor, hip.ops
+    x, table = r(rng, batch, seq, dim), r(rng, max_seq, dim)
+    for off in {0, max_seq - seq}:
+        assert_bits_equal(ops.addPositionalEmbeddingAt(D.fromHost(x), D.fromHost(table), off).toHost(),
+                          oracle.addPositionalEmbeddingAt(x, table, off))
+    di, dt = ops.addPositionalEmbeddingBackward(D.fromHost(x), max_seq)
+    assert_bits_equal(di.toHost(), x)
+    assert_bits_equal(dt.toHost(), oracle.addPositionalEmbeddingBackward(x, max_seq)[1])
+    with pytest.raises(ValueError):
+        ops.addPositionalEmbeddingAt(D.fromHost(x), D.fromHost(table), max_seq - seq + 1)
+    with pytest.raises(ValueError):
+        ops.addPositionalEmbeddingBackward(D.fromHost(x), seq - 1)
+
+
+def test_concat_seq_and_argmax(hip, oracle, rng):
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b = r(rng, 3, 4, 10), r(rng, 3, 2, 10)
+    assert_bits_equal(ops.concatSeq(D.fromHost(a), D.fromHost(b)).toHost(), np.concatenate([a, b], axis=1))
+    for vocab in (1, 5, 1000, 50257):
+        logits = r(rng, 1, 3, vocab)
+        logits[0, 2, vocab // 2] = logits[0, 2].max()  # a tie: the lower index must win
+        assert ops.argmaxLastPosition(D.fromHost(logits)) == oracle.argmaxLastPosition(logits[0])
+    logits = np.zeros((2, 9), f32)
+    assert ops.argmaxLastPosition(D.fromHost(logits)) == 0
+
+
+@pytest.mark.parametrize("rows,classes", [(1, 2), (2, 3), (7, 13), (512, 256), (5, 1000), (3, 32000), (2, 50257), (1, 70001)])
+def test_cross_entropy(hip, oracle, rng, rows, classes):
+    D, ops = hip.DeviceTensor, hip.ops
+    logits = r(rng, rows, classes, scale=3)
+    idx = rng.integers(0, classes, rows)
+    res = ops.softmaxCrossEntropySparse(D.fromHost(logits), D.fromHost(idx.astype(f32)))
+    ev, eg = oracle.softmaxCrossEntropySparse(logits, idx.astype(f32))
+    assert abs(res.value - ev) <= 1e-4 * abs(ev) + 1e-6
+    assert_close(res.grad.toHost(), eg, what="sparse CE grad")
+    if rows * classes < 10_000_000:
+        dense = np.zeros((rows, classes), f32)
+        dense[np.arange(rows), idx] = 0.7
+        dense[np.arange(rows), (idx + 1) % classes] += 0.3
+        res = ops.softmaxCrossEntropy(D.fromHost(logits), D.fromHost(dense))
+        ev, eg = oracle.softmaxCrossEntropy(logits, dense)
+        assert abs(res.value - ev) <= 1e-4 * abs(ev) + 1e-6
+        assert_close(res.grad.toHost(), eg, what="dense CE grad")
+
+
+def test_loss_literals_errors_and_accumulate(hip, oracle, rng):
+    """tests/backend/cpu/loss_tests.cpp:10-16,51-69,115-140; cuda/loss_tests.cu:124-130."""
+    import math
+    D, ops = hip.DeviceTensor, hip.ops
+    assert ops.meanSquaredError(D.fromHost(np.array([1, 2], f32)), D.fromHost(np.zeros(2, f32))).value == 2.5
+    res = ops.softmaxCrossEntropy(D.fromHost(np.zeros((1, 2), f32)), D.fromHost(np.array([[1, 0]], f32)))
+    assert abs(res.value - math.log(2)) < 1e-6
+    np.testing.assert_allclose(res.grad.toHost().ravel(), [-0.5, 0.5], atol=1e-6)
+    with pytest.raises(ValueError):
+        ops.softmaxCrossEntropySparse(D.fromHost(np.array([[0.1, 0.2, 0.3]], f32)), D.fromHost(np.array([5], f32)))
+    with pytest.raises(ValueError):
+        ops.softmaxCrossEntropySparse(D.zeros((2, 3)), D.zeros((3,)))
+    with pytest.raises(ValueError):
+        ops.meanSquaredError(D.zeros((2,)), D.zeros((3,)))
+    with pytest.raises(ValueError):
+        ops.softmaxCrossEntropy(D.zeros((2,)), D.zeros((2,)))
+    # *Accumulate: the accumulator receives the SUM of row losses of each call (loss.hpp:39-57)
+    p, t = r(rng, 6, 10), r(rng, 6, 10)
+    acc = D.zeros((1,))
+    for _ in range(3):
+        g = ops.meanSquaredErrorAccumulate(D.fromHost(p), D.fromHost(t), acc)
+    ev, eg = oracle.meanSquaredError(p, t)
+    assert_close(g.toHost(), eg)
+    assert abs(acc.toHost()[0] - 3 * ev * p.size) <= 1e-4 * 3 * ev * p.size
+    idx = rng.integers(0, 10, 6).astype(f32)
+    acc = D.zeros((1,))
+    for _ in range(2):
+        g = ops.softmaxCrossEntropySparseAccumulate(D.fromHost(p), D.fromHost(idx), acc)
+    ev, eg = oracle.softmaxCrossEntropySparse(p, idx)
+    assert_close(g.toHost(), eg)
+    assert abs(acc.toHost()[0] - 2 * ev * 6) <= 1e-4 * 2 * ev * 6
+
+
+@pytest.mark.parametrize("n", [1, 1000, 1 << 20])
+def test_mse(hip, oracle, rng, n):
+    D, ops = hip.DeviceTensor, hip.ops
+    p, t = r(rng, n), r(rng, n)
+    res = ops.meanSquaredError(D.fromHost(p), D.fromHost(t))
+    ev, eg = oracle.meanSquaredError(p, t)
+    assert abs(res.value - ev) <= 1e-4 * ev + 1e-12
+    assert_close(res.grad.toHost(), eg)
+
+
+def test_optimizers_multi_tensor(hip, oracle, rng):
+    """SGD / AdamW closed forms of tests/backend/cpu/optimizer_tests.cpp:10-59, then 10 steps on ragged tensors."""
+    import math
+    D, ops = hip.DeviceTensor, hip.ops
+    p = ops.Parameter("p", D.fromHost(np.array([1, -2], f32)), D.fromHost(np.array([0.5, 0.5], f32)))
+    ops.SGD(0.1).step([p])
+    assert_bits_equal(p.value.toHost(), np.array([1, -2], f32) - f32(0.1) * f32(0.5))
+    p = ops.Parameter("p", D.fromHost(np.array([1], f32)), D.fromHost(np.array([0.2], f32)))
+    ops.AdamW(0.1, 0.9, 0.999, 1e-8, 0.0).step([p])
+    assert abs(p.value.toHost()[0] - (1.0 - 0.1 * (0.2 / (math.sqrt(0.04) + 1e-8)))) < 1e-5
+    p = ops.Parameter("p", D.fromHost(np.array([1], f32)), D.fromHost(np.array([0], f32)))
+    ops.AdamW(0.1, 0.9, 0.999, 1e-8, 0.1).step([p])
+    assert p.value.toHost()[0] == f32(1.0) - f32(0.1) * f32(0.1)
+
+    sizes = [1, 7, 8192, 8195, 300001]
+    host_p = [r(rng, n) for n in sizes]
+    params = [ops.Parameter(f"t{i}", D.fromHost(a), D.zeros((n,))) for i, (a, n) in enumerate(zip(host_p, sizes))]
+    opt = ops.AdamW(1e-2)
+    m = [np.zeros(n, f32) for n in sizes]
+    v = [np.zeros(n, f32) for n in sizes]
+    for step in range(1, 11):
+        grads = [r(rng, n) for n in sizes]
+        for prm, g in zip(params, grads):
+            prm.grad = D.fromHost(g)
+        opt.step(params)
+        for i, g in enumerate(grads):
+            host_p[i], m[i], v[i] = oracle.adamwStep(host_p[i], g, m[i], v[i], step, 1e-2)
+    for prm, e in zip(params, host_p):
+        assert_close(prm.value.toHost(), e, what="AdamW after 10 steps")
+    sgd = ops.SGD(0.05)
+    sgd.step(params)
+    for prm, e, g in zip(params, host_p, grads):
+        assert_close(prm.value.toHost(), oracle.sgdStep(e, g, 0.05), what="SGD")

@@ -1,0 +1,124 @@
+"""GPU parity: fp32 GEMM family (fp32 MFMA) and bf16 projections (bf16 MFMA, fp32 accumulate)."""
+import numpy as np
+import pytest
+
+from parity import BF16_TOL, assert_bits_equal, assert_close
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+def r(rng, *s, scale=1.0):
+    return (rng.standard_normal(s) * scale).astype(f32)
+
+
+SHAPES = [(1, 1, 1), (2, 2, 2), (5, 7, 3), (33, 65, 17), (64, 64, 64), (128, 16, 128), (130, 200, 70), (512, 128, 256),
+          (257, 512, 129), (1024, 96, 1536)]
+
+
+def test_matmul_reference_literal(hip):
+    """tests/backend/cpu/ops_tests.cpp:36-46 and, through bf16, tests/backend/cuda/ops_tests.cu:85-103."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b = D.fromHost(np.array([[1, 2], [3, 4]], f32)), D.fromHost(np.array([[5, 6], [7, 8]], f32))
+    np.testing.assert_array_equal(ops.matmul(a, b).toHost().ravel(), [19, 22, 43, 50])
+    np.testing.assert_array_equal(ops.matmulBf16(a, b).toHost().ravel(), [19, 22, 43, 50])
+    with pytest.raises(ValueError):
+        ops.matmul(D.zeros((2, 3)), D.zeros((2, 2)))
+    with pytest.raises(ValueError):
+        ops.matmulBf16(D.zeros((2, 3)), D.zeros((2, 2)))
+    with pytest.raises(ValueError):
+        ops.matmulBackward(D.zeros((2, 3)), D.zeros((3, 2)), D.zeros((2, 3)))
+
+
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_fp32_gemm_family(hip, oracle, rng, m, k, n):
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b, bt, g = r(rng, m, k), r(rng, k, n), r(rng, n, k), r(rng, m, n)
+    da, db, dbt, dg = map(D.fromHost, (a, b, bt, g))
+    assert_close(ops.matmul(da, db).toHost(), oracle.matmul(a, b), what="matmul")
+    assert_close(ops.matmulTransposeB(da, dbt).toHost(), oracle.matmulTransposeB(a, bt), what="matmulTransposeB")
+    for got, exp, nm in zip(ops.matmulBackward(da, db, dg), oracle.matmulBackward(a, b, g), ("dA", "dB")):
+        assert_close(got.toHost(), exp, what="matmulBackward." + nm)
+    for got, exp, nm in zip(ops.matmulTransposeBBackward(da, dbt, dg), oracle.matmulTransposeBBackward(a, bt, g), ("dA", "dB")):
+        assert_close(got.toHost(), exp, what="matmulTransposeBBackward." + nm)
+    bias = r(rng, n)
+    assert_close(ops.linear(da, db, D.fromHost(bias)).toHost(), oracle.linear(a, b, bias), what="linear")
+
+
+def test_fp32_gemm_large_tile_path(hip, rng):
+    """Big enough for the 128x128-tile kernel; checked against float64 numpy on a sample of rows."""
+    D, ops = hip.DeviceTensor, hip.ops
+    m, k, n = 2048, 300, 4224
+    a, b = r(rng, m, k), r(rng, k, n)
+    c = ops.matmul(D.fromHost(a), D.fromHost(b)).toHost()
+    rows = [0, 1, 127, 128, 1000, 2047]
+    assert_close(c[rows], a[rows].astype(np.float64) @ b.astype(np.float64), what="matmul 128-tile")
+
+
+def test_linear_rank3_and_identity(hip, oracle):
+    """tests/backend/cpu/ops_tests.cpp:54-63,173-184."""
+    D, ops = hip.DeviceTensor, hip.ops
+    out = ops.linear(D.fromHost(np.array([[3, 4]], f32)), D.fromHost(np.eye(2, dtype=f32)), D.fromHost(np.array([10, 20], f32)))
+    np.testing.assert_array_equal(out.toHost().ravel(), [13, 24])
+    x = np.array([1, 1, 2, 2, 3, 3, 4, 4, 5, 5, 6, 6], f32).reshape(2, 3, 2)
+    out = ops.linear(D.fromHost(x), D.fromHost(np.ones((2, 1), f32)), D.zeros((1,)))
+    assert out.shape == (2, 3, 1)
+    np.testing.assert_array_equal(out.toHost().ravel(), x.sum(-1).ravel())
+
+
+def test_bf16_conversion_is_round_to_nearest_even(hip, oracle, rng):
+    import ctypes
+    D = hip.DeviceTensor
+    x = np.concatenate([r(rng, 1003, scale=100), np.array([1 + 2.0 ** -8, 1 + 3 * 2.0 ** -8, np.inf, -np.inf, 0.0, -0.0], f32)])
+    dx = D.fromHost(x)
+    out = D((x.size,), itemsize=2)
+    hip.capi.call("bf_hip_cvt_f32_bf16", dx.ptr, out.ptr, x.size, None)
+    bits = out.toHost().astype(np.uint32) << 16
+    assert_bits_equal(bits.view(f32), oracle.roundToBf16(x))
+    # transposing variant
+    m = r(rng, 37, 50)
+    outT = D((50, 37), itemsize=2)
+    hip.capi.call("bf_hip_cvt_f32_bf16_transpose", D.fromHost(m).ptr, outT.ptr, 37, 50, None)
+    assert_bits_equal((outT.toHost().astype(np.uint32) << 16).view(f32), oracle.roundToBf16(m).T)
+
+
+@pytest.mark.parametrize("m,k,n", SHAPES + [(256, 1024, 768)])
+@pytest.mark.parametrize("cached", [False, True])
+def test_bf16_projection_and_gradients(hip, oracle, rng, m, k, n, cached):
+    """c = bf16(a) bf16(b) with fp32 accumulation: against the fp32 oracle on bf16-rounded operands
+    (tight: only the summation order differs) and against the unrounded fp32 product (2e-2)."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b, g = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, m, n)
+    da, db, dg = map(D.fromHost, (a, b, g))
+    ar, br, gr = oracle.roundToBf16(a), oracle.roundToBf16(b), oracle.roundToBf16(g)
+    fwd = ops.matmulBf16CachedWeight if cached else ops.matmulBf16
+    bwd = ops.matmulBf16BackwardCachedWeight if cached else ops.matmulBf16Backward
+    ops.invalidateBf16WeightCache()
+    c = fwd(da, db).toHost()
+    assert_close(c, oracle.matmul(ar, br), tol=1e-4, what="bf16 fwd vs rounded operands")
+    assert_close(c, oracle.matmul(a, b), tol=BF16_TOL, what="bf16 fwd vs fp32")
+    dA, dB = bwd(da, db, dg)
+    eA, eB = oracle.matmulBackward(ar, br, gr)
+    assert_close(dA.toHost(), eA, tol=1e-4, what="bf16 dA vs rounded operands")
+    assert_close(dB.toHost(), eB, tol=1e-4, what="bf16 dB vs rounded operands")
+    fA, fB = oracle.matmulBackward(a, b, g)
+    assert_close(dA.toHost(), fA, tol=BF16_TOL, what="bf16 dA vs fp32")
+    assert_close(dB.toHost(), fB, tol=BF16_TOL, what="bf16 dB vs fp32")
+
+
+def test_bf16_weight_cache_semantics(hip, oracle, rng):
+    """A cached weight image is reused until invalidateBf16WeightCache() (ops_tensorcore.cu:98-131,448)."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b = r(rng, 16, 32), r(rng, 32, 24)
+    da, db = D.fromHost(a), D.fromHost(b)
+    ops.invalidateBf16WeightCache()
+    first = ops.matmulBf16CachedWeight(da, db).toHost()
+    b2 = r(rng, 32, 24)
+    hip.capi.call("bf_hip_memcpy_h2d", db.ptr, b2.ctypes.data, b2.nbytes)   # weights change in place
+    stale = ops.matmulBf16CachedWeight(da, db).toHost()
+    assert_bits_equal(stale, first, "cached image must be reused")
+    ops.invalidateBf16WeightCache()
+    fresh = ops.matmulBf16CachedWeight(da, db).toHost()
+    assert_close(fresh, oracle.matmul(oracle.roundToBf16(a), oracle.roundToBf16(b2)), tol=1e-4)
+    lin = ops.linearBf16(da, db, D.fromHost(np.ones(24, f32))).toHost()
+    assert_close(lin, oracle.matmul(oracle.roundToBf16(a), oracle.roundToBf16(b2)) + 1, tol=1e-4)
