@@ -83,11 +83,12 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormKernel(const float* 
     for (size_t row = firstRow; row < rows; row += rowStep) {
         Row<G, MAXE, VEC, CACHED> rx;
         rx.open(x + row * features, features, t, 0.0f);
-        float ss = 0.0f;
-        rx.reduce([&](float v) { ss += v * v; });
-        ss = groupSum<G>(ss, lds);
-        float inv = 1.0f / sqrtf(ss / float(features) + kRmsNormEps);
-        rx.map(out + row * features, [&](float v, size_t) { return v * inv; });
+        // sum of squares in double and x / rms in float, as the reference does (ops.cpp:264-275)
+        double ss = 0.0;
+        rx.reduce([&](float v) { ss += double(v) * double(v); });
+        ss = groupSum<G>(ss, ldsD);
+        float rms = float(sqrt(ss / double(features) + double(kRmsNormEps)));
+        rx.map(out + row * features, [&](float v, size_t) { return v / rms; });
     }
 }
 
@@ -99,25 +100,27 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const
         Row<G, MAXE, VEC, CACHED> rx, rg;
         rx.open(x + row * features, features, t, 0.0f);
         rg.open(g + row * features, features, t, 0.0f);
-        float ss = 0.0f, gx = 0.0f;
+        // double sums and a double final formula, as the reference does (autodiff.cpp:212-229): the two
+        // terms cancel almost completely for short rows, which float arithmetic cannot resolve
+        double ss = 0.0, gx = 0.0;
         if constexpr (CACHED) {
 #pragma unroll
-            for (int i = 0; i < MAXE; ++i) { ss += rx.c.r[i] * rx.c.r[i]; gx += rg.c.r[i] * rx.c.r[i]; }
+            for (int i = 0; i < MAXE; ++i) { double xv = rx.c.r[i]; ss += xv * xv; gx += double(rg.c.r[i]) * xv; }
         } else {
-            for (size_t e = t; e < features; e += G) { float xv = rx.p[e]; ss += xv * xv; gx += rg.p[e] * xv; }
+            for (size_t e = t; e < features; e += G) { double xv = rx.p[e]; ss += xv * xv; gx += double(rg.p[e]) * xv; }
         }
-        ss = groupSum<G>(ss, lds);
-        gx = groupSum<G>(gx, lds);
-        float r = sqrtf(ss / float(features) + kRmsNormEps);
-        float invR = 1.0f / r;
-        float k = gx / (float(features) * r * r * r);
+        ss = groupSum<G>(ss, ldsD);
+        gx = groupSum<G>(gx, ldsD);
+        const double r = sqrt(ss / double(features) + double(kRmsNormEps));
+        const double invR = 1.0 / r;
+        const double k = gx / (double(features) * r * r * r);
         float* o = out + row * features;
         if constexpr (CACHED) {
 #pragma unroll
-            for (int i = 0; i < MAXE; ++i) rg.c.r[i] = rg.c.r[i] * invR - rx.c.r[i] * k;
+            for (int i = 0; i < MAXE; ++i) rg.c.r[i] = float(double(rg.c.r[i]) * invR - double(rx.c.r[i]) * k);
             rg.c.store(o, features, t);
         } else {
-            for (size_t e = t; e < features; e += G) o[e] = rg.p[e] * invR - rx.p[e] * k;
+            for (size_t e = t; e < features; e += G) o[e] = float(double(rg.p[e]) * invR - double(rx.p[e]) * k);
         }
     }
 }

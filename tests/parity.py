@@ -4,7 +4,12 @@ fp32 ops and the attention core: every element must satisfy
     |gpu - ref| <= 1e-4 * |ref| + 1e-4 * rms(ref)
 i.e. a maximum relative error of 1e-4 with an absolute floor of 1e-4 of the tensor's typical
 magnitude, so that elements that happen to be near zero are judged against the scale of the tensor
-rather than against themselves.  bf16 projections and their gradients use 2e-2 in the same formula.
+rather than against themselves.  Where a result is a difference of nearly equal terms (attention
+gradients: dS = P * (dP - D) vanishes identically for a row with one visible key), rms(ref) can be
+arbitrarily small or zero; such tests pass `scale`, the magnitude of the terms being combined, and the
+floor becomes 1e-4 * max(rms(ref), scale).  (The reference's own GPU-vs-CPU tests use absolute
+tolerances: 1e-3 for attention, tests/backend/cuda/ops_tests.cu:342-363.)
+bf16 projections and their gradients use 2e-2 in the same formula.
 Integer / index / copy work (embedding gather, argmax, concat) must be bit-exact.
 """
 import numpy as np
@@ -13,7 +18,7 @@ FP32_TOL = 1e-4
 BF16_TOL = 2e-2
 
 
-def assert_close(actual, expected, tol=FP32_TOL, what=""):
+def assert_close(actual, expected, tol=FP32_TOL, what="", scale=0.0):
     actual = np.asarray(actual, np.float64)
     expected = np.asarray(expected, np.float64)
     assert actual.shape == expected.shape, f"{what}: shape {actual.shape} != {expected.shape}"
@@ -21,7 +26,7 @@ def assert_close(actual, expected, tol=FP32_TOL, what=""):
         return
     assert np.isfinite(actual).all(), f"{what}: non-finite values in the GPU result"
     rms = float(np.sqrt(np.mean(expected ** 2)))
-    bound = tol * np.abs(expected) + tol * rms + 1e-30
+    bound = tol * np.abs(expected) + tol * max(rms, float(scale)) + 1e-30
     err = np.abs(actual - expected)
     worst = int(np.argmax(err - bound))
     assert (err <= bound).all(), (

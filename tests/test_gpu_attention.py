@@ -15,6 +15,16 @@ def r(rng, *s, scale=1.0):
     return (rng.standard_normal(s) * scale).astype(f32)
 
 
+def rms(a):
+    return float(np.sqrt(np.mean(np.asarray(a, np.float64) ** 2)))
+
+
+def grad_scales(q, k, v, go, scale):
+    """Magnitude of the terms each gradient sums: |dS| <= |P| |dP - D| ~ |dO||V|; dQ = scale dS K, dK = scale dS^T Q, dV = P^T dO."""
+    ds = rms(go) * rms(v)
+    return {"dQ": ds * rms(k) * scale, "dK": ds * rms(q) * scale, "dV": rms(go), "O": rms(v), "m": 0.0, "l": 0.0}
+
+
 def run_gpu(hip, q, k, v, go, heads, scale, old_len):
     D, ops = hip.DeviceTensor, hip.ops
     dq_, dk_, dv_, dgo = map(D.fromHost, (q, k, v, go))
@@ -37,8 +47,9 @@ def test_attention_core_matches_the_oracle(hip, oracle, rng, batch, heads, new_l
     o, m, l, dq, dk, dv = run_gpu(hip, q, k, v, go, heads, scale, old_len)
     eo, em, el = oracle.attentionCoreForward(q, k, v, heads, scale, old_len)
     edq, edk, edv = oracle.attentionCoreBackward(go, q, k, v, heads, scale, old_len)
+    sc = grad_scales(q, k, v, go, scale)
     for got, exp, name in ((o, eo, "O"), (m, em, "m"), (l, el, "l"), (dq, edq, "dQ"), (dk, edk, "dK"), (dv, edv, "dV")):
-        assert_close(got, exp, what=f"{name} case {(batch, heads, new_len, old_len, hd)}")
+        assert_close(got, exp, what=f"{name} case {(batch, heads, new_len, old_len, hd)}", scale=sc[name])
 
 
 def test_attention_golden_fixtures(hip):
@@ -48,16 +59,17 @@ def test_attention_golden_fixtures(hip):
         g = {n: gold[f"core{i}_{n}"] for n in "q k v go o m l dq dk dv".split()}
         scale = float(f32(1.0) / np.sqrt(f32(hd)))
         got = run_gpu(hip, g["q"], g["k"], g["v"], g["go"], int(h), scale, int(ol))
-        for a, n in zip(got, "o m l dq dk dv".split()):
-            assert_close(a, g[n], what=f"golden core{i} {n}")
+        sc = grad_scales(g["q"], g["k"], g["v"], g["go"], scale)
+        for a, n, key in zip(got, "o m l dq dk dv".split(), "O m l dQ dK dV".split()):
+            assert_close(a, g[n], what=f"golden core{i} {n}", scale=sc[key])
 
 
 def test_dot_o_do(hip, rng):
     D = hip.DeviceTensor
     for batch, heads, n, hd in ((2, 3, 17, 8), (1, 2, 5, 3), (2, 16, 64, 64)):
         o, g = r(rng, batch, n, heads * hd), r(rng, batch, n, heads * hd)
-        out = D((batch, heads, n))
-        hip.capi.call("bf_hip_attention_dot_o_do", D.fromHost(o).ptr, D.fromHost(g).ptr, out.ptr, batch, heads, n, heads * hd, None)
+        out, do, dg = D((batch, heads, n)), D.fromHost(o), D.fromHost(g)   # keep the inputs alive across the call
+        hip.capi.call("bf_hip_attention_dot_o_do", do.ptr, dg.ptr, out.ptr, batch, heads, n, heads * hd, None)
         exp = (o.astype(np.float64) * g).reshape(batch, n, heads, hd).sum(-1).transpose(0, 2, 1)
         assert_close(out.toHost(), exp, what="D")
 

@@ -77,8 +77,8 @@ def test_bf16_conversion_is_round_to_nearest_even(hip, oracle, rng):
     assert_bits_equal(bits.view(f32), oracle.roundToBf16(x))
     # transposing variant
     m = r(rng, 37, 50)
-    outT = D((50, 37), itemsize=2)
-    hip.capi.call("bf_hip_cvt_f32_bf16_transpose", D.fromHost(m).ptr, outT.ptr, 37, 50, None)
+    outT, dm = D((50, 37), itemsize=2), D.fromHost(m)
+    hip.capi.call("bf_hip_cvt_f32_bf16_transpose", dm.ptr, outT.ptr, 37, 50, None)
     assert_bits_equal((outT.toHost().astype(np.uint32) << 16).view(f32), oracle.roundToBf16(m).T)
 
 
