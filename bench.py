@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X operator backend on the headline workload.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--extras]
+
+Workload (BASELINE.json configs[2], the one the fused-attention TFLOP/s metric is quoted on):
+standalone causal fused attention in fp32, batch 8, heads 16, seq 2048, head_dim 64, Q/K/V/dOut
+i.i.d. N(0,1) from a fixed seed, scale 1/sqrt(64).  One "step" = forward O plus backward dQ, dK, dV
+(bf_hip_attention_forward + bf_hip_attention_backward through the C ABI), inputs resident in HBM.
+
+Prints ONE JSON line.  `value` = algorithmic FLOPs of a step (14*hd*P with P = B*H*S(S+1)/2 causal
+pairs: 4*hd*P forward, 10*hd*P backward, the FlashAttention convention; exp/softmax not counted)
+divided by the measured time per step.  `roofline` describes the dominant kernel (the key-tile-owner
+backward kernel that produces dK and dV), timed live with HIP events on the stream the kernels run on.
+`cpu_baseline` times the CPU reference on a bounded sample of the same workload on this host.
+Everything on one GPU: this build has no multi-GPU path.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
+PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# same command (profiles/attention_c3_*.md says how they were taken and scaled); None until measured.
+MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvKernel": None}
+
+
+def attention_flops(batch, heads, seq, hd):
+    pairs = batch * heads * seq * (seq + 1) // 2
+    return {"fwd": 4 * hd * pairs, "bwd": 10 * hd * pairs, "dkv": 8 * hd * pairs, "dq": 6 * hd * pairs, "pairs": pairs}
+
+
+def time_region(bf, stream, fn, steps, warmup):
+    """Mean milliseconds per call of fn() over `steps` calls, HIP events on `stream`."""
+    for _ in range(warmup):
+        fn()
+    stream.synchronize()
+    start, stop = bf.Event(), bf.Event()
+    start.record(stream)
+    for _ in range(steps):
+        fn()
+    stop.record(stream)
+    stop.synchronize()
+    return start.elapsed_ms(stop) / steps
+
+
+def bench_attention(bf, steps, warmup):
+    D, call = bf.DeviceTensor, bf.capi.call
+    batch, heads, seq, hd = 8, 16, 2048, 64
+    dim, scale = heads * hd, 1.0 / np.sqrt(np.float32(hd))
+    rng = np.random.default_rng(42)
+    gen = lambda: D.fromHost(rng.standard_normal((batch, seq, dim), dtype=np.float32))
+    q, k, v, go = gen(), gen(), gen(), gen()
+    out, dq, dk, dv = D((batch, seq, dim)), D((batch, seq, dim)), D((batch, seq, dim)), D((batch, seq, dim))
+    m, l = D((batch, heads, seq)), D((batch, heads, seq))
+    lse2, dvec = D((batch, heads, seq)), D((batch, heads, seq))
+    stream = bf.Stream()
+    sh = stream.handle
+    dims = (batch, heads, seq, seq, dim, ctypes.c_float(scale), 0, sh)
+
+    fwd = lambda: call("bf_hip_attention_forward", q.ptr, k.ptr, v.ptr, out.ptr, m.ptr, l.ptr, *dims)
+    bwd = lambda: call("bf_hip_attention_backward", go.ptr, q.ptr, k.ptr, v.ptr, out.ptr, m.ptr, l.ptr, dq.ptr, dk.ptr,
+                       dv.ptr, *dims)
+    prep = lambda: call("bf_hip_attention_backward_prepare", out.ptr, go.ptr, m.ptr, l.ptr, lse2.ptr, dvec.ptr, batch,
+                        heads, seq, dim, sh)
+    dkv = lambda: call("bf_hip_attention_backward_dkv", go.ptr, q.ptr, k.ptr, v.ptr, lse2.ptr, dvec.ptr, dk.ptr, dv.ptr,
+                       *dims)
+    dqk = lambda: call("bf_hip_attention_backward_dq", go.ptr, q.ptr, k.ptr, v.ptr, lse2.ptr, dvec.ptr, dq.ptr, *dims)
+
+    def step():
+        fwd()
+        bwd()
+
+    # the timed region of the contract: exactly `steps` steps between two synchronisations
+    for _ in range(warmup):
+        step()
+    stream.synchronize()
+    bf.capi.call("bf_hip_synchronize")
+    t0 = time.perf_counter()
+    start, stop = bf.Event(), bf.Event()
+    start.record(stream)
+    for _ in range(steps):
+        step()
+    stop.record(stream)
+    stop.synchronize()
+    bf.capi.call("bf_hip_synchronize")
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms_step = start.elapsed_ms(stop) / steps
+
+    # per-kernel durations, live, same stream
+    per = {name: time_region(bf, stream, fn, steps, 1) for name, fn in
+           (("forward", fwd), ("prepare", prep), ("dkv", dkv), ("dq", dqk))}
+    fl = attention_flops(batch, heads, seq, hd)
+    return {"ms_per_step": ms_step, "wall_ms_per_step": wall_ms, "kernel_ms": per, "flops": fl,
+            "shape": {"batch": batch, "heads": heads, "seq": seq, "head_dim": hd}}
+
+
+def cpu_baseline_attention(seconds_budget=20.0):
+    """The CPU reference (oracle/_ref, else the restatement) on a sample of (batch, head) slices at full
+    sequence length; slices are independent, so FLOP/s on the sample is FLOP/s on the workload."""
+    from oracle import bfo
+    impl = bfo.reference() or bfo.oracle()
+    kind = "reference" if impl.is_reference else "port"
+    seq, hd = 2048, 64
+    rng = np.random.default_rng(7)
+    mk = lambda: rng.standard_normal((1, seq, hd), dtype=np.float32)
+    q, k, v, go = mk(), mk(), mk(), mk()
+    flops_slice = 14 * hd * (seq * (seq + 1) // 2)
+    done, t0 = 0, time.perf_counter()
+    while True:
+        impl.attentionCoreForward(q, k, v, 1, 0.125, 0)
+        impl.attentionCoreBackward(go, q, k, v, 1, 0.125, 0)
+        done += 1
+        elapsed = time.perf_counter() - t0
+        if elapsed + elapsed / done > seconds_budget or done >= 8:
+            break
+    return {"value": round(flops_slice * done / elapsed / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": kind,
+            "sample": f"{done} of 128 (batch, head) slices of the workload at full seq 2048, head_dim 64, fwd+bwd, "
+                      f"{elapsed:.1f} s on one host core (the reference CPU backend is single-threaded)"}
+
+
+def bench_extras(bf, steps):
+    """Secondary figures: a bandwidth-bound kernel and the bf16 projection GEMM (not part of `value`)."""
+    D, call, ops = bf.DeviceTensor, bf.capi.call, bf.ops
+    stream = bf.Stream()
+    extras = {}
+    n = 4096 * 4096
+    x, y = D.zeros((n,)), D((n,))
+    ms = time_region(bf, stream, lambda: call("bf_hip_act_forward", x.ptr, y.ptr, n, bf.capi.ACT_SILU, stream.handle), steps, 3)
+    extras["silu_4096x4096"] = {"ms": ms, "GB/s": 8 * n / ms / 1e6, "frac_hbm": 8 * n / ms / 1e6 / PEAK_HBM_GBS}
+    mdim = 4096
+    a = D.fromHost(np.random.default_rng(1).standard_normal((mdim, mdim), dtype=np.float32))
+    w = D.fromHost(np.random.default_rng(2).standard_normal((mdim, mdim), dtype=np.float32) / 64)
+    abf, wbf, c = D((mdim, mdim), itemsize=2), D((mdim, mdim), itemsize=2), D((mdim, mdim))
+    call("bf_hip_cvt_f32_bf16", a.ptr, abf.ptr, mdim * mdim, None)
+    call("bf_hip_cvt_f32_bf16_transpose", w.ptr, wbf.ptr, mdim, mdim, None)
+    ms = time_region(bf, stream, lambda: call("bf_hip_gemm_bf16_nt", abf.ptr, wbf.ptr, c.ptr, mdim, mdim, mdim, stream.handle), steps, 3)
+    tf = 2 * mdim ** 3 / ms / 1e9
+    extras["gemm_bf16_4096"] = {"ms": ms, "TFLOP/s": tf, "frac_bf16_mfma": tf / PEAK_BF16_MFMA_TFLOPS}
+    ms = time_region(bf, stream, lambda: call("bf_hip_matmul_bf16", a.ptr, w.ptr, c.ptr, mdim, mdim, mdim, 1, stream.handle), steps, 3)
+    extras["matmul_bf16_4096_fp32_io"] = {"ms": ms, "TFLOP/s": 2 * mdim ** 3 / ms / 1e9}
+    return extras
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--extras", action="store_true", help="also time a bandwidth kernel and the bf16 GEMM")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    import blackforge_amd as bf
+    bf.capi.load()
+    if bf.capi.device_count() < 1:
+        sys.exit("bench.py: no HIP device visible; the operator library has no CPU fallback")
+    props = bf.capi.device_props(0)
+
+    res = bench_attention(bf, args.steps, args.warmup)
+    fl = res["flops"]
+    total_flops = fl["fwd"] + fl["bwd"]
+    value = total_flops / (res["ms_per_step"] * 1e-3) / 1e12
+    dkv_ms = res["kernel_ms"]["dkv"]
+    achieved = fl["dkv"] / (dkv_ms * 1e-3) / 1e12
+    line = {
+        "metric": "fused-attn fwd+bwd TFLOP/s",
+        "value": round(value, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(res["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "causal fused attention fwd+bwd, fp32, batch 8, heads 16, seq 2048, head_dim 64 "
+                               "(BASELINE.json configs[2])", **res["shape"]},
+        "roofline": {"bound": "mfma", "kernel": "attnBackwardDkvKernel<64,64> (dK,dV; key-tile owner)",
+                     "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES["attnBackwardDkvKernel"],
+                     "flops_per_launch": fl["dkv"], "launch_ms": round(dkv_ms, 4)},
+        "frac_of_fp32_mfma_peak": round(value / PEAK_FP32_MFMA_TFLOPS, 4),
+        "kernel_ms": {k: round(v, 4) for k, v in res["kernel_ms"].items()},
+        "kernel_tflops": {"forward": round(fl["fwd"] / res["kernel_ms"]["forward"] / 1e9, 2),
+                          "dkv": round(fl["dkv"] / res["kernel_ms"]["dkv"] / 1e9, 2),
+                          "dq": round(fl["dq"] / res["kernel_ms"]["dq"] / 1e9, 2)},
+        "wall_ms_per_step": round(res["wall_ms_per_step"], 4),
+        "device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units},
+    }
+    if args.extras:
+        line["extras"] = bench_extras(bf, max(5, args.steps // 2))
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_attention()
+        line["cpu_baseline"]["host_cores"] = os.cpu_count()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -92,6 +92,9 @@ SIGNATURES = {
     "bf_hip_attention_dot_o_do": [P, P, P, c_size, c_size, c_size, c_size, S],
     "bf_hip_attention_backward": [P, P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float,
                                   c_size, S],
+    "bf_hip_attention_backward_prepare": [P, P, P, P, P, P, c_size, c_size, c_size, c_size, S],
+    "bf_hip_attention_backward_dkv": [P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
+    "bf_hip_attention_backward_dq": [P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_mse": [P, P, P, P, c_size, c_int, S],
     "bf_hip_cross_entropy": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse": [P, P, P, P, c_size, c_size, c_int, S],

@@ -586,6 +586,64 @@ int bf_hip_attention_dot_o_do(const float* out, const float* dOut, float* D, siz
     return BF_OK;
 }
 
+static int fillParams(AttnParams& p, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
+                      size_t oldLen) {
+    p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(totalLen);
+    p.dim = int(dim); p.hd = int(dim / heads); p.oldLen = int(oldLen); p.scale = scale;
+    return BF_OK;
+}
+
+int bf_hip_attention_backward_prepare(const float* out, const float* dOut, const float* m, const float* l, float* lse2,
+                                      float* D, size_t batch, size_t heads, size_t newLen, size_t dim,
+                                      bf_stream_t stream) {
+    BF_REQUIRE(heads != 0 && dim % heads == 0, "numHeads must divide dim");
+    if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(out && dOut && m && l && lse2 && D, "NULL pointer");
+    const int hd = int(dim / heads);
+    const size_t stats = batch * heads * newLen;
+    const bool vec4 = hd % 4 == 0 && dim % 4 == 0 && ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dOut)) & 15u) == 0;
+    const unsigned grid = gridFor(stats * 16, 256, 1u << 30);
+    hipStream_t s = asStream(stream);
+    if (vec4) attnDotKernel<true><<<grid, 256, 0, s>>>(out, dOut, m, l, D, lse2, int(batch), int(heads), int(newLen), int(dim), hd);
+    else attnDotKernel<false><<<grid, 256, 0, s>>>(out, dOut, m, l, D, lse2, int(batch), int(heads), int(newLen), int(dim), hd);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_attention_backward_dkv(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
+                                  const float* D, float* dK, float* dV, size_t batch, size_t heads, size_t newLen,
+                                  size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
+    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+    if (st != BF_OK) return st;
+    if (batch == 0 || dim == 0 || totalLen == 0) return BF_OK;
+    BF_REQUIRE(dK && dV, "NULL pointer");
+    if (newLen == 0) {   // no query: key/value gradients are zero
+        st = bf_hip_fill_zero(dK, batch * totalLen * dim * sizeof(float), stream);
+        if (st != BF_OK) return st;
+        return bf_hip_fill_zero(dV, batch * totalLen * dim * sizeof(float), stream);
+    }
+    BF_REQUIRE(dOut && q && k && v && lse2 && D, "NULL pointer");
+    AttnParams p{};
+    p.q = q; p.k = k; p.v = v; p.dO = dOut; p.dK = dK; p.dV = dV; p.lse2 = lse2; p.dvec = D;
+    fillParams(p, batch, heads, newLen, totalLen, dim, scale, oldLen);
+    p.numTiles = int((totalLen + 127) / 128);
+    return dispatch<2>(p, vec4Ok(p, {q, k, v, dOut}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
+}
+
+int bf_hip_attention_backward_dq(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
+                                 const float* D, float* dQ, size_t batch, size_t heads, size_t newLen, size_t totalLen,
+                                 size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
+    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+    if (st != BF_OK) return st;
+    if (batch == 0 || dim == 0 || newLen == 0) return BF_OK;
+    BF_REQUIRE(dOut && q && k && v && lse2 && D && dQ, "NULL pointer");
+    AttnParams p{};
+    p.q = q; p.k = k; p.v = v; p.dO = dOut; p.dQ = dQ; p.lse2 = lse2; p.dvec = D;
+    fillParams(p, batch, heads, newLen, totalLen, dim, scale, oldLen);
+    p.numTiles = int((newLen + 127) / 128);
+    return dispatch<1>(p, vec4Ok(p, {q, k, v, dOut, dQ}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
+}
+
 int bf_hip_attention_backward(const float* dOut, const float* q, const float* k, const float* v, const float* out,
                               const float* m, const float* l, float* dQ, float* dK, float* dV, size_t batch,
                               size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
@@ -593,43 +651,17 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
     int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
     if (st != BF_OK) return st;
     if (batch == 0 || dim == 0) return BF_OK;
-    hipStream_t s = asStream(stream);
-    if (newLen == 0) {   // no query: key/value gradients are zero
-        if (totalLen) {
-            BF_REQUIRE(dK && dV, "NULL pointer");
-            st = bf_hip_fill_zero(dK, batch * totalLen * dim * sizeof(float), stream);
-            if (st != BF_OK) return st;
-            return bf_hip_fill_zero(dV, batch * totalLen * dim * sizeof(float), stream);
-        }
-        return BF_OK;
-    }
-    BF_REQUIRE(dOut && q && k && v && out && m && l && dQ && dK && dV, "NULL pointer");
-    AttnParams p{};
-    p.q = q; p.k = k; p.v = v; p.o = out; p.dO = dOut; p.dQ = dQ; p.dK = dK; p.dV = dV;
-    p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(totalLen);
-    p.dim = int(dim); p.hd = int(dim / heads); p.oldLen = int(oldLen); p.scale = scale;
-
     // workspace: lse2 | D, each [batch, heads, newLen]
-    size_t stats = batch * heads * newLen;
+    const size_t stats = batch * heads * newLen;
     Scratch work(2 * stats * sizeof(float));
     if (work.status != BF_OK) return work.status;
     float* lse2 = work.as<float>();
     float* dvec = lse2 + stats;
-    {
-        bool vec4 = p.hd % 4 == 0 && dim % 4 == 0 && ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dOut)) & 15u) == 0;
-        unsigned grid = gridFor(stats * 16, 256, 1u << 30);
-        if (vec4) attnDotKernel<true><<<grid, 256, 0, s>>>(out, dOut, m, l, dvec, lse2, p.batch, p.heads, p.newLen, p.dim, p.hd);
-        else attnDotKernel<false><<<grid, 256, 0, s>>>(out, dOut, m, l, dvec, lse2, p.batch, p.heads, p.newLen, p.dim, p.hd);
-        BF_LAUNCH_CHECK();
-    }
-    p.lse2 = lse2;
-    p.dvec = dvec;
-
-    p.numTiles = int((totalLen + 127) / 128);
-    st = dispatch<2>(p, vec4Ok(p, {q, k, v, dOut}), unsigned(batch * heads * size_t(p.numTiles)), s);
+    st = bf_hip_attention_backward_prepare(out, dOut, m, l, lse2, dvec, batch, heads, newLen, dim, stream);
     if (st != BF_OK) return st;
-    p.numTiles = int((newLen + 127) / 128);
-    return dispatch<1>(p, vec4Ok(p, {q, k, v, dOut, dQ}), unsigned(batch * heads * size_t(p.numTiles)), s);
+    st = bf_hip_attention_backward_dkv(dOut, q, k, v, lse2, dvec, dK, dV, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+    if (st != BF_OK) return st;
+    return bf_hip_attention_backward_dq(dOut, q, k, v, lse2, dvec, dQ, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
 }
 
 }  // extern "C"

@@ -222,6 +222,21 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
                               size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
                               bf_stream_t stream);
 
+/* The three stages of bf_hip_attention_backward, for callers that need only one of the gradients
+ * (frozen keys/values, or a query-only probe) or want to time the stages; same kernels, same results.
+ * prepare: lse2[b,h,i] = m*log2(e) + log2(l) and D[b,h,i] = dot(out, dOut) (computeDKernel plus the
+ * statistics fold); dkv: dK, dV from a key-tile owner; dq: dQ from a query-tile owner
+ * (tiledFusedAttentionBackwardKernel, fused_attention.cu:201-303, split by which gradient is owned). */
+int bf_hip_attention_backward_prepare(const float* out, const float* dOut, const float* m, const float* l, float* lse2,
+                                      float* D, size_t batch, size_t heads, size_t newLen, size_t dim,
+                                      bf_stream_t stream);
+int bf_hip_attention_backward_dkv(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
+                                  const float* D, float* dK, float* dV, size_t batch, size_t heads, size_t newLen,
+                                  size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream);
+int bf_hip_attention_backward_dq(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
+                                 const float* D, float* dQ, size_t batch, size_t heads, size_t newLen, size_t totalLen,
+                                 size_t dim, float scale, size_t oldLen, bf_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Losses                                                      (reference: loss.hpp:20-70, loss.cu)
  * Each writes grad (same shape as the prediction) and the SUM over the batch of the per-row (per-
