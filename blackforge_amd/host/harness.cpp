@@ -1,0 +1,186 @@
+// C entry points over the C++ operator layer (blackforge::backend::hip::Model, losses, optimizers) so
+// that the benchmark and the Python parity tests can drive a whole training step of the C++ host layer.
+// Host-only code: it calls the GPU exclusively through the C ABI of libbf_hip.so.
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "blackforge/backend/hip/loss.hpp"
+#include "blackforge/backend/hip/model.hpp"
+#include "blackforge/backend/hip/optimizer.hpp"
+
+namespace hip = blackforge::backend::hip;
+
+namespace {
+thread_local std::string g_error;
+
+struct Handle {
+    std::unique_ptr<hip::Model> model;
+    std::unique_ptr<hip::AdamW> adamw;
+    std::unique_ptr<hip::SGD> sgd;
+    hip::DeviceTensor output;
+    hip::DeviceTensor lossGrad;
+    hip::DeviceTensor lossAccumulator;
+    std::vector<hip::Parameter*> params;
+};
+
+template <typename Fn>
+int guarded(Fn&& fn) {
+    try {
+        fn();
+        return 0;
+    } catch (const std::invalid_argument& e) {
+        g_error = e.what();
+        return 1;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 2;
+    }
+}
+
+// Non-owning view of caller-owned device memory as a DeviceTensor argument.
+struct Borrowed {
+    hip::DeviceTensor tensor;
+    Borrowed(const float* ptr, std::vector<std::size_t> shape) : tensor(hip::DeviceTensor::borrow(ptr, std::move(shape))) {}
+};
+}  // namespace
+
+extern "C" {
+
+const char* bfh_last_error(void) { return g_error.c_str(); }
+
+// kinds follow hip::LayerKind order: 0 linear, 1 silu, 2 relu, 3 gelu, 4 rmsnorm, 5 softmax, 6 embedding,
+// 7 positional embedding, 8 attention, 9 feedforward (arg1: 0 SiLU, 1 GELU)
+void* bfh_model_create(int numLayers, const int* kinds, const long long* arg0, const long long* arg1, size_t inputFeatures,
+                       int useBf16) {
+    Handle* handle = nullptr;
+    int st = guarded([&] {
+        std::vector<hip::LayerSpec> specs;
+        for (int i = 0; i < numLayers; ++i)
+            specs.push_back(hip::LayerSpec{static_cast<hip::LayerKind>(kinds[i]), static_cast<std::size_t>(arg0[i]),
+                                           static_cast<std::size_t>(arg1 ? arg1[i] : 0)});
+        auto h = std::make_unique<Handle>();
+        h->model = std::make_unique<hip::Model>("harness", specs, inputFeatures, useBf16 != 0);
+        h->params = h->model->parameters();
+        h->lossAccumulator = hip::DeviceTensor::zeros({1});
+        handle = h.release();
+    });
+    return st == 0 ? handle : nullptr;
+}
+
+void bfh_model_destroy(void* h) { delete static_cast<Handle*>(h); }
+
+int bfh_model_num_params(void* h) { return static_cast<int>(static_cast<Handle*>(h)->params.size()); }
+
+int bfh_model_param_info(void* h, int index, char* name, size_t capacity, size_t* count, float** value, float** grad) {
+    Handle* handle = static_cast<Handle*>(h);
+    if (index < 0 || static_cast<size_t>(index) >= handle->params.size()) return 1;
+    hip::Parameter* p = handle->params[static_cast<size_t>(index)];
+    if (name && capacity) {
+        std::strncpy(name, p->name.c_str(), capacity - 1);
+        name[capacity - 1] = '\0';
+    }
+    if (count) *count = p->value.elementCount();
+    if (value) *value = p->value.data();
+    if (grad) *grad = p->grad.data();
+    return 0;
+}
+
+// input: device pointer to [shape...] floats (token ids or features).
+int bfh_model_forward(void* h, const float* input, int rank, const size_t* shape, int trusted, float** output, size_t* outCount) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
+        handle->output = handle->model->forward(in.tensor, trusted != 0);
+        if (output) *output = handle->output.data();
+        if (outCount) *outCount = handle->output.elementCount();
+    });
+}
+
+// lossKind 0: sparse cross-entropy (targets = one class index per output row), 1: mean squared error.
+// The loss sum is accumulated on the device; bfh_model_read_loss reads and resets it.
+int bfh_model_loss(void* h, const float* target, int lossKind) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        if (lossKind == 0) {
+            std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
+            Borrowed tgt(target, {rows});
+            handle->lossGrad = hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
+        } else {
+            Borrowed tgt(target, handle->output.shape());
+            handle->lossGrad = hip::meanSquaredErrorAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
+        }
+    });
+}
+
+int bfh_model_loss_grad(void* h, float** grad, size_t* count) {
+    Handle* handle = static_cast<Handle*>(h);
+    if (grad) *grad = handle->lossGrad.data();
+    if (count) *count = handle->lossGrad.elementCount();
+    return 0;
+}
+
+int bfh_model_backward(void* h, int trusted) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] { handle->model->backward(handle->lossGrad, trusted != 0); });
+}
+
+int bfh_model_zero_grad(void* h) {
+    return guarded([&] { static_cast<Handle*>(h)->model->zeroGrad(); });
+}
+
+int bfh_model_adamw_step(void* h, float lr, float beta1, float beta2, float eps, float weightDecay) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        if (!handle->adamw) handle->adamw = std::make_unique<hip::AdamW>(lr, beta1, beta2, eps, weightDecay);
+        handle->adamw->setLearningRate(lr);
+        handle->adamw->step(handle->params);
+    });
+}
+
+int bfh_model_sgd_step(void* h, float lr) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        if (!handle->sgd) handle->sgd = std::make_unique<hip::SGD>(lr);
+        handle->sgd->setLearningRate(lr);
+        handle->sgd->step(handle->params);
+    });
+}
+
+// One whole training step with no host synchronisation: zeroGrad, forward, loss (accumulated on the
+// device), backward, optimizer (0 none, 1 AdamW with the reference defaults and the given lr).
+int bfh_model_train_step(void* h, const float* input, int rank, const size_t* shape, const float* target, int lossKind,
+                         int optimizer, float lr) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        handle->model->zeroGrad();
+        Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
+        handle->output = handle->model->forward(in.tensor, true);
+        if (lossKind == 0) {
+            std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
+            Borrowed tgt(target, {rows});
+            handle->lossGrad = hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
+        } else {
+            Borrowed tgt(target, handle->output.shape());
+            handle->lossGrad = hip::meanSquaredErrorAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
+        }
+        handle->model->backward(handle->lossGrad, true);
+        if (optimizer == 1) {
+            if (!handle->adamw) handle->adamw = std::make_unique<hip::AdamW>(lr, 0.9F, 0.999F, 1e-8F, 0.01F);
+            handle->adamw->setLearningRate(lr);
+            handle->adamw->step(handle->params);
+        }
+    });
+}
+
+// Reads the accumulated loss sum (one device->host copy) and resets the accumulator.
+int bfh_model_read_loss(void* h, float* sum) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        hip::check(bf_hip_memcpy_d2h(sum, handle->lossAccumulator.data(), sizeof(float)));
+        hip::check(bf_hip_fill_zero(handle->lossAccumulator.data(), sizeof(float), nullptr));
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,131 @@
+"""ctypes binding of blackforge_amd/lib/libbf_hip_host.so: C entry points over the C++ operator layer
+(blackforge::backend::hip::Model and friends, include/blackforge/backend/hip/).  Used by the benchmark and
+the parity tests to run whole training steps of the C++ host layer."""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import List, Sequence, Tuple
+
+import numpy as np
+
+from . import capi
+from .tensor import DeviceTensor
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libbf_hip_host.so")
+
+LINEAR, SILU, RELU, GELU, RMSNORM, SOFTMAX, EMBEDDING, POSITIONAL, ATTENTION, FEEDFORWARD = range(10)
+LOSS_SPARSE_CE, LOSS_MSE = 0, 1
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        capi.load()
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: run `make -C blackforge_amd/host` after building libbf_hip.so")
+        lib = ctypes.CDLL(LIB_PATH)
+        lib.bfh_last_error.restype = ctypes.c_char_p
+        lib.bfh_model_create.restype = ctypes.c_void_p
+        lib.bfh_model_create.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_longlong),
+                                         ctypes.POINTER(ctypes.c_longlong), ctypes.c_size_t, ctypes.c_int]
+        lib.bfh_model_destroy.argtypes = [ctypes.c_void_p]
+        lib.bfh_model_num_params.argtypes = [ctypes.c_void_p]
+        lib.bfh_model_param_info.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t,
+                                             ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_void_p),
+                                             ctypes.POINTER(ctypes.c_void_p)]
+        lib.bfh_model_forward.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_size_t),
+                                          ctypes.c_int, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_size_t)]
+        lib.bfh_model_loss.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+        lib.bfh_model_loss_grad.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_size_t)]
+        lib.bfh_model_backward.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        lib.bfh_model_zero_grad.argtypes = [ctypes.c_void_p]
+        lib.bfh_model_adamw_step.argtypes = [ctypes.c_void_p] + [ctypes.c_float] * 5
+        lib.bfh_model_sgd_step.argtypes = [ctypes.c_void_p, ctypes.c_float]
+        lib.bfh_model_train_step.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_size_t),
+                                             ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float]
+        lib.bfh_model_read_loss.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
+        _lib = lib
+    return _lib
+
+
+def _check(status: int):
+    if status == 0:
+        return
+    message = load().bfh_last_error().decode(errors="replace")
+    raise ValueError(message) if status == 1 else RuntimeError(message)
+
+
+class HostModel:
+    """A blackforge::backend::hip::Model built from ``(kind, arg0, arg1)`` layer tuples."""
+
+    def __init__(self, layers: Sequence[Tuple[int, ...]], input_features: int = 0, use_bf16: bool = False):
+        lib = load()
+        n = len(layers)
+        kinds = (ctypes.c_int * n)(*[l[0] for l in layers])
+        a0 = (ctypes.c_longlong * n)(*[(l[1] if len(l) > 1 else 0) for l in layers])
+        a1 = (ctypes.c_longlong * n)(*[(l[2] if len(l) > 2 else 0) for l in layers])
+        self.handle = ctypes.c_void_p(lib.bfh_model_create(n, kinds, a0, a1, input_features, int(use_bf16)))
+        if not self.handle:
+            _check(1)
+        self.names: List[str] = []
+        self.counts: List[int] = []
+        self._value_ptrs, self._grad_ptrs = [], []
+        for i in range(lib.bfh_model_num_params(self.handle)):
+            name = ctypes.create_string_buffer(96)
+            count, vp, gp = ctypes.c_size_t(), ctypes.c_void_p(), ctypes.c_void_p()
+            lib.bfh_model_param_info(self.handle, i, name, 96, ctypes.byref(count), ctypes.byref(vp), ctypes.byref(gp))
+            self.names.append(name.value.decode())
+            self.counts.append(count.value)
+            self._value_ptrs.append(vp)
+            self._grad_ptrs.append(gp)
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            load().bfh_model_destroy(self.handle)
+            self.handle = None
+
+    def set_value(self, i: int, host) -> None:
+        host = np.ascontiguousarray(host, np.float32).reshape(-1)
+        assert host.size == self.counts[i]
+        capi.call("bf_hip_memcpy_h2d", self._value_ptrs[i], host.ctypes.data_as(ctypes.c_void_p), host.nbytes)
+
+    def _read(self, ptr, count) -> np.ndarray:
+        out = np.empty(count, np.float32)
+        capi.call("bf_hip_memcpy_d2h", out.ctypes.data_as(ctypes.c_void_p), ptr, out.nbytes)
+        return out
+
+    def value(self, i: int) -> np.ndarray:
+        return self._read(self._value_ptrs[i], self.counts[i])
+
+    def grad(self, i: int) -> np.ndarray:
+        return self._read(self._grad_ptrs[i], self.counts[i])
+
+    def forward(self, x: DeviceTensor, trusted: bool = False) -> np.ndarray:
+        shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
+        out, count = ctypes.c_void_p(), ctypes.c_size_t()
+        _check(load().bfh_model_forward(self.handle, x.ptr, len(x.shape), shape, int(trusted), ctypes.byref(out), ctypes.byref(count)))
+        return self._read(out, count.value)
+
+    def loss(self, target: DeviceTensor, kind: int = LOSS_SPARSE_CE) -> None:
+        _check(load().bfh_model_loss(self.handle, target.ptr, kind))
+
+    def backward(self, trusted: bool = False) -> None:
+        _check(load().bfh_model_backward(self.handle, int(trusted)))
+
+    def zeroGrad(self) -> None:
+        _check(load().bfh_model_zero_grad(self.handle))
+
+    def adamwStep(self, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01) -> None:
+        _check(load().bfh_model_adamw_step(self.handle, lr, beta1, beta2, eps, wd))
+
+    def trainStep(self, x: DeviceTensor, target: DeviceTensor, loss_kind: int = LOSS_SPARSE_CE, optimizer: int = 1, lr: float = 1e-3):
+        shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
+        _check(load().bfh_model_train_step(self.handle, x.ptr, len(x.shape), shape, target.ptr, loss_kind, optimizer, lr))
+
+    def readLossSum(self) -> float:
+        v = ctypes.c_float()
+        _check(load().bfh_model_read_loss(self.handle, ctypes.byref(v)))
+        return v.value

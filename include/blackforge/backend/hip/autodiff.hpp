@@ -1,0 +1,260 @@
+#pragma once
+// Backward operators with the reference's signatures (include/blackforge/backend/cuda/autodiff.hpp:18-177).
+#include <cmath>
+#include <cstddef>
+#include <utility>
+
+#include "blackforge/backend/hip/device_tensor.hpp"
+#include "blackforge/backend/hip/ops.hpp"
+
+namespace blackforge::backend::hip {
+
+struct MatmulGrad {
+    DeviceTensor dA;
+    DeviceTensor dB;
+};
+
+namespace detail {
+inline void requireMatmulBackward(const char* op, const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& g) {
+    require(a.rank() == 2 && b.rank() == 2 && g.rank() == 2 && a.dim(1) == b.dim(0) && g.dim(0) == a.dim(0) &&
+                g.dim(1) == b.dim(1),
+            std::string(op) + ": incompatible shapes on the device");
+}
+// Gradients of c = a(as [m,k]) * b[k,n] given g (as [m,n]); mode as in detail::projection.
+inline MatmulGrad projectionBackward(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& g, int mode,
+                                     std::vector<std::size_t> dAShape) {
+    std::size_t m = rowsOf(a), k = lastDim(a), n = b.dim(1);
+    MatmulGrad r{DeviceTensor(std::move(dAShape)), DeviceTensor({k, n})};
+    if (mode == 0) {
+        check(bf_hip_gemm_f32(0, 1, g.data(), b.data(), r.dA.data(), m, k, n, nullptr));   // dA = g b^T
+        check(bf_hip_gemm_f32(1, 0, a.data(), g.data(), r.dB.data(), k, n, m, nullptr));   // dB = a^T g
+    } else {
+        check(bf_hip_matmul_bf16_backward(a.data(), b.data(), g.data(), r.dA.data(), r.dB.data(), m, k, n, mode == 2, nullptr));
+    }
+    return r;
+}
+}  // namespace detail
+
+inline MatmulGrad matmulBackward(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& gradOutput) {
+    detail::requireMatmulBackward("matmulBackward", a, b, gradOutput);
+    return detail::projectionBackward(a, b, gradOutput, 0, a.shape());
+}
+inline MatmulGrad matmulBf16Backward(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& gradOutput) {
+    detail::requireMatmulBackward("matmulBf16Backward", a, b, gradOutput);
+    return detail::projectionBackward(a, b, gradOutput, 1, a.shape());
+}
+inline MatmulGrad matmulBf16BackwardCachedWeight(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& gradOutput) {
+    detail::requireMatmulBackward("matmulBf16BackwardCachedWeight", a, b, gradOutput);
+    return detail::projectionBackward(a, b, gradOutput, 2, a.shape());
+}
+
+struct MatmulTransposeBGrad {
+    DeviceTensor dA;
+    DeviceTensor dB;
+};
+
+// Forward was a:[m,k], b:[n,k] -> a b^T:[m,n].
+inline MatmulTransposeBGrad matmulTransposeBBackward(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& gradOutput) {
+    require(a.rank() == 2 && b.rank() == 2 && gradOutput.rank() == 2 && a.dim(1) == b.dim(1) && gradOutput.dim(0) == a.dim(0) &&
+                gradOutput.dim(1) == b.dim(0),
+            "matmulTransposeBBackward: incompatible shapes on the device");
+    std::size_t m = a.dim(0), k = a.dim(1), n = b.dim(0);
+    MatmulTransposeBGrad r{DeviceTensor({m, k}), DeviceTensor({n, k})};
+    check(bf_hip_gemm_f32(0, 0, gradOutput.data(), b.data(), r.dA.data(), m, k, n, nullptr));   // dA = g b
+    check(bf_hip_gemm_f32(1, 0, gradOutput.data(), a.data(), r.dB.data(), n, k, m, nullptr));   // dB = g^T a
+    return r;
+}
+
+struct AddBiasGrad {
+    DeviceTensor dInput;
+    DeviceTensor dBias;
+};
+
+inline DeviceTensor biasGradientOnly(const DeviceTensor& gradOutput) {
+    require(gradOutput.rank() >= 2, "biasGradientOnly: needs a gradient of rank >= 2 on the device");
+    DeviceTensor dBias({detail::lastDim(gradOutput)});
+    check(bf_hip_bias_grad(gradOutput.data(), dBias.data(), detail::rowsOf(gradOutput), detail::lastDim(gradOutput), nullptr));
+    return dBias;
+}
+
+inline AddBiasGrad addBiasBackward(const DeviceTensor& gradOutput) {
+    require(gradOutput.rank() >= 2, "addBiasBackward: needs a gradient of rank >= 2 on the device");
+    return AddBiasGrad{gradOutput.clone(), biasGradientOnly(gradOutput)};
+}
+
+struct AddBiasSiluGrad {
+    DeviceTensor dGemmOutput;
+    DeviceTensor dBias;
+};
+
+inline AddBiasSiluGrad addBiasActivationBackward(const DeviceTensor& gemmOutput, const DeviceTensor& bias,
+                                                  const DeviceTensor& dHidden, Activation act) {
+    require(gemmOutput.shape() == dHidden.shape() && bias.rank() == 1 && detail::lastDim(gemmOutput) == bias.dim(0),
+            "addBiasSiluBackward: incompatible shapes on the device");
+    AddBiasSiluGrad r{DeviceTensor(gemmOutput.shape()), DeviceTensor({bias.dim(0)})};
+    check(bf_hip_add_bias_act_backward(gemmOutput.data(), bias.data(), dHidden.data(), r.dGemmOutput.data(), r.dBias.data(),
+                                       detail::rowsOf(gemmOutput), bias.dim(0), static_cast<int>(act), nullptr));
+    return r;
+}
+inline AddBiasSiluGrad addBiasSiluBackward(const DeviceTensor& gemmOutput, const DeviceTensor& bias, const DeviceTensor& dHidden) {
+    return addBiasActivationBackward(gemmOutput, bias, dHidden, Activation::Silu);
+}
+
+inline DeviceTensor activationBackward(const char* op, const DeviceTensor& input, const DeviceTensor& gradOutput, Activation act) {
+    require(input.shape() == gradOutput.shape(), std::string(op) + ": incompatible shapes on the device");
+    DeviceTensor out(input.shape());
+    check(bf_hip_act_backward(input.data(), gradOutput.data(), out.data(), input.elementCount(), static_cast<int>(act), nullptr));
+    return out;
+}
+inline DeviceTensor siluBackward(const DeviceTensor& input, const DeviceTensor& gradOutput) {
+    return activationBackward("siluBackward", input, gradOutput, Activation::Silu);
+}
+inline DeviceTensor reluBackward(const DeviceTensor& input, const DeviceTensor& gradOutput) {
+    return activationBackward("reluBackward", input, gradOutput, Activation::Relu);
+}
+inline DeviceTensor geluBackward(const DeviceTensor& input, const DeviceTensor& gradOutput) {
+    return activationBackward("geluBackward", input, gradOutput, Activation::Gelu);
+}
+
+inline DeviceTensor rmsnormBackward(const DeviceTensor& input, const DeviceTensor& gradOutput) {
+    require(input.shape() == gradOutput.shape(), "rmsnormBackward: incompatible shapes on the device");
+    require(input.rank() >= 2, "rmsnormBackward: needs a tensor of rank >= 2 on the device");
+    DeviceTensor out(input.shape());
+    check(bf_hip_rmsnorm_backward(input.data(), gradOutput.data(), out.data(), detail::rowsOf(input), detail::lastDim(input), nullptr));
+    return out;
+}
+
+inline DeviceTensor softmaxBackward(const DeviceTensor& input, const DeviceTensor& gradOutput) {
+    require(input.shape() == gradOutput.shape(), "softmaxBackward: incompatible shapes on the device");
+    require(input.rank() >= 2, "softmaxBackward: needs a tensor of rank >= 2 on the device");
+    DeviceTensor out(input.shape());
+    check(bf_hip_softmax_backward(input.data(), gradOutput.data(), out.data(), detail::rowsOf(input), detail::lastDim(input), nullptr));
+    return out;
+}
+
+inline DeviceTensor embeddingLookupBackwardPreValidated(const DeviceTensor& tokenIds, const DeviceTensor& gradOutput,
+                                                         std::size_t vocabSize) {
+    require(tokenIds.rank() == 2 && gradOutput.rank() == 3 && tokenIds.dim(0) == gradOutput.dim(0) &&
+                tokenIds.dim(1) == gradOutput.dim(1),
+            "embeddingLookupBackward: incompatible shapes on the device");
+    DeviceTensor dTable({vocabSize, gradOutput.dim(2)});
+    check(bf_hip_embedding_backward(tokenIds.data(), gradOutput.data(), dTable.data(), tokenIds.elementCount(), vocabSize,
+                                    gradOutput.dim(2), nullptr));
+    return dTable;
+}
+
+inline DeviceTensor embeddingLookupBackward(const DeviceTensor& tokenIds, const DeviceTensor& gradOutput, std::size_t vocabSize) {
+    require(tokenIds.rank() == 2 && gradOutput.rank() == 3 && tokenIds.dim(0) == gradOutput.dim(0) &&
+                tokenIds.dim(1) == gradOutput.dim(1),
+            "embeddingLookupBackward: incompatible shapes on the device");
+    detail::requireIdsInRange("embeddingLookupBackward", tokenIds, vocabSize, "token id");
+    return embeddingLookupBackwardPreValidated(tokenIds, gradOutput, vocabSize);
+}
+
+struct PositionalEmbeddingGrad {
+    DeviceTensor dInput;
+    DeviceTensor dTable;
+};
+
+inline PositionalEmbeddingGrad addPositionalEmbeddingBackward(const DeviceTensor& gradOutput, std::size_t maxSeqLen) {
+    require(gradOutput.rank() == 3, "addPositionalEmbeddingBackward: needs a gradient of rank 3 on the device");
+    PositionalEmbeddingGrad r{DeviceTensor(), DeviceTensor({maxSeqLen, gradOutput.dim(2)})};
+    check(bf_hip_positional_backward(gradOutput.data(), r.dTable.data(), gradOutput.dim(0), gradOutput.dim(1), gradOutput.dim(2),
+                                     maxSeqLen, nullptr));
+    r.dInput = gradOutput.clone();
+    return r;
+}
+
+struct FeedForwardGrad {
+    DeviceTensor dInput, dW1, dB1, dW2, dB2;
+};
+
+inline FeedForwardGrad feedForwardBackwardCached(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
+                                                  const DeviceTensor& w2, const DeviceTensor& b2, const FeedForwardCache& cache,
+                                                  const DeviceTensor& gradOutput, bool useBf16, Activation act = Activation::Silu) {
+    (void)b2;
+    require(gradOutput.shape() == input.shape(), "feedForwardBackward: gradient shape differs from the input");
+    const int mode = useBf16 ? 2 : 0;
+    DeviceTensor dB2 = biasGradientOnly(gradOutput);
+    MatmulGrad g2 = detail::projectionBackward(cache.hidden, w2, gradOutput, mode, cache.hidden.shape());
+    AddBiasSiluGrad hiddenGrad = addBiasActivationBackward(cache.gemm1, b1, g2.dA, act);
+    MatmulGrad g1 = detail::projectionBackward(cache.normed, w1, hiddenGrad.dGemmOutput, mode, cache.normed.shape());
+    DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, g1.dA));
+    return FeedForwardGrad{std::move(dInput), std::move(g1.dB), std::move(hiddenGrad.dBias), std::move(g2.dB), std::move(dB2)};
+}
+
+namespace detail {
+// Stateless variant: recomputes the forward first (reference: autodiff.cu:624-652).
+inline FeedForwardGrad feedForwardBackwardImpl(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
+                                               const DeviceTensor& w2, const DeviceTensor& b2, const DeviceTensor& gradOutput,
+                                               int mode, Activation act) {
+    FeedForwardCache cache;
+    cache.normed = rmsnorm(input);
+    cache.gemm1 = projection(cache.normed, w1, mode, withLastDim(input, w1.dim(1)));
+    cache.hidden = addBiasActivation(cache.gemm1, b1, act);
+    DeviceTensor dB2 = biasGradientOnly(gradOutput);
+    MatmulGrad g2 = projectionBackward(cache.hidden, w2, gradOutput, mode, cache.hidden.shape());
+    AddBiasSiluGrad hiddenGrad = addBiasActivationBackward(cache.gemm1, b1, g2.dA, act);
+    MatmulGrad g1 = projectionBackward(cache.normed, w1, hiddenGrad.dGemmOutput, mode, cache.normed.shape());
+    DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, g1.dA));
+    (void)b2;
+    return FeedForwardGrad{std::move(dInput), std::move(g1.dB), std::move(hiddenGrad.dBias), std::move(g2.dB), std::move(dB2)};
+}
+}  // namespace detail
+
+inline FeedForwardGrad feedForwardBackward(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
+                                            const DeviceTensor& w2, const DeviceTensor& b2, const DeviceTensor& gradOutput,
+                                            Activation act = Activation::Silu) {
+    return detail::feedForwardBackwardImpl(input, w1, b1, w2, b2, gradOutput, 0, act);
+}
+inline FeedForwardGrad feedForwardBf16Backward(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
+                                                const DeviceTensor& w2, const DeviceTensor& b2, const DeviceTensor& gradOutput,
+                                                Activation act = Activation::Silu) {
+    return detail::feedForwardBackwardImpl(input, w1, b1, w2, b2, gradOutput, 1, act);
+}
+
+struct SelfAttentionGrad {
+    DeviceTensor dInput, dWq, dWk, dWv, dWout;
+};
+
+namespace detail {
+inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                        const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                        const SelfAttentionCache& cache, const DeviceTensor& gradOutput, int mode) {
+    require(gradOutput.shape() == input.shape(), "selfAttentionBackward: gradient shape differs from the input");
+    std::size_t batch = input.dim(0), seq = input.dim(1), dim = input.dim(2);
+    float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
+    MatmulGrad outGrad = projectionBackward(cache.attnOutput, wout, gradOutput, mode, {batch, seq, dim});
+    FusedAttentionGrad attn = fusedAttentionBackward(outGrad.dA, cache.q, cache.k, cache.v, cache.attnOutput, cache.attnM,
+                                                      cache.attnL, numHeads, scaleFactor, 0);
+    MatmulGrad gq = projectionBackward(cache.normedFlat, wq, attn.dQ, mode, {batch * seq, dim});
+    MatmulGrad gk = projectionBackward(cache.normedFlat, wk, attn.dK, mode, {batch * seq, dim});
+    MatmulGrad gv = projectionBackward(cache.normedFlat, wv, attn.dV, mode, {batch * seq, dim});
+    DeviceTensor dNormed = add(add(gq.dA, gk.dA), gv.dA).reshaped({batch, seq, dim});
+    DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, dNormed));
+    return SelfAttentionGrad{std::move(dInput), std::move(gq.dB), std::move(gk.dB), std::move(gv.dB), std::move(outGrad.dB)};
+}
+}  // namespace detail
+
+inline SelfAttentionGrad selfAttentionBackwardCached(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                      const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                      const SelfAttentionCache& cache, const DeviceTensor& gradOutput, bool useBf16) {
+    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, useBf16 ? 2 : 0);
+}
+// Stateless variants: recompute the forward first (reference: autodiff.cu:654-700).
+inline SelfAttentionGrad selfAttentionBackward(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                const DeviceTensor& gradOutput) {
+    SelfAttentionCache cache;
+    detail::selfAttentionForwardImpl("selfAttentionBackward", input, wq, wk, wv, wout, numHeads, 0, cache);
+    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, 0);
+}
+inline SelfAttentionGrad selfAttentionBf16Backward(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                    const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                    const DeviceTensor& gradOutput) {
+    SelfAttentionCache cache;
+    detail::selfAttentionForwardImpl("selfAttentionBf16Backward", input, wq, wk, wv, wout, numHeads, 1, cache);
+    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, 1);
+}
+
+}  // namespace blackforge::backend::hip

@@ -1,0 +1,91 @@
+#pragma once
+// Loss functions with the reference's signatures (include/blackforge/backend/cuda/loss.hpp:7-70).
+#include <cstddef>
+
+#include "blackforge/backend/hip/device_tensor.hpp"
+#include "blackforge/backend/hip/ops.hpp"
+
+namespace blackforge::backend::hip {
+
+struct LossResult {
+    float value;
+    DeviceTensor grad;  // dL/dprediction, same shape as the prediction
+};
+
+namespace detail {
+inline float readScalar(const DeviceTensor& t) {
+    float v = 0.0F;
+    check(bf_hip_memcpy_d2h(&v, t.data(), sizeof(float)));
+    return v;
+}
+inline void requireDense(const char* op, const DeviceTensor& logits, const DeviceTensor& target) {
+    require(logits.shape() == target.shape(), std::string(op) + ": incompatible shapes on the device");
+    require(logits.rank() >= 2, std::string(op) + ": needs a tensor of rank >= 2 on the device");
+}
+inline void requireSparse(const char* op, const DeviceTensor& logits, const DeviceTensor& idx) {
+    require(logits.rank() >= 2, std::string(op) + ": needs logits of rank >= 2 on the device");
+    require(idx.elementCount() == rowsOf(logits), std::string(op) + ": targetIndices does not have one entry per logits row");
+}
+}  // namespace detail
+
+inline LossResult meanSquaredError(const DeviceTensor& prediction, const DeviceTensor& target) {
+    require(prediction.shape() == target.shape(), "meanSquaredError: incompatible shapes on the device");
+    std::size_t n = prediction.elementCount();
+    LossResult r{0.0F, DeviceTensor(prediction.shape())};
+    DeviceTensor sum({1});
+    check(bf_hip_mse(prediction.data(), target.data(), r.grad.data(), sum.data(), n, 0, nullptr));
+    if (n > 0) r.value = detail::readScalar(sum) / static_cast<float>(n);
+    return r;
+}
+
+inline LossResult softmaxCrossEntropy(const DeviceTensor& logits, const DeviceTensor& target) {
+    detail::requireDense("softmaxCrossEntropy", logits, target);
+    std::size_t rows = detail::rowsOf(logits);
+    LossResult r{0.0F, DeviceTensor(logits.shape())};
+    DeviceTensor sum({1});
+    check(bf_hip_cross_entropy(logits.data(), target.data(), r.grad.data(), sum.data(), rows, detail::lastDim(logits), 0, nullptr));
+    if (rows > 0) r.value = detail::readScalar(sum) / static_cast<float>(rows);
+    return r;
+}
+
+inline LossResult softmaxCrossEntropySparse(const DeviceTensor& logits, const DeviceTensor& targetIndices) {
+    detail::requireSparse("softmaxCrossEntropySparse", logits, targetIndices);
+    std::size_t rows = detail::rowsOf(logits), classes = detail::lastDim(logits);
+    if (rows > 0) detail::requireIdsInRange("softmaxCrossEntropySparse", targetIndices, classes, "class index");
+    LossResult r{0.0F, DeviceTensor(logits.shape())};
+    DeviceTensor sum({1});
+    check(bf_hip_cross_entropy_sparse(logits.data(), targetIndices.data(), r.grad.data(), sum.data(), rows, classes, 0, nullptr));
+    if (rows > 0) r.value = detail::readScalar(sum) / static_cast<float>(rows);
+    return r;
+}
+
+// "Accumulate" variants for the training loop: the gradient is returned, the SUM of this call's per-row
+// (per-element for MSE) losses is added on the device to lossAccumulator (one element, owned by the
+// caller); nothing is read back to the host.
+inline DeviceTensor meanSquaredErrorAccumulate(const DeviceTensor& prediction, const DeviceTensor& target, DeviceTensor& lossAccumulator) {
+    require(prediction.shape() == target.shape(), "meanSquaredErrorAccumulate: incompatible shapes on the device");
+    DeviceTensor grad(prediction.shape());
+    check(bf_hip_mse(prediction.data(), target.data(), grad.data(), lossAccumulator.data(), prediction.elementCount(), 1, nullptr));
+    return grad;
+}
+
+inline DeviceTensor softmaxCrossEntropyAccumulate(const DeviceTensor& logits, const DeviceTensor& target, DeviceTensor& lossAccumulator) {
+    detail::requireDense("softmaxCrossEntropyAccumulate", logits, target);
+    DeviceTensor grad(logits.shape());
+    check(bf_hip_cross_entropy(logits.data(), target.data(), grad.data(), lossAccumulator.data(), detail::rowsOf(logits),
+                               detail::lastDim(logits), 1, nullptr));
+    return grad;
+}
+
+// PRECONDITION (caller's responsibility): every index already lies in [0, classes); no range check and no
+// host round trip happen here.
+inline DeviceTensor softmaxCrossEntropySparseAccumulate(const DeviceTensor& logits, const DeviceTensor& targetIndices,
+                                                         DeviceTensor& lossAccumulator) {
+    detail::requireSparse("softmaxCrossEntropySparseAccumulate", logits, targetIndices);
+    DeviceTensor grad(logits.shape());
+    check(bf_hip_cross_entropy_sparse(logits.data(), targetIndices.data(), grad.data(), lossAccumulator.data(),
+                                      detail::rowsOf(logits), detail::lastDim(logits), 1, nullptr));
+    return grad;
+}
+
+}  // namespace blackforge::backend::hip

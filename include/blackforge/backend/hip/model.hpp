@@ -1,0 +1,352 @@
+#pragma once
+// Trainable pipeline on the GPU with the reference's Model interface
+// (include/blackforge/backend/cuda/model.hpp:48-159; forward/backward src/backend/cuda/model.cu:252-383).
+//
+// A model is a list of layers; each layer kind corresponds to one ir::OpKind of the reference.  Inside a
+// BlackForge build the constructor taking ir::ModelIR is available as well and initialises the weights
+// from the project's own deterministic generator, exactly like the reference backends do.
+#include <cstddef>
+#include <optional>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "blackforge/backend/hip/autodiff.hpp"
+#include "blackforge/backend/hip/device_tensor.hpp"
+#include "blackforge/backend/hip/ops.hpp"
+
+#if __has_include("blackforge/ir/module.hpp") && __has_include("blackforge/backend/cpu/random_init.hpp")
+#include "blackforge/backend/cpu/random_init.hpp"
+#include "blackforge/ir/module.hpp"
+#define BLACKFORGE_HIP_HAS_IR 1
+#endif
+
+namespace blackforge::backend::hip {
+
+struct Parameter {
+    std::string name;
+    DeviceTensor value;
+    DeviceTensor grad;
+};
+
+enum class LayerKind { Linear, Silu, Relu, Gelu, RmsNorm, Softmax, Embedding, PositionalEmbedding, Attention, FeedForward };
+
+struct LayerSpec {
+    LayerKind kind;
+    std::size_t arg0 = 0;  // Linear: out features; Embedding: vocab; PositionalEmbedding: maxSeqLen; Attention: heads; FeedForward: hidden
+    std::size_t arg1 = 0;  // Embedding: dim; FeedForward: activation (0 SiLU = reference, 1 GELU)
+};
+
+class Model {
+public:
+    // inputFeatures: last dimension of the input (ignored when the first layer is an embedding).
+    // Parameters start at zero; assign values through parameters().  useBf16 selects bf16 MFMA projections
+    // (precision.compute == BF16 in the reference, model.cu:139-140).
+    Model(std::string name, const std::vector<LayerSpec>& layers, std::size_t inputFeatures, bool useBf16)
+        : name_(std::move(name)), useBf16_(useBf16) {
+        std::size_t features = inputFeatures;
+        std::size_t valueId = 0;
+        for (const LayerSpec& spec : layers) {
+            ++valueId;  // the model input is value 0; layer i writes value i+1 (names follow the reference)
+            LayerState layer;
+            layer.spec = spec;
+            const std::string id = std::to_string(valueId);
+            switch (spec.kind) {
+                case LayerKind::Linear:
+                    layer.params.push_back(makeParameter("linear" + id + ".weight", {features, spec.arg0}));
+                    layer.params.push_back(makeParameter("linear" + id + ".bias", {spec.arg0}));
+                    features = spec.arg0;
+                    break;
+                case LayerKind::Embedding:
+                    layer.params.push_back(makeParameter("embedding" + id + ".table", {spec.arg0, spec.arg1}));
+                    features = spec.arg1;
+                    break;
+                case LayerKind::PositionalEmbedding:
+                    layer.params.push_back(makeParameter("positional_embedding" + id + ".table", {spec.arg0, features}));
+                    break;
+                case LayerKind::Attention:
+                    require(spec.arg0 != 0 && features % spec.arg0 == 0,
+                            "hip::Model: 'attention#" + id + "' needs " + std::to_string(spec.arg0) + " heads to divide dim=" +
+                                std::to_string(features));
+                    for (const char* w : {".wq", ".wk", ".wv", ".wout"})
+                        layer.params.push_back(makeParameter("attention" + id + w, {features, features}));
+                    break;
+                case LayerKind::FeedForward:
+                    layer.params.push_back(makeParameter("feedforward" + id + ".w1", {features, spec.arg0}));
+                    layer.params.push_back(makeParameter("feedforward" + id + ".b1", {spec.arg0}));
+                    layer.params.push_back(makeParameter("feedforward" + id + ".w2", {spec.arg0, features}));
+                    layer.params.push_back(makeParameter("feedforward" + id + ".b2", {features}));
+                    break;
+                default:
+                    break;
+            }
+            layers_.push_back(std::move(layer));
+        }
+    }
+
+#ifdef BLACKFORGE_HIP_HAS_IR
+    // Same construction as cuda::Model (model.cu:137-250): first pipeline of the IR, weights from
+    // cpu::randomTensor(seedFor(seed, valueId, salt)) uploaded to the device.
+    explicit Model(const ir::ModelIR& modelIR, unsigned int seed = 42, std::optional<ir::PrecisionPolicy> precision = std::nullopt)
+        : Model(modelIR.name, specsFromIr(modelIR), inputFeaturesFromIr(modelIR),
+                precision.has_value() && precision->compute == sema::DType::BF16) {
+        initialiseLikeReference(modelIR, seed);
+    }
+#endif
+
+    // Runs the pipeline, keeping what backward() needs.  inputRangeTrusted: the caller has already checked
+    // the token ids of a leading embedding layer on the host (train_runner.cu:210-212), so no device-side
+    // range check (and no host synchronisation) is done.
+    DeviceTensor forward(const DeviceTensor& input, bool inputRangeTrusted = false) {
+        invalidateBf16WeightCache();   // the optimizer may have changed the weights since the last call
+        DeviceTensor current = input.clone();
+        for (std::size_t li = 0; li < layers_.size(); ++li) {
+            LayerState& layer = layers_[li];
+            DeviceTensor next = applyForward(layer, current, inputRangeTrusted && li == 0);
+            layer.cachedInput = std::move(current);
+            current = std::move(next);
+        }
+        return current;
+    }
+
+    void backward(const DeviceTensor& outputGrad, bool inputRangeTrusted = false) {
+        DeviceTensor grad = outputGrad.clone();
+        for (std::size_t li = layers_.size(); li-- > 0;) grad = applyBackward(layers_[li], grad, inputRangeTrusted && li == 0);
+    }
+
+    void zeroGrad() {
+        std::vector<float*> ptrs;
+        std::vector<std::size_t> counts;
+        for (LayerState& layer : layers_)
+            for (Parameter& p : layer.params) {
+                ptrs.push_back(p.grad.data());
+                counts.push_back(p.grad.elementCount());
+            }
+        check(bf_hip_zero_multi(ptrs.data(), counts.data(), ptrs.size(), nullptr));
+    }
+
+    // Incremental forward for generation: only the new positions are processed, K/V of earlier positions
+    // come from the per-layer cache (model.cu:385-424).
+    DeviceTensor forwardIncremental(const DeviceTensor& newTokenIds) {
+        DeviceTensor current = newTokenIds.clone();
+        std::size_t newLen = current.rank() >= 2 ? current.dim(1) : 0;
+        for (LayerState& layer : layers_) {
+            const LayerSpec& s = layer.spec;
+            switch (s.kind) {
+                case LayerKind::PositionalEmbedding:
+                    current = addPositionalEmbeddingAt(current, layer.params[0].value, generationPosition_);
+                    break;
+                case LayerKind::Attention:
+                    current = useBf16_ ? selfAttentionIncrementalBf16(current, layer.params[0].value, layer.params[1].value,
+                                                                       layer.params[2].value, layer.params[3].value, s.arg0, layer.kvCache)
+                                       : selfAttentionIncremental(current, layer.params[0].value, layer.params[1].value,
+                                                                  layer.params[2].value, layer.params[3].value, s.arg0, layer.kvCache);
+                    break;
+                case LayerKind::FeedForward: {
+                    Activation act = s.arg1 == 1 ? Activation::Gelu : Activation::Silu;
+                    current = useBf16_ ? feedForwardBf16(current, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                         layer.params[3].value, act)
+                                       : feedForward(current, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                     layer.params[3].value, act);
+                    break;
+                }
+                case LayerKind::Linear:
+                    current = useBf16_ ? linearBf16(current, layer.params[0].value, layer.params[1].value)
+                                       : linear(current, layer.params[0].value, layer.params[1].value);
+                    break;
+                case LayerKind::Embedding: current = embeddingLookup(current, layer.params[0].value); break;
+                default: current = applyElementwise(s.kind, current); break;
+            }
+        }
+        generationPosition_ += newLen;
+        return current;
+    }
+
+    void resetGenerationState() {
+        generationPosition_ = 0;
+        for (LayerState& layer : layers_) layer.kvCache = KVCache{};
+    }
+
+    [[nodiscard]] std::vector<Parameter*> parameters() {
+        std::vector<Parameter*> result;
+        for (LayerState& layer : layers_)
+            for (Parameter& p : layer.params) result.push_back(&p);
+        return result;
+    }
+
+    [[nodiscard]] std::optional<std::size_t> firstLayerEmbeddingVocabSize() const {
+        if (layers_.empty() || layers_.front().spec.kind != LayerKind::Embedding) return std::nullopt;
+        return layers_.front().spec.arg0;
+    }
+
+    [[nodiscard]] const std::string& name() const { return name_; }
+    [[nodiscard]] bool usesBf16() const { return useBf16_; }
+
+private:
+    struct LayerState {
+        LayerSpec spec;
+        std::vector<Parameter> params;
+        DeviceTensor cachedInput;
+        SelfAttentionCache attnCache;
+        FeedForwardCache ffCache;
+        KVCache kvCache;
+    };
+
+    static Parameter makeParameter(std::string name, std::vector<std::size_t> shape) {
+        return Parameter{std::move(name), DeviceTensor::zeros(shape), DeviceTensor::zeros(shape)};
+    }
+
+    static DeviceTensor applyElementwise(LayerKind kind, const DeviceTensor& x) {
+        switch (kind) {
+            case LayerKind::Silu: return silu(x);
+            case LayerKind::Relu: return relu(x);
+            case LayerKind::Gelu: return gelu(x);
+            case LayerKind::RmsNorm: return rmsnorm(x);
+            case LayerKind::Softmax: return softmax(x);
+            default: throw std::invalid_argument("hip::Model: not an elementwise layer");
+        }
+    }
+
+    DeviceTensor applyForward(LayerState& layer, const DeviceTensor& x, bool trustedIds) {
+        const LayerSpec& s = layer.spec;
+        switch (s.kind) {
+            case LayerKind::Linear:
+                return useBf16_ ? linearBf16CachedWeight(x, layer.params[0].value, layer.params[1].value)
+                                : linear(x, layer.params[0].value, layer.params[1].value);
+            case LayerKind::Embedding:
+                return trustedIds ? embeddingLookupPreValidated(x, layer.params[0].value) : embeddingLookup(x, layer.params[0].value);
+            case LayerKind::PositionalEmbedding: return addPositionalEmbedding(x, layer.params[0].value);
+            case LayerKind::Attention:
+                return selfAttentionForwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                  layer.params[3].value, s.arg0, useBf16_, layer.attnCache);
+            case LayerKind::FeedForward:
+                return feedForwardForwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                layer.params[3].value, useBf16_, layer.ffCache,
+                                                s.arg1 == 1 ? Activation::Gelu : Activation::Silu);
+            default: return applyElementwise(s.kind, x);
+        }
+    }
+
+    static void accumulate(DeviceTensor& target, const DeviceTensor& delta) {
+        check(bf_hip_accumulate(target.data(), delta.data(), target.elementCount(), nullptr));
+    }
+
+    DeviceTensor applyBackward(LayerState& layer, const DeviceTensor& grad, bool trustedIds) {
+        const LayerSpec& s = layer.spec;
+        const DeviceTensor& x = layer.cachedInput;
+        switch (s.kind) {
+            case LayerKind::Linear: {
+                DeviceTensor dBias = biasGradientOnly(grad);
+                MatmulGrad g = detail::projectionBackward(x, layer.params[0].value, grad, useBf16_ ? 2 : 0, x.shape());
+                accumulate(layer.params[0].grad, g.dB);
+                accumulate(layer.params[1].grad, dBias);
+                return std::move(g.dA);
+            }
+            case LayerKind::Silu: return siluBackward(x, grad);
+            case LayerKind::Relu: return reluBackward(x, grad);
+            case LayerKind::Gelu: return geluBackward(x, grad);
+            case LayerKind::RmsNorm: return rmsnormBackward(x, grad);
+            case LayerKind::Softmax: return softmaxBackward(x, grad);
+            case LayerKind::Embedding: {
+                DeviceTensor dTable = trustedIds ? embeddingLookupBackwardPreValidated(x, grad, s.arg0)
+                                                 : embeddingLookupBackward(x, grad, s.arg0);
+                accumulate(layer.params[0].grad, dTable);
+                return DeviceTensor::zeros(x.shape());   // token ids carry no gradient
+            }
+            case LayerKind::PositionalEmbedding: {
+                PositionalEmbeddingGrad g = addPositionalEmbeddingBackward(grad, s.arg0);
+                accumulate(layer.params[0].grad, g.dTable);
+                return std::move(g.dInput);
+            }
+            case LayerKind::Attention: {
+                SelfAttentionGrad g = selfAttentionBackwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                                  layer.params[3].value, s.arg0, layer.attnCache, grad, useBf16_);
+                accumulate(layer.params[0].grad, g.dWq);
+                accumulate(layer.params[1].grad, g.dWk);
+                accumulate(layer.params[2].grad, g.dWv);
+                accumulate(layer.params[3].grad, g.dWout);
+                return std::move(g.dInput);
+            }
+            case LayerKind::FeedForward: {
+                FeedForwardGrad g = feedForwardBackwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                              layer.params[3].value, layer.ffCache, grad, useBf16_,
+                                                              s.arg1 == 1 ? Activation::Gelu : Activation::Silu);
+                accumulate(layer.params[0].grad, g.dW1);
+                accumulate(layer.params[1].grad, g.dB1);
+                accumulate(layer.params[2].grad, g.dW2);
+                accumulate(layer.params[3].grad, g.dB2);
+                return std::move(g.dInput);
+            }
+        }
+        throw std::invalid_argument("hip::Model: unknown layer kind");
+    }
+
+#ifdef BLACKFORGE_HIP_HAS_IR
+    static std::vector<LayerSpec> specsFromIr(const ir::ModelIR& modelIR) {
+        require(!modelIR.pipelines.empty(), "hip::Model: model '" + modelIR.name + "' has no pipeline to train");
+        std::vector<LayerSpec> specs;
+        for (const ir::Operation& op : modelIR.pipelines.front().operations) {
+            switch (op.kind) {
+                case ir::OpKind::Linear: specs.push_back({LayerKind::Linear, static_cast<std::size_t>(op.linearOutFeatures), 0}); break;
+                case ir::OpKind::Silu: specs.push_back({LayerKind::Silu}); break;
+                case ir::OpKind::Relu: specs.push_back({LayerKind::Relu}); break;
+                case ir::OpKind::Gelu: specs.push_back({LayerKind::Gelu}); break;
+                case ir::OpKind::RmsNorm: specs.push_back({LayerKind::RmsNorm}); break;
+                case ir::OpKind::Softmax: specs.push_back({LayerKind::Softmax}); break;
+                case ir::OpKind::Embedding:
+                    specs.push_back({LayerKind::Embedding, static_cast<std::size_t>(op.embeddingVocabSize), static_cast<std::size_t>(op.embeddingDim)});
+                    break;
+                case ir::OpKind::PositionalEmbedding:
+                    specs.push_back({LayerKind::PositionalEmbedding, static_cast<std::size_t>(op.positionalMaxSeqLen), 0});
+                    break;
+                case ir::OpKind::Attention: specs.push_back({LayerKind::Attention, static_cast<std::size_t>(op.attentionNumHeads), 0}); break;
+                case ir::OpKind::FeedForward: specs.push_back({LayerKind::FeedForward, static_cast<std::size_t>(op.feedForwardHiddenDim), 0}); break;
+                default:
+                    throw std::invalid_argument("hip::Model: 'bidirectional_attention' is not implemented on this backend");
+            }
+        }
+        return specs;
+    }
+    static std::size_t inputFeaturesFromIr(const ir::ModelIR& modelIR) {
+        const ir::Value& v = modelIR.valueById(modelIR.pipelines.front().sourceValue);
+        return v.shape.empty() || v.shape.back().isSymbolic ? 0 : static_cast<std::size_t>(v.shape.back().literalValue);
+    }
+    void initialiseLikeReference(const ir::ModelIR& modelIR, unsigned int seed) {
+        // salts per parameter slot: src/backend/cpu/model.cpp:14-26
+        static const unsigned int linearSalts[] = {0x2545F491U, 0x27D4EB2FU};
+        static const unsigned int attnSalts[] = {0x27D4EB2DU, 0x165667B1U, 0xD3A2646CU, 0xFD7046C5U};
+        static const unsigned int ffSalts[] = {0xB55A4F09U, 0x5BD1E995U, 0x9E3779B9U, 0x1B873593U};
+        const auto& ops = modelIR.pipelines.front().operations;
+        for (std::size_t li = 0; li < layers_.size(); ++li) {
+            const unsigned int* salts = nullptr;
+            static const unsigned int embSalt[] = {0x85EBCA6BU}, posSalt[] = {0xC2B2AE35U};
+            switch (layers_[li].spec.kind) {
+                case LayerKind::Linear: salts = linearSalts; break;
+                case LayerKind::Embedding: salts = embSalt; break;
+                case LayerKind::PositionalEmbedding: salts = posSalt; break;
+                case LayerKind::Attention: salts = attnSalts; break;
+                case LayerKind::FeedForward: salts = ffSalts; break;
+                default: break;
+            }
+            for (std::size_t pi = 0; pi < layers_[li].params.size(); ++pi) {
+                Parameter& p = layers_[li].params[pi];
+                p.name = renameForValue(p.name, ops[li].output);
+                p.value = DeviceTensor::fromHost(cpu::randomTensor(p.value.shape(), cpu::seedFor(seed, ops[li].output, salts[pi])));
+            }
+        }
+    }
+    static std::string renameForValue(const std::string& name, std::size_t valueId) {
+        std::size_t dot = name.find('.');
+        std::size_t digits = dot;
+        while (digits > 0 && name[digits - 1] >= '0' && name[digits - 1] <= '9') --digits;
+        return name.substr(0, digits) + std::to_string(valueId) + name.substr(dot);
+    }
+#endif
+
+    std::string name_;
+    bool useBf16_ = false;
+    std::vector<LayerState> layers_;
+    std::size_t generationPosition_ = 0;
+};
+
+}  // namespace blackforge::backend::hip

@@ -1,0 +1,335 @@
+#pragma once
+// Forward operators with the reference's signatures (include/blackforge/backend/cuda/ops.hpp:8-258).
+// Each function validates shapes (std::invalid_argument), takes its result from the pool and makes one or
+// a few calls into the C ABI; no computation happens on the host.
+#include <cmath>
+#include <cstddef>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "blackforge/backend/hip/device_tensor.hpp"
+#include "blackforge/backend/hip/fused_attention.hpp"
+
+namespace blackforge::backend::hip {
+
+// Feed-forward activation: Silu is the reference block; Gelu is the same block with the reference's
+// gelu / geluBackward formulas substituted.
+enum class Activation : int { Silu = BF_ACT_SILU, Gelu = BF_ACT_GELU, Relu = BF_ACT_RELU };
+
+namespace detail {
+inline std::size_t lastDim(const DeviceTensor& t) { return t.shape().back(); }
+inline std::size_t rowsOf(const DeviceTensor& t) { return lastDim(t) ? t.elementCount() / lastDim(t) : 0; }
+inline std::vector<std::size_t> withLastDim(const DeviceTensor& t, std::size_t last) {
+    std::vector<std::size_t> s = t.shape();
+    s.back() = last;
+    return s;
+}
+inline void requireBias(const char* op, const DeviceTensor& x, const DeviceTensor& bias) {
+    require(x.rank() >= 2 && bias.rank() == 1 && lastDim(x) == bias.dim(0),
+            std::string(op) + ": expected input [..., features] and bias [features]");
+}
+// c[rows(a), n] = a(as [rows, k]) * b[k, n]; bf16 = 0 fp32 MFMA, 1 bf16 MFMA, 2 bf16 with cached weight image
+inline DeviceTensor projection(const DeviceTensor& a, const DeviceTensor& b, int bf16, std::vector<std::size_t> outShape) {
+    std::size_t k = lastDim(a), m = rowsOf(a), n = b.dim(1);
+    DeviceTensor c(std::move(outShape));
+    if (bf16 == 0) check(bf_hip_gemm_f32(0, 0, a.data(), b.data(), c.data(), m, n, k, nullptr));
+    else check(bf_hip_matmul_bf16(a.data(), b.data(), c.data(), m, k, n, bf16 == 2, nullptr));
+    return c;
+}
+}  // namespace detail
+
+inline DeviceTensor add(const DeviceTensor& a, const DeviceTensor& b) {
+    require(a.shape() == b.shape(), "add: incompatible shapes on the device");
+    DeviceTensor out(a.shape());
+    check(bf_hip_add(a.data(), b.data(), out.data(), a.elementCount(), nullptr));
+    return out;
+}
+
+inline DeviceTensor scale(const DeviceTensor& x, float factor) {
+    DeviceTensor out(x.shape());
+    check(bf_hip_scale(x.data(), factor, out.data(), x.elementCount(), nullptr));
+    return out;
+}
+
+inline DeviceTensor addBias(const DeviceTensor& input, const DeviceTensor& bias) {
+    detail::requireBias("addBias", input, bias);
+    DeviceTensor out(input.shape());
+    check(bf_hip_add_bias(input.data(), bias.data(), out.data(), detail::rowsOf(input), bias.dim(0), nullptr));
+    return out;
+}
+
+inline DeviceTensor addBiasActivation(const DeviceTensor& gemmOutput, const DeviceTensor& bias, Activation act) {
+    detail::requireBias("addBiasSilu", gemmOutput, bias);
+    DeviceTensor out(gemmOutput.shape());
+    check(bf_hip_add_bias_act(gemmOutput.data(), bias.data(), out.data(), detail::rowsOf(gemmOutput), bias.dim(0),
+                              static_cast<int>(act), nullptr));
+    return out;
+}
+
+inline DeviceTensor addBiasSilu(const DeviceTensor& gemmOutput, const DeviceTensor& bias) {
+    return addBiasActivation(gemmOutput, bias, Activation::Silu);
+}
+
+inline DeviceTensor addBiasResidual(const DeviceTensor& gemmOutput, const DeviceTensor& bias, const DeviceTensor& residual) {
+    detail::requireBias("addBiasResidual", gemmOutput, bias);
+    require(gemmOutput.shape() == residual.shape(), "addBiasResidual: residual shape differs");
+    DeviceTensor out(gemmOutput.shape());
+    check(bf_hip_add_bias_residual(gemmOutput.data(), bias.data(), residual.data(), out.data(), detail::rowsOf(gemmOutput),
+                                   bias.dim(0), nullptr));
+    return out;
+}
+
+inline DeviceTensor matmul(const DeviceTensor& a, const DeviceTensor& b) {
+    require(a.rank() == 2 && b.rank() == 2 && a.dim(1) == b.dim(0), "matmul: incompatible shapes on the device");
+    return detail::projection(a, b, 0, {a.dim(0), b.dim(1)});
+}
+
+inline DeviceTensor matmulTransposeB(const DeviceTensor& a, const DeviceTensor& b) {
+    require(a.rank() == 2 && b.rank() == 2 && a.dim(1) == b.dim(1), "matmulTransposeB: incompatible shapes on the device");
+    DeviceTensor c({a.dim(0), b.dim(0)});
+    check(bf_hip_gemm_f32(0, 1, a.data(), b.data(), c.data(), a.dim(0), b.dim(0), a.dim(1), nullptr));
+    return c;
+}
+
+inline DeviceTensor matmulBf16(const DeviceTensor& a, const DeviceTensor& b) {
+    require(a.rank() == 2 && b.rank() == 2 && a.dim(1) == b.dim(0), "matmulBf16: incompatible shapes on the device");
+    return detail::projection(a, b, 1, {a.dim(0), b.dim(1)});
+}
+
+inline DeviceTensor matmulBf16CachedWeight(const DeviceTensor& a, const DeviceTensor& b) {
+    require(a.rank() == 2 && b.rank() == 2 && a.dim(1) == b.dim(0), "matmulBf16CachedWeight: incompatible shapes on the device");
+    return detail::projection(a, b, 2, {a.dim(0), b.dim(1)});
+}
+
+inline void invalidateBf16WeightCache() { check(bf_hip_invalidate_bf16_weight_cache()); }
+
+inline DeviceTensor activation(const DeviceTensor& input, Activation act) {
+    DeviceTensor out(input.shape());
+    check(bf_hip_act_forward(input.data(), out.data(), input.elementCount(), static_cast<int>(act), nullptr));
+    return out;
+}
+inline DeviceTensor silu(const DeviceTensor& input) { return activation(input, Activation::Silu); }
+inline DeviceTensor relu(const DeviceTensor& input) { return activation(input, Activation::Relu); }
+inline DeviceTensor gelu(const DeviceTensor& input) { return activation(input, Activation::Gelu); }
+
+inline DeviceTensor rmsnorm(const DeviceTensor& input) {
+    require(input.rank() >= 2, "rmsnorm: needs a tensor of rank >= 2 on the device");
+    DeviceTensor out(input.shape());
+    check(bf_hip_rmsnorm(input.data(), out.data(), detail::rowsOf(input), detail::lastDim(input), nullptr));
+    return out;
+}
+
+inline DeviceTensor softmax(const DeviceTensor& input) {
+    require(input.rank() >= 2, "softmax: needs a tensor of rank >= 2 on the device");
+    DeviceTensor out(input.shape());
+    check(bf_hip_softmax(input.data(), out.data(), detail::rowsOf(input), detail::lastDim(input), nullptr));
+    return out;
+}
+
+namespace detail {
+inline void requireIdsInRange(const char* op, const DeviceTensor& ids, std::size_t limit, const char* what) {
+    std::size_t bad = 0;
+    long long first = 0;
+    check(bf_hip_count_out_of_range(ids.data(), ids.elementCount(), limit, &bad, &first, nullptr));
+    require(bad == 0, std::string(op) + ": " + what + " " + std::to_string(first) + " outside [0, " + std::to_string(limit) + ")");
+}
+}  // namespace detail
+
+inline DeviceTensor embeddingLookupPreValidated(const DeviceTensor& tokenIds, const DeviceTensor& table) {
+    require(tokenIds.rank() == 2, "embeddingLookup: token ids must have rank 2 [batch, seq]");
+    require(table.rank() == 2, "embeddingLookup: table must have rank 2 [vocabSize, dim]");
+    DeviceTensor out({tokenIds.dim(0), tokenIds.dim(1), table.dim(1)});
+    check(bf_hip_embedding_forward(tokenIds.data(), table.data(), out.data(), tokenIds.elementCount(), table.dim(0),
+                                   table.dim(1), nullptr));
+    return out;
+}
+
+inline DeviceTensor embeddingLookup(const DeviceTensor& tokenIds, const DeviceTensor& table) {
+    require(tokenIds.rank() == 2, "embeddingLookup: token ids must have rank 2 [batch, seq]");
+    require(table.rank() == 2, "embeddingLookup: table must have rank 2 [vocabSize, dim]");
+    detail::requireIdsInRange("embeddingLookup", tokenIds, table.dim(0), "token id");
+    return embeddingLookupPreValidated(tokenIds, table);
+}
+
+inline DeviceTensor addPositionalEmbeddingAt(const DeviceTensor& input, const DeviceTensor& table, std::size_t offset) {
+    require(input.rank() == 3, "addPositionalEmbedding: needs an input of rank 3 [batch, seq, dim]");
+    require(table.rank() == 2 && table.dim(1) == input.dim(2), "addPositionalEmbedding: table must be [maxSeqLen, dim]");
+    DeviceTensor out(input.shape());
+    check(bf_hip_positional_forward(input.data(), table.data(), out.data(), input.dim(0), input.dim(1), input.dim(2),
+                                    table.dim(0), offset, nullptr));
+    return out;
+}
+
+inline DeviceTensor addPositionalEmbedding(const DeviceTensor& input, const DeviceTensor& table) {
+    return addPositionalEmbeddingAt(input, table, 0);
+}
+
+namespace detail {
+inline DeviceTensor linearImpl(const char* op, const DeviceTensor& input, const DeviceTensor& weight, const DeviceTensor& bias, int bf16) {
+    require(input.rank() >= 2, std::string(op) + ": needs a tensor of rank >= 2");
+    require(weight.rank() == 2 && lastDim(input) == weight.dim(0), std::string(op) + ": incompatible shapes on the device");
+    require(bias.rank() == 1 && bias.dim(0) == weight.dim(1), std::string(op) + ": bias does not match the weight");
+    DeviceTensor product = projection(input, weight, bf16, withLastDim(input, weight.dim(1)));
+    DeviceTensor out(product.shape());
+    check(bf_hip_add_bias(product.data(), bias.data(), out.data(), rowsOf(product), bias.dim(0), nullptr));
+    return out;
+}
+}  // namespace detail
+
+inline DeviceTensor linear(const DeviceTensor& input, const DeviceTensor& weight, const DeviceTensor& bias) {
+    return detail::linearImpl("linear", input, weight, bias, 0);
+}
+inline DeviceTensor linearBf16(const DeviceTensor& input, const DeviceTensor& weight, const DeviceTensor& bias) {
+    return detail::linearImpl("linearBf16", input, weight, bias, 1);
+}
+inline DeviceTensor linearBf16CachedWeight(const DeviceTensor& input, const DeviceTensor& weight, const DeviceTensor& bias) {
+    return detail::linearImpl("linearBf16CachedWeight", input, weight, bias, 2);
+}
+
+// ---- composite blocks ------------------------------------------------------------------------
+struct FeedForwardCache {
+    DeviceTensor normed;  // rmsnorm(input)
+    DeviceTensor gemm1;   // normed @ w1, before bias and activation
+    DeviceTensor hidden;  // act(gemm1 + b1)
+};
+
+inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
+                                              const DeviceTensor& w2, const DeviceTensor& b2, bool useBf16,
+                                              FeedForwardCache& cache, Activation act = Activation::Silu) {
+    require(input.rank() >= 2 && w1.rank() == 2 && w2.rank() == 2 && detail::lastDim(input) == w1.dim(0) && w1.dim(1) == w2.dim(0),
+            "feedForward: incompatible shapes on the device");
+    const int mode = useBf16 ? 2 : 0;
+    cache.normed = rmsnorm(input);
+    cache.gemm1 = detail::projection(cache.normed, w1, mode, detail::withLastDim(input, w1.dim(1)));
+    cache.hidden = addBiasActivation(cache.gemm1, b1, act);
+    DeviceTensor gemm2 = detail::projection(cache.hidden, w2, mode, detail::withLastDim(input, w2.dim(1)));
+    return addBiasResidual(gemm2, b2, input);
+}
+
+namespace detail {
+inline DeviceTensor feedForwardImpl(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
+                                     const DeviceTensor& w2, const DeviceTensor& b2, bool useBf16, Activation act) {
+    DeviceTensor normed = rmsnorm(input);
+    DeviceTensor hidden = activation(linearImpl("feedForward", normed, w1, b1, useBf16 ? 1 : 0), act);
+    DeviceTensor out = linearImpl("feedForward", hidden, w2, b2, useBf16 ? 1 : 0);
+    return add(input, out);
+}
+}  // namespace detail
+
+inline DeviceTensor feedForward(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
+                                 const DeviceTensor& w2, const DeviceTensor& b2, Activation act = Activation::Silu) {
+    return detail::feedForwardImpl(input, w1, b1, w2, b2, false, act);
+}
+inline DeviceTensor feedForwardBf16(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
+                                     const DeviceTensor& w2, const DeviceTensor& b2, Activation act = Activation::Silu) {
+    return detail::feedForwardImpl(input, w1, b1, w2, b2, true, act);
+}
+
+struct SelfAttentionCache {
+    DeviceTensor normedFlat;  // [batch*seq, dim]
+    DeviceTensor q, k, v;     // [batch, seq, dim]
+    DeviceTensor attnOutput;  // [batch, seq, dim], before Wout
+    DeviceTensor attnM, attnL;
+};
+
+namespace detail {
+inline void requireAttention(const char* op, const DeviceTensor& input, std::size_t numHeads) {
+    require(input.rank() == 3, std::string(op) + ": needs an input of rank 3 [batch, seq, dim] on the device");
+    require(numHeads != 0 && input.dim(2) % numHeads == 0, std::string(op) + ": numHeads must divide dim exactly");
+}
+// mode: 0 fp32, 1 bf16, 2 bf16 with cached weight images
+inline DeviceTensor selfAttentionForwardImpl(const char* op, const DeviceTensor& input, const DeviceTensor& wq,
+                                              const DeviceTensor& wk, const DeviceTensor& wv, const DeviceTensor& wout,
+                                              std::size_t numHeads, int mode, SelfAttentionCache& cache) {
+    requireAttention(op, input, numHeads);
+    std::size_t batch = input.dim(0), seq = input.dim(1), dim = input.dim(2);
+    float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
+    cache.normedFlat = rmsnorm(input).reshaped({batch * seq, dim});
+    cache.q = projection(cache.normedFlat, wq, mode, {batch, seq, dim});
+    cache.k = projection(cache.normedFlat, wk, mode, {batch, seq, dim});
+    cache.v = projection(cache.normedFlat, wv, mode, {batch, seq, dim});
+    FusedAttentionForwardResult attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, 0);
+    cache.attnOutput = std::move(attn.output);
+    cache.attnM = std::move(attn.m);
+    cache.attnL = std::move(attn.l);
+    DeviceTensor projected = projection(cache.attnOutput, wout, mode, {batch, seq, dim});
+    return add(input, projected);
+}
+}  // namespace detail
+
+inline DeviceTensor selfAttentionForwardCached(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                bool useBf16, SelfAttentionCache& cache) {
+    return detail::selfAttentionForwardImpl("selfAttentionForwardCached", input, wq, wk, wv, wout, numHeads, useBf16 ? 2 : 0, cache);
+}
+inline DeviceTensor selfAttention(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                   const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads) {
+    SelfAttentionCache cache;
+    return detail::selfAttentionForwardImpl("selfAttention", input, wq, wk, wv, wout, numHeads, 0, cache);
+}
+inline DeviceTensor selfAttentionBf16(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                       const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads) {
+    SelfAttentionCache cache;
+    return detail::selfAttentionForwardImpl("selfAttentionBf16", input, wq, wk, wv, wout, numHeads, 1, cache);
+}
+
+// K/V of the positions processed so far, for incremental decoding.
+struct KVCache {
+    DeviceTensor k;
+    DeviceTensor v;
+    std::size_t length = 0;
+};
+
+namespace detail {
+inline DeviceTensor concatSeq(const DeviceTensor& a, const DeviceTensor& b) {
+    DeviceTensor out({a.dim(0), a.dim(1) + b.dim(1), a.dim(2)});
+    check(bf_hip_concat_seq(a.data(), b.data(), out.data(), a.dim(0), a.dim(1), b.dim(1), a.dim(2), nullptr));
+    return out;
+}
+inline DeviceTensor selfAttentionIncrementalImpl(const char* op, const DeviceTensor& newInput, const DeviceTensor& wq,
+                                                  const DeviceTensor& wk, const DeviceTensor& wv, const DeviceTensor& wout,
+                                                  std::size_t numHeads, KVCache& cache, int mode) {
+    requireAttention(op, newInput, numHeads);
+    std::size_t batch = newInput.dim(0), newLen = newInput.dim(1), dim = newInput.dim(2);
+    DeviceTensor normedFlat = rmsnorm(newInput).reshaped({batch * newLen, dim});
+    DeviceTensor qNew = projection(normedFlat, wq, mode, {batch, newLen, dim});
+    DeviceTensor kNew = projection(normedFlat, wk, mode, {batch, newLen, dim});
+    DeviceTensor vNew = projection(normedFlat, wv, mode, {batch, newLen, dim});
+    std::size_t oldLen = cache.length;
+    if (oldLen == 0) {
+        cache.k = std::move(kNew);
+        cache.v = std::move(vNew);
+    } else {
+        cache.k = concatSeq(cache.k, kNew);
+        cache.v = concatSeq(cache.v, vNew);
+    }
+    cache.length = oldLen + newLen;
+    float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
+    FusedAttentionForwardResult attn = fusedAttentionForward(qNew, cache.k, cache.v, numHeads, scaleFactor, oldLen);
+    DeviceTensor projected = projection(attn.output, wout, mode, {batch, newLen, dim});
+    return add(newInput, projected);
+}
+}  // namespace detail
+
+inline DeviceTensor selfAttentionIncremental(const DeviceTensor& newInput, const DeviceTensor& wq, const DeviceTensor& wk,
+                                              const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                              KVCache& cache) {
+    return detail::selfAttentionIncrementalImpl("selfAttentionIncremental", newInput, wq, wk, wv, wout, numHeads, cache, 0);
+}
+inline DeviceTensor selfAttentionIncrementalBf16(const DeviceTensor& newInput, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                  const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                  KVCache& cache) {
+    return detail::selfAttentionIncrementalImpl("selfAttentionIncrementalBf16", newInput, wq, wk, wv, wout, numHeads, cache, 1);
+}
+
+// Greedy next-token choice over the last position of [1, seq, vocab] logits (reference: src/main.cpp:504-518),
+// computed on the device; only the index crosses to the host.
+inline std::size_t argmaxLastPosition(const DeviceTensor& logits) {
+    require(logits.rank() >= 2, "argmaxLastPosition: needs logits of rank >= 2");
+    long long index = 0;
+    check(bf_hip_argmax_last_position(logits.data(), logits.dim(logits.rank() - 2), logits.dim(logits.rank() - 1), &index, nullptr));
+    return static_cast<std::size_t>(index);
+}
+
+}  // namespace blackforge::backend::hip

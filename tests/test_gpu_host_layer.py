@@ -1,0 +1,205 @@
+"""GPU parity of the C++ operator layer (include/blackforge/backend/hip/): the C++ API test program, the
+composite blocks, and whole training steps of hip::Model against the CPU oracle and the golden fixtures."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import refvectors as rv
+from parity import BF16_TOL, assert_close
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(ROOT, "tests", "golden", "reference_vectors.npz")
+
+
+def r(rng, *s, scale=1.0):
+    return (rng.standard_normal(s) * scale).astype(f32)
+
+
+def test_cpp_api_program(hip):
+    """tests/cpp/host_api_test.cpp: the reference's literal test vectors through namespace blackforge::backend::hip."""
+    exe = os.path.join(ROOT, "blackforge_amd", "host", "bin", "host_api_test")
+    assert os.path.exists(exe), "run `make -C blackforge_amd/host` (the driver's build() does)"
+    proc = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(proc.stdout[-3000:])
+    assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-1000:]
+
+
+def test_attention_block_fixture_and_golden(hip, oracle):
+    """The reference's shared 4x4 attention fixture: forward and every gradient against the real reference's numbers."""
+    gold = np.load(GOLDEN)
+    D, ops = hip.DeviceTensor, hip.ops
+    w = [D.fromHost(a) for a in (rv.ATTN_WQ, rv.ATTN_WK, rv.ATTN_WV, rv.ATTN_WOUT)]
+    x, g = D.fromHost(rv.ATTN_INPUT), D.fromHost(gold["attnfix_grad"])
+    assert_close(ops.selfAttention(x, *w, rv.ATTN_HEADS).toHost(), gold["attnfix_out"], what="selfAttention fixture")
+    grad = ops.selfAttentionBackward(x, *w, rv.ATTN_HEADS, g)
+    for name, got in zip(("dx", "dwq", "dwk", "dwv", "dwout"), (grad.dInput, grad.dWq, grad.dWk, grad.dWv, grad.dWout)):
+        assert_close(got.toHost(), gold["attnfix_" + name], what="selfAttentionBackward fixture " + name, scale=1e-2)
+    ff = [D.fromHost(a) for a in (rv.FF_W1, rv.FF_B1, rv.FF_W2, rv.FF_B2)]
+    assert_close(ops.feedForward(D.fromHost(rv.FF_INPUT), *ff).toHost(), gold["fffix_out"], what="feedForward fixture")
+    fg = ops.feedForwardBackward(D.fromHost(rv.FF_INPUT), *ff, D.fromHost(rv.FF_GRAD))
+    for name, got in zip(("dx", "dw1", "db1", "dw2", "db2"), (fg.dInput, fg.dW1, fg.dB1, fg.dW2, fg.dB2)):
+        assert_close(got.toHost(), gold["fffix_" + name], what="feedForwardBackward fixture " + name, scale=1e-2)
+
+
+@pytest.mark.parametrize("batch,seq,dim,heads,hidden", [(2, 9, 12, 3, 20), (8, 64, 128, 4, 512), (1, 130, 64, 2, 96)])
+@pytest.mark.parametrize("act", [0, 1])
+def test_blocks_against_oracle(hip, oracle, rng, batch, seq, dim, heads, hidden, act):
+    D, ops = hip.DeviceTensor, hip.ops
+    x, g = r(rng, batch, seq, dim), r(rng, batch, seq, dim)
+    w = [r(rng, dim, dim, scale=dim ** -0.5) for _ in range(4)]
+    dw = [D.fromHost(a) for a in w]
+    dx, dg = D.fromHost(x), D.fromHost(g)
+    if act == 0:
+        assert_close(ops.selfAttention(dx, *dw, heads).toHost(), oracle.selfAttention(x, *w, heads), what="selfAttention")
+        grad = ops.selfAttentionBackward(dx, *dw, heads, dg)
+        exp = oracle.selfAttentionBackward(x, *w, heads, g)
+        for got, e, n in zip((grad.dInput, grad.dWq, grad.dWk, grad.dWv, grad.dWout), exp, ("dInput", "dWq", "dWk", "dWv", "dWout")):
+            assert_close(got.toHost(), e, what="selfAttentionBackward." + n, scale=float(np.abs(e).max()) * 0.1)
+    p = [r(rng, dim, hidden, scale=dim ** -0.5), r(rng, hidden, scale=.1), r(rng, hidden, dim, scale=hidden ** -0.5), r(rng, dim, scale=.1)]
+    dp = [D.fromHost(a) for a in p]
+    assert_close(ops.feedForward(dx, *dp, act).toHost(), oracle.feedForward(x, *p, act), what="feedForward")
+    fg = ops.feedForwardBackward(dx, *dp, dg, act)
+    for got, e, n in zip((fg.dInput, fg.dW1, fg.dB1, fg.dW2, fg.dB2), oracle.feedForwardBackward(x, *p, g, act), ("dInput", "dW1", "dB1", "dW2", "dB2")):
+        assert_close(got.toHost(), e, what="feedForwardBackward." + n, scale=float(np.abs(e).max()) * 0.1)
+
+
+def test_incremental_decode_block(hip, oracle, rng):
+    D, ops = hip.DeviceTensor, hip.ops
+    batch, dim, heads = 2, 32, 4
+    w = [r(rng, dim, dim, scale=dim ** -0.5) for _ in range(4)]
+    dw = [D.fromHost(a) for a in w]
+    cache, kc, vc = ops.KVCache(), None, None
+    for new_len in (5, 1, 1, 3):
+        x = r(rng, batch, new_len, dim)
+        got = ops.selfAttentionIncremental(D.fromHost(x), *dw, heads, cache).toHost()
+        exp, kc, vc = oracle.selfAttentionIncremental(x, *w, heads, kc, vc)
+        assert_close(got, exp, what=f"incremental newLen={new_len}")
+    assert cache.length == 10
+    assert_close(cache.k.toHost(), kc, what="KV cache K")
+
+
+def _lm_layers(hl, vocab, dim, seq, heads, hidden, act, blocks=1):
+    layers = [(hl.EMBEDDING, vocab, dim), (hl.POSITIONAL, seq)]
+    for _ in range(blocks):
+        layers += [(hl.ATTENTION, heads), (hl.FEEDFORWARD, hidden, act)]
+    return layers + [(hl.LINEAR, vocab)]
+
+
+def test_tiny_lm_three_steps_match_the_reference_fixture(hip):
+    """hip::Model against numbers produced by the reference's cpu::Model: logits, loss, every gradient and every
+    parameter after each of three AdamW steps (fixture: tests/golden/make_golden.py)."""
+    from blackforge_amd import hostlayer as hl
+    gold = np.load(GOLDEN)
+    layers = [tuple(int(v) for v in row) for row in gold["lm_layers"]]
+    model = hl.HostModel(layers)
+    for i in range(len(model.counts)):
+        model.set_value(i, gold[f"lm_init{i}"])
+    D = hip.DeviceTensor
+    for step in range(3):
+        model.zeroGrad()
+        logits = model.forward(D.fromHost(gold[f"lm_step{step}_ids"]))
+        assert_close(logits, gold[f"lm_step{step}_logits"], what=f"step {step} logits")
+        model.loss(D.fromHost(gold[f"lm_step{step}_tgt"]))
+        loss = model.readLossSum() / 16
+        assert abs(loss - float(gold[f"lm_step{step}_loss"])) <= 1e-4 * float(gold[f"lm_step{step}_loss"])
+        model.backward()
+        for i in range(len(model.counts)):
+            e = gold[f"lm_step{step}_grad{i}"]
+            assert_close(model.grad(i), e, what=f"step {step} grad {model.names[i]}", scale=float(np.abs(e).max()) * 0.05)
+        model.adamwStep(lr=1e-2)
+        for i in range(len(model.counts)):
+            # floor: 2 % of the AdamW step bound lr = 1e-2 (the update is lr * m / (sqrt(v) + eps), ill-conditioned
+            # where the gradient is comparable to eps)
+            assert_close(model.value(i), gold[f"lm_step{step}_param{i}"], what=f"step {step} param {model.names[i]}", scale=0.02 * 1e-2 / 1e-4)
+
+
+@pytest.mark.parametrize("act", [0, 1])
+def test_config1_tiny_lm_full_step_against_oracle(hip, oracle, rng, act):
+    """BASELINE config 1 shape: vocab 256, d_model 128, 4 heads, 1 attention + 1 feedforward(512) block, seq 64,
+    batch 8; forward, sparse CE, backward, one AdamW step (lr 1e-3, wd 0.01).  act=1 is the GELU variant."""
+    from blackforge_amd import hostlayer as hl
+    from oracle import bfo
+    vocab, dim, seq, batch, heads, hidden = 256, 128, 64, 8, 4, 512
+    gpu = hl.HostModel(_lm_layers(hl, vocab, dim, seq, heads, hidden, act))
+    cpu = oracle.model(_lm_layers(bfo, vocab, dim, seq, heads, hidden, act))
+    assert gpu.names == cpu.names
+    for i, c in enumerate(gpu.counts):
+        w = r(rng, c, scale=0.02)
+        gpu.set_value(i, w)
+        cpu.value(i)[:] = w
+    D = hip.DeviceTensor
+    ids = rng.integers(0, vocab, (batch, seq)).astype(f32)
+    tgt = rng.integers(0, vocab, batch * seq).astype(f32)
+    cpu.zeroGrad()
+    logits = cpu.forward(ids)
+    loss, grad = oracle.softmaxCrossEntropySparse(logits.reshape(-1, vocab), tgt)
+    cpu.backward(grad)
+    gpu.zeroGrad()
+    assert_close(gpu.forward(D.fromHost(ids), trusted=True), logits, what="logits")
+    gpu.loss(D.fromHost(tgt))
+    assert abs(gpu.readLossSum() / (batch * seq) - loss) <= 1e-4 * loss
+    gpu.backward(trusted=True)
+    for i in range(len(gpu.counts)):
+        e = cpu.grad(i)
+        assert_close(gpu.grad(i), e, what="grad " + gpu.names[i], scale=float(np.abs(e).max()) * 0.05)
+    cpu.adamwStep()
+    gpu.adamwStep()
+    for i in range(len(gpu.counts)):
+        # AdamW's first step is lr * g / (|g| + eps): where |g| is comparable to eps = 1e-8 the step depends on
+        # the gradient's last bits, but it never exceeds lr, so the floor is a small fraction (2 %) of lr = 1e-3
+        assert_close(gpu.value(i), cpu.value(i), what="param " + gpu.names[i], scale=0.02 * 1e-3 / 1e-4)
+
+
+def test_bf16_model_step_stays_within_bf16_tolerance(hip, oracle, rng):
+    """bf16 projections (precision.compute = bf16): logits and gradients within 2e-2 of the fp32 CPU reference."""
+    from blackforge_amd import hostlayer as hl
+    from oracle import bfo
+    vocab, dim, seq, batch, heads, hidden = 96, 64, 32, 4, 2, 128
+    gpu = hl.HostModel(_lm_layers(hl, vocab, dim, seq, heads, hidden, 0), use_bf16=True)
+    cpu = oracle.model(_lm_layers(bfo, vocab, dim, seq, heads, hidden, 0))
+    for i, c in enumerate(gpu.counts):
+        w = r(rng, c, scale=0.05)
+        gpu.set_value(i, w)
+        cpu.value(i)[:] = w
+    D = hip.DeviceTensor
+    ids = rng.integers(0, vocab, (batch, seq)).astype(f32)
+    tgt = rng.integers(0, vocab, batch * seq).astype(f32)
+    logits = cpu.forward(ids)
+    loss, grad = oracle.softmaxCrossEntropySparse(logits.reshape(-1, vocab), tgt)
+    cpu.zeroGrad()
+    cpu.backward(grad)
+    x, t = D.fromHost(ids), D.fromHost(tgt)
+    gpu.trainStep(x, t, optimizer=0)
+    assert abs(gpu.readLossSum() / (batch * seq) - loss) <= BF16_TOL * loss
+    for i in range(len(gpu.counts)):
+        e = cpu.grad(i)
+        assert_close(gpu.grad(i), e, tol=BF16_TOL, what="bf16 grad " + gpu.names[i], scale=float(np.abs(e).max()))
+
+
+def test_mlp_config2_shape_small(hip, oracle, rng):
+    """BASELINE config 2 pipeline (linear -> silu -> linear, MSE) at a reduced width, bf16 projections."""
+    from blackforge_amd import hostlayer as hl
+    from oracle import bfo
+    tokens, width = 256, 192
+    layers = lambda m: [(m.LINEAR, width), (m.SILU,), (m.LINEAR, width)]
+    gpu = hl.HostModel(layers(hl), input_features=width, use_bf16=True)
+    cpu = oracle.model(layers(bfo), input_features=width)
+    for i, c in enumerate(gpu.counts):
+        w = r(rng, c, scale=width ** -0.5) if gpu.names[i].endswith("weight") else np.zeros(c, f32)
+        gpu.set_value(i, w)
+        cpu.value(i)[:] = w
+    x, y = r(rng, tokens, width), r(rng, tokens, width)
+    out = cpu.forward(x)
+    loss, grad = oracle.meanSquaredError(out.reshape(tokens, width), y)
+    cpu.zeroGrad()
+    cpu.backward(grad)
+    dx, dy = hip.DeviceTensor.fromHost(x), hip.DeviceTensor.fromHost(y)
+    gpu.trainStep(dx, dy, loss_kind=hl.LOSS_MSE, optimizer=0)
+    assert abs(gpu.readLossSum() / (tokens * width) - loss) <= BF16_TOL * loss
+    for i in range(len(gpu.counts)):
+        e = cpu.grad(i)
+        assert_close(gpu.grad(i), e, tol=BF16_TOL, what="mlp grad " + gpu.names[i], scale=float(np.abs(e).max()))
