@@ -47,16 +47,18 @@ struct AttnParams {
 
 __device__ __forceinline__ float fastExp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Workgroup -> (batch*head, tile).  Workgroups are dealt round-robin to the 8 XCDs, each with its own
-// L2; this mapping gives every XCD a contiguous range of (batch, head) pairs so that the tiles that
-// share K/V (or Q/dO) hit the same L2.  Within a pair the heaviest tile comes first.
+// Workgroup -> (batch*head, tile), heaviest tiles first over ALL (batch, head) pairs: causal tiles differ in
+// work by up to numTiles x, and a heavy tile that starts late sets the kernel's makespan.  Consecutive
+// workgroup ids walk the (batch, head) pairs at one tile level; the hardware deals workgroups round-robin to
+// the 8 XCDs, so with a pair count divisible by 8 every pair stays on one XCD, and the tiles of a pair that
+// are dispatched together stream through the same K/V (or Q/dO) tiles at the same time and share them in
+// that XCD's L2.
 __device__ __forceinline__ void decodeBlock(int numTiles, int totalBlocks, bool heavyIsLast, int& bh, int& tile) {
-    int id = blockIdx.x;
-    constexpr int kXcds = 8;
-    if (totalBlocks % kXcds == 0) id = (id % kXcds) * (totalBlocks / kXcds) + id / kXcds;
-    bh = id / numTiles;
-    int t = id - bh * numTiles;
-    tile = heavyIsLast ? numTiles - 1 - t : t;
+    const int id = blockIdx.x;
+    const int numPairs = totalBlocks / numTiles;
+    const int level = id / numPairs;   // 0 = heaviest
+    bh = id - level * numPairs;
+    tile = heavyIsLast ? numTiles - 1 - level : level;
 }
 
 // Cooperative copy of ROWS rows of one head ([row][hd] slices of a [.., dim] tensor) into LDS as
@@ -84,6 +86,52 @@ __device__ __forceinline__ void loadHeadTile(float* __restrict__ lds, const floa
             }
         }
         storef4(lds + r * LDSW + c, val);
+    }
+}
+
+// The same copy split in two so that the global loads of the NEXT tile are in flight while the current
+// tile is being consumed: fetchHeadTile issues the loads into registers, commitHeadTile writes them to LDS.
+template <int HDP, int ROWS>
+struct TileRegs {
+    static constexpr int kSlots = (ROWS * (HDP / 4) + 255) / 256;
+    float4v v[kSlots];
+};
+
+template <int HDP, int ROWS, bool VEC4>
+__device__ __forceinline__ void fetchHeadTile(TileRegs<HDP, ROWS>& regs, const float* __restrict__ base, int dim, int row0,
+                                              int rowLimit, int hd, int tid) {
+    constexpr int V4 = HDP / 4;
+    constexpr int SLOTS = ROWS * V4;
+#pragma unroll
+    for (int i = 0; i < TileRegs<HDP, ROWS>::kSlots; ++i) {
+        int s = tid + i * 256;
+        int r = s / V4, c = (s % V4) * 4;
+        int row = row0 + r;
+        float4v val = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (s < SLOTS && row < rowLimit && c < hd) {
+            const float* src = base + size_t(row) * dim + c;
+            if constexpr (VEC4) {
+                val = loadf4(src);
+            } else {
+                val.x = src[0];
+                if (c + 1 < hd) val.y = src[1];
+                if (c + 2 < hd) val.z = src[2];
+                if (c + 3 < hd) val.w = src[3];
+            }
+        }
+        regs.v[i] = val;
+    }
+}
+
+template <int HDP, int ROWS>
+__device__ __forceinline__ void commitHeadTile(float* __restrict__ lds, const TileRegs<HDP, ROWS>& regs, int tid) {
+    constexpr int LDSW = HDP + 4;
+    constexpr int V4 = HDP / 4;
+    constexpr int SLOTS = ROWS * V4;
+#pragma unroll
+    for (int i = 0; i < TileRegs<HDP, ROWS>::kSlots; ++i) {
+        int s = tid + i * 256;
+        if (s < SLOTS) storef4(lds + (s / V4) * LDSW + (s % V4) * 4, regs.v[i]);
     }
 }
 
@@ -168,6 +216,61 @@ __device__ __forceinline__ void storeTransposed(float* __restrict__ dst, const f
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
+// One K/V tile (BC keys = BC/32 sub-blocks) for one wavefront, as straight-line code so that the
+// instruction scheduler can overlap the matrix pipe with the vector pipe inside a single wave: the score
+// MFMAs of sub-block sb+1 are issued BEFORE the softmax arithmetic of sub-block sb in program order, and do
+// not depend on it, so exp/max/rescale run in the shadow of those MFMAs.  MASKED = false is the interior
+// of the causal triangle (every key of the tile visible to every row of the wave).
+template <int HDP, int BC, bool MASKED>
+__device__ __forceinline__ void forwardTile(const float* __restrict__ ks, const float* __restrict__ vs,
+                                            const float (&qreg)[HDP / 2], float16v (&acc)[HDP / 32], float& mrow, float& lrow,
+                                            int kt0, int myLimit, int totalLen, int half, int li) {
+    constexpr int LDSW = HDP + 4, DT = HDP / 32, NSB = BC / 32;
+    float16v s[NSB];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[0][r] = 0.0f;
+    s[0] = headDot<HDP>(ks + li * LDSW + half * (HDP / 2), qreg, s[0]);
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+        if (sb + 1 < NSB) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[sb + 1][r] = 0.0f;
+            s[sb + 1] = headDot<HDP>(ks + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), qreg, s[sb + 1]);
+        }
+        float16v& sc = s[sb];   // sc[r] = log2-scaled score of (key = kt0 + sb*32 + dRow(r), this lane's query)
+        if constexpr (MASKED) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int key = kt0 + sb * 32 + dRow(r, half);
+                sc[r] = (key > myLimit || key >= totalLen) ? -INFINITY : sc[r];
+            }
+        }
+        float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+#pragma unroll
+        for (int r = 4; r < 16; r += 4) mx = fmaxf(mx, fmaxf(fmaxf(sc[r], sc[r + 1]), fmaxf(sc[r + 2], sc[r + 3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mnew = fmaxf(mrow, mx);
+        const float corr = fastExp2(mrow - mnew);
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { sc[r] = fastExp2(sc[r] - mnew); psum += sc[r]; }
+        lrow = lrow * corr + psum;
+        mrow = mnew;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+        // O^T += V^T * P^T : step r contracts over key dRow(r, half)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float* vrow = vs + (sb * 32 + dRow(r, half)) * LDSW + li;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[dt * 32], sc[r], acc[dt], 0, 0, 0);
+        }
+    }
+}
+
 template <int HDP, int BC, bool VEC4>
 __global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
     constexpr int LDSW = HDP + 4, DT = HDP / 32;
@@ -202,51 +305,22 @@ __global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
     const int waveKeyEnd = p.oldLen + waveQ0 + 32;                       // keys >= this are invisible to the wave
     const int myLimit = p.oldLen + i;                                    // last visible key of this lane's row
 
+    TileRegs<HDP, BC> kNext, vNext;
+    fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, 0, p.totalLen, hd, tid);
+    fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, 0, p.totalLen, hd, tid);
     for (int kt0 = 0; kt0 < blockKeyEnd; kt0 += BC) {
-        loadHeadTile<HDP, BC, VEC4>(ks, kb, dim, kt0, p.totalLen, hd, tid);
-        loadHeadTile<HDP, BC, VEC4>(vs, vb, dim, kt0, p.totalLen, hd, tid);
+        commitHeadTile<HDP, BC>(ks, kNext, tid);
+        commitHeadTile<HDP, BC>(vs, vNext, tid);
         __syncthreads();
-#pragma unroll
-        for (int sb = 0; sb < BC / 32; ++sb) {
-            const int key0 = kt0 + sb * 32;
-            if (key0 < waveKeyEnd && key0 < p.totalLen) {   // wave-uniform
-                float16v s;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) s[r] = 0.0f;
-                s = headDot<HDP>(ks + (sb * 32 + li) * LDSW + half * (HDP / 2), qreg, s);
-                // s[r] = log2-scaled score of (key = key0 + dRow(r), query = i)
-                const bool needMask = (key0 + 31 > p.oldLen + waveQ0) || (key0 + 32 > p.totalLen);
-                if (needMask) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        int key = key0 + dRow(r, half);
-                        if (key > myLimit || key >= p.totalLen) s[r] = -INFINITY;
-                    }
-                }
-                float mx = s[0];
-#pragma unroll
-                for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float mnew = fmaxf(mrow, mx);
-                const float corr = fastExp2(mrow - mnew);
-                float psum = 0.0f;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { s[r] = fastExp2(s[r] - mnew); psum += s[r]; }
-                lrow = lrow * corr + psum;
-                mrow = mnew;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
-                // O^T += V^T * P^T : step r contracts over key dRow(r, half)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float* vrow = vs + (sb * 32 + dRow(r, half)) * LDSW + li;
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
-                        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[dt * 32], s[r], acc[dt], 0, 0, 0);
-                }
-            }
+        if (kt0 + BC < blockKeyEnd) {   // next tile's loads fly while this tile is consumed
+            fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, kt0 + BC, p.totalLen, hd, tid);
+            fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, kt0 + BC, p.totalLen, hd, tid);
+        }
+        if (kt0 < waveKeyEnd) {   // wave-uniform: the tile holds keys some row of this wave can see
+            // the whole tile is visible to every row of the wave -> no masking arithmetic at all
+            const bool masked = (kt0 + BC - 1 > p.oldLen + waveQ0) || (kt0 + BC > p.totalLen);
+            if (masked) forwardTile<HDP, BC, true>(ks, vs, qreg, acc, mrow, lrow, kt0, myLimit, p.totalLen, half, li);
+            else forwardTile<HDP, BC, false>(ks, vs, qreg, acc, mrow, lrow, kt0, myLimit, p.totalLen, half, li);
         }
         __syncthreads();
     }
@@ -338,10 +412,17 @@ __global__ void __launch_bounds__(256) attnBackwardDqKernel(AttnParams p) {
     const int waveKeyEnd = p.oldLen + waveQ0 + 32;
     const int myLimit = p.oldLen + i;
 
+    TileRegs<HDP, BC> kNext, vNext;
+    fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, 0, p.totalLen, hd, tid);
+    fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, 0, p.totalLen, hd, tid);
     for (int kt0 = 0; kt0 < blockKeyEnd; kt0 += BC) {
-        loadHeadTile<HDP, BC, VEC4>(ks, kb, dim, kt0, p.totalLen, hd, tid);
-        loadHeadTile<HDP, BC, VEC4>(vs, vb, dim, kt0, p.totalLen, hd, tid);
+        commitHeadTile<HDP, BC>(ks, kNext, tid);
+        commitHeadTile<HDP, BC>(vs, vNext, tid);
         __syncthreads();
+        if (kt0 + BC < blockKeyEnd) {   // next tile's loads fly while this tile is consumed
+            fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, kt0 + BC, p.totalLen, hd, tid);
+            fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, kt0 + BC, p.totalLen, hd, tid);
+        }
 #pragma unroll
         for (int sb = 0; sb < BC / 32; ++sb) {
             const int key0 = kt0 + sb * 32;
@@ -416,15 +497,32 @@ __global__ void __launch_bounds__(256) attnBackwardDkvKernel(AttnParams p) {
     if (firstQuery < 0) firstQuery = 0;
     const int q0Start = (firstQuery / BQ) * BQ;
 
+    TileRegs<HDP, BQ> qNext, gNext;
+    float lseNext = INFINITY, dNext = 0.0f;
+    auto fetchStats = [&](int qt0) {
+        int qi = qt0 + tid;
+        bool ok = tid < BQ && qi < p.newLen;
+        lseNext = ok ? p.lse2[statOff + qi] : INFINITY;
+        dNext = ok ? p.dvec[statOff + qi] : 0.0f;
+    };
+    if (q0Start < p.newLen) {
+        fetchHeadTile<HDP, BQ, VEC4>(qNext, p.q + qOff, dim, q0Start, p.newLen, hd, tid);
+        fetchHeadTile<HDP, BQ, VEC4>(gNext, p.dO + qOff, dim, q0Start, p.newLen, hd, tid);
+        fetchStats(q0Start);
+    }
     for (int qt0 = q0Start; qt0 < p.newLen; qt0 += BQ) {
-        loadHeadTile<HDP, BQ, VEC4>(qs, p.q + qOff, dim, qt0, p.newLen, hd, tid);
-        loadHeadTile<HDP, BQ, VEC4>(gs, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+        commitHeadTile<HDP, BQ>(qs, qNext, tid);
+        commitHeadTile<HDP, BQ>(gs, gNext, tid);
         if (tid < BQ) {
-            int qi = qt0 + tid;
-            lses[tid] = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
-            dvs[tid] = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
+            lses[tid] = lseNext;
+            dvs[tid] = dNext;
         }
         __syncthreads();
+        if (qt0 + BQ < p.newLen) {
+            fetchHeadTile<HDP, BQ, VEC4>(qNext, p.q + qOff, dim, qt0 + BQ, p.newLen, hd, tid);
+            fetchHeadTile<HDP, BQ, VEC4>(gNext, p.dO + qOff, dim, qt0 + BQ, p.newLen, hd, tid);
+            fetchStats(qt0 + BQ);
+        }
 #pragma unroll
         for (int sb = 0; sb < BQ / 32; ++sb) {
             const int q0 = qt0 + sb * 32;
