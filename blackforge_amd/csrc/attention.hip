@@ -4,7 +4,8 @@
 // (absolute position oldLen+i) attends to keys j <= oldLen+i.
 //
 // Three MFMA kernels, all with 256-thread workgroups (4 wavefronts, one per SIMD), 32 rows per wave:
-//   forward : a workgroup owns 128 query rows, streams K/V tiles through LDS, online softmax.
+//   forward : a workgroup owns 128 query rows, streams K/V tiles through LDS (double buffered, one barrier
+//             per tile, next tile's global loads in flight in registers), online softmax.
 //   dQ      : same ownership; recomputes P from the saved statistics, accumulates dQ in registers.
 //   dK/dV   : a workgroup owns 128 keys (K, V and both accumulators live in registers), streams
 //             Q/dO tiles through LDS, writes dK and dV once.  No atomics anywhere, so gradients are
@@ -62,35 +63,9 @@ __device__ __forceinline__ void decodeBlock(int numTiles, int totalBlocks, bool 
 }
 
 // Cooperative copy of ROWS rows of one head ([row][hd] slices of a [.., dim] tensor) into LDS as
-// [ROWS][HDP+4], zero-filling rows >= rowLimit and columns >= hd.
-template <int HDP, int ROWS, bool VEC4>
-__device__ __forceinline__ void loadHeadTile(float* __restrict__ lds, const float* __restrict__ base, int dim, int row0,
-                                             int rowLimit, int hd, int tid) {
-    constexpr int LDSW = HDP + 4;
-    constexpr int V4 = HDP / 4;              // float4 slots per row
-    constexpr int SLOTS = ROWS * V4;
-#pragma unroll
-    for (int s = tid; s < SLOTS; s += 256) {
-        int r = s / V4, c = (s % V4) * 4;
-        int row = row0 + r;
-        float4v val = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (row < rowLimit && c < hd) {
-            const float* src = base + size_t(row) * dim + c;
-            if constexpr (VEC4) {
-                val = loadf4(src);
-            } else {
-                val.x = src[0];
-                if (c + 1 < hd) val.y = src[1];
-                if (c + 2 < hd) val.z = src[2];
-                if (c + 3 < hd) val.w = src[3];
-            }
-        }
-        storef4(lds + r * LDSW + c, val);
-    }
-}
-
-// The same copy split in two so that the global loads of the NEXT tile are in flight while the current
-// tile is being consumed: fetchHeadTile issues the loads into registers, commitHeadTile writes them to LDS.
+// [ROWS][HDP+4], zero-filling rows >= rowLimit and columns >= hd.  Split in two so that the global loads of
+// a LATER tile are in flight while the current one is being consumed: fetchHeadTile issues the loads into
+// registers, commitHeadTile writes them to LDS.
 template <int HDP, int ROWS>
 struct TileRegs {
     static constexpr int kSlots = (ROWS * (HDP / 4) + 255) / 256;
@@ -271,12 +246,16 @@ __device__ __forceinline__ void forwardTile(const float* __restrict__ ks, const 
     }
 }
 
+// Streaming schedule shared by the three kernels (LDS double buffering, ONE barrier per tile):
+//   iteration t consumes buffer t&1, then writes tile t+1 (already in registers) into buffer (t+1)&1 and
+//   issues the global loads of tile t+2; the barrier at the end of the iteration both publishes tile t+1
+//   and guarantees every wave is done reading buffer t&1 before iteration t+1 overwrites it with tile t+2.
 template <int HDP, int BC, bool VEC4>
 __global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
-    constexpr int LDSW = HDP + 4, DT = HDP / 32;
+    constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BC * LDSW;
     extern __shared__ float smem[];
-    float* ks = smem;
-    float* vs = smem + BC * LDSW;
+    float* ks = smem;               // [2][BC][LDSW]
+    float* vs = smem + 2 * TILE;    // [2][BC][LDSW]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
     int bh, qt;
@@ -304,23 +283,35 @@ __global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
     const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);   // keys >= this are invisible to the tile
     const int waveKeyEnd = p.oldLen + waveQ0 + 32;                       // keys >= this are invisible to the wave
     const int myLimit = p.oldLen + i;                                    // last visible key of this lane's row
+    const int numKeyTiles = (blockKeyEnd + BC - 1) / BC;
 
     TileRegs<HDP, BC> kNext, vNext;
     fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, 0, p.totalLen, hd, tid);
     fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, 0, p.totalLen, hd, tid);
-    for (int kt0 = 0; kt0 < blockKeyEnd; kt0 += BC) {
-        commitHeadTile<HDP, BC>(ks, kNext, tid);
-        commitHeadTile<HDP, BC>(vs, vNext, tid);
-        __syncthreads();
-        if (kt0 + BC < blockKeyEnd) {   // next tile's loads fly while this tile is consumed
-            fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, kt0 + BC, p.totalLen, hd, tid);
-            fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, kt0 + BC, p.totalLen, hd, tid);
-        }
+    commitHeadTile<HDP, BC>(ks, kNext, tid);
+    commitHeadTile<HDP, BC>(vs, vNext, tid);
+    if (numKeyTiles > 1) {
+        fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, BC, p.totalLen, hd, tid);
+        fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, BC, p.totalLen, hd, tid);
+    }
+    __syncthreads();
+    for (int t = 0; t < numKeyTiles; ++t) {
+        const int kt0 = t * BC;
+        const float* kcur = ks + (t & 1) * TILE;
+        const float* vcur = vs + (t & 1) * TILE;
         if (kt0 < waveKeyEnd) {   // wave-uniform: the tile holds keys some row of this wave can see
-            // the whole tile is visible to every row of the wave -> no masking arithmetic at all
+            // interior of the causal triangle: every key visible to every row of the wave, no masking arithmetic
             const bool masked = (kt0 + BC - 1 > p.oldLen + waveQ0) || (kt0 + BC > p.totalLen);
-            if (masked) forwardTile<HDP, BC, true>(ks, vs, qreg, acc, mrow, lrow, kt0, myLimit, p.totalLen, half, li);
-            else forwardTile<HDP, BC, false>(ks, vs, qreg, acc, mrow, lrow, kt0, myLimit, p.totalLen, half, li);
+            if (masked) forwardTile<HDP, BC, true>(kcur, vcur, qreg, acc, mrow, lrow, kt0, myLimit, p.totalLen, half, li);
+            else forwardTile<HDP, BC, false>(kcur, vcur, qreg, acc, mrow, lrow, kt0, myLimit, p.totalLen, half, li);
+        }
+        if (t + 1 < numKeyTiles) {
+            commitHeadTile<HDP, BC>(ks + ((t + 1) & 1) * TILE, kNext, tid);
+            commitHeadTile<HDP, BC>(vs + ((t + 1) & 1) * TILE, vNext, tid);
+            if (t + 2 < numKeyTiles) {
+                fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, kt0 + 2 * BC, p.totalLen, hd, tid);
+                fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, kt0 + 2 * BC, p.totalLen, hd, tid);
+            }
         }
         __syncthreads();
     }
@@ -375,12 +366,53 @@ __global__ void __launch_bounds__(256) attnDotKernel(const float* __restrict__ o
 // ---------------------------------------------------------------------------------------------
 // backward, part 1: dQ (query-tile owner).  Same streaming structure as the forward.
 // ---------------------------------------------------------------------------------------------
+// One K/V tile for one wavefront, straight-line and software-pipelined like forwardTile: the S^T and dP^T
+// MFMAs of sub-block sb+1 are issued before the exp / dS arithmetic of sub-block sb.
+template <int HDP, int BC, bool MASKED>
+__device__ __forceinline__ void dqTile(const float* __restrict__ ks, const float* __restrict__ vs, const float (&qreg)[HDP / 2],
+                                       const float (&greg)[HDP / 2], float16v (&acc)[HDP / 32], float lse, float dval, int kt0,
+                                       int myLimit, int totalLen, int half, int li) {
+    constexpr int LDSW = HDP + 4, DT = HDP / 32, NSB = BC / 32;
+    float16v s[NSB], dp[NSB];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s[0][r] = 0.0f; dp[0][r] = 0.0f; }
+    s[0] = headDot<HDP>(ks + li * LDSW + half * (HDP / 2), qreg, s[0]);      // S^T  = K * Q^T
+    dp[0] = headDot<HDP>(vs + li * LDSW + half * (HDP / 2), greg, dp[0]);    // dP^T = V * dO^T
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+        if (sb + 1 < NSB) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { s[sb + 1][r] = 0.0f; dp[sb + 1][r] = 0.0f; }
+            s[sb + 1] = headDot<HDP>(ks + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), qreg, s[sb + 1]);
+            dp[sb + 1] = headDot<HDP>(vs + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), greg, dp[sb + 1]);
+        }
+        float16v& ds = s[sb];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float prob = fastExp2(ds[r] - lse);
+            if constexpr (MASKED) {
+                int key = kt0 + sb * 32 + dRow(r, half);
+                prob = (key > myLimit || key >= totalLen) ? 0.0f : prob;
+            }
+            ds[r] = prob * (dp[sb][r] - dval);   // dS^T (without the scale factor)
+        }
+        // dQ^T += K^T * dS^T : step r contracts over key dRow(r, half)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float* krow = ks + (sb * 32 + dRow(r, half)) * LDSW + li;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[dt * 32], ds[r], acc[dt], 0, 0, 0);
+        }
+    }
+}
+
 template <int HDP, int BC, bool VEC4>
 __global__ void __launch_bounds__(256) attnBackwardDqKernel(AttnParams p) {
-    constexpr int LDSW = HDP + 4, DT = HDP / 32;
+    constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BC * LDSW;
     extern __shared__ float smem[];
     float* ks = smem;
-    float* vs = smem + BC * LDSW;
+    float* vs = smem + 2 * TILE;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
     int bh, qt;
@@ -411,45 +443,33 @@ __global__ void __launch_bounds__(256) attnBackwardDqKernel(AttnParams p) {
     const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);
     const int waveKeyEnd = p.oldLen + waveQ0 + 32;
     const int myLimit = p.oldLen + i;
+    const int numKeyTiles = (blockKeyEnd + BC - 1) / BC;
 
     TileRegs<HDP, BC> kNext, vNext;
     fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, 0, p.totalLen, hd, tid);
     fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, 0, p.totalLen, hd, tid);
-    for (int kt0 = 0; kt0 < blockKeyEnd; kt0 += BC) {
-        commitHeadTile<HDP, BC>(ks, kNext, tid);
-        commitHeadTile<HDP, BC>(vs, vNext, tid);
-        __syncthreads();
-        if (kt0 + BC < blockKeyEnd) {   // next tile's loads fly while this tile is consumed
-            fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, kt0 + BC, p.totalLen, hd, tid);
-            fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, kt0 + BC, p.totalLen, hd, tid);
+    commitHeadTile<HDP, BC>(ks, kNext, tid);
+    commitHeadTile<HDP, BC>(vs, vNext, tid);
+    if (numKeyTiles > 1) {
+        fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, BC, p.totalLen, hd, tid);
+        fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, BC, p.totalLen, hd, tid);
+    }
+    __syncthreads();
+    for (int t = 0; t < numKeyTiles; ++t) {
+        const int kt0 = t * BC;
+        const float* kcur = ks + (t & 1) * TILE;
+        const float* vcur = vs + (t & 1) * TILE;
+        if (kt0 < waveKeyEnd) {
+            const bool masked = (kt0 + BC - 1 > p.oldLen + waveQ0) || (kt0 + BC > p.totalLen);
+            if (masked) dqTile<HDP, BC, true>(kcur, vcur, qreg, greg, acc, lse, dval, kt0, myLimit, p.totalLen, half, li);
+            else dqTile<HDP, BC, false>(kcur, vcur, qreg, greg, acc, lse, dval, kt0, myLimit, p.totalLen, half, li);
         }
-#pragma unroll
-        for (int sb = 0; sb < BC / 32; ++sb) {
-            const int key0 = kt0 + sb * 32;
-            if (key0 < waveKeyEnd && key0 < p.totalLen) {
-                float16v s, dp;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { s[r] = 0.0f; dp[r] = 0.0f; }
-                s = headDot<HDP>(ks + (sb * 32 + li) * LDSW + half * (HDP / 2), qreg, s);     // S^T  = K  * Q^T
-                dp = headDot<HDP>(vs + (sb * 32 + li) * LDSW + half * (HDP / 2), greg, dp);   // dP^T = V  * dO^T
-                const bool needMask = (key0 + 31 > p.oldLen + waveQ0) || (key0 + 32 > p.totalLen);
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    float prob = fastExp2(s[r] - lse);
-                    if (needMask) {
-                        int key = key0 + dRow(r, half);
-                        if (key > myLimit || key >= p.totalLen) prob = 0.0f;
-                    }
-                    s[r] = prob * (dp[r] - dval);   // dS^T (without the scale factor)
-                }
-                // dQ^T += K^T * dS^T : step r contracts over key dRow(r, half)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float* krow = ks + (sb * 32 + dRow(r, half)) * LDSW + li;
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
-                        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[dt * 32], s[r], acc[dt], 0, 0, 0);
-                }
+        if (t + 1 < numKeyTiles) {
+            commitHeadTile<HDP, BC>(ks + ((t + 1) & 1) * TILE, kNext, tid);
+            commitHeadTile<HDP, BC>(vs + ((t + 1) & 1) * TILE, vNext, tid);
+            if (t + 2 < numKeyTiles) {
+                fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, kt0 + 2 * BC, p.totalLen, hd, tid);
+                fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, kt0 + 2 * BC, p.totalLen, hd, tid);
             }
         }
         __syncthreads();
@@ -461,14 +481,66 @@ __global__ void __launch_bounds__(256) attnBackwardDqKernel(AttnParams p) {
 // backward, part 2: dK, dV (key-tile owner).  K and V of the wave's 32 keys stay in registers as MFMA
 // B operands; Q/dO tiles and the per-row statistics are streamed through LDS.
 // ---------------------------------------------------------------------------------------------
+// One Q/dO tile (BQ queries) for one wavefront, straight-line and software-pipelined.
+// stats: [0..BQ) = lse2 of the tile's queries (+inf for padding rows), [BQ..2BQ) = D.
+template <int HDP, int BQ, bool MASKED>
+__device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const float* __restrict__ gs, const float* __restrict__ stats,
+                                        const float (&kreg)[HDP / 2], const float (&vreg)[HDP / 2], float16v (&dk)[HDP / 32],
+                                        float16v (&dv)[HDP / 32], int qt0, int key, bool keyValid, int oldLen, int half, int li) {
+    constexpr int LDSW = HDP + 4, DT = HDP / 32, NSB = BQ / 32;
+    float16v s[NSB], dp[NSB];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s[0][r] = 0.0f; dp[0][r] = 0.0f; }
+    s[0] = headDotB<HDP>(qs + li * LDSW + half * (HDP / 2), kreg, s[0]);     // S  = Q  * K^T
+    dp[0] = headDotB<HDP>(gs + li * LDSW + half * (HDP / 2), vreg, dp[0]);   // dP = dO * V^T
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+        if (sb + 1 < NSB) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { s[sb + 1][r] = 0.0f; dp[sb + 1][r] = 0.0f; }
+            s[sb + 1] = headDotB<HDP>(qs + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), kreg, s[sb + 1]);
+            dp[sb + 1] = headDotB<HDP>(gs + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), vreg, dp[sb + 1]);
+        }
+        // register r: query = qt0 + sb*32 + dRow(r, half), key = this lane's key
+        float16v& pr = s[sb];
+        float16v& dsv = dp[sb];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float4v lse4 = loadf4(stats + sb * 32 + 8 * g + 4 * half);
+            float4v d4 = loadf4(stats + BQ + sb * 32 + 8 * g + 4 * half);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int r = 4 * g + c;
+                float prob = fastExp2(pr[r] - lse4[c]);
+                if constexpr (MASKED) {
+                    int qi = qt0 + sb * 32 + dRow(r, half);
+                    prob = (key > oldLen + qi || !keyValid) ? 0.0f : prob;
+                }
+                pr[r] = prob;                          // P
+                dsv[r] = prob * (dsv[r] - d4[c]);      // dS (without the scale factor)
+            }
+        }
+        // dV += P^T * dO, dK += dS^T * Q : step r contracts over query dRow(r, half)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float* grow = gs + (sb * 32 + dRow(r, half)) * LDSW + li;
+            const float* qrow = qs + (sb * 32 + dRow(r, half)) * LDSW + li;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                dv[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pr[r], grow[dt * 32], dv[dt], 0, 0, 0);
+                dk[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(dsv[r], qrow[dt * 32], dk[dt], 0, 0, 0);
+            }
+        }
+    }
+}
+
 template <int HDP, int BQ, bool VEC4>
 __global__ void __launch_bounds__(256) attnBackwardDkvKernel(AttnParams p) {
-    constexpr int LDSW = HDP + 4, DT = HDP / 32;
+    constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BQ * LDSW;
     extern __shared__ float smem[];
-    float* qs = smem;
-    float* gs = smem + BQ * LDSW;
-    float* lses = gs + BQ * LDSW;   // [BQ]
-    float* dvs = lses + BQ;         // [BQ]
+    float* qs = smem;                   // [2][BQ][LDSW]
+    float* gs = smem + 2 * TILE;        // [2][BQ][LDSW]
+    float* stats = smem + 4 * TILE;     // [2][2*BQ]: lse2 | D
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
     int bh, kt;
@@ -496,73 +568,46 @@ __global__ void __launch_bounds__(256) attnBackwardDkvKernel(AttnParams p) {
     int firstQuery = kt * 128 - p.oldLen;
     if (firstQuery < 0) firstQuery = 0;
     const int q0Start = (firstQuery / BQ) * BQ;
+    const int numQTiles = q0Start < p.newLen ? (p.newLen - q0Start + BQ - 1) / BQ : 0;
 
     TileRegs<HDP, BQ> qNext, gNext;
-    float lseNext = INFINITY, dNext = 0.0f;
-    auto fetchStats = [&](int qt0) {
-        int qi = qt0 + tid;
-        bool ok = tid < BQ && qi < p.newLen;
-        lseNext = ok ? p.lse2[statOff + qi] : INFINITY;
-        dNext = ok ? p.dvec[statOff + qi] : 0.0f;
+    float statNext = 0.0f;
+    auto fetchStats = [&](int qt0) {   // thread t < BQ: lse2 of query qt0+t; BQ <= t < 2BQ: D of query qt0+t-BQ
+        const int j = tid < BQ ? tid : tid - BQ;
+        const int qi = qt0 + j;
+        if (tid < BQ) statNext = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
+        else if (tid < 2 * BQ) statNext = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
     };
-    if (q0Start < p.newLen) {
-        fetchHeadTile<HDP, BQ, VEC4>(qNext, p.q + qOff, dim, q0Start, p.newLen, hd, tid);
-        fetchHeadTile<HDP, BQ, VEC4>(gNext, p.dO + qOff, dim, q0Start, p.newLen, hd, tid);
-        fetchStats(q0Start);
+    auto commitAll = [&](int buf) {
+        commitHeadTile<HDP, BQ>(qs + buf * TILE, qNext, tid);
+        commitHeadTile<HDP, BQ>(gs + buf * TILE, gNext, tid);
+        if (tid < 2 * BQ) stats[buf * 2 * BQ + tid] = statNext;
+    };
+    auto fetchAll = [&](int qt0) {
+        fetchHeadTile<HDP, BQ, VEC4>(qNext, p.q + qOff, dim, qt0, p.newLen, hd, tid);
+        fetchHeadTile<HDP, BQ, VEC4>(gNext, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+        fetchStats(qt0);
+    };
+    if (numQTiles > 0) {
+        fetchAll(q0Start);
+        commitAll(0);
+        if (numQTiles > 1) fetchAll(q0Start + BQ);
     }
-    for (int qt0 = q0Start; qt0 < p.newLen; qt0 += BQ) {
-        commitHeadTile<HDP, BQ>(qs, qNext, tid);
-        commitHeadTile<HDP, BQ>(gs, gNext, tid);
-        if (tid < BQ) {
-            lses[tid] = lseNext;
-            dvs[tid] = dNext;
+    __syncthreads();
+    for (int t = 0; t < numQTiles; ++t) {
+        const int qt0 = q0Start + t * BQ;
+        // the wave's keys [waveK0, waveK0+32) are visible to some query of the tile?
+        if (p.oldLen + qt0 + BQ - 1 >= waveK0 && waveK0 < p.totalLen) {
+            const bool masked = (waveK0 + 31 > p.oldLen + qt0) || (waveK0 + 32 > p.totalLen);
+            const float* qcur = qs + (t & 1) * TILE;
+            const float* gcur = gs + (t & 1) * TILE;
+            const float* scur = stats + (t & 1) * 2 * BQ;
+            if (masked) dkvTile<HDP, BQ, true>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li);
+            else dkvTile<HDP, BQ, false>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li);
         }
-        __syncthreads();
-        if (qt0 + BQ < p.newLen) {
-            fetchHeadTile<HDP, BQ, VEC4>(qNext, p.q + qOff, dim, qt0 + BQ, p.newLen, hd, tid);
-            fetchHeadTile<HDP, BQ, VEC4>(gNext, p.dO + qOff, dim, qt0 + BQ, p.newLen, hd, tid);
-            fetchStats(qt0 + BQ);
-        }
-#pragma unroll
-        for (int sb = 0; sb < BQ / 32; ++sb) {
-            const int q0 = qt0 + sb * 32;
-            // the wave's keys [waveK0, waveK0+32) are visible to some query of [q0, q0+32)?
-            if (q0 < p.newLen && p.oldLen + q0 + 31 >= waveK0 && waveK0 < p.totalLen) {
-                float16v s, dp;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { s[r] = 0.0f; dp[r] = 0.0f; }
-                s = headDotB<HDP>(qs + (sb * 32 + li) * LDSW + half * (HDP / 2), kreg, s);    // S  = Q  * K^T
-                dp = headDotB<HDP>(gs + (sb * 32 + li) * LDSW + half * (HDP / 2), vreg, dp);  // dP = dO * V^T
-                // register r: query = q0 + dRow(r, half), key = this lane's key
-                const bool needMask = (waveK0 + 31 > p.oldLen + q0) || (waveK0 + 32 > p.totalLen);
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    float4v lse4 = loadf4(lses + sb * 32 + 8 * g + 4 * half);
-                    float4v d4 = loadf4(dvs + sb * 32 + 8 * g + 4 * half);
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const int r = 4 * g + c;
-                        float prob = fastExp2(s[r] - lse4[c]);
-                        if (needMask) {
-                            int qi = q0 + dRow(r, half);
-                            if (key > p.oldLen + qi || !keyValid) prob = 0.0f;
-                        }
-                        s[r] = prob;                        // P
-                        dp[r] = prob * (dp[r] - d4[c]);     // dS (without the scale factor)
-                    }
-                }
-                // dV += P^T * dO, dK += dS^T * Q : step r contracts over query dRow(r, half)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float* grow = gs + (sb * 32 + dRow(r, half)) * LDSW + li;
-                    const float* qrow = qs + (sb * 32 + dRow(r, half)) * LDSW + li;
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        dv[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(s[r], grow[dt * 32], dv[dt], 0, 0, 0);
-                        dk[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(dp[r], qrow[dt * 32], dk[dt], 0, 0, 0);
-                    }
-                }
-            }
+        if (t + 1 < numQTiles) {
+            commitAll((t + 1) & 1);
+            if (t + 2 < numQTiles) fetchAll(qt0 + 2 * BQ);
         }
         __syncthreads();
     }
@@ -609,8 +654,8 @@ bool vec4Ok(const AttnParams& p, std::initializer_list<const void*> ptrs) {
 // KIND 0 forward, 1 dQ, 2 dK/dV
 template <int KIND, int HDP, int TILE>
 int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
-    constexpr size_t tileBytes = size_t(2) * TILE * (HDP + 4) * sizeof(float);
-    constexpr size_t smem = KIND == 2 ? tileBytes + 2 * TILE * sizeof(float) : tileBytes;
+    constexpr size_t tileBytes = size_t(4) * TILE * (HDP + 4) * sizeof(float);   // two operands, double buffered
+    constexpr size_t smem = KIND == 2 ? tileBytes + 4 * TILE * sizeof(float) : tileBytes;
     if constexpr (KIND == 0) {
         return vec4 ? launchAttn(attnForwardKernel<HDP, TILE, true>, smem, grid, p, s)
                     : launchAttn(attnForwardKernel<HDP, TILE, false>, smem, grid, p, s);
