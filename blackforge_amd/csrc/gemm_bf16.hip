@@ -78,80 +78,111 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(const float* __
 }
 
 // ---- the GEMM ----------------------------------------------------------------------------------
-constexpr int BM = 128, BN = 128, BKK = 64;
-constexpr int LDS_ROW = BKK + 8;   // bf16 elements per LDS row (16-byte pad)
+// C[M,N] = A[M,K] * Bt[N,K]^T.  A workgroup of WAVES_M x WAVES_N wavefronts owns a BM x BN tile; each
+// wavefront a (BM/WAVES_M) x (BN/WAVES_N) sub-tile made of 32x32 MFMA accumulators.  K advances in steps
+// of 64 through a double-buffered LDS stage with one barrier per step: while step t is being multiplied
+// out of buffer t&1, the registers holding step t+1 are written to the other buffer and the global loads
+// of step t+2 are issued.
+constexpr int BKK = 64;
+constexpr int LDS_ROW = BKK + 8;   // bf16 elements per LDS row: 128 B of data + 16 B pad (conflict-free b128 reads)
 
-__global__ void __launch_bounds__(256) gemmBf16NtKernel(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
-                                                         float* __restrict__ C, int M, int N, int K, int lda, int ldb) {
-    __shared__ __attribute__((aligned(16))) unsigned short as[BM * LDS_ROW];
-    __shared__ __attribute__((aligned(16))) unsigned short bs[BN * LDS_ROW];
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const unsigned short* __restrict__ A,
+                                                                            const unsigned short* __restrict__ Bt,
+                                                                            float* __restrict__ C, int M, int N, int K, int lda,
+                                                                            int ldb) {
+    constexpr int THREADS = WAVES_M * WAVES_N * 64;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;     // per-wave tile
+    constexpr int TM = WM / 32, TN = WN / 32;               // 32x32 accumulators per wave
+    constexpr int ROWS_PER_PASS = THREADS / 8;              // 8 threads (16 B each) cover one 128-byte row
+    constexpr int A_PASSES = BM / ROWS_PER_PASS, B_PASSES = BN / ROWS_PER_PASS;
+    static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "tile rows must be a multiple of the rows loaded per pass");
+    extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
+    unsigned short* as = lds;                              // [2][BM][LDS_ROW]
+    unsigned short* bs = lds + 2 * BM * LDS_ROW;           // [2][BN][LDS_ROW]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
-    // XCD-aware tile order: the 8 XCDs take workgroups round-robin; give each XCD a contiguous band of
-    // tiles so A/Bt panels are reused out of its own L2.
-    int id = blockIdx.x;
-    const int total = gridDim.x;
-    if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
-    const int tilesN = (N + BN - 1) / BN;
-    const int m0 = (id / tilesN) * BM, n0 = (id % tilesN) * BN;
-    const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
+    // Tile order: groups of 8 tile-rows are walked column-first so that the tiles in flight at any time
+    // share A and Bt panels in L2; workgroups go round-robin to the 8 XCDs.
+    const int tilesM = (M + BM - 1) / BM, tilesN = (N + BN - 1) / BN;
+    int tm, tn;
+    {
+        constexpr int GROUP = 8;
+        const int id = blockIdx.x;
+        const int perGroup = GROUP * tilesN;
+        const int g = id / perGroup, rem = id - g * perGroup;
+        const int rowsInGroup = min(GROUP, tilesM - g * GROUP);
+        tm = g * GROUP + rem % rowsInGroup;
+        tn = rem / rowsInGroup;
+    }
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
 
-    // global -> register staging: thread t covers rows (t/8 + 32*i), 8 bf16 at column (t%8)*8
     const int lr = tid >> 3, lc = (tid & 7) * 8;
-    uint4v aReg[4], bReg[4];
+    uint4v aReg[A_PASSES], bReg[B_PASSES];
     auto loadGlobal = [&](int k0) {
+        const uint4v z = {0u, 0u, 0u, 0u};
+        const bool kOk = k0 + lc < K;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int r = lr + 32 * i;
-            uint4v z = {0u, 0u, 0u, 0u};
-            aReg[i] = (m0 + r < M && k0 + lc < K) ? *reinterpret_cast<const uint4v*>(A + size_t(m0 + r) * lda + k0 + lc) : z;
-            bReg[i] = (n0 + r < N && k0 + lc < K) ? *reinterpret_cast<const uint4v*>(Bt + size_t(n0 + r) * ldb + k0 + lc) : z;
+        for (int i = 0; i < A_PASSES; ++i) {
+            int r = m0 + lr + ROWS_PER_PASS * i;
+            aReg[i] = (r < M && kOk) ? *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k0 + lc) : z;
+        }
+#pragma unroll
+        for (int i = 0; i < B_PASSES; ++i) {
+            int r = n0 + lr + ROWS_PER_PASS * i;
+            bReg[i] = (r < N && kOk) ? *reinterpret_cast<const uint4v*>(Bt + size_t(r) * ldb + k0 + lc) : z;
         }
     };
-    auto storeLds = [&]() {
+    auto storeLds = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int r = lr + 32 * i;
-            *reinterpret_cast<uint4v*>(as + r * LDS_ROW + lc) = aReg[i];
-            *reinterpret_cast<uint4v*>(bs + r * LDS_ROW + lc) = bReg[i];
-        }
+        for (int i = 0; i < A_PASSES; ++i)
+            *reinterpret_cast<uint4v*>(as + (buf * BM + lr + ROWS_PER_PASS * i) * LDS_ROW + lc) = aReg[i];
+#pragma unroll
+        for (int i = 0; i < B_PASSES; ++i)
+            *reinterpret_cast<uint4v*>(bs + (buf * BN + lr + ROWS_PER_PASS * i) * LDS_ROW + lc) = bReg[i];
     };
 
-    float16v acc[2][2];
+    float16v acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
+    const int steps = (K + BKK - 1) / BKK;
     loadGlobal(0);
-    for (int k0 = 0; k0 < K; k0 += BKK) {
-        storeLds();
-        __syncthreads();
-        if (k0 + BKK < K) loadGlobal(k0 + BKK);
+    storeLds(0);
+    if (steps > 1) loadGlobal(BKK);
+    __syncthreads();
+    for (int t = 0; t < steps; ++t) {
+        const unsigned short* ac = as + ((t & 1) * BM + wm0 + li) * LDS_ROW + 8 * half;
+        const unsigned short* bc = bs + ((t & 1) * BN + wn0 + li) * LDS_ROW + 8 * half;
 #pragma unroll
         for (int kk = 0; kk < BKK; kk += 16) {
-            bf16x8 a[2], b[2];
+            bf16x8 a[TM], b[TN];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                a[i] = *reinterpret_cast<const bf16x8*>(as + (wm0 + i * 32 + li) * LDS_ROW + kk + 8 * half);
+            for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const bf16x8*>(ac + i * 32 * LDS_ROW + kk);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                b[j] = *reinterpret_cast<const bf16x8*>(bs + (wn0 + j * 32 + li) * LDS_ROW + kk + 8 * half);
+            for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const bf16x8*>(bc + j * 32 * LDS_ROW + kk);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (t + 1 < steps) {
+            storeLds((t + 1) & 1);
+            if (t + 2 < steps) loadGlobal((t + 2) * BKK);
         }
         __syncthreads();
     }
 
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < TN; ++j) {
             const int col = n0 + wn0 + j * 32 + li;
             if (col < N) {
 #pragma unroll
@@ -163,14 +194,27 @@ __global__ void __launch_bounds__(256) gemmBf16NtKernel(const unsigned short* __
         }
 }
 
-int launchGemmNt(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda,
-                 size_t ldb, hipStream_t s) {
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+int launchTile(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda, size_t ldb,
+               hipStream_t s) {
     size_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    if (tiles >= (size_t(1) << 31) || M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31))
-        return failInvalid("gemm_bf16", "shape too large");
-    gemmBf16NtKernel<<<unsigned(tiles), 256, 0, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb));
+    if (tiles >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+    constexpr size_t smem = size_t(2) * (BM + BN) * LDS_ROW * sizeof(unsigned short);
+    auto kernel = gemmBf16NtKernel<BM, BN, WAVES_M, WAVES_N>;
+    if (smem > 48 * 1024)
+        BF_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+    kernel<<<unsigned(tiles), WAVES_M * WAVES_N * 64, smem, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb));
     BF_LAUNCH_CHECK();
     return BF_OK;
+}
+
+int launchGemmNt(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda,
+                 size_t ldb, hipStream_t s) {
+    if (M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+    // 256x256 tiles (8 wavefronts) once they give every CU at least one tile; otherwise 128x128 (4 wavefronts)
+    const size_t bigTiles = ((M + 255) / 256) * ((N + 255) / 256);
+    if (bigTiles >= size_t(computeUnits()) * 3 / 4) return launchTile<256, 256, 2, 4>(A, Bt, C, M, N, K, lda, ldb, s);
+    return launchTile<128, 128, 2, 2>(A, Bt, C, M, N, K, lda, ldb, s);
 }
 
 int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, hipStream_t s) {
