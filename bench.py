@@ -155,6 +155,71 @@ def bench_extras(bf, steps):
     return extras
 
 
+def lm_layers(hl, vocab, dim, seq, heads, hidden, act, blocks):
+    layers = [(hl.EMBEDDING, vocab, dim), (hl.POSITIONAL, seq)]
+    for _ in range(blocks):
+        layers += [(hl.ATTENTION, heads), (hl.FEEDFORWARD, hidden, act)]
+    return layers + [(hl.LINEAR, vocab)]
+
+
+TRAIN_CONFIGS = {
+    # name: (vocab, d_model, heads, blocks, ffn, activation (0 silu / 1 gelu), seq, batch, bf16, optimizer)
+    "tiny_lm": dict(vocab=256, dim=128, heads=4, blocks=1, ffn=512, act=1, seq=64, batch=8, bf16=False, adamw=True,
+                    what="BASELINE.json configs[0]: tiny LM, fp32, full step with AdamW"),
+    "gpt_small": dict(vocab=32000, dim=768, heads=12, blocks=12, ffn=3072, act=1, seq=1024, batch=8, bf16=True, adamw=True,
+                      what="BASELINE.json configs[3]: GPT-small shape, bf16 projections + fp32 attention, full step with sparse CE and AdamW"),
+    "long_context": dict(vocab=50257, dim=2048, heads=16, blocks=8, ffn=8192, act=0, seq=4096, batch=4, bf16=True, adamw=False,
+                         what="BASELINE.json configs[4]: long-context LM, bf16 projections, forward + backward with sparse CE"),
+}
+
+
+def train_step_flops(c):
+    """Algorithmic FLOPs of one step: 6*tokens*(matmul weights) + 14*hd*P per attention layer."""
+    tokens = c["batch"] * c["seq"]
+    weights = c["blocks"] * (4 * c["dim"] ** 2 + 2 * c["dim"] * c["ffn"]) + c["dim"] * c["vocab"]
+    pairs = c["batch"] * c["heads"] * c["seq"] * (c["seq"] + 1) // 2
+    return 6 * tokens * weights + c["blocks"] * 14 * (c["dim"] // c["heads"]) * pairs
+
+
+def bench_train_step(bf, name, steps, warmup):
+    """One training step of the C++ operator layer's Model (hip::Model) through its C harness."""
+    from blackforge_amd import hostlayer as hl
+    c = TRAIN_CONFIGS[name]
+    model = hl.HostModel(lm_layers(hl, c["vocab"], c["dim"], c["seq"], c["heads"], c["ffn"], c["act"], c["blocks"]), use_bf16=c["bf16"])
+    rng = np.random.default_rng(42)
+    n_params = 0
+    for i, count in enumerate(model.counts):
+        n_params += count
+        is_bias = model.names[i].endswith((".bias", ".b1", ".b2"))
+        model.set_value(i, np.zeros(count, np.float32) if is_bias else rng.standard_normal(count, dtype=np.float32) * np.float32(0.02))
+    D = bf.DeviceTensor
+    ids = D.fromHost(rng.integers(0, c["vocab"], (c["batch"], c["seq"])).astype(np.float32))
+    tgt = D.fromHost(rng.integers(0, c["vocab"], c["batch"] * c["seq"]).astype(np.float32))
+    opt = 1 if c["adamw"] else 0
+    step = lambda: model.trainStep(ids, tgt, hl.LOSS_SPARSE_CE, opt, 1e-3)
+    for _ in range(warmup):
+        step()
+    bf.capi.call("bf_hip_synchronize")
+    model.readLossSum()
+    start, stop = bf.Event(), bf.Event()
+    t0 = time.perf_counter()
+    start.record(None)
+    for _ in range(steps):
+        step()
+    stop.record(None)
+    stop.synchronize()
+    bf.capi.call("bf_hip_synchronize")
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms = start.elapsed_ms(stop) / steps
+    loss = model.readLossSum() / (steps * c["batch"] * c["seq"])
+    tokens = c["batch"] * c["seq"]
+    flops = train_step_flops(c)
+    return {"workload": c["what"], "tokens_per_s": round(tokens / (ms * 1e-3), 1), "ms_per_step": round(ms, 3),
+            "wall_ms_per_step": round(wall_ms, 3), "tokens": tokens, "parameters": n_params,
+            "algorithmic_tflop_per_step": round(flops / 1e12, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
+            "mean_loss": round(float(loss), 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -162,6 +227,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time a bandwidth kernel and the bf16 GEMM")
+    ap.add_argument("--train", default="gpt_small", help="comma list of train-step workloads to add (tiny_lm, gpt_small, "
+                    "long_context) or 'none'")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -206,6 +273,9 @@ def main():
         "wall_ms_per_step": round(res["wall_ms_per_step"], 4),
         "device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units},
     }
+    if args.train != "none":
+        line["train_step"] = {name: bench_train_step(bf, name, max(3, args.steps // 2), max(1, args.warmup // 2))
+                              for name in args.train.split(",")}
     if args.extras:
         line["extras"] = bench_extras(bf, max(5, args.steps // 2))
     if not args.no_cpu_baseline:
