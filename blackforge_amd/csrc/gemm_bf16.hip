@@ -11,10 +11,9 @@
 //     dB = a^T g            : A = bf16(a)^T      Bt = bf16(g)^T  (transposing converts)
 // Converted operands are padded with zeros to a multiple of 8 along K so the GEMM needs no K tail.
 //
-// Kernel: 256 threads (2 x 2 wavefronts), 128 x 128 tile of C per workgroup, 64 x 64 per wavefront
-// (four 32x32 accumulators), K step 64.  Global loads of the next K step are issued into registers
-// before the MFMAs of the current one and written to LDS afterwards (register double buffering).
-// LDS rows are padded by 16 bytes so the 16-byte operand reads of 8 consecutive lanes cover all banks.
+// Two kernels, picked by tile count: a 256x256-tile kernel whose eight wavefronts alternate between moving
+// data and multiplying (large products), and a 128x128-tile kernel with one barrier per K step, optionally
+// cutting K into slices that a second kernel adds up in a fixed order (small products).
 #include "common.hpp"
 
 #include <map>
@@ -78,19 +77,78 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(const float* __
 }
 
 // ---- the GEMM ----------------------------------------------------------------------------------
-// C[M,N] = A[M,K] * Bt[N,K]^T.  A workgroup of WAVES_M x WAVES_N wavefronts owns a BM x BN tile; each
-// wavefront a (BM/WAVES_M) x (BN/WAVES_N) sub-tile made of 32x32 MFMA accumulators.  K advances in steps
-// of 64 through a double-buffered LDS stage with one barrier per step: while step t is being multiplied
-// out of buffer t&1, the registers holding step t+1 are written to the other buffer and the global loads
-// of step t+2 are issued.
+// C[M,N] = A[M,K] * Bt[N,K]^T on 32x32x16 bf16 MFMAs.  Two kernels share the operand layout: LDS rows of
+// 64 bf16 (one 128-byte line of the operand) padded by 16 bytes, so that the 16-byte fragment reads of a
+// wavefront touch every bank once.  Rows past the end of an operand are clamped to its last row (their
+// products are never stored) and chunks past the end of the K range read as zero, so neither kernel has
+// a branch around a load.
 constexpr int BKK = 64;
-constexpr int LDS_ROW = BKK + 8;   // bf16 elements per LDS row: 128 B of data + 16 B pad (conflict-free b128 reads)
+constexpr int LDS_ROW = BKK + 8;
 
+// A 16-byte chunk of an operand row at column k, or of column 0 when k is past the end of the K range: the
+// caller replaces such a chunk by zeros when it consumes the register (zeroPast), not here, so that the load
+// stays in flight across the phases in between.
+__device__ __forceinline__ uint4v loadChunk(const unsigned short* __restrict__ row, int k, int kEnd) {
+    return *reinterpret_cast<const uint4v*>(row + (k < kEnd ? k : 0));
+}
+__device__ __forceinline__ uint4v zeroPast(uint4v v, int k, int kEnd) {
+    const uint4v z = {0u, 0u, 0u, 0u};
+    return k < kEnd ? v : z;
+}
+
+// Walks tile rows in groups of 8, column-first inside a group, so tiles in flight share operand panels.
+__device__ __forceinline__ void tileIndexGrouped(int id, int tilesM, int tilesN, int& tm, int& tn) {
+    constexpr int GROUP = 8;
+    const int perGroup = GROUP * tilesN;
+    const int g = id / perGroup, rem = id - g * perGroup;
+    const int rowsInGroup = min(GROUP, tilesM - g * GROUP);
+    tm = g * GROUP + rem % rowsInGroup;
+    tn = rem / rowsInGroup;
+}
+
+// Workgroups go round-robin to the 8 XCDs (id % 8), each with its own L2.  Here every XCD walks whole
+// blocks of 2^gmLog x 2^gnLog = 32 tiles, one per CU, so the 32 tiles an XCD works on at a time share
+// 2^gmLog + 2^gnLog operand panels in its L2 instead of 33.
+__device__ __forceinline__ bool tileIndexXcd(int id, int tilesM, int tilesN, int gmLog, int gnLog, int& tm, int& tn) {
+    const int x = id & 7, j = id >> 3;
+    const int blocksN = (tilesN + (1 << gnLog) - 1) >> gnLog, blocksM = (tilesM + (1 << gmLog) - 1) >> gmLog;
+    const int b = (j >> 5) * 8 + x, q = j & 31;
+    if (b >= blocksM * blocksN) return false;
+    const int bm = b / blocksN, bn = b - bm * blocksN;
+    tm = (bm << gmLog) + (q & ((1 << gmLog) - 1));
+    tn = (bn << gnLog) + (q >> gmLog);
+    return tm < tilesM && tn < tilesN;
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void storeAccumulators(float16v (&acc)[TM][TN], float* __restrict__ C, int M, int N, int row0,
+                                                  int col0, int li, int half) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = col0 + j * 32 + li;
+            if (col < N) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = row0 + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                    if (row < M) C[size_t(row) * N + col] = acc[i][j][r];
+                }
+            }
+        }
+}
+
+// Kernel for small tile counts: a workgroup of WAVES_M x WAVES_N wavefronts owns a BM x BN tile, K advances
+// in steps of 64 through a double-buffered LDS stage with one barrier per step (while step t is multiplied
+// out of buffer t&1, the registers holding step t+1 go to the other buffer and the loads of step t+2 are
+// issued).  Several workgroups fit on a CU and cover each other's barriers and epilogues.
+// blockIdx.y selects a slice of K (split-K): slice s covers [s*kPerSplit, (s+1)*kPerSplit) and writes its
+// partial product to C + s*sliceStride.
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const unsigned short* __restrict__ A,
                                                                             const unsigned short* __restrict__ Bt,
                                                                             float* __restrict__ C, int M, int N, int K, int lda,
-                                                                            int ldb) {
+                                                                            int ldb, int kPerSplit, size_t sliceStride) {
     constexpr int THREADS = WAVES_M * WAVES_N * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;     // per-wave tile
     constexpr int TM = WM / 32, TN = WN / 32;               // 32x32 accumulators per wave
@@ -102,45 +160,34 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
     unsigned short* bs = lds + 2 * BM * LDS_ROW;           // [2][BN][LDS_ROW]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
-    // Tile order: groups of 8 tile-rows are walked column-first so that the tiles in flight at any time
-    // share A and Bt panels in L2; workgroups go round-robin to the 8 XCDs.
-    const int tilesM = (M + BM - 1) / BM, tilesN = (N + BN - 1) / BN;
     int tm, tn;
-    {
-        constexpr int GROUP = 8;
-        const int id = blockIdx.x;
-        const int perGroup = GROUP * tilesN;
-        const int g = id / perGroup, rem = id - g * perGroup;
-        const int rowsInGroup = min(GROUP, tilesM - g * GROUP);
-        tm = g * GROUP + rem % rowsInGroup;
-        tn = rem / rowsInGroup;
-    }
+    tileIndexGrouped(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+    const int kBegin = blockIdx.y * kPerSplit, kEnd = min(K, kBegin + kPerSplit);
+    C += size_t(blockIdx.y) * sliceStride;
 
     const int lr = tid >> 3, lc = (tid & 7) * 8;
+    const unsigned short* aRow[A_PASSES];
+    const unsigned short* bRow[B_PASSES];
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i) aRow[i] = A + size_t(min(m0 + lr + ROWS_PER_PASS * i, M - 1)) * lda;
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i) bRow[i] = Bt + size_t(min(n0 + lr + ROWS_PER_PASS * i, N - 1)) * ldb;
     uint4v aReg[A_PASSES], bReg[B_PASSES];
     auto loadGlobal = [&](int k0) {
-        const uint4v z = {0u, 0u, 0u, 0u};
-        const bool kOk = k0 + lc < K;
 #pragma unroll
-        for (int i = 0; i < A_PASSES; ++i) {
-            int r = m0 + lr + ROWS_PER_PASS * i;
-            aReg[i] = (r < M && kOk) ? *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k0 + lc) : z;
-        }
+        for (int i = 0; i < A_PASSES; ++i) aReg[i] = loadChunk(aRow[i], k0 + lc, kEnd);
 #pragma unroll
-        for (int i = 0; i < B_PASSES; ++i) {
-            int r = n0 + lr + ROWS_PER_PASS * i;
-            bReg[i] = (r < N && kOk) ? *reinterpret_cast<const uint4v*>(Bt + size_t(r) * ldb + k0 + lc) : z;
-        }
+        for (int i = 0; i < B_PASSES; ++i) bReg[i] = loadChunk(bRow[i], k0 + lc, kEnd);
     };
-    auto storeLds = [&](int buf) {
+    auto storeLds = [&](int buf, int k0) {   // k0: K offset of the step held in the registers
 #pragma unroll
         for (int i = 0; i < A_PASSES; ++i)
-            *reinterpret_cast<uint4v*>(as + (buf * BM + lr + ROWS_PER_PASS * i) * LDS_ROW + lc) = aReg[i];
+            *reinterpret_cast<uint4v*>(as + (buf * BM + lr + ROWS_PER_PASS * i) * LDS_ROW + lc) = zeroPast(aReg[i], k0 + lc, kEnd);
 #pragma unroll
         for (int i = 0; i < B_PASSES; ++i)
-            *reinterpret_cast<uint4v*>(bs + (buf * BN + lr + ROWS_PER_PASS * i) * LDS_ROW + lc) = bReg[i];
+            *reinterpret_cast<uint4v*>(bs + (buf * BN + lr + ROWS_PER_PASS * i) * LDS_ROW + lc) = zeroPast(bReg[i], k0 + lc, kEnd);
     };
 
     float16v acc[TM][TN];
@@ -151,10 +198,12 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    const int steps = (K + BKK - 1) / BKK;
-    loadGlobal(0);
-    storeLds(0);
-    if (steps > 1) loadGlobal(BKK);
+    const int steps = (kEnd - kBegin + BKK - 1) / BKK;   // <= 0 for an empty slice: stores zeros
+    if (steps > 0) {
+        loadGlobal(kBegin);
+        storeLds(0, kBegin);
+        if (steps > 1) loadGlobal(kBegin + BKK);
+    }
     __syncthreads();
     for (int t = 0; t < steps; ++t) {
         const unsigned short* ac = as + ((t & 1) * BM + wm0 + li) * LDS_ROW + 8 * half;
@@ -173,37 +222,192 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
         }
         if (t + 1 < steps) {
-            storeLds((t + 1) & 1);
-            if (t + 2 < steps) loadGlobal((t + 2) * BKK);
+            storeLds((t + 1) & 1, kBegin + (t + 1) * BKK);
+            if (t + 2 < steps) loadGlobal(kBegin + (t + 2) * BKK);
         }
         __syncthreads();
     }
+    storeAccumulators<TM, TN>(acc, C, M, N, m0 + wm0, n0 + wn0, li, half);
+}
 
+// Kernel for large products: 256 x 256 tile, 8 wavefronts in two groups of four.  Wavefronts w and w+4 of
+// a workgroup share a SIMD, so each SIMD holds one wavefront of either group.  A K step of 64 is worked
+// in two halves; each half has a memory phase (read the 12 operand fragments of the half step from LDS,
+// write one staged operand of the next step to the other LDS buffer, issue that operand's global loads for
+// the step after) and a compute phase (16 MFMAs out of registers).  A barrier ends every phase and group 1
+// runs one phase behind group 0: on every SIMD one wavefront multiplies while the other moves data.
+//   phase of group 0:  M(T,0) C(T,0) M(T,1) C(T,1) M(T+1,0) ...
+//   phase of group 1:     -   M(T,0) C(T,0) M(T,1) C(T,1)   ...
+// Buffer (T+1)&1 is written during the four phases after its last reader (group 1's M(T-1,1)) has passed a
+// barrier and before its first reader (group 0's M(T+1,0)) starts, and a global load has four phases to land.
+// Operand A is staged in the first half step and Bt in the second, so every load instruction still fetches
+// whole 128-byte lines.
+template <int XCD_ORDER>
+__global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned short* __restrict__ A,
+                                                                 const unsigned short* __restrict__ Bt, float* __restrict__ C,
+                                                                 int M, int N, int K, int lda, int ldb, int gmLog, int gnLog) {
+    constexpr int BM = 256, BN = 256, TM = 4, TN = 2;
+    extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
+    unsigned short* as = lds;                        // [2][256][LDS_ROW]
+    unsigned short* bs = lds + 2 * BM * LDS_ROW;     // [2][256][LDS_ROW]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    const int group = wave >> 2;
+    int tm, tn;
+    if (XCD_ORDER) {
+        if (!tileIndexXcd(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, gmLog, gnLog, tm, tn)) return;
+    } else {
+        tileIndexGrouped(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+    }
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int wm0 = group * 128, wn0 = (wave & 3) * 64;
+    const int lr = tid >> 3, lc = (tid & 7) * 8;     // 64 rows x 128 bytes per pass, 4 passes per operand
+    const unsigned short* aRow[4];
+    const unsigned short* bRow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        aRow[i] = A + size_t(min(m0 + lr + 64 * i, M - 1)) * lda;
+        bRow[i] = Bt + size_t(min(n0 + lr + 64 * i, N - 1)) * ldb;
+    }
+    uint4v stageA[4], stageB[4];
+    float16v acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int col = n0 + wn0 + j * 32 + li;
-            if (col < N) {
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                    if (row < M) C[size_t(row) * N + col] = acc[i][j][r];
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    const int steps = (K + BKK - 1) / BKK;
+    const int ldsW = lr * LDS_ROW + lc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        stageA[i] = loadChunk(aRow[i], lc, K);
+        stageB[i] = loadChunk(bRow[i], lc, K);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        *reinterpret_cast<uint4v*>(as + ldsW + 64 * i * LDS_ROW) = zeroPast(stageA[i], lc, K);
+        *reinterpret_cast<uint4v*>(bs + ldsW + 64 * i * LDS_ROW) = zeroPast(stageB[i], lc, K);
+    }
+    if (steps > 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            stageA[i] = loadChunk(aRow[i], BKK + lc, K);
+            stageB[i] = loadChunk(bRow[i], BKK + lc, K);
+        }
+    }
+    __syncthreads();
+    if (group == 1) __builtin_amdgcn_s_barrier();    // group 1 starts one phase late
+    bf16x8 a[2][TM], b[2][TN];
+    for (int T = 0; T < steps; ++T) {
+        const int par = T & 1;
+        const unsigned short* ac = as + (par * BM + wm0 + li) * LDS_ROW + 8 * half;
+        const unsigned short* bc = bs + (par * BN + wn0 + li) * LDS_ROW + 8 * half;
+        unsigned short* aw = as + (par ^ 1) * BM * LDS_ROW + ldsW;
+        unsigned short* bw = bs + (par ^ 1) * BN * LDS_ROW + ldsW;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            // ---- memory phase
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) a[kk][i] = *reinterpret_cast<const bf16x8*>(ac + i * 32 * LDS_ROW + h * 32 + kk * 16);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) b[kk][j] = *reinterpret_cast<const bf16x8*>(bc + j * 32 * LDS_ROW + h * 32 + kk * 16);
+            }
+            if (T + 1 < steps) {
+                if (h == 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(aw + 64 * i * LDS_ROW) = zeroPast(stageA[i], (T + 1) * BKK + lc, K);
+                    if (T + 2 < steps) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) stageA[i] = loadChunk(aRow[i], (T + 2) * BKK + lc, K);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(bw + 64 * i * LDS_ROW) = zeroPast(stageB[i], (T + 1) * BKK + lc, K);
+                    if (T + 2 < steps) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], (T + 2) * BKK + lc, K);
+                    }
                 }
             }
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- compute phase
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
         }
+    }
+    if (group == 0) __builtin_amdgcn_s_barrier();    // pairs with group 1's last barrier
+    storeAccumulators<TM, TN>(acc, C, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
-int launchTile(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda, size_t ldb,
-               hipStream_t s) {
-    size_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    if (tiles >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
-    constexpr size_t smem = size_t(2) * (BM + BN) * LDS_ROW * sizeof(unsigned short);
-    auto kernel = gemmBf16NtKernel<BM, BN, WAVES_M, WAVES_N>;
+// C[i] = sum over slices of partial[s*sliceStride + i], slices added in index order (deterministic).
+// sliceStride is a multiple of 4; `vec` says that C is 16-byte aligned.
+__global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restrict__ partial, float* __restrict__ C, size_t count,
+                                                            size_t sliceStride, int slices, int vec) {
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    const size_t first = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t count4 = vec ? count / 4 : 0;
+    for (size_t i = first; i < count4; i += stride) {
+        float4v sum = loadf4(partial + 4 * i);
+        for (int s = 1; s < slices; ++s) {
+            float4v p = loadf4(partial + size_t(s) * sliceStride + 4 * i);
+            sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
+        }
+        storef4(C + 4 * i, sum);
+    }
+    for (size_t i = 4 * count4 + first; i < count; i += stride) {
+        float sum = partial[i];
+        for (int s = 1; s < slices; ++s) sum += partial[size_t(s) * sliceStride + i];
+        C[i] = sum;
+    }
+}
+
+template <typename Kernel>
+int allowSharedMemory(Kernel kernel, size_t smem) {
     if (smem > 48 * 1024)
         BF_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-    kernel<<<unsigned(tiles), WAVES_M * WAVES_N * 64, smem, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb));
+    return BF_OK;
+}
+
+int launchPingPong(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda,
+                   size_t ldb, hipStream_t s) {
+    const size_t tilesM = (M + 255) / 256, tilesN = (N + 255) / 256;
+    constexpr size_t smem = size_t(2) * 512 * LDS_ROW * sizeof(unsigned short);
+    // XCD block shape: the 2^g x 2^(5-g) block that pads the tile grid least, squarest on ties
+    int gmLog = 2, gnLog = 3;
+    size_t bestCost = 0, blocks = 0;
+    for (int g = 0; g <= 5; ++g) {
+        size_t gm = size_t(1) << g, gn = size_t(32) >> g;
+        size_t nb = ((tilesM + gm - 1) / gm) * ((tilesN + gn - 1) / gn);
+        size_t cost = nb * 1000 + gm + gn;
+        if (g == 0 || cost < bestCost) { bestCost = cost; gmLog = g; gnLog = 5 - g; blocks = nb; }
+    }
+    // blocks are dealt to XCDs eight at a time: only worth it when that deal is (nearly) even
+    const bool xcdOrder = blocks * 32 <= (tilesM * tilesN) * 5 / 4 && (blocks % 8 == 0 || blocks >= 64);
+    if (xcdOrder) {
+        size_t grid = (blocks + 7) / 8 * 8 * 32;
+        if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+        auto kernel = gemmBf16PingPongKernel<1>;
+        int st = allowSharedMemory(kernel, smem);
+        if (st != BF_OK) return st;
+        kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb), gmLog, gnLog);
+    } else {
+        size_t grid = tilesM * tilesN;
+        if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+        auto kernel = gemmBf16PingPongKernel<0>;
+        int st = allowSharedMemory(kernel, smem);
+        if (st != BF_OK) return st;
+        kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb), 0, 0);
+    }
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -211,10 +415,37 @@ int launchTile(const unsigned short* A, const unsigned short* Bt, float* C, size
 int launchGemmNt(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda,
                  size_t ldb, hipStream_t s) {
     if (M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
-    // 256x256 tiles (8 wavefronts) once they give every CU at least one tile; otherwise 128x128 (4 wavefronts)
+    const size_t cus = size_t(computeUnits());
+    // 256x256 ping-pong tiles once they give three quarters of the CUs a tile; otherwise 128x128 tiles,
+    // with K cut into slices when even those leave CUs idle and K is long enough to share out.
     const size_t bigTiles = ((M + 255) / 256) * ((N + 255) / 256);
-    if (bigTiles >= size_t(computeUnits()) * 3 / 4) return launchTile<256, 256, 2, 4>(A, Bt, C, M, N, K, lda, ldb, s);
-    return launchTile<128, 128, 2, 2>(A, Bt, C, M, N, K, lda, ldb, s);
+    if (bigTiles >= cus * 3 / 4) return launchPingPong(A, Bt, C, M, N, K, lda, ldb, s);
+    const size_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    constexpr size_t smem = size_t(2) * (128 + 128) * LDS_ROW * sizeof(unsigned short);
+    auto kernel = gemmBf16NtKernel<128, 128, 2, 2>;
+    int st = allowSharedMemory(kernel, smem);
+    if (st != BF_OK) return st;
+    size_t slices = 1;
+    if (tiles < cus && K >= 2048) slices = std::min<size_t>(std::min<size_t>(8, (2 * cus) / tiles), K / 1024);
+    if (slices > 1) {
+        const size_t steps = (K + BKK - 1) / BKK;
+        const size_t kPer = (steps + slices - 1) / slices * BKK;
+        slices = (K + kPer - 1) / kPer;
+        const size_t count = M * N, sliceStride = (count + 3) / 4 * 4;
+        Scratch partial(slices * sliceStride * sizeof(float));
+        if (partial.status != BF_OK) return partial.status;
+        kernel<<<dim3(unsigned(tiles), unsigned(slices)), 256, smem, s>>>(A, Bt, partial.as<float>(), int(M), int(N), int(K),
+                                                                         int(lda), int(ldb), int(kPer), sliceStride);
+        BF_LAUNCH_CHECK();
+        const int vec = (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
+        splitReduceKernel<<<gridFor(count / 4 + 1, kBlock, unsigned(cus) * 8), kBlock, 0, s>>>(partial.as<float>(), C, count,
+                                                                                              sliceStride, int(slices), vec);
+        BF_LAUNCH_CHECK();
+        return BF_OK;
+    }
+    kernel<<<dim3(unsigned(tiles), 1), 256, smem, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb), int(K), size_t(0));
+    BF_LAUNCH_CHECK();
+    return BF_OK;
 }
 
 int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, hipStream_t s) {

@@ -106,6 +106,35 @@ def test_bf16_projection_and_gradients(hip, oracle, rng, m, k, n, cached):
     assert_close(dB.toHost(), fB, tol=BF16_TOL, what="bf16 dB vs fp32")
 
 
+@pytest.mark.parametrize("m,k,n", [(4100, 129, 71), (2050, 72, 130)])
+def test_bf16_gradients_with_long_contraction(hip, oracle, rng, m, k, n):
+    """dB contracts over m: long enough that K is cut into slices summed in a fixed order; odd output counts."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b, g = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, m, n)
+    ar, br, gr = oracle.roundToBf16(a), oracle.roundToBf16(b), oracle.roundToBf16(g)
+    dA, dB = ops.matmulBf16Backward(*map(D.fromHost, (a, b, g)))
+    eA, eB = oracle.matmulBackward(ar, br, gr)
+    assert_close(dA.toHost(), eA, tol=1e-4, what="bf16 dA vs rounded operands")
+    assert_close(dB.toHost(), eB, tol=1e-4, what="bf16 dB vs rounded operands")
+    again = ops.matmulBf16Backward(*map(D.fromHost, (a, b, g)))[1]
+    assert_bits_equal(again.toHost(), dB.toHost(), "sliced contraction must be deterministic")
+
+
+@pytest.mark.parametrize("m,k,n", [(3500, 200, 3700), (4000, 136, 4090), (8192, 64, 2048)])
+def test_bf16_projection_large_tile_kernel(hip, oracle, rng, m, k, n):
+    """Shapes with enough 256x256 tiles for the large-product kernel (ragged edges, a K tail, and a tile grid
+    that is dealt to the XCDs in blocks).  Expected value: float64 product of the bf16-rounded operands, which
+    the oracle's fp32 matmul matches to 1e-6 on the sampled rows below."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b = r(rng, m, k), r(rng, k, n, scale=0.1)
+    ar, br = oracle.roundToBf16(a), oracle.roundToBf16(b)
+    c = ops.matmulBf16(D.fromHost(a), D.fromHost(b)).toHost()
+    expected = (ar.astype(np.float64) @ br.astype(np.float64)).astype(f32)
+    rows = np.r_[0:3, m // 2:m // 2 + 3, m - 3:m]
+    assert_close(oracle.matmul(ar[rows], br), expected[rows], tol=1e-5, what="oracle vs float64 on sampled rows")
+    assert_close(c, expected, tol=1e-4, what="bf16 fwd (large tiles) vs rounded operands")
+
+
 def test_bf16_weight_cache_semantics(hip, oracle, rng):
     """A cached weight image is reused until invalidateBf16WeightCache() (ops_tensorcore.cu:98-131,448)."""
     D, ops = hip.DeviceTensor, hip.ops
