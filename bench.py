@@ -133,25 +133,89 @@ def cpu_baseline_attention(seconds_budget=20.0):
 
 
 def bench_extras(bf, steps):
-    """Secondary figures: a bandwidth-bound kernel and the bf16 projection GEMM (not part of `value`)."""
-    D, call, ops = bf.DeviceTensor, bf.capi.call, bf.ops
+    """Secondary figures (not part of `value`): the bandwidth-bound kernels at the sizes of the GPT-small and
+    long-context configurations, priced in algorithmic bytes (every distinct input read once, every output
+    written once), and the bf16 projection GEMM on N(0,1) operands."""
+    D, call = bf.DeviceTensor, bf.capi.call
     stream = bf.Stream()
+    sh = stream.handle
+    rng = np.random.default_rng(3)
     extras = {}
-    n = 4096 * 4096
-    x, y = D.zeros((n,)), D((n,))
-    ms = time_region(bf, stream, lambda: call("bf_hip_act_forward", x.ptr, y.ptr, n, bf.capi.ACT_SILU, stream.handle), steps, 3)
-    extras["silu_4096x4096"] = {"ms": ms, "GB/s": 8 * n / ms / 1e6, "frac_hbm": 8 * n / ms / 1e6 / PEAK_HBM_GBS}
-    mdim = 4096
-    a = D.fromHost(np.random.default_rng(1).standard_normal((mdim, mdim), dtype=np.float32))
-    w = D.fromHost(np.random.default_rng(2).standard_normal((mdim, mdim), dtype=np.float32) / 64)
-    abf, wbf, c = D((mdim, mdim), itemsize=2), D((mdim, mdim), itemsize=2), D((mdim, mdim))
-    call("bf_hip_cvt_f32_bf16", a.ptr, abf.ptr, mdim * mdim, None)
-    call("bf_hip_cvt_f32_bf16_transpose", w.ptr, wbf.ptr, mdim, mdim, None)
-    ms = time_region(bf, stream, lambda: call("bf_hip_gemm_bf16_nt", abf.ptr, wbf.ptr, c.ptr, mdim, mdim, mdim, stream.handle), steps, 3)
-    tf = 2 * mdim ** 3 / ms / 1e9
-    extras["gemm_bf16_4096"] = {"ms": ms, "TFLOP/s": tf, "frac_bf16_mfma": tf / PEAK_BF16_MFMA_TFLOPS}
-    ms = time_region(bf, stream, lambda: call("bf_hip_matmul_bf16", a.ptr, w.ptr, c.ptr, mdim, mdim, mdim, 1, stream.handle), steps, 3)
-    extras["matmul_bf16_4096_fp32_io"] = {"ms": ms, "TFLOP/s": 2 * mdim ** 3 / ms / 1e9}
+
+    def hbm(name, nbytes, fn):
+        ms = time_region(bf, stream, fn, steps, 2)
+        gbs = nbytes / ms / 1e6
+        extras[name] = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 3)}
+
+    def rand(*shape, scale=1.0):
+        return D.fromHost(rng.standard_normal(shape, dtype=np.float32) * np.float32(scale))
+
+    # long-context hidden activation [16384, 8192] (512 MiB) and model-width rows [16384, 2048]
+    rows, hid, dm = 16384, 8192, 2048
+    x, g, y = rand(rows, hid), rand(rows, hid), D((rows, hid))
+    bias = rand(hid)
+    n = rows * hid
+    hbm("silu_16384x8192", 8 * n, lambda: call("bf_hip_act_forward", x.ptr, y.ptr, n, bf.capi.ACT_SILU, sh))
+    hbm("gelu_backward_16384x8192", 12 * n, lambda: call("bf_hip_act_backward", x.ptr, g.ptr, y.ptr, n, bf.capi.ACT_GELU, sh))
+    hbm("add_bias_silu_16384x8192", 8 * n, lambda: call("bf_hip_add_bias_act", x.ptr, bias.ptr, y.ptr, rows, hid, bf.capi.ACT_SILU, sh))
+    hbm("add_16384x8192", 12 * n, lambda: call("bf_hip_add", x.ptr, g.ptr, y.ptr, n, sh))
+    hbm("accumulate_16384x8192", 12 * n, lambda: call("bf_hip_accumulate", y.ptr, g.ptr, n, sh))
+    dbias = D((hid,))
+    hbm("bias_grad_16384x8192", 4 * n, lambda: call("bf_hip_bias_grad", g.ptr, dbias.ptr, rows, hid, sh))
+    half = D((rows, hid // 2))
+    hbm("cvt_f32_bf16_16384x8192", 6 * n, lambda: call("bf_hip_cvt_f32_bf16", x.ptr, half.ptr, n, sh))
+    hbm("cvt_f32_bf16_transpose_16384x8192", 6 * n, lambda: call("bf_hip_cvt_f32_bf16_transpose", x.ptr, half.ptr, rows, hid, sh))
+    nr = rows * dm * 4   # [65536, 2048]: four blocks' worth of rows, 512 MiB
+    hbm("rmsnorm_65536x2048", 8 * nr, lambda: call("bf_hip_rmsnorm", x.ptr, y.ptr, nr // dm, dm, sh))
+    hbm("rmsnorm_backward_65536x2048", 12 * nr, lambda: call("bf_hip_rmsnorm_backward", x.ptr, g.ptr, y.ptr, nr // dm, dm, sh))
+    hbm("softmax_65536x2048", 8 * nr, lambda: call("bf_hip_softmax", x.ptr, y.ptr, nr // dm, dm, sh))
+    del x, g, y, half
+
+    # GPT-small logits [8192, 32000] (0.98 GiB): sparse cross-entropy reads logits once and writes the gradient
+    rows, vocab, dim = 8192, 32000, 768
+    logits, grad = rand(rows, vocab), D((rows, vocab))
+    target = D.fromHost(rng.integers(0, vocab, rows).astype(np.float32))
+    loss = D.zeros((1,))
+    hbm("cross_entropy_sparse_8192x32000", 8 * rows * vocab,
+        lambda: call("bf_hip_cross_entropy_sparse", logits.ptr, target.ptr, grad.ptr, loss.ptr, rows, vocab, 0, sh))
+    del logits, grad
+
+    # embedding table [32000, 768]: gather of 8192 tokens; scatter-add backward writes the whole table gradient
+    table, dtable = rand(vocab, dim), D((vocab, dim))
+    ids = D.fromHost(rng.integers(0, vocab, rows).astype(np.float32))
+    out, gout = D((rows, dim)), rand(rows, dim)
+    hbm("embedding_forward_8192x768", rows * dim * 8 + rows * 4,
+        lambda: call("bf_hip_embedding_forward", ids.ptr, table.ptr, out.ptr, rows, vocab, dim, sh))
+    hbm("embedding_backward_8192x768_into_32000x768", rows * dim * 4 + vocab * dim * 4,
+        lambda: call("bf_hip_embedding_backward", ids.ptr, gout.ptr, dtable.ptr, rows, vocab, dim, sh))
+
+    # AdamW over the GPT-small parameter set (134 951 168 values in 76 tensors): 28 bytes per parameter
+    counts = [vocab * dim, 1024 * dim] + [dim * dim] * 48 + [dim * 3072, 3072, 3072 * dim, dim] * 12 + [dim * vocab, vocab]
+    total = sum(counts)
+    pool = [D.zeros((total,)) for _ in range(4)]   # params, grads, m, v as slices of four big buffers
+    offs = np.concatenate([[0], np.cumsum(counts)[:-1]])
+    arr = lambda t: (ctypes.c_void_p * len(counts))(*[t.ptr.value + int(o) * 4 if hasattr(t.ptr, "value") else t.ptr + int(o) * 4 for o in offs])
+    ps, gs, ms_, vs = (arr(t) for t in pool)
+    cn = (ctypes.c_size_t * len(counts))(*counts)
+    hbm("adamw_134951168_params", 28 * total,
+        lambda: call("bf_hip_adamw_multi", ps, gs, ms_, vs, cn, len(counts), 1, ctypes.c_float(1e-3), ctypes.c_float(0.9),
+                     ctypes.c_float(0.999), ctypes.c_float(1e-8), ctypes.c_float(0.01), sh))
+    hbm("zero_multi_134951168_params", 4 * total, lambda: call("bf_hip_zero_multi", gs, cn, len(counts), sh))
+    del pool
+
+    # bf16 projection GEMM (C2 shape and a long-context shape), operands N(0,1) / N(0,1/64) rounded to bf16
+    def gemm(m, n_, k):
+        a, w = rand(m, k), rand(k, n_, scale=1 / 64)
+        abf, wbf, c = D((m, k), itemsize=2), D((n_, k), itemsize=2), D((m, n_))
+        call("bf_hip_cvt_f32_bf16", a.ptr, abf.ptr, m * k, None)
+        call("bf_hip_cvt_f32_bf16_transpose", w.ptr, wbf.ptr, k, n_, None)
+        ms = time_region(bf, stream, lambda: call("bf_hip_gemm_bf16_nt", abf.ptr, wbf.ptr, c.ptr, m, n_, k, sh), steps, 3)
+        tf = 2 * m * n_ * k / ms / 1e9
+        extras[f"gemm_bf16_{m}x{n_}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_bf16_mfma": round(tf / PEAK_BF16_MFMA_TFLOPS, 3)}
+        ms = time_region(bf, stream, lambda: call("bf_hip_matmul_bf16", a.ptr, w.ptr, c.ptr, m, k, n_, 1, sh), steps, 3)
+        extras[f"matmul_bf16_fp32_io_{m}x{n_}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(2 * m * n_ * k / ms / 1e9, 1)}
+    gemm(4096, 4096, 4096)
+    gemm(16384, 8192, 2048)
     return extras
 
 

@@ -108,6 +108,23 @@ __device__ __forceinline__ T blockReduce(T v, T identity, Op op, T* scratch) {
 struct OpSum { template <typename T> __device__ T operator()(T a, T b) const { return a + b; } };
 struct OpMaxF { __device__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 
+// For the flat multi-tensor kernels: tensors are laid end to end in units of blocks and entry i of `table`
+// (any struct with a `firstBlock` member) starts at block table[i].firstBlock.  Returns the entry that owns
+// `block`: the last one whose firstBlock is <= block (empty tensors share their successor's firstBlock and
+// are skipped by that rule).  The wavefront tests 64 entries per step, so a typical parameter list takes one
+// round of loads instead of a chain of dependent ones.
+template <typename T>
+__device__ __forceinline__ int owningTensor(const T* __restrict__ table, int numTensors, unsigned block) {
+    const int lane = threadIdx.x & 63;
+    int notAfter = 0;
+    for (int base = 0; base < numTensors; base += 64) {
+        const int i = base + lane;
+        const bool le = i < numTensors && table[i].firstBlock <= block;
+        notAfter += __popcll(__ballot(le));
+    }
+    return notAfter - 1;
+}
+
 __device__ __forceinline__ float4v loadf4(const float* p) { return *reinterpret_cast<const float4v*>(p); }
 __device__ __forceinline__ void storef4(float* p, float4v v) { *reinterpret_cast<float4v*>(p) = v; }
 

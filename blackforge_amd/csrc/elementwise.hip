@@ -31,7 +31,10 @@ __global__ void __launch_bounds__(kBlock) flat1Kernel(size_t begin, size_t n, F 
 template <typename F>
 int launchFlat(size_t n, bool canVectorise, F f, hipStream_t stream) {
     if (n == 0) return BF_OK;
-    const unsigned cap = unsigned(computeUnits()) * 16;
+    // one group of four elements per thread and a grid that covers the whole array: the access stream stays
+    // in address order across the device, which HBM rewards (grid-stride loops over a few blocks per CU lose
+    // about a fifth of the bandwidth)
+    const unsigned cap = 1u << 30;
     size_t done = 0;
     if (canVectorise && n >= 4) {
         size_t n4 = n / 4;
@@ -90,7 +93,7 @@ struct RowGeom {
     int vec;
 };
 
-RowGeom rowGeometry(size_t rows, size_t features, bool canVectorise, unsigned maxRowBlocks = 0) {
+RowGeom rowGeometry(size_t rows, size_t features, bool canVectorise, unsigned maxRowBlocks = 0, unsigned rowsPerThread = 1) {
     RowGeom g;
     g.vec = (canVectorise && features % 4 == 0) ? 4 : 1;
     size_t cols = features / g.vec;
@@ -98,10 +101,9 @@ RowGeom rowGeometry(size_t rows, size_t features, bool canVectorise, unsigned ma
     while (bx < 256 && bx < cols) bx <<= 1;
     unsigned by = 256 / bx;
     unsigned gx = unsigned((cols + bx - 1) / bx);
-    size_t rowBlocks = (rows + by - 1) / by;
-    size_t want = size_t(computeUnits()) * 16 / (gx ? gx : 1);
-    if (want < 1) want = 1;
-    if (rowBlocks > want) rowBlocks = want;
+    size_t rowBlocks = (rows + size_t(by) * rowsPerThread - 1) / (size_t(by) * rowsPerThread);
+    // streaming kernels (maxRowBlocks == 0) take every row block once, in address order; reductions cap the
+    // number of row blocks because each writes a partial row
     if (maxRowBlocks && rowBlocks > maxRowBlocks) rowBlocks = maxRowBlocks;
     if (rowBlocks > 65535) rowBlocks = 65535;
     if (rowBlocks < 1) rowBlocks = 1;
@@ -162,16 +164,32 @@ __global__ void __launch_bounds__(256) columnSumKernel(const float* __restrict__
     if (active) {
         typename Pack<VEC>::T b = {};
         if constexpr (FUSED) b = Pack<VEC>::load(bias + col);
-        size_t rowStep = size_t(gridDim.y) * blockDim.y;
-        for (size_t r = size_t(blockIdx.y) * blockDim.y + threadIdx.y; r < rows; r += rowStep) {
+        auto term = [&](size_t r) {
             size_t idx = r * features + col;
             typename Pack<VEC>::T v = Pack<VEC>::load(src + idx);
             if constexpr (FUSED) {
                 v = Pack<VEC>::load(dHidden + idx) * actD4<ACT>(v + b);
                 Pack<VEC>::store(dGemm + idx, v);
             }
-            acc = acc + v;
+            return v;
+        };
+        // In one step the whole grid reads one contiguous band of gridDim.y * 4 * blockDim.y rows (a block takes
+        // 4 * blockDim.y consecutive rows of it, a thread four of those), then all blocks move to the next band:
+        // the device streams the matrix in address order with four loads in flight per thread.  Each of a
+        // thread's four rows has its own running sum; the sums are added in a fixed order.
+        const size_t by = blockDim.y, bandRows = size_t(gridDim.y) * 4 * by;
+        typename Pack<VEC>::T acc1 = {}, acc2 = {}, acc3 = {};
+        for (size_t r = size_t(blockIdx.y) * 4 * by + threadIdx.y; r < rows; r += bandRows) {
+            if (r + 3 * by < rows) {
+                typename Pack<VEC>::T v0 = term(r), v1 = term(r + by), v2 = term(r + 2 * by), v3 = term(r + 3 * by);
+                acc = acc + v0; acc1 = acc1 + v1; acc2 = acc2 + v2; acc3 = acc3 + v3;
+            } else {
+                acc = acc + term(r);
+                if (r + by < rows) acc1 = acc1 + term(r + by);
+                if (r + 2 * by < rows) acc2 = acc2 + term(r + 2 * by);
+            }
         }
+        acc = (acc + acc1) + (acc2 + acc3);
     }
     if (partial == nullptr) return;
     // reduce over threadIdx.y (fixed order), result in the ty == 0 threads
@@ -206,7 +224,7 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
         return BF_OK;
     }
     bool vec = aligned16(src) && (!FUSED || (aligned16(bias) && aligned16(dHidden) && aligned16(dGemm)));
-    RowGeom g = rowGeometry(rows, features, vec, 128);
+    RowGeom g = rowGeometry(rows, features, vec, 128, 4);
     size_t parts = g.grid.y;
     Scratch scratch(dBias ? parts * features * sizeof(float) : 0);
     if (scratch.status != BF_OK) return scratch.status;
@@ -228,14 +246,24 @@ struct ZeroTarget {
     size_t count;
 };
 
-// One block per chunk of one tensor; chunk table built on the host so that every block has work.
-struct ZeroChunk {
+// One flat grid over all tensors laid end to end: a block owns 1024 consecutive elements of one tensor,
+// which it finds in the table of first-block indices.
+struct ZeroTensor {
     float* ptr;
-    unsigned count;
+    size_t count;
+    unsigned firstBlock;
+    unsigned pad;
 };
-__global__ void __launch_bounds__(kBlock) zeroMultiKernel(const ZeroChunk* chunks) {
-    ZeroChunk c = chunks[blockIdx.x];
-    for (unsigned i = threadIdx.x; i < c.count; i += blockDim.x) c.ptr[i] = 0.0f;
+__global__ void __launch_bounds__(kBlock) zeroMultiKernel(const ZeroTensor* __restrict__ table, int numTensors) {
+    const ZeroTensor c = table[owningTensor(table, numTensors, blockIdx.x)];
+    const size_t base = (size_t(blockIdx.x - c.firstBlock) * kBlock + threadIdx.x) * 4;
+    if (base >= c.count) return;
+    if ((reinterpret_cast<uintptr_t>(c.ptr) & 15u) == 0 && base + 4 <= c.count) {
+        const float4v z = {0.0f, 0.0f, 0.0f, 0.0f};
+        storef4(c.ptr + base, z);
+    } else {
+        for (size_t i = base; i < base + 4 && i < c.count; ++i) c.ptr[i] = 0.0f;
+    }
 }
 
 }  // namespace
@@ -350,20 +378,20 @@ int bf_hip_add_bias_act_backward(const float* gemm, const float* bias, const flo
 int bf_hip_zero_multi(float* const* ptrs, const size_t* counts, size_t numTensors, bf_stream_t stream) {
     if (numTensors == 0) return BF_OK;
     BF_REQUIRE(ptrs && counts, "NULL pointer");
-    constexpr size_t kChunk = size_t(kBlock) * 32;  // 8192 floats = 32 KiB per block
-    std::vector<ZeroChunk> chunks;
+    constexpr size_t kPerBlock = size_t(kBlock) * 4;
+    std::vector<ZeroTensor> table;
+    size_t blocks = 0;
     for (size_t t = 0; t < numTensors; ++t) {
         BF_REQUIRE(ptrs[t] != nullptr || counts[t] == 0, "NULL tensor pointer");
-        for (size_t off = 0; off < counts[t]; off += kChunk) {
-            size_t c = counts[t] - off < kChunk ? counts[t] - off : kChunk;
-            chunks.push_back(ZeroChunk{ptrs[t] + off, unsigned(c)});
-        }
+        table.push_back(ZeroTensor{ptrs[t], counts[t], unsigned(blocks), 0});
+        blocks += (counts[t] + kPerBlock - 1) / kPerBlock;
+        BF_REQUIRE(blocks < (size_t(1) << 31), "too many elements for one launch");
     }
-    if (chunks.empty()) return BF_OK;
-    const void* table = nullptr;
-    int status = uploadDescriptorTable(kSlotZero, chunks.data(), chunks.size() * sizeof(ZeroChunk), asStream(stream), &table);
+    if (blocks == 0) return BF_OK;
+    const void* device = nullptr;
+    int status = uploadDescriptorTable(kSlotZero, table.data(), table.size() * sizeof(ZeroTensor), asStream(stream), &device);
     if (status != BF_OK) return status;
-    zeroMultiKernel<<<unsigned(chunks.size()), kBlock, 0, asStream(stream)>>>(static_cast<const ZeroChunk*>(table));
+    zeroMultiKernel<<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const ZeroTensor*>(device), int(numTensors));
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

@@ -51,17 +51,21 @@ __global__ void __launch_bounds__(kBlock) histogramKernel(const float* __restric
     if (i < tokens) atomicAdd(&counts[size_t(roundId(ids[i]))], 1u);
 }
 
-// Exclusive scan of counts[0..vocab) into offsets[0..vocab], single block, fixed order.
+// Exclusive scan of counts[0..vocab) into offsets[0..vocab], single block of 1024 threads, four consecutive
+// entries per thread and pass (integer sums: any order gives the same result).
 __global__ void __launch_bounds__(1024) exclusiveScanKernel(const unsigned* __restrict__ counts, unsigned* __restrict__ offsets, size_t vocab) {
     __shared__ unsigned waveTotals[16];
     __shared__ unsigned carry;
     if (threadIdx.x == 0) carry = 0;
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (size_t base = 0; base < vocab; base += 1024) {
-        size_t i = base + threadIdx.x;
-        unsigned v = i < vocab ? counts[i] : 0u;
-        unsigned incl = v;
+    for (size_t base = 0; base < vocab; base += 4096) {
+        const size_t i = base + size_t(threadIdx.x) * 4;
+        unsigned v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = i + j < vocab ? counts[i + j] : 0u;
+        const unsigned mine = v[0] + v[1] + v[2] + v[3];
+        unsigned incl = mine;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             unsigned n = __shfl_up(incl, off, 64);
@@ -71,7 +75,12 @@ __global__ void __launch_bounds__(1024) exclusiveScanKernel(const unsigned* __re
         __syncthreads();
         unsigned before = carry;
         for (int w = 0; w < wave; ++w) before += waveTotals[w];
-        if (i < vocab) offsets[i] = before + incl - v;
+        unsigned run = before + incl - mine;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (i + j < vocab) offsets[i + j] = run;
+            run += v[j];
+        }
         __syncthreads();
         if (threadIdx.x == 1023) carry = before + incl;
         __syncthreads();
@@ -79,15 +88,29 @@ __global__ void __launch_bounds__(1024) exclusiveScanKernel(const unsigned* __re
     if (threadIdx.x == 0) offsets[vocab] = carry;
 }
 
-// order[offsets[id] + rank] = token, where rank = number of earlier tokens with the same id.
-__global__ void __launch_bounds__(kBlock) placeTokensKernel(const float* __restrict__ ids, size_t tokens,
-                                                            const unsigned* __restrict__ offsets, unsigned* __restrict__ order) {
+// Tokens are first dropped into their id's segment in whatever order the atomics resolve
+// (slot = offsets[id] + one of counts[id]-1 .. 0), then every token finds its rank among the tokens of its
+// segment (how many of them are smaller) and moves to order[offsets[id] + rank]: segments end up sorted by
+// token index whatever the atomics did, so the sums below run in token order.  The rank loop is as long as
+// the segment (the number of tokens that share the id).
+__global__ void __launch_bounds__(kBlock) scatterTokensKernel(const float* __restrict__ ids, size_t tokens,
+                                                              const unsigned* __restrict__ offsets, unsigned* __restrict__ counts,
+                                                              unsigned* __restrict__ unordered) {
     size_t t = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (t >= tokens) return;
-    long long id = roundId(ids[t]);
-    unsigned rank = 0;
-    for (size_t u = 0; u < t; ++u) rank += roundId(ids[u]) == id ? 1u : 0u;
-    order[offsets[size_t(id)] + rank] = unsigned(t);
+    size_t id = size_t(roundId(ids[t]));
+    unsigned left = atomicSub(&counts[id], 1u);   // value before the decrement: counts[id] .. 1
+    unordered[offsets[id] + left - 1u] = unsigned(t);
+}
+__global__ void __launch_bounds__(kBlock) rankTokensKernel(const float* __restrict__ ids, size_t tokens,
+                                                           const unsigned* __restrict__ offsets,
+                                                           const unsigned* __restrict__ unordered, unsigned* __restrict__ order) {
+    size_t t = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= tokens) return;
+    size_t id = size_t(roundId(ids[t]));
+    unsigned begin = offsets[id], end = offsets[id + 1], rank = 0;
+    for (unsigned j = begin; j < end; ++j) rank += unordered[j] < unsigned(t) ? 1u : 0u;
+    order[begin + rank] = unsigned(t);
 }
 
 // One wavefront per vocabulary row.
@@ -227,10 +250,7 @@ Geom2D geometry2D(size_t rows, size_t cols, bool canVectorise) {
     unsigned by = 256 / bx;
     unsigned gx = unsigned((groups + bx - 1) / bx);
     size_t gy = (rows + by - 1) / by;
-    size_t want = size_t(computeUnits()) * 16 / (gx ? gx : 1);
-    if (want < 1) want = 1;
-    if (gy > want) gy = want;
-    if (gy > 65535) gy = 65535;
+    if (gy > 65535) gy = 65535;   // every row block once, in address order
     if (gy < 1) gy = 1;
     g.block = dim3(bx, by);
     g.grid = dim3(gx, unsigned(gy));
@@ -287,22 +307,25 @@ int bf_hip_embedding_backward(const float* ids, const float* g, float* dTable, s
     hipStream_t s = asStream(stream);
     if (tokens == 0) return bf_hip_fill_zero(dTable, vocab * dim * sizeof(float), stream);
     BF_REQUIRE(ids && g, "NULL pointer");
-    // counts[vocab] | offsets[vocab+1] | order[tokens]
-    size_t words = vocab + (vocab + 1) + tokens;
+    // counts[vocab] | offsets[vocab+1] | unordered[tokens] | order[tokens]
+    size_t words = vocab + (vocab + 1) + 2 * tokens;
     Scratch work(words * sizeof(unsigned));
     if (work.status != BF_OK) return work.status;
     unsigned* counts = work.as<unsigned>();
     unsigned* offsets = counts + vocab;
-    unsigned* order = offsets + vocab + 1;
+    unsigned* unordered = offsets + vocab + 1;
+    unsigned* order = unordered + tokens;
     int st = bf_hip_fill_zero(counts, vocab * sizeof(unsigned), stream);
     if (st != BF_OK) return st;
     histogramKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, counts);
     BF_LAUNCH_CHECK();
     exclusiveScanKernel<<<1, 1024, 0, s>>>(counts, offsets, vocab);
     BF_LAUNCH_CHECK();
-    placeTokensKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, offsets, order);
+    scatterTokensKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, offsets, counts, unordered);
     BF_LAUNCH_CHECK();
-    unsigned grid = gridFor(vocab, kBlock / 64, unsigned(computeUnits()) * 16);
+    rankTokensKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, offsets, unordered, order);
+    BF_LAUNCH_CHECK();
+    unsigned grid = gridFor(vocab, kBlock / 64);
     if (aligned16(g) && aligned16(dTable) && dim % 4 == 0)
         embeddingBackwardKernel<4><<<grid, kBlock, 0, s>>>(g, dTable, offsets, order, vocab, dim);
     else

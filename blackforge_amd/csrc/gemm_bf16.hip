@@ -55,24 +55,51 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict_
     }
 }
 
-// out[c, 0..rowsPad) = bf16(x[0..rows, c]), zero padded: 64 x 64 tiles through LDS.
+// out[c, 0..rowsPad) = bf16(x[0..rows, c]), zero padded: 64 x 64 tiles through LDS.  With `vec` (x 16-byte
+// aligned, cols a multiple of 4, rowsPad a multiple of 8) a thread reads four consecutive columns of a row as
+// one 16-byte load and writes eight consecutive rows of an output row as one 16-byte store, so both sides move
+// whole 128-byte lines; otherwise elements go one by one.
 __global__ void __launch_bounds__(kBlock) convertTransposeKernel(const float* __restrict__ x, unsigned short* __restrict__ out,
-                                                                 size_t rows, size_t cols, size_t rowsPad) {
-    __shared__ unsigned short tile[64][66];
+                                                                 size_t rows, size_t cols, size_t rowsPad, int vec) {
+    __shared__ __attribute__((aligned(16))) unsigned short tile[64][72];   // [column][row], 144-byte pitch
     const size_t r0 = size_t(blockIdx.y) * 64, c0 = size_t(blockIdx.x) * 64;
+    if (vec) {
+        const int cg = threadIdx.x & 15, rr = threadIdx.x >> 4;   // 16 column groups x 16 rows per pass
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = rr + 16 * i;
+            const size_t gr = r0 + r, gc = c0 + 4 * cg;
+            float4v v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (gr < rows && gc < cols) v = loadf4(x + gr * cols + gc);   // cols % 4 == 0: all four in range
+            tile[4 * cg + 0][r] = toBf16Bits(v.x);
+            tile[4 * cg + 1][r] = toBf16Bits(v.y);
+            tile[4 * cg + 2][r] = toBf16Bits(v.z);
+            tile[4 * cg + 3][r] = toBf16Bits(v.w);
+        }
+        __syncthreads();
+        const int chunk = threadIdx.x & 7, cc = threadIdx.x >> 3;   // 8 chunks of 8 rows x 32 columns per pass
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = cc + 32 * i;
+            const size_t gc = c0 + c, gr = r0 + 8 * chunk;
+            if (gc < cols && gr < rowsPad)    // rowsPad % 8 == 0: the whole chunk is in range
+                *reinterpret_cast<uint4v*>(out + gc * rowsPad + gr) = *reinterpret_cast<const uint4v*>(&tile[c][8 * chunk]);
+        }
+        return;
+    }
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;   // 64 x 4
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         int r = ty + 4 * i;
         size_t gr = r0 + r, gc = c0 + tx;
-        tile[r][tx] = (gr < rows && gc < cols) ? toBf16Bits(x[gr * cols + gc]) : (unsigned short)0;
+        tile[tx][r] = (gr < rows && gc < cols) ? toBf16Bits(x[gr * cols + gc]) : (unsigned short)0;
     }
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         int c = ty + 4 * i;
         size_t gc = c0 + c, gr = r0 + tx;
-        if (gc < cols && gr < rowsPad) out[gc * rowsPad + gr] = tile[tx][c];
+        if (gc < cols && gr < rowsPad) out[gc * rowsPad + gr] = tile[c][tx];
     }
 }
 
@@ -453,7 +480,7 @@ int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, 
     size_t groups = rows * (colsPad / 8);
     if (groups == 0) return BF_OK;
     int vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && cols % 4 == 0;
-    convertKernel<<<gridFor(groups, kBlock, unsigned(computeUnits()) * 16), kBlock, 0, s>>>(x, out, rows, cols, colsPad, vec);
+    convertKernel<<<gridFor(groups, kBlock), kBlock, 0, s>>>(x, out, rows, cols, colsPad, vec);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -463,7 +490,8 @@ int convertTransposed(const float* x, unsigned short* out, size_t rows, size_t c
     size_t rowsPad = padRows ? pad8(rows) : rows;   // length of an output row
     dim3 grid(unsigned((cols + 63) / 64), unsigned((rowsPad + 63) / 64));
     if (grid.y > 65535) return failInvalid("cvt_f32_bf16_transpose", "too many rows");
-    convertTransposeKernel<<<grid, kBlock, 0, s>>>(x, out, rows, cols, rowsPad);
+    const int vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && cols % 4 == 0 && rowsPad % 8 == 0;
+    convertTransposeKernel<<<grid, kBlock, 0, s>>>(x, out, rows, cols, rowsPad, vec);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

@@ -75,38 +75,65 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
             for (size_t e = t; e < classes; e += G) mx = fmaxf(mx, x[e]);
         }
         mx = groupMax<G>(mx, lds);
+        // exp(x - mx) as one hardware exp2 of (x - mx) * log2(e): the argument is <= 0 and the result feeds
+        // a sum of up to `classes` terms, so its ~1e-6 relative error is far inside the 1e-4 bound
+        constexpr float kLog2e = 1.4426950408889634f;
         float sum = 0.0f;
         if constexpr (CACHED) {
 #pragma unroll
-            for (int i = 0; i < MAXE; ++i) { c.r[i] = expf(c.r[i] - mx); sum += c.r[i]; }
+            for (int i = 0; i < MAXE; ++i) { c.r[i] = __builtin_amdgcn_exp2f((c.r[i] - mx) * kLog2e); sum += c.r[i]; }
         } else {
-            for (size_t e = t; e < classes; e += G) sum += expf(x[e] - mx);
+            for (size_t e = t; e < classes; e += G) sum += __builtin_amdgcn_exp2f((x[e] - mx) * kLog2e);
         }
         sum = groupSum<G>(sum, lds);
         const float inv = 1.0f / sum;
 
         float loss = 0.0f;  // this thread's share of the row loss
-        size_t cls = 0;
-        if constexpr (SPARSE) cls = size_t(lroundf(target[row]));
-        auto emit = [&](float e, size_t idx) -> float {
-            float p = e * inv;
-            float tv;
-            if constexpr (SPARSE) tv = idx == cls ? 1.0f : 0.0f;
-            else tv = target[row * classes + idx];
-            if (tv != 0.0f) loss += -tv * logf(fmaxf(p, 1e-12f));
-            return (p - tv) * invRows;
-        };
-        if constexpr (CACHED) {
+        if constexpr (SPARSE) {
+            // grad = (p - onehot) / rows; the one thread that holds the target class keeps its probability
+            const unsigned cls = unsigned(lroundf(target[row]));
+            float pTarget = -1.0f;
+            if constexpr (CACHED) {
 #pragma unroll
-            for (int it = 0; it < MAXE / VEC; ++it)
+                for (int it = 0; it < MAXE / VEC; ++it)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    size_t idx = RowCache<G, MAXE, VEC>::index(it, t, j);
-                    if (idx < classes) c.r[it * VEC + j] = emit(c.r[it * VEC + j], idx);
+                    for (int j = 0; j < VEC; ++j) {
+                        const unsigned idx = unsigned(it * G + t) * VEC + j;   // < G * MAXE <= 65536
+                        const float p = c.r[it * VEC + j] * inv;
+                        const bool hit = idx == cls;
+                        pTarget = hit ? p : pTarget;
+                        c.r[it * VEC + j] = (p - (hit ? 1.0f : 0.0f)) * invRows;
+                    }
+                c.store(gOut, classes, t);
+            } else {
+                for (size_t e = t; e < classes; e += G) {
+                    const float p = __builtin_amdgcn_exp2f((x[e] - mx) * kLog2e) * inv;
+                    const bool hit = e == cls;
+                    pTarget = hit ? p : pTarget;
+                    gOut[e] = (p - (hit ? 1.0f : 0.0f)) * invRows;
                 }
-            c.store(gOut, classes, t);
+            }
+            if (pTarget >= 0.0f) loss = -logf(fmaxf(pTarget, 1e-12f));
         } else {
-            for (size_t e = t; e < classes; e += G) gOut[e] = emit(expf(x[e] - mx), e);
+            const float* tRow = target + row * classes;
+            auto emit = [&](float e, size_t idx) -> float {
+                const float p = e * inv;
+                const float tv = tRow[idx];
+                if (tv != 0.0f) loss += -tv * logf(fmaxf(p, 1e-12f));
+                return (p - tv) * invRows;
+            };
+            if constexpr (CACHED) {
+#pragma unroll
+                for (int it = 0; it < MAXE / VEC; ++it)
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) {
+                        size_t idx = RowCache<G, MAXE, VEC>::index(it, t, j);
+                        if (idx < classes) c.r[it * VEC + j] = emit(c.r[it * VEC + j], idx);
+                    }
+                c.store(gOut, classes, t);
+            } else {
+                for (size_t e = t; e < classes; e += G) gOut[e] = emit(__builtin_amdgcn_exp2f((x[e] - mx) * kLog2e), e);
+            }
         }
         loss = groupSum<G>(loss, lds);
         if (t == 0) rowLoss[row] = loss;
@@ -121,14 +148,19 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
     float* rl = rowLoss.as<float>();
     const float invRows = 1.0f / float(rows);
     const bool vec4 = aligned16(logits) && aligned16(grad) && classes % 4 == 0;
-    const unsigned cap = unsigned(computeUnits()) * 8;
-#define BF_CE(G, MAXE, VEC, CACHED, threads, perBlock)                                                     \
-    crossEntropyKernel<G, MAXE, VEC, CACHED, SPARSE><<<gridFor(rows, perBlock, cap), threads, 0, s>>>(      \
-        logits, target, grad, rl, rows, classes, invRows)
-    if (classes <= 64 * 16) { if (vec4) BF_CE(64, 16, 4, true, 256, 4); else BF_CE(64, 16, 1, true, 256, 4); }
-    else if (classes <= 256 * 32) { if (vec4) BF_CE(256, 32, 4, true, 256, 1); else BF_CE(256, 32, 1, true, 256, 1); }
-    else if (classes <= 1024 * 64) { if (vec4) BF_CE(1024, 64, 4, true, 1024, 1); else BF_CE(1024, 64, 1, true, 1024, 1); }
-    else BF_CE(1024, 4, 1, false, 1024, 1);
+    // smallest group and register count that hold a row (see the row kernels); a block takes its rows once
+#define BF_CE(G, MAXE)                                                                                            \
+    if (classes <= size_t(G) * MAXE) {                                                                            \
+        const unsigned threads = G > 256 ? G : 256;                                                               \
+        const unsigned grid = gridFor(rows, threads / G);                                                         \
+        if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows); \
+        else crossEntropyKernel<G, MAXE, 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows);      \
+        break;                                                                                                    \
+    }
+    do {
+        BF_CE(64, 4) BF_CE(64, 8) BF_CE(64, 16) BF_CE(256, 8) BF_CE(256, 16) BF_CE(256, 32) BF_CE(1024, 16) BF_CE(1024, 32)
+        crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows);
+    } while (0);
 #undef BF_CE
     BF_LAUNCH_CHECK();
     finishSumKernel<<<1, 1024, 0, s>>>(rl, rows, lossSum, accumulate);
@@ -152,7 +184,7 @@ int bf_hip_mse(const float* pred, const float* target, float* grad, float* lossS
         return BF_OK;
     }
     BF_REQUIRE(pred && target && grad, "NULL pointer");
-    unsigned grid = gridFor(n, size_t(kBlock) * 8, unsigned(computeUnits()) * 8);
+    unsigned grid = gridFor(n, size_t(kBlock) * 4, 65536);   // one 16-byte group per thread until the partial sums get too many
     Scratch partial(grid * sizeof(float));
     if (partial.status != BF_OK) return partial.status;
     float gradScale = 2.0f / float(n);

@@ -1,9 +1,11 @@
 // Multi-tensor optimizers: SGD and AdamW over every parameter in one launch.
 //
 // HBM-bound: AdamW moves 28 algorithmic bytes per parameter (read p, g, m, v; write p, m, v), SGD 12.
-// The host cuts every tensor into chunks of 8192 elements and launches one block per chunk, so the
-// grid is balanced however unequal the tensors are (the embedding table next to a bias vector); the
-// chunk table lives in device memory and is re-uploaded only when the parameter set changes.
+// The launch is one flat grid over all tensors laid end to end: a block owns 1024 consecutive elements of
+// one tensor (one 16-byte group per thread), finds its tensor by binary search in a small table of first
+// block indices, and touches its elements once.  The grid is balanced however unequal the tensors are (the
+// embedding table next to a bias vector) and walks every tensor in address order; the table (one entry per
+// tensor) lives in device memory and is re-uploaded only when the parameter set changes.
 #include "common.hpp"
 
 #include <cmath>
@@ -12,36 +14,35 @@
 namespace bf {
 namespace {
 
-constexpr size_t kChunk = size_t(kBlock) * 32;
+constexpr size_t kPerBlock = size_t(kBlock) * 4;
 
-struct SgdChunk {
+struct SgdTensor {
     float* p;
     const float* g;
-    unsigned count;
+    size_t count;
+    unsigned firstBlock;
     unsigned pad;
 };
-struct AdamChunk {
+struct AdamTensor {
     float* p;
     const float* g;
     float* m;
     float* v;
-    unsigned count;
+    size_t count;
+    unsigned firstBlock;
     unsigned pad;
 };
 
-inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
-__global__ void __launch_bounds__(kBlock) sgdKernel(const SgdChunk* __restrict__ chunks, float lr) {
-    SgdChunk c = chunks[blockIdx.x];
-    bool vec = ((reinterpret_cast<uintptr_t>(c.p) | reinterpret_cast<uintptr_t>(c.g)) & 15u) == 0;
-    unsigned done = 0;
+__global__ void __launch_bounds__(kBlock) sgdKernel(const SgdTensor* __restrict__ table, int numTensors, float lr) {
+    const SgdTensor c = table[owningTensor(table, numTensors, blockIdx.x)];
+    const size_t base = (size_t(blockIdx.x - c.firstBlock) * kBlock + threadIdx.x) * 4;
+    if (base >= c.count) return;
+    const bool vec = ((reinterpret_cast<uintptr_t>(c.p) | reinterpret_cast<uintptr_t>(c.g)) & 15u) == 0 && base + 4 <= c.count;
     if (vec) {
-        unsigned n4 = c.count / 4;
-        for (unsigned i = threadIdx.x; i < n4; i += blockDim.x)
-            storef4(c.p + 4 * i, loadf4(c.p + 4 * i) - loadf4(c.g + 4 * i) * lr);
-        done = n4 * 4;
+        storef4(c.p + base, loadf4(c.p + base) - loadf4(c.g + base) * lr);
+    } else {
+        for (size_t i = base; i < base + 4 && i < c.count; ++i) c.p[i] -= lr * c.g[i];
     }
-    for (unsigned i = done + threadIdx.x; i < c.count; i += blockDim.x) c.p[i] -= lr * c.g[i];
 }
 
 struct AdamParams {
@@ -56,28 +57,26 @@ __device__ __forceinline__ void adamOne(float& p, float g, float& m, float& v, c
     p -= a.lr * (mHat / (sqrtf(vHat) + a.eps) + a.weightDecay * p);
 }
 
-__global__ void __launch_bounds__(kBlock) adamwKernel(const AdamChunk* __restrict__ chunks, AdamParams a) {
-    AdamChunk c = chunks[blockIdx.x];
-    bool vec = ((reinterpret_cast<uintptr_t>(c.p) | reinterpret_cast<uintptr_t>(c.g) | reinterpret_cast<uintptr_t>(c.m) |
-                 reinterpret_cast<uintptr_t>(c.v)) & 15u) == 0;
-    unsigned done = 0;
+__global__ void __launch_bounds__(kBlock) adamwKernel(const AdamTensor* __restrict__ table, int numTensors, AdamParams a) {
+    const AdamTensor c = table[owningTensor(table, numTensors, blockIdx.x)];
+    const size_t base = (size_t(blockIdx.x - c.firstBlock) * kBlock + threadIdx.x) * 4;
+    if (base >= c.count) return;
+    const bool vec = ((reinterpret_cast<uintptr_t>(c.p) | reinterpret_cast<uintptr_t>(c.g) | reinterpret_cast<uintptr_t>(c.m) |
+                       reinterpret_cast<uintptr_t>(c.v)) & 15u) == 0 && base + 4 <= c.count;
     if (vec) {
-        unsigned n4 = c.count / 4;
-        for (unsigned i = threadIdx.x; i < n4; i += blockDim.x) {
-            float4v p = loadf4(c.p + 4 * i), g = loadf4(c.g + 4 * i), m = loadf4(c.m + 4 * i), v = loadf4(c.v + 4 * i);
+        float4v p = loadf4(c.p + base), g = loadf4(c.g + base), m = loadf4(c.m + base), v = loadf4(c.v + base);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float pj = p[j], mj = m[j], vj = v[j];
-                adamOne(pj, g[j], mj, vj, a);
-                p[j] = pj; m[j] = mj; v[j] = vj;
-            }
-            storef4(c.p + 4 * i, p);
-            storef4(c.m + 4 * i, m);
-            storef4(c.v + 4 * i, v);
+        for (int j = 0; j < 4; ++j) {
+            float pj = p[j], mj = m[j], vj = v[j];
+            adamOne(pj, g[j], mj, vj, a);
+            p[j] = pj; m[j] = mj; v[j] = vj;
         }
-        done = n4 * 4;
+        storef4(c.p + base, p);
+        storef4(c.m + base, m);
+        storef4(c.v + base, v);
+    } else {
+        for (size_t i = base; i < base + 4 && i < c.count; ++i) adamOne(c.p[i], c.g[i], c.m[i], c.v[i], a);
     }
-    for (unsigned i = done + threadIdx.x; i < c.count; i += blockDim.x) adamOne(c.p[i], c.g[i], c.m[i], c.v[i], a);
 }
 
 }  // namespace
@@ -91,19 +90,19 @@ int bf_hip_sgd_multi(float* const* params, const float* const* grads, const size
                      bf_stream_t stream) {
     if (numTensors == 0) return BF_OK;
     BF_REQUIRE(params && grads && counts, "NULL pointer");
-    std::vector<SgdChunk> chunks;
+    std::vector<SgdTensor> table;
+    size_t blocks = 0;
     for (size_t t = 0; t < numTensors; ++t) {
         BF_REQUIRE((params[t] && grads[t]) || counts[t] == 0, "NULL tensor pointer");
-        for (size_t off = 0; off < counts[t]; off += kChunk) {
-            size_t c = counts[t] - off < kChunk ? counts[t] - off : kChunk;
-            chunks.push_back(SgdChunk{params[t] + off, grads[t] + off, unsigned(c), 0});
-        }
+        table.push_back(SgdTensor{params[t], grads[t], counts[t], unsigned(blocks), 0});
+        blocks += (counts[t] + kPerBlock - 1) / kPerBlock;
+        BF_REQUIRE(blocks < (size_t(1) << 31), "too many elements for one launch");
     }
-    if (chunks.empty()) return BF_OK;
-    const void* table = nullptr;
-    int st = uploadDescriptorTable(kSlotSgd, chunks.data(), chunks.size() * sizeof(SgdChunk), asStream(stream), &table);
+    if (blocks == 0) return BF_OK;
+    const void* device = nullptr;
+    int st = uploadDescriptorTable(kSlotSgd, table.data(), table.size() * sizeof(SgdTensor), asStream(stream), &device);
     if (st != BF_OK) return st;
-    sgdKernel<<<unsigned(chunks.size()), kBlock, 0, asStream(stream)>>>(static_cast<const SgdChunk*>(table), lr);
+    sgdKernel<<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const SgdTensor*>(device), int(numTensors), lr);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -114,22 +113,22 @@ int bf_hip_adamw_multi(float* const* params, const float* const* grads, float* c
     BF_REQUIRE(step >= 1, "step must be >= 1");
     if (numTensors == 0) return BF_OK;
     BF_REQUIRE(params && grads && m && v && counts, "NULL pointer");
-    std::vector<AdamChunk> chunks;
+    std::vector<AdamTensor> table;
+    size_t blocks = 0;
     for (size_t t = 0; t < numTensors; ++t) {
         BF_REQUIRE((params[t] && grads[t] && m[t] && v[t]) || counts[t] == 0, "NULL tensor pointer");
-        for (size_t off = 0; off < counts[t]; off += kChunk) {
-            size_t c = counts[t] - off < kChunk ? counts[t] - off : kChunk;
-            chunks.push_back(AdamChunk{params[t] + off, grads[t] + off, m[t] + off, v[t] + off, unsigned(c), 0});
-        }
+        table.push_back(AdamTensor{params[t], grads[t], m[t], v[t], counts[t], unsigned(blocks), 0});
+        blocks += (counts[t] + kPerBlock - 1) / kPerBlock;
+        BF_REQUIRE(blocks < (size_t(1) << 31), "too many elements for one launch");
     }
-    if (chunks.empty()) return BF_OK;
-    const void* table = nullptr;
-    int st = uploadDescriptorTable(kSlotAdamW, chunks.data(), chunks.size() * sizeof(AdamChunk), asStream(stream), &table);
+    if (blocks == 0) return BF_OK;
+    const void* device = nullptr;
+    int st = uploadDescriptorTable(kSlotAdamW, table.data(), table.size() * sizeof(AdamTensor), asStream(stream), &device);
     if (st != BF_OK) return st;
     // bias corrections on the host in float, exactly like the reference (optimizer.cu:104-107)
     float t = static_cast<float>(step);
     AdamParams a{lr, beta1, beta2, eps, weightDecay, 1.0f - std::pow(beta1, t), 1.0f - std::pow(beta2, t)};
-    adamwKernel<<<unsigned(chunks.size()), kBlock, 0, asStream(stream)>>>(static_cast<const AdamChunk*>(table), a);
+    adamwKernel<<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const AdamTensor*>(device), int(numTensors), a);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

@@ -116,8 +116,14 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const
         const double k = gx / (double(features) * r * r * r);
         float* o = out + row * features;
         if constexpr (CACHED) {
+            if (features >= 64) {   // cancellation between the two terms is at most 1/features of either: float is enough
+                const float invRf = float(invR), kf = float(k);
 #pragma unroll
-            for (int i = 0; i < MAXE; ++i) rg.c.r[i] = float(double(rg.c.r[i]) * invR - double(rx.c.r[i]) * k);
+                for (int i = 0; i < MAXE; ++i) rg.c.r[i] = rg.c.r[i] * invRf - rx.c.r[i] * kf;
+            } else {
+#pragma unroll
+                for (int i = 0; i < MAXE; ++i) rg.c.r[i] = float(double(rg.c.r[i]) * invR - double(rx.c.r[i]) * k);
+            }
             rg.c.store(o, features, t);
         } else {
             for (size_t e = t; e < features; e += G) o[e] = float(double(rg.p[e]) * invR - double(rx.p[e]) * k);
@@ -189,34 +195,36 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) softmaxBackwardKernel(const
     }
 }
 
-// Picks the instantiation for a row length.  ONE_INPUT kernels keep up to 16/32/64 elements per
-// thread, two-input kernels half of that for the 1024-thread group (register budget of 16 waves/CU).
+// Picks the instantiation for a row length: the smallest group (64, 256 or 1024 threads per row) and the
+// smallest per-thread register count whose product holds the row, so short rows carry no padding work and
+// no variant spills.  Two-input kernels get half the registers per input at 1024 threads (16 waves per CU
+// leave 128 VGPRs each).  Every block takes its rows once: the grid covers all rows, which keeps the HBM
+// access stream in address order.
+#define BF_ROW_CASE(KERNEL, G, MAXE, limitRows)                                                                    \
+    if ((features_) <= size_t(G) * MAXE) {                                                                         \
+        const unsigned threads = G > 256 ? G : 256;                                                                \
+        const unsigned grid = gridFor(rows_, threads / G);                                                         \
+        if (vec4) KERNEL<G, MAXE, 4, true><<<grid, threads, 0, stream_>>>(ARGS_);                                  \
+        else KERNEL<G, MAXE, 1, true><<<grid, threads, 0, stream_>>>(ARGS_);                                       \
+        break;                                                                                                     \
+    }
 #define BF_ROW_LAUNCH(KERNEL, TWO_INPUTS, vecOk, rows, features, stream, ...)                                      \
     do {                                                                                                           \
-        const bool vec4 = (vecOk) && (features) % 4 == 0;                                                          \
-        const int big = (TWO_INPUTS) ? 32 : 64;                                                                    \
-        const unsigned cap = unsigned(computeUnits()) * 8;                                                         \
-        if ((features) <= 64 * 16) {                                                                               \
-            unsigned grid = gridFor(rows, 4, cap);                                                                 \
-            if (vec4) KERNEL<64, 16, 4, true><<<grid, 256, 0, stream>>>(__VA_ARGS__);                              \
-            else KERNEL<64, 16, 1, true><<<grid, 256, 0, stream>>>(__VA_ARGS__);                                   \
-        } else if ((features) <= 256 * 32) {                                                                       \
-            unsigned grid = gridFor(rows, 1, cap);                                                                 \
-            if (vec4) KERNEL<256, 32, 4, true><<<grid, 256, 0, stream>>>(__VA_ARGS__);                             \
-            else KERNEL<256, 32, 1, true><<<grid, 256, 0, stream>>>(__VA_ARGS__);                                  \
-        } else if ((features) <= size_t(1024) * big) {                                                             \
-            unsigned grid = gridFor(rows, 1, cap);                                                                 \
-            if (TWO_INPUTS) {                                                                                      \
-                if (vec4) KERNEL<1024, 32, 4, true><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                       \
-                else KERNEL<1024, 32, 1, true><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                            \
-            } else {                                                                                               \
-                if (vec4) KERNEL<1024, 64, 4, true><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                       \
-                else KERNEL<1024, 64, 1, true><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                            \
-            }                                                                                                      \
-        } else {                                                                                                   \
-            unsigned grid = gridFor(rows, 1, cap);                                                                 \
-            KERNEL<1024, 4, 1, false><<<grid, 1024, 0, stream>>>(__VA_ARGS__);                                     \
+        const size_t rows_ = (rows), features_ = (features);                                                       \
+        hipStream_t stream_ = (stream);                                                                            \
+        const bool vec4 = (vecOk) && features_ % 4 == 0;                                                           \
+        BF_ROW_CASE(KERNEL, 64, 4, 0)                                                                              \
+        BF_ROW_CASE(KERNEL, 64, 8, 0)                                                                              \
+        BF_ROW_CASE(KERNEL, 64, 16, 0)                                                                             \
+        BF_ROW_CASE(KERNEL, 256, 8, 0)                                                                             \
+        BF_ROW_CASE(KERNEL, 256, 16, 0)                                                                            \
+        BF_ROW_CASE(KERNEL, 256, 32, 0)                                                                            \
+        BF_ROW_CASE(KERNEL, 1024, 16, 0)                                                                           \
+        if (!(TWO_INPUTS)) {                                                                                       \
+            BF_ROW_CASE(KERNEL, 1024, 32, 0)                                                                       \
+            if (vec4) { BF_ROW_CASE(KERNEL, 1024, 52, 0) }                                                         \
         }                                                                                                          \
+        KERNEL<1024, 4, 1, false><<<gridFor(rows_, 1), 1024, 0, stream_>>>(ARGS_);                                 \
     } while (0)
 
 }  // namespace
@@ -230,7 +238,9 @@ int bf_hip_rmsnorm(const float* x, float* out, size_t rows, size_t features, bf_
     if (rows == 0 || features == 0) return BF_OK;
     BF_REQUIRE(x && out, "NULL pointer");
     hipStream_t s = asStream(stream);
+#define ARGS_ x, out, rows, features
     BF_ROW_LAUNCH(rmsnormKernel, false, aligned16(x) && aligned16(out), rows, features, s, x, out, rows, features);
+#undef ARGS_
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -240,8 +250,10 @@ int bf_hip_rmsnorm_backward(const float* x, const float* g, float* out, size_t r
     if (rows == 0 || features == 0) return BF_OK;
     BF_REQUIRE(x && g && out, "NULL pointer");
     hipStream_t s = asStream(stream);
+#define ARGS_ x, g, out, rows, features
     BF_ROW_LAUNCH(rmsnormBackwardKernel, true, aligned16(x) && aligned16(g) && aligned16(out), rows, features, s, x, g,
                   out, rows, features);
+#undef ARGS_
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -250,7 +262,9 @@ int bf_hip_softmax(const float* x, float* out, size_t rows, size_t features, bf_
     if (rows == 0 || features == 0) return BF_OK;
     BF_REQUIRE(x && out, "NULL pointer");
     hipStream_t s = asStream(stream);
+#define ARGS_ x, out, rows, features
     BF_ROW_LAUNCH(softmaxKernel, false, aligned16(x) && aligned16(out), rows, features, s, x, out, rows, features);
+#undef ARGS_
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -260,8 +274,10 @@ int bf_hip_softmax_backward(const float* x, const float* g, float* out, size_t r
     if (rows == 0 || features == 0) return BF_OK;
     BF_REQUIRE(x && g && out, "NULL pointer");
     hipStream_t s = asStream(stream);
+#define ARGS_ x, g, out, rows, features
     BF_ROW_LAUNCH(softmaxBackwardKernel, true, aligned16(x) && aligned16(g) && aligned16(out), rows, features, s, x, g,
                   out, rows, features);
+#undef ARGS_
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

@@ -293,7 +293,7 @@ int bf_hip_fill_zero(void* dst, size_t bytes, bf_stream_t stream) {
     BF_REQUIRE((reinterpret_cast<uintptr_t>(dst) & 3u) == 0, "dst must be 4-byte aligned");
     size_t words = bytes / 4;
     if (words) {
-        unsigned grid = gridFor(words, size_t(kBlock) * 8, unsigned(computeUnits()) * 8);
+        unsigned grid = gridFor(words, size_t(kBlock) * 4);
         fillZeroKernel<<<grid, kBlock, 0, asStream(stream)>>>(static_cast<uint32_t*>(dst), words);
         BF_LAUNCH_CHECK();
     }
