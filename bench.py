@@ -33,9 +33,10 @@ PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# same command (profiles/attention_c3_*.md says how they were taken and scaled); None until measured.
-MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvKernel": None}
+# HBM bytes per launch of the dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this workload,
+# each scaled by what the same counter reads for a plain 256 MiB copy (x2.000 and x1.000): 755.8 MB read +
+# 134.2 MB written.  profiles/attention_c3_kernel_trace.md holds the commands and the raw counter values.
+MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvKernel": 890005068}
 
 
 def attention_flops(batch, heads, seq, hd):
@@ -291,6 +292,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extras", action="store_true", help="also time a bandwidth kernel and the bf16 GEMM")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 256 MiB copy (bf_hip_scale by 1.0) so that a counter run of this command "
+                         "holds a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--train", default="gpt_small", help="comma list of train-step workloads to add (tiny_lm, gpt_small, "
                     "long_context) or 'none'")
     args = ap.parse_args()
@@ -303,6 +307,12 @@ def main():
         sys.exit("bench.py: no HIP device visible; the operator library has no CPU fallback")
     props = bf.capi.device_props(0)
 
+    if args.calibrate_copy:
+        n = 64 * 1024 * 1024   # 256 MiB read + 256 MiB written by flat4Kernel<ScaleOp>
+        src, dst = bf.DeviceTensor.zeros((n,)), bf.DeviceTensor((n,))
+        bf.capi.call("bf_hip_scale", src.ptr, ctypes.c_float(1.0), dst.ptr, n, None)
+        bf.capi.call("bf_hip_synchronize")
+        del src, dst
     res = bench_attention(bf, args.steps, args.warmup)
     fl = res["flops"]
     total_flops = fl["fwd"] + fl["bwd"]

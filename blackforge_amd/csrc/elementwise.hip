@@ -206,13 +206,19 @@ __global__ void __launch_bounds__(256) columnSumKernel(const float* __restrict__
     }
 }
 
+// out[c] = sum of the partial rows of column c.  64 columns per block; four lanes per column each add every
+// fourth partial row (in index order) and the four sums are combined in a fixed order.
 __global__ void __launch_bounds__(kBlock) columnFinishKernel(const float* __restrict__ partial, float* __restrict__ out,
                                                              size_t parts, size_t features) {
-    size_t c = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (c >= features) return;
+    __shared__ float lds[4][64];
+    const int cx = threadIdx.x & 63, lane4 = threadIdx.x >> 6;
+    const size_t c = size_t(blockIdx.x) * 64 + cx;
     float s = 0.0f;
-    for (size_t p = 0; p < parts; ++p) s += partial[p * features + c];
-    out[c] = s;
+    if (c < features)
+        for (size_t p = lane4; p < parts; p += 4) s += partial[p * features + c];
+    lds[lane4][cx] = s;
+    __syncthreads();
+    if (lane4 == 0 && c < features) out[c] = (lds[0][cx] + lds[1][cx]) + (lds[2][cx] + lds[3][cx]);
 }
 
 template <int FUSED, int ACT>
@@ -235,7 +241,7 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
         columnSumKernel<1, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
     BF_LAUNCH_CHECK();
     if (dBias) {
-        columnFinishKernel<<<gridFor(features, kBlock), kBlock, 0, stream>>>(partial, dBias, parts, features);
+        columnFinishKernel<<<gridFor(features, 64), kBlock, 0, stream>>>(partial, dBias, parts, features);
         BF_LAUNCH_CHECK();
     }
     return BF_OK;
