@@ -87,6 +87,10 @@ SIGNATURES = {
     "bf_hip_gemm_bf16_nt": [P, P, P, c_size, c_size, c_size, S],
     "bf_hip_matmul_bf16": [P, P, P, c_size, c_size, c_size, c_int, S],
     "bf_hip_matmul_bf16_backward": [P, P, P, P, P, c_size, c_size, c_size, c_int, S],
+    "bf_hip_linear_bf16": [P, P, P, P, P, c_size, c_size, c_size, c_int, S],
+    "bf_hip_matmul_bf16_shared_input": [P, ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), c_size, c_size, c_size, c_size, c_int, S],
+    "bf_hip_matmul_bf16_shared_input_backward": [P, ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), P, ctypes.POINTER(c_ptr), c_size,
+                                                 c_size, c_size, c_size, c_int, S],
     "bf_hip_invalidate_bf16_weight_cache": [],
     "bf_hip_attention_forward": [P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_attention_dot_o_do": [P, P, P, c_size, c_size, c_size, c_size, S],

@@ -33,9 +33,9 @@ __device__ __forceinline__ unsigned short toBf16Bits(float x) {
 
 inline size_t pad8(size_t n) { return (n + 7) / 8 * 8; }
 
-// out[r, 0..colsPad) = bf16(x[r, 0..cols)), zero padded.
+// out[r*ld + 0..colsPad) = bf16(x[r, 0..cols)), zero padded.
 __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict__ x, unsigned short* __restrict__ out,
-                                                        size_t rows, size_t cols, size_t colsPad, int vec) {
+                                                        size_t rows, size_t cols, size_t colsPad, int vec, size_t ld) {
     const size_t groupsPerRow = colsPad / 8;
     const size_t total = rows * groupsPerRow;
     const size_t stride = size_t(gridDim.x) * blockDim.x;
@@ -51,7 +51,7 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict_
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = c + j < cols ? toBf16Bits(src[j]) : (unsigned short)0;
         }
-        *reinterpret_cast<ushort8*>(out + r * colsPad + c) = v;
+        *reinterpret_cast<ushort8*>(out + r * ld + c) = v;
     }
 }
 
@@ -147,19 +147,40 @@ __device__ __forceinline__ bool tileIndexXcd(int id, int tilesM, int tilesN, int
     return tm < tilesM && tn < tilesN;
 }
 
+// Where a product goes.  The N columns are cut into runs of `splitN` that land in up to three separate
+// [M, splitN] outputs (one GEMM for several projections of the same input; splitN is a multiple of the tile
+// width, so a tile belongs to one output); a single output has splitN == N.  `bias` ([N]) and `residual`
+// ([M, N], single output only) are added to the accumulator in that order before the store, the order in
+// which the separate add kernels would have done it.
+struct Epilogue {
+    float* c[3];
+    int splitN;
+    const float* bias;
+    const float* residual;
+};
+
 template <int TM, int TN>
-__device__ __forceinline__ void storeAccumulators(float16v (&acc)[TM][TN], float* __restrict__ C, int M, int N, int row0,
+__device__ __forceinline__ void storeAccumulators(float16v (&acc)[TM][TN], const Epilogue& e, int M, int N, int row0,
                                                   int col0, int li, int half) {
+    const int which = col0 / e.splitN;              // uniform over the tile
+    float* __restrict__ C = e.c[which];
+    const int shift = which * e.splitN, ld = e.splitN;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int col = col0 + j * 32 + li;
             if (col < N) {
+                const float b = e.bias ? e.bias[col] : 0.0f;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int row = row0 + i * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                    if (row < M) C[size_t(row) * N + col] = acc[i][j][r];
+                    if (row < M) {
+                        float v = acc[i][j][r];
+                        if (e.bias) v += b;
+                        if (e.residual) v += e.residual[size_t(row) * N + col];
+                        C[size_t(row) * ld + (col - shift)] = v;
+                    }
                 }
             }
         }
@@ -174,7 +195,7 @@ __device__ __forceinline__ void storeAccumulators(float16v (&acc)[TM][TN], float
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const unsigned short* __restrict__ A,
                                                                             const unsigned short* __restrict__ Bt,
-                                                                            float* __restrict__ C, int M, int N, int K, int lda,
+                                                                            Epilogue epi, int M, int N, int K, int lda,
                                                                             int ldb, int kPerSplit, size_t sliceStride) {
     constexpr int THREADS = WAVES_M * WAVES_N * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;     // per-wave tile
@@ -192,7 +213,7 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
     const int m0 = tm * BM, n0 = tn * BN;
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
     const int kBegin = blockIdx.y * kPerSplit, kEnd = min(K, kBegin + kPerSplit);
-    C += size_t(blockIdx.y) * sliceStride;
+    epi.c[0] += size_t(blockIdx.y) * sliceStride;   // slices are only used with a single plain output
 
     const int lr = tid >> 3, lc = (tid & 7) * 8;
     const unsigned short* aRow[A_PASSES];
@@ -254,7 +275,7 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
         }
         __syncthreads();
     }
-    storeAccumulators<TM, TN>(acc, C, M, N, m0 + wm0, n0 + wn0, li, half);
+    storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
 // Kernel for large products: 256 x 256 tile, 8 wavefronts in two groups of four.  Wavefronts w and w+4 of
@@ -271,7 +292,7 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
 // whole 128-byte lines.
 template <int XCD_ORDER>
 __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned short* __restrict__ A,
-                                                                 const unsigned short* __restrict__ Bt, float* __restrict__ C,
+                                                                 const unsigned short* __restrict__ Bt, Epilogue epi,
                                                                  int M, int N, int K, int lda, int ldb, int gmLog, int gnLog) {
     constexpr int BM = 256, BN = 256, TM = 4, TN = 2;
     extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
@@ -373,28 +394,36 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
         }
     }
     if (group == 0) __builtin_amdgcn_s_barrier();    // pairs with group 1's last barrier
-    storeAccumulators<TM, TN>(acc, C, M, N, m0 + wm0, n0 + wn0, li, half);
+    storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
-// C[i] = sum over slices of partial[s*sliceStride + i], slices added in index order (deterministic).
-// sliceStride is a multiple of 4; `vec` says that C is 16-byte aligned.
-__global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restrict__ partial, float* __restrict__ C, size_t count,
-                                                            size_t sliceStride, int slices, int vec) {
+// out = sum over slices of partial[s*sliceStride + i] (+ bias[i % N] + residual[i]), slices added in index order
+// (deterministic), written through the epilogue's output split.  sliceStride is a multiple of 4; `vec` says
+// that every pointer is 16-byte aligned and N and splitN are multiples of 4.
+__global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restrict__ partial, Epilogue e, size_t count,
+                                                            size_t sliceStride, int slices, int vec, size_t N) {
     const size_t stride = size_t(gridDim.x) * blockDim.x;
     const size_t first = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     const size_t count4 = vec ? count / 4 : 0;
+    const size_t splitN = size_t(e.splitN);
     for (size_t i = first; i < count4; i += stride) {
         float4v sum = loadf4(partial + 4 * i);
         for (int s = 1; s < slices; ++s) {
             float4v p = loadf4(partial + size_t(s) * sliceStride + 4 * i);
             sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w;
         }
-        storef4(C + 4 * i, sum);
+        const size_t row = (4 * i) / N, col = (4 * i) - row * N, which = col / splitN;
+        if (e.bias) sum = sum + loadf4(e.bias + col);
+        if (e.residual) sum = sum + loadf4(e.residual + 4 * i);
+        storef4(e.c[which] + row * splitN + (col - which * splitN), sum);
     }
     for (size_t i = 4 * count4 + first; i < count; i += stride) {
         float sum = partial[i];
         for (int s = 1; s < slices; ++s) sum += partial[size_t(s) * sliceStride + i];
-        C[i] = sum;
+        const size_t row = i / N, col = i - row * N, which = col / splitN;
+        if (e.bias) sum += e.bias[col];
+        if (e.residual) sum += e.residual[i];
+        e.c[which][row * splitN + (col - which * splitN)] = sum;
     }
 }
 
@@ -405,8 +434,8 @@ int allowSharedMemory(Kernel kernel, size_t smem) {
     return BF_OK;
 }
 
-int launchPingPong(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda,
-                   size_t ldb, hipStream_t s) {
+int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
+                   size_t lda, size_t ldb, hipStream_t s) {
     const size_t tilesM = (M + 255) / 256, tilesN = (N + 255) / 256;
     constexpr size_t smem = size_t(2) * 512 * LDS_ROW * sizeof(unsigned short);
     // XCD block shape: the 2^g x 2^(5-g) block that pads the tile grid least, squarest on ties
@@ -426,27 +455,28 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, float* C, 
         auto kernel = gemmBf16PingPongKernel<1>;
         int st = allowSharedMemory(kernel, smem);
         if (st != BF_OK) return st;
-        kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb), gmLog, gnLog);
+        kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), gmLog, gnLog);
     } else {
         size_t grid = tilesM * tilesN;
         if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
         auto kernel = gemmBf16PingPongKernel<0>;
         int st = allowSharedMemory(kernel, smem);
         if (st != BF_OK) return st;
-        kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb), 0, 0);
+        kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), 0, 0);
     }
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
 
-int launchGemmNt(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda,
-                 size_t ldb, hipStream_t s) {
+// epi.splitN must be N (one output) or a multiple of 256 (several outputs).
+int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
+                 size_t lda, size_t ldb, hipStream_t s) {
     if (M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
     const size_t cus = size_t(computeUnits());
     // 256x256 ping-pong tiles once they give three quarters of the CUs a tile; otherwise 128x128 tiles,
     // with K cut into slices when even those leave CUs idle and K is long enough to share out.
     const size_t bigTiles = ((M + 255) / 256) * ((N + 255) / 256);
-    if (bigTiles >= cus * 3 / 4) return launchPingPong(A, Bt, C, M, N, K, lda, ldb, s);
+    if (bigTiles >= cus * 3 / 4) return launchPingPong(A, Bt, epi, M, N, K, lda, ldb, s);
     const size_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     constexpr size_t smem = size_t(2) * (128 + 128) * LDS_ROW * sizeof(unsigned short);
     auto kernel = gemmBf16NtKernel<128, 128, 2, 2>;
@@ -461,26 +491,35 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, float* C, si
         const size_t count = M * N, sliceStride = (count + 3) / 4 * 4;
         Scratch partial(slices * sliceStride * sizeof(float));
         if (partial.status != BF_OK) return partial.status;
-        kernel<<<dim3(unsigned(tiles), unsigned(slices)), 256, smem, s>>>(A, Bt, partial.as<float>(), int(M), int(N), int(K),
-                                                                         int(lda), int(ldb), int(kPer), sliceStride);
+        Epilogue plain{{partial.as<float>(), nullptr, nullptr}, int(N), nullptr, nullptr};
+        kernel<<<dim3(unsigned(tiles), unsigned(slices)), 256, smem, s>>>(A, Bt, plain, int(M), int(N), int(K), int(lda), int(ldb),
+                                                                         int(kPer), sliceStride);
         BF_LAUNCH_CHECK();
-        const int vec = (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
-        splitReduceKernel<<<gridFor(count / 4 + 1, kBlock, unsigned(cus) * 8), kBlock, 0, s>>>(partial.as<float>(), C, count,
-                                                                                              sliceStride, int(slices), vec);
+        const int vec = ((reinterpret_cast<uintptr_t>(epi.c[0]) | reinterpret_cast<uintptr_t>(epi.c[1]) |
+                          reinterpret_cast<uintptr_t>(epi.c[2]) | reinterpret_cast<uintptr_t>(epi.residual) |
+                          reinterpret_cast<uintptr_t>(epi.bias)) & 15u) == 0 && N % 4 == 0 && epi.splitN % 4 == 0;
+        splitReduceKernel<<<gridFor(count / 4 + 1, kBlock), kBlock, 0, s>>>(partial.as<float>(), epi, count, sliceStride, int(slices),
+                                                                          vec, N);
         BF_LAUNCH_CHECK();
         return BF_OK;
     }
-    kernel<<<dim3(unsigned(tiles), 1), 256, smem, s>>>(A, Bt, C, int(M), int(N), int(K), int(lda), int(ldb), int(K), size_t(0));
+    kernel<<<dim3(unsigned(tiles), 1), 256, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), int(K), size_t(0));
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
+int launchGemmNt(const unsigned short* A, const unsigned short* Bt, float* C, size_t M, size_t N, size_t K, size_t lda,
+                 size_t ldb, hipStream_t s) {
+    return launchGemmNt(A, Bt, Epilogue{{C, nullptr, nullptr}, int(N), nullptr, nullptr}, M, N, K, lda, ldb, s);
+}
 
-int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, hipStream_t s) {
+// ld: elements between rows of `out` (0 = pad8(cols), a dense image); with ld > pad8(cols) the image is a column
+// slice of a wider one.
+int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, hipStream_t s, size_t ld = 0) {
     size_t colsPad = pad8(cols);
     size_t groups = rows * (colsPad / 8);
     if (groups == 0) return BF_OK;
     int vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && cols % 4 == 0;
-    convertKernel<<<gridFor(groups, kBlock), kBlock, 0, s>>>(x, out, rows, cols, colsPad, vec);
+    convertKernel<<<gridFor(groups, kBlock), kBlock, 0, s>>>(x, out, rows, cols, colsPad, vec, ld ? ld : colsPad);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -496,34 +535,51 @@ int convertTransposed(const float* x, unsigned short* out, size_t rows, size_t c
     return BF_OK;
 }
 
-// ---- bf16 images of weights, kept per (device, pointer, layout) until invalidated -------------------
+// ---- bf16 images of weights, kept per (device, pointers, layout) until invalidated ------------------
+// Layouts: 0 plain [rows, pad8(cols)]; 1 transposed [cols, pad8(rows)]; for a group of up to three weights of one
+// shape, 2 = their transposed images stacked row-wise ([count*cols, pad8(rows)], the Bt operand of one GEMM that
+// produces all their products) and 3 = their plain images side by side ([rows, count*cols], the Bt operand of
+// the one GEMM that sums their input gradients).
 struct CachedWeight {
     size_t generation;
     void* buffer;
     size_t bytes;
 };
 size_t g_generation = 0;
-std::map<std::tuple<int, const float*, int>, CachedWeight>& weightCache() {
-    static std::map<std::tuple<int, const float*, int>, CachedWeight> cache;
+using WeightKey = std::tuple<int, const float*, const float*, const float*, int>;
+std::map<WeightKey, CachedWeight>& weightCache() {
+    static std::map<WeightKey, CachedWeight> cache;
     return cache;
 }
 
-// Returns a bf16 image of w[rows, cols]: transposed ([cols, pad8(rows)]) or plain ([rows, pad8(cols)]).
-// With `cache` the image is kept; otherwise it is a scratch buffer the caller releases with releaseImage.
-int weightImage(const float* w, size_t rows, size_t cols, bool transposed, bool cache, hipStream_t s, unsigned short** image,
-                size_t* imageBytes) {
-    size_t bytes = (transposed ? cols * pad8(rows) : rows * pad8(cols)) * sizeof(unsigned short);
+int fillWeightImage(const float* const* w, size_t count, size_t rows, size_t cols, int layout, unsigned short* image, hipStream_t s) {
+    int st = BF_OK;
+    for (size_t i = 0; i < count && st == BF_OK; ++i) {
+        if (layout == 0) st = convertPlain(w[i], image, rows, cols, s);
+        else if (layout == 1) st = convertTransposed(w[i], image, rows, cols, s);
+        else if (layout == 2) st = convertTransposed(w[i], image + i * cols * pad8(rows), rows, cols, s);
+        else st = convertPlain(w[i], image + i * cols, rows, cols, s, count * cols);   // cols % 8 == 0 checked by the caller
+    }
+    return st;
+}
+
+// Returns the bf16 image of `count` weights w[i][rows, cols] in `layout`.  With `cache` the image is kept;
+// otherwise it is a scratch buffer the caller releases with bf_hip_pool_release(image, bytes).
+int weightImage(const float* const* w, size_t count, size_t rows, size_t cols, int layout, bool cache, hipStream_t s,
+                unsigned short** image, size_t* imageBytes) {
+    size_t elems = (layout == 0 || layout == 3) ? rows * pad8(cols) * count : count * cols * pad8(rows);
+    size_t bytes = elems * sizeof(unsigned short);
     *imageBytes = bytes;
     int dev = 0;
     BF_HIP_TRY(hipGetDevice(&dev));
+    void* buf = nullptr;
     if (cache) {
-        auto key = std::make_tuple(dev, w, transposed ? 1 : 0);
+        WeightKey key{dev, w[0], count > 1 ? w[1] : nullptr, count > 2 ? w[2] : nullptr, layout};
         auto it = weightCache().find(key);
         if (it != weightCache().end() && it->second.generation == g_generation && it->second.bytes == bytes) {
             *image = static_cast<unsigned short*>(it->second.buffer);
             return BF_OK;
         }
-        void* buf = nullptr;
         if (it != weightCache().end() && it->second.bytes == bytes) buf = it->second.buffer;   // refresh in place
         else {
             if (it != weightCache().end()) bf_hip_pool_release(it->second.buffer, it->second.bytes);
@@ -531,14 +587,16 @@ int weightImage(const float* w, size_t rows, size_t cols, bool transposed, bool 
             if (st != BF_OK) return st;
         }
         weightCache()[key] = CachedWeight{g_generation, buf, bytes};
-        *image = static_cast<unsigned short*>(buf);
     } else {
-        void* buf = nullptr;
         int st = bf_hip_pool_acquire(bytes, &buf);
         if (st != BF_OK) return st;
-        *image = static_cast<unsigned short*>(buf);
     }
-    return transposed ? convertTransposed(w, *image, rows, cols, s) : convertPlain(w, *image, rows, cols, s);
+    *image = static_cast<unsigned short*>(buf);
+    return fillWeightImage(w, count, rows, cols, layout, *image, s);
+}
+int weightImage(const float* w, size_t rows, size_t cols, bool transposed, bool cache, hipStream_t s, unsigned short** image,
+                size_t* imageBytes) {
+    return weightImage(&w, 1, rows, cols, transposed ? 1 : 0, cache, s, image, imageBytes);
 }
 
 }  // namespace
@@ -641,6 +699,151 @@ int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, 
         st = convertTransposed(g, gT.as<unsigned short>(), m, n, s);
         if (st != BF_OK) return st;
         st = launchGemmNt(aT.as<unsigned short>(), gT.as<unsigned short>(), dB, k, n, mp, mp, mp, s);
+    }
+    return st;
+}
+
+int bf_hip_linear_bf16(const float* a, const float* w, const float* bias, const float* residual, float* out, size_t m, size_t k,
+                       size_t n, int cacheWeight, bf_stream_t stream) {
+    if (m == 0 || n == 0) return BF_OK;
+    BF_REQUIRE(out != nullptr, "NULL output");
+    int st = BF_OK;
+    if (k == 0) {   // empty contraction: out = bias + residual
+        st = bf_hip_fill_zero(out, m * n * sizeof(float), stream);
+        if (st == BF_OK && bias) st = bf_hip_add_bias(out, bias, out, m, n, stream);
+        if (st == BF_OK && residual) st = bf_hip_accumulate(out, residual, m * n, stream);
+        return st;
+    }
+    BF_REQUIRE(a && w, "NULL operand");
+    hipStream_t s = asStream(stream);
+    const size_t kp = pad8(k);
+    Scratch aImg(m * kp * sizeof(unsigned short));
+    if (aImg.status != BF_OK) return aImg.status;
+    unsigned short* wImg = nullptr;
+    size_t wBytes = 0;
+    st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
+    if (st != BF_OK) return st;
+    st = weightImage(w, k, n, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
+    if (st != BF_OK) return st;
+    st = launchGemmNt(aImg.as<unsigned short>(), wImg, Epilogue{{out, nullptr, nullptr}, int(n), bias, residual}, m, n, kp, kp, kp, s);
+    if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+    return st;
+}
+
+int bf_hip_matmul_bf16_shared_input(const float* a, const float* const* b, float* const* c, size_t count, size_t m, size_t k,
+                                    size_t n, int cacheWeight, bf_stream_t stream) {
+    BF_REQUIRE(count >= 1 && count <= 3, "count must be 1, 2 or 3");
+    BF_REQUIRE(b && c, "NULL pointer array");
+    if (m == 0 || n == 0) return BF_OK;
+    for (size_t i = 0; i < count; ++i) BF_REQUIRE(c[i] != nullptr, "NULL output");
+    if (k == 0) {
+        for (size_t i = 0; i < count; ++i) {
+            int st = bf_hip_fill_zero(c[i], m * n * sizeof(float), stream);
+            if (st != BF_OK) return st;
+        }
+        return BF_OK;
+    }
+    BF_REQUIRE(a != nullptr, "NULL operand");
+    for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] != nullptr, "NULL operand");
+    hipStream_t s = asStream(stream);
+    const size_t kp = pad8(k);
+    Scratch aImg(m * kp * sizeof(unsigned short));
+    if (aImg.status != BF_OK) return aImg.status;
+    int st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
+    if (st != BF_OK) return st;
+    unsigned short* wImg = nullptr;
+    size_t wBytes = 0;
+    if (count > 1 && n % 256 == 0) {   // one GEMM over the stacked weight images, tiles routed to their output
+        st = weightImage(b, count, k, n, 2, cacheWeight != 0, s, &wImg, &wBytes);
+        if (st != BF_OK) return st;
+        Epilogue epi{{c[0], count > 1 ? c[1] : nullptr, count > 2 ? c[2] : nullptr}, int(n), nullptr, nullptr};
+        st = launchGemmNt(aImg.as<unsigned short>(), wImg, epi, m, count * n, kp, kp, kp, s);
+        if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+        return st;
+    }
+    for (size_t i = 0; i < count; ++i) {
+        st = weightImage(b[i], k, n, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
+        if (st != BF_OK) return st;
+        st = launchGemmNt(aImg.as<unsigned short>(), wImg, c[i], m, n, kp, kp, kp, s);
+        if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+        if (st != BF_OK) return st;
+    }
+    return BF_OK;
+}
+
+int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const* b, const float* const* g, float* dA,
+                                             float* const* dB, size_t count, size_t m, size_t k, size_t n, int cacheWeight,
+                                             bf_stream_t stream) {
+    BF_REQUIRE(count >= 1 && count <= 3, "count must be 1, 2 or 3");
+    BF_REQUIRE(b && g, "NULL pointer array");
+    hipStream_t s = asStream(stream);
+    if (m == 0 || k == 0 || n == 0) {   // degenerate: gradients are zero
+        int st = BF_OK;
+        if (dA && m * k) st = bf_hip_fill_zero(dA, m * k * sizeof(float), stream);
+        for (size_t i = 0; dB && i < count && st == BF_OK; ++i)
+            if (dB[i] && k * n) st = bf_hip_fill_zero(dB[i], k * n * sizeof(float), stream);
+        return st;
+    }
+    BF_REQUIRE(a != nullptr, "NULL operand");
+    for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] && g[i], "NULL operand");
+    int st = BF_OK;
+    if (dA) {
+        if (count > 1 && n % 8 == 0) {
+            // dA = sum_i g_i b_i^T = [g_0 | g_1 | g_2] [b_0 | b_1 | b_2]^T: one GEMM whose contraction runs over all of them
+            const size_t nn = count * n;
+            Scratch gImg(m * nn * sizeof(unsigned short));
+            if (gImg.status != BF_OK) return gImg.status;
+            for (size_t i = 0; i < count; ++i) {
+                st = convertPlain(g[i], gImg.as<unsigned short>() + i * n, m, n, s, nn);
+                if (st != BF_OK) return st;
+            }
+            unsigned short* wImg = nullptr;
+            size_t wBytes = 0;
+            st = weightImage(b, count, k, n, 3, cacheWeight != 0, s, &wImg, &wBytes);
+            if (st != BF_OK) return st;
+            st = launchGemmNt(gImg.as<unsigned short>(), wImg, dA, m, k, nn, nn, nn, s);
+            if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+            if (st != BF_OK) return st;
+        } else {
+            Scratch extra(count > 1 ? m * k * sizeof(float) : 0);
+            if (extra.status != BF_OK) return extra.status;
+            for (size_t i = 0; i < count; ++i) {
+                float* target = i == 0 ? dA : extra.as<float>();
+                st = bf_hip_matmul_bf16_backward(a, b[i], g[i], target, nullptr, m, k, n, cacheWeight, stream);
+                if (st != BF_OK) return st;
+                if (i > 0) st = bf_hip_accumulate(dA, target, m * k, stream);
+                if (st != BF_OK) return st;
+            }
+        }
+    }
+    bool anyDb = false;
+    for (size_t i = 0; dB && i < count; ++i) anyDb = anyDb || dB[i] != nullptr;
+    if (anyDb) {
+        const size_t mp = pad8(m);
+        Scratch aT(k * mp * sizeof(unsigned short));
+        if (aT.status != BF_OK) return aT.status;
+        st = convertTransposed(a, aT.as<unsigned short>(), m, k, s);
+        if (st != BF_OK) return st;
+        bool all = true;
+        for (size_t i = 0; i < count; ++i) all = all && dB[i] != nullptr;
+        Scratch gT(count * n * mp * sizeof(unsigned short));
+        if (gT.status != BF_OK) return gT.status;
+        for (size_t i = 0; i < count; ++i) {
+            if (!dB[i]) continue;
+            st = convertTransposed(g[i], gT.as<unsigned short>() + i * n * mp, m, n, s);
+            if (st != BF_OK) return st;
+        }
+        if (all && count > 1 && n % 256 == 0) {
+            Epilogue epi{{dB[0], count > 1 ? dB[1] : nullptr, count > 2 ? dB[2] : nullptr}, int(n), nullptr, nullptr};
+            st = launchGemmNt(aT.as<unsigned short>(), gT.as<unsigned short>(), epi, k, count * n, mp, mp, mp, s);
+            if (st != BF_OK) return st;
+        } else {
+            for (size_t i = 0; i < count; ++i) {
+                if (!dB[i]) continue;
+                st = launchGemmNt(aT.as<unsigned short>(), gT.as<unsigned short>() + i * n * mp, dB[i], k, n, mp, mp, mp, s);
+                if (st != BF_OK) return st;
+            }
+        }
     }
     return st;
 }

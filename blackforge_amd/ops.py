@@ -333,9 +333,52 @@ def _linear(name, x, w, bias, mm):
     return out
 
 
+def _linear_bf16(name, x, w, bias, residual, cache):
+    """x w (+ bias) (+ residual) with the adds folded into the GEMM's store (bf_hip_linear_bf16)."""
+    _require(x.rank() >= 2, f"{name}: needs a tensor of rank >= 2")
+    _require(w.rank() == 2 and x.shape[-1] == w.shape[0], f"{name}: incompatible shapes {x.shape} x {w.shape}")
+    _require(bias is None or (bias.rank() == 1 and bias.shape[0] == w.shape[1]), f"{name}: bias does not match {w.shape}")
+    out = DeviceTensor(x.shape[:-1] + (w.shape[1],))
+    _require(residual is None or residual.shape == out.shape, f"{name}: residual shape differs from the product")
+    rows = out.elementCount() // w.shape[1] if w.shape[1] else 0
+    _call("bf_hip_linear_bf16", x.ptr, w.ptr, bias.ptr if bias is not None else None, residual.ptr if residual is not None else None,
+          out.ptr, rows, w.shape[0], w.shape[1], cache, None)
+    return out
+
+
 def linear(x, w, bias): return _linear("linear", x, w, bias, matmul)
-def linearBf16(x, w, bias): return _linear("linearBf16", x, w, bias, matmulBf16)
-def linearBf16CachedWeight(x, w, bias): return _linear("linearBf16CachedWeight", x, w, bias, matmulBf16CachedWeight)
+def linearBf16(x, w, bias): return _linear_bf16("linearBf16", x, w, bias, None, 0)
+def linearBf16CachedWeight(x, w, bias): return _linear_bf16("linearBf16CachedWeight", x, w, bias, None, 1)
+def linearBf16Fused(x, w, bias=None, residual=None, cached=False):
+    """The projection-plus-adds form the composite blocks use: bias and residual are optional."""
+    return _linear_bf16("linearBf16Fused", x, w, bias, residual, 1 if cached else 0)
+
+
+def _ptr_array(tensors):
+    """A host array of device pointers; None entries and empty tensors become NULL."""
+    return (ctypes.c_void_p * len(tensors))(*[t.ptr.value if t is not None and t.ptr else None for t in tensors])
+
+
+def matmulBf16SharedInput(a, weights, cached=False):
+    """[a w for w in weights] for up to three weights of one shape: one conversion of `a`, one GEMM when it can be."""
+    _require(1 <= len(weights) <= 3, "matmulBf16SharedInput: one to three weights")
+    _require(a.rank() == 2 and all(w.rank() == 2 and w.shape == weights[0].shape and w.shape[0] == a.shape[1] for w in weights),
+             "matmulBf16SharedInput: incompatible shapes")
+    outs = [DeviceTensor((a.shape[0], w.shape[1])) for w in weights]
+    _call("bf_hip_matmul_bf16_shared_input", a.ptr, _ptr_array(weights), _ptr_array(outs), len(weights), a.shape[0], a.shape[1],
+          weights[0].shape[1], 1 if cached else 0, None)
+    return outs
+
+
+def matmulBf16SharedInputBackward(a, weights, grads, cached=False, want_dA=True, want_dB=(True, True, True)):
+    """dA = sum_i g_i w_i^T and dB_i = a^T g_i for the products of matmulBf16SharedInput."""
+    _require(len(weights) == len(grads) and 1 <= len(weights) <= 3, "matmulBf16SharedInputBackward: one to three products")
+    dA = DeviceTensor(a.shape) if want_dA else None
+    dBs = [DeviceTensor(w.shape) if want_dB[i] else None for i, w in enumerate(weights)]
+    _call("bf_hip_matmul_bf16_shared_input_backward", a.ptr, _ptr_array(weights), _ptr_array(grads),
+          dA.ptr if dA is not None else None, _ptr_array(dBs), len(weights), a.shape[0], a.shape[1], weights[0].shape[1],
+          1 if cached else 0, None)
+    return dA, dBs
 
 
 # ------------------------------------------------------------------------------------------------
@@ -648,10 +691,6 @@ class Parameter:
     name: str
     value: DeviceTensor
     grad: DeviceTensor
-
-
-def _ptr_array(tensors):
-    return (ctypes.c_void_p * len(tensors))(*[t.ptr.value if t.ptr else None for t in tensors])
 
 
 class SGD:

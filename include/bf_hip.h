@@ -198,6 +198,24 @@ int bf_hip_matmul_bf16(const float* a, const float* b, float* c, size_t m, size_
  * dA[m,k] = bf16(g) * bf16(b)^T, dB[k,n] = bf16(a)^T * bf16(g).  Either output may be NULL. */
 int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, float* dA, float* dB, size_t m,
                                 size_t k, size_t n, int cacheWeight, bf_stream_t stream);
+/* linearBf16 ops.hpp:253 / linearBf16CachedWeight ops.hpp:258, with the adds that follow a projection in the
+ * composite blocks folded into the GEMM's store: out[m,n] = bf16(a[m,k]) * bf16(w[k,n]) + bias[n] + residual[m,n].
+ * `bias` and `residual` may each be NULL (both NULL = matmulBf16).  The sum is formed in the order the separate
+ * kernels would use (addBias ops.hpp:14, addBiasResidual ops.hpp:30, add ops.hpp:8): product, then bias, then residual. */
+int bf_hip_linear_bf16(const float* a, const float* w, const float* bias, const float* residual, float* out, size_t m,
+                       size_t k, size_t n, int cacheWeight, bf_stream_t stream);
+/* The Q, K and V projections of selfAttentionForwardCached (ops_transformer.cu:217-257: three matmulBf16 calls on
+ * the same normalised input): c[i][m,n] = bf16(a[m,k]) * bf16(b[i][k,n]) for i < count (count <= 3; `b` and `c` are
+ * HOST arrays of device pointers).  The input is converted once; when n is a multiple of 256 the products run as
+ * one GEMM over the stacked weight images, each tile stored to its own output. */
+int bf_hip_matmul_bf16_shared_input(const float* a, const float* const* b, float* const* c, size_t count, size_t m,
+                                    size_t k, size_t n, int cacheWeight, bf_stream_t stream);
+/* Their gradients in selfAttentionBackwardCached (autodiff.cu:756-798: three matmulBf16Backward calls and two adds):
+ * dA[m,k] = sum_i bf16(g[i][m,n]) * bf16(b[i][k,n])^T (one GEMM whose contraction runs over all outputs when n is a
+ * multiple of 8), dB[i][k,n] = bf16(a)^T * bf16(g[i]).  dA, dB and any dB[i] may be NULL. */
+int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const* b, const float* const* g, float* dA,
+                                             float* const* dB, size_t count, size_t m, size_t k, size_t n,
+                                             int cacheWeight, bf_stream_t stream);
 /* invalidateBf16WeightCache: ops.hpp:80 */
 int bf_hip_invalidate_bf16_weight_cache(void);
 

@@ -227,6 +227,18 @@ inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& inpu
     MatmulGrad outGrad = projectionBackward(cache.attnOutput, wout, gradOutput, mode, {batch, seq, dim});
     FusedAttentionGrad attn = fusedAttentionBackward(outGrad.dA, cache.q, cache.k, cache.v, cache.attnOutput, cache.attnM,
                                                       cache.attnL, numHeads, scaleFactor, 0);
+    if (mode != 0) {
+        // the three projection gradients share their input: one GEMM sums dQ Wq^T + dK Wk^T + dV Wv^T, one produces
+        // the three weight gradients (for widths that are multiples of 256; separate GEMMs otherwise)
+        DeviceTensor dNormed({batch, seq, dim}), dWq(wq.shape()), dWk(wk.shape()), dWv(wv.shape());
+        const float* weights[3] = {wq.data(), wk.data(), wv.data()};
+        const float* grads[3] = {attn.dQ.data(), attn.dK.data(), attn.dV.data()};
+        float* weightGrads[3] = {dWq.data(), dWk.data(), dWv.data()};
+        check(bf_hip_matmul_bf16_shared_input_backward(cache.normedFlat.data(), weights, grads, dNormed.data(), weightGrads, 3,
+                                                       batch * seq, dim, dim, mode == 2, nullptr));
+        DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, dNormed));
+        return SelfAttentionGrad{std::move(dInput), std::move(dWq), std::move(dWk), std::move(dWv), std::move(outGrad.dB)};
+    }
     MatmulGrad gq = projectionBackward(cache.normedFlat, wq, attn.dQ, mode, {batch * seq, dim});
     MatmulGrad gk = projectionBackward(cache.normedFlat, wk, attn.dK, mode, {batch * seq, dim});
     MatmulGrad gv = projectionBackward(cache.normedFlat, wv, attn.dV, mode, {batch * seq, dim});

@@ -37,6 +37,16 @@ inline DeviceTensor projection(const DeviceTensor& a, const DeviceTensor& b, int
     else check(bf_hip_matmul_bf16(a.data(), b.data(), c.data(), m, k, n, bf16 == 2, nullptr));
     return c;
 }
+// bf16 projection with the adds that follow it folded into the GEMM's store: a*b (+ bias) (+ residual).
+// bf16: 1 = fresh weight image, 2 = cached weight image.
+inline DeviceTensor projectionFused(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor* bias, const DeviceTensor* residual,
+                                    int bf16, std::vector<std::size_t> outShape) {
+    DeviceTensor c(std::move(outShape));
+    const std::size_t k = b.dim(0), n = b.dim(1), m = n ? c.elementCount() / n : 0;
+    check(bf_hip_linear_bf16(a.data(), b.data(), bias ? bias->data() : nullptr, residual ? residual->data() : nullptr, c.data(), m, k,
+                             n, bf16 == 2, nullptr));
+    return c;
+}
 }  // namespace detail
 
 inline DeviceTensor add(const DeviceTensor& a, const DeviceTensor& b) {
@@ -170,6 +180,7 @@ inline DeviceTensor linearImpl(const char* op, const DeviceTensor& input, const 
     require(input.rank() >= 2, std::string(op) + ": needs a tensor of rank >= 2");
     require(weight.rank() == 2 && lastDim(input) == weight.dim(0), std::string(op) + ": incompatible shapes on the device");
     require(bias.rank() == 1 && bias.dim(0) == weight.dim(1), std::string(op) + ": bias does not match the weight");
+    if (bf16 != 0) return projectionFused(input, weight, &bias, nullptr, bf16, withLastDim(input, weight.dim(1)));
     DeviceTensor product = projection(input, weight, bf16, withLastDim(input, weight.dim(1)));
     DeviceTensor out(product.shape());
     check(bf_hip_add_bias(product.data(), bias.data(), out.data(), rowsOf(product), bias.dim(0), nullptr));
@@ -203,6 +214,11 @@ inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const De
     cache.normed = rmsnorm(input);
     cache.gemm1 = detail::projection(cache.normed, w1, mode, detail::withLastDim(input, w1.dim(1)));
     cache.hidden = addBiasActivation(cache.gemm1, b1, act);
+    if (mode != 0) {
+        require(b2.rank() == 1 && b2.dim(0) == w2.dim(1), "addBiasResidual: expected input [..., features] and bias [features]");
+        require(w2.dim(1) == detail::lastDim(input), "addBiasResidual: residual shape differs from the product");
+        return detail::projectionFused(cache.hidden, w2, &b2, &input, mode, input.shape());
+    }
     DeviceTensor gemm2 = detail::projection(cache.hidden, w2, mode, detail::withLastDim(input, w2.dim(1)));
     return addBiasResidual(gemm2, b2, input);
 }
@@ -246,13 +262,26 @@ inline DeviceTensor selfAttentionForwardImpl(const char* op, const DeviceTensor&
     std::size_t batch = input.dim(0), seq = input.dim(1), dim = input.dim(2);
     float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
     cache.normedFlat = rmsnorm(input).reshaped({batch * seq, dim});
-    cache.q = projection(cache.normedFlat, wq, mode, {batch, seq, dim});
-    cache.k = projection(cache.normedFlat, wk, mode, {batch, seq, dim});
-    cache.v = projection(cache.normedFlat, wv, mode, {batch, seq, dim});
+    if (mode != 0) {
+        // one conversion of the normalised input and (for widths that are multiples of 256) one GEMM for Q, K and V
+        require(wq.rank() == 2 && wq.shape() == wk.shape() && wq.shape() == wv.shape() && wq.dim(0) == dim && wq.dim(1) == dim,
+                std::string(op) + ": projection weights must be [dim, dim]");
+        cache.q = DeviceTensor({batch, seq, dim});
+        cache.k = DeviceTensor({batch, seq, dim});
+        cache.v = DeviceTensor({batch, seq, dim});
+        const float* weights[3] = {wq.data(), wk.data(), wv.data()};
+        float* outputs[3] = {cache.q.data(), cache.k.data(), cache.v.data()};
+        check(bf_hip_matmul_bf16_shared_input(cache.normedFlat.data(), weights, outputs, 3, batch * seq, dim, dim, mode == 2, nullptr));
+    } else {
+        cache.q = projection(cache.normedFlat, wq, mode, {batch, seq, dim});
+        cache.k = projection(cache.normedFlat, wk, mode, {batch, seq, dim});
+        cache.v = projection(cache.normedFlat, wv, mode, {batch, seq, dim});
+    }
     FusedAttentionForwardResult attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, 0);
     cache.attnOutput = std::move(attn.output);
     cache.attnM = std::move(attn.m);
     cache.attnL = std::move(attn.l);
+    if (mode != 0) return projectionFused(cache.attnOutput, wout, nullptr, &input, mode, {batch, seq, dim});
     DeviceTensor projected = projection(cache.attnOutput, wout, mode, {batch, seq, dim});
     return add(input, projected);
 }

@@ -135,6 +135,56 @@ def test_bf16_projection_large_tile_kernel(hip, oracle, rng, m, k, n):
     assert_close(c, expected, tol=1e-4, what="bf16 fwd (large tiles) vs rounded operands")
 
 
+@pytest.mark.parametrize("m,k,n", [(33, 40, 24), (300, 72, 520), (2100, 136, 3000), (70, 4100, 90)])
+@pytest.mark.parametrize("with_bias,with_residual", [(True, False), (False, True), (True, True), (False, False)])
+def test_bf16_linear_with_adds_in_the_store(hip, oracle, rng, m, k, n, with_bias, with_residual):
+    """bf_hip_linear_bf16 = matmulBf16 followed by addBias / addBiasResidual / add (ops.hpp:14,30,8), through every
+    GEMM path: small tiles, large tiles, and a contraction cut into slices."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, w, bias, res = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, n), r(rng, m, n)
+    got = ops.linearBf16Fused(D.fromHost(a), D.fromHost(w), D.fromHost(bias) if with_bias else None,
+                              D.fromHost(res) if with_residual else None).toHost()
+    expected = (oracle.roundToBf16(a).astype(np.float64) @ oracle.roundToBf16(w).astype(np.float64)).astype(f32)
+    if m * k * n <= 5_000_000:   # small enough for the oracle's own loop
+        assert_close(oracle.matmul(oracle.roundToBf16(a), oracle.roundToBf16(w)), expected, tol=1e-5, what="oracle vs float64")
+    if with_bias: expected = oracle.addBias(expected, bias)
+    if with_residual: expected = oracle.add(expected, res)
+    assert_close(got, expected, tol=1e-4, what="fused linear")
+
+
+@pytest.mark.parametrize("m,k,n,count", [(50, 40, 24, 3), (300, 136, 256, 3), (4096, 64, 1024, 3), (4100, 256, 256, 3), (260, 72, 512, 2),
+                                         (64, 32, 48, 1)])
+@pytest.mark.parametrize("cached", [False, True])
+def test_bf16_projections_of_a_shared_input(hip, oracle, rng, m, k, n, count, cached):
+    """Q/K/V-style projections of one input and their gradients (ops_transformer.cu:217-257, autodiff.cu:756-798) against
+    the same products computed one by one: widths that fuse into one GEMM with split outputs (multiples of 256), widths
+    that do not, and a token count long enough that the weight-gradient contraction is cut into slices."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a = r(rng, m, k)
+    ws = [r(rng, k, n, scale=0.1) for _ in range(count)]
+    gs = [r(rng, m, n) for _ in range(count)]
+    da, dws, dgs = D.fromHost(a), [D.fromHost(w) for w in ws], [D.fromHost(g) for g in gs]
+    ops.invalidateBf16WeightCache()
+    ar = oracle.roundToBf16(a).astype(np.float64)
+    outs = ops.matmulBf16SharedInput(da, dws, cached=cached)
+    for i in range(count):
+        assert_close(outs[i].toHost(), (ar @ oracle.roundToBf16(ws[i]).astype(np.float64)).astype(f32), tol=1e-4, what=f"product {i}")
+    dA, dBs = ops.matmulBf16SharedInputBackward(da, dws, dgs, cached=cached)
+    eA = sum(oracle.roundToBf16(gs[i]).astype(np.float64) @ oracle.roundToBf16(ws[i]).astype(np.float64).T for i in range(count))
+    assert_close(dA.toHost(), eA.astype(f32), tol=1e-4, what="dA")
+    for i in range(count):
+        eB = ar.T @ oracle.roundToBf16(gs[i]).astype(np.float64)
+        assert_close(dBs[i].toHost(), eB.astype(f32), tol=1e-4, what=f"dB {i}")
+    # agreement with the one-by-one operators (same rounding, different summation split): tight
+    single = ops.matmulBf16(da, dws[0]).toHost()
+    assert_close(outs[0].toHost(), single, tol=1e-5, what="shared-input product vs matmulBf16")
+    # partial requests: only the input gradient, only one weight gradient
+    onlyA, none = ops.matmulBf16SharedInputBackward(da, dws, dgs, cached=cached, want_dB=(False, False, False))
+    assert_bits_equal(onlyA.toHost(), dA.toHost(), "dA must not depend on which weight gradients are requested")
+    _, some = ops.matmulBf16SharedInputBackward(da, dws, dgs, cached=cached, want_dA=False, want_dB=(True,) + (False,) * 2)
+    assert_close(some[0].toHost(), dBs[0].toHost(), tol=1e-5, what="single requested weight gradient")
+
+
 def test_bf16_weight_cache_semantics(hip, oracle, rng):
     """A cached weight image is reused until invalidateBf16WeightCache() (ops_tensorcore.cu:98-131,448)."""
     D, ops = hip.DeviceTensor, hip.ops
