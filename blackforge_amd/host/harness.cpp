@@ -8,6 +8,7 @@
 
 #include "blackforge/backend/hip/loss.hpp"
 #include "blackforge/backend/hip/model.hpp"
+#include "blackforge/backend/hip/train_runner.hpp"
 #include "blackforge/backend/hip/optimizer.hpp"
 
 namespace hip = blackforge::backend::hip;
@@ -180,6 +181,55 @@ int bfh_model_read_loss(void* h, float* sum) {
     return guarded([&] {
         hip::check(bf_hip_memcpy_d2h(sum, handle->lossAccumulator.data(), sizeof(float)));
         hip::check(bf_hip_fill_zero(handle->lossAccumulator.data(), sizeof(float), nullptr));
+    });
+}
+
+// hip::runTraining over a BFDATA1 file (lossKind: 0 mse, 1 cross_entropy, 2 cross_entropy_sparse; optimizerKind: 0 sgd,
+// 1 adamw); epochLosses receives `epochs` values.
+int bfh_model_run_training(void* h, const char* datasetPath, int lossKind, int optimizerKind, long long epochs, size_t batchSize,
+                           double learningRate, int cosineSchedule, const char* fromCheckpoint, const char* saveCheckpoint,
+                           double* epochLosses) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        hip::HostDataset dataset = hip::HostDataset::load(datasetPath);
+        hip::TrainOptions options;
+        options.loss = lossKind == 0 ? "mse" : lossKind == 1 ? "cross_entropy" : "cross_entropy_sparse";
+        options.optimizer = optimizerKind == 0 ? "sgd" : "adamw";
+        options.epochs = epochs;
+        options.batchSize = batchSize;
+        options.learningRate = learningRate;
+        options.cosineSchedule = cosineSchedule != 0;
+        options.fromCheckpointPath = fromCheckpoint ? fromCheckpoint : "";
+        options.saveCheckpointPath = saveCheckpoint ? saveCheckpoint : "";
+        hip::TrainRunResult result = hip::runTraining(*handle->model, dataset, options, nullptr);
+        for (std::size_t i = 0; i < result.epochLosses.size(); ++i) epochLosses[i] = result.epochLosses[i];
+    });
+}
+
+int bfh_model_save_checkpoint(void* h, const char* path) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] { hip::saveCheckpoint(*handle->model, path); });
+}
+
+// Parameter buffers are re-created by the load: callers must fetch bfh_model_param_info again afterwards.
+int bfh_model_load_checkpoint(void* h, const char* path) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        hip::loadCheckpoint(*handle->model, path);
+        handle->params = handle->model->parameters();
+    });
+}
+
+// The permutation HostDataset::shuffle(seed) applies to `numExamples` examples: order[i] = example at position i afterwards.
+int bfh_shuffle_order(size_t numExamples, unsigned seed, size_t* order) {
+    return guarded([&] {
+        std::vector<float> ids(numExamples), zeros(numExamples, 0.0F);
+        for (std::size_t i = 0; i < numExamples; ++i) ids[i] = static_cast<float>(i);
+        hip::HostDataset d({1}, {1}, ids, zeros, numExamples);
+        d.shuffle(seed);
+        if (numExamples == 0) return;
+        auto all = d.batch(0, numExamples);
+        for (std::size_t i = 0; i < numExamples; ++i) order[i] = static_cast<std::size_t>(all.input.data()[i]);
     });
 }
 

@@ -47,6 +47,12 @@ def load() -> ctypes.CDLL:
         lib.bfh_model_train_step.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_size_t),
                                              ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float]
         lib.bfh_model_read_loss.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
+        lib.bfh_model_run_training.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_longlong,
+                                               ctypes.c_size_t, ctypes.c_double, ctypes.c_int, ctypes.c_char_p, ctypes.c_char_p,
+                                               ctypes.POINTER(ctypes.c_double)]
+        lib.bfh_model_save_checkpoint.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
+        lib.bfh_model_load_checkpoint.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
+        lib.bfh_shuffle_order.argtypes = [ctypes.c_size_t, ctypes.c_uint, ctypes.POINTER(ctypes.c_size_t)]
         _lib = lib
     return _lib
 
@@ -125,7 +131,45 @@ class HostModel:
         shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
         _check(load().bfh_model_train_step(self.handle, x.ptr, len(x.shape), shape, target.ptr, loss_kind, optimizer, lr))
 
+    def _refresh_params(self) -> None:
+        """Re-reads names, counts and device pointers of the parameters (a checkpoint load replaces the buffers)."""
+        lib = load()
+        self.names, self.counts, self._value_ptrs, self._grad_ptrs = [], [], [], []
+        for i in range(lib.bfh_model_num_params(self.handle)):
+            buf, cnt = ctypes.create_string_buffer(96), ctypes.c_size_t()
+            val, grd = ctypes.c_void_p(), ctypes.c_void_p()
+            _check(lib.bfh_model_param_info(self.handle, i, buf, 96, ctypes.byref(cnt), ctypes.byref(val), ctypes.byref(grd)))
+            self.names.append(buf.value.decode())
+            self.counts.append(cnt.value)
+            self._value_ptrs.append(val)
+            self._grad_ptrs.append(grd)
+
+    def saveCheckpoint(self, path: str) -> None:
+        """hip::saveCheckpoint: BFCKPT1, the format of the CPU and CUDA backends."""
+        _check(load().bfh_model_save_checkpoint(self.handle, path.encode()))
+
+    def loadCheckpoint(self, path: str) -> None:
+        _check(load().bfh_model_load_checkpoint(self.handle, path.encode()))
+        self._refresh_params()
+
+    def runTraining(self, dataset_path: str, loss: str, optimizer: str, epochs: int, batch_size: int, lr: float = 1e-3,
+                    cosine: bool = False, from_checkpoint: str = "", save_checkpoint: str = ""):
+        """hip::runTraining over a BFDATA1 file; returns the epoch losses."""
+        losses = (ctypes.c_double * max(epochs, 1))()
+        _check(load().bfh_model_run_training(self.handle, dataset_path.encode(), {"mse": 0, "cross_entropy": 1, "cross_entropy_sparse": 2}[loss],
+                                             {"sgd": 0, "adamw": 1}[optimizer], epochs, batch_size, lr, int(cosine),
+                                             from_checkpoint.encode(), save_checkpoint.encode(), losses))
+        self._refresh_params()
+        return list(losses[:epochs])
+
     def readLossSum(self) -> float:
         v = ctypes.c_float()
         _check(load().bfh_model_read_loss(self.handle, ctypes.byref(v)))
         return v.value
+
+
+def shuffleOrder(num_examples: int, seed: int) -> np.ndarray:
+    """The permutation hip::HostDataset::shuffle(seed) applies: result[i] = example that moves to position i."""
+    order = (ctypes.c_size_t * max(num_examples, 1))()
+    _check(load().bfh_shuffle_order(num_examples, seed, order))
+    return np.array(order[:num_examples], dtype=np.int64)

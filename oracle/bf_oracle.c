@@ -19,6 +19,7 @@
 #include "bf_oracle.h"
 
 #include <math.h>
+#include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -743,6 +744,7 @@ int bfo_argmax_last_position(const float* logits, size_t seq, size_t vocab, long
 typedef struct {
     char name[64];
     size_t count;
+    size_t rows, cols; /* shape: [rows, cols], or [rows] when cols == 0 */
     float* value;
     float* grad;
     float* m; /* AdamW moments, allocated on first step */
@@ -769,11 +771,14 @@ struct bfo_model {
     long long adamStep;
 };
 
-static int add_param(bfo_model* model, const char* base, const char* suffix, size_t count) {
+static int add_param(bfo_model* model, const char* base, const char* suffix, size_t rows, size_t cols) {
+    const size_t count = cols ? rows * cols : rows;
     model->params = (bfo_param*)realloc(model->params, (size_t)(model->numParams + 1) * sizeof(bfo_param));
     bfo_param* p = &model->params[model->numParams];
     snprintf(p->name, sizeof(p->name), "%s.%s", base, suffix);
     p->count = count;
+    p->rows = rows;
+    p->cols = cols;
     p->value = calloc_floats(count);
     p->grad = calloc_floats(count);
     p->m = NULL;
@@ -801,20 +806,20 @@ bfo_model* bfo_model_create(int numLayers, const int* kinds, const long long* ar
             case BFO_LINEAR: {
                 size_t outF = (size_t)layer->arg0;
                 snprintf(base, sizeof(base), "linear%d", outputId);
-                layer->params[0] = add_param(model, base, "weight", features * outF);
-                layer->params[1] = add_param(model, base, "bias", outF);
+                layer->params[0] = add_param(model, base, "weight", features, outF);
+                layer->params[1] = add_param(model, base, "bias", outF, 0);
                 features = outF;
                 break;
             }
             case BFO_EMBEDDING: {
                 snprintf(base, sizeof(base), "embedding%d", outputId);
-                layer->params[0] = add_param(model, base, "table", (size_t)layer->arg0 * (size_t)layer->arg1);
+                layer->params[0] = add_param(model, base, "table", (size_t)layer->arg0, (size_t)layer->arg1);
                 features = (size_t)layer->arg1;
                 break;
             }
             case BFO_POSITIONAL: {
                 snprintf(base, sizeof(base), "positional_embedding%d", outputId);
-                layer->params[0] = add_param(model, base, "table", (size_t)layer->arg0 * features);
+                layer->params[0] = add_param(model, base, "table", (size_t)layer->arg0, features);
                 break;
             }
             case BFO_ATTENTION: {
@@ -823,19 +828,19 @@ bfo_model* bfo_model_create(int numLayers, const int* kinds, const long long* ar
                     return NULL;
                 }
                 snprintf(base, sizeof(base), "attention%d", outputId);
-                layer->params[0] = add_param(model, base, "wq", features * features);
-                layer->params[1] = add_param(model, base, "wk", features * features);
-                layer->params[2] = add_param(model, base, "wv", features * features);
-                layer->params[3] = add_param(model, base, "wout", features * features);
+                layer->params[0] = add_param(model, base, "wq", features, features);
+                layer->params[1] = add_param(model, base, "wk", features, features);
+                layer->params[2] = add_param(model, base, "wv", features, features);
+                layer->params[3] = add_param(model, base, "wout", features, features);
                 break;
             }
             case BFO_FEEDFORWARD: {
                 size_t hidden = (size_t)layer->arg0;
                 snprintf(base, sizeof(base), "feedforward%d", outputId);
-                layer->params[0] = add_param(model, base, "w1", features * hidden);
-                layer->params[1] = add_param(model, base, "b1", hidden);
-                layer->params[2] = add_param(model, base, "w2", hidden * features);
-                layer->params[3] = add_param(model, base, "b2", features);
+                layer->params[0] = add_param(model, base, "w1", features, hidden);
+                layer->params[1] = add_param(model, base, "b1", hidden, 0);
+                layer->params[2] = add_param(model, base, "w2", hidden, features);
+                layer->params[3] = add_param(model, base, "b2", features, 0);
                 break;
             }
             default:
@@ -1073,4 +1078,285 @@ int bfo_model_adamw_step(bfo_model* model, float lr, float beta1, float beta2, f
         bfo_adamw_step(p->value, p->grad, p->m, p->v, p->count, model->adamStep, lr, beta1, beta2, eps, weightDecay);
     }
     return BFO_OK;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Training run: dataset file, per-epoch shuffle, learning-rate schedule, checkpoints
+ * ------------------------------------------------------------------------------------------- */
+
+/* std::mt19937 (the 32-bit Mersenne twister of the C++ standard: fixed algorithm and constants). */
+typedef struct {
+    uint32_t state[624];
+    int index;
+} mt19937;
+static void mt_seed(mt19937* g, uint32_t seed) {
+    g->state[0] = seed;
+    for (int i = 1; i < 624; ++i) g->state[i] = 1812433253u * (g->state[i - 1] ^ (g->state[i - 1] >> 30)) + (uint32_t)i;
+    g->index = 624;
+}
+static uint32_t mt_next(mt19937* g) {
+    if (g->index >= 624) {
+        for (int i = 0; i < 624; ++i) {
+            uint32_t y = (g->state[i] & 0x80000000u) | (g->state[(i + 1) % 624] & 0x7fffffffu);
+            g->state[i] = g->state[(i + 397) % 624] ^ (y >> 1) ^ ((y & 1u) ? 0x9908b0dfu : 0u);
+        }
+        g->index = 0;
+    }
+    uint32_t y = g->state[g->index++];
+    y ^= y >> 11;
+    y ^= (y << 7) & 0x9d2c5680u;
+    y ^= (y << 15) & 0xefc60000u;
+    y ^= y >> 18;
+    return y;
+}
+/* std::uniform_int_distribution<size_t>(0, hi) drawing from a 32-bit generator, as libstdc++ (GCC 11 and later)
+ * evaluates it for hi < 2^32 - 1: Lemire's nearly divisionless reduction of one 32-bit draw to [0, hi]. */
+static uint32_t uniform_below_inclusive(mt19937* g, uint32_t hi) {
+    const uint64_t range = (uint64_t)hi + 1u;
+    uint64_t product = (uint64_t)mt_next(g) * range;
+    uint32_t low = (uint32_t)product;
+    if (low < range) {
+        const uint32_t threshold = (uint32_t)((0u - (uint32_t)range) % (uint32_t)range);
+        while (low < threshold) {
+            product = (uint64_t)mt_next(g) * range;
+            low = (uint32_t)product;
+        }
+    }
+    return (uint32_t)(product >> 32);
+}
+
+/* data::Dataset::shuffle (dataset.cpp:102-131): Fisher-Yates from the last position down, generator seeded with
+ * the epoch number; order[i] is the example that moves to position i. */
+int bfo_shuffle_order(size_t numExamples, unsigned seed, size_t* order) {
+    if (numExamples >= 0xffffffffu) return BFO_INVALID_ARGUMENT;
+    for (size_t i = 0; i < numExamples; ++i) order[i] = i;
+    if (numExamples <= 1) return BFO_OK;
+    mt19937 g;
+    mt_seed(&g, seed);
+    for (size_t i = numExamples - 1; i > 0; --i) {
+        size_t j = uniform_below_inclusive(&g, (uint32_t)i);
+        size_t t = order[i];
+        order[i] = order[j];
+        order[j] = t;
+    }
+    return BFO_OK;
+}
+
+/* cosineAnnealingLearningRate (backend/lr_schedule.hpp:...): double arithmetic, rounded to float once. */
+float bfo_cosine_learning_rate(long long epoch, long long totalEpochs, float base) {
+    if (totalEpochs <= 1) return base;
+    const double kPi = 3.14159265358979323846;
+    double progress = (double)(epoch - 1) / (double)(totalEpochs - 1);
+    return (float)(base * 0.5 * (1.0 + cos(kPi * progress)));
+}
+
+typedef struct {
+    uint32_t numExamples;
+    size_t inputRank, targetRank;
+    size_t inputShape[8], targetShape[8];
+    size_t inputSize, targetSize; /* elements per example */
+    float* inputs;
+    float* targets;
+} bfo_dataset;
+
+static int read_shape(FILE* f, size_t* rank, size_t* shape, size_t* product) {
+    uint32_t r = 0;
+    if (fread(&r, 4, 1, f) != 1 || r > 8) return 0;
+    *rank = r;
+    *product = 1;
+    for (uint32_t i = 0; i < r; ++i) {
+        uint64_t d = 0;
+        if (fread(&d, 8, 1, f) != 1) return 0;
+        shape[i] = (size_t)d;
+        *product *= (size_t)d;
+    }
+    return 1;
+}
+/* data::loadDataset (dataset.cpp:154-184): "BFDATA1\0", u32 examples, two shapes (u32 rank + u64 dims), inputs, targets. */
+static int dataset_load(const char* path, bfo_dataset* d) {
+    memset(d, 0, sizeof(*d));
+    FILE* f = fopen(path, "rb");
+    if (!f) return 0;
+    char magic[8];
+    int ok = fread(magic, 1, 8, f) == 8 && memcmp(magic, "BFDATA1\0", 8) == 0 && fread(&d->numExamples, 4, 1, f) == 1 &&
+             read_shape(f, &d->inputRank, d->inputShape, &d->inputSize) && read_shape(f, &d->targetRank, d->targetShape, &d->targetSize);
+    if (ok) {
+        d->inputs = calloc_floats((size_t)d->numExamples * d->inputSize);
+        d->targets = calloc_floats((size_t)d->numExamples * d->targetSize);
+        ok = fread(d->inputs, 4, (size_t)d->numExamples * d->inputSize, f) == (size_t)d->numExamples * d->inputSize &&
+             fread(d->targets, 4, (size_t)d->numExamples * d->targetSize, f) == (size_t)d->numExamples * d->targetSize;
+    }
+    fclose(f);
+    return ok;
+}
+static void dataset_free(bfo_dataset* d) {
+    free(d->inputs);
+    free(d->targets);
+}
+static void dataset_shuffle(bfo_dataset* d, unsigned seed) {
+    const size_t n = d->numExamples;
+    if (n <= 1) return;
+    size_t* order = (size_t*)malloc(n * sizeof(size_t));
+    bfo_shuffle_order(n, seed, order);
+    float* in2 = calloc_floats(n * d->inputSize);
+    float* tg2 = calloc_floats(n * d->targetSize);
+    for (size_t i = 0; i < n; ++i) {
+        memcpy(in2 + i * d->inputSize, d->inputs + order[i] * d->inputSize, d->inputSize * sizeof(float));
+        memcpy(tg2 + i * d->targetSize, d->targets + order[i] * d->targetSize, d->targetSize * sizeof(float));
+    }
+    free(d->inputs);
+    free(d->targets);
+    free(order);
+    d->inputs = in2;
+    d->targets = tg2;
+}
+
+/* saveCheckpoint (cpu/checkpoint.cpp:58-83): "BFCKPT1\0", u32 count, then per parameter u32 name length, name,
+ * u32 rank, u64 dims, fp32 data. */
+int bfo_model_save_checkpoint(const bfo_model* model, const char* path) {
+    FILE* f = fopen(path, "wb");
+    if (!f) return BFO_INVALID_ARGUMENT;
+    fwrite("BFCKPT1\0", 1, 8, f);
+    uint32_t count = (uint32_t)model->numParams;
+    fwrite(&count, 4, 1, f);
+    for (int i = 0; i < model->numParams; ++i) {
+        const bfo_param* p = &model->params[i];
+        uint32_t len = (uint32_t)strlen(p->name), rank = p->cols ? 2u : 1u;
+        uint64_t d0 = p->rows, d1 = p->cols;
+        fwrite(&len, 4, 1, f);
+        fwrite(p->name, 1, len, f);
+        fwrite(&rank, 4, 1, f);
+        fwrite(&d0, 8, 1, f);
+        if (rank == 2) fwrite(&d1, 8, 1, f);
+        fwrite(p->value, 4, p->count, f);
+    }
+    int bad = ferror(f);
+    fclose(f);
+    return bad ? BFO_INVALID_ARGUMENT : BFO_OK;
+}
+/* loadCheckpoint (cpu/checkpoint.cpp:85-135): parameters are matched by name; unknown names, shape mismatches and
+ * truncated files are errors; parameters the file does not mention keep their values. */
+int bfo_model_load_checkpoint(bfo_model* model, const char* path) {
+    FILE* f = fopen(path, "rb");
+    if (!f) return BFO_INVALID_ARGUMENT;
+    char magic[8];
+    uint32_t count = 0;
+    int status = BFO_OK;
+    if (fread(magic, 1, 8, f) != 8 || memcmp(magic, "BFCKPT1\0", 8) != 0 || fread(&count, 4, 1, f) != 1) status = BFO_INVALID_ARGUMENT;
+    for (uint32_t i = 0; i < count && status == BFO_OK; ++i) {
+        uint32_t len = 0, rank = 0;
+        char name[256];
+        uint64_t dims[8] = {0};
+        if (fread(&len, 4, 1, f) != 1 || len >= sizeof(name) || fread(name, 1, len, f) != len || fread(&rank, 4, 1, f) != 1 || rank > 8 ||
+            fread(dims, 8, rank, f) != rank) { status = BFO_INVALID_ARGUMENT; break; }
+        name[len] = 0;
+        bfo_param* p = NULL;
+        for (int j = 0; j < model->numParams; ++j)
+            if (strcmp(model->params[j].name, name) == 0) p = &model->params[j];
+        const uint32_t wantRank = p && p->cols ? 2u : 1u;
+        if (!p || rank != wantRank || dims[0] != p->rows || (rank == 2 && dims[1] != p->cols)) { status = BFO_INVALID_ARGUMENT; break; }
+        if (fread(p->value, 4, p->count, f) != p->count) status = BFO_INVALID_ARGUMENT;
+    }
+    fclose(f);
+    return status;
+}
+
+/* cpu::runTraining (cpu/train_runner.cpp:38-211) for a model built from a layer list: per epoch, shuffle with the
+ * epoch number as seed, optional cosine learning rate, floor(examples / batch) batches of zeroGrad, forward, loss,
+ * backward, optimizer step; the epoch loss is the mean of the batch losses (accumulated in double).
+ * lossKind: 0 mse, 1 cross_entropy, 2 cross_entropy_sparse.  optimizerKind: 0 sgd, 1 adamw (reference defaults).
+ * The model starts from `fromCheckpoint` when that is a non-empty path, else from its current values. */
+int bfo_model_run_training(bfo_model* model, const char* datasetPath, int lossKind, int optimizerKind, long long epochs,
+                           size_t batchSize, float learningRate, int cosineSchedule, const char* fromCheckpoint,
+                           const char* saveCheckpoint, double* epochLosses) {
+    bfo_dataset data;
+    if (!dataset_load(datasetPath, &data)) return BFO_INVALID_ARGUMENT;
+    int status = BFO_OK;
+    if (fromCheckpoint && fromCheckpoint[0]) status = bfo_model_load_checkpoint(model, fromCheckpoint);
+    if (status == BFO_OK && (batchSize == 0 || data.numExamples < batchSize)) status = BFO_INVALID_ARGUMENT;
+    if (status != BFO_OK) { dataset_free(&data); return status; }
+    const size_t batches = data.numExamples / batchSize;
+    float* input = calloc_floats(batchSize * data.inputSize);
+    float* target = calloc_floats(batchSize * data.targetSize);
+    size_t shape[9];
+    shape[0] = batchSize;
+    for (size_t i = 0; i < data.inputRank; ++i) shape[i + 1] = data.inputShape[i];
+    size_t outCapacity = 0;
+    float* out = NULL;
+    float* grad = NULL;
+    float lr = learningRate;
+    for (long long epoch = 1; epoch <= epochs && status == BFO_OK; ++epoch) {
+        dataset_shuffle(&data, (unsigned)epoch);
+        if (cosineSchedule) lr = bfo_cosine_learning_rate(epoch, epochs, learningRate);
+        double sum = 0.0;
+        for (size_t b = 0; b < batches && status == BFO_OK; ++b) {
+            for (size_t i = 0; i < batchSize; ++i) {
+                size_t e = (b * batchSize + i) % data.numExamples;
+                memcpy(input + i * data.inputSize, data.inputs + e * data.inputSize, data.inputSize * sizeof(float));
+                memcpy(target + i * data.targetSize, data.targets + e * data.targetSize, data.targetSize * sizeof(float));
+            }
+            bfo_model_zero_grad(model);
+            size_t outCount = 0;
+            status = bfo_model_forward(model, input, (int)data.inputRank + 1, shape, out, outCapacity, &outCount);
+            if (status != BFO_OK && outCount > outCapacity) {   /* first batch: size the output buffers and run again */
+                free(out);
+                free(grad);
+                outCapacity = outCount;
+                out = calloc_floats(outCapacity);
+                grad = calloc_floats(outCapacity);
+                status = bfo_model_forward(model, input, (int)data.inputRank + 1, shape, out, outCapacity, &outCount);
+            }
+            if (status != BFO_OK) break;
+            const size_t classes = model->layers[model->numLayers - 1].outFeatures, rows = outCount / classes;
+            float value = 0.0f;
+            if (lossKind == 0) status = bfo_mean_squared_error(out, target, grad, &value, outCount);
+            else if (lossKind == 1) status = bfo_softmax_cross_entropy(out, target, grad, &value, rows, classes);
+            else status = bfo_softmax_cross_entropy_sparse(out, target, grad, &value, rows, classes);
+            if (status != BFO_OK) break;
+            status = bfo_model_backward(model, grad, outCount);
+            if (status != BFO_OK) break;
+            if (optimizerKind == 0) {
+                for (int i = 0; i < model->numParams; ++i) bfo_sgd_step(model->params[i].value, model->params[i].grad, model->params[i].count, lr);
+            } else {
+                bfo_model_adamw_step(model, lr, 0.9f, 0.999f, 1e-8f, 0.01f);
+            }
+            sum += value;
+        }
+        epochLosses[epoch - 1] = sum / (double)batches;
+    }
+    if (status == BFO_OK && saveCheckpoint && saveCheckpoint[0]) status = bfo_model_save_checkpoint(model, saveCheckpoint);
+    free(input); free(target); free(out); free(grad);
+    dataset_free(&data);
+    return status;
+}
+
+int bfo_model_write_initial_checkpoint(bfo_model* model, const char* path) {
+    (void)model;
+    (void)path;
+    return BFO_INVALID_ARGUMENT; /* the reference's std:: random streams are not restated */
+}
+
+int bfo_save_dataset(const char* path, int inputRank, const size_t* inputShape, int targetRank, const size_t* targetShape,
+                     const float* inputs, const float* targets, size_t numExamples) {
+    FILE* f = fopen(path, "wb");
+    if (!f) return BFO_INVALID_ARGUMENT;
+    fwrite("BFDATA1\0", 1, 8, f);
+    uint32_t n = (uint32_t)numExamples;
+    fwrite(&n, 4, 1, f);
+    size_t inSize = 1, tgSize = 1;
+    for (int pass = 0; pass < 2; ++pass) {
+        uint32_t rank = (uint32_t)(pass == 0 ? inputRank : targetRank);
+        const size_t* shape = pass == 0 ? inputShape : targetShape;
+        fwrite(&rank, 4, 1, f);
+        for (uint32_t i = 0; i < rank; ++i) {
+            uint64_t d = shape[i];
+            fwrite(&d, 8, 1, f);
+            if (pass == 0) inSize *= shape[i]; else tgSize *= shape[i];
+        }
+    }
+    fwrite(inputs, 4, numExamples * inSize, f);
+    fwrite(targets, 4, numExamples * tgSize, f);
+    int bad = ferror(f);
+    fclose(f);
+    return bad ? BFO_INVALID_ARGUMENT : BFO_OK;
 }

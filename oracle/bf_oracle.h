@@ -145,6 +145,29 @@ int bfo_model_zero_grad(bfo_model* model);
 /* One AdamW step over parameters() with per-model moment state (optimizer.cpp:18-46). */
 int bfo_model_adamw_step(bfo_model* model, float lr, float beta1, float beta2, float eps, float weightDecay);
 
+
+/* ---- training run (cpu/train_runner.cpp, data/dataset.cpp, cpu/checkpoint.cpp, backend/lr_schedule.hpp) ---- */
+/* The permutation of data::Dataset::shuffle(seed) (dataset.cpp:102-131): order[i] = example that moves to position i. */
+int bfo_shuffle_order(size_t numExamples, unsigned seed, size_t* order);
+/* cosineAnnealingLearningRate (lr_schedule.hpp:7-15). */
+float bfo_cosine_learning_rate(long long epoch, long long totalEpochs, float base);
+/* saveCheckpoint / loadCheckpoint in the BFCKPT1 format (cpu/checkpoint.cpp:58-135). */
+int bfo_model_save_checkpoint(const bfo_model* model, const char* path);
+int bfo_model_load_checkpoint(bfo_model* model, const char* path);
+/* cpu::runTraining (train_runner.cpp:38-211) over a BFDATA1 dataset file (dataset.cpp:133-184).  lossKind: 0 mse,
+ * 1 cross_entropy, 2 cross_entropy_sparse; optimizerKind: 0 sgd, 1 adamw; cosineSchedule: 0/1.  The run starts from
+ * `fromCheckpoint` (required: the reference's random initialisation is not restated) and writes `saveCheckpoint`
+ * when that is a non-empty path.  epochLosses receives `epochs` values. */
+int bfo_model_run_training(bfo_model* model, const char* datasetPath, int lossKind, int optimizerKind, long long epochs,
+                           size_t batchSize, float learningRate, int cosineSchedule, const char* fromCheckpoint,
+                           const char* saveCheckpoint, double* epochLosses);
+/* Reference build only (returns BFO_INVALID_ARGUMENT in the restatement): writes the checkpoint of a model of this
+ * layer list as cpu::Model(modelIR, seed 42) initialises it (model.cpp, random_init.cpp), for use as `fromCheckpoint`. */
+int bfo_model_write_initial_checkpoint(bfo_model* model, const char* path);
+/* data::saveDataset (dataset.cpp:133-152). */
+int bfo_save_dataset(const char* path, int inputRank, const size_t* inputShape, int targetRank, const size_t* targetShape,
+                     const float* inputs, const float* targets, size_t numExamples);
+
 #ifdef __cplusplus
 }
 #endif

@@ -49,6 +49,7 @@ class Oracle:
         self.lib.bfo_model_create.restype = ctypes.c_void_p
         self.lib.bfo_model_param_value.restype = _f32p
         self.lib.bfo_model_param_grad.restype = _f32p
+        self.lib.bfo_cosine_learning_rate.restype = ctypes.c_float
         self.is_reference = bool(self.lib.bfo_is_reference())
 
     # -- plumbing ---------------------------------------------------------------------------
@@ -351,6 +352,25 @@ class Oracle:
         self._call("bfo_argmax_last_position", logits, seq, vocab, ctypes.byref(idx))
         return idx.value
 
+    def shuffleOrder(self, num_examples: int, seed: int) -> np.ndarray:
+        """The permutation data::Dataset::shuffle(seed) applies: result[i] = example that moves to position i."""
+        order = (_sz * max(num_examples, 1))()
+        if self.lib.bfo_shuffle_order(_sz(num_examples), ctypes.c_uint(seed), order) != 0:
+            raise OracleInvalidArgument("shuffle_order")
+        return np.array(order[:num_examples], dtype=np.int64)
+
+    def cosineAnnealingLearningRate(self, epoch: int, total_epochs: int, base: float) -> float:
+        return float(self.lib.bfo_cosine_learning_rate(ctypes.c_longlong(epoch), ctypes.c_longlong(total_epochs), ctypes.c_float(base)))
+
+    def saveDataset(self, path: str, inputs, targets) -> None:
+        """inputs: [examples, *inputShape], targets: [examples, *targetShape] (data::saveDataset, BFDATA1)."""
+        inputs, targets = _f(inputs), _f(targets)
+        ins, tgs = inputs.shape[1:], targets.shape[1:]
+        st = self.lib.bfo_save_dataset(path.encode(), len(ins), (_sz * max(len(ins), 1))(*ins), len(tgs), (_sz * max(len(tgs), 1))(*tgs),
+                                       _p(inputs), _p(targets), _sz(inputs.shape[0]))
+        if st != 0:
+            raise OracleInvalidArgument("save_dataset")
+
     def model(self, layers, input_features=0):
         return OracleModel(self, layers, input_features)
 
@@ -419,6 +439,33 @@ class OracleModel:
         f = ctypes.c_float
         if self.o.lib.bfo_model_adamw_step(self.handle, f(lr), f(beta1), f(beta2), f(eps), f(wd)) != 0:
             raise OracleInvalidArgument("model_adamw_step")
+
+
+    def saveCheckpoint(self, path: str) -> None:
+        if self.o.lib.bfo_model_save_checkpoint(self.handle, path.encode()) != 0:
+            raise OracleInvalidArgument("save_checkpoint")
+
+    def loadCheckpoint(self, path: str) -> None:
+        if self.o.lib.bfo_model_load_checkpoint(self.handle, path.encode()) != 0:
+            raise OracleInvalidArgument("load_checkpoint")
+
+    def writeInitialCheckpoint(self, path: str) -> None:
+        """Reference build only: the checkpoint of this model as cpu::Model(modelIR, seed 42) initialises it."""
+        if self.o.lib.bfo_model_write_initial_checkpoint(self.handle, path.encode()) != 0:
+            raise OracleInvalidArgument("write_initial_checkpoint")
+
+    def runTraining(self, dataset_path, loss, optimizer, epochs, batch_size, lr=1e-3, cosine=False, from_checkpoint="",
+                    save_checkpoint=""):
+        """cpu::runTraining.  loss: 'mse' | 'cross_entropy' | 'cross_entropy_sparse'; optimizer: 'sgd' | 'adamw'.
+        Returns the list of epoch losses; the trained values are left in this model."""
+        losses = (ctypes.c_double * max(epochs, 1))()
+        st = self.o.lib.bfo_model_run_training(self.handle, dataset_path.encode(), {"mse": 0, "cross_entropy": 1, "cross_entropy_sparse": 2}[loss],
+                                               {"sgd": 0, "adamw": 1}[optimizer], ctypes.c_longlong(epochs), _sz(batch_size),
+                                               ctypes.c_float(lr), int(bool(cosine)), from_checkpoint.encode(), save_checkpoint.encode(),
+                                               losses)
+        if st != 0:
+            raise OracleInvalidArgument("run_training")
+        return list(losses[:epochs])
 
 
 _cache = {}

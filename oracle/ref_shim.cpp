@@ -20,7 +20,12 @@
 #include <string>
 #include <vector>
 
+#include "blackforge/ast/ast.hpp"
 #include "blackforge/backend/cpu/autodiff.hpp"
+#include "blackforge/backend/cpu/checkpoint.hpp"
+#include "blackforge/backend/cpu/train_runner.hpp"
+#include "blackforge/backend/lr_schedule.hpp"
+#include "blackforge/data/dataset.hpp"
 #include "blackforge/backend/cpu/loss.hpp"
 #include "blackforge/backend/cpu/model.hpp"
 #include "blackforge/backend/cpu/ops.hpp"
@@ -502,6 +507,103 @@ int bfo_model_adamw_step(bfo_model* model, float lr, float beta1, float beta2, f
         model->adamw->setLearningRate(lr);
         model->adamw->step(model->model->parameters());
     });
+}
+
+
+// ---- training run: the reference's own runTraining, dataset, checkpoint and schedule functions ----------------
+int bfo_shuffle_order(size_t numExamples, unsigned seed, size_t* order) {
+    return guarded([&] {
+        // a dataset whose example i holds the number i: after shuffle(seed), position i holds order[i]
+        std::vector<float> ids(numExamples), zeros(numExamples, 0.0F);
+        for (std::size_t i = 0; i < numExamples; ++i) ids[i] = static_cast<float>(i);
+        if (numExamples >= (std::size_t(1) << 24)) throw std::invalid_argument("too many examples for float indices");
+        blackforge::data::Dataset d({1}, {1}, ids, zeros, numExamples);
+        d.shuffle(seed);
+        if (numExamples == 0) return;
+        auto all = d.batch(0, numExamples);
+        for (std::size_t i = 0; i < numExamples; ++i) order[i] = static_cast<std::size_t>(all.input.data()[i]);
+    });
+}
+
+float bfo_cosine_learning_rate(long long epoch, long long totalEpochs, float base) {
+    return blackforge::backend::cosineAnnealingLearningRate(epoch, totalEpochs, base);
+}
+
+int bfo_model_save_checkpoint(const bfo_model* model, const char* path) {
+    try {
+        cpu::saveCheckpoint(*model->model, path);
+        return BFO_OK;
+    } catch (const std::exception&) {
+        return BFO_INVALID_ARGUMENT;
+    }
+}
+int bfo_model_load_checkpoint(bfo_model* model, const char* path) {
+    try {
+        cpu::loadCheckpoint(*model->model, path);
+        return BFO_OK;
+    } catch (const std::exception&) {
+        return BFO_INVALID_ARGUMENT;
+    }
+}
+int bfo_model_write_initial_checkpoint(bfo_model* model, const char* path) {
+    try {
+        cpu::Model fresh(model->irModel, 42U);
+        cpu::saveCheckpoint(fresh, path);
+        return BFO_OK;
+    } catch (const std::exception&) {
+        return BFO_INVALID_ARGUMENT;
+    }
+}
+int bfo_save_dataset(const char* path, int inputRank, const size_t* inputShape, int targetRank, const size_t* targetShape,
+                     const float* inputs, const float* targets, size_t numExamples) {
+    try {
+        std::vector<std::size_t> inS(inputShape, inputShape + inputRank), tgS(targetShape, targetShape + targetRank);
+        std::size_t inN = numExamples, tgN = numExamples;
+        for (std::size_t d : inS) inN *= d;
+        for (std::size_t d : tgS) tgN *= d;
+        blackforge::data::saveDataset(path, inS, tgS, std::vector<float>(inputs, inputs + inN), std::vector<float>(targets, targets + tgN),
+                                      numExamples);
+        return BFO_OK;
+    } catch (const std::exception&) {
+        return BFO_INVALID_ARGUMENT;
+    }
+}
+
+// The real cpu::runTraining, driven by a hand-built program: one dataset declaration (path) and one train block.
+// It constructs its own cpu::Model from the IR (seed 42) and loads `fromCheckpoint` over it; the trained weights
+// come back through `saveCheckpoint`, which is then loaded into this handle's model.
+int bfo_model_run_training(bfo_model* model, const char* datasetPath, int lossKind, int optimizerKind, long long epochs,
+                           size_t batchSize, float learningRate, int cosineSchedule, const char* fromCheckpoint,
+                           const char* saveCheckpoint, double* epochLosses) {
+    namespace ast = blackforge::ast;
+    try {
+        if (!saveCheckpoint || !saveCheckpoint[0]) return BFO_INVALID_ARGUMENT;
+        ast::Program program;
+        ast::DatasetDecl dataset;
+        dataset.name = "data";
+        dataset.fields.push_back(ast::DatasetPathField{datasetPath, {}});
+        program.declarations.push_back(dataset);
+        ast::TrainDecl train;
+        train.fields.push_back(ast::TrainModelField{model->irModel.name, {}});
+        train.fields.push_back(ast::TrainDatasetField{"data", {}});
+        const char* lossNames[3] = {"mse", "cross_entropy", "cross_entropy_sparse"};
+        if (lossKind < 0 || lossKind > 2) return BFO_INVALID_ARGUMENT;
+        train.fields.push_back(ast::TrainLossField{lossNames[lossKind], {}});
+        train.fields.push_back(ast::TrainOptimizerField{optimizerKind == 0 ? "sgd" : "adamw", {}});
+        train.fields.push_back(ast::TrainEpochsField{epochs, {}});
+        train.fields.push_back(ast::TrainBatchSizeField{static_cast<long long>(batchSize), {}});
+        train.fields.push_back(ast::TrainLearningRateField{static_cast<double>(learningRate), {}});
+        if (cosineSchedule) train.fields.push_back(ast::TrainLrScheduleField{"cosine", {}});
+        program.declarations.push_back(train);
+        ir::Module module;
+        module.models.push_back(model->irModel);
+        cpu::TrainRunResult result = cpu::runTraining(program, module, fromCheckpoint ? fromCheckpoint : "", saveCheckpoint, nullptr);
+        for (std::size_t i = 0; i < result.epochLosses.size(); ++i) epochLosses[i] = result.epochLosses[i];
+        cpu::loadCheckpoint(*model->model, saveCheckpoint);
+        return BFO_OK;
+    } catch (const std::exception&) {
+        return BFO_INVALID_ARGUMENT;
+    }
 }
 
 }  // extern "C"
