@@ -534,8 +534,11 @@ __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const floa
     }
 }
 
-template <int HDP, int BQ, bool VEC4>
-__global__ void __launch_bounds__(256) attnBackwardDkvKernel(AttnParams p) {
+// OCC = wavefronts per SIMD the register allocation is held to.  At OCC 2 (head dims up to 64) two workgroups share
+// a CU and cover each other's barriers and tile hand-overs, at the price of a handful of spilled registers; it pays
+// once the grid has more workgroups than two per CU, below that one roomier workgroup per CU is faster.
+template <int HDP, int BQ, bool VEC4, int OCC>
+__global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) {
     constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BQ * LDSW;
     extern __shared__ float smem[];
     float* qs = smem;                   // [2][BQ][LDSW]
@@ -663,8 +666,12 @@ int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
         return vec4 ? launchAttn(attnBackwardDqKernel<HDP, TILE, true>, smem, grid, p, s)
                     : launchAttn(attnBackwardDqKernel<HDP, TILE, false>, smem, grid, p, s);
     } else {
-        return vec4 ? launchAttn(attnBackwardDkvKernel<HDP, TILE, true>, smem, grid, p, s)
-                    : launchAttn(attnBackwardDkvKernel<HDP, TILE, false>, smem, grid, p, s);
+        if (HDP <= 64 && grid > 2u * unsigned(computeUnits())) {
+            return vec4 ? launchAttn(attnBackwardDkvKernel<HDP, TILE, true, (HDP <= 64 ? 2 : 1)>, smem, grid, p, s)
+                        : launchAttn(attnBackwardDkvKernel<HDP, TILE, false, (HDP <= 64 ? 2 : 1)>, smem, grid, p, s);
+        }
+        return vec4 ? launchAttn(attnBackwardDkvKernel<HDP, TILE, true, 1>, smem, grid, p, s)
+                    : launchAttn(attnBackwardDkvKernel<HDP, TILE, false, 1>, smem, grid, p, s);
     }
 }
 
