@@ -196,10 +196,18 @@ __device__ __forceinline__ void storeTransposed(float* __restrict__ dst, const f
 // MFMAs of sub-block sb+1 are issued BEFORE the softmax arithmetic of sub-block sb in program order, and do
 // not depend on it, so exp/max/rescale run in the shadow of those MFMAs.  MASKED = false is the interior
 // of the causal triangle (every key of the tile visible to every row of the wave).
+//
+// Lazy rescaling: exponentials are taken relative to a reference maximum `mref` that only moves when the running row
+// maximum `mrow` has grown past it by more than kRescaleThreshold (in log2 units), so probabilities stay below 2^8 and
+// the accumulator/row-sum rescale -- 32+ multiplies that sit between two groups of dependent MFMAs -- runs only in
+// the tiles where some row of the wavefront needs it (a wave-uniform branch; for typical scores that is the first
+// tile only).  The result is the same sum taken about a different reference point; the true maximum is tracked
+// separately for the statistics the backward pass reads.
+constexpr float kRescaleThreshold = 8.0f;
 template <int HDP, int BC, bool MASKED>
 __device__ __forceinline__ void forwardTile(const float* __restrict__ ks, const float* __restrict__ vs,
-                                            const float (&qreg)[HDP / 2], float16v (&acc)[HDP / 32], float& mrow, float& lrow,
-                                            int kt0, int myLimit, int totalLen, int half, int li) {
+                                            const float (&qreg)[HDP / 2], float16v (&acc)[HDP / 32], float& mrow, float& mref,
+                                            float& lrow, int kt0, int myLimit, int totalLen, int half, int li) {
     constexpr int LDSW = HDP + 4, DT = HDP / 32, NSB = BC / 32;
     float16v s[NSB];
 #pragma unroll
@@ -224,17 +232,21 @@ __device__ __forceinline__ void forwardTile(const float* __restrict__ ks, const 
 #pragma unroll
         for (int r = 4; r < 16; r += 4) mx = fmaxf(mx, fmaxf(fmaxf(sc[r], sc[r + 1]), fmaxf(sc[r + 2], sc[r + 3])));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float mnew = fmaxf(mrow, mx);
-        const float corr = fastExp2(mrow - mnew);
+        mrow = fmaxf(mrow, mx);
+        const bool moveRef = mrow > mref + kRescaleThreshold;   // also true on the first visible key (mref = -inf)
+        if (__builtin_amdgcn_ballot_w64(moveRef) != 0) {
+            const float corr = moveRef ? fastExp2(mref - mrow) : 1.0f;   // 0 when the reference was still -inf
+            mref = moveRef ? mrow : mref;
+            lrow *= corr;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+        }
         float psum = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { sc[r] = fastExp2(sc[r] - mnew); psum += sc[r]; }
-        lrow = lrow * corr + psum;
-        mrow = mnew;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+        for (int r = 0; r < 16; ++r) { sc[r] = fastExp2(sc[r] - mref); psum += sc[r]; }
+        lrow += psum;
         // O^T += V^T * P^T : step r contracts over key dRow(r, half)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -277,7 +289,7 @@ __global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
-    float mrow = -INFINITY, lrow = 0.0f;
+    float mrow = -INFINITY, mref = -INFINITY, lrow = 0.0f;
 
     const int lastQuery = min(p.newLen, qt * 128 + 128) - 1;
     const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);   // keys >= this are invisible to the tile
@@ -302,8 +314,8 @@ __global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
         if (kt0 < waveKeyEnd) {   // wave-uniform: the tile holds keys some row of this wave can see
             // interior of the causal triangle: every key visible to every row of the wave, no masking arithmetic
             const bool masked = (kt0 + BC - 1 > p.oldLen + waveQ0) || (kt0 + BC > p.totalLen);
-            if (masked) forwardTile<HDP, BC, true>(kcur, vcur, qreg, acc, mrow, lrow, kt0, myLimit, p.totalLen, half, li);
-            else forwardTile<HDP, BC, false>(kcur, vcur, qreg, acc, mrow, lrow, kt0, myLimit, p.totalLen, half, li);
+            if (masked) forwardTile<HDP, BC, true>(kcur, vcur, qreg, acc, mrow, mref, lrow, kt0, myLimit, p.totalLen, half, li);
+            else forwardTile<HDP, BC, false>(kcur, vcur, qreg, acc, mrow, mref, lrow, kt0, myLimit, p.totalLen, half, li);
         }
         if (t + 1 < numKeyTiles) {
             commitHeadTile<HDP, BC>(ks + ((t + 1) & 1) * TILE, kNext, tid);
@@ -320,9 +332,10 @@ __global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
     if (rowValid) {
         storeTransposed<HDP, VEC4>(p.out + (size_t(b) * p.newLen + i) * dim + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
         if (half == 0) {
+            // statistics about the TRUE row maximum: l = sum exp(score - m) = (sum about mref) * 2^(mref - mrow)
             size_t idx = (size_t(b) * p.heads + h) * p.newLen + i;
             p.m[idx] = mrow * kLn2;
-            p.l[idx] = lrow;
+            p.l[idx] = lrow * fastExp2(mref - mrow);
         }
     }
 }

@@ -52,6 +52,28 @@ def test_attention_core_matches_the_oracle(hip, oracle, rng, batch, heads, new_l
         assert_close(got, exp, what=f"{name} case {(batch, heads, new_len, old_len, hd)}", scale=sc[name])
 
 
+@pytest.mark.parametrize("new_len,hd,growth,qscale", [(300, 64, 0.25, 1.0), (200, 32, 0.6, 1.0), (513, 128, 0.1, 0.3), (260, 64, -0.3, 1.0)])
+def test_attention_with_drifting_row_maximum(hip, oracle, rng, new_len, hd, growth, qscale):
+    """Scores that keep growing (or shrinking) along the key axis: the running row maximum passes the forward kernel's
+    reference maximum by more than its rescale threshold many times (growth > 0) or never after the first key
+    (growth < 0), and the saved statistics m, l must still be those of the TRUE maximum."""
+    heads, dim = 2, 2 * hd
+    t = np.arange(new_len, dtype=f32) / 8.0
+    ramp = (1.0 + growth * t if growth > 0 else 1.0 / (1.0 - growth * t))[None, :, None]   # key scale: growing, or decaying
+    q = (np.abs(r(rng, 1, new_len, dim)) + 0.5) * f32(qscale)                    # qscale keeps the largest logits near 50
+    k = (np.abs(r(rng, 1, new_len, dim)) + 0.5) * ramp.astype(f32)               # q.k > 0 and following the ramp
+    v, go = r(rng, 1, new_len, dim), r(rng, 1, new_len, dim)
+    scale = float(f32(1.0) / np.sqrt(f32(hd)))
+    o, m, l, dq, dk, dv = run_gpu(hip, q, k, v, go, heads, scale, 0)
+    eo, em, el = oracle.attentionCoreForward(q, k, v, heads, scale, 0)
+    edq, edk, edv = oracle.attentionCoreBackward(go, q, k, v, heads, scale, 0)
+    if growth > 0:
+        assert float(em.max() - em[..., 0].min()) > 8 * np.log(2.0) * 5, "the case must cross the threshold several times"
+    sc = grad_scales(q, k, v, go, scale)
+    for got, exp, name in ((o, eo, "O"), (m, em, "m"), (l, el, "l"), (dq, edq, "dQ"), (dk, edk, "dK"), (dv, edv, "dV")):
+        assert_close(got, exp, what=f"{name} drifting maximum {(new_len, hd, growth)}", scale=sc[name])
+
+
 def test_attention_golden_fixtures(hip):
     """Inputs and outputs written by the real reference build (tests/golden/make_golden.py)."""
     gold = np.load(GOLDEN)
