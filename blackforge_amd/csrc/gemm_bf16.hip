@@ -25,6 +25,7 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned short ushort8 __attribute__((ext_vector_type(8)));
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ unsigned short toBf16Bits(float x) {
     __bf16 h = static_cast<__bf16>(x);   // round to nearest even, NaN preserved
@@ -58,11 +59,15 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict_
 // out[c, 0..rowsPad) = bf16(x[0..rows, c]), zero padded: 64 x 64 tiles through LDS.  With `vec` (x 16-byte
 // aligned, cols a multiple of 4, rowsPad a multiple of 8) a thread reads four consecutive columns of a row as
 // one 16-byte load and writes eight consecutive rows of an output row as one 16-byte store, so both sides move
-// whole 128-byte lines; otherwise elements go one by one.
+// whole 128-byte lines; otherwise elements go one by one.  When `plain` is not NULL the same pass also writes
+// the untransposed image plain[r*ldPlain + 0..pad8(cols)) = bf16(x[r, :]), zero padded: a gradient that feeds
+// both the input-gradient GEMM (plain) and the weight-gradient GEMM (transposed) is read from HBM once.
 __global__ void __launch_bounds__(kBlock) convertTransposeKernel(const float* __restrict__ x, unsigned short* __restrict__ out,
-                                                                 size_t rows, size_t cols, size_t rowsPad, int vec) {
+                                                                 size_t rows, size_t cols, size_t rowsPad, int vec,
+                                                                 unsigned short* __restrict__ plain, size_t ldPlain) {
     __shared__ __attribute__((aligned(16))) unsigned short tile[64][72];   // [column][row], 144-byte pitch
     const size_t r0 = size_t(blockIdx.y) * 64, c0 = size_t(blockIdx.x) * 64;
+    const size_t colsPad = (cols + 7) / 8 * 8;
     if (vec) {
         const int cg = threadIdx.x & 15, rr = threadIdx.x >> 4;   // 16 column groups x 16 rows per pass
 #pragma unroll
@@ -71,10 +76,15 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(const float* __
             const size_t gr = r0 + r, gc = c0 + 4 * cg;
             float4v v = {0.0f, 0.0f, 0.0f, 0.0f};
             if (gr < rows && gc < cols) v = loadf4(x + gr * cols + gc);   // cols % 4 == 0: all four in range
-            tile[4 * cg + 0][r] = toBf16Bits(v.x);
-            tile[4 * cg + 1][r] = toBf16Bits(v.y);
-            tile[4 * cg + 2][r] = toBf16Bits(v.z);
-            tile[4 * cg + 3][r] = toBf16Bits(v.w);
+            const unsigned short b0 = toBf16Bits(v.x), b1 = toBf16Bits(v.y), b2 = toBf16Bits(v.z), b3 = toBf16Bits(v.w);
+            tile[4 * cg + 0][r] = b0;
+            tile[4 * cg + 1][r] = b1;
+            tile[4 * cg + 2][r] = b2;
+            tile[4 * cg + 3][r] = b3;
+            if (plain && gr < rows && gc < colsPad) {   // ldPlain % 8 == 0 and gc % 4 == 0: an aligned 8-byte store
+                uint2v packed = {unsigned(b0) | (unsigned(b1) << 16), unsigned(b2) | (unsigned(b3) << 16)};
+                *reinterpret_cast<uint2v*>(plain + gr * ldPlain + gc) = packed;
+            }
         }
         __syncthreads();
         const int chunk = threadIdx.x & 7, cc = threadIdx.x >> 3;   // 8 chunks of 8 rows x 32 columns per pass
@@ -92,7 +102,9 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(const float* __
     for (int i = 0; i < 16; ++i) {
         int r = ty + 4 * i;
         size_t gr = r0 + r, gc = c0 + tx;
-        tile[tx][r] = (gr < rows && gc < cols) ? toBf16Bits(x[gr * cols + gc]) : (unsigned short)0;
+        const unsigned short b = (gr < rows && gc < cols) ? toBf16Bits(x[gr * cols + gc]) : (unsigned short)0;
+        tile[tx][r] = b;
+        if (plain && gr < rows && gc < colsPad) plain[gr * ldPlain + gc] = b;
     }
     __syncthreads();
 #pragma unroll
@@ -524,13 +536,17 @@ int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, 
     return BF_OK;
 }
 
-int convertTransposed(const float* x, unsigned short* out, size_t rows, size_t cols, hipStream_t s, bool padRows = true) {
+// plain / ldPlain: optional second output, the untransposed image with row stride ldPlain (a multiple of 8).
+int convertTransposed(const float* x, unsigned short* out, size_t rows, size_t cols, hipStream_t s, bool padRows = true,
+                      unsigned short* plain = nullptr, size_t ldPlain = 0) {
     if (rows == 0 || cols == 0) return BF_OK;
     size_t rowsPad = padRows ? pad8(rows) : rows;   // length of an output row
-    dim3 grid(unsigned((cols + 63) / 64), unsigned((rowsPad + 63) / 64));
+    // the grid covers pad8(cols) columns so that the plain image's zero padding is written too
+    dim3 grid(unsigned(((plain ? pad8(cols) : cols) + 63) / 64), unsigned((rowsPad + 63) / 64));
     if (grid.y > 65535) return failInvalid("cvt_f32_bf16_transpose", "too many rows");
-    const int vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && cols % 4 == 0 && rowsPad % 8 == 0;
-    convertTransposeKernel<<<grid, kBlock, 0, s>>>(x, out, rows, cols, rowsPad, vec);
+    const int vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(plain)) & 15u) == 0 &&
+                    cols % 4 == 0 && rowsPad % 8 == 0 && ldPlain % 8 == 0;
+    convertTransposeKernel<<<grid, kBlock, 0, s>>>(x, out, rows, cols, rowsPad, vec, plain, ldPlain);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -674,11 +690,16 @@ int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, 
     }
     BF_REQUIRE(a && b && g, "NULL operand");
     int st = BF_OK;
+    const size_t mp = pad8(m);
+    Scratch gT(dB ? n * mp * sizeof(unsigned short) : 0);
+    if (gT.status != BF_OK) return gT.status;
     if (dA) {   // dA[m,k] = g[m,n] * b[k,n]^T : contraction over n
         const size_t np = pad8(n);
         Scratch gImg(m * np * sizeof(unsigned short));
         if (gImg.status != BF_OK) return gImg.status;
-        st = convertPlain(g, gImg.as<unsigned short>(), m, n, s);
+        // with both gradients wanted, one pass over g writes the plain image for this product and the transposed one for dB
+        if (dB) st = convertTransposed(g, gT.as<unsigned short>(), m, n, s, true, gImg.as<unsigned short>(), np);
+        else st = convertPlain(g, gImg.as<unsigned short>(), m, n, s);
         if (st != BF_OK) return st;
         unsigned short* bImg = nullptr;
         size_t bBytes = 0;
@@ -689,14 +710,11 @@ int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, 
         if (st != BF_OK) return st;
     }
     if (dB) {   // dB[k,n] = a[m,k]^T * g[m,n] : contraction over m
-        const size_t mp = pad8(m);
         Scratch aT(k * mp * sizeof(unsigned short));
-        Scratch gT(n * mp * sizeof(unsigned short));
         if (aT.status != BF_OK) return aT.status;
-        if (gT.status != BF_OK) return gT.status;
         st = convertTransposed(a, aT.as<unsigned short>(), m, k, s);
         if (st != BF_OK) return st;
-        st = convertTransposed(g, gT.as<unsigned short>(), m, n, s);
+        if (!dA) st = convertTransposed(g, gT.as<unsigned short>(), m, n, s);
         if (st != BF_OK) return st;
         st = launchGemmNt(aT.as<unsigned short>(), gT.as<unsigned short>(), dB, k, n, mp, mp, mp, s);
     }
@@ -787,6 +805,12 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
     BF_REQUIRE(a != nullptr, "NULL operand");
     for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] && g[i], "NULL operand");
     int st = BF_OK;
+    bool anyDb = false;
+    for (size_t i = 0; dB && i < count; ++i) anyDb = anyDb || dB[i] != nullptr;
+    const size_t mp = pad8(m);
+    Scratch gT(anyDb ? count * n * mp * sizeof(unsigned short) : 0);   // transposed gradient images, stacked
+    if (gT.status != BF_OK) return gT.status;
+    bool transposedDone[3] = {false, false, false};
     if (dA) {
         if (count > 1 && n % 8 == 0) {
             // dA = sum_i g_i b_i^T = [g_0 | g_1 | g_2] [b_0 | b_1 | b_2]^T: one GEMM whose contraction runs over all of them
@@ -794,7 +818,12 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
             Scratch gImg(m * nn * sizeof(unsigned short));
             if (gImg.status != BF_OK) return gImg.status;
             for (size_t i = 0; i < count; ++i) {
-                st = convertPlain(g[i], gImg.as<unsigned short>() + i * n, m, n, s, nn);
+                if (dB && dB[i]) {   // one pass over g_i writes its column slice of the plain image and its transposed image
+                    st = convertTransposed(g[i], gT.as<unsigned short>() + i * n * mp, m, n, s, true, gImg.as<unsigned short>() + i * n, nn);
+                    transposedDone[i] = true;
+                } else {
+                    st = convertPlain(g[i], gImg.as<unsigned short>() + i * n, m, n, s, nn);
+                }
                 if (st != BF_OK) return st;
             }
             unsigned short* wImg = nullptr;
@@ -816,20 +845,15 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
             }
         }
     }
-    bool anyDb = false;
-    for (size_t i = 0; dB && i < count; ++i) anyDb = anyDb || dB[i] != nullptr;
     if (anyDb) {
-        const size_t mp = pad8(m);
         Scratch aT(k * mp * sizeof(unsigned short));
         if (aT.status != BF_OK) return aT.status;
         st = convertTransposed(a, aT.as<unsigned short>(), m, k, s);
         if (st != BF_OK) return st;
         bool all = true;
         for (size_t i = 0; i < count; ++i) all = all && dB[i] != nullptr;
-        Scratch gT(count * n * mp * sizeof(unsigned short));
-        if (gT.status != BF_OK) return gT.status;
         for (size_t i = 0; i < count; ++i) {
-            if (!dB[i]) continue;
+            if (!dB[i] || transposedDone[i]) continue;
             st = convertTransposed(g[i], gT.as<unsigned short>() + i * n * mp, m, n, s);
             if (st != BF_OK) return st;
         }
