@@ -230,7 +230,7 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
         return BF_OK;
     }
     bool vec = aligned16(src) && (!FUSED || (aligned16(bias) && aligned16(dHidden) && aligned16(dGemm)));
-    RowGeom g = rowGeometry(rows, features, vec, 128, 4);
+    RowGeom g = rowGeometry(rows, features, vec, 256, 4);
     size_t parts = g.grid.y;
     Scratch scratch(dBias ? parts * features * sizeof(float) : 0);
     if (scratch.status != BF_OK) return scratch.status;
