@@ -652,9 +652,8 @@ int paddedHeadDim(int hd) { return hd <= 32 ? 32 : hd <= 64 ? 64 : hd <= 128 ? 1
 
 template <typename K>
 int launchAttn(K kernel, size_t smemBytes, unsigned grid, const AttnParams& p, hipStream_t s) {
-    if (smemBytes > 48 * 1024)
-        BF_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       int(smemBytes)));
+    int st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smemBytes);
+    if (st != BF_OK) return st;
     kernel<<<grid, 256, smemBytes, s>>>(p);
     BF_LAUNCH_CHECK();
     return BF_OK;

@@ -47,6 +47,10 @@ inline unsigned gridFor(size_t work, size_t perBlock, unsigned cap = kMaxGridX) 
 // Number of compute units of the current device (cached); used to size persistent grids.
 int computeUnits();
 
+// Raises a kernel's dynamic shared-memory limit to `bytes` on the current device (needed above 48 KiB).  The
+// setting is per (kernel, device) and sticks, so it is made once and remembered.
+int allowDynamicSharedMemory(const void* kernel, size_t bytes);
+
 // Scratch memory from the per-device pool, returned on scope exit.  The release only puts the block
 // back on the pool's free list; kernels already enqueued on a stream keep using it safely because
 // every later user of the block is enqueued behind them on the same stream or is ordered by the

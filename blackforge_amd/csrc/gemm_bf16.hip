@@ -441,9 +441,7 @@ __global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restr
 
 template <typename Kernel>
 int allowSharedMemory(Kernel kernel, size_t smem) {
-    if (smem > 48 * 1024)
-        BF_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-    return BF_OK;
+    return allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
 }
 
 int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,

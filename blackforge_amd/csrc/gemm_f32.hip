@@ -11,10 +11,47 @@
 //   D: lane l, register r holds D[i = 8*(r/4) + 4*(l/32) + r%4][j = l % 32]
 #include "common.hpp"
 
+#include <algorithm>
+
 namespace bf {
 namespace {
 
-constexpr int BK = 16;
+constexpr int BK = 32;
+
+// One thread's share of a [BK x BT] operand tile: element e = tid + 256*i of the tile, walked so that consecutive
+// threads read consecutive global addresses (along k when the tile dimension t is a row of X, along t otherwise).
+template <int BT>
+struct TileRegs {
+    static constexpr int kPer = BK * BT / 256;
+    float v[kPer];
+};
+
+// Issues the global loads of the tile of op(X) at (k0, t0) into registers, zero outside the matrix or the K slice.
+// op(X)[k][t] = X[t*ld + k] when t is the row of X (T_IS_ROW), or X[k*ld + t] when t is its column.
+template <int BT, bool T_IS_ROW>
+__device__ __forceinline__ void fetchTile(TileRegs<BT>& regs, const float* __restrict__ X, size_t ld, size_t tExtent,
+                                          size_t kEnd, size_t t0, size_t k0, int tid) {
+#pragma unroll
+    for (int i = 0; i < TileRegs<BT>::kPer; ++i) {
+        const int e = tid + 256 * i;
+        int k, t;
+        if constexpr (T_IS_ROW) { k = e % BK; t = e / BK; }
+        else { t = e % BT; k = e / BT; }
+        const size_t gt = t0 + t, gk = k0 + k;
+        regs.v[i] = (gt < tExtent && gk < kEnd) ? (T_IS_ROW ? X[gt * ld + gk] : X[gk * ld + gt]) : 0.0f;
+    }
+}
+template <int BT, bool T_IS_ROW>
+__device__ __forceinline__ void commitTile(float (*lds)[BT + 4], const TileRegs<BT>& regs, int tid) {
+#pragma unroll
+    for (int i = 0; i < TileRegs<BT>::kPer; ++i) {
+        const int e = tid + 256 * i;
+        int k, t;
+        if constexpr (T_IS_ROW) { k = e % BK; t = e / BK; }
+        else { t = e % BT; k = e / BT; }
+        lds[k][t] = regs.v[i];
+    }
+}
 
 template <int BM, int BN>
 struct GemmTile {
@@ -23,30 +60,15 @@ struct GemmTile {
     float bs[BK][BN + kPad];
 };
 
-// Copies the [BK x BT] tile of op(X) starting at (k0, t0) into lds[k][t], zero-filling outside the
-// matrix.  op(X)[k][t] = X[t*ld + k] when the tile dimension t is the row of X (contiguous along k),
-// or X[k*ld + t] when t is the column of X (contiguous along t).
-template <int BT, bool T_IS_ROW>
-__device__ __forceinline__ void loadTile(float (*lds)[BT + 4], const float* __restrict__ X, size_t ld, size_t tExtent,
-                                         size_t kExtent, size_t t0, size_t k0, int tid) {
-    constexpr int kElems = BK * BT;
-#pragma unroll
-    for (int e = tid; e < kElems; e += 256) {
-        int k, t;
-        if constexpr (T_IS_ROW) { k = e % BK; t = e / BK; }   // consecutive threads walk k (contiguous)
-        else { t = e % BT; k = e / BT; }                       // consecutive threads walk t (contiguous)
-        size_t gt = t0 + t, gk = k0 + k;
-        float v = 0.0f;
-        if (gt < tExtent && gk < kExtent) v = T_IS_ROW ? X[gt * ld + gk] : X[gk * ld + gt];
-        lds[k][t] = v;
-    }
-}
-
 // TRANS_A: A stored [K,M] (op(A)[m][k] = A[k*M + m]); otherwise A stored [M,K].
 // TRANS_B: B stored [N,K] (op(B)[k][n] = B[n*K + k]); otherwise B stored [K,N].
+// blockIdx.z selects a slice [z*kPerSlice, (z+1)*kPerSlice) of the contraction; slice z writes its partial product
+// to C + z*sliceStride.  The global loads of the next K step are in flight (in registers) while the current one is
+// multiplied out of LDS.
 template <int BM, int BN, bool TRANS_A, bool TRANS_B>
 __global__ void __launch_bounds__(256) gemmF32Kernel(const float* __restrict__ A, const float* __restrict__ B,
-                                                      float* __restrict__ C, size_t M, size_t N, size_t K) {
+                                                      float* __restrict__ C, size_t M, size_t N, size_t K, size_t kPerSlice,
+                                                      size_t sliceStride) {
     constexpr int WM = BM / 2, WN = BN / 2;      // 2 x 2 wavefronts
     constexpr int TM = WM / 32, TN = WN / 32;    // 32x32 MFMA tiles per wavefront
     __shared__ GemmTile<BM, BN> tile;
@@ -55,6 +77,8 @@ __global__ void __launch_bounds__(256) gemmF32Kernel(const float* __restrict__ A
     const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
     const size_t m0 = size_t(blockIdx.y) * BM, n0 = size_t(blockIdx.x) * BN;
     const int li = lane & 31, lk = lane >> 5;
+    const size_t kBegin = size_t(blockIdx.z) * kPerSlice, kEnd = kBegin + kPerSlice < K ? kBegin + kPerSlice : K;
+    C += size_t(blockIdx.z) * sliceStride;
 
     float16v acc[TM][TN];
 #pragma unroll
@@ -64,14 +88,22 @@ __global__ void __launch_bounds__(256) gemmF32Kernel(const float* __restrict__ A
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    for (size_t k0 = 0; k0 < K; k0 += BK) {
+    TileRegs<BM> aNext;
+    TileRegs<BN> bNext;
+    auto fetch = [&](size_t k0) {
         // A tile: tile dimension m.  A stored [M,K] -> m is the row (contiguous along k).
-        if constexpr (TRANS_A) loadTile<BM, false>(tile.as, A, M, M, K, m0, k0, tid);
-        else loadTile<BM, true>(tile.as, A, K, M, K, m0, k0, tid);
+        if constexpr (TRANS_A) fetchTile<BM, false>(aNext, A, M, M, kEnd, m0, k0, tid);
+        else fetchTile<BM, true>(aNext, A, K, M, kEnd, m0, k0, tid);
         // B tile: tile dimension n.  B stored [K,N] -> n is the column (contiguous along n).
-        if constexpr (TRANS_B) loadTile<BN, true>(tile.bs, B, K, N, K, n0, k0, tid);
-        else loadTile<BN, false>(tile.bs, B, N, N, K, n0, k0, tid);
+        if constexpr (TRANS_B) fetchTile<BN, true>(bNext, B, K, N, kEnd, n0, k0, tid);
+        else fetchTile<BN, false>(bNext, B, N, N, kEnd, n0, k0, tid);
+    };
+    if (kBegin < kEnd) fetch(kBegin);
+    for (size_t k0 = kBegin; k0 < kEnd; k0 += BK) {
+        commitTile<BM, !TRANS_A>(tile.as, aNext, tid);
+        commitTile<BN, TRANS_B>(tile.bs, bNext, tid);
         __syncthreads();
+        if (k0 + BK < kEnd) fetch(k0 + BK);
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
             float a[TM], b[TN];
@@ -101,14 +133,24 @@ __global__ void __launch_bounds__(256) gemmF32Kernel(const float* __restrict__ A
         }
 }
 
+// C[i] = sum over slices of partial[s*stride + i], slices added in index order (deterministic).
+__global__ void __launch_bounds__(kBlock) sliceSumKernel(const float* __restrict__ partial, float* __restrict__ C, size_t count,
+                                                         size_t stride, int slices) {
+    const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float sum = partial[i];
+    for (int s = 1; s < slices; ++s) sum += partial[size_t(s) * stride + i];
+    C[i] = sum;
+}
+
 template <int BM, int BN>
-int launchGemm(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K,
-               hipStream_t s) {
-    dim3 grid(unsigned((N + BN - 1) / BN), unsigned((M + BM - 1) / BM));
-    if (!transA && !transB) gemmF32Kernel<BM, BN, false, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K);
-    else if (!transA && transB) gemmF32Kernel<BM, BN, false, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K);
-    else if (transA && !transB) gemmF32Kernel<BM, BN, true, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K);
-    else gemmF32Kernel<BM, BN, true, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K);
+int launchGemm(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t slices,
+               size_t kPerSlice, size_t sliceStride, hipStream_t s) {
+    dim3 grid(unsigned((N + BN - 1) / BN), unsigned((M + BM - 1) / BM), unsigned(slices));
+    if (!transA && !transB) gemmF32Kernel<BM, BN, false, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else if (!transA && transB) gemmF32Kernel<BM, BN, false, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else if (transA && !transB) gemmF32Kernel<BM, BN, true, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else gemmF32Kernel<BM, BN, true, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -126,8 +168,27 @@ extern "C" int bf_hip_gemm_f32(int transA, int transB, const float* A, const flo
     BF_REQUIRE(A && B, "NULL operand");
     BF_REQUIRE((M + 63) / 64 <= 65535, "M too large");
     // Large tiles once they alone can fill the chip twice over; small tiles otherwise.
+    hipStream_t s = asStream(stream);
+    const size_t cus = size_t(computeUnits());
     size_t bigTiles = ((M + 127) / 128) * ((N + 127) / 128);
-    if (bigTiles >= size_t(2) * size_t(computeUnits()))
-        return launchGemm<128, 128>(transA, transB, A, B, C, M, N, K, asStream(stream));
-    return launchGemm<64, 64>(transA, transB, A, B, C, M, N, K, asStream(stream));
+    if (bigTiles >= 2 * cus) return launchGemm<128, 128>(transA, transB, A, B, C, M, N, K, 1, K, 0, s);
+    // Few tiles and a long contraction (the weight gradients of a small model: a [features x features] product
+    // over all tokens): cut K into slices so that more workgroups share it; a second kernel adds the slices in
+    // order.
+    const size_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+    size_t slices = 1;
+    if (tiles < cus && K >= 4 * BK) slices = std::min<size_t>(std::min<size_t>(16, cus / tiles), K / (2 * BK));
+    if (slices > 1) {
+        const size_t steps = (K + BK - 1) / BK, kPer = (steps + slices - 1) / slices * BK;
+        slices = (K + kPer - 1) / kPer;
+        const size_t count = M * N;
+        Scratch partial(slices * count * sizeof(float));
+        if (partial.status != BF_OK) return partial.status;
+        int st = launchGemm<64, 64>(transA, transB, A, B, partial.as<float>(), M, N, K, slices, kPer, count, s);
+        if (st != BF_OK) return st;
+        sliceSumKernel<<<gridFor(count, kBlock), kBlock, 0, s>>>(partial.as<float>(), C, count, count, int(slices));
+        BF_LAUNCH_CHECK();
+        return BF_OK;
+    }
+    return launchGemm<64, 64>(transA, transB, A, B, C, M, N, K, 1, K, 0, s);
 }

@@ -56,6 +56,18 @@ std::map<std::pair<int, int>, DescriptorTable>& descriptorTables() {
 }
 }  // namespace
 
+int allowDynamicSharedMemory(const void* kernel, size_t bytes) {
+    if (bytes <= 48 * 1024) return BF_OK;
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    static std::map<std::pair<const void*, int>, size_t> granted;
+    size_t& have = granted[{kernel, dev}];
+    if (have >= bytes) return BF_OK;
+    BF_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes)));
+    have = bytes;
+    return BF_OK;
+}
+
 int uploadDescriptorTable(int slot, const void* hostBytes, size_t bytes, hipStream_t stream, const void** devicePtr) {
     int dev = 0;
     BF_HIP_TRY(hipGetDevice(&dev));
