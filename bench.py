@@ -238,6 +238,39 @@ TRAIN_CONFIGS = {
 }
 
 
+MLP_CONFIG = dict(rows=4096, width=4096, what="BASELINE.json configs[1]: MLP [4096 tokens, 4096] -> linear(4096) -> silu -> "
+                  "linear(4096), bf16 projections with fp32 accumulation, forward + backward against an MSE loss")
+
+
+def bench_mlp(bf, steps, warmup):
+    """The README MLP: forward, MSE loss and backward through the C++ operator layer's Model (no optimizer step)."""
+    from blackforge_amd import hostlayer as hl
+    rows, width = MLP_CONFIG["rows"], MLP_CONFIG["width"]
+    model = hl.HostModel([(hl.LINEAR, width), (hl.SILU,), (hl.LINEAR, width)], input_features=width, use_bf16=True)
+    rng = np.random.default_rng(42)
+    for i, count in enumerate(model.counts):
+        bias = model.names[i].endswith(".bias")
+        model.set_value(i, np.zeros(count, np.float32) if bias else rng.standard_normal(count, dtype=np.float32) * np.float32(1 / 64))
+    x = bf.DeviceTensor.fromHost(rng.standard_normal((rows, width), dtype=np.float32))
+    y = bf.DeviceTensor.fromHost(rng.standard_normal((rows, width), dtype=np.float32))
+    step = lambda: model.trainStep(x, y, hl.LOSS_MSE, 0, 0.0)
+    for _ in range(warmup):
+        step()
+    bf.capi.call("bf_hip_synchronize")
+    model.readLossSum()
+    start, stop = bf.Event(), bf.Event()
+    start.record(None)
+    for _ in range(steps):
+        step()
+    stop.record(None)
+    stop.synchronize()
+    ms = start.elapsed_ms(stop) / steps
+    flops = 6 * 2 * rows * width * width
+    return {"workload": MLP_CONFIG["what"], "tokens_per_s": round(rows / (ms * 1e-3), 1), "ms_per_step": round(ms, 3), "tokens": rows,
+            "algorithmic_tflop_per_step": round(flops / 1e12, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
+            "mean_loss": round(model.readLossSum() / (steps * rows * width), 4)}
+
+
 def train_step_flops(c):
     """Algorithmic FLOPs of one step: 6*tokens*(matmul weights) + 14*hd*P per attention layer."""
     tokens = c["batch"] * c["seq"]
@@ -295,7 +328,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 256 MiB copy (bf_hip_scale by 1.0) so that a counter run of this command "
                          "holds a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
-    ap.add_argument("--train", default="gpt_small", help="comma list of train-step workloads to add (tiny_lm, gpt_small, "
+    ap.add_argument("--train", default="gpt_small", help="comma list of train-step workloads to add (tiny_lm, mlp, gpt_small, "
                     "long_context) or 'none'")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -348,7 +381,8 @@ def main():
         "device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units},
     }
     if args.train != "none":
-        line["train_step"] = {name: bench_train_step(bf, name, max(3, args.steps // 2), max(1, args.warmup // 2))
+        line["train_step"] = {name: (bench_mlp if name == "mlp" else lambda b, s_, w_: bench_train_step(b, name, s_, w_))(
+                                  bf, max(3, args.steps // 2), max(1, args.warmup // 2))
                               for name in args.train.split(",")}
     if args.extras:
         line["extras"] = bench_extras(bf, max(5, args.steps // 2))
