@@ -110,8 +110,14 @@ public:
     }
 
     void backward(const DeviceTensor& outputGrad, bool inputRangeTrusted = false) {
-        DeviceTensor grad = outputGrad.clone();
-        for (std::size_t li = layers_.size(); li-- > 0;) grad = applyBackward(layers_[li], grad, inputRangeTrusted && li == 0);
+        // the caller's gradient is only read: no copy of it (the logits gradient of a language model is the largest
+        // tensor of the step)
+        const DeviceTensor* grad = &outputGrad;
+        DeviceTensor owned;
+        for (std::size_t li = layers_.size(); li-- > 0;) {
+            owned = applyBackward(layers_[li], *grad, inputRangeTrusted && li == 0);
+            grad = &owned;
+        }
     }
 
     void zeroGrad() {
