@@ -263,7 +263,7 @@ __device__ __forceinline__ void forwardTile(const float* __restrict__ ks, const 
 //   issues the global loads of tile t+2; the barrier at the end of the iteration both publishes tile t+1
 //   and guarantees every wave is done reading buffer t&1 before iteration t+1 overwrites it with tile t+2.
 template <int HDP, int BC, bool VEC4>
-__global__ void __launch_bounds__(256) attnForwardKernel(AttnParams p) {
+__global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnForwardKernel(AttnParams p) {
     constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BC * LDSW;
     extern __shared__ float smem[];
     float* ks = smem;               // [2][BC][LDSW]
@@ -421,7 +421,7 @@ __device__ __forceinline__ void dqTile(const float* __restrict__ ks, const float
 }
 
 template <int HDP, int BC, bool VEC4>
-__global__ void __launch_bounds__(256) attnBackwardDqKernel(AttnParams p) {
+__global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnBackwardDqKernel(AttnParams p) {
     constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BC * LDSW;
     extern __shared__ float smem[];
     float* ks = smem;
