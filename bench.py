@@ -11,7 +11,7 @@ i.i.d. N(0,1) from a fixed seed, scale 1/sqrt(64).  One "step" = forward O plus 
 Prints ONE JSON line.  `value` = algorithmic FLOPs of a step (14*hd*P with P = B*H*S(S+1)/2 causal
 pairs: 4*hd*P forward, 10*hd*P backward, the FlashAttention convention; exp/softmax not counted)
 divided by the measured time per step.  `roofline` describes the dominant kernel (the key-tile-owner
-backward kernel that produces dK and dV), timed live with HIP events on the stream the kernels run on.
+backward kernel that produces dK and dV and leaves dS in HBM for the dQ kernel), timed live with HIP events on the stream the kernels run on.
 `cpu_baseline` times the CPU reference on a bounded sample of the same workload on this host.
 Everything on one GPU: this build has no multi-GPU path.
 """
@@ -41,7 +41,9 @@ MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvKernel": 901435591}
 
 def attention_flops(batch, heads, seq, hd):
     pairs = batch * heads * seq * (seq + 1) // 2
-    return {"fwd": 4 * hd * pairs, "bwd": 10 * hd * pairs, "dkv": 8 * hd * pairs, "dq": 6 * hd * pairs, "pairs": pairs}
+    # dkv: S, dP, dV, dK; dq: dS*K alone when dS is handed over, S and dP again when it is recomputed
+    return {"fwd": 4 * hd * pairs, "bwd": 10 * hd * pairs, "dkv": 8 * hd * pairs, "dq": 2 * hd * pairs,
+            "dq_recompute": 6 * hd * pairs, "pairs": pairs}
 
 
 def time_region(bf, stream, fn, steps, warmup):
@@ -77,9 +79,17 @@ def bench_attention(bf, steps, warmup):
                        dv.ptr, *dims)
     prep = lambda: call("bf_hip_attention_backward_prepare", out.ptr, go.ptr, m.ptr, l.ptr, lse2.ptr, dvec.ptr, batch,
                         heads, seq, dim, sh)
-    dkv = lambda: call("bf_hip_attention_backward_dkv", go.ptr, q.ptr, k.ptr, v.ptr, lse2.ptr, dvec.ptr, dk.ptr, dv.ptr,
-                       *dims)
-    dqk = lambda: call("bf_hip_attention_backward_dq", go.ptr, q.ptr, k.ptr, v.ptr, lse2.ptr, dvec.ptr, dq.ptr, *dims)
+    # the two kernels bf_hip_attention_backward launches after prepare: dK/dV leaving dS behind, dQ from that dS
+    ds_bytes = ctypes.c_size_t(0)
+    call("bf_hip_attention_ds_bytes", batch, heads, seq, seq, ctypes.byref(ds_bytes))
+    ds = D((ds_bytes.value // 4,))
+    dkv = lambda: call("bf_hip_attention_backward_dkv_ds", go.ptr, q.ptr, k.ptr, v.ptr, lse2.ptr, dvec.ptr, dk.ptr, dv.ptr,
+                       ds.ptr, *dims)
+    dqk = lambda: call("bf_hip_attention_backward_dq_from_ds", ds.ptr, k.ptr, dq.ptr, *dims)
+    # the route taken when the dS buffer does not fit: both kernels recompute S and dP
+    dkv_re = lambda: call("bf_hip_attention_backward_dkv", go.ptr, q.ptr, k.ptr, v.ptr, lse2.ptr, dvec.ptr, dk.ptr, dv.ptr,
+                          *dims)
+    dq_re = lambda: call("bf_hip_attention_backward_dq", go.ptr, q.ptr, k.ptr, v.ptr, lse2.ptr, dvec.ptr, dq.ptr, *dims)
 
     def step():
         fwd()
@@ -103,7 +113,8 @@ def bench_attention(bf, steps, warmup):
 
     # per-kernel durations, live, same stream
     per = {name: time_region(bf, stream, fn, steps, 1) for name, fn in
-           (("forward", fwd), ("prepare", prep), ("dkv", dkv), ("dq", dqk))}
+           (("forward", fwd), ("prepare", prep), ("dkv", dkv), ("dq", dqk), ("dkv_recompute", dkv_re),
+            ("dq_recompute", dq_re))}
     fl = attention_flops(batch, heads, seq, hd)
     return {"ms_per_step": ms_step, "wall_ms_per_step": wall_ms, "kernel_ms": per, "flops": fl,
             "shape": {"batch": batch, "heads": heads, "seq": seq, "head_dim": hd}}
@@ -367,7 +378,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "causal fused attention fwd+bwd, fp32, batch 8, heads 16, seq 2048, head_dim 64 "
                                "(BASELINE.json configs[2])", **res["shape"]},
-        "roofline": {"bound": "mfma", "kernel": "attnBackwardDkvKernel<64,64> (dK,dV; key-tile owner)",
+        "roofline": {"bound": "mfma", "kernel": "attnBackwardDkvKernel<64,64,..,store dS> (dK, dV and the dS hand-over; key-tile owner)",
                      "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES["attnBackwardDkvKernel"],
@@ -376,7 +387,9 @@ def main():
         "kernel_ms": {k: round(v, 4) for k, v in res["kernel_ms"].items()},
         "kernel_tflops": {"forward": round(fl["fwd"] / res["kernel_ms"]["forward"] / 1e9, 2),
                           "dkv": round(fl["dkv"] / res["kernel_ms"]["dkv"] / 1e9, 2),
-                          "dq": round(fl["dq"] / res["kernel_ms"]["dq"] / 1e9, 2)},
+                          "dq": round(fl["dq"] / res["kernel_ms"]["dq"] / 1e9, 2),
+                          "dkv_recompute": round(fl["dkv"] / res["kernel_ms"]["dkv_recompute"] / 1e9, 2),
+                          "dq_recompute": round(fl["dq_recompute"] / res["kernel_ms"]["dq_recompute"] / 1e9, 2)},
         "wall_ms_per_step": round(res["wall_ms_per_step"], 4),
         "device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units},
     }

@@ -99,6 +99,10 @@ SIGNATURES = {
     "bf_hip_attention_backward_prepare": [P, P, P, P, P, P, c_size, c_size, c_size, c_size, S],
     "bf_hip_attention_backward_dkv": [P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_attention_backward_dq": [P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
+    "bf_hip_attention_ds_bytes": [c_size, c_size, c_size, c_size, ctypes.POINTER(c_size)],
+    "bf_hip_attention_set_workspace_limit": [c_size],
+    "bf_hip_attention_backward_dkv_ds": [P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
+    "bf_hip_attention_backward_dq_from_ds": [P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_mse": [P, P, P, P, c_size, c_int, S],
     "bf_hip_cross_entropy": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse": [P, P, P, P, c_size, c_size, c_int, S],

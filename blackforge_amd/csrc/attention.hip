@@ -27,7 +27,9 @@
 // newLen/totalLen/oldLen are accepted (tiles are zero-filled and masked).
 #include "common.hpp"
 
+#include <atomic>
 #include <cmath>
+#include <cstdint>
 
 namespace bf {
 namespace {
@@ -41,6 +43,8 @@ struct AttnParams {
     const float* dvec;   // [batch, heads, newLen]: dot(O, dO)
     float* out; float* m; float* l;
     float* dQ; float* dK; float* dV;
+    float* ds;           // [batch*heads, nqb, nkb, 32 queries, 32 keys]: dS sub-blocks handed from dK/dV to dQ (or null)
+    int nqb, nkb;        // query / key sub-blocks of 32 per (batch, head)
     int batch, heads, newLen, totalLen, dim, hd, oldLen;
     float scale;
     int numTiles;        // query tiles (forward, dQ) or key tiles (dK/dV) per (batch, head)
@@ -491,15 +495,121 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnBackwardDqKernel(A
 }
 
 // ---------------------------------------------------------------------------------------------
+// backward, part 1b: dQ from stored dS.  When the dK/dV kernel has left its dS sub-blocks in HBM, dQ = dS * K is a
+// single contraction: a wave streams its 32 queries' row of sub-blocks (contiguous, 4 KiB each) into registers one
+// tile ahead, while the K tiles go through LDS as in the kernels above.  Neither S nor dP is recomputed, so the
+// backward pass executes the five products of the algorithm instead of seven.
+// A sub-block is read exactly when its first key is visible to its last query; the dK/dV kernel writes all of those.
+// ---------------------------------------------------------------------------------------------
+constexpr int kDsPatch = 32 * 36;   // floats of LDS per staged dS sub-block
+
+template <int HDP, int BC, bool VEC4>
+__global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnBackwardDqFromDsKernel(AttnParams p) {
+    constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BC * LDSW, NSB = BC / 32;
+    extern __shared__ float smem[];
+    float* ks = smem;   // [2][BC][LDSW]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, qt;
+    decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const size_t qOff = size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+
+    const int waveQ0 = qt * 128 + wave * 32;
+    const int i = waveQ0 + li;
+    // keys below waveKeyEnd are visible to some query of this wave's sub-block row (none if the row is past newLen)
+    const int waveKeyEnd = waveQ0 < p.newLen ? min(p.totalLen, p.oldLen + waveQ0 + 32) : 0;
+    // A sub-block is fetched as it lies in memory (lane l takes bytes 16*l of each KiB: whole cache lines per 8 lanes)
+    // and turned into B-operand layout (lane (li, half), registers 4g..4g+3 = dS[query li][keys 8g + 4*half ..+3])
+    // through a wave-private LDS patch with rows padded to 36 floats; no barrier is involved, a wave's LDS
+    // operations execute in order.
+    const float* dsWave = p.ds + ((size_t(bh) * p.nqb + size_t(waveQ0 >> 5)) * p.nkb) * 1024 + lane * 4;
+    float* stage = smem + 2 * TILE + wave * (NSB * kDsPatch);
+
+    float16v acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
+
+    const int lastQuery = min(p.newLen, qt * 128 + 128) - 1;
+    const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);
+    const int numKeyTiles = (blockKeyEnd + BC - 1) / BC;
+
+    float4v dsNext[NSB][4];
+    auto fetchDs = [&](int kt0) {
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb) {
+            const int k0 = kt0 + sb * 32;
+            if (k0 < waveKeyEnd) {
+                const float* src = dsWave + size_t(k0 >> 5) * 1024;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) dsNext[sb][j] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(src + j * 256));
+            }
+        }
+    };
+
+    TileRegs<HDP, BC> kNext;
+    fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, 0, p.totalLen, hd, tid);
+    fetchDs(0);
+    commitHeadTile<HDP, BC>(ks, kNext, tid);
+    if (numKeyTiles > 1) fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, BC, p.totalLen, hd, tid);
+    __syncthreads();
+    for (int t = 0; t < numKeyTiles; ++t) {
+        const int kt0 = t * BC;
+        const float* kcur = ks + (t & 1) * TILE;
+        float16v ds[NSB];
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb) {
+            if (kt0 + sb * 32 < waveKeyEnd) {
+                float* patch = stage + sb * kDsPatch;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) storef4(patch + (8 * j + (lane >> 3)) * 36 + (lane & 7) * 4, dsNext[sb][j]);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float4v val = loadf4(patch + li * 36 + (2 * g + half) * 4);
+                    ds[sb][4 * g] = val.x; ds[sb][4 * g + 1] = val.y; ds[sb][4 * g + 2] = val.z; ds[sb][4 * g + 3] = val.w;
+                }
+            }
+        }
+        if (t + 1 < numKeyTiles) fetchDs(kt0 + BC);
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb) {
+            if (kt0 + sb * 32 < waveKeyEnd) {
+                // dQ^T += K^T * dS^T : step r contracts over key dRow(r, half)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float* krow = kcur + (sb * 32 + dRow(r, half)) * LDSW + li;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+                        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[dt * 32], ds[sb][r], acc[dt], 0, 0, 0);
+                }
+            }
+        }
+        if (t + 1 < numKeyTiles) {
+            commitHeadTile<HDP, BC>(ks + ((t + 1) & 1) * TILE, kNext, tid);
+            if (t + 2 < numKeyTiles) fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, kt0 + 2 * BC, p.totalLen, hd, tid);
+        }
+        __syncthreads();
+    }
+    if (i < p.newLen) storeTransposed<HDP, VEC4>(p.dQ + qOff + size_t(i) * dim, acc, hd, half, p.scale);
+}
+
+// ---------------------------------------------------------------------------------------------
 // backward, part 2: dK, dV (key-tile owner).  K and V of the wave's 32 keys stay in registers as MFMA
 // B operands; Q/dO tiles and the per-row statistics are streamed through LDS.
 // ---------------------------------------------------------------------------------------------
 // One Q/dO tile (BQ queries) for one wavefront, straight-line and software-pipelined.
 // stats: [0..BQ) = lse2 of the tile's queries (+inf for padding rows), [BQ..2BQ) = D.
-template <int HDP, int BQ, bool MASKED>
+// STORE: also writes each dS sub-block (32 queries x 32 keys, row-major) to dsLane + sb*dsStride for the dQ kernel
+// that contracts it with K; dsLane already points at this lane's column and first row (li + 128*half floats in).
+template <int HDP, int BQ, bool MASKED, bool STORE>
 __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const float* __restrict__ gs, const float* __restrict__ stats,
                                         const float (&kreg)[HDP / 2], const float (&vreg)[HDP / 2], float16v (&dk)[HDP / 32],
-                                        float16v (&dv)[HDP / 32], int qt0, int key, bool keyValid, int oldLen, int half, int li) {
+                                        float16v (&dv)[HDP / 32], int qt0, int key, bool keyValid, int oldLen, int half, int li,
+                                        float* __restrict__ dsLane, size_t dsStride, int newLen) {
     constexpr int LDSW = HDP + 4, DT = HDP / 32, NSB = BQ / 32;
     float16v s[NSB], dp[NSB];
 #pragma unroll
@@ -533,6 +643,13 @@ __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const floa
                 dsv[r] = prob * (dsv[r] - d4[c]);      // dS (without the scale factor)
             }
         }
+        if constexpr (STORE) {
+            if (qt0 + sb * 32 < newLen) {   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave
+                float* dst = dsLane + sb * dsStride;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(dsv[r], dst + (8 * (r >> 2) + (r & 3)) * 32);
+            }
+        }
         // dV += P^T * dO, dK += dS^T * Q : step r contracts over query dRow(r, half)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -550,7 +667,7 @@ __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const floa
 // OCC = wavefronts per SIMD the register allocation is held to.  At OCC 2 (head dims up to 64) two workgroups share
 // a CU and cover each other's barriers and tile hand-overs, at the price of a handful of spilled registers; it pays
 // once the grid has more workgroups than two per CU, below that one roomier workgroup per CU is faster.
-template <int HDP, int BQ, bool VEC4, int OCC>
+template <int HDP, int BQ, bool VEC4, int OCC, bool STORE>
 __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) {
     constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BQ * LDSW;
     extern __shared__ float smem[];
@@ -586,6 +703,10 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
     const int q0Start = (firstQuery / BQ) * BQ;
     const int numQTiles = q0Start < p.newLen ? (p.newLen - q0Start + BQ - 1) / BQ : 0;
 
+    // this lane's corner of the wave's column of dS sub-blocks: key sub-block waveK0/32, row 4*half, column li
+    const size_t dsStride = size_t(p.nkb) * 1024;
+    float* const dsColumn = STORE ? p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024 + half * 128 + li : nullptr;
+
     TileRegs<HDP, BQ> qNext, gNext;
     float statNext = 0.0f;
     auto fetchStats = [&](int qt0) {   // thread t < BQ: lse2 of query qt0+t; BQ <= t < 2BQ: D of query qt0+t-BQ
@@ -618,8 +739,13 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
             const float* qcur = qs + (t & 1) * TILE;
             const float* gcur = gs + (t & 1) * TILE;
             const float* scur = stats + (t & 1) * 2 * BQ;
-            if (masked) dkvTile<HDP, BQ, true>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li);
-            else dkvTile<HDP, BQ, false>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li);
+            float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride : nullptr;
+            if (masked)
+                dkvTile<HDP, BQ, true, STORE>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride,
+                                              p.newLen);
+            else
+                dkvTile<HDP, BQ, false, STORE>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride,
+                                               p.newLen);
         }
         if (t + 1 < numQTiles) {
             commitAll((t + 1) & 1);
@@ -666,24 +792,30 @@ bool vec4Ok(const AttnParams& p, std::initializer_list<const void*> ptrs) {
     return true;
 }
 
-// KIND 0 forward, 1 dQ, 2 dK/dV
+// KIND 0 forward, 1 dQ, 2 dK/dV, 3 dK/dV that also stores dS, 4 dQ from stored dS
+template <int HDP, int TILE, bool VEC4, bool STORE>
+int launchDkv(const AttnParams& p, size_t smem, unsigned grid, hipStream_t s) {
+    if (HDP <= 64 && grid > 2u * unsigned(computeUnits()))
+        return launchAttn(attnBackwardDkvKernel<HDP, TILE, VEC4, (HDP <= 64 ? 2 : 1), STORE>, smem, grid, p, s);
+    return launchAttn(attnBackwardDkvKernel<HDP, TILE, VEC4, 1, STORE>, smem, grid, p, s);
+}
+
 template <int KIND, int HDP, int TILE>
 int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
-    constexpr size_t tileBytes = size_t(4) * TILE * (HDP + 4) * sizeof(float);   // two operands, double buffered
-    constexpr size_t smem = KIND == 2 ? tileBytes + 4 * TILE * sizeof(float) : tileBytes;
+    constexpr size_t operandBytes = size_t(2) * TILE * (HDP + 4) * sizeof(float);   // one operand, double buffered
     if constexpr (KIND == 0) {
-        return vec4 ? launchAttn(attnForwardKernel<HDP, TILE, true>, smem, grid, p, s)
-                    : launchAttn(attnForwardKernel<HDP, TILE, false>, smem, grid, p, s);
+        return vec4 ? launchAttn(attnForwardKernel<HDP, TILE, true>, 2 * operandBytes, grid, p, s)
+                    : launchAttn(attnForwardKernel<HDP, TILE, false>, 2 * operandBytes, grid, p, s);
     } else if constexpr (KIND == 1) {
-        return vec4 ? launchAttn(attnBackwardDqKernel<HDP, TILE, true>, smem, grid, p, s)
-                    : launchAttn(attnBackwardDqKernel<HDP, TILE, false>, smem, grid, p, s);
+        return vec4 ? launchAttn(attnBackwardDqKernel<HDP, TILE, true>, 2 * operandBytes, grid, p, s)
+                    : launchAttn(attnBackwardDqKernel<HDP, TILE, false>, 2 * operandBytes, grid, p, s);
+    } else if constexpr (KIND == 4) {
+        constexpr size_t smem = operandBytes + size_t(4) * (TILE / 32) * kDsPatch * sizeof(float);   // K tiles + a dS patch per wave
+        return vec4 ? launchAttn(attnBackwardDqFromDsKernel<HDP, TILE, true>, smem, grid, p, s)
+                    : launchAttn(attnBackwardDqFromDsKernel<HDP, TILE, false>, smem, grid, p, s);
     } else {
-        if (HDP <= 64 && grid > 2u * unsigned(computeUnits())) {
-            return vec4 ? launchAttn(attnBackwardDkvKernel<HDP, TILE, true, (HDP <= 64 ? 2 : 1)>, smem, grid, p, s)
-                        : launchAttn(attnBackwardDkvKernel<HDP, TILE, false, (HDP <= 64 ? 2 : 1)>, smem, grid, p, s);
-        }
-        return vec4 ? launchAttn(attnBackwardDkvKernel<HDP, TILE, true, 1>, smem, grid, p, s)
-                    : launchAttn(attnBackwardDkvKernel<HDP, TILE, false, 1>, smem, grid, p, s);
+        constexpr size_t smem = 2 * operandBytes + 4 * TILE * sizeof(float);
+        return vec4 ? launchDkv<HDP, TILE, true, KIND == 3>(p, smem, grid, s) : launchDkv<HDP, TILE, false, KIND == 3>(p, smem, grid, s);
     }
 }
 
@@ -695,6 +827,23 @@ int dispatch(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
         case 128: return dispatchVec<KIND, 128, 32>(p, vec4, grid, s);
         default: return dispatchVec<KIND, 256, 32>(p, vec4, grid, s);
     }
+}
+
+// Bytes of the dS hand-over buffer: one 32x32 fp32 sub-block per (query sub-block, key sub-block) of every (batch, head).
+size_t dsBytes(size_t batch, size_t heads, size_t newLen, size_t totalLen) {
+    return batch * heads * ((newLen + 31) / 32) * ((totalLen + 31) / 32) * 1024 * sizeof(float);
+}
+
+// Upper limit of the hand-over buffer that bf_hip_attention_backward may take from the pool; SIZE_MAX = an eighth of
+// the device's memory.  Above the limit the backward pass recomputes S and dP in the dQ kernel instead.
+std::atomic<size_t> gDsLimit{SIZE_MAX};
+
+size_t dsLimit() {
+    size_t limit = gDsLimit.load();
+    if (limit != SIZE_MAX) return limit;
+    size_t freeBytes = 0, totalBytes = 0;
+    if (hipMemGetInfo(&freeBytes, &totalBytes) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    return totalBytes / 8;
 }
 
 int checkShapes(const char* fn, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, size_t oldLen) {
@@ -752,6 +901,7 @@ static int fillParams(AttnParams& p, size_t batch, size_t heads, size_t newLen, 
                       size_t oldLen) {
     p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(totalLen);
     p.dim = int(dim); p.hd = int(dim / heads); p.oldLen = int(oldLen); p.scale = scale;
+    p.nqb = int((newLen + 31) / 32); p.nkb = int((totalLen + 31) / 32);
     return BF_OK;
 }
 
@@ -792,6 +942,49 @@ int bf_hip_attention_backward_dkv(const float* dOut, const float* q, const float
     return dispatch<2>(p, vec4Ok(p, {q, k, v, dOut}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
 }
 
+int bf_hip_attention_ds_bytes(size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t* bytes) {
+    BF_REQUIRE(bytes != nullptr, "bytes is NULL");
+    *bytes = dsBytes(batch, heads, newLen, totalLen);
+    return BF_OK;
+}
+
+int bf_hip_attention_set_workspace_limit(size_t bytes) {
+    gDsLimit.store(bytes);
+    return BF_OK;
+}
+
+int bf_hip_attention_backward_dkv_ds(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
+                                     const float* D, float* dK, float* dV, float* dS, size_t batch, size_t heads,
+                                     size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
+                                     bf_stream_t stream) {
+    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+    if (st != BF_OK) return st;
+    if (batch == 0 || dim == 0 || totalLen == 0) return BF_OK;
+    if (newLen == 0)
+        return bf_hip_attention_backward_dkv(dOut, q, k, v, lse2, D, dK, dV, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+    BF_REQUIRE(dOut && q && k && v && lse2 && D && dK && dV && dS, "NULL pointer");
+    BF_REQUIRE((reinterpret_cast<uintptr_t>(dS) & 15u) == 0, "dS must be 16-byte aligned");
+    AttnParams p{};
+    p.q = q; p.k = k; p.v = v; p.dO = dOut; p.dK = dK; p.dV = dV; p.lse2 = lse2; p.dvec = D; p.ds = dS;
+    fillParams(p, batch, heads, newLen, totalLen, dim, scale, oldLen);
+    p.numTiles = int((totalLen + 127) / 128);
+    return dispatch<3>(p, vec4Ok(p, {q, k, v, dOut}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
+}
+
+int bf_hip_attention_backward_dq_from_ds(const float* dS, const float* k, float* dQ, size_t batch, size_t heads, size_t newLen,
+                                         size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
+    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+    if (st != BF_OK) return st;
+    if (batch == 0 || dim == 0 || newLen == 0) return BF_OK;
+    BF_REQUIRE(dS && k && dQ, "NULL pointer");
+    BF_REQUIRE((reinterpret_cast<uintptr_t>(dS) & 15u) == 0, "dS must be 16-byte aligned");
+    AttnParams p{};
+    p.k = k; p.dQ = dQ; p.ds = const_cast<float*>(dS);
+    fillParams(p, batch, heads, newLen, totalLen, dim, scale, oldLen);
+    p.numTiles = int((newLen + 127) / 128);
+    return dispatch<4>(p, vec4Ok(p, {k, dQ}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
+}
+
 int bf_hip_attention_backward_dq(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
                                  const float* D, float* dQ, size_t batch, size_t heads, size_t newLen, size_t totalLen,
                                  size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
@@ -821,6 +1014,16 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
     float* dvec = lse2 + stats;
     st = bf_hip_attention_backward_prepare(out, dOut, m, l, lse2, dvec, batch, heads, newLen, dim, stream);
     if (st != BF_OK) return st;
+    // With room for the dS hand-over buffer the dK/dV kernel leaves dS behind and dQ is one contraction over it.
+    const size_t handOver = dsBytes(batch, heads, newLen, totalLen);
+    if (newLen > 0 && totalLen > 0 && handOver <= dsLimit()) {
+        Scratch ds(handOver);
+        if (ds.status != BF_OK) return ds.status;
+        st = bf_hip_attention_backward_dkv_ds(dOut, q, k, v, lse2, dvec, dK, dV, ds.as<float>(), batch, heads, newLen, totalLen, dim, scale,
+                                              oldLen, stream);
+        if (st != BF_OK) return st;
+        return bf_hip_attention_backward_dq_from_ds(ds.as<float>(), k, dQ, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+    }
     st = bf_hip_attention_backward_dkv(dOut, q, k, v, lse2, dvec, dK, dV, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
     if (st != BF_OK) return st;
     return bf_hip_attention_backward_dq(dOut, q, k, v, lse2, dvec, dQ, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);

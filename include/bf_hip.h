@@ -255,6 +255,24 @@ int bf_hip_attention_backward_dq(const float* dOut, const float* q, const float*
                                  const float* D, float* dQ, size_t batch, size_t heads, size_t newLen, size_t totalLen,
                                  size_t dim, float scale, size_t oldLen, bf_stream_t stream);
 
+/* The same backward pass with dS handed from the key-tile owner to the query-tile owner through HBM instead of
+ * being recomputed: dkv_ds also writes dS = P * (dP - D) (without the scale factor) as 32x32 fp32 sub-blocks,
+ * dS[((bh * ceil(newLen/32) + queryBlock) * ceil(totalLen/32) + keyBlock) * 1024 + query%32 * 32 + key%32], at least
+ * every sub-block whose first key is not after its last query (the others hold no visible pair and are not read);
+ * dq_from_ds contracts those sub-blocks with K (dQ = scale *
+ * dS * K), so the pass runs the five matrix products of tiledFusedAttentionBackwardKernel (fused_attention.cu:201-303)
+ * once each.  ds_bytes gives the size of that buffer (16-byte aligned device memory).  bf_hip_attention_backward
+ * takes this route by itself when the buffer fits under the workspace limit (default: an eighth of the device's
+ * memory; 0 = always recompute); the limit has no counterpart in the reference, whose kernel holds dS in registers. */
+int bf_hip_attention_ds_bytes(size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t* bytes);
+int bf_hip_attention_set_workspace_limit(size_t bytes);
+int bf_hip_attention_backward_dkv_ds(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
+                                     const float* D, float* dK, float* dV, float* dS, size_t batch, size_t heads,
+                                     size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
+                                     bf_stream_t stream);
+int bf_hip_attention_backward_dq_from_ds(const float* dS, const float* k, float* dQ, size_t batch, size_t heads, size_t newLen,
+                                         size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Losses                                                      (reference: loss.hpp:20-70, loss.cu)
  * Each writes grad (same shape as the prediction) and the SUM over the batch of the per-row (per-

@@ -52,6 +52,75 @@ def test_attention_core_matches_the_oracle(hip, oracle, rng, batch, heads, new_l
         assert_close(got, exp, what=f"{name} case {(batch, heads, new_len, old_len, hd)}", scale=sc[name])
 
 
+@pytest.fixture
+def recompute_route(hip):
+    """Workspace limit 0: bf_hip_attention_backward recomputes S and dP in the dQ kernel instead of reading dS back."""
+    hip.capi.call("bf_hip_attention_set_workspace_limit", 0)
+    yield
+    hip.capi.call("bf_hip_attention_set_workspace_limit", 2 ** 64 - 1)
+
+
+@pytest.mark.parametrize("batch,heads,new_len,old_len,hd", CASES)
+def test_attention_backward_recompute_route(hip, oracle, rng, recompute_route, batch, heads, new_len, old_len, hd):
+    dim, total = heads * hd, old_len + new_len
+    q, k, v, go = r(rng, batch, new_len, dim), r(rng, batch, total, dim), r(rng, batch, total, dim), r(rng, batch, new_len, dim)
+    scale = float(f32(1.0) / np.sqrt(f32(hd)))
+    _, _, _, dq, dk, dv = run_gpu(hip, q, k, v, go, heads, scale, old_len)
+    edq, edk, edv = oracle.attentionCoreBackward(go, q, k, v, heads, scale, old_len)
+    sc = grad_scales(q, k, v, go, scale)
+    for got, exp, name in ((dq, edq, "dQ"), (dk, edk, "dK"), (dv, edv, "dV")):
+        assert_close(got, exp, what=f"{name} case {(batch, heads, new_len, old_len, hd)}", scale=sc[name])
+
+
+@pytest.mark.parametrize("batch,heads,new_len,old_len,hd", [(2, 2, 70, 0, 16), (1, 3, 45, 100, 64), (1, 1, 130, 3, 128), (1, 2, 33, 0, 200)])
+def test_ds_hand_over_buffer(hip, rng, batch, heads, new_len, old_len, hd):
+    """The dS sub-blocks that the dK/dV kernel leaves for the dQ kernel, against dS = P * (dP - D) in float64, and
+    dQ from them; a sub-block with no visible (query, key) pair is either left alone or written as zeros."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    import ctypes
+    dim, total = heads * hd, old_len + new_len
+    scale = float(f32(1.0) / np.sqrt(f32(hd)))
+    q, k, v, go = r(rng, batch, new_len, dim), r(rng, batch, total, dim), r(rng, batch, total, dim), r(rng, batch, new_len, dim)
+    dq_, dk_, dv_, dgo = map(D.fromHost, (q, k, v, go))
+    fwd = hip.ops.fusedAttentionForward(dq_, dk_, dv_, heads, scale, old_len)
+    lse2, dvec = D((batch, heads, new_len)), D((batch, heads, new_len))
+    call("bf_hip_attention_backward_prepare", fwd.output.ptr, dgo.ptr, fwd.m.ptr, fwd.l.ptr, lse2.ptr, dvec.ptr, batch, heads, new_len, dim, None)
+    nbytes = ctypes.c_size_t(0)
+    call("bf_hip_attention_ds_bytes", batch, heads, new_len, total, ctypes.byref(nbytes))
+    nqb, nkb = (new_len + 31) // 32, (total + 31) // 32
+    assert nbytes.value == batch * heads * nqb * nkb * 4096
+    fill = f32(12345.0)
+    ds = D.fromHost(np.full((batch * heads, nqb, nkb, 32, 32), fill, f32))
+    dK, dV, dQ = D((batch, total, dim)), D((batch, total, dim)), D((batch, new_len, dim))
+    tail = (batch, heads, new_len, total, dim, ctypes.c_float(scale), old_len, None)
+    call("bf_hip_attention_backward_dkv_ds", dgo.ptr, dq_.ptr, dk_.ptr, dv_.ptr, lse2.ptr, dvec.ptr, dK.ptr, dV.ptr, ds.ptr, *tail)
+    call("bf_hip_attention_backward_dq_from_ds", ds.ptr, dk_.ptr, dQ.ptr, *tail)
+    got = ds.toHost()
+    # float64 restatement of dS
+    split = lambda t, n: t.reshape(batch, n, heads, hd).transpose(0, 2, 1, 3).astype(np.float64)
+    Q, K, V, G = split(q, new_len), split(k, total), split(v, total), split(go, new_len)
+    S = np.einsum("bhid,bhjd->bhij", Q, K) * scale
+    visible = np.arange(total)[None, :] <= old_len + np.arange(new_len)[:, None]
+    S = np.where(visible, S, -np.inf)
+    P = np.exp(S - S.max(-1, keepdims=True))
+    P /= P.sum(-1, keepdims=True)
+    dP = np.einsum("bhid,bhjd->bhij", G, V)
+    Dv = (P * dP).sum(-1, keepdims=True)
+    dS = P * (dP - Dv)
+    padded = np.zeros((batch * heads, nqb * 32, nkb * 32))
+    padded[:, :new_len, :total] = dS.reshape(batch * heads, new_len, total)
+    tiles = padded.reshape(batch * heads, nqb, 32, nkb, 32).transpose(0, 1, 3, 2, 4)
+    for qb in range(nqb):
+        for kb in range(nkb):
+            if kb * 32 <= old_len + qb * 32 + 31:   # some key of the sub-block is at or before its last query: read by the dQ kernel
+                assert_close(got[:, qb, kb], tiles[:, qb, kb].astype(f32), what=f"dS sub-block ({qb},{kb})", scale=rms(go) * rms(v))
+            else:
+                assert np.all((got[:, qb, kb] == fill) | (got[:, qb, kb] == 0)), f"masked sub-block ({qb},{kb}) holds values"
+                assert not tiles[:, qb, kb].any()
+    edq = (np.einsum("bhij,bhjd->bhid", dS, K) * scale).transpose(0, 2, 1, 3).reshape(batch, new_len, dim)
+    assert_close(dQ.toHost(), edq.astype(f32), what="dQ from dS", scale=grad_scales(q, k, v, go, scale)["dQ"])
+
+
 @pytest.mark.parametrize("new_len,hd,growth,qscale", [(300, 64, 0.25, 1.0), (200, 32, 0.6, 1.0), (513, 128, 0.1, 0.3), (260, 64, -0.3, 1.0)])
 def test_attention_with_drifting_row_maximum(hip, oracle, rng, new_len, hd, growth, qscale):
     """Scores that keep growing (or shrinking) along the key axis: the running row maximum passes the forward kernel's
@@ -70,6 +139,9 @@ def test_attention_with_drifting_row_maximum(hip, oracle, rng, new_len, hd, grow
     if growth > 0:
         assert float(em.max() - em[..., 0].min()) > 8 * np.log(2.0) * 5, "the case must cross the threshold several times"
     sc = grad_scales(q, k, v, go, scale)
+    # K carries the ramp, so the terms that dQ = scale * dS * K sums are as large as max|K|, not rms(K); against float64
+    # the CPU reference and both GPU routes are each about 3e-4 away on the growing cases.
+    sc["dQ"] = rms(go) * rms(v) * float(np.abs(k).max()) * scale
     for got, exp, name in ((o, eo, "O"), (m, em, "m"), (l, el, "l"), (dq, edq, "dQ"), (dk, edk, "dK"), (dv, edv, "dV")):
         assert_close(got, exp, what=f"{name} drifting maximum {(new_len, hd, growth)}", scale=sc[name])
 
