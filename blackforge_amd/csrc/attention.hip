@@ -605,28 +605,35 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnBackwardDqFromDsK
 // stats: [0..BQ) = lse2 of the tile's queries (+inf for padding rows), [BQ..2BQ) = D.
 // STORE: also writes each dS sub-block (32 queries x 32 keys, row-major) to dsLane + sb*dsStride for the dQ kernel
 // that contracts it with K; dsLane already points at this lane's column and first row (li + 128*half floats in).
-template <int HDP, int BQ, bool MASKED, bool STORE>
+// AHEAD: the S / dP products of sub-block sb+1 are issued before the exp / dS arithmetic of sub-block sb (two sub-blocks
+// of scores live at once).  With two waves per SIMD the other wave fills the matrix pipe during that arithmetic, and
+// the 32 registers are worth more as room that keeps the kernel from spilling.
+template <int HDP, int BQ, bool MASKED, bool STORE, bool AHEAD>
 __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const float* __restrict__ gs, const float* __restrict__ stats,
                                         const float (&kreg)[HDP / 2], const float (&vreg)[HDP / 2], float16v (&dk)[HDP / 32],
                                         float16v (&dv)[HDP / 32], int qt0, int key, bool keyValid, int oldLen, int half, int li,
                                         float* __restrict__ dsLane, size_t dsStride, int newLen) {
-    constexpr int LDSW = HDP + 4, DT = HDP / 32, NSB = BQ / 32;
-    float16v s[NSB], dp[NSB];
+    constexpr int LDSW = HDP + 4, DT = HDP / 32, NSB = BQ / 32, LIVE = AHEAD ? NSB : 1;
+    float16v s[LIVE], dp[LIVE];
+    auto scores = [&](int sb) {   // S = Q * K^T and dP = dO * V^T of sub-block sb
+        float16v& sDst = s[AHEAD ? sb : 0];
+        float16v& dpDst = dp[AHEAD ? sb : 0];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { s[0][r] = 0.0f; dp[0][r] = 0.0f; }
-    s[0] = headDotB<HDP>(qs + li * LDSW + half * (HDP / 2), kreg, s[0]);     // S  = Q  * K^T
-    dp[0] = headDotB<HDP>(gs + li * LDSW + half * (HDP / 2), vreg, dp[0]);   // dP = dO * V^T
+        for (int r = 0; r < 16; ++r) { sDst[r] = 0.0f; dpDst[r] = 0.0f; }
+        sDst = headDotB<HDP>(qs + (sb * 32 + li) * LDSW + half * (HDP / 2), kreg, sDst);
+        dpDst = headDotB<HDP>(gs + (sb * 32 + li) * LDSW + half * (HDP / 2), vreg, dpDst);
+    };
+    if constexpr (AHEAD) scores(0);
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb) {
-        if (sb + 1 < NSB) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) { s[sb + 1][r] = 0.0f; dp[sb + 1][r] = 0.0f; }
-            s[sb + 1] = headDotB<HDP>(qs + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), kreg, s[sb + 1]);
-            dp[sb + 1] = headDotB<HDP>(gs + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), vreg, dp[sb + 1]);
+        if constexpr (AHEAD) {
+            if (sb + 1 < NSB) scores(sb + 1);
+        } else {
+            scores(sb);
         }
         // register r: query = qt0 + sb*32 + dRow(r, half), key = this lane's key
-        float16v& pr = s[sb];
-        float16v& dsv = dp[sb];
+        float16v& pr = s[AHEAD ? sb : 0];
+        float16v& dsv = dp[AHEAD ? sb : 0];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             float4v lse4 = loadf4(stats + sb * 32 + 8 * g + 4 * half);
@@ -705,7 +712,8 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
 
     // this lane's corner of the wave's column of dS sub-blocks: key sub-block waveK0/32, row 4*half, column li
     const size_t dsStride = size_t(p.nkb) * 1024;
-    float* const dsColumn = STORE ? p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024 + half * 128 + li : nullptr;
+    float* const dsColumn = STORE ? p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024 : nullptr;   // wave-uniform
+    const int dsLaneOffset = half * 128 + li;
 
     TileRegs<HDP, BQ> qNext, gNext;
     float statNext = 0.0f;
@@ -739,12 +747,12 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
             const float* qcur = qs + (t & 1) * TILE;
             const float* gcur = gs + (t & 1) * TILE;
             const float* scur = stats + (t & 1) * 2 * BQ;
-            float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride : nullptr;
+            float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
             if (masked)
-                dkvTile<HDP, BQ, true, STORE>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride,
+                dkvTile<HDP, BQ, true, STORE, OCC == 1>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride,
                                               p.newLen);
             else
-                dkvTile<HDP, BQ, false, STORE>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride,
+                dkvTile<HDP, BQ, false, STORE, OCC == 1>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride,
                                                p.newLen);
         }
         if (t + 1 < numQTiles) {
