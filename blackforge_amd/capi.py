@@ -106,6 +106,7 @@ SIGNATURES = {
     "bf_hip_mse": [P, P, P, P, c_size, c_int, S],
     "bf_hip_cross_entropy": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse": [P, P, P, P, c_size, c_size, c_int, S],
+    "bf_hip_cross_entropy_masked": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_sgd_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_size), c_size, c_float, S],
     "bf_hip_adamw_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr),
                            ctypes.POINTER(c_size), c_size, c_ll, c_float, c_float, c_float, c_float, c_float, S],

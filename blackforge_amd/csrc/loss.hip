@@ -22,6 +22,31 @@ __global__ void __launch_bounds__(1024) finishSumKernel(const float* __restrict_
     if (threadIdx.x == 0) out[0] = accumulate ? out[0] + float(s) : float(s);
 }
 
+// info[0] = number of entries of `target` that do not round to -1, info[1] = 1 / info[0] (0 when there is none).
+__global__ void __launch_bounds__(1024) countUnmaskedKernel(const float* __restrict__ target, size_t rows, float* __restrict__ info) {
+    __shared__ double lds[16];
+    double n = 0.0;
+    for (size_t i = threadIdx.x; i < rows; i += blockDim.x) n += lroundf(target[i]) == -1 ? 0.0 : 1.0;
+    const double total = blockReduce(n, 0.0, OpSum{}, lds);
+    if (threadIdx.x == 0) {
+        info[0] = float(total);
+        info[1] = total > 0.0 ? 1.0f / float(total) : 0.0f;
+    }
+}
+
+// finishSumKernel with the total scaled by *scale (read on the device) before it is stored or accumulated.
+__global__ void __launch_bounds__(1024) finishScaledSumKernel(const float* __restrict__ partial, size_t count, const float* __restrict__ scale,
+                                                              float* __restrict__ out, int accumulate) {
+    __shared__ double lds[16];
+    double s = 0.0;
+    for (size_t i = threadIdx.x; i < count; i += blockDim.x) s += double(partial[i]);
+    s = blockReduce(s, 0.0, OpSum{}, lds);
+    if (threadIdx.x == 0) {
+        const float mean = float(s * double(scale[0]));
+        out[0] = accumulate ? out[0] + mean : mean;
+    }
+}
+
 template <int VEC>
 __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pred, const float* __restrict__ target,
                                                     float* __restrict__ grad, float* __restrict__ partial, size_t n,
@@ -57,15 +82,32 @@ template <int G, int MAXE, int VEC, bool CACHED, bool SPARSE>
 __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const float* __restrict__ logits,
                                                                          const float* __restrict__ target,
                                                                          float* __restrict__ grad, float* __restrict__ rowLoss,
-                                                                         size_t rows, size_t classes, float invRows) {
+                                                                         size_t rows, size_t classes, float invRows,
+                                                                         const float* __restrict__ maskInfo) {
     __shared__ float lds[16];
     const int t = threadIdx.x % G;
     const size_t rowsPerBlock = blockDim.x / G;
     const size_t rowStep = size_t(gridDim.x) * rowsPerBlock;
+    // masked form (sparse targets only): maskInfo[1] = 1 / (number of rows whose index is not -1) replaces 1 / rows,
+    // and a row with index -1 contributes nothing: zero gradient, zero loss
+    if (SPARSE && maskInfo != nullptr) invRows = maskInfo[1];
     for (size_t row = size_t(blockIdx.x) * rowsPerBlock + threadIdx.x / G; row < rows; row += rowStep) {
         const float* x = logits + row * classes;
         float* gOut = grad + row * classes;
         RowCache<G, MAXE, VEC> c;
+        if constexpr (SPARSE) {
+            if (maskInfo != nullptr && lroundf(target[row]) == -1) {   // uniform over the row's group
+                if constexpr (CACHED) {
+#pragma unroll
+                    for (int i = 0; i < MAXE; ++i) c.r[i] = 0.0f;
+                    c.store(gOut, classes, t);
+                } else {
+                    for (size_t e = t; e < classes; e += G) gOut[e] = 0.0f;
+                }
+                if (t == 0) rowLoss[row] = 0.0f;
+                continue;
+            }
+        }
         float mx = -INFINITY;
         if constexpr (CACHED) {
             c.load(x, classes, t, -INFINITY);
@@ -142,10 +184,16 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
 
 template <bool SPARSE>
 int launchCrossEntropy(const float* logits, const float* target, float* grad, float* lossSum, size_t rows,
-                       size_t classes, int accumulate, hipStream_t s) {
-    Scratch rowLoss(rows * sizeof(float));
+                       size_t classes, int accumulate, hipStream_t s, bool masked = false) {
+    Scratch rowLoss((rows + 2) * sizeof(float));   // per-row losses, then the two words of the masked form
     if (rowLoss.status != BF_OK) return rowLoss.status;
     float* rl = rowLoss.as<float>();
+    const float* maskInfo = nullptr;
+    if (masked) {
+        countUnmaskedKernel<<<1, 1024, 0, s>>>(target, rows, rl + rows);
+        BF_LAUNCH_CHECK();
+        maskInfo = rl + rows;
+    }
     const float invRows = 1.0f / float(rows);
     const bool vec4 = aligned16(logits) && aligned16(grad) && classes % 4 == 0;
     // smallest group and register count that hold a row (see the row kernels); a block takes its rows once
@@ -153,17 +201,18 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
     if (classes <= size_t(G) * MAXE) {                                                                            \
         const unsigned threads = G > 256 ? G : 256;                                                               \
         const unsigned grid = gridFor(rows, threads / G);                                                         \
-        if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows); \
-        else crossEntropyKernel<G, MAXE, 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows);      \
+        if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
+        else crossEntropyKernel<G, MAXE, 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo);      \
         break;                                                                                                    \
     }
     do {
         BF_CE(64, 4) BF_CE(64, 8) BF_CE(64, 16) BF_CE(256, 8) BF_CE(256, 16) BF_CE(256, 32) BF_CE(1024, 16) BF_CE(1024, 32)
-        crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows);
+        crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo);
     } while (0);
 #undef BF_CE
     BF_LAUNCH_CHECK();
-    finishSumKernel<<<1, 1024, 0, s>>>(rl, rows, lossSum, accumulate);
+    if (masked) finishScaledSumKernel<<<1, 1024, 0, s>>>(rl, rows, maskInfo + 1, lossSum, accumulate);
+    else finishSumKernel<<<1, 1024, 0, s>>>(rl, rows, lossSum, accumulate);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -218,6 +267,17 @@ int bf_hip_cross_entropy_sparse(const float* logits, const float* targetIdx, flo
     }
     BF_REQUIRE(logits && targetIdx && grad, "NULL pointer");
     return launchCrossEntropy<true>(logits, targetIdx, grad, lossSum, rows, classes, accumulate, asStream(stream));
+}
+
+int bf_hip_cross_entropy_masked(const float* logits, const float* targetIdx, float* grad, float* lossMean, size_t rows,
+                                size_t classes, int accumulate, bf_stream_t stream) {
+    BF_REQUIRE(lossMean != nullptr, "lossMean is NULL");
+    if (rows == 0 || classes == 0) {
+        if (!accumulate) return bf_hip_fill_zero(lossMean, sizeof(float), stream);
+        return BF_OK;
+    }
+    BF_REQUIRE(logits && targetIdx && grad, "NULL pointer");
+    return launchCrossEntropy<true>(logits, targetIdx, grad, lossMean, rows, classes, accumulate, asStream(stream), true);
 }
 
 }  // extern "C"

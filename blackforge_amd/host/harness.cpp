@@ -52,7 +52,7 @@ extern "C" {
 const char* bfh_last_error(void) { return g_error.c_str(); }
 
 // kinds follow hip::LayerKind order: 0 linear, 1 silu, 2 relu, 3 gelu, 4 rmsnorm, 5 softmax, 6 embedding,
-// 7 positional embedding, 8 attention, 9 feedforward (arg1: 0 SiLU, 1 GELU)
+// 7 positional embedding, 8 attention, 9 feedforward (arg1: 0 SiLU, 1 GELU), 10 bidirectional attention
 void* bfh_model_create(int numLayers, const int* kinds, const long long* arg0, const long long* arg1, size_t inputFeatures,
                        int useBf16) {
     Handle* handle = nullptr;
@@ -99,15 +99,17 @@ int bfh_model_forward(void* h, const float* input, int rank, const size_t* shape
     });
 }
 
-// lossKind 0: sparse cross-entropy (targets = one class index per output row), 1: mean squared error.
-// The loss sum is accumulated on the device; bfh_model_read_loss reads and resets it.
+// lossKind 0: sparse cross-entropy (targets = one class index per output row), 1: mean squared error, 2: masked sparse
+// cross-entropy (index -1 = row ignored).  The loss sum (for kind 2: the mean over the rows not ignored) is accumulated on the
+// device; bfh_model_read_loss reads and resets it.
 int bfh_model_loss(void* h, const float* target, int lossKind) {
     Handle* handle = static_cast<Handle*>(h);
     return guarded([&] {
-        if (lossKind == 0) {
+        if (lossKind == 0 || lossKind == 2) {
             std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
             Borrowed tgt(target, {rows});
-            handle->lossGrad = hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
+            handle->lossGrad = lossKind == 0 ? hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator)
+                                             : hip::softmaxCrossEntropyMaskedAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
         } else {
             Borrowed tgt(target, handle->output.shape());
             handle->lossGrad = hip::meanSquaredErrorAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
@@ -158,10 +160,11 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
         handle->model->zeroGrad();
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
         handle->output = handle->model->forward(in.tensor, true);
-        if (lossKind == 0) {
+        if (lossKind == 0 || lossKind == 2) {
             std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
             Borrowed tgt(target, {rows});
-            handle->lossGrad = hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
+            handle->lossGrad = lossKind == 0 ? hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator)
+                                             : hip::softmaxCrossEntropyMaskedAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
         } else {
             Borrowed tgt(target, handle->output.shape());
             handle->lossGrad = hip::meanSquaredErrorAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
@@ -184,7 +187,7 @@ int bfh_model_read_loss(void* h, float* sum) {
     });
 }
 
-// hip::runTraining over a BFDATA1 file (lossKind: 0 mse, 1 cross_entropy, 2 cross_entropy_sparse; optimizerKind: 0 sgd,
+// hip::runTraining over a BFDATA1 file (lossKind: 0 mse, 1 cross_entropy, 2 cross_entropy_sparse, 3 cross_entropy_masked; optimizerKind: 0 sgd,
 // 1 adamw); epochLosses receives `epochs` values.
 int bfh_model_run_training(void* h, const char* datasetPath, int lossKind, int optimizerKind, long long epochs, size_t batchSize,
                            double learningRate, int cosineSchedule, const char* fromCheckpoint, const char* saveCheckpoint,
@@ -193,7 +196,7 @@ int bfh_model_run_training(void* h, const char* datasetPath, int lossKind, int o
     return guarded([&] {
         hip::HostDataset dataset = hip::HostDataset::load(datasetPath);
         hip::TrainOptions options;
-        options.loss = lossKind == 0 ? "mse" : lossKind == 1 ? "cross_entropy" : "cross_entropy_sparse";
+        options.loss = lossKind == 0 ? "mse" : lossKind == 1 ? "cross_entropy" : lossKind == 2 ? "cross_entropy_sparse" : "cross_entropy_masked";
         options.optimizer = optimizerKind == 0 ? "sgd" : "adamw";
         options.epochs = epochs;
         options.batchSize = batchSize;

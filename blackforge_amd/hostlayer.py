@@ -14,8 +14,8 @@ from .tensor import DeviceTensor
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libbf_hip_host.so")
 
-LINEAR, SILU, RELU, GELU, RMSNORM, SOFTMAX, EMBEDDING, POSITIONAL, ATTENTION, FEEDFORWARD = range(10)
-LOSS_SPARSE_CE, LOSS_MSE = 0, 1
+LINEAR, SILU, RELU, GELU, RMSNORM, SOFTMAX, EMBEDDING, POSITIONAL, ATTENTION, FEEDFORWARD, BIDIRECTIONAL_ATTENTION = range(11)
+LOSS_SPARSE_CE, LOSS_MSE, LOSS_MASKED_CE = 0, 1, 2
 
 _lib = None
 
@@ -156,7 +156,7 @@ class HostModel:
                     cosine: bool = False, from_checkpoint: str = "", save_checkpoint: str = ""):
         """hip::runTraining over a BFDATA1 file; returns the epoch losses."""
         losses = (ctypes.c_double * max(epochs, 1))()
-        _check(load().bfh_model_run_training(self.handle, dataset_path.encode(), {"mse": 0, "cross_entropy": 1, "cross_entropy_sparse": 2}[loss],
+        _check(load().bfh_model_run_training(self.handle, dataset_path.encode(), {"mse": 0, "cross_entropy": 1, "cross_entropy_sparse": 2, "cross_entropy_masked": 3}[loss],
                                              {"sgd": 0, "adamw": 1}[optimizer], epochs, batch_size, lr, int(cosine),
                                              from_checkpoint.encode(), save_checkpoint.encode(), losses))
         self._refresh_params()

@@ -11,6 +11,8 @@ from __future__ import annotations
 
 import ctypes
 import math
+
+import numpy as np
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 
@@ -438,6 +440,7 @@ class SelfAttentionCache:
     attnOutput: Optional[DeviceTensor] = None
     attnM: Optional[DeviceTensor] = None
     attnL: Optional[DeviceTensor] = None
+    causal: bool = True   # False: bidirectionalSelfAttention
 
 
 @dataclass
@@ -527,19 +530,33 @@ def _check_attention(name, x, numHeads):
 
 
 def selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads: int, useBf16: bool, cache: SelfAttentionCache,
-                               cachedWeights: bool = True):
-    _check_attention("selfAttention", x, numHeads)
+                               cachedWeights: bool = True, causal: bool = True):
+    _check_attention("selfAttention" if causal else "bidirectionalSelfAttention", x, numHeads)
     batch, seq, dim = x.shape
+    cache.causal = causal
     scaleFactor = 1.0 / math.sqrt(dim // numHeads)
     mm = _mm(useBf16, cachedWeights)
     cache.normedFlat = rmsnorm(x).reshaped((batch * seq, dim))
     cache.q = mm(cache.normedFlat, wq).reshaped((batch, seq, dim))
     cache.k = mm(cache.normedFlat, wk).reshaped((batch, seq, dim))
     cache.v = mm(cache.normedFlat, wv).reshaped((batch, seq, dim))
-    attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, 0)
+    # query i sees keys j <= oldLen + i: an offset of seq makes every key visible (the bidirectional form)
+    attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, 0 if causal else seq)
     cache.attnOutput, cache.attnM, cache.attnL = attn.output, attn.m, attn.l
     projected = mm(_flat2d(cache.attnOutput), wout).reshaped((batch, seq, dim))
     return add(x, projected)
+
+
+def bidirectionalSelfAttention(x, wq, wk, wv, wout, numHeads: int, useBf16: bool = False):
+    """The block without the causal mask (CPU backend, ops.cpp:504-507; absent from the CUDA backend, model.cu:151-160)."""
+    return selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, useBf16, SelfAttentionCache(), False, causal=False)
+
+
+def bidirectionalSelfAttentionBackward(x, wq, wk, wv, wout, numHeads: int, g, useBf16: bool = False) -> "SelfAttentionGrad":
+    """cpu autodiff.cpp:492-496: recomputes the (non-causal) forward, then the shared backward."""
+    cache = SelfAttentionCache()
+    selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, useBf16, cache, False, causal=False)
+    return selfAttentionBackwardCached(x, wq, wk, wv, wout, numHeads, cache, g, useBf16, False)
 
 
 def selfAttention(x, wq, wk, wv, wout, numHeads: int):
@@ -567,7 +584,7 @@ def selfAttentionBackwardCached(x, wq, wk, wv, wout, numHeads: int, cache: SelfA
     dOutFlat, dWout = bwd(_flat2d(cache.attnOutput), wout, _flat2d(g))
     dOutput = dOutFlat.reshaped((batch, seq, dim))
     ag = fusedAttentionBackward(dOutput, cache.q, cache.k, cache.v, cache.attnOutput, cache.attnM, cache.attnL, numHeads,
-                                scaleFactor, 0)
+                                scaleFactor, 0 if cache.causal else seq)
     dNq, dWq = bwd(cache.normedFlat, wq, _flat2d(ag.dQ))
     dNk, dWk = bwd(cache.normedFlat, wk, _flat2d(ag.dK))
     dNv, dWv = bwd(cache.normedFlat, wv, _flat2d(ag.dV))
@@ -681,6 +698,27 @@ def softmaxCrossEntropySparse(logits, targetIndices) -> LossResult:
     grad, total = DeviceTensor(logits.shape), DeviceTensor((1,))
     _call("bf_hip_cross_entropy_sparse", logits.ptr, targetIndices.ptr, grad.ptr, total.ptr, rows, classes, 0, None)
     return LossResult(_read_scalar(total) / rows if rows else 0.0, grad)
+
+
+def softmaxCrossEntropyMasked(logits, targetIndices) -> LossResult:
+    """cpu loss.cpp:149-215: rows whose index is -1 are ignored; loss and gradient are means over the other rows."""
+    _check_sparse("softmaxCrossEntropyMasked", logits, targetIndices)
+    rows, classes = _rows(logits)
+    if rows:
+        idx = np.rint(targetIndices.toHost()).astype(np.int64).ravel()
+        bad = idx[(idx != -1) & ((idx < 0) | (idx >= classes))]
+        _require(bad.size == 0, f"softmaxCrossEntropyMasked: class index {bad[0] if bad.size else 0} outside [0, {classes}) (or -1 to ignore)")
+    grad, mean = DeviceTensor(logits.shape), DeviceTensor((1,))
+    _call("bf_hip_cross_entropy_masked", logits.ptr, targetIndices.ptr, grad.ptr, mean.ptr, rows, classes, 0, None)
+    return LossResult(_read_scalar(mean), grad)
+
+
+def softmaxCrossEntropyMaskedAccumulate(logits, targetIndices, lossAccumulator: DeviceTensor) -> DeviceTensor:
+    """Adds this call's mean over the rows that are not ignored to lossAccumulator; indices are the caller's precondition."""
+    _check_sparse("softmaxCrossEntropyMaskedAccumulate", logits, targetIndices)
+    grad = DeviceTensor(logits.shape)
+    _call("bf_hip_cross_entropy_masked", logits.ptr, targetIndices.ptr, grad.ptr, lossAccumulator.ptr, *_rows(logits), 1, None)
+    return grad
 
 
 # ------------------------------------------------------------------------------------------------

@@ -288,6 +288,13 @@ int bf_hip_cross_entropy(const float* logits, const float* target, float* grad, 
 /* softmaxCrossEntropySparse[Accumulate]: target class index per row; indices must already be in range */
 int bf_hip_cross_entropy_sparse(const float* logits, const float* targetIdx, float* grad, float* lossSum,
                                 size_t rows, size_t classes, int accumulate, bf_stream_t stream);
+/* softmaxCrossEntropyMasked (the CPU backend's loss for masked-language-model training, src/backend/cpu/loss.cpp:149-215;
+ * the CUDA backend has no counterpart): as the sparse form, except that a row whose index rounds to -1 is ignored (zero
+ * gradient, no loss term) and gradient and loss are averaged over the n rows that are not: grad = (p - onehot) / n, and
+ * lossMean[0] receives (or, with accumulate != 0, is increased by) the MEAN over those n rows, 0 when n == 0.  n is
+ * counted on the device.  Every other index must already be in [0, classes). */
+int bf_hip_cross_entropy_masked(const float* logits, const float* targetIdx, float* grad, float* lossMean, size_t rows,
+                                size_t classes, int accumulate, bf_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Optimizers                                              (reference: optimizer.hpp:28-66, optimizer.cu)

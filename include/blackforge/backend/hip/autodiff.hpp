@@ -226,7 +226,7 @@ inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& inpu
     float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
     MatmulGrad outGrad = projectionBackward(cache.attnOutput, wout, gradOutput, mode, {batch, seq, dim});
     FusedAttentionGrad attn = fusedAttentionBackward(outGrad.dA, cache.q, cache.k, cache.v, cache.attnOutput, cache.attnM,
-                                                      cache.attnL, numHeads, scaleFactor, 0);
+                                                      cache.attnL, numHeads, scaleFactor, cache.causal ? 0 : seq);
     if (mode != 0) {
         // the three projection gradients share their input: one GEMM sums dQ Wq^T + dK Wk^T + dV Wv^T, one produces
         // the three weight gradients (for widths that are multiples of 256; separate GEMMs otherwise)
@@ -266,6 +266,22 @@ inline SelfAttentionGrad selfAttentionBf16Backward(const DeviceTensor& input, co
                                                     const DeviceTensor& gradOutput) {
     SelfAttentionCache cache;
     detail::selfAttentionForwardImpl("selfAttentionBf16Backward", input, wq, wk, wv, wout, numHeads, 1, cache);
+    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, 1);
+}
+// Gradients of bidirectionalSelfAttention (src/backend/cpu/autodiff.cpp:492-496): the cache remembers that the forward
+// pass was not causal, so the cached form is selfAttentionBackwardCached; these recompute the forward pass first.
+inline SelfAttentionGrad bidirectionalSelfAttentionBackward(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                             const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                             const DeviceTensor& gradOutput) {
+    SelfAttentionCache cache;
+    detail::selfAttentionForwardImpl("bidirectionalSelfAttentionBackward", input, wq, wk, wv, wout, numHeads, 0, cache, false);
+    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, 0);
+}
+inline SelfAttentionGrad bidirectionalSelfAttentionBf16Backward(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                                 const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                                 const DeviceTensor& gradOutput) {
+    SelfAttentionCache cache;
+    detail::selfAttentionForwardImpl("bidirectionalSelfAttentionBf16Backward", input, wq, wk, wv, wout, numHeads, 1, cache, false);
     return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, 1);
 }
 

@@ -1,6 +1,8 @@
 #pragma once
 // Loss functions with the reference's signatures (include/blackforge/backend/cuda/loss.hpp:7-70).
+#include <cmath>
 #include <cstddef>
+#include <string>
 
 #include "blackforge/backend/hip/device_tensor.hpp"
 #include "blackforge/backend/hip/ops.hpp"
@@ -59,6 +61,31 @@ inline LossResult softmaxCrossEntropySparse(const DeviceTensor& logits, const De
     return r;
 }
 
+namespace detail {
+// src/backend/cpu/loss.cpp:171-178: an index is -1 (row ignored) or lies in [0, classes); checked on a host copy
+inline void requireMaskedIds(const char* op, const DeviceTensor& idx, std::size_t classes) {
+    const runtime::Tensor host = idx.toHost();
+    for (std::size_t i = 0; i < host.elementCount(); ++i) {
+        const long long index = static_cast<long long>(std::lround(host.at(i)));
+        require(index == -1 || (index >= 0 && static_cast<std::size_t>(index) < classes),
+                std::string(op) + ": class index " + std::to_string(index) + " outside [0, " + std::to_string(classes) + ") (or -1 to ignore)");
+    }
+}
+}  // namespace detail
+
+// The masked-language-model loss of the CPU backend (src/backend/cpu/loss.cpp:149-215): rows whose index is -1 are
+// ignored, loss and gradient are averaged over the others (value 0 and zero gradient when every row is ignored).
+inline LossResult softmaxCrossEntropyMasked(const DeviceTensor& logits, const DeviceTensor& targetIndices) {
+    detail::requireSparse("softmaxCrossEntropyMasked", logits, targetIndices);
+    std::size_t rows = detail::rowsOf(logits), classes = detail::lastDim(logits);
+    if (rows > 0) detail::requireMaskedIds("softmaxCrossEntropyMasked", targetIndices, classes);
+    LossResult r{0.0F, DeviceTensor(logits.shape())};
+    DeviceTensor mean({1});
+    check(bf_hip_cross_entropy_masked(logits.data(), targetIndices.data(), r.grad.data(), mean.data(), rows, classes, 0, nullptr));
+    r.value = detail::readScalar(mean);
+    return r;
+}
+
 // "Accumulate" variants for the training loop: the gradient is returned, the SUM of this call's per-row
 // (per-element for MSE) losses is added on the device to lossAccumulator (one element, owned by the
 // caller); nothing is read back to the host.
@@ -85,6 +112,17 @@ inline DeviceTensor softmaxCrossEntropySparseAccumulate(const DeviceTensor& logi
     DeviceTensor grad(logits.shape());
     check(bf_hip_cross_entropy_sparse(logits.data(), targetIndices.data(), grad.data(), lossAccumulator.data(),
                                       detail::rowsOf(logits), detail::lastDim(logits), 1, nullptr));
+    return grad;
+}
+
+// Adds this call's MEAN over the rows that are not ignored (the value softmaxCrossEntropyMasked returns) to
+// lossAccumulator; indices are the caller's precondition, as above.
+inline DeviceTensor softmaxCrossEntropyMaskedAccumulate(const DeviceTensor& logits, const DeviceTensor& targetIndices,
+                                                         DeviceTensor& lossAccumulator) {
+    detail::requireSparse("softmaxCrossEntropyMaskedAccumulate", logits, targetIndices);
+    DeviceTensor grad(logits.shape());
+    check(bf_hip_cross_entropy_masked(logits.data(), targetIndices.data(), grad.data(), lossAccumulator.data(), detail::rowsOf(logits),
+                                      detail::lastDim(logits), 1, nullptr));
     return grad;
 }
 

@@ -29,11 +29,11 @@ struct Parameter {
     DeviceTensor grad;
 };
 
-enum class LayerKind { Linear, Silu, Relu, Gelu, RmsNorm, Softmax, Embedding, PositionalEmbedding, Attention, FeedForward };
+enum class LayerKind { Linear, Silu, Relu, Gelu, RmsNorm, Softmax, Embedding, PositionalEmbedding, Attention, FeedForward, BidirectionalAttention };
 
 struct LayerSpec {
     LayerKind kind;
-    std::size_t arg0 = 0;  // Linear: out features; Embedding: vocab; PositionalEmbedding: maxSeqLen; Attention: heads; FeedForward: hidden
+    std::size_t arg0 = 0;  // Linear: out features; Embedding: vocab; PositionalEmbedding: maxSeqLen; [Bidirectional]Attention: heads; FeedForward: hidden
     std::size_t arg1 = 0;  // Embedding: dim; FeedForward: activation (0 SiLU = reference, 1 GELU)
 };
 
@@ -65,12 +65,16 @@ public:
                     layer.params.push_back(makeParameter("positional_embedding" + id + ".table", {spec.arg0, features}));
                     break;
                 case LayerKind::Attention:
+                case LayerKind::BidirectionalAttention: {
+                    // same parameters for both, named after the op (src/backend/cpu/model.cpp:124-150)
+                    const std::string label = spec.kind == LayerKind::Attention ? "attention" : "bidirectional_attention";
                     require(spec.arg0 != 0 && features % spec.arg0 == 0,
-                            "hip::Model: 'attention#" + id + "' needs " + std::to_string(spec.arg0) + " heads to divide dim=" +
+                            "hip::Model: '" + label + "#" + id + "' needs " + std::to_string(spec.arg0) + " heads to divide dim=" +
                                 std::to_string(features));
                     for (const char* w : {".wq", ".wk", ".wv", ".wout"})
-                        layer.params.push_back(makeParameter("attention" + id + w, {features, features}));
+                        layer.params.push_back(makeParameter(label + id + w, {features, features}));
                     break;
+                }
                 case LayerKind::FeedForward:
                     layer.params.push_back(makeParameter("feedforward" + id + ".w1", {features, spec.arg0}));
                     layer.params.push_back(makeParameter("feedforward" + id + ".b1", {spec.arg0}));
@@ -148,6 +152,10 @@ public:
                                        : selfAttentionIncremental(current, layer.params[0].value, layer.params[1].value,
                                                                   layer.params[2].value, layer.params[3].value, s.arg0, layer.kvCache);
                     break;
+                case LayerKind::BidirectionalAttention:
+                    // src/backend/cpu/model.cpp:365-374: a layer that sees the whole sequence has no next token to generate
+                    throw std::invalid_argument("hip::Model::forwardIncremental: the pipeline contains 'bidirectional_attention', "
+                                                "which does not support incremental generation");
                 case LayerKind::FeedForward: {
                     Activation act = s.arg1 == 1 ? Activation::Gelu : Activation::Silu;
                     current = useBf16_ ? feedForwardBf16(current, layer.params[0].value, layer.params[1].value, layer.params[2].value,
@@ -225,6 +233,9 @@ private:
             case LayerKind::Attention:
                 return selfAttentionForwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
                                                   layer.params[3].value, s.arg0, useBf16_, layer.attnCache);
+            case LayerKind::BidirectionalAttention:
+                return bidirectionalSelfAttentionForwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                               layer.params[3].value, s.arg0, useBf16_, layer.attnCache);
             case LayerKind::FeedForward:
                 return feedForwardForwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
                                                 layer.params[3].value, useBf16_, layer.ffCache,
@@ -264,7 +275,8 @@ private:
                 accumulate(layer.params[0].grad, g.dTable);
                 return std::move(g.dInput);
             }
-            case LayerKind::Attention: {
+            case LayerKind::Attention:
+            case LayerKind::BidirectionalAttention: {   // the cache records which of the two the forward pass was
                 SelfAttentionGrad g = selfAttentionBackwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
                                                                   layer.params[3].value, s.arg0, layer.attnCache, grad, useBf16_);
                 accumulate(layer.params[0].grad, g.dWq);
@@ -306,9 +318,12 @@ private:
                     specs.push_back({LayerKind::PositionalEmbedding, static_cast<std::size_t>(op.positionalMaxSeqLen), 0});
                     break;
                 case ir::OpKind::Attention: specs.push_back({LayerKind::Attention, static_cast<std::size_t>(op.attentionNumHeads), 0}); break;
+                case ir::OpKind::BidirectionalAttention:
+                    specs.push_back({LayerKind::BidirectionalAttention, static_cast<std::size_t>(op.attentionNumHeads), 0});
+                    break;
                 case ir::OpKind::FeedForward: specs.push_back({LayerKind::FeedForward, static_cast<std::size_t>(op.feedForwardHiddenDim), 0}); break;
                 default:
-                    throw std::invalid_argument("hip::Model: 'bidirectional_attention' is not implemented on this backend");
+                    throw std::invalid_argument("hip::Model: operation '" + std::string(ir::opKindName(op.kind)) + "' is not implemented on this backend");
             }
         }
         return specs;
@@ -330,7 +345,8 @@ private:
                 case LayerKind::Linear: salts = linearSalts; break;
                 case LayerKind::Embedding: salts = embSalt; break;
                 case LayerKind::PositionalEmbedding: salts = posSalt; break;
-                case LayerKind::Attention: salts = attnSalts; break;
+                case LayerKind::Attention:
+                case LayerKind::BidirectionalAttention: salts = attnSalts; break;
                 case LayerKind::FeedForward: salts = ffSalts; break;
                 default: break;
             }

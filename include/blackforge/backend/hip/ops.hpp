@@ -247,6 +247,7 @@ struct SelfAttentionCache {
     DeviceTensor q, k, v;     // [batch, seq, dim]
     DeviceTensor attnOutput;  // [batch, seq, dim], before Wout
     DeviceTensor attnM, attnL;
+    bool causal = true;       // false: bidirectionalSelfAttention (every position sees the whole sequence)
 };
 
 namespace detail {
@@ -257,9 +258,10 @@ inline void requireAttention(const char* op, const DeviceTensor& input, std::siz
 // mode: 0 fp32, 1 bf16, 2 bf16 with cached weight images
 inline DeviceTensor selfAttentionForwardImpl(const char* op, const DeviceTensor& input, const DeviceTensor& wq,
                                               const DeviceTensor& wk, const DeviceTensor& wv, const DeviceTensor& wout,
-                                              std::size_t numHeads, int mode, SelfAttentionCache& cache) {
+                                              std::size_t numHeads, int mode, SelfAttentionCache& cache, bool causal = true) {
     requireAttention(op, input, numHeads);
     std::size_t batch = input.dim(0), seq = input.dim(1), dim = input.dim(2);
+    cache.causal = causal;
     float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
     cache.normedFlat = rmsnorm(input).reshaped({batch * seq, dim});
     if (mode != 0) {
@@ -277,7 +279,8 @@ inline DeviceTensor selfAttentionForwardImpl(const char* op, const DeviceTensor&
         cache.k = projection(cache.normedFlat, wk, mode, {batch, seq, dim});
         cache.v = projection(cache.normedFlat, wv, mode, {batch, seq, dim});
     }
-    FusedAttentionForwardResult attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, 0);
+    // query i sees keys j <= oldLen + i: an offset of seq makes every key visible, which is the bidirectional form
+    FusedAttentionForwardResult attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, causal ? 0 : seq);
     cache.attnOutput = std::move(attn.output);
     cache.attnM = std::move(attn.m);
     cache.attnL = std::move(attn.l);
@@ -296,6 +299,24 @@ inline DeviceTensor selfAttention(const DeviceTensor& input, const DeviceTensor&
                                    const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads) {
     SelfAttentionCache cache;
     return detail::selfAttentionForwardImpl("selfAttention", input, wq, wk, wv, wout, numHeads, 0, cache);
+}
+// The same block without the causal mask (the CPU backend's bidirectionalSelfAttention, src/backend/cpu/ops.cpp:504-507;
+// the CUDA backend refuses the op, model.cu:151-160).
+inline DeviceTensor bidirectionalSelfAttentionForwardCached(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                             const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                             bool useBf16, SelfAttentionCache& cache) {
+    return detail::selfAttentionForwardImpl("bidirectionalSelfAttentionForwardCached", input, wq, wk, wv, wout, numHeads, useBf16 ? 2 : 0,
+                                            cache, false);
+}
+inline DeviceTensor bidirectionalSelfAttention(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads) {
+    SelfAttentionCache cache;
+    return detail::selfAttentionForwardImpl("bidirectionalSelfAttention", input, wq, wk, wv, wout, numHeads, 0, cache, false);
+}
+inline DeviceTensor bidirectionalSelfAttentionBf16(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                    const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads) {
+    SelfAttentionCache cache;
+    return detail::selfAttentionForwardImpl("bidirectionalSelfAttentionBf16", input, wq, wk, wv, wout, numHeads, 1, cache, false);
 }
 inline DeviceTensor selfAttentionBf16(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
                                        const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads) {

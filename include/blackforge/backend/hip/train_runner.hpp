@@ -30,7 +30,7 @@ struct TrainRunResult {
 };
 
 struct TrainOptions {
-    std::string loss = "mse";          // "mse", "cross_entropy", "cross_entropy_sparse"
+    std::string loss = "mse";          // "mse", "cross_entropy", "cross_entropy_sparse", "cross_entropy_masked"
     std::string optimizer = "adamw";   // "sgd", anything else = AdamW with the reference defaults (train_runner.cu:168-173)
     long long epochs = 1;
     std::size_t batchSize = 1;
@@ -58,12 +58,23 @@ inline void validateHostIndexRange(const runtime::Tensor& host, std::size_t boun
         }
     }
 }
+// src/backend/cpu/loss.cpp:171-178: -1 marks a row to ignore, every other index must lie in [0, bound)
+inline void validateHostMaskedIndexRange(const runtime::Tensor& host, std::size_t bound, const char* label) {
+    for (std::size_t i = 0; i < host.elementCount(); ++i) {
+        const long long index = static_cast<long long>(std::lround(host.at(i)));
+        if (index != -1 && (index < 0 || static_cast<std::size_t>(index) >= bound)) {
+            throw std::invalid_argument(std::string(label) + ": class index " + std::to_string(index) + " outside [0, " + std::to_string(bound) +
+                                        ") (or -1 to ignore)");
+        }
+    }
+}
 }  // namespace detail
 
 // DatasetT: HostDataset, or blackforge::data::Dataset inside a BlackForge build (same batch/shuffle/numExamples members).
 template <typename DatasetT>
 TrainRunResult runTraining(Model& model, DatasetT& dataset, const TrainOptions& options, std::ostream* progressOutput = nullptr) {
     const bool sparse = options.loss == "cross_entropy_sparse", dense = options.loss == "cross_entropy";
+    const bool maskedLoss = options.loss == "cross_entropy_masked";   // cpu/train_runner.cpp:132-133; the CUDA runner has no such loss
     const std::optional<std::size_t> vocab = model.firstLayerEmbeddingVocabSize();
     if (!options.fromCheckpointPath.empty()) {
         loadCheckpoint(model, options.fromCheckpointPath);
@@ -98,11 +109,15 @@ TrainRunResult runTraining(Model& model, DatasetT& dataset, const TrainOptions& 
             model.zeroGrad();
             DeviceTensor output = model.forward(input, vocab.has_value());
             if (sparse) detail::validateHostIndexRange(batch.target, output.shape().back(), "softmaxCrossEntropySparse");
+            if (maskedLoss) detail::validateHostMaskedIndexRange(batch.target, output.shape().back(), "softmaxCrossEntropyMasked");
             DeviceTensor target = DeviceTensor::fromHost(batch.target);
-            lossDivisor += (sparse || dense) ? output.elementCount() / output.shape().back() : output.elementCount();
-            DeviceTensor grad = sparse  ? softmaxCrossEntropySparseAccumulate(output, target, lossAccumulator)
-                                : dense ? softmaxCrossEntropyAccumulate(output, target, lossAccumulator)
-                                        : meanSquaredErrorAccumulate(output, target, lossAccumulator);
+            // the masked loss adds each batch's MEAN (its divisor, the rows not ignored, differs from batch to batch),
+            // so the epoch's figure is the mean of the batch means, as in cpu/train_runner.cpp:184-194
+            lossDivisor += maskedLoss ? 1 : (sparse || dense) ? output.elementCount() / output.shape().back() : output.elementCount();
+            DeviceTensor grad = sparse       ? softmaxCrossEntropySparseAccumulate(output, target, lossAccumulator)
+                                : maskedLoss ? softmaxCrossEntropyMaskedAccumulate(output, target, lossAccumulator)
+                                : dense      ? softmaxCrossEntropyAccumulate(output, target, lossAccumulator)
+                                             : meanSquaredErrorAccumulate(output, target, lossAccumulator);
             model.backward(grad, vocab.has_value());
             optimizer->step(model.parameters());
         }

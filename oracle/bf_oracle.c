@@ -679,6 +679,40 @@ int bfo_softmax_cross_entropy_sparse(const float* logits, const float* targetIdx
     return BFO_OK;
 }
 
+/* loss.cpp:149-215.  A row whose index rounds to -1 is skipped; gradient rows are first written unnormalised
+ * (float(prob) - t) and then multiplied by 1.0f / numMaskedRows in float (loss.cpp:194-213). */
+int bfo_softmax_cross_entropy_masked(const float* logits, const float* targetIdx, float* grad, float* value,
+                                     size_t rows, size_t classes) {
+    double* probs = (double*)malloc((classes ? classes : 1) * sizeof(double));
+    double totalLoss = 0.0;
+    size_t numMaskedRows = 0;
+    for (size_t i = 0; i < rows * classes; ++i) grad[i] = 0.0f;
+    for (size_t b = 0; b < rows; ++b) {
+        long long cls = (long long)lroundf(targetIdx[b]);
+        if (cls == -1) continue;
+        if (cls < 0 || (size_t)cls >= classes) {
+            free(probs);
+            return BFO_INVALID_ARGUMENT;
+        }
+        ++numMaskedRows;
+        row_probabilities(logits + b * classes, probs, classes);
+        double p = probs[cls] > 1e-12 ? probs[cls] : 1e-12;
+        totalLoss += -log(p);
+        for (size_t c = 0; c < classes; ++c) {
+            float t = (c == (size_t)cls) ? 1.0f : 0.0f;
+            grad[b * classes + c] = (float)probs[c] - t;
+        }
+    }
+    *value = 0.0f;
+    if (numMaskedRows > 0) {
+        *value = (float)(totalLoss / (double)numMaskedRows);
+        float invMaskedRows = 1.0f / (float)numMaskedRows;
+        for (size_t i = 0; i < rows * classes; ++i) grad[i] *= invMaskedRows;
+    }
+    free(probs);
+    return BFO_OK;
+}
+
 /* ------------------------------------------------------------------------------------------- */
 /* optimizers, quantisation, argmax                                                              */
 /* ------------------------------------------------------------------------------------------- */
@@ -822,12 +856,13 @@ bfo_model* bfo_model_create(int numLayers, const int* kinds, const long long* ar
                 layer->params[0] = add_param(model, base, "table", (size_t)layer->arg0, features);
                 break;
             }
-            case BFO_ATTENTION: {
+            case BFO_ATTENTION:
+            case BFO_BIDIRECTIONAL_ATTENTION: {   /* model.cpp:124-150: same parameters, named after the op */
                 if (layer->arg0 <= 0 || features % (size_t)layer->arg0 != 0) {
                     bfo_model_destroy(model);
                     return NULL;
                 }
-                snprintf(base, sizeof(base), "attention%d", outputId);
+                snprintf(base, sizeof(base), layer->kind == BFO_ATTENTION ? "attention%d" : "bidirectional_attention%d", outputId);
                 layer->params[0] = add_param(model, base, "wq", features, features);
                 layer->params[1] = add_param(model, base, "wk", features, features);
                 layer->params[2] = add_param(model, base, "wv", features, features);
@@ -940,12 +975,13 @@ int bfo_model_forward(bfo_model* model, const float* input, int rank, const size
                                                          curShape[2], (size_t)layer->arg0, 0);
                 break;
             }
-            case BFO_ATTENTION: {
+            case BFO_ATTENTION:
+            case BFO_BIDIRECTIONAL_ATTENTION: {   /* model.cpp:218-226 */
                 if (curRank != 3) { status = BFO_INVALID_ARGUMENT; break; }
                 next = alloc_floats(count);
                 status = bfo_self_attention(current, pv(model, layer, 0), pv(model, layer, 1), pv(model, layer, 2),
                                             pv(model, layer, 3), next, curShape[0], curShape[1], curShape[2],
-                                            (size_t)layer->arg0, 1);
+                                            (size_t)layer->arg0, layer->kind == BFO_ATTENTION);
                 break;
             }
             case BFO_FEEDFORWARD: {
@@ -1021,7 +1057,8 @@ int bfo_model_backward(bfo_model* model, const float* outputGrad, size_t count) 
                 memcpy(next, grad, inCount * sizeof(float));
                 break;
             }
-            case BFO_ATTENTION: {
+            case BFO_ATTENTION:
+            case BFO_BIDIRECTIONAL_ATTENTION: {   /* model.cpp:310-325 */
                 size_t dim = inShape[2];
                 float* dWq = alloc_floats(dim * dim);
                 float* dWk = alloc_floats(dim * dim);
@@ -1029,7 +1066,8 @@ int bfo_model_backward(bfo_model* model, const float* outputGrad, size_t count) 
                 float* dWo = alloc_floats(dim * dim);
                 status = bfo_self_attention_backward(layer->cachedInput, pv(model, layer, 0), pv(model, layer, 1),
                                                      pv(model, layer, 2), pv(model, layer, 3), grad, next, dWq, dWk,
-                                                     dWv, dWo, inShape[0], inShape[1], dim, (size_t)layer->arg0, 1);
+                                                     dWv, dWo, inShape[0], inShape[1], dim, (size_t)layer->arg0,
+                                                     layer->kind == BFO_ATTENTION);
                 accumulate(pg(model, layer, 0), dWq, dim * dim);
                 accumulate(pg(model, layer, 1), dWk, dim * dim);
                 accumulate(pg(model, layer, 2), dWv, dim * dim);
@@ -1264,7 +1302,7 @@ int bfo_model_load_checkpoint(bfo_model* model, const char* path) {
 /* cpu::runTraining (cpu/train_runner.cpp:38-211) for a model built from a layer list: per epoch, shuffle with the
  * epoch number as seed, optional cosine learning rate, floor(examples / batch) batches of zeroGrad, forward, loss,
  * backward, optimizer step; the epoch loss is the mean of the batch losses (accumulated in double).
- * lossKind: 0 mse, 1 cross_entropy, 2 cross_entropy_sparse.  optimizerKind: 0 sgd, 1 adamw (reference defaults).
+ * lossKind: 0 mse, 1 cross_entropy, 2 cross_entropy_sparse, 3 cross_entropy_masked.  optimizerKind: 0 sgd, 1 adamw (reference defaults).
  * The model starts from `fromCheckpoint` when that is a non-empty path, else from its current values. */
 int bfo_model_run_training(bfo_model* model, const char* datasetPath, int lossKind, int optimizerKind, long long epochs,
                            size_t batchSize, float learningRate, int cosineSchedule, const char* fromCheckpoint,
@@ -1311,7 +1349,8 @@ int bfo_model_run_training(bfo_model* model, const char* datasetPath, int lossKi
             float value = 0.0f;
             if (lossKind == 0) status = bfo_mean_squared_error(out, target, grad, &value, outCount);
             else if (lossKind == 1) status = bfo_softmax_cross_entropy(out, target, grad, &value, rows, classes);
-            else status = bfo_softmax_cross_entropy_sparse(out, target, grad, &value, rows, classes);
+            else if (lossKind == 2) status = bfo_softmax_cross_entropy_sparse(out, target, grad, &value, rows, classes);
+            else status = bfo_softmax_cross_entropy_masked(out, target, grad, &value, rows, classes);
             if (status != BFO_OK) break;
             status = bfo_model_backward(model, grad, outCount);
             if (status != BFO_OK) break;

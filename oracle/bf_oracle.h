@@ -101,6 +101,9 @@ int bfo_softmax_cross_entropy(const float* logits, const float* target, float* g
                               size_t classes);                                                   /* loss.cpp:30 */
 int bfo_softmax_cross_entropy_sparse(const float* logits, const float* targetIdx, float* grad, float* value,
                                      size_t rows, size_t classes);                               /* loss.cpp:84 */
+/* Index -1 = row ignored; loss and gradient are means over the other rows (0 when there is none). */
+int bfo_softmax_cross_entropy_masked(const float* logits, const float* targetIdx, float* grad, float* value,
+                                     size_t rows, size_t classes);                               /* loss.cpp:149 */
 
 /* ---- optimizers: src/backend/cpu/optimizer.cpp ---- */
 int bfo_sgd_step(float* param, const float* grad, size_t n, float lr);                           /* optimizer.cpp:7 */
@@ -124,7 +127,8 @@ enum {
     BFO_EMBEDDING = 6,   /* arg0 = vocab, arg1 = dim */
     BFO_POSITIONAL = 7,  /* arg0 = max sequence length */
     BFO_ATTENTION = 8,   /* arg0 = heads */
-    BFO_FEEDFORWARD = 9  /* arg0 = hidden, arg1 = activation (0 SiLU, 1 GELU) */
+    BFO_FEEDFORWARD = 9, /* arg0 = hidden, arg1 = activation (0 SiLU, 1 GELU) */
+    BFO_BIDIRECTIONAL_ATTENTION = 10   /* arg0 = heads; the attention block without the causal mask (ops.cpp:504) */
 };
 typedef struct bfo_model bfo_model;
 /* inputFeatures: last dimension of the model input (ignored when the first layer is an embedding). */
@@ -155,7 +159,7 @@ float bfo_cosine_learning_rate(long long epoch, long long totalEpochs, float bas
 int bfo_model_save_checkpoint(const bfo_model* model, const char* path);
 int bfo_model_load_checkpoint(bfo_model* model, const char* path);
 /* cpu::runTraining (train_runner.cpp:38-211) over a BFDATA1 dataset file (dataset.cpp:133-184).  lossKind: 0 mse,
- * 1 cross_entropy, 2 cross_entropy_sparse; optimizerKind: 0 sgd, 1 adamw; cosineSchedule: 0/1.  The run starts from
+ * 1 cross_entropy, 2 cross_entropy_sparse, 3 cross_entropy_masked; optimizerKind: 0 sgd, 1 adamw; cosineSchedule: 0/1.  The run starts from
  * `fromCheckpoint` (required: the reference's random initialisation is not restated) and writes `saveCheckpoint`
  * when that is a non-empty path.  epochLosses receives `epochs` values. */
 int bfo_model_run_training(bfo_model* model, const char* datasetPath, int lossKind, int optimizerKind, long long epochs,

@@ -22,7 +22,7 @@ REF_LIB = os.path.join(_HERE, "_ref", "libbf_ref.so")
 _f32p = ctypes.POINTER(ctypes.c_float)
 _sz = ctypes.c_size_t
 
-LINEAR, SILU, RELU, GELU, RMSNORM, SOFTMAX, EMBEDDING, POSITIONAL, ATTENTION, FEEDFORWARD = range(10)
+LINEAR, SILU, RELU, GELU, RMSNORM, SOFTMAX, EMBEDDING, POSITIONAL, ATTENTION, FEEDFORWARD, BIDIRECTIONAL_ATTENTION = range(11)
 
 
 class OracleInvalidArgument(ValueError):
@@ -330,6 +330,17 @@ class Oracle:
                    logits.size // logits.shape[-1], logits.shape[-1])
         return value.value, grad
 
+    def softmaxCrossEntropyMasked(self, logits, target_idx):
+        """loss.cpp:149-215: index -1 = row ignored; means over the other rows."""
+        logits, target_idx = _f(logits), _f(target_idx)
+        if logits.ndim < 2 or target_idx.size != logits.size // logits.shape[-1]:
+            raise OracleInvalidArgument("softmaxCrossEntropyMasked: shapes")
+        grad = np.empty_like(logits)
+        value = ctypes.c_float()
+        self._call("bfo_softmax_cross_entropy_masked", logits, target_idx, grad, ctypes.byref(value),
+                   logits.size // logits.shape[-1], logits.shape[-1])
+        return value.value, grad
+
     # -- optimizers / misc --------------------------------------------------------------------
     def sgdStep(self, param, grad, lr):
         param = _f(param).copy()
@@ -459,7 +470,7 @@ class OracleModel:
         """cpu::runTraining.  loss: 'mse' | 'cross_entropy' | 'cross_entropy_sparse'; optimizer: 'sgd' | 'adamw'.
         Returns the list of epoch losses; the trained values are left in this model."""
         losses = (ctypes.c_double * max(epochs, 1))()
-        st = self.o.lib.bfo_model_run_training(self.handle, dataset_path.encode(), {"mse": 0, "cross_entropy": 1, "cross_entropy_sparse": 2}[loss],
+        st = self.o.lib.bfo_model_run_training(self.handle, dataset_path.encode(), {"mse": 0, "cross_entropy": 1, "cross_entropy_sparse": 2, "cross_entropy_masked": 3}[loss],
                                                {"sgd": 0, "adamw": 1}[optimizer], ctypes.c_longlong(epochs), _sz(batch_size),
                                                ctypes.c_float(lr), int(bool(cosine)), from_checkpoint.encode(), save_checkpoint.encode(),
                                                losses)

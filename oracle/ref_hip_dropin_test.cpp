@@ -76,7 +76,8 @@ static ir::ModelIR makeModel(const std::string& name, const std::vector<LayerDes
             case ir::OpKind::Linear: op.linearOutFeatures = layers[i].a0; features = layers[i].a0; break;
             case ir::OpKind::Embedding: op.embeddingVocabSize = layers[i].a0; op.embeddingDim = layers[i].a1; features = layers[i].a1; break;
             case ir::OpKind::PositionalEmbedding: op.positionalMaxSeqLen = layers[i].a0; break;
-            case ir::OpKind::Attention: op.attentionNumHeads = layers[i].a0; break;
+            case ir::OpKind::Attention:
+            case ir::OpKind::BidirectionalAttention: op.attentionNumHeads = layers[i].a0; break;
             case ir::OpKind::FeedForward: op.feedForwardHiddenDim = layers[i].a0; break;
             default: break;
         }
@@ -118,9 +119,14 @@ int main(int argc, char** argv) {
     ir::ModelIR mlp = makeModel("mlp", {{ir::OpKind::Linear, 24, 0}, {ir::OpKind::Silu, 0, 0}, {ir::OpKind::Linear, 24, 0}, {ir::OpKind::Gelu, 0, 0},
                                        {ir::OpKind::Linear, 5, 0}, {ir::OpKind::Softmax, 0, 0}},
                                 {batchDim, lit(10)});
+    // a masked language model: the CPU backend runs it, the CUDA backend refuses it (model.cu:151-160)
+    ir::ModelIR mlm = makeModel("tiny_mlm",
+                                {{ir::OpKind::Embedding, 48, 32}, {ir::OpKind::PositionalEmbedding, 12, 0}, {ir::OpKind::BidirectionalAttention, 4, 0},
+                                 {ir::OpKind::FeedForward, 64, 0}, {ir::OpKind::Linear, 48, 0}},
+                                {batchDim, lit(12)});
     try {
         // 1. executors
-        for (const ir::ModelIR* m : {&lm, &mlp}) {
+        for (const ir::ModelIR* m : {&lm, &mlp, &mlm}) {
             cpu::Executor cx(42);
             hip::Executor hx(42);
             bf::runtime::Tensor in = cx.makeSyntheticInput(*m, 6), inHip = hx.makeSyntheticInput(*m, 6);
@@ -154,11 +160,15 @@ int main(int argc, char** argv) {
             for (int j = 0; j < 5; ++j) { y[i * 5 + j] = float(next() % 100 + 1); sum += y[i * 5 + j]; }
             for (int j = 0; j < 5; ++j) y[i * 5 + j] /= sum;
         }
+        std::vector<float> maskedTgt(ids.size());
+        for (std::size_t i = 0; i < ids.size(); ++i) maskedTgt[i] = next() % 4 == 0 ? ids[i] : -1.0f;   // a quarter of the positions count
+        bf::data::saveDataset(tmp + "/dropin_mlm.bfdata", {12}, {12}, ids, maskedTgt, 30);
         bf::data::saveDataset(tmp + "/dropin_lm.bfdata", {12}, {12}, ids, tgt, 30);
         bf::data::saveDataset(tmp + "/dropin_mlp.bfdata", {10}, {5}, x, y, 40);
-        std::vector<Run> runs = {{&lm, "cross_entropy_sparse", "adamw", 3, 5, 5e-3, true}, {&mlp, "mse", "sgd", 3, 8, 0.1, false}};
+        std::vector<Run> runs = {{&lm, "cross_entropy_sparse", "adamw", 3, 5, 5e-3, true}, {&mlp, "mse", "sgd", 3, 8, 0.1, false},
+                                 {&mlm, "cross_entropy_masked", "adamw", 3, 5, 5e-3, false}};
         for (const Run& r : runs) {
-            const std::string data = tmp + (r.model == &lm ? "/dropin_lm.bfdata" : "/dropin_mlp.bfdata");
+            const std::string data = tmp + (r.model == &lm ? "/dropin_lm.bfdata" : r.model == &mlm ? "/dropin_mlm.bfdata" : "/dropin_mlp.bfdata");
             ast::Program program = makeProgram(r.model->name, data, r.loss, r.optimizer, r.epochs, r.batch, r.lr, r.cosine);
             ir::Module module;
             module.models.push_back(*r.model);

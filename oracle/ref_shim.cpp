@@ -346,6 +346,15 @@ int bfo_softmax_cross_entropy_sparse(const float* logits, const float* targetIdx
     });
 }
 
+int bfo_softmax_cross_entropy_masked(const float* logits, const float* targetIdx, float* grad, float* value,
+                                     size_t rows, size_t classes) {
+    return guarded([&] {
+        cpu::LossResult r = cpu::softmaxCrossEntropyMasked(wrap(logits, {rows, classes}), wrap(targetIdx, {rows}));
+        *value = r.value;
+        store(r.grad, grad);
+    });
+}
+
 int bfo_sgd_step(float* param, const float* grad, size_t n, float lr) {
     return guarded([&] {
         cpu::Parameter p{"p", wrap(param, {n}), wrap(grad, {n})};
@@ -432,6 +441,7 @@ bfo_model* bfo_model_create(int numLayers, const int* kinds, const long long* ar
                     break;
                 case BFO_POSITIONAL: op.kind = ir::OpKind::PositionalEmbedding; op.positionalMaxSeqLen = arg0[i]; break;
                 case BFO_ATTENTION: op.kind = ir::OpKind::Attention; op.attentionNumHeads = arg0[i]; break;
+                case BFO_BIDIRECTIONAL_ATTENTION: op.kind = ir::OpKind::BidirectionalAttention; op.attentionNumHeads = arg0[i]; break;
                 case BFO_FEEDFORWARD:
                     if (a1 != 0) return nullptr;  // the reference's feedforward block is SiLU only
                     op.kind = ir::OpKind::FeedForward; op.feedForwardHiddenDim = arg0[i];
@@ -586,8 +596,8 @@ int bfo_model_run_training(bfo_model* model, const char* datasetPath, int lossKi
         ast::TrainDecl train;
         train.fields.push_back(ast::TrainModelField{model->irModel.name, {}});
         train.fields.push_back(ast::TrainDatasetField{"data", {}});
-        const char* lossNames[3] = {"mse", "cross_entropy", "cross_entropy_sparse"};
-        if (lossKind < 0 || lossKind > 2) return BFO_INVALID_ARGUMENT;
+        const char* lossNames[4] = {"mse", "cross_entropy", "cross_entropy_sparse", "cross_entropy_masked"};
+        if (lossKind < 0 || lossKind > 3) return BFO_INVALID_ARGUMENT;
         train.fields.push_back(ast::TrainLossField{lossNames[lossKind], {}});
         train.fields.push_back(ast::TrainOptimizerField{optimizerKind == 0 ? "sgd" : "adamw", {}});
         train.fields.push_back(ast::TrainEpochsField{epochs, {}});

@@ -257,6 +257,34 @@ int main() {
         EXPECT_TRUE(idx == 1);
     });
 
+    run("Model: masked-language-model pipeline (bidirectional attention, masked loss) trains; no incremental generation", [] {
+        using hip::LayerKind;
+        hip::Model model("mlm", {{LayerKind::Embedding, 16, 8}, {LayerKind::PositionalEmbedding, 4, 0}, {LayerKind::BidirectionalAttention, 2, 0},
+                                 {LayerKind::FeedForward, 16, 0}, {LayerKind::Linear, 16, 0}}, 0, false);
+        unsigned state = 777;
+        for (hip::Parameter* p : model.parameters()) {
+            std::vector<float> init(p->value.elementCount());
+            for (float& v : init) { state = state * 1664525u + 1013904223u; v = (float(state >> 8) / float(1u << 24) - 0.5F) * 0.2F; }
+            p->value = DeviceTensor::fromHost(Tensor(p->value.shape(), init));
+        }
+        EXPECT_TRUE(model.parameters()[2]->name == "bidirectional_attention3.wq");
+        DeviceTensor ids = dev({2, 4}, {1, 2, 3, 4, 5, 6, 7, 8});
+        DeviceTensor targets = dev({8}, {-1, 2, -1, -1, 5, -1, -1, 8});   // loss over three of the eight positions
+        hip::AdamW opt(1e-2F);
+        float first = 0, last = 0;
+        for (int step = 0; step < 30; ++step) {
+            model.zeroGrad();
+            hip::LossResult loss = hip::softmaxCrossEntropyMasked(model.forward(ids), targets);
+            model.backward(loss.grad);
+            opt.step(model.parameters());
+            if (step == 0) first = loss.value;
+            last = loss.value;
+        }
+        EXPECT_TRUE(last < first * 0.8F);
+        EXPECT_THROW_INVALID(hip::softmaxCrossEntropyMasked(model.forward(ids), dev({8}, {-2, 2, -1, -1, 5, -1, -1, 8})));
+        EXPECT_THROW_INVALID((void)model.forwardIncremental(dev({1, 1}, {3})));   // src/backend/cpu/model.cpp:365-374
+    });
+
     std::printf("%d checks, %d failures\n", g_checks, g_failures);
     return g_failures == 0 ? 0 : 1;
 }

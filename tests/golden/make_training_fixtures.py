@@ -2,7 +2,7 @@
 
 Run in a container that has the reference tree (oracle/_ref/libbf_ref.so is built from it by oracle/Makefile):
     python tests/golden/make_training_fixtures.py
-Data only: two small BFDATA1 datasets (seeded random numbers), the BFCKPT1 checkpoint of each model as the reference
+Data only: a few small BFDATA1 datasets (seeded random numbers), the BFCKPT1 checkpoint of each model as the reference
 initialises it (seed 42), the checkpoint the reference's own cpu::runTraining leaves after training on them, its
 epoch losses, and the permutations of data::Dataset::shuffle for a few sizes and seeds.
 """
@@ -24,6 +24,9 @@ RUNS = {
                  "cross_entropy_sparse", "adamw", 3, 4, 1e-2, True),
     "train_mlp": ([(bfo.LINEAR, 16), (bfo.SILU,), (bfo.LINEAR, 4)], 8, "mse", "sgd", 4, 5, 0.05, False),
     "train_dense": ([(bfo.LINEAR, 12), (bfo.RELU,), (bfo.LINEAR, 6)], 8, "cross_entropy", "adamw", 2, 6, 5e-3, True),
+    # masked language model: no causal mask, loss over the masked positions only (targets -1 elsewhere)
+    "train_mlm": ([(bfo.EMBEDDING, 32, 16), (bfo.POSITIONAL, 8), (bfo.BIDIRECTIONAL_ATTENTION, 2), (bfo.FEEDFORWARD, 32, 0),
+                   (bfo.LINEAR, 32)], 0, "cross_entropy_masked", "adamw", 3, 4, 1e-2, False),
 }
 SHUFFLES = [(n, seed) for n in (2, 3, 5, 17, 24, 100) for seed in (1, 2, 3)]
 
@@ -34,7 +37,10 @@ def datasets(rng):
     xd = rng.standard_normal((18, 8)).astype(f32)
     yd = rng.random((18, 6)).astype(f32)
     yd /= yd.sum(-1, keepdims=True)
-    return {"train_lm": (ids, tgt), "train_mlp": (x, y), "train_dense": (xd, yd)}
+    mlm_ids = rng.integers(0, 32, (24, 8)).astype(f32)
+    mlm_tgt = np.where(rng.random((24, 8)) < 0.3, mlm_ids, f32(-1.0)).astype(f32)
+    mlm_tgt[5] = -1.0   # an example with nothing masked
+    return {"train_lm": (ids, tgt), "train_mlp": (x, y), "train_dense": (xd, yd), "train_mlm": (mlm_ids, mlm_tgt)}
 
 
 def main():

@@ -52,6 +52,33 @@ def test_attention_core_matches_the_oracle(hip, oracle, rng, batch, heads, new_l
         assert_close(got, exp, what=f"{name} case {(batch, heads, new_len, old_len, hd)}", scale=sc[name])
 
 
+@pytest.mark.parametrize("batch,heads,new_len,total,hd", [(1, 2, 3, 3, 2), (2, 2, 70, 70, 32), (1, 3, 129, 129, 64), (1, 1, 40, 200, 128), (2, 1, 130, 37, 16)])
+@pytest.mark.parametrize("route", ["hand-over", "recompute"])
+def test_attention_without_causal_mask(hip, oracle, rng, batch, heads, new_len, total, hd, route):
+    """An offset oldLen >= totalLen - 1 makes every key visible to every query: the bidirectional form, through the
+    same kernels (also with more or fewer keys than queries)."""
+    dim = heads * hd
+    q, k, v, go = r(rng, batch, new_len, dim), r(rng, batch, total, dim), r(rng, batch, total, dim), r(rng, batch, new_len, dim)
+    scale = float(f32(1.0) / np.sqrt(f32(hd)))
+    hip.capi.call("bf_hip_attention_set_workspace_limit", 0 if route == "recompute" else 2 ** 64 - 1)
+    try:
+        o, m, l, dq, dk, dv = run_gpu(hip, q, k, v, go, heads, scale, total)
+    finally:
+        hip.capi.call("bf_hip_attention_set_workspace_limit", 2 ** 64 - 1)
+    eo, em, el = oracle.attentionCoreForward(q, k, v, heads, scale, total)
+    edq, edk, edv = oracle.attentionCoreBackward(go, q, k, v, heads, scale, total)
+    # textbook softmax(QK^T)V in float64 pins what "no mask" means independently of the oracle's oldLen handling
+    split = lambda t, n: t.reshape(batch, n, heads, hd).transpose(0, 2, 1, 3).astype(np.float64)
+    S = np.einsum("bhid,bhjd->bhij", split(q, new_len), split(k, total)) * scale
+    P = np.exp(S - S.max(-1, keepdims=True))
+    P /= P.sum(-1, keepdims=True)
+    textbook = np.einsum("bhij,bhjd->bhid", P, split(v, total)).transpose(0, 2, 1, 3).reshape(batch, new_len, dim)
+    assert_close(eo, textbook.astype(f32), what="oracle vs textbook")
+    sc = grad_scales(q, k, v, go, scale)
+    for got, exp, name in ((o, eo, "O"), (m, em, "m"), (l, el, "l"), (dq, edq, "dQ"), (dk, edk, "dK"), (dv, edv, "dV")):
+        assert_close(got, exp, what=f"{name} non-causal {(batch, heads, new_len, total, hd)} {route}", scale=sc[name])
+
+
 @pytest.fixture
 def recompute_route(hip):
     """Workspace limit 0: bf_hip_attention_backward recomputes S and dP in the dQ kernel instead of reading dS back."""

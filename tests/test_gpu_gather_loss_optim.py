@@ -91,6 +91,51 @@ def test_cross_entropy(hip, oracle, rng, rows, classes):
         assert_close(res.grad.toHost(), eg, what="dense CE grad")
 
 
+@pytest.mark.parametrize("rows,classes,keep", [(1, 2, 1.0), (7, 13, 0.5), (512, 256, 0.15), (33, 1000, 0.3), (6, 32000, 0.5), (4, 50257, 0.5),
+                                               (2, 70001, 1.0), (9, 40, 0.0)])
+def test_masked_cross_entropy(hip, oracle, rng, rows, classes, keep):
+    """softmaxCrossEntropyMasked: rows with index -1 are ignored, means over the others (cpu loss.cpp:149-215)."""
+    D, ops = hip.DeviceTensor, hip.ops
+    logits = r(rng, rows, classes, scale=3)
+    idx = np.where(rng.random(rows) < keep, rng.integers(0, classes, rows), -1).astype(f32)
+    res = ops.softmaxCrossEntropyMasked(D.fromHost(logits), D.fromHost(idx))
+    ev, eg = oracle.softmaxCrossEntropyMasked(logits, idx)
+    assert abs(res.value - ev) <= 1e-4 * abs(ev) + 1e-6
+    got = res.grad.toHost()
+    assert_close(got, eg, what="masked CE grad")
+    assert not got[idx == -1].any(), "ignored rows must have an exactly zero gradient"
+    if keep == 0.0:
+        assert res.value == 0.0 and not got.any()
+    # accumulate form: adds the mean of each call
+    acc = D.zeros((1,))
+    for _ in range(3):
+        g = ops.softmaxCrossEntropyMaskedAccumulate(D.fromHost(logits), D.fromHost(idx), acc)
+    assert_close(g.toHost(), eg, what="masked CE grad (accumulate)")
+    assert abs(acc.toHost()[0] - 3 * ev) <= 1e-4 * 3 * abs(ev) + 1e-6
+
+
+def test_masked_cross_entropy_reference_cases(hip):
+    """tests/backend/cpu/loss_tests.cpp:142-196."""
+    D, ops = hip.DeviceTensor, hip.ops
+    logits = np.array([[0.5, -1.2, 0.3], [2.0, 0.1, -0.5]], f32)
+    masked = ops.softmaxCrossEntropyMasked(D.fromHost(logits), D.fromHost(np.array([1, 0], f32)))
+    sparse = ops.softmaxCrossEntropySparse(D.fromHost(logits), D.fromHost(np.array([1, 0], f32)))
+    assert abs(masked.value - sparse.value) <= 1e-6
+    np.testing.assert_allclose(masked.grad.toHost(), sparse.grad.toHost(), atol=1e-6)
+    logits = np.array([[1, 2, 3], [0.5, -1.0, 0.2], [-0.3, 0.1, 0.4]], f32)
+    masked = ops.softmaxCrossEntropyMasked(D.fromHost(logits), D.fromHost(np.array([-1, 2, -1], f32)))
+    single = ops.softmaxCrossEntropySparse(D.fromHost(logits[1:2]), D.fromHost(np.array([2], f32)))
+    g = masked.grad.toHost()
+    assert not g[0].any() and not g[2].any()
+    assert abs(masked.value - single.value) <= 1e-5
+    none = ops.softmaxCrossEntropyMasked(D.fromHost(logits[:2]), D.fromHost(np.array([-1, -1], f32)))
+    assert none.value == 0.0 and not none.grad.toHost().any()
+    with pytest.raises(ValueError):
+        ops.softmaxCrossEntropyMasked(D.fromHost(np.array([[0.1, 0.2, 0.3]], f32)), D.fromHost(np.array([7], f32)))
+    with pytest.raises(ValueError):
+        ops.softmaxCrossEntropyMasked(D.fromHost(np.array([[0.1, 0.2, 0.3]], f32)), D.fromHost(np.array([-2], f32)))
+
+
 def test_loss_literals_errors_and_accumulate(hip, oracle, rng):
     """tests/backend/cpu/loss_tests.cpp:10-16,51-69,115-140; cuda/loss_tests.cu:124-130."""
     import math

@@ -67,6 +67,78 @@ def test_blocks_against_oracle(hip, oracle, rng, batch, seq, dim, heads, hidden,
         assert_close(got.toHost(), e, what="feedForwardBackward." + n, scale=float(np.abs(e).max()) * 0.1)
 
 
+@pytest.mark.parametrize("batch,seq,dim,heads", [(2, 9, 12, 3), (4, 64, 128, 4), (1, 130, 64, 2), (1, 200, 256, 2)])
+def test_bidirectional_attention_block(hip, oracle, rng, batch, seq, dim, heads):
+    """bidirectionalSelfAttention and its backward (cpu ops.cpp:504-507, autodiff.cpp:492-496): the block with every key
+    visible to every query."""
+    D, ops = hip.DeviceTensor, hip.ops
+    x, g = r(rng, batch, seq, dim), r(rng, batch, seq, dim)
+    w = [r(rng, dim, dim, scale=dim ** -0.5) for _ in range(4)]
+    dw = [D.fromHost(a) for a in w]
+    dx, dg = D.fromHost(x), D.fromHost(g)
+    exp = oracle.selfAttention(x, *w, heads, causal=False)
+    assert_close(ops.bidirectionalSelfAttention(dx, *dw, heads).toHost(), exp, what="bidirectionalSelfAttention")
+    assert np.abs(exp - oracle.selfAttention(x, *w, heads, causal=True)).max() > 1e-3, "the case must tell the two masks apart"
+    grad = ops.bidirectionalSelfAttentionBackward(dx, *dw, heads, dg)
+    for got, e, n in zip((grad.dInput, grad.dWq, grad.dWk, grad.dWv, grad.dWout), oracle.selfAttentionBackward(x, *w, heads, g, causal=False),
+                         ("dInput", "dWq", "dWk", "dWv", "dWout")):
+        assert_close(got.toHost(), e, what="bidirectionalSelfAttentionBackward." + n, scale=float(np.abs(e).max()) * 0.1)
+    # bf16 projections: the documented bf16 tolerance
+    got = ops.bidirectionalSelfAttention(dx, *dw, heads, useBf16=True).toHost()
+    assert_close(got, exp, tol=2e-2, what="bidirectionalSelfAttention bf16")
+
+
+def test_bidirectional_attention_reference_case(hip):
+    """tests/backend/cpu/ops_tests.cpp:359-391: a change at position 2 reaches the outputs at positions 0 and 1."""
+    D, ops = hip.DeviceTensor, hip.ops
+    wq = np.array([0.3, -0.1, 0.2, 0.05, 0.1, 0.4, -0.2, 0.15, -0.3, 0.2, 0.1, -0.05, 0.2, -0.1, 0.3, 0.1], f32).reshape(4, 4)
+    wk = np.array([0.1, 0.2, -0.1, 0.3, -0.2, 0.1, 0.4, -0.1, 0.3, -0.3, 0.1, 0.2, -0.1, 0.2, -0.2, 0.1], f32).reshape(4, 4)
+    wv = np.array([0.2, 0.1, -0.1, 0.3, 0.1, -0.2, 0.3, 0.1, -0.1, 0.3, 0.2, -0.1, 0.3, 0.1, -0.2, 0.2], f32).reshape(4, 4)
+    wo = np.array([0.1, -0.1, 0.2, 0.1, 0.2, 0.1, -0.1, 0.2, -0.1, 0.2, 0.1, -0.1, 0.1, 0.2, -0.1, 0.2], f32).reshape(4, 4)
+    a = np.array([0.1, -0.2, 0.3, 0.4, -0.5, 0.6, 0.2, -0.1, 0.3, 0.2, -0.4, 0.5], f32).reshape(1, 3, 4)
+    b = a.copy()
+    b[0, 2, 0] = 99.0
+    dw = [D.fromHost(t) for t in (wq, wk, wv, wo)]
+    ya, yb = (ops.bidirectionalSelfAttention(D.fromHost(t), *dw, 2).toHost() for t in (a, b))
+    assert np.abs(ya[0, :2] - yb[0, :2]).max() > 1e-4
+    ca, cb = (ops.selfAttention(D.fromHost(t), *dw, 2).toHost() for t in (a, b))
+    assert np.abs(ca[0, :2] - cb[0, :2]).max() == 0.0
+
+
+def test_mlm_model_steps_against_oracle(hip, oracle, rng):
+    """A masked-language-model pipeline (embedding, positions, bidirectional attention, feed-forward, linear) through the
+    C++ host layer's Model for three steps with the masked loss and AdamW, against the CPU restatement."""
+    from blackforge_amd import hostlayer as hl
+    from oracle import bfo
+    vocab, dim, seq, heads, hidden, batch = 37, 32, 12, 4, 48, 3
+    mk = lambda m: [(m.EMBEDDING, vocab, dim), (m.POSITIONAL, seq), (m.BIDIRECTIONAL_ATTENTION, heads), (m.FEEDFORWARD, hidden, 0),
+                    (m.LINEAR, vocab)]
+    gpu, cpu = hl.HostModel(mk(hl)), oracle.model(mk(bfo))
+    assert gpu.names == cpu.names and any(n.startswith("bidirectional_attention3.") for n in gpu.names)
+    for i, c in enumerate(gpu.counts):
+        w = r(rng, c, scale=0.1)
+        gpu.set_value(i, w)
+        cpu.value(i)[:] = w
+    D = hip.DeviceTensor
+    for step in range(3):
+        ids = rng.integers(0, vocab, (batch, seq)).astype(f32)
+        target = np.where(rng.random(batch * seq) < 0.3, ids.ravel(), -1).astype(f32)
+        target[1] = ids.ravel()[1]
+        cpu.zeroGrad()
+        logits = cpu.forward(ids)
+        loss, grad = oracle.softmaxCrossEntropyMasked(logits.reshape(-1, vocab), target)
+        cpu.backward(grad)
+        gpu.trainStep(D.fromHost(ids), D.fromHost(target), hl.LOSS_MASKED_CE, optimizer=0)
+        assert abs(gpu.readLossSum() - loss) <= 1e-4 * abs(loss) + 1e-6
+        for i in range(len(gpu.counts)):
+            e = cpu.grad(i)
+            assert_close(gpu.grad(i), e, what=f"step {step} grad {gpu.names[i]}", scale=float(np.abs(e).max()) * 0.05)
+        cpu.adamwStep(lr=1e-2)
+        gpu.adamwStep(lr=1e-2)
+        for i in range(len(gpu.counts)):
+            assert_close(gpu.value(i), cpu.value(i), what=f"step {step} param {gpu.names[i]}", scale=0.02 * 1e-2 / 1e-4)
+
+
 def test_incremental_decode_block(hip, oracle, rng):
     D, ops = hip.DeviceTensor, hip.ops
     batch, dim, heads = 2, 32, 4

@@ -182,3 +182,53 @@ def test_bf16_rounding_is_nearest_even(oracle):
     # 1 + 3*2^-8 is halfway between 1+2^-7 (odd) and 1+2^-6 (even): goes up.
     x = np.array([1 + 2.0 ** -8, 1 + 3 * 2.0 ** -8, 1 + 2.0 ** -8 + 2.0 ** -20, -(1 + 2.0 ** -8)], f32)
     np.testing.assert_array_equal(oracle.roundToBf16(x), np.array([1.0, 1 + 2.0 ** -6, 1 + 2.0 ** -7, -1.0], f32))
+
+
+def test_masked_cross_entropy_reduces_to_the_sparse_loss_on_the_kept_rows(oracle, rng):
+    """The cases of tests/backend/cpu/loss_tests.cpp:142-196 and their general form: with no -1 the masked loss IS the sparse
+    loss; otherwise it is the sparse loss of the kept rows alone, ignored rows get a zero gradient, and with every row
+    ignored loss and gradient are zero."""
+    f32 = np.float32
+    logits = np.array([[0.5, -1.2, 0.3], [2.0, 0.1, -0.5]], f32)
+    v, g = oracle.softmaxCrossEntropyMasked(logits, np.array([1, 0], f32))
+    sv, sg = oracle.softmaxCrossEntropySparse(logits, np.array([1, 0], f32))
+    assert abs(v - sv) <= 1e-6 and np.abs(g - sg).max() <= 1e-6
+    logits = np.array([[1, 2, 3], [0.5, -1.0, 0.2], [-0.3, 0.1, 0.4]], f32)
+    v, g = oracle.softmaxCrossEntropyMasked(logits, np.array([-1, 2, -1], f32))
+    sv, sg = oracle.softmaxCrossEntropySparse(logits[1:2], np.array([2], f32))
+    assert not g[0].any() and not g[2].any()
+    assert abs(v - sv) <= 1e-5 and np.abs(g[1] - sg[0]).max() <= 1e-6
+    v, g = oracle.softmaxCrossEntropyMasked(logits[:2], np.array([-1, -1], f32))
+    assert v == 0.0 and not g.any()
+    with pytest.raises(Exception):
+        oracle.softmaxCrossEntropyMasked(np.array([[0.1, 0.2, 0.3]], f32), np.array([7], f32))
+    # general form on random data, against float64
+    rows, classes = 50, 11
+    x = rng.standard_normal((rows, classes)).astype(f32) * 2
+    idx = np.where(rng.random(rows) < 0.3, rng.integers(0, classes, rows), -1)
+    v, g = oracle.softmaxCrossEntropyMasked(x, idx.astype(f32))
+    keep = idx >= 0
+    z = x.astype(np.float64) - x.max(-1, keepdims=True)
+    p = np.exp(z) / np.exp(z).sum(-1, keepdims=True)
+    onehot = np.zeros_like(p)
+    onehot[keep, idx[keep]] = 1
+    expect = np.where(keep[:, None], (p - onehot) / keep.sum(), 0.0)
+    assert abs(v - (-np.log(p[keep, idx[keep]])).mean()) <= 1e-6
+    assert np.abs(g - expect).max() <= 1e-7
+
+
+def test_bidirectional_attention_sees_later_positions(oracle):
+    """tests/backend/cpu/ops_tests.cpp:359-391: changing token 2 changes the outputs at positions 0 and 1, which it must
+    not do under the causal mask."""
+    f32 = np.float32
+    wq = np.array([0.3, -0.1, 0.2, 0.05, 0.1, 0.4, -0.2, 0.15, -0.3, 0.2, 0.1, -0.05, 0.2, -0.1, 0.3, 0.1], f32).reshape(4, 4)
+    wk = np.array([0.1, 0.2, -0.1, 0.3, -0.2, 0.1, 0.4, -0.1, 0.3, -0.3, 0.1, 0.2, -0.1, 0.2, -0.2, 0.1], f32).reshape(4, 4)
+    wv = np.array([0.2, 0.1, -0.1, 0.3, 0.1, -0.2, 0.3, 0.1, -0.1, 0.3, 0.2, -0.1, 0.3, 0.1, -0.2, 0.2], f32).reshape(4, 4)
+    wo = np.array([0.1, -0.1, 0.2, 0.1, 0.2, 0.1, -0.1, 0.2, -0.1, 0.2, 0.1, -0.1, 0.1, 0.2, -0.1, 0.2], f32).reshape(4, 4)
+    a = np.array([0.1, -0.2, 0.3, 0.4, -0.5, 0.6, 0.2, -0.1, 0.3, 0.2, -0.4, 0.5], f32).reshape(1, 3, 4)
+    b = a.copy()
+    b[0, 2, 0] = 99.0
+    ya, yb = (oracle.selfAttention(x, wq, wk, wv, wo, 2, causal=False) for x in (a, b))
+    assert np.abs(ya[0, :2] - yb[0, :2]).max() > 1e-4
+    ca, cb = (oracle.selfAttention(x, wq, wk, wv, wo, 2, causal=True) for x in (a, b))
+    assert np.abs(ca[0, :2] - cb[0, :2]).max() == 0.0

@@ -124,6 +124,20 @@ def test_losses(oracle, ref, rng):
         same(ga, gb)
 
 
+@pytest.mark.parametrize("rows,classes,keep", [(7, 13, 0.5), (40, 5, 0.15), (6, 9, 1.0), (5, 4, 0.0)])
+def test_masked_cross_entropy(oracle, ref, rng, rows, classes, keep):
+    logits = r(rng, rows, classes, scale=3)
+    idx = np.where(rng.random(rows) < keep, rng.integers(0, classes, rows), -1).astype(f32)
+    (va, ga), (vb, gb) = oracle.softmaxCrossEntropyMasked(logits, idx), ref.softmaxCrossEntropyMasked(logits, idx)
+    assert f32(va).view(np.uint32) == f32(vb).view(np.uint32)
+    same(ga, gb)
+    bad = idx.copy()
+    bad[0] = classes
+    for impl in (oracle, ref):
+        with pytest.raises(bfo.OracleInvalidArgument):
+            impl.softmaxCrossEntropyMasked(logits, bad)
+
+
 def test_optimizers(oracle, ref, rng):
     p, g = r(rng, 50), r(rng, 50)
     same(oracle.sgdStep(p, g, 0.05), ref.sgdStep(p, g, 0.05))
@@ -134,9 +148,10 @@ def test_optimizers(oracle, ref, rng):
 
 TINY_LM = [(bfo.EMBEDDING, 17, 8), (bfo.POSITIONAL, 6), (bfo.ATTENTION, 2), (bfo.FEEDFORWARD, 16, 0), (bfo.LINEAR, 17)]
 MLP = [(bfo.LINEAR, 12), (bfo.SILU,), (bfo.LINEAR, 5), (bfo.RMSNORM,), (bfo.GELU,), (bfo.RELU,), (bfo.SOFTMAX,)]
+TINY_MLM = [(bfo.EMBEDDING, 17, 8), (bfo.POSITIONAL, 6), (bfo.BIDIRECTIONAL_ATTENTION, 2), (bfo.FEEDFORWARD, 16, 0), (bfo.LINEAR, 17)]
 
 
-@pytest.mark.parametrize("layers,in_features,kind", [(TINY_LM, 0, "lm"), (MLP, 9, "mlp")])
+@pytest.mark.parametrize("layers,in_features,kind", [(TINY_LM, 0, "lm"), (MLP, 9, "mlp"), (TINY_MLM, 0, "mlm")])
 def test_model_training_steps(oracle, ref, rng, layers, in_features, kind):
     """Three full steps (zeroGrad, forward, loss, backward, AdamW) through cpu::Model and the restatement."""
     mo, mr = oracle.model(layers, in_features), ref.model(layers, in_features)
@@ -149,6 +164,10 @@ def test_model_training_steps(oracle, ref, rng, layers, in_features, kind):
         if kind == "lm":
             x = rng.integers(0, 17, (2, 5)).astype(f32)
             target = rng.integers(0, 17, 10).astype(f32)
+        elif kind == "mlm":
+            x = rng.integers(0, 17, (2, 5)).astype(f32)
+            target = np.where(rng.random(10) < 0.4, x.ravel(), -1).astype(f32)
+            target[3] = x.ravel()[3]   # at least one row counts
         else:
             x = r(rng, 4, 9)
             target = rng.integers(0, 5, 4).astype(f32)
@@ -156,8 +175,9 @@ def test_model_training_steps(oracle, ref, rng, layers, in_features, kind):
         for o, m in ((oracle, mo), (ref, mr)):
             m.zeroGrad()
             y = m.forward(x)
-            classes = 17 if kind == "lm" else 5
-            loss, grad = o.softmaxCrossEntropySparse(y.reshape(-1, classes), target)
+            classes = 5 if kind == "mlp" else 17
+            loss_fn = o.softmaxCrossEntropyMasked if kind == "mlm" else o.softmaxCrossEntropySparse
+            loss, grad = loss_fn(y.reshape(-1, classes), target)
             m.backward(grad)
             grads = [m.grad(i).copy() for i in range(len(m.counts))]
             m.adamwStep(lr=1e-2)

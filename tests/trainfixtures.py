@@ -8,8 +8,8 @@ import numpy as np
 GOLDEN_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 EXPECTED = os.path.join(GOLDEN_DIR, "training_expected.npz")
 
-# layer kinds as the oracle and the host layer number them (bf_oracle.h: BFO_LINEAR = 0 ... BFO_FEEDFORWARD = 9)
-LINEAR, SILU, RELU, GELU, RMSNORM, SOFTMAX, EMBEDDING, POSITIONAL, ATTENTION, FEEDFORWARD = range(10)
+# layer kinds as the oracle and the host layer number them (bf_oracle.h: BFO_LINEAR = 0 ... BFO_BIDIRECTIONAL_ATTENTION = 10)
+LINEAR, SILU, RELU, GELU, RMSNORM, SOFTMAX, EMBEDDING, POSITIONAL, ATTENTION, FEEDFORWARD, BIDIRECTIONAL_ATTENTION = range(11)
 
 # name -> (layers, input features, loss, optimizer, epochs, batch, lr, cosine): the same table the generator uses
 RUNS = {
@@ -17,6 +17,8 @@ RUNS = {
                  "cross_entropy_sparse", "adamw", 3, 4, 1e-2, True),
     "train_mlp": ([(LINEAR, 16), (SILU,), (LINEAR, 4)], 8, "mse", "sgd", 4, 5, 0.05, False),
     "train_dense": ([(LINEAR, 12), (RELU,), (LINEAR, 6)], 8, "cross_entropy", "adamw", 2, 6, 5e-3, True),
+    "train_mlm": ([(EMBEDDING, 32, 16), (POSITIONAL, 8), (BIDIRECTIONAL_ATTENTION, 2), (FEEDFORWARD, 32, 0), (LINEAR, 32)], 0,
+                  "cross_entropy_masked", "adamw", 3, 4, 1e-2, False),
 }
 SHUFFLES = [(n, seed) for n in (2, 3, 5, 17, 24, 100) for seed in (1, 2, 3)]
 
