@@ -27,6 +27,7 @@
 // newLen/totalLen/oldLen are accepted (tiles are zero-filled and masked).
 #include "common.hpp"
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstdint>
@@ -504,7 +505,7 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnBackwardDqKernel(A
 constexpr int kDsPatch = 32 * 36;   // floats of LDS per staged dS sub-block
 
 template <int HDP, int BC, bool VEC4>
-__global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnBackwardDqFromDsKernel(AttnParams p) {
+__global__ void __launch_bounds__(256, HDP <= 64 ? 3 : HDP <= 128 ? 2 : 1) attnBackwardDqFromDsKernel(AttnParams p) {
     constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BC * LDSW, NSB = BC / 32;
     extern __shared__ float smem[];
     float* ks = smem;   // [2][BC][LDSW]
@@ -526,7 +527,7 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnBackwardDqFromDsK
     // through a wave-private LDS patch with rows padded to 36 floats; no barrier is involved, a wave's LDS
     // operations execute in order.
     const float* dsWave = p.ds + ((size_t(bh) * p.nqb + size_t(waveQ0 >> 5)) * p.nkb) * 1024 + lane * 4;
-    float* stage = smem + 2 * TILE + wave * (NSB * kDsPatch);
+    float* stage = smem + 2 * TILE + wave * kDsPatch;   // one patch per wave, reused by its sub-blocks in turn
 
     float16v acc[DT];
 #pragma unroll
@@ -564,7 +565,7 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnBackwardDqFromDsK
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb) {
             if (kt0 + sb * 32 < waveKeyEnd) {
-                float* patch = stage + sb * kDsPatch;
+                float* patch = stage;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) storef4(patch + (8 * j + (lane >> 3)) * 36 + (lane & 7) * 4, dsNext[sb][j]);
 #pragma unroll
@@ -818,7 +819,10 @@ int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
         return vec4 ? launchAttn(attnBackwardDqKernel<HDP, TILE, true>, 2 * operandBytes, grid, p, s)
                     : launchAttn(attnBackwardDqKernel<HDP, TILE, false>, 2 * operandBytes, grid, p, s);
     } else if constexpr (KIND == 4) {
-        constexpr size_t smem = operandBytes + size_t(4) * (TILE / 32) * kDsPatch * sizeof(float);   // K tiles + a dS patch per wave
+        constexpr size_t need = operandBytes + size_t(4) * kDsPatch * sizeof(float);   // K tiles + a dS patch per wave
+        // Three workgroups per CU pay once the grid keeps refilling them; a grid that fits in one round is better spread
+        // two per CU, which asking for more LDS than needed (over a third of the CU's 160 KiB) enforces.
+        const size_t smem = grid > 3u * unsigned(computeUnits()) ? need : std::max(need, size_t(56) * 1024);
         return vec4 ? launchAttn(attnBackwardDqFromDsKernel<HDP, TILE, true>, smem, grid, p, s)
                     : launchAttn(attnBackwardDqFromDsKernel<HDP, TILE, false>, smem, grid, p, s);
     } else {
