@@ -192,6 +192,13 @@ def bench_extras(bf, steps):
     hbm("cross_entropy_sparse_8192x32000", 8 * rows * vocab,
         lambda: call("bf_hip_cross_entropy_sparse", logits.ptr, target.ptr, grad.ptr, loss.ptr, rows, vocab, 0, sh))
     del logits, grad
+    # long-context logits [16384, 50257] (3.07 GiB): rows of odd length, 16-byte accesses through a per-row shift
+    rows_lc, vocab_lc = 16384, 50257
+    logits, grad = rand(rows_lc, vocab_lc), D((rows_lc, vocab_lc))
+    target_lc = D.fromHost(rng.integers(0, vocab_lc, rows_lc).astype(np.float32))
+    hbm("cross_entropy_sparse_16384x50257", 8 * rows_lc * vocab_lc,
+        lambda: call("bf_hip_cross_entropy_sparse", logits.ptr, target_lc.ptr, grad.ptr, loss.ptr, rows_lc, vocab_lc, 0, sh))
+    del logits, grad
 
     # embedding table [32000, 768]: gather of 8192 tokens; scatter-add backward writes the whole table gradient
     table, dtable = rand(vocab, dim), D((vocab, dim))

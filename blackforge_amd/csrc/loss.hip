@@ -78,7 +78,8 @@ __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pr
 }
 
 // SPARSE: target holds one class index per row.  Otherwise a dense target row.
-template <int G, int MAXE, int VEC, bool CACHED, bool SPARSE>
+// SHIFTED (with VEC = 4, CACHED): rows of any length and alignment through 16-byte accesses (RowCache::loadShifted).
+template <int G, int MAXE, int VEC, bool CACHED, bool SPARSE, bool SHIFTED = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const float* __restrict__ logits,
                                                                          const float* __restrict__ target,
                                                                          float* __restrict__ grad, float* __restrict__ rowLoss,
@@ -95,12 +96,17 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
         const float* x = logits + row * classes;
         float* gOut = grad + row * classes;
         RowCache<G, MAXE, VEC> c;
+        const int shift = SHIFTED ? RowCache<G, MAXE, VEC>::shiftOf(x) : 0;   // the same for gOut: the host checks that
+        auto storeRow = [&]() __attribute__((always_inline)) {
+            if constexpr (SHIFTED) c.storeShifted(gOut, classes, t, shift);
+            else c.store(gOut, classes, t);
+        };
         if constexpr (SPARSE) {
             if (maskInfo != nullptr && lroundf(target[row]) == -1) {   // uniform over the row's group
                 if constexpr (CACHED) {
 #pragma unroll
                     for (int i = 0; i < MAXE; ++i) c.r[i] = 0.0f;
-                    c.store(gOut, classes, t);
+                    storeRow();
                 } else {
                     for (size_t e = t; e < classes; e += G) gOut[e] = 0.0f;
                 }
@@ -110,7 +116,8 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
         }
         float mx = -INFINITY;
         if constexpr (CACHED) {
-            c.load(x, classes, t, -INFINITY);
+            if constexpr (SHIFTED) c.loadShifted(x, classes, t, -INFINITY, shift);
+            else c.load(x, classes, t, -INFINITY);
 #pragma unroll
             for (int i = 0; i < MAXE; ++i) mx = fmaxf(mx, c.r[i]);
         } else {
@@ -140,13 +147,13 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                 for (int it = 0; it < MAXE / VEC; ++it)
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) {
-                        const unsigned idx = unsigned(it * G + t) * VEC + j;   // < G * MAXE <= 65536
+                        const int idx = int(it * G + t) * VEC + j - shift;   // |.| < G * MAXE + 4 <= 65540
                         const float p = c.r[it * VEC + j] * inv;
-                        const bool hit = idx == cls;
+                        const bool hit = idx == int(cls);                    // cls < classes <= G * MAXE
                         pTarget = hit ? p : pTarget;
                         c.r[it * VEC + j] = (p - (hit ? 1.0f : 0.0f)) * invRows;
                     }
-                c.store(gOut, classes, t);
+                storeRow();
             } else {
                 for (size_t e = t; e < classes; e += G) {
                     const float p = __builtin_amdgcn_exp2f((x[e] - mx) * kLog2e) * inv;
@@ -169,10 +176,10 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                 for (int it = 0; it < MAXE / VEC; ++it)
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) {
-                        size_t idx = RowCache<G, MAXE, VEC>::index(it, t, j);
-                        if (idx < classes) c.r[it * VEC + j] = emit(c.r[it * VEC + j], idx);
+                        const long idx = long(RowCache<G, MAXE, VEC>::index(it, t, j)) - shift;
+                        if (idx >= 0 && size_t(idx) < classes) c.r[it * VEC + j] = emit(c.r[it * VEC + j], size_t(idx));
                     }
-                c.store(gOut, classes, t);
+                storeRow();
             } else {
                 for (size_t e = t; e < classes; e += G) gOut[e] = emit(__builtin_amdgcn_exp2f((x[e] - mx) * kLog2e), e);
             }
@@ -196,17 +203,21 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
     }
     const float invRows = 1.0f / float(rows);
     const bool vec4 = aligned16(logits) && aligned16(grad) && classes % 4 == 0;
+    // rows that are not 16-byte aligned still get 16-byte accesses (shifted) as long as a logits row and its gradient
+    // row sit at the same offset within a 16-byte group; a row must then fit its registers with up to 3 elements to spare
+    const bool shifted = !vec4 && ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad)) & 15u) == 0;
     // smallest group and register count that hold a row (see the row kernels); a block takes its rows once
 #define BF_CE(G, MAXE)                                                                                            \
-    if (classes <= size_t(G) * MAXE) {                                                                            \
+    if (classes + (vec4 ? 0 : 3) <= size_t(G) * MAXE && (vec4 || shifted || MAXE <= 32)) {                        \
         const unsigned threads = G > 256 ? G : 256;                                                               \
         const unsigned grid = gridFor(rows, threads / G);                                                         \
         if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
-        else crossEntropyKernel<G, MAXE, 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo);      \
+        else if (shifted) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
+        else crossEntropyKernel<G, (MAXE <= 32 ? MAXE : 4), 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); /* plans above 32 registers have no one-element form */ \
         break;                                                                                                    \
     }
     do {
-        BF_CE(64, 4) BF_CE(64, 8) BF_CE(64, 16) BF_CE(256, 8) BF_CE(256, 16) BF_CE(256, 32) BF_CE(1024, 16) BF_CE(1024, 32)
+        BF_CE(64, 4) BF_CE(64, 8) BF_CE(64, 16) BF_CE(256, 8) BF_CE(256, 16) BF_CE(256, 32) BF_CE(1024, 16) BF_CE(1024, 32) BF_CE(1024, 52)
         crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo);
     } while (0);
 #undef BF_CE

@@ -4,7 +4,11 @@
 // up to MAXE elements per thread in registers, so multi-pass algorithms (max, sum, normalise) read
 // the row from HBM exactly once.  Rows longer than G*MAXE fall back to re-reading global memory
 // (served by L2).  VEC = 4 uses dwordx4 accesses and needs 16-byte aligned rows (features % 4 == 0
-// and an aligned base); VEC = 1 handles every other shape with coalesced dword accesses.
+// and an aligned base); VEC = 1 handles every other shape with coalesced dword accesses.  loadShifted /
+// storeShifted give rows of ANY length and alignment the 16-byte accesses too: the row is addressed from the
+// 16-byte boundary at or below its first element, `shift` (0..3) elements earlier, and the elements a group
+// holds from outside the row are masked.  An aligned 16-byte load that contains one element of the tensor stays
+// inside the tensor's page, so the bytes read from beyond a row are always readable; nothing is written there.
 #pragma once
 
 #include "common.hpp"
@@ -21,7 +25,7 @@ struct RowCache {
     // element index handled by (iteration it, vector slot j) for group-thread t
     __device__ static size_t index(int it, int t, int j) { return (size_t(it) * G + t) * VEC + j; }
 
-    __device__ void load(const float* __restrict__ row, size_t features, int t, float fill) {
+    __device__ __forceinline__ void load(const float* __restrict__ row, size_t features, int t, float fill) {
 #pragma unroll
         for (int it = 0; it < kIters; ++it) {
             size_t e = index(it, t, 0);
@@ -38,7 +42,54 @@ struct RowCache {
         }
     }
 
-    __device__ void store(float* __restrict__ row, size_t features, int t) const {
+    // Elements before the row's first one in the 16-byte group that holds it.
+    __device__ static int shiftOf(const float* row) { return int((reinterpret_cast<uintptr_t>(row) >> 2) & 3u); }
+
+    // Rows are shorter than 2^31 - 4 elements here (G * MAXE elements at most), so 32-bit indices do.  Only the group
+    // that holds the row's first element (thread 0, iteration 0) and the one that holds its last need any masking.
+    __device__ __forceinline__ void loadShifted(const float* __restrict__ row, size_t features, int t, float fill, int shift) {
+        static_assert(VEC == 4, "shifted access is 4 wide");
+        const float* base = row - shift;
+        const int last = int(features) + shift;   // one past the row's last element, counted from base
+        // every load first (a group past the row's end re-reads group 0 instead of branching), the masking afterwards:
+        // code between the loads that touches a loaded register would make each load wait for the one before it
+#pragma unroll
+        for (int it = 0; it < kIters; ++it) {
+            const int g = (it * G + t) * 4;
+            const float4v v = loadf4(base + (g < last ? g : 0));
+            r[it * 4 + 0] = v.x; r[it * 4 + 1] = v.y; r[it * 4 + 2] = v.z; r[it * 4 + 3] = v.w;
+        }
+        const int lo = t == 0 ? shift : 0;   // slots of thread 0's first group that belong to the row before
+#pragma unroll
+        for (int it = 0; it < kIters; ++it) {
+            const int n = last - (it * G + t) * 4;   // slots of this group before the row's end (>= 4: all of them)
+            const int first = it == 0 ? lo : 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) r[it * 4 + j] = (j >= first && j < n) ? r[it * 4 + j] : fill;
+        }
+    }
+
+    __device__ __forceinline__ void storeShifted(float* __restrict__ row, size_t features, int t, int shift) const {
+        static_assert(VEC == 4, "shifted access is 4 wide");
+        float* base = row - shift;
+        const int last = int(features) + shift;
+#pragma unroll
+        for (int it = 0; it < kIters; ++it) {
+            const int g = (it * G + t) * 4;
+            if (g < last) {
+                const bool head = it == 0 && t == 0 && shift > 0, tail = g + 4 > last;
+                if (!head && !tail) {
+                    storef4(base + g, float4v{r[it * 4 + 0], r[it * 4 + 1], r[it * 4 + 2], r[it * 4 + 3]});
+                } else {   // a group that straddles an end of the row: its own elements one by one
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (g + j >= shift && g + j < last) base[g + j] = r[it * 4 + j];
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(float* __restrict__ row, size_t features, int t) const {
 #pragma unroll
         for (int it = 0; it < kIters; ++it) {
             size_t e = index(it, t, 0);
