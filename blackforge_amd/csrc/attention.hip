@@ -853,9 +853,7 @@ std::atomic<size_t> gDsLimit{SIZE_MAX};
 size_t dsLimit() {
     size_t limit = gDsLimit.load();
     if (limit != SIZE_MAX) return limit;
-    size_t freeBytes = 0, totalBytes = 0;
-    if (hipMemGetInfo(&freeBytes, &totalBytes) != hipSuccess) { (void)hipGetLastError(); return 0; }
-    return totalBytes / 8;
+    return deviceMemoryBytes() / 8;
 }
 
 int checkShapes(const char* fn, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, size_t oldLen) {

@@ -46,6 +46,8 @@ inline unsigned gridFor(size_t work, size_t perBlock, unsigned cap = kMaxGridX) 
 
 // Number of compute units of the current device (cached); used to size persistent grids.
 int computeUnits();
+// Total memory of the current device in bytes (cached per device; 0 if it cannot be read).
+size_t deviceMemoryBytes();
 
 // Raises a kernel's dynamic shared-memory limit to `bytes` on the current device (needed above 48 KiB).  The
 // setting is per (kernel, device) and sticks, so it is made once and remembered.

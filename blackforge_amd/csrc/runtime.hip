@@ -44,6 +44,18 @@ int computeUnits() {
     return cus;
 }
 
+size_t deviceMemoryBytes() {
+    static std::unordered_map<int, size_t> cache;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    auto it = cache.find(dev);
+    if (it != cache.end()) return it->second;
+    size_t freeBytes = 0, totalBytes = 0;
+    if (hipMemGetInfo(&freeBytes, &totalBytes) != hipSuccess) { (void)hipGetLastError(); totalBytes = 0; }
+    cache[dev] = totalBytes;
+    return totalBytes;
+}
+
 namespace {
 struct DescriptorTable {
     std::vector<unsigned char> host;
