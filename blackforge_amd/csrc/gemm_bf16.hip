@@ -302,13 +302,17 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
 // barrier and before its first reader (group 0's M(T+1,0)) starts, and a global load has four phases to land.
 // Operand A is staged in the first half step and Bt in the second, so every load instruction still fetches
 // whole 128-byte lines.
-template <int XCD_ORDER>
+// BM = 256, or 128 for products whose 256-row tiles would leave compute units without one (or with a nearly empty
+// second round): half the rows per workgroup, the same eight wavefronts, each with a 64 x 64 share instead of 128 x 64.
+// The memory phase then moves 8 fragments for 8 MFMAs instead of 12 for 16, so a tile costs more than half of a full
+// one; it pays when it fills the chip.
+template <int XCD_ORDER, int BM>
 __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned short* __restrict__ A,
                                                                  const unsigned short* __restrict__ Bt, Epilogue epi,
                                                                  int M, int N, int K, int lda, int ldb, int gmLog, int gnLog) {
-    constexpr int BM = 256, BN = 256, TM = 4, TN = 2;
+    constexpr int BN = 256, TM = BM / 64, TN = 2, A_PASSES = BM / 64;
     extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
-    unsigned short* as = lds;                        // [2][256][LDS_ROW]
+    unsigned short* as = lds;                        // [2][BM][LDS_ROW]
     unsigned short* bs = lds + 2 * BM * LDS_ROW;     // [2][256][LDS_ROW]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
     const int group = wave >> 2;
@@ -319,16 +323,15 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
         tileIndexGrouped(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
     }
     const int m0 = tm * BM, n0 = tn * BN;
-    const int wm0 = group * 128, wn0 = (wave & 3) * 64;
-    const int lr = tid >> 3, lc = (tid & 7) * 8;     // 64 rows x 128 bytes per pass, 4 passes per operand
-    const unsigned short* aRow[4];
+    const int wm0 = group * (BM / 2), wn0 = (wave & 3) * 64;
+    const int lr = tid >> 3, lc = (tid & 7) * 8;     // 64 rows x 128 bytes per pass
+    const unsigned short* aRow[A_PASSES];
     const unsigned short* bRow[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        aRow[i] = A + size_t(min(m0 + lr + 64 * i, M - 1)) * lda;
-        bRow[i] = Bt + size_t(min(n0 + lr + 64 * i, N - 1)) * ldb;
-    }
-    uint4v stageA[4], stageB[4];
+    for (int i = 0; i < A_PASSES; ++i) aRow[i] = A + size_t(min(m0 + lr + 64 * i, M - 1)) * lda;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bRow[i] = Bt + size_t(min(n0 + lr + 64 * i, N - 1)) * ldb;
+    uint4v stageA[A_PASSES], stageB[4];
     float16v acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -339,21 +342,18 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
     const int steps = (K + BKK - 1) / BKK;
     const int ldsW = lr * LDS_ROW + lc;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        stageA[i] = loadChunk(aRow[i], lc, K);
-        stageB[i] = loadChunk(bRow[i], lc, K);
-    }
+    for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], lc, K);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<uint4v*>(as + ldsW + 64 * i * LDS_ROW) = zeroPast(stageA[i], lc, K);
-        *reinterpret_cast<uint4v*>(bs + ldsW + 64 * i * LDS_ROW) = zeroPast(stageB[i], lc, K);
-    }
+    for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], lc, K);
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<uint4v*>(as + ldsW + 64 * i * LDS_ROW) = zeroPast(stageA[i], lc, K);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(bs + ldsW + 64 * i * LDS_ROW) = zeroPast(stageB[i], lc, K);
     if (steps > 1) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            stageA[i] = loadChunk(aRow[i], BKK + lc, K);
-            stageB[i] = loadChunk(bRow[i], BKK + lc, K);
-        }
+        for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], BKK + lc, K);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], BKK + lc, K);
     }
     __syncthreads();
     if (group == 1) __builtin_amdgcn_s_barrier();    // group 1 starts one phase late
@@ -377,10 +377,10 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
             if (T + 1 < steps) {
                 if (h == 0) {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(aw + 64 * i * LDS_ROW) = zeroPast(stageA[i], (T + 1) * BKK + lc, K);
+                    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<uint4v*>(aw + 64 * i * LDS_ROW) = zeroPast(stageA[i], (T + 1) * BKK + lc, K);
                     if (T + 2 < steps) {
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) stageA[i] = loadChunk(aRow[i], (T + 2) * BKK + lc, K);
+                        for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], (T + 2) * BKK + lc, K);
                     }
                 } else {
 #pragma unroll
@@ -444,10 +444,11 @@ int allowSharedMemory(Kernel kernel, size_t smem) {
     return allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
 }
 
+template <int BM>
 int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
                    size_t lda, size_t ldb, hipStream_t s) {
-    const size_t tilesM = (M + 255) / 256, tilesN = (N + 255) / 256;
-    constexpr size_t smem = size_t(2) * 512 * LDS_ROW * sizeof(unsigned short);
+    const size_t tilesM = (M + BM - 1) / BM, tilesN = (N + 255) / 256;
+    constexpr size_t smem = size_t(2) * (BM + 256) * LDS_ROW * sizeof(unsigned short);
     // XCD block shape: the 2^g x 2^(5-g) block that pads the tile grid least, squarest on ties
     int gmLog = 2, gnLog = 3;
     size_t bestCost = 0, blocks = 0;
@@ -462,14 +463,14 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
     if (xcdOrder) {
         size_t grid = (blocks + 7) / 8 * 8 * 32;
         if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
-        auto kernel = gemmBf16PingPongKernel<1>;
+        auto kernel = gemmBf16PingPongKernel<1, BM>;
         int st = allowSharedMemory(kernel, smem);
         if (st != BF_OK) return st;
         kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), gmLog, gnLog);
     } else {
         size_t grid = tilesM * tilesN;
         if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
-        auto kernel = gemmBf16PingPongKernel<0>;
+        auto kernel = gemmBf16PingPongKernel<0, BM>;
         int st = allowSharedMemory(kernel, smem);
         if (st != BF_OK) return st;
         kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), 0, 0);
@@ -485,8 +486,14 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
     const size_t cus = size_t(computeUnits());
     // 256x256 ping-pong tiles once they give three quarters of the CUs a tile; otherwise 128x128 tiles,
     // with K cut into slices when even those leave CUs idle and K is long enough to share out.
-    const size_t bigTiles = ((M + 255) / 256) * ((N + 255) / 256);
-    if (bigTiles >= cus * 3 / 4) return launchPingPong(A, Bt, epi, M, N, K, lda, ldb, s);
+    // A workgroup per CU at a time, so a product takes ceil(tiles / CUs) rounds; a 128-row tile costs kHalfTileCost of a
+    // 256-row one (measured).  Either form is used only if its first round covers most of the chip.
+    const size_t bigTiles = ((M + 255) / 256) * ((N + 255) / 256), halfTiles = ((M + 127) / 128) * ((N + 255) / 256);
+    constexpr double kHalfTileCost = 0.78;
+    const double bigTime = bigTiles >= cus * 3 / 4 ? double((bigTiles + cus - 1) / cus) : 1e30;
+    const double halfTime = halfTiles >= cus * 3 / 4 ? double((halfTiles + cus - 1) / cus) * kHalfTileCost : 1e30;
+    if (bigTime <= halfTime && bigTime < 1e30) return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
+    if (halfTime < 1e30) return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s);
     const size_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     constexpr size_t smem = size_t(2) * (128 + 128) * LDS_ROW * sizeof(unsigned short);
     auto kernel = gemmBf16NtKernel<128, 128, 2, 2>;

@@ -120,10 +120,11 @@ def test_bf16_gradients_with_long_contraction(hip, oracle, rng, m, k, n):
     assert_bits_equal(again.toHost(), dB.toHost(), "sliced contraction must be deterministic")
 
 
-@pytest.mark.parametrize("m,k,n", [(3500, 200, 3700), (4000, 136, 4090), (8192, 64, 2048)])
+@pytest.mark.parametrize("m,k,n", [(3500, 200, 3700), (4000, 136, 4090), (8192, 64, 2048), (8192, 200, 768), (8100, 136, 700),
+                                   (6200, 72, 1500)])
 def test_bf16_projection_large_tile_kernel(hip, oracle, rng, m, k, n):
     """Shapes with enough 256x256 tiles for the large-product kernel (ragged edges, a K tail, and a tile grid
-    that is dealt to the XCDs in blocks).  Expected value: float64 product of the bf16-rounded operands, which
+    that is dealt to the XCDs in blocks), and tall narrow ones that take its 128-row-tile form.  Expected value: float64 product of the bf16-rounded operands, which
     the oracle's fp32 matmul matches to 1e-6 on the sampled rows below."""
     D, ops = hip.DeviceTensor, hip.ops
     a, b = r(rng, m, k), r(rng, k, n, scale=0.1)
