@@ -309,7 +309,8 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
 template <int XCD_ORDER, int BM>
 __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned short* __restrict__ A,
                                                                  const unsigned short* __restrict__ Bt, Epilogue epi,
-                                                                 int M, int N, int K, int lda, int ldb, int gmLog, int gnLog) {
+                                                                 int M, int N, int K, int lda, int ldb, int gmLog, int gnLog,
+                                                                 int kPerSplit, size_t sliceStride) {
     constexpr int BN = 256, TM = BM / 64, TN = 2, A_PASSES = BM / 64;
     extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
     unsigned short* as = lds;                        // [2][BM][LDS_ROW]
@@ -339,21 +340,24 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-    const int steps = (K + BKK - 1) / BKK;
+    // blockIdx.y selects a slice of K, as in the small-tile kernel: partial products go to C + slice * sliceStride
+    const int kBegin = blockIdx.y * kPerSplit, kEnd = min(K, kBegin + kPerSplit);
+    epi.c[0] += size_t(blockIdx.y) * sliceStride;
+    const int steps = max((kEnd - kBegin + BKK - 1) / BKK, 1);   // an empty slice runs one step of zeros
     const int ldsW = lr * LDS_ROW + lc;
 #pragma unroll
-    for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], lc, K);
+    for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], kBegin + lc, kEnd);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], lc, K);
+    for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], kBegin + lc, kEnd);
 #pragma unroll
-    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<uint4v*>(as + ldsW + 64 * i * LDS_ROW) = zeroPast(stageA[i], lc, K);
+    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<uint4v*>(as + ldsW + 64 * i * LDS_ROW) = zeroPast(stageA[i], kBegin + lc, kEnd);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(bs + ldsW + 64 * i * LDS_ROW) = zeroPast(stageB[i], lc, K);
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(bs + ldsW + 64 * i * LDS_ROW) = zeroPast(stageB[i], kBegin + lc, kEnd);
     if (steps > 1) {
 #pragma unroll
-        for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], BKK + lc, K);
+        for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], kBegin + BKK + lc, kEnd);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], BKK + lc, K);
+        for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], kBegin + BKK + lc, kEnd);
     }
     __syncthreads();
     if (group == 1) __builtin_amdgcn_s_barrier();    // group 1 starts one phase late
@@ -377,17 +381,17 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
             if (T + 1 < steps) {
                 if (h == 0) {
 #pragma unroll
-                    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<uint4v*>(aw + 64 * i * LDS_ROW) = zeroPast(stageA[i], (T + 1) * BKK + lc, K);
+                    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<uint4v*>(aw + 64 * i * LDS_ROW) = zeroPast(stageA[i], kBegin + (T + 1) * BKK + lc, kEnd);
                     if (T + 2 < steps) {
 #pragma unroll
-                        for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], (T + 2) * BKK + lc, K);
+                        for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], kBegin + (T + 2) * BKK + lc, kEnd);
                     }
                 } else {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(bw + 64 * i * LDS_ROW) = zeroPast(stageB[i], (T + 1) * BKK + lc, K);
+                    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(bw + 64 * i * LDS_ROW) = zeroPast(stageB[i], kBegin + (T + 1) * BKK + lc, kEnd);
                     if (T + 2 < steps) {
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], (T + 2) * BKK + lc, K);
+                        for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], kBegin + (T + 2) * BKK + lc, kEnd);
                     }
                 }
             }
@@ -444,9 +448,11 @@ int allowSharedMemory(Kernel kernel, size_t smem) {
     return allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
 }
 
+// slices > 1: K is cut into `slices` ranges of kPer (a multiple of 64) and range i writes to epi.c[0] + i * sliceStride
 template <int BM>
 int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
-                   size_t lda, size_t ldb, hipStream_t s) {
+                   size_t lda, size_t ldb, hipStream_t s, size_t slices = 1, size_t kPer = 0, size_t sliceStride = 0) {
+    if (slices <= 1) { slices = 1; kPer = K; sliceStride = 0; }
     const size_t tilesM = (M + BM - 1) / BM, tilesN = (N + 255) / 256;
     constexpr size_t smem = size_t(2) * (BM + 256) * LDS_ROW * sizeof(unsigned short);
     // XCD block shape: the 2^g x 2^(5-g) block that pads the tile grid least, squarest on ties
@@ -466,14 +472,16 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
         auto kernel = gemmBf16PingPongKernel<1, BM>;
         int st = allowSharedMemory(kernel, smem);
         if (st != BF_OK) return st;
-        kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), gmLog, gnLog);
+        kernel<<<dim3(unsigned(grid), unsigned(slices)), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), gmLog, gnLog,
+                                                                         int(kPer), sliceStride);
     } else {
         size_t grid = tilesM * tilesN;
         if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
         auto kernel = gemmBf16PingPongKernel<0, BM>;
         int st = allowSharedMemory(kernel, smem);
         if (st != BF_OK) return st;
-        kernel<<<unsigned(grid), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), 0, 0);
+        kernel<<<dim3(unsigned(grid), unsigned(slices)), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), 0, 0,
+                                                                         int(kPer), sliceStride);
     }
     BF_LAUNCH_CHECK();
     return BF_OK;
@@ -494,6 +502,42 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
     const double halfTime = halfTiles >= cus * 3 / 4 ? double((halfTiles + cus - 1) / cus) * kHalfTileCost : 1e30;
     if (bigTime <= halfTime && bigTime < 1e30) return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
     if (halfTime < 1e30) return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s);
+    // Few tiles but a long contraction (the weight-gradient products, K = all tokens): the same kernel with K cut into
+    // slices, one workgroup per (tile, slice), partial products summed in slice order by a second kernel.  More slices
+    // fill more CUs but write and re-read more partial sums; the estimate below (K steps at the measured ~1.4 us per
+    // step of a full tile, partial sums at ~4 TB/s) picks the form and the slice count.
+    if (K >= 4096) {
+        const size_t stepsAll = (K + BKK - 1) / BKK;
+        double best = 1e30;
+        size_t bestSlices = 0, bestTiles = 0;
+        int bestForm = 0;
+        for (int form = 0; form < 2; ++form) {
+            const size_t t = form == 0 ? bigTiles : halfTiles;
+            for (size_t sl = 2; sl <= 16 && sl * 8 <= stepsAll; ++sl) {
+                const size_t rounds = (t * sl + cus - 1) / cus;
+                const double gemmUs = double(rounds) * double((stepsAll + sl - 1) / sl) * 1.4 * (form == 0 ? 1.0 : kHalfTileCost);
+                const double reduceUs = double(sl + 1) * double(M * N) * 2.0 * sizeof(float) / 4e6;
+                if (gemmUs + reduceUs < best) { best = gemmUs + reduceUs; bestSlices = sl; bestTiles = t; bestForm = form; }
+            }
+        }
+        if (bestSlices > 1 && bestTiles * bestSlices >= cus / 2) {
+            const size_t kPer = (stepsAll + bestSlices - 1) / bestSlices * BKK;
+            const size_t sl = (K + kPer - 1) / kPer;
+            const size_t count = M * N, sliceStride = (count + 3) / 4 * 4;
+            Scratch partial(sl * sliceStride * sizeof(float));
+            if (partial.status != BF_OK) return partial.status;
+            Epilogue plain{{partial.as<float>(), nullptr, nullptr}, int(N), nullptr, nullptr};
+            int st = bestForm == 0 ? launchPingPong<256>(A, Bt, plain, M, N, K, lda, ldb, s, sl, kPer, sliceStride)
+                                   : launchPingPong<128>(A, Bt, plain, M, N, K, lda, ldb, s, sl, kPer, sliceStride);
+            if (st != BF_OK) return st;
+            const int vec = ((reinterpret_cast<uintptr_t>(epi.c[0]) | reinterpret_cast<uintptr_t>(epi.c[1]) |
+                              reinterpret_cast<uintptr_t>(epi.c[2]) | reinterpret_cast<uintptr_t>(epi.residual) |
+                              reinterpret_cast<uintptr_t>(epi.bias)) & 15u) == 0 && N % 4 == 0 && epi.splitN % 4 == 0;
+            splitReduceKernel<<<gridFor(count / 4 + 1, kBlock), kBlock, 0, s>>>(partial.as<float>(), epi, count, sliceStride, int(sl), vec, N);
+            BF_LAUNCH_CHECK();
+            return BF_OK;
+        }
+    }
     const size_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     constexpr size_t smem = size_t(2) * (128 + 128) * LDS_ROW * sizeof(unsigned short);
     auto kernel = gemmBf16NtKernel<128, 128, 2, 2>;
