@@ -236,6 +236,10 @@ def bench_extras(bf, steps):
         extras[f"matmul_bf16_fp32_io_{m}x{n_}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(2 * m * n_ * k / ms / 1e9, 1)}
     gemm(4096, 4096, 4096)
     gemm(16384, 8192, 2048)
+    # GPT-small shapes: FFN up, FFN down / its input gradient (tall and narrow: 128-row tiles), FFN weight gradient (K slices)
+    gemm(8192, 3072, 768)
+    gemm(8192, 768, 3072)
+    gemm(768, 3072, 8192)
     return extras
 
 
