@@ -99,6 +99,37 @@ def test_attention_backward_recompute_route(hip, oracle, rng, recompute_route, b
         assert_close(got, exp, what=f"{name} case {(batch, heads, new_len, old_len, hd)}", scale=sc[name])
 
 
+def test_backward_routes_agree_on_random_shapes(hip):
+    """dS hand-over against recomputation on seeded random shapes (ragged lengths, offsets from 0 up to no mask at all,
+    every head-dim class): the two routes run different kernels for dQ and must agree to fp32 rounding; dK and dV come
+    from the same arithmetic with and without the dS stores and must agree bit for bit."""
+    shapes = np.random.default_rng(77)
+    for case in range(14):
+        batch, heads = int(shapes.integers(1, 4)), int(shapes.integers(1, 5))
+        hd = int(shapes.choice([4, 20, 32, 48, 64, 100, 128, 160]))
+        new_len = int(shapes.integers(1, 330))
+        old_len = int(shapes.choice([0, 0, 1, 17, 64, 200]))
+        total = old_len + new_len if shapes.random() < 0.7 else int(shapes.integers(1, 400))
+        if total != old_len + new_len:
+            old_len = int(shapes.choice([0, total // 2, total]))   # the offset need not tie the two lengths together
+        dim = heads * hd
+        data = np.random.default_rng(1000 + case)
+        q, k, v, go = r(data, batch, new_len, dim), r(data, batch, total, dim), r(data, batch, total, dim), r(data, batch, new_len, dim)
+        scale = float(f32(1.0) / np.sqrt(f32(hd)))
+        what = f"case {case}: batch {batch} heads {heads} hd {hd} newLen {new_len} totalLen {total} oldLen {old_len}"
+        print(what, flush=True)
+        _, _, _, dq, dk, dv = run_gpu(hip, q, k, v, go, heads, scale, old_len)
+        hip.capi.call("bf_hip_attention_set_workspace_limit", 0)
+        try:
+            _, _, _, dq2, dk2, dv2 = run_gpu(hip, q, k, v, go, heads, scale, old_len)
+        finally:
+            hip.capi.call("bf_hip_attention_set_workspace_limit", 2 ** 64 - 1)
+        sc = grad_scales(q, k, v, go, scale)
+        assert_close(dq, dq2, what="dQ " + what, scale=sc["dQ"])
+        assert_bits_equal(dk, dk2, "dK " + what)
+        assert_bits_equal(dv, dv2, "dV " + what)
+
+
 @pytest.mark.parametrize("batch,heads,new_len,old_len,hd", [(2, 2, 70, 0, 16), (1, 3, 45, 100, 64), (1, 1, 130, 3, 128), (1, 2, 33, 0, 200)])
 def test_ds_hand_over_buffer(hip, rng, batch, heads, new_len, old_len, hd):
     """The dS sub-blocks that the dK/dV kernel leaves for the dQ kernel, against dS = P * (dP - D) in float64, and
