@@ -1026,9 +1026,9 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
     if (st != BF_OK) return st;
     // With room for the dS hand-over buffer the dK/dV kernel leaves dS behind and dQ is one contraction over it.
     const size_t handOver = dsBytes(batch, heads, newLen, totalLen);
-    if (newLen > 0 && totalLen > 0 && handOver <= dsLimit()) {
-        Scratch ds(handOver);
-        if (ds.status != BF_OK) return ds.status;
+    Scratch ds(newLen > 0 && totalLen > 0 && handOver <= dsLimit() ? handOver : 0);
+    if (ds.status != BF_OK) (void)hipGetLastError();   // no room for the buffer after all: recompute instead
+    if (ds.status == BF_OK && ds.ptr != nullptr) {
         st = bf_hip_attention_backward_dkv_ds(dOut, q, k, v, lse2, dvec, dK, dV, ds.as<float>(), batch, heads, newLen, totalLen, dim, scale,
                                               oldLen, stream);
         if (st != BF_OK) return st;
