@@ -85,6 +85,7 @@ SIGNATURES = {
     "bf_hip_cvt_f32_bf16": [P, P, c_size, S],
     "bf_hip_cvt_f32_bf16_transpose": [P, P, c_size, c_size, S],
     "bf_hip_gemm_bf16_nt": [P, P, P, c_size, c_size, c_size, S],
+    "bf_hip_gemm_bf16_tn": [P, P, P, c_size, c_size, c_size, S],
     "bf_hip_matmul_bf16": [P, P, P, c_size, c_size, c_size, c_int, S],
     "bf_hip_matmul_bf16_backward": [P, P, P, P, P, c_size, c_size, c_size, c_int, S],
     "bf_hip_linear_bf16": [P, P, P, P, P, c_size, c_size, c_size, c_int, S],

@@ -443,6 +443,143 @@ __global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restr
     }
 }
 
+// The same kernel for operands that lie the other way round: C[M,N] = A^T * B with A [K, lda] and B [K, ldb], the
+// contraction index K running over ROWS (a weight gradient dW = X^T * G: both the activations X and the gradient G have
+// one row per token).  A K step is 64 rows of either operand, staged in LDS as they lie in memory ([k][m], rows padded
+// to pitch = width + 32 elements); the MFMA fragments, which want eight consecutive k per lane, are gathered by the LDS
+// transposing read (ds_read_b64_tr_b16: within 16 lanes, lane j receives element j%4 of the 8-byte pieces addressed by
+// lanes j/4, j/4 + 4, j/4 + 8, j/4 + 12; with lane i addressing row i/4, columns 4*(i%4).. of a 4 x 16 block, lane j
+// ends up with the four rows of column j).  No transposed operand image is ever written to HBM.  The pitch is 64 bytes
+// more than a multiple of 256, which spreads the 4 rows x 2 column blocks that half a wavefront reads over all banks.
+typedef short short4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x8 readTransposed8(const unsigned short* p, int rowPitch) {
+    typedef __attribute__((address_space(3))) short4v* LdsPtr;
+    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(p));
+    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(p + 4 * rowPitch));
+    typedef short short8v __attribute__((ext_vector_type(8)));
+    const short8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8, both);
+}
+
+template <int XCD_ORDER, int BM>
+__global__ void __launch_bounds__(512, 2) gemmBf16TnPingPongKernel(const unsigned short* __restrict__ A,
+                                                                   const unsigned short* __restrict__ B, Epilogue epi,
+                                                                   int M, int N, int K, int lda, int ldb, int gmLog, int gnLog,
+                                                                   int kPerSplit, size_t sliceStride) {
+    constexpr int BN = 256, TM = BM / 64, TN = 2, A_PASSES = BM / 64;
+    constexpr int PITCH_A = BM + 32, PITCH_B = BN + 32;           // elements
+    constexpr int A_THREADS_PER_ROW = BM / 8, A_ROWS_PER_PASS = 512 / A_THREADS_PER_ROW;   // 16-byte pieces
+    constexpr int B_THREADS_PER_ROW = BN / 8, B_ROWS_PER_PASS = 512 / B_THREADS_PER_ROW;
+    static_assert(A_ROWS_PER_PASS * A_PASSES == 64 && B_ROWS_PER_PASS * 4 == 64, "a K step is 64 rows");
+    extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
+    unsigned short* as = lds;                             // [2][64][PITCH_A]
+    unsigned short* bs = lds + 2 * 64 * PITCH_A;          // [2][64][PITCH_B]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    const int group = wave >> 2;
+    int tm, tn;
+    if (XCD_ORDER) {
+        if (!tileIndexXcd(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, gmLog, gnLog, tm, tn)) return;
+    } else {
+        tileIndexGrouped(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+    }
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int wm0 = group * (BM / 2), wn0 = (wave & 3) * 64;
+    const int kBegin = blockIdx.y * kPerSplit, kEnd = min(K, kBegin + kPerSplit);
+    epi.c[0] += size_t(blockIdx.y) * sliceStride;
+    const int steps = max((kEnd - kBegin + BKK - 1) / BKK, 1);
+
+    // staging: thread -> (row of the K step, 16-byte piece of that row); columns past the operand's width are clamped
+    // into it (their products are never stored), rows past kEnd are clamped to the last row and stored as zeros
+    const int aRow = tid / A_THREADS_PER_ROW, aCol = (tid % A_THREADS_PER_ROW) * 8;
+    const int bRow = tid / B_THREADS_PER_ROW, bCol = (tid % B_THREADS_PER_ROW) * 8;
+    const unsigned short* aSrc = A + min(m0 + aCol, lda - 8);
+    const unsigned short* bSrc = B + min(n0 + bCol, ldb - 8);
+    uint4v stageA[A_PASSES], stageB[4];
+    auto loadA = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_PASSES; ++i)
+            stageA[i] = *reinterpret_cast<const uint4v*>(aSrc + size_t(min(k0 + aRow + A_ROWS_PER_PASS * i, K - 1)) * lda);
+    };
+    auto loadB = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            stageB[i] = *reinterpret_cast<const uint4v*>(bSrc + size_t(min(k0 + bRow + B_ROWS_PER_PASS * i, K - 1)) * ldb);
+    };
+    auto storeA = [&](int buf, int k0) {
+#pragma unroll
+        for (int i = 0; i < A_PASSES; ++i)
+            *reinterpret_cast<uint4v*>(as + (buf * 64 + aRow + A_ROWS_PER_PASS * i) * PITCH_A + aCol) =
+                zeroPast(stageA[i], k0 + aRow + A_ROWS_PER_PASS * i, kEnd);
+    };
+    auto storeB = [&](int buf, int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            *reinterpret_cast<uint4v*>(bs + (buf * 64 + bRow + B_ROWS_PER_PASS * i) * PITCH_B + bCol) =
+                zeroPast(stageB[i], k0 + bRow + B_ROWS_PER_PASS * i, kEnd);
+    };
+
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    loadA(kBegin);
+    loadB(kBegin);
+    storeA(0, kBegin);
+    storeB(0, kBegin);
+    if (steps > 1) {
+        loadA(kBegin + BKK);
+        loadB(kBegin + BKK);
+    }
+    __syncthreads();
+    if (group == 1) __builtin_amdgcn_s_barrier();    // group 1 starts one phase late
+    // this lane's corner of a fragment's 16-row x 32-column block: lanes 0-15 and 16-31 take the two 16-column halves,
+    // lanes 32-63 the rows eight further down; inside 16 lanes, lane i addresses row i/4, columns 4*(i%4)..
+    const int fragRow = (lane >> 5) * 8 + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    bf16x8 a[2][TM], b[2][TN];
+    for (int T = 0; T < steps; ++T) {
+        const int par = T & 1;
+        const unsigned short* ac = as + (par * 64 + fragRow) * PITCH_A + wm0 + fragCol;
+        const unsigned short* bc = bs + (par * 64 + fragRow) * PITCH_B + wn0 + fragCol;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            // ---- memory phase
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) a[kk][i] = readTransposed8(ac + (h * 32 + kk * 16) * PITCH_A + i * 32, PITCH_A);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) b[kk][j] = readTransposed8(bc + (h * 32 + kk * 16) * PITCH_B + j * 32, PITCH_B);
+            }
+            if (T + 1 < steps) {
+                if (h == 0) {
+                    storeA(par ^ 1, kBegin + (T + 1) * BKK);
+                    if (T + 2 < steps) loadA(kBegin + (T + 2) * BKK);
+                } else {
+                    storeB(par ^ 1, kBegin + (T + 1) * BKK);
+                    if (T + 2 < steps) loadB(kBegin + (T + 2) * BKK);
+                }
+            }
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- compute phase
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+        }
+    }
+    if (group == 0) __builtin_amdgcn_s_barrier();    // pairs with group 1's last barrier
+    storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
+}
+
 template <typename Kernel>
 int allowSharedMemory(Kernel kernel, size_t smem) {
     return allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
@@ -483,6 +620,106 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
         kernel<<<dim3(unsigned(grid), unsigned(slices)), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), 0, 0,
                                                                          int(kPer), sliceStride);
     }
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+template <int BM>
+int launchPingPongTn(const unsigned short* A, const unsigned short* B, const Epilogue& epi, size_t M, size_t N, size_t K,
+                     size_t lda, size_t ldb, hipStream_t s, size_t slices, size_t kPer, size_t sliceStride) {
+    const size_t tilesM = (M + BM - 1) / BM, tilesN = (N + 255) / 256;
+    constexpr size_t smem = size_t(2) * 64 * ((BM + 32) + (256 + 32)) * sizeof(unsigned short);
+    int gmLog = 2, gnLog = 3;
+    size_t bestCost = 0, blocks = 0;
+    for (int g = 0; g <= 5; ++g) {
+        size_t gm = size_t(1) << g, gn = size_t(32) >> g;
+        size_t nb = ((tilesM + gm - 1) / gm) * ((tilesN + gn - 1) / gn);
+        size_t cost = nb * 1000 + gm + gn;
+        if (g == 0 || cost < bestCost) { bestCost = cost; gmLog = g; gnLog = 5 - g; blocks = nb; }
+    }
+    const bool xcdOrder = blocks * 32 <= (tilesM * tilesN) * 5 / 4 && (blocks % 8 == 0 || blocks >= 64);
+    if (xcdOrder) {
+        size_t grid = (blocks + 7) / 8 * 8 * 32;
+        if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+        auto kernel = gemmBf16TnPingPongKernel<1, BM>;
+        int st = allowSharedMemory(kernel, smem);
+        if (st != BF_OK) return st;
+        kernel<<<dim3(unsigned(grid), unsigned(slices)), 512, smem, s>>>(A, B, epi, int(M), int(N), int(K), int(lda), int(ldb), gmLog, gnLog,
+                                                                         int(kPer), sliceStride);
+    } else {
+        size_t grid = tilesM * tilesN;
+        if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+        auto kernel = gemmBf16TnPingPongKernel<0, BM>;
+        int st = allowSharedMemory(kernel, smem);
+        if (st != BF_OK) return st;
+        kernel<<<dim3(unsigned(grid), unsigned(slices)), 512, smem, s>>>(A, B, epi, int(M), int(N), int(K), int(lda), int(ldb), 0, 0,
+                                                                         int(kPer), sliceStride);
+    }
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+// C = A^T B for products too small for the tile kernel to matter: one thread per output element.
+__global__ void __launch_bounds__(kBlock) gemmBf16TnSmallKernel(const unsigned short* __restrict__ A, const unsigned short* __restrict__ B,
+                                                                float* __restrict__ C, size_t M, size_t N, size_t K, size_t lda, size_t ldb) {
+    const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= M * N) return;
+    const size_t i = idx / N, j = idx - i * N;
+    float acc = 0.0f;
+    for (size_t k = 0; k < K; ++k)
+        acc += __uint_as_float(unsigned(A[k * lda + i]) << 16) * __uint_as_float(unsigned(B[k * ldb + j]) << 16);
+    C[idx] = acc;
+}
+
+// Form (256- or 128-row tiles) and number of K slices for a product on the large-tile kernels, by the estimate
+// described at launchGemmNt; false when even the best plan leaves more than half of the CUs without a workgroup.
+bool planLargeTiles(size_t M, size_t N, size_t K, int* form, size_t* slices) {
+    const size_t cus = size_t(computeUnits());
+    const size_t bigTiles = ((M + 255) / 256) * ((N + 255) / 256), halfTiles = ((M + 127) / 128) * ((N + 255) / 256);
+    const size_t stepsAll = (K + BKK - 1) / BKK;
+    constexpr double kHalfTileCost = 0.78;
+    double best = 1e30;
+    for (int f = 0; f < 2; ++f) {
+        const size_t t = f == 0 ? bigTiles : halfTiles;
+        for (size_t sl = 1; sl <= 16 && (sl == 1 || sl * 8 <= stepsAll); ++sl) {
+            if (t * sl < cus / 2) continue;
+            const size_t rounds = (t * sl + cus - 1) / cus;
+            const double gemmUs = double(rounds) * double((stepsAll + sl - 1) / sl) * 1.4 * (f == 0 ? 1.0 : kHalfTileCost);
+            const double reduceUs = sl == 1 ? 0.0 : double(sl + 1) * double(M * N) * 2.0 * sizeof(float) / 4e6;
+            if (gemmUs + reduceUs < best) { best = gemmUs + reduceUs; *form = f; *slices = sl; }
+        }
+    }
+    return best < 1e30;
+}
+
+// C[M,N] = A^T B for A [K, lda], B [K, ldb] (see gemmBf16TnPingPongKernel).  *done = false, and nothing launched, when the
+// product is too small for the large-tile kernel (the caller then builds transposed images and uses launchGemmNt).
+int launchGemmTn(const unsigned short* A, const unsigned short* B, const Epilogue& epi, size_t M, size_t N, size_t K, size_t lda,
+                 size_t ldb, hipStream_t s, bool* done) {
+    *done = false;
+    if (M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+    int form = 0;
+    size_t slices = 1;
+    if (lda < 8 || ldb < 8 || !planLargeTiles(M, N, K, &form, &slices)) return BF_OK;
+    const size_t stepsAll = (K + BKK - 1) / BKK;
+    const size_t kPer = (stepsAll + slices - 1) / slices * BKK;
+    slices = (K + kPer - 1) / kPer;
+    *done = true;
+    if (slices <= 1) {
+        return form == 0 ? launchPingPongTn<256>(A, B, epi, M, N, K, lda, ldb, s, 1, K, 0)
+                         : launchPingPongTn<128>(A, B, epi, M, N, K, lda, ldb, s, 1, K, 0);
+    }
+    const size_t count = M * N, sliceStride = (count + 3) / 4 * 4;
+    Scratch partial(slices * sliceStride * sizeof(float));
+    if (partial.status != BF_OK) return partial.status;
+    Epilogue plain{{partial.as<float>(), nullptr, nullptr}, int(N), nullptr, nullptr};
+    int st = form == 0 ? launchPingPongTn<256>(A, B, plain, M, N, K, lda, ldb, s, slices, kPer, sliceStride)
+                       : launchPingPongTn<128>(A, B, plain, M, N, K, lda, ldb, s, slices, kPer, sliceStride);
+    if (st != BF_OK) return st;
+    const int vec = ((reinterpret_cast<uintptr_t>(epi.c[0]) | reinterpret_cast<uintptr_t>(epi.c[1]) |
+                      reinterpret_cast<uintptr_t>(epi.c[2]) | reinterpret_cast<uintptr_t>(epi.residual) |
+                      reinterpret_cast<uintptr_t>(epi.bias)) & 15u) == 0 && N % 4 == 0 && epi.splitN % 4 == 0;
+    splitReduceKernel<<<gridFor(count / 4 + 1, kBlock), kBlock, 0, s>>>(partial.as<float>(), epi, count, sliceStride, int(slices), vec, N);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -707,6 +944,21 @@ int bf_hip_gemm_bf16_nt(const uint16_t* A, const uint16_t* Bt, float* C, size_t 
     return launchGemmNt(A, Bt, C, M, N, K, K, K, asStream(stream));
 }
 
+int bf_hip_gemm_bf16_tn(const uint16_t* A, const uint16_t* B, float* C, size_t M, size_t N, size_t K, bf_stream_t stream) {
+    if (M == 0 || N == 0) return BF_OK;
+    BF_REQUIRE(C != nullptr, "NULL output");
+    if (K == 0) return bf_hip_fill_zero(C, M * N * sizeof(float), stream);
+    BF_REQUIRE(A && B, "NULL operand");
+    BF_REQUIRE(M % 8 == 0 && N % 8 == 0, "M and N must be multiples of 8 (16-byte operand rows)");
+    BF_REQUIRE(((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15u) == 0, "operands must be 16-byte aligned");
+    bool done = false;
+    int st = launchGemmTn(A, B, Epilogue{{C, nullptr, nullptr}, int(N), nullptr, nullptr}, M, N, K, M, N, asStream(stream), &done);
+    if (st != BF_OK || done) return st;
+    gemmBf16TnSmallKernel<<<gridFor(M * N, kBlock, 1u << 30), kBlock, 0, asStream(stream)>>>(A, B, C, M, N, K, M, N);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
 int bf_hip_matmul_bf16(const float* a, const float* b, float* c, size_t m, size_t k, size_t n, int cacheWeight,
                        bf_stream_t stream) {
     if (m == 0 || n == 0) return BF_OK;
@@ -739,17 +991,24 @@ int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, 
     }
     BF_REQUIRE(a && b && g, "NULL operand");
     int st = BF_OK;
-    const size_t mp = pad8(m);
-    Scratch gT(dB ? n * mp * sizeof(unsigned short) : 0);
+    const size_t mp = pad8(m), np = pad8(n), kp = pad8(k);
+    // dB = a^T g contracts over the rows of both operands.  When the product is big enough for the large-tile kernel
+    // that transposes fragments on their way out of LDS, both operands are converted as they lie (g's plain image also
+    // serves dA); otherwise transposed images are built and the row-by-row kernel is used.
+    int form = 0;
+    size_t slices = 1;
+    const bool transposeInLds = dB != nullptr && planLargeTiles(k, n, m, &form, &slices);
+    Scratch gT(dB && !transposeInLds ? n * mp * sizeof(unsigned short) : 0);
     if (gT.status != BF_OK) return gT.status;
-    if (dA) {   // dA[m,k] = g[m,n] * b[k,n]^T : contraction over n
-        const size_t np = pad8(n);
-        Scratch gImg(m * np * sizeof(unsigned short));
-        if (gImg.status != BF_OK) return gImg.status;
-        // with both gradients wanted, one pass over g writes the plain image for this product and the transposed one for dB
-        if (dB) st = convertTransposed(g, gT.as<unsigned short>(), m, n, s, true, gImg.as<unsigned short>(), np);
+    Scratch gImg(dA || transposeInLds ? m * np * sizeof(unsigned short) : 0);
+    if (gImg.status != BF_OK) return gImg.status;
+    if (dA || transposeInLds) {
+        // with both gradients wanted on the transposed-image route, one pass over g writes the plain and the transposed image
+        if (dB && !transposeInLds) st = convertTransposed(g, gT.as<unsigned short>(), m, n, s, true, gImg.as<unsigned short>(), np);
         else st = convertPlain(g, gImg.as<unsigned short>(), m, n, s);
         if (st != BF_OK) return st;
+    }
+    if (dA) {   // dA[m,k] = g[m,n] * b[k,n]^T : contraction over n
         unsigned short* bImg = nullptr;
         size_t bBytes = 0;
         st = weightImage(b, k, n, /*transposed=*/false, cacheWeight != 0, s, &bImg, &bBytes);
@@ -757,6 +1016,15 @@ int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, 
         st = launchGemmNt(gImg.as<unsigned short>(), bImg, dA, m, k, np, np, np, s);
         if (!cacheWeight) bf_hip_pool_release(bImg, bBytes);
         if (st != BF_OK) return st;
+    }
+    if (dB && transposeInLds) {
+        Scratch aImg(m * kp * sizeof(unsigned short));
+        if (aImg.status != BF_OK) return aImg.status;
+        st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
+        if (st != BF_OK) return st;
+        bool done = false;
+        return launchGemmTn(aImg.as<unsigned short>(), gImg.as<unsigned short>(), Epilogue{{dB, nullptr, nullptr}, int(n), nullptr, nullptr}, k, n,
+                            m, kp, np, s, &done);
     }
     if (dB) {   // dB[k,n] = a[m,k]^T * g[m,n] : contraction over m
         Scratch aT(k * mp * sizeof(unsigned short));
@@ -854,8 +1122,41 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
     BF_REQUIRE(a != nullptr, "NULL operand");
     for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] && g[i], "NULL operand");
     int st = BF_OK;
-    bool anyDb = false;
+    bool anyDb = false, allDb = dB != nullptr;
     for (size_t i = 0; dB && i < count; ++i) anyDb = anyDb || dB[i] != nullptr;
+    for (size_t i = 0; dB && i < count; ++i) allDb = allDb && dB[i] != nullptr;
+    {
+        // Every gradient wanted and the weight-gradient product big enough for the kernel that transposes fragments in
+        // LDS: the gradients are converted once, side by side and as they lie; that image is the A operand of the
+        // input-gradient product and the B operand of the weight-gradient product, whose other operand is the plain
+        // image of `a`.  No transposed image is built.
+        int form = 0;
+        size_t slices = 1;
+        const size_t nn = count * n;
+        if (dA && allDb && count > 1 && n % 256 == 0 && planLargeTiles(k, nn, m, &form, &slices)) {
+            const size_t kp = pad8(k);
+            Scratch gImg(m * nn * sizeof(unsigned short));
+            if (gImg.status != BF_OK) return gImg.status;
+            for (size_t i = 0; i < count; ++i) {
+                st = convertPlain(g[i], gImg.as<unsigned short>() + i * n, m, n, s, nn);
+                if (st != BF_OK) return st;
+            }
+            unsigned short* wImg = nullptr;
+            size_t wBytes = 0;
+            st = weightImage(b, count, k, n, 3, cacheWeight != 0, s, &wImg, &wBytes);
+            if (st != BF_OK) return st;
+            st = launchGemmNt(gImg.as<unsigned short>(), wImg, dA, m, k, nn, nn, nn, s);
+            if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+            if (st != BF_OK) return st;
+            Scratch aImg(m * kp * sizeof(unsigned short));
+            if (aImg.status != BF_OK) return aImg.status;
+            st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
+            if (st != BF_OK) return st;
+            Epilogue epi{{dB[0], count > 1 ? dB[1] : nullptr, count > 2 ? dB[2] : nullptr}, int(n), nullptr, nullptr};
+            bool done = false;
+            return launchGemmTn(aImg.as<unsigned short>(), gImg.as<unsigned short>(), epi, k, nn, m, kp, nn, s, &done);
+        }
+    }
     const size_t mp = pad8(m);
     Scratch gT(anyDb ? count * n * mp * sizeof(unsigned short) : 0);   // transposed gradient images, stacked
     if (gT.status != BF_OK) return gT.status;

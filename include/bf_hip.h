@@ -189,6 +189,11 @@ int bf_hip_cvt_f32_bf16_transpose(const float* x, uint16_t* out, size_t rows, si
  * (the cublasLtMatmul call, ops_tensorcore.cu:293-304). */
 int bf_hip_gemm_bf16_nt(const uint16_t* A, const uint16_t* Bt, float* C, size_t M, size_t N, size_t K,
                         bf_stream_t stream);
+/* C[M,N] (fp32) = A^T * B for bf16 A[K,M] and B[K,N] (M, N multiples of 8): the contraction runs over rows, the
+ * form of a weight gradient dB = a^T g (the CUBLAS_OP_T product of matmulBf16Backward, ops_tensorcore.cu:409-411).
+ * Operand fragments are transposed on their way out of LDS; no transposed image is built. */
+int bf_hip_gemm_bf16_tn(const uint16_t* A, const uint16_t* B, float* C, size_t M, size_t N, size_t K,
+                        bf_stream_t stream);
 /* matmulBf16 ops.hpp:53 (cacheWeight = 0) / matmulBf16CachedWeight ops.hpp:72 (cacheWeight = 1):
  * c[m,n] = bf16(a[m,k]) * bf16(b[k,n]), fp32 accumulate.  With cacheWeight the bf16 image of `b` is kept
  * per (device, pointer) until bf_hip_invalidate_bf16_weight_cache(). */

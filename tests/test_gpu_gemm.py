@@ -120,6 +120,37 @@ def test_bf16_gradients_with_long_contraction(hip, oracle, rng, m, k, n):
     assert_bits_equal(again.toHost(), dB.toHost(), "sliced contraction must be deterministic")
 
 
+@pytest.mark.parametrize("m,k,n", [(8192, 520, 776), (6001, 300, 1100), (16384, 264, 520)])
+def test_bf16_weight_gradient_transposed_in_lds(hip, oracle, rng, m, k, n):
+    """Token counts long enough, and weight shapes wide enough, that dB = a^T g runs on the kernel that contracts over
+    the ROWS of both operands (fragments transposed on their way out of LDS, K cut into slices): against float64 on
+    the bf16-rounded operands, ragged in every dimension, and bit-reproducible."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b, g = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, m, n)
+    ar, br, gr = (oracle.roundToBf16(t).astype(np.float64) for t in (a, b, g))
+    dA, dB = ops.matmulBf16Backward(*map(D.fromHost, (a, b, g)))
+    assert_close(dA.toHost(), (gr @ br.T).astype(f32), tol=1e-4, what="bf16 dA vs rounded operands")
+    assert_close(dB.toHost(), (ar.T @ gr).astype(f32), tol=1e-4, what="bf16 dB vs rounded operands")
+    da_, db_, dg_, only = D.fromHost(a), D.fromHost(b), D.fromHost(g), D((k, n))
+    hip.capi.call("bf_hip_matmul_bf16_backward", da_.ptr, db_.ptr, dg_.ptr, None, only.ptr, m, k, n, 0, None)
+    assert_bits_equal(only.toHost(), dB.toHost(), "dB must not depend on whether dA is requested, and must be deterministic")
+
+
+@pytest.mark.parametrize("m,n,k", [(768, 768, 8192), (1000, 520, 4100), (264, 3080, 9000), (40, 24, 100), (8, 8, 3)])
+def test_bf16_gemm_tn_entry(hip, rng, m, n, k):
+    """bf_hip_gemm_bf16_tn: C = A^T B for bf16 A[K,M], B[K,N]: sliced large tiles, a K tail, and the small-product form."""
+    D = hip.DeviceTensor
+    def bf16(x):
+        bits = (x.view(np.uint32) >> 16).astype(np.uint16)
+        return bits, (bits.astype(np.uint32) << 16).view(f32)
+    (abits, a), (bbits, b) = bf16(r(rng, k, m)), bf16(r(rng, k, n))
+    da, db, c = D((k, m), itemsize=2), D((k, n), itemsize=2), D((m, n))
+    hip.capi.call("bf_hip_memcpy_h2d", da.ptr, abits.ctypes.data, abits.nbytes)
+    hip.capi.call("bf_hip_memcpy_h2d", db.ptr, bbits.ctypes.data, bbits.nbytes)
+    hip.capi.call("bf_hip_gemm_bf16_tn", da.ptr, db.ptr, c.ptr, m, n, k, None)
+    assert_close(c.toHost(), (a.astype(np.float64).T @ b.astype(np.float64)).astype(f32), tol=1e-5, what="gemm_bf16_tn")
+
+
 @pytest.mark.parametrize("m,k,n", [(3500, 200, 3700), (4000, 136, 4090), (8192, 64, 2048), (8192, 200, 768), (8100, 136, 700),
                                    (6200, 72, 1500)])
 def test_bf16_projection_large_tile_kernel(hip, oracle, rng, m, k, n):
@@ -154,7 +185,7 @@ def test_bf16_linear_with_adds_in_the_store(hip, oracle, rng, m, k, n, with_bias
 
 
 @pytest.mark.parametrize("m,k,n,count", [(50, 40, 24, 3), (300, 136, 256, 3), (4096, 64, 1024, 3), (4100, 256, 256, 3), (260, 72, 512, 2),
-                                         (64, 32, 48, 1)])
+                                         (64, 32, 48, 1), (8192, 520, 256, 3), (8200, 300, 512, 2)])
 @pytest.mark.parametrize("cached", [False, True])
 def test_bf16_projections_of_a_shared_input(hip, oracle, rng, m, k, n, count, cached):
     """Q/K/V-style projections of one input and their gradients (ops_transformer.cu:217-257, autodiff.cu:756-798) against
