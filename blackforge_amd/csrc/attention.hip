@@ -166,6 +166,26 @@ __device__ __forceinline__ float16v headDotB(const float* __restrict__ ldsRow, c
     return acc;
 }
 
+// Two such contractions at once (S = Q K^T and dP = dO V^T of the key-owner kernel), their MFMAs alternating: a
+// 32x32x2 MFMA whose accumulator is the previous instruction's result issues a few clocks late, so two independent
+// accumulator chains keep the matrix pipe fuller than one chain after the other.
+template <int HDP>
+__device__ __forceinline__ void headDotPairB(const float* __restrict__ ldsRow0, const float* __restrict__ ldsRow1,
+                                             const float (&reg0)[HDP / 2], const float (&reg1)[HDP / 2], float16v& acc0, float16v& acc1) {
+#pragma unroll
+    for (int t = 0; t < HDP / 2; t += 4) {
+        const float4v a0 = loadf4(ldsRow0 + t), a1 = loadf4(ldsRow1 + t);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, reg0[t], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.x, reg1[t], acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, reg0[t + 1], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.y, reg1[t + 1], acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, reg0[t + 2], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.z, reg1[t + 2], acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, reg0[t + 3], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.w, reg1[t + 3], acc1, 0, 0, 0);
+    }
+}
+
 // Row index inside a 32-row MFMA block held by register r of a lane in half `half`.
 __device__ __forceinline__ int dRow(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }
 
@@ -394,15 +414,15 @@ __device__ __forceinline__ void dqTile(const float* __restrict__ ks, const float
     float16v s[NSB], dp[NSB];
 #pragma unroll
     for (int r = 0; r < 16; ++r) { s[0][r] = 0.0f; dp[0][r] = 0.0f; }
-    s[0] = headDot<HDP>(ks + li * LDSW + half * (HDP / 2), qreg, s[0]);      // S^T  = K * Q^T
-    dp[0] = headDot<HDP>(vs + li * LDSW + half * (HDP / 2), greg, dp[0]);    // dP^T = V * dO^T
+    // S^T = K * Q^T and dP^T = V * dO^T, their MFMAs alternating
+    headDotPairB<HDP>(ks + li * LDSW + half * (HDP / 2), vs + li * LDSW + half * (HDP / 2), qreg, greg, s[0], dp[0]);
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb) {
         if (sb + 1 < NSB) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) { s[sb + 1][r] = 0.0f; dp[sb + 1][r] = 0.0f; }
-            s[sb + 1] = headDot<HDP>(ks + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), qreg, s[sb + 1]);
-            dp[sb + 1] = headDot<HDP>(vs + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), greg, dp[sb + 1]);
+            headDotPairB<HDP>(ks + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), vs + ((sb + 1) * 32 + li) * LDSW + half * (HDP / 2), qreg, greg,
+                              s[sb + 1], dp[sb + 1]);
         }
         float16v& ds = s[sb];
 #pragma unroll
@@ -621,8 +641,7 @@ __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const floa
         float16v& dpDst = dp[AHEAD ? sb : 0];
 #pragma unroll
         for (int r = 0; r < 16; ++r) { sDst[r] = 0.0f; dpDst[r] = 0.0f; }
-        sDst = headDotB<HDP>(qs + (sb * 32 + li) * LDSW + half * (HDP / 2), kreg, sDst);
-        dpDst = headDotB<HDP>(gs + (sb * 32 + li) * LDSW + half * (HDP / 2), vreg, dpDst);
+        headDotPairB<HDP>(qs + (sb * 32 + li) * LDSW + half * (HDP / 2), gs + (sb * 32 + li) * LDSW + half * (HDP / 2), kreg, vreg, sDst, dpDst);
     };
     if constexpr (AHEAD) scores(0);
 #pragma unroll
