@@ -206,19 +206,30 @@ __global__ void __launch_bounds__(256) columnSumKernel(const float* __restrict__
     }
 }
 
-// out[c] = sum of the partial rows of column c.  64 columns per block; four lanes per column each add every
-// fourth partial row (in index order) and the four sums are combined in a fixed order.
+// out[c] = sum of the partial rows of column c.  16 columns per block; sixteen lanes per column each add every
+// sixteenth partial row (in index order, eight loads in flight) and the sixteen sums are combined in a fixed order.
 __global__ void __launch_bounds__(kBlock) columnFinishKernel(const float* __restrict__ partial, float* __restrict__ out,
                                                              size_t parts, size_t features) {
-    __shared__ float lds[4][64];
-    const int cx = threadIdx.x & 63, lane4 = threadIdx.x >> 6;
-    const size_t c = size_t(blockIdx.x) * 64 + cx;
+    __shared__ float lds[16][17];
+    const int cx = threadIdx.x & 15, part = threadIdx.x >> 4;
+    const size_t c = size_t(blockIdx.x) * 16 + cx;
     float s = 0.0f;
-    if (c < features)
-        for (size_t p = lane4; p < parts; p += 4) s += partial[p * features + c];
-    lds[lane4][cx] = s;
+    if (c < features) {
+#pragma unroll 8
+        for (size_t p = part; p < parts; p += 16) s += partial[p * features + c];
+    }
+    lds[part][cx] = s;
     __syncthreads();
-    if (lane4 == 0 && c < features) out[c] = (lds[0][cx] + lds[1][cx]) + (lds[2][cx] + lds[3][cx]);
+    if (part == 0 && c < features) {
+        float t[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t[i] = lds[i][cx];
+#pragma unroll
+        for (int w = 8; w > 0; w >>= 1)
+#pragma unroll
+            for (int i = 0; i < w; ++i) t[i] += t[i + w];
+        out[c] = t[0];
+    }
 }
 
 template <int FUSED, int ACT>
@@ -241,7 +252,7 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
         columnSumKernel<1, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
     BF_LAUNCH_CHECK();
     if (dBias) {
-        columnFinishKernel<<<gridFor(features, 64), kBlock, 0, stream>>>(partial, dBias, parts, features);
+        columnFinishKernel<<<gridFor(features, 16), kBlock, 0, stream>>>(partial, dBias, parts, features);
         BF_LAUNCH_CHECK();
     }
     return BF_OK;
