@@ -92,6 +92,8 @@ SIGNATURES = {
     "bf_hip_matmul_bf16_shared_input": [P, ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), c_size, c_size, c_size, c_size, c_int, S],
     "bf_hip_matmul_bf16_shared_input_backward": [P, ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), P, ctypes.POINTER(c_ptr), c_size,
                                                  c_size, c_size, c_size, c_int, S],
+    "bf_hip_feedforward_bf16": [P, P, P, P, P, P, c_int, P, P, P, P, c_size, c_size, c_size, c_int, S],
+    "bf_hip_feedforward_bf16_backward": [P, P, P, P, P, P, P, c_int, P, P, P, P, P, c_size, c_size, c_size, c_int, S],
     "bf_hip_invalidate_bf16_weight_cache": [],
     "bf_hip_attention_forward": [P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_attention_dot_o_do": [P, P, P, c_size, c_size, c_size, c_size, S],

@@ -131,6 +131,8 @@ __device__ __forceinline__ int owningTensor(const T* __restrict__ table, int num
     return notAfter - 1;
 }
 
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float4v loadf4(const float* p) { return *reinterpret_cast<const float4v*>(p); }
 __device__ __forceinline__ void storef4(float* p, float4v v) { *reinterpret_cast<float4v*>(p) = v; }
 
@@ -163,7 +165,19 @@ template <int ACT> __device__ __forceinline__ float actD(float x) {
     else if constexpr (ACT == BF_ACT_GELU) return geluD(x);
     else return reluD(x);
 }
+// fp32 -> bf16 bits, round to nearest even, NaN preserved (floatToBf16, ops_tensorcore.cu:21-26)
+__device__ __forceinline__ unsigned short toBf16Bits(float x) {
+    __bf16 h = static_cast<__bf16>(x);
+    return __builtin_bit_cast(unsigned short, h);
+}
 
 #endif  // __HIPCC__
+
+// Feed-forward helpers defined with the elementwise kernels and used by the bf16 GEMM entry points (features % 8 == 0,
+// 16-byte aligned pointers): image[i] = bf16(act(z[i])), and dzImage = bf16(dHidden * act'(z)) with the column sums of
+// that product before rounding in dBias (may be NULL).
+int actToBf16Image(const float* z, unsigned short* image, size_t n, int act, hipStream_t stream);
+int actBackwardToBf16Image(const float* z, const float* dHidden, unsigned short* dzImage, float* dBias, size_t rows,
+                           size_t features, int act, hipStream_t stream);
 
 }  // namespace bf

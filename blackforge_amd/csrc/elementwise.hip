@@ -85,6 +85,20 @@ struct ActBackwardOp {
     __device__ void one(size_t i) const { out[i] = g[i] * actD<ACT>(x[i]); }
 };
 
+// image[8i .. 8i+7] = bf16(act(z[8i .. 8i+7])): two 16-byte loads, one 16-byte store per thread
+template <int ACT>
+struct ActImageOp {
+    const float* z; unsigned short* image;
+    __device__ void vec(size_t i) const {
+        const float4v a = loadf4(z + 8 * i), b = loadf4(z + 8 * i + 4);
+        uint4v packed = {unsigned(toBf16Bits(actF<ACT>(a.x))) | unsigned(toBf16Bits(actF<ACT>(a.y))) << 16,
+                         unsigned(toBf16Bits(actF<ACT>(a.z))) | unsigned(toBf16Bits(actF<ACT>(a.w))) << 16,
+                         unsigned(toBf16Bits(actF<ACT>(b.x))) | unsigned(toBf16Bits(actF<ACT>(b.y))) << 16,
+                         unsigned(toBf16Bits(actF<ACT>(b.z))) | unsigned(toBf16Bits(actF<ACT>(b.w))) << 16};
+        *reinterpret_cast<uint4v*>(image + 8 * i) = packed;
+    }
+};
+
 // ---- row/column kernels (bias family) ---------------------------------------------------------
 // Thread layout: blockDim = (bx, by); a thread owns column group (blockIdx.x*bx + tx) and walks rows
 // blockIdx.y*by + ty, stepping gridDim.y*by.
@@ -156,20 +170,29 @@ __global__ void __launch_bounds__(256) biasKernel(const float* __restrict__ x, c
 template <int VEC, int FUSED, int ACT>
 __global__ void __launch_bounds__(256) columnSumKernel(const float* __restrict__ src, const float* __restrict__ bias,
                                                         const float* __restrict__ dHidden, float* __restrict__ dGemm,
-                                                        float* __restrict__ partial, size_t rows, size_t features) {
+                                                        float* __restrict__ partial, size_t rows, size_t features,
+                                                        unsigned short* __restrict__ image = nullptr) {
     __shared__ float lds[256 * 4];
     size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
     bool active = col < features;
     typename Pack<VEC>::T acc = {};
     if (active) {
         typename Pack<VEC>::T b = {};
-        if constexpr (FUSED) b = Pack<VEC>::load(bias + col);
+        if constexpr (FUSED) { if (bias) b = Pack<VEC>::load(bias + col); }
+        // FUSED: either output may be absent; `image` (four-column form only) receives the product rounded to bf16
         auto term = [&](size_t r) {
             size_t idx = r * features + col;
             typename Pack<VEC>::T v = Pack<VEC>::load(src + idx);
             if constexpr (FUSED) {
                 v = Pack<VEC>::load(dHidden + idx) * actD4<ACT>(v + b);
-                Pack<VEC>::store(dGemm + idx, v);
+                if (dGemm) Pack<VEC>::store(dGemm + idx, v);
+                if constexpr (VEC == 4) {
+                    if (image) {
+                        uint2v packed = {unsigned(toBf16Bits(v.x)) | unsigned(toBf16Bits(v.y)) << 16,
+                                         unsigned(toBf16Bits(v.z)) | unsigned(toBf16Bits(v.w)) << 16};
+                        *reinterpret_cast<uint2v*>(image + idx) = packed;
+                    }
+                }
             }
             return v;
         };
@@ -234,7 +257,7 @@ __global__ void __launch_bounds__(kBlock) columnFinishKernel(const float* __rest
 
 template <int FUSED, int ACT>
 int launchColumnSum(const float* src, const float* bias, const float* dHidden, float* dGemm, float* dBias,
-                    size_t rows, size_t features, hipStream_t stream) {
+                    size_t rows, size_t features, hipStream_t stream, unsigned short* image = nullptr) {
     if (features == 0) return BF_OK;
     if (rows == 0) {
         if (dBias) return bf_hip_fill_zero(dBias, features * sizeof(float), stream);
@@ -246,8 +269,9 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
     Scratch scratch(dBias ? parts * features * sizeof(float) : 0);
     if (scratch.status != BF_OK) return scratch.status;
     float* partial = dBias ? scratch.as<float>() : nullptr;
+    if (image && g.vec != 4) return failInvalid("act_backward_image", "operands must be 16-byte aligned and the width a multiple of 4");
     if (g.vec == 4)
-        columnSumKernel<4, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
+        columnSumKernel<4, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features, image);
     else
         columnSumKernel<1, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
     BF_LAUNCH_CHECK();
@@ -284,6 +308,26 @@ __global__ void __launch_bounds__(kBlock) zeroMultiKernel(const ZeroTensor* __re
 }
 
 }  // namespace
+
+int actToBf16Image(const float* z, unsigned short* image, size_t n, int act, hipStream_t stream) {
+    if (n == 0) return BF_OK;
+    if (n % 8 != 0 || !aligned16(z) || !aligned16(image)) return failInvalid("act_image", "needs 16-byte aligned operands and a multiple of 8 elements");
+    const size_t groups = n / 8;
+    const unsigned grid = gridFor(groups, kBlock, 1u << 30);
+    if (act == BF_ACT_SILU) flat4Kernel<<<grid, kBlock, 0, stream>>>(groups, ActImageOp<BF_ACT_SILU>{z, image});
+    else if (act == BF_ACT_GELU) flat4Kernel<<<grid, kBlock, 0, stream>>>(groups, ActImageOp<BF_ACT_GELU>{z, image});
+    else flat4Kernel<<<grid, kBlock, 0, stream>>>(groups, ActImageOp<BF_ACT_RELU>{z, image});
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int actBackwardToBf16Image(const float* z, const float* dHidden, unsigned short* dzImage, float* dBias, size_t rows,
+                           size_t features, int act, hipStream_t stream) {
+    if (act == BF_ACT_SILU) return launchColumnSum<1, BF_ACT_SILU>(z, nullptr, dHidden, nullptr, dBias, rows, features, stream, dzImage);
+    if (act == BF_ACT_GELU) return launchColumnSum<1, BF_ACT_GELU>(z, nullptr, dHidden, nullptr, dBias, rows, features, stream, dzImage);
+    return launchColumnSum<1, BF_ACT_RELU>(z, nullptr, dHidden, nullptr, dBias, rows, features, stream, dzImage);
+}
+
 }  // namespace bf
 
 using namespace bf;

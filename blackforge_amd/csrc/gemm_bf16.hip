@@ -24,13 +24,7 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned short ushort8 __attribute__((ext_vector_type(8)));
-typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
-typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ unsigned short toBf16Bits(float x) {
-    __bf16 h = static_cast<__bf16>(x);   // round to nearest even, NaN preserved
-    return __builtin_bit_cast(unsigned short, h);
-}
 
 inline size_t pad8(size_t n) { return (n + 7) / 8 * 8; }
 
@@ -175,7 +169,7 @@ template <int TM, int TN>
 __device__ __forceinline__ void storeAccumulators(float16v (&acc)[TM][TN], const Epilogue& e, int M, int N, int row0,
                                                   int col0, int li, int half) {
     const int which = col0 / e.splitN;              // uniform over the tile
-    float* __restrict__ C = e.c[which];
+    float* __restrict__ C = which == 0 ? e.c[0] : which == 1 ? e.c[1] : e.c[2];   // no indexed access: the struct stays in registers
     const int shift = which * e.splitN, ld = e.splitN;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -431,7 +425,7 @@ __global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restr
         const size_t row = (4 * i) / N, col = (4 * i) - row * N, which = col / splitN;
         if (e.bias) sum = sum + loadf4(e.bias + col);
         if (e.residual) sum = sum + loadf4(e.residual + 4 * i);
-        storef4(e.c[which] + row * splitN + (col - which * splitN), sum);
+        storef4((which == 0 ? e.c[0] : which == 1 ? e.c[1] : e.c[2]) + row * splitN + (col - which * splitN), sum);
     }
     for (size_t i = 4 * count4 + first; i < count; i += stride) {
         float sum = partial[i];
@@ -439,7 +433,7 @@ __global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restr
         const size_t row = i / N, col = i - row * N, which = col / splitN;
         if (e.bias) sum += e.bias[col];
         if (e.residual) sum += e.residual[i];
-        e.c[which][row * splitN + (col - which * splitN)] = sum;
+        (which == 0 ? e.c[0] : which == 1 ? e.c[1] : e.c[2])[row * splitN + (col - which * splitN)] = sum;
     }
 }
 
@@ -837,6 +831,30 @@ int convertTransposed(const float* x, unsigned short* out, size_t rows, size_t c
     return BF_OK;
 }
 
+// out[c, r] = in[r, c] for a bf16 image `in` [rows, ldIn] (cols columns used); `out` is [cols, ldOut] with ldOut >= rows,
+// columns rows..ldOut-1 zero.
+__global__ void __launch_bounds__(kBlock) transposeBf16Kernel(const unsigned short* __restrict__ in, unsigned short* __restrict__ out,
+                                                              size_t rows, size_t cols, size_t ldIn, size_t ldOut) {
+    __shared__ unsigned short tile[64][66];
+    const size_t r0 = size_t(blockIdx.y) * 64, c0 = size_t(blockIdx.x) * 64;
+    for (int i = threadIdx.x; i < 4096; i += kBlock) {
+        const int r = i >> 6, c = i & 63;
+        tile[r][c] = (r0 + r < rows && c0 + c < cols) ? in[(r0 + r) * ldIn + c0 + c] : static_cast<unsigned short>(0);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 4096; i += kBlock) {
+        const int c = i >> 6, r = i & 63;
+        if (c0 + c < cols && r0 + r < ldOut) out[(c0 + c) * ldOut + r0 + r] = tile[r][c];
+    }
+}
+int transposeImage(const unsigned short* in, unsigned short* out, size_t rows, size_t cols, size_t ldIn, size_t ldOut, hipStream_t s) {
+    dim3 grid(unsigned((cols + 63) / 64), unsigned((ldOut + 63) / 64));
+    if (grid.y > 65535) return failInvalid("feedforward_bf16", "too many rows");
+    transposeBf16Kernel<<<grid, kBlock, 0, s>>>(in, out, rows, cols, ldIn, ldOut);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
 // ---- bf16 images of weights, kept per (device, pointers, layout) until invalidated ------------------
 // Layouts: 0 plain [rows, pad8(cols)]; 1 transposed [cols, pad8(rows)]; for a group of up to three weights of one
 // shape, 2 = their transposed images stacked row-wise ([count*cols, pad8(rows)], the Bt operand of one GEMM that
@@ -1218,6 +1236,120 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
                 if (st != BF_OK) return st;
             }
         }
+    }
+    return st;
+}
+
+int bf_hip_feedforward_bf16(const float* x, const float* w1, const float* b1, const float* w2, const float* b2, const float* residual,
+                            int act, float* z, uint16_t* hImage, uint16_t* xImage, float* out, size_t m, size_t d, size_t hidden,
+                            int cacheWeight, bf_stream_t stream) {
+    if (m == 0) return BF_OK;
+    BF_REQUIRE(d > 0 && hidden > 0 && d % 8 == 0 && hidden % 8 == 0, "d and hidden must be positive multiples of 8");
+    BF_REQUIRE(act == BF_ACT_SILU || act == BF_ACT_GELU || act == BF_ACT_RELU, "unknown activation");
+    BF_REQUIRE(x && w1 && w2 && z && hImage && out, "NULL pointer");
+    hipStream_t s = asStream(stream);
+    Scratch xScratch(xImage ? 0 : m * d * sizeof(unsigned short));
+    if (xScratch.status != BF_OK) return xScratch.status;
+    unsigned short* xImg = xImage ? xImage : xScratch.as<unsigned short>();
+    int st = convertPlain(x, xImg, m, d, s);
+    if (st != BF_OK) return st;
+    unsigned short* wImg = nullptr;
+    size_t wBytes = 0;
+    st = weightImage(w1, d, hidden, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
+    if (st != BF_OK) return st;
+    st = launchGemmNt(xImg, wImg, Epilogue{{z, nullptr, nullptr}, int(hidden), b1, nullptr}, m, hidden, d, d, d, s);
+    if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+    if (st != BF_OK) return st;
+    st = actToBf16Image(z, hImage, m * hidden, act, s);
+    if (st != BF_OK) return st;
+    st = weightImage(w2, hidden, d, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
+    if (st != BF_OK) return st;
+    st = launchGemmNt(hImage, wImg, Epilogue{{out, nullptr, nullptr}, int(d), b2, residual}, m, d, hidden, hidden, hidden, s);
+    if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+    return st;
+}
+
+int bf_hip_feedforward_bf16_backward(const float* x, const uint16_t* xImage, const float* w1, const float* w2, const float* z,
+                                     const uint16_t* hImage, const float* g, int act, float* dX, float* dW1, float* dB1, float* dW2,
+                                     float* dB2, size_t m, size_t d, size_t hidden, int cacheWeight, bf_stream_t stream) {
+    BF_REQUIRE(d > 0 && hidden > 0 && d % 8 == 0 && hidden % 8 == 0, "d and hidden must be positive multiples of 8");
+    BF_REQUIRE(act == BF_ACT_SILU || act == BF_ACT_GELU || act == BF_ACT_RELU, "unknown activation");
+    hipStream_t s = asStream(stream);
+    int st = BF_OK;
+    if (m == 0) {   // no rows: parameter gradients are zero
+        if (dW1) st = bf_hip_fill_zero(dW1, d * hidden * sizeof(float), stream);
+        if (st == BF_OK && dW2) st = bf_hip_fill_zero(dW2, d * hidden * sizeof(float), stream);
+        if (st == BF_OK && dB1) st = bf_hip_fill_zero(dB1, hidden * sizeof(float), stream);
+        if (st == BF_OK && dB2) st = bf_hip_fill_zero(dB2, d * sizeof(float), stream);
+        return st;
+    }
+    BF_REQUIRE((x || xImage) && w1 && w2 && z && hImage && g, "NULL operand");
+    const size_t mp = pad8(m);
+    Scratch gImg(m * d * sizeof(unsigned short));
+    if (gImg.status != BF_OK) return gImg.status;
+    st = convertPlain(g, gImg.as<unsigned short>(), m, d, s);
+    if (st != BF_OK) return st;
+    if (dB2) {
+        st = bf_hip_bias_grad(g, dB2, m, d, stream);
+        if (st != BF_OK) return st;
+    }
+    if (dW2) {   // dW2[hidden, d] = h^T g, contraction over the m rows
+        bool done = false;
+        st = launchGemmTn(hImage, gImg.as<unsigned short>(), Epilogue{{dW2, nullptr, nullptr}, int(d), nullptr, nullptr}, hidden, d, m,
+                          hidden, d, s, &done);
+        if (st != BF_OK) return st;
+        if (!done) {
+            Scratch hT(hidden * mp * sizeof(unsigned short)), gT(d * mp * sizeof(unsigned short));
+            if (hT.status != BF_OK) return hT.status;
+            if (gT.status != BF_OK) return gT.status;
+            st = transposeImage(hImage, hT.as<unsigned short>(), m, hidden, hidden, mp, s);
+            if (st == BF_OK) st = convertTransposed(g, gT.as<unsigned short>(), m, d, s);
+            if (st == BF_OK) st = launchGemmNt(hT.as<unsigned short>(), gT.as<unsigned short>(), dW2, hidden, d, mp, mp, mp, s);
+            if (st != BF_OK) return st;
+        }
+    }
+    if (!dX && !dW1 && !dB1) return BF_OK;
+    // dH = g w2^T; one pass over it writes bf16(dz), dz = act'(z) . dH, and dz's column sums: dz is never stored in fp32
+    Scratch dH(m * hidden * sizeof(float)), dzImg(m * hidden * sizeof(unsigned short));
+    if (dH.status != BF_OK) return dH.status;
+    if (dzImg.status != BF_OK) return dzImg.status;
+    unsigned short* wImg = nullptr;
+    size_t wBytes = 0;
+    st = weightImage(w2, hidden, d, /*transposed=*/false, cacheWeight != 0, s, &wImg, &wBytes);
+    if (st != BF_OK) return st;
+    st = launchGemmNt(gImg.as<unsigned short>(), wImg, dH.as<float>(), m, hidden, d, d, d, s);
+    if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+    if (st != BF_OK) return st;
+    st = actBackwardToBf16Image(z, dH.as<float>(), dzImg.as<unsigned short>(), dB1, m, hidden, act, s);
+    if (st != BF_OK) return st;
+    if (dW1) {   // dW1[d, hidden] = x^T dz
+        Scratch xScratch(xImage ? 0 : m * d * sizeof(unsigned short));
+        if (xScratch.status != BF_OK) return xScratch.status;
+        const unsigned short* xImg = xImage;
+        if (!xImg) {
+            st = convertPlain(x, xScratch.as<unsigned short>(), m, d, s);
+            if (st != BF_OK) return st;
+            xImg = xScratch.as<unsigned short>();
+        }
+        bool done = false;
+        st = launchGemmTn(xImg, dzImg.as<unsigned short>(), Epilogue{{dW1, nullptr, nullptr}, int(hidden), nullptr, nullptr}, d, hidden, m,
+                          d, hidden, s, &done);
+        if (st != BF_OK) return st;
+        if (!done) {
+            Scratch xT(d * mp * sizeof(unsigned short)), dzT(hidden * mp * sizeof(unsigned short));
+            if (xT.status != BF_OK) return xT.status;
+            if (dzT.status != BF_OK) return dzT.status;
+            st = transposeImage(xImg, xT.as<unsigned short>(), m, d, d, mp, s);
+            if (st == BF_OK) st = transposeImage(dzImg.as<unsigned short>(), dzT.as<unsigned short>(), m, hidden, hidden, mp, s);
+            if (st == BF_OK) st = launchGemmNt(xT.as<unsigned short>(), dzT.as<unsigned short>(), dW1, d, hidden, mp, mp, mp, s);
+            if (st != BF_OK) return st;
+        }
+    }
+    if (dX) {   // dX[m, d] = dz w1^T
+        st = weightImage(w1, d, hidden, /*transposed=*/false, cacheWeight != 0, s, &wImg, &wBytes);
+        if (st != BF_OK) return st;
+        st = launchGemmNt(dzImg.as<unsigned short>(), wImg, dX, m, d, hidden, hidden, hidden, s);
+        if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
     }
     return st;
 }

@@ -427,8 +427,10 @@ def fusedAttentionBackward(dOutput, q, k, v, output, m, l, numHeads: int, scaleF
 @dataclass
 class FeedForwardCache:
     normed: Optional[DeviceTensor] = None
-    gemm1: Optional[DeviceTensor] = None
-    hidden: Optional[DeviceTensor] = None
+    gemm1: Optional[DeviceTensor] = None    # normed @ w1; on the fused bf16 route normed @ w1 + b1
+    hidden: Optional[DeviceTensor] = None   # act(gemm1 + b1); absent on the fused bf16 route
+    hiddenImage: Optional[DeviceTensor] = None   # fused bf16 route: bf16(act(gemm1)) as raw storage [rows, hidden/2]
+    normedImage: Optional[DeviceTensor] = None   # fused bf16 route: bf16(normed) as raw storage [rows, d/2]
 
 
 @dataclass
@@ -462,8 +464,42 @@ def _mm_bwd(useBf16, cached):
     return matmulBf16BackwardCachedWeight if cached else matmulBf16Backward
 
 
+def _opt(t):
+    return t.ptr if t is not None else None
+
+
+def feedForwardBf16Fused(x, w1, b1, w2, b2, residual=None, act: int = ACT_SILU, cached=False):
+    """bf_hip_feedforward_bf16 on x:[m,d]: returns (out, z, hImage, xImage); the images are raw bf16 storage held in
+    DeviceTensors of half the width."""
+    _require(x.rank() == 2 and w1.rank() == 2 and w2.rank() == 2 and x.shape[1] == w1.shape[0] and w1.shape[1] == w2.shape[0]
+             and w2.shape[1] == x.shape[1], "feedForwardBf16Fused: incompatible shapes")
+    m, d, hidden = x.shape[0], x.shape[1], w1.shape[1]
+    _require(d % 8 == 0 and hidden % 8 == 0, "feedForwardBf16Fused: d and hidden must be multiples of 8")
+    z, hImage, xImage, out = DeviceTensor((m, hidden)), DeviceTensor((m, hidden // 2)), DeviceTensor((m, d // 2)), DeviceTensor((m, d))
+    _call("bf_hip_feedforward_bf16", x.ptr, w1.ptr, _opt(b1), w2.ptr, _opt(b2), _opt(residual), act, z.ptr, hImage.ptr, xImage.ptr,
+          out.ptr, m, d, hidden, 1 if cached else 0, None)
+    return out, z, hImage, xImage
+
+
+def feedForwardBf16FusedBackward(x, xImage, w1, w2, z, hImage, g, act: int = ACT_SILU, cached=False):
+    """bf_hip_feedforward_bf16_backward: returns (dX, dW1, dB1, dW2, dB2); x or xImage may be None."""
+    m, d, hidden = g.shape[0], g.shape[1], w1.shape[1]
+    dX, dW1, dB1, dW2, dB2 = DeviceTensor((m, d)), DeviceTensor(w1.shape), DeviceTensor((hidden,)), DeviceTensor(w2.shape), DeviceTensor((d,))
+    _call("bf_hip_feedforward_bf16_backward", _opt(x), _opt(xImage), w1.ptr, w2.ptr, z.ptr, hImage.ptr, g.ptr, act, dX.ptr, dW1.ptr,
+          dB1.ptr, dW2.ptr, dB2.ptr, m, d, hidden, 1 if cached else 0, None)
+    return dX, dW1, dB1, dW2, dB2
+
+
+def _fused_feed_forward(useBf16, x, w1):
+    return useBf16 and x.shape[-1] % 8 == 0 and w1.shape[1] % 8 == 0 and x.elementCount() > 0
+
+
 def feedForwardForwardCached(x, w1, b1, w2, b2, useBf16: bool, cache: FeedForwardCache, act: int = ACT_SILU):
     cache.normed = rmsnorm(x)
+    if _fused_feed_forward(useBf16, x, w1):
+        out, z, cache.hiddenImage, cache.normedImage = feedForwardBf16Fused(_flat2d(cache.normed), w1, b1, w2, b2, _flat2d(x), act, True)
+        cache.gemm1, cache.hidden = z.reshaped(x.shape[:-1] + (w1.shape[1],)), None
+        return out.reshaped(x.shape)
     mm = _mm(useBf16, True)
     hiddenShape = x.shape[:-1] + (w1.shape[1],)
     cache.gemm1 = mm(_flat2d(cache.normed), w1).reshaped(hiddenShape)
@@ -493,6 +529,11 @@ class FeedForwardGrad:
 
 
 def feedForwardBackwardCached(x, w1, b1, w2, b2, cache: FeedForwardCache, g, useBf16: bool, act: int = ACT_SILU) -> FeedForwardGrad:
+    if cache.hiddenImage is not None:
+        dNormedFlat, dW1, dB1, dW2, dB2 = feedForwardBf16FusedBackward(None, cache.normedImage, w1, w2, _flat2d(cache.gemm1),
+                                                                        cache.hiddenImage, _flat2d(g), act, True)
+        dInput = add(g, rmsnormBackward(x, dNormedFlat.reshaped(cache.normed.shape)))
+        return FeedForwardGrad(dInput, dW1, dB1, dW2, dB2)
     bwd = _mm_bwd(useBf16, True)
     dB2 = biasGradientOnly(g)
     dHiddenFlat, dW2 = bwd(_flat2d(cache.hidden), w2, _flat2d(g))

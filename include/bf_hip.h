@@ -221,6 +221,25 @@ int bf_hip_matmul_bf16_shared_input(const float* a, const float* const* b, float
 int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const* b, const float* const* g, float* dA,
                                              float* const* dB, size_t count, size_t m, size_t k, size_t n,
                                              int cacheWeight, bf_stream_t stream);
+/* The feed-forward block between its normalisation and its output in the bf16 mode (feedForwardForwardCached,
+ * ops_transformer.cu:182-215: linearBf16CachedWeight, activation, linearBf16CachedWeight, residual add) with the adds
+ * done by the GEMMs' stores and the activation by one pass that writes only what the second GEMM reads:
+ *   z[m,hidden]      = bf16(x[m,d]) * bf16(w1[d,hidden]) + b1       fp32, kept for the backward pass
+ *   hImage[m,hidden] = bf16(act(z))                                 the second GEMM's operand; no fp32 copy is written
+ *   out[m,d]         = hImage * bf16(w2[hidden,d]) + b2 + residual
+ * d and hidden must be multiples of 8; b1, b2 and residual may be NULL; xImage, if not NULL, receives bf16(x) ([m,d]) for
+ * the backward call.  Results equal those of bf_hip_matmul_bf16 + bf_hip_add_bias_act + bf_hip_linear_bf16. */
+int bf_hip_feedforward_bf16(const float* x, const float* w1, const float* b1, const float* w2, const float* b2,
+                            const float* residual, int act, float* z, uint16_t* hImage, uint16_t* xImage, float* out, size_t m,
+                            size_t d, size_t hidden, int cacheWeight, bf_stream_t stream);
+/* Its gradients (feedForwardBackwardCached, autodiff.cu:719-750, between the output gradient g[m,d] and the
+ * normalisation's backward): dB2 = column sums of g; dW2 = hImage^T * bf16(g); dz = act'(z) . (bf16(g) * bf16(w2)^T),
+ * of which one pass keeps the bf16 image and the column sums dB1 (taken before the rounding) and nothing else;
+ * dW1 = bf16(x)^T * bf16(dz); dX = bf16(dz) * bf16(w1)^T.  One of x and xImage may be NULL; any output may be NULL. */
+int bf_hip_feedforward_bf16_backward(const float* x, const uint16_t* xImage, const float* w1, const float* w2, const float* z,
+                                     const uint16_t* hImage, const float* g, int act, float* dX, float* dW1, float* dB1,
+                                     float* dW2, float* dB2, size_t m, size_t d, size_t hidden, int cacheWeight,
+                                     bf_stream_t stream);
 /* invalidateBf16WeightCache: ops.hpp:80 */
 int bf_hip_invalidate_bf16_weight_cache(void);
 

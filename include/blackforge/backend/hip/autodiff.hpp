@@ -175,6 +175,16 @@ inline FeedForwardGrad feedForwardBackwardCached(const DeviceTensor& input, cons
     (void)b2;
     require(gradOutput.shape() == input.shape(), "feedForwardBackward: gradient shape differs from the input");
     const int mode = useBf16 ? 2 : 0;
+    if (cache.fused) {
+        const std::size_t rows = detail::rowsOf(input), d = detail::lastDim(input), hidden = w1.dim(1);
+        DeviceTensor dNormed(cache.normed.shape()), dW1(w1.shape()), dB1({hidden}), dW2(w2.shape()), dB2({d});
+        check(bf_hip_feedforward_bf16_backward(nullptr, reinterpret_cast<const uint16_t*>(cache.normedImage.data()), w1.data(), w2.data(),
+                                               cache.gemm1.data(), reinterpret_cast<const uint16_t*>(cache.hiddenImage.data()),
+                                               gradOutput.data(), static_cast<int>(act), dNormed.data(), dW1.data(), dB1.data(),
+                                               dW2.data(), dB2.data(), rows, d, hidden, 1, nullptr));
+        DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, dNormed));
+        return FeedForwardGrad{std::move(dInput), std::move(dW1), std::move(dB1), std::move(dW2), std::move(dB2)};
+    }
     DeviceTensor dB2 = biasGradientOnly(gradOutput);
     MatmulGrad g2 = detail::projectionBackward(cache.hidden, w2, gradOutput, mode, cache.hidden.shape());
     AddBiasSiluGrad hiddenGrad = addBiasActivationBackward(cache.gemm1, b1, g2.dA, act);

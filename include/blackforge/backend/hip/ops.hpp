@@ -201,9 +201,20 @@ inline DeviceTensor linearBf16CachedWeight(const DeviceTensor& input, const Devi
 // ---- composite blocks ------------------------------------------------------------------------
 struct FeedForwardCache {
     DeviceTensor normed;  // rmsnorm(input)
-    DeviceTensor gemm1;   // normed @ w1, before bias and activation
-    DeviceTensor hidden;  // act(gemm1 + b1)
+    DeviceTensor gemm1;   // normed @ w1, before bias and activation; with `fused` normed @ w1 + b1
+    DeviceTensor hidden;  // act(gemm1 + b1); empty with `fused`
+    // bf16 mode with widths that are multiples of 8: the activation is applied where the first GEMM stores its product and
+    // only the bf16 images the later GEMMs read are kept (raw storage, two values per float)
+    bool fused = false;
+    DeviceTensor hiddenImage;  // bf16(act(gemm1)), [rows, hidden / 2]
+    DeviceTensor normedImage;  // bf16(normed), [rows, d / 2]
 };
+
+namespace detail {
+inline bool feedForwardFuses(const DeviceTensor& input, const DeviceTensor& w1, bool useBf16) {
+    return useBf16 && input.elementCount() > 0 && lastDim(input) % 8 == 0 && w1.dim(1) % 8 == 0;
+}
+}  // namespace detail
 
 inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
                                               const DeviceTensor& w2, const DeviceTensor& b2, bool useBf16,
@@ -212,6 +223,22 @@ inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const De
             "feedForward: incompatible shapes on the device");
     const int mode = useBf16 ? 2 : 0;
     cache.normed = rmsnorm(input);
+    cache.fused = detail::feedForwardFuses(input, w1, useBf16);
+    if (cache.fused) {
+        require(b1.rank() == 1 && b1.dim(0) == w1.dim(1), "addBiasSilu: expected input [..., features] and bias [features]");
+        require(b2.rank() == 1 && b2.dim(0) == w2.dim(1), "addBiasResidual: expected input [..., features] and bias [features]");
+        require(w2.dim(1) == detail::lastDim(input), "addBiasResidual: residual shape differs from the product");
+        const std::size_t rows = detail::rowsOf(input), d = detail::lastDim(input), hidden = w1.dim(1);
+        cache.gemm1 = DeviceTensor(detail::withLastDim(input, hidden));
+        cache.hidden = DeviceTensor();
+        cache.hiddenImage = DeviceTensor({rows, hidden / 2});
+        cache.normedImage = DeviceTensor({rows, d / 2});
+        DeviceTensor out(input.shape());
+        check(bf_hip_feedforward_bf16(cache.normed.data(), w1.data(), b1.data(), w2.data(), b2.data(), input.data(), static_cast<int>(act),
+                                      cache.gemm1.data(), reinterpret_cast<uint16_t*>(cache.hiddenImage.data()),
+                                      reinterpret_cast<uint16_t*>(cache.normedImage.data()), out.data(), rows, d, hidden, 1, nullptr));
+        return out;
+    }
     cache.gemm1 = detail::projection(cache.normed, w1, mode, detail::withLastDim(input, w1.dim(1)));
     cache.hidden = addBiasActivation(cache.gemm1, b1, act);
     if (mode != 0) {

@@ -233,3 +233,54 @@ def test_bf16_weight_cache_semantics(hip, oracle, rng):
     assert_close(fresh, oracle.matmul(oracle.roundToBf16(a), oracle.roundToBf16(b2)), tol=1e-4)
     lin = ops.linearBf16(da, db, D.fromHost(np.ones(24, f32))).toHost()
     assert_close(lin, oracle.matmul(oracle.roundToBf16(a), oracle.roundToBf16(b2)) + 1, tol=1e-4)
+
+
+def bf16_bits_to_f32(raw, rows, cols):
+    """Reads a bf16 image kept as raw storage in a float32 tensor of half the width."""
+    bits = np.ascontiguousarray(raw).view(np.uint16).reshape(rows, cols)
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+@pytest.mark.parametrize("m,d,hidden,act", [(64, 32, 128, 0), (64, 32, 128, 1), (64, 32, 128, 2), (300, 72, 264, 0), (300, 72, 264, 1),
+                                            (1000, 64, 2048, 2), (4096, 256, 1024, 0), (4096, 256, 1024, 1), (8192, 768, 3072, 0),
+                                            (2048, 8, 8, 0), (513, 512, 512, 1), (256, 4096, 256, 1), (256, 4096, 256, 2)])
+def test_feed_forward_with_the_elementwise_steps_in_the_gemm_stores(hip, oracle, rng, m, d, hidden, act):
+    """bf_hip_feedforward_bf16[_backward] (feedForwardForwardCached / feedForwardBackwardCached in the bf16 mode,
+    ops_transformer.cu:182-215, autodiff.cu:719-750) against the same block built from the separate operators, which are
+    themselves checked against the oracle: same roundings, so the agreement is tight.  Shapes cover the small-tile GEMM with
+    the transposed-image weight gradients, ragged row counts, and the large-tile kernels with fragments transposed in LDS;
+    act 0/1/2 = silu/gelu/relu."""
+    D, ops = hip.DeviceTensor, hip.ops
+    x, w1, b1 = r(rng, m, d), r(rng, d, hidden, scale=0.1), r(rng, hidden, scale=0.5)
+    w2, b2, res, g = r(rng, hidden, d, scale=0.1), r(rng, d), r(rng, m, d), r(rng, m, d)
+    dx, dw1, db1, dw2, db2, dres, dg = map(D.fromHost, (x, w1, b1, w2, b2, res, g))
+    ops.invalidateBf16WeightCache()
+    out, z, hImage, xImage = ops.feedForwardBf16Fused(dx, dw1, db1, dw2, db2, dres, act)
+    # the separate operators
+    gemm1 = ops.matmulBf16(dx, dw1)
+    hiddenT = ops.addBiasAct(gemm1, db1, act)
+    expectedOut = ops.linearBf16Fused(hiddenT, dw2, db2, dres)
+    assert_close(z.toHost(), ops.addBias(gemm1, db1).toHost(), tol=1e-6, what="pre-activation")
+    assert_bits_equal(bf16_bits_to_f32(hImage.toHost(), m, hidden), oracle.roundToBf16(ops._act(z, act).toHost()), "hidden image")
+    assert_bits_equal(bf16_bits_to_f32(xImage.toHost(), m, d), oracle.roundToBf16(x), "input image")
+    assert_close(out.toHost(), expectedOut.toHost(), tol=1e-5, what="block output")
+    if m * d * hidden <= 20_000_000:   # and against float64 arithmetic on the rounded operands
+        zr = oracle.roundToBf16(x).astype(np.float64) @ oracle.roundToBf16(w1).astype(np.float64) + b1
+        assert_close(z.toHost(), zr.astype(f32), tol=1e-4, what="pre-activation vs float64")
+    # gradients
+    dX, dW1, dB1, dW2, dB2 = ops.feedForwardBf16FusedBackward(dx, None, dw1, dw2, z, hImage, dg, act)
+    eHidden, eW2 = ops.matmulBf16Backward(hiddenT, dw2, dg)
+    eGemm1, eB1 = ops.addBiasActBackward(gemm1, db1, eHidden, act)
+    eX, eW1 = ops.matmulBf16Backward(dx, dw1, eGemm1)
+    for got, exp, name in ((dX, eX, "dX"), (dW1, eW1, "dW1"), (dB1, eB1, "dB1"), (dW2, eW2, "dW2"), (dB2, ops.biasGradientOnly(dg), "dB2")):
+        assert_close(got.toHost(), exp.toHost(), tol=2e-5, what=name)
+    # the same gradients from the input image alone
+    again = ops.feedForwardBf16FusedBackward(None, xImage, dw1, dw2, z, hImage, dg, act)
+    for got, exp, name in zip(again, (dX, dW1, dB1, dW2, dB2), ("dX", "dW1", "dB1", "dW2", "dB2")):
+        assert_bits_equal(got.toHost(), exp.toHost(), name + " from the input image")
+
+
+def test_feed_forward_fused_rejects_widths_that_are_not_multiples_of_eight(hip):
+    D, ops = hip.DeviceTensor, hip.ops
+    with pytest.raises(ValueError):
+        ops.feedForwardBf16Fused(D.zeros((4, 12)), D.zeros((12, 16)), D.zeros((16,)), D.zeros((16, 12)), D.zeros((12,)))
