@@ -71,6 +71,7 @@ SIGNATURES = {
     "bf_hip_zero_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_size), c_size, S],
     "bf_hip_rmsnorm": [P, P, c_size, c_size, S],
     "bf_hip_rmsnorm_backward": [P, P, P, c_size, c_size, S],
+    "bf_hip_rmsnorm_backward_add": [P, P, P, P, c_size, c_size, S],
     "bf_hip_softmax": [P, P, c_size, c_size, S],
     "bf_hip_softmax_backward": [P, P, P, c_size, c_size, S],
     "bf_hip_bias_grad": [P, P, c_size, c_size, S],

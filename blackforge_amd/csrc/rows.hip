@@ -94,7 +94,8 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormKernel(const float* 
 
 template <int G, int MAXE, int VEC, bool CACHED>
 __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const float* __restrict__ x, const float* __restrict__ g,
-                                                                            float* __restrict__ out, size_t rows, size_t features) {
+                                                                            const float* __restrict__ addend, float* __restrict__ out,
+                                                                            size_t rows, size_t features) {
     BF_ROW_PROLOGUE();
     for (size_t row = firstRow; row < rows; row += rowStep) {
         Row<G, MAXE, VEC, CACHED> rx, rg;
@@ -124,9 +125,18 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const
 #pragma unroll
                 for (int i = 0; i < MAXE; ++i) rg.c.r[i] = float(double(rg.c.r[i]) * invR - double(rx.c.r[i]) * k);
             }
+            if (addend) {   // the gradient that bypassed the normalisation (a residual connection) joins here
+                rx.open(addend + row * features, features, t, 0.0f);
+#pragma unroll
+                for (int i = 0; i < MAXE; ++i) rg.c.r[i] += rx.c.r[i];
+            }
             rg.c.store(o, features, t);
         } else {
-            for (size_t e = t; e < features; e += G) o[e] = float(double(rg.p[e]) * invR - double(rx.p[e]) * k);
+            const float* a = addend ? addend + row * features : nullptr;
+            for (size_t e = t; e < features; e += G) {
+                const float v = float(double(rg.p[e]) * invR - double(rx.p[e]) * k);
+                o[e] = a ? v + a[e] : v;
+            }
         }
     }
 }
@@ -245,17 +255,23 @@ int bf_hip_rmsnorm(const float* x, float* out, size_t rows, size_t features, bf_
     return BF_OK;
 }
 
-int bf_hip_rmsnorm_backward(const float* x, const float* g, float* out, size_t rows, size_t features,
-                            bf_stream_t stream) {
+int bf_hip_rmsnorm_backward_add(const float* x, const float* g, const float* addend, float* out, size_t rows, size_t features,
+                                bf_stream_t stream) {
     if (rows == 0 || features == 0) return BF_OK;
     BF_REQUIRE(x && g && out, "NULL pointer");
+    BF_REQUIRE(addend != out, "the output must not be the addend");
     hipStream_t s = asStream(stream);
-#define ARGS_ x, g, out, rows, features
-    BF_ROW_LAUNCH(rmsnormBackwardKernel, true, aligned16(x) && aligned16(g) && aligned16(out), rows, features, s, x, g,
-                  out, rows, features);
+#define ARGS_ x, g, addend, out, rows, features
+    BF_ROW_LAUNCH(rmsnormBackwardKernel, true, aligned16(x) && aligned16(g) && aligned16(out) && aligned16(addend), rows, features, s, x, g,
+                  addend, out, rows, features);
 #undef ARGS_
     BF_LAUNCH_CHECK();
     return BF_OK;
+}
+
+int bf_hip_rmsnorm_backward(const float* x, const float* g, float* out, size_t rows, size_t features,
+                            bf_stream_t stream) {
+    return bf_hip_rmsnorm_backward_add(x, g, nullptr, out, rows, features, stream);
 }
 
 int bf_hip_softmax(const float* x, float* out, size_t rows, size_t features, bf_stream_t stream) {

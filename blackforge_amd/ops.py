@@ -134,6 +134,15 @@ def rmsnormBackward(x: DeviceTensor, g: DeviceTensor) -> DeviceTensor:
     return out
 
 
+def rmsnormBackwardAdd(x: DeviceTensor, g: DeviceTensor, residualGrad: DeviceTensor) -> DeviceTensor:
+    """residualGrad + rmsnormBackward(x, g) in one pass."""
+    _require(x.shape == g.shape == residualGrad.shape, "rmsnormBackward: incompatible shapes")
+    _require(x.rank() >= 2, "rmsnormBackward: needs a tensor of rank >= 2")
+    out = DeviceTensor(x.shape)
+    _call("bf_hip_rmsnorm_backward_add", x.ptr, g.ptr, residualGrad.ptr, out.ptr, *_rows(x), None)
+    return out
+
+
 def softmax(x: DeviceTensor) -> DeviceTensor:
     _require(x.rank() >= 2, "softmax: needs a tensor of rank >= 2")
     out = DeviceTensor(x.shape)
@@ -532,7 +541,7 @@ def feedForwardBackwardCached(x, w1, b1, w2, b2, cache: FeedForwardCache, g, use
     if cache.hiddenImage is not None:
         dNormedFlat, dW1, dB1, dW2, dB2 = feedForwardBf16FusedBackward(None, cache.normedImage, w1, w2, _flat2d(cache.gemm1),
                                                                         cache.hiddenImage, _flat2d(g), act, True)
-        dInput = add(g, rmsnormBackward(x, dNormedFlat.reshaped(cache.normed.shape)))
+        dInput = rmsnormBackwardAdd(x, dNormedFlat.reshaped(cache.normed.shape), g)
         return FeedForwardGrad(dInput, dW1, dB1, dW2, dB2)
     bwd = _mm_bwd(useBf16, True)
     dB2 = biasGradientOnly(g)

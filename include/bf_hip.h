@@ -135,6 +135,11 @@ int bf_hip_rmsnorm(const float* x, float* out, size_t rows, size_t features, bf_
 /* rmsnormBackward: autodiff.hpp:79 */
 int bf_hip_rmsnorm_backward(const float* x, const float* g, float* out, size_t rows, size_t features,
                             bf_stream_t stream);
+/* The same with the gradient that bypassed the normalisation added in: out = addend + rmsnormBackward(x, g), the
+ * `add(gradOutput, rmsnormBackward(...))` that ends both composite blocks' backward passes (autodiff.cu:746,794).
+ * addend may be NULL; out must not be addend. */
+int bf_hip_rmsnorm_backward_add(const float* x, const float* g, const float* addend, float* out, size_t rows,
+                                size_t features, bf_stream_t stream);
 /* softmax: ops.hpp:98 */
 int bf_hip_softmax(const float* x, float* out, size_t rows, size_t features, bf_stream_t stream);
 /* softmaxBackward: autodiff.hpp:84 (takes the forward INPUT, recomputes y) */

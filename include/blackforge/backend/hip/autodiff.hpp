@@ -14,7 +14,20 @@ struct MatmulGrad {
     DeviceTensor dB;
 };
 
+// Where a backward pass may write parameter gradients directly: tensors of the gradients' shapes whose contents are to be
+// REPLACED (a model's gradient buffers straight after zeroGrad(): writing g there equals adding g to zero).  A gradient
+// written to slot i comes back as a non-owning view of that tensor instead of a tensor of its own, so callers can tell by
+// the data pointer.  Slots: Linear {weight}; self-attention {wq, wk, wv, wout}; feed-forward {w1, b1, w2, b2}.
+struct GradientTargets {
+    DeviceTensor* slot[4] = {nullptr, nullptr, nullptr, nullptr};
+};
+
 namespace detail {
+inline DeviceTensor gradientTensor(const GradientTargets* into, int i, std::vector<std::size_t> shape) {
+    if (into != nullptr && into->slot[i] != nullptr && into->slot[i]->shape() == shape && into->slot[i]->data() != nullptr)
+        return DeviceTensor::borrow(into->slot[i]->data(), std::move(shape));
+    return DeviceTensor(std::move(shape));
+}
 inline void requireMatmulBackward(const char* op, const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& g) {
     require(a.rank() == 2 && b.rank() == 2 && g.rank() == 2 && a.dim(1) == b.dim(0) && g.dim(0) == a.dim(0) &&
                 g.dim(1) == b.dim(1),
@@ -22,9 +35,9 @@ inline void requireMatmulBackward(const char* op, const DeviceTensor& a, const D
 }
 // Gradients of c = a(as [m,k]) * b[k,n] given g (as [m,n]); mode as in detail::projection.
 inline MatmulGrad projectionBackward(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& g, int mode,
-                                     std::vector<std::size_t> dAShape) {
+                                     std::vector<std::size_t> dAShape, const GradientTargets* into = nullptr, int slot = 0) {
     std::size_t m = rowsOf(a), k = lastDim(a), n = b.dim(1);
-    MatmulGrad r{DeviceTensor(std::move(dAShape)), DeviceTensor({k, n})};
+    MatmulGrad r{DeviceTensor(std::move(dAShape)), gradientTensor(into, slot, {k, n})};
     if (mode == 0) {
         check(bf_hip_gemm_f32(0, 1, g.data(), b.data(), r.dA.data(), m, k, n, nullptr));   // dA = g b^T
         check(bf_hip_gemm_f32(1, 0, a.data(), g.data(), r.dB.data(), k, n, m, nullptr));   // dB = a^T g
@@ -124,6 +137,17 @@ inline DeviceTensor rmsnormBackward(const DeviceTensor& input, const DeviceTenso
     return out;
 }
 
+// residualGrad + rmsnormBackward(input, gradOutput) in one pass: how both composite blocks' backward passes end
+// (autodiff.cu:746,794).
+inline DeviceTensor rmsnormBackwardAdd(const DeviceTensor& input, const DeviceTensor& gradOutput, const DeviceTensor& residualGrad) {
+    require(input.shape() == gradOutput.shape() && residualGrad.shape() == input.shape(), "rmsnormBackward: incompatible shapes on the device");
+    require(input.rank() >= 2, "rmsnormBackward: needs a tensor of rank >= 2 on the device");
+    DeviceTensor out(input.shape());
+    check(bf_hip_rmsnorm_backward_add(input.data(), gradOutput.data(), residualGrad.data(), out.data(), detail::rowsOf(input),
+                                      detail::lastDim(input), nullptr));
+    return out;
+}
+
 inline DeviceTensor softmaxBackward(const DeviceTensor& input, const DeviceTensor& gradOutput) {
     require(input.shape() == gradOutput.shape(), "softmaxBackward: incompatible shapes on the device");
     require(input.rank() >= 2, "softmaxBackward: needs a tensor of rank >= 2 on the device");
@@ -133,22 +157,23 @@ inline DeviceTensor softmaxBackward(const DeviceTensor& input, const DeviceTenso
 }
 
 inline DeviceTensor embeddingLookupBackwardPreValidated(const DeviceTensor& tokenIds, const DeviceTensor& gradOutput,
-                                                         std::size_t vocabSize) {
+                                                         std::size_t vocabSize, const GradientTargets* into = nullptr) {
     require(tokenIds.rank() == 2 && gradOutput.rank() == 3 && tokenIds.dim(0) == gradOutput.dim(0) &&
                 tokenIds.dim(1) == gradOutput.dim(1),
             "embeddingLookupBackward: incompatible shapes on the device");
-    DeviceTensor dTable({vocabSize, gradOutput.dim(2)});
+    DeviceTensor dTable = detail::gradientTensor(into, 0, {vocabSize, gradOutput.dim(2)});
     check(bf_hip_embedding_backward(tokenIds.data(), gradOutput.data(), dTable.data(), tokenIds.elementCount(), vocabSize,
                                     gradOutput.dim(2), nullptr));
     return dTable;
 }
 
-inline DeviceTensor embeddingLookupBackward(const DeviceTensor& tokenIds, const DeviceTensor& gradOutput, std::size_t vocabSize) {
+inline DeviceTensor embeddingLookupBackward(const DeviceTensor& tokenIds, const DeviceTensor& gradOutput, std::size_t vocabSize,
+                                            const GradientTargets* into = nullptr) {
     require(tokenIds.rank() == 2 && gradOutput.rank() == 3 && tokenIds.dim(0) == gradOutput.dim(0) &&
                 tokenIds.dim(1) == gradOutput.dim(1),
             "embeddingLookupBackward: incompatible shapes on the device");
     detail::requireIdsInRange("embeddingLookupBackward", tokenIds, vocabSize, "token id");
-    return embeddingLookupBackwardPreValidated(tokenIds, gradOutput, vocabSize);
+    return embeddingLookupBackwardPreValidated(tokenIds, gradOutput, vocabSize, into);
 }
 
 struct PositionalEmbeddingGrad {
@@ -156,9 +181,10 @@ struct PositionalEmbeddingGrad {
     DeviceTensor dTable;
 };
 
-inline PositionalEmbeddingGrad addPositionalEmbeddingBackward(const DeviceTensor& gradOutput, std::size_t maxSeqLen) {
+inline PositionalEmbeddingGrad addPositionalEmbeddingBackward(const DeviceTensor& gradOutput, std::size_t maxSeqLen,
+                                                              const GradientTargets* into = nullptr) {
     require(gradOutput.rank() == 3, "addPositionalEmbeddingBackward: needs a gradient of rank 3 on the device");
-    PositionalEmbeddingGrad r{DeviceTensor(), DeviceTensor({maxSeqLen, gradOutput.dim(2)})};
+    PositionalEmbeddingGrad r{DeviceTensor(), detail::gradientTensor(into, 0, {maxSeqLen, gradOutput.dim(2)})};
     check(bf_hip_positional_backward(gradOutput.data(), r.dTable.data(), gradOutput.dim(0), gradOutput.dim(1), gradOutput.dim(2),
                                      maxSeqLen, nullptr));
     r.dInput = gradOutput.clone();
@@ -171,25 +197,28 @@ struct FeedForwardGrad {
 
 inline FeedForwardGrad feedForwardBackwardCached(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
                                                   const DeviceTensor& w2, const DeviceTensor& b2, const FeedForwardCache& cache,
-                                                  const DeviceTensor& gradOutput, bool useBf16, Activation act = Activation::Silu) {
+                                                  const DeviceTensor& gradOutput, bool useBf16, Activation act = Activation::Silu,
+                                                  const GradientTargets* into = nullptr) {
     (void)b2;
     require(gradOutput.shape() == input.shape(), "feedForwardBackward: gradient shape differs from the input");
     const int mode = useBf16 ? 2 : 0;
     if (cache.fused) {
         const std::size_t rows = detail::rowsOf(input), d = detail::lastDim(input), hidden = w1.dim(1);
-        DeviceTensor dNormed(cache.normed.shape()), dW1(w1.shape()), dB1({hidden}), dW2(w2.shape()), dB2({d});
+        DeviceTensor dNormed(cache.normed.shape()), dW1 = detail::gradientTensor(into, 0, w1.shape()),
+                     dB1 = detail::gradientTensor(into, 1, {hidden}), dW2 = detail::gradientTensor(into, 2, w2.shape()),
+                     dB2 = detail::gradientTensor(into, 3, {d});
         check(bf_hip_feedforward_bf16_backward(nullptr, reinterpret_cast<const uint16_t*>(cache.normedImage.data()), w1.data(), w2.data(),
                                                cache.gemm1.data(), reinterpret_cast<const uint16_t*>(cache.hiddenImage.data()),
                                                gradOutput.data(), static_cast<int>(act), dNormed.data(), dW1.data(), dB1.data(),
                                                dW2.data(), dB2.data(), rows, d, hidden, 1, nullptr));
-        DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, dNormed));
+        DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput);
         return FeedForwardGrad{std::move(dInput), std::move(dW1), std::move(dB1), std::move(dW2), std::move(dB2)};
     }
     DeviceTensor dB2 = biasGradientOnly(gradOutput);
-    MatmulGrad g2 = detail::projectionBackward(cache.hidden, w2, gradOutput, mode, cache.hidden.shape());
+    MatmulGrad g2 = detail::projectionBackward(cache.hidden, w2, gradOutput, mode, cache.hidden.shape(), into, 2);
     AddBiasSiluGrad hiddenGrad = addBiasActivationBackward(cache.gemm1, b1, g2.dA, act);
-    MatmulGrad g1 = detail::projectionBackward(cache.normed, w1, hiddenGrad.dGemmOutput, mode, cache.normed.shape());
-    DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, g1.dA));
+    MatmulGrad g1 = detail::projectionBackward(cache.normed, w1, hiddenGrad.dGemmOutput, mode, cache.normed.shape(), into, 0);
+    DeviceTensor dInput = rmsnormBackwardAdd(input, g1.dA, gradOutput);
     return FeedForwardGrad{std::move(dInput), std::move(g1.dB), std::move(hiddenGrad.dBias), std::move(g2.dB), std::move(dB2)};
 }
 
@@ -206,7 +235,7 @@ inline FeedForwardGrad feedForwardBackwardImpl(const DeviceTensor& input, const 
     MatmulGrad g2 = projectionBackward(cache.hidden, w2, gradOutput, mode, cache.hidden.shape());
     AddBiasSiluGrad hiddenGrad = addBiasActivationBackward(cache.gemm1, b1, g2.dA, act);
     MatmulGrad g1 = projectionBackward(cache.normed, w1, hiddenGrad.dGemmOutput, mode, cache.normed.shape());
-    DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, g1.dA));
+    DeviceTensor dInput = rmsnormBackwardAdd(input, g1.dA, gradOutput);
     (void)b2;
     return FeedForwardGrad{std::move(dInput), std::move(g1.dB), std::move(hiddenGrad.dBias), std::move(g2.dB), std::move(dB2)};
 }
@@ -230,38 +259,41 @@ struct SelfAttentionGrad {
 namespace detail {
 inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
                                                         const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
-                                                        const SelfAttentionCache& cache, const DeviceTensor& gradOutput, int mode) {
+                                                        const SelfAttentionCache& cache, const DeviceTensor& gradOutput, int mode,
+                                                        const GradientTargets* into = nullptr) {
     require(gradOutput.shape() == input.shape(), "selfAttentionBackward: gradient shape differs from the input");
     std::size_t batch = input.dim(0), seq = input.dim(1), dim = input.dim(2);
     float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
-    MatmulGrad outGrad = projectionBackward(cache.attnOutput, wout, gradOutput, mode, {batch, seq, dim});
+    MatmulGrad outGrad = projectionBackward(cache.attnOutput, wout, gradOutput, mode, {batch, seq, dim}, into, 3);
     FusedAttentionGrad attn = fusedAttentionBackward(outGrad.dA, cache.q, cache.k, cache.v, cache.attnOutput, cache.attnM,
                                                       cache.attnL, numHeads, scaleFactor, cache.causal ? 0 : seq);
     if (mode != 0) {
         // the three projection gradients share their input: one GEMM sums dQ Wq^T + dK Wk^T + dV Wv^T, one produces
         // the three weight gradients (for widths that are multiples of 256; separate GEMMs otherwise)
-        DeviceTensor dNormed({batch, seq, dim}), dWq(wq.shape()), dWk(wk.shape()), dWv(wv.shape());
+        DeviceTensor dNormed({batch, seq, dim}), dWq = gradientTensor(into, 0, wq.shape()), dWk = gradientTensor(into, 1, wk.shape()),
+                     dWv = gradientTensor(into, 2, wv.shape());
         const float* weights[3] = {wq.data(), wk.data(), wv.data()};
         const float* grads[3] = {attn.dQ.data(), attn.dK.data(), attn.dV.data()};
         float* weightGrads[3] = {dWq.data(), dWk.data(), dWv.data()};
         check(bf_hip_matmul_bf16_shared_input_backward(cache.normedFlat.data(), weights, grads, dNormed.data(), weightGrads, 3,
                                                        batch * seq, dim, dim, mode == 2, nullptr));
-        DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, dNormed));
+        DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput);
         return SelfAttentionGrad{std::move(dInput), std::move(dWq), std::move(dWk), std::move(dWv), std::move(outGrad.dB)};
     }
-    MatmulGrad gq = projectionBackward(cache.normedFlat, wq, attn.dQ, mode, {batch * seq, dim});
-    MatmulGrad gk = projectionBackward(cache.normedFlat, wk, attn.dK, mode, {batch * seq, dim});
-    MatmulGrad gv = projectionBackward(cache.normedFlat, wv, attn.dV, mode, {batch * seq, dim});
+    MatmulGrad gq = projectionBackward(cache.normedFlat, wq, attn.dQ, mode, {batch * seq, dim}, into, 0);
+    MatmulGrad gk = projectionBackward(cache.normedFlat, wk, attn.dK, mode, {batch * seq, dim}, into, 1);
+    MatmulGrad gv = projectionBackward(cache.normedFlat, wv, attn.dV, mode, {batch * seq, dim}, into, 2);
     DeviceTensor dNormed = add(add(gq.dA, gk.dA), gv.dA).reshaped({batch, seq, dim});
-    DeviceTensor dInput = add(gradOutput, rmsnormBackward(input, dNormed));
+    DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput);
     return SelfAttentionGrad{std::move(dInput), std::move(gq.dB), std::move(gk.dB), std::move(gv.dB), std::move(outGrad.dB)};
 }
 }  // namespace detail
 
 inline SelfAttentionGrad selfAttentionBackwardCached(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
                                                       const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
-                                                      const SelfAttentionCache& cache, const DeviceTensor& gradOutput, bool useBf16) {
-    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, useBf16 ? 2 : 0);
+                                                      const SelfAttentionCache& cache, const DeviceTensor& gradOutput, bool useBf16,
+                                                      const GradientTargets* into = nullptr) {
+    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, useBf16 ? 2 : 0, into);
 }
 // Stateless variants: recompute the forward first (reference: autodiff.cu:654-700).
 inline SelfAttentionGrad selfAttentionBackward(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,

@@ -133,6 +133,7 @@ public:
                 counts.push_back(p.grad.elementCount());
             }
         check(bf_hip_zero_multi(ptrs.data(), counts.data(), ptrs.size(), nullptr));
+        for (LayerState& layer : layers_) layer.gradsAreZero = true;
     }
 
     // Incremental forward for generation: only the new positions are processed, K/V of earlier positions
@@ -204,6 +205,9 @@ private:
         SelfAttentionCache attnCache;
         FeedForwardCache ffCache;
         KVCache kvCache;
+        // true from zeroGrad() until this layer's next backward pass: its gradient buffers hold zeros, so that pass may
+        // write the gradients there instead of adding them in
+        bool gradsAreZero = true;
     };
 
     static Parameter makeParameter(std::string name, std::vector<std::size_t> shape) {
@@ -244,17 +248,26 @@ private:
         }
     }
 
+    // target += delta, unless the backward pass already wrote delta into target (see GradientTargets)
     static void accumulate(DeviceTensor& target, const DeviceTensor& delta) {
+        if (delta.data() == target.data()) return;
         check(bf_hip_accumulate(target.data(), delta.data(), target.elementCount(), nullptr));
     }
 
     DeviceTensor applyBackward(LayerState& layer, const DeviceTensor& grad, bool trustedIds) {
         const LayerSpec& s = layer.spec;
         const DeviceTensor& x = layer.cachedInput;
+        GradientTargets targets;
+        const GradientTargets* into = nullptr;
+        if (layer.gradsAreZero) {
+            for (std::size_t i = 0; i < layer.params.size() && i < 4; ++i) targets.slot[i] = &layer.params[i].grad;
+            into = &targets;
+        }
+        layer.gradsAreZero = false;
         switch (s.kind) {
             case LayerKind::Linear: {
                 DeviceTensor dBias = biasGradientOnly(grad);
-                MatmulGrad g = detail::projectionBackward(x, layer.params[0].value, grad, useBf16_ ? 2 : 0, x.shape());
+                MatmulGrad g = detail::projectionBackward(x, layer.params[0].value, grad, useBf16_ ? 2 : 0, x.shape(), into, 0);
                 accumulate(layer.params[0].grad, g.dB);
                 accumulate(layer.params[1].grad, dBias);
                 return std::move(g.dA);
@@ -265,20 +278,20 @@ private:
             case LayerKind::RmsNorm: return rmsnormBackward(x, grad);
             case LayerKind::Softmax: return softmaxBackward(x, grad);
             case LayerKind::Embedding: {
-                DeviceTensor dTable = trustedIds ? embeddingLookupBackwardPreValidated(x, grad, s.arg0)
-                                                 : embeddingLookupBackward(x, grad, s.arg0);
+                DeviceTensor dTable = trustedIds ? embeddingLookupBackwardPreValidated(x, grad, s.arg0, into)
+                                                 : embeddingLookupBackward(x, grad, s.arg0, into);
                 accumulate(layer.params[0].grad, dTable);
                 return DeviceTensor::zeros(x.shape());   // token ids carry no gradient
             }
             case LayerKind::PositionalEmbedding: {
-                PositionalEmbeddingGrad g = addPositionalEmbeddingBackward(grad, s.arg0);
+                PositionalEmbeddingGrad g = addPositionalEmbeddingBackward(grad, s.arg0, into);
                 accumulate(layer.params[0].grad, g.dTable);
                 return std::move(g.dInput);
             }
             case LayerKind::Attention:
             case LayerKind::BidirectionalAttention: {   // the cache records which of the two the forward pass was
                 SelfAttentionGrad g = selfAttentionBackwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
-                                                                  layer.params[3].value, s.arg0, layer.attnCache, grad, useBf16_);
+                                                                  layer.params[3].value, s.arg0, layer.attnCache, grad, useBf16_, into);
                 accumulate(layer.params[0].grad, g.dWq);
                 accumulate(layer.params[1].grad, g.dWk);
                 accumulate(layer.params[2].grad, g.dWv);
@@ -288,7 +301,7 @@ private:
             case LayerKind::FeedForward: {
                 FeedForwardGrad g = feedForwardBackwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
                                                               layer.params[3].value, layer.ffCache, grad, useBf16_,
-                                                              s.arg1 == 1 ? Activation::Gelu : Activation::Silu);
+                                                              s.arg1 == 1 ? Activation::Gelu : Activation::Silu, into);
                 accumulate(layer.params[0].grad, g.dW1);
                 accumulate(layer.params[1].grad, g.dB1);
                 accumulate(layer.params[2].grad, g.dW2);

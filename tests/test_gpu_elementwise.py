@@ -98,6 +98,10 @@ def test_row_ops(hip, oracle, rng, rows, features):
     dx, dg = D.fromHost(x), D.fromHost(g)
     assert_close(ops.rmsnorm(dx).toHost(), oracle.rmsnorm(x), what="rmsnorm")
     assert_close(ops.rmsnormBackward(dx, dg).toHost(), oracle.rmsnormBackward(x, g), what="rmsnormBackward")
+    # the residual connection's gradient joined in the same pass: the separate add's result, bit for bit
+    res = r(rng, rows, features)
+    assert_bits_equal(ops.rmsnormBackwardAdd(dx, dg, D.fromHost(res)).toHost(), ops.add(D.fromHost(res), ops.rmsnormBackward(dx, dg)).toHost(),
+                      "rmsnormBackwardAdd")
     assert_close(ops.softmax(dx).toHost(), oracle.softmax(x), what="softmax")
     assert_close(ops.softmaxBackward(dx, dg).toHost(), oracle.softmaxBackward(x, g), what="softmaxBackward")
 

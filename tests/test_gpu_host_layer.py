@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import refvectors as rv
-from parity import BF16_TOL, assert_close
+from parity import BF16_TOL, assert_bits_equal, assert_close
 
 pytestmark = pytest.mark.gpu
 f32 = np.float32
@@ -224,6 +224,40 @@ def test_config1_tiny_lm_full_step_against_oracle(hip, oracle, rng, act):
         # AdamW's first step is lr * g / (|g| + eps): where |g| is comparable to eps = 1e-8 the step depends on
         # the gradient's last bits, but it never exceeds lr, so the floor is a small fraction (2 %) of lr = 1e-3
         assert_close(gpu.value(i), cpu.value(i), what="param " + gpu.names[i], scale=0.02 * 1e-3 / 1e-4)
+
+
+@pytest.mark.parametrize("use_bf16", [False, True])
+def test_gradients_accumulate_over_backward_passes(hip, rng, use_bf16):
+    """cuda::Model::backward adds into the parameters' gradients (model.cu:40-46, 332-383).  The first pass after
+    zeroGrad() writes them in place of adding to zeros; a second pass without zeroGrad() must double them, and
+    zeroGrad() must bring back the single-pass values."""
+    from blackforge_amd import hostlayer as hl
+    vocab, dim, seq, batch, heads, hidden = 96, 64, 32, 4, 2, 128
+    gpu = hl.HostModel(_lm_layers(hl, vocab, dim, seq, heads, hidden, 0), use_bf16=use_bf16)
+    for i, c in enumerate(gpu.counts):
+        gpu.set_value(i, r(rng, c, scale=0.05))
+    D = hip.DeviceTensor
+    x = D.fromHost(rng.integers(0, vocab, (batch, seq)).astype(f32))
+    t = D.fromHost(rng.integers(0, vocab, batch * seq).astype(f32))
+
+    def one_pass():
+        gpu.forward(x, trusted=True)
+        gpu.loss(t)
+        gpu.backward(trusted=True)
+
+    gpu.zeroGrad()
+    one_pass()
+    single = [gpu.grad(i).copy() for i in range(len(gpu.counts))]
+    assert any(np.abs(g).max() > 0 for g in single)
+    one_pass()
+    for i, g in enumerate(single):
+        assert_close(gpu.grad(i), 2 * g, tol=1e-6, what="accumulated grad " + gpu.names[i])
+    gpu.zeroGrad()
+    for i in range(len(gpu.counts)):
+        assert not gpu.grad(i).any(), "zeroGrad " + gpu.names[i]
+    one_pass()
+    for i, g in enumerate(single):
+        assert_bits_equal(gpu.grad(i), g, "grad after zeroGrad " + gpu.names[i])
 
 
 def test_bf16_model_step_stays_within_bf16_tolerance(hip, oracle, rng):
