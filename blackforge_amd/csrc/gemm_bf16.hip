@@ -24,13 +24,14 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned short ushort8 __attribute__((ext_vector_type(8)));
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));   // a float4 that may start on any 4-byte boundary
 
 
 inline size_t pad8(size_t n) { return (n + 7) / 8 * 8; }
 
 // out[r*ld + 0..colsPad) = bf16(x[r, 0..cols)), zero padded.
 __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict__ x, unsigned short* __restrict__ out,
-                                                        size_t rows, size_t cols, size_t colsPad, int vec, size_t ld) {
+                                                        size_t rows, size_t cols, size_t colsPad, size_t ld) {
     const size_t groupsPerRow = colsPad / 8;
     const size_t total = rows * groupsPerRow;
     const size_t stride = size_t(gridDim.x) * blockDim.x;
@@ -38,8 +39,10 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict_
         size_t r = gidx / groupsPerRow, c = (gidx - r * groupsPerRow) * 8;
         const float* src = x + r * cols + c;
         ushort8 v;
-        if (vec && c + 8 <= cols) {
-            float4v a = loadf4(src), b = loadf4(src + 4);
+        if (c + 8 <= cols) {
+            // two 16-byte loads; global memory serves them from any 4-byte boundary, so rows of an odd width (which do
+            // not start on 16-byte boundaries) take the same path
+            float4u a = *reinterpret_cast<const float4u*>(src), b = *reinterpret_cast<const float4u*>(src + 4);
             v[0] = toBf16Bits(a.x); v[1] = toBf16Bits(a.y); v[2] = toBf16Bits(a.z); v[3] = toBf16Bits(a.w);
             v[4] = toBf16Bits(b.x); v[5] = toBf16Bits(b.y); v[6] = toBf16Bits(b.z); v[7] = toBf16Bits(b.w);
         } else {
@@ -810,8 +813,7 @@ int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, 
     size_t colsPad = pad8(cols);
     size_t groups = rows * (colsPad / 8);
     if (groups == 0) return BF_OK;
-    int vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && cols % 4 == 0;
-    convertKernel<<<gridFor(groups, kBlock), kBlock, 0, s>>>(x, out, rows, cols, colsPad, vec, ld ? ld : colsPad);
+    convertKernel<<<gridFor(groups, kBlock), kBlock, 0, s>>>(x, out, rows, cols, colsPad, ld ? ld : colsPad);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
