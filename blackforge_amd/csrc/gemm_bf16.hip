@@ -168,12 +168,61 @@ struct Epilogue {
     const float* residual;
 };
 
+// 4 x 4 transposition among the four lanes of a quad: lane t comes in holding one column of a 4 x 4 block (v_k = element
+// (k, t)) and leaves holding one row (v_c = element (t, c)).  Two exchange steps (with lane t^1, then lane t^2), each a
+// data-parallel move between neighbouring lanes, no LDS.
+__device__ __forceinline__ float quadXor1(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ float quadXor2(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+}
+__device__ __forceinline__ void quadTranspose(float& v0, float& v1, float& v2, float& v3, int t) {
+    const bool odd = (t & 1) != 0;
+    const float r01 = quadXor1(odd ? v0 : v1), r23 = quadXor1(odd ? v2 : v3);
+    if (odd) { v0 = r01; v2 = r23; } else { v1 = r01; v3 = r23; }
+    const bool upper = (t & 2) != 0;
+    const float r02 = quadXor2(upper ? v0 : v2), r13 = quadXor2(upper ? v1 : v3);
+    if (upper) { v0 = r02; v1 = r13; } else { v2 = r02; v3 = r13; }
+}
+
+// An accumulator tile of the 32x32 MFMA gives lane (li, half) column li of rows 8g + 4 half + 0..3 (g = 0..3).  Stored
+// as they lie, the 64 lanes of a store instruction cover two rows of 128 bytes, 4 bytes a lane: a 256 x 256 tile takes
+// 128 such instructions per lane, which costs a 768-long product a third of its time.  When everything is 16-byte aligned
+// each quad of lanes first transposes its 4 x 4 blocks, so that a lane holds four consecutive columns of ONE row and stores
+// them as 16 bytes: a quarter of the instructions, still whole 128-byte lines per row.
 template <int TM, int TN>
 __device__ __forceinline__ void storeAccumulators(float16v (&acc)[TM][TN], const Epilogue& e, int M, int N, int row0,
                                                   int col0, int li, int half) {
     const int which = col0 / e.splitN;              // uniform over the tile
     float* __restrict__ C = which == 0 ? e.c[0] : which == 1 ? e.c[1] : e.c[2];   // no indexed access: the struct stays in registers
     const int shift = which * e.splitN, ld = e.splitN;
+    const bool wide = ((N | ld) & 3) == 0 &&
+                      ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(e.bias) | reinterpret_cast<uintptr_t>(e.residual)) & 15u) == 0;
+    if (wide) {
+        const int t = li & 3, colq = 4 * (li >> 2);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int col = col0 + j * 32 + colq;
+                float4v b = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (e.bias && col < N) b = loadf4(e.bias + col);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float v0 = acc[i][j][4 * g], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
+                    quadTranspose(v0, v1, v2, v3, t);
+                    const int row = row0 + i * 32 + 8 * g + 4 * half + t;
+                    if (row < M && col < N) {
+                        float4v v = {v0, v1, v2, v3};
+                        if (e.bias) v = v + b;
+                        if (e.residual) v = v + loadf4(e.residual + size_t(row) * N + col);
+                        storef4(C + size_t(row) * ld + (col - shift), v);
+                    }
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
