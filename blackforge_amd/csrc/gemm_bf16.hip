@@ -459,6 +459,89 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
     storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
+// 128 x 256 tiles on sixteen wavefronts (four per SIMD, each with a 32 x 64 share), one barrier per K step: while step T
+// is multiplied out of LDS buffer T&1 (fragments of the next 16-deep slice are read while the current one is multiplied),
+// the registers holding step T+1 go to the other buffer and the loads of step T+2 are issued.  The K loop costs what the
+// eight-wavefront ping-pong costs for a tile of this size (the LDS pipe bounds both), but filling and draining it does
+// not: sixteen wavefronts fetch the first step and store the tile in half the time, and no group waits a phase for the
+// other.  Products with a short contraction, whose tiles live for twenty microseconds, are several microseconds faster per
+// round of tiles; long contractions stay on the 256-row ping-pong kernel, which moves fewer operand bytes per MFMA.
+template <int XCD_ORDER>
+__global__ void __launch_bounds__(1024, 4) gemmBf16SixteenWaveKernel(const unsigned short* __restrict__ A,
+                                                                    const unsigned short* __restrict__ Bt, Epilogue epi, int M,
+                                                                    int N, int K, int lda, int ldb, int gmLog, int gnLog) {
+    constexpr int BM = 128, BN = 256, TM = 1, TN = 2;
+    extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
+    unsigned short* as = lds;                        // [2][128][LDS_ROW]
+    unsigned short* bs = lds + 2 * BM * LDS_ROW;     // [2][256][LDS_ROW]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int tm, tn;
+    if (XCD_ORDER) {
+        if (!tileIndexXcd(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, gmLog, gnLog, tm, tn)) return;
+    } else {
+        tileIndexGrouped(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tm, tn);
+    }
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int wm0 = (wave & 3) * 32, wn0 = (wave >> 2) * 64;
+    const int lr = tid >> 3, lc = (tid & 7) * 8;     // 128 rows x 128 bytes per pass: A takes one pass, Bt two
+    const unsigned short* aRow = A + size_t(min(m0 + lr, M - 1)) * lda;
+    const unsigned short* bRow[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) bRow[i] = Bt + size_t(min(n0 + lr + 128 * i, N - 1)) * ldb;
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[0][j][r] = 0.0f;
+    const int steps = max((K + BKK - 1) / BKK, 1);
+    const int ldsW = lr * LDS_ROW + lc;
+    uint4v stageA = loadChunk(aRow, lc, K), stageB[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) stageB[i] = loadChunk(bRow[i], lc, K);
+    *reinterpret_cast<uint4v*>(as + ldsW) = zeroPast(stageA, lc, K);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4v*>(bs + ldsW + 128 * i * LDS_ROW) = zeroPast(stageB[i], lc, K);
+    if (steps > 1) {
+        stageA = loadChunk(aRow, BKK + lc, K);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) stageB[i] = loadChunk(bRow[i], BKK + lc, K);
+    }
+    __syncthreads();
+    bf16x8 a[2], b[2][TN];
+    for (int T = 0; T < steps; ++T) {
+        const int par = T & 1;
+        const unsigned short* ac = as + (par * BM + wm0 + li) * LDS_ROW + 8 * half;
+        const unsigned short* bc = bs + (par * BN + wn0 + li) * LDS_ROW + 8 * half;
+        if (T + 1 < steps) {
+            const int kNext = (T + 1) * BKK + lc;
+            *reinterpret_cast<uint4v*>(as + (par ^ 1) * BM * LDS_ROW + ldsW) = zeroPast(stageA, kNext, K);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                *reinterpret_cast<uint4v*>(bs + ((par ^ 1) * BN + 128 * i) * LDS_ROW + ldsW) = zeroPast(stageB[i], kNext, K);
+            if (T + 2 < steps) {
+                stageA = loadChunk(aRow, kNext + BKK, K);
+#pragma unroll
+                for (int i = 0; i < 2; ++i) stageB[i] = loadChunk(bRow[i], kNext + BKK, K);
+            }
+        }
+        a[0] = *reinterpret_cast<const bf16x8*>(ac);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[0][j] = *reinterpret_cast<const bf16x8*>(bc + j * 32 * LDS_ROW);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            if (kk < 3) {
+                a[(kk + 1) & 1] = *reinterpret_cast<const bf16x8*>(ac + (kk + 1) * 16);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) b[(kk + 1) & 1][j] = *reinterpret_cast<const bf16x8*>(bc + j * 32 * LDS_ROW + (kk + 1) * 16);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk & 1], b[kk & 1][j], acc[0][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
+}
+
 // out = sum over slices of partial[s*sliceStride + i] (+ bias[i % N] + residual[i]), slices added in index order
 // (deterministic), written through the epilogue's output split.  sliceStride is a multiple of 4; `vec` says
 // that every pointer is 16-byte aligned and N and splitN are multiples of 4.
@@ -670,6 +753,30 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
     return BF_OK;
 }
 
+int launchSixteenWave(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
+                      size_t lda, size_t ldb, hipStream_t s) {
+    const size_t tilesM = (M + 127) / 128, tilesN = (N + 255) / 256;
+    constexpr size_t smem = size_t(2) * (128 + 256) * LDS_ROW * sizeof(unsigned short);
+    int gmLog = 2, gnLog = 3;
+    size_t bestCost = 0, blocks = 0;
+    for (int g = 0; g <= 5; ++g) {
+        size_t gm = size_t(1) << g, gn = size_t(32) >> g;
+        size_t nb = ((tilesM + gm - 1) / gm) * ((tilesN + gn - 1) / gn);
+        size_t cost = nb * 1000 + gm + gn;
+        if (g == 0 || cost < bestCost) { bestCost = cost; gmLog = g; gnLog = 5 - g; blocks = nb; }
+    }
+    const bool xcdOrder = blocks * 32 <= (tilesM * tilesN) * 5 / 4 && (blocks % 8 == 0 || blocks >= 64);
+    const size_t grid = xcdOrder ? (blocks + 7) / 8 * 8 * 32 : tilesM * tilesN;
+    if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+    auto kernel = xcdOrder ? gemmBf16SixteenWaveKernel<1> : gemmBf16SixteenWaveKernel<0>;
+    int st = allowSharedMemory(kernel, smem);
+    if (st != BF_OK) return st;
+    kernel<<<dim3(unsigned(grid)), 1024, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), xcdOrder ? gmLog : 0,
+                                                    xcdOrder ? gnLog : 0);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
 template <int BM>
 int launchPingPongTn(const unsigned short* A, const unsigned short* B, const Epilogue& epi, size_t M, size_t N, size_t K,
                      size_t lda, size_t ldb, hipStream_t s, size_t slices, size_t kPer, size_t sliceStride) {
@@ -783,6 +890,14 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
     constexpr double kHalfTileCost = 0.78;
     const double bigTime = bigTiles >= cus * 3 / 4 ? double((bigTiles + cus - 1) / cus) : 1e30;
     const double halfTime = halfTiles >= cus * 3 / 4 ? double((halfTiles + cus - 1) / cus) * kHalfTileCost : 1e30;
+    if (halfTiles >= cus * 3 / 4) {
+        // measured per round of tiles, in microseconds: the 256-row ping-pong 8 + 1.56 per K step, sixteen wavefronts on
+        // 128-row tiles 5 + 0.95 per K step
+        const double stepsAll = double((K + BKK - 1) / BKK);
+        const double big = bigTiles >= cus * 3 / 4 ? double((bigTiles + cus - 1) / cus) * (8.0 + 1.56 * stepsAll) : 1e30;
+        const double wide = double((halfTiles + cus - 1) / cus) * (5.0 + 0.95 * stepsAll);
+        if (wide < big) return launchSixteenWave(A, Bt, epi, M, N, K, lda, ldb, s);
+    }
     if (bigTime <= halfTime && bigTime < 1e30) return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
     if (halfTime < 1e30) return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s);
     // Few tiles but a long contraction (the weight-gradient products, K = all tokens): the same kernel with K cut into

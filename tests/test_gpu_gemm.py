@@ -155,8 +155,9 @@ def test_bf16_gemm_tn_entry(hip, rng, m, n, k):
                                    (6200, 72, 1500)])
 def test_bf16_projection_large_tile_kernel(hip, oracle, rng, m, k, n):
     """Shapes with enough 256x256 tiles for the large-product kernel (ragged edges, a K tail, and a tile grid
-    that is dealt to the XCDs in blocks), and tall narrow ones that take its 128-row-tile form.  Expected value: float64 product of the bf16-rounded operands, which
-    the oracle's fp32 matmul matches to 1e-6 on the sampled rows below."""
+    that is dealt to the XCDs in blocks), and tall narrow ones that take the 128-row tiles of the sixteen-wavefront kernel
+    (with a K tail and ragged edges too).  Expected value: float64 product of the bf16-rounded operands, which the oracle's
+    fp32 matmul matches to 1e-6 on the sampled rows below."""
     D, ops = hip.DeviceTensor, hip.ops
     a, b = r(rng, m, k), r(rng, k, n, scale=0.1)
     ar, br = oracle.roundToBf16(a), oracle.roundToBf16(b)
