@@ -34,10 +34,10 @@ PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
 
 # HBM bytes per launch of the dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this workload,
-# each scaled by what the same counter reads for a plain 256 MiB copy (x2.000 and x1.000): 903.0 MB read +
+# each scaled by what the same counter reads for a plain 256 MiB copy (x2.000 and x1.000): 640.4 MB read +
 # 1249.9 MB written (1095 MB of that is the dS hand-over).  profiles/attention_c3_kernel_trace.md holds the commands
 # and the raw counter values.
-MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvKernel": 2152880400}
+MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvKernel": 1890348162}
 
 
 def attention_flops(batch, heads, seq, hd):
