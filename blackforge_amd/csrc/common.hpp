@@ -165,6 +165,24 @@ template <int ACT> __device__ __forceinline__ float actD(float x) {
     else if constexpr (ACT == BF_ACT_GELU) return geluD(x);
     else return reluD(x);
 }
+// 4 x 4 transposition among the four lanes of a quad: lane t comes in holding one column of a 4 x 4 block (v_k = element
+// (k, t)) and leaves holding one row (v_c = element (t, c)).  Two exchange steps (with lane t^1, then lane t^2), each a
+// data-parallel move between neighbouring lanes, no LDS.
+__device__ __forceinline__ float quadXor1(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ float quadXor2(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+}
+__device__ __forceinline__ void quadTranspose(float& v0, float& v1, float& v2, float& v3, int t) {
+    const bool odd = (t & 1) != 0;
+    const float r01 = quadXor1(odd ? v0 : v1), r23 = quadXor1(odd ? v2 : v3);
+    if (odd) { v0 = r01; v2 = r23; } else { v1 = r01; v3 = r23; }
+    const bool upper = (t & 2) != 0;
+    const float r02 = quadXor2(upper ? v0 : v2), r13 = quadXor2(upper ? v1 : v3);
+    if (upper) { v0 = r02; v1 = r13; } else { v2 = r02; v3 = r13; }
+}
+
 // fp32 -> bf16 bits, round to nearest even, NaN preserved (floatToBf16, ops_tensorcore.cu:21-26)
 __device__ __forceinline__ unsigned short toBf16Bits(float x) {
     __bf16 h = static_cast<__bf16>(x);

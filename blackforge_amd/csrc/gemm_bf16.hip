@@ -168,24 +168,6 @@ struct Epilogue {
     const float* residual;
 };
 
-// 4 x 4 transposition among the four lanes of a quad: lane t comes in holding one column of a 4 x 4 block (v_k = element
-// (k, t)) and leaves holding one row (v_c = element (t, c)).  Two exchange steps (with lane t^1, then lane t^2), each a
-// data-parallel move between neighbouring lanes, no LDS.
-__device__ __forceinline__ float quadXor1(float v) {
-    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-}
-__device__ __forceinline__ float quadXor2(float v) {
-    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-}
-__device__ __forceinline__ void quadTranspose(float& v0, float& v1, float& v2, float& v3, int t) {
-    const bool odd = (t & 1) != 0;
-    const float r01 = quadXor1(odd ? v0 : v1), r23 = quadXor1(odd ? v2 : v3);
-    if (odd) { v0 = r01; v2 = r23; } else { v1 = r01; v3 = r23; }
-    const bool upper = (t & 2) != 0;
-    const float r02 = quadXor2(upper ? v0 : v2), r13 = quadXor2(upper ? v1 : v3);
-    if (upper) { v0 = r02; v1 = r13; } else { v2 = r02; v3 = r13; }
-}
-
 // An accumulator tile of the 32x32 MFMA gives lane (li, half) column li of rows 8g + 4 half + 0..3 (g = 0..3).  Stored
 // as they lie, the 64 lanes of a store instruction cover two rows of 128 bytes, 4 bytes a lane: a 256 x 256 tile takes
 // 128 such instructions per lane, which costs a 768-long product a third of its time.  When everything is 16-byte aligned
