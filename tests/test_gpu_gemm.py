@@ -168,11 +168,14 @@ def test_bf16_projection_large_tile_kernel(hip, oracle, rng, m, k, n):
     assert_close(c, expected, tol=1e-4, what="bf16 fwd (large tiles) vs rounded operands")
 
 
-@pytest.mark.parametrize("m,k,n", [(33, 40, 24), (300, 72, 520), (2100, 136, 3000), (70, 4100, 90)])
+@pytest.mark.parametrize("m,k,n", [(33, 40, 24), (300, 72, 520), (2100, 136, 3000), (70, 4100, 90), (6200, 72, 1501), (4100, 136, 4093),
+                                   (4100, 72, 4096)])
 @pytest.mark.parametrize("with_bias,with_residual", [(True, False), (False, True), (True, True), (False, False)])
 def test_bf16_linear_with_adds_in_the_store(hip, oracle, rng, m, k, n, with_bias, with_residual):
     """bf_hip_linear_bf16 = matmulBf16 followed by addBias / addBiasResidual / add (ops.hpp:14,30,8), through every
-    GEMM path: small tiles, large tiles, and a contraction cut into slices."""
+    GEMM path: small tiles, 128-row tiles on sixteen wavefronts, 256-row tiles, and a contraction cut into slices; widths
+    that are multiples of four (16-byte stores after the transposition inside lane quads) and widths that are not
+    (element-wise stores)."""
     D, ops = hip.DeviceTensor, hip.ops
     a, w, bias, res = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, n), r(rng, m, n)
     got = ops.linearBf16Fused(D.fromHost(a), D.fromHost(w), D.fromHost(bias) if with_bias else None,
