@@ -75,6 +75,7 @@ SIGNATURES = {
     "bf_hip_softmax": [P, P, c_size, c_size, S],
     "bf_hip_softmax_backward": [P, P, P, c_size, c_size, S],
     "bf_hip_bias_grad": [P, P, c_size, c_size, S],
+    "bf_hip_bias_grad_static": [P, P, c_size, c_size, S],
     "bf_hip_count_out_of_range": [P, c_size, c_size, ctypes.POINTER(c_size), ctypes.POINTER(c_ll), S],
     "bf_hip_embedding_forward": [P, P, P, c_size, c_size, c_size, S],
     "bf_hip_embedding_backward": [P, P, P, c_size, c_size, c_size, S],

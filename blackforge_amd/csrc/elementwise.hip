@@ -9,6 +9,13 @@
 
 #include <vector>
 
+// Workspace of bf_hip_bias_grad_static: the partial rows of the column sum live in a device array that is part of the
+// library's code object, so that entry point never asks the driver or the pool for memory.  Each device that runs the
+// library holds its own copy at its own address; the address is looked up once per device (columnSumWorkspace below).
+// The name is only the host-side handle of the symbol: kernels and fills are always given the looked-up address.
+static constexpr size_t kColumnSumWorkspaceFloats = size_t(2) << 20;   // 8 MiB: 256 partial rows of up to 8192 columns
+static __device__ __align__(256) float scratch[kColumnSumWorkspaceFloats];
+
 namespace bf {
 namespace {
 
@@ -255,9 +262,12 @@ __global__ void __launch_bounds__(kBlock) columnFinishKernel(const float* __rest
     }
 }
 
+// `workspace`, when given, takes the place of the pool block for the partial rows (the caller has checked that it holds
+// workspaceFloats floats); the kernels and their geometry are the same either way.
 template <int FUSED, int ACT>
 int launchColumnSum(const float* src, const float* bias, const float* dHidden, float* dGemm, float* dBias,
-                    size_t rows, size_t features, hipStream_t stream, unsigned short* image = nullptr) {
+                    size_t rows, size_t features, hipStream_t stream, unsigned short* image = nullptr,
+                    float* workspace = nullptr, size_t workspaceFloats = 0) {
     if (features == 0) return BF_OK;
     if (rows == 0) {
         if (dBias) return bf_hip_fill_zero(dBias, features * sizeof(float), stream);
@@ -266,9 +276,12 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
     bool vec = aligned16(src) && (!FUSED || (aligned16(bias) && aligned16(dHidden) && aligned16(dGemm)));
     RowGeom g = rowGeometry(rows, features, vec, 256, 4);
     size_t parts = g.grid.y;
-    Scratch scratch(dBias ? parts * features * sizeof(float) : 0);
+    if (workspace && dBias && parts * features > workspaceFloats)
+        return failInvalid("column_sum", "the partial sums (" + std::to_string(parts) + " rows of " + std::to_string(features) +
+                                             " columns) exceed the static workspace of " + std::to_string(workspaceFloats) + " floats");
+    Scratch scratch(dBias && !workspace ? parts * features * sizeof(float) : 0);
     if (scratch.status != BF_OK) return scratch.status;
-    float* partial = dBias ? scratch.as<float>() : nullptr;
+    float* partial = dBias ? (workspace ? workspace : scratch.as<float>()) : nullptr;
     if (image && g.vec != 4) return failInvalid("act_backward_image", "operands must be 16-byte aligned and the width a multiple of 4");
     if (g.vec == 4)
         columnSumKernel<4, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features, image);
@@ -282,10 +295,21 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
     return BF_OK;
 }
 
-struct ZeroTarget {
-    float* ptr;
-    size_t count;
-};
+constexpr int kMaxDevices = 64;
+int columnSumWorkspace(float** out) {
+    static float* perDevice[kMaxDevices] = {};
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    BF_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index beyond the per-device workspace table");
+    if (perDevice[dev] == nullptr) {
+        void* address = nullptr;
+        BF_HIP_TRY(hipGetSymbolAddress(&address, HIP_SYMBOL(::scratch)));
+        BF_REQUIRE(address != nullptr, "the static workspace has no device address");
+        perDevice[dev] = static_cast<float*>(address);
+    }
+    *out = perDevice[dev];
+    return BF_OK;
+}
 
 // One flat grid over all tensors laid end to end: a block owns 1024 consecutive elements of one tensor,
 // which it finds in the table of first-block indices.
@@ -422,6 +446,16 @@ int bf_hip_bias_grad(const float* g, float* dBias, size_t rows, size_t features,
     if (features == 0) return BF_OK;
     BF_REQUIRE(dBias && (g || rows == 0), "NULL pointer");
     return launchColumnSum<0, 0>(g, nullptr, nullptr, nullptr, dBias, rows, features, asStream(stream));
+}
+
+int bf_hip_bias_grad_static(const float* g, float* dBias, size_t rows, size_t features, bf_stream_t stream) {
+    if (features == 0) return BF_OK;
+    BF_REQUIRE(dBias && (g || rows == 0), "NULL pointer");
+    float* workspace = nullptr;
+    int status = columnSumWorkspace(&workspace);
+    if (status != BF_OK) return status;
+    return launchColumnSum<0, 0>(g, nullptr, nullptr, nullptr, dBias, rows, features, asStream(stream), nullptr, workspace,
+                                 kColumnSumWorkspaceFloats);
 }
 
 int bf_hip_add_bias_act_backward(const float* gemm, const float* bias, const float* dHidden, float* dGemm,

@@ -147,6 +147,14 @@ int bf_hip_softmax_backward(const float* x, const float* g, float* out, size_t r
                             bf_stream_t stream);
 /* biasGradientOnly / addBiasBackward's dBias: autodiff.hpp:52,59   dBias[c] = sum_r g[r,c] */
 int bf_hip_bias_grad(const float* g, float* dBias, size_t rows, size_t features, bf_stream_t stream);
+/* bf_hip_bias_grad for callers that cannot allocate device memory (code under HIP graph capture, serving loops that
+ * forbid hipMalloc): no counterpart in the reference.  Same kernels and same results as bf_hip_bias_grad, but the
+ * partial sums go to an 8 MiB array that is part of the library's code object (one copy per device, held until the
+ * process ends) instead of a pool block; the call makes no hipMalloc/hipFree and takes nothing from the pool.
+ * Limit: min(256, ceil(rows / (4 * r))) * features <= 2^21, with r = 256 / min(256, 2^ceil(log2(features / 4))) rows
+ * per workgroup: any row count up to 8192 features, fewer rows above that; BF_ERR_INVALID_ARGUMENT beyond it.
+ * Calls on one device share the array, so two of them in flight at once (on different streams) race. */
+int bf_hip_bias_grad_static(const float* g, float* dBias, size_t rows, size_t features, bf_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Gather / scatter                                 (reference: ops_elementwise.cu, autodiff.cu)
