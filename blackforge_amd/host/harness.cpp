@@ -223,6 +223,172 @@ int bfh_model_load_checkpoint(void* h, const char* path) {
     });
 }
 
+// ---- composite blocks of the C++ operator layer, for parity tests against the CPU backend --------------------
+// Every pointer is device memory owned by the caller; results are copied into the caller's buffers.
+// variant: 0 the stateless fp32 operator, 1 the stateless bf16 operator, 2 the *ForwardCached / *BackwardCached pair in
+// fp32, 3 the same pair with bf16 projections (cached weight images).
+namespace {
+void copyOut(float* dst, const hip::DeviceTensor& src) {
+    if (dst != nullptr && src.elementCount() != 0)
+        hip::check(bf_hip_memcpy_d2d(dst, src.data(), src.elementCount() * sizeof(float), nullptr));
+}
+struct AttentionWeights {
+    Borrowed wq, wk, wv, wout;
+    AttentionWeights(const float* q, const float* k, const float* v, const float* o, std::size_t dim)
+        : wq(q, {dim, dim}), wk(k, {dim, dim}), wv(v, {dim, dim}), wout(o, {dim, dim}) {}
+};
+struct FeedForwardWeights {
+    Borrowed w1, b1, w2, b2;
+    FeedForwardWeights(const float* w1p, const float* b1p, const float* w2p, const float* b2p, std::size_t d, std::size_t hidden)
+        : w1(w1p, {d, hidden}), b1(b1p, {hidden}), w2(w2p, {hidden, d}), b2(b2p, {d}) {}
+};
+}  // namespace
+
+int bfh_self_attention(const float* x, const float* wq, const float* wk, const float* wv, const float* wout, size_t batch, size_t seq,
+                       size_t dim, size_t heads, int variant, int causal, float* out) {
+    return guarded([&] {
+        Borrowed in(x, {batch, seq, dim});
+        AttentionWeights w(wq, wk, wv, wout, dim);
+        hip::DeviceTensor y;
+        hip::SelfAttentionCache cache;
+        if (variant >= 2) hip::invalidateBf16WeightCache();
+        const auto &a = w.wq.tensor, &b = w.wk.tensor, &c = w.wv.tensor, &d = w.wout.tensor;
+        switch (variant * 2 + (causal ? 1 : 0)) {
+            case 1: y = hip::selfAttention(in.tensor, a, b, c, d, heads); break;
+            case 0: y = hip::bidirectionalSelfAttention(in.tensor, a, b, c, d, heads); break;
+            case 3: y = hip::selfAttentionBf16(in.tensor, a, b, c, d, heads); break;
+            case 2: y = hip::bidirectionalSelfAttentionBf16(in.tensor, a, b, c, d, heads); break;
+            case 5: case 7: y = hip::selfAttentionForwardCached(in.tensor, a, b, c, d, heads, variant == 3, cache); break;
+            case 4: case 6: y = hip::bidirectionalSelfAttentionForwardCached(in.tensor, a, b, c, d, heads, variant == 3, cache); break;
+            default: throw std::invalid_argument("bfh_self_attention: unknown variant");
+        }
+        copyOut(out, y);
+    });
+}
+
+int bfh_self_attention_backward(const float* x, const float* wq, const float* wk, const float* wv, const float* wout, const float* g,
+                                size_t batch, size_t seq, size_t dim, size_t heads, int variant, int causal, float* dInput, float* dWq,
+                                float* dWk, float* dWv, float* dWout) {
+    return guarded([&] {
+        Borrowed in(x, {batch, seq, dim}), grad(g, {batch, seq, dim});
+        AttentionWeights w(wq, wk, wv, wout, dim);
+        const auto &a = w.wq.tensor, &b = w.wk.tensor, &c = w.wv.tensor, &d = w.wout.tensor;
+        hip::SelfAttentionGrad r;
+        if (variant >= 2) {
+            hip::invalidateBf16WeightCache();
+            hip::SelfAttentionCache cache;
+            if (causal) hip::selfAttentionForwardCached(in.tensor, a, b, c, d, heads, variant == 3, cache);
+            else hip::bidirectionalSelfAttentionForwardCached(in.tensor, a, b, c, d, heads, variant == 3, cache);
+            r = hip::selfAttentionBackwardCached(in.tensor, a, b, c, d, heads, cache, grad.tensor, variant == 3);
+        } else if (variant == 0) {
+            r = causal ? hip::selfAttentionBackward(in.tensor, a, b, c, d, heads, grad.tensor)
+                       : hip::bidirectionalSelfAttentionBackward(in.tensor, a, b, c, d, heads, grad.tensor);
+        } else {
+            r = causal ? hip::selfAttentionBf16Backward(in.tensor, a, b, c, d, heads, grad.tensor)
+                       : hip::bidirectionalSelfAttentionBf16Backward(in.tensor, a, b, c, d, heads, grad.tensor);
+        }
+        copyOut(dInput, r.dInput);
+        copyOut(dWq, r.dWq);
+        copyOut(dWk, r.dWk);
+        copyOut(dWv, r.dWv);
+        copyOut(dWout, r.dWout);
+    });
+}
+
+// act: 0 SiLU (the reference block), 1 GELU, 2 ReLU.  x: [shape..., d].
+int bfh_feed_forward(const float* x, int rank, const size_t* shape, const float* w1, const float* b1, const float* w2, const float* b2,
+                     size_t hidden, int variant, int act, float* out) {
+    return guarded([&] {
+        std::vector<std::size_t> dims(shape, shape + rank);
+        if (dims.empty()) throw std::invalid_argument("bfh_feed_forward: rank 0");
+        Borrowed in(x, dims);
+        FeedForwardWeights w(w1, b1, w2, b2, dims.back(), hidden);
+        const auto activation = static_cast<hip::Activation>(act);
+        hip::DeviceTensor y;
+        hip::FeedForwardCache cache;
+        if (variant >= 2) hip::invalidateBf16WeightCache();
+        if (variant == 0) y = hip::feedForward(in.tensor, w.w1.tensor, w.b1.tensor, w.w2.tensor, w.b2.tensor, activation);
+        else if (variant == 1) y = hip::feedForwardBf16(in.tensor, w.w1.tensor, w.b1.tensor, w.w2.tensor, w.b2.tensor, activation);
+        else y = hip::feedForwardForwardCached(in.tensor, w.w1.tensor, w.b1.tensor, w.w2.tensor, w.b2.tensor, variant == 3, cache, activation);
+        copyOut(out, y);
+    });
+}
+
+int bfh_feed_forward_backward(const float* x, int rank, const size_t* shape, const float* w1, const float* b1, const float* w2,
+                              const float* b2, const float* g, size_t hidden, int variant, int act, float* dInput, float* dW1, float* dB1,
+                              float* dW2, float* dB2) {
+    return guarded([&] {
+        std::vector<std::size_t> dims(shape, shape + rank);
+        if (dims.empty()) throw std::invalid_argument("bfh_feed_forward_backward: rank 0");
+        Borrowed in(x, dims), grad(g, dims);
+        FeedForwardWeights w(w1, b1, w2, b2, dims.back(), hidden);
+        const auto activation = static_cast<hip::Activation>(act);
+        hip::FeedForwardGrad r;
+        if (variant >= 2) {
+            hip::invalidateBf16WeightCache();
+            hip::FeedForwardCache cache;
+            hip::feedForwardForwardCached(in.tensor, w.w1.tensor, w.b1.tensor, w.w2.tensor, w.b2.tensor, variant == 3, cache, activation);
+            r = hip::feedForwardBackwardCached(in.tensor, w.w1.tensor, w.b1.tensor, w.w2.tensor, w.b2.tensor, cache, grad.tensor,
+                                               variant == 3, activation);
+        } else if (variant == 0) {
+            r = hip::feedForwardBackward(in.tensor, w.w1.tensor, w.b1.tensor, w.w2.tensor, w.b2.tensor, grad.tensor, activation);
+        } else {
+            r = hip::feedForwardBf16Backward(in.tensor, w.w1.tensor, w.b1.tensor, w.w2.tensor, w.b2.tensor, grad.tensor, activation);
+        }
+        copyOut(dInput, r.dInput);
+        copyOut(dW1, r.dW1);
+        copyOut(dB1, r.dB1);
+        copyOut(dW2, r.dW2);
+        copyOut(dB2, r.dB2);
+    });
+}
+
+// hip::KVCache behind a handle, for selfAttentionIncremental[Bf16].
+void* bfh_kv_cache_create(void) { return new hip::KVCache(); }
+void bfh_kv_cache_destroy(void* cache) { delete static_cast<hip::KVCache*>(cache); }
+int bfh_kv_cache_info(void* cache, size_t* length, float** k, float** v) {
+    auto* c = static_cast<hip::KVCache*>(cache);
+    if (length) *length = c->length;
+    if (k) *k = c->k.data();
+    if (v) *v = c->v.data();
+    return 0;
+}
+int bfh_self_attention_incremental(void* cache, const float* xNew, const float* wq, const float* wk, const float* wv, const float* wout,
+                                   size_t batch, size_t newLen, size_t dim, size_t heads, int useBf16, float* out) {
+    return guarded([&] {
+        Borrowed in(xNew, {batch, newLen, dim});
+        AttentionWeights w(wq, wk, wv, wout, dim);
+        auto& kv = *static_cast<hip::KVCache*>(cache);
+        hip::DeviceTensor y = useBf16 ? hip::selfAttentionIncrementalBf16(in.tensor, w.wq.tensor, w.wk.tensor, w.wv.tensor, w.wout.tensor, heads, kv)
+                                      : hip::selfAttentionIncremental(in.tensor, w.wq.tensor, w.wk.tensor, w.wv.tensor, w.wout.tensor, heads, kv);
+        copyOut(out, y);
+    });
+}
+
+// Model::forwardIncremental on [batch, newLen] token ids (features for a model without embedding: [batch, newLen, d]);
+// the output stays owned by the handle until the next forward call.
+int bfh_model_forward_incremental(void* h, const float* input, int rank, const size_t* shape, float** output, size_t* outCount) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
+        handle->output = handle->model->forwardIncremental(in.tensor);
+        if (output) *output = handle->output.data();
+        if (outCount) *outCount = handle->output.elementCount();
+    });
+}
+int bfh_model_reset_generation(void* h) {
+    return guarded([&] { static_cast<Handle*>(h)->model->resetGenerationState(); });
+}
+// argmaxLastPosition over the handle's last output viewed as [rows, vocab].
+int bfh_model_argmax_last(void* h, size_t vocab, long long* index) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        std::size_t rows = vocab ? handle->output.elementCount() / vocab : 0;
+        Borrowed view(handle->output.data(), {rows, vocab});
+        *index = static_cast<long long>(hip::argmaxLastPosition(view.tensor));
+    });
+}
+
 // The permutation HostDataset::shuffle(seed) applies to `numExamples` examples: order[i] = example at position i afterwards.
 int bfh_shuffle_order(size_t numExamples, unsigned seed, size_t* order) {
     return guarded([&] {

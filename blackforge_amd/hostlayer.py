@@ -53,6 +53,18 @@ def load() -> ctypes.CDLL:
         lib.bfh_model_save_checkpoint.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
         lib.bfh_model_load_checkpoint.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
         lib.bfh_shuffle_order.argtypes = [ctypes.c_size_t, ctypes.c_uint, ctypes.POINTER(ctypes.c_size_t)]
+        P, Z, I = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+        lib.bfh_self_attention.argtypes = [P] * 5 + [Z] * 4 + [I, I, P]
+        lib.bfh_self_attention_backward.argtypes = [P] * 6 + [Z] * 4 + [I, I] + [P] * 5
+        lib.bfh_feed_forward.argtypes = [P, I, ctypes.POINTER(Z)] + [P] * 4 + [Z, I, I, P]
+        lib.bfh_feed_forward_backward.argtypes = [P, I, ctypes.POINTER(Z)] + [P] * 5 + [Z, I, I] + [P] * 5
+        lib.bfh_kv_cache_create.restype = P
+        lib.bfh_kv_cache_destroy.argtypes = [P]
+        lib.bfh_kv_cache_info.argtypes = [P, ctypes.POINTER(Z), ctypes.POINTER(P), ctypes.POINTER(P)]
+        lib.bfh_self_attention_incremental.argtypes = [P] * 6 + [Z] * 4 + [I, P]
+        lib.bfh_model_forward_incremental.argtypes = [P, P, I, ctypes.POINTER(Z), ctypes.POINTER(P), ctypes.POINTER(Z)]
+        lib.bfh_model_reset_generation.argtypes = [P]
+        lib.bfh_model_argmax_last.argtypes = [P, Z, ctypes.POINTER(ctypes.c_longlong)]
         _lib = lib
     return _lib
 
@@ -162,6 +174,22 @@ class HostModel:
         self._refresh_params()
         return list(losses[:epochs])
 
+    def forwardIncremental(self, x: DeviceTensor) -> np.ndarray:
+        """hip::Model::forwardIncremental on the new positions only (K/V of earlier ones come from the model's caches)."""
+        shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
+        out, count = ctypes.c_void_p(), ctypes.c_size_t()
+        _check(load().bfh_model_forward_incremental(self.handle, x.ptr, len(x.shape), shape, ctypes.byref(out), ctypes.byref(count)))
+        return self._read(out, count.value)
+
+    def resetGenerationState(self) -> None:
+        _check(load().bfh_model_reset_generation(self.handle))
+
+    def argmaxLast(self, vocab: int) -> int:
+        """hip::argmaxLastPosition over the last output of forward / forwardIncremental."""
+        index = ctypes.c_longlong()
+        _check(load().bfh_model_argmax_last(self.handle, vocab, ctypes.byref(index)))
+        return index.value
+
     def readLossSum(self) -> float:
         v = ctypes.c_float()
         _check(load().bfh_model_read_loss(self.handle, ctypes.byref(v)))
@@ -173,3 +201,86 @@ def shuffleOrder(num_examples: int, seed: int) -> np.ndarray:
     order = (ctypes.c_size_t * max(num_examples, 1))()
     _check(load().bfh_shuffle_order(num_examples, seed, order))
     return np.array(order[:num_examples], dtype=np.int64)
+
+
+# ---- composite blocks of the C++ operator layer (hip::selfAttention*, hip::feedForward*) --------------------
+# variant: 0 stateless fp32, 1 stateless bf16, 2 the ForwardCached/BackwardCached pair in fp32, 3 that pair in bf16.
+def _require_rank3(name: str, x: DeviceTensor):
+    if x.rank() != 3:
+        raise ValueError(f"{name}: needs an input of rank 3 [batch, seq, dim]")
+
+
+def selfAttention(x, wq, wk, wv, wout, heads: int, variant: int = 0, causal: bool = True) -> DeviceTensor:
+    _require_rank3("selfAttention", x)
+    batch, seq, dim = x.shape
+    out = DeviceTensor(x.shape)
+    _check(load().bfh_self_attention(x.ptr, wq.ptr, wk.ptr, wv.ptr, wout.ptr, batch, seq, dim, heads, variant, int(causal), out.ptr))
+    return out
+
+
+def selfAttentionBackward(x, wq, wk, wv, wout, heads: int, g, variant: int = 0, causal: bool = True):
+    """Returns (dInput, dWq, dWk, dWv, dWout)."""
+    _require_rank3("selfAttentionBackward", x)
+    batch, seq, dim = x.shape
+    outs = [DeviceTensor(x.shape)] + [DeviceTensor((dim, dim)) for _ in range(4)]
+    _check(load().bfh_self_attention_backward(x.ptr, wq.ptr, wk.ptr, wv.ptr, wout.ptr, g.ptr, batch, seq, dim, heads, variant,
+                                              int(causal), *[t.ptr for t in outs]))
+    return tuple(outs)
+
+
+def feedForward(x, w1, b1, w2, b2, act: int = 0, variant: int = 0) -> DeviceTensor:
+    shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
+    out = DeviceTensor(x.shape)
+    _check(load().bfh_feed_forward(x.ptr, len(x.shape), shape, w1.ptr, b1.ptr, w2.ptr, b2.ptr, w1.shape[1], variant, act, out.ptr))
+    return out
+
+
+def feedForwardBackward(x, w1, b1, w2, b2, g, act: int = 0, variant: int = 0):
+    """Returns (dInput, dW1, dB1, dW2, dB2)."""
+    shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
+    outs = [DeviceTensor(x.shape), DeviceTensor(w1.shape), DeviceTensor(b1.shape), DeviceTensor(w2.shape), DeviceTensor(b2.shape)]
+    _check(load().bfh_feed_forward_backward(x.ptr, len(x.shape), shape, w1.ptr, b1.ptr, w2.ptr, b2.ptr, g.ptr, w1.shape[1], variant,
+                                            act, *[t.ptr for t in outs]))
+    return tuple(outs)
+
+
+class KVCache:
+    """hip::KVCache behind a handle."""
+
+    def __init__(self):
+        self.handle = ctypes.c_void_p(load().bfh_kv_cache_create())
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            load().bfh_kv_cache_destroy(self.handle)
+            self.handle = None
+
+    def _info(self):
+        length, k, v = ctypes.c_size_t(), ctypes.c_void_p(), ctypes.c_void_p()
+        load().bfh_kv_cache_info(self.handle, ctypes.byref(length), ctypes.byref(k), ctypes.byref(v))
+        return length.value, k, v
+
+    @property
+    def length(self) -> int:
+        return self._info()[0]
+
+    def keys(self, batch: int, dim: int) -> np.ndarray:
+        length, k, _ = self._info()
+        out = np.empty((batch, length, dim), np.float32)
+        capi.call("bf_hip_memcpy_d2h", out.ctypes.data_as(ctypes.c_void_p), k, out.nbytes)
+        return out
+
+    def values(self, batch: int, dim: int) -> np.ndarray:
+        length, _, v = self._info()
+        out = np.empty((batch, length, dim), np.float32)
+        capi.call("bf_hip_memcpy_d2h", out.ctypes.data_as(ctypes.c_void_p), v, out.nbytes)
+        return out
+
+
+def selfAttentionIncremental(xNew, wq, wk, wv, wout, heads: int, cache: KVCache, useBf16: bool = False) -> DeviceTensor:
+    _require_rank3("selfAttentionIncremental", xNew)
+    batch, newLen, dim = xNew.shape
+    out = DeviceTensor(xNew.shape)
+    _check(load().bfh_self_attention_incremental(cache.handle, xNew.ptr, wq.ptr, wk.ptr, wv.ptr, wout.ptr, batch, newLen, dim, heads,
+                                                 int(useBf16), out.ptr))
+    return out

@@ -430,49 +430,12 @@ def fusedAttentionBackward(dOutput, q, k, v, output, m, l, numHeads: int, scaleF
 
 
 # ------------------------------------------------------------------------------------------------
-# composite blocks (ops.hpp:127-245, autodiff.hpp:117-177).  `act` selects the feed-forward
-# activation: ACT_SILU is the reference block, ACT_GELU the same block with gelu substituted.
+# composite blocks (ops.hpp:127-245, autodiff.hpp:117-177).  These are pass-throughs to the C++ operator
+# layer (include/blackforge/backend/hip/{ops,autodiff}.hpp) through blackforge_amd/hostlayer.py: the
+# orchestration (normalisation, projections, fused attention, residuals) exists once, in C++.
+# `act` selects the feed-forward activation: ACT_SILU is the reference block, ACT_GELU the same block
+# with gelu substituted.  `cached=True` runs the *ForwardCached / *BackwardCached pair that Model uses.
 # ------------------------------------------------------------------------------------------------
-@dataclass
-class FeedForwardCache:
-    normed: Optional[DeviceTensor] = None
-    gemm1: Optional[DeviceTensor] = None    # normed @ w1; on the fused bf16 route normed @ w1 + b1
-    hidden: Optional[DeviceTensor] = None   # act(gemm1 + b1); absent on the fused bf16 route
-    hiddenImage: Optional[DeviceTensor] = None   # fused bf16 route: bf16(act(gemm1)) as raw storage [rows, hidden/2]
-    normedImage: Optional[DeviceTensor] = None   # fused bf16 route: bf16(normed) as raw storage [rows, d/2]
-
-
-@dataclass
-class SelfAttentionCache:
-    normedFlat: Optional[DeviceTensor] = None
-    q: Optional[DeviceTensor] = None
-    k: Optional[DeviceTensor] = None
-    v: Optional[DeviceTensor] = None
-    attnOutput: Optional[DeviceTensor] = None
-    attnM: Optional[DeviceTensor] = None
-    attnL: Optional[DeviceTensor] = None
-    causal: bool = True   # False: bidirectionalSelfAttention
-
-
-@dataclass
-class KVCache:
-    k: Optional[DeviceTensor] = None
-    v: Optional[DeviceTensor] = None
-    length: int = 0
-
-
-def _mm(useBf16, cached):
-    if not useBf16:
-        return matmul
-    return matmulBf16CachedWeight if cached else matmulBf16
-
-
-def _mm_bwd(useBf16, cached):
-    if not useBf16:
-        return matmulBackward
-    return matmulBf16BackwardCachedWeight if cached else matmulBf16Backward
-
-
 def _opt(t):
     return t.ptr if t is not None else None
 
@@ -499,29 +462,13 @@ def feedForwardBf16FusedBackward(x, xImage, w1, w2, z, hImage, g, act: int = ACT
     return dX, dW1, dB1, dW2, dB2
 
 
-def _fused_feed_forward(useBf16, x, w1):
-    return useBf16 and x.shape[-1] % 8 == 0 and w1.shape[1] % 8 == 0 and x.elementCount() > 0
+def _variant(useBf16: bool, cached: bool) -> int:
+    return (2 if cached else 0) + (1 if useBf16 else 0)
 
 
-def feedForwardForwardCached(x, w1, b1, w2, b2, useBf16: bool, cache: FeedForwardCache, act: int = ACT_SILU):
-    cache.normed = rmsnorm(x)
-    if _fused_feed_forward(useBf16, x, w1):
-        out, z, cache.hiddenImage, cache.normedImage = feedForwardBf16Fused(_flat2d(cache.normed), w1, b1, w2, b2, _flat2d(x), act, True)
-        cache.gemm1, cache.hidden = z.reshaped(x.shape[:-1] + (w1.shape[1],)), None
-        return out.reshaped(x.shape)
-    mm = _mm(useBf16, True)
-    hiddenShape = x.shape[:-1] + (w1.shape[1],)
-    cache.gemm1 = mm(_flat2d(cache.normed), w1).reshaped(hiddenShape)
-    cache.hidden = addBiasAct(cache.gemm1, b1, act)
-    gemm2 = mm(_flat2d(cache.hidden), w2).reshaped(x.shape[:-1] + (w2.shape[1],))
-    return addBiasResidual(gemm2, b2, x)
-
-
-def feedForward(x, w1, b1, w2, b2, act: int = ACT_SILU, useBf16: bool = False):
-    normed = rmsnorm(x)
-    lin = linearBf16 if useBf16 else linear
-    hidden = _act(lin(normed, w1, b1), act)
-    return add(x, lin(hidden, w2, b2))
+def feedForward(x, w1, b1, w2, b2, act: int = ACT_SILU, useBf16: bool = False, cached: bool = False):
+    from . import hostlayer
+    return hostlayer.feedForward(x, w1, b1, w2, b2, act, _variant(useBf16, cached))
 
 
 def feedForwardBf16(x, w1, b1, w2, b2, act: int = ACT_SILU):
@@ -537,84 +484,28 @@ class FeedForwardGrad:
     dB2: DeviceTensor
 
 
-def feedForwardBackwardCached(x, w1, b1, w2, b2, cache: FeedForwardCache, g, useBf16: bool, act: int = ACT_SILU) -> FeedForwardGrad:
-    if cache.hiddenImage is not None:
-        dNormedFlat, dW1, dB1, dW2, dB2 = feedForwardBf16FusedBackward(None, cache.normedImage, w1, w2, _flat2d(cache.gemm1),
-                                                                        cache.hiddenImage, _flat2d(g), act, True)
-        dInput = rmsnormBackwardAdd(x, dNormedFlat.reshaped(cache.normed.shape), g)
-        return FeedForwardGrad(dInput, dW1, dB1, dW2, dB2)
-    bwd = _mm_bwd(useBf16, True)
-    dB2 = biasGradientOnly(g)
-    dHiddenFlat, dW2 = bwd(_flat2d(cache.hidden), w2, _flat2d(g))
-    dHidden = dHiddenFlat.reshaped(cache.hidden.shape)
-    dGemm1, dB1 = addBiasActBackward(cache.gemm1, b1, dHidden, act)
-    dNormedFlat, dW1 = bwd(_flat2d(cache.normed), w1, _flat2d(dGemm1))
-    dNormed = dNormedFlat.reshaped(cache.normed.shape)
-    dInput = add(g, rmsnormBackward(x, dNormed))
-    return FeedForwardGrad(dInput, dW1, dB1, dW2, dB2)
-
-
-def feedForwardBackward(x, w1, b1, w2, b2, g, act: int = ACT_SILU, useBf16: bool = False) -> FeedForwardGrad:
-    """Stateless variant: recomputes the forward, like autodiff.cu:624-652."""
-    cache = FeedForwardCache()
-    cache.normed = rmsnorm(x)
-    mm = _mm(useBf16, False)
-    cache.gemm1 = mm(_flat2d(cache.normed), w1).reshaped(x.shape[:-1] + (w1.shape[1],))
-    cache.hidden = addBiasAct(cache.gemm1, b1, act)
-    bwd = _mm_bwd(useBf16, False)
-    dB2 = biasGradientOnly(g)
-    dHiddenFlat, dW2 = bwd(_flat2d(cache.hidden), w2, _flat2d(g))
-    dGemm1, dB1 = addBiasActBackward(cache.gemm1, b1, dHiddenFlat.reshaped(cache.hidden.shape), act)
-    dNormedFlat, dW1 = bwd(_flat2d(cache.normed), w1, _flat2d(dGemm1))
-    dInput = add(g, rmsnormBackward(x, dNormedFlat.reshaped(x.shape)))
-    return FeedForwardGrad(dInput, dW1, dB1, dW2, dB2)
+def feedForwardBackward(x, w1, b1, w2, b2, g, act: int = ACT_SILU, useBf16: bool = False, cached: bool = False) -> FeedForwardGrad:
+    from . import hostlayer
+    return FeedForwardGrad(*hostlayer.feedForwardBackward(x, w1, b1, w2, b2, g, act, _variant(useBf16, cached)))
 
 
 def feedForwardBf16Backward(x, w1, b1, w2, b2, g, act: int = ACT_SILU):
     return feedForwardBackward(x, w1, b1, w2, b2, g, act, True)
 
 
-def _check_attention(name, x, numHeads):
-    _require(x.rank() == 3, f"{name}: needs an input of rank 3 [batch, seq, dim]")
-    _require(numHeads != 0 and x.shape[2] % numHeads == 0, f"{name}: numHeads must divide dim exactly")
-
-
-def selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads: int, useBf16: bool, cache: SelfAttentionCache,
-                               cachedWeights: bool = True, causal: bool = True):
-    _check_attention("selfAttention" if causal else "bidirectionalSelfAttention", x, numHeads)
-    batch, seq, dim = x.shape
-    cache.causal = causal
-    scaleFactor = 1.0 / math.sqrt(dim // numHeads)
-    mm = _mm(useBf16, cachedWeights)
-    cache.normedFlat = rmsnorm(x).reshaped((batch * seq, dim))
-    cache.q = mm(cache.normedFlat, wq).reshaped((batch, seq, dim))
-    cache.k = mm(cache.normedFlat, wk).reshaped((batch, seq, dim))
-    cache.v = mm(cache.normedFlat, wv).reshaped((batch, seq, dim))
-    # query i sees keys j <= oldLen + i: an offset of seq makes every key visible (the bidirectional form)
-    attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, 0 if causal else seq)
-    cache.attnOutput, cache.attnM, cache.attnL = attn.output, attn.m, attn.l
-    projected = mm(_flat2d(cache.attnOutput), wout).reshaped((batch, seq, dim))
-    return add(x, projected)
-
-
-def bidirectionalSelfAttention(x, wq, wk, wv, wout, numHeads: int, useBf16: bool = False):
-    """The block without the causal mask (CPU backend, ops.cpp:504-507; absent from the CUDA backend, model.cu:151-160)."""
-    return selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, useBf16, SelfAttentionCache(), False, causal=False)
-
-
-def bidirectionalSelfAttentionBackward(x, wq, wk, wv, wout, numHeads: int, g, useBf16: bool = False) -> "SelfAttentionGrad":
-    """cpu autodiff.cpp:492-496: recomputes the (non-causal) forward, then the shared backward."""
-    cache = SelfAttentionCache()
-    selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, useBf16, cache, False, causal=False)
-    return selfAttentionBackwardCached(x, wq, wk, wv, wout, numHeads, cache, g, useBf16, False)
-
-
-def selfAttention(x, wq, wk, wv, wout, numHeads: int):
-    return selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, False, SelfAttentionCache(), False)
+def selfAttention(x, wq, wk, wv, wout, numHeads: int, useBf16: bool = False, cached: bool = False):
+    from . import hostlayer
+    return hostlayer.selfAttention(x, wq, wk, wv, wout, numHeads, _variant(useBf16, cached), True)
 
 
 def selfAttentionBf16(x, wq, wk, wv, wout, numHeads: int):
-    return selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, True, SelfAttentionCache(), False)
+    return selfAttention(x, wq, wk, wv, wout, numHeads, True)
+
+
+def bidirectionalSelfAttention(x, wq, wk, wv, wout, numHeads: int, useBf16: bool = False, cached: bool = False):
+    """The block without the causal mask (CPU backend, ops.cpp:504-507; absent from the CUDA backend, model.cu:151-160)."""
+    from . import hostlayer
+    return hostlayer.selfAttention(x, wq, wk, wv, wout, numHeads, _variant(useBf16, cached), False)
 
 
 @dataclass
@@ -626,55 +517,33 @@ class SelfAttentionGrad:
     dWout: DeviceTensor
 
 
-def selfAttentionBackwardCached(x, wq, wk, wv, wout, numHeads: int, cache: SelfAttentionCache, g, useBf16: bool,
-                                cachedWeights: bool = True) -> SelfAttentionGrad:
-    batch, seq, dim = x.shape
-    scaleFactor = 1.0 / math.sqrt(dim // numHeads)
-    bwd = _mm_bwd(useBf16, cachedWeights)
-    dOutFlat, dWout = bwd(_flat2d(cache.attnOutput), wout, _flat2d(g))
-    dOutput = dOutFlat.reshaped((batch, seq, dim))
-    ag = fusedAttentionBackward(dOutput, cache.q, cache.k, cache.v, cache.attnOutput, cache.attnM, cache.attnL, numHeads,
-                                scaleFactor, 0 if cache.causal else seq)
-    dNq, dWq = bwd(cache.normedFlat, wq, _flat2d(ag.dQ))
-    dNk, dWk = bwd(cache.normedFlat, wk, _flat2d(ag.dK))
-    dNv, dWv = bwd(cache.normedFlat, wv, _flat2d(ag.dV))
-    dNormed = add(add(dNq, dNk), dNv).reshaped((batch, seq, dim))
-    dInput = add(g, rmsnormBackward(x, dNormed))
-    return SelfAttentionGrad(dInput, dWq, dWk, dWv, dWout)
-
-
-def selfAttentionBackward(x, wq, wk, wv, wout, numHeads: int, g, useBf16: bool = False) -> SelfAttentionGrad:
-    """Stateless variant: recomputes the forward, like autodiff.cu:654-700."""
-    cache = SelfAttentionCache()
-    selfAttentionForwardCached(x, wq, wk, wv, wout, numHeads, useBf16, cache, False)
-    return selfAttentionBackwardCached(x, wq, wk, wv, wout, numHeads, cache, g, useBf16, False)
+def selfAttentionBackward(x, wq, wk, wv, wout, numHeads: int, g, useBf16: bool = False, cached: bool = False) -> SelfAttentionGrad:
+    from . import hostlayer
+    return SelfAttentionGrad(*hostlayer.selfAttentionBackward(x, wq, wk, wv, wout, numHeads, g, _variant(useBf16, cached), True))
 
 
 def selfAttentionBf16Backward(x, wq, wk, wv, wout, numHeads: int, g):
     return selfAttentionBackward(x, wq, wk, wv, wout, numHeads, g, True)
 
 
-def selfAttentionIncremental(xNew, wq, wk, wv, wout, numHeads: int, cache: KVCache, useBf16: bool = False):
-    _check_attention("selfAttentionIncremental", xNew, numHeads)
-    batch, newLen, dim = xNew.shape
-    mm = _mm(useBf16, False)
-    normedFlat = rmsnorm(xNew).reshaped((batch * newLen, dim))
-    qNew = mm(normedFlat, wq).reshaped((batch, newLen, dim))
-    kNew = mm(normedFlat, wk).reshaped((batch, newLen, dim))
-    vNew = mm(normedFlat, wv).reshaped((batch, newLen, dim))
-    oldLen = cache.length
-    if oldLen == 0:
-        cache.k, cache.v = kNew, vNew
-    else:
-        cache.k, cache.v = concatSeq(cache.k, kNew), concatSeq(cache.v, vNew)
-    cache.length = oldLen + newLen
-    scaleFactor = 1.0 / math.sqrt(dim // numHeads)
-    attn = fusedAttentionForward(qNew, cache.k, cache.v, numHeads, scaleFactor, oldLen)
-    projected = mm(_flat2d(attn.output), wout).reshaped((batch, newLen, dim))
-    return add(xNew, projected)
+def bidirectionalSelfAttentionBackward(x, wq, wk, wv, wout, numHeads: int, g, useBf16: bool = False, cached: bool = False) -> SelfAttentionGrad:
+    """cpu autodiff.cpp:492-496."""
+    from . import hostlayer
+    return SelfAttentionGrad(*hostlayer.selfAttentionBackward(x, wq, wk, wv, wout, numHeads, g, _variant(useBf16, cached), False))
 
 
-def selfAttentionIncrementalBf16(xNew, wq, wk, wv, wout, numHeads: int, cache: KVCache):
+def KVCache():
+    """hip::KVCache (ops.hpp of the C++ layer): K/V of the positions processed so far."""
+    from . import hostlayer
+    return hostlayer.KVCache()
+
+
+def selfAttentionIncremental(xNew, wq, wk, wv, wout, numHeads: int, cache, useBf16: bool = False):
+    from . import hostlayer
+    return hostlayer.selfAttentionIncremental(xNew, wq, wk, wv, wout, numHeads, cache, useBf16)
+
+
+def selfAttentionIncrementalBf16(xNew, wq, wk, wv, wout, numHeads: int, cache):
     return selfAttentionIncremental(xNew, wq, wk, wv, wout, numHeads, cache, True)
 
 

@@ -285,6 +285,47 @@ int main() {
         EXPECT_THROW_INVALID((void)model.forwardIncremental(dev({1, 1}, {3})));   // src/backend/cpu/model.cpp:365-374
     });
 
+    // tests/backend/cuda/model_tests.cu:536-611: generating token by token gives the logits of the full forward pass
+    for (bool bf16 : {false, true}) {
+        run(bf16 ? "Model::forwardIncremental == forward, bf16 projections" : "Model::forwardIncremental == forward, fp32", [bf16] {
+            using hip::LayerKind;
+            const std::size_t vocab = 24, dim = 16, maxSeq = 8;
+            hip::Model model("decode", {{LayerKind::Embedding, vocab, dim}, {LayerKind::PositionalEmbedding, maxSeq, 0}, {LayerKind::Attention, 2, 0},
+                                        {LayerKind::FeedForward, 32, 0}, {LayerKind::Attention, 4, 0}, {LayerKind::Linear, vocab, 0}}, 0, bf16);
+            unsigned state = 4242;
+            for (hip::Parameter* p : model.parameters()) {
+                std::vector<float> init(p->value.elementCount());
+                for (float& v : init) { state = state * 1664525u + 1013904223u; v = (float(state >> 8) / float(1u << 24) - 0.5F) * 0.6F; }
+                p->value = DeviceTensor::fromHost(Tensor(p->value.shape(), init));
+            }
+            const std::vector<float> tokens = {3, 17, 5, 9, 21, 0};
+            const double tol = bf16 ? 2e-2 : 1e-4;
+            for (int round = 0; round < 2; ++round) {   // the second round checks resetGenerationState()
+                std::size_t done = 0;
+                for (std::size_t newLen : {std::size_t(3), std::size_t(1), std::size_t(1), std::size_t(1)}) {
+                    std::vector<float> piece(tokens.begin() + long(done), tokens.begin() + long(done + newLen));
+                    Tensor inc = model.forwardIncremental(dev({1, newLen}, piece)).toHost();
+                    done += newLen;
+                    Tensor full = model.forward(dev({1, done}, std::vector<float>(tokens.begin(), tokens.begin() + long(done)))).toHost();
+                    EXPECT_TRUE(inc.shape() == (std::vector<std::size_t>{1, newLen, vocab}));
+                    double scale = 0;
+                    for (float v : full.data()) scale = std::fmax(scale, std::fabs(v));
+                    for (std::size_t i = 0; i < newLen * vocab; ++i)
+                        EXPECT_NEAR(inc.data()[i], full.data()[(done - newLen) * vocab + i], tol * scale);
+                    std::size_t choice = hip::argmaxLastPosition(DeviceTensor::fromHost(inc));
+                    std::size_t best = 0;
+                    for (std::size_t c = 1; c < vocab; ++c)
+                        if (inc.data()[(newLen - 1) * vocab + c] > inc.data()[(newLen - 1) * vocab + best]) best = c;
+                    EXPECT_TRUE(choice == best);
+                }
+                model.resetGenerationState();
+            }
+            // positions continue without a reset: 6 + 3 > maxSeq rows of the positional table
+            (void)model.forwardIncremental(dev({1, 6}, tokens));
+            EXPECT_THROW_INVALID((void)model.forwardIncremental(dev({1, 3}, {1, 2, 3})));
+        });
+    }
+
     std::printf("%d checks, %d failures\n", g_checks, g_failures);
     return g_failures == 0 ? 0 : 1;
 }

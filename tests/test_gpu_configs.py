@@ -1,0 +1,234 @@
+"""GPU parity at the sizes the benchmark configurations name: the large-tile bf16 GEMMs with long contractions against
+float64 on sampled rows and columns, one (batch, head) slice of long-context attention against float64, multi-block bf16
+language models against the CPU oracle, and the GPT-small and long-context models at FULL size through properties that
+do not depend on size (bit-reproducibility, finiteness, causality-exact logits of a short prefix against the oracle)."""
+import numpy as np
+import pytest
+
+from parity import BF16_TOL, assert_bits_equal, assert_close
+from textbook import attention_slice
+
+pytestmark = pytest.mark.gpu
+f32, f64 = np.float32, np.float64
+
+
+def r(rng, *s, scale=1.0):
+    return (rng.standard_normal(s, dtype=f32) * f32(scale))
+
+
+def sample(rng, n, count=48):
+    """Indices that cover the edges and the middle of [0, n) plus seeded random picks (every tile row and wavefront row
+    of a 256-row tile is hit with high probability)."""
+    picks = np.r_[0:3, n // 2 - 1:n // 2 + 2, n - 3:n, rng.integers(0, n, count)]
+    return np.unique(picks[(picks >= 0) & (picks < n)])
+
+
+# ---- bf16 projections with long contractions, at the shapes of configs 2, 4 and 5 ------------------------------------
+@pytest.mark.parametrize("m,k,n", [(4096, 4096, 4096), (8192, 3072, 768), (8192, 768, 3072), (16384, 2048, 8192), (8192, 768, 2304)])
+def test_long_contraction_projection_against_float64(hip, oracle, m, k, n):
+    """matmulBf16 / linearBf16 with bias and residual, and both gradients, through the 256x256 ping-pong, 128-row and
+    sixteen-wavefront kernels with 12 to 128 K steps: float64 products of the bf16-rounded operands on sampled rows
+    (forward, dA) and sampled columns (dB, whose contraction runs over all m rows)."""
+    rng = np.random.default_rng(m + k + n)
+    D, ops = hip.DeviceTensor, hip.ops
+    a, w, g = r(rng, m, k), r(rng, k, n, scale=k ** -0.5), r(rng, m, n)
+    bias, res = r(rng, n), r(rng, m, n)
+    ar, wr, gr = (oracle.roundToBf16(t) for t in (a, w, g))
+    rows, cols = sample(rng, m), sample(rng, n, 24)
+    # the oracle's own fp32 loop on a few of the sampled rows ties the float64 product to the reference arithmetic
+    few = rows[:4]
+    assert_close(oracle.matmul(ar[few], wr), (ar[few].astype(f64) @ wr.astype(f64)).astype(f32), tol=1e-5, what="oracle vs float64")
+    da, dw, dg = D.fromHost(a), D.fromHost(w), D.fromHost(g)
+    ops.invalidateBf16WeightCache()
+    expected = ar[rows].astype(f64) @ wr.astype(f64)
+    c = ops.matmulBf16(da, dw).toHost()
+    assert_close(c[rows], expected.astype(f32), tol=1e-4, what="matmulBf16 sampled rows")
+    fused = ops.linearBf16Fused(da, dw, D.fromHost(bias), D.fromHost(res)).toHost()
+    assert_close(fused[rows], oracle.add(oracle.addBias(expected.astype(f32), bias), res[rows]), tol=1e-4, what="linear with bias and residual")
+    # the rest of the output must be the same kernel's work: whole-matrix agreement of the two entry points
+    assert_close(fused, c + bias[None, :] + res, tol=1e-5, what="fused store vs separate adds, whole matrix")
+    del c, fused
+    dA, dB = ops.matmulBf16Backward(da, dw, dg)
+    dA, dB = dA.toHost(), dB.toHost()
+    assert_close(dA[rows], (gr[rows].astype(f64) @ wr.astype(f64).T).astype(f32), tol=1e-4, what="dA sampled rows")
+    assert_close(dB[:, cols], (ar.astype(f64).T @ gr[:, cols].astype(f64)).astype(f32), tol=1e-4, what="dB sampled columns")
+    # sampled rows of dB as well (a different slice of the tile grid)
+    krows = sample(rng, k, 16)
+    assert_close(dB[krows], (ar[:, krows].astype(f64).T @ gr.astype(f64)).astype(f32), tol=1e-4, what="dB sampled rows")
+    assert np.isfinite(dA).all() and np.isfinite(dB).all()
+
+
+# ---- long-context attention (config 5 layer shape) -------------------------------------------------------------------
+@pytest.mark.parametrize("route", ["hand-over", "recompute"])
+def test_config5_attention_slice_against_float64(hip, route):
+    """batch 4, heads 16, seq 4096, head_dim 128 in fp32: (batch, head) slices against the float64 textbook form, and the
+    size-independent properties, on both backward routes."""
+    rng = np.random.default_rng(5)
+    batch, heads, seq, hd = 4, 16, 4096, 128
+    dim, scale = heads * hd, float(f32(1.0) / np.sqrt(f32(hd)))
+    q, k, v, go = (r(rng, batch, seq, dim) for _ in range(4))
+    D, ops = hip.DeviceTensor, hip.ops
+
+    def run(qh, kh, vh, gh):
+        dq_, dk_, dv_, dg_ = map(D.fromHost, (qh, kh, vh, gh))
+        fwd = ops.fusedAttentionForward(dq_, dk_, dv_, heads, scale, 0)
+        grad = ops.fusedAttentionBackward(dg_, dq_, dk_, dv_, fwd.output, fwd.m, fwd.l, heads, scale, 0)
+        return [t.toHost() for t in (fwd.output, fwd.m, fwd.l, grad.dQ, grad.dK, grad.dV)]
+
+    hip.capi.call("bf_hip_attention_set_workspace_limit", 0 if route == "recompute" else 2 ** 64 - 1)
+    try:
+        o, m, l, dq, dk, dv = run(q, k, v, go)
+        again = run(q, k, v, go)
+        doubled = run(q, k, v, 2 * go)
+    finally:
+        hip.capi.call("bf_hip_attention_set_workspace_limit", 2 ** 64 - 1)
+    rms = lambda t: float(np.sqrt(np.mean(np.asarray(t, f64) ** 2)))
+    ds = rms(go) * rms(v)
+    floors = {"O": rms(v), "dQ": ds * rms(k) * scale, "dK": ds * rms(q) * scale, "dV": rms(go)}
+    for b, h in ((0, 0), (3, 15), (1, 6)):
+        sl = lambda t: t[b, :, h * hd:(h + 1) * hd]
+        eo, em, el, edq, edk, edv = attention_slice(sl(q), sl(k), sl(v), sl(go), scale)
+        for got, exp, name in ((sl(o), eo, "O"), (sl(dq), edq, "dQ"), (sl(dk), edk, "dK"), (sl(dv), edv, "dV")):
+            assert_close(got, exp.astype(f32), what=f"{name} slice ({b},{h}) at the long-context shape, {route}", scale=floors[name])
+        assert_close(m[b, h], em.astype(f32), what="m slice")
+        assert_close(l[b, h], el.astype(f32), what="l slice")
+    for a, bb, name in zip((o, m, l, dq, dk, dv), again, "O m l dQ dK dV".split()):
+        assert_bits_equal(a, bb, name + " is not bit-reproducible")
+    for a, bb, name in zip((dq, dk, dv), doubled[3:], ("dQ", "dK", "dV")):
+        assert_bits_equal(bb, 2 * a, f"{name}(2 dO) != 2 {name}(dO)")
+    np.testing.assert_allclose(o[:, 0], v[:, 0], rtol=1e-6, atol=1e-6)     # the first query sees only the first key
+    lhs, rhs = (dq.astype(f64) * q).sum(), (dk.astype(f64) * k).sum()         # rows of dS sum to zero
+    assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), abs(rhs), 1.0)
+
+
+# ---- multi-block bf16 language models against the oracle -------------------------------------------------------------
+def lm_layers(mod, vocab, dim, seq, heads, hidden, act, blocks):
+    layers = [(mod.EMBEDDING, vocab, dim), (mod.POSITIONAL, seq)]
+    for _ in range(blocks):
+        layers += [(mod.ATTENTION, heads), (mod.FEEDFORWARD, hidden, act)]
+    return layers + [(mod.LINEAR, vocab)]
+
+
+def init(rng, names, counts, scale=0.02):
+    """Weights N(0, scale), biases zero (the benchmark's initialisation)."""
+    return [np.zeros(c, f32) if n.endswith((".bias", ".b1", ".b2")) else r(rng, c, scale=scale) for n, c in zip(names, counts)]
+
+
+@pytest.mark.parametrize("what,vocab,dim,seq,heads,hidden,act,blocks,batch,adamw", [
+    ("gpt-small pipeline: GELU, head_dim 64, AdamW", 512, 256, 64, 4, 1024, 1, 2, 4, True),
+    ("long-context pipeline: SiLU, head_dim 128, no optimizer", 384, 256, 96, 2, 512, 0, 2, 2, False)])
+def test_two_block_bf16_model_against_oracle(hip, oracle, what, vocab, dim, seq, heads, hidden, act, blocks, batch, adamw):
+    """The pipelines of configs 4 and 5 (several attention + feed-forward blocks, bf16 projections with the fused
+    feed-forward and shared-input Q/K/V routes, fp32 attention, sparse cross-entropy) at a size the oracle finishes in
+    seconds: loss, every gradient and (with AdamW) every updated parameter within the bf16 bound of the fp32 CPU model."""
+    from blackforge_amd import hostlayer as hl
+    from oracle import bfo
+    rng = np.random.default_rng(vocab + dim)
+    gpu = hl.HostModel(lm_layers(hl, vocab, dim, seq, heads, hidden, act, blocks), use_bf16=True)
+    cpu = oracle.model(lm_layers(bfo, vocab, dim, seq, heads, hidden, act, blocks))
+    assert gpu.names == cpu.names
+    for i, w in enumerate(init(rng, gpu.names, gpu.counts, scale=0.05)):
+        gpu.set_value(i, w)
+        cpu.value(i)[:] = w
+    D = hip.DeviceTensor
+    ids = rng.integers(0, vocab, (batch, seq)).astype(f32)
+    tgt = rng.integers(0, vocab, batch * seq).astype(f32)
+    cpu.zeroGrad()
+    logits = cpu.forward(ids)
+    loss, grad = oracle.softmaxCrossEntropySparse(logits.reshape(-1, vocab), tgt)
+    cpu.backward(grad)
+    x, t = D.fromHost(ids), D.fromHost(tgt)
+    assert_close(gpu.forward(x, trusted=True), logits.ravel(), tol=BF16_TOL, what=what + ": logits", scale=float(np.abs(logits).max()))
+    gpu.trainStep(x, t, optimizer=0)
+    assert abs(gpu.readLossSum() / (batch * seq) - loss) <= BF16_TOL * loss
+    for i in range(len(gpu.counts)):
+        e = cpu.grad(i)
+        assert_close(gpu.grad(i), e, tol=BF16_TOL, what=f"{what}: grad {gpu.names[i]}", scale=float(np.abs(e).max()))
+    if adamw:
+        before = [gpu.value(i) for i in range(len(gpu.counts))]
+        cpu.adamwStep()
+        gpu.adamwStep()
+        for i in range(len(gpu.counts)):
+            # the first AdamW step moves a parameter by at most lr (1 + wd |p|); where bf16 noise flips the sign of a
+            # gradient near zero the two updates differ by up to 2 lr, so the comparison is of the step, not the bits
+            step_gpu, step_cpu = gpu.value(i) - before[i], cpu.value(i) - before[i]
+            assert np.abs(step_gpu).max() <= 1e-3 * (1 + 0.01 * np.abs(before[i]).max()) * 1.001 + 1e-9
+            agree = np.mean(np.sign(step_gpu) == np.sign(step_cpu))
+            assert agree > 0.95, f"{what}: AdamW step direction of {gpu.names[i]} agrees on {agree:.3f} of elements"
+
+
+# ---- configs 4 and 5 at full size --------------------------------------------------------------------------------------
+FULL = {
+    "gpt_small": dict(vocab=32000, dim=768, heads=12, blocks=12, ffn=3072, act=1, seq=1024, batch=8, adamw=True),
+    "long_context": dict(vocab=50257, dim=2048, heads=16, blocks=8, ffn=8192, act=0, seq=4096, batch=4, adamw=False),
+}
+
+
+@pytest.mark.parametrize("name", ["gpt_small", "long_context"])
+def test_full_size_training_step(hip, oracle, name):
+    """BASELINE configs 4 and 5 exactly as the benchmark runs them (hip::Model, bf16 projections, fp32 attention, sparse CE,
+    AdamW for GPT-small).  The CPU reference would take hours, so: (1) the logits of the first two positions of two
+    sequences depend only on those two tokens (causal mask) and are checked against the oracle run on the two-token
+    prefixes with the same weights; (2) loss and every gradient are finite and bit-identical across two runs; (3) the loss
+    equals the float64 cross-entropy of the model's own logits; (4) the AdamW step is bounded by lr (1 + wd |p|) and finite."""
+    from blackforge_amd import hostlayer as hl
+    from oracle import bfo
+    c = FULL[name]
+    rng = np.random.default_rng(42)
+    layers = lambda mod: lm_layers(mod, c["vocab"], c["dim"], c["seq"], c["heads"], c["ffn"], c["act"], c["blocks"])
+    gpu, cpu = hl.HostModel(layers(hl), use_bf16=True), oracle.model(layers(bfo))
+    assert gpu.names == cpu.names
+    for i, (n, count) in enumerate(zip(gpu.names, gpu.counts)):
+        w = np.zeros(count, f32) if n.endswith((".bias", ".b1", ".b2")) else r(rng, count, scale=0.02)
+        gpu.set_value(i, w)
+        cpu.value(i)[:] = w
+    D = hip.DeviceTensor
+    batch, seq, vocab = c["batch"], c["seq"], c["vocab"]
+    ids = rng.integers(0, vocab, (batch, seq)).astype(f32)
+    tgt = rng.integers(0, vocab, batch * seq).astype(f32)
+    x, t = D.fromHost(ids), D.fromHost(tgt)
+    print(f"{name}: {sum(gpu.counts)} parameters", flush=True)
+    # (1) prefix logits
+    logits = gpu.forward(x, trusted=True).reshape(batch, seq, vocab)
+    assert np.isfinite(logits).all()
+    for b in (0, batch - 1):
+        expected = cpu.forward(ids[b:b + 1, :2]).reshape(2, vocab)
+        assert_close(logits[b, :2], expected, tol=BF16_TOL, what=f"{name}: logits of the first two positions of sequence {b}",
+                     scale=float(np.abs(expected).max()))
+    # the loss the step must report, from these logits in float64 (row chunks keep the float64 copies small)
+    rows = logits.reshape(batch * seq, vocab)
+    expected_loss = 0.0
+    for lo in range(0, batch * seq, 1024):
+        chunk = rows[lo:lo + 1024].astype(f64)
+        top = chunk.max(1)
+        lse = top + np.log(np.exp(chunk - top[:, None]).sum(1))
+        expected_loss += float((lse - chunk[np.arange(len(chunk)), tgt[lo:lo + 1024].astype(np.int64)]).sum())
+    expected_loss /= batch * seq
+    del logits, rows
+    # (2) reproducibility and finiteness of a whole step without the optimizer
+    gpu.trainStep(x, t, optimizer=0)
+    loss1 = gpu.readLossSum()
+    first = [gpu.grad(i) for i in range(len(gpu.counts))]
+    gpu.trainStep(x, t, optimizer=0)
+    loss2 = gpu.readLossSum()
+    assert np.float32(loss1).tobytes() == np.float32(loss2).tobytes(), "loss is not bit-reproducible"
+    for i, g1 in enumerate(first):
+        assert np.isfinite(g1).all(), f"{name}: non-finite gradient in {gpu.names[i]}"
+        assert_bits_equal(gpu.grad(i), g1, f"{name}: gradient of {gpu.names[i]} is not bit-reproducible")
+    assert any(np.abs(g).max() > 0 for g in first)
+    # (3) the reported loss is the cross-entropy of the logits checked above
+    mean_loss = loss1 / (batch * seq)
+    assert abs(mean_loss - expected_loss) <= 1e-4 * expected_loss, (mean_loss, expected_loss)
+    del first
+    # (4) one AdamW step (GPT-small runs one in the benchmark)
+    if c["adamw"]:
+        probe = [0, len(gpu.counts) // 2, len(gpu.counts) - 2]
+        before = {i: gpu.value(i) for i in probe}
+        gpu.trainStep(x, t, optimizer=1, lr=1e-3)
+        gpu.readLossSum()
+        for i in probe:
+            after = gpu.value(i)
+            assert np.isfinite(after).all()
+            step = np.abs(after - before[i])
+            assert step.max() <= 1e-3 * (1 + 0.01 * np.abs(before[i]).max()) * 1.001 + 1e-9, f"{name}: AdamW step of {gpu.names[i]} exceeds lr"
+            assert step.max() > 0

@@ -45,26 +45,41 @@ def test_attention_block_fixture_and_golden(hip, oracle):
         assert_close(got.toHost(), gold["fffix_" + name], what="feedForwardBackward fixture " + name, scale=1e-2)
 
 
-@pytest.mark.parametrize("batch,seq,dim,heads,hidden", [(2, 9, 12, 3, 20), (8, 64, 128, 4, 512), (1, 130, 64, 2, 96)])
+@pytest.mark.parametrize("batch,seq,dim,heads,hidden", [(2, 9, 12, 3, 20), (8, 64, 128, 4, 512), (1, 130, 64, 2, 96), (2, 40, 256, 2, 264)])
 @pytest.mark.parametrize("act", [0, 1])
-def test_blocks_against_oracle(hip, oracle, rng, batch, seq, dim, heads, hidden, act):
+@pytest.mark.parametrize("cached", [False, True])
+def test_blocks_against_oracle(hip, oracle, rng, batch, seq, dim, heads, hidden, act, cached):
+    """The composite blocks of the C++ operator layer (hip::selfAttention[Backward], hip::feedForward[Backward], and with
+    `cached` the *ForwardCached / *BackwardCached pair that hip::Model calls) against the CPU backend's blocks: fp32 at
+    the fp32 bound, the bf16 variants (stateless, and cached with the fused feed-forward and shared-input routes) at 2e-2."""
     D, ops = hip.DeviceTensor, hip.ops
     x, g = r(rng, batch, seq, dim), r(rng, batch, seq, dim)
     w = [r(rng, dim, dim, scale=dim ** -0.5) for _ in range(4)]
     dw = [D.fromHost(a) for a in w]
     dx, dg = D.fromHost(x), D.fromHost(g)
+    names = ("dInput", "dWq", "dWk", "dWv", "dWout")
     if act == 0:
-        assert_close(ops.selfAttention(dx, *dw, heads).toHost(), oracle.selfAttention(x, *w, heads), what="selfAttention")
-        grad = ops.selfAttentionBackward(dx, *dw, heads, dg)
-        exp = oracle.selfAttentionBackward(x, *w, heads, g)
-        for got, e, n in zip((grad.dInput, grad.dWq, grad.dWk, grad.dWv, grad.dWout), exp, ("dInput", "dWq", "dWk", "dWv", "dWout")):
+        eo, eg = oracle.selfAttention(x, *w, heads), oracle.selfAttentionBackward(x, *w, heads, g)
+        assert_close(ops.selfAttention(dx, *dw, heads, cached=cached).toHost(), eo, what="selfAttention")
+        grad = ops.selfAttentionBackward(dx, *dw, heads, dg, cached=cached)
+        for got, e, n in zip((grad.dInput, grad.dWq, grad.dWk, grad.dWv, grad.dWout), eg, names):
             assert_close(got.toHost(), e, what="selfAttentionBackward." + n, scale=float(np.abs(e).max()) * 0.1)
+        assert_close(ops.selfAttention(dx, *dw, heads, useBf16=True, cached=cached).toHost(), eo, tol=BF16_TOL, what="selfAttentionBf16")
+        grad = ops.selfAttentionBackward(dx, *dw, heads, dg, useBf16=True, cached=cached)
+        for got, e, n in zip((grad.dInput, grad.dWq, grad.dWk, grad.dWv, grad.dWout), eg, names):
+            assert_close(got.toHost(), e, tol=BF16_TOL, what="selfAttentionBf16Backward." + n, scale=float(np.abs(e).max()))
     p = [r(rng, dim, hidden, scale=dim ** -0.5), r(rng, hidden, scale=.1), r(rng, hidden, dim, scale=hidden ** -0.5), r(rng, dim, scale=.1)]
     dp = [D.fromHost(a) for a in p]
-    assert_close(ops.feedForward(dx, *dp, act).toHost(), oracle.feedForward(x, *p, act), what="feedForward")
-    fg = ops.feedForwardBackward(dx, *dp, dg, act)
-    for got, e, n in zip((fg.dInput, fg.dW1, fg.dB1, fg.dW2, fg.dB2), oracle.feedForwardBackward(x, *p, g, act), ("dInput", "dW1", "dB1", "dW2", "dB2")):
+    eo, eg = oracle.feedForward(x, *p, act), oracle.feedForwardBackward(x, *p, g, act)
+    names = ("dInput", "dW1", "dB1", "dW2", "dB2")
+    assert_close(ops.feedForward(dx, *dp, act, cached=cached).toHost(), eo, what="feedForward")
+    fg = ops.feedForwardBackward(dx, *dp, dg, act, cached=cached)
+    for got, e, n in zip((fg.dInput, fg.dW1, fg.dB1, fg.dW2, fg.dB2), eg, names):
         assert_close(got.toHost(), e, what="feedForwardBackward." + n, scale=float(np.abs(e).max()) * 0.1)
+    assert_close(ops.feedForward(dx, *dp, act, useBf16=True, cached=cached).toHost(), eo, tol=BF16_TOL, what="feedForwardBf16")
+    fg = ops.feedForwardBackward(dx, *dp, dg, act, useBf16=True, cached=cached)
+    for got, e, n in zip((fg.dInput, fg.dW1, fg.dB1, fg.dW2, fg.dB2), eg, names):
+        assert_close(got.toHost(), e, tol=BF16_TOL, what="feedForwardBf16Backward." + n, scale=float(np.abs(e).max()))
 
 
 @pytest.mark.parametrize("batch,seq,dim,heads", [(2, 9, 12, 3), (4, 64, 128, 4), (1, 130, 64, 2), (1, 200, 256, 2)])
@@ -139,19 +154,24 @@ def test_mlm_model_steps_against_oracle(hip, oracle, rng):
             assert_close(gpu.value(i), cpu.value(i), what=f"step {step} param {gpu.names[i]}", scale=0.02 * 1e-2 / 1e-4)
 
 
-def test_incremental_decode_block(hip, oracle, rng):
+@pytest.mark.parametrize("use_bf16", [False, True])
+def test_incremental_decode_block(hip, oracle, rng, use_bf16):
+    """hip::selfAttentionIncremental[Bf16] with a growing hip::KVCache against the CPU backend's incremental block
+    (ops.cpp:509-566): prefill, single tokens, a longer continuation."""
     D, ops = hip.DeviceTensor, hip.ops
     batch, dim, heads = 2, 32, 4
     w = [r(rng, dim, dim, scale=dim ** -0.5) for _ in range(4)]
     dw = [D.fromHost(a) for a in w]
     cache, kc, vc = ops.KVCache(), None, None
+    tol = BF16_TOL if use_bf16 else 1e-4
     for new_len in (5, 1, 1, 3):
         x = r(rng, batch, new_len, dim)
-        got = ops.selfAttentionIncremental(D.fromHost(x), *dw, heads, cache).toHost()
+        got = ops.selfAttentionIncremental(D.fromHost(x), *dw, heads, cache, useBf16=use_bf16).toHost()
         exp, kc, vc = oracle.selfAttentionIncremental(x, *w, heads, kc, vc)
-        assert_close(got, exp, what=f"incremental newLen={new_len}")
+        assert_close(got, exp, tol=tol, what=f"incremental newLen={new_len}")
     assert cache.length == 10
-    assert_close(cache.k.toHost(), kc, what="KV cache K")
+    assert_close(cache.keys(batch, dim), kc, tol=tol, what="KV cache K")
+    assert_close(cache.values(batch, dim), vc, tol=tol, what="KV cache V")
 
 
 def _lm_layers(hl, vocab, dim, seq, heads, hidden, act, blocks=1):
@@ -187,6 +207,54 @@ def test_tiny_lm_three_steps_match_the_reference_fixture(hip):
             # floor: 2 % of the AdamW step bound lr = 1e-2 (the update is lr * m / (sqrt(v) + eps), ill-conditioned
             # where the gradient is comparable to eps)
             assert_close(model.value(i), gold[f"lm_step{step}_param{i}"], what=f"step {step} param {model.names[i]}", scale=0.02 * 1e-2 / 1e-4)
+
+
+@pytest.mark.parametrize("use_bf16", [False, True])
+def test_model_forward_incremental_matches_full_forward(hip, oracle, rng, use_bf16):
+    """hip::Model::forwardIncremental (model.cu:385-424; the reference's own check is token-by-token == full forward,
+    tests/backend/cuda/model_tests.cu:536-611): prefill five tokens, then single tokens; each call's logits against
+    Model::forward over the whole prefix at the same positions and against the CPU model; greedy argmax of the last
+    position; resetGenerationState() starts over at position 0."""
+    from blackforge_amd import hostlayer as hl
+    from oracle import bfo
+    vocab, dim, seq, heads, hidden, blocks = 61, 64, 16, 4, 96, 2
+    gpu = hl.HostModel(_lm_layers(hl, vocab, dim, seq, heads, hidden, 0, blocks), use_bf16=use_bf16)
+    cpu = oracle.model(_lm_layers(bfo, vocab, dim, seq, heads, hidden, 0, blocks))
+    for i, c in enumerate(gpu.counts):
+        w = r(rng, c, scale=0.2)
+        gpu.set_value(i, w)
+        cpu.value(i)[:] = w
+    D = hip.DeviceTensor
+    ids = rng.integers(0, vocab, (1, 9)).astype(f32)
+    tol = BF16_TOL if use_bf16 else 1e-4
+
+    def decode():
+        done, outs = 0, []
+        for new_len in (5, 1, 1, 2):
+            logits = gpu.forwardIncremental(D.fromHost(ids[:, done:done + new_len])).reshape(new_len, vocab)
+            choice = gpu.argmaxLast(vocab)
+            done += new_len
+            full = gpu.forward(D.fromHost(ids[:, :done])).reshape(done, vocab)
+            # same kernels on the same rows: only the attention tiling (one call over the prefix against new rows over a
+            # cache) and, in bf16 mode, the cached weight images differ
+            assert_close(logits, full[done - new_len:], tol=1e-4 if not use_bf16 else 5e-3, what=f"incremental vs full forward at {done}")
+            expected = cpu.forward(ids[:, :done]).reshape(done, vocab)
+            assert_close(logits, expected[done - new_len:], tol=tol, what=f"incremental vs CPU model at {done}",
+                         scale=float(np.abs(expected).max()) if use_bf16 else 0.0)
+            assert choice == int(np.argmax(logits[-1])), "argmaxLastPosition over the incremental logits"
+            if not use_bf16:
+                assert choice == oracle.argmaxLastPosition(expected[None])
+            outs.append(logits)
+        return outs
+
+    first = decode()
+    gpu.resetGenerationState()
+    second = decode()
+    for a, b in zip(first, second):
+        assert_bits_equal(a, b, "decode after resetGenerationState")
+    # without a reset the positions continue: the positional table has 16 rows, so 9 + 9 > 16 must be refused
+    with pytest.raises(ValueError):
+        gpu.forwardIncremental(D.fromHost(ids))
 
 
 @pytest.mark.parametrize("act", [0, 1])

@@ -232,3 +232,17 @@ def test_bidirectional_attention_sees_later_positions(oracle):
     assert np.abs(ya[0, :2] - yb[0, :2]).max() > 1e-4
     ca, cb = (oracle.selfAttention(x, wq, wk, wv, wo, 2, causal=True) for x in (a, b))
     assert np.abs(ca[0, :2] - cb[0, :2]).max() == 0.0
+
+
+def test_textbook_attention_slice_helper_agrees_with_the_oracle(oracle, rng):
+    """tests/textbook.attention_slice is the float64 reference of the GPU tests at sizes the C oracle is too slow for;
+    here it is held against the oracle (itself pinned above and against the reference build) on a small slice."""
+    from textbook import attention_slice
+    for nl, ol, hd in ((37, 0, 16), (20, 9, 128)):
+        q, k, v, go = r(rng, 1, nl, hd), r(rng, 1, nl + ol, hd), r(rng, 1, nl + ol, hd), r(rng, 1, nl, hd)
+        scale = 1.0 / np.sqrt(hd)
+        o, m, l = oracle.attentionCoreForward(q, k, v, 1, scale, ol)
+        dq, dk, dv = oracle.attentionCoreBackward(go, q, k, v, 1, scale, ol)
+        got = attention_slice(q[0], k[0], v[0], go[0], scale, ol)
+        for a, e in zip(got, (o[0], m[0, 0], l[0, 0], dq[0], dk[0], dv[0])):
+            np.testing.assert_allclose(a, e, rtol=0, atol=1e-5 * np.abs(e).max() + 1e-6)
