@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X operator backend on the headline workload.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras] [--train LIST]
 
 Workload (BASELINE.json configs[2], the one the fused-attention TFLOP/s metric is quoted on):
 standalone causal fused attention in fp32, batch 8, heads 16, seq 2048, head_dim 64, Q/K/V/dOut
@@ -289,9 +289,38 @@ def bench_mlp(bf, steps, warmup):
     stop.synchronize()
     ms = start.elapsed_ms(stop) / steps
     flops = 6 * 2 * rows * width * width
+    # floor: six 4096^3 products at the bf16 MFMA peak, plus the fp32 passes the pipeline cannot avoid at the HBM peak
+    # (input, two outputs, SiLU and its backward, loss gradient, two bias gradients: ~14 passes over [rows, width])
+    floor_ms = flops / PEAK_BF16_MFMA_TFLOPS / 1e9 + 14 * rows * width * 4 / PEAK_HBM_GBS / 1e6
     return {"workload": MLP_CONFIG["what"], "tokens_per_s": round(rows / (ms * 1e-3), 1), "ms_per_step": round(ms, 3), "tokens": rows,
             "algorithmic_tflop_per_step": round(flops / 1e12, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
-            "mean_loss": round(model.readLossSum() / (steps * rows * width), 4)}
+            "mean_loss": round(model.readLossSum() / (steps * rows * width), 4),
+            "roofline": {"bound": "mfma", "achieved": round(flops / ms / 1e9, 2), "peak": round(flops / floor_ms / 1e9, 2), "unit": "TFLOP/s",
+                         "frac": round(floor_ms / ms, 4), "floor_ms": round(floor_ms, 3),
+                         "note": "peak = algorithmic FLOPs / (six products at the bf16 MFMA peak + 14 fp32 passes over [rows, width] at the HBM peak)"}}
+
+
+def cpu_baseline_mlp():
+    """The reference CPU backend on the MLP: cpu::Model linear -> silu -> linear with an MSE loss on a sample of rows
+    (its cost is linear in the row count)."""
+    from oracle import bfo
+    impl = bfo.reference() or bfo.oracle()
+    rows, width, sample = MLP_CONFIG["rows"], MLP_CONFIG["width"], 16
+    rng = np.random.default_rng(5)
+    model = impl.model([(bfo.LINEAR, width), (bfo.SILU,), (bfo.LINEAR, width)], input_features=width)
+    for i, count in enumerate(model.counts):
+        model.value(i)[:] = np.resize(rng.standard_normal(4099, dtype=np.float32) * np.float32(1 / 64), count)
+    x = rng.standard_normal((sample, width), dtype=np.float32)
+    y = rng.standard_normal((sample, width), dtype=np.float32)
+    t0 = time.perf_counter()
+    model.zeroGrad()
+    out = model.forward(x, out_capacity=x.size)
+    _, grad = impl.meanSquaredError(out.reshape(sample, width), y)
+    model.backward(grad)
+    elapsed = time.perf_counter() - t0
+    return {"value": round(sample / elapsed, 3), "unit": "tokens/s", "cores": 1, "kind": "reference" if impl.is_reference else "port",
+            "extrapolated": True,
+            "sample": f"{sample} of {rows} rows through cpu::Model (forward, MSE, backward) in {elapsed:.2f} s on one host core; rows are independent"}
 
 
 def train_step_flops(c):
@@ -300,6 +329,108 @@ def train_step_flops(c):
     weights = c["blocks"] * (4 * c["dim"] ** 2 + 2 * c["dim"] * c["ffn"]) + c["dim"] * c["vocab"]
     pairs = c["batch"] * c["heads"] * c["seq"] * (c["seq"] + 1) // 2
     return 6 * tokens * weights + c["blocks"] * 14 * (c["dim"] // c["heads"]) * pairs
+
+
+def train_step_roofline(c, ms):
+    """The step against its matrix-pipe floor: bf16 MFMA peak for the projections, fp32 MFMA peak for the attention core
+    (the elementwise and loss kernels are HBM-bound and add to the floor what their algorithmic bytes cost at HBM peak)."""
+    tokens = c["batch"] * c["seq"]
+    weights = c["blocks"] * (4 * c["dim"] ** 2 + 2 * c["dim"] * c["ffn"]) + c["dim"] * c["vocab"]
+    pairs = c["batch"] * c["heads"] * c["seq"] * (c["seq"] + 1) // 2
+    gemm_flops = 6 * tokens * weights
+    attn_flops = c["blocks"] * 14 * (c["dim"] // c["heads"]) * pairs
+    peak_gemm = PEAK_BF16_MFMA_TFLOPS if c["bf16"] else PEAK_FP32_MFMA_TFLOPS
+    floor_ms = gemm_flops / peak_gemm / 1e9 + attn_flops / PEAK_FP32_MFMA_TFLOPS / 1e9
+    # bandwidth part: cross-entropy 8 B per logit, AdamW 28 B per parameter, per block ~14 passes over [tokens, dim] and
+    # ~5 over [tokens, ffn] in fp32 (normalisations, residuals, activations and the bf16 images the GEMMs read)
+    params = weights + c["vocab"] * c["dim"] + c["seq"] * c["dim"]
+    hbm_bytes = 8 * tokens * c["vocab"] + (28 * params if c["adamw"] else 4 * params) + \
+        c["blocks"] * tokens * 4 * (14 * c["dim"] + 5 * c["ffn"])
+    floor_ms += hbm_bytes / PEAK_HBM_GBS / 1e6
+    return {"bound": "mfma", "achieved": round((gemm_flops + attn_flops) / ms / 1e9, 2),
+            "peak": round((gemm_flops + attn_flops) / floor_ms / 1e9, 2), "unit": "TFLOP/s", "frac": round(floor_ms / ms, 4),
+            "floor_ms": round(floor_ms, 3),
+            "note": "peak = algorithmic FLOPs / (projection FLOPs at the bf16 MFMA peak + attention FLOPs at the fp32 MFMA peak "
+                    "+ elementwise, loss and optimizer bytes at the HBM peak)"}
+
+
+def cpu_baseline_train_step(name):
+    """The reference CPU backend's training step, measured on a bounded sample and extrapolated (it would take an hour or
+    more at full size): cpu::Model with ONE block + the LM head and with the LM head alone, batch 1, a short sequence at
+    full widths and vocabulary (projection cost is linear in tokens), plus the attention core of one (batch, head) slice
+    at a sequence length the host finishes in seconds (its cost is quadratic in the sequence length)."""
+    from oracle import bfo
+    impl = bfo.reference() or bfo.oracle()
+    c = TRAIN_CONFIGS[name]
+    rng = np.random.default_rng(11)
+    s0 = {"tiny_lm": c["seq"], "gpt_small": 32, "long_context": 8}[name]
+
+    def timed_model(blocks, batch=1, seq=None):
+        seq = seq or s0
+        # the reference's feed-forward block is SiLU only; where the configuration says GELU the real reference is timed
+        # with SiLU (same projections, one transcendental per hidden element either way)
+        act = 0 if impl.is_reference else c["act"]
+        model = impl.model(lm_layers(bfo, c["vocab"], c["dim"], c["seq"], c["heads"], c["ffn"], act, blocks))
+        for i, count in enumerate(model.counts):   # the loops' cost does not depend on the values: a cheap non-constant fill
+            model.value(i)[:] = np.resize(rng.standard_normal(4099, dtype=np.float32) * np.float32(0.02), count)
+        ids = rng.integers(0, c["vocab"], (batch, seq)).astype(np.float32)
+        tgt = rng.integers(0, c["vocab"], batch * seq).astype(np.float32)
+        t0 = time.perf_counter()
+        model.zeroGrad()
+        logits = model.forward(ids, out_capacity=batch * seq * c["vocab"])
+        _, grad = impl.softmaxCrossEntropySparse(logits.reshape(batch * seq, c["vocab"]), tgt)
+        model.backward(grad)
+        if c["adamw"]:
+            model.adamwStep()
+        return time.perf_counter() - t0
+
+    if name == "tiny_lm":   # small enough to run whole
+        step_s = min(timed_model(c["blocks"], c["batch"], c["seq"]) for _ in range(3))
+        return {"value": round(c["batch"] * c["seq"] / step_s, 1), "unit": "tokens/s", "cores": 1,
+                "kind": "reference" if impl.is_reference else "port", "extrapolated": False,
+                "sample": ("feed-forward activation SiLU in place of GELU (the reference block has no GELU); " if impl.is_reference else "") +
+                          f"the whole step (zeroGrad, forward, sparse CE, backward, AdamW) through cpu::Model, best of 3, {step_s * 1e3:.1f} ms on one host core"}
+    def timed_block():
+        """One attention + feed-forward block alone on [1, s0, dim] features: forward, backward, optimizer."""
+        act = 0 if impl.is_reference else c["act"]
+        model = impl.model([(bfo.ATTENTION, c["heads"]), (bfo.FEEDFORWARD, c["ffn"], act)], input_features=c["dim"])
+        for i, count in enumerate(model.counts):
+            model.value(i)[:] = np.resize(rng.standard_normal(4099, dtype=np.float32) * np.float32(0.02), count)
+        x = rng.standard_normal((1, s0, c["dim"]), dtype=np.float32)
+        g = rng.standard_normal((1, s0, c["dim"]), dtype=np.float32)
+        t0 = time.perf_counter()
+        model.zeroGrad()
+        model.forward(x, out_capacity=x.size)
+        model.backward(g)
+        if c["adamw"]:
+            model.adamwStep()
+        return time.perf_counter() - t0
+
+    # embedding + head + loss at two token counts: a cost per step (zeroing and scatter-add over the whole embedding table,
+    # the optimizer over the parameters) and a cost per token
+    t_head, t_head2 = timed_model(0), timed_model(0, 1, 2 * s0)
+    head_per_token = max(t_head2 - t_head, 0.0) / s0
+    head_fixed = max(t_head - head_per_token * s0, 0.0)
+    t_block = timed_block()
+    hd = c["dim"] // c["heads"]
+    s_attn = min(c["seq"], 1024)
+    mk = lambda: rng.standard_normal((1, s_attn, hd), dtype=np.float32)
+    q, k, v, go = mk(), mk(), mk(), mk()
+    t0 = time.perf_counter()
+    impl.attentionCoreForward(q, k, v, 1, hd ** -0.5, 0)
+    impl.attentionCoreBackward(go, q, k, v, 1, hd ** -0.5, 0)
+    t_core = (time.perf_counter() - t0) * (c["seq"] / s_attn) ** 2
+    # per step: every token passes the head once and every block once; every (batch, head) slice runs the attention core
+    tokens = c["batch"] * c["seq"]
+    step_s = head_fixed + tokens * head_per_token + tokens / s0 * c["blocks"] * t_block + c["blocks"] * c["batch"] * c["heads"] * t_core
+    return {"value": round(c["batch"] * c["seq"] / step_s, 3), "unit": "tokens/s", "cores": 1,
+            "kind": "reference" if impl.is_reference else "port", "extrapolated": True,
+            "sample": ("feed-forward activation SiLU in place of GELU (the reference block has no GELU); " if impl.is_reference and c["act"] == 1 else "") +
+                      f"cpu::Model of one attention + feed-forward block, and of embedding + LM head + loss, each on batch 1 x {s0} tokens at full widths "
+                      f"(head {head_fixed:.2f} s per step + {head_per_token * 1e3:.1f} ms per token from runs at {s0} and {2 * s0} tokens, block {t_block:.2f} s), "
+                      f"scaled by tokens x {c['blocks']} blocks; attention core of one "
+                      f"(batch, head) slice at seq {s_attn} ({t_core * (s_attn / c['seq']) ** 2:.2f} s) scaled quadratically to seq {c['seq']} "
+                      f"and by {c['batch'] * c['heads']} slices x {c['blocks']} blocks; one host core, extrapolated step {step_s:.0f} s"}
 
 
 def bench_train_step(bf, name, steps, warmup):
@@ -338,7 +469,20 @@ def bench_train_step(bf, name, steps, warmup):
     return {"workload": c["what"], "tokens_per_s": round(tokens / (ms * 1e-3), 1), "ms_per_step": round(ms, 3),
             "wall_ms_per_step": round(wall_ms, 3), "tokens": tokens, "parameters": n_params,
             "algorithmic_tflop_per_step": round(flops / 1e12, 4), "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
-            "mean_loss": round(float(loss), 4)}
+            "mean_loss": round(float(loss), 4), "roofline": train_step_roofline(c, ms)}
+
+
+def extras_summary(extras):
+    """The north-star targets in three numbers: the bf16 projection at 4096^3 against the bf16 MFMA peak, and the worst and
+    the median bandwidth kernel against the HBM peak."""
+    hbm = sorted((v["frac_hbm"], k) for k, v in extras.items() if "frac_hbm" in v)
+    gemms = {k: v["frac_bf16_mfma"] for k, v in extras.items() if "frac_bf16_mfma" in v}
+    out = {"bf16_gemm_frac_of_peak": gemms}
+    if hbm:
+        out["hbm_min"] = {"kernel": hbm[0][1], "frac": hbm[0][0]}
+        out["hbm_median"] = {"kernel": hbm[len(hbm) // 2][1], "frac": hbm[len(hbm) // 2][0]}
+        out["hbm_below_0.70"] = [k for f, k in hbm if f < 0.70]
+    return out
 
 
 def main():
@@ -347,11 +491,11 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--extras", action="store_true", help="also time a bandwidth kernel and the bf16 GEMM")
+    ap.add_argument("--no-extras", action="store_true", help="skip the bandwidth kernels and the bf16 GEMMs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 256 MiB copy (bf_hip_scale by 1.0) so that a counter run of this command "
                          "holds a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
-    ap.add_argument("--train", default="gpt_small", help="comma list of train-step workloads to add (tiny_lm, mlp, gpt_small, "
+    ap.add_argument("--train", default="gpt_small,long_context,mlp,tiny_lm", help="comma list of train-step workloads to add (tiny_lm, mlp, gpt_small, "
                     "long_context) or 'none'")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -394,6 +538,8 @@ def main():
                      "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES["attnBackwardDkvKernel"],
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this kernel on this workload, recorded in "
+                                       "profiles/attention_c3_kernel_trace.md (counters cannot be read from inside this run)",
                      "flops_per_launch": fl["dkv"], "launch_ms": round(dkv_ms, 4)},
         "frac_of_fp32_mfma_peak": round(value / PEAK_FP32_MFMA_TFLOPS, 4),
         "kernel_ms": {k: round(v, 4) for k, v in res["kernel_ms"].items()},
@@ -409,11 +555,14 @@ def main():
         line["train_step"] = {name: (bench_mlp if name == "mlp" else lambda b, s_, w_: bench_train_step(b, name, s_, w_))(
                                   bf, max(3, args.steps // 2), max(1, args.warmup // 2))
                               for name in args.train.split(",")}
-    if args.extras:
+    if not args.no_extras:
         line["extras"] = bench_extras(bf, max(5, args.steps // 2))
+        line["extras_summary"] = extras_summary(line["extras"])
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_attention()
         line["cpu_baseline"]["host_cores"] = os.cpu_count()
+        for name in line.get("train_step", {}):
+            line["train_step"][name]["cpu_baseline"] = cpu_baseline_mlp() if name == "mlp" else cpu_baseline_train_step(name)
     print(json.dumps(line))
 
 

@@ -21,7 +21,13 @@
  *     documented as synchronous block the host.
  *   - Outputs never alias inputs unless a parameter says "in/out".  Zero-sized tensors are accepted
  *     and launch nothing (reference: device_pool.cu:30-32).
- *   - One host thread at a time per device, like the reference (device_pool.hpp:39-40).
+ *   - One host thread at a time per PROCESS, like the reference (device_pool.hpp:39-40): the pool, the cached bf16
+ *     weight images and the descriptor tables are unguarded registries.
+ *   - One stream in flight at a time per device.  Workspace and result blocks return to the pool when the host call
+ *     returns, while the kernels using them may still be queued; the next user of such a block is ordered behind them
+ *     only if it is enqueued on the same stream.  The cached weight images and descriptor tables are shared across
+ *     streams in the same way.  A caller that switches streams on a device synchronises the old one first
+ *     (bf_hip_stream_synchronize); overlapping two streams on one device is not supported.
  */
 #ifndef BF_HIP_H
 #define BF_HIP_H

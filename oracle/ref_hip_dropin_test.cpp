@@ -6,7 +6,9 @@
 //   2. Model(ir, 42): same parameter names, shapes and initial values as cpu::Model;
 //   3. runTraining(program, module, "", save): same epoch losses (1e-4) and final checkpoints (tolerance below),
 //      both backends starting from their own seed-42 initialisation and reading the same BFDATA1 file;
-//   4. checkpoint interop: the CPU run's file loads into hip::Model and the other way round.
+//   4. checkpoint interop: the CPU run's file loads into hip::Model and the other way round;
+//   5. device dispatch (hip/dispatch.hpp): `--device hip` / `hip:0` reach hip::Executor, hip::Model and hip::runTraining
+//      through runOnDevice / trainOnDevice with the results of steps 1 and 3; `hip:99` and `cuda` are refused.
 // Prints one line per check and exits non-zero on the first failure.
 #include <cmath>
 #include <cstdio>
@@ -20,6 +22,7 @@
 #include "blackforge/backend/cpu/model.hpp"
 #include "blackforge/backend/cpu/train_runner.hpp"
 #include "blackforge/backend/hip/checkpoint.hpp"
+#include "blackforge/backend/hip/dispatch.hpp"
 #include "blackforge/backend/hip/executor.hpp"
 #include "blackforge/backend/hip/model.hpp"
 #include "blackforge/backend/hip/train_runner.hpp"
@@ -191,6 +194,44 @@ int main(int argc, char** argv) {
             double werr = 0.0;
             for (std::size_t i = 0; i < cp.size(); ++i) werr = std::max(werr, maxRelError(cp[i]->value.data(), hp[i]->value.toHost().data(), 2e-2));
             report(werr <= 2e-2, r.model->name + ": checkpoints interchange between the backends; trained weights agree (max rel err " + std::to_string(werr) + ")");
+        }
+        // 5. the dispatch a CLI would go through
+        {
+            hip::DeviceSpec spec;
+            std::string error;
+            ir::Module module;
+            module.models.push_back(lm);
+            for (const char* name : {"hip", "hip:0"}) {
+                bool parsed = hip::parseDeviceSpec(name, spec, error);
+                hip::RunOutcome outcome = hip::runOnDevice(spec, module, 6);
+                cpu::Executor cx(42);
+                bf::runtime::Tensor want = cx.run(lm, cx.makeSyntheticInput(lm, 6));
+                double err = maxRelError(outcome.output.data(), want.data(), 1e-6);
+                report(parsed && outcome.output.shape() == want.shape() && err <= 1e-4,
+                       std::string("--device ") + name + ": runOnDevice gives the CPU executor's output (max rel err " + std::to_string(err) + ")");
+            }
+            const std::string ckpt = tmp + "/dropin_tiny_lm_cpu.bfckpt";   // written by the CPU training run above
+            hip::parseDeviceSpec("hip:0", spec, error);
+            hip::RunOutcome fromFile = hip::runOnDevice(spec, module, 4, ckpt);
+            cpu::Model cm(lm, 42U);
+            cpu::loadCheckpoint(cm, ckpt);
+            double err = maxRelError(fromFile.output.data(), cm.forward(fromFile.input).data(), 1e-6);
+            report(fromFile.loadedCheckpoint && err <= 1e-4, "--device hip:0 --from-checkpoint: output of the loaded weights matches cpu::Model (max rel err " + std::to_string(err) + ")");
+            ast::Program program = makeProgram(lm.name, tmp + "/dropin_lm.bfdata", "cross_entropy_sparse", "adamw", 2, 5, 5e-3, false);
+            cpu::TrainRunResult want = cpu::runTraining(program, module, "", "", nullptr);
+            hip::TrainRunResult got = hip::trainOnDevice(spec, program, module, "", "", nullptr);
+            double worst = 0.0;
+            for (std::size_t e = 0; e < want.epochLosses.size() && e < got.epochLosses.size(); ++e)
+                worst = std::max(worst, std::fabs(got.epochLosses[e] - want.epochLosses[e]) / std::fabs(want.epochLosses[e]));
+            report(got.epochLosses.size() == want.epochLosses.size() && worst <= 1e-4, "--device hip:0: trainOnDevice epoch losses match cpu::runTraining");
+            auto refused = [&](const char* name) {
+                if (!hip::parseDeviceSpec(name, spec, error)) return false;
+                try { (void)hip::runOnDevice(spec, module, 2); } catch (const std::invalid_argument&) { return true; }
+                return false;
+            };
+            report(refused("hip:99"), "--device hip:99 parses and is refused at selection (std::invalid_argument)");
+            report(refused("cuda"), "--device cuda parses and is refused by the HIP backend");
+            report(!hip::parseDeviceSpec("hip:x", spec, error) && error == "indice GPU non valido in 'hip:x'", "--device hip:x is a parse error");
         }
     } catch (const std::exception& e) {
         report(false, std::string("exception: ") + e.what());
