@@ -22,10 +22,10 @@ namespace {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---- flat kernels -----------------------------------------------------------------------------
-template <typename F>
+template <bool NT, typename F>
 __global__ void __launch_bounds__(kBlock) flat4Kernel(size_t n4, F f) {
     size_t stride = size_t(gridDim.x) * blockDim.x;
-    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) f.vec(i);
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) f.template vec<NT>(i);
 }
 template <typename F>
 __global__ void __launch_bounds__(kBlock) flat1Kernel(size_t begin, size_t n, F f) {
@@ -34,9 +34,10 @@ __global__ void __launch_bounds__(kBlock) flat1Kernel(size_t begin, size_t n, F 
 }
 
 // Runs f.vec(i) over groups of four elements when every pointer is 16-byte aligned, then f.one(i) over
-// the tail (or over everything otherwise).
+// the tail (or over everything otherwise).  bytesPerElement: what the op reads and writes per element, which decides
+// whether the launch streams past the last-level cache.
 template <typename F>
-int launchFlat(size_t n, bool canVectorise, F f, hipStream_t stream) {
+int launchFlat(size_t n, bool canVectorise, F f, hipStream_t stream, size_t bytesPerElement = 8) {
     if (n == 0) return BF_OK;
     // one group of four elements per thread and a grid that covers the whole array: the access stream stays
     // in address order across the device, which HBM rewards (grid-stride loops over a few blocks per CU lose
@@ -45,7 +46,8 @@ int launchFlat(size_t n, bool canVectorise, F f, hipStream_t stream) {
     size_t done = 0;
     if (canVectorise && n >= 4) {
         size_t n4 = n / 4;
-        flat4Kernel<<<gridFor(n4, kBlock, cap), kBlock, 0, stream>>>(n4, f);
+        if (streamsPastCache(n * bytesPerElement)) flat4Kernel<true><<<gridFor(n4, kBlock, cap), kBlock, 0, stream>>>(n4, f);
+        else flat4Kernel<false><<<gridFor(n4, kBlock, cap), kBlock, 0, stream>>>(n4, f);
         BF_LAUNCH_CHECK();
         done = n4 * 4;
     }
@@ -58,36 +60,36 @@ int launchFlat(size_t n, bool canVectorise, F f, hipStream_t stream) {
 
 struct AddOp {
     const float* a; const float* b; float* out;
-    __device__ void vec(size_t i) const { storef4(out + 4 * i, loadf4(a + 4 * i) + loadf4(b + 4 * i)); }
+    template <bool NT> __device__ void vec(size_t i) const { stf4<NT>(out + 4 * i, ldf4<NT>(a + 4 * i) + ldf4<NT>(b + 4 * i)); }
     __device__ void one(size_t i) const { out[i] = a[i] + b[i]; }
 };
 struct ScaleOp {
     const float* x; float* out; float factor;
-    __device__ void vec(size_t i) const { storef4(out + 4 * i, loadf4(x + 4 * i) * factor); }
+    template <bool NT> __device__ void vec(size_t i) const { stf4<NT>(out + 4 * i, ldf4<NT>(x + 4 * i) * factor); }
     __device__ void one(size_t i) const { out[i] = x[i] * factor; }
 };
 struct AccumulateOp {
     float* target; const float* delta;
-    __device__ void vec(size_t i) const { storef4(target + 4 * i, loadf4(target + 4 * i) + loadf4(delta + 4 * i)); }
+    template <bool NT> __device__ void vec(size_t i) const { stf4<NT>(target + 4 * i, ldf4<NT>(target + 4 * i) + ldf4<NT>(delta + 4 * i)); }
     __device__ void one(size_t i) const { target[i] += delta[i]; }
 };
 template <int ACT>
 struct ActForwardOp {
     const float* x; float* out;
-    __device__ void vec(size_t i) const {
-        float4v v = loadf4(x + 4 * i);
+    template <bool NT> __device__ void vec(size_t i) const {
+        float4v v = ldf4<NT>(x + 4 * i);
         v.x = actF<ACT>(v.x); v.y = actF<ACT>(v.y); v.z = actF<ACT>(v.z); v.w = actF<ACT>(v.w);
-        storef4(out + 4 * i, v);
+        stf4<NT>(out + 4 * i, v);
     }
     __device__ void one(size_t i) const { out[i] = actF<ACT>(x[i]); }
 };
 template <int ACT>
 struct ActBackwardOp {
     const float* x; const float* g; float* out;
-    __device__ void vec(size_t i) const {
-        float4v v = loadf4(x + 4 * i), gv = loadf4(g + 4 * i);
+    template <bool NT> __device__ void vec(size_t i) const {
+        float4v v = ldf4<NT>(x + 4 * i), gv = ldf4<NT>(g + 4 * i);
         v.x = gv.x * actD<ACT>(v.x); v.y = gv.y * actD<ACT>(v.y); v.z = gv.z * actD<ACT>(v.z); v.w = gv.w * actD<ACT>(v.w);
-        storef4(out + 4 * i, v);
+        stf4<NT>(out + 4 * i, v);
     }
     __device__ void one(size_t i) const { out[i] = g[i] * actD<ACT>(x[i]); }
 };
@@ -96,13 +98,13 @@ struct ActBackwardOp {
 template <int ACT>
 struct ActImageOp {
     const float* z; unsigned short* image;
-    __device__ void vec(size_t i) const {
-        const float4v a = loadf4(z + 8 * i), b = loadf4(z + 8 * i + 4);
+    template <bool NT> __device__ void vec(size_t i) const {
+        const float4v a = ldf4<NT>(z + 8 * i), b = ldf4<NT>(z + 8 * i + 4);
         uint4v packed = {unsigned(toBf16Bits(actF<ACT>(a.x))) | unsigned(toBf16Bits(actF<ACT>(a.y))) << 16,
                          unsigned(toBf16Bits(actF<ACT>(a.z))) | unsigned(toBf16Bits(actF<ACT>(a.w))) << 16,
                          unsigned(toBf16Bits(actF<ACT>(b.x))) | unsigned(toBf16Bits(actF<ACT>(b.y))) << 16,
                          unsigned(toBf16Bits(actF<ACT>(b.z))) | unsigned(toBf16Bits(actF<ACT>(b.w))) << 16};
-        *reinterpret_cast<uint4v*>(image + 8 * i) = packed;
+        stu4<NT>(image + 8 * i, packed);
     }
 };
 
@@ -136,13 +138,13 @@ RowGeom rowGeometry(size_t rows, size_t features, bool canVectorise, unsigned ma
 template <int VEC> struct Pack;
 template <> struct Pack<4> {
     using T = float4v;
-    static __device__ T load(const float* p) { return loadf4(p); }
-    static __device__ void store(float* p, T v) { storef4(p, v); }
+    template <bool NT = false> static __device__ T load(const float* p) { return ldf4<NT>(p); }
+    template <bool NT = false> static __device__ void store(float* p, T v) { stf4<NT>(p, v); }
 };
 template <> struct Pack<1> {
     using T = float;
-    static __device__ T load(const float* p) { return *p; }
-    static __device__ void store(float* p, T v) { *p = v; }
+    template <bool NT = false> static __device__ T load(const float* p) { return ldf1<NT>(p); }
+    template <bool NT = false> static __device__ void store(float* p, T v) { stf1<NT>(p, v); }
 };
 template <int ACT> __device__ float4v actF4(float4v v) {
     v.x = actF<ACT>(v.x); v.y = actF<ACT>(v.y); v.z = actF<ACT>(v.z); v.w = actF<ACT>(v.w); return v;
@@ -154,7 +156,7 @@ template <int ACT> __device__ float4v actD4(float4v v) {
 template <int ACT> __device__ float actD4(float v) { return actD<ACT>(v); }
 
 // MODE 0: x + bias; 1: act(x + bias); 2: x + bias + residual
-template <int VEC, int MODE, int ACT>
+template <int VEC, int MODE, int ACT, bool NT>
 __global__ void __launch_bounds__(256) biasKernel(const float* __restrict__ x, const float* __restrict__ bias,
                                                    const float* __restrict__ residual, float* __restrict__ out,
                                                    size_t rows, size_t features) {
@@ -164,17 +166,17 @@ __global__ void __launch_bounds__(256) biasKernel(const float* __restrict__ x, c
     size_t rowStep = size_t(gridDim.y) * blockDim.y;
     for (size_t r = size_t(blockIdx.y) * blockDim.y + threadIdx.y; r < rows; r += rowStep) {
         size_t idx = r * features + col;
-        typename Pack<VEC>::T v = Pack<VEC>::load(x + idx) + b;
+        typename Pack<VEC>::T v = Pack<VEC>::template load<NT>(x + idx) + b;
         if constexpr (MODE == 1) v = actF4<ACT>(v);
-        if constexpr (MODE == 2) v = v + Pack<VEC>::load(residual + idx);
-        Pack<VEC>::store(out + idx, v);
+        if constexpr (MODE == 2) v = v + Pack<VEC>::template load<NT>(residual + idx);
+        Pack<VEC>::template store<NT>(out + idx, v);
     }
 }
 
 // Column sums, optionally fused with dGemm = dHidden * act'(gemm + bias) (FUSED = 1).
 // Each block reduces its rows per column in registers, then over threadIdx.y through LDS, and writes
 // one partial row per blockIdx.y; columnFinishKernel adds the partial rows in a fixed order.
-template <int VEC, int FUSED, int ACT>
+template <int VEC, int FUSED, int ACT, bool NT>
 __global__ void __launch_bounds__(256) columnSumKernel(const float* __restrict__ src, const float* __restrict__ bias,
                                                         const float* __restrict__ dHidden, float* __restrict__ dGemm,
                                                         float* __restrict__ partial, size_t rows, size_t features,
@@ -189,15 +191,15 @@ __global__ void __launch_bounds__(256) columnSumKernel(const float* __restrict__
         // FUSED: either output may be absent; `image` (four-column form only) receives the product rounded to bf16
         auto term = [&](size_t r) {
             size_t idx = r * features + col;
-            typename Pack<VEC>::T v = Pack<VEC>::load(src + idx);
+            typename Pack<VEC>::T v = Pack<VEC>::template load<NT>(src + idx);
             if constexpr (FUSED) {
-                v = Pack<VEC>::load(dHidden + idx) * actD4<ACT>(v + b);
-                if (dGemm) Pack<VEC>::store(dGemm + idx, v);
+                v = Pack<VEC>::template load<NT>(dHidden + idx) * actD4<ACT>(v + b);
+                if (dGemm) Pack<VEC>::template store<NT>(dGemm + idx, v);
                 if constexpr (VEC == 4) {
                     if (image) {
                         uint2v packed = {unsigned(toBf16Bits(v.x)) | unsigned(toBf16Bits(v.y)) << 16,
                                          unsigned(toBf16Bits(v.z)) | unsigned(toBf16Bits(v.w)) << 16};
-                        *reinterpret_cast<uint2v*>(image + idx) = packed;
+                        stu2<NT>(image + idx, packed);
                     }
                 }
             }
@@ -283,10 +285,16 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
     if (scratch.status != BF_OK) return scratch.status;
     float* partial = dBias ? (workspace ? workspace : scratch.as<float>()) : nullptr;
     if (image && g.vec != 4) return failInvalid("act_backward_image", "operands must be 16-byte aligned and the width a multiple of 4");
-    if (g.vec == 4)
-        columnSumKernel<4, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features, image);
-    else
-        columnSumKernel<1, FUSED, ACT><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
+    // bytes per element: the source, and on the fused route the second input and whichever outputs are written
+    const size_t perElement = 4 + (FUSED ? 4 + (dGemm ? 4 : 0) + (image ? 2 : 0) : 0);
+    const bool nt = streamsPastCache(rows * features * perElement);
+    if (g.vec == 4) {
+        if (nt) columnSumKernel<4, FUSED, ACT, true><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features, image);
+        else columnSumKernel<4, FUSED, ACT, false><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features, image);
+    } else {
+        if (nt) columnSumKernel<1, FUSED, ACT, true><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
+        else columnSumKernel<1, FUSED, ACT, false><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
+    }
     BF_LAUNCH_CHECK();
     if (dBias) {
         columnFinishKernel<<<gridFor(features, 16), kBlock, 0, stream>>>(partial, dBias, parts, features);
@@ -319,13 +327,14 @@ struct ZeroTensor {
     unsigned firstBlock;
     unsigned pad;
 };
+template <bool NT>
 __global__ void __launch_bounds__(kBlock) zeroMultiKernel(const ZeroTensor* __restrict__ table, int numTensors) {
     const ZeroTensor c = table[owningTensor(table, numTensors, blockIdx.x)];
     const size_t base = (size_t(blockIdx.x - c.firstBlock) * kBlock + threadIdx.x) * 4;
     if (base >= c.count) return;
     if ((reinterpret_cast<uintptr_t>(c.ptr) & 15u) == 0 && base + 4 <= c.count) {
         const float4v z = {0.0f, 0.0f, 0.0f, 0.0f};
-        storef4(c.ptr + base, z);
+        stf4<NT>(c.ptr + base, z);
     } else {
         for (size_t i = base; i < base + 4 && i < c.count; ++i) c.ptr[i] = 0.0f;
     }
@@ -338,9 +347,16 @@ int actToBf16Image(const float* z, unsigned short* image, size_t n, int act, hip
     if (n % 8 != 0 || !aligned16(z) || !aligned16(image)) return failInvalid("act_image", "needs 16-byte aligned operands and a multiple of 8 elements");
     const size_t groups = n / 8;
     const unsigned grid = gridFor(groups, kBlock, 1u << 30);
-    if (act == BF_ACT_SILU) flat4Kernel<<<grid, kBlock, 0, stream>>>(groups, ActImageOp<BF_ACT_SILU>{z, image});
-    else if (act == BF_ACT_GELU) flat4Kernel<<<grid, kBlock, 0, stream>>>(groups, ActImageOp<BF_ACT_GELU>{z, image});
-    else flat4Kernel<<<grid, kBlock, 0, stream>>>(groups, ActImageOp<BF_ACT_RELU>{z, image});
+    const bool nt = streamsPastCache(n * 6);
+#define BF_ACT_IMAGE(ACT)                                                                                  \
+    do {                                                                                                   \
+        if (nt) flat4Kernel<true><<<grid, kBlock, 0, stream>>>(groups, ActImageOp<ACT>{z, image});         \
+        else flat4Kernel<false><<<grid, kBlock, 0, stream>>>(groups, ActImageOp<ACT>{z, image});           \
+    } while (0)
+    if (act == BF_ACT_SILU) BF_ACT_IMAGE(BF_ACT_SILU);
+    else if (act == BF_ACT_GELU) BF_ACT_IMAGE(BF_ACT_GELU);
+    else BF_ACT_IMAGE(BF_ACT_RELU);
+#undef BF_ACT_IMAGE
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -361,7 +377,7 @@ extern "C" {
 int bf_hip_add(const float* a, const float* b, float* out, size_t n, bf_stream_t stream) {
     if (n == 0) return BF_OK;
     BF_REQUIRE(a && b && out, "NULL pointer");
-    return launchFlat(n, aligned16(a) && aligned16(b) && aligned16(out), AddOp{a, b, out}, asStream(stream));
+    return launchFlat(n, aligned16(a) && aligned16(b) && aligned16(out), AddOp{a, b, out}, asStream(stream), 12);
 }
 
 int bf_hip_scale(const float* x, float factor, float* out, size_t n, bf_stream_t stream) {
@@ -373,7 +389,7 @@ int bf_hip_scale(const float* x, float factor, float* out, size_t n, bf_stream_t
 int bf_hip_accumulate(float* target, const float* delta, size_t n, bf_stream_t stream) {
     if (n == 0) return BF_OK;
     BF_REQUIRE(target && delta, "NULL pointer");
-    return launchFlat(n, aligned16(target) && aligned16(delta), AccumulateOp{target, delta}, asStream(stream));
+    return launchFlat(n, aligned16(target) && aligned16(delta), AccumulateOp{target, delta}, asStream(stream), 12);
 }
 
 int bf_hip_act_forward(const float* x, float* out, size_t n, int act, bf_stream_t stream) {
@@ -393,19 +409,24 @@ int bf_hip_act_backward(const float* x, const float* g, float* out, size_t n, in
     BF_REQUIRE(x && g && out, "NULL pointer");
     bool vec = aligned16(x) && aligned16(g) && aligned16(out);
     switch (act) {
-        case BF_ACT_SILU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_SILU>{x, g, out}, asStream(stream));
-        case BF_ACT_GELU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_GELU>{x, g, out}, asStream(stream));
-        case BF_ACT_RELU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_RELU>{x, g, out}, asStream(stream));
+        case BF_ACT_SILU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_SILU>{x, g, out}, asStream(stream), 12);
+        case BF_ACT_GELU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_GELU>{x, g, out}, asStream(stream), 12);
+        case BF_ACT_RELU: return launchFlat(n, vec, ActBackwardOp<BF_ACT_RELU>{x, g, out}, asStream(stream), 12);
         default: return failInvalid(__func__, "unknown activation " + std::to_string(act));
     }
 }
 
 #define BF_BIAS_LAUNCH(MODE, ACT)                                                                               \
     do {                                                                                                        \
-        if (g.vec == 4)                                                                                         \
-            biasKernel<4, MODE, ACT><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
+        const bool nt = streamsPastCache(rows * features * (MODE == 2 ? 12 : 8));                               \
+        if (g.vec == 4 && nt)                                                                                   \
+            biasKernel<4, MODE, ACT, true><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
+        else if (g.vec == 4)                                                                                    \
+            biasKernel<4, MODE, ACT, false><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
+        else if (nt)                                                                                            \
+            biasKernel<1, MODE, ACT, true><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
         else                                                                                                    \
-            biasKernel<1, MODE, ACT><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
+            biasKernel<1, MODE, ACT, false><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
     } while (0)
 
 int bf_hip_add_bias(const float* x, const float* bias, float* out, size_t rows, size_t features, bf_stream_t stream) {
@@ -486,7 +507,8 @@ int bf_hip_zero_multi(float* const* ptrs, const size_t* counts, size_t numTensor
     const void* device = nullptr;
     int status = uploadDescriptorTable(kSlotZero, table.data(), table.size() * sizeof(ZeroTensor), asStream(stream), &device);
     if (status != BF_OK) return status;
-    zeroMultiKernel<<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const ZeroTensor*>(device), int(numTensors));
+    // plain stores: the hint pays only for kernels that also read (0.87 of HBM peak without it, 0.85 with it)
+    zeroMultiKernel<false><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const ZeroTensor*>(device), int(numTensors));
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

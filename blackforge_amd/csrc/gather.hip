@@ -2,11 +2,15 @@
 // KV-cache concatenation, token-id range check and last-position argmax.
 //
 // All HBM-bound.  The embedding gradient avoids both the memset and the per-element global atomics of
-// the usual scatter-add: tokens are bucketed by id with a counting sort (integer work only), then one
-// wavefront per vocabulary row adds that row's tokens in token order and writes the row once (rows
-// nobody used are written as zeros).  The result is deterministic and equals a sequential
-// token-order sum in fp32.
+// the usual scatter-add.  A training batch (up to 16384 tokens) runs as ONE launch in which a wavefront per
+// token finds the other tokens with its id through bitmaps in LDS and the workgroups share out the rows
+// that stay zero; longer token lists are bucketed by id with a counting sort (integer work only), then one
+// wavefront per vocabulary row adds that row's tokens.  Either way a row's tokens are added in token order
+// and every row is written once: the result is deterministic and equals the CPU loop's sum bit for bit.
 #include "common.hpp"
+
+#include <algorithm>
+#include <type_traits>
 
 namespace bf {
 namespace {
@@ -34,21 +38,28 @@ __global__ void __launch_bounds__(kBlock) countOutOfRangeKernel(const float* __r
 // One row of `dim` floats per (token); 2-D layout as in the bias kernels: no division on the memory path.
 template <int VEC>
 __global__ void __launch_bounds__(256) embeddingForwardKernel(const float* __restrict__ ids, const float* __restrict__ table,
-                                                              float* __restrict__ out, size_t tokens, size_t dim) {
+                                                              float* __restrict__ out, size_t tokens, size_t dim, long long vocab) {
     size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
     if (col >= dim) return;
     size_t step = size_t(gridDim.y) * blockDim.y;
     for (size_t t = size_t(blockIdx.y) * blockDim.y + threadIdx.y; t < tokens; t += step) {
-        size_t id = size_t(roundId(ids[t]));
-        if constexpr (VEC == 4) storef4(out + t * dim + col, loadf4(table + id * dim + col));
-        else out[t * dim + col] = table[id * dim + col];
+        // an id outside the table (the validating variant rejects those before the launch) reads nothing: zeros
+        const long long id = roundId(ids[t]);
+        const bool inside = id >= 0 && id < vocab;
+        if constexpr (VEC == 4) storef4(out + t * dim + col, inside ? loadf4(table + size_t(id) * dim + col) : float4v{0.0f, 0.0f, 0.0f, 0.0f});
+        else out[t * dim + col] = inside ? table[size_t(id) * dim + col] : 0.0f;
     }
 }
 
 // ---- embedding backward: counting sort by id ---------------------------------------------------
-__global__ void __launch_bounds__(kBlock) histogramKernel(const float* __restrict__ ids, size_t tokens, unsigned* __restrict__ counts) {
+// Ids outside [0, vocab) take no part in any of the kernels below (no count, no slot, no sum).
+__device__ __forceinline__ bool idInside(long long id, size_t vocab) { return id >= 0 && (unsigned long long)id < vocab; }
+
+__global__ void __launch_bounds__(kBlock) histogramKernel(const float* __restrict__ ids, size_t tokens, unsigned* __restrict__ counts, size_t vocab) {
     size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < tokens) atomicAdd(&counts[size_t(roundId(ids[i]))], 1u);
+    if (i >= tokens) return;
+    const long long id = roundId(ids[i]);
+    if (idInside(id, vocab)) atomicAdd(&counts[size_t(id)], 1u);
 }
 
 // Exclusive scan of counts[0..vocab) into offsets[0..vocab], single block of 1024 threads, four consecutive
@@ -95,24 +106,148 @@ __global__ void __launch_bounds__(1024) exclusiveScanKernel(const unsigned* __re
 // the segment (the number of tokens that share the id).
 __global__ void __launch_bounds__(kBlock) scatterTokensKernel(const float* __restrict__ ids, size_t tokens,
                                                               const unsigned* __restrict__ offsets, unsigned* __restrict__ counts,
-                                                              unsigned* __restrict__ unordered) {
+                                                              unsigned* __restrict__ unordered, size_t vocab) {
     size_t t = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (t >= tokens) return;
+    if (!idInside(roundId(ids[t]), vocab)) return;
     size_t id = size_t(roundId(ids[t]));
     unsigned left = atomicSub(&counts[id], 1u);   // value before the decrement: counts[id] .. 1
     unordered[offsets[id] + left - 1u] = unsigned(t);
 }
 __global__ void __launch_bounds__(kBlock) rankTokensKernel(const float* __restrict__ ids, size_t tokens,
                                                            const unsigned* __restrict__ offsets,
-                                                           const unsigned* __restrict__ unordered, unsigned* __restrict__ order) {
+                                                           const unsigned* __restrict__ unordered, unsigned* __restrict__ order, size_t vocab) {
     size_t t = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (t >= tokens) return;
+    if (!idInside(roundId(ids[t]), vocab)) return;
     size_t id = size_t(roundId(ids[t]));
     unsigned begin = offsets[id], end = offsets[id + 1], rank = 0;
     for (unsigned j = begin; j < end; ++j) rank += unordered[j] < unsigned(t) ? 1u : 0u;
     order[begin + rank] = unsigned(t);
 }
 
+// Few tokens (at most kByTokenMax: a training batch) against a large table: no sort, ONE launch.  A workgroup takes 16
+// tokens, one per wavefront, and a share of consecutive table rows.  All 1024 threads together look at every token's id
+// once: they compare it with the workgroup's 16 ids (a register compare away) and mark the matches in 16 bitmaps in LDS,
+// one bit per token, and they mark the rows of the workgroup's share that some token uses.  The rows of the share that
+// no token uses are then written as zeros.  A wavefront whose token is not the first with its id (a bit below its own
+// is set) has nothing more to do; otherwise it walks its bitmap upwards, adds the rows of the tokens it finds, in token
+// order, and writes the table row.  Every table row is written exactly once, by whoever knows its value, with no chain
+// of small dependent launches in front of the 98 MB that the gradient of a 32000 x 768 table has to move (the counting
+// sort below spends more time in its five small launches than in that write).
+constexpr size_t kByTokenMax = 16384;
+constexpr int kTokensPerGroup = 16;
+template <int VEC>
+__global__ void __launch_bounds__(1024) embeddingBackwardByTokenKernel(const float* __restrict__ ids, const float* __restrict__ g,
+                                                                       float* __restrict__ dTable, unsigned tokens, size_t vocab,
+                                                                       size_t dim) {
+    extern __shared__ unsigned bitmaps[];   // [16][words]: bit j of bitmaps[s] = token j has the id of the group's token s
+    __shared__ int groupId[kTokensPerGroup];
+    const unsigned words = (tokens + 31) / 32;
+    // this workgroup's share of the table rows, and (after the 16 bitmaps) one bit per row of it: some token uses the row
+    const unsigned share = unsigned((vocab + gridDim.x - 1) / gridDim.x);
+    const long long rowLo = (long long)blockIdx.x * share, rowHi = rowLo + share < (long long)vocab ? rowLo + share : (long long)vocab;
+    unsigned* used = bitmaps + words * kTokensPerGroup;
+    const unsigned usedWords = (share + 31) / 32;
+    const unsigned lane = threadIdx.x & 63, slot = threadIdx.x >> 6, t0 = blockIdx.x * kTokensPerGroup;
+    auto toId = [&](float v) { const long long id = roundId(v); return idInside(id, vocab) ? int(id) : -2; };   // -2: matches nothing
+    for (unsigned w = threadIdx.x; w < words * kTokensPerGroup + usedWords; w += 1024) bitmaps[w] = 0u;
+    if (threadIdx.x < kTokensPerGroup) {
+        const unsigned t = t0 + threadIdx.x;
+        const int id = t < tokens ? toId(ids[t]) : -2;
+        groupId[threadIdx.x] = id == -2 ? -1 : id;   // -1: no row to write; never equal to a token's -2
+    }
+    __syncthreads();
+    int mine[kTokensPerGroup];
+#pragma unroll
+    for (int s = 0; s < kTokensPerGroup; ++s) mine[s] = groupId[s];
+    auto mark = [&](unsigned j, int id) {
+#pragma unroll
+        for (int s = 0; s < kTokensPerGroup; ++s)
+            if (id == mine[s]) atomicOr(&bitmaps[s * words + (j >> 5)], 1u << (j & 31u));
+        if (id >= rowLo && id < rowHi) atomicOr(&used[unsigned(id - rowLo) >> 5], 1u << (unsigned(id - rowLo) & 31u));
+    };
+    if ((reinterpret_cast<uintptr_t>(ids) & 15u) == 0) {
+        // four ids per load and every load of a thread issued before the first is used: one memory latency, not one per id
+        constexpr int PER = int(kByTokenMax / 4 / 1024);
+        float4v v[PER];
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const unsigned i4 = threadIdx.x + 1024u * u;
+            v[u] = 4 * i4 + 4 <= tokens ? loadf4(ids + 4 * i4) : float4v{-1.0f, -1.0f, -1.0f, -1.0f};
+        }
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const unsigned j = 4 * (threadIdx.x + 1024u * u);
+            if (j + 4 <= tokens) { mark(j, toId(v[u].x)); mark(j + 1, toId(v[u].y)); mark(j + 2, toId(v[u].z)); mark(j + 3, toId(v[u].w)); }
+        }
+        for (unsigned j = (tokens & ~3u) + threadIdx.x; j < tokens; j += 1024) mark(j, toId(ids[j]));
+    } else {
+        for (unsigned j = threadIdx.x; j < tokens; j += 1024) mark(j, toId(ids[j]));
+    }
+    __syncthreads();
+    // zeros for the rows of the share that no token uses: a wavefront per row, 64 * VEC columns per store
+    for (long long row = rowLo + slot; row < rowHi; row += kTokensPerGroup) {
+        const unsigned r = unsigned(row - rowLo);
+        if ((used[r >> 5] >> (r & 31u)) & 1u) continue;
+        float* out = dTable + size_t(row) * dim;
+        for (size_t col = size_t(lane) * VEC; col < dim; col += size_t(64) * VEC) {
+            if constexpr (VEC == 4) storef4(out + col, float4v{0.0f, 0.0f, 0.0f, 0.0f});
+            else out[col] = 0.0f;
+        }
+    }
+    const unsigned t = t0 + slot;
+    if (t >= tokens) return;
+    const int id = groupId[slot];
+    if (id < 0) return;
+    const unsigned* bits = bitmaps + slot * words;
+    // wave-uniform: a set bit below this token's own means an earlier token owns the id's row
+    for (unsigned base = 0; base <= (t >> 5); base += 64) {
+        const unsigned w = base + lane;
+        unsigned word = w <= (t >> 5) ? bits[w] : 0u;
+        if (w == (t >> 5)) word &= (1u << (t & 31u)) - 1u;
+        if (__ballot(word != 0u) != 0) return;
+    }
+    constexpr int CHUNKS = 4;   // column groups of 64 * VEC held in registers per pass over the bitmap
+    typedef typename std::conditional<VEC == 4, float4v, float>::type V;
+    for (size_t col0 = 0; col0 < dim; col0 += size_t(64) * VEC * CHUNKS) {
+        V acc[CHUNKS];
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) acc[c] = V{};
+        for (unsigned base = (t >> 5) & ~63u; base < words; base += 64) {
+            const unsigned w = base + lane;
+            const unsigned word = w < words ? bits[w] : 0u;
+            unsigned long long lanes = __ballot(word != 0u);
+            while (lanes != 0) {   // words in ascending order, bits of a word in ascending order: token order
+                const int src = __ffsll((long long)lanes) - 1;
+                lanes &= lanes - 1;
+                unsigned pending = unsigned(__builtin_amdgcn_readlane(int(word), src));
+                while (pending != 0) {
+                    const unsigned k = (base + unsigned(src)) * 32u + unsigned(__ffs(int(pending))) - 1u;   // >= t: lower bits were ruled out above
+                    pending &= pending - 1;
+                    const float* row = g + size_t(k) * dim;
+#pragma unroll
+                    for (int c = 0; c < CHUNKS; ++c) {
+                        const size_t col = col0 + (size_t(c) * 64 + lane) * VEC;
+                        if (col < dim) {
+                            if constexpr (VEC == 4) acc[c] = acc[c] + loadf4(row + col);
+                            else acc[c] += row[col];
+                        }
+                    }
+                }
+            }
+        }
+        float* out = dTable + size_t(id) * dim;
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+            const size_t col = col0 + (size_t(c) * 64 + lane) * VEC;
+            if (col < dim) {
+                if constexpr (VEC == 4) storef4(out + col, acc[c]);
+                else out[col] = acc[c];
+            }
+        }
+    }
+}
 // One wavefront per vocabulary row.
 template <int VEC>
 __global__ void __launch_bounds__(kBlock) embeddingBackwardKernel(const float* __restrict__ g, float* __restrict__ dTable,
@@ -289,12 +424,11 @@ int bf_hip_count_out_of_range(const float* ids, size_t count, size_t limit, size
 
 int bf_hip_embedding_forward(const float* ids, const float* table, float* out, size_t tokens, size_t vocab, size_t dim,
                              bf_stream_t stream) {
-    (void)vocab;
     if (tokens == 0 || dim == 0) return BF_OK;
     BF_REQUIRE(ids && table && out, "NULL pointer");
     Geom2D g = geometry2D(tokens, dim, aligned16(table) && aligned16(out));
-    if (g.vec == 4) embeddingForwardKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(ids, table, out, tokens, dim);
-    else embeddingForwardKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(ids, table, out, tokens, dim);
+    if (g.vec == 4) embeddingForwardKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(ids, table, out, tokens, dim, (long long)vocab);
+    else embeddingForwardKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(ids, table, out, tokens, dim, (long long)vocab);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -307,6 +441,21 @@ int bf_hip_embedding_backward(const float* ids, const float* g, float* dTable, s
     hipStream_t s = asStream(stream);
     if (tokens == 0) return bf_hip_fill_zero(dTable, vocab * dim * sizeof(float), stream);
     BF_REQUIRE(ids && g, "NULL pointer");
+    if (tokens <= kByTokenMax && vocab * 2 >= tokens && vocab < (size_t(1) << 31)) {   // a batch of tokens against a table at least half as large
+        const bool vec = aligned16(g) && aligned16(dTable) && dim % 4 == 0;
+        // a workgroup per 16 tokens, and never fewer than two per compute unit: they also share out the rows to zero
+        const unsigned grid = std::max(unsigned((tokens + kTokensPerGroup - 1) / kTokensPerGroup), unsigned(computeUnits()) * 2u);
+        const size_t share = (vocab + grid - 1) / grid;
+        const size_t lds = ((tokens + 31) / 32 * kTokensPerGroup + (share + 31) / 32) * sizeof(unsigned);
+        const void* kernel = vec ? reinterpret_cast<const void*>(embeddingBackwardByTokenKernel<4>)
+                                 : reinterpret_cast<const void*>(embeddingBackwardByTokenKernel<1>);
+        int st = allowDynamicSharedMemory(kernel, lds);
+        if (st != BF_OK) return st;
+        if (vec) embeddingBackwardByTokenKernel<4><<<grid, 1024, lds, s>>>(ids, g, dTable, unsigned(tokens), vocab, dim);
+        else embeddingBackwardByTokenKernel<1><<<grid, 1024, lds, s>>>(ids, g, dTable, unsigned(tokens), vocab, dim);
+        BF_LAUNCH_CHECK();
+        return BF_OK;
+    }
     // counts[vocab] | offsets[vocab+1] | unordered[tokens] | order[tokens]
     size_t words = vocab + (vocab + 1) + 2 * tokens;
     Scratch work(words * sizeof(unsigned));
@@ -317,13 +466,13 @@ int bf_hip_embedding_backward(const float* ids, const float* g, float* dTable, s
     unsigned* order = unordered + tokens;
     int st = bf_hip_fill_zero(counts, vocab * sizeof(unsigned), stream);
     if (st != BF_OK) return st;
-    histogramKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, counts);
+    histogramKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, counts, vocab);
     BF_LAUNCH_CHECK();
     exclusiveScanKernel<<<1, 1024, 0, s>>>(counts, offsets, vocab);
     BF_LAUNCH_CHECK();
-    scatterTokensKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, offsets, counts, unordered);
+    scatterTokensKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, offsets, counts, unordered, vocab);
     BF_LAUNCH_CHECK();
-    rankTokensKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, offsets, unordered, order);
+    rankTokensKernel<<<gridFor(tokens, kBlock), kBlock, 0, s>>>(ids, tokens, offsets, unordered, order, vocab);
     BF_LAUNCH_CHECK();
     unsigned grid = gridFor(vocab, kBlock / 64);
     if (aligned16(g) && aligned16(dTable) && dim % 4 == 0)

@@ -30,6 +30,7 @@ typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));   // a fl
 inline size_t pad8(size_t n) { return (n + 7) / 8 * 8; }
 
 // out[r*ld + 0..colsPad) = bf16(x[r, 0..cols)), zero padded.
+template <bool NT>
 __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict__ x, unsigned short* __restrict__ out,
                                                         size_t rows, size_t cols, size_t colsPad, size_t ld) {
     const size_t groupsPerRow = colsPad / 8;
@@ -42,14 +43,17 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict_
         if (c + 8 <= cols) {
             // two 16-byte loads; global memory serves them from any 4-byte boundary, so rows of an odd width (which do
             // not start on 16-byte boundaries) take the same path
-            float4u a = *reinterpret_cast<const float4u*>(src), b = *reinterpret_cast<const float4u*>(src + 4);
+            float4u a, b;
+            if constexpr (NT) { a = __builtin_nontemporal_load(reinterpret_cast<const float4u*>(src)); b = __builtin_nontemporal_load(reinterpret_cast<const float4u*>(src + 4)); }
+            else { a = *reinterpret_cast<const float4u*>(src); b = *reinterpret_cast<const float4u*>(src + 4); }
             v[0] = toBf16Bits(a.x); v[1] = toBf16Bits(a.y); v[2] = toBf16Bits(a.z); v[3] = toBf16Bits(a.w);
             v[4] = toBf16Bits(b.x); v[5] = toBf16Bits(b.y); v[6] = toBf16Bits(b.z); v[7] = toBf16Bits(b.w);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = c + j < cols ? toBf16Bits(src[j]) : (unsigned short)0;
         }
-        *reinterpret_cast<ushort8*>(out + r * ld + c) = v;
+        if constexpr (NT) __builtin_nontemporal_store(v, reinterpret_cast<ushort8*>(out + r * ld + c));
+        else *reinterpret_cast<ushort8*>(out + r * ld + c) = v;
     }
 }
 
@@ -959,7 +963,8 @@ int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, 
     size_t colsPad = pad8(cols);
     size_t groups = rows * (colsPad / 8);
     if (groups == 0) return BF_OK;
-    convertKernel<<<gridFor(groups, kBlock), kBlock, 0, s>>>(x, out, rows, cols, colsPad, ld ? ld : colsPad);
+    if (streamsPastCache(rows * cols * 6)) convertKernel<true><<<gridFor(groups, kBlock), kBlock, 0, s>>>(x, out, rows, cols, colsPad, ld ? ld : colsPad);
+    else convertKernel<false><<<gridFor(groups, kBlock), kBlock, 0, s>>>(x, out, rows, cols, colsPad, ld ? ld : colsPad);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(1024) finishScaledSumKernel(const float* __res
     }
 }
 
-template <int VEC>
+template <int VEC, bool NT = false>
 __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pred, const float* __restrict__ target,
                                                     float* __restrict__ grad, float* __restrict__ partial, size_t n,
                                                     float gradScale) {
@@ -57,9 +57,9 @@ __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pr
     if constexpr (VEC == 4) {
         size_t n4 = n / 4;
         for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) {
-            float4v d = loadf4(pred + 4 * i) - loadf4(target + 4 * i);
+            float4v d = ldf4<NT>(pred + 4 * i) - ldf4<NT>(target + 4 * i);
             acc += d.x * d.x + d.y * d.y + d.z * d.z + d.w * d.w;
-            storef4(grad + 4 * i, d * gradScale);
+            stf4<NT>(grad + 4 * i, d * gradScale);
         }
         for (size_t i = n4 * 4 + size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
             float d = pred[i] - target[i];
@@ -79,7 +79,7 @@ __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pr
 
 // SPARSE: target holds one class index per row.  Otherwise a dense target row.
 // SHIFTED (with VEC = 4, CACHED): rows of any length and alignment through 16-byte accesses (RowCache::loadShifted).
-template <int G, int MAXE, int VEC, bool CACHED, bool SPARSE, bool SHIFTED = false>
+template <int G, int MAXE, int VEC, bool CACHED, bool SPARSE, bool SHIFTED = false, bool NT = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const float* __restrict__ logits,
                                                                          const float* __restrict__ target,
                                                                          float* __restrict__ grad, float* __restrict__ rowLoss,
@@ -92,11 +92,29 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
     // masked form (sparse targets only): maskInfo[1] = 1 / (number of rows whose index is not -1) replaces 1 / rows,
     // and a row with index -1 contributes nothing: zero gradient, zero loss
     if (SPARSE && maskInfo != nullptr) invRows = maskInfo[1];
-    for (size_t row = size_t(blockIdx.x) * rowsPerBlock + threadIdx.x / G; row < rows; row += rowStep) {
+    // Rows that leave room for a second copy in registers (MAXE <= 32) run on a grid of two waves of blocks per SIMD that
+    // walks the rows: the next row's loads are issued before the current row is reduced, so they are in flight during
+    // its two block-wide reductions and its stores (8192 x 32000: 0.405 -> 0.367 ms together with the streaming hint).
+    constexpr bool AHEAD = CACHED && MAXE <= 32;
+    RowCache<G, AHEAD ? MAXE : VEC, VEC, NT> ahead;
+    const size_t firstRow = size_t(blockIdx.x) * rowsPerBlock + threadIdx.x / G;
+    auto fetch = [&](auto& into, size_t r) __attribute__((always_inline)) {
+        const float* src = logits + r * classes;
+        if constexpr (SHIFTED) into.loadShifted(src, classes, t, -INFINITY, RowCache<G, MAXE, VEC, NT>::shiftOf(src));
+        else into.load(src, classes, t, -INFINITY);
+    };
+    if constexpr (AHEAD) { if (firstRow < rows) fetch(ahead, firstRow); }
+    for (size_t row = firstRow; row < rows; row += rowStep) {
         const float* x = logits + row * classes;
         float* gOut = grad + row * classes;
-        RowCache<G, MAXE, VEC> c;
-        const int shift = SHIFTED ? RowCache<G, MAXE, VEC>::shiftOf(x) : 0;   // the same for gOut: the host checks that
+        RowCache<G, MAXE, VEC, NT> c;
+        if constexpr (AHEAD) {
+            c = ahead;
+            if (row + rowStep < rows) fetch(ahead, row + rowStep);
+        } else if constexpr (CACHED) {
+            fetch(c, row);
+        }
+        const int shift = SHIFTED ? RowCache<G, MAXE, VEC, NT>::shiftOf(x) : 0;   // the same for gOut: the host checks that
         auto storeRow = [&]() __attribute__((always_inline)) {
             if constexpr (SHIFTED) c.storeShifted(gOut, classes, t, shift);
             else c.store(gOut, classes, t);
@@ -116,8 +134,6 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
         }
         float mx = -INFINITY;
         if constexpr (CACHED) {
-            if constexpr (SHIFTED) c.loadShifted(x, classes, t, -INFINITY, shift);
-            else c.load(x, classes, t, -INFINITY);
 #pragma unroll
             for (int i = 0; i < MAXE; ++i) mx = fmaxf(mx, c.r[i]);
         } else {
@@ -176,7 +192,7 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                 for (int it = 0; it < MAXE / VEC; ++it)
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) {
-                        const long idx = long(RowCache<G, MAXE, VEC>::index(it, t, j)) - shift;
+                        const long idx = long(RowCache<G, MAXE, VEC, NT>::index(it, t, j)) - shift;
                         if (idx >= 0 && size_t(idx) < classes) c.r[it * VEC + j] = emit(c.r[it * VEC + j], size_t(idx));
                     }
                 storeRow();
@@ -206,12 +222,16 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
     // rows that are not 16-byte aligned still get 16-byte accesses (shifted) as long as a logits row and its gradient
     // row sit at the same offset within a 16-byte group; a row must then fit its registers with up to 3 elements to spare
     const bool shifted = !vec4 && ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad)) & 15u) == 0;
+    const bool streaming = streamsPastCache(rows * classes * (SPARSE ? 8 : 12));   // logits in, gradient out (and a dense target in)
     // smallest group and register count that hold a row (see the row kernels); a block takes its rows once
 #define BF_CE(G, MAXE)                                                                                            \
     if (classes + (vec4 ? 0 : 3) <= size_t(G) * MAXE && (vec4 || shifted || MAXE <= 32)) {                        \
         const unsigned threads = G > 256 ? G : 256;                                                               \
-        const unsigned grid = gridFor(rows, threads / G);                                                         \
-        if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
+        const bool nt = streaming && MAXE <= 32;   /* measured: the hint only pays together with the look-ahead */ \
+        const unsigned grid = gridFor(rows, threads / G, MAXE <= 32 ? unsigned(computeUnits()) * (2048 / threads) : kMaxGridX); \
+        if (vec4 && nt) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
+        else if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
+        else if (shifted && nt) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
         else if (shifted) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
         else crossEntropyKernel<G, (MAXE <= 32 ? MAXE : 4), 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); /* plans above 32 registers have no one-element form */ \
         break;                                                                                                    \
@@ -248,7 +268,9 @@ int bf_hip_mse(const float* pred, const float* target, float* grad, float* lossS
     Scratch partial(grid * sizeof(float));
     if (partial.status != BF_OK) return partial.status;
     float gradScale = 2.0f / float(n);
-    if (aligned16(pred) && aligned16(target) && aligned16(grad))
+    if (aligned16(pred) && aligned16(target) && aligned16(grad) && streamsPastCache(n * 12))
+        mseKernel<4, true><<<grid, kBlock, 0, s>>>(pred, target, grad, partial.as<float>(), n, gradScale);
+    else if (aligned16(pred) && aligned16(target) && aligned16(grad))
         mseKernel<4><<<grid, kBlock, 0, s>>>(pred, target, grad, partial.as<float>(), n, gradScale);
     else
         mseKernel<1><<<grid, kBlock, 0, s>>>(pred, target, grad, partial.as<float>(), n, gradScale);

@@ -33,13 +33,14 @@ struct AdamTensor {
     unsigned pad;
 };
 
+template <bool NT>
 __global__ void __launch_bounds__(kBlock) sgdKernel(const SgdTensor* __restrict__ table, int numTensors, float lr) {
     const SgdTensor c = table[owningTensor(table, numTensors, blockIdx.x)];
     const size_t base = (size_t(blockIdx.x - c.firstBlock) * kBlock + threadIdx.x) * 4;
     if (base >= c.count) return;
     const bool vec = ((reinterpret_cast<uintptr_t>(c.p) | reinterpret_cast<uintptr_t>(c.g)) & 15u) == 0 && base + 4 <= c.count;
     if (vec) {
-        storef4(c.p + base, loadf4(c.p + base) - loadf4(c.g + base) * lr);
+        stf4<NT>(c.p + base, ldf4<NT>(c.p + base) - ldf4<NT>(c.g + base) * lr);
     } else {
         for (size_t i = base; i < base + 4 && i < c.count; ++i) c.p[i] -= lr * c.g[i];
     }
@@ -57,6 +58,7 @@ __device__ __forceinline__ void adamOne(float& p, float g, float& m, float& v, c
     p -= a.lr * (mHat / (sqrtf(vHat) + a.eps) + a.weightDecay * p);
 }
 
+template <bool NT>
 __global__ void __launch_bounds__(kBlock) adamwKernel(const AdamTensor* __restrict__ table, int numTensors, AdamParams a) {
     const AdamTensor c = table[owningTensor(table, numTensors, blockIdx.x)];
     const size_t base = (size_t(blockIdx.x - c.firstBlock) * kBlock + threadIdx.x) * 4;
@@ -64,16 +66,16 @@ __global__ void __launch_bounds__(kBlock) adamwKernel(const AdamTensor* __restri
     const bool vec = ((reinterpret_cast<uintptr_t>(c.p) | reinterpret_cast<uintptr_t>(c.g) | reinterpret_cast<uintptr_t>(c.m) |
                        reinterpret_cast<uintptr_t>(c.v)) & 15u) == 0 && base + 4 <= c.count;
     if (vec) {
-        float4v p = loadf4(c.p + base), g = loadf4(c.g + base), m = loadf4(c.m + base), v = loadf4(c.v + base);
+        float4v p = ldf4<NT>(c.p + base), g = ldf4<NT>(c.g + base), m = ldf4<NT>(c.m + base), v = ldf4<NT>(c.v + base);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             float pj = p[j], mj = m[j], vj = v[j];
             adamOne(pj, g[j], mj, vj, a);
             p[j] = pj; m[j] = mj; v[j] = vj;
         }
-        storef4(c.p + base, p);
-        storef4(c.m + base, m);
-        storef4(c.v + base, v);
+        stf4<NT>(c.p + base, p);
+        stf4<NT>(c.m + base, m);
+        stf4<NT>(c.v + base, v);
     } else {
         for (size_t i = base; i < base + 4 && i < c.count; ++i) adamOne(c.p[i], c.g[i], c.m[i], c.v[i], a);
     }
@@ -102,7 +104,8 @@ int bf_hip_sgd_multi(float* const* params, const float* const* grads, const size
     const void* device = nullptr;
     int st = uploadDescriptorTable(kSlotSgd, table.data(), table.size() * sizeof(SgdTensor), asStream(stream), &device);
     if (st != BF_OK) return st;
-    sgdKernel<<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const SgdTensor*>(device), int(numTensors), lr);
+    if (streamsPastCache(blocks * kPerBlock * 12)) sgdKernel<true><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const SgdTensor*>(device), int(numTensors), lr);
+    else sgdKernel<false><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const SgdTensor*>(device), int(numTensors), lr);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -128,7 +131,8 @@ int bf_hip_adamw_multi(float* const* params, const float* const* grads, float* c
     // bias corrections on the host in float, exactly like the reference (optimizer.cu:104-107)
     float t = static_cast<float>(step);
     AdamParams a{lr, beta1, beta2, eps, weightDecay, 1.0f - std::pow(beta1, t), 1.0f - std::pow(beta2, t)};
-    adamwKernel<<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const AdamTensor*>(device), int(numTensors), a);
+    if (streamsPastCache(blocks * kPerBlock * 28)) adamwKernel<true><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const AdamTensor*>(device), int(numTensors), a);
+    else adamwKernel<false><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const AdamTensor*>(device), int(numTensors), a);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

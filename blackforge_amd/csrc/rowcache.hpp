@@ -17,7 +17,8 @@ namespace bf {
 
 #if defined(__HIPCC__)
 
-template <int G, int MAXE, int VEC>
+// NT: accesses carry the non-temporal hint (rows streamed past the last-level cache, see ldf4 / stf4).
+template <int G, int MAXE, int VEC, bool NT = false>
 struct RowCache {
     static constexpr int kIters = MAXE / VEC;
     float r[MAXE];
@@ -31,13 +32,13 @@ struct RowCache {
             size_t e = index(it, t, 0);
             if constexpr (VEC == 4) {
                 if (e < features) {
-                    float4v v = loadf4(row + e);
+                    float4v v = ldf4<NT>(row + e);
                     r[it * 4 + 0] = v.x; r[it * 4 + 1] = v.y; r[it * 4 + 2] = v.z; r[it * 4 + 3] = v.w;
                 } else {
                     r[it * 4 + 0] = r[it * 4 + 1] = r[it * 4 + 2] = r[it * 4 + 3] = fill;
                 }
             } else {
-                r[it] = e < features ? row[e] : fill;
+                r[it] = e < features ? ldf1<NT>(row + e) : fill;
             }
         }
     }
@@ -56,7 +57,7 @@ struct RowCache {
 #pragma unroll
         for (int it = 0; it < kIters; ++it) {
             const int g = (it * G + t) * 4;
-            const float4v v = loadf4(base + (g < last ? g : 0));
+            const float4v v = ldf4<NT>(base + (g < last ? g : 0));
             r[it * 4 + 0] = v.x; r[it * 4 + 1] = v.y; r[it * 4 + 2] = v.z; r[it * 4 + 3] = v.w;
         }
         const int lo = t == 0 ? shift : 0;   // slots of thread 0's first group that belong to the row before
@@ -79,7 +80,7 @@ struct RowCache {
             if (g < last) {
                 const bool head = it == 0 && t == 0 && shift > 0, tail = g + 4 > last;
                 if (!head && !tail) {
-                    storef4(base + g, float4v{r[it * 4 + 0], r[it * 4 + 1], r[it * 4 + 2], r[it * 4 + 3]});
+                    stf4<NT>(base + g, float4v{r[it * 4 + 0], r[it * 4 + 1], r[it * 4 + 2], r[it * 4 + 3]});
                 } else {   // a group that straddles an end of the row: its own elements one by one
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
@@ -96,9 +97,9 @@ struct RowCache {
             if (e < features) {
                 if constexpr (VEC == 4) {
                     float4v v = {r[it * 4 + 0], r[it * 4 + 1], r[it * 4 + 2], r[it * 4 + 3]};
-                    storef4(row + e, v);
+                    stf4<NT>(row + e, v);
                 } else {
-                    row[e] = r[it];
+                    stf1<NT>(row + e, r[it]);
                 }
             }
         }

@@ -14,9 +14,9 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 constexpr float kRmsNormEps = 1e-6f;
 
 // Visits the row either from the register cache or (CACHED == false) from global memory.
-template <int G, int MAXE, int VEC, bool CACHED>
+template <int G, int MAXE, int VEC, bool CACHED, bool NT = false>
 struct Row {
-    RowCache<G, MAXE, VEC> c;
+    RowCache<G, MAXE, VEC, NT> c;
     const float* p;
     size_t n;
     int t;
@@ -40,7 +40,7 @@ struct Row {
             for (int it = 0; it < MAXE / VEC; ++it)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
-                    size_t e = RowCache<G, MAXE, VEC>::index(it, t, j);
+                    size_t e = RowCache<G, MAXE, VEC, NT>::index(it, t, j);
                     if (e < n) f(c.r[it * VEC + j], e);
                 }
         } else {
@@ -54,7 +54,7 @@ struct Row {
             for (int it = 0; it < MAXE / VEC; ++it)
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) {
-                    size_t e = RowCache<G, MAXE, VEC>::index(it, t, j);
+                    size_t e = RowCache<G, MAXE, VEC, NT>::index(it, t, j);
                     c.r[it * VEC + j] = f(c.r[it * VEC + j], e);
                 }
             c.store(out, n, t);
@@ -76,12 +76,12 @@ struct Row {
 // When a whole block shares a row (G > 64) every thread must take part in the LDS reductions, so
 // the row loop is uniform across the block: rowsPerBlock == 1 there.
 
-template <int G, int MAXE, int VEC, bool CACHED>
+template <int G, int MAXE, int VEC, bool CACHED, bool NT = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormKernel(const float* __restrict__ x, float* __restrict__ out,
                                                                     size_t rows, size_t features) {
     BF_ROW_PROLOGUE();
     for (size_t row = firstRow; row < rows; row += rowStep) {
-        Row<G, MAXE, VEC, CACHED> rx;
+        Row<G, MAXE, VEC, CACHED, NT> rx;
         rx.open(x + row * features, features, t, 0.0f);
         // sum of squares in double and x / rms in float, as the reference does (ops.cpp:264-275)
         double ss = 0.0;
@@ -92,13 +92,13 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormKernel(const float* 
     }
 }
 
-template <int G, int MAXE, int VEC, bool CACHED>
+template <int G, int MAXE, int VEC, bool CACHED, bool NT = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const float* __restrict__ x, const float* __restrict__ g,
                                                                             const float* __restrict__ addend, float* __restrict__ out,
                                                                             size_t rows, size_t features) {
     BF_ROW_PROLOGUE();
     for (size_t row = firstRow; row < rows; row += rowStep) {
-        Row<G, MAXE, VEC, CACHED> rx, rg;
+        Row<G, MAXE, VEC, CACHED, NT> rx, rg;
         rx.open(x + row * features, features, t, 0.0f);
         rg.open(g + row * features, features, t, 0.0f);
         // double sums and a double final formula, as the reference does (autodiff.cpp:212-229): the two
@@ -141,12 +141,12 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const
     }
 }
 
-template <int G, int MAXE, int VEC, bool CACHED>
+template <int G, int MAXE, int VEC, bool CACHED, bool NT = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) softmaxKernel(const float* __restrict__ x, float* __restrict__ out,
                                                                     size_t rows, size_t features) {
     BF_ROW_PROLOGUE();
     for (size_t row = firstRow; row < rows; row += rowStep) {
-        Row<G, MAXE, VEC, CACHED> rx;
+        Row<G, MAXE, VEC, CACHED, NT> rx;
         rx.open(x + row * features, features, t, -INFINITY);
         float mx = -INFINITY;
         rx.reduce([&](float v) { mx = fmaxf(mx, v); });
@@ -172,12 +172,12 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) softmaxKernel(const float* 
 }
 
 // dx = y * (g - sum(g*y)) with y = softmax(x) recomputed in registers.
-template <int G, int MAXE, int VEC, bool CACHED>
+template <int G, int MAXE, int VEC, bool CACHED, bool NT = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) softmaxBackwardKernel(const float* __restrict__ x, const float* __restrict__ g,
                                                                             float* __restrict__ out, size_t rows, size_t features) {
     BF_ROW_PROLOGUE();
     for (size_t row = firstRow; row < rows; row += rowStep) {
-        Row<G, MAXE, VEC, CACHED> rx, rg;
+        Row<G, MAXE, VEC, CACHED, NT> rx, rg;
         rx.open(x + row * features, features, t, -INFINITY);
         rg.open(g + row * features, features, t, 0.0f);
         float mx = -INFINITY;
@@ -214,7 +214,8 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) softmaxBackwardKernel(const
     if ((features_) <= size_t(G) * MAXE) {                                                                         \
         const unsigned threads = G > 256 ? G : 256;                                                                \
         const unsigned grid = gridFor(rows_, threads / G);                                                         \
-        if (vec4) KERNEL<G, MAXE, 4, true><<<grid, threads, 0, stream_>>>(ARGS_);                                  \
+        if (vec4 && nt_) KERNEL<G, MAXE, 4, true, true><<<grid, threads, 0, stream_>>>(ARGS_);                      \
+        else if (vec4) KERNEL<G, MAXE, 4, true><<<grid, threads, 0, stream_>>>(ARGS_);                             \
         else KERNEL<G, MAXE, 1, true><<<grid, threads, 0, stream_>>>(ARGS_);                                       \
         break;                                                                                                     \
     }
@@ -223,6 +224,7 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) softmaxBackwardKernel(const
         const size_t rows_ = (rows), features_ = (features);                                                       \
         hipStream_t stream_ = (stream);                                                                            \
         const bool vec4 = (vecOk) && features_ % 4 == 0;                                                           \
+        const bool nt_ = !(TWO_INPUTS) && streamsPastCache(rows_ * features_ * 8);   /* measured: no gain with two inputs */ \
         BF_ROW_CASE(KERNEL, 64, 4, 0)                                                                              \
         BF_ROW_CASE(KERNEL, 64, 8, 0)                                                                              \
         BF_ROW_CASE(KERNEL, 64, 16, 0)                                                                             \

@@ -25,6 +25,46 @@ def test_embedding_gather_and_scatter_are_bit_exact(hip, oracle, rng, batch, seq
                       oracle.embeddingLookupBackward(ids, g, vocab))
 
 
+@pytest.mark.parametrize("tokens,vocab,dim,hot", [(8192, 32000, 64, 0), (8192, 300, 32, 3000), (16384, 50257, 16, 5000), (70000, 1000, 8, 100),
+                                                  (500, 200001, 4, 50), (65535, 76800, 4, 0), (16384, 8192, 1028, 0), (777, 5000, 770, 30), (300, 4000, 7, 4)])
+def test_embedding_scatter_routes(hip, oracle, tokens, vocab, dim, hot):
+    """The route without a sort (up to 16384 tokens against a table at least half as large: one wavefront per token, the
+    first token of an id sums its row) and the counting-sort route (more tokens, or a small table), with an id that `hot`
+    tokens share: every route sums in token order, so the result is the CPU loop's bit for bit."""
+    rng = np.random.default_rng(tokens + vocab)
+    D, ops = hip.DeviceTensor, hip.ops
+    ids = rng.integers(0, vocab, (1, tokens)).astype(f32)
+    if hot:
+        ids[0, rng.choice(tokens, hot, replace=False)] = 7 % vocab
+    ids[0, -1] = vocab - 1
+    g = r(rng, 1, tokens, dim)
+    assert_bits_equal(ops.embeddingLookupBackwardPreValidated(D.fromHost(ids), D.fromHost(g), vocab).toHost(),
+                      oracle.embeddingLookupBackward(ids, g, vocab))
+
+
+def test_embedding_ids_outside_the_table_touch_nothing(hip, oracle, rng):
+    """The pre-validated entry points trust their caller; an id outside [0, vocab) must still not read or write outside
+    the tensors: the lookup gives zeros for it and the gradient ignores it (both routes of the sort)."""
+    D, ops = hip.DeviceTensor, hip.ops
+    vocab, dim = 50, 12
+    for tokens in (40, 70000):
+        ids = rng.integers(0, vocab, (1, tokens)).astype(f32)
+        bad = np.array([3, 11, tokens - 1])
+        ids[0, bad] = [-1.0, float(vocab), 1e9]
+        table, g = r(rng, vocab, dim), r(rng, 1, tokens, dim)
+        out = ops.embeddingLookupPreValidated(D.fromHost(ids), D.fromHost(table)).toHost()
+        good = np.ones(tokens, bool)
+        good[bad] = False
+        clipped = np.where(good, ids[0], 0).astype(f32)[None]
+        expected = oracle.embeddingLookup(clipped, table)
+        expected[0, bad] = 0
+        assert_bits_equal(out, expected)
+        gz = g.copy()
+        gz[0, bad] = 0   # the ignored tokens contribute nothing; their stand-in id 0 then only adds zeros
+        assert_bits_equal(ops.embeddingLookupBackwardPreValidated(D.fromHost(ids), D.fromHost(g), vocab).toHost(),
+                          oracle.embeddingLookupBackward(clipped, gz, vocab))
+
+
 def test_embedding_reference_literals_and_range_errors(hip):
     """tests/backend/cpu/ops_tests.cpp:238-262, autodiff_tests.cpp:180-199, cuda/ops_tests.cu:300-306."""
     D, ops = hip.DeviceTensor, hip.ops
