@@ -72,6 +72,8 @@ SIGNATURES = {
     "bf_hip_rmsnorm": [P, P, c_size, c_size, S],
     "bf_hip_rmsnorm_backward": [P, P, P, c_size, c_size, S],
     "bf_hip_rmsnorm_backward_add": [P, P, P, P, c_size, c_size, S],
+    "bf_hip_rmsnorm_img": [P, P, P, c_size, c_size, S],
+    "bf_hip_rmsnorm_backward_add_img": [P, P, P, P, P, c_size, c_size, S],
     "bf_hip_softmax": [P, P, c_size, c_size, S],
     "bf_hip_softmax_backward": [P, P, P, c_size, c_size, S],
     "bf_hip_bias_grad": [P, P, c_size, c_size, S],
@@ -96,8 +98,17 @@ SIGNATURES = {
                                                  c_size, c_size, c_size, c_int, S],
     "bf_hip_feedforward_bf16": [P, P, P, P, P, P, c_int, P, P, P, P, c_size, c_size, c_size, c_int, S],
     "bf_hip_feedforward_bf16_backward": [P, P, P, P, P, P, P, c_int, P, P, P, P, P, c_size, c_size, c_size, c_int, S],
+    "bf_hip_linear_bf16_img": [P, P, P, P, P, P, c_size, c_size, c_size, c_int, S],
+    "bf_hip_matmul_bf16_backward_img": [P, P, P, P, P, P, P, c_size, c_size, c_size, c_int, S],
+    "bf_hip_matmul_bf16_shared_input_img": [P, P, ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), c_size, c_size, c_size, c_size, c_int, S],
+    "bf_hip_matmul_bf16_shared_input_backward_img": [P, P, ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), P, P, ctypes.POINTER(c_ptr), c_size,
+                                                     c_size, c_size, c_size, c_int, S],
+    "bf_hip_feedforward_bf16_backward_img": [P, P, P, P, P, P, P, P, c_int, P, P, P, P, P, c_size, c_size, c_size, c_int, S],
     "bf_hip_invalidate_bf16_weight_cache": [],
     "bf_hip_attention_forward": [P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
+    "bf_hip_attention_forward_img": [P, P, P, P, P, c_size, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
+    "bf_hip_attention_backward_img": [P, P, P, P, P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_size, c_float,
+                                      c_size, S],
     "bf_hip_attention_dot_o_do": [P, P, P, c_size, c_size, c_size, c_size, S],
     "bf_hip_attention_backward": [P, P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float,
                                   c_size, S],
@@ -111,6 +122,7 @@ SIGNATURES = {
     "bf_hip_mse": [P, P, P, P, c_size, c_int, S],
     "bf_hip_cross_entropy": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse": [P, P, P, P, c_size, c_size, c_int, S],
+    "bf_hip_cross_entropy_sparse_img": [P, P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_masked": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_sgd_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_size), c_size, c_float, S],
     "bf_hip_adamw_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr),

@@ -44,6 +44,11 @@ struct AttnParams {
     const float* dvec;   // [batch, heads, newLen]: dot(O, dO)
     float* out; float* m; float* l;
     float* dQ; float* dK; float* dV;
+    // bf16 images (rounded to nearest even) of the outputs, for consumers that are bf16 GEMMs: row r of a [rows, dim]
+    // output lies at img + r * imgLd (imgLd >= dim, so that dQ, dK and dV can be column slices of one wider image).
+    // Each is optional; with an image given the fp32 tensor of the same output may be NULL.
+    unsigned short* outImg; unsigned short* dQImg; unsigned short* dKImg; unsigned short* dVImg;
+    size_t imgLd;
     float* ds;           // [batch*heads, nqb, nkb, 32 queries, 32 keys]: dS sub-blocks handed from dK/dV to dQ (or null)
     int nqb, nkb;        // query / key sub-blocks of 32 per (batch, head)
     int batch, heads, newLen, totalLen, dim, hd, oldLen;
@@ -213,6 +218,31 @@ __device__ __forceinline__ void storeTransposed(float* __restrict__ dst, const f
         }
 }
 
+// The same accumulator as a row of a bf16 image: four consecutive head-dim elements are one 8-byte store.
+template <int HDP, bool VEC4>
+__device__ __forceinline__ void storeTransposedBf16(unsigned short* __restrict__ dst, const float16v (&acc)[HDP / 32], int hd, int half,
+                                                    float mul) {
+#pragma unroll
+    for (int dt = 0; dt < HDP / 32; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            int d = dt * 32 + 8 * g + 4 * half;
+            if (d < hd) {
+                const unsigned short b0 = toBf16Bits(acc[dt][4 * g] * mul), b1 = toBf16Bits(acc[dt][4 * g + 1] * mul),
+                                     b2 = toBf16Bits(acc[dt][4 * g + 2] * mul), b3 = toBf16Bits(acc[dt][4 * g + 3] * mul);
+                if constexpr (VEC4) {
+                    const uint2v packed = {unsigned(b0) | unsigned(b1) << 16, unsigned(b2) | unsigned(b3) << 16};
+                    *reinterpret_cast<uint2v*>(dst + d) = packed;
+                } else {
+                    dst[d] = b0;
+                    if (d + 1 < hd) dst[d + 1] = b1;
+                    if (d + 2 < hd) dst[d + 2] = b2;
+                    if (d + 3 < hd) dst[d + 3] = b3;
+                }
+            }
+        }
+}
+
 // ---------------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------------
@@ -355,7 +385,8 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnForwardKernel(Att
 
     lrow += __shfl_xor(lrow, 32, 64);
     if (rowValid) {
-        storeTransposed<HDP, VEC4>(p.out + (size_t(b) * p.newLen + i) * dim + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
+        if (p.out) storeTransposed<HDP, VEC4>(p.out + (size_t(b) * p.newLen + i) * dim + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
+        if (p.outImg) storeTransposedBf16<HDP, VEC4>(p.outImg + (size_t(b) * p.newLen + i) * p.imgLd + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
         if (half == 0) {
             // statistics about the TRUE row maximum: l = sum exp(score - m) = (sum about mref) * 2^(mref - mrow)
             size_t idx = (size_t(b) * p.heads + h) * p.newLen + i;
@@ -512,7 +543,10 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnBackwardDqKernel(A
         }
         __syncthreads();
     }
-    if (rowValid) storeTransposed<HDP, VEC4>(p.dQ + qOff + size_t(i) * dim, acc, hd, half, p.scale);
+    if (rowValid) {
+        if (p.dQ) storeTransposed<HDP, VEC4>(p.dQ + qOff + size_t(i) * dim, acc, hd, half, p.scale);
+        if (p.dQImg) storeTransposedBf16<HDP, VEC4>(p.dQImg + (size_t(b) * p.newLen + i) * p.imgLd + size_t(h) * hd, acc, hd, half, p.scale);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -615,7 +649,10 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 3 : HDP <= 128 ? 2 : 1) attnB
         }
         __syncthreads();
     }
-    if (i < p.newLen) storeTransposed<HDP, VEC4>(p.dQ + qOff + size_t(i) * dim, acc, hd, half, p.scale);
+    if (i < p.newLen) {
+        if (p.dQ) storeTransposed<HDP, VEC4>(p.dQ + qOff + size_t(i) * dim, acc, hd, half, p.scale);
+        if (p.dQImg) storeTransposedBf16<HDP, VEC4>(p.dQImg + (size_t(b) * p.newLen + i) * p.imgLd + size_t(h) * hd, acc, hd, half, p.scale);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -783,6 +820,9 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
     }
 
     // dk/dv[dt][r]: key = waveK0 + dRow(r, half), d = dt*32 + li  -> 128-byte coalesced rows
+    const bool images = p.dKImg != nullptr || p.dVImg != nullptr;
+    // with an even head dim, row pitch and base every even column of an image row is 4-byte aligned and has its neighbour
+    const bool pairs = (hd & 1) == 0 && (p.imgLd & 1u) == 0 && ((reinterpret_cast<uintptr_t>(p.dKImg) | reinterpret_cast<uintptr_t>(p.dVImg)) & 3u) == 0;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
         const int d = dt * 32 + li;
@@ -791,8 +831,22 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
             for (int r = 0; r < 16; ++r) {
                 const int kk = waveK0 + dRow(r, half);
                 if (kk < p.totalLen) {
-                    p.dK[kOff + size_t(kk) * dim + d] = dk[dt][r] * p.scale;
-                    p.dV[kOff + size_t(kk) * dim + d] = dv[dt][r];
+                    const float dkv = dk[dt][r] * p.scale, dvv = dv[dt][r];
+                    if (p.dK) p.dK[kOff + size_t(kk) * dim + d] = dkv;
+                    if (p.dV) p.dV[kOff + size_t(kk) * dim + d] = dvv;
+                    if (images) {
+                        const size_t at = (size_t(b) * p.totalLen + kk) * p.imgLd + size_t(h) * hd + d;
+                        if (pairs) {   // lanes 2i and 2i+1 hold neighbouring columns: lane 2i stores both, four bytes at once
+                            const float dkNext = __shfl_down(dkv, 1, 64), dvNext = __shfl_down(dvv, 1, 64);
+                            if ((li & 1) == 0) {
+                                if (p.dKImg) *reinterpret_cast<unsigned*>(p.dKImg + at) = unsigned(toBf16Bits(dkv)) | unsigned(toBf16Bits(dkNext)) << 16;
+                                if (p.dVImg) *reinterpret_cast<unsigned*>(p.dVImg + at) = unsigned(toBf16Bits(dvv)) | unsigned(toBf16Bits(dvNext)) << 16;
+                            }
+                        } else {
+                            if (p.dKImg) p.dKImg[at] = toBf16Bits(dkv);
+                            if (p.dVImg) p.dVImg[at] = toBf16Bits(dvv);
+                        }
+                    }
                 }
             }
         }
@@ -895,20 +949,41 @@ using namespace bf;
 
 extern "C" {
 
-int bf_hip_attention_forward(const float* q, const float* k, const float* v, float* out, float* m, float* l,
-                             size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
-                             size_t oldLen, bf_stream_t stream) {
+static int checkImages(const char* fn, std::initializer_list<const void*> images, size_t imageLd, size_t dim) {
+    bool any = false;
+    for (const void* img : images) {
+        any = any || img != nullptr;
+        if (reinterpret_cast<uintptr_t>(img) & 15u) return failInvalid(fn, "bf16 images must be 16-byte aligned");
+    }
+    if (any && (imageLd < dim || imageLd % 8 != 0 || dim % 8 != 0))
+        return failInvalid(fn, "bf16 images need dim and the image row pitch to be multiples of 8, and a pitch of at least dim");
+    return BF_OK;
+}
+
+int bf_hip_attention_forward_img(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
+                                 float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
+                                 size_t oldLen, bf_stream_t stream) {
     int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
     if (st != BF_OK) return st;
     if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
-    BF_REQUIRE(q && k && v && out && m && l, "NULL pointer");
+    BF_REQUIRE(q && k && v && (out || outImage) && m && l, "NULL pointer");
+    st = checkImages(__func__, {outImage}, imageLd, dim);
+    if (st != BF_OK) return st;
     AttnParams p{};
+    p.outImg = outImage; p.imgLd = imageLd;
     p.q = q; p.k = k; p.v = v; p.out = out; p.m = m; p.l = l;
     p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(totalLen);
     p.dim = int(dim); p.hd = int(dim / heads); p.oldLen = int(oldLen); p.scale = scale;
     p.numTiles = int((newLen + 127) / 128);
     unsigned grid = unsigned(batch * heads * size_t(p.numTiles));
     return dispatch<0>(p, vec4Ok(p, {q, k, v, out}), grid, asStream(stream));
+}
+
+int bf_hip_attention_forward(const float* q, const float* k, const float* v, float* out, float* m, float* l,
+                             size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
+                             size_t oldLen, bf_stream_t stream) {
+    if (batch != 0 && newLen != 0 && dim != 0) BF_REQUIRE(out != nullptr, "NULL pointer");
+    return bf_hip_attention_forward_img(q, k, v, out, nullptr, 0, m, l, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
 }
 
 int bf_hip_attention_dot_o_do(const float* out, const float* dOut, float* D, size_t batch, size_t heads, size_t newLen,
@@ -951,24 +1026,44 @@ int bf_hip_attention_backward_prepare(const float* out, const float* dOut, const
     return BF_OK;
 }
 
-int bf_hip_attention_backward_dkv(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
-                                  const float* D, float* dK, float* dV, size_t batch, size_t heads, size_t newLen,
-                                  size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
-    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+// bf16 images of the gradients (each optional; with an image the fp32 tensor of the same gradient may be NULL)
+struct GradImages {
+    uint16_t* dQ = nullptr;
+    uint16_t* dK = nullptr;
+    uint16_t* dV = nullptr;
+    size_t ld = 0;
+};
+
+// dK, dV from the key-tile owner; dS != NULL also leaves the dS sub-blocks behind for dqFromDs
+static int dkvStage(const char* fn, const float* dOut, const float* q, const float* k, const float* v, const float* lse2, const float* D,
+                    float* dK, float* dV, float* dS, const GradImages& img, size_t batch, size_t heads, size_t newLen, size_t totalLen,
+                    size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
+    int st = checkShapes(fn, batch, heads, newLen, totalLen, dim, oldLen);
     if (st != BF_OK) return st;
     if (batch == 0 || dim == 0 || totalLen == 0) return BF_OK;
-    BF_REQUIRE(dK && dV, "NULL pointer");
+    if (!(dK || img.dK) || !(dV || img.dV)) return failInvalid(fn, "NULL pointer");
     if (newLen == 0) {   // no query: key/value gradients are zero
+        if (img.dK || img.dV) return failInvalid(fn, "bf16 gradient images need at least one query row");
         st = bf_hip_fill_zero(dK, batch * totalLen * dim * sizeof(float), stream);
         if (st != BF_OK) return st;
         return bf_hip_fill_zero(dV, batch * totalLen * dim * sizeof(float), stream);
     }
-    BF_REQUIRE(dOut && q && k && v && lse2 && D, "NULL pointer");
+    if (!(dOut && q && k && v && lse2 && D)) return failInvalid(fn, "NULL pointer");
+    if (dS != nullptr && (reinterpret_cast<uintptr_t>(dS) & 15u) != 0) return failInvalid(fn, "dS must be 16-byte aligned");
     AttnParams p{};
-    p.q = q; p.k = k; p.v = v; p.dO = dOut; p.dK = dK; p.dV = dV; p.lse2 = lse2; p.dvec = D;
+    p.q = q; p.k = k; p.v = v; p.dO = dOut; p.dK = dK; p.dV = dV; p.lse2 = lse2; p.dvec = D; p.ds = dS;
+    p.dKImg = img.dK; p.dVImg = img.dV; p.imgLd = img.ld;
     fillParams(p, batch, heads, newLen, totalLen, dim, scale, oldLen);
     p.numTiles = int((totalLen + 127) / 128);
-    return dispatch<2>(p, vec4Ok(p, {q, k, v, dOut}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
+    const unsigned grid = unsigned(batch * heads * size_t(p.numTiles));
+    return dS ? dispatch<3>(p, vec4Ok(p, {q, k, v, dOut}), grid, asStream(stream)) : dispatch<2>(p, vec4Ok(p, {q, k, v, dOut}), grid, asStream(stream));
+}
+
+int bf_hip_attention_backward_dkv(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
+                                  const float* D, float* dK, float* dV, size_t batch, size_t heads, size_t newLen,
+                                  size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
+    if (batch != 0 && dim != 0 && totalLen != 0) BF_REQUIRE(dK && dV, "NULL pointer");
+    return dkvStage(__func__, dOut, q, k, v, lse2, D, dK, dV, nullptr, GradImages{}, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
 }
 
 int bf_hip_attention_ds_bytes(size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t* bytes) {
@@ -986,55 +1081,67 @@ int bf_hip_attention_backward_dkv_ds(const float* dOut, const float* q, const fl
                                      const float* D, float* dK, float* dV, float* dS, size_t batch, size_t heads,
                                      size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
                                      bf_stream_t stream) {
-    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
-    if (st != BF_OK) return st;
-    if (batch == 0 || dim == 0 || totalLen == 0) return BF_OK;
-    if (newLen == 0)
-        return bf_hip_attention_backward_dkv(dOut, q, k, v, lse2, D, dK, dV, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
-    BF_REQUIRE(dOut && q && k && v && lse2 && D && dK && dV && dS, "NULL pointer");
-    BF_REQUIRE((reinterpret_cast<uintptr_t>(dS) & 15u) == 0, "dS must be 16-byte aligned");
-    AttnParams p{};
-    p.q = q; p.k = k; p.v = v; p.dO = dOut; p.dK = dK; p.dV = dV; p.lse2 = lse2; p.dvec = D; p.ds = dS;
-    fillParams(p, batch, heads, newLen, totalLen, dim, scale, oldLen);
-    p.numTiles = int((totalLen + 127) / 128);
-    return dispatch<3>(p, vec4Ok(p, {q, k, v, dOut}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
+    if (batch != 0 && dim != 0 && totalLen != 0) BF_REQUIRE(dK && dV && (dS || newLen == 0), "NULL pointer");
+    return dkvStage(__func__, dOut, q, k, v, lse2, D, dK, dV, newLen == 0 ? nullptr : dS, GradImages{}, batch, heads, newLen, totalLen, dim,
+                    scale, oldLen, stream);
 }
+
+static int dqFromDsStage(const char* fn, const float* dS, const float* k, float* dQ, const GradImages& img, size_t batch, size_t heads,
+                         size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream);
 
 int bf_hip_attention_backward_dq_from_ds(const float* dS, const float* k, float* dQ, size_t batch, size_t heads, size_t newLen,
                                          size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
-    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+    if (batch != 0 && dim != 0 && newLen != 0) BF_REQUIRE(dQ != nullptr, "NULL pointer");
+    return dqFromDsStage(__func__, dS, k, dQ, GradImages{}, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+}
+
+static int dqFromDsStage(const char* fn, const float* dS, const float* k, float* dQ, const GradImages& img, size_t batch, size_t heads,
+                         size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
+    int st = checkShapes(fn, batch, heads, newLen, totalLen, dim, oldLen);
     if (st != BF_OK) return st;
     if (batch == 0 || dim == 0 || newLen == 0) return BF_OK;
-    BF_REQUIRE(dS && k && dQ, "NULL pointer");
-    BF_REQUIRE((reinterpret_cast<uintptr_t>(dS) & 15u) == 0, "dS must be 16-byte aligned");
+    if (!(dS && k && (dQ || img.dQ))) return failInvalid(fn, "NULL pointer");
+    if ((reinterpret_cast<uintptr_t>(dS) & 15u) != 0) return failInvalid(fn, "dS must be 16-byte aligned");
     AttnParams p{};
+    p.dQImg = img.dQ; p.imgLd = img.ld;
     p.k = k; p.dQ = dQ; p.ds = const_cast<float*>(dS);
     fillParams(p, batch, heads, newLen, totalLen, dim, scale, oldLen);
     p.numTiles = int((newLen + 127) / 128);
     return dispatch<4>(p, vec4Ok(p, {k, dQ}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
 }
 
-int bf_hip_attention_backward_dq(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
-                                 const float* D, float* dQ, size_t batch, size_t heads, size_t newLen, size_t totalLen,
-                                 size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
-    int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
+static int dqStage(const char* fn, const float* dOut, const float* q, const float* k, const float* v, const float* lse2, const float* D,
+                   float* dQ, const GradImages& img, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
+                   size_t oldLen, bf_stream_t stream) {
+    int st = checkShapes(fn, batch, heads, newLen, totalLen, dim, oldLen);
     if (st != BF_OK) return st;
     if (batch == 0 || dim == 0 || newLen == 0) return BF_OK;
-    BF_REQUIRE(dOut && q && k && v && lse2 && D && dQ, "NULL pointer");
+    if (!(dOut && q && k && v && lse2 && D && (dQ || img.dQ))) return failInvalid(fn, "NULL pointer");
     AttnParams p{};
     p.q = q; p.k = k; p.v = v; p.dO = dOut; p.dQ = dQ; p.lse2 = lse2; p.dvec = D;
+    p.dQImg = img.dQ; p.imgLd = img.ld;
     fillParams(p, batch, heads, newLen, totalLen, dim, scale, oldLen);
     p.numTiles = int((newLen + 127) / 128);
     return dispatch<1>(p, vec4Ok(p, {q, k, v, dOut, dQ}), unsigned(batch * heads * size_t(p.numTiles)), asStream(stream));
 }
 
-int bf_hip_attention_backward(const float* dOut, const float* q, const float* k, const float* v, const float* out,
-                              const float* m, const float* l, float* dQ, float* dK, float* dV, size_t batch,
-                              size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
-                              bf_stream_t stream) {
+int bf_hip_attention_backward_dq(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
+                                 const float* D, float* dQ, size_t batch, size_t heads, size_t newLen, size_t totalLen,
+                                 size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
+    if (batch != 0 && dim != 0 && newLen != 0) BF_REQUIRE(dQ != nullptr, "NULL pointer");
+    return dqStage(__func__, dOut, q, k, v, lse2, D, dQ, GradImages{}, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+}
+
+int bf_hip_attention_backward_img(const float* dOut, const float* q, const float* k, const float* v, const float* out, const float* m,
+                                  const float* l, float* dQ, float* dK, float* dV, uint16_t* dQImage, uint16_t* dKImage,
+                                  uint16_t* dVImage, size_t imageLd, size_t batch, size_t heads, size_t newLen, size_t totalLen,
+                                  size_t dim, float scale, size_t oldLen, bf_stream_t stream) {
     int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
     if (st != BF_OK) return st;
     if (batch == 0 || dim == 0) return BF_OK;
+    st = checkImages(__func__, {dQImage, dKImage, dVImage}, imageLd, dim);
+    if (st != BF_OK) return st;
+    const GradImages img{dQImage, dKImage, dVImage, imageLd};
     // workspace: lse2 | D, each [batch, heads, newLen]
     const size_t stats = batch * heads * newLen;
     Scratch work(2 * stats * sizeof(float));
@@ -1048,14 +1155,22 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
     Scratch ds(newLen > 0 && totalLen > 0 && handOver <= dsLimit() ? handOver : 0);
     if (ds.status != BF_OK) (void)hipGetLastError();   // no room for the buffer after all: recompute instead
     if (ds.status == BF_OK && ds.ptr != nullptr) {
-        st = bf_hip_attention_backward_dkv_ds(dOut, q, k, v, lse2, dvec, dK, dV, ds.as<float>(), batch, heads, newLen, totalLen, dim, scale,
-                                              oldLen, stream);
+        st = dkvStage(__func__, dOut, q, k, v, lse2, dvec, dK, dV, ds.as<float>(), img, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
         if (st != BF_OK) return st;
-        return bf_hip_attention_backward_dq_from_ds(ds.as<float>(), k, dQ, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+        return dqFromDsStage(__func__, ds.as<float>(), k, dQ, img, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
     }
-    st = bf_hip_attention_backward_dkv(dOut, q, k, v, lse2, dvec, dK, dV, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+    st = dkvStage(__func__, dOut, q, k, v, lse2, dvec, dK, dV, nullptr, img, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
     if (st != BF_OK) return st;
-    return bf_hip_attention_backward_dq(dOut, q, k, v, lse2, dvec, dQ, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+    return dqStage(__func__, dOut, q, k, v, lse2, dvec, dQ, img, batch, heads, newLen, totalLen, dim, scale, oldLen, stream);
+}
+
+int bf_hip_attention_backward(const float* dOut, const float* q, const float* k, const float* v, const float* out,
+                              const float* m, const float* l, float* dQ, float* dK, float* dV, size_t batch,
+                              size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
+                              bf_stream_t stream) {
+    if (batch != 0 && dim != 0) BF_REQUIRE((dQ || newLen == 0) && ((dK && dV) || totalLen == 0), "NULL pointer");
+    return bf_hip_attention_backward_img(dOut, q, k, v, out, m, l, dQ, dK, dV, nullptr, nullptr, nullptr, 0, batch, heads, newLen, totalLen, dim,
+                                         scale, oldLen, stream);
 }
 
 }  // extern "C"

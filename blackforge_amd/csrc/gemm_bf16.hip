@@ -1132,27 +1132,11 @@ int bf_hip_gemm_bf16_tn(const uint16_t* A, const uint16_t* B, float* C, size_t M
 
 int bf_hip_matmul_bf16(const float* a, const float* b, float* c, size_t m, size_t k, size_t n, int cacheWeight,
                        bf_stream_t stream) {
-    if (m == 0 || n == 0) return BF_OK;
-    BF_REQUIRE(c != nullptr, "NULL output");
-    if (k == 0) return bf_hip_fill_zero(c, m * n * sizeof(float), stream);
-    BF_REQUIRE(a && b, "NULL operand");
-    hipStream_t s = asStream(stream);
-    const size_t kp = pad8(k);
-    Scratch aImg(m * kp * sizeof(unsigned short));
-    if (aImg.status != BF_OK) return aImg.status;
-    int st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
-    if (st != BF_OK) return st;
-    unsigned short* bImg = nullptr;
-    size_t bBytes = 0;
-    st = weightImage(b, k, n, /*transposed=*/true, cacheWeight != 0, s, &bImg, &bBytes);
-    if (st != BF_OK) return st;
-    st = launchGemmNt(aImg.as<unsigned short>(), bImg, c, m, n, kp, kp, kp, s);
-    if (!cacheWeight) bf_hip_pool_release(bImg, bBytes);
-    return st;
+    return bf_hip_linear_bf16_img(a, nullptr, b, nullptr, nullptr, c, m, k, n, cacheWeight, stream);
 }
 
-int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, float* dA, float* dB, size_t m,
-                                size_t k, size_t n, int cacheWeight, bf_stream_t stream) {
+int bf_hip_matmul_bf16_backward_img(const float* a, const uint16_t* aImage, const float* b, const float* g, const uint16_t* gImage,
+                                    float* dA, float* dB, size_t m, size_t k, size_t n, int cacheWeight, bf_stream_t stream) {
     hipStream_t s = asStream(stream);
     if (m == 0 || k == 0 || n == 0) {   // degenerate: gradients are zero (ops_tensorcore.cu:412-415)
         int st = BF_OK;
@@ -1160,57 +1144,69 @@ int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, 
         if (st == BF_OK && dB && k * n) st = bf_hip_fill_zero(dB, k * n * sizeof(float), stream);
         return st;
     }
-    BF_REQUIRE(a && b && g, "NULL operand");
+    BF_REQUIRE((a || aImage || !dB) && b && (g || gImage), "NULL operand");
+    BF_REQUIRE(((reinterpret_cast<uintptr_t>(aImage) | reinterpret_cast<uintptr_t>(gImage)) & 15u) == 0, "operand images must be 16-byte aligned");
     int st = BF_OK;
     const size_t mp = pad8(m), np = pad8(n), kp = pad8(k);
     // dB = a^T g contracts over the rows of both operands.  When the product is big enough for the large-tile kernel
-    // that transposes fragments on their way out of LDS, both operands are converted as they lie (g's plain image also
+    // that transposes fragments on their way out of LDS, both operands are used as they lie (g's plain image also
     // serves dA); otherwise transposed images are built and the row-by-row kernel is used.
     int form = 0;
     size_t slices = 1;
     const bool transposeInLds = dB != nullptr && planLargeTiles(k, n, m, &form, &slices);
+    const bool needPlainG = dA || transposeInLds || (dB && !g);   // without the fp32 gradient its transposed image comes from the plain one
     Scratch gT(dB && !transposeInLds ? n * mp * sizeof(unsigned short) : 0);
     if (gT.status != BF_OK) return gT.status;
-    Scratch gImg(dA || transposeInLds ? m * np * sizeof(unsigned short) : 0);
+    Scratch gImg(needPlainG && !gImage ? m * np * sizeof(unsigned short) : 0);
     if (gImg.status != BF_OK) return gImg.status;
-    if (dA || transposeInLds) {
+    bool gTransposed = false;
+    if (needPlainG && !gImage) {
         // with both gradients wanted on the transposed-image route, one pass over g writes the plain and the transposed image
-        if (dB && !transposeInLds) st = convertTransposed(g, gT.as<unsigned short>(), m, n, s, true, gImg.as<unsigned short>(), np);
+        if (dB && !transposeInLds) { st = convertTransposed(g, gT.as<unsigned short>(), m, n, s, true, gImg.as<unsigned short>(), np); gTransposed = true; }
         else st = convertPlain(g, gImg.as<unsigned short>(), m, n, s);
         if (st != BF_OK) return st;
+        gImage = gImg.as<unsigned short>();
     }
     if (dA) {   // dA[m,k] = g[m,n] * b[k,n]^T : contraction over n
         unsigned short* bImg = nullptr;
         size_t bBytes = 0;
         st = weightImage(b, k, n, /*transposed=*/false, cacheWeight != 0, s, &bImg, &bBytes);
         if (st != BF_OK) return st;
-        st = launchGemmNt(gImg.as<unsigned short>(), bImg, dA, m, k, np, np, np, s);
+        st = launchGemmNt(gImage, bImg, dA, m, k, np, np, np, s);
         if (!cacheWeight) bf_hip_pool_release(bImg, bBytes);
         if (st != BF_OK) return st;
     }
     if (dB && transposeInLds) {
-        Scratch aImg(m * kp * sizeof(unsigned short));
+        Scratch aImg(aImage ? 0 : m * kp * sizeof(unsigned short));
         if (aImg.status != BF_OK) return aImg.status;
-        st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
-        if (st != BF_OK) return st;
+        if (!aImage) {
+            st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
+            if (st != BF_OK) return st;
+            aImage = aImg.as<unsigned short>();
+        }
         bool done = false;
-        return launchGemmTn(aImg.as<unsigned short>(), gImg.as<unsigned short>(), Epilogue{{dB, nullptr, nullptr}, int(n), nullptr, nullptr}, k, n,
-                            m, kp, np, s, &done);
+        return launchGemmTn(aImage, gImage, Epilogue{{dB, nullptr, nullptr}, int(n), nullptr, nullptr}, k, n, m, kp, np, s, &done);
     }
     if (dB) {   // dB[k,n] = a[m,k]^T * g[m,n] : contraction over m
         Scratch aT(k * mp * sizeof(unsigned short));
         if (aT.status != BF_OK) return aT.status;
-        st = convertTransposed(a, aT.as<unsigned short>(), m, k, s);
+        st = a ? convertTransposed(a, aT.as<unsigned short>(), m, k, s) : transposeImage(aImage, aT.as<unsigned short>(), m, k, kp, mp, s);
         if (st != BF_OK) return st;
-        if (!dA) st = convertTransposed(g, gT.as<unsigned short>(), m, n, s);
+        if (!gTransposed) st = g ? convertTransposed(g, gT.as<unsigned short>(), m, n, s) : transposeImage(gImage, gT.as<unsigned short>(), m, n, np, mp, s);
         if (st != BF_OK) return st;
         st = launchGemmNt(aT.as<unsigned short>(), gT.as<unsigned short>(), dB, k, n, mp, mp, mp, s);
     }
     return st;
 }
 
-int bf_hip_linear_bf16(const float* a, const float* w, const float* bias, const float* residual, float* out, size_t m, size_t k,
-                       size_t n, int cacheWeight, bf_stream_t stream) {
+int bf_hip_matmul_bf16_backward(const float* a, const float* b, const float* g, float* dA, float* dB, size_t m,
+                                size_t k, size_t n, int cacheWeight, bf_stream_t stream) {
+    if (m != 0 && k != 0 && n != 0) BF_REQUIRE(a && g, "NULL operand");
+    return bf_hip_matmul_bf16_backward_img(a, nullptr, b, g, nullptr, dA, dB, m, k, n, cacheWeight, stream);
+}
+
+int bf_hip_linear_bf16_img(const float* a, const uint16_t* aImage, const float* w, const float* bias, const float* residual, float* out,
+                           size_t m, size_t k, size_t n, int cacheWeight, bf_stream_t stream) {
     if (m == 0 || n == 0) return BF_OK;
     BF_REQUIRE(out != nullptr, "NULL output");
     int st = BF_OK;
@@ -1220,24 +1216,40 @@ int bf_hip_linear_bf16(const float* a, const float* w, const float* bias, const 
         if (st == BF_OK && residual) st = bf_hip_accumulate(out, residual, m * n, stream);
         return st;
     }
-    BF_REQUIRE(a && w, "NULL operand");
+    BF_REQUIRE((a || aImage) && w, "NULL operand");
+    BF_REQUIRE((reinterpret_cast<uintptr_t>(aImage) & 15u) == 0, "operand images must be 16-byte aligned");
     hipStream_t s = asStream(stream);
     const size_t kp = pad8(k);
-    Scratch aImg(m * kp * sizeof(unsigned short));
+    Scratch aImg(aImage ? 0 : m * kp * sizeof(unsigned short));
     if (aImg.status != BF_OK) return aImg.status;
     unsigned short* wImg = nullptr;
     size_t wBytes = 0;
-    st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
-    if (st != BF_OK) return st;
+    if (!aImage) {
+        st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
+        if (st != BF_OK) return st;
+        aImage = aImg.as<unsigned short>();
+    }
     st = weightImage(w, k, n, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
     if (st != BF_OK) return st;
-    st = launchGemmNt(aImg.as<unsigned short>(), wImg, Epilogue{{out, nullptr, nullptr}, int(n), bias, residual}, m, n, kp, kp, kp, s);
+    st = launchGemmNt(aImage, wImg, Epilogue{{out, nullptr, nullptr}, int(n), bias, residual}, m, n, kp, kp, kp, s);
     if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
     return st;
 }
 
+int bf_hip_linear_bf16(const float* a, const float* w, const float* bias, const float* residual, float* out, size_t m, size_t k,
+                       size_t n, int cacheWeight, bf_stream_t stream) {
+    if (m != 0 && n != 0 && k != 0) BF_REQUIRE(a != nullptr, "NULL operand");
+    return bf_hip_linear_bf16_img(a, nullptr, w, bias, residual, out, m, k, n, cacheWeight, stream);
+}
+
 int bf_hip_matmul_bf16_shared_input(const float* a, const float* const* b, float* const* c, size_t count, size_t m, size_t k,
                                     size_t n, int cacheWeight, bf_stream_t stream) {
+    if (m != 0 && n != 0 && k != 0) BF_REQUIRE(a != nullptr, "NULL operand");
+    return bf_hip_matmul_bf16_shared_input_img(a, nullptr, b, c, count, m, k, n, cacheWeight, stream);
+}
+
+int bf_hip_matmul_bf16_shared_input_img(const float* a, const uint16_t* aImage, const float* const* b, float* const* c, size_t count,
+                                        size_t m, size_t k, size_t n, int cacheWeight, bf_stream_t stream) {
     BF_REQUIRE(count >= 1 && count <= 3, "count must be 1, 2 or 3");
     BF_REQUIRE(b && c, "NULL pointer array");
     if (m == 0 || n == 0) return BF_OK;
@@ -1249,28 +1261,33 @@ int bf_hip_matmul_bf16_shared_input(const float* a, const float* const* b, float
         }
         return BF_OK;
     }
-    BF_REQUIRE(a != nullptr, "NULL operand");
+    BF_REQUIRE(a != nullptr || aImage != nullptr, "NULL operand");
+    BF_REQUIRE((reinterpret_cast<uintptr_t>(aImage) & 15u) == 0, "operand images must be 16-byte aligned");
     for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] != nullptr, "NULL operand");
     hipStream_t s = asStream(stream);
     const size_t kp = pad8(k);
-    Scratch aImg(m * kp * sizeof(unsigned short));
+    Scratch aImg(aImage ? 0 : m * kp * sizeof(unsigned short));
     if (aImg.status != BF_OK) return aImg.status;
-    int st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
-    if (st != BF_OK) return st;
+    int st = BF_OK;
+    if (!aImage) {
+        st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
+        if (st != BF_OK) return st;
+        aImage = aImg.as<unsigned short>();
+    }
     unsigned short* wImg = nullptr;
     size_t wBytes = 0;
     if (count > 1 && n % 256 == 0) {   // one GEMM over the stacked weight images, tiles routed to their output
         st = weightImage(b, count, k, n, 2, cacheWeight != 0, s, &wImg, &wBytes);
         if (st != BF_OK) return st;
         Epilogue epi{{c[0], count > 1 ? c[1] : nullptr, count > 2 ? c[2] : nullptr}, int(n), nullptr, nullptr};
-        st = launchGemmNt(aImg.as<unsigned short>(), wImg, epi, m, count * n, kp, kp, kp, s);
+        st = launchGemmNt(aImage, wImg, epi, m, count * n, kp, kp, kp, s);
         if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
         return st;
     }
     for (size_t i = 0; i < count; ++i) {
         st = weightImage(b[i], k, n, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
         if (st != BF_OK) return st;
-        st = launchGemmNt(aImg.as<unsigned short>(), wImg, c[i], m, n, kp, kp, kp, s);
+        st = launchGemmNt(aImage, wImg, c[i], m, n, kp, kp, kp, s);
         if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
         if (st != BF_OK) return st;
     }
@@ -1280,8 +1297,19 @@ int bf_hip_matmul_bf16_shared_input(const float* a, const float* const* b, float
 int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const* b, const float* const* g, float* dA,
                                              float* const* dB, size_t count, size_t m, size_t k, size_t n, int cacheWeight,
                                              bf_stream_t stream) {
+    BF_REQUIRE(g != nullptr, "NULL pointer array");
+    if (m != 0 && k != 0 && n != 0) {
+        BF_REQUIRE(a != nullptr, "NULL operand");
+        for (size_t i = 0; i < count && i < 3; ++i) BF_REQUIRE(g[i] != nullptr, "NULL operand");
+    }
+    return bf_hip_matmul_bf16_shared_input_backward_img(a, nullptr, b, g, nullptr, dA, dB, count, m, k, n, cacheWeight, stream);
+}
+
+int bf_hip_matmul_bf16_shared_input_backward_img(const float* a, const uint16_t* aImage, const float* const* b, const float* const* g,
+                                                 const uint16_t* gImage, float* dA, float* const* dB, size_t count, size_t m, size_t k,
+                                                 size_t n, int cacheWeight, bf_stream_t stream) {
     BF_REQUIRE(count >= 1 && count <= 3, "count must be 1, 2 or 3");
-    BF_REQUIRE(b && g, "NULL pointer array");
+    BF_REQUIRE(b && (g || gImage), "NULL pointer array");
     hipStream_t s = asStream(stream);
     if (m == 0 || k == 0 || n == 0) {   // degenerate: gradients are zero
         int st = BF_OK;
@@ -1290,8 +1318,10 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
             if (dB[i] && k * n) st = bf_hip_fill_zero(dB[i], k * n * sizeof(float), stream);
         return st;
     }
-    BF_REQUIRE(a != nullptr, "NULL operand");
-    for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] && g[i], "NULL operand");
+    BF_REQUIRE(a != nullptr || aImage != nullptr, "NULL operand");
+    for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] && (gImage || g[i]), "NULL operand");
+    BF_REQUIRE(gImage == nullptr || n % 8 == 0, "a side-by-side gradient image needs a width that is a multiple of 8");
+    BF_REQUIRE(((reinterpret_cast<uintptr_t>(aImage) | reinterpret_cast<uintptr_t>(gImage)) & 15u) == 0, "operand images must be 16-byte aligned");
     int st = BF_OK;
     bool anyDb = false, allDb = dB != nullptr;
     for (size_t i = 0; dB && i < count; ++i) anyDb = anyDb || dB[i] != nullptr;
@@ -1306,26 +1336,32 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
         const size_t nn = count * n;
         if (dA && allDb && count > 1 && n % 256 == 0 && planLargeTiles(k, nn, m, &form, &slices)) {
             const size_t kp = pad8(k);
-            Scratch gImg(m * nn * sizeof(unsigned short));
+            Scratch gImg(gImage ? 0 : m * nn * sizeof(unsigned short));
             if (gImg.status != BF_OK) return gImg.status;
-            for (size_t i = 0; i < count; ++i) {
-                st = convertPlain(g[i], gImg.as<unsigned short>() + i * n, m, n, s, nn);
-                if (st != BF_OK) return st;
+            if (!gImage) {
+                for (size_t i = 0; i < count; ++i) {
+                    st = convertPlain(g[i], gImg.as<unsigned short>() + i * n, m, n, s, nn);
+                    if (st != BF_OK) return st;
+                }
+                gImage = gImg.as<unsigned short>();
             }
             unsigned short* wImg = nullptr;
             size_t wBytes = 0;
             st = weightImage(b, count, k, n, 3, cacheWeight != 0, s, &wImg, &wBytes);
             if (st != BF_OK) return st;
-            st = launchGemmNt(gImg.as<unsigned short>(), wImg, dA, m, k, nn, nn, nn, s);
+            st = launchGemmNt(gImage, wImg, dA, m, k, nn, nn, nn, s);
             if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
             if (st != BF_OK) return st;
-            Scratch aImg(m * kp * sizeof(unsigned short));
+            Scratch aImg(aImage ? 0 : m * kp * sizeof(unsigned short));
             if (aImg.status != BF_OK) return aImg.status;
-            st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
-            if (st != BF_OK) return st;
+            if (!aImage) {
+                st = convertPlain(a, aImg.as<unsigned short>(), m, k, s);
+                if (st != BF_OK) return st;
+                aImage = aImg.as<unsigned short>();
+            }
             Epilogue epi{{dB[0], count > 1 ? dB[1] : nullptr, count > 2 ? dB[2] : nullptr}, int(n), nullptr, nullptr};
             bool done = false;
-            return launchGemmTn(aImg.as<unsigned short>(), gImg.as<unsigned short>(), epi, k, nn, m, kp, nn, s, &done);
+            return launchGemmTn(aImage, gImage, epi, k, nn, m, kp, nn, s, &done);
         }
     }
     const size_t mp = pad8(m);
@@ -1336,9 +1372,9 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
         if (count > 1 && n % 8 == 0) {
             // dA = sum_i g_i b_i^T = [g_0 | g_1 | g_2] [b_0 | b_1 | b_2]^T: one GEMM whose contraction runs over all of them
             const size_t nn = count * n;
-            Scratch gImg(m * nn * sizeof(unsigned short));
+            Scratch gImg(gImage ? 0 : m * nn * sizeof(unsigned short));
             if (gImg.status != BF_OK) return gImg.status;
-            for (size_t i = 0; i < count; ++i) {
+            for (size_t i = 0; i < count && !gImage; ++i) {
                 if (dB && dB[i]) {   // one pass over g_i writes its column slice of the plain image and its transposed image
                     st = convertTransposed(g[i], gT.as<unsigned short>() + i * n * mp, m, n, s, true, gImg.as<unsigned short>() + i * n, nn);
                     transposedDone[i] = true;
@@ -1351,7 +1387,7 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
             size_t wBytes = 0;
             st = weightImage(b, count, k, n, 3, cacheWeight != 0, s, &wImg, &wBytes);
             if (st != BF_OK) return st;
-            st = launchGemmNt(gImg.as<unsigned short>(), wImg, dA, m, k, nn, nn, nn, s);
+            st = launchGemmNt(gImage ? gImage : gImg.as<unsigned short>(), wImg, dA, m, k, nn, nn, nn, s);
             if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
             if (st != BF_OK) return st;
         } else {
@@ -1359,7 +1395,9 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
             if (extra.status != BF_OK) return extra.status;
             for (size_t i = 0; i < count; ++i) {
                 float* target = i == 0 ? dA : extra.as<float>();
-                st = bf_hip_matmul_bf16_backward(a, b[i], g[i], target, nullptr, m, k, n, cacheWeight, stream);
+                // a side-by-side image exists only for widths that are multiples of 8, which the branch above takes unless count == 1
+                st = bf_hip_matmul_bf16_backward_img(a, aImage, b[i], g ? g[i] : nullptr, count == 1 ? gImage : nullptr, target, nullptr, m, k, n,
+                                                     cacheWeight, stream);
                 if (st != BF_OK) return st;
                 if (i > 0) st = bf_hip_accumulate(dA, target, m * k, stream);
                 if (st != BF_OK) return st;
@@ -1369,13 +1407,14 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
     if (anyDb) {
         Scratch aT(k * mp * sizeof(unsigned short));
         if (aT.status != BF_OK) return aT.status;
-        st = convertTransposed(a, aT.as<unsigned short>(), m, k, s);
+        st = a ? convertTransposed(a, aT.as<unsigned short>(), m, k, s) : transposeImage(aImage, aT.as<unsigned short>(), m, k, pad8(k), mp, s);
         if (st != BF_OK) return st;
         bool all = true;
         for (size_t i = 0; i < count; ++i) all = all && dB[i] != nullptr;
         for (size_t i = 0; i < count; ++i) {
             if (!dB[i] || transposedDone[i]) continue;
-            st = convertTransposed(g[i], gT.as<unsigned short>() + i * n * mp, m, n, s);
+            st = (g && g[i]) ? convertTransposed(g[i], gT.as<unsigned short>() + i * n * mp, m, n, s)
+                             : transposeImage(gImage + i * n, gT.as<unsigned short>() + i * n * mp, m, n, count * n, mp, s);
             if (st != BF_OK) return st;
         }
         if (all && count > 1 && n % 256 == 0) {
@@ -1399,13 +1438,17 @@ int bf_hip_feedforward_bf16(const float* x, const float* w1, const float* b1, co
     if (m == 0) return BF_OK;
     BF_REQUIRE(d > 0 && hidden > 0 && d % 8 == 0 && hidden % 8 == 0, "d and hidden must be positive multiples of 8");
     BF_REQUIRE(act == BF_ACT_SILU || act == BF_ACT_GELU || act == BF_ACT_RELU, "unknown activation");
-    BF_REQUIRE(x && w1 && w2 && z && hImage && out, "NULL pointer");
+    BF_REQUIRE((x || xImage) && w1 && w2 && z && hImage && out, "NULL pointer");
+    BF_REQUIRE(((reinterpret_cast<uintptr_t>(xImage) | reinterpret_cast<uintptr_t>(hImage)) & 15u) == 0, "operand images must be 16-byte aligned");
     hipStream_t s = asStream(stream);
     Scratch xScratch(xImage ? 0 : m * d * sizeof(unsigned short));
     if (xScratch.status != BF_OK) return xScratch.status;
     unsigned short* xImg = xImage ? xImage : xScratch.as<unsigned short>();
-    int st = convertPlain(x, xImg, m, d, s);
-    if (st != BF_OK) return st;
+    int st = BF_OK;
+    if (x) {   // x == NULL: xImage already holds bf16(x)
+        st = convertPlain(x, xImg, m, d, s);
+        if (st != BF_OK) return st;
+    }
     unsigned short* wImg = nullptr;
     size_t wBytes = 0;
     st = weightImage(w1, d, hidden, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
@@ -1425,6 +1468,14 @@ int bf_hip_feedforward_bf16(const float* x, const float* w1, const float* b1, co
 int bf_hip_feedforward_bf16_backward(const float* x, const uint16_t* xImage, const float* w1, const float* w2, const float* z,
                                      const uint16_t* hImage, const float* g, int act, float* dX, float* dW1, float* dB1, float* dW2,
                                      float* dB2, size_t m, size_t d, size_t hidden, int cacheWeight, bf_stream_t stream) {
+    return bf_hip_feedforward_bf16_backward_img(x, xImage, w1, w2, z, hImage, g, nullptr, act, dX, dW1, dB1, dW2, dB2, m, d, hidden,
+                                                cacheWeight, stream);
+}
+
+int bf_hip_feedforward_bf16_backward_img(const float* x, const uint16_t* xImage, const float* w1, const float* w2, const float* z,
+                                         const uint16_t* hImage, const float* g, const uint16_t* gImage, int act, float* dX, float* dW1,
+                                         float* dB1, float* dW2, float* dB2, size_t m, size_t d, size_t hidden, int cacheWeight,
+                                         bf_stream_t stream) {
     BF_REQUIRE(d > 0 && hidden > 0 && d % 8 == 0 && hidden % 8 == 0, "d and hidden must be positive multiples of 8");
     BF_REQUIRE(act == BF_ACT_SILU || act == BF_ACT_GELU || act == BF_ACT_RELU, "unknown activation");
     hipStream_t s = asStream(stream);
@@ -1436,19 +1487,25 @@ int bf_hip_feedforward_bf16_backward(const float* x, const uint16_t* xImage, con
         if (st == BF_OK && dB2) st = bf_hip_fill_zero(dB2, d * sizeof(float), stream);
         return st;
     }
-    BF_REQUIRE((x || xImage) && w1 && w2 && z && hImage && g, "NULL operand");
+    BF_REQUIRE((x || xImage) && w1 && w2 && z && hImage && (g || gImage), "NULL operand");
+    BF_REQUIRE(g != nullptr || dB2 == nullptr, "the bias gradient dB2 is taken from the fp32 gradient");
+    BF_REQUIRE(((reinterpret_cast<uintptr_t>(xImage) | reinterpret_cast<uintptr_t>(hImage) | reinterpret_cast<uintptr_t>(gImage)) & 15u) == 0,
+               "operand images must be 16-byte aligned");
     const size_t mp = pad8(m);
-    Scratch gImg(m * d * sizeof(unsigned short));
+    Scratch gImg(gImage ? 0 : m * d * sizeof(unsigned short));
     if (gImg.status != BF_OK) return gImg.status;
-    st = convertPlain(g, gImg.as<unsigned short>(), m, d, s);
-    if (st != BF_OK) return st;
+    if (!gImage) {   // gImage: bf16(g) made by whoever produced g
+        st = convertPlain(g, gImg.as<unsigned short>(), m, d, s);
+        if (st != BF_OK) return st;
+        gImage = gImg.as<unsigned short>();
+    }
     if (dB2) {
         st = bf_hip_bias_grad(g, dB2, m, d, stream);
         if (st != BF_OK) return st;
     }
     if (dW2) {   // dW2[hidden, d] = h^T g, contraction over the m rows
         bool done = false;
-        st = launchGemmTn(hImage, gImg.as<unsigned short>(), Epilogue{{dW2, nullptr, nullptr}, int(d), nullptr, nullptr}, hidden, d, m,
+        st = launchGemmTn(hImage, gImage, Epilogue{{dW2, nullptr, nullptr}, int(d), nullptr, nullptr}, hidden, d, m,
                           hidden, d, s, &done);
         if (st != BF_OK) return st;
         if (!done) {
@@ -1456,7 +1513,7 @@ int bf_hip_feedforward_bf16_backward(const float* x, const uint16_t* xImage, con
             if (hT.status != BF_OK) return hT.status;
             if (gT.status != BF_OK) return gT.status;
             st = transposeImage(hImage, hT.as<unsigned short>(), m, hidden, hidden, mp, s);
-            if (st == BF_OK) st = convertTransposed(g, gT.as<unsigned short>(), m, d, s);
+            if (st == BF_OK) st = g ? convertTransposed(g, gT.as<unsigned short>(), m, d, s) : transposeImage(gImage, gT.as<unsigned short>(), m, d, d, mp, s);
             if (st == BF_OK) st = launchGemmNt(hT.as<unsigned short>(), gT.as<unsigned short>(), dW2, hidden, d, mp, mp, mp, s);
             if (st != BF_OK) return st;
         }
@@ -1470,7 +1527,7 @@ int bf_hip_feedforward_bf16_backward(const float* x, const uint16_t* xImage, con
     size_t wBytes = 0;
     st = weightImage(w2, hidden, d, /*transposed=*/false, cacheWeight != 0, s, &wImg, &wBytes);
     if (st != BF_OK) return st;
-    st = launchGemmNt(gImg.as<unsigned short>(), wImg, dH.as<float>(), m, hidden, d, d, d, s);
+    st = launchGemmNt(gImage, wImg, dH.as<float>(), m, hidden, d, d, d, s);
     if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
     if (st != BF_OK) return st;
     st = actBackwardToBf16Image(z, dH.as<float>(), dzImg.as<unsigned short>(), dB1, m, hidden, act, s);

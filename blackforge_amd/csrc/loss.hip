@@ -84,7 +84,8 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                                                                          const float* __restrict__ target,
                                                                          float* __restrict__ grad, float* __restrict__ rowLoss,
                                                                          size_t rows, size_t classes, float invRows,
-                                                                         const float* __restrict__ maskInfo) {
+                                                                         const float* __restrict__ maskInfo,
+                                                                         unsigned short* __restrict__ gradImage) {
     __shared__ float lds[16];
     const int t = threadIdx.x % G;
     const size_t rowsPerBlock = blockDim.x / G;
@@ -115,9 +116,14 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
             fetch(c, row);
         }
         const int shift = SHIFTED ? RowCache<G, MAXE, VEC, NT>::shiftOf(x) : 0;   // the same for gOut: the host checks that
+        // gradImage (aligned rows only; the host checks): the gradient row rounded to bf16, for the bf16 GEMMs that consume it
+        unsigned short* gImg = gradImage ? gradImage + row * classes : nullptr;
         auto storeRow = [&]() __attribute__((always_inline)) {
             if constexpr (SHIFTED) c.storeShifted(gOut, classes, t, shift);
-            else c.store(gOut, classes, t);
+            else {
+                c.store(gOut, classes, t);
+                if (gImg) c.storeBf16(gImg, classes, t);
+            }
         };
         if constexpr (SPARSE) {
             if (maskInfo != nullptr && lroundf(target[row]) == -1) {   // uniform over the row's group
@@ -126,7 +132,7 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                     for (int i = 0; i < MAXE; ++i) c.r[i] = 0.0f;
                     storeRow();
                 } else {
-                    for (size_t e = t; e < classes; e += G) gOut[e] = 0.0f;
+                    for (size_t e = t; e < classes; e += G) { gOut[e] = 0.0f; if (gImg) gImg[e] = 0; }
                 }
                 if (t == 0) rowLoss[row] = 0.0f;
                 continue;
@@ -175,7 +181,9 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                     const float p = __builtin_amdgcn_exp2f((x[e] - mx) * kLog2e) * inv;
                     const bool hit = e == cls;
                     pTarget = hit ? p : pTarget;
-                    gOut[e] = (p - (hit ? 1.0f : 0.0f)) * invRows;
+                    const float gv = (p - (hit ? 1.0f : 0.0f)) * invRows;
+                    gOut[e] = gv;
+                    if (gImg) gImg[e] = toBf16Bits(gv);
                 }
             }
             if (pTarget >= 0.0f) loss = -logf(fmaxf(pTarget, 1e-12f));
@@ -197,7 +205,11 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                     }
                 storeRow();
             } else {
-                for (size_t e = t; e < classes; e += G) gOut[e] = emit(__builtin_amdgcn_exp2f((x[e] - mx) * kLog2e), e);
+                for (size_t e = t; e < classes; e += G) {
+                    const float gv = emit(__builtin_amdgcn_exp2f((x[e] - mx) * kLog2e), e);
+                    gOut[e] = gv;
+                    if (gImg) gImg[e] = toBf16Bits(gv);
+                }
             }
         }
         loss = groupSum<G>(loss, lds);
@@ -207,7 +219,9 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
 
 template <bool SPARSE>
 int launchCrossEntropy(const float* logits, const float* target, float* grad, float* lossSum, size_t rows,
-                       size_t classes, int accumulate, hipStream_t s, bool masked = false) {
+                       size_t classes, int accumulate, hipStream_t s, bool masked = false, unsigned short* gradImage = nullptr) {
+    if (gradImage != nullptr && (classes % 8 != 0 || !aligned16(logits) || !aligned16(grad) || !aligned16(gradImage)))
+        return failInvalid("cross_entropy", "the bf16 gradient image needs 16-byte aligned tensors and a class count that is a multiple of 8");
     Scratch rowLoss((rows + 2) * sizeof(float));   // per-row losses, then the two words of the masked form
     if (rowLoss.status != BF_OK) return rowLoss.status;
     float* rl = rowLoss.as<float>();
@@ -229,16 +243,16 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
         const unsigned threads = G > 256 ? G : 256;                                                               \
         const bool nt = streaming && MAXE <= 32;   /* measured: the hint only pays together with the look-ahead */ \
         const unsigned grid = gridFor(rows, threads / G, MAXE <= 32 ? unsigned(computeUnits()) * (2048 / threads) : kMaxGridX); \
-        if (vec4 && nt) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
-        else if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
-        else if (shifted && nt) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
-        else if (shifted) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); \
-        else crossEntropyKernel<G, (MAXE <= 32 ? MAXE : 4), 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo); /* plans above 32 registers have no one-element form */ \
+        if (vec4 && nt) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
+        else if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
+        else if (shifted && nt) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
+        else if (shifted) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
+        else crossEntropyKernel<G, (MAXE <= 32 ? MAXE : 4), 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); /* plans above 32 registers have no one-element form */ \
         break;                                                                                                    \
     }
     do {
         BF_CE(64, 4) BF_CE(64, 8) BF_CE(64, 16) BF_CE(256, 8) BF_CE(256, 16) BF_CE(256, 32) BF_CE(1024, 16) BF_CE(1024, 32) BF_CE(1024, 52)
-        crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo);
+        crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage);
     } while (0);
 #undef BF_CE
     BF_LAUNCH_CHECK();
@@ -291,15 +305,20 @@ int bf_hip_cross_entropy(const float* logits, const float* target, float* grad, 
     return launchCrossEntropy<false>(logits, target, grad, lossSum, rows, classes, accumulate, asStream(stream));
 }
 
-int bf_hip_cross_entropy_sparse(const float* logits, const float* targetIdx, float* grad, float* lossSum,
-                                size_t rows, size_t classes, int accumulate, bf_stream_t stream) {
+int bf_hip_cross_entropy_sparse_img(const float* logits, const float* targetIdx, float* grad, uint16_t* gradImage, float* lossSum,
+                                    size_t rows, size_t classes, int accumulate, bf_stream_t stream) {
     BF_REQUIRE(lossSum != nullptr, "lossSum is NULL");
     if (rows == 0 || classes == 0) {
         if (!accumulate) return bf_hip_fill_zero(lossSum, sizeof(float), stream);
         return BF_OK;
     }
     BF_REQUIRE(logits && targetIdx && grad, "NULL pointer");
-    return launchCrossEntropy<true>(logits, targetIdx, grad, lossSum, rows, classes, accumulate, asStream(stream));
+    return launchCrossEntropy<true>(logits, targetIdx, grad, lossSum, rows, classes, accumulate, asStream(stream), false, gradImage);
+}
+
+int bf_hip_cross_entropy_sparse(const float* logits, const float* targetIdx, float* grad, float* lossSum,
+                                size_t rows, size_t classes, int accumulate, bf_stream_t stream) {
+    return bf_hip_cross_entropy_sparse_img(logits, targetIdx, grad, nullptr, lossSum, rows, classes, accumulate, stream);
 }
 
 int bf_hip_cross_entropy_masked(const float* logits, const float* targetIdx, float* grad, float* lossMean, size_t rows,

@@ -90,6 +90,23 @@ struct RowCache {
         }
     }
 
+    // The row rounded to bf16 (nearest even), for rows that are the operand of a bf16 GEMM: row[e] = bf16(r[e]).
+    __device__ __forceinline__ void storeBf16(unsigned short* __restrict__ row, size_t features, int t) const {
+#pragma unroll
+        for (int it = 0; it < kIters; ++it) {
+            size_t e = index(it, t, 0);
+            if (e < features) {
+                if constexpr (VEC == 4) {
+                    const uint2v packed = {unsigned(toBf16Bits(r[it * 4 + 0])) | unsigned(toBf16Bits(r[it * 4 + 1])) << 16,
+                                           unsigned(toBf16Bits(r[it * 4 + 2])) | unsigned(toBf16Bits(r[it * 4 + 3])) << 16};
+                    stu2<NT>(row + e, packed);
+                } else {
+                    row[e] = toBf16Bits(r[it]);
+                }
+            }
+        }
+    }
+
     __device__ __forceinline__ void store(float* __restrict__ row, size_t features, int t) const {
 #pragma unroll
         for (int it = 0; it < kIters; ++it) {

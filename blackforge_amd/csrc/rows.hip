@@ -78,7 +78,7 @@ struct Row {
 
 template <int G, int MAXE, int VEC, bool CACHED, bool NT = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormKernel(const float* __restrict__ x, float* __restrict__ out,
-                                                                    size_t rows, size_t features) {
+                                                                    unsigned short* __restrict__ image, size_t rows, size_t features) {
     BF_ROW_PROLOGUE();
     for (size_t row = firstRow; row < rows; row += rowStep) {
         Row<G, MAXE, VEC, CACHED, NT> rx;
@@ -88,14 +88,27 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormKernel(const float* 
         rx.reduce([&](float v) { ss += double(v) * double(v); });
         ss = groupSum<G>(ss, ldsD);
         float rms = float(sqrt(ss / double(features) + double(kRmsNormEps)));
-        rx.map(out + row * features, [&](float v, size_t) { return v / rms; });
+        // either output may be absent: the fp32 row, and its bf16 image for a consumer that is a bf16 GEMM
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int i = 0; i < MAXE; ++i) rx.c.r[i] = rx.c.r[i] / rms;
+            if (out) rx.c.store(out + row * features, features, t);
+            if (image) rx.c.storeBf16(image + row * features, features, t);
+        } else {
+            for (size_t e = t; e < features; e += G) {
+                const float v = rx.p[e] / rms;
+                if (out) out[row * features + e] = v;
+                if (image) image[row * features + e] = toBf16Bits(v);
+            }
+        }
     }
 }
 
 template <int G, int MAXE, int VEC, bool CACHED, bool NT = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const float* __restrict__ x, const float* __restrict__ g,
                                                                             const float* __restrict__ addend, float* __restrict__ out,
-                                                                            size_t rows, size_t features) {
+                                                                            unsigned short* __restrict__ outImage, size_t rows,
+                                                                            size_t features) {
     BF_ROW_PROLOGUE();
     for (size_t row = firstRow; row < rows; row += rowStep) {
         Row<G, MAXE, VEC, CACHED, NT> rx, rg;
@@ -131,11 +144,14 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) rmsnormBackwardKernel(const
                 for (int i = 0; i < MAXE; ++i) rg.c.r[i] += rx.c.r[i];
             }
             rg.c.store(o, features, t);
+            if (outImage) rg.c.storeBf16(outImage + row * features, features, t);
         } else {
             const float* a = addend ? addend + row * features : nullptr;
             for (size_t e = t; e < features; e += G) {
-                const float v = float(double(rg.p[e]) * invR - double(rx.p[e]) * k);
-                o[e] = a ? v + a[e] : v;
+                float v = float(double(rg.p[e]) * invR - double(rx.p[e]) * k);
+                if (a) v += a[e];
+                o[e] = v;
+                if (outImage) outImage[row * features + e] = toBf16Bits(v);
             }
         }
     }
@@ -246,12 +262,34 @@ using namespace bf;
 
 extern "C" {
 
+int bf_hip_rmsnorm_img(const float* x, float* out, uint16_t* image, size_t rows, size_t features, bf_stream_t stream) {
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && (out || image), "NULL pointer");
+    BF_REQUIRE(image == nullptr || features % 8 == 0, "the bf16 image needs a feature count that is a multiple of 8");
+    hipStream_t s = asStream(stream);
+#define ARGS_ x, out, image, rows, features
+    BF_ROW_LAUNCH(rmsnormKernel, false, aligned16(x) && aligned16(out) && aligned16(image), rows, features, s, x, out, image, rows, features);
+#undef ARGS_
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
 int bf_hip_rmsnorm(const float* x, float* out, size_t rows, size_t features, bf_stream_t stream) {
     if (rows == 0 || features == 0) return BF_OK;
     BF_REQUIRE(x && out, "NULL pointer");
+    return bf_hip_rmsnorm_img(x, out, nullptr, rows, features, stream);
+}
+
+int bf_hip_rmsnorm_backward_add_img(const float* x, const float* g, const float* addend, float* out, uint16_t* outImage, size_t rows,
+                                    size_t features, bf_stream_t stream) {
+    if (rows == 0 || features == 0) return BF_OK;
+    BF_REQUIRE(x && g && out, "NULL pointer");
+    BF_REQUIRE(addend != out, "the output must not be the addend");
+    BF_REQUIRE(outImage == nullptr || features % 8 == 0, "the bf16 image needs a feature count that is a multiple of 8");
     hipStream_t s = asStream(stream);
-#define ARGS_ x, out, rows, features
-    BF_ROW_LAUNCH(rmsnormKernel, false, aligned16(x) && aligned16(out), rows, features, s, x, out, rows, features);
+#define ARGS_ x, g, addend, out, outImage, rows, features
+    BF_ROW_LAUNCH(rmsnormBackwardKernel, true, aligned16(x) && aligned16(g) && aligned16(out) && aligned16(addend) && aligned16(outImage), rows,
+                  features, s, x, g, addend, out, outImage, rows, features);
 #undef ARGS_
     BF_LAUNCH_CHECK();
     return BF_OK;
@@ -259,16 +297,7 @@ int bf_hip_rmsnorm(const float* x, float* out, size_t rows, size_t features, bf_
 
 int bf_hip_rmsnorm_backward_add(const float* x, const float* g, const float* addend, float* out, size_t rows, size_t features,
                                 bf_stream_t stream) {
-    if (rows == 0 || features == 0) return BF_OK;
-    BF_REQUIRE(x && g && out, "NULL pointer");
-    BF_REQUIRE(addend != out, "the output must not be the addend");
-    hipStream_t s = asStream(stream);
-#define ARGS_ x, g, addend, out, rows, features
-    BF_ROW_LAUNCH(rmsnormBackwardKernel, true, aligned16(x) && aligned16(g) && aligned16(out) && aligned16(addend), rows, features, s, x, g,
-                  addend, out, rows, features);
-#undef ARGS_
-    BF_LAUNCH_CHECK();
-    return BF_OK;
+    return bf_hip_rmsnorm_backward_add_img(x, g, addend, out, nullptr, rows, features, stream);
 }
 
 int bf_hip_rmsnorm_backward(const float* x, const float* g, float* out, size_t rows, size_t features,

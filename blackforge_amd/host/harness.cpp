@@ -108,7 +108,8 @@ int bfh_model_loss(void* h, const float* target, int lossKind) {
         if (lossKind == 0 || lossKind == 2) {
             std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
             Borrowed tgt(target, {rows});
-            handle->lossGrad = lossKind == 0 ? hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator)
+            handle->lossGrad = lossKind == 0 ? hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator,
+                                                                                       handle->model->usesBf16())
                                              : hip::softmaxCrossEntropyMaskedAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
         } else {
             Borrowed tgt(target, handle->output.shape());
@@ -163,7 +164,8 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
         if (lossKind == 0 || lossKind == 2) {
             std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
             Borrowed tgt(target, {rows});
-            handle->lossGrad = lossKind == 0 ? hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator)
+            handle->lossGrad = lossKind == 0 ? hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator,
+                                                                                       handle->model->usesBf16())
                                              : hip::softmaxCrossEntropyMaskedAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
         } else {
             Borrowed tgt(target, handle->output.shape());

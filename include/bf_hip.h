@@ -146,6 +146,13 @@ int bf_hip_rmsnorm_backward(const float* x, const float* g, float* out, size_t r
  * addend may be NULL; out must not be addend. */
 int bf_hip_rmsnorm_backward_add(const float* x, const float* g, const float* addend, float* out, size_t rows,
                                 size_t features, bf_stream_t stream);
+/* rmsnorm / rmsnorm_backward_add that also (or only) write the bf16 image of their result (round to nearest even,
+ * [rows, features], features a multiple of 8): a result whose consumers are bf16 GEMMs needs no conversion pass, and
+ * rmsnorm's fp32 output may be NULL when nothing else reads it.  No counterpart in the reference, whose cuBLASLt
+ * operands are converted by floatToBf16Kernel (ops_tensorcore.cu:21-26,80-87) on every call. */
+int bf_hip_rmsnorm_img(const float* x, float* out, uint16_t* image, size_t rows, size_t features, bf_stream_t stream);
+int bf_hip_rmsnorm_backward_add_img(const float* x, const float* g, const float* addend, float* out, uint16_t* outImage, size_t rows,
+                                    size_t features, bf_stream_t stream);
 /* softmax: ops.hpp:98 */
 int bf_hip_softmax(const float* x, float* out, size_t rows, size_t features, bf_stream_t stream);
 /* softmaxBackward: autodiff.hpp:84 (takes the forward INPUT, recomputes y) */
@@ -247,7 +254,7 @@ int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const*
  *   hImage[m,hidden] = bf16(act(z))                                 the second GEMM's operand; no fp32 copy is written
  *   out[m,d]         = hImage * bf16(w2[hidden,d]) + b2 + residual
  * d and hidden must be multiples of 8; b1, b2 and residual may be NULL; xImage, if not NULL, receives bf16(x) ([m,d]) for
- * the backward call.  Results equal those of bf_hip_matmul_bf16 + bf_hip_add_bias_act + bf_hip_linear_bf16. */
+ * the backward call -- or, with x == NULL, already holds it.  Results equal those of bf_hip_matmul_bf16 + bf_hip_add_bias_act + bf_hip_linear_bf16. */
 int bf_hip_feedforward_bf16(const float* x, const float* w1, const float* b1, const float* w2, const float* b2,
                             const float* residual, int act, float* z, uint16_t* hImage, uint16_t* xImage, float* out, size_t m,
                             size_t d, size_t hidden, int cacheWeight, bf_stream_t stream);
@@ -259,6 +266,26 @@ int bf_hip_feedforward_bf16_backward(const float* x, const uint16_t* xImage, con
                                      const uint16_t* hImage, const float* g, int act, float* dX, float* dW1, float* dB1,
                                      float* dW2, float* dB2, size_t m, size_t d, size_t hidden, int cacheWeight,
                                      bf_stream_t stream);
+/* The projection entry points above with operands that already exist as bf16 images (made by the *_img producers, or
+ * kept from the forward pass): wherever a fp32 operand `a` / `g` / `x` is paired with an image pointer, a non-NULL image
+ * ([rows, pad8(width)] bf16, 16-byte aligned) is used as it is and the fp32 pointer may be NULL.  For the shared-input
+ * backward the image holds the `count` gradients side by side: gImage[m, count * n], gradient i in columns i*n .. (n a
+ * multiple of 8).  Results are those of the fp32-operand entry points, bit for bit: the images hold the same roundings. */
+int bf_hip_linear_bf16_img(const float* a, const uint16_t* aImage, const float* w, const float* bias, const float* residual, float* out,
+                           size_t m, size_t k, size_t n, int cacheWeight, bf_stream_t stream);
+int bf_hip_matmul_bf16_backward_img(const float* a, const uint16_t* aImage, const float* b, const float* g, const uint16_t* gImage,
+                                    float* dA, float* dB, size_t m, size_t k, size_t n, int cacheWeight, bf_stream_t stream);
+int bf_hip_matmul_bf16_shared_input_img(const float* a, const uint16_t* aImage, const float* const* b, float* const* c, size_t count,
+                                        size_t m, size_t k, size_t n, int cacheWeight, bf_stream_t stream);
+int bf_hip_matmul_bf16_shared_input_backward_img(const float* a, const uint16_t* aImage, const float* const* b, const float* const* g,
+                                                 const uint16_t* gImage, float* dA, float* const* dB, size_t count, size_t m, size_t k,
+                                                 size_t n, int cacheWeight, bf_stream_t stream);
+/* bf_hip_feedforward_bf16 itself accepts x == NULL with xImage holding bf16(x) on entry; the backward pass takes the
+ * image of g beside g (g is still read for dB2; with dB2 == NULL it may be NULL). */
+int bf_hip_feedforward_bf16_backward_img(const float* x, const uint16_t* xImage, const float* w1, const float* w2, const float* z,
+                                         const uint16_t* hImage, const float* g, const uint16_t* gImage, int act, float* dX, float* dW1,
+                                         float* dB1, float* dW2, float* dB2, size_t m, size_t d, size_t hidden, int cacheWeight,
+                                         bf_stream_t stream);
 /* invalidateBf16WeightCache: ops.hpp:80 */
 int bf_hip_invalidate_bf16_weight_cache(void);
 
@@ -272,6 +299,11 @@ int bf_hip_invalidate_bf16_weight_cache(void);
 int bf_hip_attention_forward(const float* q, const float* k, const float* v, float* out, float* m, float* l,
                              size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
                              size_t oldLen, bf_stream_t stream);
+/* The same with the bf16 image of the output written as well (outImage[batch*newLen, imageLd], imageLd >= dim, both
+ * multiples of 8), for the output projection that consumes it; `out` is still needed by the backward pass. */
+int bf_hip_attention_forward_img(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
+                                 float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
+                                 size_t oldLen, bf_stream_t stream);
 /* computeDKernel: fused_attention.cu:166-190   D[b,h,i] = dot(out[b,i,h,:], dOut[b,i,h,:]) */
 int bf_hip_attention_dot_o_do(const float* out, const float* dOut, float* D, size_t batch, size_t heads,
                               size_t newLen, size_t dim, bf_stream_t stream);
@@ -282,6 +314,14 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
                               const float* m, const float* l, float* dQ, float* dK, float* dV, size_t batch,
                               size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
                               bf_stream_t stream);
+
+/* fusedAttentionBackward whose gradients go to bf16 images (row r of a gradient at image + r * imageLd; the three images
+ * may be column slices of one [rows, 3 * dim] image, the operand layout of bf_hip_matmul_bf16_shared_input_backward_img).
+ * Any image may be NULL; a gradient with an image may have a NULL fp32 tensor, which then is not written at all. */
+int bf_hip_attention_backward_img(const float* dOut, const float* q, const float* k, const float* v, const float* out, const float* m,
+                                  const float* l, float* dQ, float* dK, float* dV, uint16_t* dQImage, uint16_t* dKImage,
+                                  uint16_t* dVImage, size_t imageLd, size_t batch, size_t heads, size_t newLen, size_t totalLen,
+                                  size_t dim, float scale, size_t oldLen, bf_stream_t stream);
 
 /* The three stages of bf_hip_attention_backward, for callers that need only one of the gradients
  * (frozen keys/values, or a query-only probe) or want to time the stages; same kernels, same results.
@@ -331,6 +371,10 @@ int bf_hip_cross_entropy(const float* logits, const float* target, float* grad, 
 /* softmaxCrossEntropySparse[Accumulate]: target class index per row; indices must already be in range */
 int bf_hip_cross_entropy_sparse(const float* logits, const float* targetIdx, float* grad, float* lossSum,
                                 size_t rows, size_t classes, int accumulate, bf_stream_t stream);
+/* The same with the gradient's bf16 image written too (gradImage[rows, classes], classes a multiple of 8, 16-byte
+ * aligned tensors), for the language-model head's backward GEMMs. */
+int bf_hip_cross_entropy_sparse_img(const float* logits, const float* targetIdx, float* grad, uint16_t* gradImage, float* lossSum,
+                                    size_t rows, size_t classes, int accumulate, bf_stream_t stream);
 /* softmaxCrossEntropyMasked (the CPU backend's loss for masked-language-model training, src/backend/cpu/loss.cpp:149-215;
  * the CUDA backend has no counterpart): as the sparse form, except that a row whose index rounds to -1 is ignored (zero
  * gradient, no loss term) and gradient and loss are averaged over the n rows that are not: grad = (p - onehot) / n, and

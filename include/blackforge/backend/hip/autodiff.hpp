@@ -2,6 +2,7 @@
 // Backward operators with the reference's signatures (include/blackforge/backend/cuda/autodiff.hpp:18-177).
 #include <cmath>
 #include <cstddef>
+#include <cstdint>
 #include <utility>
 
 #include "blackforge/backend/hip/device_tensor.hpp"
@@ -41,8 +42,9 @@ inline MatmulGrad projectionBackward(const DeviceTensor& a, const DeviceTensor& 
     if (mode == 0) {
         check(bf_hip_gemm_f32(0, 1, g.data(), b.data(), r.dA.data(), m, k, n, nullptr));   // dA = g b^T
         check(bf_hip_gemm_f32(1, 0, a.data(), g.data(), r.dB.data(), k, n, m, nullptr));   // dB = a^T g
-    } else {
-        check(bf_hip_matmul_bf16_backward(a.data(), b.data(), g.data(), r.dA.data(), r.dB.data(), m, k, n, mode == 2, nullptr));
+    } else {   // a gradient that carries its bf16 image (made by the kernel that produced it) is not converted again
+        check(bf_hip_matmul_bf16_backward_img(a.data(), a.image(), b.data(), g.data(), g.image(), r.dA.data(), r.dB.data(), m, k, n,
+                                              mode == 2, nullptr));
     }
     return r;
 }
@@ -139,12 +141,15 @@ inline DeviceTensor rmsnormBackward(const DeviceTensor& input, const DeviceTenso
 
 // residualGrad + rmsnormBackward(input, gradOutput) in one pass: how both composite blocks' backward passes end
 // (autodiff.cu:746,794).
-inline DeviceTensor rmsnormBackwardAdd(const DeviceTensor& input, const DeviceTensor& gradOutput, const DeviceTensor& residualGrad) {
+// withImage: the result also carries its bf16 image (DeviceTensor::image()), for a reader that is a bf16 GEMM.
+inline DeviceTensor rmsnormBackwardAdd(const DeviceTensor& input, const DeviceTensor& gradOutput, const DeviceTensor& residualGrad,
+                                       bool withImage = false) {
     require(input.shape() == gradOutput.shape() && residualGrad.shape() == input.shape(), "rmsnormBackward: incompatible shapes on the device");
     require(input.rank() >= 2, "rmsnormBackward: needs a tensor of rank >= 2 on the device");
     DeviceTensor out(input.shape());
-    check(bf_hip_rmsnorm_backward_add(input.data(), gradOutput.data(), residualGrad.data(), out.data(), detail::rowsOf(input),
-                                      detail::lastDim(input), nullptr));
+    std::uint16_t* image = withImage && detail::lastDim(input) % 8 == 0 && input.elementCount() > 0 ? out.attachImage() : nullptr;
+    check(bf_hip_rmsnorm_backward_add_img(input.data(), gradOutput.data(), residualGrad.data(), out.data(), image, detail::rowsOf(input),
+                                          detail::lastDim(input), nullptr));
     return out;
 }
 
@@ -198,27 +203,27 @@ struct FeedForwardGrad {
 inline FeedForwardGrad feedForwardBackwardCached(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
                                                   const DeviceTensor& w2, const DeviceTensor& b2, const FeedForwardCache& cache,
                                                   const DeviceTensor& gradOutput, bool useBf16, Activation act = Activation::Silu,
-                                                  const GradientTargets* into = nullptr) {
+                                                  const GradientTargets* into = nullptr, bool imageForConsumer = false) {
     (void)b2;
     require(gradOutput.shape() == input.shape(), "feedForwardBackward: gradient shape differs from the input");
     const int mode = useBf16 ? 2 : 0;
     if (cache.fused) {
         const std::size_t rows = detail::rowsOf(input), d = detail::lastDim(input), hidden = w1.dim(1);
-        DeviceTensor dNormed(cache.normed.shape()), dW1 = detail::gradientTensor(into, 0, w1.shape()),
+        DeviceTensor dNormed(input.shape()), dW1 = detail::gradientTensor(into, 0, w1.shape()),
                      dB1 = detail::gradientTensor(into, 1, {hidden}), dW2 = detail::gradientTensor(into, 2, w2.shape()),
                      dB2 = detail::gradientTensor(into, 3, {d});
-        check(bf_hip_feedforward_bf16_backward(nullptr, reinterpret_cast<const uint16_t*>(cache.normedImage.data()), w1.data(), w2.data(),
-                                               cache.gemm1.data(), reinterpret_cast<const uint16_t*>(cache.hiddenImage.data()),
-                                               gradOutput.data(), static_cast<int>(act), dNormed.data(), dW1.data(), dB1.data(),
-                                               dW2.data(), dB2.data(), rows, d, hidden, 1, nullptr));
-        DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput);
+        check(bf_hip_feedforward_bf16_backward_img(nullptr, reinterpret_cast<const uint16_t*>(cache.normedImage.data()), w1.data(), w2.data(),
+                                                   cache.gemm1.data(), reinterpret_cast<const uint16_t*>(cache.hiddenImage.data()),
+                                                   gradOutput.data(), gradOutput.image(), static_cast<int>(act), dNormed.data(), dW1.data(),
+                                                   dB1.data(), dW2.data(), dB2.data(), rows, d, hidden, 1, nullptr));
+        DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput, imageForConsumer);
         return FeedForwardGrad{std::move(dInput), std::move(dW1), std::move(dB1), std::move(dW2), std::move(dB2)};
     }
     DeviceTensor dB2 = biasGradientOnly(gradOutput);
     MatmulGrad g2 = detail::projectionBackward(cache.hidden, w2, gradOutput, mode, cache.hidden.shape(), into, 2);
     AddBiasSiluGrad hiddenGrad = addBiasActivationBackward(cache.gemm1, b1, g2.dA, act);
     MatmulGrad g1 = detail::projectionBackward(cache.normed, w1, hiddenGrad.dGemmOutput, mode, cache.normed.shape(), into, 0);
-    DeviceTensor dInput = rmsnormBackwardAdd(input, g1.dA, gradOutput);
+    DeviceTensor dInput = rmsnormBackwardAdd(input, g1.dA, gradOutput, imageForConsumer && useBf16);
     return FeedForwardGrad{std::move(dInput), std::move(g1.dB), std::move(hiddenGrad.dBias), std::move(g2.dB), std::move(dB2)};
 }
 
@@ -260,11 +265,29 @@ namespace detail {
 inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
                                                         const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
                                                         const SelfAttentionCache& cache, const DeviceTensor& gradOutput, int mode,
-                                                        const GradientTargets* into = nullptr) {
+                                                        const GradientTargets* into = nullptr, bool imageForConsumer = false) {
     require(gradOutput.shape() == input.shape(), "selfAttentionBackward: gradient shape differs from the input");
     std::size_t batch = input.dim(0), seq = input.dim(1), dim = input.dim(2);
     float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
     MatmulGrad outGrad = projectionBackward(cache.attnOutput, wout, gradOutput, mode, {batch, seq, dim}, into, 3);
+    if (mode != 0 && cache.normedImage.data() != nullptr) {
+        // the forward pass kept bf16 images of the normalised input and of the attention output; here the attention
+        // gradients go straight to one side-by-side bf16 image [rows, 3 dim] (they have no reader but the two GEMMs below)
+        const std::size_t rows = batch * seq;
+        DeviceTensor gradImage({rows, 3 * dim / 2});   // raw bf16 storage
+        std::uint16_t* gi = reinterpret_cast<std::uint16_t*>(gradImage.data());
+        check(bf_hip_attention_backward_img(outGrad.dA.data(), cache.q.data(), cache.k.data(), cache.v.data(), cache.attnOutput.data(),
+                                            cache.attnM.data(), cache.attnL.data(), nullptr, nullptr, nullptr, gi, gi + dim, gi + 2 * dim, 3 * dim,
+                                            batch, numHeads, seq, seq, dim, scaleFactor, cache.causal ? 0 : seq, nullptr));
+        DeviceTensor dNormed({batch, seq, dim}), dWq = gradientTensor(into, 0, wq.shape()), dWk = gradientTensor(into, 1, wk.shape()),
+                     dWv = gradientTensor(into, 2, wv.shape());
+        const float* weights[3] = {wq.data(), wk.data(), wv.data()};
+        float* weightGrads[3] = {dWq.data(), dWk.data(), dWv.data()};
+        check(bf_hip_matmul_bf16_shared_input_backward_img(nullptr, reinterpret_cast<const std::uint16_t*>(cache.normedImage.data()), weights,
+                                                           nullptr, gi, dNormed.data(), weightGrads, 3, rows, dim, dim, mode == 2, nullptr));
+        DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput, imageForConsumer);
+        return SelfAttentionGrad{std::move(dInput), std::move(dWq), std::move(dWk), std::move(dWv), std::move(outGrad.dB)};
+    }
     FusedAttentionGrad attn = fusedAttentionBackward(outGrad.dA, cache.q, cache.k, cache.v, cache.attnOutput, cache.attnM,
                                                       cache.attnL, numHeads, scaleFactor, cache.causal ? 0 : seq);
     if (mode != 0) {
@@ -277,7 +300,7 @@ inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& inpu
         float* weightGrads[3] = {dWq.data(), dWk.data(), dWv.data()};
         check(bf_hip_matmul_bf16_shared_input_backward(cache.normedFlat.data(), weights, grads, dNormed.data(), weightGrads, 3,
                                                        batch * seq, dim, dim, mode == 2, nullptr));
-        DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput);
+        DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput, imageForConsumer);
         return SelfAttentionGrad{std::move(dInput), std::move(dWq), std::move(dWk), std::move(dWv), std::move(outGrad.dB)};
     }
     MatmulGrad gq = projectionBackward(cache.normedFlat, wq, attn.dQ, mode, {batch * seq, dim}, into, 0);
@@ -292,8 +315,9 @@ inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& inpu
 inline SelfAttentionGrad selfAttentionBackwardCached(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,
                                                       const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
                                                       const SelfAttentionCache& cache, const DeviceTensor& gradOutput, bool useBf16,
-                                                      const GradientTargets* into = nullptr) {
-    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, useBf16 ? 2 : 0, into);
+                                                      const GradientTargets* into = nullptr, bool imageForConsumer = false) {
+    return detail::selfAttentionBackwardFromCache(input, wq, wk, wv, wout, numHeads, cache, gradOutput, useBf16 ? 2 : 0, into,
+                                                  imageForConsumer && useBf16);
 }
 // Stateless variants: recompute the forward first (reference: autodiff.cu:654-700).
 inline SelfAttentionGrad selfAttentionBackward(const DeviceTensor& input, const DeviceTensor& wq, const DeviceTensor& wk,

@@ -3,6 +3,7 @@
 // (include/blackforge/backend/cuda/device_tensor.hpp:19-75): move-only, fromHost/toHost/zeros/clone,
 // reshaped() && transfers ownership.  Memory comes from the library's per-device pool.
 #include <cstddef>
+#include <cstdint>
 #include <utility>
 #include <vector>
 
@@ -24,9 +25,12 @@ public:
     DeviceTensor(const DeviceTensor&) = delete;
     DeviceTensor& operator=(const DeviceTensor&) = delete;
 
-    DeviceTensor(DeviceTensor&& other) noexcept : data_(other.data_), shape_(std::move(other.shape_)), owns_(other.owns_) {
+    DeviceTensor(DeviceTensor&& other) noexcept
+        : data_(other.data_), shape_(std::move(other.shape_)), owns_(other.owns_), image_(other.image_), imageBytes_(other.imageBytes_) {
         other.data_ = nullptr;
         other.shape_.clear();
+        other.image_ = nullptr;
+        other.imageBytes_ = 0;
     }
     DeviceTensor& operator=(DeviceTensor&& other) noexcept {
         if (this != &other) {
@@ -34,11 +38,28 @@ public:
             data_ = other.data_;
             shape_ = std::move(other.shape_);
             owns_ = other.owns_;
+            image_ = other.image_;
+            imageBytes_ = other.imageBytes_;
             other.data_ = nullptr;
             other.shape_.clear();
+            other.image_ = nullptr;
+            other.imageBytes_ = 0;
         }
         return *this;
     }
+
+    // A bf16 image of the same values (round to nearest even, same row-major layout, two bytes per element), for tensors
+    // whose readers include bf16 GEMMs: the kernel that produces the tensor writes the image in the same pass, and the
+    // GEMM entry points take it in place of a conversion pass of their own.  attachImage() gives the tensor an (unwritten)
+    // image buffer from the pool; it travels with the tensor through moves and reshaped() and is returned with it.  Only
+    // for tensors that are not modified after the producing call.  Not part of the reference's DeviceTensor.
+    [[nodiscard]] std::uint16_t* attachImage() {
+        releaseImage();
+        imageBytes_ = elementCount() * sizeof(std::uint16_t);
+        image_ = static_cast<std::uint16_t*>(devicePoolAcquire(imageBytes_));
+        return image_;
+    }
+    [[nodiscard]] const std::uint16_t* image() const { return image_; }
 
     // A non-owning view of device memory that belongs to someone else (an application buffer handed in
     // through a C interface): usable wherever a const DeviceTensor& is expected, never returned to the pool.
@@ -82,8 +103,12 @@ public:
         t.data_ = data_;
         t.shape_ = std::move(newShape);
         t.owns_ = owns_;
+        t.image_ = image_;
+        t.imageBytes_ = imageBytes_;
         data_ = nullptr;
         shape_.clear();
+        image_ = nullptr;
+        imageBytes_ = 0;
         return t;
     }
 
@@ -100,14 +125,22 @@ public:
     }
 
 private:
+    void releaseImage() noexcept {
+        if (image_ != nullptr) bf_hip_pool_release(image_, imageBytes_);
+        image_ = nullptr;
+        imageBytes_ = 0;
+    }
     void release() noexcept {
         if (data_ != nullptr && owns_) bf_hip_pool_release(data_, elementCount() * sizeof(float));
         data_ = nullptr;
+        releaseImage();
     }
 
     float* data_ = nullptr;
     std::vector<std::size_t> shape_;
     bool owns_ = true;
+    std::uint16_t* image_ = nullptr;
+    std::size_t imageBytes_ = 0;
 };
 
 }  // namespace blackforge::backend::hip

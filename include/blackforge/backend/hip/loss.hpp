@@ -2,6 +2,7 @@
 // Loss functions with the reference's signatures (include/blackforge/backend/cuda/loss.hpp:7-70).
 #include <cmath>
 #include <cstddef>
+#include <cstdint>
 #include <string>
 
 #include "blackforge/backend/hip/device_tensor.hpp"
@@ -106,12 +107,15 @@ inline DeviceTensor softmaxCrossEntropyAccumulate(const DeviceTensor& logits, co
 
 // PRECONDITION (caller's responsibility): every index already lies in [0, classes); no range check and no
 // host round trip happen here.
+// gradImage: the gradient also carries its bf16 image (DeviceTensor::image()) when the class count allows it (a multiple
+// of 8): a model with bf16 projections feeds it to the GEMMs of its last layer without a conversion pass.
 inline DeviceTensor softmaxCrossEntropySparseAccumulate(const DeviceTensor& logits, const DeviceTensor& targetIndices,
-                                                         DeviceTensor& lossAccumulator) {
+                                                         DeviceTensor& lossAccumulator, bool gradImage = false) {
     detail::requireSparse("softmaxCrossEntropySparseAccumulate", logits, targetIndices);
     DeviceTensor grad(logits.shape());
-    check(bf_hip_cross_entropy_sparse(logits.data(), targetIndices.data(), grad.data(), lossAccumulator.data(),
-                                      detail::rowsOf(logits), detail::lastDim(logits), 1, nullptr));
+    std::uint16_t* image = gradImage && detail::lastDim(logits) % 8 == 0 && logits.elementCount() > 0 ? grad.attachImage() : nullptr;
+    check(bf_hip_cross_entropy_sparse_img(logits.data(), targetIndices.data(), grad.data(), image, lossAccumulator.data(),
+                                          detail::rowsOf(logits), detail::lastDim(logits), 1, nullptr));
     return grad;
 }
 

@@ -119,7 +119,9 @@ public:
         const DeviceTensor* grad = &outputGrad;
         DeviceTensor owned;
         for (std::size_t li = layers_.size(); li-- > 0;) {
-            owned = applyBackward(layers_[li], *grad, inputRangeTrusted && li == 0);
+            // a block whose gradient goes on to another block's bf16 GEMMs writes that gradient's bf16 image with it
+            const bool imageForConsumer = useBf16_ && li > 0 && isBlock(layers_[li - 1].spec.kind);
+            owned = applyBackward(layers_[li], *grad, inputRangeTrusted && li == 0, imageForConsumer);
             grad = &owned;
         }
     }
@@ -254,7 +256,11 @@ private:
         check(bf_hip_accumulate(target.data(), delta.data(), target.elementCount(), nullptr));
     }
 
-    DeviceTensor applyBackward(LayerState& layer, const DeviceTensor& grad, bool trustedIds) {
+    static bool isBlock(LayerKind kind) {
+        return kind == LayerKind::Attention || kind == LayerKind::BidirectionalAttention || kind == LayerKind::FeedForward;
+    }
+
+    DeviceTensor applyBackward(LayerState& layer, const DeviceTensor& grad, bool trustedIds, bool imageForConsumer) {
         const LayerSpec& s = layer.spec;
         const DeviceTensor& x = layer.cachedInput;
         GradientTargets targets;
@@ -291,7 +297,8 @@ private:
             case LayerKind::Attention:
             case LayerKind::BidirectionalAttention: {   // the cache records which of the two the forward pass was
                 SelfAttentionGrad g = selfAttentionBackwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
-                                                                  layer.params[3].value, s.arg0, layer.attnCache, grad, useBf16_, into);
+                                                                  layer.params[3].value, s.arg0, layer.attnCache, grad, useBf16_, into,
+                                                                  imageForConsumer);
                 accumulate(layer.params[0].grad, g.dWq);
                 accumulate(layer.params[1].grad, g.dWk);
                 accumulate(layer.params[2].grad, g.dWv);
@@ -301,7 +308,7 @@ private:
             case LayerKind::FeedForward: {
                 FeedForwardGrad g = feedForwardBackwardCached(x, layer.params[0].value, layer.params[1].value, layer.params[2].value,
                                                               layer.params[3].value, layer.ffCache, grad, useBf16_,
-                                                              s.arg1 == 1 ? Activation::Gelu : Activation::Silu, into);
+                                                              s.arg1 == 1 ? Activation::Gelu : Activation::Silu, into, imageForConsumer);
                 accumulate(layer.params[0].grad, g.dW1);
                 accumulate(layer.params[1].grad, g.dB1);
                 accumulate(layer.params[2].grad, g.dW2);

@@ -4,6 +4,7 @@
 // a few calls into the C ABI; no computation happens on the host.
 #include <cmath>
 #include <cstddef>
+#include <cstdint>
 #include <string>
 #include <utility>
 #include <vector>
@@ -200,7 +201,7 @@ inline DeviceTensor linearBf16CachedWeight(const DeviceTensor& input, const Devi
 
 // ---- composite blocks ------------------------------------------------------------------------
 struct FeedForwardCache {
-    DeviceTensor normed;  // rmsnorm(input)
+    DeviceTensor normed;  // rmsnorm(input); empty with `fused` (only normedImage exists)
     DeviceTensor gemm1;   // normed @ w1, before bias and activation; with `fused` normed @ w1 + b1
     DeviceTensor hidden;  // act(gemm1 + b1); empty with `fused`
     // bf16 mode with widths that are multiples of 8: the activation is applied where the first GEMM stores its product and
@@ -222,8 +223,8 @@ inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const De
     require(input.rank() >= 2 && w1.rank() == 2 && w2.rank() == 2 && detail::lastDim(input) == w1.dim(0) && w1.dim(1) == w2.dim(0),
             "feedForward: incompatible shapes on the device");
     const int mode = useBf16 ? 2 : 0;
-    cache.normed = rmsnorm(input);
     cache.fused = detail::feedForwardFuses(input, w1, useBf16);
+    if (!cache.fused) cache.normed = rmsnorm(input);
     if (cache.fused) {
         require(b1.rank() == 1 && b1.dim(0) == w1.dim(1), "addBiasSilu: expected input [..., features] and bias [features]");
         require(b2.rank() == 1 && b2.dim(0) == w2.dim(1), "addBiasResidual: expected input [..., features] and bias [features]");
@@ -233,8 +234,11 @@ inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const De
         cache.hidden = DeviceTensor();
         cache.hiddenImage = DeviceTensor({rows, hidden / 2});
         cache.normedImage = DeviceTensor({rows, d / 2});
+        cache.normed = DeviceTensor();
+        // the normalised input has no reader but the GEMMs: it is written as a bf16 image only
+        check(bf_hip_rmsnorm_img(input.data(), nullptr, reinterpret_cast<uint16_t*>(cache.normedImage.data()), rows, d, nullptr));
         DeviceTensor out(input.shape());
-        check(bf_hip_feedforward_bf16(cache.normed.data(), w1.data(), b1.data(), w2.data(), b2.data(), input.data(), static_cast<int>(act),
+        check(bf_hip_feedforward_bf16(nullptr, w1.data(), b1.data(), w2.data(), b2.data(), input.data(), static_cast<int>(act),
                                       cache.gemm1.data(), reinterpret_cast<uint16_t*>(cache.hiddenImage.data()),
                                       reinterpret_cast<uint16_t*>(cache.normedImage.data()), out.data(), rows, d, hidden, 1, nullptr));
         return out;
@@ -270,6 +274,9 @@ inline DeviceTensor feedForwardBf16(const DeviceTensor& input, const DeviceTenso
 }
 
 struct SelfAttentionCache {
+    // bf16 mode with a width that is a multiple of 8: the normalised input exists only as the bf16 image the projections
+    // read (raw storage, [batch*seq, dim / 2]; normedFlat is empty) and attnOutput carries its own image
+    DeviceTensor normedImage;
     DeviceTensor normedFlat;  // [batch*seq, dim]
     DeviceTensor q, k, v;     // [batch, seq, dim]
     DeviceTensor attnOutput;  // [batch, seq, dim], before Wout
@@ -290,6 +297,36 @@ inline DeviceTensor selfAttentionForwardImpl(const char* op, const DeviceTensor&
     std::size_t batch = input.dim(0), seq = input.dim(1), dim = input.dim(2);
     cache.causal = causal;
     float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
+    cache.normedImage = DeviceTensor();
+    if (mode != 0 && dim % 8 == 0 && input.elementCount() > 0) {
+        // bf16 operands are written where they are produced: the normalised input only as an image, the attention output
+        // with an image beside it (the fp32 copy feeds the backward pass); Q, K and V are one GEMM for widths that are
+        // multiples of 256
+        require(wq.rank() == 2 && wq.shape() == wk.shape() && wq.shape() == wv.shape() && wq.dim(0) == dim && wq.dim(1) == dim &&
+                    wout.shape() == wq.shape(),
+                std::string(op) + ": projection weights must be [dim, dim]");
+        const std::size_t rows = batch * seq;
+        cache.normedFlat = DeviceTensor();
+        cache.normedImage = DeviceTensor({rows, dim / 2});
+        const std::uint16_t* normedImage = reinterpret_cast<const std::uint16_t*>(cache.normedImage.data());
+        check(bf_hip_rmsnorm_img(input.data(), nullptr, reinterpret_cast<std::uint16_t*>(cache.normedImage.data()), rows, dim, nullptr));
+        cache.q = DeviceTensor({batch, seq, dim});
+        cache.k = DeviceTensor({batch, seq, dim});
+        cache.v = DeviceTensor({batch, seq, dim});
+        const float* weights[3] = {wq.data(), wk.data(), wv.data()};
+        float* outputs[3] = {cache.q.data(), cache.k.data(), cache.v.data()};
+        check(bf_hip_matmul_bf16_shared_input_img(nullptr, normedImage, weights, outputs, 3, rows, dim, dim, mode == 2, nullptr));
+        cache.attnOutput = DeviceTensor({batch, seq, dim});
+        cache.attnM = DeviceTensor({batch, numHeads, seq});
+        cache.attnL = DeviceTensor({batch, numHeads, seq});
+        std::uint16_t* outImage = cache.attnOutput.attachImage();
+        check(bf_hip_attention_forward_img(cache.q.data(), cache.k.data(), cache.v.data(), cache.attnOutput.data(), outImage, dim,
+                                           cache.attnM.data(), cache.attnL.data(), batch, numHeads, seq, seq, dim, scaleFactor,
+                                           causal ? 0 : seq, nullptr));
+        DeviceTensor out({batch, seq, dim});
+        check(bf_hip_linear_bf16_img(nullptr, outImage, wout.data(), nullptr, input.data(), out.data(), rows, dim, dim, mode == 2, nullptr));
+        return out;
+    }
     cache.normedFlat = rmsnorm(input).reshaped({batch * seq, dim});
     if (mode != 0) {
         // one conversion of the normalised input and (for widths that are multiples of 256) one GEMM for Q, K and V

@@ -114,7 +114,7 @@ TrainRunResult runTraining(Model& model, DatasetT& dataset, const TrainOptions& 
             // the masked loss adds each batch's MEAN (its divisor, the rows not ignored, differs from batch to batch),
             // so the epoch's figure is the mean of the batch means, as in cpu/train_runner.cpp:184-194
             lossDivisor += maskedLoss ? 1 : (sparse || dense) ? output.elementCount() / output.shape().back() : output.elementCount();
-            DeviceTensor grad = sparse       ? softmaxCrossEntropySparseAccumulate(output, target, lossAccumulator)
+            DeviceTensor grad = sparse       ? softmaxCrossEntropySparseAccumulate(output, target, lossAccumulator, model.usesBf16())
                                 : maskedLoss ? softmaxCrossEntropyMaskedAccumulate(output, target, lossAccumulator)
                                 : dense      ? softmaxCrossEntropyAccumulate(output, target, lossAccumulator)
                                              : meanSquaredErrorAccumulate(output, target, lossAccumulator);

@@ -1,0 +1,196 @@
+"""GPU parity of the bf16 operand images that producers write in place of a separate conversion pass, and of the
+projection entry points that consume them.
+
+An image must hold exactly the round-to-nearest-even bf16 of the fp32 values the same kernel writes (checked against the
+oracle's roundToBf16 of the fp32 output), and a projection fed an image must give the bits of the same projection fed
+the fp32 tensor (which the other GEMM tests hold against the oracle)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from parity import assert_bits_equal, assert_close
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+def r(rng, *s, scale=1.0):
+    return rng.standard_normal(s, dtype=f32) * f32(scale)
+
+
+def image_of(hip, shape):
+    """Raw bf16 storage for a [rows, cols] image."""
+    return hip.DeviceTensor(shape, itemsize=2)
+
+
+def as_f32(image_host):
+    return (image_host.astype(np.uint32) << 16).view(f32)
+
+
+def to_image(hip, host):
+    """Device bf16 image of a host fp32 matrix (through the library's own conversion entry point)."""
+    t = hip.DeviceTensor.fromHost(host)
+    img = image_of(hip, host.shape)
+    hip.capi.call("bf_hip_cvt_f32_bf16", t.ptr, img.ptr, host.size, None)
+    return img
+
+
+@pytest.mark.parametrize("rows,features", [(3, 8), (37, 64), (512, 128), (9, 768), (4, 1024), (5, 2048), (3, 8192), (2, 16384), (2, 70000)])
+def test_rmsnorm_images(hip, oracle, rng, rows, features):
+    D, call = hip.DeviceTensor, hip.capi.call
+    x, g, res = r(rng, rows, features, scale=2), r(rng, rows, features), r(rng, rows, features)
+    dx, dg, dres = D.fromHost(x), D.fromHost(g), D.fromHost(res)
+    out, img = D((rows, features)), image_of(hip, (rows, features))
+    call("bf_hip_rmsnorm_img", dx.ptr, out.ptr, img.ptr, rows, features, None)
+    plain = hip.ops.rmsnorm(dx).toHost()
+    assert_bits_equal(out.toHost(), plain, "rmsnorm fp32 output with an image beside it")
+    assert_bits_equal(as_f32(img.toHost()), oracle.roundToBf16(plain), "rmsnorm image")
+    only = image_of(hip, (rows, features))
+    call("bf_hip_rmsnorm_img", dx.ptr, None, only.ptr, rows, features, None)
+    np.testing.assert_array_equal(only.toHost(), img.toHost())
+    # backward with the residual gradient joined and the image of the sum
+    out2, img2 = D((rows, features)), image_of(hip, (rows, features))
+    call("bf_hip_rmsnorm_backward_add_img", dx.ptr, dg.ptr, dres.ptr, out2.ptr, img2.ptr, rows, features, None)
+    plain2 = hip.ops.rmsnormBackwardAdd(dx, dg, dres).toHost()
+    assert_bits_equal(out2.toHost(), plain2, "rmsnormBackwardAdd with an image beside it")
+    assert_bits_equal(as_f32(img2.toHost()), oracle.roundToBf16(plain2), "rmsnormBackwardAdd image")
+
+
+def test_image_shape_requirements(hip):
+    D, call = hip.DeviceTensor, hip.capi.call
+    x, out, img = D.zeros((4, 12)), D((4, 12)), image_of(hip, (4, 12))
+    with pytest.raises(ValueError, match="multiple of 8"):
+        call("bf_hip_rmsnorm_img", x.ptr, out.ptr, img.ptr, 4, 12, None)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        call("bf_hip_rmsnorm_backward_add_img", x.ptr, x.ptr, None, out.ptr, img.ptr, 4, 12, None)
+    call("bf_hip_rmsnorm_img", x.ptr, out.ptr, None, 4, 12, None)   # no image: any width
+
+
+@pytest.mark.parametrize("batch,heads,seq,hd,old_len", [(2, 2, 70, 32, 0), (1, 3, 129, 64, 0), (2, 2, 40, 128, 0), (1, 2, 200, 24, 0),
+                                                        (1, 4, 33, 16, 33), (1, 1, 300, 256, 0)])
+@pytest.mark.parametrize("route", ["hand-over", "recompute"])
+def test_attention_images(hip, oracle, rng, batch, heads, seq, hd, old_len, route):
+    """O with its image; dQ, dK, dV as column slices of one [rows, 3 dim] image with no fp32 gradient written at all."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    dim, scale = heads * hd, float(f32(1.0) / np.sqrt(f32(hd)))
+    q, k, v, go = (r(rng, batch, seq, dim) for _ in range(4))
+    dq_, dk_, dv_, dgo = map(D.fromHost, (q, k, v, go))
+    fwd = hip.ops.fusedAttentionForward(dq_, dk_, dv_, heads, scale, old_len)
+    out, m, l = D((batch, seq, dim)), D((batch, heads, seq)), D((batch, heads, seq))
+    out_img = image_of(hip, (batch * seq, dim))
+    call("bf_hip_attention_forward_img", dq_.ptr, dk_.ptr, dv_.ptr, out.ptr, out_img.ptr, dim, m.ptr, l.ptr, batch, heads, seq, seq, dim,
+         ctypes.c_float(scale), old_len, None)
+    assert_bits_equal(out.toHost(), fwd.output.toHost(), "O with an image beside it")
+    assert_bits_equal(as_f32(out_img.toHost()).reshape(batch, seq, dim), oracle.roundToBf16(fwd.output.toHost()), "O image")
+    hip.capi.call("bf_hip_attention_set_workspace_limit", 0 if route == "recompute" else 2 ** 64 - 1)
+    try:
+        grad = hip.ops.fusedAttentionBackward(dgo, dq_, dk_, dv_, fwd.output, fwd.m, fwd.l, heads, scale, old_len)
+        img = image_of(hip, (batch * seq, 3 * dim))
+        base = img.ptr.value
+        call("bf_hip_attention_backward_img", dgo.ptr, dq_.ptr, dk_.ptr, dv_.ptr, fwd.output.ptr, fwd.m.ptr, fwd.l.ptr, None, None, None,
+             ctypes.c_void_p(base), ctypes.c_void_p(base + 2 * dim), ctypes.c_void_p(base + 4 * dim), 3 * dim, batch, heads, seq, seq, dim,
+             ctypes.c_float(scale), old_len, None)
+    finally:
+        hip.capi.call("bf_hip_attention_set_workspace_limit", 2 ** 64 - 1)
+    got = as_f32(img.toHost()).reshape(batch, seq, 3, dim)
+    for i, (name, t) in enumerate((("dQ", grad.dQ), ("dK", grad.dK), ("dV", grad.dV))):
+        assert_bits_equal(got[:, :, i], oracle.roundToBf16(t.toHost()), name + " image")
+
+
+@pytest.mark.parametrize("rows,classes", [(5, 16), (7, 1000), (300, 256), (3, 32000), (2, 40000)])
+def test_cross_entropy_gradient_image(hip, oracle, rng, rows, classes):
+    D, call = hip.DeviceTensor, hip.capi.call
+    logits = r(rng, rows, classes, scale=3)
+    idx = rng.integers(0, classes, rows).astype(f32)
+    dl, di = D.fromHost(logits), D.fromHost(idx)
+    plain = hip.ops.softmaxCrossEntropySparse(dl, di)
+    grad, img, loss = D((rows, classes)), image_of(hip, (rows, classes)), D.zeros((1,))
+    call("bf_hip_cross_entropy_sparse_img", dl.ptr, di.ptr, grad.ptr, img.ptr, loss.ptr, rows, classes, 0, None)
+    assert_bits_equal(grad.toHost(), plain.grad.toHost(), "CE gradient with an image beside it")
+    assert_bits_equal(as_f32(img.toHost()), oracle.roundToBf16(plain.grad.toHost()), "CE gradient image")
+    assert abs(loss.toHost()[0] / rows - plain.value) <= 1e-6 * abs(plain.value)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        call("bf_hip_cross_entropy_sparse_img", dl.ptr, di.ptr, grad.ptr, img.ptr, loss.ptr, rows, classes - 4, 0, None)
+
+
+# (m, k, n): the small-tile route with transposed images, a ragged one, and the large-tile routes (fragments transposed in LDS)
+GEMM_SHAPES = [(64, 40, 24), (300, 72, 520), (4100, 136, 264), (8192, 256, 768), (6001, 520, 1032)]
+
+
+@pytest.mark.parametrize("m,k,n", GEMM_SHAPES)
+def test_projections_fed_with_images(hip, rng, m, k, n):
+    """linear, its two gradients: fp32 operands against the same operands as bf16 images, bit for bit."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    a, w, g, bias, res = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, m, n), r(rng, n), r(rng, m, n)
+    da, dw, dg, db, dres = map(D.fromHost, (a, w, g, bias, res))
+    a_img, g_img = to_image(hip, a), to_image(hip, g)
+    out0, out1 = D((m, n)), D((m, n))
+    call("bf_hip_linear_bf16", da.ptr, dw.ptr, db.ptr, dres.ptr, out0.ptr, m, k, n, 0, None)
+    call("bf_hip_linear_bf16_img", None, a_img.ptr, dw.ptr, db.ptr, dres.ptr, out1.ptr, m, k, n, 0, None)
+    assert_bits_equal(out1.toHost(), out0.toHost(), "linear from an image")
+    dA0, dB0, dA1, dB1 = D((m, k)), D((k, n)), D((m, k)), D((k, n))
+    call("bf_hip_matmul_bf16_backward", da.ptr, dw.ptr, dg.ptr, dA0.ptr, dB0.ptr, m, k, n, 0, None)
+    call("bf_hip_matmul_bf16_backward_img", None, a_img.ptr, dw.ptr, None, g_img.ptr, dA1.ptr, dB1.ptr, m, k, n, 0, None)
+    assert_bits_equal(dA1.toHost(), dA0.toHost(), "dA from images")
+    assert_bits_equal(dB1.toHost(), dB0.toHost(), "dB from images")
+    # mixed: one operand as an image, the other in fp32; and a single gradient requested
+    call("bf_hip_matmul_bf16_backward_img", da.ptr, None, dw.ptr, dg.ptr, g_img.ptr, dA1.ptr, dB1.ptr, m, k, n, 0, None)
+    assert_bits_equal(dB1.toHost(), dB0.toHost(), "dB from the gradient's image and the fp32 input")
+    only = D((k, n))
+    call("bf_hip_matmul_bf16_backward_img", None, a_img.ptr, dw.ptr, None, g_img.ptr, None, only.ptr, m, k, n, 0, None)
+    assert_bits_equal(only.toHost(), dB0.toHost(), "dB alone from images")
+
+
+@pytest.mark.parametrize("m,k,n,count", [(50, 40, 24, 3), (300, 136, 256, 3), (4100, 256, 256, 3), (8192, 520, 256, 3), (260, 72, 512, 2),
+                                         (64, 32, 48, 1)])
+def test_shared_input_projections_fed_with_images(hip, rng, m, k, n, count):
+    D, call = hip.DeviceTensor, hip.capi.call
+    a = r(rng, m, k)
+    ws = [r(rng, k, n, scale=0.1) for _ in range(count)]
+    gs = [r(rng, m, n) for _ in range(count)]
+    da, dws, dgs = D.fromHost(a), [D.fromHost(w) for w in ws], [D.fromHost(g) for g in gs]
+    arr = lambda ts: (ctypes.c_void_p * count)(*[t.ptr for t in ts])
+    a_img = to_image(hip, a)
+    g_img = to_image(hip, np.concatenate(gs, axis=1))   # side by side: [m, count * n]
+    c0, c1 = [D((m, n)) for _ in range(count)], [D((m, n)) for _ in range(count)]
+    call("bf_hip_matmul_bf16_shared_input", da.ptr, arr(dws), arr(c0), count, m, k, n, 0, None)
+    call("bf_hip_matmul_bf16_shared_input_img", None, a_img.ptr, arr(dws), arr(c1), count, m, k, n, 0, None)
+    for x, y in zip(c0, c1):
+        assert_bits_equal(y.toHost(), x.toHost(), "shared-input product from an image")
+    dA0, dA1 = D((m, k)), D((m, k))
+    dB0, dB1 = [D((k, n)) for _ in range(count)], [D((k, n)) for _ in range(count)]
+    call("bf_hip_matmul_bf16_shared_input_backward", da.ptr, arr(dws), arr(dgs), dA0.ptr, arr(dB0), count, m, k, n, 0, None)
+    call("bf_hip_matmul_bf16_shared_input_backward_img", None, a_img.ptr, arr(dws), None, g_img.ptr, dA1.ptr, arr(dB1), count, m, k, n, 0, None)
+    assert_bits_equal(dA1.toHost(), dA0.toHost(), "dA from images")
+    for x, y in zip(dB0, dB1):
+        assert_bits_equal(y.toHost(), x.toHost(), "dB from images")
+
+
+@pytest.mark.parametrize("m,d,hidden,act", [(64, 32, 128, 0), (300, 72, 264, 1), (4096, 256, 1024, 0), (8192, 768, 3072, 1)])
+def test_feed_forward_fed_with_images(hip, rng, m, d, hidden, act):
+    D, ops, call = hip.DeviceTensor, hip.ops, hip.capi.call
+    x, w1, b1 = r(rng, m, d), r(rng, d, hidden, scale=0.1), r(rng, hidden, scale=0.5)
+    w2, b2, res, g = r(rng, hidden, d, scale=0.1), r(rng, d), r(rng, m, d), r(rng, m, d)
+    dx, dw1, db1, dw2, db2, dres, dg = map(D.fromHost, (x, w1, b1, w2, b2, res, g))
+    out0, z0, h0, xi0 = ops.feedForwardBf16Fused(dx, dw1, db1, dw2, db2, dres, act)
+    x_img, g_img = to_image(hip, x), to_image(hip, g)
+    z1, h1, out1 = D((m, hidden)), D((m, hidden // 2)), D((m, d))
+    call("bf_hip_feedforward_bf16", None, dw1.ptr, db1.ptr, dw2.ptr, db2.ptr, dres.ptr, act, z1.ptr, h1.ptr, x_img.ptr, out1.ptr, m, d, hidden, 0, None)
+    assert_bits_equal(out1.toHost(), out0.toHost(), "feed-forward from the input's image")
+    assert_bits_equal(z1.toHost(), z0.toHost(), "pre-activation from the input's image")
+    ref = ops.feedForwardBf16FusedBackward(dx, None, dw1, dw2, z0, h0, dg, act)
+    outs = [D((m, d)), D(w1.shape), D((hidden,)), D(w2.shape), D((d,))]
+    call("bf_hip_feedforward_bf16_backward_img", None, x_img.ptr, dw1.ptr, dw2.ptr, z0.ptr, h0.ptr, dg.ptr, g_img.ptr, act,
+         *[t.ptr for t in outs], m, d, hidden, 0, None)
+    for got, exp, name in zip(outs, ref, ("dX", "dW1", "dB1", "dW2", "dB2")):
+        assert_bits_equal(got.toHost(), exp.toHost(), name + " from images")
+    # without the fp32 gradient only the bias gradient of the second projection is unavailable
+    outs2 = [D((m, d)), D(w1.shape), D((hidden,)), D(w2.shape)]
+    call("bf_hip_feedforward_bf16_backward_img", None, x_img.ptr, dw1.ptr, dw2.ptr, z0.ptr, h0.ptr, None, g_img.ptr, act,
+         *[t.ptr for t in outs2], None, m, d, hidden, 0, None)
+    for got, exp, name in zip(outs2, ref, ("dX", "dW1", "dB1", "dW2")):
+        assert_bits_equal(got.toHost(), exp.toHost(), name + " from the gradient image alone")
+    with pytest.raises(ValueError, match="dB2"):
+        call("bf_hip_feedforward_bf16_backward_img", None, x_img.ptr, dw1.ptr, dw2.ptr, z0.ptr, h0.ptr, None, g_img.ptr, act,
+             *[t.ptr for t in outs], m, d, hidden, 0, None)
