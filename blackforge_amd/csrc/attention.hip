@@ -3,13 +3,17 @@
 // Layout: q [batch,newLen,dim], k/v [batch,totalLen,dim], heads contiguous in dim.  Query row i
 // (absolute position oldLen+i) attends to keys j <= oldLen+i.
 //
-// Three MFMA kernels, all with 256-thread workgroups (4 wavefronts, one per SIMD), 32 rows per wave:
+// MFMA kernels, all with 256-thread workgroups (4 wavefronts, one per SIMD), 32 rows per wave:
 //   forward : a workgroup owns 128 query rows, streams K/V tiles through LDS (double buffered, one barrier
 //             per tile, next tile's global loads in flight in registers), online softmax.
-//   dQ      : same ownership; recomputes P from the saved statistics, accumulates dQ in registers.
 //   dK/dV   : a workgroup owns 128 keys (K, V and both accumulators live in registers), streams
-//             Q/dO tiles through LDS, writes dK and dV once.  No atomics anywhere, so gradients are
-//             bit-reproducible; the price is that S and dP are recomputed in both backward kernels.
+//             Q/dO tiles through LDS, writes dK and dV once.  On the default route it also leaves
+//             dS = P o (dP - D) behind in a hand-over buffer [batch, heads, totalLen, newLen].
+//   dQ      : default route: one contraction dQ = scale * dS * K over the hand-over buffer (no exp, no second
+//             pass over Q and dO).  When the buffer would exceed the workspace limit, the recompute route: the
+//             same ownership as forward, P rebuilt from the saved statistics, and the dK/dV kernel keeps dS to itself.
+// No atomics anywhere, so gradients are bit-reproducible.  Every kernel can write a bf16 image of its result beside
+// (or instead of) the fp32 tensor, for the projections that read it next.
 //
 // Orientation trick (what makes the softmax cheap on 64-wide waves).  With the 32x32x2 MFMA
 //   A: lane l holds A[i = l%32][k = l/32]      B: lane l holds B[k = l/32][j = l%32]

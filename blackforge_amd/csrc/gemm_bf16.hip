@@ -1014,58 +1014,96 @@ int transposeImage(const unsigned short* in, unsigned short* out, size_t rows, s
 // produces all their products) and 3 = their plain images side by side ([rows, count*cols], the Bt operand of
 // the one GEMM that sums their input gradients).
 struct CachedWeight {
-    size_t generation;
+    size_t generation;   // the generation whose weights the image holds; 0 = never filled
     void* buffer;
     size_t bytes;
 };
-size_t g_generation = 0;
+size_t g_generation = 1;
 using WeightKey = std::tuple<int, const float*, const float*, const float*, int>;
 std::map<WeightKey, CachedWeight>& weightCache() {
     static std::map<WeightKey, CachedWeight> cache;
     return cache;
 }
 
-int fillWeightImage(const float* const* w, size_t count, size_t rows, size_t cols, int layout, unsigned short* image, hipStream_t s) {
+// `plain`: for the transposed layouts (1, 2) the plain counterpart (0, 3) written in the same pass, or NULL.
+int fillWeightImage(const float* const* w, size_t count, size_t rows, size_t cols, int layout, unsigned short* image, unsigned short* plain,
+                    hipStream_t s) {
     int st = BF_OK;
     for (size_t i = 0; i < count && st == BF_OK; ++i) {
         if (layout == 0) st = convertPlain(w[i], image, rows, cols, s);
-        else if (layout == 1) st = convertTransposed(w[i], image, rows, cols, s);
-        else if (layout == 2) st = convertTransposed(w[i], image + i * cols * pad8(rows), rows, cols, s);
+        else if (layout == 1) st = convertTransposed(w[i], image, rows, cols, s, true, plain, pad8(cols));
+        else if (layout == 2) st = convertTransposed(w[i], image + i * cols * pad8(rows), rows, cols, s, true, plain ? plain + i * cols : nullptr, count * cols);
         else st = convertPlain(w[i], image + i * cols, rows, cols, s, count * cols);   // cols % 8 == 0 checked by the caller
     }
     return st;
 }
 
-// Returns the bf16 image of `count` weights w[i][rows, cols] in `layout`.  With `cache` the image is kept;
-// otherwise it is a scratch buffer the caller releases with bf_hip_pool_release(image, bytes).
-int weightImage(const float* const* w, size_t count, size_t rows, size_t cols, int layout, bool cache, hipStream_t s,
-                unsigned short** image, size_t* imageBytes) {
-    size_t elems = (layout == 0 || layout == 3) ? rows * pad8(cols) * count : count * cols * pad8(rows);
-    size_t bytes = elems * sizeof(unsigned short);
-    *imageBytes = bytes;
-    int dev = 0;
-    BF_HIP_TRY(hipGetDevice(&dev));
-    void* buf = nullptr;
-    if (cache) {
-        WeightKey key{dev, w[0], count > 1 ? w[1] : nullptr, count > 2 ? w[2] : nullptr, layout};
-        auto it = weightCache().find(key);
-        if (it != weightCache().end() && it->second.generation == g_generation && it->second.bytes == bytes) {
-            *image = static_cast<unsigned short*>(it->second.buffer);
-            return BF_OK;
-        }
-        if (it != weightCache().end() && it->second.bytes == bytes) buf = it->second.buffer;   // refresh in place
-        else {
-            if (it != weightCache().end()) bf_hip_pool_release(it->second.buffer, it->second.bytes);
-            int st = bf_hip_pool_acquire(bytes, &buf);
-            if (st != BF_OK) return st;
-        }
-        weightCache()[key] = CachedWeight{g_generation, buf, bytes};
-    } else {
+size_t weightImageBytes(size_t count, size_t rows, size_t cols, int layout) {
+    return ((layout == 0 || layout == 3) ? rows * pad8(cols) * count : count * cols * pad8(rows)) * sizeof(unsigned short);
+}
+
+// The cache entry of `key` with a buffer of `bytes` (acquired, or re-acquired when the size changed); its generation
+// says whether the buffer's contents are current.  Entries stay where they are in the map, so the pointer holds.
+int cacheSlot(const WeightKey& key, size_t bytes, CachedWeight** slot) {
+    auto& cache = weightCache();
+    auto it = cache.find(key);
+    if (it != cache.end() && it->second.bytes != bytes) {
+        bf_hip_pool_release(it->second.buffer, it->second.bytes);
+        cache.erase(it);
+        it = cache.end();
+    }
+    if (it == cache.end()) {
+        void* buf = nullptr;
         int st = bf_hip_pool_acquire(bytes, &buf);
         if (st != BF_OK) return st;
+        it = cache.emplace(key, CachedWeight{0, buf, bytes}).first;
     }
-    *image = static_cast<unsigned short*>(buf);
-    return fillWeightImage(w, count, rows, cols, layout, *image, s);
+    *slot = &it->second;
+    return BF_OK;
+}
+
+// Returns the bf16 image of `count` weights w[i][rows, cols] in `layout`.  With `cache` the image is kept;
+// otherwise it is a scratch buffer the caller releases with bf_hip_pool_release(image, bytes).  A cached transposed
+// image (the forward operand) is filled together with its plain counterpart (the operand of the input-gradient
+// product of the same weights), one pass over the fp32 weights for both.  An entry is marked current only once its
+// conversion has been launched, so a failed launch is never served as an image.
+int weightImage(const float* const* w, size_t count, size_t rows, size_t cols, int layout, bool cache, hipStream_t s,
+                unsigned short** image, size_t* imageBytes) {
+    const size_t bytes = weightImageBytes(count, rows, cols, layout);
+    *imageBytes = bytes;
+    if (!cache) {
+        void* buf = nullptr;
+        int st = bf_hip_pool_acquire(bytes, &buf);
+        if (st != BF_OK) return st;
+        st = fillWeightImage(w, count, rows, cols, layout, static_cast<unsigned short*>(buf), nullptr, s);
+        if (st != BF_OK) {
+            bf_hip_pool_release(buf, bytes);
+            return st;
+        }
+        *image = static_cast<unsigned short*>(buf);
+        return BF_OK;
+    }
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    const float* w1 = count > 1 ? w[1] : nullptr;
+    const float* w2 = count > 2 ? w[2] : nullptr;
+    CachedWeight* slot = nullptr;
+    int st = cacheSlot(WeightKey{dev, w[0], w1, w2, layout}, bytes, &slot);
+    if (st != BF_OK) return st;
+    *image = static_cast<unsigned short*>(slot->buffer);
+    if (slot->generation == g_generation) return BF_OK;
+    CachedWeight* mate = nullptr;
+    if (layout == 1 || (layout == 2 && cols % 8 == 0)) {
+        const int mateLayout = layout == 1 ? 0 : 3;
+        st = cacheSlot(WeightKey{dev, w[0], w1, w2, mateLayout}, weightImageBytes(count, rows, cols, mateLayout), &mate);
+        if (st != BF_OK) return st;
+        if (mate->generation == g_generation) mate = nullptr;   // already current
+    }
+    st = fillWeightImage(w, count, rows, cols, layout, *image, mate ? static_cast<unsigned short*>(mate->buffer) : nullptr, s);
+    if (st != BF_OK) return st;
+    slot->generation = g_generation;
+    if (mate) mate->generation = g_generation;
+    return BF_OK;
 }
 int weightImage(const float* w, size_t rows, size_t cols, bool transposed, bool cache, hipStream_t s, unsigned short** image,
                 size_t* imageBytes) {
@@ -1565,7 +1603,18 @@ int bf_hip_feedforward_bf16_backward_img(const float* x, const uint16_t* xImage,
 }
 
 int bf_hip_invalidate_bf16_weight_cache(void) {
-    ++g_generation;
+    // Images that nobody asked for during the generation that ends here belong to weights that are gone (a destroyed
+    // model) or idle: their buffers go back to the pool.  An idle weight that is used again just converts once more.
+    auto& cache = bf::weightCache();
+    for (auto it = cache.begin(); it != cache.end();) {
+        if (it->second.generation != bf::g_generation) {
+            bf_hip_pool_release(it->second.buffer, it->second.bytes);
+            it = cache.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    ++bf::g_generation;
     return BF_OK;
 }
 

@@ -5,6 +5,7 @@
 //   "BFCKPT1\0" | u32 parameter count | per parameter: u32 name length, name bytes, u32 rank, u64 dims[rank], fp32 data
 // Parameters are matched by NAME on load; a name the model does not have, a shape that differs, or a short file is
 // a std::runtime_error, and parameters the file does not mention keep their values.
+#include <algorithm>
 #include <cerrno>
 #include <cstdint>
 #include <cstring>
@@ -48,40 +49,109 @@ inline void saveCheckpoint(Model& model, const std::string& path) {
     if (!out) throw std::runtime_error("saveCheckpoint: write to '" + path + "' failed");
 }
 
-inline void loadCheckpoint(Model& model, const std::string& path) {
-    std::ifstream in(path, std::ios::binary);
-    if (!in) throw std::runtime_error("loadCheckpoint: cannot open '" + path + "'");
-    char magic[8];
-    in.read(magic, sizeof(magic));
-    if (!in || std::memcmp(magic, detail::kCheckpointMagic, sizeof(magic)) != 0) {
-        throw std::runtime_error("loadCheckpoint: '" + path + "' is not a BlackForge checkpoint");
+namespace detail {
+
+// One parameter of a checkpoint file: where its values lie, not the values.
+struct CheckpointRecord {
+    std::string name;
+    std::vector<std::size_t> shape;
+    std::size_t elementCount = 0;
+    std::streamoff dataOffset = 0;
+};
+
+// The table of contents of a BFCKPT1 file.  Walks the records by seeking over their values and checks every length
+// against the size of the file, so that a truncated or corrupt file is refused before anything is read into a model.
+class CheckpointIndex {
+public:
+    explicit CheckpointIndex(const std::string& path) : path_(path), in_(path, std::ios::binary | std::ios::ate) {
+        if (!in_) throw std::runtime_error("loadCheckpoint: cannot open '" + path + "'");
+        fileBytes_ = static_cast<std::uint64_t>(in_.tellg());
+        in_.seekg(0);
+        char magic[sizeof(kCheckpointMagic)] = {};
+        in_.read(magic, sizeof(magic));
+        if (!in_ || std::memcmp(magic, kCheckpointMagic, sizeof(magic)) != 0)
+            throw std::runtime_error("loadCheckpoint: '" + path + "' is not a BlackForge checkpoint");
+        const std::uint32_t count = take<std::uint32_t>();
+        records_.reserve(std::min<std::uint32_t>(count, 1U << 16));
+        for (std::uint32_t i = 0; i < count; ++i) records_.push_back(nextRecord());
     }
+
+    [[nodiscard]] const std::vector<CheckpointRecord>& records() const { return records_; }
+
+    // The values of one record, read into `host` (resized to fit).
+    void readValues(const CheckpointRecord& record, std::vector<float>& host) {
+        host.resize(record.elementCount);
+        in_.clear();
+        in_.seekg(record.dataOffset);
+        in_.read(reinterpret_cast<char*>(host.data()), static_cast<std::streamsize>(record.elementCount * sizeof(float)));
+        if (!in_) corrupt();
+    }
+
+private:
+    [[noreturn]] void corrupt() const { throw std::runtime_error("loadCheckpoint: '" + path_ + "' is truncated or corrupt"); }
+    [[nodiscard]] std::uint64_t remaining() {
+        const std::uint64_t at = static_cast<std::uint64_t>(in_.tellg());
+        return at <= fileBytes_ ? fileBytes_ - at : 0;
+    }
+    template <typename T> T take() {
+        if (remaining() < sizeof(T)) corrupt();
+        return readRaw<T>(in_);
+    }
+    CheckpointRecord nextRecord() {
+        CheckpointRecord record;
+        const std::uint32_t nameLength = take<std::uint32_t>();
+        if (nameLength > remaining()) corrupt();
+        record.name.resize(nameLength);
+        in_.read(record.name.data(), nameLength);
+        const std::uint32_t rank = take<std::uint32_t>();
+        if (std::uint64_t(rank) * sizeof(std::uint64_t) > remaining()) corrupt();
+        record.shape.resize(rank);
+        std::uint64_t elements = 1;
+        for (std::size_t& extent : record.shape) {
+            const std::uint64_t value = take<std::uint64_t>();
+            if (value != 0 && elements > fileBytes_ / value) corrupt();   // more values than the file has bytes
+            elements *= value;
+            extent = static_cast<std::size_t>(value);
+        }
+        if (elements > remaining() / sizeof(float)) corrupt();
+        record.elementCount = static_cast<std::size_t>(elements);
+        record.dataOffset = in_.tellg();
+        in_.seekg(static_cast<std::streamoff>(elements * sizeof(float)), std::ios::cur);
+        return record;
+    }
+
+    std::string path_;
+    std::ifstream in_;
+    std::uint64_t fileBytes_ = 0;
+    std::vector<CheckpointRecord> records_;
+};
+
+}  // namespace detail
+
+// Loads in two phases.  First the file's table of contents is matched against the model: every record must name a
+// parameter of the model with the same shape (the reference's conditions, src/backend/cpu/checkpoint.cpp:118-129), and a
+// file that fails leaves the model exactly as it was.  Then the values are copied over the parameters' existing device
+// buffers, so the addresses that the bf16 weight-image cache and a captured step hold stay valid.
+inline void loadCheckpoint(Model& model, const std::string& path) {
+    detail::CheckpointIndex index(path);
     std::unordered_map<std::string, Parameter*> byName;
     for (Parameter* p : model.parameters()) byName[p->name] = p;
-    const std::uint32_t count = detail::readRaw<std::uint32_t>(in);
-    for (std::uint32_t i = 0; i < count; ++i) {
-        const std::uint32_t nameLength = detail::readRaw<std::uint32_t>(in);
-        if (!in || nameLength > (1U << 20)) throw std::runtime_error("loadCheckpoint: '" + path + "' is truncated or corrupt");
-        std::string name(nameLength, '\0');
-        in.read(name.data(), nameLength);
-        const std::uint32_t rank = detail::readRaw<std::uint32_t>(in);
-        if (!in || rank > 16) throw std::runtime_error("loadCheckpoint: '" + path + "' is truncated or corrupt");
-        std::vector<std::size_t> shape(rank);
-        std::size_t elementCount = 1;
-        for (std::uint32_t d = 0; d < rank; ++d) {
-            shape[d] = static_cast<std::size_t>(detail::readRaw<std::uint64_t>(in));
-            elementCount *= shape[d];
-        }
-        auto it = byName.find(name);
-        if (!in) throw std::runtime_error("loadCheckpoint: '" + path + "' is truncated or corrupt");
-        if (it == byName.end()) throw std::runtime_error("loadCheckpoint: the model has no parameter called '" + name + "'");
-        if (it->second->value.shape() != shape) throw std::runtime_error("loadCheckpoint: shape mismatch for '" + name + "'");
-        std::vector<float> data(elementCount);
-        in.read(reinterpret_cast<char*>(data.data()), static_cast<std::streamsize>(elementCount * sizeof(float)));
-        if (!in) throw std::runtime_error("loadCheckpoint: '" + path + "' is truncated or corrupt");
-        it->second->value = DeviceTensor::fromHost(runtime::Tensor(shape, std::move(data)));
+    std::vector<Parameter*> targets;
+    targets.reserve(index.records().size());
+    for (const detail::CheckpointRecord& record : index.records()) {
+        const auto found = byName.find(record.name);
+        if (found == byName.end()) throw std::runtime_error("loadCheckpoint: the model has no parameter called '" + record.name + "'");
+        if (found->second->value.shape() != record.shape) throw std::runtime_error("loadCheckpoint: shape mismatch for '" + record.name + "'");
+        targets.push_back(found->second);
     }
-    // the next Model::forward() refreshes the bf16 weight images, as after an optimizer step
+    std::vector<float> staging;
+    for (std::size_t i = 0; i < targets.size(); ++i) {
+        const detail::CheckpointRecord& record = index.records()[i];
+        if (record.elementCount == 0) continue;
+        index.readValues(record, staging);
+        check(bf_hip_memcpy_h2d(targets[i]->value.data(), staging.data(), record.elementCount * sizeof(float)));
+    }
+    invalidateBf16WeightCache();   // images of the old values must not outlive them
 }
 
 }  // namespace blackforge::backend::hip

@@ -194,3 +194,46 @@ def test_feed_forward_fed_with_images(hip, rng, m, d, hidden, act):
     with pytest.raises(ValueError, match="dB2"):
         call("bf_hip_feedforward_bf16_backward_img", None, x_img.ptr, dw1.ptr, dw2.ptr, z0.ptr, h0.ptr, None, g_img.ptr, act,
              *[t.ptr for t in outs], m, d, hidden, 0, None)
+
+
+def in_use(hip):
+    stats = hip.capi.PoolStats()
+    hip.capi.call("bf_hip_pool_stats", ctypes.byref(stats))
+    return stats.bytes_in_use
+
+
+def test_weight_image_cache_fills_pairs_and_lets_go_of_idle_weights(hip, rng):
+    """The cached forward image of a weight comes with the plain image its input-gradient product reads (same bits as
+    the uncached route); images of weights that sat out a whole generation go back to the pool."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    m, k, n = 300, 136, 264
+    a, w, g = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, m, n)
+    da, dw, dg = map(D.fromHost, (a, w, g))
+    call("bf_hip_invalidate_bf16_weight_cache")
+    call("bf_hip_invalidate_bf16_weight_cache")   # two in a row: nothing of earlier tests is left in the cache
+    out0, out1, dA0, dA1 = D((m, n)), D((m, n)), D((m, k)), D((m, k))
+    base = in_use(hip)   # the pool counts whole size classes, so compare levels rather than sums of tensor sizes
+    call("bf_hip_linear_bf16", da.ptr, dw.ptr, None, None, out0.ptr, m, k, n, 0, None)
+    assert in_use(hip) == base, "the uncached route returns its images"
+    call("bf_hip_linear_bf16", da.ptr, dw.ptr, None, None, out1.ptr, m, k, n, 1, None)
+    assert_bits_equal(out1.toHost(), out0.toHost(), "linear with a cached weight image")
+    assert in_use(hip) - base >= 2 * (k * n * 2), "the transposed image and its plain counterpart are both held"
+    call("bf_hip_matmul_bf16_backward", da.ptr, dw.ptr, dg.ptr, dA0.ptr, None, m, k, n, 0, None)
+    before = in_use(hip)
+    call("bf_hip_matmul_bf16_backward", da.ptr, dw.ptr, dg.ptr, dA1.ptr, None, m, k, n, 1, None)
+    assert in_use(hip) == before, "the plain image was there already"
+    assert_bits_equal(dA1.toHost(), dA0.toHost(), "dA from the plain image that the forward pass left")
+    # the weights change (an optimizer step): the next forward must not be served the old image
+    w2 = r(rng, k, n, scale=0.1)
+    hip.capi.call("bf_hip_memcpy_h2d", dw.ptr, w2.ctypes.data_as(ctypes.c_void_p), w2.nbytes)
+    call("bf_hip_invalidate_bf16_weight_cache")
+    call("bf_hip_linear_bf16", da.ptr, dw.ptr, None, None, out0.ptr, m, k, n, 0, None)
+    call("bf_hip_linear_bf16", da.ptr, dw.ptr, None, None, out1.ptr, m, k, n, 1, None)
+    assert_bits_equal(out1.toHost(), out0.toHost(), "linear after the weights changed")
+    call("bf_hip_matmul_bf16_backward", da.ptr, dw.ptr, dg.ptr, dA0.ptr, None, m, k, n, 0, None)
+    call("bf_hip_matmul_bf16_backward", da.ptr, dw.ptr, dg.ptr, dA1.ptr, None, m, k, n, 1, None)
+    assert_bits_equal(dA1.toHost(), dA0.toHost(), "dA after the weights changed")
+    # a generation in which nobody asks for them, and the images are returned
+    call("bf_hip_invalidate_bf16_weight_cache")
+    call("bf_hip_invalidate_bf16_weight_cache")
+    assert in_use(hip) == base, "only this test's own tensors are still checked out"
