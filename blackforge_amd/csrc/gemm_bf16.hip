@@ -16,6 +16,7 @@
 // cutting K into slices that a second kernel adds up in a fixed order (small products).
 #include "common.hpp"
 
+#include <atomic>
 #include <map>
 #include <unordered_map>
 
@@ -122,6 +123,7 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(const float* __
 // wavefront touch every bank once.  Rows past the end of an operand are clamped to its last row (their
 // products are never stored) and chunks past the end of the K range read as zero, so neither kernel has
 // a branch around a load.
+std::atomic<int> g_ntRoute{BF_GEMM_ROUTE_AUTO};
 constexpr int BKK = 64;
 constexpr int LDS_ROW = BKK + 8;
 
@@ -445,21 +447,26 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
     storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
-// 128 x 256 tiles on sixteen wavefronts (four per SIMD, each with a 32 x 64 share), one barrier per K step: while step T
-// is multiplied out of LDS buffer T&1 (fragments of the next 16-deep slice are read while the current one is multiplied),
-// the registers holding step T+1 go to the other buffer and the loads of step T+2 are issued.  The K loop costs what the
-// eight-wavefront ping-pong costs for a tile of this size (the LDS pipe bounds both), but filling and draining it does
-// not: sixteen wavefronts fetch the first step and store the tile in half the time, and no group waits a phase for the
-// other.  Products with a short contraction, whose tiles live for twenty microseconds, are several microseconds faster per
-// round of tiles; long contractions stay on the 256-row ping-pong kernel, which moves fewer operand bytes per MFMA.
-template <int XCD_ORDER>
-__global__ void __launch_bounds__(1024, 4) gemmBf16SixteenWaveKernel(const unsigned short* __restrict__ A,
-                                                                    const unsigned short* __restrict__ Bt, Epilogue epi, int M,
-                                                                    int N, int K, int lda, int ldb, int gmLog, int gnLog) {
-    constexpr int BM = 128, BN = 256, TM = 1, TN = 2;
-    extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
-    unsigned short* as = lds;                        // [2][128][LDS_ROW]
-    unsigned short* bs = lds + 2 * BM * LDS_ROW;     // [2][256][LDS_ROW]
+// 128-row tiles on twelve or sixteen wavefronts (three or four per SIMD, each with a 32 x 64 share: tiles 192 or 256
+// wide), one barrier per K step: while step T is multiplied out of LDS buffer T&1 (fragments of the next 16-deep slice are
+// read while the current one is multiplied), the registers holding step T+1 go to the other buffer and the loads of step
+// T+2 are issued.  The K loop costs what the eight-wavefront ping-pong costs for a tile of this size (the LDS pipe bounds
+// both), but filling and draining it does not: all wavefronts fetch the first step and store the tile together, and no
+// group waits a phase for the other.  Products with a short contraction, whose tiles live for twenty microseconds, are
+// several microseconds faster per round of tiles; long contractions stay on the 256-row ping-pong kernel, which moves
+// fewer operand bytes per MFMA.  The 192-wide form is for widths that 256 does not divide into whole rounds of tiles:
+// 768 columns are 3 tiles of 256 (192 tiles for 8192 rows, three quarters of the compute units) or 4 of 192 (256 tiles).
+// The 128 + BN operand rows of a K step are staged as one run of rows, 32 * WAVES_N per pass, A first.
+template <int XCD_ORDER, int WAVES_N>
+__global__ void __launch_bounds__(256 * WAVES_N, WAVES_N) gemmBf16WideWaveKernel(const unsigned short* __restrict__ A,
+                                                                                 const unsigned short* __restrict__ Bt, Epilogue epi,
+                                                                                 int M, int N, int K, int lda, int ldb, int gmLog,
+                                                                                 int gnLog) {
+    constexpr int BM = 128, BN = 64 * WAVES_N, TM = 1, TN = 2;
+    constexpr int ROWS = BM + BN, ROWS_PER_PASS = 32 * WAVES_N, PASSES = (ROWS + ROWS_PER_PASS - 1) / ROWS_PER_PASS;
+    constexpr int LAST_ROWS = ROWS - (PASSES - 1) * ROWS_PER_PASS;   // rows of the last pass (the pass is whole waves: 32 rows = 4 waves)
+    static_assert(LAST_ROWS % 8 == 0, "the threads of the last pass must be whole wavefronts");
+    extern __shared__ __attribute__((aligned(16))) unsigned short lds[];   // [2][ROWS][LDS_ROW]: A rows, then Bt rows
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
     int tm, tn;
     if (XCD_ORDER) {
@@ -469,11 +476,14 @@ __global__ void __launch_bounds__(1024, 4) gemmBf16SixteenWaveKernel(const unsig
     }
     const int m0 = tm * BM, n0 = tn * BN;
     const int wm0 = (wave & 3) * 32, wn0 = (wave >> 2) * 64;
-    const int lr = tid >> 3, lc = (tid & 7) * 8;     // 128 rows x 128 bytes per pass: A takes one pass, Bt two
-    const unsigned short* aRow = A + size_t(min(m0 + lr, M - 1)) * lda;
-    const unsigned short* bRow[2];
+    const int lr = tid >> 3, lc = (tid & 7) * 8;     // ROWS_PER_PASS rows x 128 bytes per pass
+    const bool lastPass = LAST_ROWS == ROWS_PER_PASS || lr < LAST_ROWS;   // uniform over a wavefront
+    const unsigned short* src[PASSES];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) bRow[i] = Bt + size_t(min(n0 + lr + 128 * i, N - 1)) * ldb;
+    for (int p = 0; p < PASSES; ++p) {
+        const int row = min(lr + ROWS_PER_PASS * p, ROWS - 1);
+        src[p] = row < BM ? A + size_t(min(m0 + row, M - 1)) * lda : Bt + size_t(min(n0 + row - BM, N - 1)) * ldb;
+    }
     float16v acc[TM][TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -481,34 +491,31 @@ __global__ void __launch_bounds__(1024, 4) gemmBf16SixteenWaveKernel(const unsig
         for (int r = 0; r < 16; ++r) acc[0][j][r] = 0.0f;
     const int steps = max((K + BKK - 1) / BKK, 1);
     const int ldsW = lr * LDS_ROW + lc;
-    uint4v stageA = loadChunk(aRow, lc, K), stageB[2];
+    uint4v stage[PASSES];
+    auto loadStep = [&](int k) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) stageB[i] = loadChunk(bRow[i], lc, K);
-    *reinterpret_cast<uint4v*>(as + ldsW) = zeroPast(stageA, lc, K);
+        for (int p = 0; p < PASSES; ++p)
+            if (p + 1 < PASSES || lastPass) stage[p] = loadChunk(src[p], k, K);
+    };
+    auto storeStep = [&](int buf, int k) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) *reinterpret_cast<uint4v*>(bs + ldsW + 128 * i * LDS_ROW) = zeroPast(stageB[i], lc, K);
-    if (steps > 1) {
-        stageA = loadChunk(aRow, BKK + lc, K);
-#pragma unroll
-        for (int i = 0; i < 2; ++i) stageB[i] = loadChunk(bRow[i], BKK + lc, K);
-    }
+        for (int p = 0; p < PASSES; ++p)
+            if (p + 1 < PASSES || lastPass)
+                *reinterpret_cast<uint4v*>(lds + (buf * ROWS + ROWS_PER_PASS * p) * LDS_ROW + ldsW) = zeroPast(stage[p], k, K);
+    };
+    loadStep(lc);
+    storeStep(0, lc);
+    if (steps > 1) loadStep(BKK + lc);
     __syncthreads();
     bf16x8 a[2], b[2][TN];
     for (int T = 0; T < steps; ++T) {
         const int par = T & 1;
-        const unsigned short* ac = as + (par * BM + wm0 + li) * LDS_ROW + 8 * half;
-        const unsigned short* bc = bs + (par * BN + wn0 + li) * LDS_ROW + 8 * half;
+        const unsigned short* ac = lds + (par * ROWS + wm0 + li) * LDS_ROW + 8 * half;
+        const unsigned short* bc = lds + (par * ROWS + BM + wn0 + li) * LDS_ROW + 8 * half;
         if (T + 1 < steps) {
             const int kNext = (T + 1) * BKK + lc;
-            *reinterpret_cast<uint4v*>(as + (par ^ 1) * BM * LDS_ROW + ldsW) = zeroPast(stageA, kNext, K);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-                *reinterpret_cast<uint4v*>(bs + ((par ^ 1) * BN + 128 * i) * LDS_ROW + ldsW) = zeroPast(stageB[i], kNext, K);
-            if (T + 2 < steps) {
-                stageA = loadChunk(aRow, kNext + BKK, K);
-#pragma unroll
-                for (int i = 0; i < 2; ++i) stageB[i] = loadChunk(bRow[i], kNext + BKK, K);
-            }
+            storeStep(par ^ 1, kNext);
+            if (T + 2 < steps) loadStep(kNext + BKK);
         }
         a[0] = *reinterpret_cast<const bf16x8*>(ac);
 #pragma unroll
@@ -739,10 +746,12 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
     return BF_OK;
 }
 
-int launchSixteenWave(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
-                      size_t lda, size_t ldb, hipStream_t s) {
-    const size_t tilesM = (M + 127) / 128, tilesN = (N + 255) / 256;
-    constexpr size_t smem = size_t(2) * (128 + 256) * LDS_ROW * sizeof(unsigned short);
+template <int WAVES_N>
+int launchWideWave(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
+                   size_t lda, size_t ldb, hipStream_t s) {
+    constexpr size_t BN = 64 * WAVES_N;
+    const size_t tilesM = (M + 127) / 128, tilesN = (N + BN - 1) / BN;
+    constexpr size_t smem = size_t(2) * (128 + BN) * LDS_ROW * sizeof(unsigned short);
     int gmLog = 2, gnLog = 3;
     size_t bestCost = 0, blocks = 0;
     for (int g = 0; g <= 5; ++g) {
@@ -754,11 +763,11 @@ int launchSixteenWave(const unsigned short* A, const unsigned short* Bt, const E
     const bool xcdOrder = blocks * 32 <= (tilesM * tilesN) * 5 / 4 && (blocks % 8 == 0 || blocks >= 64);
     const size_t grid = xcdOrder ? (blocks + 7) / 8 * 8 * 32 : tilesM * tilesN;
     if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
-    auto kernel = xcdOrder ? gemmBf16SixteenWaveKernel<1> : gemmBf16SixteenWaveKernel<0>;
+    auto kernel = xcdOrder ? gemmBf16WideWaveKernel<1, WAVES_N> : gemmBf16WideWaveKernel<0, WAVES_N>;
     int st = allowSharedMemory(kernel, smem);
     if (st != BF_OK) return st;
-    kernel<<<dim3(unsigned(grid)), 1024, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), xcdOrder ? gmLog : 0,
-                                                    xcdOrder ? gnLog : 0);
+    kernel<<<dim3(unsigned(grid)), 256 * WAVES_N, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), xcdOrder ? gmLog : 0,
+                                                             xcdOrder ? gnLog : 0);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -863,11 +872,20 @@ int launchGemmTn(const unsigned short* A, const unsigned short* B, const Epilogu
     return BF_OK;
 }
 
-// epi.splitN must be N (one output) or a multiple of 256 (several outputs).
+// epi.splitN must be N (one output) or a multiple of 256 (several outputs: a tile must lie in one of them).
 int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
                  size_t lda, size_t ldb, hipStream_t s) {
     if (M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
     const size_t cus = size_t(computeUnits());
+    switch (g_ntRoute.load()) {   // a kernel named by the caller (tests and tuning); BF_GEMM_ROUTE_AUTO otherwise
+        case BF_GEMM_ROUTE_PINGPONG_256: return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
+        case BF_GEMM_ROUTE_PINGPONG_128: return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s);
+        case BF_GEMM_ROUTE_WIDE_256: return launchWideWave<4>(A, Bt, epi, M, N, K, lda, ldb, s);
+        case BF_GEMM_ROUTE_WIDE_192:
+            if (size_t(epi.splitN) != N && epi.splitN % 192 != 0) return failInvalid("gemm_bf16", "192-wide tiles need outputs whose width is a multiple of 192");
+            return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s);
+        default: break;
+    }
     // 256x256 ping-pong tiles once they give three quarters of the CUs a tile; otherwise 128x128 tiles,
     // with K cut into slices when even those leave CUs idle and K is long enough to share out.
     // A workgroup per CU at a time, so a product takes ceil(tiles / CUs) rounds; a 128-row tile costs kHalfTileCost of a
@@ -876,13 +894,18 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
     constexpr double kHalfTileCost = 0.78;
     const double bigTime = bigTiles >= cus * 3 / 4 ? double((bigTiles + cus - 1) / cus) : 1e30;
     const double halfTime = halfTiles >= cus * 3 / 4 ? double((halfTiles + cus - 1) / cus) * kHalfTileCost : 1e30;
-    if (halfTiles >= cus * 3 / 4) {
+    {
         // measured per round of tiles, in microseconds: the 256-row ping-pong 8 + 1.56 per K step, sixteen wavefronts on
-        // 128-row tiles 5 + 0.95 per K step
+        // 128 x 256 tiles 5 + 0.95 per K step, twelve on 128 x 192 tiles 5 + kNarrowStep per K step
+        constexpr double kNarrowStep = 0.86;
         const double stepsAll = double((K + BKK - 1) / BKK);
+        const size_t narrowTiles = ((M + 127) / 128) * ((N + 191) / 192);
+        const bool narrowFits = size_t(epi.splitN) == N || epi.splitN % 192 == 0;   // a tile must lie in one output
         const double big = bigTiles >= cus * 3 / 4 ? double((bigTiles + cus - 1) / cus) * (8.0 + 1.56 * stepsAll) : 1e30;
-        const double wide = double((halfTiles + cus - 1) / cus) * (5.0 + 0.95 * stepsAll);
-        if (wide < big) return launchSixteenWave(A, Bt, epi, M, N, K, lda, ldb, s);
+        const double wide = halfTiles >= cus * 3 / 4 ? double((halfTiles + cus - 1) / cus) * (5.0 + 0.95 * stepsAll) : 1e30;
+        const double narrow = narrowFits && narrowTiles >= cus * 3 / 4 ? double((narrowTiles + cus - 1) / cus) * (5.0 + kNarrowStep * stepsAll) : 1e30;
+        if (narrow < wide && narrow < big) return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s);
+        if (wide < big) return launchWideWave<4>(A, Bt, epi, M, N, K, lda, ldb, s);
     }
     if (bigTime <= halfTime && bigTime < 1e30) return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
     if (halfTime < 1e30) return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s);
@@ -1600,6 +1623,12 @@ int bf_hip_feedforward_bf16_backward_img(const float* x, const uint16_t* xImage,
         if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
     }
     return st;
+}
+
+int bf_hip_gemm_bf16_set_route(int route) {
+    BF_REQUIRE(route >= BF_GEMM_ROUTE_AUTO && route <= BF_GEMM_ROUTE_WIDE_192, "unknown route");
+    bf::g_ntRoute.store(route);
+    return BF_OK;
 }
 
 int bf_hip_invalidate_bf16_weight_cache(void) {

@@ -286,6 +286,18 @@ int bf_hip_feedforward_bf16_backward_img(const float* x, const uint16_t* xImage,
                                          const uint16_t* hImage, const float* g, const uint16_t* gImage, int act, float* dX, float* dW1,
                                          float* dB1, float* dW2, float* dB2, size_t m, size_t d, size_t hidden, int cacheWeight,
                                          bf_stream_t stream);
+/* Which kernel bf_hip_gemm_bf16_nt and the projections built on it use for C = A * Bt^T.  AUTO (the default) picks by
+ * a cost estimate from the shape; the others name one tile form whatever the shape, for tests that must reach every
+ * kernel with the same operands and for tuning the estimate.  Every form gives the same bits (each output element is
+ * accumulated in the same order of k).  No counterpart in the reference. */
+enum {
+    BF_GEMM_ROUTE_AUTO = 0,
+    BF_GEMM_ROUTE_PINGPONG_256 = 1,   /* 256 x 256 tiles, eight wavefronts in two alternating groups */
+    BF_GEMM_ROUTE_PINGPONG_128 = 2,   /* 128 x 256 tiles, same schedule */
+    BF_GEMM_ROUTE_WIDE_256 = 3,       /* 128 x 256 tiles, sixteen wavefronts */
+    BF_GEMM_ROUTE_WIDE_192 = 4        /* 128 x 192 tiles, twelve wavefronts */
+};
+int bf_hip_gemm_bf16_set_route(int route);
 /* invalidateBf16WeightCache: ops.hpp:80 */
 int bf_hip_invalidate_bf16_weight_cache(void);
 

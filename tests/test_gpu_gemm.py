@@ -1,4 +1,6 @@
 """GPU parity: fp32 GEMM family (fp32 MFMA) and bf16 projections (bf16 MFMA, fp32 accumulate)."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -166,6 +168,61 @@ def test_bf16_projection_large_tile_kernel(hip, oracle, rng, m, k, n):
     rows = np.r_[0:3, m // 2:m // 2 + 3, m - 3:m]
     assert_close(oracle.matmul(ar[rows], br), expected[rows], tol=1e-5, what="oracle vs float64 on sampled rows")
     assert_close(c, expected, tol=1e-4, what="bf16 fwd (large tiles) vs rounded operands")
+
+
+ROUTES = {"ping-pong 256": 1, "ping-pong 128": 2, "sixteen wavefronts, 128 x 256": 3, "twelve wavefronts, 128 x 192": 4}
+
+
+@pytest.mark.parametrize("m,k,n", [(8192, 768, 768), (8192, 200, 2304), (700, 136, 1000), (1, 8, 1), (130, 72, 193), (4100, 64, 4093), (257, 1032, 385)])
+def test_bf16_gemm_every_tile_form_on_the_same_operands(hip, oracle, rng, m, k, n):
+    """Each large-tile kernel named through bf_hip_gemm_bf16_set_route, whatever the cost estimate would pick: float64 of
+    the rounded operands to 1e-4 for one of them, and the same bits from all (an output element is accumulated over k
+    in the same order by every form).  Shapes: whole rounds of tiles for the 192-wide form, ragged edges in both
+    directions, a K tail, single tiles, one element."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    a, b = oracle.roundToBf16(r(rng, m, k)), oracle.roundToBf16(r(rng, n, k, scale=0.1))
+    ai, bi = D((m, k), itemsize=2), D((n, k), itemsize=2)
+    call("bf_hip_cvt_f32_bf16", D.fromHost(a).ptr, ai.ptr, m * k, None)
+    call("bf_hip_cvt_f32_bf16", D.fromHost(b).ptr, bi.ptr, n * k, None)
+    expected = (a.astype(np.float64) @ b.astype(np.float64).T).astype(f32)
+    first = None
+    try:
+        for name, route in ROUTES.items():
+            call("bf_hip_gemm_bf16_set_route", route)
+            guard = D.fromHost(np.full((m + 2, n), 7.0, f32))   # a row of sevens on either side of the output
+            out_ptr = ctypes.c_void_p(guard.ptr.value + 4 * n)
+            call("bf_hip_gemm_bf16_nt", ai.ptr, bi.ptr, out_ptr, m, n, k, None)
+            got = guard.toHost()
+            assert (got[0] == 7).all() and (got[-1] == 7).all(), name + ": wrote outside the output"
+            if first is None:
+                first = got[1:-1]
+                assert_close(first, expected, tol=1e-4, what=name)
+            else:
+                assert_bits_equal(got[1:-1], first, name + " vs " + next(iter(ROUTES)))
+    finally:
+        call("bf_hip_gemm_bf16_set_route", 0)
+    with pytest.raises(ValueError):
+        call("bf_hip_gemm_bf16_set_route", 17)
+
+
+def test_bf16_shared_input_projections_on_192_wide_tiles(hip, rng):
+    """Three projections of width 768 in one product of width 2304 with split outputs: 768 = 4 x 192, so the twelve-wavefront
+    form may serve it (and does for 8192 rows); the same bits as the sixteen-wavefront form and as three separate products."""
+    D, ops, call = hip.DeviceTensor, hip.ops, hip.capi.call
+    m, k, n = 8192, 264, 768
+    da = D.fromHost(r(rng, m, k))
+    dws = [D.fromHost(r(rng, k, n, scale=0.1)) for _ in range(3)]
+    results = {}
+    try:
+        for route in (0, 3, 4):
+            call("bf_hip_gemm_bf16_set_route", route)
+            results[route] = [t.toHost() for t in ops.matmulBf16SharedInput(da, dws)]
+    finally:
+        call("bf_hip_gemm_bf16_set_route", 0)
+    singles = [ops.matmulBf16(da, w).toHost() for w in dws]
+    for route, outs in results.items():
+        for got, single in zip(outs, singles):
+            assert_bits_equal(got, single, f"route {route}: split output vs its own product")
 
 
 @pytest.mark.parametrize("m,k,n", [(33, 40, 24), (300, 72, 520), (2100, 136, 3000), (70, 4100, 90), (6200, 72, 1501), (4100, 136, 4093),
