@@ -58,6 +58,10 @@ SIGNATURES = {
     "bf_hip_memcpy_h2d": [P, c_ptr, c_size],
     "bf_hip_memcpy_d2h": [c_ptr, P, c_size],
     "bf_hip_memcpy_d2d": [P, P, c_size, S],
+    "bf_hip_capture_begin": [S],
+    "bf_hip_capture_end": [ctypes.POINTER(c_ptr)],
+    "bf_hip_graph_launch": [c_ptr, S],
+    "bf_hip_graph_destroy": [c_ptr],
     "bf_hip_fill_zero": [P, c_size, S],
     "bf_hip_add": [P, P, P, c_size, S],
     "bf_hip_scale": [P, c_float, P, c_size, S],
@@ -125,6 +129,11 @@ SIGNATURES = {
     "bf_hip_cross_entropy_sparse": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse_img": [P, P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_masked": [P, P, P, P, c_size, c_size, c_int, S],
+    "bf_hip_sgd_publish": [P, c_float, S],
+    "bf_hip_sgd_multi_indirect": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_size), c_size, P, S],
+    "bf_hip_adamw_publish": [P, c_ll, c_float, c_float, c_float, c_float, c_float, S],
+    "bf_hip_adamw_multi_indirect": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr),
+                                    ctypes.POINTER(c_size), c_size, P, S],
     "bf_hip_sgd_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_size), c_size, c_float, S],
     "bf_hip_adamw_multi": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr),
                            ctypes.POINTER(c_size), c_size, c_ll, c_float, c_float, c_float, c_float, c_float, S],

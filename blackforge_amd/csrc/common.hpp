@@ -30,7 +30,17 @@ int failRuntime(const char* function, hipError_t error, const char* file, int li
 
 #define BF_LAUNCH_CHECK() BF_HIP_TRY(hipGetLastError())
 
-inline hipStream_t asStream(bf_stream_t s) { return static_cast<hipStream_t>(s); }
+// The stream a NULL bf_stream_t stands for: the device's default stream, or, between bf_hip_capture_begin and
+// bf_hip_capture_end, the stream that is being captured (so that code written against the default stream, like the
+// C++ operator layer, records into the graph unchanged).
+extern hipStream_t g_defaultStream;
+inline hipStream_t asStream(bf_stream_t s) { return s ? static_cast<hipStream_t>(s) : g_defaultStream; }
+// True between bf_hip_capture_begin and bf_hip_capture_end.  While it holds, pool blocks come from and return to the
+// capture's own arena, descriptor tables are private copies, and weight images are cached per capture: nothing the
+// recorded kernels address can be handed to anyone else while the graph lives.
+bool capturing();
+// gemm_bf16.hip: returns the weight images cached during the capture to the pool (the arena, at that point).
+void dropCaptureWeightImages();
 
 // ---- launch geometry ---------------------------------------------------------------------------
 constexpr int kWave = 64;            // CDNA wavefront

@@ -276,14 +276,16 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
         return BF_OK;
     }
     bool vec = aligned16(src) && (!FUSED || (aligned16(bias) && aligned16(dHidden) && aligned16(dGemm)));
-    RowGeom g = rowGeometry(rows, features, vec, 256, 4);
+    // a matrix small enough for one row of blocks to walk is summed in one launch, straight into dBias
+    const bool single = rows * features <= (size_t(1) << 16);
+    RowGeom g = rowGeometry(rows, features, vec, single ? 1 : 256, 4);
     size_t parts = g.grid.y;
     if (workspace && dBias && parts * features > workspaceFloats)
         return failInvalid("column_sum", "the partial sums (" + std::to_string(parts) + " rows of " + std::to_string(features) +
                                              " columns) exceed the static workspace of " + std::to_string(workspaceFloats) + " floats");
-    Scratch scratch(dBias && !workspace ? parts * features * sizeof(float) : 0);
+    Scratch scratch(dBias && !workspace && parts > 1 ? parts * features * sizeof(float) : 0);
     if (scratch.status != BF_OK) return scratch.status;
-    float* partial = dBias ? (workspace ? workspace : scratch.as<float>()) : nullptr;
+    float* partial = dBias ? (parts == 1 ? dBias : workspace ? workspace : scratch.as<float>()) : nullptr;
     if (image && g.vec != 4) return failInvalid("act_backward_image", "operands must be 16-byte aligned and the width a multiple of 4");
     // bytes per element: the source, and on the fused route the second input and whichever outputs are written
     const size_t perElement = 4 + (FUSED ? 4 + (dGemm ? 4 : 0) + (image ? 2 : 0) : 0);
@@ -296,7 +298,7 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
         else columnSumKernel<1, FUSED, ACT, false><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
     }
     BF_LAUNCH_CHECK();
-    if (dBias) {
+    if (dBias && parts > 1) {
         columnFinishKernel<<<gridFor(features, 16), kBlock, 0, stream>>>(partial, dBias, parts, features);
         BF_LAUNCH_CHECK();
     }

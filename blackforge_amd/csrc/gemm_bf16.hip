@@ -1043,9 +1043,11 @@ struct CachedWeight {
 };
 size_t g_generation = 1;
 using WeightKey = std::tuple<int, const float*, const float*, const float*, int>;
+// While a graph is being captured the images live in a cache of their own, filled and emptied inside the capture: the
+// recorded conversions and products address arena blocks that no later eager call can be handed.
 std::map<WeightKey, CachedWeight>& weightCache() {
-    static std::map<WeightKey, CachedWeight> cache;
-    return cache;
+    static std::map<WeightKey, CachedWeight> eager, captured;
+    return capturing() ? captured : eager;
 }
 
 // `plain`: for the transposed layouts (1, 2) the plain counterpart (0, 3) written in the same pass, or NULL.
@@ -1134,6 +1136,13 @@ int weightImage(const float* w, size_t rows, size_t cols, bool transposed, bool 
 }
 
 }  // namespace
+
+void dropCaptureWeightImages() {
+    if (!capturing()) return;
+    auto& cache = weightCache();
+    for (auto& entry : cache) bf_hip_pool_release(entry.second.buffer, entry.second.bytes);
+    cache.clear();
+}
 }  // namespace bf
 
 using namespace bf;

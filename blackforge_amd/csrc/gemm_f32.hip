@@ -175,9 +175,12 @@ extern "C" int bf_hip_gemm_f32(int transA, int transB, const float* A, const flo
     // Few tiles and a long contraction (the weight gradients of a small model: a [features x features] product
     // over all tokens): cut K into slices so that more workgroups share it; a second kernel adds the slices in
     // order.
+    // The second launch must pay for itself: with a workgroup alone on its compute unit a K step of 32 takes about a
+    // microsecond (nothing hides its latencies) and a dependent launch about five, so contractions under 256 stay whole
+    // (a small model's step is bounded by its launch count) and longer ones are cut into slices of at least two steps.
     const size_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
     size_t slices = 1;
-    if (tiles < cus && K >= 4 * BK) slices = std::min<size_t>(std::min<size_t>(16, cus / tiles), K / (2 * BK));
+    if (tiles < cus && K >= 8 * BK) slices = std::min<size_t>(std::min<size_t>(16, cus / tiles), K / (2 * BK));
     if (slices > 1) {
         const size_t steps = (K + BK - 1) / BK, kPer = (steps + slices - 1) / slices * BK;
         slices = (K + kPer - 1) / kPer;

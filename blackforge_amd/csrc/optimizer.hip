@@ -33,8 +33,11 @@ struct AdamTensor {
     unsigned pad;
 };
 
+// lrDevice: when not NULL the learning rate is read from there (a launch recorded in a graph must not freeze it)
 template <bool NT>
-__global__ void __launch_bounds__(kBlock) sgdKernel(const SgdTensor* __restrict__ table, int numTensors, float lr) {
+__global__ void __launch_bounds__(kBlock) sgdKernel(const SgdTensor* __restrict__ table, int numTensors, float lr,
+                                                    const float* __restrict__ lrDevice) {
+    if (lrDevice) lr = *lrDevice;
     const SgdTensor c = table[owningTensor(table, numTensors, blockIdx.x)];
     const size_t base = (size_t(blockIdx.x - c.firstBlock) * kBlock + threadIdx.x) * 4;
     if (base >= c.count) return;
@@ -58,8 +61,14 @@ __device__ __forceinline__ void adamOne(float& p, float g, float& m, float& v, c
     p -= a.lr * (mHat / (sqrtf(vHat) + a.eps) + a.weightDecay * p);
 }
 
+__global__ void publishHyperKernel(AdamParams* dst, AdamParams value) { *dst = value; }
+__global__ void publishFloatKernel(float* dst, float value) { *dst = value; }
+
+// hyper: when not NULL the hyper-parameters and bias corrections are read from there
 template <bool NT>
-__global__ void __launch_bounds__(kBlock) adamwKernel(const AdamTensor* __restrict__ table, int numTensors, AdamParams a) {
+__global__ void __launch_bounds__(kBlock) adamwKernel(const AdamTensor* __restrict__ table, int numTensors, AdamParams a,
+                                                      const AdamParams* __restrict__ hyper) {
+    if (hyper) a = *hyper;
     const AdamTensor c = table[owningTensor(table, numTensors, blockIdx.x)];
     const size_t base = (size_t(blockIdx.x - c.firstBlock) * kBlock + threadIdx.x) * 4;
     if (base >= c.count) return;
@@ -88,8 +97,8 @@ using namespace bf;
 
 extern "C" {
 
-int bf_hip_sgd_multi(float* const* params, const float* const* grads, const size_t* counts, size_t numTensors, float lr,
-                     bf_stream_t stream) {
+static int sgdMulti(float* const* params, const float* const* grads, const size_t* counts, size_t numTensors, float lr,
+                    const float* lrDevice, bf_stream_t stream) {
     if (numTensors == 0) return BF_OK;
     BF_REQUIRE(params && grads && counts, "NULL pointer");
     std::vector<SgdTensor> table;
@@ -104,16 +113,14 @@ int bf_hip_sgd_multi(float* const* params, const float* const* grads, const size
     const void* device = nullptr;
     int st = uploadDescriptorTable(kSlotSgd, table.data(), table.size() * sizeof(SgdTensor), asStream(stream), &device);
     if (st != BF_OK) return st;
-    if (streamsPastCache(blocks * kPerBlock * 12)) sgdKernel<true><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const SgdTensor*>(device), int(numTensors), lr);
-    else sgdKernel<false><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const SgdTensor*>(device), int(numTensors), lr);
+    if (streamsPastCache(blocks * kPerBlock * 12)) sgdKernel<true><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const SgdTensor*>(device), int(numTensors), lr, lrDevice);
+    else sgdKernel<false><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const SgdTensor*>(device), int(numTensors), lr, lrDevice);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
 
-int bf_hip_adamw_multi(float* const* params, const float* const* grads, float* const* m, float* const* v,
-                       const size_t* counts, size_t numTensors, long long step, float lr, float beta1, float beta2,
-                       float eps, float weightDecay, bf_stream_t stream) {
-    BF_REQUIRE(step >= 1, "step must be >= 1");
+static int adamwMulti(float* const* params, const float* const* grads, float* const* m, float* const* v, const size_t* counts,
+                      size_t numTensors, const AdamParams& byValue, const AdamParams* hyperDevice, bf_stream_t stream) {
     if (numTensors == 0) return BF_OK;
     BF_REQUIRE(params && grads && m && v && counts, "NULL pointer");
     std::vector<AdamTensor> table;
@@ -128,11 +135,55 @@ int bf_hip_adamw_multi(float* const* params, const float* const* grads, float* c
     const void* device = nullptr;
     int st = uploadDescriptorTable(kSlotAdamW, table.data(), table.size() * sizeof(AdamTensor), asStream(stream), &device);
     if (st != BF_OK) return st;
-    // bias corrections on the host in float, exactly like the reference (optimizer.cu:104-107)
-    float t = static_cast<float>(step);
-    AdamParams a{lr, beta1, beta2, eps, weightDecay, 1.0f - std::pow(beta1, t), 1.0f - std::pow(beta2, t)};
-    if (streamsPastCache(blocks * kPerBlock * 28)) adamwKernel<true><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const AdamTensor*>(device), int(numTensors), a);
-    else adamwKernel<false><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const AdamTensor*>(device), int(numTensors), a);
+    if (streamsPastCache(blocks * kPerBlock * 28)) adamwKernel<true><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const AdamTensor*>(device), int(numTensors), byValue, hyperDevice);
+    else adamwKernel<false><<<unsigned(blocks), kBlock, 0, asStream(stream)>>>(static_cast<const AdamTensor*>(device), int(numTensors), byValue, hyperDevice);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+// bias corrections on the host in float, exactly like the reference (optimizer.cu:104-107)
+static AdamParams adamParams(long long step, float lr, float beta1, float beta2, float eps, float weightDecay) {
+    const float t = static_cast<float>(step);
+    return AdamParams{lr, beta1, beta2, eps, weightDecay, 1.0f - std::pow(beta1, t), 1.0f - std::pow(beta2, t)};
+}
+
+int bf_hip_sgd_multi(float* const* params, const float* const* grads, const size_t* counts, size_t numTensors, float lr,
+                     bf_stream_t stream) {
+    return sgdMulti(params, grads, counts, numTensors, lr, nullptr, stream);
+}
+
+int bf_hip_sgd_multi_indirect(float* const* params, const float* const* grads, const size_t* counts, size_t numTensors,
+                              const float* lrDevice, bf_stream_t stream) {
+    BF_REQUIRE(lrDevice != nullptr, "lrDevice is NULL");
+    return sgdMulti(params, grads, counts, numTensors, 0.0f, lrDevice, stream);
+}
+
+int bf_hip_sgd_publish(float* lrDevice, float lr, bf_stream_t stream) {
+    BF_REQUIRE(lrDevice != nullptr, "lrDevice is NULL");
+    publishFloatKernel<<<1, 1, 0, asStream(stream)>>>(lrDevice, lr);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_adamw_multi(float* const* params, const float* const* grads, float* const* m, float* const* v,
+                       const size_t* counts, size_t numTensors, long long step, float lr, float beta1, float beta2,
+                       float eps, float weightDecay, bf_stream_t stream) {
+    BF_REQUIRE(step >= 1, "step must be >= 1");
+    return adamwMulti(params, grads, m, v, counts, numTensors, adamParams(step, lr, beta1, beta2, eps, weightDecay), nullptr, stream);
+}
+
+int bf_hip_adamw_multi_indirect(float* const* params, const float* const* grads, float* const* m, float* const* v,
+                                const size_t* counts, size_t numTensors, const bf_adamw_hyper* hyperDevice, bf_stream_t stream) {
+    BF_REQUIRE(hyperDevice != nullptr, "hyperDevice is NULL");
+    static_assert(sizeof(bf_adamw_hyper) == sizeof(AdamParams), "the public block and the kernel's must match");
+    return adamwMulti(params, grads, m, v, counts, numTensors, AdamParams{}, reinterpret_cast<const AdamParams*>(hyperDevice), stream);
+}
+
+int bf_hip_adamw_publish(bf_adamw_hyper* hyperDevice, long long step, float lr, float beta1, float beta2, float eps,
+                         float weightDecay, bf_stream_t stream) {
+    BF_REQUIRE(hyperDevice != nullptr, "hyperDevice is NULL");
+    BF_REQUIRE(step >= 1, "step must be >= 1");
+    publishHyperKernel<<<1, 1, 0, asStream(stream)>>>(reinterpret_cast<AdamParams*>(hyperDevice), adamParams(step, lr, beta1, beta2, eps, weightDecay));
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

@@ -32,6 +32,8 @@ int failRuntime(const char* function, hipError_t error, const char* file, int li
     return BF_ERR_RUNTIME;
 }
 
+hipStream_t g_defaultStream = nullptr;
+
 int computeUnits() {
     static std::unordered_map<int, int> cache;
     int dev = 0;
@@ -68,6 +70,8 @@ std::map<std::pair<int, int>, DescriptorTable>& descriptorTables() {
 }
 }  // namespace
 
+int uploadPrivateTable(const void* hostBytes, size_t bytes, const void** devicePtr);
+
 int allowDynamicSharedMemory(const void* kernel, size_t bytes) {
     if (bytes <= 48 * 1024) return BF_OK;
     int dev = 0;
@@ -83,6 +87,7 @@ int allowDynamicSharedMemory(const void* kernel, size_t bytes) {
 int uploadDescriptorTable(int slot, const void* hostBytes, size_t bytes, hipStream_t stream, const void** devicePtr) {
     int dev = 0;
     BF_HIP_TRY(hipGetDevice(&dev));
+    if (capturing()) return uploadPrivateTable(hostBytes, bytes, devicePtr);
     DescriptorTable& t = descriptorTables()[{dev, slot}];
     const auto* src = static_cast<const unsigned char*>(hostBytes);
     bool same = t.device != nullptr && t.host.size() == bytes && std::equal(src, src + bytes, t.host.begin());
@@ -129,6 +134,73 @@ std::unordered_map<int, DevicePool>& pools() {
     return registry;
 }
 
+// The memory of one captured graph.  Every block acquired while the capture runs belongs to the arena: when it is
+// released (during the capture or later, by whoever holds it) it goes to the arena's own free lists, where only the
+// same capture can take it again, and it reaches the device's general free lists only when the graph is destroyed.
+// A replay therefore never finds one of its buffers in somebody else's hands, and bf_hip_pool_trim cannot free them.
+struct CaptureArena {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::unordered_map<size_t, std::vector<void*>> freeLists;
+    std::vector<std::pair<void*, size_t>> blocks;   // (pointer, size class) of every block taken during the capture
+    std::vector<void*> tables;                      // descriptor tables of recorded launches (hipMalloc, not pool blocks)
+};
+CaptureArena* g_capture = nullptr;                               // the capture in progress
+std::unordered_map<void*, CaptureArena*>& arenaOwners() {        // block -> arena, for arenas that still exist
+    static std::unordered_map<void*, CaptureArena*> owners;
+    return owners;
+}
+hipStream_t g_utilityStream = nullptr;   // non-blocking, for copies that must not touch a capturing stream
+
+struct CapturedGraph {
+    hipGraphExec_t exec = nullptr;
+    CaptureArena* arena = nullptr;
+};
+
+// hipMalloc with one retry after returning every cached block to the driver: size classes above 64 MiB are 2 MiB
+// apart, so a process that has seen many shapes can hold most of the card in free lists that fit nothing new.
+hipError_t mallocWithTrim(void** ptr, size_t bytes, DevicePool& pool) {
+    hipError_t err = hipMalloc(ptr, bytes);
+    if (err != hipErrorOutOfMemory || capturing()) return err;
+    (void)hipGetLastError();
+    if (hipDeviceSynchronize() != hipSuccess) return err;
+    for (auto& entry : pool.freeLists) {
+        for (void* p : entry.second) {
+            if (hipFree(p) == hipSuccess) pool.stats.bytes_from_driver -= entry.first;
+        }
+        entry.second.clear();
+    }
+    return hipMalloc(ptr, bytes);
+}
+
+void retireArena(CaptureArena* arena) {
+    DevicePool& pool = pools()[arena->device];
+    for (const auto& block : arena->blocks) arenaOwners().erase(block.first);
+    for (auto& entry : arena->freeLists)
+        for (void* p : entry.second) pool.freeLists[entry.first].push_back(p);
+    for (void* table : arena->tables) (void)hipFree(table);
+    delete arena;
+}
+
+}  // namespace
+
+bool capturing() { return g_capture != nullptr; }
+
+// A descriptor table for kernels that are being recorded: memory of its own, written now (on a stream that has nothing
+// to do with the capturing one) and never again, so that replays read what the recording saw.  It must not come from
+// the pool: a block that recorded kernels used as a temporary earlier in the capture and released would be rewritten
+// by those kernels on every replay, under the table.
+int uploadPrivateTable(const void* hostBytes, size_t bytes, const void** devicePtr) {
+    void* block = nullptr;
+    BF_HIP_TRY(hipMalloc(&block, bytes < 256 ? 256 : bytes));
+    g_capture->tables.push_back(block);   // freed with the graph
+    BF_HIP_TRY(hipMemcpyAsync(block, hostBytes, bytes, hipMemcpyHostToDevice, g_utilityStream));
+    BF_HIP_TRY(hipStreamSynchronize(g_utilityStream));
+    *devicePtr = block;
+    return BF_OK;
+}
+
+namespace {
 __global__ void fillZeroKernel(uint32_t* dst, size_t words) {
     size_t stride = size_t(gridDim.x) * blockDim.x;
     for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < words; i += stride) dst[i] = 0u;
@@ -244,15 +316,17 @@ int bf_hip_pool_acquire(size_t bytes, void** ptr) {
     BF_HIP_TRY(hipGetDevice(&dev));
     DevicePool& pool = pools()[dev];
     size_t cls = sizeClass(bytes);
-    std::vector<void*>& list = pool.freeLists[cls];
-    if (!list.empty()) {
-        *ptr = list.back();
-        list.pop_back();
+    std::vector<void*>* list = &pool.freeLists[cls];
+    if (g_capture != nullptr && !g_capture->freeLists[cls].empty()) list = &g_capture->freeLists[cls];
+    if (!list->empty()) {
+        *ptr = list->back();
+        list->pop_back();
     } else {
-        BF_HIP_TRY(hipMalloc(ptr, cls));
+        BF_HIP_TRY(mallocWithTrim(ptr, cls, pool));
         pool.stats.bytes_from_driver += cls;
         pool.stats.driver_allocations += 1;
     }
+    if (g_capture != nullptr && arenaOwners().emplace(*ptr, g_capture).second) g_capture->blocks.emplace_back(*ptr, cls);
     pool.stats.bytes_in_use += cls;
     pool.stats.acquires += 1;
     return BF_OK;
@@ -264,7 +338,9 @@ int bf_hip_pool_release(void* ptr, size_t bytes) {
     BF_HIP_TRY(hipGetDevice(&dev));
     DevicePool& pool = pools()[dev];
     size_t cls = sizeClass(bytes);
-    pool.freeLists[cls].push_back(ptr);
+    const auto owner = arenaOwners().find(ptr);
+    if (owner != arenaOwners().end()) owner->second->freeLists[cls].push_back(ptr);
+    else pool.freeLists[cls].push_back(ptr);
     pool.stats.bytes_in_use -= cls < pool.stats.bytes_in_use ? cls : pool.stats.bytes_in_use;
     return BF_OK;
 }
@@ -308,6 +384,60 @@ int bf_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, bf_stream_t stre
     if (bytes == 0) return BF_OK;
     BF_REQUIRE(dst && src, "NULL pointer");
     BF_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, asStream(stream)));
+    return BF_OK;
+}
+
+int bf_hip_capture_begin(bf_stream_t stream) {
+    BF_REQUIRE(stream != nullptr, "a capture needs a stream made by bf_hip_stream_create");
+    BF_REQUIRE(g_capture == nullptr, "a capture is already in progress");
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    if (g_utilityStream == nullptr) BF_HIP_TRY(hipStreamCreateWithFlags(&g_utilityStream, hipStreamNonBlocking));
+    BF_HIP_TRY(hipDeviceSynchronize());   // nothing of the eager work before may still be in flight on another stream
+    BF_HIP_TRY(hipStreamBeginCapture(static_cast<hipStream_t>(stream), hipStreamCaptureModeRelaxed));
+    g_capture = new CaptureArena;
+    g_capture->device = dev;
+    g_capture->stream = static_cast<hipStream_t>(stream);
+    g_defaultStream = g_capture->stream;
+    return BF_OK;
+}
+
+int bf_hip_capture_end(bf_graph_t* graph) {
+    BF_REQUIRE(g_capture != nullptr, "no capture in progress");
+    CaptureArena* arena = g_capture;
+    dropCaptureWeightImages();   // while releases still go to the arena
+    g_capture = nullptr;
+    g_defaultStream = nullptr;
+    hipGraph_t recorded = nullptr;
+    hipError_t err = hipStreamEndCapture(arena->stream, &recorded);
+    hipGraphExec_t exec = nullptr;
+    if (err == hipSuccess && graph != nullptr) err = hipGraphInstantiate(&exec, recorded, nullptr, nullptr, 0);
+    if (recorded != nullptr) (void)hipGraphDestroy(recorded);
+    if (err != hipSuccess || graph == nullptr) {   // failed, or the caller abandons the capture (graph == NULL)
+        (void)hipGetLastError();
+        retireArena(arena);
+        if (graph != nullptr) *graph = nullptr;
+        if (err != hipSuccess) return failRuntime(__func__, err, __FILE__, __LINE__);
+        return BF_OK;
+    }
+    *graph = new CapturedGraph{exec, arena};
+    return BF_OK;
+}
+
+int bf_hip_graph_launch(bf_graph_t graph, bf_stream_t stream) {
+    BF_REQUIRE(graph != nullptr, "graph is NULL");
+    BF_REQUIRE(g_capture == nullptr, "a graph cannot be launched into a capture");
+    BF_HIP_TRY(hipGraphLaunch(static_cast<CapturedGraph*>(graph)->exec, asStream(stream)));
+    return BF_OK;
+}
+
+int bf_hip_graph_destroy(bf_graph_t graph) {
+    if (graph == nullptr) return BF_OK;
+    CapturedGraph* g = static_cast<CapturedGraph*>(graph);
+    BF_HIP_TRY(hipDeviceSynchronize());   // a replay still running keeps using the arena's blocks
+    if (g->exec != nullptr) (void)hipGraphExecDestroy(g->exec);
+    retireArena(g->arena);
+    delete g;
     return BF_OK;
 }
 

@@ -6,6 +6,7 @@
 #include <string>
 #include <vector>
 
+#include "blackforge/backend/hip/captured_step.hpp"
 #include "blackforge/backend/hip/loss.hpp"
 #include "blackforge/backend/hip/model.hpp"
 #include "blackforge/backend/hip/train_runner.hpp"
@@ -178,6 +179,42 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
             handle->adamw->step(handle->params);
         }
     });
+}
+
+// The same step recorded as a graph (hip::CapturedTrainStep) over the caller's input and target buffers: optimizer 1 =
+// AdamW with the reference defaults, 2 = SGD.  The handle keeps the optimizer; *step is released with
+// bfh_captured_step_destroy before the model is.
+int bfh_model_capture_train_step(void* h, const float* input, int rank, const size_t* shape, const float* target, int targetRank,
+                                 const size_t* targetShape, int lossKind, int optimizer, float lr, void** step) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        hip::require(optimizer == 1 || optimizer == 2, "capture_train_step: optimizer must be 1 (AdamW) or 2 (SGD)");
+        hip::Optimizer* opt = nullptr;
+        if (optimizer == 1) {
+            if (!handle->adamw) handle->adamw = std::make_unique<hip::AdamW>(lr, 0.9F, 0.999F, 1e-8F, 0.01F);
+            opt = handle->adamw.get();
+        } else {
+            if (!handle->sgd) handle->sgd = std::make_unique<hip::SGD>(lr);
+            opt = handle->sgd.get();
+        }
+        opt->setLearningRate(lr);
+        Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
+        Borrowed tgt(target, std::vector<std::size_t>(targetShape, targetShape + targetRank));
+        const char* lossName = lossKind == 0 ? "cross_entropy_sparse" : lossKind == 2 ? "cross_entropy_masked" : "mse";
+        *step = new hip::CapturedTrainStep(*handle->model, *opt, lossName, in.tensor, tgt.tensor, handle->lossAccumulator);
+    });
+}
+int bfh_captured_step_run(void* h, void* step, float lr, int optimizer) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        hip::Optimizer* opt = optimizer == 1 ? static_cast<hip::Optimizer*>(handle->adamw.get()) : handle->sgd.get();
+        hip::require(opt != nullptr, "captured_step_run: no such optimizer on this model");
+        opt->setLearningRate(lr);
+        static_cast<hip::CapturedTrainStep*>(step)->run();
+    });
+}
+int bfh_captured_step_destroy(void* step) {
+    return guarded([&] { delete static_cast<hip::CapturedTrainStep*>(step); });
 }
 
 // Reads the accumulated loss sum (one device->host copy) and resets the accumulator.

@@ -46,6 +46,11 @@ def load() -> ctypes.CDLL:
         lib.bfh_model_sgd_step.argtypes = [ctypes.c_void_p, ctypes.c_float]
         lib.bfh_model_train_step.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_size_t),
                                              ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float]
+        lib.bfh_model_capture_train_step.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_size_t),
+                                                     ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_size_t), ctypes.c_int,
+                                                     ctypes.c_int, ctypes.c_float, ctypes.POINTER(ctypes.c_void_p)]
+        lib.bfh_captured_step_run.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_int]
+        lib.bfh_captured_step_destroy.argtypes = [ctypes.c_void_p]
         lib.bfh_model_read_loss.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
         lib.bfh_model_run_training.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_longlong,
                                                ctypes.c_size_t, ctypes.c_double, ctypes.c_int, ctypes.c_char_p, ctypes.c_char_p,
@@ -74,6 +79,27 @@ def _check(status: int):
         return
     message = load().bfh_last_error().decode(errors="replace")
     raise ValueError(message) if status == 1 else RuntimeError(message)
+
+
+class CapturedStep:
+    """A recorded training step of a HostModel; keeps the model and the input tensors alive, and goes before them."""
+
+    def __init__(self, model, handle, optimizer, tensors):
+        self.model, self.handle, self.optimizer, self.tensors = model, handle, optimizer, tensors
+
+    def run(self, lr: float = 1e-3) -> None:
+        _check(load().bfh_captured_step_run(self.model.handle, self.handle, lr, self.optimizer))
+
+    def close(self) -> None:
+        if self.handle:
+            _check(load().bfh_captured_step_destroy(self.handle))
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class HostModel:
@@ -139,9 +165,21 @@ class HostModel:
     def adamwStep(self, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01) -> None:
         _check(load().bfh_model_adamw_step(self.handle, lr, beta1, beta2, eps, wd))
 
+    def sgdStep(self, lr: float) -> None:
+        _check(load().bfh_model_sgd_step(self.handle, lr))
+
     def trainStep(self, x: DeviceTensor, target: DeviceTensor, loss_kind: int = LOSS_SPARSE_CE, optimizer: int = 1, lr: float = 1e-3):
         shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
         _check(load().bfh_model_train_step(self.handle, x.ptr, len(x.shape), shape, target.ptr, loss_kind, optimizer, lr))
+
+    def captureTrainStep(self, x: DeviceTensor, target: DeviceTensor, loss_kind: int = LOSS_SPARSE_CE, optimizer: int = 1, lr: float = 1e-3):
+        """hip::CapturedTrainStep over x and target: the step recorded once (nothing executes), replayed by run()."""
+        shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
+        tshape = (ctypes.c_size_t * len(target.shape))(*target.shape)
+        step = ctypes.c_void_p()
+        _check(load().bfh_model_capture_train_step(self.handle, x.ptr, len(x.shape), shape, target.ptr, len(target.shape), tshape, loss_kind,
+                                                   optimizer, lr, ctypes.byref(step)))
+        return CapturedStep(self, step, optimizer, (x, target))
 
     def _refresh_params(self) -> None:
         """Re-reads names, counts and device pointers of the parameters (a checkpoint load replaces the buffers)."""

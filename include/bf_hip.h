@@ -96,6 +96,27 @@ typedef struct {
 int bf_hip_pool_stats(bf_pool_stats* stats);
 int bf_hip_pool_trim(void);                          /* hipFree every cached block of the current device */
 
+/* ---------------------------------------------------------------------------------------------
+ * Recording a sequence of calls once and replaying it (HIP graphs).  No counterpart in the reference, which launches
+ * every kernel of every step from the host; for small models a step is bounded by those launches.
+ *
+ * Between capture_begin(stream) and capture_end every call of this library that takes a stream records its kernels
+ * instead of running them; a NULL stream argument stands for `stream` while the capture lasts, so code written against
+ * the default stream records unchanged.  Memory the calls take from the pool during the capture belongs to the graph
+ * until bf_hip_graph_destroy: a replay never shares a buffer with anyone else, and pool_trim cannot free it.
+ * Rules for the recorded region: no call that copies to or from the host or waits for the device (memcpy_h2d/d2h,
+ * synchronize, the validating embedding entry points, argmax read-backs); tensors that the region reads without writing
+ * them first (parameters, optimizer state, inputs) must exist before capture_begin and stay where they are; values
+ * passed BY VALUE (learning rate, AdamW step) are frozen into the graph: use the *_indirect optimizer entry points,
+ * which read them from device memory.  capture_end(NULL) abandons the recording.  Replays are asynchronous on the
+ * stream they are launched on; one capture at a time per process.
+ * ------------------------------------------------------------------------------------------- */
+typedef void* bf_graph_t;
+int bf_hip_capture_begin(bf_stream_t stream);
+int bf_hip_capture_end(bf_graph_t* graph);
+int bf_hip_graph_launch(bf_graph_t graph, bf_stream_t stream);
+int bf_hip_graph_destroy(bf_graph_t graph);
+
 int bf_hip_memcpy_h2d(void* dst, const void* src, size_t bytes);   /* synchronous (fromHost) */
 int bf_hip_memcpy_d2h(void* dst, const void* src, size_t bytes);   /* synchronous (toHost)   */
 int bf_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, bf_stream_t stream);  /* clone() */
@@ -412,6 +433,20 @@ int bf_hip_sgd_multi(float* const* params, const float* const* grads, const size
 int bf_hip_adamw_multi(float* const* params, const float* const* grads, float* const* m, float* const* v,
                        const size_t* counts, size_t numTensors, long long step, float lr, float beta1, float beta2,
                        float eps, float weightDecay, bf_stream_t stream);
+/* The same steps with what changes from step to step read from DEVICE memory, for launches that are recorded in a
+ * graph (a value passed by value would be frozen into it).  bf_hip_adamw_publish / bf_hip_sgd_publish write the block
+ * for one step (a one-thread kernel on `stream`, bias corrections computed on the host exactly as bf_hip_adamw_multi
+ * does): call it before each replay.  No counterpart in the reference. */
+typedef struct {
+    float lr, beta1, beta2, eps, weight_decay, bias1, bias2;   /* bias1 = 1 - beta1^t, bias2 = 1 - beta2^t */
+} bf_adamw_hyper;
+int bf_hip_adamw_publish(bf_adamw_hyper* hyperDevice, long long step, float lr, float beta1, float beta2, float eps,
+                         float weightDecay, bf_stream_t stream);
+int bf_hip_adamw_multi_indirect(float* const* params, const float* const* grads, float* const* m, float* const* v,
+                                const size_t* counts, size_t numTensors, const bf_adamw_hyper* hyperDevice, bf_stream_t stream);
+int bf_hip_sgd_publish(float* lrDevice, float lr, bf_stream_t stream);
+int bf_hip_sgd_multi_indirect(float* const* params, const float* const* grads, const size_t* counts, size_t numTensors,
+                              const float* lrDevice, bf_stream_t stream);
 
 #ifdef __cplusplus
 }

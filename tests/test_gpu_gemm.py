@@ -57,6 +57,21 @@ def test_fp32_gemm_large_tile_path(hip, rng):
     assert_close(c[rows], a[rows].astype(np.float64) @ b.astype(np.float64), what="matmul 128-tile")
 
 
+@pytest.mark.parametrize("m,k,n", [(70, 4100, 90), (130, 2500, 64), (128, 2047, 128)])
+def test_fp32_gemm_long_contraction(hip, rng, m, k, n):
+    """Few tiles and a contraction of 2048 or more: K is cut into slices that a second kernel adds in order (and one
+    just under the limit, which stays whole).  Against float64."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, b, g = r(rng, m, k), r(rng, k, n), r(rng, m, n)
+    da, db, dg = map(D.fromHost, (a, b, g))
+    assert_close(ops.matmul(da, db).toHost(), (a.astype(np.float64) @ b.astype(np.float64)).astype(f32), what="matmul", scale=float(np.sqrt(k)))
+    # a weight gradient: dB = X^T G over k rows of tokens
+    x, w, gy = r(rng, k, m), r(rng, m, n), r(rng, k, n)
+    dX, dW = ops.matmulBackward(D.fromHost(x), D.fromHost(w), D.fromHost(gy))
+    assert_close(dW.toHost(), (x.astype(np.float64).T @ gy.astype(np.float64)).astype(f32), what="dW", scale=float(np.sqrt(k)))
+    assert_close(dX.toHost(), (gy.astype(np.float64) @ w.astype(np.float64).T).astype(f32), what="dX", scale=float(np.sqrt(n)))
+
+
 def test_linear_rank3_and_identity(hip, oracle):
     """tests/backend/cpu/ops_tests.cpp:54-63,173-184."""
     D, ops = hip.DeviceTensor, hip.ops
