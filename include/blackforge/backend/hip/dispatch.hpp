@@ -1,15 +1,18 @@
 #pragma once
 // Device dispatch for the HIP backend: what `blackforge run|train|devices --device ...` needs in order to reach
-// hip::Executor, hip::Model and hip::runTraining.  The reference's CLI parses `cpu | cuda | cuda:N` into a DeviceSpec
+// hip::Executor, hip::Model and hip::runTraining; likewise the GPU branches of `generate` and `benchmark`.  The reference's CLI parses `cpu | cuda | cuda:N` into a DeviceSpec
 // and branches on it (src/main.cpp:118-186 parse, :298-395 run, :397-476 train, :86-112 devices); its runtime has
 // DeviceKind{CPU, CUDA} (include/blackforge/runtime/device.hpp:8) and its semantic analyser a closed list of target
 // names (src/sema/semantic_analyzer.cpp:12-17,139-144).  This header supplies the same pieces with `hip | hip:N` added:
 // the parser (same diagnostics, same exit-code meaning), the device family, the target-name check, the `devices`
 // listing, and the bodies of the run / train branches as functions over the reference's own ir / ast types, so the
-// CLI's edit is one `else if (spec.family == DeviceFamily::Hip)` per command.  Nothing here parses .bf programs.
+// CLI's edit is one `else if (spec.family == DeviceFamily::Hip)` per command.  Nothing here parses .bf programs or
+// text: `generate` starts from token ids (the tokenizer stays on the host side of the CLI).
 #include <algorithm>
 #include <cctype>
+#include <chrono>
 #include <cstddef>
+#include <cstdint>
 #include <iosfwd>
 #include <ostream>
 #include <string>
@@ -129,6 +132,72 @@ inline TrainRunResult trainOnDevice(const DeviceSpec& spec, const ast::Program& 
                                     const std::string& fromCheckpoint, const std::string& saveCheckpointPath, std::ostream* progress) {
     selectDevice(spec);
     return runTraining(program, module, fromCheckpoint, saveCheckpointPath, progress);
+}
+
+// The GPU branch of runGenerate (main.cpp:594-617), from token ids to token ids: the model of the module's precision
+// policy loads the checkpoint, the prompt goes through forwardIncremental once and every further token alone, each
+// chosen as the first maximum of the last position's logits (main.cpp:504-518).  The choice is made on the device, so
+// one index per token crosses to the host instead of the logits.  Like the CLI, generation stops quietly when the model
+// refuses a further position (its positional table is exhausted); `stoppedAtCapacity` reports that.
+struct GenerateOutcome {
+    std::vector<std::uint32_t> tokens;   // the prompt followed by the generated ids
+    bool stoppedAtCapacity = false;
+};
+
+inline GenerateOutcome generateOnDevice(const DeviceSpec& spec, const ir::Module& module, const std::string& fromCheckpoint,
+                                        const std::vector<std::uint32_t>& promptIds, std::size_t maxNewTokens) {
+    require(!module.models.empty(), "il programma non definisce alcun modello da eseguire");
+    require(!promptIds.empty(), "il prompt codificato e' vuoto (prompt vuoto?)");
+    selectDevice(spec);
+    Model loaded(module.models.front(), 42U, module.precision);
+    loadCheckpoint(loaded, fromCheckpoint);
+    loaded.resetGenerationState();
+    GenerateOutcome outcome;
+    outcome.tokens = promptIds;
+    const std::vector<float> promptFloats(promptIds.begin(), promptIds.end());
+    DeviceTensor logits = loaded.forwardIncremental(DeviceTensor::fromHost(runtime::Tensor({1, promptIds.size()}, promptFloats)));
+    for (std::size_t step = 0; step < maxNewTokens; ++step) {
+        const auto best = static_cast<std::uint32_t>(argmaxLastPosition(logits));
+        outcome.tokens.push_back(best);
+        try {
+            logits = loaded.forwardIncremental(DeviceTensor::fromHost(runtime::Tensor({1, 1}, {static_cast<float>(best)})));
+        } catch (const std::exception&) {
+            outcome.stoppedAtCapacity = true;
+            break;
+        }
+    }
+    return outcome;
+}
+
+// The GPU branch of runBenchmark (main.cpp:801-850): the executor on a synthetic batch, `warmupIterations` untimed runs,
+// then `measuredIterations` timed with the host clock (each run ends in a device-to-host copy, so the clock sees
+// finished work), mean milliseconds and examples per second, and the last output for the comparison with the CPU run.
+struct BenchmarkOutcome {
+    std::string deviceName;
+    std::vector<std::size_t> inputShape;
+    double meanMilliseconds = 0.0;
+    double throughputSamplesPerSecond = 0.0;
+    runtime::Tensor output;
+};
+
+inline BenchmarkOutcome benchmarkOnDevice(const DeviceSpec& spec, const ir::ModelIR& model, std::size_t batchSize,
+                                          std::size_t warmupIterations, std::size_t measuredIterations) {
+    require(measuredIterations > 0, "benchmarkOnDevice: needs at least one measured iteration");
+    selectDevice(spec);
+    BenchmarkOutcome outcome;
+    outcome.deviceName = "GPU sconosciuta";
+    for (const HipDeviceInfo& d : enumerateDevices())
+        if (d.index == spec.index) outcome.deviceName = d.name.empty() ? d.arch : d.name;   // some drivers report no marketing name
+    Executor executor;
+    const runtime::Tensor input = executor.makeSyntheticInput(model, batchSize);
+    outcome.inputShape = input.shape();
+    for (std::size_t i = 0; i < warmupIterations; ++i) (void)executor.run(model, input);
+    const auto start = std::chrono::steady_clock::now();
+    for (std::size_t i = 0; i < measuredIterations; ++i) outcome.output = executor.run(model, input);
+    const auto end = std::chrono::steady_clock::now();
+    outcome.meanMilliseconds = std::chrono::duration<double, std::milli>(end - start).count() / static_cast<double>(measuredIterations);
+    outcome.throughputSamplesPerSecond = outcome.meanMilliseconds > 0.0 ? static_cast<double>(batchSize) * 1000.0 / outcome.meanMilliseconds : 0.0;
+    return outcome;
 }
 
 }  // namespace blackforge::backend::hip

@@ -8,7 +8,10 @@
 //      both backends starting from their own seed-42 initialisation and reading the same BFDATA1 file;
 //   4. checkpoint interop: the CPU run's file loads into hip::Model and the other way round;
 //   5. device dispatch (hip/dispatch.hpp): `--device hip` / `hip:0` reach hip::Executor, hip::Model and hip::runTraining
-//      through runOnDevice / trainOnDevice with the results of steps 1 and 3; `hip:99` and `cuda` are refused.
+//      through runOnDevice / trainOnDevice with the results of steps 1 and 3; `hip:99` and `cuda` are refused;
+//   6. generate: greedy decoding from a trained checkpoint through generateOnDevice gives the token ids of the CPU
+//      model's forwardIncremental + first-maximum loop, including the stop when the positional table is exhausted;
+//   7. benchmark: benchmarkOnDevice times the executor and its last output matches the CPU executor's.
 // Prints one line per check and exits non-zero on the first failure.
 #include <cmath>
 #include <cstdio>
@@ -232,6 +235,59 @@ int main(int argc, char** argv) {
             report(refused("hip:99"), "--device hip:99 parses and is refused at selection (std::invalid_argument)");
             report(refused("cuda"), "--device cuda parses and is refused by the HIP backend");
             report(!hip::parseDeviceSpec("hip:x", spec, error) && error == "indice GPU non valido in 'hip:x'", "--device hip:x is a parse error");
+        }
+        // 6. greedy generation from the CPU run's checkpoint (the loop of runGenerate, src/main.cpp:575-592)
+        {
+            hip::DeviceSpec spec;
+            std::string error;
+            hip::parseDeviceSpec("hip:0", spec, error);
+            ir::Module module;
+            module.models.push_back(lm);
+            const std::string ckpt = tmp + "/dropin_tiny_lm_cpu.bfckpt";
+            auto cpuGenerate = [&](const std::vector<std::uint32_t>& prompt, std::size_t maxNew, bool& stopped) {
+                cpu::Model cm(lm);
+                cpu::loadCheckpoint(cm, ckpt);
+                cm.resetGenerationState();
+                std::vector<std::uint32_t> out = prompt;
+                std::vector<float> pf(prompt.begin(), prompt.end());
+                bf::runtime::Tensor logits = cm.forwardIncremental(bf::runtime::Tensor({1, prompt.size()}, pf));
+                stopped = false;
+                for (std::size_t step = 0; step < maxNew; ++step) {
+                    const std::size_t vocab = logits.dim(2), last = logits.dim(1) - 1;
+                    std::size_t best = 0;
+                    for (std::size_t v = 1; v < vocab; ++v)
+                        if (logits.at(last * vocab + v) > logits.at(last * vocab + best)) best = v;
+                    out.push_back(static_cast<std::uint32_t>(best));
+                    try {
+                        logits = cm.forwardIncremental(bf::runtime::Tensor({1, 1}, {static_cast<float>(best)}));
+                    } catch (const std::exception&) { stopped = true; break; }
+                }
+                return out;
+            };
+            for (const auto& [prompt, maxNew] : std::vector<std::pair<std::vector<std::uint32_t>, std::size_t>>{{{3, 17, 40}, 4}, {{5}, 8}, {{1, 2, 3, 4, 5, 6, 7}, 20}}) {
+                bool stopped = false;
+                std::vector<std::uint32_t> want = cpuGenerate(prompt, maxNew, stopped);
+                hip::GenerateOutcome got = hip::generateOnDevice(spec, module, ckpt, prompt, maxNew);
+                report(got.tokens == want && got.stoppedAtCapacity == stopped,
+                       "generate: " + std::to_string(prompt.size()) + " prompt tokens + " + std::to_string(maxNew) + " requested -> " +
+                           std::to_string(got.tokens.size()) + " ids identical to the CPU loop" + (stopped ? " (both stop at the positional table's end)" : ""));
+            }
+        }
+        // 7. the benchmark command's GPU branch (src/main.cpp:801-850)
+        {
+            hip::DeviceSpec spec;
+            std::string error;
+            hip::parseDeviceSpec("hip", spec, error);
+            hip::BenchmarkOutcome outcome = hip::benchmarkOnDevice(spec, mlp, 16, 2, 5);
+            cpu::Executor cx;
+            bf::runtime::Tensor want = cx.run(mlp, cx.makeSyntheticInput(mlp, 16));
+            float maxAbsDiff = 0.0F;
+            for (std::size_t i = 0; i < want.elementCount() && i < outcome.output.elementCount(); ++i)
+                maxAbsDiff = std::max(maxAbsDiff, std::fabs(want.at(i) - outcome.output.at(i)));
+            report(outcome.output.shape() == want.shape() && maxAbsDiff <= 1e-5F && outcome.meanMilliseconds > 0.0 && outcome.throughputSamplesPerSecond > 0.0 &&
+                       outcome.inputShape == std::vector<std::size_t>{16, 10} && !outcome.deviceName.empty(),
+                   "benchmark: benchmarkOnDevice on '" + outcome.deviceName + "' " + std::to_string(outcome.meanMilliseconds) + " ms per run, max abs diff vs the CPU executor " +
+                       std::to_string(maxAbsDiff));
         }
     } catch (const std::exception& e) {
         report(false, std::string("exception: ") + e.what());
