@@ -20,34 +20,34 @@ constexpr int BK = 32;
 
 // One thread's share of a [BK x BT] operand tile: element e = tid + 256*i of the tile, walked so that consecutive
 // threads read consecutive global addresses (along k when the tile dimension t is a row of X, along t otherwise).
-template <int BT>
+template <int BT, int BKT = BK>
 struct TileRegs {
-    static constexpr int kPer = BK * BT / 256;
+    static constexpr int kPer = BKT * BT / 256;
     float v[kPer];
 };
 
 // Issues the global loads of the tile of op(X) at (k0, t0) into registers, zero outside the matrix or the K slice.
 // op(X)[k][t] = X[t*ld + k] when t is the row of X (T_IS_ROW), or X[k*ld + t] when t is its column.
-template <int BT, bool T_IS_ROW>
-__device__ __forceinline__ void fetchTile(TileRegs<BT>& regs, const float* __restrict__ X, size_t ld, size_t tExtent,
+template <int BT, bool T_IS_ROW, int BKT = BK>
+__device__ __forceinline__ void fetchTile(TileRegs<BT, BKT>& regs, const float* __restrict__ X, size_t ld, size_t tExtent,
                                           size_t kEnd, size_t t0, size_t k0, int tid) {
 #pragma unroll
-    for (int i = 0; i < TileRegs<BT>::kPer; ++i) {
+    for (int i = 0; i < TileRegs<BT, BKT>::kPer; ++i) {
         const int e = tid + 256 * i;
         int k, t;
-        if constexpr (T_IS_ROW) { k = e % BK; t = e / BK; }
+        if constexpr (T_IS_ROW) { k = e % BKT; t = e / BKT; }
         else { t = e % BT; k = e / BT; }
         const size_t gt = t0 + t, gk = k0 + k;
         regs.v[i] = (gt < tExtent && gk < kEnd) ? (T_IS_ROW ? X[gt * ld + gk] : X[gk * ld + gt]) : 0.0f;
     }
 }
-template <int BT, bool T_IS_ROW>
-__device__ __forceinline__ void commitTile(float (*lds)[BT + 4], const TileRegs<BT>& regs, int tid) {
+template <int BT, bool T_IS_ROW, int BKT = BK, int PAD = 4>
+__device__ __forceinline__ void commitTile(float (*lds)[BT + PAD], const TileRegs<BT, BKT>& regs, int tid) {
 #pragma unroll
-    for (int i = 0; i < TileRegs<BT>::kPer; ++i) {
+    for (int i = 0; i < TileRegs<BT, BKT>::kPer; ++i) {
         const int e = tid + 256 * i;
         int k, t;
-        if constexpr (T_IS_ROW) { k = e % BK; t = e / BK; }
+        if constexpr (T_IS_ROW) { k = e % BKT; t = e / BKT; }
         else { t = e % BT; k = e / BT; }
         lds[k][t] = regs.v[i];
     }
@@ -133,6 +133,101 @@ __global__ void __launch_bounds__(256) gemmF32Kernel(const float* __restrict__ A
         }
 }
 
+// Small products (a model a few hundred wide: every product of it is a handful of 64 x 64 tiles whose four K steps
+// each wait a full round trip to memory): 32 x 32 tiles, four wavefronts with a 16 x 16 share each on the
+// 16x16x4 fp32 MFMA, and K steps of 128, so that a contraction up to 128 long is ONE round of loads and one barrier
+// and a workgroup's MFMA chain is 32 instructions long.  Two accumulators alternate so that consecutive MFMAs do not
+// depend on each other; they are added at the end (a fixed order: results are reproducible).
+//   A: lane l holds A[i = l % 16][k = l / 16]   B: lane l holds B[k = l / 16][j = l % 16]
+//   D: lane l, register r holds D[i = 4*(l/16) + r][j = l % 16]
+// An operand tile lies in LDS the way it lies in memory, so that the copy writes consecutive words: [t][k] with rows of
+// 132 floats when k is the contiguous dimension (the 16 rows x 4 k a wavefront reads cover all 64 banks), [k][t] with
+// rows of 48 floats otherwise (4 k rows x 16 t: likewise).
+constexpr int SBK = 128, SBT = 32;
+constexpr int SROW_K = SBK + 4, SROW_T = SBT + 16;
+constexpr int SWORDS = SBK * SROW_T > SBT * SROW_K ? SBK * SROW_T : SBT * SROW_K;
+
+template <bool K_CONTIG>
+struct SmallOperand {
+    static constexpr int kPer = SBK * SBT / 256;
+    float v[kPer];
+    // X[t*ld + k] when k is contiguous, X[k*ld + t] otherwise; zero outside the matrix or the K slice
+    __device__ __forceinline__ void fetch(const float* __restrict__ X, size_t ld, size_t tExtent, size_t kEnd, size_t t0, size_t k0, int tid) {
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int e = tid + 256 * i;
+            const int k = K_CONTIG ? e % SBK : e / SBT, t = K_CONTIG ? e / SBK : e % SBT;
+            const size_t gt = t0 + t, gk = k0 + k;
+            v[i] = (gt < tExtent && gk < kEnd) ? (K_CONTIG ? X[gt * ld + gk] : X[gk * ld + gt]) : 0.0f;
+        }
+    }
+    __device__ __forceinline__ void commit(float* lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int e = tid + 256 * i;
+            if constexpr (K_CONTIG) lds[(e / SBK) * SROW_K + e % SBK] = v[i];
+            else lds[(e / SBT) * SROW_T + e % SBT] = v[i];
+        }
+    }
+    // element (t, k) of the tile
+    static __device__ __forceinline__ float at(const float* lds, int t, int k) {
+        return K_CONTIG ? lds[t * SROW_K + k] : lds[k * SROW_T + t];
+    }
+};
+
+template <bool TRANS_A, bool TRANS_B>
+__global__ void __launch_bounds__(256) gemmF32SmallKernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                           float* __restrict__ C, size_t M, size_t N, size_t K, size_t kPerSlice,
+                                                           size_t sliceStride) {
+    __shared__ float as[SWORDS];
+    __shared__ float bs[SWORDS];
+    using OpA = SmallOperand<!TRANS_A>;   // A stored [M,K]: k contiguous
+    using OpB = SmallOperand<TRANS_B>;    // B stored [N,K]: k contiguous
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave >> 1) * 16, wn0 = (wave & 1) * 16;
+    const size_t m0 = size_t(blockIdx.y) * SBT, n0 = size_t(blockIdx.x) * SBT;
+    const int li = lane & 15, lk = lane >> 4;
+    const size_t kBegin = size_t(blockIdx.z) * kPerSlice, kEnd = kBegin + kPerSlice < K ? kBegin + kPerSlice : K;
+    C += size_t(blockIdx.z) * sliceStride;
+    float4v acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+    OpA aNext;
+    OpB bNext;
+    auto fetch = [&](size_t k0) {
+        aNext.fetch(A, TRANS_A ? M : K, M, kEnd, m0, k0, tid);
+        bNext.fetch(B, TRANS_B ? K : N, N, kEnd, n0, k0, tid);
+    };
+    if (kBegin < kEnd) fetch(kBegin);
+    for (size_t k0 = kBegin; k0 < kEnd; k0 += SBK) {
+        aNext.commit(as, tid);
+        bNext.commit(bs, tid);
+        __syncthreads();
+        if (k0 + SBK < kEnd) fetch(k0 + SBK);
+#pragma unroll
+        for (int kk = 0; kk < SBK; kk += 8) {
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(OpA::at(as, wm0 + li, kk + lk), OpB::at(bs, wn0 + li, kk + lk), acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(OpA::at(as, wm0 + li, kk + 4 + lk), OpB::at(bs, wn0 + li, kk + 4 + lk), acc1, 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    const size_t col = n0 + wn0 + li;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const size_t row = m0 + wm0 + 4 * lk + r;
+        if (row < M && col < N) C[row * N + col] = acc0[r] + acc1[r];
+    }
+}
+
+int launchSmallGemm(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t slices,
+                    size_t kPerSlice, size_t sliceStride, hipStream_t s) {
+    dim3 grid(unsigned((N + SBT - 1) / SBT), unsigned((M + SBT - 1) / SBT), unsigned(slices));
+    if (!transA && !transB) gemmF32SmallKernel<false, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else if (!transA && transB) gemmF32SmallKernel<false, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else if (transA && !transB) gemmF32SmallKernel<true, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else gemmF32SmallKernel<true, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
 // C[i] = sum over slices of partial[s*stride + i], slices added in index order (deterministic).
 __global__ void __launch_bounds__(kBlock) sliceSumKernel(const float* __restrict__ partial, float* __restrict__ C, size_t count,
                                                          size_t stride, int slices) {
@@ -179,6 +274,26 @@ extern "C" int bf_hip_gemm_f32(int transA, int transB, const float* A, const flo
     // microsecond (nothing hides its latencies) and a dependent launch about five, so contractions under 256 stay whole
     // (a small model's step is bounded by its launch count) and longer ones are cut into slices of at least two steps.
     const size_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+    // Fewer 64 x 64 tiles than half the chip: 32 x 32 tiles with K steps of 128.  A contraction is cut into slices (of
+    // at least four steps) only when it is long enough for a second launch to pay: 2048 and up.
+    if (tiles * 2 <= cus && (M + SBT - 1) / SBT <= 65535) {
+        const size_t smallTiles = ((M + SBT - 1) / SBT) * ((N + SBT - 1) / SBT);
+        size_t cut = 1;
+        if (K >= 16 * SBK && smallTiles < cus) cut = std::min<size_t>(std::min<size_t>(16, 2 * cus / smallTiles), K / (4 * SBK));
+        if (cut > 1) {
+            const size_t steps = (K + SBK - 1) / SBK, kPer = (steps + cut - 1) / cut * SBK;
+            cut = (K + kPer - 1) / kPer;
+            const size_t count = M * N;
+            Scratch partial(cut * count * sizeof(float));
+            if (partial.status != BF_OK) return partial.status;
+            int st = launchSmallGemm(transA, transB, A, B, partial.as<float>(), M, N, K, cut, kPer, count, s);
+            if (st != BF_OK) return st;
+            sliceSumKernel<<<gridFor(count, kBlock), kBlock, 0, s>>>(partial.as<float>(), C, count, count, int(cut));
+            BF_LAUNCH_CHECK();
+            return BF_OK;
+        }
+        return launchSmallGemm(transA, transB, A, B, C, M, N, K, 1, K, 0, s);
+    }
     size_t slices = 1;
     if (tiles < cus && K >= 8 * BK) slices = std::min<size_t>(std::min<size_t>(16, cus / tiles), K / (2 * BK));
     if (slices > 1) {
