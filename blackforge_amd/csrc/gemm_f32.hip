@@ -12,6 +12,7 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <cstdint>
 
 namespace bf {
 namespace {
@@ -147,26 +148,38 @@ constexpr int SBK = 128, SBT = 32;
 constexpr int SROW_K = SBK + 4, SROW_T = SBT + 16;
 constexpr int SWORDS = SBK * SROW_T > SBT * SROW_K ? SBK * SROW_T : SBT * SROW_K;
 
-template <bool K_CONTIG>
+// VEC = 4: every access is 16 bytes (the contiguous extent and the row pitch are multiples of 4 and the base is 16-byte
+// aligned; a group of four is then wholly inside or wholly outside the matrix); VEC = 1 takes any shape.
+template <bool K_CONTIG, int VEC>
 struct SmallOperand {
-    static constexpr int kPer = SBK * SBT / 256;
-    float v[kPer];
+    static constexpr int kPer = SBK * SBT / 256 / VEC;
+    static constexpr int kGroupsK = SBK / VEC, kGroupsT = SBT / VEC;
+    float v[kPer * VEC];
     // X[t*ld + k] when k is contiguous, X[k*ld + t] otherwise; zero outside the matrix or the K slice
     __device__ __forceinline__ void fetch(const float* __restrict__ X, size_t ld, size_t tExtent, size_t kEnd, size_t t0, size_t k0, int tid) {
 #pragma unroll
         for (int i = 0; i < kPer; ++i) {
             const int e = tid + 256 * i;
-            const int k = K_CONTIG ? e % SBK : e / SBT, t = K_CONTIG ? e / SBK : e % SBT;
+            const int k = K_CONTIG ? (e % kGroupsK) * VEC : e / kGroupsT, t = K_CONTIG ? e / kGroupsK : (e % kGroupsT) * VEC;
             const size_t gt = t0 + t, gk = k0 + k;
-            v[i] = (gt < tExtent && gk < kEnd) ? (K_CONTIG ? X[gt * ld + gk] : X[gk * ld + gt]) : 0.0f;
+            const bool inside = gt < tExtent && gk < kEnd;
+            const float* src = K_CONTIG ? X + gt * ld + gk : X + gk * ld + gt;
+            if constexpr (VEC == 4) {
+                const float4v q = inside ? loadf4(src) : float4v{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[4 * i + j] = q[j];
+            } else {
+                v[i] = inside ? *src : 0.0f;
+            }
         }
     }
     __device__ __forceinline__ void commit(float* lds, int tid) const {
 #pragma unroll
         for (int i = 0; i < kPer; ++i) {
             const int e = tid + 256 * i;
-            if constexpr (K_CONTIG) lds[(e / SBK) * SROW_K + e % SBK] = v[i];
-            else lds[(e / SBT) * SROW_T + e % SBT] = v[i];
+            float* dst = K_CONTIG ? lds + (e / kGroupsK) * SROW_K + (e % kGroupsK) * VEC : lds + (e / kGroupsT) * SROW_T + (e % kGroupsT) * VEC;
+            if constexpr (VEC == 4) storef4(dst, float4v{v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]});
+            else *dst = v[i];
         }
     }
     // element (t, k) of the tile
@@ -175,14 +188,16 @@ struct SmallOperand {
     }
 };
 
-template <bool TRANS_A, bool TRANS_B>
+// DEPTH register stages hold the K steps that follow the one being multiplied: a contraction of up to DEPTH steps has
+// all its loads in flight at once (a 512-token weight gradient waits for memory once, not four times).
+template <bool TRANS_A, bool TRANS_B, int VEC, int DEPTH>
 __global__ void __launch_bounds__(256) gemmF32SmallKernel(const float* __restrict__ A, const float* __restrict__ B,
                                                            float* __restrict__ C, size_t M, size_t N, size_t K, size_t kPerSlice,
                                                            size_t sliceStride) {
-    __shared__ float as[SWORDS];
-    __shared__ float bs[SWORDS];
-    using OpA = SmallOperand<!TRANS_A>;   // A stored [M,K]: k contiguous
-    using OpB = SmallOperand<TRANS_B>;    // B stored [N,K]: k contiguous
+    __shared__ __attribute__((aligned(16))) float as[SWORDS];
+    __shared__ __attribute__((aligned(16))) float bs[SWORDS];
+    using OpA = SmallOperand<!TRANS_A, VEC>;   // A stored [M,K]: k contiguous
+    using OpB = SmallOperand<TRANS_B, VEC>;    // B stored [N,K]: k contiguous
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm0 = (wave >> 1) * 16, wn0 = (wave & 1) * 16;
     const size_t m0 = size_t(blockIdx.y) * SBT, n0 = size_t(blockIdx.x) * SBT;
@@ -190,24 +205,33 @@ __global__ void __launch_bounds__(256) gemmF32SmallKernel(const float* __restric
     const size_t kBegin = size_t(blockIdx.z) * kPerSlice, kEnd = kBegin + kPerSlice < K ? kBegin + kPerSlice : K;
     C += size_t(blockIdx.z) * sliceStride;
     float4v acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
-    OpA aNext;
-    OpB bNext;
-    auto fetch = [&](size_t k0) {
-        aNext.fetch(A, TRANS_A ? M : K, M, kEnd, m0, k0, tid);
-        bNext.fetch(B, TRANS_B ? K : N, N, kEnd, n0, k0, tid);
-    };
-    if (kBegin < kEnd) fetch(kBegin);
-    for (size_t k0 = kBegin; k0 < kEnd; k0 += SBK) {
-        aNext.commit(as, tid);
-        bNext.commit(bs, tid);
-        __syncthreads();
-        if (k0 + SBK < kEnd) fetch(k0 + SBK);
+    OpA aStage[DEPTH];
+    OpB bStage[DEPTH];
 #pragma unroll
-        for (int kk = 0; kk < SBK; kk += 8) {
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(OpA::at(as, wm0 + li, kk + lk), OpB::at(bs, wn0 + li, kk + lk), acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(OpA::at(as, wm0 + li, kk + 4 + lk), OpB::at(bs, wn0 + li, kk + 4 + lk), acc1, 0, 0, 0);
+    for (int d = 0; d < DEPTH; ++d)
+        if (kBegin + size_t(d) * SBK < kEnd) {
+            aStage[d].fetch(A, TRANS_A ? M : K, M, kEnd, m0, kBegin + size_t(d) * SBK, tid);
+            bStage[d].fetch(B, TRANS_B ? K : N, N, kEnd, n0, kBegin + size_t(d) * SBK, tid);
         }
-        __syncthreads();
+    for (size_t base = kBegin; base < kEnd; base += size_t(DEPTH) * SBK) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const size_t k0 = base + size_t(d) * SBK;
+            if (k0 >= kEnd) break;
+            aStage[d].commit(as, tid);
+            bStage[d].commit(bs, tid);
+            __syncthreads();
+            if (k0 + size_t(DEPTH) * SBK < kEnd) {
+                aStage[d].fetch(A, TRANS_A ? M : K, M, kEnd, m0, k0 + size_t(DEPTH) * SBK, tid);
+                bStage[d].fetch(B, TRANS_B ? K : N, N, kEnd, n0, k0 + size_t(DEPTH) * SBK, tid);
+            }
+#pragma unroll
+            for (int kk = 0; kk < SBK; kk += 8) {
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(OpA::at(as, wm0 + li, kk + lk), OpB::at(bs, wn0 + li, kk + lk), acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(OpA::at(as, wm0 + li, kk + 4 + lk), OpB::at(bs, wn0 + li, kk + 4 + lk), acc1, 0, 0, 0);
+            }
+            __syncthreads();
+        }
     }
     const size_t col = n0 + wn0 + li;
 #pragma unroll
@@ -217,15 +241,26 @@ __global__ void __launch_bounds__(256) gemmF32SmallKernel(const float* __restric
     }
 }
 
-int launchSmallGemm(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t slices,
-                    size_t kPerSlice, size_t sliceStride, hipStream_t s) {
+template <int VEC, int DEPTH>
+int launchSmallGemmAs(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t slices,
+                      size_t kPerSlice, size_t sliceStride, hipStream_t s) {
     dim3 grid(unsigned((N + SBT - 1) / SBT), unsigned((M + SBT - 1) / SBT), unsigned(slices));
-    if (!transA && !transB) gemmF32SmallKernel<false, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else if (!transA && transB) gemmF32SmallKernel<false, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else if (transA && !transB) gemmF32SmallKernel<true, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else gemmF32SmallKernel<true, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    if (!transA && !transB) gemmF32SmallKernel<false, false, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else if (!transA && transB) gemmF32SmallKernel<false, true, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else if (transA && !transB) gemmF32SmallKernel<true, false, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    else gemmF32SmallKernel<true, true, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
     BF_LAUNCH_CHECK();
     return BF_OK;
+}
+
+int launchSmallGemm(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t slices,
+                    size_t kPerSlice, size_t sliceStride, hipStream_t s) {
+    // 16-byte accesses need the contiguous extent of either operand (K, or M / N for an operand stored with K as its rows)
+    // to be a multiple of 4 and 16-byte aligned bases
+    auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    const bool vec = aligned16(A) && aligned16(B) && (transA ? M : K) % 4 == 0 && (transB ? K : N) % 4 == 0;
+    if (vec) return launchSmallGemmAs<4, 4>(transA, transB, A, B, C, M, N, K, slices, kPerSlice, sliceStride, s);
+    return launchSmallGemmAs<1, 1>(transA, transB, A, B, C, M, N, K, slices, kPerSlice, sliceStride, s);
 }
 
 // C[i] = sum over slices of partial[s*stride + i], slices added in index order (deterministic).
