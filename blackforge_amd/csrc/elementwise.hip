@@ -116,13 +116,14 @@ struct RowGeom {
     int vec;
 };
 
-RowGeom rowGeometry(size_t rows, size_t features, bool canVectorise, unsigned maxRowBlocks = 0, unsigned rowsPerThread = 1) {
+RowGeom rowGeometry(size_t rows, size_t features, bool canVectorise, unsigned maxRowBlocks = 0, unsigned rowsPerThread = 1,
+                    unsigned threads = 256) {
     RowGeom g;
     g.vec = (canVectorise && features % 4 == 0) ? 4 : 1;
     size_t cols = features / g.vec;
     unsigned bx = 1;
     while (bx < 256 && bx < cols) bx <<= 1;
-    unsigned by = 256 / bx;
+    unsigned by = std::max(threads / bx, 1u);
     unsigned gx = unsigned((cols + bx - 1) / bx);
     size_t rowBlocks = (rows + size_t(by) * rowsPerThread - 1) / (size_t(by) * rowsPerThread);
     // streaming kernels (maxRowBlocks == 0) take every row block once, in address order; reductions cap the
@@ -176,12 +177,12 @@ __global__ void __launch_bounds__(256) biasKernel(const float* __restrict__ x, c
 // Column sums, optionally fused with dGemm = dHidden * act'(gemm + bias) (FUSED = 1).
 // Each block reduces its rows per column in registers, then over threadIdx.y through LDS, and writes
 // one partial row per blockIdx.y; columnFinishKernel adds the partial rows in a fixed order.
-template <int VEC, int FUSED, int ACT, bool NT>
-__global__ void __launch_bounds__(256) columnSumKernel(const float* __restrict__ src, const float* __restrict__ bias,
+template <int VEC, int FUSED, int ACT, bool NT, int THREADS = 256>
+__global__ void __launch_bounds__(THREADS) columnSumKernel(const float* __restrict__ src, const float* __restrict__ bias,
                                                         const float* __restrict__ dHidden, float* __restrict__ dGemm,
                                                         float* __restrict__ partial, size_t rows, size_t features,
                                                         unsigned short* __restrict__ image = nullptr) {
-    __shared__ float lds[256 * 4];
+    __shared__ float lds[THREADS * 4];
     size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
     bool active = col < features;
     typename Pack<VEC>::T acc = {};
@@ -278,7 +279,9 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
     bool vec = aligned16(src) && (!FUSED || (aligned16(bias) && aligned16(dHidden) && aligned16(dGemm)));
     // a matrix small enough for one row of blocks to walk is summed in one launch, straight into dBias
     const bool single = rows * features <= (size_t(1) << 16);
-    RowGeom g = rowGeometry(rows, features, vec, single ? 1 : 256, 4);
+    // the lone block of the one-launch form takes 1024 threads when the matrix is narrow: a quarter of the rounds of loads
+    const bool wide = single && rows >= 256 && features <= 1024;
+    RowGeom g = rowGeometry(rows, features, vec, single ? 1 : 256, 4, wide ? 1024 : 256);
     size_t parts = g.grid.y;
     if (workspace && dBias && parts * features > workspaceFloats)
         return failInvalid("column_sum", "the partial sums (" + std::to_string(parts) + " rows of " + std::to_string(features) +
@@ -290,7 +293,10 @@ int launchColumnSum(const float* src, const float* bias, const float* dHidden, f
     // bytes per element: the source, and on the fused route the second input and whichever outputs are written
     const size_t perElement = 4 + (FUSED ? 4 + (dGemm ? 4 : 0) + (image ? 2 : 0) : 0);
     const bool nt = streamsPastCache(rows * features * perElement);
-    if (g.vec == 4) {
+    if (wide) {
+        if (g.vec == 4) columnSumKernel<4, FUSED, ACT, false, 1024><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features, image);
+        else columnSumKernel<1, FUSED, ACT, false, 1024><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features);
+    } else if (g.vec == 4) {
         if (nt) columnSumKernel<4, FUSED, ACT, true><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features, image);
         else columnSumKernel<4, FUSED, ACT, false><<<g.grid, g.block, 0, stream>>>(src, bias, dHidden, dGemm, partial, rows, features, image);
     } else {
