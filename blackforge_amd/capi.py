@@ -90,6 +90,7 @@ SIGNATURES = {
     "bf_hip_concat_seq": [P, P, P, c_size, c_size, c_size, c_size, S],
     "bf_hip_argmax_last_position": [P, c_size, c_size, ctypes.POINTER(c_ll), S],
     "bf_hip_gemm_f32": [c_int, c_int, P, P, P, c_size, c_size, c_size, S],
+    "bf_hip_gemm_f32_adds": [c_int, c_int, P, P, P, P, P, c_size, c_size, c_size, S],
     "bf_hip_cvt_f32_bf16": [P, P, c_size, S],
     "bf_hip_cvt_f32_bf16_transpose": [P, P, c_size, c_size, S],
     "bf_hip_gemm_bf16_nt": [P, P, P, c_size, c_size, c_size, S],

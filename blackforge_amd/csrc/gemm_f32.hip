@@ -54,6 +54,14 @@ __device__ __forceinline__ void commitTile(float (*lds)[BT + PAD], const TileReg
     }
 }
 
+// What the store adds to a finished product: an optional bias row, then an optional residual matrix (which may be the
+// output itself: each element is read and written by one thread), in the order the separate add kernels use.
+__device__ __forceinline__ float withAdds(float v, const float* __restrict__ bias, const float* residual, size_t index, size_t col) {
+    if (bias) v += bias[col];
+    if (residual) v += residual[index];
+    return v;
+}
+
 template <int BM, int BN>
 struct GemmTile {
     static constexpr int kPad = 4;
@@ -68,8 +76,8 @@ struct GemmTile {
 // multiplied out of LDS.
 template <int BM, int BN, bool TRANS_A, bool TRANS_B>
 __global__ void __launch_bounds__(256) gemmF32Kernel(const float* __restrict__ A, const float* __restrict__ B,
-                                                      float* __restrict__ C, size_t M, size_t N, size_t K, size_t kPerSlice,
-                                                      size_t sliceStride) {
+                                                      float* C, size_t M, size_t N, size_t K, size_t kPerSlice,
+                                                      size_t sliceStride, const float* __restrict__ bias, const float* residual) {
     constexpr int WM = BM / 2, WN = BN / 2;      // 2 x 2 wavefronts
     constexpr int TM = WM / 32, TN = WN / 32;    // 32x32 MFMA tiles per wavefront
     __shared__ GemmTile<BM, BN> tile;
@@ -129,7 +137,7 @@ __global__ void __launch_bounds__(256) gemmF32Kernel(const float* __restrict__ A
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 size_t row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * lk + (r % 4);
-                if (row < M && col < N) C[row * N + col] = acc[i][j][r];
+                if (row < M && col < N) C[row * N + col] = withAdds(acc[i][j][r], bias, residual, row * N + col, col);
             }
         }
 }
@@ -192,8 +200,8 @@ struct SmallOperand {
 // all its loads in flight at once (a 512-token weight gradient waits for memory once, not four times).
 template <bool TRANS_A, bool TRANS_B, int VEC, int DEPTH>
 __global__ void __launch_bounds__(256) gemmF32SmallKernel(const float* __restrict__ A, const float* __restrict__ B,
-                                                           float* __restrict__ C, size_t M, size_t N, size_t K, size_t kPerSlice,
-                                                           size_t sliceStride) {
+                                                           float* C, size_t M, size_t N, size_t K, size_t kPerSlice,
+                                                           size_t sliceStride, const float* __restrict__ bias, const float* residual) {
     __shared__ __attribute__((aligned(16))) float as[SWORDS];
     __shared__ __attribute__((aligned(16))) float bs[SWORDS];
     using OpA = SmallOperand<!TRANS_A, VEC>;   // A stored [M,K]: k contiguous
@@ -237,50 +245,51 @@ __global__ void __launch_bounds__(256) gemmF32SmallKernel(const float* __restric
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const size_t row = m0 + wm0 + 4 * lk + r;
-        if (row < M && col < N) C[row * N + col] = acc0[r] + acc1[r];
+        if (row < M && col < N) C[row * N + col] = withAdds(acc0[r] + acc1[r], bias, residual, row * N + col, col);
     }
 }
 
 template <int VEC, int DEPTH>
 int launchSmallGemmAs(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t slices,
-                      size_t kPerSlice, size_t sliceStride, hipStream_t s) {
+                      size_t kPerSlice, size_t sliceStride, const float* bias, const float* residual, hipStream_t s) {
     dim3 grid(unsigned((N + SBT - 1) / SBT), unsigned((M + SBT - 1) / SBT), unsigned(slices));
-    if (!transA && !transB) gemmF32SmallKernel<false, false, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else if (!transA && transB) gemmF32SmallKernel<false, true, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else if (transA && !transB) gemmF32SmallKernel<true, false, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else gemmF32SmallKernel<true, true, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    if (!transA && !transB) gemmF32SmallKernel<false, false, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride, bias, residual);
+    else if (!transA && transB) gemmF32SmallKernel<false, true, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride, bias, residual);
+    else if (transA && !transB) gemmF32SmallKernel<true, false, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride, bias, residual);
+    else gemmF32SmallKernel<true, true, VEC, DEPTH><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride, bias, residual);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
 
 int launchSmallGemm(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t slices,
-                    size_t kPerSlice, size_t sliceStride, hipStream_t s) {
+                    size_t kPerSlice, size_t sliceStride, const float* bias, const float* residual, hipStream_t s) {
     // 16-byte accesses need the contiguous extent of either operand (K, or M / N for an operand stored with K as its rows)
     // to be a multiple of 4 and 16-byte aligned bases
     auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     const bool vec = aligned16(A) && aligned16(B) && (transA ? M : K) % 4 == 0 && (transB ? K : N) % 4 == 0;
-    if (vec) return launchSmallGemmAs<4, 4>(transA, transB, A, B, C, M, N, K, slices, kPerSlice, sliceStride, s);
-    return launchSmallGemmAs<1, 1>(transA, transB, A, B, C, M, N, K, slices, kPerSlice, sliceStride, s);
+    if (vec) return launchSmallGemmAs<4, 4>(transA, transB, A, B, C, M, N, K, slices, kPerSlice, sliceStride, bias, residual, s);
+    return launchSmallGemmAs<1, 1>(transA, transB, A, B, C, M, N, K, slices, kPerSlice, sliceStride, bias, residual, s);
 }
 
 // C[i] = sum over slices of partial[s*stride + i], slices added in index order (deterministic).
-__global__ void __launch_bounds__(kBlock) sliceSumKernel(const float* __restrict__ partial, float* __restrict__ C, size_t count,
-                                                         size_t stride, int slices) {
+__global__ void __launch_bounds__(kBlock) sliceSumKernel(const float* __restrict__ partial, float* C, size_t count,
+                                                         size_t stride, int slices, size_t N, const float* __restrict__ bias,
+                                                         const float* residual) {
     const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= count) return;
     float sum = partial[i];
     for (int s = 1; s < slices; ++s) sum += partial[size_t(s) * stride + i];
-    C[i] = sum;
+    C[i] = withAdds(sum, bias, residual, i, i % N);
 }
 
 template <int BM, int BN>
 int launchGemm(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, size_t slices,
-               size_t kPerSlice, size_t sliceStride, hipStream_t s) {
+               size_t kPerSlice, size_t sliceStride, const float* bias, const float* residual, hipStream_t s) {
     dim3 grid(unsigned((N + BN - 1) / BN), unsigned((M + BM - 1) / BM), unsigned(slices));
-    if (!transA && !transB) gemmF32Kernel<BM, BN, false, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else if (!transA && transB) gemmF32Kernel<BM, BN, false, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else if (transA && !transB) gemmF32Kernel<BM, BN, true, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
-    else gemmF32Kernel<BM, BN, true, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride);
+    if (!transA && !transB) gemmF32Kernel<BM, BN, false, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride, bias, residual);
+    else if (!transA && transB) gemmF32Kernel<BM, BN, false, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride, bias, residual);
+    else if (transA && !transB) gemmF32Kernel<BM, BN, true, false><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride, bias, residual);
+    else gemmF32Kernel<BM, BN, true, true><<<grid, 256, 0, s>>>(A, B, C, M, N, K, kPerSlice, sliceStride, bias, residual);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -290,18 +299,24 @@ int launchGemm(int transA, int transB, const float* A, const float* B, float* C,
 
 using namespace bf;
 
-extern "C" int bf_hip_gemm_f32(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N,
-                               size_t K, bf_stream_t stream) {
+namespace bf {
+namespace {
+// C = op(A) op(B) (+ bias per column) (+ residual); with K slices the adds move to the kernel that sums the slices.
+int gemmF32(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K, const float* bias,
+            const float* residual, bf_stream_t stream) {
     if (M == 0 || N == 0) return BF_OK;
     BF_REQUIRE(C != nullptr, "NULL output");
-    if (K == 0) return bf_hip_fill_zero(C, M * N * sizeof(float), stream);
+    if (K == 0) {
+        BF_REQUIRE(!bias && !residual, "an empty contraction with a bias or residual is not supported");
+        return bf_hip_fill_zero(C, M * N * sizeof(float), stream);
+    }
     BF_REQUIRE(A && B, "NULL operand");
     BF_REQUIRE((M + 63) / 64 <= 65535, "M too large");
     // Large tiles once they alone can fill the chip twice over; small tiles otherwise.
     hipStream_t s = asStream(stream);
     const size_t cus = size_t(computeUnits());
     size_t bigTiles = ((M + 127) / 128) * ((N + 127) / 128);
-    if (bigTiles >= 2 * cus) return launchGemm<128, 128>(transA, transB, A, B, C, M, N, K, 1, K, 0, s);
+    if (bigTiles >= 2 * cus) return launchGemm<128, 128>(transA, transB, A, B, C, M, N, K, 1, K, 0, bias, residual, s);
     // Few tiles and a long contraction (the weight gradients of a small model: a [features x features] product
     // over all tokens): cut K into slices so that more workgroups share it; a second kernel adds the slices in
     // order.
@@ -321,13 +336,13 @@ extern "C" int bf_hip_gemm_f32(int transA, int transB, const float* A, const flo
             const size_t count = M * N;
             Scratch partial(cut * count * sizeof(float));
             if (partial.status != BF_OK) return partial.status;
-            int st = launchSmallGemm(transA, transB, A, B, partial.as<float>(), M, N, K, cut, kPer, count, s);
+            int st = launchSmallGemm(transA, transB, A, B, partial.as<float>(), M, N, K, cut, kPer, count, nullptr, nullptr, s);
             if (st != BF_OK) return st;
-            sliceSumKernel<<<gridFor(count, kBlock), kBlock, 0, s>>>(partial.as<float>(), C, count, count, int(cut));
+            sliceSumKernel<<<gridFor(count, kBlock), kBlock, 0, s>>>(partial.as<float>(), C, count, count, int(cut), N, bias, residual);
             BF_LAUNCH_CHECK();
             return BF_OK;
         }
-        return launchSmallGemm(transA, transB, A, B, C, M, N, K, 1, K, 0, s);
+        return launchSmallGemm(transA, transB, A, B, C, M, N, K, 1, K, 0, bias, residual, s);
     }
     size_t slices = 1;
     if (tiles < cus && K >= 8 * BK) slices = std::min<size_t>(std::min<size_t>(16, cus / tiles), K / (2 * BK));
@@ -337,11 +352,23 @@ extern "C" int bf_hip_gemm_f32(int transA, int transB, const float* A, const flo
         const size_t count = M * N;
         Scratch partial(slices * count * sizeof(float));
         if (partial.status != BF_OK) return partial.status;
-        int st = launchGemm<64, 64>(transA, transB, A, B, partial.as<float>(), M, N, K, slices, kPer, count, s);
+        int st = launchGemm<64, 64>(transA, transB, A, B, partial.as<float>(), M, N, K, slices, kPer, count, nullptr, nullptr, s);
         if (st != BF_OK) return st;
-        sliceSumKernel<<<gridFor(count, kBlock), kBlock, 0, s>>>(partial.as<float>(), C, count, count, int(slices));
+        sliceSumKernel<<<gridFor(count, kBlock), kBlock, 0, s>>>(partial.as<float>(), C, count, count, int(slices), N, bias, residual);
         BF_LAUNCH_CHECK();
         return BF_OK;
     }
-    return launchGemm<64, 64>(transA, transB, A, B, C, M, N, K, 1, K, 0, s);
+    return launchGemm<64, 64>(transA, transB, A, B, C, M, N, K, 1, K, 0, bias, residual, s);
+}
+}  // namespace
+}  // namespace bf
+
+extern "C" int bf_hip_gemm_f32(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N,
+                               size_t K, bf_stream_t stream) {
+    return gemmF32(transA, transB, A, B, C, M, N, K, nullptr, nullptr, stream);
+}
+
+extern "C" int bf_hip_gemm_f32_adds(int transA, int transB, const float* A, const float* B, const float* bias, const float* residual,
+                                    float* C, size_t M, size_t N, size_t K, bf_stream_t stream) {
+    return gemmF32(transA, transB, A, B, C, M, N, K, bias, residual, stream);
 }

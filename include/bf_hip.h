@@ -228,6 +228,14 @@ int bf_hip_argmax_last_position(const float* logits, size_t seq, size_t vocab, l
  * G,B; dB: 1,0 on A,G); matmulTransposeBBackward autodiff.hpp:44 (dA: 0,0 on G,B; dB: 1,0 on G,A). */
 int bf_hip_gemm_f32(int transA, int transB, const float* A, const float* B, float* C, size_t M, size_t N, size_t K,
                     bf_stream_t stream);
+/* The same product with the adds that follow it done where the product is stored: C = op(A) op(B) + bias (a row of N,
+ * optional) + residual ([M,N], optional, may be C itself: C += op(A) op(B)), in that order, bit-identical to the
+ * product followed by addBias / addBiasResidual / add.  linear ops.hpp:46 (ops_gemm.cu:112-132: cublasSgemm, then the
+ * addBias kernel); the fp32 attention block's output projection + residual and the feed-forward block's second
+ * projection + bias + residual (ops_transformer.cu:121-130,207-214); the sum of the Q, K and V input gradients
+ * (autodiff.cu:693-699). */
+int bf_hip_gemm_f32_adds(int transA, int transB, const float* A, const float* B, const float* bias, const float* residual,
+                         float* C, size_t M, size_t N, size_t K, bf_stream_t stream);
 /* floatToBf16 (round to nearest even): ops_tensorcore.cu:21-26,80-87.  `out` holds n bf16 values. */
 int bf_hip_cvt_f32_bf16(const float* x, uint16_t* out, size_t n, bf_stream_t stream);
 /* Same rounding, writing out[c,r] = bf16(x[r,c]) for x:[rows,cols]. */

@@ -35,9 +35,18 @@ inline void requireMatmulBackward(const char* op, const DeviceTensor& a, const D
             std::string(op) + ": incompatible shapes on the device");
 }
 // Gradients of c = a(as [m,k]) * b[k,n] given g (as [m,n]); mode as in detail::projection.
+// `dAInto` (fp32 mode): the input gradient is ADDED to that tensor, which becomes dA (several projections of one input
+// sum their input gradients where the products are stored instead of in separate add kernels).
 inline MatmulGrad projectionBackward(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& g, int mode,
-                                     std::vector<std::size_t> dAShape, const GradientTargets* into = nullptr, int slot = 0) {
+                                     std::vector<std::size_t> dAShape, const GradientTargets* into = nullptr, int slot = 0,
+                                     DeviceTensor* dAInto = nullptr) {
     std::size_t m = rowsOf(a), k = lastDim(a), n = b.dim(1);
+    if (mode == 0 && dAInto != nullptr && n != 0) {
+        MatmulGrad r{std::move(*dAInto), gradientTensor(into, slot, {k, n})};
+        check(bf_hip_gemm_f32_adds(0, 1, g.data(), b.data(), nullptr, r.dA.data(), r.dA.data(), m, k, n, nullptr));   // dA += g b^T
+        check(bf_hip_gemm_f32(1, 0, a.data(), g.data(), r.dB.data(), k, n, m, nullptr));                              // dB = a^T g
+        return r;
+    }
     MatmulGrad r{DeviceTensor(std::move(dAShape)), gradientTensor(into, slot, {k, n})};
     if (mode == 0) {
         check(bf_hip_gemm_f32(0, 1, g.data(), b.data(), r.dA.data(), m, k, n, nullptr));   // dA = g b^T
@@ -304,9 +313,10 @@ inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& inpu
         return SelfAttentionGrad{std::move(dInput), std::move(dWq), std::move(dWk), std::move(dWv), std::move(outGrad.dB)};
     }
     MatmulGrad gq = projectionBackward(cache.normedFlat, wq, attn.dQ, mode, {batch * seq, dim}, into, 0);
-    MatmulGrad gk = projectionBackward(cache.normedFlat, wk, attn.dK, mode, {batch * seq, dim}, into, 1);
-    MatmulGrad gv = projectionBackward(cache.normedFlat, wv, attn.dV, mode, {batch * seq, dim}, into, 2);
-    DeviceTensor dNormed = add(add(gq.dA, gk.dA), gv.dA).reshaped({batch, seq, dim});
+    // (dQ Wq^T + dK Wk^T) + dV Wv^T, each product added to the running sum where it is stored
+    MatmulGrad gk = projectionBackward(cache.normedFlat, wk, attn.dK, mode, {batch * seq, dim}, into, 1, &gq.dA);
+    MatmulGrad gv = projectionBackward(cache.normedFlat, wv, attn.dV, mode, {batch * seq, dim}, into, 2, &gk.dA);
+    DeviceTensor dNormed = std::move(gv.dA).reshaped({batch, seq, dim});
     DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput);
     return SelfAttentionGrad{std::move(dInput), std::move(gq.dB), std::move(gk.dB), std::move(gv.dB), std::move(outGrad.dB)};
 }

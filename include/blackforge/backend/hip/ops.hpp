@@ -38,12 +38,25 @@ inline DeviceTensor projection(const DeviceTensor& a, const DeviceTensor& b, int
     else check(bf_hip_matmul_bf16(a.data(), b.data(), c.data(), m, k, n, bf16 == 2, nullptr));
     return c;
 }
-// bf16 projection with the adds that follow it folded into the GEMM's store: a*b (+ bias) (+ residual).
-// bf16: 1 = fresh weight image, 2 = cached weight image.
+// A projection with the adds that follow it folded into the GEMM's store: a*b (+ bias) (+ residual).
+// bf16: 0 = fp32 product, 1 = fresh weight image, 2 = cached weight image.
 inline DeviceTensor projectionFused(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor* bias, const DeviceTensor* residual,
                                     int bf16, std::vector<std::size_t> outShape) {
     DeviceTensor c(std::move(outShape));
     const std::size_t k = b.dim(0), n = b.dim(1), m = n ? c.elementCount() / n : 0;
+    if (bf16 == 0) {
+        if (k == 0 && m != 0 && n != 0) {   // an empty contraction: the product is zero, the adds remain
+            DeviceTensor zero = DeviceTensor::zeros(c.shape());
+            if (bias && residual) check(bf_hip_add_bias_residual(zero.data(), bias->data(), residual->data(), c.data(), m, n, nullptr));
+            else if (bias) check(bf_hip_add_bias(zero.data(), bias->data(), c.data(), m, n, nullptr));
+            else if (residual) return residual->clone();
+            else return zero;
+            return c;
+        }
+        check(bf_hip_gemm_f32_adds(0, 0, a.data(), b.data(), bias ? bias->data() : nullptr, residual ? residual->data() : nullptr, c.data(),
+                                   m, n, k, nullptr));
+        return c;
+    }
     check(bf_hip_linear_bf16(a.data(), b.data(), bias ? bias->data() : nullptr, residual ? residual->data() : nullptr, c.data(), m, k,
                              n, bf16 == 2, nullptr));
     return c;
@@ -181,11 +194,7 @@ inline DeviceTensor linearImpl(const char* op, const DeviceTensor& input, const 
     require(input.rank() >= 2, std::string(op) + ": needs a tensor of rank >= 2");
     require(weight.rank() == 2 && lastDim(input) == weight.dim(0), std::string(op) + ": incompatible shapes on the device");
     require(bias.rank() == 1 && bias.dim(0) == weight.dim(1), std::string(op) + ": bias does not match the weight");
-    if (bf16 != 0) return projectionFused(input, weight, &bias, nullptr, bf16, withLastDim(input, weight.dim(1)));
-    DeviceTensor product = projection(input, weight, bf16, withLastDim(input, weight.dim(1)));
-    DeviceTensor out(product.shape());
-    check(bf_hip_add_bias(product.data(), bias.data(), out.data(), rowsOf(product), bias.dim(0), nullptr));
-    return out;
+    return projectionFused(input, weight, &bias, nullptr, bf16, withLastDim(input, weight.dim(1)));
 }
 }  // namespace detail
 
@@ -245,13 +254,9 @@ inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const De
     }
     cache.gemm1 = detail::projection(cache.normed, w1, mode, detail::withLastDim(input, w1.dim(1)));
     cache.hidden = addBiasActivation(cache.gemm1, b1, act);
-    if (mode != 0) {
-        require(b2.rank() == 1 && b2.dim(0) == w2.dim(1), "addBiasResidual: expected input [..., features] and bias [features]");
-        require(w2.dim(1) == detail::lastDim(input), "addBiasResidual: residual shape differs from the product");
-        return detail::projectionFused(cache.hidden, w2, &b2, &input, mode, input.shape());
-    }
-    DeviceTensor gemm2 = detail::projection(cache.hidden, w2, mode, detail::withLastDim(input, w2.dim(1)));
-    return addBiasResidual(gemm2, b2, input);
+    require(b2.rank() == 1 && b2.dim(0) == w2.dim(1), "addBiasResidual: expected input [..., features] and bias [features]");
+    require(w2.dim(1) == detail::lastDim(input), "addBiasResidual: residual shape differs from the product");
+    return detail::projectionFused(cache.hidden, w2, &b2, &input, mode, input.shape());
 }
 
 namespace detail {
@@ -348,9 +353,7 @@ inline DeviceTensor selfAttentionForwardImpl(const char* op, const DeviceTensor&
     cache.attnOutput = std::move(attn.output);
     cache.attnM = std::move(attn.m);
     cache.attnL = std::move(attn.l);
-    if (mode != 0) return projectionFused(cache.attnOutput, wout, nullptr, &input, mode, {batch, seq, dim});
-    DeviceTensor projected = projection(cache.attnOutput, wout, mode, {batch, seq, dim});
-    return add(input, projected);
+    return projectionFused(cache.attnOutput, wout, nullptr, &input, mode, {batch, seq, dim});
 }
 }  // namespace detail
 

@@ -360,3 +360,29 @@ def test_feed_forward_fused_rejects_widths_that_are_not_multiples_of_eight(hip):
     D, ops = hip.DeviceTensor, hip.ops
     with pytest.raises(ValueError):
         ops.feedForwardBf16Fused(D.zeros((4, 12)), D.zeros((12, 16)), D.zeros((16,)), D.zeros((16, 12)), D.zeros((12,)))
+
+
+@pytest.mark.parametrize("m,k,n", [(512, 128, 256), (70, 300, 33), (257, 4100, 129), (2048, 300, 4224), (64, 64, 64)])
+def test_fp32_gemm_with_adds_in_the_store(hip, rng, m, k, n):
+    """bf_hip_gemm_f32_adds: the product with bias and residual added where it is stored is bit-identical to the product
+    followed by the separate add kernels, in every tile form (32 x 32, 64 x 64, 128 x 128, K slices), and the residual
+    may be the output itself (accumulation in place)."""
+    D, ops, call = hip.DeviceTensor, hip.ops, hip.capi.call
+    a, b, bias, res = r(rng, m, k), r(rng, k, n), r(rng, n), r(rng, m, n)
+    da, db, dbias, dres = map(D.fromHost, (a, b, bias, res))
+    product = ops.matmul(da, db)
+    out = D((m, n))
+    call("bf_hip_gemm_f32_adds", 0, 0, da.ptr, db.ptr, dbias.ptr, dres.ptr, out.ptr, m, n, k, None)
+    assert_bits_equal(out.toHost(), ops.addBiasResidual(product, dbias, dres).toHost(), "product + bias + residual")
+    call("bf_hip_gemm_f32_adds", 0, 0, da.ptr, db.ptr, dbias.ptr, None, out.ptr, m, n, k, None)
+    assert_bits_equal(out.toHost(), ops.addBias(product, dbias).toHost(), "product + bias")
+    acc = D.fromHost(res)
+    call("bf_hip_gemm_f32_adds", 0, 0, da.ptr, db.ptr, None, acc.ptr, acc.ptr, m, n, k, None)
+    assert_bits_equal(acc.toHost(), ops.add(product, dres).toHost(), "residual += product")
+    # transposed operands take the same store: dA += g b^T
+    g = r(rng, m, n)
+    dg = D.fromHost(g)
+    dA, _ = ops.matmulBackward(da, db, dg)
+    acc = D.fromHost(a)
+    call("bf_hip_gemm_f32_adds", 0, 1, dg.ptr, db.ptr, None, acc.ptr, acc.ptr, m, k, n, None)
+    assert_bits_equal(acc.toHost(), ops.add(dA, da).toHost(), "a += g b^T")
