@@ -33,6 +33,12 @@ class PoolStats(ctypes.Structure):
                 ("acquires", c_size)]
 
 
+class GemmF32Problem(ctypes.Structure):
+    """bf_gemm_f32_problem: one member of a bf_hip_gemm_f32_group call."""
+    _fields_ = [("A", c_ptr), ("B", c_ptr), ("C", c_ptr), ("bias", c_ptr), ("residual", c_ptr),
+                ("M", c_size), ("N", c_size), ("K", c_size), ("transA", ctypes.c_int), ("transB", ctypes.c_int)]
+
+
 P = c_ptr  # device pointer
 S = c_ptr  # stream
 
@@ -91,6 +97,7 @@ SIGNATURES = {
     "bf_hip_argmax_last_position": [P, c_size, c_size, ctypes.POINTER(c_ll), S],
     "bf_hip_gemm_f32": [c_int, c_int, P, P, P, c_size, c_size, c_size, S],
     "bf_hip_gemm_f32_adds": [c_int, c_int, P, P, P, P, P, c_size, c_size, c_size, S],
+    "bf_hip_gemm_f32_group": [ctypes.POINTER(GemmF32Problem), c_size, S],
     "bf_hip_cvt_f32_bf16": [P, P, c_size, S],
     "bf_hip_cvt_f32_bf16_transpose": [P, P, c_size, c_size, S],
     "bf_hip_gemm_bf16_nt": [P, P, P, c_size, c_size, c_size, S],

@@ -271,6 +271,92 @@ int launchSmallGemm(int transA, int transB, const float* A, const float* B, floa
     return launchSmallGemmAs<1, 1>(transA, transB, A, B, C, M, N, K, slices, kPerSlice, sliceStride, bias, residual, s);
 }
 
+// Several independent small products in ONE launch (blockIdx.z selects the product): the two gradient products of a
+// projection, or the Q, K and V projections of one input.  A small model's step is a chain of launches of a few
+// microseconds each, most of that the launch and one round trip to memory; products that do not depend on each other
+// share both.  The orientation of the operands is a run-time property of each product here.
+constexpr int kMaxGroup = 8;
+struct GroupProblem {
+    const float* A;
+    const float* B;
+    float* C;
+    const float* bias;
+    const float* residual;
+    unsigned M, N, K;
+    int transA, transB;
+};
+struct GroupArgs {
+    GroupProblem p[kMaxGroup];
+};
+
+template <int VEC>
+struct SmallOperandRt {
+    float v[SBK * SBT / 256];
+    __device__ __forceinline__ void fetch(bool kContig, const float* __restrict__ X, size_t ld, size_t tExtent, size_t kEnd, size_t t0, size_t k0,
+                                          int tid) {
+        if (kContig) reinterpret_cast<SmallOperand<true, VEC>*>(this)->fetch(X, ld, tExtent, kEnd, t0, k0, tid);
+        else reinterpret_cast<SmallOperand<false, VEC>*>(this)->fetch(X, ld, tExtent, kEnd, t0, k0, tid);
+    }
+    __device__ __forceinline__ void commit(bool kContig, float* lds, int tid) const {
+        if (kContig) reinterpret_cast<const SmallOperand<true, VEC>*>(this)->commit(lds, tid);
+        else reinterpret_cast<const SmallOperand<false, VEC>*>(this)->commit(lds, tid);
+    }
+};
+
+template <int VEC, int DEPTH>
+__global__ void __launch_bounds__(256) gemmF32SmallGroupKernel(GroupArgs args) {
+    __shared__ __attribute__((aligned(16))) float as[SWORDS];
+    __shared__ __attribute__((aligned(16))) float bs[SWORDS];
+    const GroupProblem& g = args.p[blockIdx.z];
+    const size_t M = g.M, N = g.N, kEnd = g.K;
+    const size_t m0 = size_t(blockIdx.y) * SBT, n0 = size_t(blockIdx.x) * SBT;
+    if (m0 >= M || n0 >= N) return;   // the grid covers the largest product of the group
+    const bool aContig = !g.transA, bContig = g.transB != 0;
+    const float* A = g.A;
+    const float* B = g.B;
+    const size_t lda = g.transA ? M : kEnd, ldb = g.transB ? kEnd : N;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave >> 1) * 16, wn0 = (wave & 1) * 16;
+    const int li = lane & 15, lk = lane >> 4;
+    // where a lane finds element (t, k) of either tile: base + k * stride
+    const int aBase = aContig ? (wm0 + li) * SROW_K : wm0 + li, aStep = aContig ? 1 : SROW_T;
+    const int bBase = bContig ? (wn0 + li) * SROW_K : wn0 + li, bStep = bContig ? 1 : SROW_T;
+    float4v acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+    SmallOperandRt<VEC> aStage[DEPTH], bStage[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (size_t(d) * SBK < kEnd) {
+            aStage[d].fetch(aContig, A, lda, M, kEnd, m0, size_t(d) * SBK, tid);
+            bStage[d].fetch(bContig, B, ldb, N, kEnd, n0, size_t(d) * SBK, tid);
+        }
+    for (size_t base = 0; base < kEnd; base += size_t(DEPTH) * SBK) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const size_t k0 = base + size_t(d) * SBK;
+            if (k0 >= kEnd) break;
+            aStage[d].commit(aContig, as, tid);
+            bStage[d].commit(bContig, bs, tid);
+            __syncthreads();
+            if (k0 + size_t(DEPTH) * SBK < kEnd) {
+                aStage[d].fetch(aContig, A, lda, M, kEnd, m0, k0 + size_t(DEPTH) * SBK, tid);
+                bStage[d].fetch(bContig, B, ldb, N, kEnd, n0, k0 + size_t(DEPTH) * SBK, tid);
+            }
+#pragma unroll
+            for (int kk = 0; kk < SBK; kk += 8) {
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(as[aBase + (kk + lk) * aStep], bs[bBase + (kk + lk) * bStep], acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(as[aBase + (kk + 4 + lk) * aStep], bs[bBase + (kk + 4 + lk) * bStep], acc1, 0, 0, 0);
+            }
+            __syncthreads();
+        }
+    }
+    const size_t col = n0 + wn0 + li;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const size_t row = m0 + wm0 + 4 * lk + r;
+        if (row < M && col < N) g.C[row * N + col] = withAdds(acc0[r] + acc1[r], g.bias, g.residual, row * N + col, col);
+    }
+}
+
 // C[i] = sum over slices of partial[s*stride + i], slices added in index order (deterministic).
 __global__ void __launch_bounds__(kBlock) sliceSumKernel(const float* __restrict__ partial, float* C, size_t count,
                                                          size_t stride, int slices, size_t N, const float* __restrict__ bias,
@@ -371,4 +457,43 @@ extern "C" int bf_hip_gemm_f32(int transA, int transB, const float* A, const flo
 extern "C" int bf_hip_gemm_f32_adds(int transA, int transB, const float* A, const float* B, const float* bias, const float* residual,
                                     float* C, size_t M, size_t N, size_t K, bf_stream_t stream) {
     return gemmF32(transA, transB, A, B, C, M, N, K, bias, residual, stream);
+}
+
+extern "C" int bf_hip_gemm_f32_group(const bf_gemm_f32_problem* problems, size_t count, bf_stream_t stream) {
+    if (count == 0) return BF_OK;
+    BF_REQUIRE(problems != nullptr, "NULL problem list");
+    // one launch when every product is small enough for the 32 x 32 form without K slices (the form bf_hip_gemm_f32 itself
+    // would pick); otherwise, or beyond eight products, the products are launched one after the other
+    const size_t cus = size_t(computeUnits());
+    auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    bool together = count <= size_t(kMaxGroup) && count > 1, vec = true;
+    size_t tilesM = 0, tilesN = 0;
+    for (size_t i = 0; i < count && together; ++i) {
+        const bf_gemm_f32_problem& p = problems[i];
+        if (p.M == 0 || p.N == 0) continue;
+        BF_REQUIRE(p.C != nullptr, "NULL output");
+        const size_t tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
+        together = p.K > 0 && p.K < size_t(16) * SBK && tiles * 2 <= cus && p.M < (size_t(1) << 31) && p.N < (size_t(1) << 31) && p.A && p.B;
+        vec = vec && aligned16(p.A) && aligned16(p.B) && (p.transA ? p.M : p.K) % 4 == 0 && (p.transB ? p.K : p.N) % 4 == 0;
+        tilesM = std::max(tilesM, (p.M + SBT - 1) / SBT);
+        tilesN = std::max(tilesN, (p.N + SBT - 1) / SBT);
+    }
+    if (!together || tilesM == 0 || tilesM > 65535) {
+        for (size_t i = 0; i < count; ++i) {
+            const bf_gemm_f32_problem& p = problems[i];
+            int st = gemmF32(p.transA, p.transB, p.A, p.B, p.C, p.M, p.N, p.K, p.bias, p.residual, stream);
+            if (st != BF_OK) return st;
+        }
+        return BF_OK;
+    }
+    GroupArgs args = {};
+    for (size_t i = 0; i < count; ++i) {
+        const bf_gemm_f32_problem& p = problems[i];
+        args.p[i] = GroupProblem{p.A, p.B, p.C, p.bias, p.residual, unsigned(p.M), unsigned(p.N), unsigned(p.K), p.transA, p.transB};
+    }
+    const dim3 grid = dim3(static_cast<unsigned>(tilesN), static_cast<unsigned>(tilesM), static_cast<unsigned>(count));
+    if (vec) gemmF32SmallGroupKernel<4, 4><<<grid, 256, 0, asStream(stream)>>>(args);
+    else gemmF32SmallGroupKernel<1, 1><<<grid, 256, 0, asStream(stream)>>>(args);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
 }

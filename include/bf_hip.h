@@ -236,6 +236,21 @@ int bf_hip_gemm_f32(int transA, int transB, const float* A, const float* B, floa
  * (autodiff.cu:693-699). */
 int bf_hip_gemm_f32_adds(int transA, int transB, const float* A, const float* B, const float* bias, const float* residual,
                          float* C, size_t M, size_t N, size_t K, bf_stream_t stream);
+/* Several independent fp32 products at once (`problems` is a HOST array): each is what bf_hip_gemm_f32_adds computes,
+ * bit for bit.  Small products (the ones a model a few hundred wide consists of) share ONE launch; anything else is
+ * launched product by product.  The outputs must not overlap each other or another product's operands.  Serves the two
+ * gradient products of matmulBackward (autodiff.cu:294-322: two kernels, one after the other) and the three
+ * projections of one input in the attention block (ops_transformer.cu:107-111) and their gradients. */
+typedef struct {
+    const float* A;
+    const float* B;
+    float* C;
+    const float* bias;      /* [N] or NULL */
+    const float* residual;  /* [M,N] or NULL; may be C */
+    size_t M, N, K;
+    int transA, transB;
+} bf_gemm_f32_problem;
+int bf_hip_gemm_f32_group(const bf_gemm_f32_problem* problems, size_t count, bf_stream_t stream);
 /* floatToBf16 (round to nearest even): ops_tensorcore.cu:21-26,80-87.  `out` holds n bf16 values. */
 int bf_hip_cvt_f32_bf16(const float* x, uint16_t* out, size_t n, bf_stream_t stream);
 /* Same rounding, writing out[c,r] = bf16(x[r,c]) for x:[rows,cols]. */

@@ -35,22 +35,12 @@ inline void requireMatmulBackward(const char* op, const DeviceTensor& a, const D
             std::string(op) + ": incompatible shapes on the device");
 }
 // Gradients of c = a(as [m,k]) * b[k,n] given g (as [m,n]); mode as in detail::projection.
-// `dAInto` (fp32 mode): the input gradient is ADDED to that tensor, which becomes dA (several projections of one input
-// sum their input gradients where the products are stored instead of in separate add kernels).
 inline MatmulGrad projectionBackward(const DeviceTensor& a, const DeviceTensor& b, const DeviceTensor& g, int mode,
-                                     std::vector<std::size_t> dAShape, const GradientTargets* into = nullptr, int slot = 0,
-                                     DeviceTensor* dAInto = nullptr) {
+                                     std::vector<std::size_t> dAShape, const GradientTargets* into = nullptr, int slot = 0) {
     std::size_t m = rowsOf(a), k = lastDim(a), n = b.dim(1);
-    if (mode == 0 && dAInto != nullptr && n != 0) {
-        MatmulGrad r{std::move(*dAInto), gradientTensor(into, slot, {k, n})};
-        check(bf_hip_gemm_f32_adds(0, 1, g.data(), b.data(), nullptr, r.dA.data(), r.dA.data(), m, k, n, nullptr));   // dA += g b^T
-        check(bf_hip_gemm_f32(1, 0, a.data(), g.data(), r.dB.data(), k, n, m, nullptr));                              // dB = a^T g
-        return r;
-    }
     MatmulGrad r{DeviceTensor(std::move(dAShape)), gradientTensor(into, slot, {k, n})};
-    if (mode == 0) {
-        check(bf_hip_gemm_f32(0, 1, g.data(), b.data(), r.dA.data(), m, k, n, nullptr));   // dA = g b^T
-        check(bf_hip_gemm_f32(1, 0, a.data(), g.data(), r.dB.data(), k, n, m, nullptr));   // dB = a^T g
+    if (mode == 0) {   // dA = g b^T and dB = a^T g do not depend on each other: one call
+        productsF32({{0, 1, g.data(), b.data(), r.dA.data(), m, k, n}, {1, 0, a.data(), g.data(), r.dB.data(), k, n, m}});
     } else {   // a gradient that carries its bf16 image (made by the kernel that produced it) is not converted again
         check(bf_hip_matmul_bf16_backward_img(a.data(), a.image(), b.data(), g.data(), g.image(), r.dA.data(), r.dB.data(), m, k, n,
                                               mode == 2, nullptr));
@@ -84,8 +74,8 @@ inline MatmulTransposeBGrad matmulTransposeBBackward(const DeviceTensor& a, cons
             "matmulTransposeBBackward: incompatible shapes on the device");
     std::size_t m = a.dim(0), k = a.dim(1), n = b.dim(0);
     MatmulTransposeBGrad r{DeviceTensor({m, k}), DeviceTensor({n, k})};
-    check(bf_hip_gemm_f32(0, 0, gradOutput.data(), b.data(), r.dA.data(), m, k, n, nullptr));   // dA = g b
-    check(bf_hip_gemm_f32(1, 0, gradOutput.data(), a.data(), r.dB.data(), n, k, m, nullptr));   // dB = g^T a
+    // dA = g b and dB = g^T a
+    detail::productsF32({{0, 0, gradOutput.data(), b.data(), r.dA.data(), m, k, n}, {1, 0, gradOutput.data(), a.data(), r.dB.data(), n, k, m}});
     return r;
 }
 
@@ -312,13 +302,17 @@ inline SelfAttentionGrad selfAttentionBackwardFromCache(const DeviceTensor& inpu
         DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput, imageForConsumer);
         return SelfAttentionGrad{std::move(dInput), std::move(dWq), std::move(dWk), std::move(dWv), std::move(outGrad.dB)};
     }
-    MatmulGrad gq = projectionBackward(cache.normedFlat, wq, attn.dQ, mode, {batch * seq, dim}, into, 0);
-    // (dQ Wq^T + dK Wk^T) + dV Wv^T, each product added to the running sum where it is stored
-    MatmulGrad gk = projectionBackward(cache.normedFlat, wk, attn.dK, mode, {batch * seq, dim}, into, 1, &gq.dA);
-    MatmulGrad gv = projectionBackward(cache.normedFlat, wv, attn.dV, mode, {batch * seq, dim}, into, 2, &gk.dA);
-    DeviceTensor dNormed = std::move(gv.dA).reshaped({batch, seq, dim});
+    // the six gradient products of the three projections are independent of each other: one call, then
+    // (dQ Wq^T + dK Wk^T) + dV Wv^T
+    const std::size_t rows = batch * seq;
+    DeviceTensor dAq({rows, dim}), dAk({rows, dim}), dAv({rows, dim});
+    DeviceTensor dWq = gradientTensor(into, 0, wq.shape()), dWk = gradientTensor(into, 1, wk.shape()), dWv = gradientTensor(into, 2, wv.shape());
+    productsF32({{0, 1, attn.dQ.data(), wq.data(), dAq.data(), rows, dim, dim}, {1, 0, cache.normedFlat.data(), attn.dQ.data(), dWq.data(), dim, dim, rows},
+                 {0, 1, attn.dK.data(), wk.data(), dAk.data(), rows, dim, dim}, {1, 0, cache.normedFlat.data(), attn.dK.data(), dWk.data(), dim, dim, rows},
+                 {0, 1, attn.dV.data(), wv.data(), dAv.data(), rows, dim, dim}, {1, 0, cache.normedFlat.data(), attn.dV.data(), dWv.data(), dim, dim, rows}});
+    DeviceTensor dNormed = add(add(dAq, dAk), dAv).reshaped({batch, seq, dim});
     DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput);
-    return SelfAttentionGrad{std::move(dInput), std::move(gq.dB), std::move(gk.dB), std::move(gv.dB), std::move(outGrad.dB)};
+    return SelfAttentionGrad{std::move(dInput), std::move(dWq), std::move(dWk), std::move(dWv), std::move(outGrad.dB)};
 }
 }  // namespace detail
 

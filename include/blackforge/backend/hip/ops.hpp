@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstddef>
 #include <cstdint>
+#include <initializer_list>
 #include <string>
 #include <utility>
 #include <vector>
@@ -37,6 +38,20 @@ inline DeviceTensor projection(const DeviceTensor& a, const DeviceTensor& b, int
     if (bf16 == 0) check(bf_hip_gemm_f32(0, 0, a.data(), b.data(), c.data(), m, n, k, nullptr));
     else check(bf_hip_matmul_bf16(a.data(), b.data(), c.data(), m, k, n, bf16 == 2, nullptr));
     return c;
+}
+// Independent fp32 products in one call (one launch when they are small): {transA, transB, A, B, C, M, N, K}.
+struct F32Product {
+    int transA, transB;
+    const float* a;
+    const float* b;
+    float* c;
+    std::size_t m, n, k;
+};
+inline void productsF32(std::initializer_list<F32Product> products) {
+    bf_gemm_f32_problem list[8];
+    std::size_t count = 0;
+    for (const F32Product& p : products) list[count++] = bf_gemm_f32_problem{p.a, p.b, p.c, nullptr, nullptr, p.m, p.n, p.k, p.transA, p.transB};
+    check(bf_hip_gemm_f32_group(list, count, nullptr));
 }
 // A projection with the adds that follow it folded into the GEMM's store: a*b (+ bias) (+ residual).
 // bf16: 0 = fp32 product, 1 = fresh weight image, 2 = cached weight image.
@@ -344,9 +359,17 @@ inline DeviceTensor selfAttentionForwardImpl(const char* op, const DeviceTensor&
         float* outputs[3] = {cache.q.data(), cache.k.data(), cache.v.data()};
         check(bf_hip_matmul_bf16_shared_input(cache.normedFlat.data(), weights, outputs, 3, batch * seq, dim, dim, mode == 2, nullptr));
     } else {
-        cache.q = projection(cache.normedFlat, wq, mode, {batch, seq, dim});
-        cache.k = projection(cache.normedFlat, wk, mode, {batch, seq, dim});
-        cache.v = projection(cache.normedFlat, wv, mode, {batch, seq, dim});
+        // three products of one input, independent of each other: one call
+        require(wq.rank() == 2 && wk.rank() == 2 && wv.rank() == 2 && wq.dim(0) == dim && wk.dim(0) == dim && wv.dim(0) == dim &&
+                    wq.dim(1) == dim && wk.dim(1) == dim && wv.dim(1) == dim,
+                std::string(op) + ": projection weights must be [dim, dim]");
+        cache.q = DeviceTensor({batch, seq, dim});
+        cache.k = DeviceTensor({batch, seq, dim});
+        cache.v = DeviceTensor({batch, seq, dim});
+        const std::size_t rows = batch * seq;
+        productsF32({{0, 0, cache.normedFlat.data(), wq.data(), cache.q.data(), rows, dim, dim},
+                     {0, 0, cache.normedFlat.data(), wk.data(), cache.k.data(), rows, dim, dim},
+                     {0, 0, cache.normedFlat.data(), wv.data(), cache.v.data(), rows, dim, dim}});
     }
     // query i sees keys j <= oldLen + i: an offset of seq makes every key visible, which is the bidirectional form
     FusedAttentionForwardResult attn = fusedAttentionForward(cache.q, cache.k, cache.v, numHeads, scaleFactor, causal ? 0 : seq);

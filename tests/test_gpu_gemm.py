@@ -386,3 +386,36 @@ def test_fp32_gemm_with_adds_in_the_store(hip, rng, m, k, n):
     acc = D.fromHost(a)
     call("bf_hip_gemm_f32_adds", 0, 1, dg.ptr, db.ptr, None, acc.ptr, acc.ptr, m, k, n, None)
     assert_bits_equal(acc.toHost(), ops.add(dA, da).toHost(), "a += g b^T")
+
+
+def test_fp32_gemm_group_matches_single_products(hip, rng):
+    """bf_hip_gemm_f32_group: products of different shapes and orientations in one call (one launch when they are small)
+    give the bits of the same products launched one by one, adds included; a member too large for the shared launch
+    sends the whole group down the one-by-one road with the same results."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    Problem = hip.capi.GemmF32Problem
+
+    def run(specs):
+        # specs: (transA, transB, M, N, K, with_bias, accumulate)
+        problems, singles, tensors = [], [], []
+        for ta, tb, m, n, k, with_bias, accumulate in specs:
+            a = D.fromHost(r(rng, *((k, m) if ta else (m, k))))
+            b = D.fromHost(r(rng, *((n, k) if tb else (k, n))))
+            bias = D.fromHost(r(rng, n)) if with_bias else None
+            start = r(rng, m, n)
+            c_group, c_single = D.fromHost(start), D.fromHost(start)
+            tensors += [a, b, bias, c_group, c_single]
+            problems.append(Problem(a.ptr, b.ptr, c_group.ptr, bias.ptr if bias else None, c_group.ptr if accumulate else None, m, n, k, ta, tb))
+            call("bf_hip_gemm_f32_adds", ta, tb, a.ptr, b.ptr, bias.ptr if bias else None, c_single.ptr if accumulate else None, c_single.ptr,
+                 m, n, k, None)
+            singles.append((c_group, c_single))
+        array = (Problem * len(problems))(*problems)
+        call("bf_hip_gemm_f32_group", array, len(problems), None)
+        for i, (got, want) in enumerate(singles):
+            assert_bits_equal(got.toHost(), want.toHost(), f"member {i} of {specs}")
+
+    run([(0, 1, 512, 128, 256, False, False), (1, 0, 128, 256, 512, False, False)])                    # a projection's two gradients
+    run([(0, 0, 512, 128, 128, False, False)] * 3)                                                      # Q, K and V of one input
+    run([(0, 1, 70, 33, 45, True, False), (1, 1, 5, 7, 300, False, True), (1, 0, 130, 64, 513, True, True), (0, 0, 1, 1, 1, False, False)])
+    run([(0, 0, 64, 64, 64, False, False), (0, 0, 2048, 4224, 300, True, False)])                       # one member needs the large tiles
+    run([(0, 1, 96, 96, 4100, False, False), (1, 0, 96, 96, 96, False, False)])                         # one member needs K slices
