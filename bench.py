@@ -118,7 +118,16 @@ def bench_attention(bf, steps, warmup):
            (("forward", fwd), ("prepare", prep), ("dkv", dkv), ("dq", dqk), ("dkv_recompute", dkv_re),
             ("dq_recompute", dq_re))}
     fl = attention_flops(batch, heads, seq, hd)
+    # the same forward pass with its two products as six bf16 MFMAs each on operands split into three bf16 terms
+    # (bf_hip_attention_set_route; not the default route: `value` and `roofline` above are the fp32-MFMA kernels')
+    call("bf_hip_attention_set_route", 1)
+    try:
+        split_fwd = time_region(bf, stream, fwd, steps, 2)
+        split_step = time_region(bf, stream, step, steps, 1)
+    finally:
+        call("bf_hip_attention_set_route", 0)
     return {"ms_per_step": ms_step, "wall_ms_per_step": wall_ms, "kernel_ms": per, "flops": fl,
+            "split_bf16_forward": {"forward_ms": split_fwd, "step_ms": split_step},
             "shape": {"batch": batch, "heads": heads, "seq": seq, "head_dim": hd}}
 
 
@@ -578,6 +587,13 @@ def main():
                           "dkv_recompute": round(fl["dkv"] / res["kernel_ms"]["dkv_recompute"] / 1e9, 2),
                           "dq_recompute": round(fl["dq_recompute"] / res["kernel_ms"]["dq_recompute"] / 1e9, 2)},
         "wall_ms_per_step": round(res["wall_ms_per_step"], 4),
+        # an opt-in route (bf_hip_attention_set_route), NOT what `value` measures: the forward kernel with each fp32 product
+        # as six bf16 MFMAs on operands split into three bf16 terms (24 mantissa bits, fp32 accumulation)
+        "split_bf16_forward_route": {
+            "forward_ms": round(res["split_bf16_forward"]["forward_ms"], 4),
+            "forward_tflops_fp32_equivalent": round(fl["fwd"] / res["split_bf16_forward"]["forward_ms"] / 1e9, 2),
+            "step_ms": round(res["split_bf16_forward"]["step_ms"], 4),
+            "step_tflops_fp32_equivalent": round(total_flops / res["split_bf16_forward"]["step_ms"] / 1e9, 2)},
         "device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units},
     }
     if args.train != "none":

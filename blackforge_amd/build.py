@@ -43,7 +43,8 @@ def _compile(src: str, force: bool) -> str:
     deps = [src] + glob.glob(os.path.join(CSRC, "*.hpp")) + glob.glob(os.path.join(ROOT, "include", "*.h"))
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) >= os.path.getmtime(d) for d in deps):
         return obj
-    cmd = [hipcc()] + HIPCC_FLAGS + ["-c", src, "-o", obj]
+    # BF_HIPCC_EXTRA: extra compiler flags for experiments (e.g. "-DSOME_SWITCH"); empty in normal builds
+    cmd = [hipcc()] + HIPCC_FLAGS + os.environ.get("BF_HIPCC_EXTRA", "").split() + ["-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass warns that it does not know the packed-fp32 feature: harmless, filtered out
     err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)

@@ -130,6 +130,7 @@ SIGNATURES = {
     "bf_hip_attention_backward_dq": [P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_attention_ds_bytes": [c_size, c_size, c_size, c_size, ctypes.POINTER(c_size)],
     "bf_hip_attention_set_workspace_limit": [c_size],
+    "bf_hip_attention_set_route": [c_int],
     "bf_hip_attention_backward_dkv_ds": [P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_attention_backward_dq_from_ds": [P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_mse": [P, P, P, P, c_size, c_int, S],

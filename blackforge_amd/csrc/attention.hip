@@ -401,6 +401,266 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnForwardKernel(Att
 }
 
 // ---------------------------------------------------------------------------------------------
+// forward on the bf16 matrix pipe at fp32 accuracy
+// ---------------------------------------------------------------------------------------------
+// An fp32 value is the exact sum of three bf16 values, x = h + m + l (h = bf16(x), m = bf16(x - h), l = bf16(x - h - m);
+// the remainders are exact in fp32), so a product of two fp32 operands is the sum of nine bf16 products, of which the six
+// largest (h h', h m', m h', h l', l h', m m') carry everything above 2^-24 of the product: as accurate as the fp32 MFMA
+// (closer to float64 in measurement), accumulated in fp32 by the same matrix unit.  v_mfma_f32_32x32x16_bf16 contracts
+// sixteen elements in 32 clocks where v_mfma_f32_32x32x2_f32 contracts two in 64, so the six products cost 6/16 of the
+// matrix time.  What it takes: operands as bf16 triples in the layout of that instruction (eight consecutive
+// contraction elements per lane).
+//   * K and V tiles are split when they are written to LDS (three bf16 images each, row-major).  S^T = K Q^T contracts
+//     over the head dimension: a K fragment is 16 bytes of a row, Q fragments live in registers for the whole kernel.
+//   * O^T += V^T P^T contracts over keys.  The score tile leaves the MFMA with lane (query, half) holding keys
+//     8g + 4 half + 0..3; the contraction index may be permuted freely as long as both operands agree, so contraction
+//     slot e of step s of a lane in `half` is DEFINED as key 16 s + 8 (e / 4) + 4 half + e % 4: the P operand is then
+//     eight consecutive accumulator registers, split in place, and the V fragment is gathered for the same keys by the
+//     transposing LDS read (two reads of four rows, eight rows apart).
+// Everything else (online softmax, lazy rescaling, masks, statistics, stores) is the fp32 kernel's.
+typedef __bf16 bf16x8a __attribute__((ext_vector_type(8)));
+typedef short short4a __attribute__((ext_vector_type(4)));
+typedef short short8a __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ void split3(float x, __bf16& h, __bf16& m, __bf16& l) {
+    h = static_cast<__bf16>(x);
+    const float r1 = x - static_cast<float>(h);
+    m = static_cast<__bf16>(r1);
+    l = static_cast<__bf16>(r1 - static_cast<float>(m));
+}
+
+// rows p, p + pitch, p + 2 pitch, p + 3 pitch (as addressed by the lanes) and the same eight rows further down
+__device__ __forceinline__ bf16x8a readTransposedApart(const unsigned short* p, int rowPitch) {
+    typedef __attribute__((address_space(3))) short4a* LdsPtr;
+    const short4a lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(p));
+    const short4a hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(p + 8 * rowPitch));
+    const short8a both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8a, both);
+}
+
+constexpr int splitKeyPitch(int hdp) { return hdp + 8; }                       // plain 16-byte fragment reads
+constexpr int splitValuePitch(int hdp) { return hdp + 32 < 96 ? 96 : hdp + 32; }   // transposing reads: an odd multiple of 64 bytes
+
+// One tile of ROWS rows from registers to three bf16 images [3][ROWS][PITCH].
+template <int HDP, int ROWS, int PITCH>
+__device__ __forceinline__ void commitSplitTile(unsigned short* __restrict__ img, const TileRegs<HDP, ROWS>& regs, int tid) {
+    constexpr int V4 = HDP / 4, SLOTS = ROWS * V4, IMG = ROWS * PITCH;
+#pragma unroll
+    for (int i = 0; i < TileRegs<HDP, ROWS>::kSlots; ++i) {
+        const int s = tid + i * 256;
+        if (s < SLOTS) {
+            __bf16 h[4], m[4], l[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) split3(regs.v[i][j], h[j], m[j], l[j]);
+            auto pack = [](const __bf16 (&v)[4]) {
+                return uint2v{unsigned(__builtin_bit_cast(unsigned short, v[0])) | unsigned(__builtin_bit_cast(unsigned short, v[1])) << 16,
+                              unsigned(__builtin_bit_cast(unsigned short, v[2])) | unsigned(__builtin_bit_cast(unsigned short, v[3])) << 16};
+            };
+            unsigned short* dst = img + (s / V4) * PITCH + (s % V4) * 4;
+            *reinterpret_cast<uint2v*>(dst) = pack(h);
+            *reinterpret_cast<uint2v*>(dst + IMG) = pack(m);
+            *reinterpret_cast<uint2v*>(dst + 2 * IMG) = pack(l);
+        }
+    }
+}
+
+template <int HDP, bool MASKED>
+__device__ __forceinline__ void forwardSplitTile(const unsigned short* __restrict__ kimg, const unsigned short* __restrict__ vimg,
+                                                 const bf16x8a (&qf)[HDP / 16][3], float16v (&acc)[HDP / 32], float& mrow, float& mref,
+                                                 float& lrow, int kt0, int myLimit, int totalLen, int lane) {
+    constexpr int KP = splitKeyPitch(HDP), VP = splitValuePitch(HDP), KIMG = 32 * KP, VIMG = 32 * VP, DT = HDP / 32, KS = HDP / 16;
+    const int half = lane >> 5, li = lane & 31;
+    // S^T = K Q^T in two accumulator chains (the MFMAs of one chain depend on each other)
+    float16v s0, s1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const unsigned short* krow = kimg + li * KP + ks * 16 + half * 8;
+        bf16x8a a[3];
+#pragma unroll
+        for (int im = 0; im < 3; ++im) a[im] = *reinterpret_cast<const bf16x8a*>(krow + im * KIMG);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][1], s1, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][0], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], qf[ks][0], s1, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][1], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][2], s1, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][0], s0, 0, 0, 0);
+    }
+    float16v sc;   // sc[r] = log2-scaled score of (key = kt0 + dRow(r), this lane's query)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = s0[r] + s1[r];
+    if constexpr (MASKED) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = kt0 + dRow(r, half);
+            sc[r] = (key > myLimit || key >= totalLen) ? -INFINITY : sc[r];
+        }
+    }
+    float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+#pragma unroll
+    for (int r = 4; r < 16; r += 4) mx = fmaxf(mx, fmaxf(fmaxf(sc[r], sc[r + 1]), fmaxf(sc[r + 2], sc[r + 3])));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mrow = fmaxf(mrow, mx);
+    const bool moveRef = mrow > mref + kRescaleThreshold;   // also true on the first visible key (mref = -inf)
+    if (__builtin_amdgcn_ballot_w64(moveRef) != 0) {
+        const float corr = moveRef ? fastExp2(mref - mrow) : 1.0f;   // 0 when the reference was still -inf
+        mref = moveRef ? mrow : mref;
+        lrow *= corr;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+    }
+    float psum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { sc[r] = fastExp2(sc[r] - mref); psum += sc[r]; }
+    lrow += psum;
+    // O^T += V^T P^T: step s contracts over keys 16 s + 8 (e / 4) + 4 half + e % 4, i.e. registers 8 s .. 8 s + 7 of sc
+    const int fragRow = 4 * (lane >> 5) + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+        bf16x8a pf[3];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            __bf16 h, m, l;
+            split3(sc[8 * st + e], h, m, l);
+            pf[0][e] = h; pf[1][e] = m; pf[2][e] = l;
+        }
+        bf16x8a vf[DT][3];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int im = 0; im < 3; ++im) vf[dt][im] = readTransposedApart(vimg + im * VIMG + (16 * st + fragRow) * VP + dt * 32 + fragCol, VP);
+        // the six products of each head-dim block, the blocks taking turns: consecutive MFMAs do not depend on each other
+        constexpr int order[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};   // (V term, P term), small products first
+#pragma unroll
+        for (int pr = 0; pr < 6; ++pr)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][order[pr][0]], pf[order[pr][1]], acc[dt], 0, 0, 0);
+    }
+}
+
+template <int HDP, bool VEC4>
+__global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnForwardSplitKernel(AttnParams p) {
+    constexpr int BC = 32, KP = splitKeyPitch(HDP), VP = splitValuePitch(HDP), KTILE = 3 * BC * KP, VTILE = 3 * BC * VP, DT = HDP / 32, KS = HDP / 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned short smemSplit[];
+    unsigned short* ks = smemSplit;               // [2][3][BC][KP]
+    unsigned short* vs = smemSplit + 2 * KTILE;   // [2][3][BC][VP]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, qt;
+    decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const float* qb = p.q + size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const float* vb = p.v + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+
+    const int waveQ0 = qt * 128 + wave * 32;
+    const int i = waveQ0 + li;                    // this lane's query row
+    const bool rowValid = i < p.newLen;
+    // Q fragments: step ks of a lane in `half` holds head-dim elements 16 ks + 8 half + 0..7 of its query, scaled
+    bf16x8a qf[KS][3];
+    {
+        const float* row = qb + size_t(i) * dim;
+        const float mul = p.scale * kLog2e;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            float x[8];
+#pragma unroll
+            for (int c = 0; c < 8; c += 4) {
+                const int d = 16 * s + 8 * half + c;
+                float4v val = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (rowValid && d < hd) {
+                    if constexpr (VEC4) {
+                        val = loadf4(row + d);
+                    } else {
+                        val.x = row[d];
+                        if (d + 1 < hd) val.y = row[d + 1];
+                        if (d + 2 < hd) val.z = row[d + 2];
+                        if (d + 3 < hd) val.w = row[d + 3];
+                    }
+                }
+                x[c] = val.x * mul; x[c + 1] = val.y * mul; x[c + 2] = val.z * mul; x[c + 3] = val.w * mul;
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                __bf16 hh, mm, ll;
+                split3(x[e], hh, mm, ll);
+                qf[s][0][e] = hh; qf[s][1][e] = mm; qf[s][2][e] = ll;
+            }
+        }
+    }
+
+    float16v acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
+    float mrow = -INFINITY, mref = -INFINITY, lrow = 0.0f;
+
+    const int lastQuery = min(p.newLen, qt * 128 + 128) - 1;
+    const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);   // keys >= this are invisible to the tile
+    const int waveKeyEnd = p.oldLen + waveQ0 + 32;                       // keys >= this are invisible to the wave
+    const int myLimit = p.oldLen + i;                                    // last visible key of this lane's row
+    const int numKeyTiles = (blockKeyEnd + BC - 1) / BC;
+
+    // Tiles are short (32 keys), so the loads of a tile are issued TWO tiles before it is written to LDS: tile t + 1 waits
+    // in register set (t + 1) & 1 while tile t is multiplied, and that set is refilled with tile t + 3 once it is written.
+    TileRegs<HDP, BC> kStage[2], vStage[2];
+    fetchHeadTile<HDP, BC, VEC4>(kStage[0], kb, dim, 0, p.totalLen, hd, tid);
+    fetchHeadTile<HDP, BC, VEC4>(vStage[0], vb, dim, 0, p.totalLen, hd, tid);
+    if (numKeyTiles > 1) {
+        fetchHeadTile<HDP, BC, VEC4>(kStage[1], kb, dim, BC, p.totalLen, hd, tid);
+        fetchHeadTile<HDP, BC, VEC4>(vStage[1], vb, dim, BC, p.totalLen, hd, tid);
+    }
+    commitSplitTile<HDP, BC, KP>(ks, kStage[0], tid);
+    commitSplitTile<HDP, BC, VP>(vs, vStage[0], tid);
+    if (numKeyTiles > 2) {
+        fetchHeadTile<HDP, BC, VEC4>(kStage[0], kb, dim, 2 * BC, p.totalLen, hd, tid);
+        fetchHeadTile<HDP, BC, VEC4>(vStage[0], vb, dim, 2 * BC, p.totalLen, hd, tid);
+    }
+    __syncthreads();
+    for (int t0 = 0; t0 < numKeyTiles; t0 += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int t = t0 + u;
+            if (t >= numKeyTiles) break;
+            const int kt0 = t * BC;
+            const unsigned short* kcur = ks + u * KTILE;
+            const unsigned short* vcur = vs + u * VTILE;
+            if (kt0 < waveKeyEnd) {   // wave-uniform: the tile holds keys some row of this wave can see
+                const bool masked = (kt0 + BC - 1 > p.oldLen + waveQ0) || (kt0 + BC > p.totalLen);
+                if (masked) forwardSplitTile<HDP, true>(kcur, vcur, qf, acc, mrow, mref, lrow, kt0, myLimit, p.totalLen, lane);
+                else forwardSplitTile<HDP, false>(kcur, vcur, qf, acc, mrow, mref, lrow, kt0, myLimit, p.totalLen, lane);
+            }
+            if (t + 1 < numKeyTiles) {
+                commitSplitTile<HDP, BC, KP>(ks + (u ^ 1) * KTILE, kStage[u ^ 1], tid);
+                commitSplitTile<HDP, BC, VP>(vs + (u ^ 1) * VTILE, vStage[u ^ 1], tid);
+                if (t + 3 < numKeyTiles) {
+                    fetchHeadTile<HDP, BC, VEC4>(kStage[u ^ 1], kb, dim, kt0 + 3 * BC, p.totalLen, hd, tid);
+                    fetchHeadTile<HDP, BC, VEC4>(vStage[u ^ 1], vb, dim, kt0 + 3 * BC, p.totalLen, hd, tid);
+                }
+            }
+            __syncthreads();
+        }
+    }
+
+    lrow += __shfl_xor(lrow, 32, 64);
+    if (rowValid) {
+        if (p.out) storeTransposed<HDP, VEC4>(p.out + (size_t(b) * p.newLen + i) * dim + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
+        if (p.outImg) storeTransposedBf16<HDP, VEC4>(p.outImg + (size_t(b) * p.newLen + i) * p.imgLd + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
+        if (half == 0) {
+            size_t idx = (size_t(b) * p.heads + h) * p.newLen + i;
+            p.m[idx] = mrow * kLn2;
+            p.l[idx] = lrow * fastExp2(mref - mrow);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // backward, part 0: D = dot(O, dO) per (batch, head, row), and optionally the log2-domain
 // log-sum-exp lse2 = m*log2(e) + log2(l).  16 lanes per (row, head); HBM-bound.
 // ---------------------------------------------------------------------------------------------
@@ -886,9 +1146,19 @@ int launchDkv(const AttnParams& p, size_t smem, unsigned grid, hipStream_t s) {
     return launchAttn(attnBackwardDkvKernel<HDP, TILE, VEC4, 1, STORE>, smem, grid, p, s);
 }
 
+// 0 = every product on the fp32 MFMA; 1 = the forward kernel's products as six bf16 MFMAs each (head dims up to 128)
+std::atomic<int> gAttnRoute{0};
+
 template <int KIND, int HDP, int TILE>
 int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
     constexpr size_t operandBytes = size_t(2) * TILE * (HDP + 4) * sizeof(float);   // one operand, double buffered
+    if constexpr (KIND == 0 && HDP <= 128) {
+        if (gAttnRoute.load() == 1) {
+            constexpr size_t splitBytes = size_t(2) * 3 * 32 * (splitKeyPitch(HDP) + splitValuePitch(HDP)) * sizeof(unsigned short);
+            return vec4 ? launchAttn(attnForwardSplitKernel<HDP, true>, splitBytes, grid, p, s)
+                        : launchAttn(attnForwardSplitKernel<HDP, false>, splitBytes, grid, p, s);
+        }
+    }
     if constexpr (KIND == 0) {
         return vec4 ? launchAttn(attnForwardKernel<HDP, TILE, true>, 2 * operandBytes, grid, p, s)
                     : launchAttn(attnForwardKernel<HDP, TILE, false>, 2 * operandBytes, grid, p, s);
@@ -1175,6 +1445,12 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
     if (batch != 0 && dim != 0) BF_REQUIRE((dQ || newLen == 0) && ((dK && dV) || totalLen == 0), "NULL pointer");
     return bf_hip_attention_backward_img(dOut, q, k, v, out, m, l, dQ, dK, dV, nullptr, nullptr, nullptr, 0, batch, heads, newLen, totalLen, dim,
                                          scale, oldLen, stream);
+}
+
+int bf_hip_attention_set_route(int route) {
+    BF_REQUIRE(route == BF_ATTN_ROUTE_FP32_MFMA || route == BF_ATTN_ROUTE_SPLIT_BF16, "unknown route");
+    bf::gAttnRoute.store(route);
+    return BF_OK;
 }
 
 }  // extern "C"

@@ -409,6 +409,11 @@ int bf_hip_attention_backward_dq(const float* dOut, const float* q, const float*
  * memory; 0 = always recompute); the limit has no counterpart in the reference, whose kernel holds dS in registers. */
 int bf_hip_attention_ds_bytes(size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t* bytes);
 int bf_hip_attention_set_workspace_limit(size_t bytes);
+/* Which matrix instruction the attention products use (a tuning and test switch; results agree to fp32 rounding):
+ * FP32_MFMA = v_mfma_f32_32x32x2_f32 throughout; SPLIT_BF16 = the forward kernel's two products as six bf16 MFMAs each on
+ * operands split into three bf16 terms (24 mantissa bits, fp32 accumulation), head dims up to 128. */
+enum { BF_ATTN_ROUTE_FP32_MFMA = 0, BF_ATTN_ROUTE_SPLIT_BF16 = 1 };
+int bf_hip_attention_set_route(int route);
 int bf_hip_attention_backward_dkv_ds(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
                                      const float* D, float* dK, float* dV, float* dS, size_t batch, size_t heads,
                                      size_t newLen, size_t totalLen, size_t dim, float scale, size_t oldLen,
