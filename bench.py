@@ -38,7 +38,7 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
 # 1249.8 MB written (1095 MB of that is the dS hand-over; the read side moves between 0.64 and 0.90 GB from run to run
 # with what the L2s happen to keep).  profiles/attention_c3_kernel_trace.md holds the commands
 # and the raw counter values.
-MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvKernel": 1932533824}
+MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvPipedKernel": 1932533824}
 
 
 def attention_flops(batch, heads, seq, hd):
@@ -118,16 +118,15 @@ def bench_attention(bf, steps, warmup):
            (("forward", fwd), ("prepare", prep), ("dkv", dkv), ("dq", dqk), ("dkv_recompute", dkv_re),
             ("dq_recompute", dq_re))}
     fl = attention_flops(batch, heads, seq, hd)
-    # the same forward pass with its two products as six bf16 MFMAs each on operands split into three bf16 terms
-    # (bf_hip_attention_set_route; not the default route: `value` and `roofline` above are the fp32-MFMA kernels')
-    call("bf_hip_attention_set_route", 1)
+    # the same pass with every product on the fp32 MFMA (bf_hip_attention_set_route(0)); everything above ran on the
+    # default route, whose forward and dK/dV kernels put each fp32 product on the bf16 matrix pipe as six MFMAs
+    call("bf_hip_attention_set_route", 0)
     try:
-        split_fwd = time_region(bf, stream, fwd, steps, 2)
-        split_step = time_region(bf, stream, step, steps, 1)
+        fp32 = {"forward_ms": time_region(bf, stream, fwd, steps, 2), "dkv_ms": time_region(bf, stream, dkv, steps, 1),
+                "step_ms": time_region(bf, stream, step, steps, 1)}
     finally:
-        call("bf_hip_attention_set_route", 0)
-    return {"ms_per_step": ms_step, "wall_ms_per_step": wall_ms, "kernel_ms": per, "flops": fl,
-            "split_bf16_forward": {"forward_ms": split_fwd, "step_ms": split_step},
+        call("bf_hip_attention_set_route", 3)
+    return {"ms_per_step": ms_step, "wall_ms_per_step": wall_ms, "kernel_ms": per, "flops": fl, "fp32_mfma_route": fp32,
             "shape": {"batch": batch, "heads": heads, "seq": seq, "head_dim": hd}}
 
 
@@ -570,12 +569,19 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "causal fused attention fwd+bwd, fp32, batch 8, heads 16, seq 2048, head_dim 64 "
-                               "(BASELINE.json configs[2])", **res["shape"]},
-        "roofline": {"bound": "mfma", "kernel": "attnBackwardDkvKernel<64,64,..,store dS> (dK, dV and the dS hand-over; key-tile owner)",
+        "config": {"workload": "causal fused attention fwd+bwd, fp32 in and out, batch 8, heads 16, seq 2048, head_dim 64 "
+                               "(BASELINE.json configs[2])", **res["shape"],
+                   "route": "default: forward and dK/dV products as six bf16 MFMAs each on operands split into three bf16 terms "
+                            "(fp32 accuracy, fp32 accumulation); dQ on the fp32 MFMA"},
+        # `achieved` counts the algorithm's fp32 flops (8 hd per visible pair), priced against the fp32 MFMA peak, the
+        # published peak of the arithmetic type the path computes; the kernel issues six bf16 MFMA flops for each of them,
+        # and `bf16_pipe` prices those against the bf16 peak
+        "roofline": {"bound": "mfma", "kernel": "attnBackwardDkvPipedKernel<64,..,store dS> (dK, dV and the dS hand-over; key-tile owner)",
                      "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES["attnBackwardDkvKernel"],
+                     "bf16_pipe": {"executed": round(6 * achieved, 2), "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
+                                   "frac": round(6 * achieved / PEAK_BF16_MFMA_TFLOPS, 4)},
+                     "traffic": MEASURED_TRAFFIC_BYTES["attnBackwardDkvPipedKernel"],
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this kernel on this workload, recorded in "
                                        "profiles/attention_c3_kernel_trace.md (counters cannot be read from inside this run)",
                      "flops_per_launch": fl["dkv"], "launch_ms": round(dkv_ms, 4)},
@@ -587,13 +593,15 @@ def main():
                           "dkv_recompute": round(fl["dkv"] / res["kernel_ms"]["dkv_recompute"] / 1e9, 2),
                           "dq_recompute": round(fl["dq_recompute"] / res["kernel_ms"]["dq_recompute"] / 1e9, 2)},
         "wall_ms_per_step": round(res["wall_ms_per_step"], 4),
-        # an opt-in route (bf_hip_attention_set_route), NOT what `value` measures: the forward kernel with each fp32 product
-        # as six bf16 MFMAs on operands split into three bf16 terms (24 mantissa bits, fp32 accumulation)
-        "split_bf16_forward_route": {
-            "forward_ms": round(res["split_bf16_forward"]["forward_ms"], 4),
-            "forward_tflops_fp32_equivalent": round(fl["fwd"] / res["split_bf16_forward"]["forward_ms"] / 1e9, 2),
-            "step_ms": round(res["split_bf16_forward"]["step_ms"], 4),
-            "step_tflops_fp32_equivalent": round(total_flops / res["split_bf16_forward"]["step_ms"] / 1e9, 2)},
+        # bf_hip_attention_set_route(0), NOT what `value` measures: every product on v_mfma_f32_32x32x2_f32
+        "fp32_mfma_route": {
+            "forward_ms": round(res["fp32_mfma_route"]["forward_ms"], 4),
+            "forward_tflops": round(fl["fwd"] / res["fp32_mfma_route"]["forward_ms"] / 1e9, 2),
+            "dkv_ms": round(res["fp32_mfma_route"]["dkv_ms"], 4),
+            "dkv_tflops": round(fl["dkv"] / res["fp32_mfma_route"]["dkv_ms"] / 1e9, 2),
+            "dkv_frac_of_fp32_mfma_peak": round(fl["dkv"] / res["fp32_mfma_route"]["dkv_ms"] / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
+            "step_ms": round(res["fp32_mfma_route"]["step_ms"], 4),
+            "step_tflops": round(total_flops / res["fp32_mfma_route"]["step_ms"] / 1e9, 2)},
         "device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units},
     }
     if args.train != "none":

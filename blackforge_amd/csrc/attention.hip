@@ -470,26 +470,28 @@ __device__ __forceinline__ void forwardSplitTile(const unsigned short* __restric
                                                  float& lrow, int kt0, int myLimit, int totalLen, int lane) {
     constexpr int KP = splitKeyPitch(HDP), VP = splitValuePitch(HDP), KIMG = 32 * KP, VIMG = 32 * VP, DT = HDP / 32, KS = HDP / 16;
     const int half = lane >> 5, li = lane & 31;
-    // S^T = K Q^T in two accumulator chains (the MFMAs of one chain depend on each other)
-    float16v s0, s1;
+    // S^T = K Q^T in three accumulator chains by magnitude: h h' | h m' + m h' | the three small products.  The chains are
+    // independent (consecutive MFMAs never wait for each other), and the large chain takes one accumulation per step: the
+    // matrix unit rounds every accumulation, and with logits in the tens the roundings of the large chain are the error.
+    float16v s0, s1, s2;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; }
+    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; s2[r] = 0.0f; }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const unsigned short* krow = kimg + li * KP + ks * 16 + half * 8;
         bf16x8a a[3];
 #pragma unroll
         for (int im = 0; im < 3; ++im) a[im] = *reinterpret_cast<const bf16x8a*>(krow + im * KIMG);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][1], s1, 0, 0, 0);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][0], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], qf[ks][0], s1, 0, 0, 0);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][1], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][2], s1, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][1], s2, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][0], s1, 0, 0, 0);
         s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][0], s0, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], qf[ks][0], s2, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][1], s1, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][2], s2, 0, 0, 0);
     }
     float16v sc;   // sc[r] = log2-scaled score of (key = kt0 + dRow(r), this lane's query)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) sc[r] = s0[r] + s1[r];
+    for (int r = 0; r < 16; ++r) sc[r] = (s2[r] + s1[r]) + s0[r];
     if constexpr (MASKED) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -992,6 +994,45 @@ __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const floa
     }
 }
 
+// dk/dv[dt][r]: key = waveK0 + dRow(r, half), d = dt*32 + li  -> 128-byte coalesced rows (fp32 tensors and bf16 images)
+template <int HDP>
+__device__ __forceinline__ void storeKeyGradients(const AttnParams& p, const float16v (&dk)[HDP / 32], const float16v (&dv)[HDP / 32], int b,
+                                                  int h, int waveK0, size_t kOff, int half, int li) {
+    constexpr int DT = HDP / 32;
+    const int hd = p.hd, dim = p.dim;
+    const bool images = p.dKImg != nullptr || p.dVImg != nullptr;
+    // with an even head dim, row pitch and base every even column of an image row is 4-byte aligned and has its neighbour
+    const bool pairs = (hd & 1) == 0 && (p.imgLd & 1u) == 0 && ((reinterpret_cast<uintptr_t>(p.dKImg) | reinterpret_cast<uintptr_t>(p.dVImg)) & 3u) == 0;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const int d = dt * 32 + li;
+        if (d < hd) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int kk = waveK0 + dRow(r, half);
+                if (kk < p.totalLen) {
+                    const float dkv = dk[dt][r] * p.scale, dvv = dv[dt][r];
+                    if (p.dK) p.dK[kOff + size_t(kk) * dim + d] = dkv;
+                    if (p.dV) p.dV[kOff + size_t(kk) * dim + d] = dvv;
+                    if (images) {
+                        const size_t at = (size_t(b) * p.totalLen + kk) * p.imgLd + size_t(h) * hd + d;
+                        if (pairs) {   // lanes 2i and 2i+1 hold neighbouring columns: lane 2i stores both, four bytes at once
+                            const float dkNext = __shfl_down(dkv, 1, 64), dvNext = __shfl_down(dvv, 1, 64);
+                            if ((li & 1) == 0) {
+                                if (p.dKImg) *reinterpret_cast<unsigned*>(p.dKImg + at) = unsigned(toBf16Bits(dkv)) | unsigned(toBf16Bits(dkNext)) << 16;
+                                if (p.dVImg) *reinterpret_cast<unsigned*>(p.dVImg + at) = unsigned(toBf16Bits(dvv)) | unsigned(toBf16Bits(dvNext)) << 16;
+                            }
+                        } else {
+                            if (p.dKImg) p.dKImg[at] = toBf16Bits(dkv);
+                            if (p.dVImg) p.dVImg[at] = toBf16Bits(dvv);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
 // OCC = wavefronts per SIMD the register allocation is held to.  At OCC 2 (head dims up to 64) two workgroups share
 // a CU and cover each other's barriers and tile hand-overs, at the price of a handful of spilled registers; it pays
 // once the grid has more workgroups than two per CU, below that one roomier workgroup per CU is faster.
@@ -1083,38 +1124,556 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
         __syncthreads();
     }
 
-    // dk/dv[dt][r]: key = waveK0 + dRow(r, half), d = dt*32 + li  -> 128-byte coalesced rows
-    const bool images = p.dKImg != nullptr || p.dVImg != nullptr;
-    // with an even head dim, row pitch and base every even column of an image row is 4-byte aligned and has its neighbour
-    const bool pairs = (hd & 1) == 0 && (p.imgLd & 1u) == 0 && ((reinterpret_cast<uintptr_t>(p.dKImg) | reinterpret_cast<uintptr_t>(p.dVImg)) & 3u) == 0;
+    storeKeyGradients<HDP>(p, dk, dv, b, h, waveK0, kOff, half, li);
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward, part 2 on the bf16 matrix pipe at fp32 accuracy: dK, dV (key-tile owner) with every product as six bf16
+// MFMAs on operands split into three bf16 terms (see the forward kernel above).  The wavefront's K and V rows are split
+// once into register fragments (B operands of S = Q K^T and dP = dO V^T, eight head-dim elements per lane and step);
+// Q and dO tiles are split when they are written to LDS and read two ways: 16 bytes of a row as the A operand of S and
+// dP, and through the transposing read as the B operand of dV += P^T dO and dK += dS^T Q, whose contraction runs over
+// queries in the permuted order that makes P^T and dS^T (the A operands) eight consecutive accumulator registers.
+// One wavefront per SIMD: the fragments of K and V alone take 96 registers at head dim 64 and 192 at 128.
+// ---------------------------------------------------------------------------------------------
+template <int HDP, bool MASKED, bool STORE>
+__device__ __forceinline__ void dkvSplitTile(const unsigned short* __restrict__ qimg, const unsigned short* __restrict__ gimg,
+                                             const float* __restrict__ stats, const bf16x8a (&kf)[HDP / 16][3],
+                                             const bf16x8a (&vf)[HDP / 16][3], float16v (&dk)[HDP / 32], float16v (&dv)[HDP / 32], int qt0,
+                                             int key, bool keyValid, int oldLen, int lane, float* __restrict__ dsLane, int newLen) {
+    constexpr int QP = splitKeyPitch(HDP), IMG = 32 * QP, DT = HDP / 32, KS = HDP / 16;
+    const int half = lane >> 5, li = lane & 31;
+    // S = Q K^T in three accumulator chains by magnitude (see the forward kernel), dP = dO V^T in two
+    float16v s0, s1, s2, p0, p1;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        const int d = dt * 32 + li;
-        if (d < hd) {
+    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; s2[r] = 0.0f; p0[r] = 0.0f; p1[r] = 0.0f; }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int kk = waveK0 + dRow(r, half);
-                if (kk < p.totalLen) {
-                    const float dkv = dk[dt][r] * p.scale, dvv = dv[dt][r];
-                    if (p.dK) p.dK[kOff + size_t(kk) * dim + d] = dkv;
-                    if (p.dV) p.dV[kOff + size_t(kk) * dim + d] = dvv;
-                    if (images) {
-                        const size_t at = (size_t(b) * p.totalLen + kk) * p.imgLd + size_t(h) * hd + d;
-                        if (pairs) {   // lanes 2i and 2i+1 hold neighbouring columns: lane 2i stores both, four bytes at once
-                            const float dkNext = __shfl_down(dkv, 1, 64), dvNext = __shfl_down(dvv, 1, 64);
-                            if ((li & 1) == 0) {
-                                if (p.dKImg) *reinterpret_cast<unsigned*>(p.dKImg + at) = unsigned(toBf16Bits(dkv)) | unsigned(toBf16Bits(dkNext)) << 16;
-                                if (p.dVImg) *reinterpret_cast<unsigned*>(p.dVImg + at) = unsigned(toBf16Bits(dvv)) | unsigned(toBf16Bits(dvNext)) << 16;
-                            }
-                        } else {
-                            if (p.dKImg) p.dKImg[at] = toBf16Bits(dkv);
-                            if (p.dVImg) p.dVImg[at] = toBf16Bits(dvv);
-                        }
-                    }
+    for (int ks = 0; ks < KS; ++ks) {
+        const unsigned short* qrow = qimg + li * QP + ks * 16 + half * 8;
+        const unsigned short* grow = gimg + li * QP + ks * 16 + half * 8;
+        bf16x8a a[3], g[3];
+#pragma unroll
+        for (int im = 0; im < 3; ++im) {
+            a[im] = *reinterpret_cast<const bf16x8a*>(qrow + im * IMG);
+            g[im] = *reinterpret_cast<const bf16x8a*>(grow + im * IMG);
+        }
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], kf[ks][1], s2, 0, 0, 0);
+        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[1], vf[ks][1], p1, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], kf[ks][0], s1, 0, 0, 0);
+        p0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[1], vf[ks][0], p0, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], kf[ks][0], s2, 0, 0, 0);
+        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[2], vf[ks][0], p1, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kf[ks][1], s1, 0, 0, 0);
+        p0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[0], vf[ks][1], p0, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kf[ks][2], s2, 0, 0, 0);
+        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[0], vf[ks][2], p1, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kf[ks][0], s0, 0, 0, 0);
+        p0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[0], vf[ks][0], p0, 0, 0, 0);
+    }
+    // register r: query = qt0 + dRow(r, half), key = this lane's key
+    float16v pr, dsv;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const float4v lse4 = loadf4(stats + 8 * g + 4 * half);
+        const float4v d4 = loadf4(stats + 32 + 8 * g + 4 * half);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int r = 4 * g + c;
+            float prob = fastExp2(((s2[r] + s1[r]) + s0[r]) - lse4[c]);
+            if constexpr (MASKED) {
+                const int qi = qt0 + dRow(r, half);
+                prob = (key > oldLen + qi || !keyValid) ? 0.0f : prob;
+            }
+            pr[r] = prob;                                      // P
+            dsv[r] = prob * ((p0[r] + p1[r]) - d4[c]);         // dS (without the scale factor)
+        }
+    }
+    if constexpr (STORE) {
+        if (qt0 < newLen) {   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave
+#pragma unroll
+            for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(dsv[r], dsLane + (8 * (r >> 2) + (r & 3)) * 32);
+        }
+    }
+    // dV += P^T dO, dK += dS^T Q: step st contracts over queries 16 st + 8 (e / 4) + 4 half + e % 4 = registers 8 st + e
+    const int fragRow = 4 * (lane >> 5) + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+    constexpr int order[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};   // (register term, LDS term), small products first
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+        bf16x8a pf[3], df[3];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            __bf16 h, m, l;
+            split3(pr[8 * st + e], h, m, l);
+            pf[0][e] = h; pf[1][e] = m; pf[2][e] = l;
+            split3(dsv[8 * st + e], h, m, l);
+            df[0][e] = h; df[1][e] = m; df[2][e] = l;
+        }
+        bf16x8a gfr[DT][3], qfr[DT][3];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int im = 0; im < 3; ++im) {
+                gfr[dt][im] = readTransposedApart(gimg + im * IMG + (16 * st + fragRow) * QP + dt * 32 + fragCol, QP);
+                qfr[dt][im] = readTransposedApart(qimg + im * IMG + (16 * st + fragRow) * QP + dt * 32 + fragCol, QP);
+            }
+#pragma unroll
+        for (int pr6 = 0; pr6 < 6; ++pr6)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[order[pr6][0]], gfr[dt][order[pr6][1]], dv[dt], 0, 0, 0);
+                dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(df[order[pr6][0]], qfr[dt][order[pr6][1]], dk[dt], 0, 0, 0);
+            }
+    }
+}
+
+// The wavefront's K or V rows as split register fragments: step s of a lane in `half` holds head-dim elements
+// 16 s + 8 half + 0..7 of the lane's key, times `mul`, as three bf16 terms.
+template <int HDP, bool VEC4>
+__device__ __forceinline__ void loadSplitFragments(bf16x8a (&dst)[HDP / 16][3], const float* __restrict__ row, float mul, bool keyValid,
+                                                   int hd, int half) {
+#pragma unroll
+    for (int s = 0; s < HDP / 16; ++s) {
+        float x[8];
+#pragma unroll
+        for (int c = 0; c < 8; c += 4) {
+            const int d = 16 * s + 8 * half + c;
+            float4v val = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (keyValid && d < hd) {
+                if constexpr (VEC4) {
+                    val = loadf4(row + d);
+                } else {
+                    val.x = row[d];
+                    if (d + 1 < hd) val.y = row[d + 1];
+                    if (d + 2 < hd) val.z = row[d + 2];
+                    if (d + 3 < hd) val.w = row[d + 3];
                 }
+            }
+            x[c] = val.x * mul; x[c + 1] = val.y * mul; x[c + 2] = val.z * mul; x[c + 3] = val.w * mul;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            __bf16 hh, mm, ll;
+            split3(x[e], hh, mm, ll);
+            dst[s][0][e] = hh; dst[s][1][e] = mm; dst[s][2][e] = ll;
+        }
+    }
+}
+
+template <int HDP, bool VEC4, bool STORE>
+__global__ void __launch_bounds__(256, 1) attnBackwardDkvSplitKernel(AttnParams p) {
+    constexpr int BQ = 32, QP = splitKeyPitch(HDP), TILE = 3 * BQ * QP, DT = HDP / 32, KS = HDP / 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned short smemSplit[];
+    unsigned short* qs = smemSplit;                 // [2][3][BQ][QP]
+    unsigned short* gs = smemSplit + 2 * TILE;      // [2][3][BQ][QP]
+    float* stats = reinterpret_cast<float*>(smemSplit + 4 * TILE);   // [2][2*BQ]: lse2 | D
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, kt;
+    decodeBlock(p.numTiles, gridDim.x, false, bh, kt);   // the first key tile is seen by every query: heaviest
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const size_t qOff = size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const size_t kOff = size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const size_t statOff = (size_t(b) * p.heads + h) * p.newLen;
+
+    const int waveK0 = kt * 128 + wave * 32;
+    const int key = waveK0 + li;                       // this lane's key (as B-operand column)
+    const bool keyValid = key < p.totalLen;
+    // K (scaled) and V fragments: step ks of a lane in `half` holds head-dim elements 16 ks + 8 half + 0..7 of its key
+    bf16x8a kf[KS][3], vf[KS][3];
+    loadSplitFragments<HDP, VEC4>(kf, p.k + kOff + size_t(key) * dim, p.scale * kLog2e, keyValid, hd, half);
+    loadSplitFragments<HDP, VEC4>(vf, p.v + kOff + size_t(key) * dim, 1.0f, keyValid, hd, half);
+
+    float16v dk[DT], dv[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.0f; dv[dt][r] = 0.0f; }
+
+    // first query that can see any key of this workgroup's tile: oldLen + i >= kt*128
+    int firstQuery = kt * 128 - p.oldLen;
+    if (firstQuery < 0) firstQuery = 0;
+    const int q0Start = (firstQuery / BQ) * BQ;
+    const int numQTiles = q0Start < p.newLen ? (p.newLen - q0Start + BQ - 1) / BQ : 0;
+
+    const size_t dsStride = size_t(p.nkb) * 1024;
+    float* const dsColumn = STORE ? p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024 : nullptr;   // wave-uniform
+    const int dsLaneOffset = half * 128 + li;
+
+    // tiles are short: the loads of a tile are issued two tiles before it is written to LDS (two register stages)
+    TileRegs<HDP, BQ> qStage[2], gStage[2];
+    float statStage[2] = {0.0f, 0.0f};
+    auto fetchAll = [&](int qt0, TileRegs<HDP, BQ>& qr, TileRegs<HDP, BQ>& gr, float& st) {
+        fetchHeadTile<HDP, BQ, VEC4>(qr, p.q + qOff, dim, qt0, p.newLen, hd, tid);
+        fetchHeadTile<HDP, BQ, VEC4>(gr, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+        const int j = tid < BQ ? tid : tid - BQ;
+        const int qi = qt0 + j;
+        if (tid < BQ) st = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
+        else if (tid < 2 * BQ) st = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
+    };
+    auto commitAll = [&](int buf, const TileRegs<HDP, BQ>& qr, const TileRegs<HDP, BQ>& gr, float st) {
+        commitSplitTile<HDP, BQ, QP>(qs + buf * TILE, qr, tid);
+        commitSplitTile<HDP, BQ, QP>(gs + buf * TILE, gr, tid);
+        if (tid < 2 * BQ) stats[buf * 2 * BQ + tid] = st;
+    };
+    if (numQTiles > 0) {
+        fetchAll(q0Start, qStage[0], gStage[0], statStage[0]);
+        if (numQTiles > 1) fetchAll(q0Start + BQ, qStage[1], gStage[1], statStage[1]);
+        commitAll(0, qStage[0], gStage[0], statStage[0]);
+        if (numQTiles > 2) fetchAll(q0Start + 2 * BQ, qStage[0], gStage[0], statStage[0]);
+    }
+    __syncthreads();
+    for (int t0 = 0; t0 < numQTiles; t0 += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int t = t0 + u;
+            if (t >= numQTiles) break;
+            const int qt0 = q0Start + t * BQ;
+            // the wave's keys [waveK0, waveK0+32) are visible to some query of the tile?
+            if (p.oldLen + qt0 + BQ - 1 >= waveK0 && waveK0 < p.totalLen) {
+                const bool masked = (waveK0 + 31 > p.oldLen + qt0) || (waveK0 + 32 > p.totalLen);
+                const unsigned short* qcur = qs + u * TILE;
+                const unsigned short* gcur = gs + u * TILE;
+                const float* scur = stats + u * 2 * BQ;
+                float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
+                if (masked) dkvSplitTile<HDP, true, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane, p.newLen);
+                else dkvSplitTile<HDP, false, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane, p.newLen);
+            }
+            if (t + 1 < numQTiles) {
+                commitAll(u ^ 1, qStage[u ^ 1], gStage[u ^ 1], statStage[u ^ 1]);
+                if (t + 3 < numQTiles) fetchAll(qt0 + 3 * BQ, qStage[u ^ 1], gStage[u ^ 1], statStage[u ^ 1]);
+            }
+            __syncthreads();
+        }
+    }
+    storeKeyGradients<HDP>(p, dk, dv, b, h, waveK0, kOff, half, li);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same dK/dV kernel as a two-stage pipeline over query tiles (head dims up to 64).  A wavefront per SIMD has nobody to
+// hide behind, so the matrix pipe and the vector unit take turns unless one instruction stream feeds both: here the
+// products of two neighbouring tiles are interleaved.  While S and dP of tile t run on the matrix pipe the vector unit
+// splits P and dS of tile t-1 into their bf16 terms; while dV and dK of tile t-1 run, it makes P and dS of tile t from
+// the finished S and dP and stores dS.  LDS reads are issued a step ahead of the MFMAs that consume them.  The order is
+// given to the scheduler as groups (sched_group_barrier); the data flow alone would let it put each kind of work in one
+// run.  Tile t-1 is read (transposed) while tile t is read (plain) and tile t+1 is written: three LDS buffers.
+// ---------------------------------------------------------------------------------------------
+template <int HDP>
+__device__ __forceinline__ void readSplitTransposed(bf16x8a (&gfr)[HDP / 32][3], bf16x8a (&qfr)[HDP / 32][3],
+                                                    const unsigned short* __restrict__ qimg, const unsigned short* __restrict__ gimg,
+                                                    int st, int lane) {
+    constexpr int QP = splitKeyPitch(HDP), IMG = 32 * QP;
+    const int fragRow = 4 * (lane >> 5) + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+#pragma unroll
+    for (int dt = 0; dt < HDP / 32; ++dt)
+#pragma unroll
+        for (int im = 0; im < 3; ++im) {
+            gfr[dt][im] = readTransposedApart(gimg + im * IMG + (16 * st + fragRow) * QP + dt * 32 + fragCol, QP);
+            qfr[dt][im] = readTransposedApart(qimg + im * IMG + (16 * st + fragRow) * QP + dt * 32 + fragCol, QP);
+        }
+}
+
+constexpr int kSchedValu = 0x002, kSchedMfma = 0x008;   // instruction classes of sched_group_barrier
+
+// (register term, LDS term) of the six products of dV += P^T dO and dK += dS^T Q: the LDS terms retire in the order low,
+// middle, high, so that their registers are free for the next fragments; the largest product comes last
+__device__ constexpr int kSplitOrder[6][2] = {{0, 2}, {1, 1}, {0, 1}, {2, 0}, {1, 0}, {0, 0}};
+
+// One step of the pipeline on an unmasked tile: S, dP, P and dS of the tile in (qimg, gimg, stats); dV and dK of the
+// tile before it (qprev, gprev), whose P and dS come in through (pr, dsv) and are replaced by this tile's.  The source
+// is laid out in slices of three MFMAs and a share of the vector work, with a scheduling fence after each.
+template <int HDP, bool STORE>
+__device__ __forceinline__ void dkvSplitStep(const unsigned short* __restrict__ qimg, const unsigned short* __restrict__ gimg,
+                                             const float* __restrict__ stats, const unsigned short* __restrict__ qprev,
+                                             const unsigned short* __restrict__ gprev, const bf16x8a (&kf)[HDP / 16][3],
+                                             const bf16x8a (&vf)[HDP / 16][3], float16v (&dk)[HDP / 32], float16v (&dv)[HDP / 32],
+                                             float16v& pr, float16v& dsv, int lane, float* __restrict__ dsLane) {
+    constexpr int QP = splitKeyPitch(HDP), IMG = 32 * QP, DT = HDP / 32, KS = HDP / 16;
+    static_assert(KS == 2 || KS == 4, "the pipelined form is laid out for head dims 32 and 64");
+    const int half = lane >> 5, li = lane & 31;
+    float16v s, dp;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s[r] = 0.0f; dp[r] = 0.0f; }
+    bf16x8a pf[2][3], df[2][3];
+    // sixteen pairs of neighbouring registers: P first, then dS; step st contracts over registers 8 st + e
+    auto splitPair = [&](int i) {
+        const int st = (i >> 2) & 1, e = (i & 3) * 2;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            __bf16 h, m, l;
+            if (i < 8) {
+                split3(pr[8 * st + e + c], h, m, l);
+                pf[st][0][e + c] = h; pf[st][1][e + c] = m; pf[st][2][e + c] = l;
+            } else {
+                split3(dsv[8 * st + e + c], h, m, l);
+                df[st][0][e + c] = h; df[st][1][e + c] = m; df[st][2][e + c] = l;
+            }
+        }
+    };
+
+    // Stage one: S = Q K^T and dP = dO V^T, one accumulator chain each, the products in the order of their size: the
+    // three small ones (middle x middle, low x high, high x low) of every head-dim step, then the two middle ones, then
+    // high x high, so that a small product is never added to a sum of large ones.  The chains take turns, so an MFMA
+    // never waits for the one before it.  The products come in groups (a size class of one head-dim step); a group's
+    // Q and dO terms are read from LDS while the group before it runs, and read again by a later group rather than
+    // kept: registers are what limits this kernel, LDS bandwidth is not.
+    constexpr int groups1 = 3 * KS;
+    bf16x8a fa[2][3], fg[2][3];
+    auto readGroup1 = [&](int gi) {
+        const int ks = gi % KS, cls = gi / KS;   // 0 small (terms 0, 1, 2), 1 middle (0, 1), 2 large (0)
+        const unsigned short* qrow = qimg + li * QP + ks * 16 + half * 8;
+        const unsigned short* grow = gimg + li * QP + ks * 16 + half * 8;
+#pragma unroll
+        for (int im = 0; im < 3 - cls; ++im) {
+            fa[gi & 1][im] = *reinterpret_cast<const bf16x8a*>(qrow + im * IMG);
+            fg[gi & 1][im] = *reinterpret_cast<const bf16x8a*>(grow + im * IMG);
+        }
+    };
+    // Stage two's operands: the transposed reads of one LDS term of one half (st) at a time, two groups ahead
+    bf16x8a tg[3][DT], tq[3][DT];
+    auto readGroup2 = [&](int gi) {
+        const int st = gi / 3, im = 2 - gi % 3;   // LDS terms in the order low, middle, high
+        const int fragRow = 4 * (lane >> 5) + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            tg[gi % 3][dt] = readTransposedApart(gprev + im * IMG + (16 * st + fragRow) * QP + dt * 32 + fragCol, QP);
+            tq[gi % 3][dt] = readTransposedApart(qprev + im * IMG + (16 * st + fragRow) * QP + dt * 32 + fragCol, QP);
+        }
+    };
+    constexpr int pairsPerSlice = 4 / KS;   // 16 pairs over the 4 KS slices of stage one
+    readGroup1(0);
+#pragma unroll
+    for (int i = 0; i < 12 * KS; ++i) {
+        int gi, at, bt;
+        bool first;
+        if (i < 6 * KS) {
+            gi = i / 6;
+            first = i % 6 == 0;
+            const int pair = (i % 6) >> 1;
+            at = pair == 0 ? 1 : pair == 1 ? 2 : 0;
+            bt = pair == 0 ? 1 : pair == 1 ? 0 : 2;
+        } else if (i < 10 * KS) {
+            gi = KS + (i - 6 * KS) / 4;
+            first = (i - 6 * KS) % 4 == 0;
+            const int pair = ((i - 6 * KS) % 4) >> 1;
+            at = pair == 0 ? 1 : 0;
+            bt = pair == 0 ? 0 : 1;
+        } else {
+            gi = 2 * KS + (i - 10 * KS) / 2;
+            first = (i - 10 * KS) % 2 == 0;
+            at = 0;
+            bt = 0;
+        }
+        const int ks = gi % KS;
+        if (first) {
+            if (gi + 1 < groups1) readGroup1(gi + 1);
+            if (gi == groups1 - 2) readGroup2(0);
+            if (gi == groups1 - 1) readGroup2(1);
+        }
+        if (i & 1) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fg[gi & 1][at], vf[ks][bt], dp, 0, 0, 0);
+        else s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[gi & 1][at], kf[ks][bt], s, 0, 0, 0);
+        if (i % 3 == 2) {
+#pragma unroll
+            for (int c = 0; c < pairsPerSlice; ++c) splitPair((i / 3) * pairsPerSlice + c);
+            // within the slice: some of the split, then each MFMA followed by its share of it (a wavefront alone on
+            // its SIMD issues a vector instruction every five clocks or so, an MFMA occupies the matrix pipe for 32)
+            __builtin_amdgcn_sched_group_barrier(kSchedValu, 2 * pairsPerSlice, 0);
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kSchedValu, 5 * pairsPerSlice, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // Stage two: dV += P^T dO, dK += dS^T Q of the previous tile; P and dS of this one.
+    // register r: query = tile start + dRow(r, half), key = this lane's key
+    float4v lse4[2], d4[2];
+    auto readStats = [&](int grp) {
+        lse4[grp & 1] = loadf4(stats + 8 * grp + 4 * half);
+        d4[grp & 1] = loadf4(stats + 32 + 8 * grp + 4 * half);
+    };
+    auto softmaxRegister = [&](int r) {
+        const int grp = r >> 2, c = r & 3;
+        const float prob = fastExp2(s[r] - lse4[grp & 1][c]);
+        pr[r] = prob;                                       // P
+        dsv[r] = prob * (dp[r] - d4[grp & 1][c]);           // dS (without the scale factor)
+        if constexpr (STORE)   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave
+            __builtin_nontemporal_store(dsv[r], dsLane + (8 * (r >> 2) + (r & 3)) * 32);
+    };
+    constexpr int slices = 4 * DT;                  // slices of three MFMAs in each half of stage two
+    constexpr int registersPerSlice = 2 / DT;       // 16 registers over the 8 DT slices
+    static_assert(DT == 1 || DT == 2, "the pipelined form is laid out for head dims 32 and 64");
+    readStats(0);
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+        for (int q = 0; q < 12 * DT; ++q) {
+            const int pr6 = q / (2 * DT), dt = (q / 2) % DT;
+            const int regTerm = kSplitOrder[pr6][0], ldsTerm = kSplitOrder[pr6][1];
+            const int gi = 3 * st + (2 - ldsTerm);
+            const bool first = q == 0 || kSplitOrder[(q - 1) / (2 * DT)][1] != ldsTerm;
+            if (first && gi + 2 < 6) readGroup2(gi + 2);
+            if (q & 1) dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(df[st][regTerm], tq[gi % 3][dt], dk[dt], 0, 0, 0);
+            else dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[st][regTerm], tg[gi % 3][dt], dv[dt], 0, 0, 0);
+            if (q % 3 == 2) {
+#pragma unroll
+                for (int c = 0; c < registersPerSlice; ++c) {
+                    const int r = (st * slices + q / 3) * registersPerSlice + c;
+                    if ((r & 3) == 0 && r + 4 < 16) readStats((r >> 2) + 1);
+                    softmaxRegister(r);
+                }
+#pragma unroll
+                for (int c = 0; c < 3; ++c) {
+                    __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(kSchedValu, 3 * registersPerSlice, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
+}
+
+// The last pending tile's dV and dK (no tile follows to share the step with).
+template <int HDP>
+__device__ __forceinline__ void dkvSplitDrain(const unsigned short* __restrict__ qprev, const unsigned short* __restrict__ gprev,
+                                              float16v (&dk)[HDP / 32], float16v (&dv)[HDP / 32], const float16v& pr, const float16v& dsv,
+                                              int lane) {
+    constexpr int DT = HDP / 32;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+        bf16x8a pf[3], df[3];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            __bf16 h, m, l;
+            split3(pr[8 * st + e], h, m, l);
+            pf[0][e] = h; pf[1][e] = m; pf[2][e] = l;
+            split3(dsv[8 * st + e], h, m, l);
+            df[0][e] = h; df[1][e] = m; df[2][e] = l;
+        }
+        bf16x8a gfr[DT][3], qfr[DT][3];
+        readSplitTransposed<HDP>(gfr, qfr, qprev, gprev, st, lane);
+#pragma unroll
+        for (int pr6 = 0; pr6 < 6; ++pr6)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[kSplitOrder[pr6][0]], gfr[dt][kSplitOrder[pr6][1]], dv[dt], 0, 0, 0);
+                dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(df[kSplitOrder[pr6][0]], qfr[dt][kSplitOrder[pr6][1]], dk[dt], 0, 0, 0);
+            }
+    }
+}
+
+template <int HDP, bool VEC4, bool STORE>
+__global__ void __launch_bounds__(256, 1) attnBackwardDkvPipedKernel(AttnParams p) {
+    constexpr int BQ = 32, QP = splitKeyPitch(HDP), TILE = 3 * BQ * QP, DT = HDP / 32, KS = HDP / 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned short smemSplit[];
+    unsigned short* qs = smemSplit;                 // [3][3][BQ][QP]
+    unsigned short* gs = smemSplit + 3 * TILE;      // [3][3][BQ][QP]
+    float* stats = reinterpret_cast<float*>(smemSplit + 6 * TILE);   // [3][2*BQ]: lse2 | D
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, kt;
+    decodeBlock(p.numTiles, gridDim.x, false, bh, kt);   // the first key tile is seen by every query: heaviest
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const size_t qOff = size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const size_t kOff = size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const size_t statOff = (size_t(b) * p.heads + h) * p.newLen;
+
+    const int waveK0 = kt * 128 + wave * 32;
+    const int key = waveK0 + li;                       // this lane's key (as B-operand column)
+    const bool keyValid = key < p.totalLen;
+    bf16x8a kf[KS][3], vf[KS][3];
+    loadSplitFragments<HDP, VEC4>(kf, p.k + kOff + size_t(key) * dim, p.scale * kLog2e, keyValid, hd, half);
+    loadSplitFragments<HDP, VEC4>(vf, p.v + kOff + size_t(key) * dim, 1.0f, keyValid, hd, half);
+
+    float16v dk[DT], dv[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.0f; dv[dt][r] = 0.0f; }
+
+    // first query that can see any key of this workgroup's tile: oldLen + i >= kt*128
+    int firstQuery = kt * 128 - p.oldLen;
+    if (firstQuery < 0) firstQuery = 0;
+    const int q0Start = (firstQuery / BQ) * BQ;
+    const int numQTiles = q0Start < p.newLen ? (p.newLen - q0Start + BQ - 1) / BQ : 0;
+
+    const size_t dsStride = size_t(p.nkb) * 1024;
+    float* const dsColumn = STORE ? p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024 : nullptr;   // wave-uniform
+    const int dsLaneOffset = half * 128 + li;
+
+    // a tile's loads are issued one step before it is written to LDS and two before it is read
+    TileRegs<HDP, BQ> qStage, gStage;
+    float statStage = 0.0f;
+    auto fetchAll = [&](int qt0) {
+        fetchHeadTile<HDP, BQ, VEC4>(qStage, p.q + qOff, dim, qt0, p.newLen, hd, tid);
+        fetchHeadTile<HDP, BQ, VEC4>(gStage, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+        const int j = tid < BQ ? tid : tid - BQ;
+        const int qi = qt0 + j;
+        if (tid < BQ) statStage = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
+        else if (tid < 2 * BQ) statStage = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
+    };
+    auto commitAll = [&](int buf) {
+        commitSplitTile<HDP, BQ, QP>(qs + buf * TILE, qStage, tid);
+        commitSplitTile<HDP, BQ, QP>(gs + buf * TILE, gStage, tid);
+        if (tid < 2 * BQ) stats[buf * 2 * BQ + tid] = statStage;
+    };
+    if (numQTiles > 0) {
+        fetchAll(q0Start);
+        commitAll(0);
+        if (numQTiles > 1) fetchAll(q0Start + BQ);
+    }
+    __syncthreads();
+    float16v pr, dsv;       // P and dS of the tile whose dV and dK products are still to come
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { pr[r] = 0.0f; dsv[r] = 0.0f; }
+    int cur = 0, prev = 0;   // LDS buffers of tile t and tile t-1 (at t = 0 any initialised buffer); tile t+1 goes to a third
+    int t = 0;
+    // the end of every tile's step: the next tile goes to LDS, the loads of the one after it are issued, buffers turn
+    auto advance = [&]() {
+        const int next = cur == 2 ? 0 : cur + 1;
+        if (t + 1 < numQTiles) {
+            commitAll(next);
+            if (t + 2 < numQTiles) fetchAll(q0Start + (t + 2) * BQ);
+        }
+        prev = cur;
+        cur = next;
+        ++t;
+        __syncthreads();
+    };
+    // A wavefront's tiles come in three runs: tiles none of whose queries sees its keys, masked tiles (the diagonal;
+    // every tile when the key block runs past the sequence), unmasked tiles.  Both conditions fall as the queries
+    // advance, so the runs follow each other.  The first two go through one loop with the unpiped form, the third
+    // through the pipeline; each loop has the one barrier per tile, so the wavefronts of a workgroup stay in step
+    // although they change loops at different tiles.
+    const bool waveHasKeys = waveK0 < p.totalLen;
+    const bool tailBlock = waveK0 + 32 > p.totalLen;
+    for (; t < numQTiles; advance()) {
+        const int qt0 = q0Start + t * BQ;
+        const bool visible = waveHasKeys && p.oldLen + qt0 + BQ - 1 >= waveK0;
+        const bool masked = tailBlock || waveK0 + 31 > p.oldLen + qt0;
+        if (visible && !masked) break;
+        if (visible) {
+            float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
+            dkvSplitTile<HDP, true, STORE>(qs + cur * TILE, gs + cur * TILE, stats + cur * 2 * BQ, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane,
+                                           dsLane, p.newLen);
+        }
+    }
+    if (t == numQTiles) {   // no unmasked tile; the stores appear on both paths so that neither loop copies registers for the other
+        storeKeyGradients<HDP>(p, dk, dv, b, h, waveK0, kOff, half, li);
+        return;
+    }
+    for (; t < numQTiles; advance()) {
+        // with nothing pending P and dS are zero and the second stage adds zeros (the operands it reads are finite)
+        const int qt0 = q0Start + t * BQ;
+        float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
+        dkvSplitStep<HDP, STORE>(qs + cur * TILE, gs + cur * TILE, stats + cur * 2 * BQ, qs + prev * TILE, gs + prev * TILE, kf, vf, dk, dv, pr, dsv,
+                                 lane, dsLane);
+    }
+    dkvSplitDrain<HDP>(qs + prev * TILE, gs + prev * TILE, dk, dv, pr, dsv, lane);
+    storeKeyGradients<HDP>(p, dk, dv, b, h, waveK0, kOff, half, li);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1146,14 +1705,15 @@ int launchDkv(const AttnParams& p, size_t smem, unsigned grid, hipStream_t s) {
     return launchAttn(attnBackwardDkvKernel<HDP, TILE, VEC4, 1, STORE>, smem, grid, p, s);
 }
 
-// 0 = every product on the fp32 MFMA; 1 = the forward kernel's products as six bf16 MFMAs each (head dims up to 128)
-std::atomic<int> gAttnRoute{0};
+// bit 0: the forward kernel's products as six bf16 MFMAs each; bit 1: the dK/dV kernel's (head dims up to 128 both);
+// 0 = every product on the fp32 MFMA
+std::atomic<int> gAttnRoute{BF_ATTN_ROUTE_SPLIT};
 
 template <int KIND, int HDP, int TILE>
 int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
     constexpr size_t operandBytes = size_t(2) * TILE * (HDP + 4) * sizeof(float);   // one operand, double buffered
     if constexpr (KIND == 0 && HDP <= 128) {
-        if (gAttnRoute.load() == 1) {
+        if (gAttnRoute.load() & 1) {
             constexpr size_t splitBytes = size_t(2) * 3 * 32 * (splitKeyPitch(HDP) + splitValuePitch(HDP)) * sizeof(unsigned short);
             return vec4 ? launchAttn(attnForwardSplitKernel<HDP, true>, splitBytes, grid, p, s)
                         : launchAttn(attnForwardSplitKernel<HDP, false>, splitBytes, grid, p, s);
@@ -1173,6 +1733,18 @@ int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
         return vec4 ? launchAttn(attnBackwardDqFromDsKernel<HDP, TILE, true>, smem, grid, p, s)
                     : launchAttn(attnBackwardDqFromDsKernel<HDP, TILE, false>, smem, grid, p, s);
     } else {
+        if constexpr (HDP <= 128) {
+            if (gAttnRoute.load() & 2) {
+                if constexpr (HDP <= 64) {   // Q and dO images in three buffers, statistics likewise
+                    constexpr size_t pipedBytes = size_t(6) * 3 * 32 * splitKeyPitch(HDP) * sizeof(unsigned short) + size_t(3) * 64 * sizeof(float);
+                    return vec4 ? launchAttn(attnBackwardDkvPipedKernel<HDP, true, KIND == 3>, pipedBytes, grid, p, s)
+                                : launchAttn(attnBackwardDkvPipedKernel<HDP, false, KIND == 3>, pipedBytes, grid, p, s);
+                }
+                constexpr size_t splitBytes = size_t(4) * 3 * 32 * splitKeyPitch(HDP) * sizeof(unsigned short) + size_t(2) * 64 * sizeof(float);
+                return vec4 ? launchAttn(attnBackwardDkvSplitKernel<HDP, true, KIND == 3>, splitBytes, grid, p, s)
+                            : launchAttn(attnBackwardDkvSplitKernel<HDP, false, KIND == 3>, splitBytes, grid, p, s);
+            }
+        }
         constexpr size_t smem = 2 * operandBytes + 4 * TILE * sizeof(float);
         return vec4 ? launchDkv<HDP, TILE, true, KIND == 3>(p, smem, grid, s) : launchDkv<HDP, TILE, false, KIND == 3>(p, smem, grid, s);
     }
@@ -1448,7 +2020,7 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
 }
 
 int bf_hip_attention_set_route(int route) {
-    BF_REQUIRE(route == BF_ATTN_ROUTE_FP32_MFMA || route == BF_ATTN_ROUTE_SPLIT_BF16, "unknown route");
+    BF_REQUIRE(route >= 0 && route <= BF_ATTN_ROUTE_SPLIT, "unknown route");
     bf::gAttnRoute.store(route);
     return BF_OK;
 }

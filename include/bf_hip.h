@@ -409,10 +409,16 @@ int bf_hip_attention_backward_dq(const float* dOut, const float* q, const float*
  * memory; 0 = always recompute); the limit has no counterpart in the reference, whose kernel holds dS in registers. */
 int bf_hip_attention_ds_bytes(size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t* bytes);
 int bf_hip_attention_set_workspace_limit(size_t bytes);
-/* Which matrix instruction the attention products use (a tuning and test switch; results agree to fp32 rounding):
- * FP32_MFMA = v_mfma_f32_32x32x2_f32 throughout; SPLIT_BF16 = the forward kernel's two products as six bf16 MFMAs each on
- * operands split into three bf16 terms (24 mantissa bits, fp32 accumulation), head dims up to 128. */
-enum { BF_ATTN_ROUTE_FP32_MFMA = 0, BF_ATTN_ROUTE_SPLIT_BF16 = 1 };
+/* Which matrix instruction the attention products use (a tuning and test switch; no counterpart in the reference, whose
+ * kernel has one form).  The SPLIT bits put a kernel's products on the bf16 matrix pipe at fp32 accuracy: each fp32
+ * operand is the exact sum of three bf16 terms and each product six bf16 MFMAs (everything above 2^-24 of the product),
+ * accumulated in fp32 in the order of the terms' sizes; head dims up to 128, larger ones stay on the fp32 MFMA
+ * (v_mfma_f32_32x32x2_f32), which route 0 uses throughout.  The default is both bits: the two kernels then recompute
+ * the same scores S, and the results are as close to a float64 evaluation as route 0's (the forward output closer).
+ * With one bit alone the forward statistics (m, l) and the backward pass's S differ in the last bits, which a row
+ * whose maximum drifts by hundreds shows as an error about 1.2 times route 0's.  The dQ kernels run on the fp32 MFMA
+ * on every route. */
+enum { BF_ATTN_ROUTE_FP32_MFMA = 0, BF_ATTN_ROUTE_SPLIT_FORWARD = 1, BF_ATTN_ROUTE_SPLIT_DKV = 2, BF_ATTN_ROUTE_SPLIT = 3 };
 int bf_hip_attention_set_route(int route);
 int bf_hip_attention_backward_dkv_ds(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
                                      const float* D, float* dK, float* dV, float* dS, size_t batch, size_t heads,

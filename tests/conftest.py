@@ -41,7 +41,7 @@ def hip():
     lib = bf.capi.load()
     if bf.capi.device_count() < 1:
         pytest.fail("no HIP device visible: gpu-marked tests need a real MI355X")
-    route = os.environ.get("BF_ATTN_ROUTE")   # run the whole suite on one attention route: BF_ATTN_ROUTE=1 pytest -m gpu
+    route = os.environ.get("BF_ATTN_ROUTE")   # run the whole suite on another attention route: BF_ATTN_ROUTE=0 pytest -m gpu
     if route is not None:
         bf.capi.call("bf_hip_attention_set_route", int(route))
     return bf
