@@ -422,11 +422,36 @@ typedef __bf16 bf16x8a __attribute__((ext_vector_type(8)));
 typedef short short4a __attribute__((ext_vector_type(4)));
 typedef short short8a __attribute__((ext_vector_type(8)));
 
-__device__ __forceinline__ void split3(float x, __bf16& h, __bf16& m, __bf16& l) {
-    h = static_cast<__bf16>(x);
-    const float r1 = x - static_cast<float>(h);
-    m = static_cast<__bf16>(r1);
-    l = static_cast<__bf16>(r1 - static_cast<float>(m));
+typedef __bf16 bf16x2a __attribute__((ext_vector_type(2)));
+typedef float float2a __attribute__((ext_vector_type(2)));
+typedef unsigned uint4a __attribute__((ext_vector_type(4)));
+
+// two floats as a pair of bf16 (round to nearest even), the first in the low half: one v_cvt_pk_bf16_f32
+__device__ __forceinline__ unsigned packBf16(float x0, float x1) {
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(float2a{x0, x1}, bf16x2a));
+}
+
+// x = h + m + l exactly, each term the bf16 nearest to what the terms before it leave; two values at a time so that
+// every conversion fills both halves of its result (eleven instructions a pair)
+__device__ __forceinline__ void splitPair3(float x0, float x1, unsigned& h, unsigned& m, unsigned& l) {
+    h = packBf16(x0, x1);
+    const float r0 = x0 - __builtin_bit_cast(float, h << 16), r1 = x1 - __builtin_bit_cast(float, h & 0xffff0000u);
+    m = packBf16(r0, r1);
+    l = packBf16(r0 - __builtin_bit_cast(float, m << 16), r1 - __builtin_bit_cast(float, m & 0xffff0000u));
+}
+
+// eight values (consecutive elements of an MFMA operand) as three operand terms
+__device__ __forceinline__ void splitOperand(const float (&x)[8], bf16x8a& h, bf16x8a& m, bf16x8a& l) {
+    uint4a hh, mm, ll;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        unsigned a, b, c;
+        splitPair3(x[2 * e], x[2 * e + 1], a, b, c);
+        hh[e] = a; mm[e] = b; ll[e] = c;
+    }
+    h = __builtin_bit_cast(bf16x8a, hh);
+    m = __builtin_bit_cast(bf16x8a, mm);
+    l = __builtin_bit_cast(bf16x8a, ll);
 }
 
 // rows p, p + pitch, p + 2 pitch, p + 3 pitch (as addressed by the lanes) and the same eight rows further down
@@ -449,17 +474,14 @@ __device__ __forceinline__ void commitSplitTile(unsigned short* __restrict__ img
     for (int i = 0; i < TileRegs<HDP, ROWS>::kSlots; ++i) {
         const int s = tid + i * 256;
         if (s < SLOTS) {
-            __bf16 h[4], m[4], l[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) split3(regs.v[i][j], h[j], m[j], l[j]);
-            auto pack = [](const __bf16 (&v)[4]) {
-                return uint2v{unsigned(__builtin_bit_cast(unsigned short, v[0])) | unsigned(__builtin_bit_cast(unsigned short, v[1])) << 16,
-                              unsigned(__builtin_bit_cast(unsigned short, v[2])) | unsigned(__builtin_bit_cast(unsigned short, v[3])) << 16};
-            };
+            unsigned h0, m0, l0, h1, m1, l1;
+            splitPair3(regs.v[i][0], regs.v[i][1], h0, m0, l0);
+            splitPair3(regs.v[i][2], regs.v[i][3], h1, m1, l1);
+            const uint2v h = {h0, h1}, m = {m0, m1}, l = {l0, l1};
             unsigned short* dst = img + (s / V4) * PITCH + (s % V4) * 4;
-            *reinterpret_cast<uint2v*>(dst) = pack(h);
-            *reinterpret_cast<uint2v*>(dst + IMG) = pack(m);
-            *reinterpret_cast<uint2v*>(dst + 2 * IMG) = pack(l);
+            *reinterpret_cast<uint2v*>(dst) = h;
+            *reinterpret_cast<uint2v*>(dst + IMG) = m;
+            *reinterpret_cast<uint2v*>(dst + 2 * IMG) = l;
         }
     }
 }
@@ -523,11 +545,11 @@ __device__ __forceinline__ void forwardSplitTile(const unsigned short* __restric
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
         bf16x8a pf[3];
+        {
+            float x[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            __bf16 h, m, l;
-            split3(sc[8 * st + e], h, m, l);
-            pf[0][e] = h; pf[1][e] = m; pf[2][e] = l;
+            for (int e = 0; e < 8; ++e) x[e] = sc[8 * st + e];
+            splitOperand(x, pf[0], pf[1], pf[2]);
         }
         bf16x8a vf[DT][3];
 #pragma unroll
@@ -587,12 +609,7 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnForwardSplitKernel
                 }
                 x[c] = val.x * mul; x[c + 1] = val.y * mul; x[c + 2] = val.z * mul; x[c + 3] = val.w * mul;
             }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                __bf16 hh, mm, ll;
-                split3(x[e], hh, mm, ll);
-                qf[s][0][e] = hh; qf[s][1][e] = mm; qf[s][2][e] = ll;
-            }
+            splitOperand(x, qf[s][0], qf[s][1], qf[s][2]);
         }
     }
 
@@ -1200,13 +1217,12 @@ __device__ __forceinline__ void dkvSplitTile(const unsigned short* __restrict__ 
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
         bf16x8a pf[3], df[3];
+        {
+            float x[8], y[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            __bf16 h, m, l;
-            split3(pr[8 * st + e], h, m, l);
-            pf[0][e] = h; pf[1][e] = m; pf[2][e] = l;
-            split3(dsv[8 * st + e], h, m, l);
-            df[0][e] = h; df[1][e] = m; df[2][e] = l;
+            for (int e = 0; e < 8; ++e) { x[e] = pr[8 * st + e]; y[e] = dsv[8 * st + e]; }
+            splitOperand(x, pf[0], pf[1], pf[2]);
+            splitOperand(y, df[0], df[1], df[2]);
         }
         bf16x8a gfr[DT][3], qfr[DT][3];
 #pragma unroll
@@ -1250,12 +1266,7 @@ __device__ __forceinline__ void loadSplitFragments(bf16x8a (&dst)[HDP / 16][3], 
             }
             x[c] = val.x * mul; x[c + 1] = val.y * mul; x[c + 2] = val.z * mul; x[c + 3] = val.w * mul;
         }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            __bf16 hh, mm, ll;
-            split3(x[e], hh, mm, ll);
-            dst[s][0][e] = hh; dst[s][1][e] = mm; dst[s][2][e] = ll;
-        }
+        splitOperand(x, dst[s][0], dst[s][1], dst[s][2]);
     }
 }
 
@@ -1394,20 +1405,17 @@ __device__ __forceinline__ void dkvSplitStep(const unsigned short* __restrict__ 
     float16v s, dp;
 #pragma unroll
     for (int r = 0; r < 16; ++r) { s[r] = 0.0f; dp[r] = 0.0f; }
-    bf16x8a pf[2][3], df[2][3];
+    uint4a pf[2][3], df[2][3];   // bf16 pairs; an operand is one of these as eight bf16
     // sixteen pairs of neighbouring registers: P first, then dS; step st contracts over registers 8 st + e
     auto splitPair = [&](int i) {
-        const int st = (i >> 2) & 1, e = (i & 3) * 2;
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            __bf16 h, m, l;
-            if (i < 8) {
-                split3(pr[8 * st + e + c], h, m, l);
-                pf[st][0][e + c] = h; pf[st][1][e + c] = m; pf[st][2][e + c] = l;
-            } else {
-                split3(dsv[8 * st + e + c], h, m, l);
-                df[st][0][e + c] = h; df[st][1][e + c] = m; df[st][2][e + c] = l;
-            }
+        const int st = (i >> 2) & 1, e = i & 3;
+        unsigned a, b, c;
+        if (i < 8) {
+            splitPair3(pr[8 * st + 2 * e], pr[8 * st + 2 * e + 1], a, b, c);
+            pf[st][0][e] = a; pf[st][1][e] = b; pf[st][2][e] = c;
+        } else {
+            splitPair3(dsv[8 * st + 2 * e], dsv[8 * st + 2 * e + 1], a, b, c);
+            df[st][0][e] = a; df[st][1][e] = b; df[st][2][e] = c;
         }
     };
 
@@ -1481,7 +1489,7 @@ __device__ __forceinline__ void dkvSplitStep(const unsigned short* __restrict__ 
 #pragma unroll
             for (int c = 0; c < 3; ++c) {
                 __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(kSchedValu, 5 * pairsPerSlice, 0);
+                __builtin_amdgcn_sched_group_barrier(kSchedValu, 3 * pairsPerSlice, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -1515,8 +1523,8 @@ __device__ __forceinline__ void dkvSplitStep(const unsigned short* __restrict__ 
             const int gi = 3 * st + (2 - ldsTerm);
             const bool first = q == 0 || kSplitOrder[(q - 1) / (2 * DT)][1] != ldsTerm;
             if (first && gi + 2 < 6) readGroup2(gi + 2);
-            if (q & 1) dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(df[st][regTerm], tq[gi % 3][dt], dk[dt], 0, 0, 0);
-            else dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[st][regTerm], tg[gi % 3][dt], dv[dt], 0, 0, 0);
+            if (q & 1) dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8a, df[st][regTerm]), tq[gi % 3][dt], dk[dt], 0, 0, 0);
+            else dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8a, pf[st][regTerm]), tg[gi % 3][dt], dv[dt], 0, 0, 0);
             if (q % 3 == 2) {
 #pragma unroll
                 for (int c = 0; c < registersPerSlice; ++c) {
@@ -1544,13 +1552,12 @@ __device__ __forceinline__ void dkvSplitDrain(const unsigned short* __restrict__
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
         bf16x8a pf[3], df[3];
+        {
+            float x[8], y[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            __bf16 h, m, l;
-            split3(pr[8 * st + e], h, m, l);
-            pf[0][e] = h; pf[1][e] = m; pf[2][e] = l;
-            split3(dsv[8 * st + e], h, m, l);
-            df[0][e] = h; df[1][e] = m; df[2][e] = l;
+            for (int e = 0; e < 8; ++e) { x[e] = pr[8 * st + e]; y[e] = dsv[8 * st + e]; }
+            splitOperand(x, pf[0], pf[1], pf[2]);
+            splitOperand(y, df[0], df[1], df[2]);
         }
         bf16x8a gfr[DT][3], qfr[DT][3];
         readSplitTransposed<HDP>(gfr, qfr, qprev, gprev, st, lane);
