@@ -112,6 +112,21 @@ __device__ __forceinline__ void fetchHeadTile(TileRegs<HDP, ROWS>& regs, const f
     }
 }
 
+// The same tile for a caller that can take any finite values in rows past the limit (it multiplies them by zero): the
+// row index is clamped instead of tested, and the column's pointer and validity are the thread's constants.  16-byte
+// aligned rows only.
+template <int HDP, int ROWS>
+__device__ __forceinline__ void fetchRowsClamped(TileRegs<HDP, ROWS>& regs, const float* __restrict__ columnBase, bool columnValid, int dim,
+                                                 int row0, int lastRow, int tid) {
+    constexpr int V4 = HDP / 4;
+    static_assert((ROWS * V4) % 256 == 0, "every thread takes the same number of slots");
+#pragma unroll
+    for (int i = 0; i < TileRegs<HDP, ROWS>::kSlots; ++i) {
+        const int row = min(row0 + (tid + i * 256) / V4, lastRow);
+        regs.v[i] = columnValid ? loadf4(columnBase + size_t(row) * dim) : float4v{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+}
+
 template <int HDP, int ROWS>
 __device__ __forceinline__ void commitHeadTile(float* __restrict__ lds, const TileRegs<HDP, ROWS>& regs, int tid) {
     constexpr int LDSW = HDP + 4;
@@ -1384,8 +1399,6 @@ __device__ __forceinline__ void readSplitTransposed(bf16x8a (&gfr)[HDP / 32][3],
         }
 }
 
-constexpr int kSchedValu = 0x002, kSchedMfma = 0x008;   // instruction classes of sched_group_barrier
-
 // (register term, LDS term) of the six products of dV += P^T dO and dK += dS^T Q: the LDS terms retire in the order low,
 // middle, high, so that their registers are free for the next fragments; the largest product comes last
 __device__ constexpr int kSplitOrder[6][2] = {{0, 2}, {1, 1}, {0, 1}, {2, 0}, {1, 0}, {0, 0}};
@@ -1407,15 +1420,25 @@ __device__ __forceinline__ void dkvSplitStep(const unsigned short* __restrict__ 
     for (int r = 0; r < 16; ++r) { s[r] = 0.0f; dp[r] = 0.0f; }
     uint4a pf[2][3], df[2][3];   // bf16 pairs; an operand is one of these as eight bf16
     // sixteen pairs of neighbouring registers: P first, then dS; step st contracts over registers 8 st + e
-    auto splitPair = [&](int i) {
+    // The split of pair i in three parts (high term and what it leaves; middle term and what it leaves; low term), one
+    // after each MFMA of a slice; `rest` carries the remainders from part to part.
+    float rest[2][2];
+    auto splitPairPart = [&](int i, int c, int part) {
         const int st = (i >> 2) & 1, e = i & 3;
-        unsigned a, b, c;
-        if (i < 8) {
-            splitPair3(pr[8 * st + 2 * e], pr[8 * st + 2 * e + 1], a, b, c);
-            pf[st][0][e] = a; pf[st][1][e] = b; pf[st][2][e] = c;
+        uint4a(&dst)[3] = i < 8 ? pf[st] : df[st];
+        if (part == 0) {
+            const float x0 = i < 8 ? pr[8 * st + 2 * e] : dsv[8 * st + 2 * e], x1 = i < 8 ? pr[8 * st + 2 * e + 1] : dsv[8 * st + 2 * e + 1];
+            const unsigned h = packBf16(x0, x1);
+            dst[0][e] = h;
+            rest[c][0] = x0 - __builtin_bit_cast(float, h << 16);
+            rest[c][1] = x1 - __builtin_bit_cast(float, h & 0xffff0000u);
+        } else if (part == 1) {
+            const unsigned m = packBf16(rest[c][0], rest[c][1]);
+            dst[1][e] = m;
+            rest[c][0] -= __builtin_bit_cast(float, m << 16);
+            rest[c][1] -= __builtin_bit_cast(float, m & 0xffff0000u);
         } else {
-            splitPair3(dsv[8 * st + 2 * e], dsv[8 * st + 2 * e + 1], a, b, c);
-            df[st][0][e] = a; df[st][1][e] = b; df[st][2][e] = c;
+            dst[2][e] = packBf16(rest[c][0], rest[c][1]);
         }
     };
 
@@ -1480,19 +1503,11 @@ __device__ __forceinline__ void dkvSplitStep(const unsigned short* __restrict__ 
         }
         if (i & 1) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fg[gi & 1][at], vf[ks][bt], dp, 0, 0, 0);
         else s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[gi & 1][at], kf[ks][bt], s, 0, 0, 0);
-        if (i % 3 == 2) {
+        // a third of a pair's split after every MFMA, and a fence: nothing moves across, so the matrix pipe (32 clocks an
+        // MFMA) and the vector unit (a wavefront alone on its SIMD issues an instruction every five clocks or so) alternate
 #pragma unroll
-            for (int c = 0; c < pairsPerSlice; ++c) splitPair((i / 3) * pairsPerSlice + c);
-            // within the slice: some of the split, then each MFMA followed by its share of it (a wavefront alone on
-            // its SIMD issues a vector instruction every five clocks or so, an MFMA occupies the matrix pipe for 32)
-            __builtin_amdgcn_sched_group_barrier(kSchedValu, 2 * pairsPerSlice, 0);
-#pragma unroll
-            for (int c = 0; c < 3; ++c) {
-                __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(kSchedValu, 3 * pairsPerSlice, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        for (int c = 0; c < pairsPerSlice; ++c) splitPairPart((i / 3) * pairsPerSlice + c, c, i % 3);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // Stage two: dV += P^T dO, dK += dS^T Q of the previous tile; P and dS of this one.
@@ -1502,13 +1517,17 @@ __device__ __forceinline__ void dkvSplitStep(const unsigned short* __restrict__ 
         lse4[grp & 1] = loadf4(stats + 8 * grp + 4 * half);
         d4[grp & 1] = loadf4(stats + 32 + 8 * grp + 4 * half);
     };
-    auto softmaxRegister = [&](int r) {
+    // P and dS of register r in three parts, one after each MFMA of a slice
+    auto softmaxPart = [&](int r, int part) {
         const int grp = r >> 2, c = r & 3;
-        const float prob = fastExp2(s[r] - lse4[grp & 1][c]);
-        pr[r] = prob;                                       // P
-        dsv[r] = prob * (dp[r] - d4[grp & 1][c]);           // dS (without the scale factor)
-        if constexpr (STORE)   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave
-            __builtin_nontemporal_store(dsv[r], dsLane + (8 * (r >> 2) + (r & 3)) * 32);
+        if (part == 0) {
+            pr[r] = fastExp2(s[r] - lse4[grp & 1][c]);            // P
+        } else if (part == 1) {
+            dsv[r] = pr[r] * (dp[r] - d4[grp & 1][c]);            // dS (without the scale factor)
+        } else {
+            if constexpr (STORE)   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave
+                __builtin_nontemporal_store(dsv[r], dsLane + (8 * (r >> 2) + (r & 3)) * 32);
+        }
     };
     constexpr int slices = 4 * DT;                  // slices of three MFMAs in each half of stage two
     constexpr int registersPerSlice = 2 / DT;       // 16 registers over the 8 DT slices
@@ -1525,20 +1544,13 @@ __device__ __forceinline__ void dkvSplitStep(const unsigned short* __restrict__ 
             if (first && gi + 2 < 6) readGroup2(gi + 2);
             if (q & 1) dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8a, df[st][regTerm]), tq[gi % 3][dt], dk[dt], 0, 0, 0);
             else dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8a, pf[st][regTerm]), tg[gi % 3][dt], dv[dt], 0, 0, 0);
-            if (q % 3 == 2) {
 #pragma unroll
-                for (int c = 0; c < registersPerSlice; ++c) {
-                    const int r = (st * slices + q / 3) * registersPerSlice + c;
-                    if ((r & 3) == 0 && r + 4 < 16) readStats((r >> 2) + 1);
-                    softmaxRegister(r);
-                }
-#pragma unroll
-                for (int c = 0; c < 3; ++c) {
-                    __builtin_amdgcn_sched_group_barrier(kSchedMfma, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(kSchedValu, 3 * registersPerSlice, 0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
+            for (int c = 0; c < registersPerSlice; ++c) {
+                const int r = (st * slices + q / 3) * registersPerSlice + c;
+                if (q % 3 == 0 && (r & 3) == 0 && r + 4 < 16) readStats((r >> 2) + 1);
+                softmaxPart(r, q % 3);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -1611,12 +1623,21 @@ __global__ void __launch_bounds__(256, 1) attnBackwardDkvPipedKernel(AttnParams 
     float* const dsColumn = STORE ? p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024 : nullptr;   // wave-uniform
     const int dsLaneOffset = half * 128 + li;
 
-    // a tile's loads are issued one step before it is written to LDS and two before it is read
+    // a tile's loads are issued one step before it is written to LDS and two before it is read.  Rows past the last
+    // query repeat it: their statistic is +inf, so their P and dS are zero whatever Q and dO hold there.
     TileRegs<HDP, BQ> qStage, gStage;
     float statStage = 0.0f;
+    const int fetchColumn = (tid % (HDP / 4)) * 4;
+    const float* const qColumn = p.q + qOff + fetchColumn;
+    const float* const gColumn = p.dO + qOff + fetchColumn;
     auto fetchAll = [&](int qt0) {
-        fetchHeadTile<HDP, BQ, VEC4>(qStage, p.q + qOff, dim, qt0, p.newLen, hd, tid);
-        fetchHeadTile<HDP, BQ, VEC4>(gStage, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+        if constexpr (VEC4) {
+            fetchRowsClamped<HDP, BQ>(qStage, qColumn, fetchColumn < hd, dim, qt0, p.newLen - 1, tid);
+            fetchRowsClamped<HDP, BQ>(gStage, gColumn, fetchColumn < hd, dim, qt0, p.newLen - 1, tid);
+        } else {
+            fetchHeadTile<HDP, BQ, false>(qStage, p.q + qOff, dim, qt0, p.newLen, hd, tid);
+            fetchHeadTile<HDP, BQ, false>(gStage, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+        }
         const int j = tid < BQ ? tid : tid - BQ;
         const int qi = qt0 + j;
         if (tid < BQ) statStage = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
