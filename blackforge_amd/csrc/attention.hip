@@ -1,4 +1,8 @@
-// Fused causal attention, forward and backward, fp32 on the fp32 MFMA pipe (v_mfma_f32_32x32x2_f32).
+// Fused causal attention, forward and backward, fp32 in and out.  Two sets of kernels for the forward pass and for
+// dK/dV, chosen by bf_hip_attention_set_route: every product on the fp32 MFMA (v_mfma_f32_32x32x2_f32; the kernels
+// described first), or, by default, every fp32 product as six bf16 MFMAs on operands split into three bf16 terms
+// (attnForwardSplitKernel, attnBackwardDkvSplitKernel, attnBackwardDkvPipedKernel further down; same ownership, tiling
+// and statistics, fp32 accuracy).  The dQ kernels run on the fp32 MFMA on both routes.
 //
 // Layout: q [batch,newLen,dim], k/v [batch,totalLen,dim], heads contiguous in dim.  Query row i
 // (absolute position oldLen+i) attends to keys j <= oldLen+i.
