@@ -1,7 +1,7 @@
 // Fused causal attention, forward and backward, fp32 in and out.  Two sets of kernels for the forward pass and for
 // dK/dV, chosen by bf_hip_attention_set_route: every product on the fp32 MFMA (v_mfma_f32_32x32x2_f32; the kernels
 // described first), or, by default, every fp32 product as six bf16 MFMAs on operands split into three bf16 terms
-// (attnForwardSplitKernel, attnBackwardDkvSplitKernel, attnBackwardDkvPipedKernel further down; same ownership, tiling
+// (attnForwardPipedKernel, attnBackwardDkvSplitKernel, attnBackwardDkvPipedKernel further down; same ownership, tiling
 // and statistics, fp32 accuracy).  The dQ kernels run on the fp32 MFMA on both routes.
 //
 // Layout: q [batch,newLen,dim], k/v [batch,totalLen,dim], heads contiguous in dim.  Query row i
@@ -501,199 +501,6 @@ __device__ __forceinline__ void commitSplitTile(unsigned short* __restrict__ img
             *reinterpret_cast<uint2v*>(dst) = h;
             *reinterpret_cast<uint2v*>(dst + IMG) = m;
             *reinterpret_cast<uint2v*>(dst + 2 * IMG) = l;
-        }
-    }
-}
-
-template <int HDP, bool MASKED>
-__device__ __forceinline__ void forwardSplitTile(const unsigned short* __restrict__ kimg, const unsigned short* __restrict__ vimg,
-                                                 const bf16x8a (&qf)[HDP / 16][3], float16v (&acc)[HDP / 32], float& mrow, float& mref,
-                                                 float& lrow, int kt0, int myLimit, int totalLen, int lane) {
-    constexpr int KP = splitKeyPitch(HDP), VP = splitValuePitch(HDP), KIMG = 32 * KP, VIMG = 32 * VP, DT = HDP / 32, KS = HDP / 16;
-    const int half = lane >> 5, li = lane & 31;
-    // S^T = K Q^T in three accumulator chains by magnitude: h h' | h m' + m h' | the three small products.  The chains are
-    // independent (consecutive MFMAs never wait for each other), and the large chain takes one accumulation per step: the
-    // matrix unit rounds every accumulation, and with logits in the tens the roundings of the large chain are the error.
-    float16v s0, s1, s2;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; s2[r] = 0.0f; }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        const unsigned short* krow = kimg + li * KP + ks * 16 + half * 8;
-        bf16x8a a[3];
-#pragma unroll
-        for (int im = 0; im < 3; ++im) a[im] = *reinterpret_cast<const bf16x8a*>(krow + im * KIMG);
-        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][1], s2, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][0], s1, 0, 0, 0);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][0], s0, 0, 0, 0);
-        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], qf[ks][0], s2, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][1], s1, 0, 0, 0);
-        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][2], s2, 0, 0, 0);
-    }
-    float16v sc;   // sc[r] = log2-scaled score of (key = kt0 + dRow(r), this lane's query)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) sc[r] = (s2[r] + s1[r]) + s0[r];
-    if constexpr (MASKED) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int key = kt0 + dRow(r, half);
-            sc[r] = (key > myLimit || key >= totalLen) ? -INFINITY : sc[r];
-        }
-    }
-    float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
-#pragma unroll
-    for (int r = 4; r < 16; r += 4) mx = fmaxf(mx, fmaxf(fmaxf(sc[r], sc[r + 1]), fmaxf(sc[r + 2], sc[r + 3])));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    mrow = fmaxf(mrow, mx);
-    const bool moveRef = mrow > mref + kRescaleThreshold;   // also true on the first visible key (mref = -inf)
-    if (__builtin_amdgcn_ballot_w64(moveRef) != 0) {
-        const float corr = moveRef ? fastExp2(mref - mrow) : 1.0f;   // 0 when the reference was still -inf
-        mref = moveRef ? mrow : mref;
-        lrow *= corr;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
-    }
-    float psum = 0.0f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { sc[r] = fastExp2(sc[r] - mref); psum += sc[r]; }
-    lrow += psum;
-    // O^T += V^T P^T: step s contracts over keys 16 s + 8 (e / 4) + 4 half + e % 4, i.e. registers 8 s .. 8 s + 7 of sc
-    const int fragRow = 4 * (lane >> 5) + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-#pragma unroll
-    for (int st = 0; st < 2; ++st) {
-        bf16x8a pf[3];
-        {
-            float x[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = sc[8 * st + e];
-            splitOperand(x, pf[0], pf[1], pf[2]);
-        }
-        bf16x8a vf[DT][3];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int im = 0; im < 3; ++im) vf[dt][im] = readTransposedApart(vimg + im * VIMG + (16 * st + fragRow) * VP + dt * 32 + fragCol, VP);
-        // the six products of each head-dim block, the blocks taking turns: consecutive MFMAs do not depend on each other
-        constexpr int order[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};   // (V term, P term), small products first
-#pragma unroll
-        for (int pr = 0; pr < 6; ++pr)
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][order[pr][0]], pf[order[pr][1]], acc[dt], 0, 0, 0);
-    }
-}
-
-template <int HDP, bool VEC4>
-__global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnForwardSplitKernel(AttnParams p) {
-    constexpr int BC = 32, KP = splitKeyPitch(HDP), VP = splitValuePitch(HDP), KTILE = 3 * BC * KP, VTILE = 3 * BC * VP, DT = HDP / 32, KS = HDP / 16;
-    extern __shared__ __attribute__((aligned(16))) unsigned short smemSplit[];
-    unsigned short* ks = smemSplit;               // [2][3][BC][KP]
-    unsigned short* vs = smemSplit + 2 * KTILE;   // [2][3][BC][VP]
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
-    int bh, qt;
-    decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
-    const int b = bh / p.heads, h = bh - b * p.heads;
-    const int hd = p.hd, dim = p.dim;
-    const float* qb = p.q + size_t(b) * p.newLen * dim + size_t(h) * hd;
-    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
-    const float* vb = p.v + size_t(b) * p.totalLen * dim + size_t(h) * hd;
-
-    const int waveQ0 = qt * 128 + wave * 32;
-    const int i = waveQ0 + li;                    // this lane's query row
-    const bool rowValid = i < p.newLen;
-    // Q fragments: step ks of a lane in `half` holds head-dim elements 16 ks + 8 half + 0..7 of its query, scaled
-    bf16x8a qf[KS][3];
-    {
-        const float* row = qb + size_t(i) * dim;
-        const float mul = p.scale * kLog2e;
-#pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            float x[8];
-#pragma unroll
-            for (int c = 0; c < 8; c += 4) {
-                const int d = 16 * s + 8 * half + c;
-                float4v val = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (rowValid && d < hd) {
-                    if constexpr (VEC4) {
-                        val = loadf4(row + d);
-                    } else {
-                        val.x = row[d];
-                        if (d + 1 < hd) val.y = row[d + 1];
-                        if (d + 2 < hd) val.z = row[d + 2];
-                        if (d + 3 < hd) val.w = row[d + 3];
-                    }
-                }
-                x[c] = val.x * mul; x[c + 1] = val.y * mul; x[c + 2] = val.z * mul; x[c + 3] = val.w * mul;
-            }
-            splitOperand(x, qf[s][0], qf[s][1], qf[s][2]);
-        }
-    }
-
-    float16v acc[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
-    float mrow = -INFINITY, mref = -INFINITY, lrow = 0.0f;
-
-    const int lastQuery = min(p.newLen, qt * 128 + 128) - 1;
-    const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);   // keys >= this are invisible to the tile
-    const int waveKeyEnd = p.oldLen + waveQ0 + 32;                       // keys >= this are invisible to the wave
-    const int myLimit = p.oldLen + i;                                    // last visible key of this lane's row
-    const int numKeyTiles = (blockKeyEnd + BC - 1) / BC;
-
-    // Tiles are short (32 keys), so the loads of a tile are issued TWO tiles before it is written to LDS: tile t + 1 waits
-    // in register set (t + 1) & 1 while tile t is multiplied, and that set is refilled with tile t + 3 once it is written.
-    TileRegs<HDP, BC> kStage[2], vStage[2];
-    fetchHeadTile<HDP, BC, VEC4>(kStage[0], kb, dim, 0, p.totalLen, hd, tid);
-    fetchHeadTile<HDP, BC, VEC4>(vStage[0], vb, dim, 0, p.totalLen, hd, tid);
-    if (numKeyTiles > 1) {
-        fetchHeadTile<HDP, BC, VEC4>(kStage[1], kb, dim, BC, p.totalLen, hd, tid);
-        fetchHeadTile<HDP, BC, VEC4>(vStage[1], vb, dim, BC, p.totalLen, hd, tid);
-    }
-    commitSplitTile<HDP, BC, KP>(ks, kStage[0], tid);
-    commitSplitTile<HDP, BC, VP>(vs, vStage[0], tid);
-    if (numKeyTiles > 2) {
-        fetchHeadTile<HDP, BC, VEC4>(kStage[0], kb, dim, 2 * BC, p.totalLen, hd, tid);
-        fetchHeadTile<HDP, BC, VEC4>(vStage[0], vb, dim, 2 * BC, p.totalLen, hd, tid);
-    }
-    __syncthreads();
-    for (int t0 = 0; t0 < numKeyTiles; t0 += 2) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int t = t0 + u;
-            if (t >= numKeyTiles) break;
-            const int kt0 = t * BC;
-            const unsigned short* kcur = ks + u * KTILE;
-            const unsigned short* vcur = vs + u * VTILE;
-            if (kt0 < waveKeyEnd) {   // wave-uniform: the tile holds keys some row of this wave can see
-                const bool masked = (kt0 + BC - 1 > p.oldLen + waveQ0) || (kt0 + BC > p.totalLen);
-                if (masked) forwardSplitTile<HDP, true>(kcur, vcur, qf, acc, mrow, mref, lrow, kt0, myLimit, p.totalLen, lane);
-                else forwardSplitTile<HDP, false>(kcur, vcur, qf, acc, mrow, mref, lrow, kt0, myLimit, p.totalLen, lane);
-            }
-            if (t + 1 < numKeyTiles) {
-                commitSplitTile<HDP, BC, KP>(ks + (u ^ 1) * KTILE, kStage[u ^ 1], tid);
-                commitSplitTile<HDP, BC, VP>(vs + (u ^ 1) * VTILE, vStage[u ^ 1], tid);
-                if (t + 3 < numKeyTiles) {
-                    fetchHeadTile<HDP, BC, VEC4>(kStage[u ^ 1], kb, dim, kt0 + 3 * BC, p.totalLen, hd, tid);
-                    fetchHeadTile<HDP, BC, VEC4>(vStage[u ^ 1], vb, dim, kt0 + 3 * BC, p.totalLen, hd, tid);
-                }
-            }
-            __syncthreads();
-        }
-    }
-
-    lrow += __shfl_xor(lrow, 32, 64);
-    if (rowValid) {
-        if (p.out) storeTransposed<HDP, VEC4>(p.out + (size_t(b) * p.newLen + i) * dim + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
-        if (p.outImg) storeTransposedBf16<HDP, VEC4>(p.outImg + (size_t(b) * p.newLen + i) * p.imgLd + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
-        if (half == 0) {
-            size_t idx = (size_t(b) * p.heads + h) * p.newLen + i;
-            p.m[idx] = mrow * kLn2;
-            p.l[idx] = lrow * fastExp2(mref - mrow);
         }
     }
 }
@@ -1709,6 +1516,292 @@ __global__ void __launch_bounds__(256, 1) attnBackwardDkvPipedKernel(AttnParams 
 }
 
 // ---------------------------------------------------------------------------------------------
+// The forward kernel on the split route as a two-stage pipeline over key tiles (the scheme of the dK/dV pipeline
+// above).  While S^T of tile t+1 runs on the matrix pipe the vector unit splits P of tile t; while O^T += V^T P^T of
+// tile t runs, it takes the row maximum, the exponentials and the row sum of tile t+1.  One MFMA and one part of the
+// vector work at a time, a scheduling fence after each.  A move of the reference maximum found while the products of
+// the tile before are still in flight is applied to the accumulator after them.  K tiles are written to LDS two tiles
+// ahead of their products and V tiles one tile ahead, so two buffers of each suffice.  A wavefront's masked tiles are
+// its last ones, so it passes from the loop with unmasked next tiles to the loop with masked ones, then to the last
+// tile's products alone, then waits out the workgroup's remaining tiles; every loop has the one barrier per tile.
+// ---------------------------------------------------------------------------------------------
+template <int HDP>
+__device__ __forceinline__ float16v forwardSplitScores(const unsigned short* __restrict__ kimg, const bf16x8a (&qf)[HDP / 16][3], int lane) {
+    constexpr int KP = splitKeyPitch(HDP), KIMG = 32 * KP, KS = HDP / 16;
+    const int half = lane >> 5, li = lane & 31;
+    float16v s0, s1, s2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; s2[r] = 0.0f; }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const unsigned short* krow = kimg + li * KP + ks * 16 + half * 8;
+        bf16x8a a[3];
+#pragma unroll
+        for (int im = 0; im < 3; ++im) a[im] = *reinterpret_cast<const bf16x8a*>(krow + im * KIMG);
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][1], s2, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], qf[ks][0], s1, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][0], s0, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], qf[ks][0], s2, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][1], s1, 0, 0, 0);
+        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], qf[ks][2], s2, 0, 0, 0);
+    }
+    float16v sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = (s2[r] + s1[r]) + s0[r];
+    return sc;
+}
+
+// Scores of the first tile to probabilities about a fresh reference maximum (nothing accumulated yet).
+template <bool MASKED>
+__device__ __forceinline__ void forwardFirstSoftmax(float16v& sc, float& mrow, float& mref, float& lrow, int kt0, int myLimit, int totalLen,
+                                                    int lane) {
+    const int half = lane >> 5;
+    if constexpr (MASKED) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = kt0 + dRow(r, half);
+            sc[r] = (key > myLimit || key >= totalLen) ? -INFINITY : sc[r];
+        }
+    }
+    float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+#pragma unroll
+    for (int r = 4; r < 16; r += 4) mx = fmaxf(mx, fmaxf(fmaxf(sc[r], sc[r + 1]), fmaxf(sc[r + 2], sc[r + 3])));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mrow = mx;
+    mref = mx;   // key 0 is visible to every query, so this is finite
+    float psum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { sc[r] = fastExp2(sc[r] - mref); psum += sc[r]; }
+    lrow = psum;
+}
+
+// One step: `pc` comes in as P of the current tile (probabilities about mref, accumulator layout) and leaves as P of the
+// next one; knext = K images of the next tile, vcur = V images of the current one.
+template <int HDP, bool MASKED, bool HAS_NEXT>
+__device__ __forceinline__ void forwardPipedStep(const unsigned short* __restrict__ knext, const unsigned short* __restrict__ vcur,
+                                                 const bf16x8a (&qf)[HDP / 16][3], float16v (&acc)[HDP / 32], float16v& pc, float& mrow,
+                                                 float& mref, float& lrow, int ktNext0, int myLimit, int totalLen, int lane) {
+    constexpr int KP = splitKeyPitch(HDP), VP = splitValuePitch(HDP), KIMG = 32 * KP, VIMG = 32 * VP, DT = HDP / 32, KS = HDP / 16;
+    const int half = lane >> 5, li = lane & 31;
+    uint4a pf[2][3];   // bf16 pairs; an operand is one of these as eight bf16
+    float rest[2];
+    // the split of pair i of P (registers 2 i, 2 i + 1; step st = i / 4 contracts over registers 8 st + e) in three parts
+    auto splitPart = [&](int i, int part) {
+        const int st = i >> 2, e = i & 3;
+        if (part == 0) {
+            const float x0 = pc[2 * i], x1 = pc[2 * i + 1];
+            const unsigned h = packBf16(x0, x1);
+            pf[st][0][e] = h;
+            rest[0] = x0 - __builtin_bit_cast(float, h << 16);
+            rest[1] = x1 - __builtin_bit_cast(float, h & 0xffff0000u);
+        } else if (part == 1) {
+            const unsigned m = packBf16(rest[0], rest[1]);
+            pf[st][1][e] = m;
+            rest[0] -= __builtin_bit_cast(float, m << 16);
+            rest[1] -= __builtin_bit_cast(float, m & 0xffff0000u);
+        } else {
+            pf[st][2][e] = packBf16(rest[0], rest[1]);
+        }
+    };
+    // V^T operands of stage two: the transposed reads of one LDS term of one half (st) at a time, two groups ahead
+    bf16x8a tv[3][DT];
+    auto readV = [&](int gi) {
+        const int st = gi / 3, im = 2 - gi % 3;   // LDS terms in the order low, middle, high
+        const int fragRow = 4 * (lane >> 5) + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) tv[gi % 3][dt] = readTransposedApart(vcur + im * VIMG + (16 * st + fragRow) * VP + dt * 32 + fragCol, VP);
+    };
+
+    // stage one: S^T = K Q^T of the next tile, one chain, the products in the order of their size (see the dK/dV pipeline)
+    float16v s;
+    if constexpr (HAS_NEXT) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+        bf16x8a a[KS][3];
+        auto readK = [&](int ks) {
+            const unsigned short* krow = knext + li * KP + ks * 16 + half * 8;
+#pragma unroll
+            for (int im = 0; im < 3; ++im) a[ks][im] = *reinterpret_cast<const bf16x8a*>(krow + im * KIMG);
+        };
+        readK(0);
+        if (KS > 1) readK(1);
+#pragma unroll
+        for (int j = 0; j < 6 * KS; ++j) {
+            int ks, at, bt;
+            if (j < 3 * KS) {
+                ks = j / 3;
+                at = j % 3 == 0 ? 1 : j % 3 == 1 ? 2 : 0;
+                bt = j % 3 == 0 ? 1 : j % 3 == 1 ? 0 : 2;
+                if (j % 3 == 0 && ks + 2 < KS) readK(ks + 2);
+            } else if (j < 5 * KS) {
+                ks = (j - 3 * KS) / 2;
+                at = (j - 3 * KS) % 2 == 0 ? 1 : 0;
+                bt = (j - 3 * KS) % 2 == 0 ? 0 : 1;
+                if (j == 3 * KS) readV(0);
+            } else {
+                ks = j - 5 * KS;
+                at = 0;
+                bt = 0;
+                if (j == 5 * KS) readV(1);
+            }
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks][at], qf[ks][bt], s, 0, 0, 0);
+            // 24 parts of the split over 6 KS MFMAs
+#pragma unroll
+            for (int c = (24 * j) / (6 * KS); c < (24 * (j + 1)) / (6 * KS); ++c) splitPart(c / 3, c % 3);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+        readV(0);
+        readV(1);
+#pragma unroll
+        for (int c = 0; c < 24; ++c) splitPart(c / 3, c % 3);
+    }
+
+    // stage two: O^T += V^T P^T of the current tile; maximum, exponentials and sum of the next one in 22 parts
+    float mx4[4], mrefNew = mref, psum = 0.0f;
+    bool moved = false;
+    auto softmaxPart = [&](int part) {
+        if (part < 4) {          // mask and maximum of four registers
+            if constexpr (MASKED) {
+#pragma unroll
+                for (int r = 4 * part; r < 4 * part + 4; ++r) {
+                    const int key = ktNext0 + dRow(r, half);
+                    s[r] = (key > myLimit || key >= totalLen) ? -INFINITY : s[r];
+                }
+            }
+            mx4[part] = fmaxf(fmaxf(s[4 * part], s[4 * part + 1]), fmaxf(s[4 * part + 2], s[4 * part + 3]));
+        } else if (part == 4) {  // row maximum; the reference moves when the maximum has outgrown it
+            float mx = fmaxf(fmaxf(mx4[0], mx4[1]), fmaxf(mx4[2], mx4[3]));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mrow = fmaxf(mrow, mx);
+            moved = mrow > mref + kRescaleThreshold;
+            mrefNew = moved ? mrow : mref;
+        } else if (part < 21) {  // one exponential
+            const int r = part - 5;
+            pc[r] = fastExp2(s[r] - mrefNew);
+            psum += pc[r];
+        }
+    };
+    constexpr int slots = 12 * DT;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+        for (int q = 0; q < 6 * DT; ++q) {
+            const int pr6 = q / DT, dt = q % DT;
+            const int regTerm = kSplitOrder[pr6][0], ldsTerm = kSplitOrder[pr6][1];
+            const int gi = 3 * st + (2 - ldsTerm);
+            const bool first = q == 0 || kSplitOrder[(q - 1) / DT][1] != ldsTerm;
+            if (first && gi + 2 < 6) readV(gi + 2);
+            acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tv[gi % 3][dt], __builtin_bit_cast(bf16x8a, pf[st][regTerm]), acc[dt], 0, 0, 0);
+            if constexpr (HAS_NEXT) {
+                const int n = st * 6 * DT + q;
+#pragma unroll
+                for (int c = (21 * n) / slots; c < (21 * (n + 1)) / slots; ++c) softmaxPart(c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if constexpr (HAS_NEXT) {
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {   // the products above used the old reference: rescale what they left
+            const float corr = moved ? fastExp2(mref - mrefNew) : 1.0f;
+            lrow *= corr;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+        }
+        mref = mrefNew;
+        lrow += psum;
+    }
+}
+
+template <int HDP, bool VEC4>
+__global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnForwardPipedKernel(AttnParams p) {
+    constexpr int BC = 32, KP = splitKeyPitch(HDP), VP = splitValuePitch(HDP), KTILE = 3 * BC * KP, VTILE = 3 * BC * VP, DT = HDP / 32, KS = HDP / 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned short smemSplit[];
+    unsigned short* ks = smemSplit;               // [2][3][BC][KP]
+    unsigned short* vs = smemSplit + 2 * KTILE;   // [2][3][BC][VP]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, qt;
+    decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const float* qb = p.q + size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const float* vb = p.v + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+
+    const int waveQ0 = qt * 128 + wave * 32;
+    const int i = waveQ0 + li;                    // this lane's query row
+    const bool rowValid = i < p.newLen;
+    // Q fragments: step ks of a lane in `half` holds head-dim elements 16 ks + 8 half + 0..7 of its query, scaled
+    bf16x8a qf[KS][3];
+    loadSplitFragments<HDP, VEC4>(qf, qb + size_t(i) * dim, p.scale * kLog2e, rowValid, hd, half);
+
+    float16v acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
+    float mrow = -INFINITY, mref = -INFINITY, lrow = 0.0f;
+
+    const int lastQuery = min(p.newLen, qt * 128 + 128) - 1;
+    const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);   // keys >= this are invisible to the tile
+    const int waveKeyEnd = p.oldLen + waveQ0 + 32;                       // keys >= this are invisible to the wave
+    const int myLimit = p.oldLen + i;                                    // last visible key of this lane's row
+    const int numKeyTiles = (blockKeyEnd + BC - 1) / BC;
+    const int waveTiles = min(numKeyTiles, (waveKeyEnd + BC - 1) / BC);  // the wave's tiles are the first waveTiles ones
+    auto maskedTile = [&](int t) { return (t * BC + BC - 1 > p.oldLen + waveQ0) || (t * BC + BC > p.totalLen); };
+
+    // K tiles 0 and 1 and V tile 0 to LDS; K tile 2 and V tile 1 on their way in registers
+    TileRegs<HDP, BC> kStage, vStage;
+    fetchHeadTile<HDP, BC, VEC4>(kStage, kb, dim, 0, p.totalLen, hd, tid);
+    fetchHeadTile<HDP, BC, VEC4>(vStage, vb, dim, 0, p.totalLen, hd, tid);
+    commitSplitTile<HDP, BC, KP>(ks, kStage, tid);
+    commitSplitTile<HDP, BC, VP>(vs, vStage, tid);
+    if (numKeyTiles > 1) {
+        fetchHeadTile<HDP, BC, VEC4>(kStage, kb, dim, BC, p.totalLen, hd, tid);
+        commitSplitTile<HDP, BC, KP>(ks + KTILE, kStage, tid);
+        fetchHeadTile<HDP, BC, VEC4>(vStage, vb, dim, BC, p.totalLen, hd, tid);
+    }
+    if (numKeyTiles > 2) fetchHeadTile<HDP, BC, VEC4>(kStage, kb, dim, 2 * BC, p.totalLen, hd, tid);
+    __syncthreads();
+    // the first tile's scores and probabilities (every wavefront has a first tile: key 0 is visible to every query)
+    float16v pc = forwardSplitScores<HDP>(ks, qf, lane);
+    if (maskedTile(0)) forwardFirstSoftmax<true>(pc, mrow, mref, lrow, 0, myLimit, p.totalLen, lane);
+    else forwardFirstSoftmax<false>(pc, mrow, mref, lrow, 0, myLimit, p.totalLen, lane);
+    __syncthreads();   // K tile 0's buffer is written again in the first step
+
+    int t = 0;
+    // the end of every tile's step: K tile t+2 and V tile t+1 go to LDS, the loads of K tile t+3 and V tile t+2 are issued
+    auto advance = [&]() {
+        if (t + 2 < numKeyTiles) commitSplitTile<HDP, BC, KP>(ks + (t & 1) * KTILE, kStage, tid);
+        if (t + 1 < numKeyTiles) commitSplitTile<HDP, BC, VP>(vs + ((t + 1) & 1) * VTILE, vStage, tid);
+        if (t + 3 < numKeyTiles) fetchHeadTile<HDP, BC, VEC4>(kStage, kb, dim, (t + 3) * BC, p.totalLen, hd, tid);
+        if (t + 2 < numKeyTiles) fetchHeadTile<HDP, BC, VEC4>(vStage, vb, dim, (t + 2) * BC, p.totalLen, hd, tid);
+        ++t;
+        __syncthreads();
+    };
+    for (; t + 1 < waveTiles && !maskedTile(t + 1); advance())
+        forwardPipedStep<HDP, false, true>(ks + ((t + 1) & 1) * KTILE, vs + (t & 1) * VTILE, qf, acc, pc, mrow, mref, lrow, (t + 1) * BC, myLimit, p.totalLen, lane);
+    for (; t + 1 < waveTiles; advance())
+        forwardPipedStep<HDP, true, true>(ks + ((t + 1) & 1) * KTILE, vs + (t & 1) * VTILE, qf, acc, pc, mrow, mref, lrow, (t + 1) * BC, myLimit, p.totalLen, lane);
+    forwardPipedStep<HDP, false, false>(nullptr, vs + (t & 1) * VTILE, qf, acc, pc, mrow, mref, lrow, 0, myLimit, p.totalLen, lane);
+    for (advance(); t < numKeyTiles; advance()) {}
+
+    lrow += __shfl_xor(lrow, 32, 64);
+    if (rowValid) {
+        if (p.out) storeTransposed<HDP, VEC4>(p.out + (size_t(b) * p.newLen + i) * dim + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
+        if (p.outImg) storeTransposedBf16<HDP, VEC4>(p.outImg + (size_t(b) * p.newLen + i) * p.imgLd + size_t(h) * hd, acc, hd, half, 1.0f / lrow);
+        if (half == 0) {
+            size_t idx = (size_t(b) * p.heads + h) * p.newLen + i;
+            p.m[idx] = mrow * kLn2;
+            p.l[idx] = lrow * fastExp2(mref - mrow);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 int paddedHeadDim(int hd) { return hd <= 32 ? 32 : hd <= 64 ? 64 : hd <= 128 ? 128 : 256; }
@@ -1747,8 +1840,8 @@ int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
     if constexpr (KIND == 0 && HDP <= 128) {
         if (gAttnRoute.load() & 1) {
             constexpr size_t splitBytes = size_t(2) * 3 * 32 * (splitKeyPitch(HDP) + splitValuePitch(HDP)) * sizeof(unsigned short);
-            return vec4 ? launchAttn(attnForwardSplitKernel<HDP, true>, splitBytes, grid, p, s)
-                        : launchAttn(attnForwardSplitKernel<HDP, false>, splitBytes, grid, p, s);
+            return vec4 ? launchAttn(attnForwardPipedKernel<HDP, true>, splitBytes, grid, p, s)
+                        : launchAttn(attnForwardPipedKernel<HDP, false>, splitBytes, grid, p, s);
         }
     }
     if constexpr (KIND == 0) {
