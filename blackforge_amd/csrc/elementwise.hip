@@ -174,6 +174,31 @@ __global__ void __launch_bounds__(256) biasKernel(const float* __restrict__ x, c
     }
 }
 
+// The same over four consecutive rows per thread (rows % 4 == 0, one row of threads per block): the bias is fetched
+// once for the four, and their loads are in flight together.
+template <int MODE, int ACT, bool NT>
+__global__ void __launch_bounds__(256) biasRows4Kernel(const float* __restrict__ x, const float* __restrict__ bias,
+                                                        const float* __restrict__ residual, float* __restrict__ out,
+                                                        size_t rows, size_t features) {
+    const size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+    if (col >= features) return;
+    const float4v b = loadf4(bias + col);
+    const size_t idx = size_t(blockIdx.y) * 4 * features + col;
+    float4v v[4], res[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        v[j] = ldf4<NT>(x + idx + j * features);
+        if constexpr (MODE == 2) res[j] = ldf4<NT>(residual + idx + j * features);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float4v y = v[j] + b;
+        if constexpr (MODE == 1) y = actF4<ACT>(y);
+        if constexpr (MODE == 2) y = y + res[j];
+        stf4<NT>(out + idx + j * features, y);
+    }
+}
+
 // Column sums, optionally fused with dGemm = dHidden * act'(gemm + bias) (FUSED = 1).
 // Each block reduces its rows per column in registers, then over threadIdx.y through LDS, and writes
 // one partial row per blockIdx.y; columnFinishKernel adds the partial rows in a fixed order.
@@ -427,7 +452,9 @@ int bf_hip_act_backward(const float* x, const float* g, float* out, size_t n, in
 #define BF_BIAS_LAUNCH(MODE, ACT)                                                                               \
     do {                                                                                                        \
         const bool nt = streamsPastCache(rows * features * (MODE == 2 ? 12 : 8));                               \
-        if (g.vec == 4 && nt)                                                                                   \
+        if (g.vec == 4 && nt && g.block.y == 1 && rows % 4 == 0 && rows / 4 <= 65535)                            \
+            biasRows4Kernel<MODE, ACT, true><<<dim3(g.grid.x, unsigned(rows / 4)), g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
+        else if (g.vec == 4 && nt)                                                                              \
             biasKernel<4, MODE, ACT, true><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
         else if (g.vec == 4)                                                                                    \
             biasKernel<4, MODE, ACT, false><<<g.grid, g.block, 0, asStream(stream)>>>(x, bias, residual, out, rows, features); \
