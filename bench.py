@@ -572,7 +572,10 @@ def main():
         "config": {"workload": "causal fused attention fwd+bwd, fp32 in and out, batch 8, heads 16, seq 2048, head_dim 64 "
                                "(BASELINE.json configs[2])", **res["shape"],
                    "route": "default: forward and dK/dV products as six bf16 MFMAs each on operands split into three bf16 terms "
-                            "(fp32 accuracy, fp32 accumulation); dQ on the fp32 MFMA"},
+                            "(fp32 accuracy, fp32 accumulation); dQ on the fp32 MFMA",
+                   "precision": "fp32 inputs, outputs, statistics and accumulation; every product keeps all term products above 2^-24 "
+                                "of it, and the parity tests hold this route to the same bounds against the CPU reference as the "
+                                "fp32-MFMA route (fp32_mfma_route below: the same step with every product on v_mfma_f32_32x32x2_f32)"},
         # `achieved` counts the algorithm's fp32 flops (8 hd per visible pair), priced against the fp32 MFMA peak, the
         # published peak of the arithmetic type the path computes; the kernel issues six bf16 MFMA flops for each of them,
         # and `bf16_pipe` prices those against the bf16 peak
