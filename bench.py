@@ -523,8 +523,9 @@ def extras_summary(extras):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=20, help="untimed steps first; the chip needs some 30 ms of work to reach its "
+                    "steady clocks (3 warm-up steps read 6 %% slower than 20)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the bandwidth kernels and the bf16 GEMMs")
     ap.add_argument("--no-graph", action="store_true", help="skip the recorded (HIP graph) variant of the tiny-LM step; for runs under a "
@@ -612,7 +613,7 @@ def main():
                                   bf, max(3, args.steps // 2), max(1, args.warmup // 2))
                               for name in args.train.split(",")}
     if not args.no_extras:
-        line["extras"] = bench_extras(bf, max(5, args.steps // 2))
+        line["extras"] = bench_extras(bf, min(10, max(5, args.steps // 2)))   # ten launches a kernel: what profiles/hbm_kernels_and_gemm.md describes
         line["extras_summary"] = extras_summary(line["extras"])
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_attention()
