@@ -125,7 +125,7 @@ def bench_attention(bf, steps, warmup):
         fp32 = {"forward_ms": time_region(bf, stream, fwd, steps, 2), "dkv_ms": time_region(bf, stream, dkv, steps, 1),
                 "step_ms": time_region(bf, stream, step, steps, 1)}
     finally:
-        call("bf_hip_attention_set_route", 3)
+        call("bf_hip_attention_set_route", 7)
     return {"ms_per_step": ms_step, "wall_ms_per_step": wall_ms, "kernel_ms": per, "flops": fl, "fp32_mfma_route": fp32,
             "shape": {"batch": batch, "heads": heads, "seq": seq, "head_dim": hd}}
 
@@ -572,8 +572,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "causal fused attention fwd+bwd, fp32 in and out, batch 8, heads 16, seq 2048, head_dim 64 "
                                "(BASELINE.json configs[2])", **res["shape"],
-                   "route": "default: forward and dK/dV products as six bf16 MFMAs each on operands split into three bf16 terms "
-                            "(fp32 accuracy, fp32 accumulation); dQ on the fp32 MFMA",
+                   "route": "default: every product (forward, dK/dV, dQ from the stored dS) as six bf16 MFMAs on operands split into "
+                            "three bf16 terms (fp32 accuracy, fp32 accumulation)",
                    "precision": "fp32 inputs, outputs, statistics and accumulation; every product keeps all term products above 2^-24 "
                                 "of it, and the parity tests hold this route to the same bounds against the CPU reference as the "
                                 "fp32-MFMA route (fp32_mfma_route below: the same step with every product on v_mfma_f32_32x32x2_f32)"},

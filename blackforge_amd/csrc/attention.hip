@@ -2,7 +2,8 @@
 // dK/dV, chosen by bf_hip_attention_set_route: every product on the fp32 MFMA (v_mfma_f32_32x32x2_f32; the kernels
 // described first), or, by default, every fp32 product as six bf16 MFMAs on operands split into three bf16 terms
 // (attnForwardPipedKernel, attnBackwardDkvSplitKernel, attnBackwardDkvPipedKernel further down; same ownership, tiling
-// and statistics, fp32 accuracy).  The dQ kernels run on the fp32 MFMA on both routes.
+// and statistics, fp32 accuracy), and likewise for the dQ kernel that reads the stored dS
+// (attnBackwardDqFromDsSplitKernel).  The dQ kernel that recomputes S and dP runs on the fp32 MFMA on both routes.
 //
 // Layout: q [batch,newLen,dim], k/v [batch,totalLen,dim], heads contiguous in dim.  Query row i
 // (absolute position oldLen+i) attends to keys j <= oldLen+i.
@@ -1516,6 +1517,141 @@ __global__ void __launch_bounds__(256, 1) attnBackwardDkvPipedKernel(AttnParams 
 }
 
 // ---------------------------------------------------------------------------------------------
+// dQ from stored dS on the split route: dQ^T += K^T dS^T with both operands as three bf16 terms.  K tiles (32 keys) are
+// split when they are written to LDS (images [3][32][pitch], read through the transposing LDS read as A operands: eight
+// consecutive keys per lane); a dS sub-block goes through the wave's LDS patch as in the fp32 kernel and is split in
+// registers (B operand: lane (query, half) holds keys 16 ks + 8 half + 0..7).  Several sub-blocks of the wave's row are
+// kept in flight in registers: the kernel is bound by that stream, which is why it gains less than the others.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ bf16x8a readTransposedNear(const unsigned short* p, int rowPitch) {
+    typedef __attribute__((address_space(3))) short4a* LdsPtr;
+    const short4a lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(p));
+    const short4a hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(p + 4 * rowPitch));
+    const short8a both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8a, both);
+}
+
+template <int HDP, bool VEC4>
+__global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnBackwardDqFromDsSplitKernel(AttnParams p) {
+    constexpr int DEPTH = HDP <= 64 ? 3 : 2;   // dS sub-blocks in flight per wavefront
+    constexpr int BC = 32, PITCH = splitValuePitch(HDP), IMG = BC * PITCH, KTILE = 3 * IMG, DT = HDP / 32;
+    extern __shared__ __attribute__((aligned(16))) unsigned short smemSplit[];
+    unsigned short* kimg = smemSplit;                                          // [2][3][BC][PITCH]
+    float* patches = reinterpret_cast<float*>(smemSplit + 2 * KTILE);          // [4][kDsPatch]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    int bh, qt;
+    decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
+    const int b = bh / p.heads, h = bh - b * p.heads;
+    const int hd = p.hd, dim = p.dim;
+    const size_t qOff = size_t(b) * p.newLen * dim + size_t(h) * hd;
+    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+
+    const int waveQ0 = qt * 128 + wave * 32;
+    const int i = waveQ0 + li;
+    // keys below waveKeyEnd are visible to some query of this wave's sub-block row (none if the row is past newLen)
+    const int waveKeyEnd = waveQ0 < p.newLen ? min(p.totalLen, p.oldLen + waveQ0 + 32) : 0;
+    const float* dsWave = p.ds + ((size_t(bh) * p.nqb + size_t(waveQ0 >> 5)) * p.nkb) * 1024 + lane * 4;
+    float* patch = patches + wave * kDsPatch;
+
+    // small term products in one accumulator, large ones in the other where the head dim alone gives too few independent chains
+    constexpr int NACC = DT >= 4 ? 1 : 2, SM = NACC - 1;
+    float16v acc[NACC][DT];
+#pragma unroll
+    for (int a = 0; a < NACC; ++a)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][dt][r] = 0.0f;
+
+    const int lastQuery = min(p.newLen, qt * 128 + 128) - 1;
+    const int blockKeyEnd = min(p.totalLen, p.oldLen + lastQuery + 1);
+    const int numKeyTiles = (blockKeyEnd + BC - 1) / BC;
+
+    float4v dsStage[DEPTH][4];
+    auto fetchDs = [&](int t, float4v (&dst)[4]) {
+        if (t * BC < waveKeyEnd) {
+            const float* src = dsWave + size_t(t) * 1024;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dst[j] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(src + j * 256));
+        }
+    };
+    const int fragRow = (lane >> 5) * 8 + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+
+    TileRegs<HDP, BC> kNext;
+    fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, 0, p.totalLen, hd, tid);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (d < numKeyTiles) fetchDs(d, dsStage[d]);
+    commitSplitTile<HDP, BC, PITCH>(kimg, kNext, tid);
+    if (numKeyTiles > 1) fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, BC, p.totalLen, hd, tid);
+    __syncthreads();
+    for (int t0 = 0; t0 < numKeyTiles; t0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int t = t0 + d;
+            if (t >= numKeyTiles) break;
+            const unsigned short* kcur = kimg + (t & 1) * KTILE;
+            const bool live = t * BC < waveKeyEnd;
+            bf16x8a b3[2][3];
+            if (live) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) storef4(patch + (8 * j + (lane >> 3)) * 36 + (lane & 7) * 4, dsStage[d][j]);
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    const float4v lo = loadf4(patch + li * 36 + ks * 16 + half * 8);
+                    const float4v hi = loadf4(patch + li * 36 + ks * 16 + half * 8 + 4);
+                    const float x[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                    splitOperand(x, b3[ks][0], b3[ks][1], b3[ks][2]);
+                }
+            }
+            if (t + DEPTH < numKeyTiles) fetchDs(t + DEPTH, dsStage[d]);
+            if (live) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    bf16x8a a3[DT][3];
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int im = 0; im < 3; ++im) a3[dt][im] = readTransposedNear(kcur + im * IMG + (ks * 16 + fragRow) * PITCH + dt * 32 + fragCol, PITCH);
+                    // (K term, dS term): consecutive MFMAs alternate accumulators
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        acc[SM][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[dt][1], b3[ks][1], acc[SM][dt], 0, 0, 0);
+                        acc[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[dt][0], b3[ks][0], acc[0][dt], 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        acc[SM][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[dt][2], b3[ks][0], acc[SM][dt], 0, 0, 0);
+                        acc[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[dt][1], b3[ks][0], acc[0][dt], 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        acc[SM][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[dt][0], b3[ks][2], acc[SM][dt], 0, 0, 0);
+                        acc[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a3[dt][0], b3[ks][1], acc[0][dt], 0, 0, 0);
+                    }
+                }
+            }
+            if (t + 1 < numKeyTiles) {
+                commitSplitTile<HDP, BC, PITCH>(kimg + ((t + 1) & 1) * KTILE, kNext, tid);
+                if (t + 2 < numKeyTiles) fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, (t + 2) * BC, p.totalLen, hd, tid);
+            }
+            __syncthreads();
+        }
+    }
+    if constexpr (NACC == 2) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[0][dt][r] += acc[SM][dt][r];
+    }
+    if (i < p.newLen) {
+        if (p.dQ) storeTransposed<HDP, VEC4>(p.dQ + qOff + size_t(i) * dim, acc[0], hd, half, p.scale);
+        if (p.dQImg) storeTransposedBf16<HDP, VEC4>(p.dQImg + (size_t(b) * p.newLen + i) * p.imgLd + size_t(h) * hd, acc[0], hd, half, p.scale);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // The forward kernel on the split route as a two-stage pipeline over key tiles (the scheme of the dK/dV pipeline
 // above).  While S^T of tile t+1 runs on the matrix pipe the vector unit splits P of tile t; while O^T += V^T P^T of
 // tile t runs, it takes the row maximum, the exponentials and the row sum of tile t+1.  One MFMA and one part of the
@@ -1830,8 +1966,8 @@ int launchDkv(const AttnParams& p, size_t smem, unsigned grid, hipStream_t s) {
     return launchAttn(attnBackwardDkvKernel<HDP, TILE, VEC4, 1, STORE>, smem, grid, p, s);
 }
 
-// bit 0: the forward kernel's products as six bf16 MFMAs each; bit 1: the dK/dV kernel's (head dims up to 128 both);
-// 0 = every product on the fp32 MFMA
+// bit 0: the forward kernel's products as six bf16 MFMAs each; bit 1: the dK/dV kernel's; bit 2: those of the dQ kernel
+// that reads the stored dS (head dims up to 128 all three); 0 = every product on the fp32 MFMA
 std::atomic<int> gAttnRoute{BF_ATTN_ROUTE_SPLIT};
 
 template <int KIND, int HDP, int TILE>
@@ -1851,6 +1987,13 @@ int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
         return vec4 ? launchAttn(attnBackwardDqKernel<HDP, TILE, true>, 2 * operandBytes, grid, p, s)
                     : launchAttn(attnBackwardDqKernel<HDP, TILE, false>, 2 * operandBytes, grid, p, s);
     } else if constexpr (KIND == 4) {
+        if constexpr (HDP <= 128) {
+            if (gAttnRoute.load() & BF_ATTN_ROUTE_SPLIT_DQ) {
+                constexpr size_t splitBytes = size_t(2) * 3 * 32 * splitValuePitch(HDP) * sizeof(unsigned short) + size_t(4) * kDsPatch * sizeof(float);
+                return vec4 ? launchAttn(attnBackwardDqFromDsSplitKernel<HDP, true>, splitBytes, grid, p, s)
+                            : launchAttn(attnBackwardDqFromDsSplitKernel<HDP, false>, splitBytes, grid, p, s);
+            }
+        }
         constexpr size_t need = operandBytes + size_t(4) * kDsPatch * sizeof(float);   // K tiles + a dS patch per wave
         // Three workgroups per CU pay once the grid keeps refilling them; a grid that fits in one round is better spread
         // two per CU, which asking for more LDS than needed (over a third of the CU's 160 KiB) enforces.

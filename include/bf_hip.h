@@ -413,12 +413,14 @@ int bf_hip_attention_set_workspace_limit(size_t bytes);
  * kernel has one form).  The SPLIT bits put a kernel's products on the bf16 matrix pipe at fp32 accuracy: each fp32
  * operand is the exact sum of three bf16 terms and each product six bf16 MFMAs (everything above 2^-24 of the product),
  * accumulated in fp32 in the order of the terms' sizes; head dims up to 128, larger ones stay on the fp32 MFMA
- * (v_mfma_f32_32x32x2_f32), which route 0 uses throughout.  The default is both bits: the two kernels then recompute
- * the same scores S, and the results are as close to a float64 evaluation as route 0's (the forward output closer).
- * With one bit alone the forward statistics (m, l) and the backward pass's S differ in the last bits, which a row
- * whose maximum drifts by hundreds shows as an error about 1.2 times route 0's.  The dQ kernels run on the fp32 MFMA
- * on every route. */
-enum { BF_ATTN_ROUTE_FP32_MFMA = 0, BF_ATTN_ROUTE_SPLIT_FORWARD = 1, BF_ATTN_ROUTE_SPLIT_DKV = 2, BF_ATTN_ROUTE_SPLIT = 3 };
+ * (v_mfma_f32_32x32x2_f32), which route 0 uses throughout.  The default is all three bits: the forward and dK/dV
+ * kernels then recompute the same scores S, and the results are as close to a float64 evaluation as route 0's (the
+ * forward output closer).  With the forward or the dK/dV bit alone the forward statistics (m, l) and the backward
+ * pass's S differ in the last bits, which a row whose maximum drifts by hundreds shows as an error about 1.2 times
+ * route 0's.  The DQ bit covers the kernel that forms dQ from the stored dS; the dQ kernel that recomputes S and dP
+ * (taken when the dS buffer would exceed the workspace limit) runs on the fp32 MFMA on every route. */
+enum { BF_ATTN_ROUTE_FP32_MFMA = 0, BF_ATTN_ROUTE_SPLIT_FORWARD = 1, BF_ATTN_ROUTE_SPLIT_DKV = 2, BF_ATTN_ROUTE_SPLIT_DQ = 4,
+       BF_ATTN_ROUTE_SPLIT = 7 };
 int bf_hip_attention_set_route(int route);
 int bf_hip_attention_backward_dkv_ds(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
                                      const float* D, float* dK, float* dV, float* dS, size_t batch, size_t heads,

@@ -294,12 +294,12 @@ def test_incremental_equals_full(hip, rng):
         assert_close(part, full[:, old:], what=f"oldLen={old}")
 
 
-# ---- the routes of bf_hip_attention_set_route: every test above runs on the default (forward and dK/dV products as six
-# ---- bf16 MFMAs on operands split into three bf16 terms); these run the others ----
-DEFAULT_ROUTE, FP32_ROUTE = 3, 0
+# ---- the routes of bf_hip_attention_set_route: every test above runs on the default (forward, dK/dV and dQ-from-dS
+# ---- products as six bf16 MFMAs on operands split into three bf16 terms); these run the others ----
+DEFAULT_ROUTE, FP32_ROUTE = 7, 0
 
 
-@pytest.fixture(params=[0, 1, 2], ids=["fp32-mfma", "split-forward-only", "split-dkv-only"])
+@pytest.fixture(params=[0, 1, 2, 4, 3], ids=["fp32-mfma", "split-forward-only", "split-dkv-only", "split-dq-only", "split-forward-and-dkv"])
 def other_route(hip, request):
     hip.capi.call("bf_hip_attention_set_route", request.param)
     yield request.param
@@ -322,7 +322,7 @@ def test_other_routes_match_the_oracle(hip, oracle, rng, other_route, batch, hea
 
 
 def test_route_argument(hip):
-    assert hip.capi.load().bf_hip_attention_set_route(4) != 0
+    assert hip.capi.load().bf_hip_attention_set_route(8) != 0
     assert hip.capi.load().bf_hip_attention_set_route(-1) != 0
     hip.capi.call("bf_hip_attention_set_route", DEFAULT_ROUTE)
 
