@@ -34,11 +34,11 @@ PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
 
 # HBM bytes per launch of the dominant kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this workload,
-# each scaled by what the same counter reads for a plain 256 MiB copy (x2.000 and x1.000): 992 MB read +
-# 1225 MB written (1095 MB of that is the dS hand-over; the read side moves between 0.6 and 1.0 GB from run to run
+# each scaled by what the same counter reads for a plain 256 MiB copy (x2.000 and x1.000): 979 MB read +
+# 1224 MB written (1095 MB of that is the dS hand-over; the read side moves between 0.6 and 1.0 GB from run to run
 # with what the L2s happen to keep).  profiles/attention_c3_kernel_trace.md holds the commands
 # and the raw counter values.
-MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvPipedKernel": 2216655490}
+MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvPipedKernel": 2203713462}
 
 
 def attention_flops(batch, heads, seq, hd):
