@@ -34,10 +34,11 @@ def run_gpu(hip, q, k, v, go, heads, scale, old_len):
     return [t.toHost() for t in (fwd.output, fwd.m, fwd.l, grad.dQ, grad.dK, grad.dV)]
 
 
-# (batch, heads, newLen, oldLen, headDim): tiny, ragged, every padded head-dim class, incremental decode
+# (batch, heads, newLen, oldLen, headDim): tiny, ragged, every padded head-dim class, incremental decode, head dims
+# that are not multiples of four (element-wise loads) in every class
 CASES = [(1, 1, 1, 0, 2), (1, 2, 3, 0, 2), (2, 2, 5, 0, 4), (2, 3, 33, 0, 32), (1, 2, 70, 0, 64), (1, 1, 40, 0, 128),
          (1, 1, 37, 0, 256), (2, 2, 3, 9, 16), (1, 2, 1, 37, 32), (1, 2, 129, 0, 64), (1, 1, 200, 57, 40), (2, 1, 130, 130, 8),
-         (1, 4, 256, 0, 32), (1, 2, 300, 0, 100), (1, 1, 64, 0, 7)]
+         (1, 4, 256, 0, 32), (1, 2, 300, 0, 100), (1, 1, 64, 0, 7), (1, 2, 70, 5, 62), (1, 1, 45, 0, 126)]
 
 
 @pytest.mark.parametrize("batch,heads,new_len,old_len,hd", CASES)
