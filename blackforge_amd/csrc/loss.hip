@@ -79,13 +79,16 @@ __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pr
 
 // SPARSE: target holds one class index per row.  Otherwise a dense target row.
 // SHIFTED (with VEC = 4, CACHED): rows of any length and alignment through 16-byte accesses (RowCache::loadShifted).
-template <int G, int MAXE, int VEC, bool CACHED, bool SPARSE, bool SHIFTED = false, bool NT = false>
+// AHEAD (CACHED only): a grid that fills the chip walks the rows, each block with its next row's loads in flight
+// (requested into a second set of registers before the current row is reduced).  Otherwise one block per group of rows.
+template <int G, int MAXE, int VEC, bool CACHED, bool SPARSE, bool SHIFTED = false, bool NT = false, bool AHEAD = false>
 __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const float* __restrict__ logits,
                                                                          const float* __restrict__ target,
                                                                          float* __restrict__ grad, float* __restrict__ rowLoss,
                                                                          size_t rows, size_t classes, float invRows,
                                                                          const float* __restrict__ maskInfo,
                                                                          unsigned short* __restrict__ gradImage) {
+    static_assert(CACHED || !AHEAD, "only rows held in registers are fetched ahead");
     __shared__ float lds[16];
     const int t = threadIdx.x % G;
     const size_t rowsPerBlock = blockDim.x / G;
@@ -93,29 +96,29 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
     // masked form (sparse targets only): maskInfo[1] = 1 / (number of rows whose index is not -1) replaces 1 / rows,
     // and a row with index -1 contributes nothing: zero gradient, zero loss
     if (SPARSE && maskInfo != nullptr) invRows = maskInfo[1];
-    // Rows that leave room for a second copy in registers (MAXE <= 32) run on a grid of two waves of blocks per SIMD that
-    // walks the rows: the next row's loads are issued before the current row is reduced, so they are in flight during
-    // its two block-wide reductions and its stores (8192 x 32000: 0.405 -> 0.367 ms together with the streaming hint).
-    constexpr bool AHEAD = CACHED && MAXE <= 32;
+    using Row = RowCache<G, MAXE, VEC, NT>;
     RowCache<G, AHEAD ? MAXE : VEC, VEC, NT> ahead;
     const size_t firstRow = size_t(blockIdx.x) * rowsPerBlock + threadIdx.x / G;
+    // the loads only: a shifted row is masked (Row::maskShifted) where it is first used, so that a row fetched ahead
+    // is not waited for here
     auto fetch = [&](auto& into, size_t r) __attribute__((always_inline)) {
         const float* src = logits + r * classes;
-        if constexpr (SHIFTED) into.loadShifted(src, classes, t, -INFINITY, RowCache<G, MAXE, VEC, NT>::shiftOf(src));
+        if constexpr (SHIFTED) into.template issueShifted<0, MAXE / VEC>(src, classes, t, Row::shiftOf(src));
         else into.load(src, classes, t, -INFINITY);
     };
     if constexpr (AHEAD) { if (firstRow < rows) fetch(ahead, firstRow); }
     for (size_t row = firstRow; row < rows; row += rowStep) {
         const float* x = logits + row * classes;
         float* gOut = grad + row * classes;
-        RowCache<G, MAXE, VEC, NT> c;
+        Row c;
         if constexpr (AHEAD) {
             c = ahead;
             if (row + rowStep < rows) fetch(ahead, row + rowStep);
         } else if constexpr (CACHED) {
             fetch(c, row);
         }
-        const int shift = SHIFTED ? RowCache<G, MAXE, VEC, NT>::shiftOf(x) : 0;   // the same for gOut: the host checks that
+        const int shift = SHIFTED ? Row::shiftOf(x) : 0;   // the same for gOut: the host checks that
+        if constexpr (CACHED && SHIFTED) c.maskShifted(classes, t, -INFINITY, shift);
         // gradImage (aligned rows only; the host checks): the gradient row rounded to bf16, for the bf16 GEMMs that consume it
         unsigned short* gImg = gradImage ? gradImage + row * classes : nullptr;
         auto storeRow = [&]() __attribute__((always_inline)) {
@@ -151,8 +154,9 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
         constexpr float kLog2e = 1.4426950408889634f;
         float sum = 0.0f;
         if constexpr (CACHED) {
+            const float top = mx * kLog2e;   // one fused multiply-add per element; its rounding is common to the row and cancels in p
 #pragma unroll
-            for (int i = 0; i < MAXE; ++i) { c.r[i] = __builtin_amdgcn_exp2f((c.r[i] - mx) * kLog2e); sum += c.r[i]; }
+            for (int i = 0; i < MAXE; ++i) { c.r[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(c.r[i], kLog2e, -top)); sum += c.r[i]; }
         } else {
             for (size_t e = t; e < classes; e += G) sum += __builtin_amdgcn_exp2f((x[e] - mx) * kLog2e);
         }
@@ -165,16 +169,29 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
             const unsigned cls = unsigned(lroundf(target[row]));
             float pTarget = -1.0f;
             if constexpr (CACHED) {
+                // Element e of the row sits at position e + shift of the held row: iteration pos / (G * VEC), thread
+                // (pos / VEC) % G, slot pos % VEC.  Only the iteration that holds the target looks for it (the same
+                // for the whole group), every other element is one multiplication.
+                const unsigned pos = cls + unsigned(shift);
+                const int targetIt = cls < classes ? int(pos / unsigned(G * VEC)) : -1;
+                const bool mine = int((pos / VEC) % G) == t;
+                const int targetSlot = int(pos % VEC);
+                const float scale = inv * invRows;
 #pragma unroll
-                for (int it = 0; it < MAXE / VEC; ++it)
+                for (int it = 0; it < MAXE / VEC; ++it) {
+                    if (it == targetIt) {
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) {
-                        const int idx = int(it * G + t) * VEC + j - shift;   // |.| < G * MAXE + 4 <= 65540
-                        const float p = c.r[it * VEC + j] * inv;
-                        const bool hit = idx == int(cls);                    // cls < classes <= G * MAXE
-                        pTarget = hit ? p : pTarget;
-                        c.r[it * VEC + j] = (p - (hit ? 1.0f : 0.0f)) * invRows;
+                        for (int j = 0; j < VEC; ++j) {
+                            const bool hit = mine && j == targetSlot;
+                            const float p = c.r[it * VEC + j] * inv;
+                            pTarget = hit ? p : pTarget;
+                            c.r[it * VEC + j] = hit ? (p - 1.0f) * invRows : c.r[it * VEC + j] * scale;
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) c.r[it * VEC + j] *= scale;
                     }
+                }
                 storeRow();
             } else {
                 for (size_t e = t; e < classes; e += G) {
@@ -200,7 +217,7 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                 for (int it = 0; it < MAXE / VEC; ++it)
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) {
-                        const long idx = long(RowCache<G, MAXE, VEC, NT>::index(it, t, j)) - shift;
+                        const long idx = long(Row::index(it, t, j)) - shift;
                         if (idx >= 0 && size_t(idx) < classes) c.r[it * VEC + j] = emit(c.r[it * VEC + j], size_t(idx));
                     }
                 storeRow();
@@ -237,21 +254,25 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
     // row sit at the same offset within a 16-byte group; a row must then fit its registers with up to 3 elements to spare
     const bool shifted = !vec4 && ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad)) & 15u) == 0;
     const bool streaming = streamsPastCache(rows * classes * (SPARSE ? 8 : 12));   // logits in, gradient out (and a dense target in)
-    // smallest group and register count that hold a row (see the row kernels); a block takes its rows once
-#define BF_CE(G, MAXE)                                                                                            \
+    // smallest group and register count that hold a row (see the row kernels)
+    // AHEAD as measured (8 B per logit over the launch, 16-byte aligned rows): rows of up to 8192 classes are faster
+    // one block per group of rows (65536 x 2048: 5.4 against 4.9 TB/s walking, 16384 x 4096: 5.9 against 5.3), 16384
+    // classes the same either way, 32000 faster walking (5.9 against 5.4-5.7), and rows past 32768, which leave no
+    // registers for a second row, no faster with part of one fetched ahead on half the wavefronts
+#define BF_CE(G, MAXE, AHEAD)                                                                                     \
     if (classes + (vec4 ? 0 : 3) <= size_t(G) * MAXE && (vec4 || shifted || MAXE <= 32)) {                        \
         const unsigned threads = G > 256 ? G : 256;                                                               \
-        const bool nt = streaming && MAXE <= 32;   /* measured: the hint only pays together with the look-ahead */ \
-        const unsigned grid = gridFor(rows, threads / G, MAXE <= 32 ? unsigned(computeUnits()) * (2048 / threads) : kMaxGridX); \
-        if (vec4 && nt) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
-        else if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
-        else if (shifted && nt) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
-        else if (shifted) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
-        else crossEntropyKernel<G, (MAXE <= 32 ? MAXE : 4), 1, true, SPARSE><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); /* plans above 32 registers have no one-element form */ \
+        const unsigned grid = gridFor(rows, threads / G, AHEAD ? unsigned(computeUnits()) * (2048 / threads) : kMaxGridX); \
+        if (vec4 && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
+        else if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
+        else if (shifted && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
+        else if (shifted) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
+        else crossEntropyKernel<G, (MAXE <= 32 ? MAXE : 4), 1, true, SPARSE, false, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); /* plans above 32 registers have no one-element form */ \
         break;                                                                                                    \
     }
     do {
-        BF_CE(64, 4) BF_CE(64, 8) BF_CE(64, 16) BF_CE(256, 8) BF_CE(256, 16) BF_CE(256, 32) BF_CE(1024, 16) BF_CE(1024, 32) BF_CE(1024, 52)
+        BF_CE(64, 4, false) BF_CE(64, 8, false) BF_CE(64, 16, false) BF_CE(256, 8, false) BF_CE(256, 16, false) BF_CE(256, 32, false)
+        BF_CE(1024, 16, true) BF_CE(1024, 32, true) BF_CE(1024, 52, false)
         crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage);
     } while (0);
 #undef BF_CE

@@ -27,8 +27,15 @@ struct RowCache {
     __device__ static size_t index(int it, int t, int j) { return (size_t(it) * G + t) * VEC + j; }
 
     __device__ __forceinline__ void load(const float* __restrict__ row, size_t features, int t, float fill) {
+        issue<0, kIters>(row, features, t, fill);
+    }
+
+    // Iterations [B, E) of the row only: a kernel that walks rows issues the next row's loads in pieces, as registers
+    // come free.
+    template <int B, int E>
+    __device__ __forceinline__ void issue(const float* __restrict__ row, size_t features, int t, float fill) {
 #pragma unroll
-        for (int it = 0; it < kIters; ++it) {
+        for (int it = B; it < E; ++it) {
             size_t e = index(it, t, 0);
             if constexpr (VEC == 4) {
                 if (e < features) {
@@ -49,17 +56,29 @@ struct RowCache {
     // Rows are shorter than 2^31 - 4 elements here (G * MAXE elements at most), so 32-bit indices do.  Only the group
     // that holds the row's first element (thread 0, iteration 0) and the one that holds its last need any masking.
     __device__ __forceinline__ void loadShifted(const float* __restrict__ row, size_t features, int t, float fill, int shift) {
+        // every load first (a group past the row's end re-reads group 0 instead of branching), the masking afterwards:
+        // code between the loads that touches a loaded register would make each load wait for the one before it
+        issueShifted<0, kIters>(row, features, t, shift);
+        maskShifted(features, t, fill, shift);
+    }
+
+    // The loads of iterations [B, E) of a shifted row, unmasked: maskShifted (with the same row's shift) comes before
+    // the first use, and is the first thing that waits for the loads.
+    template <int B, int E>
+    __device__ __forceinline__ void issueShifted(const float* __restrict__ row, size_t features, int t, int shift) {
         static_assert(VEC == 4, "shifted access is 4 wide");
         const float* base = row - shift;
         const int last = int(features) + shift;   // one past the row's last element, counted from base
-        // every load first (a group past the row's end re-reads group 0 instead of branching), the masking afterwards:
-        // code between the loads that touches a loaded register would make each load wait for the one before it
 #pragma unroll
-        for (int it = 0; it < kIters; ++it) {
+        for (int it = B; it < E; ++it) {
             const int g = (it * G + t) * 4;
             const float4v v = ldf4<NT>(base + (g < last ? g : 0));
             r[it * 4 + 0] = v.x; r[it * 4 + 1] = v.y; r[it * 4 + 2] = v.z; r[it * 4 + 3] = v.w;
         }
+    }
+
+    __device__ __forceinline__ void maskShifted(size_t features, int t, float fill, int shift) {
+        const int last = int(features) + shift;
         const int lo = t == 0 ? shift : 0;   // slots of thread 0's first group that belong to the row before
 #pragma unroll
         for (int it = 0; it < kIters; ++it) {
