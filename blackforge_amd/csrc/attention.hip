@@ -987,10 +987,11 @@ __device__ __forceinline__ void dkvSplitTile(const unsigned short* __restrict__ 
                                              int key, bool keyValid, int oldLen, int lane, float* __restrict__ dsLane, int newLen) {
     constexpr int QP = splitKeyPitch(HDP), IMG = 32 * QP, DT = HDP / 32, KS = HDP / 16;
     const int half = lane >> 5, li = lane & 31;
-    // S = Q K^T in three accumulator chains by magnitude (see the forward kernel), dP = dO V^T in two
-    float16v s0, s1, s2, p0, p1;
+    // S = Q K^T and dP = dO V^T in two accumulator chains each: the products of the two high terms, and everything
+    // smaller (at most 2^-7 of the first), whose own rounding is then far below the first chain's
+    float16v s0, s1, p0, p1;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; s2[r] = 0.0f; p0[r] = 0.0f; p1[r] = 0.0f; }
+    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; p0[r] = 0.0f; p1[r] = 0.0f; }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const unsigned short* qrow = qimg + li * QP + ks * 16 + half * 8;
@@ -1001,18 +1002,18 @@ __device__ __forceinline__ void dkvSplitTile(const unsigned short* __restrict__ 
             a[im] = *reinterpret_cast<const bf16x8a*>(qrow + im * IMG);
             g[im] = *reinterpret_cast<const bf16x8a*>(grow + im * IMG);
         }
-        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], kf[ks][1], s2, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], kf[ks][1], s1, 0, 0, 0);
         p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[1], vf[ks][1], p1, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], kf[ks][0], s1, 0, 0, 0);
-        p0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[1], vf[ks][0], p0, 0, 0, 0);
-        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], kf[ks][0], s2, 0, 0, 0);
-        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[2], vf[ks][0], p1, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kf[ks][1], s1, 0, 0, 0);
-        p0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[0], vf[ks][1], p0, 0, 0, 0);
-        s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kf[ks][2], s2, 0, 0, 0);
-        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[0], vf[ks][2], p1, 0, 0, 0);
         s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kf[ks][0], s0, 0, 0, 0);
         p0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[0], vf[ks][0], p0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], kf[ks][0], s1, 0, 0, 0);
+        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[2], vf[ks][0], p1, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kf[ks][2], s1, 0, 0, 0);
+        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[0], vf[ks][2], p1, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], kf[ks][0], s1, 0, 0, 0);
+        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[1], vf[ks][0], p1, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], kf[ks][1], s1, 0, 0, 0);
+        p1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(g[0], vf[ks][1], p1, 0, 0, 0);
     }
     // register r: query = qt0 + dRow(r, half), key = this lane's key
     float16v pr, dsv;
@@ -1023,13 +1024,13 @@ __device__ __forceinline__ void dkvSplitTile(const unsigned short* __restrict__ 
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const int r = 4 * g + c;
-            float prob = fastExp2(((s2[r] + s1[r]) + s0[r]) - lse4[c]);
+            float prob = fastExp2((s1[r] + s0[r]) - lse4[c]);
             if constexpr (MASKED) {
                 const int qi = qt0 + dRow(r, half);
                 prob = (key > oldLen + qi || !keyValid) ? 0.0f : prob;
             }
             pr[r] = prob;                                      // P
-            dsv[r] = prob * ((p0[r] + p1[r]) - d4[c]);         // dS (without the scale factor)
+            dsv[r] = prob * ((p1[r] + p0[r]) - d4[c]);         // dS (without the scale factor)
         }
     }
     if constexpr (STORE) {
@@ -1051,21 +1052,27 @@ __device__ __forceinline__ void dkvSplitTile(const unsigned short* __restrict__ 
             splitOperand(x, pf[0], pf[1], pf[2]);
             splitOperand(y, df[0], df[1], df[2]);
         }
-        bf16x8a gfr[DT][3], qfr[DT][3];
+        // two 32-wide blocks of the head dim at a time: four accumulator chains alternate, and twelve operand fragments
+        // are live instead of six per block of the head dim
+        constexpr int DG = DT >= 2 ? 2 : 1;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+        for (int d0 = 0; d0 < DT; d0 += DG) {
+            bf16x8a gfr[DG][3], qfr[DG][3];
 #pragma unroll
-            for (int im = 0; im < 3; ++im) {
-                gfr[dt][im] = readTransposedApart(gimg + im * IMG + (16 * st + fragRow) * QP + dt * 32 + fragCol, QP);
-                qfr[dt][im] = readTransposedApart(qimg + im * IMG + (16 * st + fragRow) * QP + dt * 32 + fragCol, QP);
-            }
+            for (int dt = 0; dt < DG; ++dt)
 #pragma unroll
-        for (int pr6 = 0; pr6 < 6; ++pr6)
+                for (int im = 0; im < 3; ++im) {
+                    gfr[dt][im] = readTransposedApart(gimg + im * IMG + (16 * st + fragRow) * QP + (d0 + dt) * 32 + fragCol, QP);
+                    qfr[dt][im] = readTransposedApart(qimg + im * IMG + (16 * st + fragRow) * QP + (d0 + dt) * 32 + fragCol, QP);
+                }
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[order[pr6][0]], gfr[dt][order[pr6][1]], dv[dt], 0, 0, 0);
-                dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(df[order[pr6][0]], qfr[dt][order[pr6][1]], dk[dt], 0, 0, 0);
-            }
+            for (int pr6 = 0; pr6 < 6; ++pr6)
+#pragma unroll
+                for (int dt = 0; dt < DG; ++dt) {
+                    dv[d0 + dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[order[pr6][0]], gfr[dt][order[pr6][1]], dv[d0 + dt], 0, 0, 0);
+                    dk[d0 + dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(df[order[pr6][0]], qfr[dt][order[pr6][1]], dk[d0 + dt], 0, 0, 0);
+                }
+        }
     }
 }
 
@@ -1138,51 +1145,45 @@ __global__ void __launch_bounds__(256, 1) attnBackwardDkvSplitKernel(AttnParams 
     float* const dsColumn = STORE ? p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024 : nullptr;   // wave-uniform
     const int dsLaneOffset = half * 128 + li;
 
-    // tiles are short: the loads of a tile are issued two tiles before it is written to LDS (two register stages)
-    TileRegs<HDP, BQ> qStage[2], gStage[2];
-    float statStage[2] = {0.0f, 0.0f};
-    auto fetchAll = [&](int qt0, TileRegs<HDP, BQ>& qr, TileRegs<HDP, BQ>& gr, float& st) {
-        fetchHeadTile<HDP, BQ, VEC4>(qr, p.q + qOff, dim, qt0, p.newLen, hd, tid);
-        fetchHeadTile<HDP, BQ, VEC4>(gr, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+    // a tile's loads are issued one tile before it is written to LDS and two before it is read
+    TileRegs<HDP, BQ> qStage, gStage;
+    float statStage = 0.0f;
+    auto fetchAll = [&](int qt0) {
+        fetchHeadTile<HDP, BQ, VEC4>(qStage, p.q + qOff, dim, qt0, p.newLen, hd, tid);
+        fetchHeadTile<HDP, BQ, VEC4>(gStage, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
         const int j = tid < BQ ? tid : tid - BQ;
         const int qi = qt0 + j;
-        if (tid < BQ) st = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
-        else if (tid < 2 * BQ) st = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
+        if (tid < BQ) statStage = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
+        else if (tid < 2 * BQ) statStage = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
     };
-    auto commitAll = [&](int buf, const TileRegs<HDP, BQ>& qr, const TileRegs<HDP, BQ>& gr, float st) {
-        commitSplitTile<HDP, BQ, QP>(qs + buf * TILE, qr, tid);
-        commitSplitTile<HDP, BQ, QP>(gs + buf * TILE, gr, tid);
-        if (tid < 2 * BQ) stats[buf * 2 * BQ + tid] = st;
+    auto commitAll = [&](int buf) {
+        commitSplitTile<HDP, BQ, QP>(qs + buf * TILE, qStage, tid);
+        commitSplitTile<HDP, BQ, QP>(gs + buf * TILE, gStage, tid);
+        if (tid < 2 * BQ) stats[buf * 2 * BQ + tid] = statStage;
     };
     if (numQTiles > 0) {
-        fetchAll(q0Start, qStage[0], gStage[0], statStage[0]);
-        if (numQTiles > 1) fetchAll(q0Start + BQ, qStage[1], gStage[1], statStage[1]);
-        commitAll(0, qStage[0], gStage[0], statStage[0]);
-        if (numQTiles > 2) fetchAll(q0Start + 2 * BQ, qStage[0], gStage[0], statStage[0]);
+        fetchAll(q0Start);
+        commitAll(0);
+        if (numQTiles > 1) fetchAll(q0Start + BQ);
     }
     __syncthreads();
-    for (int t0 = 0; t0 < numQTiles; t0 += 2) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int t = t0 + u;
-            if (t >= numQTiles) break;
-            const int qt0 = q0Start + t * BQ;
-            // the wave's keys [waveK0, waveK0+32) are visible to some query of the tile?
-            if (p.oldLen + qt0 + BQ - 1 >= waveK0 && waveK0 < p.totalLen) {
-                const bool masked = (waveK0 + 31 > p.oldLen + qt0) || (waveK0 + 32 > p.totalLen);
-                const unsigned short* qcur = qs + u * TILE;
-                const unsigned short* gcur = gs + u * TILE;
-                const float* scur = stats + u * 2 * BQ;
-                float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
-                if (masked) dkvSplitTile<HDP, true, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane, p.newLen);
-                else dkvSplitTile<HDP, false, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane, p.newLen);
-            }
-            if (t + 1 < numQTiles) {
-                commitAll(u ^ 1, qStage[u ^ 1], gStage[u ^ 1], statStage[u ^ 1]);
-                if (t + 3 < numQTiles) fetchAll(qt0 + 3 * BQ, qStage[u ^ 1], gStage[u ^ 1], statStage[u ^ 1]);
-            }
-            __syncthreads();
+    for (int t = 0; t < numQTiles; ++t) {
+        const int qt0 = q0Start + t * BQ, u = t & 1;
+        // the wave's keys [waveK0, waveK0+32) are visible to some query of the tile?
+        if (p.oldLen + qt0 + BQ - 1 >= waveK0 && waveK0 < p.totalLen) {
+            const bool masked = (waveK0 + 31 > p.oldLen + qt0) || (waveK0 + 32 > p.totalLen);
+            const unsigned short* qcur = qs + u * TILE;
+            const unsigned short* gcur = gs + u * TILE;
+            const float* scur = stats + u * 2 * BQ;
+            float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
+            if (masked) dkvSplitTile<HDP, true, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane, p.newLen);
+            else dkvSplitTile<HDP, false, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane, p.newLen);
         }
+        if (t + 1 < numQTiles) {
+            commitAll(u ^ 1);
+            if (t + 2 < numQTiles) fetchAll(qt0 + 2 * BQ);
+        }
+        __syncthreads();
     }
     storeKeyGradients<HDP>(p, dk, dv, b, h, waveK0, kOff, half, li);
 }
@@ -2007,10 +2008,11 @@ int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
                     constexpr size_t pipedBytes = size_t(6) * 3 * 32 * splitKeyPitch(HDP) * sizeof(unsigned short) + size_t(3) * 64 * sizeof(float);
                     return vec4 ? launchAttn(attnBackwardDkvPipedKernel<HDP, true, KIND == 3>, pipedBytes, grid, p, s)
                                 : launchAttn(attnBackwardDkvPipedKernel<HDP, false, KIND == 3>, pipedBytes, grid, p, s);
+                } else {
+                    constexpr size_t splitBytes = size_t(4) * 3 * 32 * splitKeyPitch(HDP) * sizeof(unsigned short) + size_t(2) * 64 * sizeof(float);
+                    return vec4 ? launchAttn(attnBackwardDkvSplitKernel<HDP, true, KIND == 3>, splitBytes, grid, p, s)
+                                : launchAttn(attnBackwardDkvSplitKernel<HDP, false, KIND == 3>, splitBytes, grid, p, s);
                 }
-                constexpr size_t splitBytes = size_t(4) * 3 * 32 * splitKeyPitch(HDP) * sizeof(unsigned short) + size_t(2) * 64 * sizeof(float);
-                return vec4 ? launchAttn(attnBackwardDkvSplitKernel<HDP, true, KIND == 3>, splitBytes, grid, p, s)
-                            : launchAttn(attnBackwardDkvSplitKernel<HDP, false, KIND == 3>, splitBytes, grid, p, s);
             }
         }
         constexpr size_t smem = 2 * operandBytes + 4 * TILE * sizeof(float);
