@@ -984,7 +984,7 @@ template <int HDP, bool MASKED, bool STORE>
 __device__ __forceinline__ void dkvSplitTile(const unsigned short* __restrict__ qimg, const unsigned short* __restrict__ gimg,
                                              const float* __restrict__ stats, const bf16x8a (&kf)[HDP / 16][3],
                                              const bf16x8a (&vf)[HDP / 16][3], float16v (&dk)[HDP / 32], float16v (&dv)[HDP / 32], int qt0,
-                                             int key, bool keyValid, int oldLen, int lane, float* __restrict__ dsLane, int newLen) {
+                                             int key, bool keyValid, int oldLen, int lane, float* __restrict__ dsLane) {
     constexpr int QP = splitKeyPitch(HDP), IMG = 32 * QP, DT = HDP / 32, KS = HDP / 16;
     const int half = lane >> 5, li = lane & 31;
     // S = Q K^T and dP = dO V^T in two accumulator chains each: the products of the two high terms, and everything
@@ -1033,11 +1033,10 @@ __device__ __forceinline__ void dkvSplitTile(const unsigned short* __restrict__ 
             dsv[r] = prob * ((p1[r] + p0[r]) - d4[c]);         // dS (without the scale factor)
         }
     }
-    if constexpr (STORE) {
-        if (qt0 < newLen) {   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave
+    if constexpr (STORE) {   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave (every tile a caller
+                             // passes starts inside the sequence, and the buffer holds whole sub-blocks)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(dsv[r], dsLane + (8 * (r >> 2) + (r & 3)) * 32);
-        }
+        for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(dsv[r], dsLane + (8 * (r >> 2) + (r & 3)) * 32);
     }
     // dV += P^T dO, dK += dS^T Q: step st contracts over queries 16 st + 8 (e / 4) + 4 half + e % 4 = registers 8 st + e
     const int fragRow = 4 * (lane >> 5) + ((lane & 15) >> 2), fragCol = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
@@ -1176,8 +1175,8 @@ __global__ void __launch_bounds__(256, 1) attnBackwardDkvSplitKernel(AttnParams 
             const unsigned short* gcur = gs + u * TILE;
             const float* scur = stats + u * 2 * BQ;
             float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
-            if (masked) dkvSplitTile<HDP, true, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane, p.newLen);
-            else dkvSplitTile<HDP, false, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane, p.newLen);
+            if (masked) dkvSplitTile<HDP, true, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane);
+            else dkvSplitTile<HDP, false, STORE>(qcur, gcur, scur, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane, dsLane);
         }
         if (t + 1 < numQTiles) {
             commitAll(u ^ 1);
@@ -1499,7 +1498,7 @@ __global__ void __launch_bounds__(256, 1) attnBackwardDkvPipedKernel(AttnParams 
         if (visible) {
             float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
             dkvSplitTile<HDP, true, STORE>(qs + cur * TILE, gs + cur * TILE, stats + cur * 2 * BQ, kf, vf, dk, dv, qt0, key, keyValid, p.oldLen, lane,
-                                           dsLane, p.newLen);
+                                           dsLane);
         }
     }
     if (t == numQTiles) {   // no unmasked tile; the stores appear on both paths so that neither loop copies registers for the other
