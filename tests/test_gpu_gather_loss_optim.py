@@ -131,6 +131,25 @@ def test_cross_entropy(hip, oracle, rng, rows, classes):
         assert_close(res.grad.toHost(), eg, what="dense CE grad")
 
 
+@pytest.mark.parametrize("classes", [37, 1000, 4099, 16384, 32000, 32003, 50257])
+def test_cross_entropy_target_at_every_kind_of_position(hip, oracle, rng, classes):
+    """The target class at the ends of the row and either side of every boundary the kernel's layouts have (16-byte
+    groups, wavefronts, 256- and 1024-thread iterations), on rows of every alignment (odd class counts shift each row
+    by a different amount): the one element whose gradient is (p - 1) / rows must be exactly that one."""
+    D, ops = hip.DeviceTensor, hip.ops
+    marks = [0, 1, 3, 4, 5, 63, 64, 255, 256, 257, 1023, 1024, 1027, 4095, 4096, 4097, 16383, 16384, 32767, 32768, 32771,
+             classes // 2, classes - 5, classes - 4, classes - 2, classes - 1]
+    idx = np.array(sorted({m for m in marks if 0 <= m < classes}))
+    rows = len(idx)
+    logits = r(rng, rows, classes, scale=3)
+    res = ops.softmaxCrossEntropySparse(D.fromHost(logits), D.fromHost(idx.astype(f32)))
+    ev, eg = oracle.softmaxCrossEntropySparse(logits, idx.astype(f32))
+    got = res.grad.toHost()
+    assert abs(res.value - ev) <= 1e-4 * abs(ev) + 1e-6
+    assert_close(got, eg, what="sparse CE grad")
+    assert (got[np.arange(rows), idx] < 0).all() and (np.delete(got, idx[0], axis=1)[0] >= 0).all()
+
+
 @pytest.mark.parametrize("rows,classes,keep", [(1, 2, 1.0), (7, 13, 0.5), (512, 256, 0.15), (33, 1000, 0.3), (6, 32000, 0.5), (4, 50257, 0.5),
                                                (2, 70001, 1.0), (9, 40, 0.0)])
 def test_masked_cross_entropy(hip, oracle, rng, rows, classes, keep):
