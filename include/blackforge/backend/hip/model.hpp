@@ -227,10 +227,14 @@ private:
         }
     }
 
-    DeviceTensor applyForward(LayerState& layer, const DeviceTensor& x, bool trustedIds) {
+    // x is about to become the layer's cached input: a bf16 linear layer gives it the bf16 image that both its forward
+    // product and, in the backward pass, its weight-gradient product read.
+    DeviceTensor applyForward(LayerState& layer, DeviceTensor& x, bool trustedIds) {
         const LayerSpec& s = layer.spec;
         switch (s.kind) {
             case LayerKind::Linear:
+                if (useBf16_ && x.image() == nullptr && x.rank() >= 2 && x.elementCount() > 0 && x.dim(x.rank() - 1) % 8 == 0)
+                    check(bf_hip_cvt_f32_bf16(x.data(), x.attachImage(), x.elementCount(), nullptr));
                 return useBf16_ ? linearBf16CachedWeight(x, layer.params[0].value, layer.params[1].value)
                                 : linear(x, layer.params[0].value, layer.params[1].value);
             case LayerKind::Embedding:

@@ -72,8 +72,9 @@ inline DeviceTensor projectionFused(const DeviceTensor& a, const DeviceTensor& b
                                    m, n, k, nullptr));
         return c;
     }
-    check(bf_hip_linear_bf16(a.data(), b.data(), bias ? bias->data() : nullptr, residual ? residual->data() : nullptr, c.data(), m, k,
-                             n, bf16 == 2, nullptr));
+    // an input that carries its bf16 image is not converted again
+    check(bf_hip_linear_bf16_img(a.data(), a.image(), b.data(), bias ? bias->data() : nullptr, residual ? residual->data() : nullptr,
+                                 c.data(), m, k, n, bf16 == 2, nullptr));
     return c;
 }
 }  // namespace detail
