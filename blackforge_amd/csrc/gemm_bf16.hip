@@ -64,10 +64,17 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict_
 // whole 128-byte lines; otherwise elements go one by one.  When `plain` is not NULL the same pass also writes
 // the untransposed image plain[r*ldPlain + 0..pad8(cols)) = bf16(x[r, :]), zero padded: a gradient that feeds
 // both the input-gradient GEMM (plain) and the weight-gradient GEMM (transposed) is read from HBM once.
-__global__ void __launch_bounds__(kBlock) convertTransposeKernel(const float* __restrict__ x, unsigned short* __restrict__ out,
+// Up to three matrices of one shape in one launch (blockIdx.z): matrix z is read from xs.p[z] and written `outStep`
+// (and `plainStep`) elements after the one before.
+struct ConvertSources { const float* p[3]; };
+__global__ void __launch_bounds__(kBlock) convertTransposeKernel(ConvertSources xs, unsigned short* __restrict__ out,
                                                                  size_t rows, size_t cols, size_t rowsPad, int vec,
-                                                                 unsigned short* __restrict__ plain, size_t ldPlain) {
+                                                                 unsigned short* __restrict__ plain, size_t ldPlain, size_t outStep,
+                                                                 size_t plainStep) {
     __shared__ __attribute__((aligned(16))) unsigned short tile[64][72];   // [column][row], 144-byte pitch
+    const float* __restrict__ x = blockIdx.z == 0 ? xs.p[0] : blockIdx.z == 1 ? xs.p[1] : xs.p[2];
+    out += blockIdx.z * outStep;
+    if (plain) plain += blockIdx.z * plainStep;
     const size_t r0 = size_t(blockIdx.y) * 64, c0 = size_t(blockIdx.x) * 64;
     const size_t colsPad = (cols + 7) / 8 * 8;
     if (vec) {
@@ -993,18 +1000,25 @@ int convertPlain(const float* x, unsigned short* out, size_t rows, size_t cols, 
 }
 
 // plain / ldPlain: optional second output, the untransposed image with row stride ldPlain (a multiple of 8).
-int convertTransposed(const float* x, unsigned short* out, size_t rows, size_t cols, hipStream_t s, bool padRows = true,
-                      unsigned short* plain = nullptr, size_t ldPlain = 0) {
-    if (rows == 0 || cols == 0) return BF_OK;
+// `count` matrices (at most three) of one shape in one launch: matrix i goes to out + i * outStep and plain + i * plainStep.
+int convertTransposedGroup(const float* const* x, size_t count, unsigned short* out, size_t outStep, size_t rows, size_t cols, hipStream_t s,
+                           bool padRows, unsigned short* plain, size_t ldPlain, size_t plainStep) {
+    if (rows == 0 || cols == 0 || count == 0) return BF_OK;
     size_t rowsPad = padRows ? pad8(rows) : rows;   // length of an output row
     // the grid covers pad8(cols) columns so that the plain image's zero padding is written too
-    dim3 grid(unsigned(((plain ? pad8(cols) : cols) + 63) / 64), unsigned((rowsPad + 63) / 64));
+    dim3 grid(unsigned(((plain ? pad8(cols) : cols) + 63) / 64), unsigned((rowsPad + 63) / 64), unsigned(count));
     if (grid.y > 65535) return failInvalid("cvt_f32_bf16_transpose", "too many rows");
-    const int vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(plain)) & 15u) == 0 &&
-                    cols % 4 == 0 && rowsPad % 8 == 0 && ldPlain % 8 == 0;
-    convertTransposeKernel<<<grid, kBlock, 0, s>>>(x, out, rows, cols, rowsPad, vec, plain, ldPlain);
+    ConvertSources xs{{x[0], count > 1 ? x[1] : nullptr, count > 2 ? x[2] : nullptr}};
+    uintptr_t bits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(plain) | (outStep * 2) | (plainStep * 2);
+    for (size_t i = 0; i < count; ++i) bits |= reinterpret_cast<uintptr_t>(x[i]);
+    const int vec = (bits & 15u) == 0 && cols % 4 == 0 && rowsPad % 8 == 0 && ldPlain % 8 == 0;
+    convertTransposeKernel<<<grid, kBlock, 0, s>>>(xs, out, rows, cols, rowsPad, vec, plain, ldPlain, outStep, plainStep);
     BF_LAUNCH_CHECK();
     return BF_OK;
+}
+int convertTransposed(const float* x, unsigned short* out, size_t rows, size_t cols, hipStream_t s, bool padRows = true,
+                      unsigned short* plain = nullptr, size_t ldPlain = 0) {
+    return convertTransposedGroup(&x, 1, out, 0, rows, cols, s, padRows, plain, ldPlain, 0);
 }
 
 // out[c, r] = in[r, c] for a bf16 image `in` [rows, ldIn] (cols columns used); `out` is [cols, ldOut] with ldOut >= rows,
@@ -1053,6 +1067,8 @@ std::map<WeightKey, CachedWeight>& weightCache() {
 // `plain`: for the transposed layouts (1, 2) the plain counterpart (0, 3) written in the same pass, or NULL.
 int fillWeightImage(const float* const* w, size_t count, size_t rows, size_t cols, int layout, unsigned short* image, unsigned short* plain,
                     hipStream_t s) {
+    if (layout == 2 && count <= 3)   // the stacked transposed images of a group (and their plain ones side by side) in one launch
+        return convertTransposedGroup(w, count, image, cols * pad8(rows), rows, cols, s, true, plain, count * cols, cols);
     int st = BF_OK;
     for (size_t i = 0; i < count && st == BF_OK; ++i) {
         if (layout == 0) st = convertPlain(w[i], image, rows, cols, s);
