@@ -255,7 +255,49 @@ def bench_extras(bf, steps):
     gemm(8192, 3072, 768)
     gemm(8192, 768, 3072)
     gemm(768, 3072, 8192)
+    extras.update(vendor_gemm_reference([(4096, 4096, 4096), (16384, 8192, 2048), (8192, 3072, 768), (8192, 768, 3072), (768, 3072, 8192)]))
     return extras
+
+
+_VENDOR_GEMM_CHILD = r"""
+import json, sys, torch
+shapes, peak = json.loads(sys.argv[1]), float(sys.argv[2])
+out = {}
+for m, n, k in shapes:
+    a = torch.randn(m, k, device="cuda", dtype=torch.bfloat16)
+    bt = (torch.randn(n, k, device="cuda", dtype=torch.bfloat16) / 8).t()
+    run = lambda: torch.mm(a, bt, out_dtype=torch.float32)
+    for _ in range(3):
+        run()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(3):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(10):
+            run()
+        end.record()
+        torch.cuda.synchronize()
+        best = min(best, start.elapsed_time(end) / 10)
+    tf = 2 * m * n * k / best / 1e9
+    out["vendor_library_gemm_bf16_%dx%dx%d" % (m, n, k)] = {"ms": round(best, 4), "TFLOP/s": round(tf, 1), "frac_bf16_mfma": round(tf / peak, 3)}
+    del a, bt
+print(json.dumps(out))
+"""
+
+
+def vendor_gemm_reference(shapes):
+    """The same products (bf16 operands, second one stored transposed, fp32 result) through the vendor's GEMM library as
+    PyTorch calls it (torch.mm -> hipBLASLt): what a library call delivers on this box, beside the hand-written kernels
+    above.  In a child process (PyTorch brings a HIP runtime of its own, which cannot share a process with the one this
+    library is linked to) while this one is idle; best of three runs of ten launches.  Empty where that fails."""
+    import subprocess
+    try:
+        proc = subprocess.run([sys.executable, "-c", _VENDOR_GEMM_CHILD, json.dumps(shapes), str(PEAK_BF16_MFMA_TFLOPS)],
+                              capture_output=True, text=True, timeout=240)
+        return json.loads(proc.stdout.strip().splitlines()[-1])
+    except Exception as err:   # no torch, an older torch without out_dtype, a time-out: no comparison
+        return {"vendor_library_gemm_bf16": {"skipped": str(err)[:120]}}
 
 
 def lm_layers(hl, vocab, dim, seq, heads, hidden, act, blocks):
@@ -511,8 +553,11 @@ def extras_summary(extras):
     """The north-star targets in three numbers: the bf16 projection at 4096^3 against the bf16 MFMA peak, and the worst and
     the median bandwidth kernel against the HBM peak."""
     hbm = sorted((v["frac_hbm"], k) for k, v in extras.items() if "frac_hbm" in v)
-    gemms = {k: v["frac_bf16_mfma"] for k, v in extras.items() if "frac_bf16_mfma" in v}
+    gemms = {k: v["frac_bf16_mfma"] for k, v in extras.items() if "frac_bf16_mfma" in v and not k.startswith("vendor_")}
+    vendor = {k[len("vendor_library_"):]: v["frac_bf16_mfma"] for k, v in extras.items() if "frac_bf16_mfma" in v and k.startswith("vendor_")}
     out = {"bf16_gemm_frac_of_peak": gemms}
+    if vendor:
+        out["vendor_library_frac_of_peak"] = vendor
     if hbm:
         out["hbm_min"] = {"kernel": hbm[0][1], "frac": hbm[0][0]}
         out["hbm_median"] = {"kernel": hbm[len(hbm) // 2][1], "frac": hbm[len(hbm) // 2][0]}
