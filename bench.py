@@ -265,20 +265,23 @@ shapes, peak = json.loads(sys.argv[1]), float(sys.argv[2])
 out = {}
 for m, n, k in shapes:
     a = torch.randn(m, k, device="cuda", dtype=torch.bfloat16)
-    bt = (torch.randn(n, k, device="cuda", dtype=torch.bfloat16) / 8).t()
+    bt = (torch.randn(n, k, device="cuda", dtype=torch.bfloat16) / 64).t()   # the operand statistics of the kernels above
     run = lambda: torch.mm(a, bt, out_dtype=torch.float32)
     for _ in range(3):
         run()
     torch.cuda.synchronize()
-    best = float("inf")
-    for _ in range(3):
+    count = 10
+    while True:   # as `timed` above: ten launches, or as many as make 2 ms
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
-        for _ in range(10):
+        for _ in range(count):
             run()
         end.record()
         torch.cuda.synchronize()
-        best = min(best, start.elapsed_time(end) / 10)
+        best = start.elapsed_time(end) / count
+        if best * count >= 0.5 or count > 10:
+            break
+        count = max(11, int(2.0 / best))
     tf = 2 * m * n * k / best / 1e9
     out["vendor_library_gemm_bf16_%dx%dx%d" % (m, n, k)] = {"ms": round(best, 4), "TFLOP/s": round(tf, 1), "frac_bf16_mfma": round(tf / peak, 3)}
     del a, bt
@@ -290,7 +293,7 @@ def vendor_gemm_reference(shapes):
     """The same products (bf16 operands, second one stored transposed, fp32 result) through the vendor's GEMM library as
     PyTorch calls it (torch.mm -> hipBLASLt): what a library call delivers on this box, beside the hand-written kernels
     above.  In a child process (PyTorch brings a HIP runtime of its own, which cannot share a process with the one this
-    library is linked to) while this one is idle; best of three runs of ten launches.  Empty where that fails."""
+    library is linked to) while this one is idle, timed as the kernels above are.  Empty where that fails."""
     import subprocess
     try:
         proc = subprocess.run([sys.executable, "-c", _VENDOR_GEMM_CHILD, json.dumps(shapes), str(PEAK_BF16_MFMA_TFLOPS)],
