@@ -776,12 +776,14 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 3 : HDP <= 128 ? 2 : 1) attnB
 // AHEAD: the S / dP products of sub-block sb+1 are issued before the exp / dS arithmetic of sub-block sb (two sub-blocks
 // of scores live at once).  With two waves per SIMD the other wave fills the matrix pipe during that arithmetic, and
 // the 32 registers are worth more as room that keeps the kernel from spilling.
-template <int HDP, int BQ, bool MASKED, bool STORE, bool AHEAD>
+// DTP, dOff: the pass accumulates DTP 32-wide blocks of the head dim starting at element dOff (all of them unless the
+// kernel takes the head dim in two passes); dsLane == nullptr: a pass that does not store dS.
+template <int HDP, int BQ, bool MASKED, bool STORE, bool AHEAD, int DTP = HDP / 32>
 __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const float* __restrict__ gs, const float* __restrict__ stats,
-                                        const float (&kreg)[HDP / 2], const float (&vreg)[HDP / 2], float16v (&dk)[HDP / 32],
-                                        float16v (&dv)[HDP / 32], int qt0, int key, bool keyValid, int oldLen, int half, int li,
-                                        float* __restrict__ dsLane, size_t dsStride, int newLen) {
-    constexpr int LDSW = HDP + 4, DT = HDP / 32, NSB = BQ / 32, LIVE = AHEAD ? NSB : 1;
+                                        const float (&kreg)[HDP / 2], const float (&vreg)[HDP / 2], float16v (&dk)[DTP],
+                                        float16v (&dv)[DTP], int qt0, int key, bool keyValid, int oldLen, int half, int li,
+                                        float* __restrict__ dsLane, size_t dsStride, int newLen, int dOff = 0) {
+    constexpr int LDSW = HDP + 4, DT = DTP, NSB = BQ / 32, LIVE = AHEAD ? NSB : 1;
     float16v s[LIVE], dp[LIVE];
     auto scores = [&](int sb) {   // S = Q * K^T and dP = dO * V^T of sub-block sb
         float16v& sDst = s[AHEAD ? sb : 0];
@@ -818,7 +820,7 @@ __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const floa
             }
         }
         if constexpr (STORE) {
-            if (qt0 + sb * 32 < newLen) {   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave
+            if (dsLane != nullptr && qt0 + sb * 32 < newLen) {   // row dRow(r, half) of the sub-block, 128 contiguous bytes per half wave
                 float* dst = dsLane + sb * dsStride;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(dsv[r], dst + (8 * (r >> 2) + (r & 3)) * 32);
@@ -827,8 +829,8 @@ __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const floa
         // dV += P^T * dO, dK += dS^T * Q : step r contracts over query dRow(r, half)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float* grow = gs + (sb * 32 + dRow(r, half)) * LDSW + li;
-            const float* qrow = qs + (sb * 32 + dRow(r, half)) * LDSW + li;
+            const float* grow = gs + (sb * 32 + dRow(r, half)) * LDSW + dOff + li;
+            const float* qrow = qs + (sb * 32 + dRow(r, half)) * LDSW + dOff + li;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 dv[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pr[r], grow[dt * 32], dv[dt], 0, 0, 0);
@@ -839,17 +841,17 @@ __device__ __forceinline__ void dkvTile(const float* __restrict__ qs, const floa
 }
 
 // dk/dv[dt][r]: key = waveK0 + dRow(r, half), d = dt*32 + li  -> 128-byte coalesced rows (fp32 tensors and bf16 images)
-template <int HDP>
-__device__ __forceinline__ void storeKeyGradients(const AttnParams& p, const float16v (&dk)[HDP / 32], const float16v (&dv)[HDP / 32], int b,
-                                                  int h, int waveK0, size_t kOff, int half, int li) {
-    constexpr int DT = HDP / 32;
+template <int HDP, int DTP = HDP / 32>
+__device__ __forceinline__ void storeKeyGradients(const AttnParams& p, const float16v (&dk)[DTP], const float16v (&dv)[DTP], int b,
+                                                  int h, int waveK0, size_t kOff, int half, int li, int dOff = 0) {
+    constexpr int DT = DTP;
     const int hd = p.hd, dim = p.dim;
     const bool images = p.dKImg != nullptr || p.dVImg != nullptr;
     // with an even head dim, row pitch and base every even column of an image row is 4-byte aligned and has its neighbour
     const bool pairs = (hd & 1) == 0 && (p.imgLd & 1u) == 0 && ((reinterpret_cast<uintptr_t>(p.dKImg) | reinterpret_cast<uintptr_t>(p.dVImg)) & 3u) == 0;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-        const int d = dt * 32 + li;
+        const int d = dOff + dt * 32 + li;
         if (d < hd) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -904,11 +906,11 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
     loadRowOperand<HDP, VEC4>(kreg, p.k + kOff + size_t(key) * dim, keyValid, hd, half, p.scale * kLog2e);
     loadRowOperand<HDP, VEC4>(vreg, p.v + kOff + size_t(key) * dim, keyValid, hd, half, 1.0f);
 
-    float16v dk[DT], dv[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.0f; dv[dt][r] = 0.0f; }
+    // Head dim 256: K and V rows (256 registers) and both accumulators (256 more) do not fit a wavefront's 512 registers,
+    // so the accumulators take the head dim in two passes of 128, each over all the query tiles (S and dP are formed
+    // again in the second pass: half again as many MFMAs, against spilling most of the accumulators).
+    constexpr int PASSES = HDP > 128 ? 2 : 1, DTP = DT / PASSES;
+    float16v dk[DTP], dv[DTP];
 
     // first query that can see any key of this workgroup's tile: oldLen + i >= kt*128
     int firstQuery = kt * 128 - p.oldLen;
@@ -921,6 +923,12 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
     float* const dsColumn = STORE ? p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024 : nullptr;   // wave-uniform
     const int dsLaneOffset = half * 128 + li;
 
+    for (int pass = 0; pass < PASSES; ++pass) {
+    const int dOff = pass * DTP * 32;
+#pragma unroll
+    for (int dt = 0; dt < DTP; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.0f; dv[dt][r] = 0.0f; }
     TileRegs<HDP, BQ> qNext, gNext;
     float statNext = 0.0f;
     auto fetchStats = [&](int qt0) {   // thread t < BQ: lse2 of query qt0+t; BQ <= t < 2BQ: D of query qt0+t-BQ
@@ -953,22 +961,23 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
             const float* qcur = qs + (t & 1) * TILE;
             const float* gcur = gs + (t & 1) * TILE;
             const float* scur = stats + (t & 1) * 2 * BQ;
-            float* dsLane = STORE ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;
+            float* dsLane = STORE && pass == 0 ? dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset : nullptr;   // dS once
             if (masked)
-                dkvTile<HDP, BQ, true, STORE, OCC == 1>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride,
-                                              p.newLen);
+                dkvTile<HDP, BQ, true, STORE, OCC == 1, DTP>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane,
+                                                             dsStride, p.newLen, dOff);
             else
-                dkvTile<HDP, BQ, false, STORE, OCC == 1>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride,
-                                               p.newLen);
+                dkvTile<HDP, BQ, false, STORE, OCC == 1, DTP>(qcur, gcur, scur, kreg, vreg, dk, dv, qt0, key, keyValid, p.oldLen, half, li, dsLane,
+                                                              dsStride, p.newLen, dOff);
         }
         if (t + 1 < numQTiles) {
             commitAll((t + 1) & 1);
             if (t + 2 < numQTiles) fetchAll(qt0 + 2 * BQ);
         }
-        __syncthreads();
+        __syncthreads();   // after the last tile too: the next pass writes the LDS buffers again
     }
 
-    storeKeyGradients<HDP>(p, dk, dv, b, h, waveK0, kOff, half, li);
+    storeKeyGradients<HDP, DTP>(p, dk, dv, b, h, waveK0, kOff, half, li, dOff);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
