@@ -87,7 +87,7 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                                                                          float* __restrict__ grad, float* __restrict__ rowLoss,
                                                                          size_t rows, size_t classes, float invRows,
                                                                          const float* __restrict__ maskInfo,
-                                                                         unsigned short* __restrict__ gradImage) {
+                                                                         unsigned short* __restrict__ gradImage, unsigned shiftMask) {
     static_assert(CACHED || !AHEAD, "only rows held in registers are fetched ahead");
     __shared__ float lds[16];
     const int t = threadIdx.x % G;
@@ -103,7 +103,7 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
     // is not waited for here
     auto fetch = [&](auto& into, size_t r) __attribute__((always_inline)) {
         const float* src = logits + r * classes;
-        if constexpr (SHIFTED) into.template issueShifted<0, MAXE / VEC>(src, classes, t, Row::shiftOf(src));
+        if constexpr (SHIFTED) into.template issueShifted<0, MAXE / VEC>(src, classes, t, Row::shiftOf(src, shiftMask));
         else into.load(src, classes, t, -INFINITY);
     };
     if constexpr (AHEAD) { if (firstRow < rows) fetch(ahead, firstRow); }
@@ -117,7 +117,7 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
         } else if constexpr (CACHED) {
             fetch(c, row);
         }
-        const int shift = SHIFTED ? Row::shiftOf(x) : 0;   // the same for gOut: the host checks that
+        const int shift = SHIFTED ? Row::shiftOf(x, shiftMask) : 0;   // the same for gOut: the host checks that
         if constexpr (CACHED && SHIFTED) c.maskShifted(classes, t, -INFINITY, shift);
         // gradImage (aligned rows only; the host checks): the gradient row rounded to bf16, for the bf16 GEMMs that consume it
         unsigned short* gImg = gradImage ? gradImage + row * classes : nullptr;
@@ -253,6 +253,9 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
     // rows that are not 16-byte aligned still get 16-byte accesses (shifted) as long as a logits row and its gradient
     // row sit at the same offset within a 16-byte group; a row must then fit its registers with up to 3 elements to spare
     const bool shifted = !vec4 && ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad)) & 15u) == 0;
+    // shifted rows are addressed from the 128-byte line below their first element when logits and gradient rows sit at
+    // the same offset within a line (every wavefront access then covers whole lines), else from the 16-byte group below
+    const bool sameLine = ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad)) & 127u) == 0;
     const bool streaming = streamsPastCache(rows * classes * (SPARSE ? 8 : 12));   // logits in, gradient out (and a dense target in)
     // smallest group and register count that hold a row (see the row kernels)
     // AHEAD as measured (8 B per logit over the launch, 16-byte aligned rows): rows of up to 8192 classes are faster
@@ -262,18 +265,24 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
 #define BF_CE(G, MAXE, AHEAD)                                                                                     \
     if (classes + (vec4 ? 0 : 3) <= size_t(G) * MAXE && (vec4 || shifted || MAXE <= 32)) {                        \
         const unsigned threads = G > 256 ? G : 256;                                                               \
+        /* whole lines pay on the long rows (1024 threads a row: +5..8 %); rows of 4100 measured 12 % slower that way */ \
+        const unsigned shiftMask = sameLine && G == 1024 && classes + 31 <= size_t(G) * MAXE ? 31u : 3u;           \
         const unsigned grid = gridFor(rows, threads / G, AHEAD ? unsigned(computeUnits()) * (2048 / threads) : kMaxGridX); \
-        if (vec4 && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
-        else if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
-        else if (shifted && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
-        else if (shifted) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); \
-        else crossEntropyKernel<G, (MAXE <= 32 ? MAXE : 4), 1, true, SPARSE, false, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage); /* plans above 32 registers have no one-element form */ \
+        /* 16-byte aligned rows that start inside a 128-byte line go the shifted way as well, for the whole lines */ \
+        const bool lineShift = vec4 && classes % 32 != 0 && shiftMask == 31u && gradImage == nullptr;               \
+        if (lineShift && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \
+        else if (lineShift) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \
+        else if (vec4 && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \
+        else if (vec4) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \
+        else if (shifted && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \
+        else if (shifted) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \
+        else crossEntropyKernel<G, (MAXE <= 32 ? MAXE : 4), 1, true, SPARSE, false, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); /* plans above 32 registers have no one-element form */ \
         break;                                                                                                    \
     }
     do {
         BF_CE(64, 4, false) BF_CE(64, 8, false) BF_CE(64, 16, false) BF_CE(256, 8, false) BF_CE(256, 16, false) BF_CE(256, 32, false)
         BF_CE(1024, 16, true) BF_CE(1024, 32, true) BF_CE(1024, 52, false)
-        crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage);
+        crossEntropyKernel<1024, 4, 1, false, SPARSE><<<gridFor(rows, 1), 1024, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, 3u);
     } while (0);
 #undef BF_CE
     BF_LAUNCH_CHECK();

@@ -5,10 +5,12 @@
 // the row from HBM exactly once.  Rows longer than G*MAXE fall back to re-reading global memory
 // (served by L2).  VEC = 4 uses dwordx4 accesses and needs 16-byte aligned rows (features % 4 == 0
 // and an aligned base); VEC = 1 handles every other shape with coalesced dword accesses.  loadShifted /
-// storeShifted give rows of ANY length and alignment the 16-byte accesses too: the row is addressed from the
-// 16-byte boundary at or below its first element, `shift` (0..3) elements earlier, and the elements a group
-// holds from outside the row are masked.  An aligned 16-byte load that contains one element of the tensor stays
-// inside the tensor's page, so the bytes read from beyond a row are always readable; nothing is written there.
+// storeShifted give rows of ANY length and alignment the 16-byte accesses too: the row is addressed from an
+// aligned boundary at or below its first element, `shift` elements earlier (the 16-byte boundary, shift 0..3, or
+// the 128-byte line, shift 0..31, after which every wavefront access covers whole lines: 8 % faster on rows of
+// 50 257 floats), and the elements a group holds from outside the row are masked.  The aligned line that holds the
+// row's first element, and the aligned 16 bytes that hold its last, stay inside the pages of the tensor, so the
+// bytes read from beyond a row are always readable; nothing is written there.
 #pragma once
 
 #include "common.hpp"
@@ -50,11 +52,12 @@ struct RowCache {
         }
     }
 
-    // Elements before the row's first one in the 16-byte group that holds it.
-    __device__ static int shiftOf(const float* row) { return int((reinterpret_cast<uintptr_t>(row) >> 2) & 3u); }
+    // Elements before the row's first one in the 16-byte group that holds it (mask 3), or in the 128-byte line that holds
+    // it (mask 31: every wavefront access then covers whole lines).
+    __device__ static int shiftOf(const float* row, unsigned mask = 3u) { return int((reinterpret_cast<uintptr_t>(row) >> 2) & mask); }
 
-    // Rows are shorter than 2^31 - 4 elements here (G * MAXE elements at most), so 32-bit indices do.  Only the group
-    // that holds the row's first element (thread 0, iteration 0) and the one that holds its last need any masking.
+    // Rows are shorter than 2^31 - 32 elements here (G * MAXE elements at most), so 32-bit indices do.  Only the groups
+    // up to the one that holds the row's first element (iteration 0) and the one that holds its last need any masking.
     __device__ __forceinline__ void loadShifted(const float* __restrict__ row, size_t features, int t, float fill, int shift) {
         // every load first (a group past the row's end re-reads group 0 instead of branching), the masking afterwards:
         // code between the loads that touches a loaded register would make each load wait for the one before it
@@ -79,7 +82,7 @@ struct RowCache {
 
     __device__ __forceinline__ void maskShifted(size_t features, int t, float fill, int shift) {
         const int last = int(features) + shift;
-        const int lo = t == 0 ? shift : 0;   // slots of thread 0's first group that belong to the row before
+        const int lo = shift - 4 * t;   // slots of this thread's first group that lie before the row (<= 0: none)
 #pragma unroll
         for (int it = 0; it < kIters; ++it) {
             const int n = last - (it * G + t) * 4;   // slots of this group before the row's end (>= 4: all of them)
@@ -97,7 +100,7 @@ struct RowCache {
         for (int it = 0; it < kIters; ++it) {
             const int g = (it * G + t) * 4;
             if (g < last) {
-                const bool head = it == 0 && t == 0 && shift > 0, tail = g + 4 > last;
+                const bool head = it == 0 && g < shift, tail = g + 4 > last;   // a group that starts before the row
                 if (!head && !tail) {
                     stf4<NT>(base + g, float4v{r[it * 4 + 0], r[it * 4 + 1], r[it * 4 + 2], r[it * 4 + 3]});
                 } else {   // a group that straddles an end of the row: its own elements one by one
