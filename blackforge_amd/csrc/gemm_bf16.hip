@@ -218,6 +218,48 @@ __device__ __forceinline__ void storeAccumulators(float16v (&acc)[TM][TN], const
             }
         return;
     }
+    // One output of any width and alignment (an odd vocabulary): the same transposition, and the four columns of a lane as
+    // one 16-byte access from whatever 4-byte boundary they start on (global memory serves those); the last group of a
+    // row, which may hold fewer than four columns, goes element by element.
+    if (ld == N && shift == 0) {
+        const int t = li & 3, colq = 4 * (li >> 2);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int col = col0 + j * 32 + colq;
+                const bool whole = col + 4 <= N;
+                float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (e.bias) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) b[c] = col + c < N ? e.bias[col + c] : 0.0f;
+                }
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float v[4] = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    quadTranspose(v[0], v[1], v[2], v[3], t);
+                    const int row = row0 + i * 32 + 8 * g + 4 * half + t;
+                    if (row < M && col < N) {
+                        float* dst = C + size_t(row) * N + col;
+                        const float* res = e.residual ? e.residual + size_t(row) * N + col : nullptr;
+                        if (e.bias) {   // the same additions, in the same order, as the other two forms
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) v[c] += b[c];
+                        }
+                        if (whole) {
+                            float4u out = {v[0], v[1], v[2], v[3]};
+                            if (res) out = out + *reinterpret_cast<const float4u*>(res);
+                            *reinterpret_cast<float4u*>(dst) = out;
+                        } else {
+#pragma unroll
+                            for (int c = 0; c < 4; ++c)
+                                if (col + c < N) dst[c] = res ? v[c] + res[c] : v[c];
+                        }
+                    }
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
