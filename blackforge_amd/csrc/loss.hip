@@ -269,7 +269,9 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
         const unsigned shiftMask = sameLine && G == 1024 && classes + 31 <= size_t(G) * MAXE ? 31u : 3u;           \
         const unsigned grid = gridFor(rows, threads / G, AHEAD ? unsigned(computeUnits()) * (2048 / threads) : kMaxGridX); \
         /* 16-byte aligned rows that start inside a 128-byte line go the shifted way as well, for the whole lines */ \
-        const bool lineShift = vec4 && classes % 32 != 0 && shiftMask == 31u && gradImage == nullptr;               \
+        /* so do the long 16-byte aligned rows of a dense target: the form without a branch per load keeps to its registers */ \
+        const bool lineShift = vec4 && gradImage == nullptr &&                                                      \
+                               ((classes % 32 != 0 && shiftMask == 31u) || (!SPARSE && MAXE > 32));                  \
         if (lineShift && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \
         else if (lineShift) crossEntropyKernel<G, MAXE, 4, true, SPARSE, true, false, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \
         else if (vec4 && streaming) crossEntropyKernel<G, MAXE, 4, true, SPARSE, false, true, AHEAD><<<grid, threads, 0, s>>>(logits, target, grad, rl, rows, classes, invRows, maskInfo, gradImage, shiftMask); \

@@ -112,7 +112,8 @@ def test_concat_seq_and_argmax(hip, oracle, rng):
     assert ops.argmaxLastPosition(D.fromHost(logits)) == 0
 
 
-@pytest.mark.parametrize("rows,classes", [(1, 2), (2, 3), (7, 13), (512, 256), (5, 1000), (3, 32000), (2, 50257), (1, 70001)])
+@pytest.mark.parametrize("rows,classes", [(1, 2), (2, 3), (7, 13), (512, 256), (5, 1000), (3, 32000), (2, 50257), (1, 70001), (3, 40000),
+                                          (2, 50260)])
 def test_cross_entropy(hip, oracle, rng, rows, classes):
     D, ops = hip.DeviceTensor, hip.ops
     logits = r(rng, rows, classes, scale=3)
