@@ -83,8 +83,15 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(ConvertSources 
         for (int i = 0; i < 4; ++i) {
             const int r = rr + 16 * i;
             const size_t gr = r0 + r, gc = c0 + 4 * cg;
-            float4v v = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (gr < rows && gc < cols) v = loadf4(x + gr * cols + gc);   // cols % 4 == 0: all four in range
+            float4u v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (gr < rows && gc + 4 <= cols) {
+                v = *reinterpret_cast<const float4u*>(x + gr * cols + gc);   // from any 4-byte boundary (rows of odd length)
+            } else if (gr < rows && gc < cols) {   // the last, partial group of a row
+                const float* src = x + gr * cols + gc;
+                v.x = src[0];
+                if (gc + 1 < cols) v.y = src[1];
+                if (gc + 2 < cols) v.z = src[2];
+            }
             const unsigned short b0 = toBf16Bits(v.x), b1 = toBf16Bits(v.y), b2 = toBf16Bits(v.z), b3 = toBf16Bits(v.w);
             tile[4 * cg + 0][r] = b0;
             tile[4 * cg + 1][r] = b1;
@@ -1051,9 +1058,9 @@ int convertTransposedGroup(const float* const* x, size_t count, unsigned short* 
     dim3 grid(unsigned(((plain ? pad8(cols) : cols) + 63) / 64), unsigned((rowsPad + 63) / 64), unsigned(count));
     if (grid.y > 65535) return failInvalid("cvt_f32_bf16_transpose", "too many rows");
     ConvertSources xs{{x[0], count > 1 ? x[1] : nullptr, count > 2 ? x[2] : nullptr}};
-    uintptr_t bits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(plain) | (outStep * 2) | (plainStep * 2);
-    for (size_t i = 0; i < count; ++i) bits |= reinterpret_cast<uintptr_t>(x[i]);
-    const int vec = (bits & 15u) == 0 && cols % 4 == 0 && rowsPad % 8 == 0 && ldPlain % 8 == 0;
+    // the sources need no alignment beyond a float's and rows of any length do (16-byte loads from any 4-byte boundary)
+    uintptr_t outBits = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(plain) | (outStep * 2) | (plainStep * 2);
+    const int vec = (outBits & 15u) == 0 && rowsPad % 8 == 0 && ldPlain % 8 == 0;
     convertTransposeKernel<<<grid, kBlock, 0, s>>>(xs, out, rows, cols, rowsPad, vec, plain, ldPlain, outStep, plainStep);
     BF_LAUNCH_CHECK();
     return BF_OK;
