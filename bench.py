@@ -38,7 +38,7 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
 # 1224 MB written (1095 MB of that is the dS hand-over; the read side moves between 0.6 and 1.0 GB from run to run
 # with what the L2s happen to keep).  profiles/attention_c3_kernel_trace.md holds the commands
 # and the raw counter values.
-MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvPipedKernel": 1980923267}
+MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvPipedKernel": 1969678618}
 
 
 def attention_flops(batch, heads, seq, hd):
