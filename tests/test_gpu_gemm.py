@@ -247,7 +247,7 @@ def test_bf16_linear_with_adds_in_the_store(hip, oracle, rng, m, k, n, with_bias
     """bf_hip_linear_bf16 = matmulBf16 followed by addBias / addBiasResidual / add (ops.hpp:14,30,8), through every
     GEMM path: small tiles, 128-row tiles on sixteen wavefronts, 256-row tiles, and a contraction cut into slices; widths
     that are multiples of four (16-byte stores after the transposition inside lane quads) and widths that are not
-    (element-wise stores)."""
+    (the same stores from 4-byte boundaries, the last group of a row element by element)."""
     D, ops = hip.DeviceTensor, hip.ops
     a, w, bias, res = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, n), r(rng, m, n)
     got = ops.linearBf16Fused(D.fromHost(a), D.fromHost(w), D.fromHost(bias) if with_bias else None,
