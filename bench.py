@@ -39,6 +39,8 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E peak
 # with what the L2s happen to keep).  profiles/attention_c3_kernel_trace.md holds the commands
 # and the raw counter values.
 MEASURED_TRAFFIC_BYTES = {"attnBackwardDkvPipedKernel": 1969678618}
+# Share of cycles with the matrix pipe busy, same kernel, same workload, by counter (same profile file)
+MEASURED_MFMA_BUSY = {"attnBackwardDkvPipedKernel": 0.44}
 
 
 def attention_flops(batch, heads, seq, hd):
@@ -238,6 +240,24 @@ def bench_extras(bf, steps):
     hbm("zero_multi_134951168_params", 4 * total, lambda: call("bf_hip_zero_multi", gs, cn, len(counts), sh))
     del pool
 
+    # what the matrix pipes deliver with nothing else running: the K loop of the 256 x 256 tile with its operand fragments
+    # held in registers (random N(0,1) bf16 values), one workgroup of eight wavefronts per compute unit, for both bf16 MFMA
+    # shapes; `implied_clock_ghz` is the clock at which 4096 flop per clock and compute unit give that rate
+    cus = bf.capi.device_props(0).compute_units
+    operands = D((32768,), itemsize=2)
+    call("bf_hip_cvt_f32_bf16", rand(32768).ptr, operands.ptr, 32768, None)
+    sink = D((cus * 512,))
+    ceiling = {}
+    k_steps = 2048   # 2048 steps of 2*256*256*64 flop per workgroup: ~3 ms a launch, as long as the largest product below
+    for shape, name in ((0, "32x32x16"), (1, "16x16x32")):
+        ms = timed(lambda: call("bf_hip_mfma_only_loop", operands.ptr, sink.ptr, shape, cus, k_steps, sh), 3)
+        tf = 2 * 256 * 256 * 64 * k_steps * cus / ms / 1e9
+        ceiling[name] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_bf16_mfma": round(tf / PEAK_BF16_MFMA_TFLOPS, 3),
+                         "implied_clock_ghz": round(tf * 1e12 / (4096 * cus) / 1e9, 3)}
+    extras["mfma_only_ceiling"] = {"what": "K loop of the shipped 256x256x64 bf16 tile, operands in registers (no LDS, no global memory), "
+                                           f"{cus} workgroups x 8 wavefronts, {k_steps} K steps a launch, N(0,1) operands", **ceiling}
+    ceiling_tf = ceiling["32x32x16"]["TFLOP/s"]   # the instruction the shipped kernels issue
+
     # bf16 projection GEMM (C2 shape and a long-context shape), operands N(0,1) / N(0,1/64) rounded to bf16
     def gemm(m, n_, k):
         a, w = rand(m, k), rand(k, n_, scale=1 / 64)
@@ -246,7 +266,8 @@ def bench_extras(bf, steps):
         call("bf_hip_cvt_f32_bf16_transpose", w.ptr, wbf.ptr, k, n_, None)
         ms = timed(lambda: call("bf_hip_gemm_bf16_nt", abf.ptr, wbf.ptr, c.ptr, m, n_, k, sh), 3)
         tf = 2 * m * n_ * k / ms / 1e9
-        extras[f"gemm_bf16_{m}x{n_}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_bf16_mfma": round(tf / PEAK_BF16_MFMA_TFLOPS, 3)}
+        extras[f"gemm_bf16_{m}x{n_}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1), "frac_bf16_mfma": round(tf / PEAK_BF16_MFMA_TFLOPS, 3),
+                                             "frac_of_measured_mfma_ceiling": round(tf / ceiling_tf, 3)}
         ms = timed(lambda: call("bf_hip_matmul_bf16", a.ptr, w.ptr, c.ptr, m, k, n_, 1, sh), 3)
         extras[f"matmul_bf16_fp32_io_{m}x{n_}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(2 * m * n_ * k / ms / 1e9, 1)}
     gemm(4096, 4096, 4096)
@@ -294,13 +315,27 @@ def vendor_gemm_reference(shapes):
     PyTorch calls it (torch.mm -> hipBLASLt): what a library call delivers on this box, beside the hand-written kernels
     above.  In a child process (PyTorch brings a HIP runtime of its own, which cannot share a process with the one this
     library is linked to) while this one is idle, timed as the kernels above are.  Empty where that fails."""
+    import signal
     import subprocess
+    child = None
     try:
-        proc = subprocess.run([sys.executable, "-c", _VENDOR_GEMM_CHILD, json.dumps(shapes), str(PEAK_BF16_MFMA_TFLOPS)],
-                              capture_output=True, text=True, timeout=240)
-        return json.loads(proc.stdout.strip().splitlines()[-1])
+        # a session of its own, so that whatever helpers the child starts can be ended with it by process group
+        child = subprocess.Popen([sys.executable, "-c", _VENDOR_GEMM_CHILD, json.dumps(shapes), str(PEAK_BF16_MFMA_TFLOPS)],
+                                 stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, start_new_session=True)
+        out, _ = child.communicate(timeout=240)
+        return json.loads(out.strip().splitlines()[-1])
     except Exception as err:   # no torch, an older torch without out_dtype, a time-out: no comparison
         return {"vendor_library_gemm_bf16": {"skipped": str(err)[:120]}}
+    finally:
+        if child is not None:
+            try:
+                os.killpg(child.pid, signal.SIGKILL)   # the group this function created: the child if it hangs, and anything it left
+            except (ProcessLookupError, PermissionError):
+                pass
+            try:
+                child.wait(timeout=10)
+            except Exception:
+                pass
 
 
 def lm_layers(hl, vocab, dim, seq, heads, hidden, act, blocks):
@@ -631,8 +666,12 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "attnBackwardDkvPipedKernel<64,..,store dS> (dK, dV and the dS hand-over; key-tile owner)",
                      "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                     "bf16_pipe": {"executed": round(6 * achieved, 2), "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
-                                   "frac": round(6 * achieved / PEAK_BF16_MFMA_TFLOPS, 4)},
+                     # what the kernel executes: six bf16 MFMA flops per algorithmic fp32 flop, on the bf16 matrix pipe;
+                     # mfma_busy is the share of cycles the matrix pipe is busy by counter (SQ_VALU_MFMA_BUSY_CYCLES over
+                     # GRBM_GUI_ACTIVE / 8 x 1024 SIMDs for this kernel on this workload, profiles/attention_c3_kernel_trace.md)
+                     "executed": {"pipe": "bf16", "instruction": "v_mfma_f32_32x32x16_bf16", "flops_per_launch": 6 * fl["dkv"],
+                                  "achieved": round(6 * achieved, 2), "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s",
+                                  "frac_of_pipe": round(6 * achieved / PEAK_BF16_MFMA_TFLOPS, 4), "mfma_busy": MEASURED_MFMA_BUSY["attnBackwardDkvPipedKernel"]},
                      "traffic": MEASURED_TRAFFIC_BYTES["attnBackwardDkvPipedKernel"],
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this kernel on this workload, recorded in "
                                        "profiles/attention_c3_kernel_trace.md (counters cannot be read from inside this run)",

@@ -17,6 +17,7 @@
 #include "common.hpp"
 
 #include <atomic>
+#include <type_traits>
 #include <map>
 #include <unordered_map>
 
@@ -591,6 +592,388 @@ __global__ void __launch_bounds__(256 * WAVES_N, WAVES_N) gemmBf16WideWaveKernel
     storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
+// The next tile this workgroup owns at or after `id`, walking in steps of `stride`; -1 past the end.  With the XCD order
+// some ids name no tile (the padding of a block of 32) and are skipped.
+template <int XCD_ORDER>
+__device__ __forceinline__ int seekTile(int id, int stride, int idEnd, int tilesM, int tilesN, int gmLog, int gnLog, int& tm, int& tn) {
+    for (; id < idEnd; id += stride) {
+        if (XCD_ORDER) {
+            if (tileIndexXcd(id, tilesM, tilesN, gmLog, gnLog, tm, tn)) return id;
+        } else {
+            tileIndexGrouped(id, tilesM, tilesN, tm, tn);
+            return id;
+        }
+    }
+    return -1;
+}
+
+// One eighth of a 32 x 64 accumulator share (chunk C = registers 4*(C&3).. of acc[C>>2]: rows 8*(C&3) + 4*half + 0..3),
+// stored the way storeAccumulators stores 16-byte aligned outputs.  `adds` holds this lane's four bias and residual values
+// of the chunk, loaded by the caller ahead of time.
+struct ChunkAdds { float4v b, res; };
+template <int C>
+__device__ __forceinline__ void loadChunkAdds(ChunkAdds& adds, const Epilogue& e, int M, int N, int row0, int col0, int li, int half) {
+    const int t = li & 3, col = col0 + (C >> 2) * 32 + 4 * (li >> 2), row = row0 + 8 * (C & 3) + 4 * half + t;
+    // rows and columns past the edge read the last ones (their sums are never stored): no branch around a load
+    const int rowIn = min(row, M - 1), colIn = min(col, N - 4);
+    if (e.bias) adds.b = loadf4(e.bias + colIn);
+    if (e.residual) adds.res = loadf4(e.residual + size_t(rowIn) * N + colIn);
+}
+// Cout / shift: the output the tile's columns belong to and the column where that output starts (uniform over a tile).
+template <int C, bool ADDS>
+__device__ __forceinline__ void storeChunk(const float16v (&acc)[2], const ChunkAdds& adds, const Epilogue& e, float* __restrict__ Cout,
+                                           int shift, int M, int N, int row0, int col0, int li, int half) {
+    constexpr int j = C >> 2, g = C & 3;
+    const int ld = e.splitN;
+    const int t = li & 3, colq = 4 * (li >> 2);
+    float v0 = acc[j][4 * g], v1 = acc[j][4 * g + 1], v2 = acc[j][4 * g + 2], v3 = acc[j][4 * g + 3];
+    quadTranspose(v0, v1, v2, v3, t);
+    const int row = row0 + 8 * g + 4 * half + t, col = col0 + j * 32 + colq;
+    float4v v = {v0, v1, v2, v3};
+    if constexpr (ADDS) {
+        if (e.bias) v = v + adds.b;
+        if (e.residual) v = v + adds.res;
+    }
+    // Everything but the store itself sits outside the condition: a one-instruction body is predicated, not branched
+    // around, and a store that every path issues lets the compiler count it when it waits for the loads around it
+    // (a store on one path only would make it wait for ALL outstanding memory operations, this store included).
+    float* dst = Cout + size_t(min(row, M - 1)) * ld + (min(col, N - 4) - shift);
+    if (row < M && col < N) storef4(dst, v);
+}
+
+// The sixteen- (twelve-) wavefront kernel as ONE workgroup per compute unit that walks a list of tiles (ids blockIdx.x,
+// blockIdx.x + gridDim.x, ...).  The K steps of all its tiles form one pipeline: while step g is multiplied, step g+1
+// is written to the other LDS buffer and step g+2 is loaded, whichever tile those belong to, so a tile's first steps are
+// already in flight while the tile before is still being multiplied.  A wavefront's share is only 32 registers of
+// accumulators, so it keeps the finished tile's share in a second set and stores it one eighth per K step of the next
+// tile, between the MFMAs; bias and residual values of an eighth (ADDS) are fetched at the start of the K step that
+// stores it.  Nothing of a tile's fill, drain or store is left outside the MFMA stream except for the first and the last
+// tile of a workgroup.  Outputs must be 16-byte aligned with widths that are multiples of 4 (the launcher checks).
+// Every output element sees the same MFMAs in the same order as in gemmBf16WideWaveKernel: the same bits.
+template <int XCD_ORDER, int WAVES_N, bool ADDS>
+__global__ void __launch_bounds__(256 * WAVES_N, WAVES_N) gemmBf16WidePersistentKernel(const unsigned short* __restrict__ A,
+                                                                                       const unsigned short* __restrict__ Bt, Epilogue epi,
+                                                                                       int M, int N, int K, int lda, int ldb, int gmLog,
+                                                                                       int gnLog, int idEnd) {
+    constexpr int BM = 128, BN = 64 * WAVES_N, TN = 2;
+    constexpr int ROWS = BM + BN, ROWS_PER_PASS = 32 * WAVES_N, PASSES = (ROWS + ROWS_PER_PASS - 1) / ROWS_PER_PASS;
+    constexpr int LAST_ROWS = ROWS - (PASSES - 1) * ROWS_PER_PASS;
+    static_assert(LAST_ROWS % 8 == 0, "the threads of the last pass must be whole wavefronts");
+    extern __shared__ __attribute__((aligned(16))) unsigned short lds[];   // [2][ROWS][LDS_ROW]: A rows, then Bt rows
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    const int tilesM = (M + BM - 1) / BM, tilesN = (N + BN - 1) / BN, stride = gridDim.x;
+    const int wm0 = (wave & 3) * 32, wn0 = (wave >> 2) * 64;
+    const int lr = tid >> 3, lc = (tid & 7) * 8;
+    const bool lastPass = LAST_ROWS == ROWS_PER_PASS || lr < LAST_ROWS;   // uniform over a wavefront
+    const int steps = max((K + BKK - 1) / BKK, 1);
+    int myTiles = 0;
+    {
+        int tm, tn;
+        for (int id = seekTile<XCD_ORDER>(blockIdx.x, stride, idEnd, tilesM, tilesN, gmLog, gnLog, tm, tn); id >= 0;
+             id = seekTile<XCD_ORDER>(id + stride, stride, idEnd, tilesM, tilesN, gmLog, gnLog, tm, tn))
+            ++myTiles;
+    }
+    if (myTiles == 0) return;
+    const int total = myTiles * steps;   // K steps of all this workgroup's tiles
+
+    // the load side of the pipeline: (tile, K step) of the next loads, two steps ahead of the MFMAs
+    int ldTm, ldTn, ldT = 0;
+    int ldId = seekTile<XCD_ORDER>(blockIdx.x, stride, idEnd, tilesM, tilesN, gmLog, gnLog, ldTm, ldTn);
+    const unsigned short* src[PASSES];
+    auto setSources = [&]() {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const int row = min(lr + ROWS_PER_PASS * p, ROWS - 1);
+            src[p] = row < BM ? A + size_t(min(ldTm * BM + row, M - 1)) * lda : Bt + size_t(min(ldTn * BN + row - BM, N - 1)) * ldb;
+        }
+    };
+    setSources();
+    uint4v stage[PASSES];
+    int kStaged = 0;   // K offset (this thread's chunk) of the step the stage registers hold
+    auto loadStep = [&]() {
+        kStaged = ldT * BKK + lc;
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p)
+            if (p + 1 < PASSES || lastPass) stage[p] = loadChunk(src[p], kStaged, K);
+        if (++ldT == steps) {
+            ldT = 0;
+            ldId = seekTile<XCD_ORDER>(ldId + stride, stride, idEnd, tilesM, tilesN, gmLog, gnLog, ldTm, ldTn);
+            if (ldId >= 0) setSources();
+        }
+    };
+    const int ldsW = lr * LDS_ROW + lc;
+    auto storeStep = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p)
+            if (p + 1 < PASSES || lastPass)
+                *reinterpret_cast<uint4v*>(lds + (buf * ROWS + ROWS_PER_PASS * p) * LDS_ROW + ldsW) = zeroPast(stage[p], kStaged, K);
+    };
+
+    float16v acc[TN], done[TN];   // the tile being multiplied; the finished tile whose store is in progress
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { acc[j][r] = 0.0f; done[j][r] = 0.0f; }
+    int doneRow0 = 0, doneCol0 = 0, doneShift = 0;
+    float* doneOut = epi.c[0];
+    ChunkAdds adds;
+    adds.b = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+    adds.res = adds.b;
+    bf16x8 a[2], b[2][TN];
+    int g = 0;
+    // one K step: C >= 0 also stores chunk C of the finished tile
+    auto step = [&](auto chunkTag) {
+        constexpr int C = decltype(chunkTag)::value;
+        const int par = g & 1;
+        const unsigned short* ac = lds + (par * ROWS + wm0 + li) * LDS_ROW + 8 * half;
+        const unsigned short* bc = lds + (par * ROWS + BM + wn0 + li) * LDS_ROW + 8 * half;
+        if constexpr (C >= 0 && ADDS) {
+            loadChunkAdds<C>(adds, epi, M, N, doneRow0, doneCol0, li, half);
+            __builtin_amdgcn_sched_barrier(0);   // the chunk's loads stay ahead of the step's: its wait leaves those in flight
+        }
+        if (g + 1 < total) {
+            storeStep(par ^ 1);
+            if (g + 2 < total) loadStep();
+        }
+        a[0] = *reinterpret_cast<const bf16x8*>(ac);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[0][j] = *reinterpret_cast<const bf16x8*>(bc + j * 32 * LDS_ROW);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            if (kk < 3) {
+                a[(kk + 1) & 1] = *reinterpret_cast<const bf16x8*>(ac + (kk + 1) * 16);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) b[(kk + 1) & 1][j] = *reinterpret_cast<const bf16x8*>(bc + j * 32 * LDS_ROW + (kk + 1) * 16);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk & 1], b[kk & 1][j], acc[j], 0, 0, 0);
+        }
+        if constexpr (C >= 0) storeChunk<C, ADDS>(done, adds, epi, doneOut, doneShift, M, N, doneRow0, doneCol0, li, half);
+        __syncthreads();
+        ++g;
+    };
+    auto chunkAlone = [&](auto chunkTag) {
+        constexpr int C = decltype(chunkTag)::value;
+        if constexpr (ADDS) loadChunkAdds<C>(adds, epi, M, N, doneRow0, doneCol0, li, half);
+        storeChunk<C, ADDS>(done, adds, epi, doneOut, doneShift, M, N, doneRow0, doneCol0, li, half);
+    };
+    // the first eight K steps of a tile carry the eight chunks of the tile before (a shorter contraction stores the rest at once)
+    auto stepsWithChunks = [&](int& T) {
+#define BF_CHUNK_STEP(C)                                              \
+        if (T < steps) { step(std::integral_constant<int, C>{}); ++T; } \
+        else chunkAlone(std::integral_constant<int, C>{});
+        BF_CHUNK_STEP(0) BF_CHUNK_STEP(1) BF_CHUNK_STEP(2) BF_CHUNK_STEP(3)
+        BF_CHUNK_STEP(4) BF_CHUNK_STEP(5) BF_CHUNK_STEP(6) BF_CHUNK_STEP(7)
+#undef BF_CHUNK_STEP
+    };
+
+    loadStep();
+    storeStep(0);
+    if (total > 1) loadStep();
+    __syncthreads();
+    int curTm, curTn;
+    int curId = seekTile<XCD_ORDER>(blockIdx.x, stride, idEnd, tilesM, tilesN, gmLog, gnLog, curTm, curTn);
+    for (int tile = 0; tile < myTiles; ++tile) {
+        int T = 0;
+        if (tile > 0) stepsWithChunks(T);
+        for (; T < steps; ++T) step(std::integral_constant<int, -1>{});
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            done[j] = acc[j];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+        }
+        doneRow0 = curTm * BM + wm0;
+        doneCol0 = curTn * BN + wn0;
+        {
+            const int which = (curTn * BN) / epi.splitN;   // a tile lies in one output
+            doneOut = which == 0 ? epi.c[0] : which == 1 ? epi.c[1] : epi.c[2];
+            doneShift = which * epi.splitN;
+        }
+        curId = seekTile<XCD_ORDER>(curId + stride, stride, idEnd, tilesM, tilesN, gmLog, gnLog, curTm, curTn);
+    }
+    chunkAlone(std::integral_constant<int, 0>{}); chunkAlone(std::integral_constant<int, 1>{});
+    chunkAlone(std::integral_constant<int, 2>{}); chunkAlone(std::integral_constant<int, 3>{});
+    chunkAlone(std::integral_constant<int, 4>{}); chunkAlone(std::integral_constant<int, 5>{});
+    chunkAlone(std::integral_constant<int, 6>{}); chunkAlone(std::integral_constant<int, 7>{});
+}
+
+// storeAccumulators for 16-byte aligned outputs with no branch around a memory instruction (clamped addresses, the
+// store alone under its condition): inside a kernel that keeps loads in flight across the store, the compiler can then
+// count every store when it waits for those loads instead of waiting for all memory operations.  Same values, same order
+// of additions.
+template <int TM, int TN>
+__device__ __forceinline__ void storeAccumulatorsFlat(float16v (&acc)[TM][TN], const Epilogue& e, float* __restrict__ C, int shift,
+                                                      int M, int N, int row0, int col0, int li, int half) {
+    const int ld = e.splitN;
+    const int t = li & 3, colq = 4 * (li >> 2);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = col0 + j * 32 + colq, colIn = min(col, N - 4);
+            float4v b = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (e.bias) b = loadf4(e.bias + colIn);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float v0 = acc[i][j][4 * g], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
+                quadTranspose(v0, v1, v2, v3, t);
+                const int row = row0 + i * 32 + 8 * g + 4 * half + t, rowIn = min(row, M - 1);
+                float4v v = {v0, v1, v2, v3};
+                if (e.bias) v = v + b;
+                if (e.residual) v = v + loadf4(e.residual + size_t(rowIn) * N + colIn);
+                float* dst = C + size_t(rowIn) * ld + (colIn - shift);
+                if (row < M && col < N) storef4(dst, v);
+            }
+        }
+}
+
+// The ping-pong kernel as one workgroup per compute unit walking a list of tiles, with the K steps of all its tiles as ONE
+// pipeline: the loads of a tile's first two K steps are issued, and its first step written to LDS, while the tile
+// before is still being multiplied, and the two groups of wavefronts keep their one-phase offset across tile boundaries,
+// so a group stores its accumulators while the other group multiplies.  A tile costs its K loop plus the store's issue
+// time; the workgroup launch, the first loads' latency and the pipeline's fill and drain are paid once per workgroup.
+// Same MFMAs in the same order per output element as gemmBf16PingPongKernel: the same bits.
+template <int XCD_ORDER, int BM>
+__global__ void __launch_bounds__(512, 2) gemmBf16PingPongPersistentKernel(const unsigned short* __restrict__ A,
+                                                                           const unsigned short* __restrict__ Bt, Epilogue epi,
+                                                                           int M, int N, int K, int lda, int ldb, int gmLog, int gnLog,
+                                                                           int idEnd) {
+    constexpr int BN = 256, TM = BM / 64, TN = 2, A_PASSES = BM / 64;
+    extern __shared__ __attribute__((aligned(16))) unsigned short lds[];
+    unsigned short* as = lds;                        // [2][BM][LDS_ROW]
+    unsigned short* bs = lds + 2 * BM * LDS_ROW;     // [2][256][LDS_ROW]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, li = lane & 31;
+    const int group = wave >> 2;
+    const int tilesM = (M + BM - 1) / BM, tilesN = (N + BN - 1) / BN, stride = gridDim.x;
+    const int wm0 = group * (BM / 2), wn0 = (wave & 3) * 64;
+    const int lr = tid >> 3, lc = (tid & 7) * 8;     // 64 rows x 128 bytes per pass
+    const int steps = max((K + BKK - 1) / BKK, 1);
+    int myTiles = 0;
+    {
+        int tm, tn;
+        for (int id = seekTile<XCD_ORDER>(blockIdx.x, stride, idEnd, tilesM, tilesN, gmLog, gnLog, tm, tn); id >= 0;
+             id = seekTile<XCD_ORDER>(id + stride, stride, idEnd, tilesM, tilesN, gmLog, gnLog, tm, tn))
+            ++myTiles;
+    }
+    if (myTiles == 0) return;
+    const int total = myTiles * steps;
+    const bool wideStores = ((N | epi.splitN) & 3) == 0 &&
+                            ((reinterpret_cast<uintptr_t>(epi.c[0]) | reinterpret_cast<uintptr_t>(epi.c[1]) | reinterpret_cast<uintptr_t>(epi.c[2]) |
+                              reinterpret_cast<uintptr_t>(epi.bias) | reinterpret_cast<uintptr_t>(epi.residual)) & 15u) == 0;
+
+    int ldTm, ldTn, ldT = 0;
+    int ldId = seekTile<XCD_ORDER>(blockIdx.x, stride, idEnd, tilesM, tilesN, gmLog, gnLog, ldTm, ldTn);
+    const unsigned short* aRow[A_PASSES];
+    const unsigned short* bRow[4];
+    auto setSources = [&]() {
+#pragma unroll
+        for (int i = 0; i < A_PASSES; ++i) aRow[i] = A + size_t(min(ldTm * BM + lr + 64 * i, M - 1)) * lda;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bRow[i] = Bt + size_t(min(ldTn * BN + lr + 64 * i, N - 1)) * ldb;
+    };
+    setSources();
+    uint4v stageA[A_PASSES], stageB[4];
+    int kA = 0, kB = 0;   // K offsets (this thread's chunk) of the steps the stage registers hold
+    auto loadA = [&]() {
+        kA = ldT * BKK + lc;
+#pragma unroll
+        for (int i = 0; i < A_PASSES; ++i) stageA[i] = loadChunk(aRow[i], kA, K);
+    };
+    auto loadB = [&]() {   // the second operand of a step: the load side then moves on to the next step
+        kB = ldT * BKK + lc;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) stageB[i] = loadChunk(bRow[i], kB, K);
+        if (++ldT == steps) {
+            ldT = 0;
+            ldId = seekTile<XCD_ORDER>(ldId + stride, stride, idEnd, tilesM, tilesN, gmLog, gnLog, ldTm, ldTn);
+            if (ldId >= 0) setSources();
+        }
+    };
+    float16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    const int ldsW = lr * LDS_ROW + lc;
+    loadA();
+    loadB();
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<uint4v*>(as + ldsW + 64 * i * LDS_ROW) = zeroPast(stageA[i], kA, K);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(bs + ldsW + 64 * i * LDS_ROW) = zeroPast(stageB[i], kB, K);
+    if (total > 1) {
+        loadA();
+        loadB();
+    }
+    __syncthreads();
+    if (group == 1) __builtin_amdgcn_s_barrier();    // group 1 runs one phase late from here to the end
+    int curTm, curTn;
+    int curId = seekTile<XCD_ORDER>(blockIdx.x, stride, idEnd, tilesM, tilesN, gmLog, gnLog, curTm, curTn);
+    bf16x8 a[2][TM], b[2][TN];
+    int g = 0;
+    for (int tile = 0; tile < myTiles; ++tile) {
+        for (int T = 0; T < steps; ++T, ++g) {
+            const int par = g & 1;
+            const unsigned short* ac = as + (par * BM + wm0 + li) * LDS_ROW + 8 * half;
+            const unsigned short* bc = bs + (par * BN + wn0 + li) * LDS_ROW + 8 * half;
+            unsigned short* aw = as + (par ^ 1) * BM * LDS_ROW + ldsW;
+            unsigned short* bw = bs + (par ^ 1) * BN * LDS_ROW + ldsW;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                // ---- memory phase
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) a[kk][i] = *reinterpret_cast<const bf16x8*>(ac + i * 32 * LDS_ROW + h * 32 + kk * 16);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) b[kk][j] = *reinterpret_cast<const bf16x8*>(bc + j * 32 * LDS_ROW + h * 32 + kk * 16);
+                }
+                if (g + 1 < total) {
+                    if (h == 0) {
+#pragma unroll
+                        for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<uint4v*>(aw + 64 * i * LDS_ROW) = zeroPast(stageA[i], kA, K);
+                        if (g + 2 < total) loadA();
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4v*>(bw + 64 * i * LDS_ROW) = zeroPast(stageB[i], kB, K);
+                        if (g + 2 < total) loadB();
+                    }
+                }
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                // ---- compute phase
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+            }
+        }
+        if (wideStores) {
+            const int which = (curTn * BN) / epi.splitN;   // a tile lies in one output
+            float* out = which == 0 ? epi.c[0] : which == 1 ? epi.c[1] : epi.c[2];
+            storeAccumulatorsFlat<TM, TN>(acc, epi, out, which * epi.splitN, M, N, curTm * BM + wm0, curTn * BN + wn0, li, half);
+        } else {
+            storeAccumulators<TM, TN>(acc, epi, M, N, curTm * BM + wm0, curTn * BN + wn0, li, half);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        curId = seekTile<XCD_ORDER>(curId + stride, stride, idEnd, tilesM, tilesN, gmLog, gnLog, curTm, curTn);
+    }
+    if (group == 0) __builtin_amdgcn_s_barrier();    // pairs with group 1's last barrier
+}
+
 // out = sum over slices of partial[s*sliceStride + i] (+ bias[i % N] + residual[i]), slices added in index order
 // (deterministic), written through the epilogue's output split.  sliceStride is a multiple of 4; `vec` says
 // that every pointer is 16-byte aligned and N and splitN are multiples of 4.
@@ -758,6 +1141,66 @@ __global__ void __launch_bounds__(512, 2) gemmBf16TnPingPongKernel(const unsigne
     storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
+// What the matrix pipes deliver when nothing else runs: the K loop of the 256 x 256 ping-pong tile (eight wavefronts of a
+// 128 x 64 share each, two per SIMD) with every memory instruction removed.  The operand fragments of one 64-deep K step
+// are read once from `operands` and stay in registers; `steps` K steps are then multiplied out of them.  SHAPE 0: 32 MFMAs
+// 32x32x16 per step and wavefront; SHAPE 1: 64 MFMAs 16x16x32.  One workgroup per compute unit; the accumulators' sums go
+// to `out` so that the loop cannot be removed.
+template <int SHAPE>
+__global__ void __launch_bounds__(512, 2) mfmaOnlyKernel(const uint4v* __restrict__ operands, float* __restrict__ out, int steps) {
+    const int tid = threadIdx.x;
+    bf16x8 fa[16], fb[8];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) fa[i] = __builtin_bit_cast(bf16x8, operands[(tid * 24 + i) & 4095]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) fb[i] = __builtin_bit_cast(bf16x8, operands[(tid * 24 + 16 + i) & 4095]);
+    float sum = 0.0f;
+    if constexpr (SHAPE == 0) {
+        float16v acc[4][2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        for (int t = 0; t < steps; ++t) {
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk * 4 + i], fb[kk * 2 + j], acc[i][j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum += acc[i][j][r];
+    } else {
+        float4v acc[8][4];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int t = 0; t < steps; ++t) {
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[kk * 8 + i], fb[kk * 4 + j], acc[i][j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sum += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+    }
+    out[size_t(blockIdx.x) * 512 + tid] = sum;
+}
+
 template <typename Kernel>
 int allowSharedMemory(Kernel kernel, size_t smem) {
     return allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
@@ -766,7 +1209,7 @@ int allowSharedMemory(Kernel kernel, size_t smem) {
 // slices > 1: K is cut into `slices` ranges of kPer (a multiple of 64) and range i writes to epi.c[0] + i * sliceStride
 template <int BM>
 int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
-                   size_t lda, size_t ldb, hipStream_t s, size_t slices = 1, size_t kPer = 0, size_t sliceStride = 0) {
+                   size_t lda, size_t ldb, hipStream_t s, size_t slices = 1, size_t kPer = 0, size_t sliceStride = 0, bool persistent = true) {
     if (slices <= 1) { slices = 1; kPer = K; sliceStride = 0; }
     const size_t tilesM = (M + BM - 1) / BM, tilesN = (N + 255) / 256;
     constexpr size_t smem = size_t(2) * (BM + 256) * LDS_ROW * sizeof(unsigned short);
@@ -781,6 +1224,20 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
     }
     // blocks are dealt to XCDs eight at a time: only worth it when that deal is (nearly) even
     const bool xcdOrder = blocks * 32 <= (tilesM * tilesN) * 5 / 4 && (blocks % 8 == 0 || blocks >= 64);
+    const size_t cus = size_t(computeUnits());
+    if (persistent && slices == 1 && tilesM * tilesN > cus) {
+        // one workgroup per compute unit walks ids blockIdx.x + r * cus (see launchWideWave)
+        const bool xcd = xcdOrder && cus % 8 == 0;
+        const size_t idEnd = xcd ? (blocks + 7) / 8 * 8 * 32 : tilesM * tilesN;
+        if (idEnd >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+        auto kernel = xcd ? gemmBf16PingPongPersistentKernel<1, BM> : gemmBf16PingPongPersistentKernel<0, BM>;
+        int st = allowSharedMemory(kernel, smem);
+        if (st != BF_OK) return st;
+        kernel<<<dim3(unsigned(cus)), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), xcd ? gmLog : 0, xcd ? gnLog : 0,
+                                                      int(idEnd));
+        BF_LAUNCH_CHECK();
+        return BF_OK;
+    }
     if (xcdOrder) {
         size_t grid = (blocks + 7) / 8 * 8 * 32;
         if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
@@ -804,7 +1261,7 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
 
 template <int WAVES_N>
 int launchWideWave(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
-                   size_t lda, size_t ldb, hipStream_t s) {
+                   size_t lda, size_t ldb, hipStream_t s, bool persistent = true) {
     constexpr size_t BN = 64 * WAVES_N;
     const size_t tilesM = (M + 127) / 128, tilesN = (N + BN - 1) / BN;
     constexpr size_t smem = size_t(2) * (128 + BN) * LDS_ROW * sizeof(unsigned short);
@@ -819,6 +1276,27 @@ int launchWideWave(const unsigned short* A, const unsigned short* Bt, const Epil
     const bool xcdOrder = blocks * 32 <= (tilesM * tilesN) * 5 / 4 && (blocks % 8 == 0 || blocks >= 64);
     const size_t grid = xcdOrder ? (blocks + 7) / 8 * 8 * 32 : tilesM * tilesN;
     if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+    const size_t cus = size_t(computeUnits());
+    const bool wideStores = ((N | size_t(epi.splitN)) & 3) == 0 &&
+                            ((reinterpret_cast<uintptr_t>(epi.c[0]) | reinterpret_cast<uintptr_t>(epi.c[1]) | reinterpret_cast<uintptr_t>(epi.c[2]) |
+                              reinterpret_cast<uintptr_t>(epi.bias) | reinterpret_cast<uintptr_t>(epi.residual)) & 15u) == 0;
+    // With sixteen wavefronts (128 registers each) the second accumulator set leaves no room for the bias and residual
+    // values fetched ahead: such products keep the one-tile-per-workgroup form.
+    const bool adds = epi.bias || epi.residual;
+    constexpr bool kAddsFit = WAVES_N < 4;
+    if (persistent && wideStores && tilesM * tilesN > cus && (!adds || kAddsFit)) {
+        // one workgroup per compute unit walks ids blockIdx.x + r * cus; with a CU count that is a multiple of 8 a workgroup
+        // stays on its XCD and round r of the XCD order is one block of 32 tiles per XCD, as in the one-tile-per-workgroup launch
+        const bool xcd = xcdOrder && cus % 8 == 0;
+        auto kernel = xcd ? (adds ? gemmBf16WidePersistentKernel<1, WAVES_N, kAddsFit> : gemmBf16WidePersistentKernel<1, WAVES_N, false>)
+                          : (adds ? gemmBf16WidePersistentKernel<0, WAVES_N, kAddsFit> : gemmBf16WidePersistentKernel<0, WAVES_N, false>);
+        int st = allowSharedMemory(kernel, smem);
+        if (st != BF_OK) return st;
+        kernel<<<dim3(unsigned(cus)), 256 * WAVES_N, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), xcd ? gmLog : 0,
+                                                                 xcd ? gnLog : 0, int(xcd ? grid : tilesM * tilesN));
+        BF_LAUNCH_CHECK();
+        return BF_OK;
+    }
     auto kernel = xcdOrder ? gemmBf16WideWaveKernel<1, WAVES_N> : gemmBf16WideWaveKernel<0, WAVES_N>;
     int st = allowSharedMemory(kernel, smem);
     if (st != BF_OK) return st;
@@ -934,12 +1412,16 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
     if (M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
     const size_t cus = size_t(computeUnits());
     switch (g_ntRoute.load()) {   // a kernel named by the caller (tests and tuning); BF_GEMM_ROUTE_AUTO otherwise
-        case BF_GEMM_ROUTE_PINGPONG_256: return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
-        case BF_GEMM_ROUTE_PINGPONG_128: return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s);
-        case BF_GEMM_ROUTE_WIDE_256: return launchWideWave<4>(A, Bt, epi, M, N, K, lda, ldb, s);
+        case BF_GEMM_ROUTE_PINGPONG_256: return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
+        case BF_GEMM_ROUTE_PINGPONG_128: return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
+        case BF_GEMM_ROUTE_PINGPONG_256_PERSISTENT: return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
+        case BF_GEMM_ROUTE_PINGPONG_128_PERSISTENT: return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s);
+        case BF_GEMM_ROUTE_WIDE_256: return launchWideWave<4>(A, Bt, epi, M, N, K, lda, ldb, s, false);
+        case BF_GEMM_ROUTE_WIDE_256_PERSISTENT: return launchWideWave<4>(A, Bt, epi, M, N, K, lda, ldb, s, true);
         case BF_GEMM_ROUTE_WIDE_192:
+        case BF_GEMM_ROUTE_WIDE_192_PERSISTENT:
             if (size_t(epi.splitN) != N && epi.splitN % 192 != 0) return failInvalid("gemm_bf16", "192-wide tiles need outputs whose width is a multiple of 192");
-            return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s);
+            return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s, g_ntRoute.load() == BF_GEMM_ROUTE_WIDE_192_PERSISTENT);
         default: break;
     }
     // 256x256 ping-pong tiles once they give three quarters of the CUs a tile; otherwise 128x128 tiles,
@@ -963,8 +1445,9 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
         if (narrow < wide && narrow < big) return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s);
         if (wide < big) return launchWideWave<4>(A, Bt, epi, M, N, K, lda, ldb, s);
     }
-    if (bigTime <= halfTime && bigTime < 1e30) return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
-    if (halfTime < 1e30) return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s);
+    // (the ping-pong kernel keeps one tile per workgroup: its tile-walking form measured no faster, see below)
+    if (bigTime <= halfTime && bigTime < 1e30) return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
+    if (halfTime < 1e30) return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
     // Few tiles but a long contraction (the weight-gradient products, K = all tokens): the same kernel with K cut into
     // slices, one workgroup per (tile, slice), partial products summed in slice order by a second kernel.  More slices
     // fill more CUs but write and re-read more partial sums; the estimate below (K steps at the measured ~1.4 us per
@@ -990,8 +1473,8 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
             Scratch partial(sl * sliceStride * sizeof(float));
             if (partial.status != BF_OK) return partial.status;
             Epilogue plain{{partial.as<float>(), nullptr, nullptr}, int(N), nullptr, nullptr};
-            int st = bestForm == 0 ? launchPingPong<256>(A, Bt, plain, M, N, K, lda, ldb, s, sl, kPer, sliceStride)
-                                   : launchPingPong<128>(A, Bt, plain, M, N, K, lda, ldb, s, sl, kPer, sliceStride);
+            int st = bestForm == 0 ? launchPingPong<256>(A, Bt, plain, M, N, K, lda, ldb, s, sl, kPer, sliceStride, false)
+                                   : launchPingPong<128>(A, Bt, plain, M, N, K, lda, ldb, s, sl, kPer, sliceStride, false);
             if (st != BF_OK) return st;
             const int vec = ((reinterpret_cast<uintptr_t>(epi.c[0]) | reinterpret_cast<uintptr_t>(epi.c[1]) |
                               reinterpret_cast<uintptr_t>(epi.c[2]) | reinterpret_cast<uintptr_t>(epi.residual) |
@@ -1699,8 +2182,20 @@ int bf_hip_feedforward_bf16_backward_img(const float* x, const uint16_t* xImage,
     return st;
 }
 
+int bf_hip_mfma_only_loop(const uint16_t* operands, float* out, int shape, int workgroups, int kSteps, bf_stream_t stream) {
+    BF_REQUIRE(operands && out, "NULL pointer");
+    BF_REQUIRE((reinterpret_cast<uintptr_t>(operands) & 15u) == 0, "operands must be 16-byte aligned");
+    BF_REQUIRE(shape == 0 || shape == 1, "shape: 0 (32x32x16) or 1 (16x16x32)");
+    BF_REQUIRE(workgroups > 0 && workgroups <= 65536 && kSteps > 0, "workgroups in 1..65536, kSteps > 0");
+    hipStream_t s = asStream(stream);
+    if (shape == 0) bf::mfmaOnlyKernel<0><<<dim3(unsigned(workgroups)), 512, 0, s>>>(reinterpret_cast<const uint4v*>(operands), out, kSteps);
+    else bf::mfmaOnlyKernel<1><<<dim3(unsigned(workgroups)), 512, 0, s>>>(reinterpret_cast<const uint4v*>(operands), out, kSteps);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
 int bf_hip_gemm_bf16_set_route(int route) {
-    BF_REQUIRE(route >= BF_GEMM_ROUTE_AUTO && route <= BF_GEMM_ROUTE_WIDE_192, "unknown route");
+    BF_REQUIRE(route >= BF_GEMM_ROUTE_AUTO && route <= BF_GEMM_ROUTE_PINGPONG_128_PERSISTENT, "unknown route");
     bf::g_ntRoute.store(route);
     return BF_OK;
 }

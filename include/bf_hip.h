@@ -339,9 +339,22 @@ enum {
     BF_GEMM_ROUTE_PINGPONG_256 = 1,   /* 256 x 256 tiles, eight wavefronts in two alternating groups */
     BF_GEMM_ROUTE_PINGPONG_128 = 2,   /* 128 x 256 tiles, same schedule */
     BF_GEMM_ROUTE_WIDE_256 = 3,       /* 128 x 256 tiles, sixteen wavefronts */
-    BF_GEMM_ROUTE_WIDE_192 = 4        /* 128 x 192 tiles, twelve wavefronts */
+    BF_GEMM_ROUTE_WIDE_192 = 4,       /* 128 x 192 tiles, twelve wavefronts */
+    /* one workgroup per compute unit walking a list of tiles, K steps pipelined across tile boundaries (products of
+     * more tiles than compute units; with fewer they fall back to the form of the same tile shape above) */
+    BF_GEMM_ROUTE_WIDE_256_PERSISTENT = 5,
+    BF_GEMM_ROUTE_WIDE_192_PERSISTENT = 6,
+    BF_GEMM_ROUTE_PINGPONG_256_PERSISTENT = 7,
+    BF_GEMM_ROUTE_PINGPONG_128_PERSISTENT = 8
 };
 int bf_hip_gemm_bf16_set_route(int route);
+/* A measurement aid with no counterpart in the reference: the K loop of the 256 x 256 bf16 GEMM tile with every memory
+ * instruction removed (operand fragments held in registers), `workgroups` workgroups of eight wavefronts, `kSteps`
+ * 64-deep K steps each = 2*256*256*64 flops per step and workgroup.  shape 0 issues v_mfma_f32_32x32x16_bf16, shape 1
+ * v_mfma_f32_16x16x32_bf16.  `operands`: 32768 bf16 values the fragments are drawn from (16-byte aligned);
+ * `out`: workgroups*512 floats (sums of the accumulators, so the loop has a result).  What this loop reaches on a box
+ * is the ceiling of any bf16 GEMM there: the matrix pipes' rate at the clock the chip holds under that load. */
+int bf_hip_mfma_only_loop(const uint16_t* operands, float* out, int shape, int workgroups, int kSteps, bf_stream_t stream);
 /* invalidateBf16WeightCache: ops.hpp:80 */
 int bf_hip_invalidate_bf16_weight_cache(void);
 

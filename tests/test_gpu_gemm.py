@@ -185,15 +185,20 @@ def test_bf16_projection_large_tile_kernel(hip, oracle, rng, m, k, n):
     assert_close(c, expected, tol=1e-4, what="bf16 fwd (large tiles) vs rounded operands")
 
 
-ROUTES = {"ping-pong 256": 1, "ping-pong 128": 2, "sixteen wavefronts, 128 x 256": 3, "twelve wavefronts, 128 x 192": 4}
+ROUTES = {"ping-pong 256": 1, "ping-pong 128": 2, "sixteen wavefronts, 128 x 256": 3, "twelve wavefronts, 128 x 192": 4,
+          "sixteen wavefronts, one workgroup per CU walking tiles": 5, "twelve wavefronts, walking tiles": 6,
+          "ping-pong 256, walking tiles": 7, "ping-pong 128, walking tiles": 8}
 
 
-@pytest.mark.parametrize("m,k,n", [(8192, 768, 768), (8192, 200, 2304), (700, 136, 1000), (1, 8, 1), (130, 72, 193), (4100, 64, 4093), (257, 1032, 385)])
+@pytest.mark.parametrize("m,k,n", [(8192, 768, 768), (8192, 200, 2304), (700, 136, 1000), (1, 8, 1), (130, 72, 193), (4100, 64, 4093), (257, 1032, 385),
+                                   (4100, 1032, 4096), (9000, 520, 2500)])
 def test_bf16_gemm_every_tile_form_on_the_same_operands(hip, oracle, rng, m, k, n):
     """Each large-tile kernel named through bf_hip_gemm_bf16_set_route, whatever the cost estimate would pick: float64 of
     the rounded operands to 1e-4 for one of them, and the same bits from all (an output element is accumulated over k
     in the same order by every form).  Shapes: whole rounds of tiles for the 192-wide form, ragged edges in both
-    directions, a K tail, single tiles, one element."""
+    directions, a K tail, single tiles, one element; for the forms that walk a list of tiles per workgroup, products of
+    more tiles than compute units with contractions shorter and longer than the eight K steps over which a finished tile
+    is stored, and a ragged last tile in both directions."""
     D, call = hip.DeviceTensor, hip.capi.call
     a, b = oracle.roundToBf16(r(rng, m, k)), oracle.roundToBf16(r(rng, n, k, scale=0.1))
     ai, bi = D((m, k), itemsize=2), D((n, k), itemsize=2)
@@ -238,6 +243,36 @@ def test_bf16_shared_input_projections_on_192_wide_tiles(hip, rng):
     for route, outs in results.items():
         for got, single in zip(outs, singles):
             assert_bits_equal(got, single, f"route {route}: split output vs its own product")
+
+
+@pytest.mark.parametrize("route", [5, 6, 7, 8])
+@pytest.mark.parametrize("m,k,n,with_bias,with_residual", [(4100, 72, 4096, True, True), (8192, 648, 2304, True, False), (5000, 1100, 3072, False, True),
+                                                           (4100, 136, 4093, True, True)])
+def test_bf16_linear_with_adds_on_the_tile_walking_forms(hip, rng, route, m, k, n, with_bias, with_residual):
+    """bias and residual added in the store of the kernels that walk a list of tiles (the sixteen- and twelve-wavefront
+    forms fetch an eighth of a tile's bias and residual values a K step ahead of storing it): the same bits as the
+    one-tile-per-workgroup form of the same tile shape, on products of more tiles than compute units, with contractions of
+    2, 11 and 18 K steps, and a width that is no multiple of four (which the wide forms leave to the plain kernel)."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    a, w = r(rng, m, k), r(rng, k, n, scale=0.1)
+    bias, res = r(rng, n), r(rng, m, n)
+    da, dw = D.fromHost(a), D.fromHost(w)
+    db, dr = (D.fromHost(bias) if with_bias else None), (D.fromHost(res) if with_residual else None)
+    outs = {}
+    try:
+        for rt in (route, {5: 3, 6: 4, 7: 1, 8: 2}[route]):
+            call("bf_hip_gemm_bf16_set_route", rt)
+            out = D.fromHost(np.full((m, n), 7.0, f32))
+            call("bf_hip_linear_bf16", da.ptr, dw.ptr, db.ptr if db else None, dr.ptr if dr else None, out.ptr, m, k, n, 0, None)
+            outs[rt] = out.toHost()
+    finally:
+        call("bf_hip_gemm_bf16_set_route", 0)
+    (r1, o1), (r2, o2) = outs.items()
+    assert_bits_equal(o1, o2, f"route {r1} vs route {r2}")
+    plain = a.astype(np.float64)  # float64 of rounded operands on a sample of rows, to 2e-2 of the bf16 contract
+    rows = rng.integers(0, m, 16)
+    ref = plain[rows] @ w.astype(np.float64) + (bias if with_bias else 0) + (res[rows] if with_residual else 0)
+    assert_close(o1[rows], ref.astype(f32), tol=2e-2, what="sampled rows against float64")
 
 
 @pytest.mark.parametrize("m,k,n", [(33, 40, 24), (300, 72, 520), (2100, 136, 3000), (70, 4100, 90), (6200, 72, 1501), (4100, 136, 4093),
