@@ -135,6 +135,7 @@ SIGNATURES = {
     "bf_hip_attention_backward_dkv_ds": [P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_attention_backward_dq_from_ds": [P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_mse": [P, P, P, P, c_size, c_int, S],
+    "bf_hip_mse_img": [P, P, P, P, P, c_size, c_int, S],
     "bf_hip_cross_entropy": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse_img": [P, P, P, P, P, c_size, c_size, c_int, S],

@@ -47,10 +47,12 @@ __global__ void __launch_bounds__(1024) finishScaledSumKernel(const float* __res
     }
 }
 
+// gradImage (VEC == 4 only; may be NULL): the bf16 image of the gradient, written in the same pass (8 bytes per thread
+// and step), for a model whose last layer's gradient products read it.
 template <int VEC, bool NT = false>
 __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pred, const float* __restrict__ target,
                                                     float* __restrict__ grad, float* __restrict__ partial, size_t n,
-                                                    float gradScale) {
+                                                    float gradScale, unsigned short* __restrict__ gradImage = nullptr) {
     __shared__ float lds[16];
     float acc = 0.0f;
     size_t stride = size_t(gridDim.x) * blockDim.x;
@@ -59,12 +61,19 @@ __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pr
         for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += stride) {
             float4v d = ldf4<NT>(pred + 4 * i) - ldf4<NT>(target + 4 * i);
             acc += d.x * d.x + d.y * d.y + d.z * d.z + d.w * d.w;
-            stf4<NT>(grad + 4 * i, d * gradScale);
+            const float4v gv = d * gradScale;
+            stf4<NT>(grad + 4 * i, gv);
+            if (gradImage) {
+                const uint2v packed = {unsigned(toBf16Bits(gv.x)) | (unsigned(toBf16Bits(gv.y)) << 16),
+                                       unsigned(toBf16Bits(gv.z)) | (unsigned(toBf16Bits(gv.w)) << 16)};
+                stu2<NT>(gradImage + 4 * i, packed);
+            }
         }
         for (size_t i = n4 * 4 + size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
             float d = pred[i] - target[i];
             acc += d * d;
             grad[i] = d * gradScale;
+            if (gradImage) gradImage[i] = toBf16Bits(d * gradScale);
         }
     } else {
         for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
@@ -303,6 +312,11 @@ extern "C" {
 
 int bf_hip_mse(const float* pred, const float* target, float* grad, float* lossSum, size_t n, int accumulate,
                bf_stream_t stream) {
+    return bf_hip_mse_img(pred, target, grad, nullptr, lossSum, n, accumulate, stream);
+}
+
+int bf_hip_mse_img(const float* pred, const float* target, float* grad, uint16_t* gradImage, float* lossSum, size_t n, int accumulate,
+                   bf_stream_t stream) {
     BF_REQUIRE(lossSum != nullptr, "lossSum is NULL");
     hipStream_t s = asStream(stream);
     if (n == 0) {
@@ -314,10 +328,13 @@ int bf_hip_mse(const float* pred, const float* target, float* grad, float* lossS
     Scratch partial(grid * sizeof(float));
     if (partial.status != BF_OK) return partial.status;
     float gradScale = 2.0f / float(n);
-    if (aligned16(pred) && aligned16(target) && aligned16(grad) && streamsPastCache(n * 12))
-        mseKernel<4, true><<<grid, kBlock, 0, s>>>(pred, target, grad, partial.as<float>(), n, gradScale);
-    else if (aligned16(pred) && aligned16(target) && aligned16(grad))
-        mseKernel<4><<<grid, kBlock, 0, s>>>(pred, target, grad, partial.as<float>(), n, gradScale);
+    const bool vec = aligned16(pred) && aligned16(target) && aligned16(grad);
+    BF_REQUIRE(gradImage == nullptr || (vec && (reinterpret_cast<uintptr_t>(gradImage) & 7u) == 0),
+               "a gradient image needs 16-byte aligned tensors and an 8-byte aligned image");
+    if (vec && streamsPastCache(n * 12))
+        mseKernel<4, true><<<grid, kBlock, 0, s>>>(pred, target, grad, partial.as<float>(), n, gradScale, gradImage);
+    else if (vec)
+        mseKernel<4><<<grid, kBlock, 0, s>>>(pred, target, grad, partial.as<float>(), n, gradScale, gradImage);
     else
         mseKernel<1><<<grid, kBlock, 0, s>>>(pred, target, grad, partial.as<float>(), n, gradScale);
     BF_LAUNCH_CHECK();

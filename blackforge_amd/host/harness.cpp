@@ -25,6 +25,9 @@ struct Handle {
     hip::DeviceTensor lossGrad;
     hip::DeviceTensor lossAccumulator;
     std::vector<hip::Parameter*> params;
+    // no parameter value has changed since the model's last forward pass: every path that changes one (optimizer steps,
+    // replays, training runs, checkpoint loads, bfh_model_weights_changed for uploads through the raw pointers) clears it
+    bool weightImagesCurrent = false;
 };
 
 template <typename Fn>
@@ -95,6 +98,7 @@ int bfh_model_forward(void* h, const float* input, int rank, const size_t* shape
     return guarded([&] {
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
         handle->output = handle->model->forward(in.tensor, trusted != 0);
+        handle->weightImagesCurrent = true;
         if (output) *output = handle->output.data();
         if (outCount) *outCount = handle->output.elementCount();
     });
@@ -140,6 +144,7 @@ int bfh_model_adamw_step(void* h, float lr, float beta1, float beta2, float eps,
     return guarded([&] {
         if (!handle->adamw) handle->adamw = std::make_unique<hip::AdamW>(lr, beta1, beta2, eps, weightDecay);
         handle->adamw->setLearningRate(lr);
+        handle->weightImagesCurrent = false;
         handle->adamw->step(handle->params);
     });
 }
@@ -149,8 +154,15 @@ int bfh_model_sgd_step(void* h, float lr) {
     return guarded([&] {
         if (!handle->sgd) handle->sgd = std::make_unique<hip::SGD>(lr);
         handle->sgd->setLearningRate(lr);
+        handle->weightImagesCurrent = false;
         handle->sgd->step(handle->params);
     });
+}
+
+// To be called after parameter values were changed through the pointers of bfh_model_param_info (an upload).
+int bfh_model_weights_changed(void* h) {
+    static_cast<Handle*>(h)->weightImagesCurrent = false;
+    return 0;
 }
 
 // One whole training step with no host synchronisation: zeroGrad, forward, loss (accumulated on the
@@ -160,8 +172,11 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
     Handle* handle = static_cast<Handle*>(h);
     return guarded([&] {
         handle->model->zeroGrad();
+        // the caller's input buffer outlives the step, so the model keeps a view of it instead of a copy; weight images
+        // made by the previous step stay in use when nothing has changed a weight since
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
-        handle->output = handle->model->forward(in.tensor, true);
+        handle->output = handle->model->forward(std::move(in.tensor), true, handle->weightImagesCurrent);
+        handle->weightImagesCurrent = true;
         if (lossKind == 0 || lossKind == 2) {
             std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
             Borrowed tgt(target, {rows});
@@ -170,12 +185,13 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
                                              : hip::softmaxCrossEntropyMaskedAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
         } else {
             Borrowed tgt(target, handle->output.shape());
-            handle->lossGrad = hip::meanSquaredErrorAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
+            handle->lossGrad = hip::meanSquaredErrorAccumulate(handle->output, tgt.tensor, handle->lossAccumulator, handle->model->usesBf16());
         }
         handle->model->backward(handle->lossGrad, true);
         if (optimizer == 1) {
             if (!handle->adamw) handle->adamw = std::make_unique<hip::AdamW>(lr, 0.9F, 0.999F, 1e-8F, 0.01F);
             handle->adamw->setLearningRate(lr);
+            handle->weightImagesCurrent = false;
             handle->adamw->step(handle->params);
         }
     });
@@ -210,6 +226,7 @@ int bfh_captured_step_run(void* h, void* step, float lr, int optimizer) {
         hip::Optimizer* opt = optimizer == 1 ? static_cast<hip::Optimizer*>(handle->adamw.get()) : handle->sgd.get();
         hip::require(opt != nullptr, "captured_step_run: no such optimizer on this model");
         opt->setLearningRate(lr);
+        handle->weightImagesCurrent = false;
         static_cast<hip::CapturedTrainStep*>(step)->run();
     });
 }
@@ -243,6 +260,7 @@ int bfh_model_run_training(void* h, const char* datasetPath, int lossKind, int o
         options.cosineSchedule = cosineSchedule != 0;
         options.fromCheckpointPath = fromCheckpoint ? fromCheckpoint : "";
         options.saveCheckpointPath = saveCheckpoint ? saveCheckpoint : "";
+        handle->weightImagesCurrent = false;
         hip::TrainRunResult result = hip::runTraining(*handle->model, dataset, options, nullptr);
         for (std::size_t i = 0; i < result.epochLosses.size(); ++i) epochLosses[i] = result.epochLosses[i];
     });
@@ -258,6 +276,7 @@ int bfh_model_load_checkpoint(void* h, const char* path) {
     Handle* handle = static_cast<Handle*>(h);
     return guarded([&] {
         hip::loadCheckpoint(*handle->model, path);
+        handle->weightImagesCurrent = false;
         handle->params = handle->model->parameters();
     });
 }

@@ -42,6 +42,7 @@ def load() -> ctypes.CDLL:
         lib.bfh_model_loss_grad.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_size_t)]
         lib.bfh_model_backward.argtypes = [ctypes.c_void_p, ctypes.c_int]
         lib.bfh_model_zero_grad.argtypes = [ctypes.c_void_p]
+        lib.bfh_model_weights_changed.argtypes = [ctypes.c_void_p]
         lib.bfh_model_adamw_step.argtypes = [ctypes.c_void_p] + [ctypes.c_float] * 5
         lib.bfh_model_sgd_step.argtypes = [ctypes.c_void_p, ctypes.c_float]
         lib.bfh_model_train_step.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_size_t),
@@ -135,6 +136,7 @@ class HostModel:
         host = np.ascontiguousarray(host, np.float32).reshape(-1)
         assert host.size == self.counts[i]
         capi.call("bf_hip_memcpy_h2d", self._value_ptrs[i], host.ctypes.data_as(ctypes.c_void_p), host.nbytes)
+        _check(load().bfh_model_weights_changed(self.handle))   # the model's cached bf16 weight images are stale now
 
     def _read(self, ptr, count) -> np.ndarray:
         out = np.empty(count, np.float32)

@@ -451,6 +451,10 @@ int bf_hip_attention_backward_dq_from_ds(const float* dS, const float* k, float*
 /* meanSquaredError[Accumulate]: grad = 2 (p - t) / n, lossSum = sum (p - t)^2 */
 int bf_hip_mse(const float* pred, const float* target, float* grad, float* lossSum, size_t n, int accumulate,
                bf_stream_t stream);
+/* The same with the gradient's bf16 image written too (gradImage[n], round to nearest even; needs 16-byte aligned
+ * tensors): the gradient products of a bf16 model's last linear layer read it in place of a conversion pass. */
+int bf_hip_mse_img(const float* pred, const float* target, float* grad, uint16_t* gradImage, float* lossSum, size_t n, int accumulate,
+                   bf_stream_t stream);
 /* softmaxCrossEntropy[Accumulate]: dense targets */
 int bf_hip_cross_entropy(const float* logits, const float* target, float* grad, float* lossSum, size_t rows,
                          size_t classes, int accumulate, bf_stream_t stream);

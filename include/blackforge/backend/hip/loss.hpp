@@ -90,10 +90,14 @@ inline LossResult softmaxCrossEntropyMasked(const DeviceTensor& logits, const De
 // "Accumulate" variants for the training loop: the gradient is returned, the SUM of this call's per-row
 // (per-element for MSE) losses is added on the device to lossAccumulator (one element, owned by the
 // caller); nothing is read back to the host.
-inline DeviceTensor meanSquaredErrorAccumulate(const DeviceTensor& prediction, const DeviceTensor& target, DeviceTensor& lossAccumulator) {
+// gradImage: as for softmaxCrossEntropySparseAccumulate below (rows whose length is a multiple of 8).
+inline DeviceTensor meanSquaredErrorAccumulate(const DeviceTensor& prediction, const DeviceTensor& target, DeviceTensor& lossAccumulator,
+                                               bool gradImage = false) {
     require(prediction.shape() == target.shape(), "meanSquaredErrorAccumulate: incompatible shapes on the device");
     DeviceTensor grad(prediction.shape());
-    check(bf_hip_mse(prediction.data(), target.data(), grad.data(), lossAccumulator.data(), prediction.elementCount(), 1, nullptr));
+    std::uint16_t* image = gradImage && prediction.rank() >= 1 && prediction.elementCount() > 0 &&
+                                   prediction.dim(prediction.rank() - 1) % 8 == 0 ? grad.attachImage() : nullptr;
+    check(bf_hip_mse_img(prediction.data(), target.data(), grad.data(), image, lossAccumulator.data(), prediction.elementCount(), 1, nullptr));
     return grad;
 }
 

@@ -86,6 +86,7 @@ public:
             }
             layers_.push_back(std::move(layer));
         }
+        planFusedTriples();
     }
 
 #ifdef BLACKFORGE_HIP_HAS_IR
@@ -102,10 +103,24 @@ public:
     // the token ids of a leading embedding layer on the host (train_runner.cu:210-212), so no device-side
     // range check (and no host synchronisation) is done.
     DeviceTensor forward(const DeviceTensor& input, bool inputRangeTrusted = false) {
-        invalidateBf16WeightCache();   // the optimizer may have changed the weights since the last call
-        DeviceTensor current = input.clone();
+        return forward(input.clone(), inputRangeTrusted, false);
+    }
+
+    // The same pass over an input the model may keep instead of copying it: `input` becomes the first layer's cached input
+    // (a DeviceTensor::borrow view must stay valid and unchanged until backward() has run).  weightImagesCurrent is the
+    // caller's promise that no parameter value has changed since this model's previous forward pass (no optimizer step,
+    // no upload, no checkpoint load): the cached bf16 weight images are then kept instead of being dropped and converted
+    // again.  Without the promise every call drops them, as the reference does per forward pass (ops_tensorcore.cu:448).
+    DeviceTensor forward(DeviceTensor&& input, bool inputRangeTrusted = false, bool weightImagesCurrent = false) {
+        if (!weightImagesCurrent) invalidateBf16WeightCache();   // the optimizer may have changed the weights since the last call
+        DeviceTensor current = std::move(input);
         for (std::size_t li = 0; li < layers_.size(); ++li) {
             LayerState& layer = layers_[li];
+            if (layer.fusedRole == 1) {
+                current = forwardFusedTriple(li, current);
+                li += 2;
+                continue;
+            }
             DeviceTensor next = applyForward(layer, current, inputRangeTrusted && li == 0);
             layer.cachedInput = std::move(current);
             current = std::move(next);
@@ -119,9 +134,17 @@ public:
         const DeviceTensor* grad = &outputGrad;
         DeviceTensor owned;
         for (std::size_t li = layers_.size(); li-- > 0;) {
+            if (layers_[li].fusedRole == 3) {
+                owned = backwardFusedTriple(li - 2, *grad);
+                grad = &owned;
+                li -= 2;
+                continue;
+            }
             // a block whose gradient goes on to another block's bf16 GEMMs writes that gradient's bf16 image with it
             const bool imageForConsumer = useBf16_ && li > 0 && isBlock(layers_[li - 1].spec.kind);
-            owned = applyBackward(layers_[li], *grad, inputRangeTrusted && li == 0, imageForConsumer);
+            // the gradient with respect to the model's input has no reader (backward() returns nothing): the first layer
+            // does not form it
+            owned = applyBackward(layers_[li], *grad, inputRangeTrusted && li == 0, imageForConsumer, /*needInputGrad=*/li > 0);
             grad = &owned;
         }
     }
@@ -210,6 +233,10 @@ private:
         // true from zeroGrad() until this layer's next backward pass: its gradient buffers hold zeros, so that pass may
         // write the gradients there instead of adding them in
         bool gradsAreZero = true;
+        // linear -> silu/gelu/relu -> linear with bf16 projections runs as one unit (1, 2, 3 = the three layers of such a
+        // triple, 0 = a layer on its own): see planFusedTriples
+        int fusedRole = 0;
+        DeviceTensor hiddenImage;   // role 1: bf16(act(z)) of the last forward pass, raw storage [rows, hidden / 2]
     };
 
     static Parameter makeParameter(std::string name, std::vector<std::size_t> shape) {
@@ -225,6 +252,75 @@ private:
             case LayerKind::Softmax: return softmax(x);
             default: throw std::invalid_argument("hip::Model: not an elementwise layer");
         }
+    }
+
+    static bool isActivation(LayerKind kind) { return kind == LayerKind::Silu || kind == LayerKind::Gelu || kind == LayerKind::Relu; }
+    static int activationCode(LayerKind kind) { return kind == LayerKind::Silu ? BF_ACT_SILU : kind == LayerKind::Gelu ? BF_ACT_GELU : BF_ACT_RELU; }
+
+    // linear(d -> hidden) -> activation -> linear(hidden -> d) with bf16 projections is the feed-forward block's pair of
+    // projections without its normalisation and residual: the three layers run through bf_hip_feedforward_bf16, which keeps
+    // the activated hidden tensor as a bf16 image only (its sole readers are GEMMs) and, in the backward pass, forms the
+    // pre-activation gradient as a bf16 image plus its column sums in one pass.  Same roundings at the same places as the
+    // three layers on their own (the operands of every product, nothing else), so the same results; four passes over
+    // [rows, hidden] in fp32 fewer.
+    void planFusedTriples() {
+        if (!useBf16_) return;
+        for (std::size_t li = 0; li + 2 < layers_.size(); ++li) {
+            LayerState &l1 = layers_[li], &la = layers_[li + 1], &l2 = layers_[li + 2];
+            if (l1.spec.kind != LayerKind::Linear || !isActivation(la.spec.kind) || l2.spec.kind != LayerKind::Linear) continue;
+            const std::size_t d = l1.params[0].value.dim(0), hidden = l1.params[0].value.dim(1);
+            if (d == 0 || hidden == 0 || d % 8 != 0 || hidden % 8 != 0 || l2.params[0].value.dim(1) != d) continue;
+            l1.fusedRole = 1;
+            la.fusedRole = 2;
+            l2.fusedRole = 3;
+            li += 2;
+        }
+    }
+
+    DeviceTensor forwardFusedTriple(std::size_t li, DeviceTensor& x) {
+        LayerState &l1 = layers_[li], &la = layers_[li + 1], &l2 = layers_[li + 2];
+        const std::size_t d = l1.params[0].value.dim(0), hidden = l1.params[0].value.dim(1);
+        require(x.rank() >= 2 && detail::lastDim(x) == d, "linear: incompatible shapes on the device");
+        const std::size_t rows = detail::rowsOf(x);
+        DeviceTensor z(detail::withLastDim(x, hidden)), out(x.shape());
+        l1.hiddenImage = DeviceTensor({rows, hidden / 2});
+        if (rows > 0) {
+            // x's bf16 image is kept with it for the weight gradient; a producer may have written it already
+            const bool haveImage = x.image() != nullptr;
+            std::uint16_t* xImage = haveImage ? const_cast<std::uint16_t*>(x.image()) : x.attachImage();
+            check(bf_hip_feedforward_bf16(haveImage ? nullptr : x.data(), l1.params[0].value.data(), l1.params[1].value.data(),
+                                          l2.params[0].value.data(), l2.params[1].value.data(), nullptr, activationCode(la.spec.kind), z.data(),
+                                          reinterpret_cast<std::uint16_t*>(l1.hiddenImage.data()), xImage, out.data(), rows, d, hidden, 1,
+                                          nullptr));
+        }
+        l1.cachedInput = std::move(x);
+        la.cachedInput = std::move(z);
+        l2.cachedInput = DeviceTensor();   // the activated hidden tensor exists as l1.hiddenImage only
+        return out;
+    }
+
+    DeviceTensor backwardFusedTriple(std::size_t li, const DeviceTensor& grad) {
+        LayerState &l1 = layers_[li], &la = layers_[li + 1], &l2 = layers_[li + 2];
+        const DeviceTensor& x = l1.cachedInput;
+        const std::size_t d = l1.params[0].value.dim(0), hidden = l1.params[0].value.dim(1), rows = detail::rowsOf(x);
+        require(grad.shape() == x.shape(), "linear backward: gradient shape differs from the output");
+        GradientTargets t1, t2;
+        if (l1.gradsAreZero) { t1.slot[0] = &l1.params[0].grad; t1.slot[1] = &l1.params[1].grad; }
+        if (l2.gradsAreZero) { t2.slot[0] = &l2.params[0].grad; t2.slot[1] = &l2.params[1].grad; }
+        l1.gradsAreZero = la.gradsAreZero = l2.gradsAreZero = false;
+        DeviceTensor dW1 = detail::gradientTensor(&t1, 0, l1.params[0].value.shape()), dB1 = detail::gradientTensor(&t1, 1, {hidden}),
+                     dW2 = detail::gradientTensor(&t2, 0, l2.params[0].value.shape()), dB2 = detail::gradientTensor(&t2, 1, {d});
+        const bool needInputGrad = li > 0;   // the model input's gradient has no reader
+        DeviceTensor dX = needInputGrad ? DeviceTensor(x.shape()) : DeviceTensor();
+        check(bf_hip_feedforward_bf16_backward_img(x.data(), x.image(), l1.params[0].value.data(), l2.params[0].value.data(), la.cachedInput.data(),
+                                                   reinterpret_cast<const std::uint16_t*>(l1.hiddenImage.data()), grad.data(), grad.image(),
+                                                   activationCode(la.spec.kind), needInputGrad ? dX.data() : nullptr, dW1.data(), dB1.data(),
+                                                   dW2.data(), dB2.data(), rows, d, hidden, 1, nullptr));
+        accumulate(l1.params[0].grad, dW1);
+        accumulate(l1.params[1].grad, dB1);
+        accumulate(l2.params[0].grad, dW2);
+        accumulate(l2.params[1].grad, dB2);
+        return dX;
     }
 
     // x is about to become the layer's cached input: a bf16 linear layer gives it the bf16 image that both its forward
@@ -264,7 +360,7 @@ private:
         return kind == LayerKind::Attention || kind == LayerKind::BidirectionalAttention || kind == LayerKind::FeedForward;
     }
 
-    DeviceTensor applyBackward(LayerState& layer, const DeviceTensor& grad, bool trustedIds, bool imageForConsumer) {
+    DeviceTensor applyBackward(LayerState& layer, const DeviceTensor& grad, bool trustedIds, bool imageForConsumer, bool needInputGrad = true) {
         const LayerSpec& s = layer.spec;
         const DeviceTensor& x = layer.cachedInput;
         GradientTargets targets;
@@ -277,6 +373,15 @@ private:
         switch (s.kind) {
             case LayerKind::Linear: {
                 DeviceTensor dBias = biasGradientOnly(grad);
+                if (useBf16_ && !needInputGrad) {   // the weight gradient alone
+                    const DeviceTensor& w = layer.params[0].value;
+                    DeviceTensor dW = detail::gradientTensor(into, 0, w.shape());
+                    check(bf_hip_matmul_bf16_backward_img(x.data(), x.image(), w.data(), grad.data(), grad.image(), nullptr, dW.data(),
+                                                          detail::rowsOf(x), w.dim(0), w.dim(1), 1, nullptr));
+                    accumulate(layer.params[0].grad, dW);
+                    accumulate(layer.params[1].grad, dBias);
+                    return DeviceTensor();
+                }
                 MatmulGrad g = detail::projectionBackward(x, layer.params[0].value, grad, useBf16_ ? 2 : 0, x.shape(), into, 0);
                 accumulate(layer.params[0].grad, g.dB);
                 accumulate(layer.params[1].grad, dBias);

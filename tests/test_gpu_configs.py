@@ -23,6 +23,88 @@ def sample(rng, n, count=48):
     return np.unique(picks[(picks >= 0) & (picks < n)])
 
 
+# ---- config 2 end to end at full size: linear(4096) -> silu -> linear(4096), MSE, forward + backward -------------------
+def _silu64(z):
+    return z / (1.0 + np.exp(-z))
+
+
+def _silu_d64(z):
+    s = 1.0 / (1.0 + np.exp(-z))
+    return s * (1.0 + z * (1.0 - s))
+
+
+def test_mlp_config2_full_size_pipeline(hip, oracle):
+    """BASELINE config 2 at its real size through hip::Model: [4096, 4096] -> linear(4096) -> silu -> linear(4096), MSE,
+    forward + backward, bf16 projections.  The CPU reference would take a quarter of an hour, so the expected values are
+    float64 evaluations of the same chain with operands rounded to bf16 where the pipeline rounds them (both operands of
+    every product; everything else fp32), on sampled rows (output) and sampled hidden units (all four gradients, whose
+    contractions run over all 4096 tokens).  The loss is checked against float64 of the model's own output, and two
+    steps from the same state must give the same bits.  Bound 5e-4 (the contract for bf16 projections is 2e-2; measured:
+    9e-5 of the largest value for the output, 1e-5 to 2e-5 for the weight gradients, printed by the test)."""
+    from blackforge_amd import hostlayer as hl
+    tokens = width = 4096
+    rng = np.random.default_rng(2)
+    model = hl.HostModel([(hl.LINEAR, width), (hl.SILU,), (hl.LINEAR, width)], input_features=width, use_bf16=True)
+    params = {}
+    for i, count in enumerate(model.counts):
+        name = model.names[i]
+        # config 2 has zero biases; small non-zero ones here so that a dropped bias term would show
+        value = r(rng, count, scale=1 / 64) if name.endswith("weight") else r(rng, count, scale=0.05)
+        model.set_value(i, value)
+        params[i] = value
+    (iw1, ib1, iw2, ib2) = range(4)
+    w1, b1, w2, b2 = params[iw1].reshape(width, width), params[ib1], params[iw2].reshape(width, width), params[ib2]
+    x, y = r(rng, tokens, width), r(rng, tokens, width)
+    D = hip.DeviceTensor
+    dx, dy = D.fromHost(x), D.fromHost(y)
+
+    model.trainStep(dx, dy, loss_kind=hl.LOSS_MSE, optimizer=0)
+    loss = model.readLossSum() / (tokens * width)
+    grads = [model.grad(i).copy() for i in range(4)]
+    out = model.forward(dx).reshape(tokens, width)
+
+    rb = lambda t: oracle.roundToBf16(np.ascontiguousarray(t, dtype=f32)).astype(f64)
+    xb, w1b, w2b = rb(x), rb(w1), rb(w2)
+    rows, units = sample(rng, tokens, 24), sample(rng, width, 16)
+    worst = {}
+
+    def check(name, got, expected, tol=5e-4):
+        expected = np.asarray(expected, f64)
+        scale = float(np.sqrt(np.mean(expected ** 2)))
+        worst[name] = float(np.max(np.abs(got.astype(f64) - expected)) / (np.abs(expected).max() + 1e-30))
+        assert_close(got, expected.astype(f32), tol=tol, what=name, scale=scale)
+
+    # forward on sampled rows: z = x w1 + b1 (fp32 out), h = silu(z) rounded to bf16 for the second product
+    z_rows = (xb[rows] @ w1b + b1).astype(f32).astype(f64)
+    h_rows = rb(_silu64(z_rows).astype(f32))
+    check("output rows", out[rows], h_rows @ w2b + b2)
+    # the loss of the model's own output
+    loss64 = float(np.mean((out.astype(f64) - y.astype(f64)) ** 2))
+    print(f"config 2 loss {loss:.6f} (float64 of the output: {loss64:.6f})")
+    assert abs(loss - loss64) <= 1e-5 * loss64
+    # gradient of the loss with respect to the output, from the model's own output (fp32 on the GPU)
+    g = (2.0 * (out.astype(f64) - y.astype(f64)) / (tokens * width)).astype(f32)
+    gb = rb(g)
+    check("linear2.bias grad", grads[ib2], g.astype(f64).sum(axis=0), tol=1e-4)
+    # hidden units `units`: their pre-activations over ALL tokens need only those columns of w1
+    z_units = (xb @ w1b[:, units] + b1[units]).astype(f32).astype(f64)            # [tokens, |units|]
+    h_units = rb(_silu64(z_units).astype(f32))
+    check("linear2.weight grad rows", grads[iw2].reshape(width, width)[units], h_units.T @ gb)
+    dh_units = (gb @ w2b[units].T).astype(f32).astype(f64)                        # dH[:, units], fp32 out of its product
+    dz_units = (dh_units * _silu_d64(z_units)).astype(f32)
+    check("linear1.bias grad", grads[ib1][units], dz_units.astype(f64).sum(axis=0), tol=1e-3)
+    check("linear1.weight grad columns", grads[iw1].reshape(width, width)[:, units], xb.T @ rb(dz_units))
+    print("config 2 at full size, max |gpu - float64| / max |float64|: " + ", ".join(f"{k} {v:.2e}" for k, v in worst.items()))
+    assert all(np.isfinite(t).all() for t in grads)
+
+    # the same step again from the same state: same bits
+    model.trainStep(dx, dy, loss_kind=hl.LOSS_MSE, optimizer=0)
+    loss2 = model.readLossSum() / (tokens * width)
+    assert loss2 == loss
+    for i in range(4):
+        assert_bits_equal(model.grad(i), grads[i], "second step, " + model.names[i])
+
+
 # ---- bf16 projections with long contractions, at the shapes of configs 2, 4 and 5 ------------------------------------
 @pytest.mark.parametrize("m,k,n", [(4096, 4096, 4096), (8192, 3072, 768), (8192, 768, 3072), (16384, 2048, 8192), (8192, 768, 2304)])
 def test_long_contraction_projection_against_float64(hip, oracle, m, k, n):
