@@ -1977,13 +1977,13 @@ int launchDkv(const AttnParams& p, size_t smem, unsigned grid, hipStream_t s) {
 
 // bit 0: the forward kernel's products as six bf16 MFMAs each; bit 1: the dK/dV kernel's; bit 2: those of the dQ kernel
 // that reads the stored dS (head dims up to 128 all three); 0 = every product on the fp32 MFMA
-std::atomic<int> gAttnRoute{BF_ATTN_ROUTE_SPLIT};
+thread_local int gAttnRoute = BF_ATTN_ROUTE_SPLIT;   // per host thread: a test naming kernels does not change other threads' calls
 
 template <int KIND, int HDP, int TILE>
 int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
     constexpr size_t operandBytes = size_t(2) * TILE * (HDP + 4) * sizeof(float);   // one operand, double buffered
     if constexpr (KIND == 0 && HDP <= 128) {
-        if (gAttnRoute.load() & 1) {
+        if (gAttnRoute & 1) {
             constexpr size_t splitBytes = size_t(2) * 3 * 32 * (splitKeyPitch(HDP) + splitValuePitch(HDP)) * sizeof(unsigned short);
             return vec4 ? launchAttn(attnForwardPipedKernel<HDP, true>, splitBytes, grid, p, s)
                         : launchAttn(attnForwardPipedKernel<HDP, false>, splitBytes, grid, p, s);
@@ -1997,7 +1997,7 @@ int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
                     : launchAttn(attnBackwardDqKernel<HDP, TILE, false>, 2 * operandBytes, grid, p, s);
     } else if constexpr (KIND == 4) {
         if constexpr (HDP <= 128) {
-            if (gAttnRoute.load() & BF_ATTN_ROUTE_SPLIT_DQ) {
+            if (gAttnRoute & BF_ATTN_ROUTE_SPLIT_DQ) {
                 constexpr size_t splitBytes = size_t(2) * 3 * 32 * splitValuePitch(HDP) * sizeof(unsigned short) + size_t(4) * kDsPatch * sizeof(float);
                 return vec4 ? launchAttn(attnBackwardDqFromDsSplitKernel<HDP, true>, splitBytes, grid, p, s)
                             : launchAttn(attnBackwardDqFromDsSplitKernel<HDP, false>, splitBytes, grid, p, s);
@@ -2011,7 +2011,7 @@ int dispatchVec(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
                     : launchAttn(attnBackwardDqFromDsKernel<HDP, TILE, false>, smem, grid, p, s);
     } else {
         if constexpr (HDP <= 128) {
-            if (gAttnRoute.load() & 2) {
+            if (gAttnRoute & 2) {
                 if constexpr (HDP <= 64) {   // Q and dO images in three buffers, statistics likewise
                     constexpr size_t pipedBytes = size_t(6) * 3 * 32 * splitKeyPitch(HDP) * sizeof(unsigned short) + size_t(3) * 64 * sizeof(float);
                     return vec4 ? launchAttn(attnBackwardDkvPipedKernel<HDP, true, KIND == 3>, pipedBytes, grid, p, s)
@@ -2045,10 +2045,10 @@ size_t dsBytes(size_t batch, size_t heads, size_t newLen, size_t totalLen) {
 
 // Upper limit of the hand-over buffer that bf_hip_attention_backward may take from the pool; SIZE_MAX = an eighth of
 // the device's memory.  Above the limit the backward pass recomputes S and dP in the dQ kernel instead.
-std::atomic<size_t> gDsLimit{SIZE_MAX};
+thread_local size_t gDsLimit = SIZE_MAX;   // per host thread, as the route
 
 size_t dsLimit() {
-    size_t limit = gDsLimit.load();
+    size_t limit = gDsLimit;
     if (limit != SIZE_MAX) return limit;
     return deviceMemoryBytes() / 8;
 }
@@ -2197,7 +2197,7 @@ int bf_hip_attention_ds_bytes(size_t batch, size_t heads, size_t newLen, size_t 
 }
 
 int bf_hip_attention_set_workspace_limit(size_t bytes) {
-    gDsLimit.store(bytes);
+    gDsLimit = bytes;
     return BF_OK;
 }
 
@@ -2299,7 +2299,7 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
 
 int bf_hip_attention_set_route(int route) {
     BF_REQUIRE(route >= 0 && route <= BF_ATTN_ROUTE_SPLIT, "unknown route");
-    bf::gAttnRoute.store(route);
+    bf::gAttnRoute = route;
     return BF_OK;
 }
 

@@ -34,13 +34,28 @@ int failRuntime(const char* function, hipError_t error, const char* file, int li
 // bf_hip_capture_end, the stream that is being captured (so that code written against the default stream, like the
 // C++ operator layer, records into the graph unchanged).
 extern hipStream_t g_defaultStream;
-inline hipStream_t asStream(bf_stream_t s) { return s ? static_cast<hipStream_t>(s) : g_defaultStream; }
+// The stream the library last enqueued work on (per process; NULL = the default stream) and whether one is known.
+extern hipStream_t g_currentStream;
+extern bool g_currentStreamKnown;
+// Orders `next` behind everything enqueued on the current stream (an event recorded there, waited for on `next`) and
+// makes it the current stream.  Pool blocks, cached weight images and descriptor tables return to their registries at
+// host-call exit while kernels using them may still be queued; their next user is then ordered behind those kernels
+// whichever stream it runs on, because every change of stream passes through here.  Nothing happens while a graph is
+// being captured (a capture uses one stream).
+void switchStream(hipStream_t next);
+inline hipStream_t asStream(bf_stream_t s) {
+    hipStream_t r = s ? static_cast<hipStream_t>(s) : g_defaultStream;
+    if (r != g_currentStream || !g_currentStreamKnown) switchStream(r);
+    return r;
+}
 // True between bf_hip_capture_begin and bf_hip_capture_end.  While it holds, pool blocks come from and return to the
 // capture's own arena, descriptor tables are private copies, and weight images are cached per capture: nothing the
 // recorded kernels address can be handed to anyone else while the graph lives.
 bool capturing();
 // gemm_bf16.hip: returns the weight images cached during the capture to the pool (the arena, at that point).
 void dropCaptureWeightImages();
+// gemm_bf16.hip: a recorded graph is about to run; whatever weights it updates, the eager weight images are stale after it.
+void noteGraphLaunched();
 
 // ---- launch geometry ---------------------------------------------------------------------------
 constexpr int kWave = 64;            // CDNA wavefront

@@ -138,7 +138,7 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(ConvertSources 
 // wavefront touch every bank once.  Rows past the end of an operand are clamped to its last row (their
 // products are never stored) and chunks past the end of the K range read as zero, so neither kernel has
 // a branch around a load.
-std::atomic<int> g_ntRoute{BF_GEMM_ROUTE_AUTO};
+thread_local int g_ntRoute = BF_GEMM_ROUTE_AUTO;   // per host thread
 constexpr int BKK = 64;
 constexpr int LDS_ROW = BKK + 8;
 
@@ -1411,7 +1411,7 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
                  size_t lda, size_t ldb, hipStream_t s) {
     if (M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
     const size_t cus = size_t(computeUnits());
-    switch (g_ntRoute.load()) {   // a kernel named by the caller (tests and tuning); BF_GEMM_ROUTE_AUTO otherwise
+    switch (g_ntRoute) {   // a kernel named by the caller (tests and tuning); BF_GEMM_ROUTE_AUTO otherwise
         case BF_GEMM_ROUTE_PINGPONG_256: return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
         case BF_GEMM_ROUTE_PINGPONG_128: return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
         case BF_GEMM_ROUTE_PINGPONG_256_PERSISTENT: return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s);
@@ -1421,7 +1421,7 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
         case BF_GEMM_ROUTE_WIDE_192:
         case BF_GEMM_ROUTE_WIDE_192_PERSISTENT:
             if (size_t(epi.splitN) != N && epi.splitN % 192 != 0) return failInvalid("gemm_bf16", "192-wide tiles need outputs whose width is a multiple of 192");
-            return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s, g_ntRoute.load() == BF_GEMM_ROUTE_WIDE_192_PERSISTENT);
+            return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s, g_ntRoute == BF_GEMM_ROUTE_WIDE_192_PERSISTENT);
         default: break;
     }
     // 256x256 ping-pong tiles once they give three quarters of the CUs a tile; otherwise 128x128 tiles,
@@ -1587,7 +1587,11 @@ struct CachedWeight {
     void* buffer;
     size_t bytes;
 };
-size_t g_generation = 1;
+// One generation per cache: an invalidation recorded into a graph must not mark the eager images stale, and the eager
+// generation also advances whenever a recorded graph is launched (its kernels may step an optimizer over the weights
+// whose images the eager cache holds: noteGraphLaunched).
+size_t g_generationEager = 1, g_generationCaptured = 1;
+size_t& generation() { return capturing() ? g_generationCaptured : g_generationEager; }
 using WeightKey = std::tuple<int, const float*, const float*, const float*, int>;
 // While a graph is being captured the images live in a cache of their own, filled and emptied inside the capture: the
 // recorded conversions and products address arena blocks that no later eager call can be handed.
@@ -1664,18 +1668,18 @@ int weightImage(const float* const* w, size_t count, size_t rows, size_t cols, i
     int st = cacheSlot(WeightKey{dev, w[0], w1, w2, layout}, bytes, &slot);
     if (st != BF_OK) return st;
     *image = static_cast<unsigned short*>(slot->buffer);
-    if (slot->generation == g_generation) return BF_OK;
+    if (slot->generation == generation()) return BF_OK;
     CachedWeight* mate = nullptr;
     if (layout == 1 || (layout == 2 && cols % 8 == 0)) {
         const int mateLayout = layout == 1 ? 0 : 3;
         st = cacheSlot(WeightKey{dev, w[0], w1, w2, mateLayout}, weightImageBytes(count, rows, cols, mateLayout), &mate);
         if (st != BF_OK) return st;
-        if (mate->generation == g_generation) mate = nullptr;   // already current
+        if (mate->generation == generation()) mate = nullptr;   // already current
     }
     st = fillWeightImage(w, count, rows, cols, layout, *image, mate ? static_cast<unsigned short*>(mate->buffer) : nullptr, s);
     if (st != BF_OK) return st;
-    slot->generation = g_generation;
-    if (mate) mate->generation = g_generation;
+    slot->generation = generation();
+    if (mate) mate->generation = generation();
     return BF_OK;
 }
 int weightImage(const float* w, size_t rows, size_t cols, bool transposed, bool cache, hipStream_t s, unsigned short** image,
@@ -1684,6 +1688,8 @@ int weightImage(const float* w, size_t rows, size_t cols, bool transposed, bool 
 }
 
 }  // namespace
+
+void noteGraphLaunched() { ++g_generationEager; }
 
 void dropCaptureWeightImages() {
     if (!capturing()) return;
@@ -2196,7 +2202,7 @@ int bf_hip_mfma_only_loop(const uint16_t* operands, float* out, int shape, int w
 
 int bf_hip_gemm_bf16_set_route(int route) {
     BF_REQUIRE(route >= BF_GEMM_ROUTE_AUTO && route <= BF_GEMM_ROUTE_PINGPONG_128_PERSISTENT, "unknown route");
-    bf::g_ntRoute.store(route);
+    bf::g_ntRoute = route;
     return BF_OK;
 }
 
@@ -2205,14 +2211,14 @@ int bf_hip_invalidate_bf16_weight_cache(void) {
     // model) or idle: their buffers go back to the pool.  An idle weight that is used again just converts once more.
     auto& cache = bf::weightCache();
     for (auto it = cache.begin(); it != cache.end();) {
-        if (it->second.generation != bf::g_generation) {
+        if (it->second.generation != bf::generation()) {
             bf_hip_pool_release(it->second.buffer, it->second.bytes);
             it = cache.erase(it);
         } else {
             ++it;
         }
     }
-    ++bf::g_generation;
+    ++bf::generation();
     return BF_OK;
 }
 

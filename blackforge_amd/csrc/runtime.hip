@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <map>
 #include <mutex>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -33,6 +34,29 @@ int failRuntime(const char* function, hipError_t error, const char* file, int li
 }
 
 hipStream_t g_defaultStream = nullptr;
+hipStream_t g_currentStream = nullptr;
+bool g_currentStreamKnown = false;
+
+void switchStream(hipStream_t next) {
+    if (capturing()) return;
+    if (g_currentStreamKnown && next != g_currentStream) {
+        // one event per device, recorded again at every switch: only the latest record matters to the waiter
+        static std::unordered_map<int, hipEvent_t> fences;
+        int dev = 0;
+        if (hipGetDevice(&dev) == hipSuccess) {
+            hipEvent_t& fence = fences[dev];
+            if (fence == nullptr && hipEventCreateWithFlags(&fence, hipEventDisableTiming) != hipSuccess) fence = nullptr;
+            // a failure here (a stream that no longer exists) leaves the old stream's work unordered with the new one's:
+            // fall back to waiting for the whole device
+            if (fence == nullptr || hipEventRecord(fence, g_currentStream) != hipSuccess || hipStreamWaitEvent(next, fence, 0) != hipSuccess) {
+                (void)hipGetLastError();
+                (void)hipDeviceSynchronize();
+            }
+        }
+    }
+    g_currentStream = next;
+    g_currentStreamKnown = true;
+}
 
 int computeUnits() {
     static std::unordered_map<int, int> cache;
@@ -141,6 +165,7 @@ std::unordered_map<int, DevicePool>& pools() {
 struct CaptureArena {
     int device = 0;
     hipStream_t stream = nullptr;
+    std::thread::id thread;   // the host thread that records: nobody else may take pool memory meanwhile
     std::unordered_map<size_t, std::vector<void*>> freeLists;
     std::vector<std::pair<void*, size_t>> blocks;   // (pointer, size class) of every block taken during the capture
     std::vector<void*> tables;                      // descriptor tables of recorded launches (hipMalloc, not pool blocks)
@@ -150,7 +175,12 @@ std::unordered_map<void*, CaptureArena*>& arenaOwners() {        // block -> are
     static std::unordered_map<void*, CaptureArena*> owners;
     return owners;
 }
-hipStream_t g_utilityStream = nullptr;   // non-blocking, for copies that must not touch a capturing stream
+// non-blocking stream of the capturing device, for copies that must not touch a capturing stream (one per device)
+hipStream_t g_utilityStream = nullptr;
+std::unordered_map<int, hipStream_t>& utilityStreams() {
+    static std::unordered_map<int, hipStream_t> streams;
+    return streams;
+}
 
 struct CapturedGraph {
     hipGraphExec_t exec = nullptr;
@@ -165,10 +195,12 @@ hipError_t mallocWithTrim(void** ptr, size_t bytes, DevicePool& pool) {
     (void)hipGetLastError();
     if (hipDeviceSynchronize() != hipSuccess) return err;
     for (auto& entry : pool.freeLists) {
+        std::vector<void*> kept;   // a block the driver refuses to take back stays on its free list
         for (void* p : entry.second) {
             if (hipFree(p) == hipSuccess) pool.stats.bytes_from_driver -= entry.first;
+            else { (void)hipGetLastError(); kept.push_back(p); }
         }
-        entry.second.clear();
+        entry.second.swap(kept);
     }
     return hipMalloc(ptr, bytes);
 }
@@ -251,7 +283,16 @@ int bf_hip_set_device(int index) {
     bf_hip_device_count(&n);
     BF_REQUIRE(index >= 0 && index < n, "device index " + std::to_string(index) + " out of range (" +
                                             std::to_string(n) + " devices)");
+    int before = index;
+    (void)hipGetDevice(&before);
     BF_HIP_TRY(hipSetDevice(index));
+    if (before != index) {   // the stream last used is a per-device fact (pools are per device): park it, fetch the other device's
+        static std::unordered_map<int, std::pair<hipStream_t, bool>> parked;
+        parked[before] = {g_currentStream, g_currentStreamKnown};
+        const auto it = parked.find(index);
+        g_currentStream = it != parked.end() ? it->second.first : nullptr;
+        g_currentStreamKnown = it != parked.end() && it->second.second;
+    }
     return BF_OK;
 }
 
@@ -276,7 +317,15 @@ int bf_hip_stream_create(bf_stream_t* stream) {
     return BF_OK;
 }
 int bf_hip_stream_destroy(bf_stream_t stream) {
-    if (stream) BF_HIP_TRY(hipStreamDestroy(asStream(stream)));
+    if (stream == nullptr) return BF_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (g_currentStreamKnown && g_currentStream == s) {
+        // its queued work may still use pool blocks that are free again on the host: it finishes before the stream goes,
+        // and the next stream has nothing to be ordered behind
+        BF_HIP_TRY(hipStreamSynchronize(s));
+        g_currentStreamKnown = false;
+    }
+    BF_HIP_TRY(hipStreamDestroy(s));
     return BF_OK;
 }
 int bf_hip_stream_synchronize(bf_stream_t stream) {
@@ -314,6 +363,8 @@ int bf_hip_pool_acquire(size_t bytes, void** ptr) {
     if (bytes == 0) return BF_OK;
     int dev = 0;
     BF_HIP_TRY(hipGetDevice(&dev));
+    if (g_capture != nullptr && g_capture->thread != std::this_thread::get_id())
+        return failInvalid(__func__, "another host thread is recording a graph: its pool memory belongs to the recording");
     DevicePool& pool = pools()[dev];
     size_t cls = sizeClass(bytes);
     std::vector<void*>* list = &pool.freeLists[cls];
@@ -392,13 +443,18 @@ int bf_hip_capture_begin(bf_stream_t stream) {
     BF_REQUIRE(g_capture == nullptr, "a capture is already in progress");
     int dev = 0;
     BF_HIP_TRY(hipGetDevice(&dev));
-    if (g_utilityStream == nullptr) BF_HIP_TRY(hipStreamCreateWithFlags(&g_utilityStream, hipStreamNonBlocking));
+    hipStream_t& utility = utilityStreams()[dev];
+    if (utility == nullptr) BF_HIP_TRY(hipStreamCreateWithFlags(&utility, hipStreamNonBlocking));
+    g_utilityStream = utility;
     BF_HIP_TRY(hipDeviceSynchronize());   // nothing of the eager work before may still be in flight on another stream
     BF_HIP_TRY(hipStreamBeginCapture(static_cast<hipStream_t>(stream), hipStreamCaptureModeRelaxed));
     g_capture = new CaptureArena;
     g_capture->device = dev;
     g_capture->stream = static_cast<hipStream_t>(stream);
+    g_capture->thread = std::this_thread::get_id();
     g_defaultStream = g_capture->stream;
+    g_currentStream = g_capture->stream;   // the device is idle: nothing to be ordered behind
+    g_currentStreamKnown = true;
     return BF_OK;
 }
 
@@ -428,6 +484,7 @@ int bf_hip_graph_launch(bf_graph_t graph, bf_stream_t stream) {
     BF_REQUIRE(graph != nullptr, "graph is NULL");
     BF_REQUIRE(g_capture == nullptr, "a graph cannot be launched into a capture");
     BF_HIP_TRY(hipGraphLaunch(static_cast<CapturedGraph*>(graph)->exec, asStream(stream)));
+    noteGraphLaunched();
     return BF_OK;
 }
 

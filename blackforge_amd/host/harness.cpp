@@ -104,23 +104,31 @@ int bfh_model_forward(void* h, const float* input, int rank, const size_t* shape
     });
 }
 
+}  // extern "C"
+
+namespace {
+const char* lossName(int lossKind) {
+    return lossKind == 0 ? "cross_entropy_sparse" : lossKind == 2 ? "cross_entropy_masked" : lossKind == 3 ? "cross_entropy" : "mse";
+}
+// The loss of handle->output against `target`, accumulated on the device, and its gradient (with a bf16 image where the
+// model's last layer reads one).
+void accumulateLoss(Handle* handle, const float* target, int lossKind) {
+    std::vector<std::size_t> shape = handle->output.shape();
+    if (lossKind == 0 || lossKind == 2) shape = {handle->output.elementCount() / handle->output.shape().back()};
+    Borrowed tgt(target, shape);
+    handle->lossGrad = hip::lossGradientAccumulate(lossName(lossKind), handle->output, tgt.tensor, handle->lossAccumulator,
+                                                   handle->model->usesBf16());
+}
+}  // namespace
+
+extern "C" {
+
 // lossKind 0: sparse cross-entropy (targets = one class index per output row), 1: mean squared error, 2: masked sparse
-// cross-entropy (index -1 = row ignored).  The loss sum (for kind 2: the mean over the rows not ignored) is accumulated on the
-// device; bfh_model_read_loss reads and resets it.
+// cross-entropy (index -1 = row ignored), 3: dense cross-entropy (targets = one probability row per output row).  The loss
+// sum (for kind 2: the mean over the rows not ignored) is accumulated on the device; bfh_model_read_loss reads and resets it.
 int bfh_model_loss(void* h, const float* target, int lossKind) {
     Handle* handle = static_cast<Handle*>(h);
-    return guarded([&] {
-        if (lossKind == 0 || lossKind == 2) {
-            std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
-            Borrowed tgt(target, {rows});
-            handle->lossGrad = lossKind == 0 ? hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator,
-                                                                                       handle->model->usesBf16())
-                                             : hip::softmaxCrossEntropyMaskedAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
-        } else {
-            Borrowed tgt(target, handle->output.shape());
-            handle->lossGrad = hip::meanSquaredErrorAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
-        }
-    });
+    return guarded([&] { accumulateLoss(handle, target, lossKind); });
 }
 
 int bfh_model_loss_grad(void* h, float** grad, size_t* count) {
@@ -177,16 +185,7 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
         handle->output = handle->model->forward(std::move(in.tensor), true, handle->weightImagesCurrent);
         handle->weightImagesCurrent = true;
-        if (lossKind == 0 || lossKind == 2) {
-            std::size_t rows = handle->output.elementCount() / handle->output.shape().back();
-            Borrowed tgt(target, {rows});
-            handle->lossGrad = lossKind == 0 ? hip::softmaxCrossEntropySparseAccumulate(handle->output, tgt.tensor, handle->lossAccumulator,
-                                                                                       handle->model->usesBf16())
-                                             : hip::softmaxCrossEntropyMaskedAccumulate(handle->output, tgt.tensor, handle->lossAccumulator);
-        } else {
-            Borrowed tgt(target, handle->output.shape());
-            handle->lossGrad = hip::meanSquaredErrorAccumulate(handle->output, tgt.tensor, handle->lossAccumulator, handle->model->usesBf16());
-        }
+        accumulateLoss(handle, target, lossKind);
         handle->model->backward(handle->lossGrad, true);
         if (optimizer == 1) {
             if (!handle->adamw) handle->adamw = std::make_unique<hip::AdamW>(lr, 0.9F, 0.999F, 1e-8F, 0.01F);
@@ -216,8 +215,8 @@ int bfh_model_capture_train_step(void* h, const float* input, int rank, const si
         opt->setLearningRate(lr);
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
         Borrowed tgt(target, std::vector<std::size_t>(targetShape, targetShape + targetRank));
-        const char* lossName = lossKind == 0 ? "cross_entropy_sparse" : lossKind == 2 ? "cross_entropy_masked" : "mse";
-        *step = new hip::CapturedTrainStep(*handle->model, *opt, lossName, in.tensor, tgt.tensor, handle->lossAccumulator);
+        const char* name = lossName(lossKind);
+        *step = new hip::CapturedTrainStep(*handle->model, *opt, name, in.tensor, tgt.tensor, handle->lossAccumulator);
     });
 }
 int bfh_captured_step_run(void* h, void* step, float lr, int optimizer) {

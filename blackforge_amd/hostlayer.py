@@ -15,7 +15,7 @@ from .tensor import DeviceTensor
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libbf_hip_host.so")
 
 LINEAR, SILU, RELU, GELU, RMSNORM, SOFTMAX, EMBEDDING, POSITIONAL, ATTENTION, FEEDFORWARD, BIDIRECTIONAL_ATTENTION = range(11)
-LOSS_SPARSE_CE, LOSS_MSE, LOSS_MASKED_CE = 0, 1, 2
+LOSS_SPARSE_CE, LOSS_MSE, LOSS_MASKED_CE, LOSS_DENSE_CE = 0, 1, 2, 3
 
 _lib = None
 

@@ -23,11 +23,14 @@
  *     and launch nothing (reference: device_pool.cu:30-32).
  *   - One host thread at a time per PROCESS, like the reference (device_pool.hpp:39-40): the pool, the cached bf16
  *     weight images and the descriptor tables are unguarded registries.
- *   - One stream in flight at a time per device.  Workspace and result blocks return to the pool when the host call
- *     returns, while the kernels using them may still be queued; the next user of such a block is ordered behind them
- *     only if it is enqueued on the same stream.  The cached weight images and descriptor tables are shared across
- *     streams in the same way.  A caller that switches streams on a device synchronises the old one first
- *     (bf_hip_stream_synchronize); overlapping two streams on one device is not supported.
+ *   - Streams: workspace and result blocks return to the pool when the host call returns, while the kernels using
+ *     them may still be queued, and the cached weight images and descriptor tables are shared by all streams.  The
+ *     library therefore orders streams itself: whenever a call names another stream than the call before it (on the
+ *     same device), the new stream first waits for everything enqueued on the old one (an event recorded there).
+ *     Calls on different streams are correct in any interleaving; they do not overlap on the device.  Devices are
+ *     selected with bf_hip_set_device (the stream last used is remembered per device).
+ *   - The tuning switches (bf_hip_gemm_bf16_set_route, bf_hip_attention_set_route, bf_hip_attention_set_workspace_limit)
+ *     are per host thread: a thread that names a kernel for a test does not change what another thread's calls run.
  */
 #ifndef BF_HIP_H
 #define BF_HIP_H

@@ -33,13 +33,16 @@ inline DeviceTensor lossGradientAccumulate(const std::string& loss, const Device
     if (loss == "cross_entropy_sparse") return softmaxCrossEntropySparseAccumulate(output, target, lossAccumulator, gradImage);
     if (loss == "cross_entropy_masked") return softmaxCrossEntropyMaskedAccumulate(output, target, lossAccumulator);
     if (loss == "cross_entropy") return softmaxCrossEntropyAccumulate(output, target, lossAccumulator);
-    return meanSquaredErrorAccumulate(output, target, lossAccumulator);   // every other name, as in the runner
+    return meanSquaredErrorAccumulate(output, target, lossAccumulator, gradImage);   // every other name, as in the runner
 }
 
 class CapturedTrainStep {
 public:
     // Records zeroGrad + forward + loss + backward + optimizer update for tensors of these shapes.  Nothing is executed:
-    // parameters, optimizer state and lossAccumulator are as they were when the constructor returns.
+    // parameters, optimizer state and lossAccumulator are as they were when the constructor returns.  The model's
+    // activation caches are NOT: recording walked the layers for their host side effects and left the caches pointing at
+    // buffers no kernel has written, so the constructor marks them invalid (Model::invalidateCaches): an eager backward()
+    // needs an eager forward() after the recording, and throws otherwise.  The same holds after a recording that failed.
     CapturedTrainStep(Model& model, Optimizer& optimizer, const std::string& loss, const DeviceTensor& input, const DeviceTensor& target,
                       DeviceTensor& lossAccumulator)
         : optimizer_(optimizer) {
@@ -61,8 +64,10 @@ public:
         } catch (...) {
             bf_hip_capture_end(nullptr);   // abandon the recording, return its memory
             bf_hip_stream_destroy(stream_);
+            model.invalidateCaches();
             throw;
         }
+        model.invalidateCaches();
         status = bf_hip_capture_end(&graph_);
         if (status != BF_OK) {
             bf_hip_stream_destroy(stream_);

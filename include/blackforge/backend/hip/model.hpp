@@ -125,10 +125,20 @@ public:
             layer.cachedInput = std::move(current);
             current = std::move(next);
         }
+        cachesValid_ = true;
         return current;
     }
 
+    // The activation caches no longer describe a forward pass that ran (a recording into a graph walked the layers without
+    // executing anything): backward() throws until forward() has run again, and gradients are added, not written.
+    void invalidateCaches() {
+        cachesValid_ = false;
+        for (LayerState& layer : layers_) layer.gradsAreZero = false;
+    }
+
     void backward(const DeviceTensor& outputGrad, bool inputRangeTrusted = false) {
+        require(cachesValid_, "hip::Model::backward: no forward pass to differentiate (none has run yet, or the last one was only "
+                              "recorded into a graph)");
         // the caller's gradient is only read: no copy of it (the logits gradient of a language model is the largest
         // tensor of the step)
         const DeviceTensor* grad = &outputGrad;
@@ -496,6 +506,7 @@ private:
 
     std::string name_;
     bool useBf16_ = false;
+    bool cachesValid_ = false;
     std::vector<LayerState> layers_;
     std::size_t generationPosition_ = 0;
 };

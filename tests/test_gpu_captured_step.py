@@ -115,3 +115,92 @@ def test_capture_rules_are_reported(hip):
     hip.capi.call("bf_hip_capture_end", None)               # abandon
     a = hip.DeviceTensor.fromHost(np.ones(8, f32))
     assert (hip.ops.scale(a, 2.0).toHost() == 2).all()      # eager calls run again
+
+
+def test_eager_backward_after_a_recording_is_refused(hip, rng):
+    """Recording walks the layers without running a kernel, so the activation caches it leaves describe nothing: an eager
+    backward pass right after it must raise, not differentiate against unwritten buffers; after an eager forward pass it
+    works again."""
+    from blackforge_amd import hostlayer as hl
+    D = hip.DeviceTensor
+    model, _ = twin_models(hl, rng, lm_layers(hl, 64, 32, 16, 2, 64), False)
+    x, t = D.fromHost(rng.integers(0, 64, (2, 16)).astype(f32)), D.fromHost(rng.integers(0, 64, 32).astype(f32))
+    model.forward(x)
+    model.loss(t)
+    model.backward()          # an ordinary eager pass works
+    step = model.captureTrainStep(x, t, hl.LOSS_SPARSE_CE, 1, 1e-3)
+    with pytest.raises(ValueError, match="no forward pass to differentiate"):
+        model.backward()
+    model.forward(x)
+    model.loss(t)
+    model.backward()
+    step.close()
+
+
+def test_cached_weight_image_follows_a_replay(hip, oracle, rng):
+    """A replay steps the optimizer over the weights; a cached-weight projection called afterwards through the C ABI must
+    multiply by the NEW weights (the eager weight-image cache is marked stale by every graph launch)."""
+    from blackforge_amd import hostlayer as hl
+    D, call = hip.DeviceTensor, hip.capi.call
+    width, rows = 64, 32
+    model = hl.HostModel([(hl.LINEAR, width)], input_features=width, use_bf16=True)
+    model.set_value(0, (rng.standard_normal(width * width) * 0.1).astype(f32))
+    model.set_value(1, np.zeros(width, f32))
+    x, y = D.fromHost(rng.standard_normal((rows, width)).astype(f32)), D.fromHost(rng.standard_normal((rows, width)).astype(f32))
+    step = model.captureTrainStep(x, y, hl.LOSS_MSE, 2, 0.5)
+    a = rng.standard_normal((rows, width)).astype(f32)
+    da, out = D.fromHost(a), D((rows, width))
+    w_ptr = model._value_ptrs[0]
+
+    def product():
+        call("bf_hip_linear_bf16", da.ptr, w_ptr, None, None, out.ptr, rows, width, width, 1, None)
+        return out.toHost()
+
+    def expected():
+        w = model.value(0).reshape(width, width)
+        return oracle.matmul(oracle.roundToBf16(a), oracle.roundToBf16(w))
+
+    np.testing.assert_allclose(product(), expected(), rtol=1e-4, atol=1e-5)
+    before = model.value(0).copy()
+    step.run(0.5)
+    hip.capi.call("bf_hip_synchronize")
+    assert np.abs(model.value(0) - before).max() > 1e-3          # the replay did move the weights
+    np.testing.assert_allclose(product(), expected(), rtol=1e-4, atol=1e-5)
+    step.close()
+
+
+@pytest.mark.parametrize("loss_kind,use_bf16,optimizer", [(2, False, 1), (3, False, 1), (1, False, 2), (1, True, 2), (0, True, 2)])
+def test_replays_equal_eager_steps_for_every_loss(hip, rng, loss_kind, use_bf16, optimizer):
+    """The masked and the dense cross-entropy and the mean squared error recorded into the graph (a device-side count of
+    the rows that are not ignored, the partial sums of the squared error), and SGD over bf16 projections: replays against
+    eager steps, bit for bit, over three batches."""
+    from blackforge_amd import hostlayer as hl
+    D = hip.DeviceTensor
+    vocab, dim, seq, batch, heads, hidden = 64, 32, 16, 4, 2, 64
+    eager, recorded = twin_models(hl, rng, lm_layers(hl, vocab, dim, seq, heads, hidden), use_bf16)
+
+    def targets():
+        if loss_kind in (0, 2):
+            t = rng.integers(0, vocab, batch * seq).astype(f32)
+            if loss_kind == 2:
+                t[rng.random(batch * seq) < 0.3] = -1.0
+            return t
+        if loss_kind == 3:
+            p = rng.random((batch, seq, vocab)).astype(f32)
+            return (p / p.sum(axis=-1, keepdims=True)).astype(f32)
+        return rng.standard_normal((batch, seq, vocab)).astype(f32)
+
+    batches = [(rng.integers(0, vocab, (batch, seq)).astype(f32), targets()) for _ in range(3)]
+    x, t = D.fromHost(batches[0][0]), D.fromHost(batches[0][1])
+    step = recorded.captureTrainStep(x, t, loss_kind, optimizer, 1e-2)
+    for n, (ids, tgt) in enumerate(batches):
+        hip.capi.call("bf_hip_memcpy_h2d", x.ptr, ids.ctypes.data_as(ctypes.c_void_p), ids.nbytes)
+        hip.capi.call("bf_hip_memcpy_h2d", t.ptr, tgt.ctypes.data_as(ctypes.c_void_p), tgt.nbytes)
+        step.run(1e-2)
+        eager.trainStep(D.fromHost(ids), D.fromHost(tgt), loss_kind, optimizer if optimizer == 1 else 0, 1e-2)
+        if optimizer == 2:
+            eager.sgdStep(1e-2)
+        for i in range(len(eager.counts)):
+            assert_bits_equal(recorded.value(i), eager.value(i), f"step {n + 1}: {eager.names[i]}")
+        assert recorded.readLossSum() == eager.readLossSum(), f"step {n + 1}: accumulated loss"
+    step.close()
