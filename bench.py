@@ -201,6 +201,24 @@ def bench_extras(bf, steps):
     hbm("softmax_65536x2048", 8 * nr, lambda: call("bf_hip_softmax", x.ptr, y.ptr, nr // dm, dm, sh))
     del x, g, y, half
 
+    # the row kernels at the sizes a GPT-small step runs them (24 and 12 launches a step): 8192 tokens x 768 features
+    # (25 MB a tensor: the last-level cache holds all of it, so these read faster than HBM could deliver) and the
+    # feed-forward block's backward pass over 8192 x 3072
+    rows_s, dm_s, hid_s = 8192, 768, 3072
+    xs, gs, ads, ys = rand(rows_s, dm_s), rand(rows_s, dm_s), rand(rows_s, dm_s), D((rows_s, dm_s))
+    ims = D((rows_s, dm_s), itemsize=2)
+    ns = rows_s * dm_s
+    hbm("rmsnorm_to_image_8192x768", 6 * ns, lambda: call("bf_hip_rmsnorm_img", xs.ptr, None, ims.ptr, rows_s, dm_s, sh))
+    hbm("rmsnorm_backward_add_with_image_8192x768", 18 * ns,
+        lambda: call("bf_hip_rmsnorm_backward_add_img", xs.ptr, gs.ptr, ads.ptr, ys.ptr, ims.ptr, rows_s, dm_s, sh))
+    zs, dhs, bs_ = rand(rows_s, hid_s), rand(rows_s, hid_s), rand(hid_s)
+    dzs = D((rows_s, hid_s))
+    dbs = D((hid_s,))
+    nh = rows_s * hid_s
+    hbm("add_bias_gelu_backward_8192x3072", 12 * nh,
+        lambda: call("bf_hip_add_bias_act_backward", zs.ptr, bs_.ptr, dhs.ptr, dzs.ptr, dbs.ptr, rows_s, hid_s, bf.capi.ACT_GELU, sh))
+    del xs, gs, ads, ys, ims, zs, dhs, dzs
+
     # GPT-small logits [8192, 32000] (0.98 GiB): sparse cross-entropy reads logits once and writes the gradient
     rows, vocab, dim = 8192, 32000, 768
     logits, grad = rand(rows, vocab), D((rows, vocab))

@@ -139,6 +139,7 @@ SIGNATURES = {
     "bf_hip_cross_entropy": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_sparse_img": [P, P, P, P, P, c_size, c_size, c_int, S],
+    "bf_hip_cross_entropy_sparse_head": [P, P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_cross_entropy_masked": [P, P, P, P, c_size, c_size, c_int, S],
     "bf_hip_sgd_publish": [P, c_float, S],
     "bf_hip_sgd_multi_indirect": [ctypes.POINTER(c_ptr), ctypes.POINTER(c_ptr), ctypes.POINTER(c_size), c_size, P, S],

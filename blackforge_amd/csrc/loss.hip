@@ -243,6 +243,91 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
     }
 }
 
+// The sparse cross-entropy of a language-model head whose gradient has no reader but the head's own gradient products:
+// the gradient row goes out as its bf16 image only (no fp32 copy is written), and its column sums, the bias gradient of
+// the head, are collected on the way: a thread holds the same columns of every row its block walks, so it adds each
+// gradient value (fp32, before the rounding) to a register per column and the block writes one partial row at the end;
+// columnPartialsFinishKernel adds the partial rows in index order.  Same arithmetic per element as crossEntropyKernel
+// (1024 threads a row, rows in registers, the next row's loads in flight): the same loss, the same image.
+template <int MAXE, bool NT>
+__global__ void __launch_bounds__(1024) crossEntropyImageKernel(const float* __restrict__ logits, const float* __restrict__ target,
+                                                                unsigned short* __restrict__ gradImage, float* __restrict__ rowLoss,
+                                                                float* __restrict__ colPartial, size_t rows, size_t classes, float invRows) {
+    constexpr int G = 1024, VEC = 4;
+    __shared__ float lds[16];
+    const int t = threadIdx.x;
+    using Row = RowCache<G, MAXE, VEC, NT>;
+    Row ahead, col;
+#pragma unroll
+    for (int i = 0; i < MAXE; ++i) col.r[i] = 0.0f;
+    const size_t rowStep = gridDim.x;
+    if (blockIdx.x < rows) ahead.load(logits + size_t(blockIdx.x) * classes, classes, t, -INFINITY);
+    for (size_t row = blockIdx.x; row < rows; row += rowStep) {
+        Row c = ahead;
+        if (row + rowStep < rows) ahead.load(logits + (row + rowStep) * classes, classes, t, -INFINITY);
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < MAXE; ++i) mx = fmaxf(mx, c.r[i]);
+        mx = groupMax<G>(mx, lds);
+        constexpr float kLog2e = 1.4426950408889634f;
+        const float top = mx * kLog2e;
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < MAXE; ++i) { c.r[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(c.r[i], kLog2e, -top)); sum += c.r[i]; }
+        sum = groupSum<G>(sum, lds);
+        const float inv = 1.0f / sum;
+        const unsigned cls = unsigned(lroundf(target[row]));
+        const int targetIt = cls < classes ? int(cls / unsigned(G * VEC)) : -1;
+        const bool mine = int((cls / VEC) % G) == t;
+        const int targetSlot = int(cls % VEC);
+        const float scale = inv * invRows;
+        float pTarget = -1.0f;
+#pragma unroll
+        for (int it = 0; it < MAXE / VEC; ++it) {
+            if (it == targetIt) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const bool hit = mine && j == targetSlot;
+                    const float p = c.r[it * VEC + j] * inv;
+                    pTarget = hit ? p : pTarget;
+                    c.r[it * VEC + j] = hit ? (p - 1.0f) * invRows : c.r[it * VEC + j] * scale;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) c.r[it * VEC + j] *= scale;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MAXE; ++i) col.r[i] += c.r[i];   // slots past the row's end hold exp2(-inf) * scale = 0
+        c.storeBf16(gradImage + row * classes, classes, t);
+        float loss = pTarget >= 0.0f ? -logf(fmaxf(pTarget, 1e-12f)) : 0.0f;
+        loss = groupSum<G>(loss, lds);
+        if (t == 0) rowLoss[row] = loss;
+    }
+    col.store(colPartial + size_t(blockIdx.x) * classes, classes, t);
+}
+
+// out[c] = sum over p of partial[p * features + c], rows added in index order: sixteen lanes per group of four columns
+// each add every sixteenth partial row, and the sixteen sums are combined in a fixed order (features % 4 == 0).
+__global__ void __launch_bounds__(kBlock) columnPartialsFinishKernel(const float* __restrict__ partial, float* __restrict__ out,
+                                                                     size_t parts, size_t features) {
+    __shared__ float4v lds[16][17];
+    const int cx = threadIdx.x & 15, part = threadIdx.x >> 4;
+    const size_t c = (size_t(blockIdx.x) * 16 + cx) * 4;
+    float4v s = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (c < features) {
+#pragma unroll 8
+        for (size_t p = part; p < parts; p += 16) s = s + loadf4(partial + p * features + c);
+    }
+    lds[part][cx] = s;
+    __syncthreads();
+    if (part == 0 && c < features) {
+        float4v total = lds[0][cx];
+        for (int i = 1; i < 16; ++i) total = total + lds[i][cx];
+        storef4(out + c, total);
+    }
+}
+
 template <bool SPARSE>
 int launchCrossEntropy(const float* logits, const float* target, float* grad, float* lossSum, size_t rows,
                        size_t classes, int accumulate, hipStream_t s, bool masked = false, unsigned short* gradImage = nullptr) {
@@ -264,7 +349,10 @@ int launchCrossEntropy(const float* logits, const float* target, float* grad, fl
     const bool shifted = !vec4 && ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad)) & 15u) == 0;
     // shifted rows are addressed from the 128-byte line below their first element when logits and gradient rows sit at
     // the same offset within a line (every wavefront access then covers whole lines), else from the 16-byte group below
-    const bool sameLine = ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad)) & 127u) == 0;
+    // ... and only when both tensors START on a line: the first row then has shift 0 and is addressed from its own first
+    // element, and every later row's line lies inside the tensor (it holds the tail of the row before), so nothing below
+    // the tensor's first byte is ever read.  Past the last row's end at most the rest of its 16-byte group is read.
+    const bool sameLine = ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(grad)) & 127u) == 0;
     const bool streaming = streamsPastCache(rows * classes * (SPARSE ? 8 : 12));   // logits in, gradient out (and a dense target in)
     // smallest group and register count that hold a row (see the row kernels)
     // AHEAD as measured (8 B per logit over the launch, 16-byte aligned rows): rows of up to 8192 classes are faster
@@ -363,6 +451,39 @@ int bf_hip_cross_entropy_sparse_img(const float* logits, const float* targetIdx,
     }
     BF_REQUIRE(logits && targetIdx && grad, "NULL pointer");
     return launchCrossEntropy<true>(logits, targetIdx, grad, lossSum, rows, classes, accumulate, asStream(stream), false, gradImage);
+}
+
+int bf_hip_cross_entropy_sparse_head(const float* logits, const float* targetIdx, uint16_t* gradImage, float* biasGrad, float* lossSum,
+                                     size_t rows, size_t classes, int accumulate, bf_stream_t stream) {
+    BF_REQUIRE(lossSum != nullptr, "lossSum is NULL");
+    // the rows a 1024-thread block can hold in 16 or 32 registers a thread, 16-byte aligned throughout, with a whole bf16 image
+    if (rows == 0 || classes == 0 || classes % 8 != 0 || classes > size_t(1024) * 32 || classes < 4096 || !aligned16(logits) ||
+        !aligned16(gradImage) || !aligned16(biasGrad)) {
+        setLastError("bf_hip_cross_entropy_sparse_head: shape or alignment not served by the fused form (use bf_hip_cross_entropy_sparse_img and bf_hip_bias_grad)");
+        return BF_ERR_UNSUPPORTED;
+    }
+    BF_REQUIRE(logits && targetIdx && gradImage && biasGrad, "NULL pointer");
+    hipStream_t s = asStream(stream);
+    const unsigned grid = unsigned(std::min<size_t>(rows, size_t(computeUnits()) * 2));
+    Scratch rowLoss(rows * sizeof(float));
+    if (rowLoss.status != BF_OK) return rowLoss.status;
+    Scratch partial(size_t(grid) * classes * sizeof(float));
+    if (partial.status != BF_OK) return partial.status;
+    const float invRows = 1.0f / float(rows);
+    const bool streaming = streamsPastCache(rows * classes * 6);
+    if (classes <= size_t(1024) * 16) {
+        if (streaming) crossEntropyImageKernel<16, true><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
+        else crossEntropyImageKernel<16, false><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
+    } else {
+        if (streaming) crossEntropyImageKernel<32, true><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
+        else crossEntropyImageKernel<32, false><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
+    }
+    BF_LAUNCH_CHECK();
+    columnPartialsFinishKernel<<<gridFor(classes / 4, 16), kBlock, 0, s>>>(partial.as<float>(), biasGrad, grid, classes);
+    BF_LAUNCH_CHECK();
+    finishSumKernel<<<1, 1024, 0, s>>>(rowLoss.as<float>(), rows, lossSum, accumulate);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
 }
 
 int bf_hip_cross_entropy_sparse(const float* logits, const float* targetIdx, float* grad, float* lossSum,

@@ -8,9 +8,11 @@
 // storeShifted give rows of ANY length and alignment the 16-byte accesses too: the row is addressed from an
 // aligned boundary at or below its first element, `shift` elements earlier (the 16-byte boundary, shift 0..3, or
 // the 128-byte line, shift 0..31, after which every wavefront access covers whole lines: 8 % faster on rows of
-// 50 257 floats), and the elements a group holds from outside the row are masked.  The aligned line that holds the
-// row's first element, and the aligned 16 bytes that hold its last, stay inside the pages of the tensor, so the
-// bytes read from beyond a row are always readable; nothing is written there.
+// 50 257 floats), and the elements a group holds from outside the row are masked.  A shifted access touches the bytes
+// from the row's first element rounded DOWN to the boundary (16 or 128 bytes) to its end rounded UP to 16 bytes, and
+// nothing else; nothing outside the row is written.  Callers use the 128-byte boundary only for tensors that start on
+// a 128-byte line (the first row then has shift 0, every other row's line holds the tail of the row before it), so
+// reads stay inside the tensor except for at most 12 bytes after its last element, inside the same 16-byte group.
 #pragma once
 
 #include "common.hpp"

@@ -185,8 +185,12 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
         handle->output = handle->model->forward(std::move(in.tensor), true, handle->weightImagesCurrent);
         handle->weightImagesCurrent = true;
-        accumulateLoss(handle, target, lossKind);
-        handle->model->backward(handle->lossGrad, true);
+        {
+            std::vector<std::size_t> targetShape = handle->output.shape();
+            if (lossKind == 0 || lossKind == 2) targetShape = {handle->output.elementCount() / handle->output.shape().back()};
+            Borrowed tgt(target, targetShape);
+            hip::lossAndBackward(*handle->model, lossName(lossKind), handle->output, tgt.tensor, handle->lossAccumulator, true);
+        }
         if (optimizer == 1) {
             if (!handle->adamw) handle->adamw = std::make_unique<hip::AdamW>(lr, 0.9F, 0.999F, 1e-8F, 0.01F);
             handle->adamw->setLearningRate(lr);

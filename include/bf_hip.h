@@ -468,6 +468,15 @@ int bf_hip_cross_entropy_sparse(const float* logits, const float* targetIdx, flo
  * aligned tensors), for the language-model head's backward GEMMs. */
 int bf_hip_cross_entropy_sparse_img(const float* logits, const float* targetIdx, float* grad, uint16_t* gradImage, float* lossSum,
                                     size_t rows, size_t classes, int accumulate, bf_stream_t stream);
+/* The loss of a language-model head whose gradient is read by nothing but the head's own gradient products
+ * (softmaxCrossEntropySparseAccumulate followed by the backward pass of the last linear layer, loss.cu:381-411 and
+ * model.cu:278-284 in one pass over the logits): gradImage[rows, classes] receives the gradient rounded to bf16 (the
+ * operand of bf_hip_matmul_bf16_backward_img), biasGrad[classes] its column sums taken in fp32 before the rounding (the
+ * bias gradient), and no fp32 gradient is written.  Same loss and same image as bf_hip_cross_entropy_sparse_img; the
+ * column sums are added in another (fixed) order than bf_hip_bias_grad adds them.  Served shapes: 16-byte aligned
+ * tensors, classes a multiple of 8 between 4096 and 32768; anything else returns BF_ERR_UNSUPPORTED and launches nothing. */
+int bf_hip_cross_entropy_sparse_head(const float* logits, const float* targetIdx, uint16_t* gradImage, float* biasGrad, float* lossSum,
+                                     size_t rows, size_t classes, int accumulate, bf_stream_t stream);
 /* softmaxCrossEntropyMasked (the CPU backend's loss for masked-language-model training, src/backend/cpu/loss.cpp:149-215;
  * the CUDA backend has no counterpart): as the sparse form, except that a row whose index rounds to -1 is ignored (zero
  * gradient, no loss term) and gradient and loss are averaged over the n rows that are not: grad = (p - onehot) / n, and

@@ -36,6 +36,23 @@ inline DeviceTensor lossGradientAccumulate(const std::string& loss, const Device
     return meanSquaredErrorAccumulate(output, target, lossAccumulator, gradImage);   // every other name, as in the runner
 }
 
+// Loss (added to lossAccumulator) and backward pass of one step.  A bf16 model that ends in a linear head takes the
+// sparse cross-entropy through the fused form (softmaxCrossEntropySparseHeadAccumulate: gradient as a bf16 image plus the
+// head's bias gradient, no fp32 gradient), every other combination through lossGradientAccumulate.  Everyone who runs a
+// training step (the runner, the recorded step, the harness) comes through here, so that their steps agree bit for bit.
+inline void lossAndBackward(Model& model, const std::string& loss, const DeviceTensor& output, const DeviceTensor& target,
+                            DeviceTensor& lossAccumulator, bool inputRangeTrusted) {
+    if (loss == "cross_entropy_sparse" && model.headTakesImageGradient()) {
+        DeviceTensor grad, biasGrad;
+        if (softmaxCrossEntropySparseHeadAccumulate(output, target, lossAccumulator, grad, biasGrad)) {
+            model.backward(grad, inputRangeTrusted, &biasGrad);
+            return;
+        }
+    }
+    DeviceTensor grad = lossGradientAccumulate(loss, output, target, lossAccumulator, model.usesBf16());
+    model.backward(grad, inputRangeTrusted);
+}
+
 class CapturedTrainStep {
 public:
     // Records zeroGrad + forward + loss + backward + optimizer update for tensors of these shapes.  Nothing is executed:
@@ -58,8 +75,7 @@ public:
             DeviceTensor output = model.forward(input, /*inputRangeTrusted=*/true);
             outputRows_ = output.elementCount() / output.shape().back();
             outputElements_ = output.elementCount();
-            DeviceTensor grad = lossGradientAccumulate(loss, output, target, lossAccumulator, model.usesBf16());
-            model.backward(grad, /*inputRangeTrusted=*/true);
+            lossAndBackward(model, loss, output, target, lossAccumulator, /*inputRangeTrusted=*/true);
             optimizer.recordStep(model.parameters());
         } catch (...) {
             bf_hip_capture_end(nullptr);   // abandon the recording, return its memory

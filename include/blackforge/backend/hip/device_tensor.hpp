@@ -71,6 +71,16 @@ public:
         return t;
     }
 
+    // A tensor that exists as its bf16 image only (data() is NULL): for a value whose readers are all bf16 GEMMs, written
+    // by a producer that never forms the fp32 copy.  Only functions documented to accept one may be handed it.
+    static DeviceTensor imageOnly(std::vector<std::size_t> shape) {
+        DeviceTensor t;
+        t.shape_ = std::move(shape);
+        t.owns_ = false;
+        (void)t.attachImage();
+        return t;
+    }
+
     static DeviceTensor fromHost(const runtime::Tensor& host) {
         DeviceTensor t(host.shape());
         check(bf_hip_memcpy_h2d(t.data_, host.data().data(), t.elementCount() * sizeof(float)));

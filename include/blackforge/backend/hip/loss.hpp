@@ -123,6 +123,27 @@ inline DeviceTensor softmaxCrossEntropySparseAccumulate(const DeviceTensor& logi
     return grad;
 }
 
+// The loss of a bf16 language-model head, for a caller that hands the gradient to nothing but that head's backward pass
+// (Model::backward with headBiasGrad): the gradient comes back as a bf16 image only (DeviceTensor::imageOnly) together
+// with its column sums, the head's bias gradient; no fp32 gradient is written.  Same loss, same image, same precondition
+// as softmaxCrossEntropySparseAccumulate(..., gradImage = true).  Returns false, and does nothing, for shapes the fused
+// kernel does not serve (the caller then takes the ordinary route).
+inline bool softmaxCrossEntropySparseHeadAccumulate(const DeviceTensor& logits, const DeviceTensor& targetIndices, DeviceTensor& lossAccumulator,
+                                                    DeviceTensor& gradImageOnly, DeviceTensor& biasGrad) {
+    detail::requireSparse("softmaxCrossEntropySparseAccumulate", logits, targetIndices);
+    const std::size_t rows = detail::rowsOf(logits), classes = detail::lastDim(logits);
+    if (rows == 0 || classes % 8 != 0 || classes < 4096 || classes > 32768) return false;
+    DeviceTensor grad = DeviceTensor::imageOnly(logits.shape());
+    DeviceTensor bias({classes});
+    const int status = bf_hip_cross_entropy_sparse_head(logits.data(), targetIndices.data(), const_cast<std::uint16_t*>(grad.image()), bias.data(),
+                                                        lossAccumulator.data(), rows, classes, 1, nullptr);
+    if (status == BF_ERR_UNSUPPORTED) return false;
+    check(status);
+    gradImageOnly = std::move(grad);
+    biasGrad = std::move(bias);
+    return true;
+}
+
 // Adds this call's MEAN over the rows that are not ignored (the value softmaxCrossEntropyMasked returns) to
 // lossAccumulator; indices are the caller's precondition, as above.
 inline DeviceTensor softmaxCrossEntropyMaskedAccumulate(const DeviceTensor& logits, const DeviceTensor& targetIndices,

@@ -136,7 +136,17 @@ public:
         for (LayerState& layer : layers_) layer.gradsAreZero = false;
     }
 
-    void backward(const DeviceTensor& outputGrad, bool inputRangeTrusted = false) {
+    // True when the last layer is a bf16 linear layer on its own: its backward pass reads the output gradient only as a
+    // bf16 image (both gradient products) and through its column sums (the bias gradient), so backward() accepts an
+    // image-only gradient together with those sums (headBiasGrad).
+    [[nodiscard]] bool headTakesImageGradient() const {
+        return useBf16_ && !layers_.empty() && layers_.back().spec.kind == LayerKind::Linear && layers_.back().fusedRole == 0;
+    }
+
+    // headBiasGrad: the column sums of outputGrad, already formed by the producer of the gradient (the loss kernel); the
+    // last layer, a linear one, then does not sum the gradient's columns itself, and outputGrad may be image-only.
+    void backward(const DeviceTensor& outputGrad, bool inputRangeTrusted = false, const DeviceTensor* headBiasGrad = nullptr) {
+        require(headBiasGrad == nullptr || headTakesImageGradient(), "hip::Model::backward: this model's last layer takes no precomputed bias gradient");
         require(cachesValid_, "hip::Model::backward: no forward pass to differentiate (none has run yet, or the last one was only "
                               "recorded into a graph)");
         // the caller's gradient is only read: no copy of it (the logits gradient of a language model is the largest
@@ -154,7 +164,8 @@ public:
             const bool imageForConsumer = useBf16_ && li > 0 && isBlock(layers_[li - 1].spec.kind);
             // the gradient with respect to the model's input has no reader (backward() returns nothing): the first layer
             // does not form it
-            owned = applyBackward(layers_[li], *grad, inputRangeTrusted && li == 0, imageForConsumer, /*needInputGrad=*/li > 0);
+            owned = applyBackward(layers_[li], *grad, inputRangeTrusted && li == 0, imageForConsumer, /*needInputGrad=*/li > 0,
+                                  li + 1 == layers_.size() ? headBiasGrad : nullptr);
             grad = &owned;
         }
     }
@@ -370,7 +381,8 @@ private:
         return kind == LayerKind::Attention || kind == LayerKind::BidirectionalAttention || kind == LayerKind::FeedForward;
     }
 
-    DeviceTensor applyBackward(LayerState& layer, const DeviceTensor& grad, bool trustedIds, bool imageForConsumer, bool needInputGrad = true) {
+    DeviceTensor applyBackward(LayerState& layer, const DeviceTensor& grad, bool trustedIds, bool imageForConsumer, bool needInputGrad = true,
+                               const DeviceTensor* givenBiasGrad = nullptr) {
         const LayerSpec& s = layer.spec;
         const DeviceTensor& x = layer.cachedInput;
         GradientTargets targets;
@@ -382,7 +394,8 @@ private:
         layer.gradsAreZero = false;
         switch (s.kind) {
             case LayerKind::Linear: {
-                DeviceTensor dBias = biasGradientOnly(grad);
+                DeviceTensor dBias = givenBiasGrad != nullptr ? DeviceTensor::borrow(givenBiasGrad->data(), givenBiasGrad->shape())
+                                                              : biasGradientOnly(grad);
                 if (useBf16_ && !needInputGrad) {   // the weight gradient alone
                     const DeviceTensor& w = layer.params[0].value;
                     DeviceTensor dW = detail::gradientTensor(into, 0, w.shape());

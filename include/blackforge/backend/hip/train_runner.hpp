@@ -16,6 +16,7 @@
 #include <string>
 #include <vector>
 
+#include "blackforge/backend/hip/captured_step.hpp"
 #include "blackforge/backend/hip/checkpoint.hpp"
 #include "blackforge/backend/hip/dataset.hpp"
 #include "blackforge/backend/hip/loss.hpp"
@@ -114,11 +115,8 @@ TrainRunResult runTraining(Model& model, DatasetT& dataset, const TrainOptions& 
             // the masked loss adds each batch's MEAN (its divisor, the rows not ignored, differs from batch to batch),
             // so the epoch's figure is the mean of the batch means, as in cpu/train_runner.cpp:184-194
             lossDivisor += maskedLoss ? 1 : (sparse || dense) ? output.elementCount() / output.shape().back() : output.elementCount();
-            DeviceTensor grad = sparse       ? softmaxCrossEntropySparseAccumulate(output, target, lossAccumulator, model.usesBf16())
-                                : maskedLoss ? softmaxCrossEntropyMaskedAccumulate(output, target, lossAccumulator)
-                                : dense      ? softmaxCrossEntropyAccumulate(output, target, lossAccumulator)
-                                             : meanSquaredErrorAccumulate(output, target, lossAccumulator);
-            model.backward(grad, vocab.has_value());
+            lossAndBackward(model, sparse ? "cross_entropy_sparse" : maskedLoss ? "cross_entropy_masked" : dense ? "cross_entropy" : "mse", output,
+                            target, lossAccumulator, vocab.has_value());
             optimizer->step(model.parameters());
         }
         const float lossSum = lossAccumulator.toHost().at(0);

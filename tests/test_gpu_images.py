@@ -114,6 +114,44 @@ def test_cross_entropy_gradient_image(hip, oracle, rng, rows, classes):
         call("bf_hip_cross_entropy_sparse_img", dl.ptr, di.ptr, grad.ptr, img.ptr, loss.ptr, rows, classes - 4, 0, None)
 
 
+@pytest.mark.parametrize("rows,classes", [(3, 4096), (700, 4104), (5, 16384), (1100, 16392), (9, 32000), (600, 32768), (1, 8192)])
+def test_cross_entropy_of_a_language_model_head(hip, oracle, rng, rows, classes):
+    """bf_hip_cross_entropy_sparse_head: the loss and the gradient image of bf_hip_cross_entropy_sparse_img (bit for bit
+    where that kernel holds a row the same way) without the fp32 gradient, and the gradient's column sums (the head's bias gradient) against float64 sums of the
+    oracle's gradient.  Row counts below and above the number of workgroups that walk the rows (one partial row of
+    column sums per workgroup), class counts at both register plans, their upper ends, and just past a multiple of 4096."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    logits = r(rng, rows, classes, scale=3)
+    idx = rng.integers(0, classes, rows).astype(f32)
+    idx[0], idx[-1] = 0, classes - 1
+    dl, di = D.fromHost(logits), D.fromHost(idx)
+    grad, img, loss = D((rows, classes)), image_of(hip, (rows, classes)), D.zeros((1,))
+    call("bf_hip_cross_entropy_sparse_img", dl.ptr, di.ptr, grad.ptr, img.ptr, loss.ptr, rows, classes, 0, None)
+    img2, bias, loss2 = image_of(hip, (rows, classes)), D.fromHost(np.full(classes, 7.0, f32)), D.fromHost(np.array([2.5], f32))
+    call("bf_hip_cross_entropy_sparse_head", dl.ptr, di.ptr, img2.ptr, bias.ptr, loss2.ptr, rows, classes, 1, None)
+    if classes > 8192:   # the separate kernel holds such rows the same way (1024 threads a row): the same bits
+        np.testing.assert_array_equal(img2.toHost(), img.toHost(), err_msg="gradient image")
+        assert loss2.toHost()[0] == np.float32(2.5) + loss.toHost()[0], "the loss is added to the accumulator"
+    else:                # shorter rows are summed in another order there: the same values to an fp32 rounding
+        a, b = as_f32(img2.toHost()).astype(np.float64), as_f32(img.toHost()).astype(np.float64)
+        assert (np.abs(a - b) <= 2.0 ** -7 * np.abs(b)).all(), "gradient image: more than one bf16 step apart"
+        assert (a != b).mean() < 1e-3, "gradient image: too many values on the other side of a rounding boundary"
+        assert abs(loss2.toHost()[0] - 2.5 - loss.toHost()[0]) <= 1e-6 * abs(loss.toHost()[0]) + 1e-6
+    expected_loss, expected_grad = oracle.softmaxCrossEntropySparse(logits, idx)
+    assert abs(loss.toHost()[0] / rows - expected_loss) <= 1e-5 * abs(expected_loss)
+    sums = expected_grad.astype(np.float64).sum(axis=0)
+    assert_close(bias.toHost(), sums.astype(f32), tol=1e-4, what="column sums of the gradient", scale=float(np.abs(expected_grad).max()))
+
+
+def test_cross_entropy_head_refuses_what_it_does_not_serve(hip, rng):
+    D, call = hip.DeviceTensor, hip.capi.call
+    for rows, classes in ((4, 1000), (4, 50257), (4, 40000), (4, 4100)):
+        dl, di = D.fromHost(r(rng, rows, classes)), D.fromHost(np.zeros(rows, f32))
+        img, bias, loss = image_of(hip, (rows, classes + 8)), D((classes,)), D.zeros((1,))
+        with pytest.raises(Exception, match="not served"):
+            call("bf_hip_cross_entropy_sparse_head", dl.ptr, di.ptr, img.ptr, bias.ptr, loss.ptr, rows, classes, 0, None)
+
+
 # (m, k, n): the small-tile route with transposed images, a ragged one, and the large-tile routes (fragments transposed in LDS)
 GEMM_SHAPES = [(64, 40, 24), (300, 72, 520), (4100, 136, 264), (8192, 256, 768), (6001, 520, 1032)]
 
