@@ -246,7 +246,7 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
 // The sparse cross-entropy of a language-model head whose gradient has no reader but the head's own gradient products:
 // the gradient row goes out as its bf16 image only (no fp32 copy is written), and its column sums, the bias gradient of
 // the head, are collected on the way: a thread holds the same columns of every row its block walks, so it adds each
-// gradient value (fp32, before the rounding) to a register per column and the block writes one partial row at the end;
+// gradient value (fp32, before the rounding) to a sum per column and the block writes one partial row at the end;
 // columnPartialsFinishKernel adds the partial rows in index order.  Same arithmetic per element as crossEntropyKernel
 // (1024 threads a row, rows in registers, the next row's loads in flight): the same loss, the same image.
 template <int MAXE, bool NT>
@@ -255,11 +255,14 @@ __global__ void __launch_bounds__(1024) crossEntropyImageKernel(const float* __r
                                                                 float* __restrict__ colPartial, size_t rows, size_t classes, float invRows) {
     constexpr int G = 1024, VEC = 4;
     __shared__ float lds[16];
+    // the column sums live in LDS ([iteration][thread] groups of four: a thread touches only its own, 16 bytes at a time,
+    // consecutive threads consecutive groups), so that two rows' worth of registers remain for the rows themselves
+    extern __shared__ __attribute__((aligned(16))) float colSums[];
     const int t = threadIdx.x;
     using Row = RowCache<G, MAXE, VEC, NT>;
-    Row ahead, col;
+    Row ahead;
 #pragma unroll
-    for (int i = 0; i < MAXE; ++i) col.r[i] = 0.0f;
+    for (int it = 0; it < MAXE / VEC; ++it) *reinterpret_cast<float4v*>(colSums + (it * G + t) * VEC) = float4v{0.0f, 0.0f, 0.0f, 0.0f};
     const size_t rowStep = gridDim.x;
     if (blockIdx.x < rows) ahead.load(logits + size_t(blockIdx.x) * classes, classes, t, -INFINITY);
     for (size_t row = blockIdx.x; row < rows; row += rowStep) {
@@ -298,11 +301,20 @@ __global__ void __launch_bounds__(1024) crossEntropyImageKernel(const float* __r
             }
         }
 #pragma unroll
-        for (int i = 0; i < MAXE; ++i) col.r[i] += c.r[i];   // slots past the row's end hold exp2(-inf) * scale = 0
+        for (int it = 0; it < MAXE / VEC; ++it) {   // slots past the row's end hold exp2(-inf) * scale = 0
+            float4v* sums = reinterpret_cast<float4v*>(colSums + (it * G + t) * VEC);
+            *sums = *sums + float4v{c.r[it * VEC + 0], c.r[it * VEC + 1], c.r[it * VEC + 2], c.r[it * VEC + 3]};
+        }
         c.storeBf16(gradImage + row * classes, classes, t);
         float loss = pTarget >= 0.0f ? -logf(fmaxf(pTarget, 1e-12f)) : 0.0f;
         loss = groupSum<G>(loss, lds);
         if (t == 0) rowLoss[row] = loss;
+    }
+    Row col;
+#pragma unroll
+    for (int it = 0; it < MAXE / VEC; ++it) {
+        const float4v v = *reinterpret_cast<const float4v*>(colSums + (it * G + t) * VEC);
+        col.r[it * VEC + 0] = v.x; col.r[it * VEC + 1] = v.y; col.r[it * VEC + 2] = v.z; col.r[it * VEC + 3] = v.w;
     }
     col.store(colPartial + size_t(blockIdx.x) * classes, classes, t);
 }
@@ -471,13 +483,16 @@ int bf_hip_cross_entropy_sparse_head(const float* logits, const float* targetIdx
     if (partial.status != BF_OK) return partial.status;
     const float invRows = 1.0f / float(rows);
     const bool streaming = streamsPastCache(rows * classes * 6);
-    if (classes <= size_t(1024) * 16) {
-        if (streaming) crossEntropyImageKernel<16, true><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
-        else crossEntropyImageKernel<16, false><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
-    } else {
-        if (streaming) crossEntropyImageKernel<32, true><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
-        else crossEntropyImageKernel<32, false><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
-    }
+    auto launch = [&](auto kernel, size_t ldsBytes) -> int {
+        int st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), ldsBytes);
+        if (st != BF_OK) return st;
+        kernel<<<grid, 1024, ldsBytes, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), partial.as<float>(), rows, classes, invRows);
+        return BF_OK;
+    };
+    int st = BF_OK;
+    if (classes <= size_t(1024) * 16) st = streaming ? launch(crossEntropyImageKernel<16, true>, 1024 * 16 * sizeof(float)) : launch(crossEntropyImageKernel<16, false>, 1024 * 16 * sizeof(float));
+    else st = streaming ? launch(crossEntropyImageKernel<32, true>, 1024 * 32 * sizeof(float)) : launch(crossEntropyImageKernel<32, false>, 1024 * 32 * sizeof(float));
+    if (st != BF_OK) return st;
     BF_LAUNCH_CHECK();
     columnPartialsFinishKernel<<<gridFor(classes / 4, 16), kBlock, 0, s>>>(partial.as<float>(), biasGrad, grid, classes);
     BF_LAUNCH_CHECK();
