@@ -18,7 +18,21 @@ FP32_TOL = 1e-4
 BF16_TOL = 2e-2
 
 
+# largest |gpu - ref| / max|ref| seen by assert_close since the last take_worst(), per first word of `what`
+_worst = {}
+
+
+def take_worst():
+    """The measured errors collected since the last call ({first word of `what`: max |gpu-ref| / max|ref|}), and a reset."""
+    out = dict(_worst)
+    _worst.clear()
+    return out
+
+
 def assert_close(actual, expected, tol=FP32_TOL, what="", scale=0.0):
+    """|gpu - ref| <= tol * |ref| + tol * max(rms(ref), scale) for every element: a relative bound with an ABSOLUTE floor of
+    tol times the tensor's rms (or `scale`, for tensors that are differences of nearly equal terms).  With the default
+    tol = 1e-4 a `scale` of 0.05 * max|ref| is an absolute floor of 5e-6 of the largest element."""
     actual = np.asarray(actual, np.float64)
     expected = np.asarray(expected, np.float64)
     assert actual.shape == expected.shape, f"{what}: shape {actual.shape} != {expected.shape}"
@@ -29,6 +43,8 @@ def assert_close(actual, expected, tol=FP32_TOL, what="", scale=0.0):
     bound = tol * np.abs(expected) + tol * max(rms, float(scale)) + 1e-30
     err = np.abs(actual - expected)
     worst = int(np.argmax(err - bound))
+    _worst[what.split(" ")[0] if what else ""] = max(_worst.get(what.split(" ")[0] if what else "", 0.0),
+                                                     float(err.max() / (np.abs(expected).max() + 1e-30)))
     assert (err <= bound).all(), (
         f"{what}: |gpu-ref|={err.flat[worst]:.3e} > bound {bound.flat[worst]:.3e} at flat index {worst} "
         f"(ref={expected.flat[worst]:.6e}, gpu={actual.flat[worst]:.6e}, rms={rms:.3e}); "

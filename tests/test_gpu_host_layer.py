@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import refvectors as rv
-from parity import BF16_TOL, assert_bits_equal, assert_close
+from parity import BF16_TOL, assert_bits_equal, assert_close, take_worst
 
 pytestmark = pytest.mark.gpu
 f32 = np.float32
@@ -152,6 +152,7 @@ def test_mlm_model_steps_against_oracle(hip, oracle, rng):
         gpu.adamwStep(lr=1e-2)
         for i in range(len(gpu.counts)):
             assert_close(gpu.value(i), cpu.value(i), what=f"step {step} param {gpu.names[i]}", scale=0.02 * 1e-2 / 1e-4)
+        print(f"step {step}: measured max |gpu - cpu| / max |cpu| over all gradients and parameters: {max(take_worst().values()):.2e}")
 
 
 @pytest.mark.parametrize("use_bf16", [False, True])
@@ -207,6 +208,7 @@ def test_tiny_lm_three_steps_match_the_reference_fixture(hip):
             # floor: 2 % of the AdamW step bound lr = 1e-2 (the update is lr * m / (sqrt(v) + eps), ill-conditioned
             # where the gradient is comparable to eps)
             assert_close(model.value(i), gold[f"lm_step{step}_param{i}"], what=f"step {step} param {model.names[i]}", scale=0.02 * 1e-2 / 1e-4)
+        print(f"step {step}: measured max |gpu - reference| / max |reference| over all gradients and parameters: {max(take_worst().values()):.2e}")
 
 
 @pytest.mark.parametrize("use_bf16", [False, True])
@@ -292,6 +294,7 @@ def test_config1_tiny_lm_full_step_against_oracle(hip, oracle, rng, act):
         # AdamW's first step is lr * g / (|g| + eps): where |g| is comparable to eps = 1e-8 the step depends on
         # the gradient's last bits, but it never exceeds lr, so the floor is a small fraction (2 %) of lr = 1e-3
         assert_close(gpu.value(i), cpu.value(i), what="param " + gpu.names[i], scale=0.02 * 1e-3 / 1e-4)
+    print(f"config 1 step: measured max |gpu - cpu| / max |cpu| over all gradients and parameters: {max(take_worst().values()):.2e}")
 
 
 @pytest.mark.parametrize("use_bf16", [False, True])
