@@ -365,10 +365,11 @@ int bf_hip_invalidate_bf16_weight_cache(void);
  * Fused causal attention                                  (reference: fused_attention.hpp:55,73)
  * q:[batch,newLen,dim]  k,v:[batch,totalLen,dim]  heads contiguous in dim, headDim = dim/heads <= 256.
  * Query row i (absolute position oldLen+i) attends to keys j <= oldLen+i.
- * Tuned head dims are 32, 64 and 128 (110-125 TFLOP/s of fp32 MFMA work at 2048-4096 positions).  Head dims above 128
- * are accepted, like the reference accepts them, and give the same results, but run on kernels whose key-tile
- * accumulators do not fit the register file: about 19 TFLOP/s in the dK/dV pass at headDim 256, a sixth of the tuned
- * rate.  Prefer more heads of at most 128.
+ * Tuned head dims are 32, 64 and 128 (forward and backward 110-175 TFLOP/s of fp32 work at 1024-4096 positions).  Head
+ * dims above 128 are accepted, like the reference accepts them, and give the same results, but only on the fp32-MFMA
+ * kernels, whose key-tile accumulators do not fit the register file there: measured at batch 4, 8 heads, 2048
+ * positions, headDim 256: forward 69, dQ 94, dK/dV 40 TFLOP/s, forward + backward 50 TFLOP/s = 0.32 of the fp32 MFMA
+ * peak (headDim 192: 56 / 72 / 34).  Prefer more heads of at most 128.
  * ------------------------------------------------------------------------------------------- */
 /* fusedAttentionForward: out:[batch,newLen,dim]; m,l:[batch,heads,newLen] = row max of the scaled
  * scores and sum of exp(score - m) (the statistics the backward reuses). */
