@@ -179,7 +179,7 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
                          int optimizer, float lr) {
     Handle* handle = static_cast<Handle*>(h);
     return guarded([&] {
-        handle->model->zeroGrad();
+        handle->model->zeroGrad(/*deferred=*/true);
         // the caller's input buffer outlives the step, so the model keeps a view of it instead of a copy; weight images
         // made by the previous step stay in use when nothing has changed a weight since
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));

@@ -71,7 +71,7 @@ public:
             check(status);
         }
         try {
-            model.zeroGrad();
+            model.zeroGrad(/*deferred=*/true);
             DeviceTensor output = model.forward(input, /*inputRangeTrusted=*/true);
             outputRows_ = output.elementCount() / output.shape().back();
             outputElements_ = output.elementCount();

@@ -154,7 +154,10 @@ public:
         const DeviceTensor* grad = &outputGrad;
         DeviceTensor owned;
         for (std::size_t li = layers_.size(); li-- > 0;) {
+            // a deferred zeroGrad(): this layer's gradients are written, not added (see accumulate)
+            overwriteGrads_ = zeroPending_ && layers_[li].gradsAreZero;
             if (layers_[li].fusedRole == 3) {
+                overwriteGrads_ = zeroPending_ && layers_[li].gradsAreZero && layers_[li - 2].gradsAreZero;
                 owned = backwardFusedTriple(li - 2, *grad);
                 grad = &owned;
                 li -= 2;
@@ -168,18 +171,18 @@ public:
                                   li + 1 == layers_.size() ? headBiasGrad : nullptr);
             grad = &owned;
         }
+        overwriteGrads_ = false;
+        zeroPending_ = false;   // every layer has written its gradients
     }
 
-    void zeroGrad() {
-        std::vector<float*> ptrs;
-        std::vector<std::size_t> counts;
-        for (LayerState& layer : layers_)
-            for (Parameter& p : layer.params) {
-                ptrs.push_back(p.grad.data());
-                counts.push_back(p.grad.elementCount());
-            }
-        check(bf_hip_zero_multi(ptrs.data(), counts.data(), ptrs.size(), nullptr));
+    // deferred: nothing is written now.  The next backward pass WRITES every gradient it would have added to a zeroed
+    // buffer (the products straight into the buffers, the rest by a copy in place of the add), which is what a training
+    // step wants: the pass over all gradient buffers that zeroes them is saved.  Until that backward pass the buffers hold
+    // their old values; parameters() zeroes whatever is still pending before it hands the parameters out.
+    void zeroGrad(bool deferred = false) {
         for (LayerState& layer : layers_) layer.gradsAreZero = true;
+        zeroPending_ = deferred;
+        if (!deferred) zeroPendingGradients();
     }
 
     // Incremental forward for generation: only the new positions are processed, K/V of earlier positions
@@ -229,6 +232,10 @@ public:
     }
 
     [[nodiscard]] std::vector<Parameter*> parameters() {
+        if (zeroPending_) {   // a deferred zeroGrad() that no backward pass has made good yet
+            zeroPendingGradients();
+            zeroPending_ = false;
+        }
         std::vector<Parameter*> result;
         for (LayerState& layer : layers_)
             for (Parameter& p : layer.params) result.push_back(&p);
@@ -371,10 +378,26 @@ private:
         }
     }
 
-    // target += delta, unless the backward pass already wrote delta into target (see GradientTargets)
-    static void accumulate(DeviceTensor& target, const DeviceTensor& delta) {
+    // The gradient buffers of every layer whose gradients still count as zero (all of them straight after zeroGrad()).
+    void zeroPendingGradients() {
+        std::vector<float*> ptrs;
+        std::vector<std::size_t> counts;
+        for (LayerState& layer : layers_) {
+            if (!layer.gradsAreZero) continue;
+            for (Parameter& p : layer.params) {
+                ptrs.push_back(p.grad.data());
+                counts.push_back(p.grad.elementCount());
+            }
+        }
+        if (!ptrs.empty()) check(bf_hip_zero_multi(ptrs.data(), counts.data(), ptrs.size(), nullptr));
+    }
+
+    // target += delta, unless the backward pass already wrote delta into target (see GradientTargets); after a deferred
+    // zeroGrad() target = delta (0 + delta without the pass that writes the zeros)
+    void accumulate(DeviceTensor& target, const DeviceTensor& delta) const {
         if (delta.data() == target.data()) return;
-        check(bf_hip_accumulate(target.data(), delta.data(), target.elementCount(), nullptr));
+        if (overwriteGrads_) check(bf_hip_memcpy_d2d(target.data(), delta.data(), target.elementCount() * sizeof(float), nullptr));
+        else check(bf_hip_accumulate(target.data(), delta.data(), target.elementCount(), nullptr));
     }
 
     static bool isBlock(LayerKind kind) {
@@ -520,6 +543,8 @@ private:
     std::string name_;
     bool useBf16_ = false;
     bool cachesValid_ = false;
+    bool zeroPending_ = false;     // a deferred zeroGrad() is outstanding
+    bool overwriteGrads_ = false;  // during backward(): the layer at hand writes its gradients instead of adding them
     std::vector<LayerState> layers_;
     std::size_t generationPosition_ = 0;
 };

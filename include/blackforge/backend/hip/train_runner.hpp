@@ -107,7 +107,7 @@ TrainRunResult runTraining(Model& model, DatasetT& dataset, const TrainOptions& 
             auto batch = dataset.batch(b * options.batchSize, options.batchSize);
             if (vocab.has_value()) detail::validateHostIndexRange(batch.input, *vocab, "embeddingLookup");
             DeviceTensor input = DeviceTensor::fromHost(batch.input);
-            model.zeroGrad();
+            model.zeroGrad(/*deferred=*/true);
             DeviceTensor output = model.forward(input, vocab.has_value());
             if (sparse) detail::validateHostIndexRange(batch.target, output.shape().back(), "softmaxCrossEntropySparse");
             if (maskedLoss) detail::validateHostMaskedIndexRange(batch.target, output.shape().back(), "softmaxCrossEntropyMasked");

@@ -383,3 +383,38 @@ def test_mlp_config2_shape_small(hip, oracle, rng):
     for i in range(len(gpu.counts)):
         e = cpu.grad(i)
         assert_close(gpu.grad(i), e, tol=BF16_TOL, what="mlp grad " + gpu.names[i], scale=float(np.abs(e).max()))
+
+
+@pytest.mark.parametrize("use_bf16", [False, True])
+def test_train_steps_do_not_carry_gradients_over(hip, rng, use_bf16):
+    """A training step zeroes the gradients by having its backward pass WRITE them (no zeroing pass): the gradients after
+    steps on batch A and then batch B must be the bits of a twin model that only ever saw batch B, for every layer kind
+    (embedding, positional table, attention, feed-forward, linear head, and a linear-gelu-linear triple on its own model),
+    and zeroGrad() on its own must still leave zeros behind."""
+    from blackforge_amd import hostlayer as hl
+    D = hip.DeviceTensor
+    vocab, dim, seq, batch, heads, hidden = 64, 32, 16, 4, 2, 64
+    models = []
+    for layers, kw in ((_lm_layers(hl, vocab, dim, seq, heads, hidden, 0), {}),
+                       ([(hl.LINEAR, 48), (hl.GELU,), (hl.LINEAR, 40), (hl.SILU,), (hl.LINEAR, 24)], {"input_features": 40})):
+        a, b = hl.HostModel(layers, use_bf16=use_bf16, **kw), hl.HostModel(layers, use_bf16=use_bf16, **kw)
+        for i, c in enumerate(a.counts):
+            w = r(rng, c, scale=0.1)
+            a.set_value(i, w)
+            b.set_value(i, w)
+        models.append((a, b, not kw))
+    for a, b, is_lm in models:
+        def make():
+            if is_lm:
+                return D.fromHost(rng.integers(0, vocab, (batch, seq)).astype(f32)), D.fromHost(rng.integers(0, vocab, batch * seq).astype(f32)), hl.LOSS_SPARSE_CE
+            return D.fromHost(r(rng, 12, 40)), D.fromHost(r(rng, 12, 24)), hl.LOSS_MSE
+        xa, ta, kind = make()
+        xb, tb, _ = make()
+        a.trainStep(xa, ta, kind, optimizer=0)
+        a.trainStep(xb, tb, kind, optimizer=0)
+        b.trainStep(xb, tb, kind, optimizer=0)
+        for i in range(len(a.counts)):
+            assert_bits_equal(a.grad(i), b.grad(i), "gradient of " + a.names[i] + " after two steps against one")
+        a.zeroGrad()
+        for i in range(len(a.counts)):
+            assert not a.grad(i).any(), "zeroGrad() leaves zeros: " + a.names[i]
