@@ -879,6 +879,269 @@ __device__ __forceinline__ void storeKeyGradients(const AttnParams& p, const flo
     }
 }
 
+// Head dims above 128 with the dS hand-over: the key-tile owner works in two passes over the query tiles that share out
+// the four products instead of repeating two of them.  Pass "P" (dkvTileP) forms S = Q K^T, the probabilities P, parks
+// P where dS will go (same 32 x 32 sub-blocks, the lane's own sixteen values) and accumulates dV += P^T dO over the whole
+// head dim; it holds the K rows and one accumulator set.  Pass "dS" (dkvTileDs) forms dP = dO V^T, reads P back (each lane
+// the values it wrote), turns it into dS = P (dP - D) in place and accumulates dK += dS^T Q; it holds the V rows and
+// one accumulator set.  Every product is formed once, each output element sees the same MFMAs in the same order as in
+// the one-pass kernel, and a wavefront stays inside its 512 registers, where K rows, V rows and both accumulator sets
+// (512 registers by themselves) made the kernel form S and dP twice and spill half its state.
+// The contraction over the head dim and the rank-one updates of an accumulator set, as fenced slices: left to itself the
+// scheduler hoists every LDS read of the unrolled loop ahead of the MFMAs (128 registers of operands at head dim 256),
+// which is what drove these kernels out of their registers.  One group of reads is in flight ahead of the MFMAs that
+// use the group before it; a scheduling fence closes each group.
+template <int HDP>
+__device__ __forceinline__ float16v headDotFenced(const float* __restrict__ ldsRow, const float (&reg)[HDP / 2], float16v acc) {
+    float4v a = loadf4(ldsRow);
+#pragma unroll
+    for (int t = 0; t < HDP / 2; t += 4) {
+        float4v next = a;
+        if (t + 4 < HDP / 2) next = loadf4(ldsRow + t + 4);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, reg[t], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, reg[t + 1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, reg[t + 2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, reg[t + 3], acc, 0, 0, 0);
+        a = next;
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    return acc;
+}
+// acc[dt] += w[r] (x) row_r[dt*32 + li] for the sixteen rows dRow(r, half) of a 32-row block at `rows`
+template <int HDP>
+__device__ __forceinline__ void rankUpdatesFenced(const float* __restrict__ rows, const float16v& w, float16v (&acc)[HDP / 32], int half, int li) {
+    constexpr int LDSW = HDP + 4, DT = HDP / 32;
+    float cur[DT], nxt[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) cur[dt] = rows[dRow(0, half) * LDSW + li + dt * 32];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        if (r + 1 < 16) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) nxt[dt] = rows[dRow(r + 1, half) * LDSW + li + dt * 32];
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[r], cur[dt], acc[dt], 0, 0, 0);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) cur[dt] = nxt[dt];
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+template <int HDP, int BQ, bool MASKED>
+__device__ __forceinline__ void dkvTileP(const float* __restrict__ qs, const float* __restrict__ gs, const float* __restrict__ stats,
+                                         const float (&kreg)[HDP / 2], float16v (&dv)[HDP / 32], int qt0, int key, bool keyValid, int oldLen,
+                                         int half, int li, float* __restrict__ dsLane, size_t dsStride, int newLen) {
+    constexpr int LDSW = HDP + 4, NSB = BQ / 32;
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+        float16v pr;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) pr[r] = 0.0f;
+        pr = headDotFenced<HDP>(qs + (sb * 32 + li) * LDSW + half * (HDP / 2), kreg, pr);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const float4v lse4 = loadf4(stats + sb * 32 + 8 * g + 4 * half);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int r = 4 * g + c;
+                float prob = fastExp2(pr[r] - lse4[c]);
+                if constexpr (MASKED) {
+                    const int qi = qt0 + sb * 32 + dRow(r, half);
+                    prob = (key > oldLen + qi || !keyValid) ? 0.0f : prob;
+                }
+                pr[r] = prob;
+            }
+        }
+        if (qt0 + sb * 32 < newLen) {
+            float* dst = dsLane + sb * dsStride;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(pr[r], dst + (8 * (r >> 2) + (r & 3)) * 32);
+        }
+        rankUpdatesFenced<HDP>(gs + sb * 32 * LDSW, pr, dv, half, li);
+    }
+}
+
+template <int HDP, int BQ>
+__device__ __forceinline__ void dkvTileDs(const float* __restrict__ qs, const float* __restrict__ gs, const float* __restrict__ stats,
+                                          const float (&vreg)[HDP / 2], float16v (&dk)[HDP / 32], int qt0, int half, int li,
+                                          float* __restrict__ dsLane, size_t dsStride, int newLen) {
+    constexpr int LDSW = HDP + 4, NSB = BQ / 32;
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+        float* dst = dsLane + sb * dsStride;
+        const bool stored = qt0 + sb * 32 < newLen;   // rows past the sequence hold no P (it is zero there)
+        float16v pr;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) pr[r] = stored ? __builtin_nontemporal_load(dst + (8 * (r >> 2) + (r & 3)) * 32) : 0.0f;
+        float16v dsv;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dsv[r] = 0.0f;
+        dsv = headDotFenced<HDP>(gs + (sb * 32 + li) * LDSW + half * (HDP / 2), vreg, dsv);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const float4v d4 = loadf4(stats + BQ + sb * 32 + 8 * g + 4 * half);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int r = 4 * g + c;
+                dsv[r] = pr[r] * (dsv[r] - d4[c]);      // dS (without the scale factor)
+            }
+        }
+        if (stored) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(dsv[r], dst + (8 * (r >> 2) + (r & 3)) * 32);
+        }
+        rankUpdatesFenced<HDP>(qs + sb * 32 * LDSW, dsv, dk, half, li);
+    }
+}
+
+// One pass of the key-tile owner over its query tiles for head dims above 128: Q and dO tiles (and lse2, D) through the
+// double-buffered LDS stage, one barrier per tile.  MODE 0: dkvTileP with `reg` = the K rows and `acc` = dV; MODE 1:
+// dkvTileDs with `reg` = the V rows and `acc` = dK.  With 16-byte aligned rows (VEC4) the tiles go from global memory
+// straight into LDS (global_load_lds, one 1 KiB row per wavefront instruction, lanes past the head dim switched off: those
+// columns were zeroed once), which frees the 64 registers a tile in flight would occupy; rows past the sequence repeat
+// its last row (finite values that meet P = 0 and dS = 0).  Otherwise tiles are staged through registers as in
+// attnBackwardDkvKernel.
+typedef __attribute__((address_space(1))) const void* GlobalPtr;
+typedef __attribute__((address_space(3))) void* LdsPtr;
+template <int HDP, int BQ, bool VEC4, int MODE>
+__device__ __forceinline__ void dkvStreamPass(const AttnParams& p, float* __restrict__ qs, float* __restrict__ gs, float* __restrict__ stats,
+                                              const float (&reg)[HDP / 2], float16v (&acc)[HDP / 32], int bh, int kt, size_t qOff,
+                                              size_t statOff, int waveK0, int key, bool keyValid, int half, int li, int tid) {
+    constexpr int LDSW = HDP + 4, TILE = BQ * LDSW;
+    const int hd = p.hd, dim = p.dim;
+    int firstQuery = kt * 128 - p.oldLen;
+    if (firstQuery < 0) firstQuery = 0;
+    const int q0Start = (firstQuery / BQ) * BQ;
+    const int numQTiles = q0Start < p.newLen ? (p.newLen - q0Start + BQ - 1) / BQ : 0;
+    const size_t dsStride = size_t(p.nkb) * 1024;
+    float* const dsColumn = p.ds + (size_t(bh) * p.nqb * p.nkb + size_t(waveK0 >> 5)) * 1024;   // wave-uniform
+    const int dsLaneOffset = half * 128 + li;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    auto tileBody = [&](int t, int qt0) __attribute__((always_inline)) {
+        if (p.oldLen + qt0 + BQ - 1 >= waveK0 && waveK0 < p.totalLen) {
+            const float* qcur = qs + (t & 1) * TILE;
+            const float* gcur = gs + (t & 1) * TILE;
+            const float* scur = stats + (t & 1) * 2 * BQ;
+            float* dsLane = dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset;
+            if constexpr (MODE == 0) {
+                const bool masked = (waveK0 + 31 > p.oldLen + qt0) || (waveK0 + 32 > p.totalLen);
+                if (masked) dkvTileP<HDP, BQ, true>(qcur, gcur, scur, reg, acc, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride, p.newLen);
+                else dkvTileP<HDP, BQ, false>(qcur, gcur, scur, reg, acc, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride, p.newLen);
+            } else {
+                dkvTileDs<HDP, BQ>(qcur, gcur, scur, reg, acc, qt0, half, li, dsLane, dsStride, p.newLen);
+            }
+        }
+    };
+    float statNext = 0.0f;
+    auto fetchStats = [&](int qt0) __attribute__((always_inline)) {
+        const int qi = qt0 + (tid < BQ ? tid : tid - BQ);
+        if (tid < BQ) statNext = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
+        else if (tid < 2 * BQ) statNext = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
+    };
+    if constexpr (VEC4) {
+        // wavefront w brings rows w, w + 4, ... of either tile; lane l the 16 bytes at column 4 l
+        const bool columnValid = 4 * lane < hd;
+        const float* qBase = p.q + qOff + 4 * lane;
+        const float* gBase = p.dO + qOff + 4 * lane;
+        auto issueTile = [&](int qt0, int buf) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < BQ / 4; ++i) {
+                const int r = wave + 4 * i;
+                const size_t row = size_t(min(qt0 + r, p.newLen - 1)) * dim;
+                if (columnValid) {
+                    __builtin_amdgcn_global_load_lds((GlobalPtr)(qBase + row), (LdsPtr)(qs + buf * TILE + r * LDSW), 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((GlobalPtr)(gBase + row), (LdsPtr)(gs + buf * TILE + r * LDSW), 16, 0, 0);
+                }
+            }
+        };
+        if (hd < HDP) {   // the columns past the head dim are never loaded: zero them once (both buffers of both tiles)
+            for (int i = tid; i < 4 * BQ * (LDSW / 4); i += 256) storef4(qs + 4 * i, float4v{0.0f, 0.0f, 0.0f, 0.0f});
+            __syncthreads();
+        }
+        if (numQTiles > 0) {
+            issueTile(q0Start, 0);
+            fetchStats(q0Start);
+            if (tid < 2 * BQ) stats[tid] = statNext;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        for (int t = 0; t < numQTiles; ++t) {
+            const int qt0 = q0Start + t * BQ;
+            if (t + 1 < numQTiles) {   // buffer (t+1)&1 was last read before the barrier that ended the tile before
+                issueTile(qt0 + BQ, (t + 1) & 1);
+                fetchStats(qt0 + BQ);
+            }
+            tileBody(t, qt0);
+            if (t + 1 < numQTiles && tid < 2 * BQ) stats[((t + 1) & 1) * 2 * BQ + tid] = statNext;
+            // the tile's loads have landed in LDS (the stores of the tile body, issued a hundred MFMAs ago, are long done)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();   // after the last tile too: the next pass writes the LDS buffers again
+        }
+    } else {
+        TileRegs<HDP, BQ> qNext, gNext;
+        auto fetchAll = [&](int qt0) __attribute__((always_inline)) {
+            fetchHeadTile<HDP, BQ, VEC4>(qNext, p.q + qOff, dim, qt0, p.newLen, hd, tid);
+            fetchHeadTile<HDP, BQ, VEC4>(gNext, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+            fetchStats(qt0);
+        };
+        auto commitAll = [&](int buf) __attribute__((always_inline)) {
+            commitHeadTile<HDP, BQ>(qs + buf * TILE, qNext, tid);
+            commitHeadTile<HDP, BQ>(gs + buf * TILE, gNext, tid);
+            if (tid < 2 * BQ) stats[buf * 2 * BQ + tid] = statNext;
+        };
+        if (numQTiles > 0) {
+            fetchAll(q0Start);
+            commitAll(0);
+            if (numQTiles > 1) fetchAll(q0Start + BQ);
+        }
+        __syncthreads();
+        for (int t = 0; t < numQTiles; ++t) {
+            const int qt0 = q0Start + t * BQ;
+            tileBody(t, qt0);
+            if (t + 1 < numQTiles) {
+                commitAll((t + 1) & 1);
+                if (t + 2 < numQTiles) fetchAll(qt0 + 2 * BQ);
+            }
+            __syncthreads();   // after the last tile too: the next pass writes the LDS buffers again
+        }
+    }
+}
+
+// One of the two key gradients (IS_K: dK, scaled; else dV), fp32 tensor and bf16 image, as storeKeyGradients stores them.
+template <int HDP, bool IS_K>
+__device__ __forceinline__ void storeOneKeyGradient(const AttnParams& p, const float16v (&acc)[HDP / 32], int b, int h, int waveK0,
+                                                    size_t kOff, int half, int li) {
+    const int hd = p.hd, dim = p.dim;
+    float* __restrict__ out = IS_K ? p.dK : p.dV;
+    unsigned short* __restrict__ img = IS_K ? p.dKImg : p.dVImg;
+    const float mul = IS_K ? p.scale : 1.0f;
+    const bool pairs = (hd & 1) == 0 && (p.imgLd & 1u) == 0 && (reinterpret_cast<uintptr_t>(img) & 3u) == 0;
+#pragma unroll
+    for (int dt = 0; dt < HDP / 32; ++dt) {
+        const int d = dt * 32 + li;
+        if (d < hd) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int kk = waveK0 + dRow(r, half);
+                if (kk < p.totalLen) {
+                    const float v = acc[dt][r] * mul;
+                    if (out) out[kOff + size_t(kk) * dim + d] = v;
+                    if (img) {
+                        const size_t at = (size_t(b) * p.totalLen + kk) * p.imgLd + size_t(h) * hd + d;
+                        if (pairs) {
+                            const float next = __shfl_down(v, 1, 64);
+                            if ((li & 1) == 0) *reinterpret_cast<unsigned*>(img + at) = unsigned(toBf16Bits(v)) | unsigned(toBf16Bits(next)) << 16;
+                        } else {
+                            img[at] = toBf16Bits(v);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
 // OCC = wavefronts per SIMD the register allocation is held to.  At OCC 2 (head dims up to 64) two workgroups share
 // a CU and cover each other's barriers and tile hand-overs, at the price of a handful of spilled registers; it pays
 // once the grid has more workgroups than two per CU, below that one roomier workgroup per CU is faster.
@@ -902,6 +1165,32 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
     const int waveK0 = kt * 128 + wave * 32;
     const int key = waveK0 + li;                       // this lane's key (as B-operand column)
     const bool keyValid = key < p.totalLen;
+    if constexpr (HDP > 128 && STORE) {
+        // two passes that share out the products (dkvTileP / dkvTileDs above)
+        {
+            float kreg[HDP / 2];
+            loadRowOperand<HDP, VEC4>(kreg, p.k + kOff + size_t(key) * dim, keyValid, hd, half, p.scale * kLog2e);
+            float16v dv[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) dv[dt][r] = 0.0f;
+            dkvStreamPass<HDP, BQ, VEC4, 0>(p, qs, gs, stats, kreg, dv, bh, kt, qOff, statOff, waveK0, key, keyValid, half, li, tid);
+            storeOneKeyGradient<HDP, false>(p, dv, b, h, waveK0, kOff, half, li);
+        }
+        {
+            float vreg[HDP / 2];
+            loadRowOperand<HDP, VEC4>(vreg, p.v + kOff + size_t(key) * dim, keyValid, hd, half, 1.0f);
+            float16v dk[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) dk[dt][r] = 0.0f;
+            dkvStreamPass<HDP, BQ, VEC4, 1>(p, qs, gs, stats, vreg, dk, bh, kt, qOff, statOff, waveK0, key, keyValid, half, li, tid);
+            storeOneKeyGradient<HDP, true>(p, dk, b, h, waveK0, kOff, half, li);
+        }
+        return;
+    }
     float kreg[HDP / 2], vreg[HDP / 2];
     loadRowOperand<HDP, VEC4>(kreg, p.k + kOff + size_t(key) * dim, keyValid, hd, half, p.scale * kLog2e);
     loadRowOperand<HDP, VEC4>(vreg, p.v + kOff + size_t(key) * dim, keyValid, hd, half, 1.0f);

@@ -39,7 +39,10 @@ def run_gpu(hip, q, k, v, go, heads, scale, old_len):
 CASES = [(1, 1, 1, 0, 2), (1, 2, 3, 0, 2), (2, 2, 5, 0, 4), (2, 3, 33, 0, 32), (1, 2, 70, 0, 64), (1, 1, 40, 0, 128),
          (1, 1, 37, 0, 256), (2, 2, 3, 9, 16), (1, 2, 1, 37, 32), (1, 2, 129, 0, 64), (1, 1, 200, 57, 40), (2, 1, 130, 130, 8),
          (1, 4, 256, 0, 32), (1, 2, 300, 0, 100), (1, 1, 64, 0, 7), (1, 2, 70, 5, 62), (1, 1, 45, 0, 126), (1, 2, 150, 0, 256),
-         (1, 1, 70, 30, 200)]
+         (1, 1, 70, 30, 200),
+         # head dims above 128 over several key tiles and query tiles (the key-tile owner's two passes that share out
+         # the products: P parked in the dS buffer, read back and replaced by dS), ragged ends, an offset, a 4-byte aligned dim
+         (2, 2, 300, 0, 192), (1, 2, 260, 40, 256), (1, 1, 129, 129, 136), (1, 1, 140, 0, 130)]
 
 
 @pytest.mark.parametrize("batch,heads,new_len,old_len,hd", CASES)
