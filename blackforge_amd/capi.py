@@ -117,6 +117,7 @@ SIGNATURES = {
                                                      c_size, c_size, c_size, c_int, S],
     "bf_hip_feedforward_bf16_backward_img": [P, P, P, P, P, P, P, P, c_int, P, P, P, P, P, c_size, c_size, c_size, c_int, S],
     "bf_hip_invalidate_bf16_weight_cache": [],
+    "bf_hip_bf16_weight_cache_refresh": [ctypes.POINTER(c_ptr), c_size, S],
     "bf_hip_gemm_bf16_set_route": [c_int],
     "bf_hip_mfma_only_loop": [P, P, c_int, c_int, c_int, S],
     "bf_hip_attention_forward": [P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],

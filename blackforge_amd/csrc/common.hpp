@@ -101,8 +101,8 @@ struct Scratch {
 // A small table of descriptors (pointers, counts, chunk lists) that a multi-tensor kernel reads from
 // device memory.  The same table is needed step after step, so the device copy is kept per (device,
 // slot) and re-uploaded only when the host bytes change; an unchanged table costs no copy and no
-// host synchronisation.  `slot` separates users (zero, sgd, adamw).
-enum { kSlotZero = 0, kSlotSgd = 1, kSlotAdamW = 2, kSlotCount = 3 };
+// host synchronisation.  `slot` separates users (zero, sgd, adamw, the weight-image refresh).
+enum { kSlotZero = 0, kSlotSgd = 1, kSlotAdamW = 2, kSlotConvert = 3, kSlotCount = 4 };
 int uploadDescriptorTable(int slot, const void* hostBytes, size_t bytes, hipStream_t stream, const void** devicePtr);
 
 // ---- device helpers ----------------------------------------------------------------------------

@@ -16,10 +16,14 @@
 // cutting K into slices that a second kernel adds up in a fixed order (small products).
 #include "common.hpp"
 
+#include <algorithm>
 #include <atomic>
 #include <type_traits>
 #include <map>
+#include <set>
+#include <tuple>
 #include <unordered_map>
+#include <vector>
 
 namespace bf {
 namespace {
@@ -68,15 +72,11 @@ __global__ void __launch_bounds__(kBlock) convertKernel(const float* __restrict_
 // Up to three matrices of one shape in one launch (blockIdx.z): matrix z is read from xs.p[z] and written `outStep`
 // (and `plainStep`) elements after the one before.
 struct ConvertSources { const float* p[3]; };
-__global__ void __launch_bounds__(kBlock) convertTransposeKernel(ConvertSources xs, unsigned short* __restrict__ out,
-                                                                 size_t rows, size_t cols, size_t rowsPad, int vec,
-                                                                 unsigned short* __restrict__ plain, size_t ldPlain, size_t outStep,
-                                                                 size_t plainStep) {
-    __shared__ __attribute__((aligned(16))) unsigned short tile[64][72];   // [column][row], 144-byte pitch
-    const float* __restrict__ x = blockIdx.z == 0 ? xs.p[0] : blockIdx.z == 1 ? xs.p[1] : xs.p[2];
-    out += blockIdx.z * outStep;
-    if (plain) plain += blockIdx.z * plainStep;
-    const size_t r0 = size_t(blockIdx.y) * 64, c0 = size_t(blockIdx.x) * 64;
+// One 64 x 64 tile (rows r0.., columns c0..) of that conversion; `tile` is the workgroup's [64][72] LDS array.
+// `out` may be NULL when `plain` is not: the plain image alone is written.
+__device__ __forceinline__ void convertTransposeTile(const float* __restrict__ x, unsigned short* __restrict__ out, size_t rows,
+                                                     size_t cols, size_t rowsPad, int vec, unsigned short* __restrict__ plain,
+                                                     size_t ldPlain, size_t r0, size_t c0, unsigned short (*tile)[72]) {
     const size_t colsPad = (cols + 7) / 8 * 8;
     if (vec) {
         const int cg = threadIdx.x & 15, rr = threadIdx.x >> 4;   // 16 column groups x 16 rows per pass
@@ -103,6 +103,7 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(ConvertSources 
                 *reinterpret_cast<uint2v*>(plain + gr * ldPlain + gc) = packed;
             }
         }
+        if (!out) return;   // (uniform) the plain image alone was asked for
         __syncthreads();
         const int chunk = threadIdx.x & 7, cc = threadIdx.x >> 3;   // 8 chunks of 8 rows x 32 columns per pass
 #pragma unroll
@@ -123,6 +124,7 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(ConvertSources 
         tile[tx][r] = b;
         if (plain && gr < rows && gc < colsPad) plain[gr * ldPlain + gc] = b;
     }
+    if (!out) return;
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -130,6 +132,35 @@ __global__ void __launch_bounds__(kBlock) convertTransposeKernel(ConvertSources 
         size_t gc = c0 + c, gr = r0 + tx;
         if (gc < cols && gr < rowsPad) out[gc * rowsPad + gr] = tile[c][tx];
     }
+}
+__global__ void __launch_bounds__(kBlock) convertTransposeKernel(ConvertSources xs, unsigned short* __restrict__ out,
+                                                                 size_t rows, size_t cols, size_t rowsPad, int vec,
+                                                                 unsigned short* __restrict__ plain, size_t ldPlain, size_t outStep,
+                                                                 size_t plainStep) {
+    __shared__ __attribute__((aligned(16))) unsigned short tile[64][72];   // [column][row], 144-byte pitch
+    const float* __restrict__ x = blockIdx.z == 0 ? xs.p[0] : blockIdx.z == 1 ? xs.p[1] : xs.p[2];
+    convertTransposeTile(x, out + blockIdx.z * outStep, rows, cols, rowsPad, vec, plain ? plain + blockIdx.z * plainStep : nullptr, ldPlain,
+                         size_t(blockIdx.y) * 64, size_t(blockIdx.x) * 64, tile);
+}
+
+// The same conversion for a list of matrices of any shapes in one launch (every weight of a model after an optimizer
+// step): the tiles of all matrices are laid end to end, a workgroup finds its matrix in the table (owningTensor) and
+// its tile inside it, column tiles fastest.
+struct ConvertEntry {
+    const float* x;
+    unsigned short* out;
+    unsigned short* plain;
+    unsigned rows, cols, rowsPad, ldPlain;
+    unsigned firstBlock, tilesX;
+    int vec;
+    unsigned pad;
+};
+__global__ void __launch_bounds__(kBlock) convertTransposeMultiKernel(const ConvertEntry* __restrict__ table, int numEntries) {
+    __shared__ __attribute__((aligned(16))) unsigned short tile[64][72];
+    const ConvertEntry e = table[owningTensor(table, numEntries, blockIdx.x)];
+    const unsigned local = blockIdx.x - e.firstBlock;
+    const unsigned ty = local / e.tilesX, tx = local - ty * e.tilesX;
+    convertTransposeTile(e.x, e.out, e.rows, e.cols, e.rowsPad, e.vec, e.plain, e.ldPlain, size_t(ty) * 64, size_t(tx) * 64, tile);
 }
 
 // ---- the GEMM ----------------------------------------------------------------------------------
@@ -1586,6 +1617,7 @@ struct CachedWeight {
     size_t generation;   // the generation whose weights the image holds; 0 = never filled
     void* buffer;
     size_t bytes;
+    size_t count, rows, cols;   // the weights behind the image: `count` matrices [rows, cols]
 };
 // One generation per cache: an invalidation recorded into a graph must not mark the eager images stale, and the eager
 // generation also advances whenever a recorded graph is launched (its kernels may step an optimizer over the weights
@@ -1621,7 +1653,8 @@ size_t weightImageBytes(size_t count, size_t rows, size_t cols, int layout) {
 
 // The cache entry of `key` with a buffer of `bytes` (acquired, or re-acquired when the size changed); its generation
 // says whether the buffer's contents are current.  Entries stay where they are in the map, so the pointer holds.
-int cacheSlot(const WeightKey& key, size_t bytes, CachedWeight** slot) {
+int cacheSlot(const WeightKey& key, size_t count, size_t rows, size_t cols, CachedWeight** slot) {
+    const size_t bytes = weightImageBytes(count, rows, cols, std::get<4>(key));
     auto& cache = weightCache();
     auto it = cache.find(key);
     if (it != cache.end() && it->second.bytes != bytes) {
@@ -1633,8 +1666,11 @@ int cacheSlot(const WeightKey& key, size_t bytes, CachedWeight** slot) {
         void* buf = nullptr;
         int st = bf_hip_pool_acquire(bytes, &buf);
         if (st != BF_OK) return st;
-        it = cache.emplace(key, CachedWeight{0, buf, bytes}).first;
+        it = cache.emplace(key, CachedWeight{0, buf, bytes, count, rows, cols}).first;
     }
+    it->second.count = count;   // (equal bytes do not pin the shape)
+    it->second.rows = rows;
+    it->second.cols = cols;
     *slot = &it->second;
     return BF_OK;
 }
@@ -1665,14 +1701,14 @@ int weightImage(const float* const* w, size_t count, size_t rows, size_t cols, i
     const float* w1 = count > 1 ? w[1] : nullptr;
     const float* w2 = count > 2 ? w[2] : nullptr;
     CachedWeight* slot = nullptr;
-    int st = cacheSlot(WeightKey{dev, w[0], w1, w2, layout}, bytes, &slot);
+    int st = cacheSlot(WeightKey{dev, w[0], w1, w2, layout}, count, rows, cols, &slot);
     if (st != BF_OK) return st;
     *image = static_cast<unsigned short*>(slot->buffer);
     if (slot->generation == generation()) return BF_OK;
     CachedWeight* mate = nullptr;
     if (layout == 1 || (layout == 2 && cols % 8 == 0)) {
         const int mateLayout = layout == 1 ? 0 : 3;
-        st = cacheSlot(WeightKey{dev, w[0], w1, w2, mateLayout}, weightImageBytes(count, rows, cols, mateLayout), &mate);
+        st = cacheSlot(WeightKey{dev, w[0], w1, w2, mateLayout}, count, rows, cols, &mate);
         if (st != BF_OK) return st;
         if (mate->generation == generation()) mate = nullptr;   // already current
     }
@@ -1685,6 +1721,79 @@ int weightImage(const float* const* w, size_t count, size_t rows, size_t cols, i
 int weightImage(const float* w, size_t rows, size_t cols, bool transposed, bool cache, hipStream_t s, unsigned short** image,
                 size_t* imageBytes) {
     return weightImage(&w, 1, rows, cols, transposed ? 1 : 0, cache, s, image, imageBytes);
+}
+
+
+// After an optimizer step over `changed`: every transposed image (with its plain mate) that was in use during the
+// generation that just ended and whose weights are all among `changed` is made again, all of them in one launch, and
+// is current in the new generation.  The caller has already advanced the generation.
+int refreshImagesOf(const float* const* changed, size_t count, size_t ending, hipStream_t s) {
+    int dev = 0;
+    BF_HIP_TRY(hipGetDevice(&dev));
+    const std::set<const float*> touched(changed, changed + count);
+    auto& cache = weightCache();
+    std::vector<ConvertEntry> table;
+    std::vector<CachedWeight*> made;
+    size_t blocks = 0;
+    for (auto& [key, slot] : cache) {
+        const int layout = std::get<4>(key);
+        if (std::get<0>(key) != dev || (layout != 1 && layout != 2) || slot.generation != ending) continue;
+        const float* w[3] = {std::get<1>(key), std::get<2>(key), std::get<3>(key)};
+        bool all = slot.count >= 1 && slot.count <= 3;
+        for (size_t i = 0; i < slot.count && all; ++i) all = w[i] != nullptr && touched.count(w[i]) != 0;
+        if (!all || slot.rows >= (size_t(1) << 31) || slot.cols >= (size_t(1) << 31)) continue;
+        CachedWeight* mate = nullptr;
+        if (layout == 1 || slot.cols % 8 == 0) {
+            auto it = cache.find(WeightKey{dev, w[0], w[1], w[2], layout == 1 ? 0 : 3});
+            if (it != cache.end() && it->second.generation == ending && it->second.rows == slot.rows && it->second.cols == slot.cols &&
+                it->second.count == slot.count)
+                mate = &it->second;
+        }
+        const size_t rowsPad = pad8(slot.rows);
+        const size_t ldPlain = layout == 1 ? pad8(slot.cols) : slot.count * slot.cols;
+        for (size_t i = 0; i < slot.count; ++i) {
+            unsigned short* out = static_cast<unsigned short*>(slot.buffer) + i * slot.cols * rowsPad;
+            unsigned short* plain = mate ? static_cast<unsigned short*>(mate->buffer) + i * slot.cols : nullptr;
+            const size_t tilesX = ((plain ? pad8(slot.cols) : slot.cols) + 63) / 64, tilesY = (rowsPad + 63) / 64;
+            const int vec = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(plain)) & 15u) == 0 && ldPlain % 8 == 0;
+            table.push_back(ConvertEntry{w[i], out, plain, unsigned(slot.rows), unsigned(slot.cols), unsigned(rowsPad), unsigned(ldPlain),
+                                         unsigned(blocks), unsigned(tilesX), vec, 0});
+            blocks += tilesX * tilesY;
+            if (blocks >= (size_t(1) << 31)) return failInvalid("bf16_weight_cache_refresh", "too many elements for one launch");
+        }
+        made.push_back(&slot);
+        if (mate) made.push_back(mate);
+    }
+    // plain images in use without a transposed one (the input-gradient product of weights whose forward pass took
+    // another form): the same kernel, writing the plain image only
+    for (auto& [key, slot] : cache) {
+        const int layout = std::get<4>(key);
+        if (std::get<0>(key) != dev || (layout != 0 && layout != 3) || slot.generation != ending) continue;
+        if (std::find(made.begin(), made.end(), &slot) != made.end()) continue;
+        const float* w[3] = {std::get<1>(key), std::get<2>(key), std::get<3>(key)};
+        bool all = slot.count >= 1 && slot.count <= 3;
+        for (size_t i = 0; i < slot.count && all; ++i) all = w[i] != nullptr && touched.count(w[i]) != 0;
+        if (!all || slot.rows >= (size_t(1) << 31) || slot.cols >= (size_t(1) << 31)) continue;
+        const size_t ldPlain = layout == 0 ? pad8(slot.cols) : slot.count * slot.cols;
+        for (size_t i = 0; i < slot.count; ++i) {
+            unsigned short* plain = static_cast<unsigned short*>(slot.buffer) + i * slot.cols;
+            const size_t tilesX = (pad8(slot.cols) + 63) / 64, tilesY = (slot.rows + 63) / 64;
+            const int vec = (reinterpret_cast<uintptr_t>(plain) & 15u) == 0 && ldPlain % 8 == 0;
+            table.push_back(ConvertEntry{w[i], nullptr, plain, unsigned(slot.rows), unsigned(slot.cols), unsigned(pad8(slot.rows)),
+                                         unsigned(ldPlain), unsigned(blocks), unsigned(tilesX), vec, 0});
+            blocks += tilesX * tilesY;
+            if (blocks >= (size_t(1) << 31)) return failInvalid("bf16_weight_cache_refresh", "too many elements for one launch");
+        }
+        made.push_back(&slot);
+    }
+    if (blocks == 0) return BF_OK;
+    const void* device = nullptr;
+    int st = uploadDescriptorTable(kSlotConvert, table.data(), table.size() * sizeof(ConvertEntry), s, &device);
+    if (st != BF_OK) return st;
+    convertTransposeMultiKernel<<<unsigned(blocks), kBlock, 0, s>>>(static_cast<const ConvertEntry*>(device), int(table.size()));
+    BF_LAUNCH_CHECK();
+    for (CachedWeight* slot : made) slot->generation = generation();
+    return BF_OK;
 }
 
 }  // namespace
@@ -2220,6 +2329,16 @@ int bf_hip_invalidate_bf16_weight_cache(void) {
     }
     ++bf::generation();
     return BF_OK;
+}
+
+int bf_hip_bf16_weight_cache_refresh(const float* const* changed, size_t count, bf_stream_t stream) {
+    BF_REQUIRE(changed || count == 0, "NULL pointer");
+    const size_t ending = bf::generation();
+    int st = bf_hip_invalidate_bf16_weight_cache();
+    // (a recording makes its images where its products need them: a refresh recorded at the end of a step would only
+    // be repeated by the conversions recorded at its beginning)
+    if (st != BF_OK || count == 0 || bf::capturing()) return st;
+    return bf::refreshImagesOf(changed, count, ending, bf::asStream(stream));
 }
 
 }  // extern "C"

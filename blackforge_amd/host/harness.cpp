@@ -194,8 +194,9 @@ int bfh_model_train_step(void* h, const float* input, int rank, const size_t* sh
         if (optimizer == 1) {
             if (!handle->adamw) handle->adamw = std::make_unique<hip::AdamW>(lr, 0.9F, 0.999F, 1e-8F, 0.01F);
             handle->adamw->setLearningRate(lr);
-            handle->weightImagesCurrent = false;
             handle->adamw->step(handle->params);
+            if (handle->model->usesBf16()) hip::refreshWeightImages(handle->params);   // all their images in one launch
+            else handle->weightImagesCurrent = false;
         }
     });
 }

@@ -360,6 +360,13 @@ int bf_hip_gemm_bf16_set_route(int route);
 int bf_hip_mfma_only_loop(const uint16_t* operands, float* out, int shape, int workgroups, int kSteps, bf_stream_t stream);
 /* invalidateBf16WeightCache: ops.hpp:80 */
 int bf_hip_invalidate_bf16_weight_cache(void);
+/* For the caller that has just changed `count` weights in place (an optimizer step over changed[0..count)): the same
+ * as bf_hip_invalidate_bf16_weight_cache(), and then every cached transposed image (with the plain image of the same
+ * weights) that was used since the previous invalidation and whose weights are all among `changed` is made again from
+ * the new values, all of them in ONE launch, and counts as current.  The reference converts each weight again inside
+ * the next forward pass (ops_tensorcore.cu:117-131 after :448); the images and the products are the same, only the
+ * dozens of small conversion launches of a step become one.  Inside a recording it only invalidates. */
+int bf_hip_bf16_weight_cache_refresh(const float* const* changed, size_t count, bf_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Fused causal attention                                  (reference: fused_attention.hpp:55,73)

@@ -102,15 +102,16 @@ public:
     // Runs the pipeline, keeping what backward() needs.  inputRangeTrusted: the caller has already checked
     // the token ids of a leading embedding layer on the host (train_runner.cu:210-212), so no device-side
     // range check (and no host synchronisation) is done.
-    DeviceTensor forward(const DeviceTensor& input, bool inputRangeTrusted = false) {
-        return forward(input.clone(), inputRangeTrusted, false);
+    DeviceTensor forward(const DeviceTensor& input, bool inputRangeTrusted = false, bool weightImagesCurrent = false) {
+        return forward(input.clone(), inputRangeTrusted, weightImagesCurrent);
     }
 
     // The same pass over an input the model may keep instead of copying it: `input` becomes the first layer's cached input
     // (a DeviceTensor::borrow view must stay valid and unchanged until backward() has run).  weightImagesCurrent is the
     // caller's promise that no parameter value has changed since this model's previous forward pass (no optimizer step,
-    // no upload, no checkpoint load): the cached bf16 weight images are then kept instead of being dropped and converted
-    // again.  Without the promise every call drops them, as the reference does per forward pass (ops_tensorcore.cu:448).
+    // no upload, no checkpoint load), or that whoever changed them has brought the images up to date
+    // (refreshWeightImages after an optimizer step): the cached bf16 weight images are then kept instead of being
+    // dropped and converted again.  Without the promise every call drops them, as the reference does per forward pass (ops_tensorcore.cu:448).
     DeviceTensor forward(DeviceTensor&& input, bool inputRangeTrusted = false, bool weightImagesCurrent = false) {
         if (!weightImagesCurrent) invalidateBf16WeightCache();   // the optimizer may have changed the weights since the last call
         DeviceTensor current = std::move(input);

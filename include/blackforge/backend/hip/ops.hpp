@@ -143,6 +143,11 @@ inline DeviceTensor matmulBf16CachedWeight(const DeviceTensor& a, const DeviceTe
 }
 
 inline void invalidateBf16WeightCache() { check(bf_hip_invalidate_bf16_weight_cache()); }
+// The same for a caller that knows which weights it has just changed in place (an optimizer step): their cached images
+// are made again at once, in one launch, instead of one by one inside the next forward pass (not in the reference).
+inline void refreshBf16WeightImages(const std::vector<const float*>& changed) {
+    check(bf_hip_bf16_weight_cache_refresh(changed.data(), changed.size(), nullptr));
+}
 
 inline DeviceTensor activation(const DeviceTensor& input, Activation act) {
     DeviceTensor out(input.shape());

@@ -26,6 +26,14 @@ public:
     virtual void publishStep(bf_stream_t stream) = 0;
 };
 
+// After an optimizer step over `updated`: the cached bf16 images of those weights are made again, all in one launch
+// (refreshBf16WeightImages), so that the next Model::forward may be told that the images are current.
+inline void refreshWeightImages(const std::vector<Parameter*>& updated) {
+    std::vector<const float*> changed;
+    for (const Parameter* param : updated) changed.push_back(param->value.data());
+    refreshBf16WeightImages(changed);
+}
+
 class SGD : public Optimizer {
 public:
     explicit SGD(float learningRate) : learningRate_(learningRate) {}

@@ -103,12 +103,14 @@ TrainRunResult runTraining(Model& model, DatasetT& dataset, const TrainOptions& 
         }
         DeviceTensor lossAccumulator = DeviceTensor::zeros({1});
         std::size_t lossDivisor = 0;
+        // only the optimizer changes weights inside the loop; after its step it brings their bf16 images up to date
+        bool weightImagesCurrent = false;
         for (std::size_t b = 0; b < batchesPerEpoch; ++b) {
             auto batch = dataset.batch(b * options.batchSize, options.batchSize);
             if (vocab.has_value()) detail::validateHostIndexRange(batch.input, *vocab, "embeddingLookup");
             DeviceTensor input = DeviceTensor::fromHost(batch.input);
             model.zeroGrad(/*deferred=*/true);
-            DeviceTensor output = model.forward(input, vocab.has_value());
+            DeviceTensor output = model.forward(input, vocab.has_value(), weightImagesCurrent);
             if (sparse) detail::validateHostIndexRange(batch.target, output.shape().back(), "softmaxCrossEntropySparse");
             if (maskedLoss) detail::validateHostMaskedIndexRange(batch.target, output.shape().back(), "softmaxCrossEntropyMasked");
             DeviceTensor target = DeviceTensor::fromHost(batch.target);
@@ -117,7 +119,12 @@ TrainRunResult runTraining(Model& model, DatasetT& dataset, const TrainOptions& 
             lossDivisor += maskedLoss ? 1 : (sparse || dense) ? output.elementCount() / output.shape().back() : output.elementCount();
             lossAndBackward(model, sparse ? "cross_entropy_sparse" : maskedLoss ? "cross_entropy_masked" : dense ? "cross_entropy" : "mse", output,
                             target, lossAccumulator, vocab.has_value());
-            optimizer->step(model.parameters());
+            const std::vector<Parameter*> parameters = model.parameters();
+            optimizer->step(parameters);
+            if (model.usesBf16()) {
+                refreshWeightImages(parameters);
+                weightImagesCurrent = true;
+            }
         }
         const float lossSum = lossAccumulator.toHost().at(0);
         const double avgLoss = static_cast<double>(lossSum) / static_cast<double>(lossDivisor);

@@ -275,3 +275,59 @@ def test_weight_image_cache_fills_pairs_and_lets_go_of_idle_weights(hip, rng):
     call("bf_hip_invalidate_bf16_weight_cache")
     call("bf_hip_invalidate_bf16_weight_cache")
     assert in_use(hip) == base, "only this test's own tensors are still checked out"
+
+
+def test_weight_images_refreshed_in_one_launch_after_an_update(hip, rng):
+    """bf_hip_bf16_weight_cache_refresh after weights changed in place: the images of the listed weights (single weights
+    of aligned and odd shapes, and a group of three that share an input) are made again at the call, bit for bit what a
+    fresh conversion gives; a weight left out of the list is only invalidated."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    m = 200
+    shapes = [(136, 264), (77, 50), (64, 512), (130, 8)]
+    a = {k: D.fromHost(r(rng, m, k)) for k in {s[0] for s in shapes} | {128}}
+    singles = [D.fromHost(r(rng, k, n, scale=0.1)) for k, n in shapes]
+    group = [D.fromHost(r(rng, 128, 96, scale=0.1)) for _ in range(3)]
+    left_out = D.fromHost(r(rng, 136, 264, scale=0.1))
+    arr = lambda ts: (ctypes.c_void_p * len(ts))(*[t.ptr for t in ts])
+
+    def run(cached):
+        outs = []
+        for (k, n), w in zip(shapes, singles):
+            out, dA = D((m, n)), D((m, k))
+            call("bf_hip_linear_bf16", a[k].ptr, w.ptr, None, None, out.ptr, m, k, n, cached, None)
+            call("bf_hip_matmul_bf16_backward", a[k].ptr, w.ptr, out.ptr, dA.ptr, None, m, k, n, cached, None)
+            outs += [out.toHost(), dA.toHost()]
+        cs = [D((m, 96)) for _ in range(3)]
+        call("bf_hip_matmul_bf16_shared_input", a[128].ptr, arr(group), arr(cs), 3, m, 128, 96, cached, None)
+        dA, dBs = D((m, 128)), [D((128, 96)) for _ in range(3)]
+        call("bf_hip_matmul_bf16_shared_input_backward", a[128].ptr, arr(group), arr(cs), dA.ptr, arr(dBs), 3, m, 128, 96, cached, None)
+        outs += [c.toHost() for c in cs] + [dA.toHost()]
+        out = D((m, 264))
+        call("bf_hip_linear_bf16", a[136].ptr, left_out.ptr, None, None, out.ptr, m, 136, 264, cached, None)
+        return outs + [out.toHost()]
+
+    def rewrite(tensors):
+        for t in tensors:
+            fresh = r(rng, *t.shape, scale=0.1)
+            call("bf_hip_memcpy_h2d", t.ptr, fresh.ctypes.data_as(ctypes.c_void_p), fresh.nbytes)
+
+    call("bf_hip_invalidate_bf16_weight_cache")
+    for got, exp in zip(run(1), run(0)):
+        assert_bits_equal(got, exp, "cached images before the update")
+    everything = singles + group + [left_out]
+    rewrite(everything)   # "an optimizer step"
+    listed = singles + group + [a[128]]   # a tensor that has no image may be in the list; left_out is not
+    call("bf_hip_bf16_weight_cache_refresh", arr(listed), len(listed), None)
+    expected = run(0)
+    # the images were made AT the call: weights rewritten behind the cache's back afterwards do not show in the cached
+    # route until the next invalidation (left_out, only invalidated, converts at its next use and does show them)
+    rewrite(singles + group)
+    got = run(1)
+    for i, (g, e) in enumerate(zip(got[:-1], expected[:-1])):
+        assert_bits_equal(g, e, f"result {i} from the images made by the refresh")
+    assert_bits_equal(got[-1], expected[-1], "a weight that was not listed is converted again at its next use")
+    call("bf_hip_invalidate_bf16_weight_cache")
+    for g, e in zip(run(1), run(0)):
+        assert_bits_equal(g, e, "after the next invalidation the cache follows the weights again")
+    call("bf_hip_bf16_weight_cache_refresh", None, 0, None)   # an empty list only invalidates
+    call("bf_hip_invalidate_bf16_weight_cache")
