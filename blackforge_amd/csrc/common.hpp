@@ -195,24 +195,30 @@ template <bool NT> __device__ __forceinline__ void stu2(void* p, uint2v v) {
     else *reinterpret_cast<uint2v*>(p) = v;
 }
 
-// Accurate activations: the formulas of the reference CPU backend, evaluated with the accurate
-// libm-style device functions (no fast-math approximations), so results stay within 1e-6 relative.
-__device__ __forceinline__ float siluF(float x) { return x / (1.0f + expf(-x)); }
+// Activations: the functions of the reference CPU backend (ops.cpp: silu x / (1 + e^-x), gelu 0.5 x (1 + tanh u) with
+// u = 0.79788456 (x + 0.044715 x^3)), written through the logistic function s(y) = 1 / (1 + e^-y), which both reduce to
+// without a subtraction of nearly equal numbers: silu = x s(x); 0.5 (1 + tanh u) = s(2u), so gelu = x s(2u) and
+// 1 - tanh^2 u = 4 s (1 - s).  s is one hardware exponential and one hardware reciprocal (each within one unit in the
+// last place), so a value costs about ten instructions instead of the forty of tanhf and an IEEE division, and is
+// within 1e-6 of the exact function relative to max(|x|, 1): these kernels move 8 to 12 bytes per element and were bound
+// by their arithmetic as much as by memory.
+__device__ __forceinline__ float logisticF(float y) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504f * y)); }
+__device__ __forceinline__ float siluF(float x) { return x * logisticF(x); }
 __device__ __forceinline__ float reluF(float x) { return x > 0.0f ? x : 0.0f; }
 __device__ __forceinline__ float geluF(float x) {
     float inner = 0.7978845608f * (x + 0.044715f * x * x * x);
-    return 0.5f * x * (1.0f + tanhf(inner));
+    return x * logisticF(2.0f * inner);
 }
 __device__ __forceinline__ float siluD(float x) {
-    float s = 1.0f / (1.0f + expf(-x));
+    float s = logisticF(x);
     return s * (1.0f + x * (1.0f - s));
 }
 __device__ __forceinline__ float reluD(float x) { return x > 0.0f ? 1.0f : 0.0f; }
 __device__ __forceinline__ float geluD(float x) {
     float inner = 0.7978845608f * (x + 0.044715f * x * x * x);
-    float t = tanhf(inner);
+    float s = logisticF(2.0f * inner);
     float dInner = 0.7978845608f * (1.0f + 3.0f * 0.044715f * x * x);
-    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * dInner;
+    return s + 2.0f * x * (s * (1.0f - s)) * dInner;
 }
 template <int ACT> __device__ __forceinline__ float actF(float x) {
     if constexpr (ACT == BF_ACT_SILU) return siluF(x);

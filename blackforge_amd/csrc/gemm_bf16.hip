@@ -213,11 +213,22 @@ __device__ __forceinline__ bool tileIndexXcd(int id, int tilesM, int tilesN, int
 // width, so a tile belongs to one output); a single output has splitN == N.  `bias` ([N]) and `residual`
 // ([M, N], single output only) are added to the accumulator in that order before the store, the order in
 // which the separate add kernels would have done it.
+//
+// A feed-forward block's activation fused into the store (`fuse`, single output, everything 16-byte aligned, N a
+// multiple of 8; only the one-tile-per-workgroup wide-wave and ping-pong kernels take it):
+//   fuse 1 (forward):  c[0] = acc + bias as usual, and image[row, col] = bf16(act(c[0][row, col])) beside it;
+//   fuse 2 (backward): image[row, col] = bf16(acc * act'(actZ[row, col])) and nothing else: the fp32 product is never
+//                      stored; colPartial[row / 32, col] = the sum of those products, before rounding, over the rows of
+//                      a 32-row block (the bias gradient is the sum of these partial rows, in order).
 struct Epilogue {
     float* c[3];
     int splitN;
     const float* bias;
     const float* residual;
+    int fuse, act;
+    unsigned short* image;   // [M, N]
+    const float* actZ;       // [M, N]
+    float* colPartial;       // [ceil(M / 32), N]
 };
 
 // An accumulator tile of the 32x32 MFMA gives lane (li, half) column li of rows 8g + 4 half + 0..3 (g = 0..3).  Stored
@@ -318,6 +329,89 @@ __device__ __forceinline__ void storeAccumulators(float16v (&acc)[TM][TN], const
                 }
             }
         }
+}
+
+__device__ __forceinline__ float4v actF4(int act, float4v v) {
+    if (act == BF_ACT_SILU) return float4v{siluF(v.x), siluF(v.y), siluF(v.z), siluF(v.w)};
+    if (act == BF_ACT_GELU) return float4v{geluF(v.x), geluF(v.y), geluF(v.z), geluF(v.w)};
+    return float4v{reluF(v.x), reluF(v.y), reluF(v.z), reluF(v.w)};
+}
+__device__ __forceinline__ float4v actD4(int act, float4v v) {
+    if (act == BF_ACT_SILU) return float4v{siluD(v.x), siluD(v.y), siluD(v.z), siluD(v.w)};
+    if (act == BF_ACT_GELU) return float4v{geluD(v.x), geluD(v.y), geluD(v.z), geluD(v.w)};
+    return float4v{reluD(v.x), reluD(v.y), reluD(v.z), reluD(v.w)};
+}
+__device__ __forceinline__ uint2v packBf16x4(float4v v) {
+    return uint2v{unsigned(toBf16Bits(v.x)) | unsigned(toBf16Bits(v.y)) << 16, unsigned(toBf16Bits(v.z)) | unsigned(toBf16Bits(v.w)) << 16};
+}
+
+// The store with a fused activation (Epilogue::fuse = FUSE): the 16-byte form of storeAccumulators, a lane holding four
+// consecutive columns of one row.  The values written are bit for bit those of the separate passes (the fp32 sum or
+// product is the one they would have read back); the column sums of fuse 2 add the rows of a 32-row block in the order
+// rows 8g (in the lane), then the four lanes of a quad, then the two halves of the wavefront.
+template <int TM, int TN, int FUSE>
+__device__ __forceinline__ void storeAccumulatorsFused(float16v (&acc)[TM][TN], const Epilogue& e, int M, int N, int row0, int col0,
+                                                       int li, int half) {
+    const int t = li & 3, colq = 4 * (li >> 2);
+    // fuse 2 reads z where it writes the image: the four 16-byte loads of a 32 x 32 block are issued one block ahead of
+    // their use (the image stores in between may alias them for all the compiler knows, so it would not move them itself)
+    float4v zAhead[2][4];
+    auto fetchZ = [&](int blk, float4v (&z)[4]) {
+        const int i = blk / TN, j = blk % TN;
+        const int colIn = min(col0 + j * 32 + colq, N - 4);   // columns past the edge read the last ones: no branch around a load
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int row = min(row0 + i * 32 + 8 * g + 4 * half + t, M - 1);
+            z[g] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(e.actZ + size_t(row) * N + colIn));
+        }
+    };
+    if constexpr (FUSE == 2) fetchZ(0, zAhead[0]);
+#pragma unroll
+    for (int blk = 0; blk < TM * TN; ++blk) {
+        const int i = blk / TN, j = blk % TN;
+        if constexpr (FUSE == 2) {
+            if (blk + 1 < TM * TN) fetchZ(blk + 1, zAhead[(blk + 1) & 1]);
+        }
+        const int col = col0 + j * 32 + colq;
+        float4v b = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (FUSE == 1 && e.bias) b = loadf4(e.bias + min(col, N - 4));
+        float4v sums = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float v0 = acc[i][j][4 * g], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
+            quadTranspose(v0, v1, v2, v3, t);
+            const int row = row0 + i * 32 + 8 * g + 4 * half + t;
+            const bool inside = row < M && col < N;
+            float4v v = {v0, v1, v2, v3};
+            if constexpr (FUSE == 1) {
+                if (e.bias) v = v + b;
+                if (inside) {
+                    storef4(e.c[0] + size_t(row) * N + col, v);
+                    *reinterpret_cast<uint2v*>(e.image + size_t(row) * N + col) = packBf16x4(actF4(e.act, v));
+                }
+            } else {
+                v = v * actD4(e.act, zAhead[blk & 1][g]);
+                if (inside) {
+                    *reinterpret_cast<uint2v*>(e.image + size_t(row) * N + col) = packBf16x4(v);
+                    sums = sums + v;
+                }
+            }
+        }
+        if constexpr (FUSE == 2) {
+            if (e.colPartial) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float x = sums[c];
+                    x += quadXor1(x);
+                    x += quadXor2(x);
+                    x += __shfl_xor(x, 32, 64);
+                    sums[c] = x;
+                }
+                const int blockRow = row0 + i * 32;
+                if (t == 0 && half == 0 && blockRow < M && col < N) storef4(e.colPartial + size_t(blockRow >> 5) * N + col, sums);
+            }
+        }
+    }
 }
 
 // Kernel for small tile counts: a workgroup of WAVES_M x WAVES_N wavefronts owns a BM x BN tile, K advances
@@ -428,7 +522,7 @@ __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64) gemmBf16NtKernel(const
 // second round): half the rows per workgroup, the same eight wavefronts, each with a 64 x 64 share instead of 128 x 64.
 // The memory phase then moves 8 fragments for 8 MFMAs instead of 12 for 16, so a tile costs more than half of a full
 // one; it pays when it fills the chip.
-template <int XCD_ORDER, int BM>
+template <int XCD_ORDER, int BM, int FUSE = 0>
 __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned short* __restrict__ A,
                                                                  const unsigned short* __restrict__ Bt, Epilogue epi,
                                                                  int M, int N, int K, int lda, int ldb, int gmLog, int gnLog,
@@ -532,7 +626,8 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
         }
     }
     if (group == 0) __builtin_amdgcn_s_barrier();    // pairs with group 1's last barrier
-    storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
+    if constexpr (FUSE != 0) storeAccumulatorsFused<TM, TN, FUSE>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
+    else storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
 // 128-row tiles on twelve or sixteen wavefronts (three or four per SIMD, each with a 32 x 64 share: tiles 192 or 256
@@ -545,7 +640,7 @@ __global__ void __launch_bounds__(512, 2) gemmBf16PingPongKernel(const unsigned 
 // fewer operand bytes per MFMA.  The 192-wide form is for widths that 256 does not divide into whole rounds of tiles:
 // 768 columns are 3 tiles of 256 (192 tiles for 8192 rows, three quarters of the compute units) or 4 of 192 (256 tiles).
 // The 128 + BN operand rows of a K step are staged as one run of rows, 32 * WAVES_N per pass, A first.
-template <int XCD_ORDER, int WAVES_N>
+template <int XCD_ORDER, int WAVES_N, int FUSE = 0>
 __global__ void __launch_bounds__(256 * WAVES_N, WAVES_N) gemmBf16WideWaveKernel(const unsigned short* __restrict__ A,
                                                                                  const unsigned short* __restrict__ Bt, Epilogue epi,
                                                                                  int M, int N, int K, int lda, int ldb, int gmLog,
@@ -620,7 +715,8 @@ __global__ void __launch_bounds__(256 * WAVES_N, WAVES_N) gemmBf16WideWaveKernel
         }
         __syncthreads();
     }
-    storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
+    if constexpr (FUSE != 0) storeAccumulatorsFused<TM, TN, FUSE>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
+    else storeAccumulators<TM, TN>(acc, epi, M, N, m0 + wm0, n0 + wn0, li, half);
 }
 
 // The next tile this workgroup owns at or after `id`, walking in steps of `stride`; -1 past the end.  With the XCD order
@@ -1256,7 +1352,8 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
     // blocks are dealt to XCDs eight at a time: only worth it when that deal is (nearly) even
     const bool xcdOrder = blocks * 32 <= (tilesM * tilesN) * 5 / 4 && (blocks % 8 == 0 || blocks >= 64);
     const size_t cus = size_t(computeUnits());
-    if (persistent && slices == 1 && tilesM * tilesN > cus) {
+    if (epi.fuse != 0 && slices != 1) return failInvalid("gemm_bf16", "a fused activation does not go with K slices");
+    if (persistent && epi.fuse == 0 && slices == 1 && tilesM * tilesN > cus) {
         // one workgroup per compute unit walks ids blockIdx.x + r * cus (see launchWideWave)
         const bool xcd = xcdOrder && cus % 8 == 0;
         const size_t idEnd = xcd ? (blocks + 7) / 8 * 8 * 32 : tilesM * tilesN;
@@ -1272,7 +1369,7 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
     if (xcdOrder) {
         size_t grid = (blocks + 7) / 8 * 8 * 32;
         if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
-        auto kernel = gemmBf16PingPongKernel<1, BM>;
+        auto kernel = epi.fuse == 1 ? gemmBf16PingPongKernel<1, BM, 1> : epi.fuse == 2 ? gemmBf16PingPongKernel<1, BM, 2> : gemmBf16PingPongKernel<1, BM>;
         int st = allowSharedMemory(kernel, smem);
         if (st != BF_OK) return st;
         kernel<<<dim3(unsigned(grid), unsigned(slices)), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), gmLog, gnLog,
@@ -1280,7 +1377,7 @@ int launchPingPong(const unsigned short* A, const unsigned short* Bt, const Epil
     } else {
         size_t grid = tilesM * tilesN;
         if (grid >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
-        auto kernel = gemmBf16PingPongKernel<0, BM>;
+        auto kernel = epi.fuse == 1 ? gemmBf16PingPongKernel<0, BM, 1> : epi.fuse == 2 ? gemmBf16PingPongKernel<0, BM, 2> : gemmBf16PingPongKernel<0, BM>;
         int st = allowSharedMemory(kernel, smem);
         if (st != BF_OK) return st;
         kernel<<<dim3(unsigned(grid), unsigned(slices)), 512, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), 0, 0,
@@ -1315,7 +1412,7 @@ int launchWideWave(const unsigned short* A, const unsigned short* Bt, const Epil
     // values fetched ahead: such products keep the one-tile-per-workgroup form.
     const bool adds = epi.bias || epi.residual;
     constexpr bool kAddsFit = WAVES_N < 4;
-    if (persistent && wideStores && tilesM * tilesN > cus && (!adds || kAddsFit)) {
+    if (persistent && epi.fuse == 0 && wideStores && tilesM * tilesN > cus && (!adds || kAddsFit)) {
         // one workgroup per compute unit walks ids blockIdx.x + r * cus; with a CU count that is a multiple of 8 a workgroup
         // stays on its XCD and round r of the XCD order is one block of 32 tiles per XCD, as in the one-tile-per-workgroup launch
         const bool xcd = xcdOrder && cus % 8 == 0;
@@ -1328,7 +1425,9 @@ int launchWideWave(const unsigned short* A, const unsigned short* Bt, const Epil
         BF_LAUNCH_CHECK();
         return BF_OK;
     }
-    auto kernel = xcdOrder ? gemmBf16WideWaveKernel<1, WAVES_N> : gemmBf16WideWaveKernel<0, WAVES_N>;
+    auto kernel = epi.fuse == 1 ? (xcdOrder ? gemmBf16WideWaveKernel<1, WAVES_N, 1> : gemmBf16WideWaveKernel<0, WAVES_N, 1>)
+                : epi.fuse == 2 ? (xcdOrder ? gemmBf16WideWaveKernel<1, WAVES_N, 2> : gemmBf16WideWaveKernel<0, WAVES_N, 2>)
+                                : (xcdOrder ? gemmBf16WideWaveKernel<1, WAVES_N> : gemmBf16WideWaveKernel<0, WAVES_N>);
     int st = allowSharedMemory(kernel, smem);
     if (st != BF_OK) return st;
     kernel<<<dim3(unsigned(grid)), 256 * WAVES_N, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), xcdOrder ? gmLog : 0,
@@ -1437,6 +1536,16 @@ int launchGemmTn(const unsigned short* A, const unsigned short* B, const Epilogu
     return BF_OK;
 }
 
+// Whether launchGemmNt takes a product of this shape with Epilogue::fuse set: a kernel chosen by the caller (tests and
+// tuning) never does, so that the separate passes stay reachable, and neither do products too small for the
+// one-tile-per-workgroup kernels.
+bool fusedActivationFits(size_t M, size_t N) {
+    if (g_ntRoute != BF_GEMM_ROUTE_AUTO || N % 8 != 0) return false;
+    const size_t cus = size_t(computeUnits());
+    const size_t halfTiles = ((M + 127) / 128) * ((N + 255) / 256);   // the 256-row form needs no fewer
+    return halfTiles >= cus * 3 / 4 || (N % 192 == 0 && ((M + 127) / 128) * (N / 192) >= cus * 3 / 4);
+}
+
 // epi.splitN must be N (one output) or a multiple of 256 (several outputs: a tile must lie in one of them).
 int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
                  size_t lda, size_t ldb, hipStream_t s) {
@@ -1479,6 +1588,7 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
     // (the ping-pong kernel keeps one tile per workgroup: its tile-walking form measured no faster, see below)
     if (bigTime <= halfTime && bigTime < 1e30) return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
     if (halfTime < 1e30) return launchPingPong<128>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
+    if (epi.fuse != 0) return failInvalid("gemm_bf16", "a fused activation needs a product of at least three quarters of a round of tiles");
     // Few tiles but a long contraction (the weight-gradient products, K = all tokens): the same kernel with K cut into
     // slices, one workgroup per (tile, slice), partial products summed in slice order by a second kernel.  More slices
     // fill more CUs but write and re-read more partial sums; the estimate below (K steps at the measured ~1.4 us per
@@ -2186,11 +2296,18 @@ int bf_hip_feedforward_bf16(const float* x, const float* w1, const float* b1, co
     size_t wBytes = 0;
     st = weightImage(w1, d, hidden, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
     if (st != BF_OK) return st;
-    st = launchGemmNt(xImg, wImg, Epilogue{{z, nullptr, nullptr}, int(hidden), b1, nullptr}, m, hidden, d, d, d, s);
+    // the activation's image is written by the product's own store when the product is large enough for the kernels
+    // that can do it (the same bits as the separate pass over z)
+    const bool fused = fusedActivationFits(m, hidden) && ((reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(b1)) & 15u) == 0;
+    Epilogue first{{z, nullptr, nullptr}, int(hidden), b1, nullptr};
+    if (fused) { first.fuse = 1; first.act = act; first.image = hImage; }
+    st = launchGemmNt(xImg, wImg, first, m, hidden, d, d, d, s);
     if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
     if (st != BF_OK) return st;
-    st = actToBf16Image(z, hImage, m * hidden, act, s);
-    if (st != BF_OK) return st;
+    if (!fused) {
+        st = actToBf16Image(z, hImage, m * hidden, act, s);
+        if (st != BF_OK) return st;
+    }
     st = weightImage(w2, hidden, d, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
     if (st != BF_OK) return st;
     st = launchGemmNt(hImage, wImg, Epilogue{{out, nullptr, nullptr}, int(d), b2, residual}, m, d, hidden, hidden, hidden, s);
@@ -2253,17 +2370,33 @@ int bf_hip_feedforward_bf16_backward_img(const float* x, const uint16_t* xImage,
     }
     if (!dX && !dW1 && !dB1) return BF_OK;
     // dH = g w2^T; one pass over it writes bf16(dz), dz = act'(z) . dH, and dz's column sums: dz is never stored in fp32
-    Scratch dH(m * hidden * sizeof(float)), dzImg(m * hidden * sizeof(unsigned short));
+    // When the product is large enough for the kernels that can do it, its store multiplies by act'(z) and writes the image
+    // itself (dH never exists in memory; the same bits as the separate pass), with dz's column sums per 32-row block, which
+    // a bias-gradient pass over those few rows finishes.
+    const bool fused = fusedActivationFits(m, hidden) && ((reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(dB1)) & 15u) == 0;
+    const size_t rowBlocks = (m + 31) / 32;
+    Scratch dH(fused ? 0 : m * hidden * sizeof(float)), dzImg(m * hidden * sizeof(unsigned short));
+    Scratch partial(fused && dB1 ? rowBlocks * hidden * sizeof(float) : 0);
     if (dH.status != BF_OK) return dH.status;
     if (dzImg.status != BF_OK) return dzImg.status;
+    if (partial.status != BF_OK) return partial.status;
     unsigned short* wImg = nullptr;
     size_t wBytes = 0;
     st = weightImage(w2, hidden, d, /*transposed=*/false, cacheWeight != 0, s, &wImg, &wBytes);
     if (st != BF_OK) return st;
-    st = launchGemmNt(gImage, wImg, dH.as<float>(), m, hidden, d, d, d, s);
+    Epilogue toDz{{dH.as<float>(), nullptr, nullptr}, int(hidden), nullptr, nullptr};
+    if (fused) {
+        toDz.fuse = 2;
+        toDz.act = act;
+        toDz.image = dzImg.as<unsigned short>();
+        toDz.actZ = z;
+        toDz.colPartial = dB1 ? partial.as<float>() : nullptr;
+    }
+    st = launchGemmNt(gImage, wImg, toDz, m, hidden, d, d, d, s);
     if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
     if (st != BF_OK) return st;
-    st = actBackwardToBf16Image(z, dH.as<float>(), dzImg.as<unsigned short>(), dB1, m, hidden, act, s);
+    if (!fused) st = actBackwardToBf16Image(z, dH.as<float>(), dzImg.as<unsigned short>(), dB1, m, hidden, act, s);
+    else if (dB1) st = bf_hip_bias_grad(partial.as<float>(), dB1, rowBlocks, hidden, stream);
     if (st != BF_OK) return st;
     if (dW1) {   // dW1[d, hidden] = x^T dz
         Scratch xScratch(xImage ? 0 : m * d * sizeof(unsigned short));

@@ -331,3 +331,61 @@ def test_weight_images_refreshed_in_one_launch_after_an_update(hip, rng):
         assert_bits_equal(g, e, "after the next invalidation the cache follows the weights again")
     call("bf_hip_bf16_weight_cache_refresh", None, 0, None)   # an empty list only invalidates
     call("bf_hip_invalidate_bf16_weight_cache")
+
+
+@pytest.mark.parametrize("m,d,hidden,act", [(2048, 256, 3072, 1), (2000, 264, 3080, 0), (4096, 1024, 4096, 0), (3000, 128, 2304, 2),
+                                            (8192, 768, 3072, 1)])
+def test_feed_forward_activation_fused_into_the_products(hip, rng, m, d, hidden, act):
+    """Products large enough for the one-tile-per-workgroup kernels write the activation's image (forward) and
+    bf16(dH . act'(z)) with its column sums (backward) from their own store.  A kernel named by the caller keeps the
+    separate passes: z, the image of act(z) and the weight gradients (dW1 is made from the image of dz) must have the
+    same bits either way; the bias gradient dB1 adds its rows in another order."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    x, w1, b1 = r(rng, m, d), r(rng, d, hidden, scale=0.1), r(rng, hidden, scale=0.5)
+    w2, b2, res, g = r(rng, hidden, d, scale=0.1), r(rng, d), r(rng, m, d), r(rng, m, d)
+    dx, dw1, db1, dw2, db2, dres, dg = map(D.fromHost, (x, w1, b1, w2, b2, res, g))
+
+    def run(route):
+        call("bf_hip_gemm_bf16_set_route", route)
+        try:
+            z, h, xi, out = D((m, hidden)), D((m, hidden // 2)), D((m, d // 2)), D((m, d))
+            call("bf_hip_feedforward_bf16", dx.ptr, dw1.ptr, db1.ptr, dw2.ptr, db2.ptr, dres.ptr, act, z.ptr, h.ptr, xi.ptr, out.ptr, m, d,
+                 hidden, 0, None)
+            outs = [D((m, d)), D(w1.shape), D((hidden,)), D(w2.shape), D((d,))]
+            call("bf_hip_feedforward_bf16_backward", dx.ptr, xi.ptr, dw1.ptr, dw2.ptr, z.ptr, h.ptr, dg.ptr, act, *[t.ptr for t in outs],
+                 m, d, hidden, 0, None)
+            return [t.toHost() for t in (z, h, out, *outs)]
+        finally:
+            call("bf_hip_gemm_bf16_set_route", 0)
+
+    names = ("z", "image of act(z)", "out", "dX", "dW1", "dB1", "dW2", "dB2")
+    fused, separate = run(0), run(1)
+    for name, a, b in zip(names, fused, separate):
+        if name == "dB1":
+            scale = float(np.abs(b).max())
+            assert float(np.abs(a - b).max()) <= 2e-6 * scale * np.sqrt(m), "dB1 from the products' partial column sums"
+        elif name not in ("z", "image of act(z)") and m * d < 8192 * 768:
+            # narrow products (d columns) of a long contraction: the named kernel adds all of K in one workgroup, the
+            # library's own choice may cut K into slices, so the order of the fp32 additions differs; the largest case
+            # has no such products and must agree bit for bit (dW1 is made from the image of dz)
+            assert float(np.abs(a - b).max()) <= 1e-5 * float(np.abs(b).max()), name
+        else:
+            assert_bits_equal(a, b, name + " with the activation fused into the product's store")
+    # and dB1 against float64 of the same terms (the fp32 products are summed, not their bf16 roundings)
+    def rounded(a):   # round-to-nearest-even bf16 of finite fp32 values
+        bits = np.ascontiguousarray(a, dtype=f32).view(np.uint32).astype(np.uint64)
+        bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+        return bits.astype(np.uint32).view(f32).astype(np.float64)
+
+    zf = fused[0].astype(np.float64)
+    dH = rounded(g) @ rounded(w2).T
+    if act == 0:
+        sg = 1.0 / (1.0 + np.exp(-zf))
+        dact = sg * (1.0 + zf * (1.0 - sg))
+    elif act == 1:
+        t = np.tanh(0.7978845608 * (zf + 0.044715 * zf ** 3))
+        dact = 0.5 * (1.0 + t) + 0.5 * zf * (1.0 - t * t) * 0.7978845608 * (1.0 + 3.0 * 0.044715 * zf * zf)
+    else:
+        dact = (zf > 0).astype(np.float64)
+    expect = (dH * dact).sum(axis=0)
+    assert float(np.abs(fused[5] - expect).max()) <= 1e-4 * float(np.abs(expect).max()), "dB1 against float64"
