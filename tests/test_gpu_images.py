@@ -287,6 +287,7 @@ def test_weight_images_refreshed_in_one_launch_after_an_update(hip, rng):
     a = {k: D.fromHost(r(rng, m, k)) for k in {s[0] for s in shapes} | {128}}
     singles = [D.fromHost(r(rng, k, n, scale=0.1)) for k, n in shapes]
     group = [D.fromHost(r(rng, 128, 96, scale=0.1)) for _ in range(3)]
+    wide_group = [D.fromHost(r(rng, 128, 256, scale=0.1)) for _ in range(3)]   # stacked images: one product for the three
     left_out = D.fromHost(r(rng, 136, 264, scale=0.1))
     arr = lambda ts: (ctypes.c_void_p * len(ts))(*[t.ptr for t in ts])
 
@@ -302,6 +303,11 @@ def test_weight_images_refreshed_in_one_launch_after_an_update(hip, rng):
         dA, dBs = D((m, 128)), [D((128, 96)) for _ in range(3)]
         call("bf_hip_matmul_bf16_shared_input_backward", a[128].ptr, arr(group), arr(cs), dA.ptr, arr(dBs), 3, m, 128, 96, cached, None)
         outs += [c.toHost() for c in cs] + [dA.toHost()]
+        cs = [D((m, 256)) for _ in range(3)]
+        call("bf_hip_matmul_bf16_shared_input", a[128].ptr, arr(wide_group), arr(cs), 3, m, 128, 256, cached, None)
+        dA, dBs = D((m, 128)), [D((128, 256)) for _ in range(3)]
+        call("bf_hip_matmul_bf16_shared_input_backward", a[128].ptr, arr(wide_group), arr(cs), dA.ptr, arr(dBs), 3, m, 128, 256, cached, None)
+        outs += [c.toHost() for c in cs] + [dA.toHost()]
         out = D((m, 264))
         call("bf_hip_linear_bf16", a[136].ptr, left_out.ptr, None, None, out.ptr, m, 136, 264, cached, None)
         return outs + [out.toHost()]
@@ -314,14 +320,14 @@ def test_weight_images_refreshed_in_one_launch_after_an_update(hip, rng):
     call("bf_hip_invalidate_bf16_weight_cache")
     for got, exp in zip(run(1), run(0)):
         assert_bits_equal(got, exp, "cached images before the update")
-    everything = singles + group + [left_out]
+    everything = singles + group + wide_group + [left_out]
     rewrite(everything)   # "an optimizer step"
-    listed = singles + group + [a[128]]   # a tensor that has no image may be in the list; left_out is not
+    listed = singles + group + wide_group + [a[128]]   # a tensor that has no image may be in the list; left_out is not
     call("bf_hip_bf16_weight_cache_refresh", arr(listed), len(listed), None)
     expected = run(0)
     # the images were made AT the call: weights rewritten behind the cache's back afterwards do not show in the cached
     # route until the next invalidation (left_out, only invalidated, converts at its next use and does show them)
-    rewrite(singles + group)
+    rewrite(singles + group + wide_group)
     got = run(1)
     for i, (g, e) in enumerate(zip(got[:-1], expected[:-1])):
         assert_bits_equal(g, e, f"result {i} from the images made by the refresh")
