@@ -84,9 +84,10 @@ struct AddBiasGrad {
     DeviceTensor dBias;
 };
 
-inline DeviceTensor biasGradientOnly(const DeviceTensor& gradOutput) {
+// into / slot: where the caller wants the gradient written (a model's own gradient tensor), see GradientTargets
+inline DeviceTensor biasGradientOnly(const DeviceTensor& gradOutput, const GradientTargets* into = nullptr, int slot = 0) {
     require(gradOutput.rank() >= 2, "biasGradientOnly: needs a gradient of rank >= 2 on the device");
-    DeviceTensor dBias({detail::lastDim(gradOutput)});
+    DeviceTensor dBias = detail::gradientTensor(into, slot, {detail::lastDim(gradOutput)});
     check(bf_hip_bias_grad(gradOutput.data(), dBias.data(), detail::rowsOf(gradOutput), detail::lastDim(gradOutput), nullptr));
     return dBias;
 }
@@ -102,10 +103,11 @@ struct AddBiasSiluGrad {
 };
 
 inline AddBiasSiluGrad addBiasActivationBackward(const DeviceTensor& gemmOutput, const DeviceTensor& bias,
-                                                  const DeviceTensor& dHidden, Activation act) {
+                                                  const DeviceTensor& dHidden, Activation act, const GradientTargets* into = nullptr,
+                                                  int slot = 0) {
     require(gemmOutput.shape() == dHidden.shape() && bias.rank() == 1 && detail::lastDim(gemmOutput) == bias.dim(0),
             "addBiasSiluBackward: incompatible shapes on the device");
-    AddBiasSiluGrad r{DeviceTensor(gemmOutput.shape()), DeviceTensor({bias.dim(0)})};
+    AddBiasSiluGrad r{DeviceTensor(gemmOutput.shape()), detail::gradientTensor(into, slot, {bias.dim(0)})};
     check(bf_hip_add_bias_act_backward(gemmOutput.data(), bias.data(), dHidden.data(), r.dGemmOutput.data(), r.dBias.data(),
                                        detail::rowsOf(gemmOutput), bias.dim(0), static_cast<int>(act), nullptr));
     return r;
@@ -218,9 +220,9 @@ inline FeedForwardGrad feedForwardBackwardCached(const DeviceTensor& input, cons
         DeviceTensor dInput = rmsnormBackwardAdd(input, dNormed, gradOutput, imageForConsumer);
         return FeedForwardGrad{std::move(dInput), std::move(dW1), std::move(dB1), std::move(dW2), std::move(dB2)};
     }
-    DeviceTensor dB2 = biasGradientOnly(gradOutput);
+    DeviceTensor dB2 = biasGradientOnly(gradOutput, into, 3);
     MatmulGrad g2 = detail::projectionBackward(cache.hidden, w2, gradOutput, mode, cache.hidden.shape(), into, 2);
-    AddBiasSiluGrad hiddenGrad = addBiasActivationBackward(cache.gemm1, b1, g2.dA, act);
+    AddBiasSiluGrad hiddenGrad = addBiasActivationBackward(cache.gemm1, b1, g2.dA, act, into, 1);
     MatmulGrad g1 = detail::projectionBackward(cache.normed, w1, hiddenGrad.dGemmOutput, mode, cache.normed.shape(), into, 0);
     DeviceTensor dInput = rmsnormBackwardAdd(input, g1.dA, gradOutput, imageForConsumer && useBf16);
     return FeedForwardGrad{std::move(dInput), std::move(g1.dB), std::move(hiddenGrad.dBias), std::move(g2.dB), std::move(dB2)};

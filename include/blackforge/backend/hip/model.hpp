@@ -419,7 +419,7 @@ private:
         switch (s.kind) {
             case LayerKind::Linear: {
                 DeviceTensor dBias = givenBiasGrad != nullptr ? DeviceTensor::borrow(givenBiasGrad->data(), givenBiasGrad->shape())
-                                                              : biasGradientOnly(grad);
+                                                              : biasGradientOnly(grad, into, 1);
                 if (useBf16_ && !needInputGrad) {   // the weight gradient alone
                     const DeviceTensor& w = layer.params[0].value;
                     DeviceTensor dW = detail::gradientTensor(into, 0, w.shape());
@@ -443,7 +443,8 @@ private:
                 DeviceTensor dTable = trustedIds ? embeddingLookupBackwardPreValidated(x, grad, s.arg0, into)
                                                  : embeddingLookupBackward(x, grad, s.arg0, into);
                 accumulate(layer.params[0].grad, dTable);
-                return DeviceTensor::zeros(x.shape());   // token ids carry no gradient
+                // token ids carry no gradient: zeros, as in the reference, for a caller that will look at them
+                return needInputGrad ? DeviceTensor::zeros(x.shape()) : DeviceTensor();
             }
             case LayerKind::PositionalEmbedding: {
                 PositionalEmbeddingGrad g = addPositionalEmbeddingBackward(grad, s.arg0, into);
