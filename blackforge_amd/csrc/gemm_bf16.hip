@@ -1550,6 +1550,13 @@ bool fusedActivationFits(size_t M, size_t N) {
 int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K,
                  size_t lda, size_t ldb, hipStream_t s) {
     if (M >= (size_t(1) << 31) || N >= (size_t(1) << 31) || K >= (size_t(1) << 31)) return failInvalid("gemm_bf16", "shape too large");
+    if (epi.fuse != 0) {   // what the fused stores assume (storeAccumulatorsFused); callers ask fusedActivationFits() first
+        const uintptr_t bits = reinterpret_cast<uintptr_t>(epi.c[0]) | reinterpret_cast<uintptr_t>(epi.bias) | reinterpret_cast<uintptr_t>(epi.image) |
+                               reinterpret_cast<uintptr_t>(epi.actZ) | reinterpret_cast<uintptr_t>(epi.colPartial);
+        const bool operands = epi.fuse == 1 ? (epi.c[0] && epi.image) : (epi.fuse == 2 && epi.image && epi.actZ && !epi.bias);
+        if (!operands || epi.residual || size_t(epi.splitN) != N || N % 8 != 0 || (bits & 15u) != 0 || g_ntRoute != BF_GEMM_ROUTE_AUTO)
+            return failInvalid("gemm_bf16", "fused activation: one 16-byte aligned output of a width that is a multiple of 8, no residual");
+    }
     const size_t cus = size_t(computeUnits());
     switch (g_ntRoute) {   // a kernel named by the caller (tests and tuning); BF_GEMM_ROUTE_AUTO otherwise
         case BF_GEMM_ROUTE_PINGPONG_256: return launchPingPong<256>(A, Bt, epi, M, N, K, lda, ldb, s, 1, 0, 0, false);
