@@ -15,11 +15,15 @@
 // reads stay inside the tensor except for at most 12 bytes after its last element, inside the same 16-byte group.
 #pragma once
 
+// BF_ROWCACHE_HOST_MODEL: a host program (tests/cpp/rowcache_bounds_test.cpp) compiles RowCache itself with accessors
+// of its own (ldf4, stf4, ...) that check every address the shifted accesses touch; it defines what common.hpp would.
+#if !defined(BF_ROWCACHE_HOST_MODEL)
 #include "common.hpp"
+#endif
 
 namespace bf {
 
-#if defined(__HIPCC__)
+#if defined(__HIPCC__) || defined(BF_ROWCACHE_HOST_MODEL)
 
 // NT: accesses carry the non-temporal hint (rows streamed past the last-level cache, see ldf4 / stf4).
 template <int G, int MAXE, int VEC, bool NT = false>
@@ -165,7 +169,7 @@ __device__ __forceinline__ float groupMax(float v, float* lds) {
     else return blockReduce(v, -INFINITY, OpMaxF{}, lds);
 }
 
-#endif  // __HIPCC__
+#endif  // __HIPCC__ || BF_ROWCACHE_HOST_MODEL
 
 // Host-side choice of group size for a row length: the smallest group whose registers hold the row.
 struct RowPlan {
