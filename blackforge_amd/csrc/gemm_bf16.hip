@@ -349,66 +349,87 @@ __device__ __forceinline__ uint2v packBf16x4(float4v v) {
 // consecutive columns of one row.  The values written are bit for bit those of the separate passes (the fp32 sum or
 // product is the one they would have read back); the column sums of fuse 2 add the rows of a 32-row block in the order
 // rows 8g (in the lane), then the four lanes of a quad, then the two halves of the wavefront.
+// The image goes out in whole 128-byte lines: a wavefront's share is 64 columns wide (two accumulator blocks side by
+// side), and neighbouring lanes (column groups q and q^1) trade one of their two packed groups, so that an even lane
+// holds eight consecutive columns of the left block and an odd lane eight of the right one: one 16-byte store per lane
+// and row instead of two 8-byte ones that each leave half a line to be merged (measured on 8192 x 3072: 16 us for the
+// image stored in halves, as much as the fp32 tensor of twice its size).
 template <int TM, int TN, int FUSE>
 __device__ __forceinline__ void storeAccumulatorsFused(float16v (&acc)[TM][TN], const Epilogue& e, int M, int N, int row0, int col0,
                                                        int li, int half) {
-    const int t = li & 3, colq = 4 * (li >> 2);
-    // fuse 2 reads z where it writes the image: the four 16-byte loads of a 32 x 32 block are issued one block ahead of
-    // their use (the image stores in between may alias them for all the compiler knows, so it would not move them itself)
-    float4v zAhead[2][4];
-    auto fetchZ = [&](int blk, float4v (&z)[4]) {
-        const int i = blk / TN, j = blk % TN;
-        const int colIn = min(col0 + j * 32 + colq, N - 4);   // columns past the edge read the last ones: no branch around a load
+    static_assert(TN == 2, "the image store pairs the two accumulator blocks of a 64-column share");
+    const int t = li & 3, q = li >> 2, colq = 4 * q;
+    const bool odd = (q & 1) != 0;
+    // fuse 2 reads z where it writes the image: the 16-byte loads of a 32-row strip are issued one strip ahead of their
+    // use (the image stores in between may alias them for all the compiler knows, so it would not move them itself)
+    float4v zAhead[TM > 1 ? 2 : 1][2][4];
+    auto fetchZ = [&](int i, float4v (&z)[2][4]) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int row = min(row0 + i * 32 + 8 * g + 4 * half + t, M - 1);
-            z[g] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(e.actZ + size_t(row) * N + colIn));
+        for (int j = 0; j < 2; ++j) {
+            const int colIn = min(col0 + j * 32 + colq, N - 4);   // columns past the edge read the last ones: no branch around a load
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int row = min(row0 + i * 32 + 8 * g + 4 * half + t, M - 1);
+                z[j][g] = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(e.actZ + size_t(row) * N + colIn));
+            }
         }
     };
     if constexpr (FUSE == 2) fetchZ(0, zAhead[0]);
 #pragma unroll
-    for (int blk = 0; blk < TM * TN; ++blk) {
-        const int i = blk / TN, j = blk % TN;
-        if constexpr (FUSE == 2) {
-            if (blk + 1 < TM * TN) fetchZ(blk + 1, zAhead[(blk + 1) & 1]);
+    for (int i = 0; i < TM; ++i) {
+        if constexpr (FUSE == 2 && TM > 1) {
+            if (i + 1 < TM) fetchZ(i + 1, zAhead[(i + 1) & 1]);
         }
-        const int col = col0 + j * 32 + colq;
-        float4v b = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (FUSE == 1 && e.bias) b = loadf4(e.bias + min(col, N - 4));
-        float4v sums = {0.0f, 0.0f, 0.0f, 0.0f};
+        float4v b[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+        if (FUSE == 1 && e.bias) {
+            b[0] = loadf4(e.bias + min(col0 + colq, N - 4));
+            b[1] = loadf4(e.bias + min(col0 + 32 + colq, N - 4));
+        }
+        float4v sums[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            float v0 = acc[i][j][4 * g], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
-            quadTranspose(v0, v1, v2, v3, t);
             const int row = row0 + i * 32 + 8 * g + 4 * half + t;
-            const bool inside = row < M && col < N;
-            float4v v = {v0, v1, v2, v3};
-            if constexpr (FUSE == 1) {
-                if (e.bias) v = v + b;
-                if (inside) {
-                    storef4(e.c[0] + size_t(row) * N + col, v);
-                    *reinterpret_cast<uint2v*>(e.image + size_t(row) * N + col) = packBf16x4(actF4(e.act, v));
-                }
-            } else {
-                v = v * actD4(e.act, zAhead[blk & 1][g]);
-                if (inside) {
-                    *reinterpret_cast<uint2v*>(e.image + size_t(row) * N + col) = packBf16x4(v);
-                    sums = sums + v;
+            uint2v packed[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                float v0 = acc[i][j][4 * g], v1 = acc[i][j][4 * g + 1], v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
+                quadTranspose(v0, v1, v2, v3, t);
+                const int col = col0 + j * 32 + colq;
+                const bool inside = row < M && col < N;
+                float4v v = {v0, v1, v2, v3};
+                if constexpr (FUSE == 1) {
+                    if (e.bias) v = v + b[j];
+                    if (inside) storef4(e.c[0] + size_t(row) * N + col, v);
+                    packed[j] = packBf16x4(actF4(e.act, v));
+                } else {
+                    v = v * actD4(e.act, zAhead[TM > 1 ? (i & 1) : 0][j][g]);
+                    if (inside) sums[j] = sums[j] + v;
+                    packed[j] = packBf16x4(v);
                 }
             }
+            // an even lane sends its right-block group and receives the left-block group of the odd lane beside it
+            const uint2v send = odd ? packed[0] : packed[1];
+            const uint2v recv = {unsigned(__shfl_xor(int(send.x), 4, 64)), unsigned(__shfl_xor(int(send.y), 4, 64))};
+            const uint4v line = odd ? uint4v{recv.x, recv.y, packed[1].x, packed[1].y} : uint4v{packed[0].x, packed[0].y, recv.x, recv.y};
+            const int ocol = odd ? col0 + 32 + colq - 4 : col0 + colq;   // a multiple of 8, like N: the eight columns are inside or outside together
+            if (row < M && ocol < N) *reinterpret_cast<uint4v*>(e.image + size_t(row) * N + ocol) = line;
         }
         if constexpr (FUSE == 2) {
             if (e.colPartial) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    float x = sums[c];
-                    x += quadXor1(x);
-                    x += quadXor2(x);
-                    x += __shfl_xor(x, 32, 64);
-                    sums[c] = x;
-                }
                 const int blockRow = row0 + i * 32;
-                if (t == 0 && half == 0 && blockRow < M && col < N) storef4(e.colPartial + size_t(blockRow >> 5) * N + col, sums);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float x = sums[j][c];
+                        x += quadXor1(x);
+                        x += quadXor2(x);
+                        x += __shfl_xor(x, 32, 64);
+                        sums[j][c] = x;
+                    }
+                    const int col = col0 + j * 32 + colq;
+                    if (t == 0 && half == 0 && blockRow < M && col < N) storef4(e.colPartial + size_t(blockRow >> 5) * N + col, sums[j]);
+                }
             }
         }
     }
