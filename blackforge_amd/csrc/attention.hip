@@ -2238,7 +2238,7 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnForwardPipedKernel
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
-int paddedHeadDim(int hd) { return hd <= 32 ? 32 : hd <= 64 ? 64 : hd <= 128 ? 128 : 256; }
+int paddedHeadDim(int hd) { return hd <= 32 ? 32 : hd <= 64 ? 64 : hd <= 128 ? 128 : hd <= 192 ? 192 : 256; }
 
 template <typename K>
 int launchAttn(K kernel, size_t smemBytes, unsigned grid, const AttnParams& p, hipStream_t s) {
@@ -2323,6 +2323,7 @@ int dispatch(const AttnParams& p, bool vec4, unsigned grid, hipStream_t s) {
         case 32: return dispatchVec<KIND, 32, 64>(p, vec4, grid, s);
         case 64: return dispatchVec<KIND, 64, 64>(p, vec4, grid, s);
         case 128: return dispatchVec<KIND, 128, 32>(p, vec4, grid, s);
+        case 192: return dispatchVec<KIND, 192, 32>(p, vec4, grid, s);
         default: return dispatchVec<KIND, 256, 32>(p, vec4, grid, s);
     }
 }

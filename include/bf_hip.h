@@ -373,10 +373,11 @@ int bf_hip_bf16_weight_cache_refresh(const float* const* changed, size_t count, 
  * q:[batch,newLen,dim]  k,v:[batch,totalLen,dim]  heads contiguous in dim, headDim = dim/heads <= 256.
  * Query row i (absolute position oldLen+i) attends to keys j <= oldLen+i.
  * Tuned head dims are 32, 64 and 128 (forward and backward 110-175 TFLOP/s of fp32 work at 1024-4096 positions).  Head
- * dims above 128 are accepted, like the reference accepts them, and run on the fp32-MFMA kernels padded to 256:
- * measured at batch 4, 8 heads, 2048 positions, headDim 256: forward 70, dK/dV 68, dQ 96 TFLOP/s, forward + backward
- * 71 TFLOP/s = 0.45 of the fp32 MFMA peak (headDim 192, a quarter of it padding: 55 / 55 / 72).  When the dS hand-over
- * buffer is refused (bf_hip_attention_set_workspace_limit) the dK/dV pass of such heads falls to 40 TFLOP/s.
+ * dims above 128 are accepted, like the reference accepts them, and run on the fp32-MFMA kernels padded to 192 or 256:
+ * measured at batch 4, 8 heads, 2048 positions, headDim 192: forward 94, dK/dV 96, dQ 95 TFLOP/s = 0.60 of the fp32
+ * MFMA peak for forward + backward (headDim 160, a sixth of it padding: 81 / 83 / 81); headDim 256: 70 / 68 / 95 =
+ * 0.45.  When the dS hand-over buffer is refused (bf_hip_attention_set_workspace_limit) the dK/dV pass of such heads
+ * falls to about half of that.
  * ------------------------------------------------------------------------------------------- */
 /* fusedAttentionForward: out:[batch,newLen,dim]; m,l:[batch,heads,newLen] = row max of the scaled
  * scores and sum of exp(score - m) (the statistics the backward reuses). */
