@@ -337,6 +337,10 @@ __device__ __forceinline__ void forwardTile(const float* __restrict__ ks, const 
     }
 }
 
+// operands of __builtin_amdgcn_global_load_lds (global memory straight into LDS)
+typedef __attribute__((address_space(1))) const void* GlobalPtr;
+typedef __attribute__((address_space(3))) void* LdsPtr;
+
 // Streaming schedule shared by the three kernels (LDS double buffering, ONE barrier per tile):
 //   iteration t consumes buffer t&1, then writes tile t+1 (already in registers) into buffer (t+1)&1 and
 //   issues the global loads of tile t+2; the barrier at the end of the iteration both publishes tile t+1
@@ -376,17 +380,7 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnForwardKernel(Att
     const int myLimit = p.oldLen + i;                                    // last visible key of this lane's row
     const int numKeyTiles = (blockKeyEnd + BC - 1) / BC;
 
-    TileRegs<HDP, BC> kNext, vNext;
-    fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, 0, p.totalLen, hd, tid);
-    fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, 0, p.totalLen, hd, tid);
-    commitHeadTile<HDP, BC>(ks, kNext, tid);
-    commitHeadTile<HDP, BC>(vs, vNext, tid);
-    if (numKeyTiles > 1) {
-        fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, BC, p.totalLen, hd, tid);
-        fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, BC, p.totalLen, hd, tid);
-    }
-    __syncthreads();
-    for (int t = 0; t < numKeyTiles; ++t) {
+    auto tileBody = [&](int t) __attribute__((always_inline)) {
         const int kt0 = t * BC;
         const float* kcur = ks + (t & 1) * TILE;
         const float* vcur = vs + (t & 1) * TILE;
@@ -396,15 +390,64 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnForwardKernel(Att
             if (masked) forwardTile<HDP, BC, true>(kcur, vcur, qreg, acc, mrow, mref, lrow, kt0, myLimit, p.totalLen, half, li);
             else forwardTile<HDP, BC, false>(kcur, vcur, qreg, acc, mrow, mref, lrow, kt0, myLimit, p.totalLen, half, li);
         }
-        if (t + 1 < numKeyTiles) {
-            commitHeadTile<HDP, BC>(ks + ((t + 1) & 1) * TILE, kNext, tid);
-            commitHeadTile<HDP, BC>(vs + ((t + 1) & 1) * TILE, vNext, tid);
-            if (t + 2 < numKeyTiles) {
-                fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, kt0 + 2 * BC, p.totalLen, hd, tid);
-                fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, kt0 + 2 * BC, p.totalLen, hd, tid);
+    };
+    if constexpr (VEC4 && HDP > 128) {
+        // Head dims above 128: the Q rows and the accumulators leave no registers for two tiles in flight (53 spilled at 256),
+        // so K and V tiles go from global memory straight into LDS (global_load_lds: one row per wavefront instruction,
+        // 16 bytes a lane, lanes past the head dim switched off and their columns zeroed once), one tile ahead of its
+        // use: a tile's products last several microseconds.  Rows past the sequence repeat its last row: finite values
+        // under a mask.
+        const int waveU = __builtin_amdgcn_readfirstlane(wave);
+        const bool columnValid = 4 * lane < hd;
+        const float* kBase = kb + 4 * lane;
+        const float* vBase = vb + 4 * lane;
+        auto issueTile = [&](int kt0, int buf) __attribute__((always_inline)) {
+#pragma unroll
+            for (int r4 = 0; r4 < BC / 4; ++r4) {
+                const int r = waveU + 4 * r4;
+                const size_t row = size_t(min(kt0 + r, p.totalLen - 1)) * dim;
+                if (columnValid) {
+                    __builtin_amdgcn_global_load_lds((GlobalPtr)(kBase + row), (LdsPtr)(ks + buf * TILE + r * LDSW), 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((GlobalPtr)(vBase + row), (LdsPtr)(vs + buf * TILE + r * LDSW), 16, 0, 0);
+                }
             }
+        };
+        if (hd < HDP) {   // the columns past the head dim are never loaded: zero them once (both buffers of both tiles)
+            for (int z = tid; z < 4 * BC * (LDSW / 4); z += 256) storef4(ks + 4 * z, float4v{0.0f, 0.0f, 0.0f, 0.0f});
+            __syncthreads();
+        }
+        issueTile(0, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        for (int t = 0; t < numKeyTiles; ++t) {
+            if (t + 1 < numKeyTiles) issueTile((t + 1) * BC, (t + 1) & 1);   // that buffer was last read before the barrier above
+            tileBody(t);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+    } else {
+        TileRegs<HDP, BC> kNext, vNext;
+        fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, 0, p.totalLen, hd, tid);
+        fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, 0, p.totalLen, hd, tid);
+        commitHeadTile<HDP, BC>(ks, kNext, tid);
+        commitHeadTile<HDP, BC>(vs, vNext, tid);
+        if (numKeyTiles > 1) {
+            fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, BC, p.totalLen, hd, tid);
+            fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, BC, p.totalLen, hd, tid);
         }
         __syncthreads();
+        for (int t = 0; t < numKeyTiles; ++t) {
+            tileBody(t);
+            if (t + 1 < numKeyTiles) {
+                commitHeadTile<HDP, BC>(ks + ((t + 1) & 1) * TILE, kNext, tid);
+                commitHeadTile<HDP, BC>(vs + ((t + 1) & 1) * TILE, vNext, tid);
+                if (t + 2 < numKeyTiles) {
+                    fetchHeadTile<HDP, BC, VEC4>(kNext, kb, dim, t * BC + 2 * BC, p.totalLen, hd, tid);
+                    fetchHeadTile<HDP, BC, VEC4>(vNext, vb, dim, t * BC + 2 * BC, p.totalLen, hd, tid);
+                }
+            }
+            __syncthreads();
+        }
     }
 
     lrow += __shfl_xor(lrow, 32, 64);
@@ -907,18 +950,19 @@ __device__ __forceinline__ float16v headDotFenced(const float* __restrict__ ldsR
     }
     return acc;
 }
-// acc[dt] += w[r] (x) row_r[dt*32 + li] for the sixteen rows dRow(r, half) of a 32-row block at `rows`
-template <int HDP>
-__device__ __forceinline__ void rankUpdatesFenced(const float* __restrict__ rows, const float16v& w, float16v (&acc)[HDP / 32], int half, int li) {
-    constexpr int LDSW = HDP + 4, DT = HDP / 32;
+// acc[dt] += w[r] (x) row_r[(DT0 + dt)*32 + li] for the sixteen rows dRow(r, half) of a 32-row block at `rows`: the
+// DT head-dim blocks from block DT0 on
+template <int HDP, int DT0, int DT>
+__device__ __forceinline__ void rankUpdatesFenced(const float* __restrict__ rows, const float16v& w, float16v (&acc)[DT], int half, int li) {
+    constexpr int LDSW = HDP + 4;
     float cur[DT], nxt[DT];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) cur[dt] = rows[dRow(0, half) * LDSW + li + dt * 32];
+    for (int dt = 0; dt < DT; ++dt) cur[dt] = rows[dRow(0, half) * LDSW + li + (DT0 + dt) * 32];
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         if (r + 1 < 16) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) nxt[dt] = rows[dRow(r + 1, half) * LDSW + li + dt * 32];
+            for (int dt = 0; dt < DT; ++dt) nxt[dt] = rows[dRow(r + 1, half) * LDSW + li + (DT0 + dt) * 32];
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[r], cur[dt], acc[dt], 0, 0, 0);
@@ -928,9 +972,29 @@ __device__ __forceinline__ void rankUpdatesFenced(const float* __restrict__ rows
     }
 }
 
-template <int HDP, int BQ, bool MASKED>
+// The sixteen values a lane parked in (or will park in) its 32 x 32 sub-block of the dS buffer; zero for rows past the sequence.
+__device__ __forceinline__ float16v readParked(const float* __restrict__ src, bool stored) {
+    float16v v;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) v[r] = stored ? __builtin_nontemporal_load(src + (8 * (r >> 2) + (r & 3)) * 32) : 0.0f;
+    return v;
+}
+// The second half of pass P or of pass dS when the accumulators take the head dim in two halves (head dim 256): the
+// parked P (or dS) is read back and meets the other half of the dO (or Q) columns; no product over the head dim.
+template <int HDP, int BQ, int DT0, int DTN>
+__device__ __forceinline__ void dkvTileAgain(const float* __restrict__ rowsTile, float16v (&acc)[DTN], int qt0, int half, int li,
+                                             const float* __restrict__ dsLane, size_t dsStride, int newLen) {
+    constexpr int LDSW = HDP + 4, NSB = BQ / 32;
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb) {
+        const float16v w = readParked(dsLane + sb * dsStride, qt0 + sb * 32 < newLen);
+        rankUpdatesFenced<HDP, DT0, DTN>(rowsTile + sb * 32 * LDSW, w, acc, half, li);
+    }
+}
+
+template <int HDP, int BQ, bool MASKED, int DTN>
 __device__ __forceinline__ void dkvTileP(const float* __restrict__ qs, const float* __restrict__ gs, const float* __restrict__ stats,
-                                         const float (&kreg)[HDP / 2], float16v (&dv)[HDP / 32], int qt0, int key, bool keyValid, int oldLen,
+                                         const float (&kreg)[HDP / 2], float16v (&dv)[DTN], int qt0, int key, bool keyValid, int oldLen,
                                          int half, int li, float* __restrict__ dsLane, size_t dsStride, int newLen) {
     constexpr int LDSW = HDP + 4, NSB = BQ / 32;
 #pragma unroll
@@ -958,22 +1022,20 @@ __device__ __forceinline__ void dkvTileP(const float* __restrict__ qs, const flo
 #pragma unroll
             for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(pr[r], dst + (8 * (r >> 2) + (r & 3)) * 32);
         }
-        rankUpdatesFenced<HDP>(gs + sb * 32 * LDSW, pr, dv, half, li);
+        rankUpdatesFenced<HDP, 0, DTN>(gs + sb * 32 * LDSW, pr, dv, half, li);
     }
 }
 
-template <int HDP, int BQ>
+template <int HDP, int BQ, int DTN>
 __device__ __forceinline__ void dkvTileDs(const float* __restrict__ qs, const float* __restrict__ gs, const float* __restrict__ stats,
-                                          const float (&vreg)[HDP / 2], float16v (&dk)[HDP / 32], int qt0, int half, int li,
+                                          const float (&vreg)[HDP / 2], float16v (&dk)[DTN], int qt0, int half, int li,
                                           float* __restrict__ dsLane, size_t dsStride, int newLen) {
     constexpr int LDSW = HDP + 4, NSB = BQ / 32;
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb) {
         float* dst = dsLane + sb * dsStride;
         const bool stored = qt0 + sb * 32 < newLen;   // rows past the sequence hold no P (it is zero there)
-        float16v pr;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) pr[r] = stored ? __builtin_nontemporal_load(dst + (8 * (r >> 2) + (r & 3)) * 32) : 0.0f;
+        const float16v pr = readParked(dst, stored);
         float16v dsv;
 #pragma unroll
         for (int r = 0; r < 16; ++r) dsv[r] = 0.0f;
@@ -991,22 +1053,23 @@ __device__ __forceinline__ void dkvTileDs(const float* __restrict__ qs, const fl
 #pragma unroll
             for (int r = 0; r < 16; ++r) __builtin_nontemporal_store(dsv[r], dst + (8 * (r >> 2) + (r & 3)) * 32);
         }
-        rankUpdatesFenced<HDP>(qs + sb * 32 * LDSW, dsv, dk, half, li);
+        rankUpdatesFenced<HDP, 0, DTN>(qs + sb * 32 * LDSW, dsv, dk, half, li);
     }
 }
 
 // One pass of the key-tile owner over its query tiles for head dims above 128: Q and dO tiles (and lse2, D) through the
 // double-buffered LDS stage, one barrier per tile.  MODE 0: dkvTileP with `reg` = the K rows and `acc` = dV; MODE 1:
-// dkvTileDs with `reg` = the V rows and `acc` = dK.  With 16-byte aligned rows (VEC4) the tiles go from global memory
+// dkvTileDs with `reg` = the V rows and `acc` = dK; `acc` holds the first DTN head-dim blocks.  MODE 2 / MODE 3
+// (dkvTileAgain, head dim 256, whose accumulators take the head dim in two halves): the parked P meets the dO columns
+// of blocks DT0.. for the rest of dV / the stored dS meets the Q columns of blocks DT0.. for the rest of dK; `reg` is
+// not read and only the tile that is needed is brought in.  With 16-byte aligned rows (VEC4) the tiles go from global memory
 // straight into LDS (global_load_lds, one 1 KiB row per wavefront instruction, lanes past the head dim switched off: those
 // columns were zeroed once), which frees the 64 registers a tile in flight would occupy; rows past the sequence repeat
 // its last row (finite values that meet P = 0 and dS = 0).  Otherwise tiles are staged through registers as in
 // attnBackwardDkvKernel.
-typedef __attribute__((address_space(1))) const void* GlobalPtr;
-typedef __attribute__((address_space(3))) void* LdsPtr;
-template <int HDP, int BQ, bool VEC4, int MODE>
+template <int HDP, int BQ, bool VEC4, int MODE, int DT0, int DTN>
 __device__ __forceinline__ void dkvStreamPass(const AttnParams& p, float* __restrict__ qs, float* __restrict__ gs, float* __restrict__ stats,
-                                              const float (&reg)[HDP / 2], float16v (&acc)[HDP / 32], int bh, int kt, size_t qOff,
+                                              const float (&reg)[HDP / 2], float16v (&acc)[DTN], int bh, int kt, size_t qOff,
                                               size_t statOff, int waveK0, int key, bool keyValid, int half, int li, int tid) {
     constexpr int LDSW = HDP + 4, TILE = BQ * LDSW;
     const int hd = p.hd, dim = p.dim;
@@ -1026,15 +1089,19 @@ __device__ __forceinline__ void dkvStreamPass(const AttnParams& p, float* __rest
             float* dsLane = dsColumn + size_t(qt0 >> 5) * dsStride + dsLaneOffset;
             if constexpr (MODE == 0) {
                 const bool masked = (waveK0 + 31 > p.oldLen + qt0) || (waveK0 + 32 > p.totalLen);
-                if (masked) dkvTileP<HDP, BQ, true>(qcur, gcur, scur, reg, acc, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride, p.newLen);
-                else dkvTileP<HDP, BQ, false>(qcur, gcur, scur, reg, acc, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride, p.newLen);
+                if (masked) dkvTileP<HDP, BQ, true, DTN>(qcur, gcur, scur, reg, acc, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride, p.newLen);
+                else dkvTileP<HDP, BQ, false, DTN>(qcur, gcur, scur, reg, acc, qt0, key, keyValid, p.oldLen, half, li, dsLane, dsStride, p.newLen);
+            } else if constexpr (MODE == 1) {
+                dkvTileDs<HDP, BQ, DTN>(qcur, gcur, scur, reg, acc, qt0, half, li, dsLane, dsStride, p.newLen);
             } else {
-                dkvTileDs<HDP, BQ>(qcur, gcur, scur, reg, acc, qt0, half, li, dsLane, dsStride, p.newLen);
+                dkvTileAgain<HDP, BQ, DT0, DTN>(MODE == 2 ? gcur : qcur, acc, qt0, half, li, dsLane, dsStride, p.newLen);
             }
         }
     };
     float statNext = 0.0f;
+    constexpr bool kNeedQ = MODE != 2, kNeedG = MODE != 3, kNeedStats = MODE < 2;
     auto fetchStats = [&](int qt0) __attribute__((always_inline)) {
+        if constexpr (!kNeedStats) return;
         const int qi = qt0 + (tid < BQ ? tid : tid - BQ);
         if (tid < BQ) statNext = qi < p.newLen ? p.lse2[statOff + qi] : INFINITY;
         else if (tid < 2 * BQ) statNext = qi < p.newLen ? p.dvec[statOff + qi] : 0.0f;
@@ -1050,8 +1117,8 @@ __device__ __forceinline__ void dkvStreamPass(const AttnParams& p, float* __rest
                 const int r = wave + 4 * i;
                 const size_t row = size_t(min(qt0 + r, p.newLen - 1)) * dim;
                 if (columnValid) {
-                    __builtin_amdgcn_global_load_lds((GlobalPtr)(qBase + row), (LdsPtr)(qs + buf * TILE + r * LDSW), 16, 0, 0);
-                    __builtin_amdgcn_global_load_lds((GlobalPtr)(gBase + row), (LdsPtr)(gs + buf * TILE + r * LDSW), 16, 0, 0);
+                    if constexpr (kNeedQ) __builtin_amdgcn_global_load_lds((GlobalPtr)(qBase + row), (LdsPtr)(qs + buf * TILE + r * LDSW), 16, 0, 0);
+                    if constexpr (kNeedG) __builtin_amdgcn_global_load_lds((GlobalPtr)(gBase + row), (LdsPtr)(gs + buf * TILE + r * LDSW), 16, 0, 0);
                 }
             }
         };
@@ -1062,7 +1129,7 @@ __device__ __forceinline__ void dkvStreamPass(const AttnParams& p, float* __rest
         if (numQTiles > 0) {
             issueTile(q0Start, 0);
             fetchStats(q0Start);
-            if (tid < 2 * BQ) stats[tid] = statNext;
+            if (kNeedStats && tid < 2 * BQ) stats[tid] = statNext;
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -1073,7 +1140,7 @@ __device__ __forceinline__ void dkvStreamPass(const AttnParams& p, float* __rest
                 fetchStats(qt0 + BQ);
             }
             tileBody(t, qt0);
-            if (t + 1 < numQTiles && tid < 2 * BQ) stats[((t + 1) & 1) * 2 * BQ + tid] = statNext;
+            if (kNeedStats && t + 1 < numQTiles && tid < 2 * BQ) stats[((t + 1) & 1) * 2 * BQ + tid] = statNext;
             // the tile's loads have landed in LDS (the stores of the tile body, issued a hundred MFMAs ago, are long done)
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();   // after the last tile too: the next pass writes the LDS buffers again
@@ -1081,14 +1148,14 @@ __device__ __forceinline__ void dkvStreamPass(const AttnParams& p, float* __rest
     } else {
         TileRegs<HDP, BQ> qNext, gNext;
         auto fetchAll = [&](int qt0) __attribute__((always_inline)) {
-            fetchHeadTile<HDP, BQ, VEC4>(qNext, p.q + qOff, dim, qt0, p.newLen, hd, tid);
-            fetchHeadTile<HDP, BQ, VEC4>(gNext, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
+            if constexpr (kNeedQ) fetchHeadTile<HDP, BQ, VEC4>(qNext, p.q + qOff, dim, qt0, p.newLen, hd, tid);
+            if constexpr (kNeedG) fetchHeadTile<HDP, BQ, VEC4>(gNext, p.dO + qOff, dim, qt0, p.newLen, hd, tid);
             fetchStats(qt0);
         };
         auto commitAll = [&](int buf) __attribute__((always_inline)) {
-            commitHeadTile<HDP, BQ>(qs + buf * TILE, qNext, tid);
-            commitHeadTile<HDP, BQ>(gs + buf * TILE, gNext, tid);
-            if (tid < 2 * BQ) stats[buf * 2 * BQ + tid] = statNext;
+            if constexpr (kNeedQ) commitHeadTile<HDP, BQ>(qs + buf * TILE, qNext, tid);
+            if constexpr (kNeedG) commitHeadTile<HDP, BQ>(gs + buf * TILE, gNext, tid);
+            if (kNeedStats && tid < 2 * BQ) stats[buf * 2 * BQ + tid] = statNext;
         };
         if (numQTiles > 0) {
             fetchAll(q0Start);
@@ -1109,8 +1176,8 @@ __device__ __forceinline__ void dkvStreamPass(const AttnParams& p, float* __rest
 }
 
 // One of the two key gradients (IS_K: dK, scaled; else dV), fp32 tensor and bf16 image, as storeKeyGradients stores them.
-template <int HDP, bool IS_K>
-__device__ __forceinline__ void storeOneKeyGradient(const AttnParams& p, const float16v (&acc)[HDP / 32], int b, int h, int waveK0,
+template <int HDP, bool IS_K, int DT0, int DTN>
+__device__ __forceinline__ void storeOneKeyGradient(const AttnParams& p, const float16v (&acc)[DTN], int b, int h, int waveK0,
                                                     size_t kOff, int half, int li) {
     const int hd = p.hd, dim = p.dim;
     float* __restrict__ out = IS_K ? p.dK : p.dV;
@@ -1118,8 +1185,8 @@ __device__ __forceinline__ void storeOneKeyGradient(const AttnParams& p, const f
     const float mul = IS_K ? p.scale : 1.0f;
     const bool pairs = (hd & 1) == 0 && (p.imgLd & 1u) == 0 && (reinterpret_cast<uintptr_t>(img) & 3u) == 0;
 #pragma unroll
-    for (int dt = 0; dt < HDP / 32; ++dt) {
-        const int d = dt * 32 + li;
+    for (int dt = 0; dt < DTN; ++dt) {
+        const int d = (DT0 + dt) * 32 + li;
         if (d < hd) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -1166,28 +1233,46 @@ __global__ void __launch_bounds__(256, OCC) attnBackwardDkvKernel(AttnParams p) 
     const int key = waveK0 + li;                       // this lane's key (as B-operand column)
     const bool keyValid = key < p.totalLen;
     if constexpr (HDP > 128 && STORE) {
-        // two passes that share out the products (dkvTileP / dkvTileDs above)
+        // two passes that share out the products (dkvTileP / dkvTileDs above).  At head dim 256 an accumulator set is 128
+        // registers beside the 128 of the K or V rows: each pass keeps the first half of its accumulators, and a second walk
+        // over the tiles (dkvTileAgain: the parked P or dS against the other half of the columns, no K or V rows, one
+        // tile instead of two) makes the rest, so that no walk leaves its registers (the one-walk form spilled 171).
+        constexpr int HALVES = HDP > 192 ? 2 : 1, DTN = DT / HALVES;
+        auto zero = [](float16v (&acc)[DTN]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int dt = 0; dt < DTN; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
+        };
         {
             float kreg[HDP / 2];
             loadRowOperand<HDP, VEC4>(kreg, p.k + kOff + size_t(key) * dim, keyValid, hd, half, p.scale * kLog2e);
-            float16v dv[DT];
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) dv[dt][r] = 0.0f;
-            dkvStreamPass<HDP, BQ, VEC4, 0>(p, qs, gs, stats, kreg, dv, bh, kt, qOff, statOff, waveK0, key, keyValid, half, li, tid);
-            storeOneKeyGradient<HDP, false>(p, dv, b, h, waveK0, kOff, half, li);
+            float16v dv[DTN];
+            zero(dv);
+            dkvStreamPass<HDP, BQ, VEC4, 0, 0, DTN>(p, qs, gs, stats, kreg, dv, bh, kt, qOff, statOff, waveK0, key, keyValid, half, li, tid);
+            storeOneKeyGradient<HDP, false, 0, DTN>(p, dv, b, h, waveK0, kOff, half, li);
+        }
+        if constexpr (HALVES == 2) {
+            float none[HDP / 2];   // never read
+            float16v dv[DTN];
+            zero(dv);
+            dkvStreamPass<HDP, BQ, VEC4, 2, DTN, DTN>(p, qs, gs, stats, none, dv, bh, kt, qOff, statOff, waveK0, key, keyValid, half, li, tid);
+            storeOneKeyGradient<HDP, false, DTN, DTN>(p, dv, b, h, waveK0, kOff, half, li);
         }
         {
             float vreg[HDP / 2];
             loadRowOperand<HDP, VEC4>(vreg, p.v + kOff + size_t(key) * dim, keyValid, hd, half, 1.0f);
-            float16v dk[DT];
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) dk[dt][r] = 0.0f;
-            dkvStreamPass<HDP, BQ, VEC4, 1>(p, qs, gs, stats, vreg, dk, bh, kt, qOff, statOff, waveK0, key, keyValid, half, li, tid);
-            storeOneKeyGradient<HDP, true>(p, dk, b, h, waveK0, kOff, half, li);
+            float16v dk[DTN];
+            zero(dk);
+            dkvStreamPass<HDP, BQ, VEC4, 1, 0, DTN>(p, qs, gs, stats, vreg, dk, bh, kt, qOff, statOff, waveK0, key, keyValid, half, li, tid);
+            storeOneKeyGradient<HDP, true, 0, DTN>(p, dk, b, h, waveK0, kOff, half, li);
+        }
+        if constexpr (HALVES == 2) {
+            float none[HDP / 2];   // never read
+            float16v dk[DTN];
+            zero(dk);
+            dkvStreamPass<HDP, BQ, VEC4, 3, DTN, DTN>(p, qs, gs, stats, none, dk, bh, kt, qOff, statOff, waveK0, key, keyValid, half, li, tid);
+            storeOneKeyGradient<HDP, true, DTN, DTN>(p, dk, b, h, waveK0, kOff, half, li);
         }
         return;
     }

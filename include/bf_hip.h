@@ -374,9 +374,9 @@ int bf_hip_bf16_weight_cache_refresh(const float* const* changed, size_t count, 
  * Query row i (absolute position oldLen+i) attends to keys j <= oldLen+i.
  * Tuned head dims are 32, 64 and 128 (forward and backward 110-175 TFLOP/s of fp32 work at 1024-4096 positions).  Head
  * dims above 128 are accepted, like the reference accepts them, and run on the fp32-MFMA kernels padded to 192 or 256:
- * measured at batch 4, 8 heads, 2048 positions, headDim 192: forward 94, dK/dV 96, dQ 95 TFLOP/s = 0.60 of the fp32
- * MFMA peak for forward + backward (headDim 160, a sixth of it padding: 81 / 83 / 81); headDim 256: 70 / 68 / 95 =
- * 0.45.  When the dS hand-over buffer is refused (bf_hip_attention_set_workspace_limit) the dK/dV pass of such heads
+ * measured at batch 4, 8 heads, 2048 positions, headDim 192: forward 100, dK/dV 96, dQ 96 TFLOP/s = 0.61 of the fp32
+ * MFMA peak for forward + backward; headDim 256: 100 / 92 / 97 = 0.60 (headDim 224, an eighth of it padding: 90 / 81 /
+ * 85).  When the dS hand-over buffer is refused (bf_hip_attention_set_workspace_limit) the dK/dV pass of such heads
  * falls to about half of that.
  * ------------------------------------------------------------------------------------------- */
 /* fusedAttentionForward: out:[batch,newLen,dim]; m,l:[batch,heads,newLen] = row max of the scaled
