@@ -42,7 +42,10 @@ CASES = [(1, 1, 1, 0, 2), (1, 2, 3, 0, 2), (2, 2, 5, 0, 4), (2, 3, 33, 0, 32), (
          (1, 1, 70, 30, 200),
          # head dims above 128 over several key tiles and query tiles (the key-tile owner's two passes that share out
          # the products: P parked in the dS buffer, read back and replaced by dS), ragged ends, an offset, a 4-byte aligned dim
-         (2, 2, 300, 0, 192), (1, 2, 260, 40, 256), (1, 1, 129, 129, 136), (1, 1, 140, 0, 130)]
+         (2, 2, 300, 0, 192), (1, 2, 260, 40, 256), (1, 1, 129, 129, 136), (1, 1, 140, 0, 130),
+         # the 256-wide padding class on rows that are not 16-byte aligned (tiles staged through registers), and the
+         # widest head that is padded to 192
+         (1, 2, 140, 20, 250), (2, 1, 200, 0, 224), (1, 3, 170, 0, 192)]
 
 
 @pytest.mark.parametrize("batch,heads,new_len,old_len,hd", CASES)
