@@ -288,6 +288,35 @@ def bench_extras(bf, steps):
                                              "frac_of_measured_mfma_ceiling": round(tf / ceiling_tf, 3)}
         ms = timed(lambda: call("bf_hip_matmul_bf16", a.ptr, w.ptr, c.ptr, m, k, n_, 1, sh), 3)
         extras[f"matmul_bf16_fp32_io_{m}x{n_}x{k}"] = {"ms": round(ms, 4), "TFLOP/s": round(2 * m * n_ * k / ms / 1e9, 1)}
+    # fused attention at the other shapes the library serves: the GPT-small and long-context layers, and head dims
+    # above 128 (fp32-MFMA kernels padded to 192 or 256); forward, dK/dV with the dS hand-over, dQ from dS
+    def attention(batch, heads, seq, hd):
+        dim, scale = heads * hd, 1.0 / np.sqrt(np.float32(hd))
+        q, k, v, go = (rand(batch, seq, dim) for _ in range(4))
+        out, dq, dk, dv = (D((batch, seq, dim)) for _ in range(4))
+        m, l, lse2, dvec = (D((batch, heads, seq)) for _ in range(4))
+        dims = (batch, heads, seq, seq, dim, ctypes.c_float(scale), 0, sh)
+        ds_bytes = ctypes.c_size_t(0)
+        call("bf_hip_attention_ds_bytes", batch, heads, seq, seq, ctypes.byref(ds_bytes))
+        ds = D((ds_bytes.value // 4,))
+        fwd = lambda: call("bf_hip_attention_forward", q.ptr, k.ptr, v.ptr, out.ptr, m.ptr, l.ptr, *dims)
+        fwd()
+        call("bf_hip_attention_backward_prepare", out.ptr, go.ptr, m.ptr, l.ptr, lse2.ptr, dvec.ptr, batch, heads, seq, dim, sh)
+        dkv = lambda: call("bf_hip_attention_backward_dkv_ds", go.ptr, q.ptr, k.ptr, v.ptr, lse2.ptr, dvec.ptr, dk.ptr, dv.ptr, ds.ptr, *dims)
+        dqk = lambda: call("bf_hip_attention_backward_dq_from_ds", ds.ptr, k.ptr, dq.ptr, *dims)
+        fl = attention_flops(batch, heads, seq, hd)
+        t = {name: timed(fn, 5) for name, fn in (("forward", fwd), ("dkv", dkv), ("dq", dqk))}
+        total = (fl["fwd"] + fl["dkv"] + fl["dq"]) / (t["forward"] + t["dkv"] + t["dq"]) / 1e9
+        extras[f"attention_b{batch}_h{heads}_s{seq}_hd{hd}"] = {
+            "ms": {name: round(ms, 4) for name, ms in t.items()},
+            "TFLOP/s": {"forward": round(fl["fwd"] / t["forward"] / 1e9, 1), "dkv": round(fl["dkv"] / t["dkv"] / 1e9, 1),
+                        "dq": round(fl["dq"] / t["dq"] / 1e9, 1), "forward_dkv_dq": round(total, 1)},
+            "frac_fp32_mfma": round(total / PEAK_FP32_MFMA_TFLOPS, 3)}
+    attention(8, 12, 1024, 64)
+    attention(4, 16, 4096, 128)
+    attention(4, 8, 2048, 192)
+    attention(4, 8, 2048, 256)
+
     gemm(4096, 4096, 4096)
     gemm(16384, 8192, 2048)
     # GPT-small shapes: FFN up, FFN down / its input gradient (tall and narrow: 128-row tiles), FFN weight gradient (K slices)
