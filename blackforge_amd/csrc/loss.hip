@@ -340,6 +340,134 @@ __global__ void __launch_bounds__(kBlock) columnPartialsFinishKernel(const float
     }
 }
 
+// The head's loss for rows that the kernel above does not serve: more classes than its column sums have LDS for
+// (up to 1024 x 52), or a class count that is not a multiple of 8 (rows that start on any 4-byte boundary; the image's
+// rows are `pitch` = classes rounded up to 8 apart, the columns past the row zero).  One row at a time in 52 registers a
+// thread, read with 16-byte loads from whatever boundary the row starts on (global memory serves those), the gradient
+// written as its bf16 image only; same arithmetic per element as crossEntropyKernel.  The bias gradient is then the
+// column sums of that image (columnSumBf16Kernel): the sum of the gradient values as the head's products see them.
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));   // a float4 that may start on any 4-byte boundary
+template <bool NT>
+__global__ void __launch_bounds__(1024) crossEntropyImageWideKernel(const float* __restrict__ logits, const float* __restrict__ target,
+                                                                    unsigned short* __restrict__ gradImage, float* __restrict__ rowLoss,
+                                                                    size_t rows, size_t classes, size_t pitch, float invRows) {
+    constexpr int G = 1024, MAXE = 52, VEC = 4;
+    __shared__ float lds[16];
+    const int t = threadIdx.x;
+    const int n = int(classes), wide = int(pitch);   // at most 1024 x 52
+    const int tailStart = n & ~3, tailIt = (n & 3) ? tailStart / (G * VEC) : -1, tailThread = (tailStart / VEC) % G;
+    for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const float* __restrict__ x = logits + row * classes;
+        float r[MAXE];
+        // every load first, without a branch (a group that is not wholly inside the row re-reads group 0), the masking
+        // afterwards; the row's last, partial group (one thread's, if the length is not a multiple of 4) element by element
+#pragma unroll
+        for (int it = 0; it < MAXE / VEC; ++it) {
+            const int e = (it * G + t) * VEC;
+            const float* src = x + (e + VEC <= n ? e : 0);
+            float4u v;
+            if constexpr (NT) v = __builtin_nontemporal_load(reinterpret_cast<const float4u*>(src));
+            else v = *reinterpret_cast<const float4u*>(src);
+            r[it * VEC + 0] = v.x; r[it * VEC + 1] = v.y; r[it * VEC + 2] = v.z; r[it * VEC + 3] = v.w;
+        }
+#pragma unroll
+        for (int it = 0; it < MAXE / VEC; ++it) {
+            const int e = (it * G + t) * VEC;
+            const bool whole = e + VEC <= n;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) r[it * VEC + j] = whole ? r[it * VEC + j] : -INFINITY;
+            if (it == tailIt && t == tailThread) {   // (the first condition is the same for the whole block)
+#pragma unroll
+                for (int j = 0; j < VEC - 1; ++j)
+                    if (tailStart + j < n) r[it * VEC + j] = x[tailStart + j];
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < MAXE; ++i) mx = fmaxf(mx, r[i]);
+        mx = groupMax<G>(mx, lds);
+        constexpr float kLog2e = 1.4426950408889634f;
+        const float top = mx * kLog2e;
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < MAXE; ++i) { r[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(r[i], kLog2e, -top)); sum += r[i]; }
+        sum = groupSum<G>(sum, lds);
+        const float inv = 1.0f / sum;
+        const unsigned cls = unsigned(lroundf(target[row]));
+        const int targetIt = cls < classes ? int(cls / unsigned(G * VEC)) : -1;
+        const bool mine = int((cls / VEC) % G) == t;
+        const int targetSlot = int(cls % VEC);
+        const float scale = inv * invRows;
+        float pTarget = -1.0f;
+#pragma unroll
+        for (int it = 0; it < MAXE / VEC; ++it) {
+            if (it == targetIt) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const bool hit = mine && j == targetSlot;
+                    const float p = r[it * VEC + j] * inv;
+                    pTarget = hit ? p : pTarget;
+                    r[it * VEC + j] = hit ? (p - 1.0f) * invRows : r[it * VEC + j] * scale;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) r[it * VEC + j] *= scale;
+            }
+        }
+        unsigned short* __restrict__ out = gradImage + row * pitch;
+#pragma unroll
+        for (int it = 0; it < MAXE / VEC; ++it) {   // slots past the row's end hold exp2(-inf) * scale = 0: the image's padding
+            const int e = (it * G + t) * VEC;
+            if (e < wide) {
+                const uint2v packed = {unsigned(toBf16Bits(r[it * VEC + 0])) | unsigned(toBf16Bits(r[it * VEC + 1])) << 16,
+                                       unsigned(toBf16Bits(r[it * VEC + 2])) | unsigned(toBf16Bits(r[it * VEC + 3])) << 16};
+                stu2<NT>(out + e, packed);
+            }
+        }
+        float loss = pTarget >= 0.0f ? -logf(fmaxf(pTarget, 1e-12f)) : 0.0f;
+        loss = groupSum<G>(loss, lds);
+        if (t == 0) rowLoss[row] = loss;
+    }
+}
+
+// partial[band * pitch + c] = sum of image[row * pitch + c] over the rows of band `blockIdx.y` (rowsPerBand each), in row
+// order: a thread owns eight columns (16 bytes of a row) and keeps four rows' loads in flight.
+__global__ void __launch_bounds__(kBlock) columnSumBf16Kernel(const unsigned short* __restrict__ image, float* __restrict__ partial,
+                                                              size_t rows, size_t pitch, size_t rowsPerBand) {
+    const size_t c = (size_t(blockIdx.x) * kBlock + threadIdx.x) * 8;
+    if (c >= pitch) return;
+    const size_t rowBegin = size_t(blockIdx.y) * rowsPerBand, rowEnd = rowBegin + rowsPerBand < rows ? rowBegin + rowsPerBand : rows;
+    float sums[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    auto add = [&](uint4v v) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            sums[2 * j] += __builtin_bit_cast(float, v[j] << 16);
+            sums[2 * j + 1] += __builtin_bit_cast(float, v[j] & 0xffff0000u);
+        }
+    };
+    size_t row = rowBegin;
+    for (; row + 4 <= rowEnd; row += 4) {
+        uint4v v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(image + (row + i) * pitch + c));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) add(v[i]);
+    }
+    for (; row < rowEnd; ++row) add(__builtin_nontemporal_load(reinterpret_cast<const uint4v*>(image + row * pitch + c)));
+    float* __restrict__ out = partial + size_t(blockIdx.y) * pitch + c;
+    storef4(out, float4v{sums[0], sums[1], sums[2], sums[3]});
+    storef4(out + 4, float4v{sums[4], sums[5], sums[6], sums[7]});
+}
+// out[c] = sum over the bands, in band order, for the `features` columns that exist (pitch >= features)
+__global__ void __launch_bounds__(kBlock) columnBandsFinishKernel(const float* __restrict__ partial, float* __restrict__ out, size_t bands,
+                                                                  size_t pitch, size_t features) {
+    const size_t c = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (c >= features) return;
+    float total = 0.0f;
+    for (size_t b = 0; b < bands; ++b) total += partial[b * pitch + c];
+    out[c] = total;
+}
+
 template <bool SPARSE>
 int launchCrossEntropy(const float* logits, const float* target, float* grad, float* lossSum, size_t rows,
                        size_t classes, int accumulate, hipStream_t s, bool masked = false, unsigned short* gradImage = nullptr) {
@@ -468,14 +596,40 @@ int bf_hip_cross_entropy_sparse_img(const float* logits, const float* targetIdx,
 int bf_hip_cross_entropy_sparse_head(const float* logits, const float* targetIdx, uint16_t* gradImage, float* biasGrad, float* lossSum,
                                      size_t rows, size_t classes, int accumulate, bf_stream_t stream) {
     BF_REQUIRE(lossSum != nullptr, "lossSum is NULL");
-    // the rows a 1024-thread block can hold in 16 or 32 registers a thread, 16-byte aligned throughout, with a whole bf16 image
-    if (rows == 0 || classes == 0 || classes % 8 != 0 || classes > size_t(1024) * 32 || classes < 4096 || !aligned16(logits) ||
-        !aligned16(gradImage) || !aligned16(biasGrad)) {
+    // the rows a 1024-thread block can hold in its registers, with a 16-byte aligned bf16 image
+    if (rows == 0 || classes < 4096 || classes > size_t(1024) * 52 || !aligned16(gradImage)) {
         setLastError("bf_hip_cross_entropy_sparse_head: shape or alignment not served by the fused form (use bf_hip_cross_entropy_sparse_img and bf_hip_bias_grad)");
         return BF_ERR_UNSUPPORTED;
     }
     BF_REQUIRE(logits && targetIdx && gradImage && biasGrad, "NULL pointer");
     hipStream_t s = asStream(stream);
+    if (classes % 8 != 0 || classes > size_t(1024) * 32 || !aligned16(logits) || !aligned16(biasGrad)) {
+        // rows of any length up to 1024 x 52 and any alignment: the loss with the image alone, then the image's column sums
+        const size_t pitch = (classes + 7) / 8 * 8;
+        const float invRows = 1.0f / float(rows);
+        const unsigned grid = unsigned(std::min<size_t>(rows, kMaxGridX));
+        Scratch rowLoss(rows * sizeof(float));
+        if (rowLoss.status != BF_OK) return rowLoss.status;
+        if (streamsPastCache(rows * classes * 6))
+            crossEntropyImageWideKernel<true><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), rows, classes, pitch, invRows);
+        else
+            crossEntropyImageWideKernel<false><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), rows, classes, pitch, invRows);
+        BF_LAUNCH_CHECK();
+        // bands of rows so that the grid has a few thousand workgroups
+        const size_t columnBlocks = (pitch / 8 + kBlock - 1) / kBlock;
+        size_t bands = std::max<size_t>(1, std::min<size_t>((rows + 63) / 64, (size_t(computeUnits()) * 8 + columnBlocks - 1) / columnBlocks));
+        const size_t rowsPerBand = (rows + bands - 1) / bands;
+        bands = (rows + rowsPerBand - 1) / rowsPerBand;
+        Scratch partial(bands * pitch * sizeof(float));
+        if (partial.status != BF_OK) return partial.status;
+        columnSumBf16Kernel<<<dim3(unsigned(columnBlocks), unsigned(bands)), kBlock, 0, s>>>(gradImage, partial.as<float>(), rows, pitch, rowsPerBand);
+        BF_LAUNCH_CHECK();
+        columnBandsFinishKernel<<<gridFor(classes, kBlock), kBlock, 0, s>>>(partial.as<float>(), biasGrad, bands, pitch, classes);
+        BF_LAUNCH_CHECK();
+        finishSumKernel<<<1, 1024, 0, s>>>(rowLoss.as<float>(), rows, lossSum, accumulate);
+        BF_LAUNCH_CHECK();
+        return BF_OK;
+    }
     const unsigned grid = unsigned(std::min<size_t>(rows, size_t(computeUnits()) * 2));
     Scratch rowLoss(rows * sizeof(float));
     if (rowLoss.status != BF_OK) return rowLoss.status;

@@ -479,11 +479,16 @@ int bf_hip_cross_entropy_sparse_img(const float* logits, const float* targetIdx,
                                     size_t rows, size_t classes, int accumulate, bf_stream_t stream);
 /* The loss of a language-model head whose gradient is read by nothing but the head's own gradient products
  * (softmaxCrossEntropySparseAccumulate followed by the backward pass of the last linear layer, loss.cu:381-411 and
- * model.cu:278-284 in one pass over the logits): gradImage[rows, classes] receives the gradient rounded to bf16 (the
- * operand of bf_hip_matmul_bf16_backward_img), biasGrad[classes] its column sums taken in fp32 before the rounding (the
- * bias gradient), and no fp32 gradient is written.  Same loss and same image as bf_hip_cross_entropy_sparse_img; the
- * column sums are added in another (fixed) order than bf_hip_bias_grad adds them.  Served shapes: 16-byte aligned
- * tensors, classes a multiple of 8 between 4096 and 32768; anything else returns BF_ERR_UNSUPPORTED and launches nothing. */
+ * model.cu:278-284 in one pass over the logits): gradImage receives the gradient rounded to bf16 (the operand of
+ * bf_hip_matmul_bf16_backward_img: rows of classes rounded up to 8 elements, the extra columns zero), biasGrad[classes]
+ * the bias gradient, and no fp32 gradient is written.  16-byte aligned tensors with classes a multiple of 8 between
+ * 4096 and 32768 take one pass: same loss and same image as bf_hip_cross_entropy_sparse_img, the column sums taken in fp32
+ * before the rounding, added in another (fixed) order than bf_hip_bias_grad adds them.  Other class counts from 4096 to
+ * 53248 (an odd vocabulary such as 50257: rows on any 4-byte boundary) and unaligned logits take two: the loss with the
+ * image (an element may differ from the other kernels' image by one bf16 step: the row sums add in another order), then
+ * the image's column sums, i.e. the bias gradient of the rounded gradient values that the head's products use.  Anything
+ * else (fewer than 4096 or more than 53248 classes, an image that is not 16-byte aligned) returns BF_ERR_UNSUPPORTED and
+ * launches nothing. */
 int bf_hip_cross_entropy_sparse_head(const float* logits, const float* targetIdx, uint16_t* gradImage, float* biasGrad, float* lossSum,
                                      size_t rows, size_t classes, int accumulate, bf_stream_t stream);
 /* softmaxCrossEntropyMasked (the CPU backend's loss for masked-language-model training, src/backend/cpu/loss.cpp:149-215;

@@ -55,7 +55,10 @@ public:
     // for tensors that are not modified after the producing call.  Not part of the reference's DeviceTensor.
     [[nodiscard]] std::uint16_t* attachImage() {
         releaseImage();
-        imageBytes_ = elementCount() * sizeof(std::uint16_t);
+        // rows of the last dimension rounded up to 8 elements (16 bytes), the row pitch of every bf16 operand image
+        const std::size_t cols = shape_.empty() ? 0 : shape_.back();
+        const std::size_t rows = cols != 0 ? elementCount() / cols : 0;
+        imageBytes_ = rows * ((cols + 7) / 8 * 8) * sizeof(std::uint16_t);
         image_ = static_cast<std::uint16_t*>(devicePoolAcquire(imageBytes_));
         return image_;
     }

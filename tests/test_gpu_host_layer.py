@@ -331,11 +331,12 @@ def test_gradients_accumulate_over_backward_passes(hip, rng, use_bf16):
         assert_bits_equal(gpu.grad(i), g, "grad after zeroGrad " + gpu.names[i])
 
 
-@pytest.mark.parametrize("vocab", [96, 4096])
+@pytest.mark.parametrize("vocab", [96, 4096, 4099])
 def test_bf16_model_step_stays_within_bf16_tolerance(hip, oracle, rng, vocab):
     """bf16 projections (precision.compute = bf16): logits and gradients within 2e-2 of the fp32 CPU reference.  With a
     vocabulary of 4096 the step takes the loss of the language-model head in its fused form (gradient as a bf16 image
-    plus the head's bias gradient, no fp32 gradient)."""
+    plus the head's bias gradient, no fp32 gradient); with an odd vocabulary of 4099 the form whose image rows are
+    padded to a multiple of 8 and whose bias gradient is the image's column sums."""
     from blackforge_amd import hostlayer as hl
     from oracle import bfo
     dim, seq, batch, heads, hidden = 64, 32, 4, 2, 128

@@ -143,13 +143,51 @@ def test_cross_entropy_of_a_language_model_head(hip, oracle, rng, rows, classes)
     assert_close(bias.toHost(), sums.astype(f32), tol=1e-4, what="column sums of the gradient", scale=float(np.abs(expected_grad).max()))
 
 
+@pytest.mark.parametrize("rows,classes,offset", [(3, 50257, 0), (300, 50257, 0), (5, 40000, 0), (64, 4099, 0), (130, 53248, 0), (7, 4100, 0),
+                                                 (33, 8192, 1), (2, 53241, 3)])
+def test_cross_entropy_of_a_head_with_an_odd_or_large_vocabulary(hip, oracle, rng, rows, classes, offset):
+    """bf_hip_cross_entropy_sparse_head beyond its one-pass form (class counts that are not multiples of 8, more than
+    32768 classes, logits that do not start on a 16-byte boundary): the loss, the gradient image in rows of classes
+    rounded up to 8 (the padding zero), within one bf16 step of the rounded fp32 gradient of bf_hip_cross_entropy_sparse,
+    and as bias gradient the column sums of that image."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    logits = r(rng, rows, classes, scale=3)
+    idx = rng.integers(0, classes, rows).astype(f32)
+    idx[0], idx[-1] = 0, classes - 1
+    flat = np.concatenate([np.zeros(offset, f32), logits.ravel()])
+    dflat, di = D.fromHost(flat), D.fromHost(idx)
+    at = ctypes.c_void_p(dflat.ptr.value + 4 * offset)   # the logits start `offset` floats into the allocation
+    grad, loss = D((rows, classes)), D.zeros((1,))
+    call("bf_hip_cross_entropy_sparse", at, di.ptr, grad.ptr, loss.ptr, rows, classes, 0, None)
+    pitch = (classes + 7) // 8 * 8
+    img = D.fromHost(np.full((rows, pitch // 2), 7.0, f32))   # raw storage of the image, filled with something else
+    bias, loss2 = D.fromHost(np.full(classes, 7.0, f32)), D.fromHost(np.array([2.5], f32))
+    call("bf_hip_cross_entropy_sparse_head", at, di.ptr, img.ptr, bias.ptr, loss2.ptr, rows, classes, 1, None)
+    image = as_f32(img.toHost().view(np.uint16).reshape(rows, pitch)).astype(np.float64)
+    assert (image[:, classes:] == 0).all(), "the columns past the row are zero"
+    g = grad.toHost().astype(np.float64)
+    assert (np.abs(image[:, :classes] - g) <= 2.0 ** -8 * np.abs(g) + 1e-30).all(), "gradient image: more than half a bf16 step from the fp32 gradient"
+    assert abs(loss2.toHost()[0] - 2.5 - loss.toHost()[0]) <= 1e-6 * abs(loss.toHost()[0]) + 1e-6
+    expected_loss, expected_grad = oracle.softmaxCrossEntropySparse(logits, idx)
+    assert abs(loss.toHost()[0] / rows - expected_loss) <= 1e-5 * abs(expected_loss)
+    sums = image[:, :classes].sum(axis=0)
+    assert_close(bias.toHost(), sums.astype(f32), tol=1e-5, what="column sums of the image", scale=float(np.abs(image).max()))
+    exact = expected_grad.astype(np.float64).sum(axis=0)   # the bias gradient proper: within the rounding of its terms
+    room = 2.0 ** -8 * np.abs(expected_grad).astype(np.float64).sum(axis=0) + 1e-12
+    assert (np.abs(bias.toHost() - exact) <= room).all(), "bias gradient: further from the fp32 sums than the rounding of the terms allows"
+
+
 def test_cross_entropy_head_refuses_what_it_does_not_serve(hip, rng):
     D, call = hip.DeviceTensor, hip.capi.call
-    for rows, classes in ((4, 1000), (4, 50257), (4, 40000), (4, 4100)):
+    for rows, classes in ((4, 1000), (4, 4095), (2, 53249), (2, 60000)):
         dl, di = D.fromHost(r(rng, rows, classes)), D.fromHost(np.zeros(rows, f32))
         img, bias, loss = image_of(hip, (rows, classes + 8)), D((classes,)), D.zeros((1,))
         with pytest.raises(Exception, match="not served"):
             call("bf_hip_cross_entropy_sparse_head", dl.ptr, di.ptr, img.ptr, bias.ptr, loss.ptr, rows, classes, 0, None)
+    dl, di = D.fromHost(r(rng, 4, 8192)), D.fromHost(np.zeros(4, f32))
+    img, bias, loss = image_of(hip, (4, 8200)), D((8192,)), D.zeros((1,))
+    with pytest.raises(Exception, match="not served"):   # an image that does not start on a 16-byte boundary
+        call("bf_hip_cross_entropy_sparse_head", dl.ptr, di.ptr, ctypes.c_void_p(img.ptr.value + 2), bias.ptr, loss.ptr, 4, 8192, 0, None)
 
 
 # (m, k, n): the small-tile route with transposed images, a ragged one, and the large-tile routes (fragments transposed in LDS)
