@@ -430,6 +430,71 @@ __global__ void __launch_bounds__(1024) crossEntropyImageWideKernel(const float*
     }
 }
 
+// The same for rows too long for a block's registers (more than 1024 x 52 classes: the vocabularies of 128 256, 151 936
+// or 256 000 words): the row is walked twice, the second time out of the last-level cache (a row of 256 000 floats is
+// 1 MB).  First walk: the maximum and, in the same walk, the sum of exponentials about the maximum so far (the sum is
+// rescaled whenever a thread's maximum moves; the threads' pairs are then combined about the row's maximum).  Second
+// walk: the gradient's image.  Element by element the values are those of the kernels above up to the order of the
+// additions in the sum.
+template <bool NT>
+__global__ void __launch_bounds__(1024) crossEntropyImageLongKernel(const float* __restrict__ logits, const float* __restrict__ target,
+                                                                    unsigned short* __restrict__ gradImage, float* __restrict__ rowLoss,
+                                                                    size_t rows, size_t classes, size_t pitch, float invRows) {
+    constexpr int G = 1024, VEC = 4;
+    constexpr float kLog2e = 1.4426950408889634f;
+    __shared__ float lds[16];
+    const int t = threadIdx.x;
+    const size_t whole = classes & ~size_t(3);   // elements in whole groups of four
+    for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const float* __restrict__ x = logits + row * classes;
+        // base-2 logarithms throughout: y = x * log2(e)
+        float mx = -INFINITY, sum = 0.0f;
+        auto take = [&](float v) {
+            const float y = v * kLog2e;
+            if (y > mx) { sum = sum * __builtin_amdgcn_exp2f(mx - y) + 1.0f; mx = y; }   // (0 * exp2(-inf - y) = 0 for the first element)
+            else sum += __builtin_amdgcn_exp2f(y - mx);
+        };
+        for (size_t e = size_t(t) * VEC; e < whole; e += size_t(G) * VEC) {
+            const float4u v = *reinterpret_cast<const float4u*>(x + e);   // stays in the cache for the second walk
+            take(v.x); take(v.y); take(v.z); take(v.w);
+        }
+        if (t < int(classes - whole)) take(x[whole + t]);
+        const float rowMax = groupMax<G>(mx, lds);
+        sum = mx > -INFINITY ? sum * __builtin_amdgcn_exp2f(mx - rowMax) : 0.0f;
+        sum = groupSum<G>(sum, lds);
+        const float inv = 1.0f / sum, scale = inv * invRows;
+        const size_t cls = size_t(lroundf(target[row]));
+        float pTarget = -1.0f;
+        unsigned short* __restrict__ out = gradImage + row * pitch;
+        for (size_t e = size_t(t) * VEC; e < pitch; e += size_t(G) * VEC) {
+            float g[VEC];
+            if (e + VEC <= classes) {
+                float4u v;
+                if constexpr (NT) v = __builtin_nontemporal_load(reinterpret_cast<const float4u*>(x + e));
+                else v = *reinterpret_cast<const float4u*>(x + e);
+                g[0] = v.x; g[1] = v.y; g[2] = v.z; g[3] = v.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) g[j] = e + j < classes ? x[e + j] : -INFINITY;
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(g[j], kLog2e, -rowMax));
+                const bool hit = e + j == cls;
+                const float p = ex * inv;
+                pTarget = hit ? p : pTarget;
+                g[j] = hit ? (p - 1.0f) * invRows : ex * scale;
+            }
+            const uint2v packed = {unsigned(toBf16Bits(g[0])) | unsigned(toBf16Bits(g[1])) << 16,
+                                   unsigned(toBf16Bits(g[2])) | unsigned(toBf16Bits(g[3])) << 16};
+            stu2<NT>(out + e, packed);
+        }
+        float loss = pTarget >= 0.0f ? -logf(fmaxf(pTarget, 1e-12f)) : 0.0f;
+        loss = groupSum<G>(loss, lds);
+        if (t == 0) rowLoss[row] = loss;
+    }
+}
+
 // partial[band * pitch + c] = sum of image[row * pitch + c] over the rows of band `blockIdx.y` (rowsPerBand each), in row
 // order: a thread owns eight columns (16 bytes of a row) and keeps four rows' loads in flight.
 __global__ void __launch_bounds__(kBlock) columnSumBf16Kernel(const unsigned short* __restrict__ image, float* __restrict__ partial,
@@ -597,23 +662,28 @@ int bf_hip_cross_entropy_sparse_head(const float* logits, const float* targetIdx
                                      size_t rows, size_t classes, int accumulate, bf_stream_t stream) {
     BF_REQUIRE(lossSum != nullptr, "lossSum is NULL");
     // the rows a 1024-thread block can hold in its registers, with a 16-byte aligned bf16 image
-    if (rows == 0 || classes < 4096 || classes > size_t(1024) * 52 || !aligned16(gradImage)) {
+    if (rows == 0 || classes < 4096 || classes > (size_t(1) << 20) || !aligned16(gradImage)) {
         setLastError("bf_hip_cross_entropy_sparse_head: shape or alignment not served by the fused form (use bf_hip_cross_entropy_sparse_img and bf_hip_bias_grad)");
         return BF_ERR_UNSUPPORTED;
     }
     BF_REQUIRE(logits && targetIdx && gradImage && biasGrad, "NULL pointer");
     hipStream_t s = asStream(stream);
     if (classes % 8 != 0 || classes > size_t(1024) * 32 || !aligned16(logits) || !aligned16(biasGrad)) {
-        // rows of any length up to 1024 x 52 and any alignment: the loss with the image alone, then the image's column sums
+        // rows of any length (up to 2^20 classes) and any alignment: the loss with the image alone, then the image's column sums
         const size_t pitch = (classes + 7) / 8 * 8;
         const float invRows = 1.0f / float(rows);
         const unsigned grid = unsigned(std::min<size_t>(rows, kMaxGridX));
         Scratch rowLoss(rows * sizeof(float));
         if (rowLoss.status != BF_OK) return rowLoss.status;
-        if (streamsPastCache(rows * classes * 6))
+        const bool streaming = streamsPastCache(rows * classes * 6);
+        if (classes > size_t(1024) * 52) {   // rows that a block's registers do not hold: two walks over each row
+            if (streaming) crossEntropyImageLongKernel<true><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), rows, classes, pitch, invRows);
+            else crossEntropyImageLongKernel<false><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), rows, classes, pitch, invRows);
+        } else if (streaming) {
             crossEntropyImageWideKernel<true><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), rows, classes, pitch, invRows);
-        else
+        } else {
             crossEntropyImageWideKernel<false><<<grid, 1024, 0, s>>>(logits, targetIdx, gradImage, rowLoss.as<float>(), rows, classes, pitch, invRows);
+        }
         BF_LAUNCH_CHECK();
         // bands of rows so that the grid has a few thousand workgroups
         const size_t columnBlocks = (pitch / 8 + kBlock - 1) / kBlock;

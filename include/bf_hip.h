@@ -484,11 +484,11 @@ int bf_hip_cross_entropy_sparse_img(const float* logits, const float* targetIdx,
  * the bias gradient, and no fp32 gradient is written.  16-byte aligned tensors with classes a multiple of 8 between
  * 4096 and 32768 take one pass: same loss and same image as bf_hip_cross_entropy_sparse_img, the column sums taken in fp32
  * before the rounding, added in another (fixed) order than bf_hip_bias_grad adds them.  Other class counts from 4096 to
- * 53248 (an odd vocabulary such as 50257: rows on any 4-byte boundary) and unaligned logits take two: the loss with the
- * image (an element may differ from the other kernels' image by one bf16 step: the row sums add in another order), then
- * the image's column sums, i.e. the bias gradient of the rounded gradient values that the head's products use.  Anything
- * else (fewer than 4096 or more than 53248 classes, an image that is not 16-byte aligned) returns BF_ERR_UNSUPPORTED and
- * launches nothing. */
+ * 2^20 (an odd vocabulary such as 50257: rows on any 4-byte boundary; 128256 or 256000 words: rows walked twice, the
+ * second time out of the cache) and unaligned logits take two: the loss with the image (an element may differ from the
+ * other kernels' image by one bf16 step: the row sums add in another order), then the image's column sums, i.e. the
+ * bias gradient of the rounded gradient values that the head's products use.  Anything else (fewer than 4096 or more
+ * than 2^20 classes, an image that is not 16-byte aligned) returns BF_ERR_UNSUPPORTED and launches nothing. */
 int bf_hip_cross_entropy_sparse_head(const float* logits, const float* targetIdx, uint16_t* gradImage, float* biasGrad, float* lossSum,
                                      size_t rows, size_t classes, int accumulate, bf_stream_t stream);
 /* softmaxCrossEntropyMasked (the CPU backend's loss for masked-language-model training, src/backend/cpu/loss.cpp:149-215;

@@ -132,7 +132,7 @@ inline bool softmaxCrossEntropySparseHeadAccumulate(const DeviceTensor& logits, 
                                                     DeviceTensor& gradImageOnly, DeviceTensor& biasGrad) {
     detail::requireSparse("softmaxCrossEntropySparseAccumulate", logits, targetIndices);
     const std::size_t rows = detail::rowsOf(logits), classes = detail::lastDim(logits);
-    if (rows == 0 || classes < 4096 || classes > 53248) return false;   // what the library serves (it says so itself otherwise)
+    if (rows == 0 || classes < 4096 || classes > (std::size_t(1) << 20)) return false;   // what the library serves (it says so itself otherwise)
     DeviceTensor grad = DeviceTensor::imageOnly(logits.shape());
     DeviceTensor bias({classes});
     const int status = bf_hip_cross_entropy_sparse_head(logits.data(), targetIndices.data(), const_cast<std::uint16_t*>(grad.image()), bias.data(),

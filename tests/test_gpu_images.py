@@ -144,10 +144,12 @@ def test_cross_entropy_of_a_language_model_head(hip, oracle, rng, rows, classes)
 
 
 @pytest.mark.parametrize("rows,classes,offset", [(3, 50257, 0), (300, 50257, 0), (5, 40000, 0), (64, 4099, 0), (130, 53248, 0), (7, 4100, 0),
-                                                 (33, 8192, 1), (2, 53241, 3)])
+                                                 (33, 8192, 1), (2, 53241, 3),
+                                                 # rows longer than a block's registers: walked twice
+                                                 (3, 53249, 0), (40, 128256, 0), (2, 151937, 1), (1, 256000, 0)])
 def test_cross_entropy_of_a_head_with_an_odd_or_large_vocabulary(hip, oracle, rng, rows, classes, offset):
     """bf_hip_cross_entropy_sparse_head beyond its one-pass form (class counts that are not multiples of 8, more than
-    32768 classes, logits that do not start on a 16-byte boundary): the loss, the gradient image in rows of classes
+    32768 classes up to vocabularies of 256000 words, logits that do not start on a 16-byte boundary): the loss, the gradient image in rows of classes
     rounded up to 8 (the padding zero), within one bf16 step of the rounded fp32 gradient of bf_hip_cross_entropy_sparse,
     and as bias gradient the column sums of that image."""
     D, call = hip.DeviceTensor, hip.capi.call
@@ -179,7 +181,7 @@ def test_cross_entropy_of_a_head_with_an_odd_or_large_vocabulary(hip, oracle, rn
 
 def test_cross_entropy_head_refuses_what_it_does_not_serve(hip, rng):
     D, call = hip.DeviceTensor, hip.capi.call
-    for rows, classes in ((4, 1000), (4, 4095), (2, 53249), (2, 60000)):
+    for rows, classes in ((4, 1000), (4, 4095), (1, (1 << 20) + 8)):
         dl, di = D.fromHost(r(rng, rows, classes)), D.fromHost(np.zeros(rows, f32))
         img, bias, loss = image_of(hip, (rows, classes + 8)), D((classes,)), D.zeros((1,))
         with pytest.raises(Exception, match="not served"):
