@@ -86,6 +86,18 @@ __global__ void __launch_bounds__(kBlock) mseKernel(const float* __restrict__ pr
     if (threadIdx.x == 0) partial[blockIdx.x] = acc;
 }
 
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));   // a float4 that may start on any 4-byte boundary
+
+// The elements of a row that is not held in registers, for thread t of the G that share it: whole groups of four as one
+// 16-byte access from whatever 4-byte boundary the row starts on (global memory serves those), then the last one to
+// three elements one by one.
+template <int G, typename Four, typename One>
+__device__ __forceinline__ void forRowElements(size_t classes, int t, Four four, One one) {
+    const size_t whole = classes & ~size_t(3);
+    for (size_t e = size_t(t) * 4; e < whole; e += size_t(G) * 4) four(e);
+    for (size_t e = whole + t; e < classes; e += G) one(e);
+}
+
 // SPARSE: target holds one class index per row.  Otherwise a dense target row.
 // SHIFTED (with VEC = 4, CACHED): rows of any length and alignment through 16-byte accesses (RowCache::loadShifted).
 // AHEAD (CACHED only): a grid that fills the chip walks the rows, each block with its next row's loads in flight
@@ -144,7 +156,12 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                     for (int i = 0; i < MAXE; ++i) c.r[i] = 0.0f;
                     storeRow();
                 } else {
-                    for (size_t e = t; e < classes; e += G) { gOut[e] = 0.0f; if (gImg) gImg[e] = 0; }
+                    forRowElements<G>(classes, t,
+                                      [&](size_t e) {
+                                          *reinterpret_cast<float4u*>(gOut + e) = float4u{0.0f, 0.0f, 0.0f, 0.0f};
+                                          if (gImg) *reinterpret_cast<uint2v*>(gImg + e) = uint2v{0u, 0u};
+                                      },
+                                      [&](size_t e) { gOut[e] = 0.0f; if (gImg) gImg[e] = 0; });
                 }
                 if (t == 0) rowLoss[row] = 0.0f;
                 continue;
@@ -155,7 +172,12 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
 #pragma unroll
             for (int i = 0; i < MAXE; ++i) mx = fmaxf(mx, c.r[i]);
         } else {
-            for (size_t e = t; e < classes; e += G) mx = fmaxf(mx, x[e]);
+            forRowElements<G>(classes, t,
+                              [&](size_t e) {
+                                  const float4u v = *reinterpret_cast<const float4u*>(x + e);
+                                  mx = fmaxf(fmaxf(mx, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+                              },
+                              [&](size_t e) { mx = fmaxf(mx, x[e]); });
         }
         mx = groupMax<G>(mx, lds);
         // exp(x - mx) as one hardware exp2 of (x - mx) * log2(e): the argument is <= 0 and the result feeds
@@ -167,7 +189,15 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
 #pragma unroll
             for (int i = 0; i < MAXE; ++i) { c.r[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(c.r[i], kLog2e, -top)); sum += c.r[i]; }
         } else {
-            for (size_t e = t; e < classes; e += G) sum += __builtin_amdgcn_exp2f((x[e] - mx) * kLog2e);
+            forRowElements<G>(classes, t,
+                              [&](size_t e) {
+                                  const float4u v = *reinterpret_cast<const float4u*>(x + e);
+                                  sum += __builtin_amdgcn_exp2f((v.x - mx) * kLog2e);
+                                  sum += __builtin_amdgcn_exp2f((v.y - mx) * kLog2e);
+                                  sum += __builtin_amdgcn_exp2f((v.z - mx) * kLog2e);
+                                  sum += __builtin_amdgcn_exp2f((v.w - mx) * kLog2e);
+                              },
+                              [&](size_t e) { sum += __builtin_amdgcn_exp2f((x[e] - mx) * kLog2e); });
         }
         sum = groupSum<G>(sum, lds);
         const float inv = 1.0f / sum;
@@ -203,14 +233,26 @@ __global__ void __launch_bounds__(G > 256 ? G : 256) crossEntropyKernel(const fl
                 }
                 storeRow();
             } else {
-                for (size_t e = t; e < classes; e += G) {
-                    const float p = __builtin_amdgcn_exp2f((x[e] - mx) * kLog2e) * inv;
+                auto element = [&](float xe, size_t e) -> float {
+                    const float p = __builtin_amdgcn_exp2f((xe - mx) * kLog2e) * inv;
                     const bool hit = e == cls;
                     pTarget = hit ? p : pTarget;
-                    const float gv = (p - (hit ? 1.0f : 0.0f)) * invRows;
-                    gOut[e] = gv;
-                    if (gImg) gImg[e] = toBf16Bits(gv);
-                }
+                    return (p - (hit ? 1.0f : 0.0f)) * invRows;
+                };
+                forRowElements<G>(classes, t,
+                                  [&](size_t e) {
+                                      const float4u v = *reinterpret_cast<const float4u*>(x + e);
+                                      const float4u gv = {element(v.x, e), element(v.y, e + 1), element(v.z, e + 2), element(v.w, e + 3)};
+                                      *reinterpret_cast<float4u*>(gOut + e) = gv;
+                                      if (gImg)   // (aligned rows of a multiple of 8 classes only: an 8-byte group)
+                                          *reinterpret_cast<uint2v*>(gImg + e) = uint2v{unsigned(toBf16Bits(gv.x)) | unsigned(toBf16Bits(gv.y)) << 16,
+                                                                                        unsigned(toBf16Bits(gv.z)) | unsigned(toBf16Bits(gv.w)) << 16};
+                                  },
+                                  [&](size_t e) {
+                                      const float gv = element(x[e], e);
+                                      gOut[e] = gv;
+                                      if (gImg) gImg[e] = toBf16Bits(gv);
+                                  });
             }
             if (pTarget >= 0.0f) loss = -logf(fmaxf(pTarget, 1e-12f));
         } else {
@@ -346,7 +388,6 @@ __global__ void __launch_bounds__(kBlock) columnPartialsFinishKernel(const float
 // thread, read with 16-byte loads from whatever boundary the row starts on (global memory serves those), the gradient
 // written as its bf16 image only; same arithmetic per element as crossEntropyKernel.  The bias gradient is then the
 // column sums of that image (columnSumBf16Kernel): the sum of the gradient values as the head's products see them.
-typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));   // a float4 that may start on any 4-byte boundary
 template <bool NT>
 __global__ void __launch_bounds__(1024) crossEntropyImageWideKernel(const float* __restrict__ logits, const float* __restrict__ target,
                                                                     unsigned short* __restrict__ gradImage, float* __restrict__ rowLoss,
