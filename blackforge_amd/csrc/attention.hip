@@ -63,7 +63,29 @@ struct AttnParams {
     int batch, heads, newLen, totalLen, dim, hd, oldLen;
     float scale;
     int numTiles;        // query tiles (forward, dQ) or key tiles (dK/dV) per (batch, head)
+    // Forward pass over the keys in chunks (few queries, many keys: one step of incremental decoding): workgroup row
+    // blockIdx.y takes keys [y * chunkKeys, ...), the last chunk everything that is left, and writes its normalised
+    // output and its statistics `partOutStride` / `partStatStride` floats after the chunk before it (applyKeyChunk);
+    // attnCombineChunksKernel puts the chunks together.  numChunks <= 1: the whole key range, as everywhere else.
+    int kvRows;          // rows per batch element of the K and V tensors (totalLen, whatever the chunk)
+    int chunkKeys, numChunks;
+    size_t partOutStride, partStatStride;
 };
+
+// A forward kernel's first statement: narrows the parameters to this workgroup's chunk of keys.  Every chunk starts at
+// or before the first query's own position (the host sees to that), so every query sees a key in every chunk.
+__device__ __forceinline__ void applyKeyChunk(AttnParams& p) {
+    if (p.numChunks <= 1) return;
+    const int c = blockIdx.y, c0 = c * p.chunkKeys;
+    const size_t skip = size_t(c0) * p.dim;
+    p.k += skip;
+    p.v += skip;
+    p.totalLen = c == p.numChunks - 1 ? p.totalLen - c0 : p.chunkKeys;
+    p.oldLen -= c0;
+    p.out += size_t(c) * p.partOutStride;
+    p.m += size_t(c) * p.partStatStride;
+    p.l += size_t(c) * p.partStatStride;
+}
 
 __device__ __forceinline__ float fastExp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -347,6 +369,7 @@ typedef __attribute__((address_space(3))) void* LdsPtr;
 //   and guarantees every wave is done reading buffer t&1 before iteration t+1 overwrites it with tile t+2.
 template <int HDP, int BC, bool VEC4>
 __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnForwardKernel(AttnParams p) {
+    applyKeyChunk(p);
     constexpr int LDSW = HDP + 4, DT = HDP / 32, TILE = BC * LDSW;
     extern __shared__ float smem[];
     float* ks = smem;               // [2][BC][LDSW]
@@ -358,8 +381,8 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnForwardKernel(Att
     const int b = bh / p.heads, h = bh - b * p.heads;
     const int hd = p.hd, dim = p.dim;
     const float* qb = p.q + size_t(b) * p.newLen * dim + size_t(h) * hd;
-    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
-    const float* vb = p.v + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const float* kb = p.k + size_t(b) * p.kvRows * dim + size_t(h) * hd;
+    const float* vb = p.v + size_t(b) * p.kvRows * dim + size_t(h) * hd;
 
     const int waveQ0 = qt * 128 + wave * 32;
     const int i = waveQ0 + li;                    // this lane's query row
@@ -2236,6 +2259,7 @@ __device__ __forceinline__ void forwardPipedStep(const unsigned short* __restric
 
 template <int HDP, bool VEC4>
 __global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnForwardPipedKernel(AttnParams p) {
+    applyKeyChunk(p);
     constexpr int BC = 32, KP = splitKeyPitch(HDP), VP = splitValuePitch(HDP), KTILE = 3 * BC * KP, VTILE = 3 * BC * VP, DT = HDP / 32, KS = HDP / 16;
     extern __shared__ __attribute__((aligned(16))) unsigned short smemSplit[];
     unsigned short* ks = smemSplit;               // [2][3][BC][KP]
@@ -2247,8 +2271,8 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnForwardPipedKernel
     const int b = bh / p.heads, h = bh - b * p.heads;
     const int hd = p.hd, dim = p.dim;
     const float* qb = p.q + size_t(b) * p.newLen * dim + size_t(h) * hd;
-    const float* kb = p.k + size_t(b) * p.totalLen * dim + size_t(h) * hd;
-    const float* vb = p.v + size_t(b) * p.totalLen * dim + size_t(h) * hd;
+    const float* kb = p.k + size_t(b) * p.kvRows * dim + size_t(h) * hd;
+    const float* vb = p.v + size_t(b) * p.kvRows * dim + size_t(h) * hd;
 
     const int waveQ0 = qt * 128 + wave * 32;
     const int i = waveQ0 + li;                    // this lane's query row
@@ -2329,9 +2353,42 @@ template <typename K>
 int launchAttn(K kernel, size_t smemBytes, unsigned grid, const AttnParams& p, hipStream_t s) {
     int st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smemBytes);
     if (st != BF_OK) return st;
-    kernel<<<grid, 256, smemBytes, s>>>(p);
+    kernel<<<dim3(grid, unsigned(p.numChunks > 1 ? p.numChunks : 1)), 256, smemBytes, s>>>(p);
     BF_LAUNCH_CHECK();
     return BF_OK;
+}
+
+// The chunks of a forward pass over the keys in chunks, put together: with chunk c's row maximum m_c, sum l_c of
+// exp(score - m_c) and normalised output O_c, the row's maximum is M = max m_c, its sum L = sum_c l_c exp(m_c - M), and
+// its output sum_c (l_c exp(m_c - M) / L) O_c, the chunks added in order.  One wavefront per (batch, query, head).
+__global__ void __launch_bounds__(256) attnCombineChunksKernel(const float* __restrict__ partOut, const float* __restrict__ partM,
+                                                               const float* __restrict__ partL, float* __restrict__ out,
+                                                               unsigned short* __restrict__ outImg, size_t imgLd, float* __restrict__ m,
+                                                               float* __restrict__ l, int batch, int heads, int newLen, int dim, int hd,
+                                                               int numChunks, size_t partOutStride, size_t partStatStride) {
+    const int lane = threadIdx.x & 63;
+    const size_t group = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6);   // (b, i, h), h fastest
+    if (group >= size_t(batch) * newLen * heads) return;
+    const int h = int(group % heads);
+    const size_t bi = group / heads;                                    // b * newLen + i
+    const size_t b = bi / newLen, i = bi - b * newLen;
+    const size_t stat = (b * heads + h) * newLen + i;
+    float rowMax = -INFINITY;
+    for (int c = 0; c < numChunks; ++c) rowMax = fmaxf(rowMax, partM[c * partStatStride + stat]);
+    float total = 0.0f;
+    for (int c = 0; c < numChunks; ++c) total += partL[c * partStatStride + stat] * expf(partM[c * partStatStride + stat] - rowMax);
+    const float inv = 1.0f / total;
+    const size_t at = bi * dim + size_t(h) * hd;
+    for (int d = lane; d < hd; d += 64) {
+        float acc = 0.0f;
+        for (int c = 0; c < numChunks; ++c) {
+            const float w = partL[c * partStatStride + stat] * expf(partM[c * partStatStride + stat] - rowMax) * inv;
+            acc += w * partOut[c * partOutStride + at + d];
+        }
+        if (out) out[at + d] = acc;
+        if (outImg) outImg[bi * imgLd + size_t(h) * hd + d] = toBf16Bits(acc);
+    }
+    if (lane == 0) { m[stat] = rowMax; l[stat] = total; }
 }
 
 bool vec4Ok(const AttnParams& p, std::initializer_list<const void*> ptrs) {
@@ -2474,8 +2531,42 @@ int bf_hip_attention_forward_img(const float* q, const float* k, const float* v,
     p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(totalLen);
     p.dim = int(dim); p.hd = int(dim / heads); p.oldLen = int(oldLen); p.scale = scale;
     p.numTiles = int((newLen + 127) / 128);
+    p.kvRows = p.totalLen;
     unsigned grid = unsigned(batch * heads * size_t(p.numTiles));
-    return dispatch<0>(p, vec4Ok(p, {q, k, v, out}), grid, asStream(stream));
+    hipStream_t s = asStream(stream);
+    // Few queries against many keys (a step of incremental decoding: one workgroup per head would walk all the keys alone):
+    // the keys go to the workgroups in chunks, each with its own statistics, and a second kernel puts the chunks together.
+    // A chunk must start at or before the first query's own position, so that every query sees a key in every chunk: the
+    // last chunk takes everything from the last such start.
+    const size_t cus = size_t(computeUnits());
+    if (size_t(grid) * 2 <= cus && totalLen >= 1024) {
+        const size_t wanted = (4 * cus + grid - 1) / grid;   // about four workgroups per compute unit
+        size_t chunkKeys = ((totalLen + wanted - 1) / wanted + 127) / 128 * 128;
+        if (chunkKeys < 128) chunkKeys = 128;
+        const size_t numChunks = std::min((totalLen + chunkKeys - 1) / chunkKeys, oldLen / chunkKeys + 1);
+        if (numChunks > 1) {
+            const size_t outFloats = batch * newLen * dim, statFloats = batch * heads * newLen;
+            Scratch part(numChunks * (outFloats + 2 * statFloats) * sizeof(float));
+            if (part.status != BF_OK) return part.status;
+            AttnParams c = p;
+            c.chunkKeys = int(chunkKeys);
+            c.numChunks = int(numChunks);
+            c.partOutStride = outFloats;
+            c.partStatStride = statFloats;
+            c.out = part.as<float>();
+            c.m = c.out + numChunks * outFloats;
+            c.l = c.m + numChunks * statFloats;
+            c.outImg = nullptr;
+            st = dispatch<0>(c, vec4Ok(c, {q, k, v, c.out}), grid, s);
+            if (st != BF_OK) return st;
+            const size_t groups = batch * newLen * heads;
+            attnCombineChunksKernel<<<unsigned((groups + 3) / 4), 256, 0, s>>>(c.out, c.m, c.l, out, outImage, imageLd, m, l, int(batch), int(heads),
+                                                                            int(newLen), int(dim), p.hd, int(numChunks), outFloats, statFloats);
+            BF_LAUNCH_CHECK();
+            return BF_OK;
+        }
+    }
+    return dispatch<0>(p, vec4Ok(p, {q, k, v, out}), grid, s);
 }
 
 int bf_hip_attention_forward(const float* q, const float* k, const float* v, float* out, float* m, float* l,

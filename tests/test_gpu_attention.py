@@ -45,7 +45,11 @@ CASES = [(1, 1, 1, 0, 2), (1, 2, 3, 0, 2), (2, 2, 5, 0, 4), (2, 3, 33, 0, 32), (
          (2, 2, 300, 0, 192), (1, 2, 260, 40, 256), (1, 1, 129, 129, 136), (1, 1, 140, 0, 130),
          # the 256-wide padding class on rows that are not 16-byte aligned (tiles staged through registers), and the
          # widest head that is padded to 192
-         (1, 2, 140, 20, 250), (2, 1, 200, 0, 224), (1, 3, 170, 0, 192)]
+         (1, 2, 140, 20, 250), (2, 1, 200, 0, 224), (1, 3, 170, 0, 192),
+         # a few queries against a long cache (a step of incremental decoding): the forward pass takes the keys in chunks
+         # and puts the chunks together (chunk ends inside and outside the new tokens, every head-dim class, ragged ends)
+         (1, 2, 1, 2047, 64), (2, 3, 5, 3000, 32), (1, 1, 1, 4500, 128), (1, 2, 16, 1500, 256), (1, 2, 3, 1100, 100), (1, 1, 130, 1024, 64),
+         (1, 1, 1, 1023, 192)]
 
 
 @pytest.mark.parametrize("batch,heads,new_len,old_len,hd", CASES)
