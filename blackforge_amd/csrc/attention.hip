@@ -2360,35 +2360,63 @@ int launchAttn(K kernel, size_t smemBytes, unsigned grid, const AttnParams& p, h
 
 // The chunks of a forward pass over the keys in chunks, put together: with chunk c's row maximum m_c, sum l_c of
 // exp(score - m_c) and normalised output O_c, the row's maximum is M = max m_c, its sum L = sum_c l_c exp(m_c - M), and
-// its output sum_c (l_c exp(m_c - M) / L) O_c, the chunks added in order.  One wavefront per (batch, query, head).
+// its output sum_c (l_c exp(m_c - M) / L) O_c.  One workgroup per (batch, query, head): the threads read the chunks'
+// statistics side by side, and each of the four wavefronts adds every fourth chunk's output (head dims up to 256: four
+// columns a lane), the four sums joined in wavefront order.
 __global__ void __launch_bounds__(256) attnCombineChunksKernel(const float* __restrict__ partOut, const float* __restrict__ partM,
                                                                const float* __restrict__ partL, float* __restrict__ out,
                                                                unsigned short* __restrict__ outImg, size_t imgLd, float* __restrict__ m,
-                                                               float* __restrict__ l, int batch, int heads, int newLen, int dim, int hd,
-                                                               int numChunks, size_t partOutStride, size_t partStatStride) {
-    const int lane = threadIdx.x & 63;
-    const size_t group = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6);   // (b, i, h), h fastest
-    if (group >= size_t(batch) * newLen * heads) return;
+                                                               float* __restrict__ l, int heads, int newLen, int dim, int hd, int numChunks,
+                                                               size_t partOutStride, size_t partStatStride) {
+    __shared__ float sReduce[4];
+    __shared__ float sWeight[256];
+    __shared__ float sAcc[4][256];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const size_t group = blockIdx.x;                                    // (b, i, h), h fastest
     const int h = int(group % heads);
     const size_t bi = group / heads;                                    // b * newLen + i
     const size_t b = bi / newLen, i = bi - b * newLen;
     const size_t stat = (b * heads + h) * newLen + i;
+
     float rowMax = -INFINITY;
-    for (int c = 0; c < numChunks; ++c) rowMax = fmaxf(rowMax, partM[c * partStatStride + stat]);
+    for (int c = t; c < numChunks; c += 256) rowMax = fmaxf(rowMax, partM[c * partStatStride + stat]);
+    for (int o = 32; o > 0; o >>= 1) rowMax = fmaxf(rowMax, __shfl_xor(rowMax, o, 64));
+    if (lane == 0) sReduce[wave] = rowMax;
+    __syncthreads();
+    rowMax = fmaxf(fmaxf(sReduce[0], sReduce[1]), fmaxf(sReduce[2], sReduce[3]));
+    __syncthreads();
     float total = 0.0f;
-    for (int c = 0; c < numChunks; ++c) total += partL[c * partStatStride + stat] * expf(partM[c * partStatStride + stat] - rowMax);
-    const float inv = 1.0f / total;
+    for (int c = t; c < numChunks; c += 256) total += partL[c * partStatStride + stat] * expf(partM[c * partStatStride + stat] - rowMax);
+    for (int o = 32; o > 0; o >>= 1) total += __shfl_xor(total, o, 64);
+    if (lane == 0) sReduce[wave] = total;
+    __syncthreads();
+    total = (sReduce[0] + sReduce[1]) + (sReduce[2] + sReduce[3]);
+
     const size_t at = bi * dim + size_t(h) * hd;
-    for (int d = lane; d < hd; d += 64) {
-        float acc = 0.0f;
-        for (int c = 0; c < numChunks; ++c) {
-            const float w = partL[c * partStatStride + stat] * expf(partM[c * partStatStride + stat] - rowMax) * inv;
-            acc += w * partOut[c * partOutStride + at + d];
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c0 = 0; c0 < numChunks; c0 += 256) {
+        __syncthreads();                                                // the previous round's weights have been read
+        if (c0 + t < numChunks) sWeight[t] = partL[(c0 + t) * partStatStride + stat] * expf(partM[(c0 + t) * partStatStride + stat] - rowMax);
+        __syncthreads();
+        const int count = min(256, numChunks - c0);
+#pragma unroll 4
+        for (int c = wave; c < count; c += 4) {
+            const float w = sWeight[c];
+            const float* src = partOut + (c0 + c) * partOutStride + at;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (lane + 64 * j < hd) acc[j] += w * src[lane + 64 * j];
         }
-        if (out) out[at + d] = acc;
-        if (outImg) outImg[bi * imgLd + size_t(h) * hd + d] = toBf16Bits(acc);
     }
-    if (lane == 0) { m[stat] = rowMax; l[stat] = total; }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sAcc[wave][lane + 64 * j] = acc[j];
+    __syncthreads();
+    if (t < hd) {
+        const float value = ((sAcc[0][t] + sAcc[1][t]) + (sAcc[2][t] + sAcc[3][t])) / total;
+        if (out) out[at + t] = value;
+        if (outImg) outImg[bi * imgLd + size_t(h) * hd + t] = toBf16Bits(value);
+    }
+    if (t == 0) { m[stat] = rowMax; l[stat] = total; }
 }
 
 bool vec4Ok(const AttnParams& p, std::initializer_list<const void*> ptrs) {
@@ -2560,8 +2588,8 @@ int bf_hip_attention_forward_img(const float* q, const float* k, const float* v,
             st = dispatch<0>(c, vec4Ok(c, {q, k, v, c.out}), grid, s);
             if (st != BF_OK) return st;
             const size_t groups = batch * newLen * heads;
-            attnCombineChunksKernel<<<unsigned((groups + 3) / 4), 256, 0, s>>>(c.out, c.m, c.l, out, outImage, imageLd, m, l, int(batch), int(heads),
-                                                                            int(newLen), int(dim), p.hd, int(numChunks), outFloats, statFloats);
+            attnCombineChunksKernel<<<unsigned(groups), 256, 0, s>>>(c.out, c.m, c.l, out, outImage, imageLd, m, l, int(heads), int(newLen), int(dim),
+                                                                  p.hd, int(numChunks), outFloats, statFloats);
             BF_LAUNCH_CHECK();
             return BF_OK;
         }

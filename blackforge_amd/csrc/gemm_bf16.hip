@@ -1152,6 +1152,76 @@ __global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restr
     }
 }
 
+// Products of at most eight rows (a step of incremental decoding: one new token per sequence).  A 128 x 128 tile would
+// be all padding and six workgroups would walk a 768-wide weight alone; here the product is what it is by nature, a walk
+// over the weights: a wavefront owns COLS output columns (rows of Bt), each lane takes 16 bytes (eight bf16) of every
+// column per step and multiplies them with the same eight elements of the MR rows of A (which every wavefront reads: they
+// stay in cache), the lanes' sums are added by a butterfly, and lane r * COLS + j stores element (r, n0 + j) through the
+// epilogue.  Products in fp32 of the bf16 values, as on the MFMA; the order of additions is fixed (even and odd elements
+// of a lane's eight apart, then the butterfly), so results repeat bit for bit.  K, lda and ldb multiples of 8, operands
+// 16-byte aligned.
+__device__ __forceinline__ void dot8(const uint4v& a, const uint4v& b, float& even, float& odd) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        even = fmaf(__uint_as_float(a[i] << 16), __uint_as_float(b[i] << 16), even);
+        odd = fmaf(__uint_as_float(a[i] & 0xffff0000u), __uint_as_float(b[i] & 0xffff0000u), odd);
+    }
+}
+template <int MR, int COLS>
+__global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
+                                                             Epilogue e, int M, int N, int K, int lda, int ldb) {
+    const int lane = threadIdx.x & 63;
+    const int n0 = (int(blockIdx.x) * 4 + int(threadIdx.x >> 6)) * COLS;
+    if (n0 >= N) return;                                     // whole wavefronts, no barrier below
+    float even[MR][COLS], odd[MR][COLS];
+#pragma unroll
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) even[r][j] = odd[r][j] = 0.0f;
+    const unsigned short* bRow[COLS];
+#pragma unroll
+    for (int j = 0; j < COLS; ++j) bRow[j] = Bt + size_t(min(n0 + j, N - 1)) * ldb;   // a column past the end repeats the last one, unstored
+#pragma unroll 2
+    for (int k = lane * 8; k < K; k += 512) {
+        uint4v b[COLS];
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) b[j] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(bRow[j] + k));
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+            if (r < M) {
+                const uint4v a = *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k);
+#pragma unroll
+                for (int j = 0; j < COLS; ++j) dot8(a, b[j], even[r][j], odd[r][j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) {
+            float v = even[r][j] + odd[r][j];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            const int col = n0 + j;
+            if (lane == r * COLS + j && r < M && col < N) {
+                const int which = col / e.splitN;
+                float* C = which == 0 ? e.c[0] : which == 1 ? e.c[1] : e.c[2];
+                if (e.bias) v += e.bias[col];
+                if (e.residual) v += e.residual[size_t(r) * N + col];
+                C[size_t(r) * e.splitN + (col - which * e.splitN)] = v;
+            }
+        }
+}
+template <int MR>
+int launchFewRows(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K, size_t lda, size_t ldb,
+                  hipStream_t s) {
+    // one column a wavefront until that gives every SIMD several wavefronts; four from there on (fewer butterflies per byte)
+    if (N <= 8192) gemmBf16FewRowsKernel<MR, 1><<<unsigned((N + 3) / 4), 256, 0, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb));
+    else gemmBf16FewRowsKernel<MR, 4><<<unsigned((N + 15) / 16), 256, 0, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb));
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
 // The same kernel for operands that lie the other way round: C[M,N] = A^T * B with A [K, lda] and B [K, ldb], the
 // contraction index K running over ROWS (a weight gradient dW = X^T * G: both the activations X and the gradient G have
 // one row per token).  A K step is 64 rows of either operand, staged in LDS as they lie in memory ([k][m], rows padded
@@ -1591,6 +1661,12 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
             if (size_t(epi.splitN) != N && epi.splitN % 192 != 0) return failInvalid("gemm_bf16", "192-wide tiles need outputs whose width is a multiple of 192");
             return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s, g_ntRoute == BF_GEMM_ROUTE_WIDE_192_PERSISTENT);
         default: break;
+    }
+    if (M <= 8 && epi.fuse == 0 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
+        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) & 15u) == 0) {   // a walk over the weights, no tiles
+        if (M == 0 || N == 0) return BF_OK;
+        return M == 1 ? launchFewRows<1>(A, Bt, epi, M, N, K, lda, ldb, s) : M == 2 ? launchFewRows<2>(A, Bt, epi, M, N, K, lda, ldb, s)
+             : M <= 4 ? launchFewRows<4>(A, Bt, epi, M, N, K, lda, ldb, s) : launchFewRows<8>(A, Bt, epi, M, N, K, lda, ldb, s);
     }
     // 256x256 ping-pong tiles once they give three quarters of the CUs a tile; otherwise 128x128 tiles,
     // with K cut into slices when even those leave CUs idle and K is long enough to share out.

@@ -433,6 +433,8 @@ int bfh_model_forward_incremental(void* h, const float* input, int rank, const s
     Handle* handle = static_cast<Handle*>(h);
     return guarded([&] {
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
+        if (!handle->weightImagesCurrent) hip::invalidateBf16WeightCache();   // weights set or trained since the images were made
+        handle->weightImagesCurrent = true;
         handle->output = handle->model->forwardIncremental(in.tensor);
         if (output) *output = handle->output.data();
         if (outCount) *outCount = handle->output.elementCount();

@@ -188,7 +188,11 @@ public:
 
     // Incremental forward for generation: only the new positions are processed, K/V of earlier positions
     // come from the per-layer cache (model.cu:385-424).
+    // The weights must not change while a generation runs (the cached keys and values were made with them): in bf16
+    // mode their images are converted at the first call after resetGenerationState() (or after anything else that
+    // invalidated them) and kept for the calls that follow, where the reference converts them in every call.
     DeviceTensor forwardIncremental(const DeviceTensor& newTokenIds) {
+        if (useBf16_ && generationPosition_ == 0) invalidateBf16WeightCache();
         DeviceTensor current = newTokenIds.clone();
         std::size_t newLen = current.rank() >= 2 ? current.dim(1) : 0;
         for (LayerState& layer : layers_) {
@@ -198,8 +202,9 @@ public:
                     current = addPositionalEmbeddingAt(current, layer.params[0].value, generationPosition_);
                     break;
                 case LayerKind::Attention:
-                    current = useBf16_ ? selfAttentionIncrementalBf16(current, layer.params[0].value, layer.params[1].value,
-                                                                       layer.params[2].value, layer.params[3].value, s.arg0, layer.kvCache)
+                    current = useBf16_ ? selfAttentionIncrementalBf16CachedWeights(current, layer.params[0].value, layer.params[1].value,
+                                                                                    layer.params[2].value, layer.params[3].value, s.arg0,
+                                                                                    layer.kvCache)
                                        : selfAttentionIncremental(current, layer.params[0].value, layer.params[1].value,
                                                                   layer.params[2].value, layer.params[3].value, s.arg0, layer.kvCache);
                     break;
@@ -208,15 +213,16 @@ public:
                     throw std::invalid_argument("hip::Model::forwardIncremental: the pipeline contains 'bidirectional_attention', "
                                                 "which does not support incremental generation");
                 case LayerKind::FeedForward: {
+                    // the block as the training pass runs it (bias, activation and residual in the products' stores, cached
+                    // weight images); what it keeps for a backward pass is dropped
                     Activation act = s.arg1 == 1 ? Activation::Gelu : Activation::Silu;
-                    current = useBf16_ ? feedForwardBf16(current, layer.params[0].value, layer.params[1].value, layer.params[2].value,
-                                                         layer.params[3].value, act)
-                                       : feedForward(current, layer.params[0].value, layer.params[1].value, layer.params[2].value,
-                                                     layer.params[3].value, act);
+                    FeedForwardCache unused;
+                    current = feedForwardForwardCached(current, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                       layer.params[3].value, useBf16_, unused, act);
                     break;
                 }
                 case LayerKind::Linear:
-                    current = useBf16_ ? linearBf16(current, layer.params[0].value, layer.params[1].value)
+                    current = useBf16_ ? linearBf16CachedWeight(current, layer.params[0].value, layer.params[1].value)
                                        : linear(current, layer.params[0].value, layer.params[1].value);
                     break;
                 case LayerKind::Embedding: current = embeddingLookup(current, layer.params[0].value); break;

@@ -438,10 +438,26 @@ inline DeviceTensor selfAttentionIncrementalImpl(const char* op, const DeviceTen
                                                   std::size_t numHeads, KVCache& cache, int mode) {
     requireAttention(op, newInput, numHeads);
     std::size_t batch = newInput.dim(0), newLen = newInput.dim(1), dim = newInput.dim(2);
-    DeviceTensor normedFlat = rmsnorm(newInput).reshaped({batch * newLen, dim});
-    DeviceTensor qNew = projection(normedFlat, wq, mode, {batch, newLen, dim});
-    DeviceTensor kNew = projection(normedFlat, wk, mode, {batch, newLen, dim});
-    DeviceTensor vNew = projection(normedFlat, wv, mode, {batch, newLen, dim});
+    DeviceTensor qNew, kNew, vNew;
+    if (mode != 0 && dim % 8 == 0 && batch * newLen > 0) {
+        // the normalised rows have no reader but the three projections: written as a bf16 image only, and the three
+        // products made by one call over that image
+        const std::size_t rows = batch * newLen;
+        DeviceTensor normedImage({rows, dim / 2});
+        check(bf_hip_rmsnorm_img(newInput.data(), nullptr, reinterpret_cast<std::uint16_t*>(normedImage.data()), rows, dim, nullptr));
+        qNew = DeviceTensor({batch, newLen, dim});
+        kNew = DeviceTensor({batch, newLen, dim});
+        vNew = DeviceTensor({batch, newLen, dim});
+        const float* weights[3] = {wq.data(), wk.data(), wv.data()};
+        float* outs[3] = {qNew.data(), kNew.data(), vNew.data()};
+        check(bf_hip_matmul_bf16_shared_input_img(nullptr, reinterpret_cast<const std::uint16_t*>(normedImage.data()), weights, outs, 3, rows, dim,
+                                                  dim, mode == 2, nullptr));
+    } else {
+        DeviceTensor normedFlat = rmsnorm(newInput).reshaped({batch * newLen, dim});
+        qNew = projection(normedFlat, wq, mode, {batch, newLen, dim});
+        kNew = projection(normedFlat, wk, mode, {batch, newLen, dim});
+        vNew = projection(normedFlat, wv, mode, {batch, newLen, dim});
+    }
     std::size_t oldLen = cache.length;
     if (oldLen == 0) {
         cache.k = std::move(kNew);
@@ -453,8 +469,7 @@ inline DeviceTensor selfAttentionIncrementalImpl(const char* op, const DeviceTen
     cache.length = oldLen + newLen;
     float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
     FusedAttentionForwardResult attn = fusedAttentionForward(qNew, cache.k, cache.v, numHeads, scaleFactor, oldLen);
-    DeviceTensor projected = projection(attn.output, wout, mode, {batch, newLen, dim});
-    return add(newInput, projected);
+    return projectionFused(attn.output, wout, nullptr, &newInput, mode, {batch, newLen, dim});   // the residual joins in the product's store
 }
 }  // namespace detail
 
@@ -467,6 +482,13 @@ inline DeviceTensor selfAttentionIncrementalBf16(const DeviceTensor& newInput, c
                                                   const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
                                                   KVCache& cache) {
     return detail::selfAttentionIncrementalImpl("selfAttentionIncrementalBf16", newInput, wq, wk, wv, wout, numHeads, cache, 1);
+}
+// The same with the weights' bf16 images kept between calls (until invalidateBf16WeightCache): for a generation loop,
+// during which the weights do not change (not part of the reference's interface).
+inline DeviceTensor selfAttentionIncrementalBf16CachedWeights(const DeviceTensor& newInput, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                               const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
+                                                               KVCache& cache) {
+    return detail::selfAttentionIncrementalImpl("selfAttentionIncrementalBf16", newInput, wq, wk, wv, wout, numHeads, cache, 2);
 }
 
 // Greedy next-token choice over the last position of [1, seq, vocab] logits (reference: src/main.cpp:504-518),

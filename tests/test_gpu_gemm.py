@@ -295,6 +295,36 @@ def test_bf16_linear_with_adds_in_the_store(hip, oracle, rng, m, k, n, with_bias
     assert_close(got, expected, tol=1e-4, what="fused linear")
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 768, 768), (1, 3072, 768), (1, 768, 32003), (2, 72, 9000), (3, 520, 41), (5, 1032, 8200), (8, 768, 2304),
+                                   (7, 8, 1), (1, 4100, 16), (4, 44, 300)])
+@pytest.mark.parametrize("with_bias,with_residual", [(True, True), (False, False)])
+def test_bf16_products_of_a_few_rows(hip, oracle, rng, m, k, n, with_bias, with_residual):
+    """matmulBf16 / linearBf16 (ops.hpp:14,30,8) with at most eight rows, the shape of a step of incremental decoding
+    (model.cpp:169, one new token per sequence): served by a walk over the weights instead of MFMA tiles.  Widths on both
+    sides of the switch from one to four columns a wavefront, odd widths, a contraction of several steps a lane, and one
+    that is not a multiple of eight (which stays on the tiles)."""
+    D, ops = hip.DeviceTensor, hip.ops
+    a, w, bias, res = r(rng, m, k), r(rng, k, n, scale=0.1), r(rng, n), r(rng, m, n)
+    expected = (oracle.roundToBf16(a).astype(np.float64) @ oracle.roundToBf16(w).astype(np.float64)).astype(f32)
+    if m * k * n <= 5_000_000:
+        assert_close(oracle.matmul(oracle.roundToBf16(a), oracle.roundToBf16(w)), expected, tol=1e-5, what="oracle vs float64")
+    plain = ops.matmulBf16(D.fromHost(a), D.fromHost(w)).toHost()
+    assert_close(plain, expected, tol=1e-4, what="few-row product")
+    again = ops.matmulBf16(D.fromHost(a), D.fromHost(w)).toHost()
+    assert_bits_equal(again, plain, "the same product twice")
+    got = ops.linearBf16Fused(D.fromHost(a), D.fromHost(w), D.fromHost(bias) if with_bias else None,
+                              D.fromHost(res) if with_residual else None).toHost()
+    if with_bias: expected = oracle.addBias(expected, bias)
+    if with_residual: expected = oracle.add(expected, res)
+    assert_close(got, expected, tol=1e-4, what="few-row product with the adds in its store")
+    if n % 256 == 0 or n <= 300:   # three projections of one input: one product with split outputs when the width allows
+        ws = [w, r(rng, k, n, scale=0.1), r(rng, k, n, scale=0.1)]
+        outs = ops.matmulBf16SharedInput(D.fromHost(a), [D.fromHost(x) for x in ws])
+        for i in range(3):
+            e = (oracle.roundToBf16(a).astype(np.float64) @ oracle.roundToBf16(ws[i]).astype(np.float64)).astype(f32)
+            assert_close(outs[i].toHost(), e, tol=1e-4, what=f"shared-input product {i}")
+
+
 @pytest.mark.parametrize("m,k,n,count", [(50, 40, 24, 3), (300, 136, 256, 3), (4096, 64, 1024, 3), (4100, 256, 256, 3), (260, 72, 512, 2),
                                          (64, 32, 48, 1), (8192, 520, 256, 3), (8200, 300, 512, 2)])
 @pytest.mark.parametrize("cached", [False, True])
