@@ -122,6 +122,8 @@ SIGNATURES = {
     "bf_hip_mfma_only_loop": [P, P, c_int, c_int, c_int, S],
     "bf_hip_attention_forward": [P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_attention_forward_img": [P, P, P, P, P, c_size, P, P, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
+    "bf_hip_attention_forward_rows": [P, P, P, P, P, c_size, P, P, c_size, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
+    "bf_hip_copy_pitched": [P, c_size, P, c_size, c_size, c_size, S],
     "bf_hip_attention_backward_img": [P, P, P, P, P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_size, c_float,
                                       c_size, S],
     "bf_hip_attention_dot_o_do": [P, P, P, c_size, c_size, c_size, c_size, S],

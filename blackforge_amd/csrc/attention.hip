@@ -2419,6 +2419,115 @@ __global__ void __launch_bounds__(256) attnCombineChunksKernel(const float* __re
     if (t == 0) { m[stat] = rowMax; l[stat] = total; }
 }
 
+// Forward pass of at most a few queries per sequence (a step of incremental decoding) without tiles: a 128-query tile
+// would hold one live row, and the pass is a walk over the cached keys and values anyway.  LPK lanes share a key: each
+// holds four of the head's columns (16 bytes of the key's row, the same of the value's), the dot product is a butterfly
+// over those lanes, and each such group of lanes walks every (256 / LPK)-th key of the workgroup's chunk, four keys a
+// round, with its own running maximum, sum and output; the groups of a wavefront are joined by a butterfly, the four
+// wavefronts in order through LDS.  blockIdx.x is the chunk of keys, blockIdx.y the (batch, head, query).  Head dims that
+// are multiples of 4, 16-byte aligned operands.  Chunk c of numChunks > 1 writes its normalised output and statistics as
+// the tile kernels do (attnCombineChunksKernel joins them); a single chunk writes the results themselves.
+template <int LPK>
+__global__ void __launch_bounds__(256) attnFewQueriesKernel(AttnParams p) {
+    constexpr int GROUPS = 256 / LPK, KEYS = 4;
+    __shared__ float sM[4], sL[4];
+    __shared__ float4v sAcc[4][LPK];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int sub = t % LPK, group = t / LPK;
+    const int c = blockIdx.x;
+    const int h = int(blockIdx.y) % p.heads, bi = int(blockIdx.y) / p.heads;   // bi = b * newLen + i
+    const int b = bi / p.newLen, i = bi - b * p.newLen;
+    const int hd = p.hd, dim = p.dim, d0 = sub * 4;
+    const bool live = d0 < hd;                                 // lanes past the head's columns carry zeros
+    const size_t column = size_t(h) * hd + (live ? d0 : 0);
+    const float* kb = p.k + size_t(b) * p.kvRows * dim + column;
+    const float* vb = p.v + size_t(b) * p.kvRows * dim + column;
+    const float4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const float4v q4 = live ? loadf4(p.q + size_t(bi) * dim + column) : zero;
+    const int limit = p.oldLen + i + 1;                        // keys 0 .. oldLen + i are visible to query i
+    const int start = c * p.chunkKeys;
+    const int end = c == p.numChunks - 1 ? limit : min(start + p.chunkKeys, limit);
+
+    float m = -INFINITY, l = 0.0f;
+    float4v acc = zero;
+    for (int j0 = start + group; j0 < end; j0 += KEYS * GROUPS) {
+        float4v k4[KEYS], v4[KEYS];
+#pragma unroll
+        for (int u = 0; u < KEYS; ++u) {
+            const int j = j0 + u * GROUPS;
+            const bool in = live && j < end;
+            k4[u] = in ? loadf4(kb + size_t(j) * dim) : zero;
+            v4[u] = in ? loadf4(vb + size_t(j) * dim) : zero;
+        }
+        float sc[KEYS];
+        float roundMax = m;
+#pragma unroll
+        for (int u = 0; u < KEYS; ++u) {
+            float dot = (q4.x * k4[u].x + q4.y * k4[u].y) + (q4.z * k4[u].z + q4.w * k4[u].w);
+#pragma unroll
+            for (int o = LPK / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);
+            sc[u] = j0 + u * GROUPS < end ? dot * p.scale : -INFINITY;
+            roundMax = fmaxf(roundMax, sc[u]);
+        }
+        const float keep = expf(m - roundMax);                 // m = -inf at the first round: 0 (key j0 itself is below `end`)
+        l *= keep;
+        acc = acc * keep;
+#pragma unroll
+        for (int u = 0; u < KEYS; ++u) {
+            const float w = expf(sc[u] - roundMax);
+            l += w;
+            acc = acc + v4[u] * w;
+        }
+        m = roundMax;
+    }
+    // join two running states: (m, l, acc) with the lanes' partners at distance `o`
+    auto join = [&](float om, float ol, float4v oacc) {
+        const float mm = fmaxf(m, om);
+        if (mm == -INFINITY) return;                           // neither side has seen a key
+        const float mine = expf(m - mm), theirs = expf(om - mm);
+        l = l * mine + ol * theirs;
+        acc = acc * mine + oacc * theirs;
+        m = mm;
+    };
+#pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) {
+        const float om = __shfl_xor(m, o, 64), ol = __shfl_xor(l, o, 64);
+        float4v oacc;
+        oacc.x = __shfl_xor(acc.x, o, 64); oacc.y = __shfl_xor(acc.y, o, 64);
+        oacc.z = __shfl_xor(acc.z, o, 64); oacc.w = __shfl_xor(acc.w, o, 64);
+        join(om, ol, oacc);
+    }
+    if (lane < LPK) {
+        sAcc[wave][lane] = acc;
+        if (lane == 0) { sM[wave] = m; sL[wave] = l; }
+    }
+    __syncthreads();
+    if (t < LPK) {
+        m = sM[0]; l = sL[0]; acc = sAcc[0][t];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) join(sM[w], sL[w], sAcc[w][t]);
+        const float inv = 1.0f / l;                            // every chunk holds a key visible to every query
+        const float4v o4 = acc * inv;
+        const size_t stat = (size_t(b) * p.heads + h) * p.newLen + i;
+        const size_t at = size_t(bi) * dim + size_t(h) * hd + d0;
+        const bool whole = p.numChunks <= 1;
+        float* out = whole ? p.out : p.out + size_t(c) * p.partOutStride;
+        if (live) {
+            if (out) storef4(out + at, o4);
+            if (whole && p.outImg) {
+                uint2v packed = {unsigned(toBf16Bits(o4.x)) | unsigned(toBf16Bits(o4.y)) << 16,
+                                 unsigned(toBf16Bits(o4.z)) | unsigned(toBf16Bits(o4.w)) << 16};
+                *reinterpret_cast<uint2v*>(p.outImg + size_t(bi) * p.imgLd + size_t(h) * hd + d0) = packed;
+            }
+        }
+        if (t == 0) {
+            const size_t off = whole ? 0 : size_t(c) * p.partStatStride;
+            p.m[off + stat] = m;
+            p.l[off + stat] = l;
+        }
+    }
+}
+
 bool vec4Ok(const AttnParams& p, std::initializer_list<const void*> ptrs) {
     if (p.hd % 4 != 0 || p.dim % 4 != 0) return false;
     for (const void* q : ptrs)
@@ -2544,13 +2653,14 @@ static int checkImages(const char* fn, std::initializer_list<const void*> images
     return BF_OK;
 }
 
-int bf_hip_attention_forward_img(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
-                                 float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
-                                 size_t oldLen, bf_stream_t stream) {
+int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
+                                  float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t kvRows, size_t dim, float scale,
+                                  size_t oldLen, bf_stream_t stream) {
     int st = checkShapes(__func__, batch, heads, newLen, totalLen, dim, oldLen);
     if (st != BF_OK) return st;
     if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
     BF_REQUIRE(q && k && v && (out || outImage) && m && l, "NULL pointer");
+    if (kvRows < totalLen || kvRows >= (size_t(1) << 31)) return failInvalid(__func__, "kvRows must be at least totalLen");
     st = checkImages(__func__, {outImage}, imageLd, dim);
     if (st != BF_OK) return st;
     AttnParams p{};
@@ -2559,14 +2669,49 @@ int bf_hip_attention_forward_img(const float* q, const float* k, const float* v,
     p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(totalLen);
     p.dim = int(dim); p.hd = int(dim / heads); p.oldLen = int(oldLen); p.scale = scale;
     p.numTiles = int((newLen + 127) / 128);
-    p.kvRows = p.totalLen;
+    p.kvRows = int(kvRows);
     unsigned grid = unsigned(batch * heads * size_t(p.numTiles));
     hipStream_t s = asStream(stream);
+    const size_t cus = size_t(computeUnits());
+    // At most eight queries per sequence (incremental decoding): the walk over the cache, LPK lanes a key
+    if (newLen <= 8 && batch * heads * newLen <= 65535 && vec4Ok(p, {q, k, v, out}) && (gAttnRoute & BF_ATTN_ROUTE_TILES_ONLY) == 0) {
+        const size_t rows = batch * heads * newLen;
+        const size_t wanted = std::max<size_t>(1, (4 * cus + rows - 1) / rows);   // about four workgroups per compute unit
+        size_t chunkKeys = std::max<size_t>(128, ((totalLen + wanted - 1) / wanted + 127) / 128 * 128);
+        const size_t numChunks = std::max<size_t>(1, std::min((totalLen + chunkKeys - 1) / chunkKeys, oldLen / chunkKeys + 1));
+        AttnParams c = p;
+        c.chunkKeys = int(chunkKeys);
+        c.numChunks = int(numChunks);
+        const size_t outFloats = batch * newLen * dim, statFloats = batch * heads * newLen;
+        Scratch part(numChunks > 1 ? numChunks * (outFloats + 2 * statFloats) * sizeof(float) : 0);
+        if (part.status != BF_OK) return part.status;
+        if (numChunks > 1) {
+            c.partOutStride = outFloats;
+            c.partStatStride = statFloats;
+            c.out = part.as<float>();
+            c.m = c.out + numChunks * outFloats;
+            c.l = c.m + numChunks * statFloats;
+        }
+        const dim3 g{unsigned(numChunks), unsigned(rows), 1u};
+        const int lanes = p.hd <= 32 ? 8 : p.hd <= 64 ? 16 : p.hd <= 128 ? 32 : 64;
+        switch (lanes) {
+            case 8: attnFewQueriesKernel<8><<<g, 256, 0, s>>>(c); break;
+            case 16: attnFewQueriesKernel<16><<<g, 256, 0, s>>>(c); break;
+            case 32: attnFewQueriesKernel<32><<<g, 256, 0, s>>>(c); break;
+            default: attnFewQueriesKernel<64><<<g, 256, 0, s>>>(c); break;
+        }
+        BF_LAUNCH_CHECK();
+        if (numChunks > 1) {
+            attnCombineChunksKernel<<<unsigned(rows), 256, 0, s>>>(c.out, c.m, c.l, out, outImage, imageLd, m, l, int(heads), int(newLen), int(dim), p.hd,
+                                                                int(numChunks), outFloats, statFloats);
+            BF_LAUNCH_CHECK();
+        }
+        return BF_OK;
+    }
     // Few queries against many keys (a step of incremental decoding: one workgroup per head would walk all the keys alone):
     // the keys go to the workgroups in chunks, each with its own statistics, and a second kernel puts the chunks together.
     // A chunk must start at or before the first query's own position, so that every query sees a key in every chunk: the
     // last chunk takes everything from the last such start.
-    const size_t cus = size_t(computeUnits());
     if (size_t(grid) * 2 <= cus && totalLen >= 1024) {
         const size_t wanted = (4 * cus + grid - 1) / grid;   // about four workgroups per compute unit
         size_t chunkKeys = ((totalLen + wanted - 1) / wanted + 127) / 128 * 128;
@@ -2595,6 +2740,12 @@ int bf_hip_attention_forward_img(const float* q, const float* k, const float* v,
         }
     }
     return dispatch<0>(p, vec4Ok(p, {q, k, v, out}), grid, s);
+}
+
+int bf_hip_attention_forward_img(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
+                                 float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
+                                 size_t oldLen, bf_stream_t stream) {
+    return bf_hip_attention_forward_rows(q, k, v, out, outImage, imageLd, m, l, batch, heads, newLen, totalLen, totalLen, dim, scale, oldLen, stream);
 }
 
 int bf_hip_attention_forward(const float* q, const float* k, const float* v, float* out, float* m, float* l,
@@ -2792,7 +2943,7 @@ int bf_hip_attention_backward(const float* dOut, const float* q, const float* k,
 }
 
 int bf_hip_attention_set_route(int route) {
-    BF_REQUIRE(route >= 0 && route <= BF_ATTN_ROUTE_SPLIT, "unknown route");
+    BF_REQUIRE(route >= 0 && route <= (BF_ATTN_ROUTE_SPLIT | BF_ATTN_ROUTE_TILES_ONLY), "unknown route");
     bf::gAttnRoute = route;
     return BF_OK;
 }

@@ -336,6 +336,20 @@ __global__ void __launch_bounds__(256) concatSeqKernel(const float* __restrict__
     }
 }
 
+// dst[r * dstPitch + c] = src[r * srcPitch + c] for c < width: blocks of `width` floats that lie `pitch` floats apart
+// (the rows of a sequence in a key/value cache that has room to grow); rows walked by threadIdx.y
+template <int VEC>
+__global__ void __launch_bounds__(256) copyPitchedKernel(float* __restrict__ dst, size_t dstPitch, const float* __restrict__ src,
+                                                         size_t srcPitch, size_t width, size_t rows) {
+    size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
+    if (col >= width) return;
+    size_t step = size_t(gridDim.y) * blockDim.y;
+    for (size_t r = size_t(blockIdx.y) * blockDim.y + threadIdx.y; r < rows; r += step) {
+        if constexpr (VEC == 4) storef4(dst + r * dstPitch + col, loadf4(src + r * srcPitch + col));
+        else dst[r * dstPitch + col] = src[r * srcPitch + col];
+    }
+}
+
 // Lowest index of the maximum of one row: the result of the host loop "best = 0; if (row[c] > row[best])
 // best = c" it replaces.  A NaN never wins a strict '>' and, at index 0, is never beaten; the key
 // below encodes exactly that.
@@ -515,6 +529,17 @@ int bf_hip_concat_seq(const float* a, const float* b, float* out, size_t batch, 
     Geom2D g = geometry2D(batch * (seqA + seqB), dim, aligned16(a) && aligned16(b) && aligned16(out));
     if (g.vec == 4) concatSeqKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(a, b, out, batch, seqA, seqB, dim);
     else concatSeqKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(a, b, out, batch, seqA, seqB, dim);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_copy_pitched(float* dst, size_t dstPitch, const float* src, size_t srcPitch, size_t width, size_t rows, bf_stream_t stream) {
+    if (width == 0 || rows == 0) return BF_OK;
+    BF_REQUIRE(dst && src, "NULL pointer");
+    BF_REQUIRE(dstPitch >= width && srcPitch >= width, "a pitch must be at least the width");
+    Geom2D g = geometry2D(rows, width, aligned16(dst) && aligned16(src) && dstPitch % 4 == 0 && srcPitch % 4 == 0);
+    if (g.vec == 4) copyPitchedKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(dst, dstPitch, src, srcPitch, width, rows);
+    else copyPitchedKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(dst, dstPitch, src, srcPitch, width, rows);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

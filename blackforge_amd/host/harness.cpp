@@ -405,22 +405,29 @@ int bfh_feed_forward_backward(const float* x, int rank, const size_t* shape, con
     });
 }
 
-// hip::KVCache behind a handle, for selfAttentionIncremental[Bf16].
-void* bfh_kv_cache_create(void) { return new hip::KVCache(); }
-void bfh_kv_cache_destroy(void* cache) { delete static_cast<hip::KVCache*>(cache); }
-int bfh_kv_cache_info(void* cache, size_t* length, float** k, float** v) {
-    auto* c = static_cast<hip::KVCache*>(cache);
-    if (length) *length = c->length;
-    if (k) *k = c->k.data();
-    if (v) *v = c->v.data();
-    return 0;
+// hip::KVCache behind a handle, for selfAttentionIncremental[Bf16]; k and v are reported as the dense
+// [batch, length, dim] tensors, copies that live until the next call.
+struct KvHandle {
+    hip::KVCache cache;
+    hip::DeviceTensor keys, values;
+};
+void* bfh_kv_cache_create(void) { return new KvHandle(); }
+void bfh_kv_cache_destroy(void* cache) { delete static_cast<KvHandle*>(cache); }
+int bfh_kv_cache_info(void* cache, size_t* length, size_t* capacity, float** k, float** v) {
+    return guarded([&] {
+        auto* c = static_cast<KvHandle*>(cache);
+        if (length) *length = c->cache.length;
+        if (capacity) *capacity = c->cache.capacity;
+        if (k) { c->keys = c->cache.keys(); *k = c->keys.data(); }
+        if (v) { c->values = c->cache.values(); *v = c->values.data(); }
+    });
 }
 int bfh_self_attention_incremental(void* cache, const float* xNew, const float* wq, const float* wk, const float* wv, const float* wout,
                                    size_t batch, size_t newLen, size_t dim, size_t heads, int useBf16, float* out) {
     return guarded([&] {
         Borrowed in(xNew, {batch, newLen, dim});
         AttentionWeights w(wq, wk, wv, wout, dim);
-        auto& kv = *static_cast<hip::KVCache*>(cache);
+        auto& kv = static_cast<KvHandle*>(cache)->cache;
         hip::DeviceTensor y = useBf16 ? hip::selfAttentionIncrementalBf16(in.tensor, w.wq.tensor, w.wk.tensor, w.wv.tensor, w.wout.tensor, heads, kv)
                                       : hip::selfAttentionIncremental(in.tensor, w.wq.tensor, w.wk.tensor, w.wv.tensor, w.wout.tensor, heads, kv);
         copyOut(out, y);

@@ -66,7 +66,7 @@ def load() -> ctypes.CDLL:
         lib.bfh_feed_forward_backward.argtypes = [P, I, ctypes.POINTER(Z)] + [P] * 5 + [Z, I, I] + [P] * 5
         lib.bfh_kv_cache_create.restype = P
         lib.bfh_kv_cache_destroy.argtypes = [P]
-        lib.bfh_kv_cache_info.argtypes = [P, ctypes.POINTER(Z), ctypes.POINTER(P), ctypes.POINTER(P)]
+        lib.bfh_kv_cache_info.argtypes = [P, ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(P), ctypes.POINTER(P)]
         lib.bfh_self_attention_incremental.argtypes = [P] * 6 + [Z] * 4 + [I, P]
         lib.bfh_model_forward_incremental.argtypes = [P, P, I, ctypes.POINTER(Z), ctypes.POINTER(P), ctypes.POINTER(Z)]
         lib.bfh_model_reset_generation.argtypes = [P]
@@ -295,14 +295,23 @@ class KVCache:
             load().bfh_kv_cache_destroy(self.handle)
             self.handle = None
 
-    def _info(self):
-        length, k, v = ctypes.c_size_t(), ctypes.c_void_p(), ctypes.c_void_p()
-        load().bfh_kv_cache_info(self.handle, ctypes.byref(length), ctypes.byref(k), ctypes.byref(v))
+    def _info(self, tensors=True):
+        length, capacity, k, v = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_void_p(), ctypes.c_void_p()
+        st = load().bfh_kv_cache_info(self.handle, ctypes.byref(length), ctypes.byref(capacity), ctypes.byref(k) if tensors else None,
+                                      ctypes.byref(v) if tensors else None)
+        if st != 0:
+            raise RuntimeError("bfh_kv_cache_info failed")
+        self._capacity = capacity.value
         return length.value, k, v
 
     @property
     def length(self) -> int:
-        return self._info()[0]
+        return self._info(False)[0]
+
+    @property
+    def capacity(self) -> int:
+        self._info(False)
+        return self._capacity
 
     def keys(self, batch: int, dim: int) -> np.ndarray:
         length, k, _ = self._info()

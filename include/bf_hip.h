@@ -218,6 +218,10 @@ int bf_hip_positional_backward(const float* g, float* dTable, size_t batch, size
 /* concatSeq (KV-cache growth): ops_transformer.cu:22-58   [batch,seqA,dim] ++ [batch,seqB,dim] */
 int bf_hip_concat_seq(const float* a, const float* b, float* out, size_t batch, size_t seqA, size_t seqB, size_t dim,
                       bf_stream_t stream);
+/* dst[r * dstPitch + c] = src[r * srcPitch + c], c < width, r < rows (floats; pitches >= width): the copy that appends
+ * new keys and values to a cache with room to grow (hip::KVCache), where the reference concatenates into a new tensor at
+ * every step (ops_transformer.cu:22-58). */
+int bf_hip_copy_pitched(float* dst, size_t dstPitch, const float* src, size_t srcPitch, size_t width, size_t rows, bf_stream_t stream);
 /* argmaxLastPosition: main.cpp:504-518, moved to the device.  logits: [seq, vocab]; *index (HOST) gets
  * the lowest index of the maximum of the last row.  Synchronous. */
 int bf_hip_argmax_last_position(const float* logits, size_t seq, size_t vocab, long long* index, bf_stream_t stream);
@@ -393,6 +397,16 @@ int bf_hip_attention_forward(const float* q, const float* k, const float* v, flo
 int bf_hip_attention_forward_img(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
                                  float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t dim, float scale,
                                  size_t oldLen, bf_stream_t stream);
+/* The same with the keys and values of a sequence `kvRows` >= totalLen rows apart (k, v: [batch, kvRows, dim], the first
+ * totalLen rows of each sequence used): attention over a cache with room to grow.  bf_hip_attention_forward_img is this
+ * with kvRows = totalLen.  (No counterpart in the reference, whose cache is exactly totalLen rows long.)
+ * At most eight queries per sequence with 16-byte aligned operands and a head dim that is a multiple of 4 (a step of
+ * incremental decoding) are served without tiles, as a walk over the cache: the lanes that share a key hold four of the
+ * head's columns each, the keys go to the workgroups in chunks of 128 or more so that about four workgroups per compute
+ * unit run, and the chunks are joined by a second kernel when there are several. */
+int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
+                                  float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t kvRows, size_t dim, float scale,
+                                  size_t oldLen, bf_stream_t stream);
 /* computeDKernel: fused_attention.cu:166-190   D[b,h,i] = dot(out[b,i,h,:], dOut[b,i,h,:]) */
 int bf_hip_attention_dot_o_do(const float* out, const float* dOut, float* D, size_t batch, size_t heads,
                               size_t newLen, size_t dim, bf_stream_t stream);
@@ -449,7 +463,8 @@ int bf_hip_attention_set_workspace_limit(size_t bytes);
  * route 0's.  The DQ bit covers the kernel that forms dQ from the stored dS; the dQ kernel that recomputes S and dP
  * (taken when the dS buffer would exceed the workspace limit) runs on the fp32 MFMA on every route. */
 enum { BF_ATTN_ROUTE_FP32_MFMA = 0, BF_ATTN_ROUTE_SPLIT_FORWARD = 1, BF_ATTN_ROUTE_SPLIT_DKV = 2, BF_ATTN_ROUTE_SPLIT_DQ = 4,
-       BF_ATTN_ROUTE_SPLIT = 7 };
+       BF_ATTN_ROUTE_SPLIT = 7,
+       BF_ATTN_ROUTE_TILES_ONLY = 8 /* added to any of the above: forward passes of few queries stay on the tile kernels */ };
 int bf_hip_attention_set_route(int route);
 int bf_hip_attention_backward_dkv_ds(const float* dOut, const float* q, const float* k, const float* v, const float* lse2,
                                      const float* D, float* dK, float* dV, float* dS, size_t batch, size_t heads,

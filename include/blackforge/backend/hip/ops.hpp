@@ -420,56 +420,94 @@ inline DeviceTensor selfAttentionBf16(const DeviceTensor& input, const DeviceTen
     return detail::selfAttentionForwardImpl("selfAttentionBf16", input, wq, wk, wv, wout, numHeads, 1, cache);
 }
 
-// K/V of the positions processed so far, for incremental decoding.
+// K/V of the positions processed so far, for incremental decoding.  The buffers have room to grow: k and v are
+// [batch, capacity, dim] with the first `length` rows of every sequence valid, and a call appends its rows in place
+// (the reference's k and v are exactly [batch, length, dim] and are re-made, old rows copied, at every call:
+// ops.hpp:213, ops_transformer.cu:22-58).  keys() / values() give the [batch, length, dim] tensors.
 struct KVCache {
     DeviceTensor k;
     DeviceTensor v;
     std::size_t length = 0;
+    std::size_t capacity = 0;   // rows per sequence in k and v
+
+    [[nodiscard]] DeviceTensor keys() const { return dense(k); }
+    [[nodiscard]] DeviceTensor values() const { return dense(v); }
+
+    // Room for `rows` positions per sequence: a first allocation takes 64 spare rows, later ones double.
+    void reserve(std::size_t batch, std::size_t rows, std::size_t dim) {
+        if (rows <= capacity && k.rank() == 3) return;
+        const std::size_t grown = (std::max(rows + 64, 2 * capacity) + 63) / 64 * 64;
+        DeviceTensor newK({batch, grown, dim}), newV({batch, grown, dim});
+        if (length != 0) {
+            check(bf_hip_copy_pitched(newK.data(), grown * dim, k.data(), capacity * dim, length * dim, batch, nullptr));
+            check(bf_hip_copy_pitched(newV.data(), grown * dim, v.data(), capacity * dim, length * dim, batch, nullptr));
+        }
+        k = std::move(newK);
+        v = std::move(newV);
+        capacity = grown;
+    }
+
+private:
+    [[nodiscard]] DeviceTensor dense(const DeviceTensor& store) const {
+        if (length == 0 || store.rank() != 3) return DeviceTensor();
+        const std::size_t batch = store.dim(0), dim = store.dim(2);
+        DeviceTensor out({batch, length, dim});
+        check(bf_hip_copy_pitched(out.data(), length * dim, store.data(), capacity * dim, length * dim, batch, nullptr));
+        return out;
+    }
 };
 
 namespace detail {
-inline DeviceTensor concatSeq(const DeviceTensor& a, const DeviceTensor& b) {
-    DeviceTensor out({a.dim(0), a.dim(1) + b.dim(1), a.dim(2)});
-    check(bf_hip_concat_seq(a.data(), b.data(), out.data(), a.dim(0), a.dim(1), b.dim(1), a.dim(2), nullptr));
-    return out;
-}
 inline DeviceTensor selfAttentionIncrementalImpl(const char* op, const DeviceTensor& newInput, const DeviceTensor& wq,
                                                   const DeviceTensor& wk, const DeviceTensor& wv, const DeviceTensor& wout,
                                                   std::size_t numHeads, KVCache& cache, int mode) {
     requireAttention(op, newInput, numHeads);
     std::size_t batch = newInput.dim(0), newLen = newInput.dim(1), dim = newInput.dim(2);
-    DeviceTensor qNew, kNew, vNew;
-    if (mode != 0 && dim % 8 == 0 && batch * newLen > 0) {
-        // the normalised rows have no reader but the three projections: written as a bf16 image only, and the three
-        // products made by one call over that image
-        const std::size_t rows = batch * newLen;
-        DeviceTensor normedImage({rows, dim / 2});
-        check(bf_hip_rmsnorm_img(newInput.data(), nullptr, reinterpret_cast<std::uint16_t*>(normedImage.data()), rows, dim, nullptr));
-        qNew = DeviceTensor({batch, newLen, dim});
+    const std::size_t oldLen = cache.length, rows = batch * newLen;
+    if (cache.length != 0) require(cache.k.rank() == 3 && cache.k.dim(0) == batch && cache.k.dim(2) == dim, std::string(op) + ": the cache was filled with another batch size or width");
+    cache.reserve(batch, oldLen + newLen, dim);
+    // one sequence: its new keys and values are rows oldLen.. of the cache, and the projections write them there;
+    // several: the projections' rows lie batch by batch and a copy spreads them over the sequences
+    const bool inPlace = batch == 1;
+    DeviceTensor qNew({batch, newLen, dim}), kNew, vNew;
+    if (!inPlace) {
         kNew = DeviceTensor({batch, newLen, dim});
         vNew = DeviceTensor({batch, newLen, dim});
+    }
+    float* kRows = inPlace ? cache.k.data() + oldLen * dim : kNew.data();
+    float* vRows = inPlace ? cache.v.data() + oldLen * dim : vNew.data();
+    if (mode != 0 && dim % 8 == 0 && rows > 0) {
+        // the normalised rows have no reader but the three projections: written as a bf16 image only, and the three
+        // products made by one call over that image
+        DeviceTensor normedImage({rows, dim / 2});
+        check(bf_hip_rmsnorm_img(newInput.data(), nullptr, reinterpret_cast<std::uint16_t*>(normedImage.data()), rows, dim, nullptr));
         const float* weights[3] = {wq.data(), wk.data(), wv.data()};
-        float* outs[3] = {qNew.data(), kNew.data(), vNew.data()};
+        float* outs[3] = {qNew.data(), kRows, vRows};
         check(bf_hip_matmul_bf16_shared_input_img(nullptr, reinterpret_cast<const std::uint16_t*>(normedImage.data()), weights, outs, 3, rows, dim,
                                                   dim, mode == 2, nullptr));
     } else {
-        DeviceTensor normedFlat = rmsnorm(newInput).reshaped({batch * newLen, dim});
-        qNew = projection(normedFlat, wq, mode, {batch, newLen, dim});
-        kNew = projection(normedFlat, wk, mode, {batch, newLen, dim});
-        vNew = projection(normedFlat, wv, mode, {batch, newLen, dim});
+        DeviceTensor normedFlat = rmsnorm(newInput).reshaped({rows, dim});
+        const DeviceTensor* w[3] = {&wq, &wk, &wv};
+        float* outs[3] = {qNew.data(), kRows, vRows};
+        for (int i = 0; i < 3; ++i) {
+            if (mode == 0) check(bf_hip_gemm_f32_adds(0, 0, normedFlat.data(), w[i]->data(), nullptr, nullptr, outs[i], rows, dim, dim, nullptr));
+            else check(bf_hip_linear_bf16_img(normedFlat.data(), nullptr, w[i]->data(), nullptr, nullptr, outs[i], rows, dim, dim, mode == 2, nullptr));
+        }
     }
-    std::size_t oldLen = cache.length;
-    if (oldLen == 0) {
-        cache.k = std::move(kNew);
-        cache.v = std::move(vNew);
-    } else {
-        cache.k = concatSeq(cache.k, kNew);
-        cache.v = concatSeq(cache.v, vNew);
+    if (!inPlace) {
+        check(bf_hip_copy_pitched(cache.k.data() + oldLen * dim, cache.capacity * dim, kNew.data(), newLen * dim, newLen * dim, batch, nullptr));
+        check(bf_hip_copy_pitched(cache.v.data() + oldLen * dim, cache.capacity * dim, vNew.data(), newLen * dim, newLen * dim, batch, nullptr));
     }
     cache.length = oldLen + newLen;
-    float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
-    FusedAttentionForwardResult attn = fusedAttentionForward(qNew, cache.k, cache.v, numHeads, scaleFactor, oldLen);
-    return projectionFused(attn.output, wout, nullptr, &newInput, mode, {batch, newLen, dim});   // the residual joins in the product's store
+    const float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
+    // the attention output has one reader, the output projection: in bf16 mode it is written as that product's operand image only
+    const bool imageOnly = mode != 0 && dim % 8 == 0;
+    DeviceTensor attnOut = imageOnly ? DeviceTensor::imageOnly({batch, newLen, dim}) : DeviceTensor({batch, newLen, dim});
+    DeviceTensor m({batch, numHeads, newLen}), l({batch, numHeads, newLen});
+    check(bf_hip_attention_forward_rows(qNew.data(), cache.k.data(), cache.v.data(), attnOut.data(),
+                                        imageOnly ? const_cast<std::uint16_t*>(attnOut.image()) : nullptr, imageOnly ? dim : 0, m.data(), l.data(), batch,
+                                        numHeads, newLen, cache.length, cache.capacity, dim, scaleFactor, oldLen, nullptr));
+    return projectionFused(attnOut, wout, nullptr, &newInput, mode, {batch, newLen, dim});   // the residual joins in the product's store
 }
 }  // namespace detail
 

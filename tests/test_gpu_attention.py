@@ -334,7 +334,7 @@ def test_other_routes_match_the_oracle(hip, oracle, rng, other_route, batch, hea
 
 
 def test_route_argument(hip):
-    assert hip.capi.load().bf_hip_attention_set_route(8) != 0
+    assert hip.capi.load().bf_hip_attention_set_route(16) != 0
     assert hip.capi.load().bf_hip_attention_set_route(-1) != 0
     hip.capi.call("bf_hip_attention_set_route", DEFAULT_ROUTE)
 

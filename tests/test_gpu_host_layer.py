@@ -173,6 +173,18 @@ def test_incremental_decode_block(hip, oracle, rng, use_bf16):
     assert cache.length == 10
     assert_close(cache.keys(batch, dim), kc, tol=tol, what="KV cache K")
     assert_close(cache.values(batch, dim), vc, tol=tol, what="KV cache V")
+    # the cache has room to grow and is re-made only when that runs out: continuations across two such moments
+    seen = {cache.capacity}
+    for new_len in (120, 1, 1, 130, 1, 2):
+        x = r(rng, batch, new_len, dim)
+        got = ops.selfAttentionIncremental(D.fromHost(x), *dw, heads, cache, useBf16=use_bf16).toHost()
+        exp, kc, vc = oracle.selfAttentionIncremental(x, *w, heads, kc, vc)
+        assert_close(got, exp, tol=tol, what=f"incremental newLen={new_len} at length {cache.length}")
+        assert cache.capacity >= cache.length
+        seen.add(cache.capacity)
+    assert cache.length == 265 and len(seen) == 3, seen
+    assert_close(cache.keys(batch, dim), kc, tol=tol, what="KV cache K after growing")
+    assert_close(cache.values(batch, dim), vc, tol=tol, what="KV cache V after growing")
 
 
 def _lm_layers(hl, vocab, dim, seq, heads, hidden, act, blocks=1):

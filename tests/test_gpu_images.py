@@ -98,6 +98,46 @@ def test_attention_images(hip, oracle, rng, batch, heads, seq, hd, old_len, rout
         assert_bits_equal(got[:, :, i], oracle.roundToBf16(t.toHost()), name + " image")
 
 
+@pytest.mark.parametrize("batch,heads,new_len,old_len,hd,kv_rows", [(1, 12, 1, 1023, 64, 1088), (2, 3, 1, 4000, 64, 4001), (3, 2, 8, 300, 128, 1024),
+                                                                    (1, 2, 5, 0, 32, 64), (2, 2, 1, 77, 192, 128), (1, 1, 2, 5000, 256, 8192),
+                                                                    (1, 3, 4, 130, 48, 200), (70, 4, 1, 200, 16, 256), (1, 2, 1, 0, 8, 1)])
+def test_few_queries_over_a_cache_with_room_to_grow(hip, oracle, rng, batch, heads, new_len, old_len, hd, kv_rows):
+    """bf_hip_attention_forward_rows: the forward pass of fusedAttentionForward (fused_attention.cu:297) over K and V that
+    lie in buffers of kv_rows rows per sequence (hip::KVCache).  At most eight queries are served by a walk over the
+    cache instead of the tile kernels: compared with the oracle, with the tile kernels on the same operands, and with
+    rows past totalLen holding NaN, which no kernel may read; the output image is the rounded output."""
+    D, call = hip.DeviceTensor, hip.capi.call
+    dim, total, scale = heads * hd, old_len + new_len, float(f32(1.0) / np.sqrt(f32(hd)))
+    q, k, v = r(rng, batch, new_len, dim), r(rng, batch, total, dim), r(rng, batch, total, dim)
+    wide_k, wide_v = (np.full((batch, kv_rows, dim), np.nan, f32) for _ in range(2))
+    wide_k[:, :total], wide_v[:, :total] = k, v
+    dq_, dk_, dv_ = map(D.fromHost, (q, wide_k, wide_v))
+
+    def run(with_image):
+        out, m, l = D((batch, new_len, dim)), D((batch, heads, new_len)), D((batch, heads, new_len))
+        img = image_of(hip, (batch * new_len, dim)) if with_image else None
+        call("bf_hip_attention_forward_rows", dq_.ptr, dk_.ptr, dv_.ptr, out.ptr, img.ptr if img else None, dim if img else 0, m.ptr, l.ptr, batch,
+             heads, new_len, total, kv_rows, dim, ctypes.c_float(scale), old_len, None)
+        return out.toHost(), m.toHost(), l.toHost(), (as_f32(img.toHost()).reshape(batch, new_len, dim) if img else None)
+
+    o, m, l, img = run(True)
+    eo, em, el = oracle.attentionCoreForward(q, k, v, heads, scale, old_len)
+    for got, exp, name in ((o, eo, "O"), (m, em, "m"), (l, el, "l")):
+        assert_close(got, exp, what=f"{name} from the walk over the cache")
+    assert_bits_equal(img, oracle.roundToBf16(o), "O image")
+    o2, m2, l2, _ = run(False)
+    for got, exp, name in ((o2, o, "O"), (m2, m, "m"), (l2, l, "l")):
+        assert_bits_equal(got, exp, f"{name} of the same call again, without the image")
+    call("bf_hip_attention_set_route", 7 | 8)   # the default products, tile kernels only
+    try:
+        to, tm, tl, timg = run(True)
+    finally:
+        call("bf_hip_attention_set_route", 7)
+    for got, exp, name in ((to, o, "O"), (tm, m, "m"), (tl, l, "l")):
+        assert_close(got, exp, tol=2e-5, what=f"{name}: tile kernels against the walk")
+    assert_bits_equal(timg, oracle.roundToBf16(to), "O image of the tile kernels")
+
+
 @pytest.mark.parametrize("rows,classes", [(5, 16), (7, 1000), (300, 256), (3, 32000), (2, 40000)])
 def test_cross_entropy_gradient_image(hip, oracle, rng, rows, classes):
     D, call = hip.DeviceTensor, hip.capi.call
