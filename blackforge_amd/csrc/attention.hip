@@ -2422,14 +2422,14 @@ __global__ void __launch_bounds__(256) attnCombineChunksKernel(const float* __re
 // Forward pass of at most a few queries per sequence (a step of incremental decoding) without tiles: a 128-query tile
 // would hold one live row, and the pass is a walk over the cached keys and values anyway.  LPK lanes share a key: each
 // holds four of the head's columns (16 bytes of the key's row, the same of the value's), the dot product is a butterfly
-// over those lanes, and each such group of lanes walks every (256 / LPK)-th key of the workgroup's chunk, four keys a
+// over those lanes, and each such group of lanes walks every (256 / LPK)-th key of the workgroup's chunk, eight keys a
 // round, with its own running maximum, sum and output; the groups of a wavefront are joined by a butterfly, the four
 // wavefronts in order through LDS.  blockIdx.x is the chunk of keys, blockIdx.y the (batch, head, query).  Head dims that
 // are multiples of 4, 16-byte aligned operands.  Chunk c of numChunks > 1 writes its normalised output and statistics as
 // the tile kernels do (attnCombineChunksKernel joins them); a single chunk writes the results themselves.
 template <int LPK>
 __global__ void __launch_bounds__(256) attnFewQueriesKernel(AttnParams p) {
-    constexpr int GROUPS = 256 / LPK, KEYS = 4;
+    constexpr int GROUPS = 256 / LPK, KEYS = LPK <= 8 ? 4 : 8;   // keys a group of lanes has in flight per round
     __shared__ float sM[4], sL[4];
     __shared__ float4v sAcc[4][LPK];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;

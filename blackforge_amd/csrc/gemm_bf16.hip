@@ -1155,11 +1155,12 @@ __global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restr
 // Products of at most eight rows (a step of incremental decoding: one new token per sequence).  A 128 x 128 tile would
 // be all padding and six workgroups would walk a 768-wide weight alone; here the product is what it is by nature, a walk
 // over the weights: a wavefront owns COLS output columns (rows of Bt), each lane takes 16 bytes (eight bf16) of every
-// column per step and multiplies them with the same eight elements of the MR rows of A (which every wavefront reads: they
-// stay in cache), the lanes' sums are added by a butterfly, and lane r * COLS + j stores element (r, n0 + j) through the
-// epilogue.  Products in fp32 of the bf16 values, as on the MFMA; the order of additions is fixed (even and odd elements
-// of a lane's eight apart, then the butterfly), so results repeat bit for bit.  K, lda and ldb multiples of 8, operands
-// 16-byte aligned.
+// column per step, U steps loaded before any is used (a weight of a few MB is in flight all at once, which is what the
+// memory's latency asks for), and multiplies them with the same eight elements of the M rows of A, which the workgroup
+// holds in LDS.  The lanes' sums are added by a butterfly and lane r * COLS + j stores element (r, n0 + j) through the
+// epilogue (fuse 1 included: z and the image of act(z)).  Products in fp32 of the bf16 values, as on the MFMA; the order of
+// additions is fixed (even and odd elements of a lane's eight apart, then the butterfly), so results repeat bit for bit.
+// K, lda and ldb multiples of 8, operands 16-byte aligned, M * K bf16 within the LDS.
 __device__ __forceinline__ void dot8(const uint4v& a, const uint4v& b, float& even, float& odd) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1167,12 +1168,14 @@ __device__ __forceinline__ void dot8(const uint4v& a, const uint4v& b, float& ev
         odd = fmaf(__uint_as_float(a[i] & 0xffff0000u), __uint_as_float(b[i] & 0xffff0000u), odd);
     }
 }
-template <int MR, int COLS>
+__device__ __forceinline__ float actF1(int act, float v) { return act == BF_ACT_SILU ? siluF(v) : act == BF_ACT_GELU ? geluF(v) : reluF(v); }
+template <int MR, int COLS, int U>
 __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
                                                              Epilogue e, int M, int N, int K, int lda, int ldb) {
+    extern __shared__ __attribute__((aligned(16))) unsigned short aRows[];   // [M][K]
     const int lane = threadIdx.x & 63;
     const int n0 = (int(blockIdx.x) * 4 + int(threadIdx.x >> 6)) * COLS;
-    if (n0 >= N) return;                                     // whole wavefronts, no barrier below
+    const bool owner = n0 < N;                               // a wavefront past the last column only helps to stage A
     float even[MR][COLS], odd[MR][COLS];
 #pragma unroll
     for (int r = 0; r < MR; ++r)
@@ -1181,19 +1184,40 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
     const unsigned short* bRow[COLS];
 #pragma unroll
     for (int j = 0; j < COLS; ++j) bRow[j] = Bt + size_t(min(n0 + j, N - 1)) * ldb;   // a column past the end repeats the last one, unstored
-#pragma unroll 2
-    for (int k = lane * 8; k < K; k += 512) {
-        uint4v b[COLS];
+    uint4v b[U][COLS];
+    const uint4v none = {0u, 0u, 0u, 0u};
+    auto loadSteps = [&](int k0) {
 #pragma unroll
-        for (int j = 0; j < COLS; ++j) b[j] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(bRow[j] + k));
+        for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int r = 0; r < MR; ++r) {
-            if (r < M) {
-                const uint4v a = *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k);
+            for (int j = 0; j < COLS; ++j)
+                b[u][j] = owner && k0 + u * 512 < K ? __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(bRow[j] + k0 + u * 512)) : none;
+    };
+    int k0 = lane * 8;
+    loadSteps(k0);                                           // in flight while A is staged
+    for (int at = int(threadIdx.x) * 8; at < M * K; at += 2048) {
+        const int r = at / K, k = at - r * K;                // K is a multiple of 8: a group of eight lies in one row
+        *reinterpret_cast<uint4v*>(aRows + at) = *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k);
+    }
+    __syncthreads();
+    if (!owner) return;
+    while (k0 < K) {
 #pragma unroll
-                for (int j = 0; j < COLS; ++j) dot8(a, b[j], even[r][j], odd[r][j]);
+        for (int u = 0; u < U; ++u) {
+            const int k = k0 + u * 512;
+            if (k < K) {
+#pragma unroll
+                for (int r = 0; r < MR; ++r) {
+                    if (r < M) {
+                        const uint4v a = *reinterpret_cast<const uint4v*>(aRows + r * K + k);
+#pragma unroll
+                        for (int j = 0; j < COLS; ++j) dot8(a, b[u][j], even[r][j], odd[r][j]);
+                    }
+                }
             }
         }
+        k0 += 512 * U;
+        if (k0 < K) loadSteps(k0);
     }
 #pragma unroll
     for (int r = 0; r < MR; ++r)
@@ -1209,18 +1233,30 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
                 if (e.bias) v += e.bias[col];
                 if (e.residual) v += e.residual[size_t(r) * N + col];
                 C[size_t(r) * e.splitN + (col - which * e.splitN)] = v;
+                if (e.fuse == 1) e.image[size_t(r) * N + col] = toBf16Bits(actF1(e.act, v));
             }
         }
 }
 template <int MR>
 int launchFewRows(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K, size_t lda, size_t ldb,
                   hipStream_t s) {
+    const size_t smem = M * K * sizeof(unsigned short);
     // one column a wavefront until that gives every SIMD several wavefronts; four from there on (fewer butterflies per byte)
-    if (N <= 8192) gemmBf16FewRowsKernel<MR, 1><<<unsigned((N + 3) / 4), 256, 0, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb));
-    else gemmBf16FewRowsKernel<MR, 4><<<unsigned((N + 15) / 16), 256, 0, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb));
+    if (N <= 8192) {
+        auto kernel = gemmBf16FewRowsKernel<MR, 1, 8>;
+        int st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
+        if (st != BF_OK) return st;
+        kernel<<<unsigned((N + 3) / 4), 256, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb));
+    } else {
+        auto kernel = gemmBf16FewRowsKernel<MR, 4, 2>;
+        int st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
+        if (st != BF_OK) return st;
+        kernel<<<unsigned((N + 15) / 16), 256, smem, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb));
+    }
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
+constexpr size_t kFewRowsLds = 128 * 1024;   // what the rows of A may take of a compute unit's 160 KB
 
 // The same kernel for operands that lie the other way round: C[M,N] = A^T * B with A [K, lda] and B [K, ldb], the
 // contraction index K running over ROWS (a weight gradient dW = X^T * G: both the activations X and the gradient G have
@@ -1630,9 +1666,10 @@ int launchGemmTn(const unsigned short* A, const unsigned short* B, const Epilogu
 // Whether launchGemmNt takes a product of this shape with Epilogue::fuse set: a kernel chosen by the caller (tests and
 // tuning) never does, so that the separate passes stay reachable, and neither do products too small for the
 // one-tile-per-workgroup kernels.
-bool fusedActivationFits(size_t M, size_t N) {
+bool fusedActivationFits(size_t M, size_t N, size_t K, int fuse) {
     if (g_ntRoute != BF_GEMM_ROUTE_AUTO || N % 8 != 0) return false;
     const size_t cus = size_t(computeUnits());
+    if (M <= 8) return fuse == 1 && K % 8 == 0 && M * K * sizeof(unsigned short) <= kFewRowsLds;   // the walk over the weights
     const size_t halfTiles = ((M + 127) / 128) * ((N + 255) / 256);   // the 256-row form needs no fewer
     return halfTiles >= cus * 3 / 4 || (N % 192 == 0 && ((M + 127) / 128) * (N / 192) >= cus * 3 / 4);
 }
@@ -1662,7 +1699,7 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
             return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s, g_ntRoute == BF_GEMM_ROUTE_WIDE_192_PERSISTENT);
         default: break;
     }
-    if (M <= 8 && epi.fuse == 0 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
+    if (M <= 8 && epi.fuse != 2 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && M * K * sizeof(unsigned short) <= kFewRowsLds &&
         ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) & 15u) == 0) {   // a walk over the weights, no tiles
         if (M == 0 || N == 0) return BF_OK;
         return M == 1 ? launchFewRows<1>(A, Bt, epi, M, N, K, lda, ldb, s) : M == 2 ? launchFewRows<2>(A, Bt, epi, M, N, K, lda, ldb, s)
@@ -2402,7 +2439,7 @@ int bf_hip_feedforward_bf16(const float* x, const float* w1, const float* b1, co
     if (st != BF_OK) return st;
     // the activation's image is written by the product's own store when the product is large enough for the kernels
     // that can do it (the same bits as the separate pass over z)
-    const bool fused = fusedActivationFits(m, hidden) && ((reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(b1)) & 15u) == 0;
+    const bool fused = fusedActivationFits(m, hidden, d, 1) && ((reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(b1)) & 15u) == 0;
     Epilogue first{{z, nullptr, nullptr}, int(hidden), b1, nullptr};
     if (fused) { first.fuse = 1; first.act = act; first.image = hImage; }
     st = launchGemmNt(xImg, wImg, first, m, hidden, d, d, d, s);
@@ -2477,7 +2514,7 @@ int bf_hip_feedforward_bf16_backward_img(const float* x, const uint16_t* xImage,
     // When the product is large enough for the kernels that can do it, its store multiplies by act'(z) and writes the image
     // itself (dH never exists in memory; the same bits as the separate pass), with dz's column sums per 32-row block, which
     // a bias-gradient pass over those few rows finishes.
-    const bool fused = fusedActivationFits(m, hidden) && ((reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(dB1)) & 15u) == 0;
+    const bool fused = fusedActivationFits(m, hidden, d, 2) && ((reinterpret_cast<uintptr_t>(z) | reinterpret_cast<uintptr_t>(dB1)) & 15u) == 0;
     const size_t rowBlocks = (m + 31) / 32;
     Scratch dH(fused ? 0 : m * hidden * sizeof(float)), dzImg(m * hidden * sizeof(unsigned short));
     Scratch partial(fused && dB1 ? rowBlocks * hidden * sizeof(float) : 0);

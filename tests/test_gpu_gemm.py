@@ -384,13 +384,15 @@ def bf16_bits_to_f32(raw, rows, cols):
 
 @pytest.mark.parametrize("m,d,hidden,act", [(64, 32, 128, 0), (64, 32, 128, 1), (64, 32, 128, 2), (300, 72, 264, 0), (300, 72, 264, 1),
                                             (1000, 64, 2048, 2), (4096, 256, 1024, 0), (4096, 256, 1024, 1), (8192, 768, 3072, 0),
-                                            (2048, 8, 8, 0), (513, 512, 512, 1), (256, 4096, 256, 1), (256, 4096, 256, 2)])
+                                            (2048, 8, 8, 0), (513, 512, 512, 1), (256, 4096, 256, 1), (256, 4096, 256, 2),
+                                            (1, 768, 3072, 1), (3, 72, 264, 0), (8, 1032, 520, 2), (1, 8, 8, 1), (8, 8200, 64, 0)])
 def test_feed_forward_with_the_elementwise_steps_in_the_gemm_stores(hip, oracle, rng, m, d, hidden, act):
     """bf_hip_feedforward_bf16[_backward] (feedForwardForwardCached / feedForwardBackwardCached in the bf16 mode,
     ops_transformer.cu:182-215, autodiff.cu:719-750) against the same block built from the separate operators, which are
     themselves checked against the oracle: same roundings, so the agreement is tight.  Shapes cover the small-tile GEMM with
-    the transposed-image weight gradients, ragged row counts, and the large-tile kernels with fragments transposed in LDS;
-    act 0/1/2 = silu/gelu/relu."""
+    the transposed-image weight gradients, ragged row counts, the large-tile kernels with fragments transposed in LDS, and
+    blocks of at most eight rows (a step of incremental decoding: products as walks over the weights, the activation in the
+    first one's store; the last case's rows are too long for that walk's LDS); act 0/1/2 = silu/gelu/relu."""
     D, ops = hip.DeviceTensor, hip.ops
     x, w1, b1 = r(rng, m, d), r(rng, d, hidden, scale=0.1), r(rng, hidden, scale=0.5)
     w2, b2, res, g = r(rng, hidden, d, scale=0.1), r(rng, d), r(rng, m, d), r(rng, m, d)
