@@ -2427,6 +2427,9 @@ __global__ void __launch_bounds__(256) attnCombineChunksKernel(const float* __re
 // wavefronts in order through LDS.  blockIdx.x is the chunk of keys, blockIdx.y the (batch, head, query).  Head dims that
 // are multiples of 4, 16-byte aligned operands.  Chunk c of numChunks > 1 writes its normalised output and statistics as
 // the tile kernels do (attnCombineChunksKernel joins them); a single chunk writes the results themselves.
+// exp(x) for x <= 0 as the hardware's 2^(x log2 e): the walk below is a chain of a few dozen dependent steps on one
+// wavefront, where the library routine's forty instructions apiece are a large part of the kernel's time
+__device__ __forceinline__ float expFast(float x) { return fastExp2(x * kLog2e); }
 template <int LPK>
 __global__ void __launch_bounds__(256) attnFewQueriesKernel(AttnParams p) {
     constexpr int GROUPS = 256 / LPK, KEYS = LPK <= 8 ? 4 : 8;   // keys a group of lanes has in flight per round
@@ -2469,12 +2472,12 @@ __global__ void __launch_bounds__(256) attnFewQueriesKernel(AttnParams p) {
             sc[u] = j0 + u * GROUPS < end ? dot * p.scale : -INFINITY;
             roundMax = fmaxf(roundMax, sc[u]);
         }
-        const float keep = expf(m - roundMax);                 // m = -inf at the first round: 0 (key j0 itself is below `end`)
+        const float keep = expFast(m - roundMax);                 // m = -inf at the first round: 0 (key j0 itself is below `end`)
         l *= keep;
         acc = acc * keep;
 #pragma unroll
         for (int u = 0; u < KEYS; ++u) {
-            const float w = expf(sc[u] - roundMax);
+            const float w = expFast(sc[u] - roundMax);
             l += w;
             acc = acc + v4[u] * w;
         }
@@ -2484,7 +2487,7 @@ __global__ void __launch_bounds__(256) attnFewQueriesKernel(AttnParams p) {
     auto join = [&](float om, float ol, float4v oacc) {
         const float mm = fmaxf(m, om);
         if (mm == -INFINITY) return;                           // neither side has seen a key
-        const float mine = expf(m - mm), theirs = expf(om - mm);
+        const float mine = expFast(m - mm), theirs = expFast(om - mm);
         l = l * mine + ol * theirs;
         acc = acc * mine + oacc * theirs;
         m = mm;

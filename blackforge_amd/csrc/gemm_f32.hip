@@ -364,8 +364,136 @@ __global__ void __launch_bounds__(kBlock) sliceSumKernel(const float* __restrict
     const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= count) return;
     float sum = partial[i];
-    for (int s = 1; s < slices; ++s) sum += partial[size_t(s) * stride + i];
+    for (int s0 = 1; s0 < slices; s0 += 8) {   // eight loads in flight, added in index order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = s0 + u < slices ? partial[size_t(s0 + u) * stride + i] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (s0 + u < slices) sum += v[u];
+    }
     C[i] = withAdds(sum, bias, residual, i, i % N);
+}
+
+// Products of at most eight rows, C[M, N] = A[M, K] B[K, N] (a step of incremental decoding: one new token per sequence),
+// as a walk over B: a lane owns VEC adjacent columns, the WAVES wavefronts of a workgroup take every WAVES-th row of the
+// workgroup's K slice, eight rows loaded before any is used, and multiply them with the slice's elements of A, which the
+// workgroup holds in LDS (read as broadcasts).  The wavefronts' sums are added in order through LDS; with several K
+// slices (blockIdx.y) a slice writes its sums `sliceStride` floats after the slice before it and sliceSumKernel adds them,
+// with one slice the adds of the epilogue are made here.  VEC 4: N a multiple of 4 and B 16-byte aligned.
+template <int MR, int VEC, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) gemmF32FewRowsKernel(const float* __restrict__ A, const float* __restrict__ B, float* out,
+                                                            int M, int N, int K, int kPer, size_t sliceStride,
+                                                            const float* __restrict__ bias, const float* residual) {   // residual may be out
+    extern __shared__ float fewRowsLds[];
+    constexpr int U = 8, WIDTH = 64 * VEC;
+    float* aRows = fewRowsLds;                      // [MR][kPer]
+    float* sums = fewRowsLds + MR * kPer;           // [WAVES][MR][WIDTH]
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int col = (int(blockIdx.x) * 64 + lane) * VEC;
+    const int kBeg = int(blockIdx.y) * kPer, kEnd = min(K, kBeg + kPer), kLen = kEnd - kBeg;
+    float b[U][VEC];
+    auto loadRows = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = k0 + WAVES * u;
+            const bool in = k < kEnd && col < N;
+            if constexpr (VEC == 4) {
+                const float4v v = in ? __builtin_nontemporal_load(reinterpret_cast<const float4v*>(B + size_t(k) * N + col)) : float4v{0.0f, 0.0f, 0.0f, 0.0f};
+                b[u][0] = v.x; b[u][1] = v.y; b[u][2] = v.z; b[u][3] = v.w;
+            } else {
+                b[u][0] = in ? __builtin_nontemporal_load(B + size_t(k) * N + col) : 0.0f;
+            }
+        }
+    };
+    int k0 = kBeg + wave;
+    loadRows(k0);                                   // in flight while A is staged
+    for (int i = t; i < M * kLen; i += 64 * WAVES) {
+        const int r = i / kLen, k = i - r * kLen;
+        aRows[r * kPer + k] = A[size_t(r) * K + kBeg + k];
+    }
+    __syncthreads();
+    float acc[MR][VEC];
+#pragma unroll
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[r][v] = 0.0f;
+    while (k0 < kEnd) {                             // the same for every lane of a wavefront
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = k0 + WAVES * u;
+            if (k < kEnd) {
+#pragma unroll
+                for (int r = 0; r < MR; ++r) {
+                    if (r < M) {
+                        const float a = aRows[r * kPer + (k - kBeg)];
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) acc[r][v] = fmaf(a, b[u][v], acc[r][v]);
+                    }
+                }
+            }
+        }
+        k0 += WAVES * U;
+        if (k0 < kEnd) loadRows(k0);
+    }
+#pragma unroll
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) sums[((wave * MR + r) * 64 + lane) * VEC + v] = acc[r][v];
+    __syncthreads();
+    float* dst = out + size_t(blockIdx.y) * sliceStride;
+    for (int i = t; i < M * WIDTH; i += 64 * WAVES) {
+        const int r = i / WIDTH, c = i - r * WIDTH, column = int(blockIdx.x) * WIDTH + c;
+        if (column < N) {
+            float total = sums[r * WIDTH + c];
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) total += sums[(w * MR + r) * WIDTH + c];
+            const size_t at = size_t(r) * N + column;
+            dst[at] = withAdds(total, bias, residual, at, size_t(column));
+        }
+    }
+}
+template <int MR>
+int launchFewRowsF32(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, const float* bias, const float* residual,
+                     hipStream_t s, bool* served) {
+    *served = false;
+    constexpr int WAVES = MR <= 4 ? 8 : 4;          // WAVES * MR * 256 sums in LDS
+    const bool vec = N % 4 == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
+    const size_t width = vec ? 256 : 64, colBlocks = (N + width - 1) / width;
+    // K slices of at least one round of loads per wavefront (8 * WAVES rows), at most 32 of them, about two workgroups
+    // per compute unit; the slices are summed by a second kernel
+    const size_t cus = size_t(computeUnits()), round = size_t(8) * WAVES;
+    size_t slices = std::max<size_t>(1, std::min<size_t>(std::min<size_t>((K + round - 1) / round, 32), 2 * cus / colBlocks));
+    size_t kPer = ((K + slices - 1) / slices + 3) / 4 * 4;
+    slices = (K + kPer - 1) / kPer;
+    const size_t smem = (size_t(MR) * kPer + size_t(WAVES) * MR * width) * sizeof(float);
+    if (smem > 96 * 1024) return BF_OK;             // rows of A too long for the LDS: the tile kernels serve
+    const size_t count = M * N;
+    Scratch partial(slices > 1 ? slices * count * sizeof(float) : 0);
+    if (partial.status != BF_OK) return partial.status;
+    float* out = slices > 1 ? partial.as<float>() : C;
+    const dim3 grid{unsigned(colBlocks), unsigned(slices), 1u};
+    int st;
+    if (vec) {
+        auto kernel = gemmF32FewRowsKernel<MR, 4, WAVES>;
+        st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
+        if (st != BF_OK) return st;
+        kernel<<<grid, 64 * WAVES, smem, s>>>(A, B, out, int(M), int(N), int(K), int(kPer), count, slices > 1 ? nullptr : bias,
+                                              slices > 1 ? nullptr : residual);
+    } else {
+        auto kernel = gemmF32FewRowsKernel<MR, 1, WAVES>;
+        st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
+        if (st != BF_OK) return st;
+        kernel<<<grid, 64 * WAVES, smem, s>>>(A, B, out, int(M), int(N), int(K), int(kPer), count, slices > 1 ? nullptr : bias,
+                                              slices > 1 ? nullptr : residual);
+    }
+    BF_LAUNCH_CHECK();
+    if (slices > 1) {
+        sliceSumKernel<<<gridFor(count, kBlock), kBlock, 0, s>>>(partial.as<float>(), C, count, count, int(slices), N, bias, residual);
+        BF_LAUNCH_CHECK();
+    }
+    *served = true;
+    return BF_OK;
 }
 
 template <int BM, int BN>
@@ -398,8 +526,16 @@ int gemmF32(int transA, int transB, const float* A, const float* B, float* C, si
     }
     BF_REQUIRE(A && B, "NULL operand");
     BF_REQUIRE((M + 63) / 64 <= 65535, "M too large");
-    // Large tiles once they alone can fill the chip twice over; small tiles otherwise.
     hipStream_t s = asStream(stream);
+    if (!transA && !transB && M <= 8 && N < (size_t(1) << 31) && K < (size_t(1) << 31)) {   // a walk over B, no tiles
+        bool served = false;
+        int st = M == 1 ? launchFewRowsF32<1>(A, B, C, M, N, K, bias, residual, s, &served)
+               : M == 2 ? launchFewRowsF32<2>(A, B, C, M, N, K, bias, residual, s, &served)
+               : M <= 4 ? launchFewRowsF32<4>(A, B, C, M, N, K, bias, residual, s, &served)
+                        : launchFewRowsF32<8>(A, B, C, M, N, K, bias, residual, s, &served);
+        if (st != BF_OK || served) return st;
+    }
+    // Large tiles once they alone can fill the chip twice over; small tiles otherwise.
     const size_t cus = size_t(computeUnits());
     size_t bigTiles = ((M + 127) / 128) * ((N + 127) / 128);
     if (bigTiles >= 2 * cus) return launchGemm<128, 128>(transA, transB, A, B, C, M, N, K, 1, K, 0, bias, residual, s);

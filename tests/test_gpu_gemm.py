@@ -47,6 +47,30 @@ def test_fp32_gemm_family(hip, oracle, rng, m, k, n):
     assert_close(ops.linear(da, db, D.fromHost(bias)).toHost(), oracle.linear(a, b, bias), what="linear")
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 768, 768), (1, 3072, 768), (1, 768, 32003), (2, 72, 9000), (3, 520, 41), (5, 1032, 8200), (8, 768, 2304),
+                                   (7, 8, 1), (1, 4100, 16), (4, 44, 300), (8, 30000, 64), (2, 1, 5)])
+def test_fp32_products_of_a_few_rows(hip, oracle, rng, m, k, n):
+    """matmul / linear (ops.hpp:14,30) with at most eight rows, the shape of a step of incremental decoding (model.cpp:169):
+    served by a walk over the weights with the contraction cut into slices.  Widths that take 16-byte loads and widths that
+    do not, one slice and many, rows of A too long for the walk's LDS (the tile kernels serve), adds in the store and after
+    the slices are summed, accumulation in place."""
+    D, ops, call = hip.DeviceTensor, hip.ops, hip.capi.call
+    a, b, bias, res = r(rng, m, k), r(rng, k, n), r(rng, n), r(rng, m, n)
+    da, db, dbias, dres = map(D.fromHost, (a, b, bias, res))
+    expected = (a.astype(np.float64) @ b.astype(np.float64)).astype(f32)
+    if m * k * n <= 5_000_000:
+        assert_close(oracle.matmul(a, b), expected, tol=1e-5, what="oracle vs float64")
+    product = ops.matmul(da, db)
+    assert_close(product.toHost(), expected, tol=1e-5, what="few-row product")
+    assert_bits_equal(ops.matmul(da, db).toHost(), product.toHost(), "the same product twice")
+    out = D((m, n))
+    call("bf_hip_gemm_f32_adds", 0, 0, da.ptr, db.ptr, dbias.ptr, dres.ptr, out.ptr, m, n, k, None)
+    assert_bits_equal(out.toHost(), ops.addBiasResidual(product, dbias, dres).toHost(), "product + bias + residual")
+    acc = D.fromHost(res)
+    call("bf_hip_gemm_f32_adds", 0, 0, da.ptr, db.ptr, None, acc.ptr, acc.ptr, m, n, k, None)
+    assert_bits_equal(acc.toHost(), ops.add(product, dres).toHost(), "residual += product")
+
+
 def test_fp32_gemm_large_tile_path(hip, rng):
     """Big enough for the 128x128-tile kernel; checked against float64 numpy on a sample of rows."""
     D, ops = hip.DeviceTensor, hip.ops
