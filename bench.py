@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X operator backend on the headline workload.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras] [--train LIST]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras] [--no-decode] [--train LIST]
 
 Workload (BASELINE.json configs[2], the one the fused-attention TFLOP/s metric is quoted on):
 standalone causal fused attention in fp32, batch 8, heads 16, seq 2048, head_dim 64, Q/K/V/dOut
@@ -640,6 +640,68 @@ def bench_train_step(bf, name, steps, warmup, with_graph=True):
     return out
 
 
+def bench_decode(bf, tokens=32, prompt=1024):
+    """Incremental decoding (Model::forwardIncremental, model.cu:385-424) of the GPT-small shape, one sequence: a prompt,
+    then `tokens` single-token steps, timed.  A step reads every Linear weight once (bf16 images in bf16 mode, 2 bytes a
+    parameter; fp32 otherwise) and the cached keys and values (fp32): that is the algorithmic traffic the rate is set against."""
+    from blackforge_amd import hostlayer as hl
+    c = TRAIN_CONFIGS["gpt_small"]
+    out = {}
+    for mode, bf16 in (("bf16", True), ("fp32", False)):
+        model = hl.HostModel(lm_layers(hl, c["vocab"], c["dim"], 2 * prompt, c["heads"], c["ffn"], c["act"], c["blocks"]), use_bf16=bf16)
+        rng = np.random.default_rng(42)
+        for i, count in enumerate(model.counts):
+            model.set_value(i, np.resize(rng.standard_normal(65537, dtype=np.float32) * np.float32(0.02), count))
+        D = bf.DeviceTensor
+        model.resetGenerationState()
+        model.forwardIncremental(D.fromHost(rng.integers(0, c["vocab"], (1, prompt)).astype(np.float32)), read=False)
+        # greedy generation as the reference's `generate` runs it (main.cpp:594-617): the next token is the device-side
+        # argmax of the last position's logits, one index read back per step
+        def step():
+            token = D.fromHost(np.array([[float(model.argmaxLast(c["vocab"]))]], np.float32))
+            model.forwardIncremental(token, read=False)
+        for _ in range(3):
+            step()
+        bf.capi.call("bf_hip_synchronize")
+        t0 = time.perf_counter()
+        for _ in range(tokens):
+            step()
+        bf.capi.call("bf_hip_synchronize")
+        ms = (time.perf_counter() - t0) * 1e3 / tokens
+        # the same generation with token and position kept on the device (Model::generateGreedy: no read-back inside the
+        # loop); the prompt is inside the clock, so two lengths are timed and their difference is the cost of the extra tokens
+        prompt_ids = D.fromHost(rng.integers(0, c["vocab"], (1, prompt)).astype(np.float32))
+        model.generateGreedy(prompt_ids, 4)
+        times = {}
+        for n in (tokens, 9 * tokens):
+            bf.capi.call("bf_hip_synchronize")
+            t0 = time.perf_counter()
+            model.generateGreedy(prompt_ids, n)
+            times[n] = (time.perf_counter() - t0) * 1e3
+        on_device_ms = (times[9 * tokens] - times[tokens]) / (8 * tokens)
+        matrix_params = c["blocks"] * (4 * c["dim"] ** 2 + 2 * c["dim"] * c["ffn"]) + c["dim"] * c["vocab"]
+        context = prompt + 3 + tokens // 2
+        bytes_per_token = matrix_params * (2 if bf16 else 4) + c["blocks"] * 2 * context * c["dim"] * 4
+        gbs = bytes_per_token / (ms * 1e-3) / 1e9
+        on_device_context = prompt + 5 * tokens
+        on_device_bytes = matrix_params * (2 if bf16 else 4) + c["blocks"] * 2 * on_device_context * c["dim"] * 4
+        on_device_gbs = on_device_bytes / (on_device_ms * 1e-3) / 1e9
+        out[mode] = {"ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1), "context": context,
+                     "algorithmic_bytes_per_token": bytes_per_token,
+                     "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)},
+                     "on_device_loop": {"what": "Model::generateGreedy: argmax, token and position stay on the device, the host launches ahead; "
+                                               f"(time of {9 * tokens} tokens - time of {tokens}) / {8 * tokens}",
+                                       "ms_per_token": round(on_device_ms, 4), "tokens_per_s": round(1e3 / on_device_ms, 1), "context": on_device_context,
+                                       "algorithmic_bytes_per_token": on_device_bytes,
+                                       "roofline": {"bound": "hbm", "achieved": round(on_device_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                                    "frac": round(on_device_gbs / PEAK_HBM_GBS, 4)}}}
+        del model
+    out["workload"] = (f"GPT-small shape (BASELINE.json configs[3]), one sequence, prompt of {prompt} tokens, then {tokens} single-token steps "
+                       "of greedy generation: device-side argmax of the last logits, then Model::forwardIncremental on that token (wall clock around "
+                       "the steps: about a hundred launches a token, bounded by their latency)")
+    return out
+
+
 def extras_summary(extras):
     """The north-star targets in three numbers: the bf16 projection at 4096^3 against the bf16 MFMA peak, and the worst and
     the median bandwidth kernel against the HBM peak."""
@@ -664,6 +726,7 @@ def main():
                     "steady clocks (3 warm-up steps read 6 %% slower than 20)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the bandwidth kernels and the bf16 GEMMs")
+    ap.add_argument("--no-decode", action="store_true", help="skip the incremental-decoding leg")
     ap.add_argument("--no-graph", action="store_true", help="skip the recorded (HIP graph) variant of the tiny-LM step; for runs under a "
                     "profiler, whose kernel tracing does not survive a stream capture on this stack")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -752,6 +815,8 @@ def main():
         line["train_step"] = {name: (bench_mlp if name == "mlp" else lambda b, s_, w_: bench_train_step(b, name, s_, w_, not args.no_graph))(
                                   bf, max(3, args.steps // 2), max(1, args.warmup // 2))
                               for name in args.train.split(",")}
+    if not args.no_decode:
+        line["decode"] = bench_decode(bf)
     if not args.no_extras:
         line["extras"] = bench_extras(bf, min(10, max(5, args.steps // 2)))   # ten launches a kernel: what profiles/hbm_kernels_and_gemm.md describes
         line["extras_summary"] = extras_summary(line["extras"])

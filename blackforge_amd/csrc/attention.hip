@@ -70,6 +70,9 @@ struct AttnParams {
     int kvRows;          // rows per batch element of the K and V tensors (totalLen, whatever the chunk)
     int chunkKeys, numChunks;
     size_t partOutStride, partStatStride;
+    // attnFewQueriesKernel only: when set, the number of cached positions is read from here instead of oldLen (a step
+    // launched before the host knows the position); the chunks then cover all kvRows and may be empty
+    const int* oldLenPtr;
 };
 
 // A forward kernel's first statement: narrows the parameters to this workgroup's chunk of keys.  Every chunk starts at
@@ -2447,7 +2450,8 @@ __global__ void __launch_bounds__(256) attnFewQueriesKernel(AttnParams p) {
     const float* vb = p.v + size_t(b) * p.kvRows * dim + column;
     const float4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
     const float4v q4 = live ? loadf4(p.q + size_t(bi) * dim + column) : zero;
-    const int limit = p.oldLen + i + 1;                        // keys 0 .. oldLen + i are visible to query i
+    const int oldLen = p.oldLenPtr ? *p.oldLenPtr : p.oldLen;
+    const int limit = min(oldLen + i + 1, p.kvRows);           // keys 0 .. oldLen + i are visible to query i
     const int start = c * p.chunkKeys;
     const int end = c == p.numChunks - 1 ? limit : min(start + p.chunkKeys, limit);
 
@@ -2509,7 +2513,7 @@ __global__ void __launch_bounds__(256) attnFewQueriesKernel(AttnParams p) {
         m = sM[0]; l = sL[0]; acc = sAcc[0][t];
 #pragma unroll
         for (int w = 1; w < 4; ++w) join(sM[w], sL[w], sAcc[w][t]);
-        const float inv = 1.0f / l;                            // every chunk holds a key visible to every query
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;          // an empty chunk (a cache read by its device-side length) gives zeros
         const float4v o4 = acc * inv;
         const size_t stat = (size_t(b) * p.heads + h) * p.newLen + i;
         const size_t at = size_t(bi) * dim + size_t(h) * hd + d0;
@@ -2536,6 +2540,43 @@ bool vec4Ok(const AttnParams& p, std::initializer_list<const void*> ptrs) {
     for (const void* q : ptrs)
         if (q && (reinterpret_cast<uintptr_t>(q) & 15u)) return false;
     return true;
+}
+
+// The walk over the cache for at most eight queries per sequence: what it asks of the operands
+bool fewQueriesFit(const AttnParams& p, size_t batch, size_t heads, size_t newLen) {
+    return newLen <= 8 && batch * heads * newLen <= 65535 && vec4Ok(p, {p.q, p.k, p.v, p.out});
+}
+// p: the whole problem, outputs included; the keys in numChunks chunks of chunkKeys
+int launchFewQueries(const AttnParams& p, size_t batch, size_t heads, size_t newLen, size_t chunkKeys, size_t numChunks, hipStream_t s) {
+    const size_t rows = batch * heads * newLen;
+    AttnParams c = p;
+    c.chunkKeys = int(chunkKeys);
+    c.numChunks = int(numChunks);
+    const size_t outFloats = batch * newLen * size_t(p.dim), statFloats = batch * heads * newLen;
+    Scratch part(numChunks > 1 ? numChunks * (outFloats + 2 * statFloats) * sizeof(float) : 0);
+    if (part.status != BF_OK) return part.status;
+    if (numChunks > 1) {
+        c.partOutStride = outFloats;
+        c.partStatStride = statFloats;
+        c.out = part.as<float>();
+        c.m = c.out + numChunks * outFloats;
+        c.l = c.m + numChunks * statFloats;
+    }
+    const dim3 g{unsigned(numChunks), unsigned(rows), 1u};
+    const int lanes = p.hd <= 32 ? 8 : p.hd <= 64 ? 16 : p.hd <= 128 ? 32 : 64;
+    switch (lanes) {
+        case 8: attnFewQueriesKernel<8><<<g, 256, 0, s>>>(c); break;
+        case 16: attnFewQueriesKernel<16><<<g, 256, 0, s>>>(c); break;
+        case 32: attnFewQueriesKernel<32><<<g, 256, 0, s>>>(c); break;
+        default: attnFewQueriesKernel<64><<<g, 256, 0, s>>>(c); break;
+    }
+    BF_LAUNCH_CHECK();
+    if (numChunks > 1) {
+        attnCombineChunksKernel<<<unsigned(rows), 256, 0, s>>>(c.out, c.m, c.l, p.out, p.outImg, p.imgLd, p.m, p.l, int(heads), int(newLen), p.dim, p.hd,
+                                                            int(numChunks), outFloats, statFloats);
+        BF_LAUNCH_CHECK();
+    }
+    return BF_OK;
 }
 
 // KIND 0 forward, 1 dQ, 2 dK/dV, 3 dK/dV that also stores dS, 4 dQ from stored dS
@@ -2677,39 +2718,13 @@ int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v
     hipStream_t s = asStream(stream);
     const size_t cus = size_t(computeUnits());
     // At most eight queries per sequence (incremental decoding): the walk over the cache, LPK lanes a key
-    if (newLen <= 8 && batch * heads * newLen <= 65535 && vec4Ok(p, {q, k, v, out}) && (gAttnRoute & BF_ATTN_ROUTE_TILES_ONLY) == 0) {
+    if (fewQueriesFit(p, batch, heads, newLen) && (gAttnRoute & BF_ATTN_ROUTE_TILES_ONLY) == 0) {
         const size_t rows = batch * heads * newLen;
         const size_t wanted = std::max<size_t>(1, (4 * cus + rows - 1) / rows);   // about four workgroups per compute unit
-        size_t chunkKeys = std::max<size_t>(128, ((totalLen + wanted - 1) / wanted + 127) / 128 * 128);
+        const size_t chunkKeys = std::max<size_t>(128, ((totalLen + wanted - 1) / wanted + 127) / 128 * 128);
+        // a chunk starts at or before the first query's own position, so that every query sees a key in every chunk
         const size_t numChunks = std::max<size_t>(1, std::min((totalLen + chunkKeys - 1) / chunkKeys, oldLen / chunkKeys + 1));
-        AttnParams c = p;
-        c.chunkKeys = int(chunkKeys);
-        c.numChunks = int(numChunks);
-        const size_t outFloats = batch * newLen * dim, statFloats = batch * heads * newLen;
-        Scratch part(numChunks > 1 ? numChunks * (outFloats + 2 * statFloats) * sizeof(float) : 0);
-        if (part.status != BF_OK) return part.status;
-        if (numChunks > 1) {
-            c.partOutStride = outFloats;
-            c.partStatStride = statFloats;
-            c.out = part.as<float>();
-            c.m = c.out + numChunks * outFloats;
-            c.l = c.m + numChunks * statFloats;
-        }
-        const dim3 g{unsigned(numChunks), unsigned(rows), 1u};
-        const int lanes = p.hd <= 32 ? 8 : p.hd <= 64 ? 16 : p.hd <= 128 ? 32 : 64;
-        switch (lanes) {
-            case 8: attnFewQueriesKernel<8><<<g, 256, 0, s>>>(c); break;
-            case 16: attnFewQueriesKernel<16><<<g, 256, 0, s>>>(c); break;
-            case 32: attnFewQueriesKernel<32><<<g, 256, 0, s>>>(c); break;
-            default: attnFewQueriesKernel<64><<<g, 256, 0, s>>>(c); break;
-        }
-        BF_LAUNCH_CHECK();
-        if (numChunks > 1) {
-            attnCombineChunksKernel<<<unsigned(rows), 256, 0, s>>>(c.out, c.m, c.l, out, outImage, imageLd, m, l, int(heads), int(newLen), int(dim), p.hd,
-                                                                int(numChunks), outFloats, statFloats);
-            BF_LAUNCH_CHECK();
-        }
-        return BF_OK;
+        return launchFewQueries(p, batch, heads, newLen, chunkKeys, numChunks, s);
     }
     // Few queries against many keys (a step of incremental decoding: one workgroup per head would walk all the keys alone):
     // the keys go to the workgroups in chunks, each with its own statistics, and a second kernel puts the chunks together.
@@ -2743,6 +2758,31 @@ int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v
         }
     }
     return dispatch<0>(p, vec4Ok(p, {q, k, v, out}), grid, s);
+}
+
+int bf_hip_attention_forward_rows_indirect(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd,
+                                           float* m, float* l, size_t batch, size_t heads, size_t newLen, size_t kvRows, size_t dim, float scale,
+                                           const int* oldLen, bf_stream_t stream) {
+    int st = checkShapes(__func__, batch, heads, newLen, kvRows, dim, 0);
+    if (st != BF_OK) return st;
+    if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(q && k && v && (out || outImage) && m && l && oldLen, "NULL pointer");
+    BF_REQUIRE(kvRows < (size_t(1) << 31), "kvRows too large");
+    st = checkImages(__func__, {outImage}, imageLd, dim);
+    if (st != BF_OK) return st;
+    AttnParams p{};
+    p.outImg = outImage; p.imgLd = imageLd;
+    p.q = q; p.k = k; p.v = v; p.out = out; p.m = m; p.l = l;
+    p.batch = int(batch); p.heads = int(heads); p.newLen = int(newLen); p.totalLen = int(kvRows);
+    p.dim = int(dim); p.hd = int(dim / heads); p.scale = scale;
+    p.kvRows = int(kvRows);
+    p.oldLenPtr = oldLen;
+    if (!fewQueriesFit(p, batch, heads, newLen))
+        return failInvalid(__func__, "at most eight queries per sequence, a head dim that is a multiple of 4 and 16-byte aligned operands");
+    const size_t rows = batch * heads * newLen, cus = size_t(computeUnits());
+    const size_t wanted = std::max<size_t>(1, (4 * cus + rows - 1) / rows);
+    const size_t chunkKeys = std::max<size_t>(128, ((kvRows + wanted - 1) / wanted + 127) / 128 * 128);
+    return launchFewQueries(p, batch, heads, newLen, chunkKeys, (kvRows + chunkKeys - 1) / chunkKeys, asStream(stream));
 }
 
 int bf_hip_attention_forward_img(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,

@@ -275,9 +275,13 @@ __global__ void __launch_bounds__(kBlock) embeddingBackwardKernel(const float* _
 template <int VEC>
 __global__ void __launch_bounds__(256) positionalForwardKernel(const float* __restrict__ x, const float* __restrict__ table,
                                                                float* __restrict__ out, size_t batch, size_t seq, size_t dim,
-                                                               size_t offset) {
+                                                               size_t offset, const int* __restrict__ offsetOnDevice, size_t maxSeq) {
     size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
     if (col >= dim) return;
+    if (offsetOnDevice) {                      // launched ahead of the device: the position is whatever the device-side counter says by then
+        offset = size_t(*offsetOnDevice);
+        if (offset + seq > maxSeq) return;     // the caller's promise, broken: nothing is written rather than read out of bounds
+    }
     size_t step = size_t(gridDim.y) * blockDim.y;
     for (size_t s = size_t(blockIdx.y) * blockDim.y + threadIdx.y; s < seq; s += step) {
         if constexpr (VEC == 4) {
@@ -350,6 +354,30 @@ __global__ void __launch_bounds__(256) copyPitchedKernel(float* __restrict__ dst
     }
 }
 
+// New keys and values, [batch, newLen, dim] each, to rows *position .. of every sequence of caches with `capacity` rows a
+// sequence: the append of a step launched before the position is known to the host.  blockIdx.z picks
+// the cache; nothing is written when the rows would not fit.
+template <int VEC>
+__global__ void __launch_bounds__(256) kvAppendKernel(float* __restrict__ kCache, float* __restrict__ vCache, const float* __restrict__ kNew,
+                                                      const float* __restrict__ vNew, size_t batch, size_t newLen, size_t dim, size_t capacity,
+                                                      const int* __restrict__ position) {
+    const size_t at = size_t(*position);
+    if (at + newLen > capacity) return;
+    float* cache = blockIdx.z == 0 ? kCache : vCache;
+    const float* rows = blockIdx.z == 0 ? kNew : vNew;
+    size_t col = (size_t(blockIdx.x) * blockDim.x + threadIdx.x) * VEC;
+    if (col >= dim) return;
+    size_t step = size_t(gridDim.y) * blockDim.y;
+    for (size_t r = size_t(blockIdx.y) * blockDim.y + threadIdx.y; r < batch * newLen; r += step) {
+        const size_t b = r / newLen, i = r - b * newLen;
+        float* dst = cache + (b * capacity + at + i) * dim + col;
+        if constexpr (VEC == 4) storef4(dst, loadf4(rows + r * dim + col));
+        else *dst = rows[r * dim + col];
+    }
+}
+
+__global__ void addToCounterKernel(int* counter, int by) { *counter += by; }
+
 // Lowest index of the maximum of one row: the result of the host loop "best = 0; if (row[c] > row[best])
 // best = c" it replaces.  A NaN never wins a strict '>' and, at index 0, is never beaten; the key
 // below encodes exactly that.
@@ -357,7 +385,8 @@ __device__ __forceinline__ float argmaxKey(float v, size_t i) {
     if (v != v) return i == 0 ? INFINITY : -INFINITY;
     return v;
 }
-__global__ void __launch_bounds__(1024) argmaxRowKernel(const float* __restrict__ row, size_t n, long long* __restrict__ result) {
+// thread 0 returns the index; every thread of the 1024 takes part
+__device__ __forceinline__ unsigned long long argmaxOfRow(const float* __restrict__ row, size_t n) {
     __shared__ float vals[16];
     __shared__ unsigned long long idxs[16];
     float best = -INFINITY;
@@ -382,7 +411,25 @@ __global__ void __launch_bounds__(1024) argmaxRowKernel(const float* __restrict_
     if (threadIdx.x == 0) {
         for (unsigned w = 1; w < (blockDim.x >> 6); ++w)
             if (takeOther(best, bestIdx, vals[w], idxs[w])) { best = vals[w]; bestIdx = idxs[w]; }
-        result[0] = (long long)bestIdx;
+    }
+    return bestIdx;
+}
+__global__ void __launch_bounds__(1024) argmaxRowKernel(const float* __restrict__ row, size_t n, long long* __restrict__ result) {
+    const unsigned long long best = argmaxOfRow(row, n);
+    if (threadIdx.x == 0) result[0] = (long long)best;
+}
+// The same index left on the device: as a float token id in token[0] (the next step's input) and, when `history` is
+// given, in history[*position + historyOffset] if that lies within historyLen.
+__global__ void __launch_bounds__(1024) argmaxToTokenKernel(const float* __restrict__ row, size_t n, float* __restrict__ token,
+                                                            float* __restrict__ history, size_t historyLen, const int* __restrict__ position,
+                                                            long long historyOffset) {
+    const unsigned long long best = argmaxOfRow(row, n);
+    if (threadIdx.x == 0) {
+        token[0] = float(best);
+        if (history) {
+            const long long slot = (position ? (long long)(*position) : 0) + historyOffset;
+            if (slot >= 0 && size_t(slot) < historyLen) history[slot] = float(best);
+        }
     }
 }
 
@@ -504,8 +551,20 @@ int bf_hip_positional_forward(const float* x, const float* table, float* out, si
     if (batch == 0 || seq == 0 || dim == 0) return BF_OK;
     BF_REQUIRE(x && table && out, "NULL pointer");
     Geom2D g = geometry2D(seq, dim, aligned16(x) && aligned16(table) && aligned16(out));
-    if (g.vec == 4) positionalForwardKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(x, table, out, batch, seq, dim, offset);
-    else positionalForwardKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(x, table, out, batch, seq, dim, offset);
+    if (g.vec == 4) positionalForwardKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(x, table, out, batch, seq, dim, offset, nullptr, maxSeq);
+    else positionalForwardKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(x, table, out, batch, seq, dim, offset, nullptr, maxSeq);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_positional_forward_indirect(const float* x, const float* table, float* out, size_t batch, size_t seq, size_t dim, size_t maxSeq,
+                                       const int* offset, bf_stream_t stream) {
+    BF_REQUIRE(seq <= maxSeq, "sequence " + std::to_string(seq) + " exceeds maxSeqLen " + std::to_string(maxSeq));
+    if (batch == 0 || seq == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(x && table && out && offset, "NULL pointer");
+    Geom2D g = geometry2D(seq, dim, aligned16(x) && aligned16(table) && aligned16(out));
+    if (g.vec == 4) positionalForwardKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(x, table, out, batch, seq, dim, 0, offset, maxSeq);
+    else positionalForwardKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(x, table, out, batch, seq, dim, 0, offset, maxSeq);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }
@@ -555,6 +614,36 @@ int bf_hip_argmax_last_position(const float* logits, size_t seq, size_t vocab, l
     BF_LAUNCH_CHECK();
     BF_HIP_TRY(hipMemcpyAsync(index, result.ptr, sizeof(long long), hipMemcpyDeviceToHost, s));
     BF_HIP_TRY(hipStreamSynchronize(s));
+    return BF_OK;
+}
+
+int bf_hip_argmax_last_position_device(const float* logits, size_t seq, size_t vocab, float* token, float* history, size_t historyLen,
+                                       const int* position, long long historyOffset, bf_stream_t stream) {
+    BF_REQUIRE(seq > 0 && vocab > 0, "empty logits");
+    BF_REQUIRE(vocab <= (size_t(1) << 24), "a token id beyond 2^24 has no exact float");
+    BF_REQUIRE(logits && token, "NULL pointer");
+    argmaxToTokenKernel<<<1, 1024, 0, asStream(stream)>>>(logits + (seq - 1) * vocab, vocab, token, history, historyLen, position, historyOffset);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_kv_append_indirect(float* kCache, float* vCache, const float* kNew, const float* vNew, size_t batch, size_t newLen, size_t dim,
+                              size_t capacity, const int* position, bf_stream_t stream) {
+    if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(kCache && vCache && kNew && vNew && position, "NULL pointer");
+    BF_REQUIRE(newLen <= capacity, "more new rows than the cache holds");
+    Geom2D g = geometry2D(batch * newLen, dim, aligned16(kCache) && aligned16(vCache) && aligned16(kNew) && aligned16(vNew));
+    g.grid.z = 2;
+    if (g.vec == 4) kvAppendKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(kCache, vCache, kNew, vNew, batch, newLen, dim, capacity, position);
+    else kvAppendKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(kCache, vCache, kNew, vNew, batch, newLen, dim, capacity, position);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_counter_add(int* counter, int by, bf_stream_t stream) {
+    BF_REQUIRE(counter != nullptr, "NULL pointer");
+    addToCounterKernel<<<1, 1, 0, asStream(stream)>>>(counter, by);
+    BF_LAUNCH_CHECK();
     return BF_OK;
 }
 

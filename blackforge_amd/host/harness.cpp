@@ -447,6 +447,17 @@ int bfh_model_forward_incremental(void* h, const float* input, int rank, const s
         if (outCount) *outCount = handle->output.elementCount();
     });
 }
+// Model::generateGreedy on a [1, n] prompt of token ids (device memory); `tokens` (HOST) receives `count` ids.
+int bfh_model_generate_greedy(void* h, const float* promptIds, size_t n, size_t count, long long* tokens) {
+    Handle* handle = static_cast<Handle*>(h);
+    return guarded([&] {
+        Borrowed in(promptIds, {1, n});
+        if (!handle->weightImagesCurrent) hip::invalidateBf16WeightCache();
+        handle->weightImagesCurrent = true;
+        std::vector<std::size_t> ids = handle->model->generateGreedy(in.tensor, count);
+        for (std::size_t i = 0; i < ids.size(); ++i) tokens[i] = static_cast<long long>(ids[i]);
+    });
+}
 int bfh_model_reset_generation(void* h) {
     return guarded([&] { static_cast<Handle*>(h)->model->resetGenerationState(); });
 }

@@ -70,6 +70,7 @@ def load() -> ctypes.CDLL:
         lib.bfh_self_attention_incremental.argtypes = [P] * 6 + [Z] * 4 + [I, P]
         lib.bfh_model_forward_incremental.argtypes = [P, P, I, ctypes.POINTER(Z), ctypes.POINTER(P), ctypes.POINTER(Z)]
         lib.bfh_model_reset_generation.argtypes = [P]
+        lib.bfh_model_generate_greedy.argtypes = [P, P, Z, Z, ctypes.POINTER(ctypes.c_longlong)]
         lib.bfh_model_argmax_last.argtypes = [P, Z, ctypes.POINTER(ctypes.c_longlong)]
         _lib = lib
     return _lib
@@ -214,12 +215,19 @@ class HostModel:
         self._refresh_params()
         return list(losses[:epochs])
 
-    def forwardIncremental(self, x: DeviceTensor) -> np.ndarray:
-        """hip::Model::forwardIncremental on the new positions only (K/V of earlier ones come from the model's caches)."""
+    def forwardIncremental(self, x: DeviceTensor, read: bool = True):
+        """hip::Model::forwardIncremental on the new positions only (K/V of earlier ones come from the model's caches).
+        read=False leaves the logits on the device (argmaxLast picks the next token there) and returns None."""
         shape = (ctypes.c_size_t * len(x.shape))(*x.shape)
         out, count = ctypes.c_void_p(), ctypes.c_size_t()
         _check(load().bfh_model_forward_incremental(self.handle, x.ptr, len(x.shape), shape, ctypes.byref(out), ctypes.byref(count)))
-        return self._read(out, count.value)
+        return self._read(out, count.value) if read else None
+
+    def generateGreedy(self, prompt: DeviceTensor, count: int) -> list:
+        """hip::Model::generateGreedy: `count` greedy tokens after a [1, n] prompt; token and position stay on the device between steps."""
+        tokens = (ctypes.c_longlong * max(count, 1))()
+        _check(load().bfh_model_generate_greedy(self.handle, prompt.ptr, prompt.shape[1], count, tokens))
+        return list(tokens[:count])
 
     def resetGenerationState(self) -> None:
         _check(load().bfh_model_reset_generation(self.handle))

@@ -407,6 +407,27 @@ int bf_hip_attention_forward_img(const float* q, const float* k, const float* v,
 int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
                                   float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t kvRows, size_t dim, float scale,
                                   size_t oldLen, bf_stream_t stream);
+/* ---- A decoding step whose position lives on the device (no counterparts in the reference, whose generation loop
+ * reads the next token back and passes the position from the host at every step, main.cpp:594-617).  These entry points
+ * read the number of cached positions from device memory instead, so that the host can launch step after step without
+ * waiting for the one before: positional_forward_indirect adds the table rows *offset.., kv_append_indirect copies the new
+ * keys and values to rows *position.. of caches with `capacity` rows a sequence, attention_forward_rows_indirect attends
+ * to the first *oldLen + newLen rows of k and v (the walk over the cache of bf_hip_attention_forward_rows, at most eight
+ * queries per sequence; its chunks cover all kvRows and those past the current length do nothing),
+ * argmax_last_position_device leaves the index on the device as a float token id (and in history[*position +
+ * historyOffset] when that lies within historyLen), counter_add advances the counter.  The caller promises that the
+ * positions fit (table rows, cache capacity): a kernel that finds otherwise writes nothing.  (They may also be recorded
+ * in a graph, whose arguments are frozen; replaying a whole decoding step that way measured slower than launching it.) */
+int bf_hip_positional_forward_indirect(const float* x, const float* table, float* out, size_t batch, size_t seq, size_t dim, size_t maxSeq,
+                                       const int* offset, bf_stream_t stream);
+int bf_hip_kv_append_indirect(float* kCache, float* vCache, const float* kNew, const float* vNew, size_t batch, size_t newLen, size_t dim,
+                              size_t capacity, const int* position, bf_stream_t stream);
+int bf_hip_attention_forward_rows_indirect(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd,
+                                           float* m, float* l, size_t batch, size_t heads, size_t newLen, size_t kvRows, size_t dim, float scale,
+                                           const int* oldLen, bf_stream_t stream);
+int bf_hip_argmax_last_position_device(const float* logits, size_t seq, size_t vocab, float* token, float* history, size_t historyLen,
+                                       const int* position, long long historyOffset, bf_stream_t stream);
+int bf_hip_counter_add(int* counter, int by, bf_stream_t stream);
 /* computeDKernel: fused_attention.cu:166-190   D[b,h,i] = dot(out[b,i,h,:], dOut[b,i,h,:]) */
 int bf_hip_attention_dot_o_do(const float* out, const float* dOut, float* D, size_t batch, size_t heads,
                               size_t newLen, size_t dim, bf_stream_t stream);

@@ -193,44 +193,55 @@ public:
     // invalidated them) and kept for the calls that follow, where the reference converts them in every call.
     DeviceTensor forwardIncremental(const DeviceTensor& newTokenIds) {
         if (useBf16_ && generationPosition_ == 0) invalidateBf16WeightCache();
-        DeviceTensor current = newTokenIds.clone();
-        std::size_t newLen = current.rank() >= 2 ? current.dim(1) : 0;
-        for (LayerState& layer : layers_) {
-            const LayerSpec& s = layer.spec;
-            switch (s.kind) {
-                case LayerKind::PositionalEmbedding:
-                    current = addPositionalEmbeddingAt(current, layer.params[0].value, generationPosition_);
-                    break;
-                case LayerKind::Attention:
-                    current = useBf16_ ? selfAttentionIncrementalBf16CachedWeights(current, layer.params[0].value, layer.params[1].value,
-                                                                                    layer.params[2].value, layer.params[3].value, s.arg0,
-                                                                                    layer.kvCache)
-                                       : selfAttentionIncremental(current, layer.params[0].value, layer.params[1].value,
-                                                                  layer.params[2].value, layer.params[3].value, s.arg0, layer.kvCache);
-                    break;
-                case LayerKind::BidirectionalAttention:
-                    // src/backend/cpu/model.cpp:365-374: a layer that sees the whole sequence has no next token to generate
-                    throw std::invalid_argument("hip::Model::forwardIncremental: the pipeline contains 'bidirectional_attention', "
-                                                "which does not support incremental generation");
-                case LayerKind::FeedForward: {
-                    // the block as the training pass runs it (bias, activation and residual in the products' stores, cached
-                    // weight images); what it keeps for a backward pass is dropped
-                    Activation act = s.arg1 == 1 ? Activation::Gelu : Activation::Silu;
-                    FeedForwardCache unused;
-                    current = feedForwardForwardCached(current, layer.params[0].value, layer.params[1].value, layer.params[2].value,
-                                                       layer.params[3].value, useBf16_, unused, act);
-                    break;
-                }
-                case LayerKind::Linear:
-                    current = useBf16_ ? linearBf16CachedWeight(current, layer.params[0].value, layer.params[1].value)
-                                       : linear(current, layer.params[0].value, layer.params[1].value);
-                    break;
-                case LayerKind::Embedding: current = embeddingLookup(current, layer.params[0].value); break;
-                default: current = applyElementwise(s.kind, current); break;
-            }
-        }
+        std::size_t newLen = newTokenIds.rank() >= 2 ? newTokenIds.dim(1) : 0;
+        DeviceTensor output = incrementalStep(newTokenIds, nullptr);
         generationPosition_ += newLen;
-        return current;
+        return output;
+    }
+
+    // Greedy continuation of a prompt of one sequence by `count` tokens: what the reference's `generate` command does
+    // from the host, one forwardIncremental and one read-back of the logits' argmax per token (main.cpp:594-617).  Here
+    // the host never waits inside the loop: the prompt is processed by forwardIncremental, and every step that follows
+    // (argmax of the last logits on the device, embed that token, all layers, the head, advance the position) takes the
+    // position and the token from device memory, so the host launches step after step ahead of the GPU and reads the
+    // tokens back once, at the end.  The caches get their room for all the tokens first.  (Replaying the step from a HIP
+    // graph instead of launching it was measured at nearly twice the time per token on this runtime: not done.)
+    // Starts a new generation (resetGenerationState) and leaves the model as count - 1 further calls of
+    // forwardIncremental would: the last token returned has not been fed.  Needs a pipeline that starts with an
+    // embedding; the ids are returned in order.  Not part of the reference's interface.
+    [[nodiscard]] std::vector<std::size_t> generateGreedy(const DeviceTensor& promptIds, std::size_t count) {
+        require(promptIds.rank() == 2 && promptIds.dim(0) == 1 && promptIds.dim(1) >= 1, "generateGreedy: the prompt must be [1, n] token ids, n >= 1");
+        require(!layers_.empty() && layers_.front().spec.kind == LayerKind::Embedding, "generateGreedy: the pipeline must start with an embedding");
+        const std::size_t promptLen = promptIds.dim(1), vocab = layers_.front().spec.arg0;
+        for (const LayerState& layer : layers_)
+            if (layer.spec.kind == LayerKind::PositionalEmbedding && count > 1)
+                require(promptLen + count - 1 <= layer.params[0].value.dim(0), "generateGreedy: the positions exceed the positional table");
+        resetGenerationState();
+        if (count == 0) return {};
+        DeviceTensor logits = forwardIncremental(promptIds);
+        require(logits.rank() == 3 && logits.dim(2) == vocab, "generateGreedy: the pipeline must end in logits over the embedding's vocabulary");
+        for (LayerState& layer : layers_)
+            if (layer.spec.kind == LayerKind::Attention) layer.kvCache.reserve(1, promptLen + count, layer.kvCache.k.dim(2));
+        DeviceTensor token({1, 1}), history({count}), position({1});   // position: one int, the number of positions processed
+        const int start = static_cast<int>(promptLen);
+        check(bf_hip_memcpy_h2d(position.data(), &start, sizeof(int)));
+        const int* devicePosition = reinterpret_cast<const int*>(position.data());
+        const long long firstSlot = -static_cast<long long>(promptLen);    // a token goes to history[*position - promptLen]
+        check(bf_hip_argmax_last_position_device(logits.data(), promptLen, vocab, token.data(), history.data(), count, devicePosition, firstSlot,
+                                                 nullptr));
+        for (std::size_t i = 1; i < count; ++i) {
+            DeviceTensor next = incrementalStep(token, devicePosition);
+            check(bf_hip_counter_add(reinterpret_cast<int*>(position.data()), 1, nullptr));
+            check(bf_hip_argmax_last_position_device(next.data(), 1, vocab, token.data(), history.data(), count, devicePosition, firstSlot, nullptr));
+        }
+        generationPosition_ += count - 1;
+        for (LayerState& layer : layers_)
+            if (layer.spec.kind == LayerKind::Attention) layer.kvCache.length += count - 1;
+        std::vector<float> ids(count);
+        check(bf_hip_memcpy_d2h(ids.data(), history.data(), count * sizeof(float)));   // waits for the steps
+        std::vector<std::size_t> result(count);
+        for (std::size_t i = 0; i < count; ++i) result[i] = static_cast<std::size_t>(ids[i]);
+        return result;
     }
 
     void resetGenerationState() {
@@ -258,6 +269,67 @@ public:
     [[nodiscard]] bool usesBf16() const { return useBf16_; }
 
 private:
+    struct LayerState;
+    // The layers of one incremental step.  devicePosition == nullptr: the eager step (positions from the host-side
+    // counters, which the caller advances; token ids checked).  Otherwise the step that needs nothing from the host:
+    // positions read from *devicePosition by the kernels, token ids trusted, host-side counters untouched.
+    DeviceTensor incrementalStep(const DeviceTensor& newTokenIds, const int* devicePosition) {
+        const DeviceTensor* input = &newTokenIds;
+        DeviceTensor current;
+        for (LayerState& layer : layers_) {
+            const LayerSpec& s = layer.spec;
+            const DeviceTensor& in = *input;
+            switch (s.kind) {
+                case LayerKind::PositionalEmbedding:
+                    if (devicePosition == nullptr) {
+                        current = addPositionalEmbeddingAt(in, layer.params[0].value, generationPosition_);
+                    } else {
+                        const DeviceTensor& table = layer.params[0].value;
+                        require(in.rank() == 3 && table.rank() == 2 && table.dim(1) == in.dim(2), "addPositionalEmbedding: table must be [maxSeqLen, dim]");
+                        DeviceTensor out(in.shape());
+                        check(bf_hip_positional_forward_indirect(in.data(), table.data(), out.data(), in.dim(0), in.dim(1), in.dim(2), table.dim(0),
+                                                                 devicePosition, nullptr));
+                        current = std::move(out);
+                    }
+                    break;
+                case LayerKind::Attention:
+                    if (devicePosition != nullptr)
+                        current = selfAttentionIncrementalOnDevicePosition(in, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                                   layer.params[3].value, s.arg0, layer.kvCache, useBf16_, devicePosition);
+                    else
+                        current = useBf16_ ? selfAttentionIncrementalBf16CachedWeights(in, layer.params[0].value, layer.params[1].value,
+                                                                                        layer.params[2].value, layer.params[3].value, s.arg0,
+                                                                                        layer.kvCache)
+                                           : selfAttentionIncremental(in, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                                      layer.params[3].value, s.arg0, layer.kvCache);
+                    break;
+                case LayerKind::BidirectionalAttention:
+                    // src/backend/cpu/model.cpp:365-374: a layer that sees the whole sequence has no next token to generate
+                    throw std::invalid_argument("hip::Model::forwardIncremental: the pipeline contains 'bidirectional_attention', "
+                                                "which does not support incremental generation");
+                case LayerKind::FeedForward: {
+                    // the block as the training pass runs it (bias, activation and residual in the products' stores, cached
+                    // weight images); what it keeps for a backward pass is dropped
+                    Activation act = s.arg1 == 1 ? Activation::Gelu : Activation::Silu;
+                    FeedForwardCache unused;
+                    current = feedForwardForwardCached(in, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                       layer.params[3].value, useBf16_, unused, act);
+                    break;
+                }
+                case LayerKind::Linear:
+                    current = useBf16_ ? linearBf16CachedWeight(in, layer.params[0].value, layer.params[1].value)
+                                       : linear(in, layer.params[0].value, layer.params[1].value);
+                    break;
+                case LayerKind::Embedding:
+                    current = devicePosition != nullptr ? embeddingLookupPreValidated(in, layer.params[0].value) : embeddingLookup(in, layer.params[0].value);
+                    break;
+                default: current = applyElementwise(s.kind, in); break;
+            }
+            input = &current;
+        }
+        return layers_.empty() ? newTokenIds.clone() : std::move(current);
+    }
+
     struct LayerState {
         LayerSpec spec;
         std::vector<Parameter> params;

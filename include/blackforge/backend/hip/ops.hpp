@@ -458,12 +458,62 @@ private:
 };
 
 namespace detail {
+// The normalised input's three projections of an incremental step, written where `outs` point
+inline void incrementalProjections(const DeviceTensor& newInput, const DeviceTensor& wq, const DeviceTensor& wk, const DeviceTensor& wv,
+                                   float* const (&outs)[3], int mode) {
+    const std::size_t dim = newInput.dim(2), rows = newInput.dim(0) * newInput.dim(1);
+    if (mode != 0 && dim % 8 == 0 && rows > 0) {
+        // the normalised rows have no reader but the three projections: written as a bf16 image only, and the three
+        // products made by one call over that image
+        DeviceTensor normedImage({rows, dim / 2});
+        check(bf_hip_rmsnorm_img(newInput.data(), nullptr, reinterpret_cast<std::uint16_t*>(normedImage.data()), rows, dim, nullptr));
+        const float* weights[3] = {wq.data(), wk.data(), wv.data()};
+        float* targets[3] = {outs[0], outs[1], outs[2]};
+        check(bf_hip_matmul_bf16_shared_input_img(nullptr, reinterpret_cast<const std::uint16_t*>(normedImage.data()), weights, targets, 3, rows, dim,
+                                                  dim, mode == 2, nullptr));
+    } else {
+        DeviceTensor normedFlat = rmsnorm(newInput).reshaped({rows, dim});
+        const DeviceTensor* w[3] = {&wq, &wk, &wv};
+        for (int i = 0; i < 3; ++i) {
+            if (mode == 0) check(bf_hip_gemm_f32_adds(0, 0, normedFlat.data(), w[i]->data(), nullptr, nullptr, outs[i], rows, dim, dim, nullptr));
+            else check(bf_hip_linear_bf16_img(normedFlat.data(), nullptr, w[i]->data(), nullptr, nullptr, outs[i], rows, dim, dim, mode == 2, nullptr));
+        }
+    }
+}
+
+// The step for a host that runs ahead of the device (Model::generateGreedy): the number of cached positions is read from
+// *devicePosition by the kernels (append, attention), nothing of it is in the arguments, and the host-side cache.length
+// is left alone.  The cache must already hold room for every position the steps will reach (KVCache::reserve).
+inline DeviceTensor selfAttentionIncrementalOnDevicePosition(const char* op, const DeviceTensor& newInput, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                      const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads, KVCache& cache,
+                                                      int mode, const int* devicePosition) {
+    const std::size_t batch = newInput.dim(0), newLen = newInput.dim(1), dim = newInput.dim(2);
+    require(cache.capacity != 0 && cache.k.rank() == 3 && cache.k.dim(0) == batch && cache.k.dim(2) == dim,
+            std::string(op) + ": a step on a device-side position needs a cache that already holds the prompt, for this batch size and width");
+    DeviceTensor qNew({batch, newLen, dim}), kNew({batch, newLen, dim}), vNew({batch, newLen, dim});
+    float* const outs[3] = {qNew.data(), kNew.data(), vNew.data()};
+    incrementalProjections(newInput, wq, wk, wv, outs, mode);
+    check(bf_hip_kv_append_indirect(cache.k.data(), cache.v.data(), kNew.data(), vNew.data(), batch, newLen, dim, cache.capacity, devicePosition,
+                                    nullptr));
+    const float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
+    const bool imageOnly = mode != 0 && dim % 8 == 0;
+    DeviceTensor attnOut = imageOnly ? DeviceTensor::imageOnly({batch, newLen, dim}) : DeviceTensor({batch, newLen, dim});
+    DeviceTensor m({batch, numHeads, newLen}), l({batch, numHeads, newLen});
+    check(bf_hip_attention_forward_rows_indirect(qNew.data(), cache.k.data(), cache.v.data(), attnOut.data(),
+                                                 imageOnly ? const_cast<std::uint16_t*>(attnOut.image()) : nullptr, imageOnly ? dim : 0, m.data(),
+                                                 l.data(), batch, numHeads, newLen, cache.capacity, dim, scaleFactor, devicePosition, nullptr));
+    return projectionFused(attnOut, wout, nullptr, &newInput, mode, {batch, newLen, dim});
+}
+
 inline DeviceTensor selfAttentionIncrementalImpl(const char* op, const DeviceTensor& newInput, const DeviceTensor& wq,
                                                   const DeviceTensor& wk, const DeviceTensor& wv, const DeviceTensor& wout,
-                                                  std::size_t numHeads, KVCache& cache, int mode) {
+                                                  std::size_t numHeads, KVCache& cache, int mode,
+                                                  const int* devicePosition = nullptr) {
     requireAttention(op, newInput, numHeads);
     std::size_t batch = newInput.dim(0), newLen = newInput.dim(1), dim = newInput.dim(2);
-    const std::size_t oldLen = cache.length, rows = batch * newLen;
+    const std::size_t oldLen = cache.length;
+    if (devicePosition != nullptr)
+        return selfAttentionIncrementalOnDevicePosition(op, newInput, wq, wk, wv, wout, numHeads, cache, mode, devicePosition);
     if (cache.length != 0) require(cache.k.rank() == 3 && cache.k.dim(0) == batch && cache.k.dim(2) == dim, std::string(op) + ": the cache was filled with another batch size or width");
     cache.reserve(batch, oldLen + newLen, dim);
     // one sequence: its new keys and values are rows oldLen.. of the cache, and the projections write them there;
@@ -476,24 +526,8 @@ inline DeviceTensor selfAttentionIncrementalImpl(const char* op, const DeviceTen
     }
     float* kRows = inPlace ? cache.k.data() + oldLen * dim : kNew.data();
     float* vRows = inPlace ? cache.v.data() + oldLen * dim : vNew.data();
-    if (mode != 0 && dim % 8 == 0 && rows > 0) {
-        // the normalised rows have no reader but the three projections: written as a bf16 image only, and the three
-        // products made by one call over that image
-        DeviceTensor normedImage({rows, dim / 2});
-        check(bf_hip_rmsnorm_img(newInput.data(), nullptr, reinterpret_cast<std::uint16_t*>(normedImage.data()), rows, dim, nullptr));
-        const float* weights[3] = {wq.data(), wk.data(), wv.data()};
-        float* outs[3] = {qNew.data(), kRows, vRows};
-        check(bf_hip_matmul_bf16_shared_input_img(nullptr, reinterpret_cast<const std::uint16_t*>(normedImage.data()), weights, outs, 3, rows, dim,
-                                                  dim, mode == 2, nullptr));
-    } else {
-        DeviceTensor normedFlat = rmsnorm(newInput).reshaped({rows, dim});
-        const DeviceTensor* w[3] = {&wq, &wk, &wv};
-        float* outs[3] = {qNew.data(), kRows, vRows};
-        for (int i = 0; i < 3; ++i) {
-            if (mode == 0) check(bf_hip_gemm_f32_adds(0, 0, normedFlat.data(), w[i]->data(), nullptr, nullptr, outs[i], rows, dim, dim, nullptr));
-            else check(bf_hip_linear_bf16_img(normedFlat.data(), nullptr, w[i]->data(), nullptr, nullptr, outs[i], rows, dim, dim, mode == 2, nullptr));
-        }
-    }
+    float* const outs[3] = {qNew.data(), kRows, vRows};
+    incrementalProjections(newInput, wq, wk, wv, outs, mode);
     if (!inPlace) {
         check(bf_hip_copy_pitched(cache.k.data() + oldLen * dim, cache.capacity * dim, kNew.data(), newLen * dim, newLen * dim, batch, nullptr));
         check(bf_hip_copy_pitched(cache.v.data() + oldLen * dim, cache.capacity * dim, vNew.data(), newLen * dim, newLen * dim, batch, nullptr));
@@ -527,6 +561,15 @@ inline DeviceTensor selfAttentionIncrementalBf16CachedWeights(const DeviceTensor
                                                                const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads,
                                                                KVCache& cache) {
     return detail::selfAttentionIncrementalImpl("selfAttentionIncrementalBf16", newInput, wq, wk, wv, wout, numHeads, cache, 2);
+}
+// One incremental step that needs nothing from the host (Model::generateGreedy): the number of cached positions comes
+// from *devicePosition, read by the kernels; cache.length stays as it is.
+inline DeviceTensor selfAttentionIncrementalOnDevicePosition(const DeviceTensor& newInput, const DeviceTensor& wq, const DeviceTensor& wk,
+                                                      const DeviceTensor& wv, const DeviceTensor& wout, std::size_t numHeads, KVCache& cache,
+                                                      bool useBf16, const int* devicePosition) {
+    require(devicePosition != nullptr, "selfAttentionIncrementalOnDevicePosition: no device-side position");
+    return detail::selfAttentionIncrementalImpl(useBf16 ? "selfAttentionIncrementalBf16" : "selfAttentionIncremental", newInput, wq, wk, wv, wout,
+                                                numHeads, cache, useBf16 ? 2 : 0, devicePosition);
 }
 
 // Greedy next-token choice over the last position of [1, seq, vocab] logits (reference: src/main.cpp:504-518),

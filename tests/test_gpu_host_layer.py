@@ -271,6 +271,42 @@ def test_model_forward_incremental_matches_full_forward(hip, oracle, rng, use_bf
         gpu.forwardIncremental(D.fromHost(ids))
 
 
+@pytest.mark.parametrize("use_bf16,heads,dim", [(False, 4, 32), (True, 4, 32), (True, 2, 264)])
+def test_greedy_generation_without_reading_back(hip, rng, use_bf16, heads, dim):
+    """hip::Model::generateGreedy: the loop of the reference's `generate` command (main.cpp:594-617: forwardIncremental, argmax
+    of the last logits, feed it back) with token and position kept on the device, so that no step waits for a read-back.
+    Checked against the loop over forwardIncremental fed with the same tokens: every token is the argmax of that loop's logits
+    at its step (up to a near tie: the attention splits the cache into chunks differently), across the 128-key chunk
+    boundary of the attention walk, and the model is left where the eager loop would be."""
+    from blackforge_amd import hostlayer as hl
+    vocab, seq, hidden, blocks = 96, 400, 64, 2
+    D = hip.DeviceTensor
+    model = hl.HostModel(_lm_layers(hl, vocab, dim, seq, heads, hidden, 1, blocks), use_bf16=use_bf16)
+    for i, c in enumerate(model.counts):
+        model.set_value(i, r(rng, c, scale=0.3))
+    prompt = rng.integers(0, vocab, (1, 7)).astype(f32)
+    count = 200
+    tokens = model.generateGreedy(D.fromHost(prompt), count)
+    assert len(tokens) == count and all(0 <= t < vocab for t in tokens)
+    after = model.forwardIncremental(D.fromHost(np.array([[tokens[-1]]], f32))).reshape(vocab)   # the generation continues eagerly
+    assert model.generateGreedy(D.fromHost(prompt), count) == tokens, "the same generation twice"
+    assert model.generateGreedy(D.fromHost(prompt), 1) == tokens[:1] and model.generateGreedy(D.fromHost(prompt), 0) == []
+
+    model.resetGenerationState()
+    logits = model.forwardIncremental(D.fromHost(prompt)).reshape(-1, vocab)[-1]
+    near_ties = 0
+    for step, t in enumerate(tokens):
+        best = int(np.argmax(logits))
+        if t != best:   # generateGreedy's logits differ from these in the last bits
+            near_ties += 1
+            assert logits[best] - logits[t] <= (5e-3 if use_bf16 else 1e-4) * np.abs(logits).max(), f"token {step}: {t} is not the eager argmax {best}"
+        logits = model.forwardIncremental(D.fromHost(np.array([[t]], f32))).reshape(vocab)
+    assert near_ties <= 2
+    assert_close(after, logits, tol=5e-3 if use_bf16 else 1e-4, what="logits after the generation vs the eager loop's")
+    with pytest.raises(ValueError):
+        model.generateGreedy(D.fromHost(prompt), seq)   # positions past the positional table
+
+
 @pytest.mark.parametrize("act", [0, 1])
 def test_config1_tiny_lm_full_step_against_oracle(hip, oracle, rng, act):
     """BASELINE config 1 shape: vocab 256, d_model 128, 4 heads, 1 attention + 1 feedforward(512) block, seq 64,
