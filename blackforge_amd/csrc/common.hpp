@@ -102,6 +102,8 @@ struct Scratch {
 // device memory.  The same table is needed step after step, so the device copy is kept per (device,
 // slot) and re-uploaded only when the host bytes change; an unchanged table costs no copy and no
 // host synchronisation.  `slot` separates users (zero, sgd, adamw, the weight-image refresh).
+constexpr float kRmsNormEps = 1e-6f;   // rmsnorm: x / sqrt(mean(x^2) + eps), ops.cpp:250-275
+
 enum { kSlotZero = 0, kSlotSgd = 1, kSlotAdamW = 2, kSlotConvert = 3, kSlotCount = 4 };
 int uploadDescriptorTable(int slot, const void* hostBytes, size_t bytes, hipStream_t stream, const void** devicePtr);
 

@@ -229,6 +229,9 @@ struct Epilogue {
     unsigned short* image;   // [M, N]
     const float* actZ;       // [M, N]
     float* colPartial;       // [ceil(M / 32), N]
+    // products of at most eight rows only (gemmBf16FewRowsKernel), A == NULL: the rows of A are those of rmsnorm(normInput)
+    // ([M, K] fp32, dense) rounded to bf16, made while the kernel stages them
+    const float* normInput;
 };
 
 // An accumulator tile of the 32x32 MFMA gives lane (li, half) column li of rows 8g + 4 half + 0..3 (g = 0..3).  Stored
@@ -1195,9 +1198,27 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
     };
     int k0 = lane * 8;
     loadSteps(k0);                                           // in flight while A is staged
-    for (int at = int(threadIdx.x) * 8; at < M * K; at += 2048) {
-        const int r = at / K, k = at - r * K;                // K is a multiple of 8: a group of eight lies in one row
-        *reinterpret_cast<uint4v*>(aRows + at) = *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k);
+    if (e.normInput == nullptr) {
+        for (int at = int(threadIdx.x) * 8; at < M * K; at += 2048) {
+            const int r = at / K, k = at - r * K;            // K is a multiple of 8: a group of eight lies in one row
+            *reinterpret_cast<uint4v*>(aRows + at) = *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k);
+        }
+    } else {
+        // x / sqrt(mean(x^2) + eps) with the sum of squares in double and the division in float, as the row kernel that
+        // this replaces forms it (ops.cpp:264-275), rounded to bf16; every workgroup normalises all M rows for itself
+        __shared__ double squares[4];
+        for (int r = 0; r < M; ++r) {
+            const float* row = e.normInput + size_t(r) * K;
+            double ss = 0.0;
+            for (int k = int(threadIdx.x); k < K; k += 256) ss += double(row[k]) * double(row[k]);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            if (lane == 0) squares[threadIdx.x >> 6] = ss;
+            __syncthreads();
+            const float rms = float(sqrt(((squares[0] + squares[1]) + (squares[2] + squares[3])) / double(K) + double(kRmsNormEps)));
+            for (int k = int(threadIdx.x); k < K; k += 256) aRows[r * K + k] = toBf16Bits(row[k] / rms);
+            __syncthreads();                                 // `squares` is free for the next row
+        }
     }
     __syncthreads();
     if (!owner) return;
@@ -1666,6 +1687,11 @@ int launchGemmTn(const unsigned short* A, const unsigned short* B, const Epilogu
 // Whether launchGemmNt takes a product of this shape with Epilogue::fuse set: a kernel chosen by the caller (tests and
 // tuning) never does, so that the separate passes stay reachable, and neither do products too small for the
 // one-tile-per-workgroup kernels.
+// what the walk over the weights (gemmBf16FewRowsKernel) asks for; launchGemmNt sends every such product there
+bool fewRowsServe(const void* A, const void* Bt, int fuse, size_t M, size_t K, size_t lda, size_t ldb) {
+    return g_ntRoute == BF_GEMM_ROUTE_AUTO && M <= 8 && fuse != 2 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
+           M * K * sizeof(unsigned short) <= kFewRowsLds && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) & 15u) == 0;
+}
 bool fusedActivationFits(size_t M, size_t N, size_t K, int fuse) {
     if (g_ntRoute != BF_GEMM_ROUTE_AUTO || N % 8 != 0) return false;
     const size_t cus = size_t(computeUnits());
@@ -1699,8 +1725,7 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
             return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s, g_ntRoute == BF_GEMM_ROUTE_WIDE_192_PERSISTENT);
         default: break;
     }
-    if (M <= 8 && epi.fuse != 2 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && M * K * sizeof(unsigned short) <= kFewRowsLds &&
-        ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) & 15u) == 0) {   // a walk over the weights, no tiles
+    if (fewRowsServe(A, Bt, epi.fuse, M, K, lda, ldb)) {   // a walk over the weights, no tiles
         if (M == 0 || N == 0) return BF_OK;
         return M == 1 ? launchFewRows<1>(A, Bt, epi, M, N, K, lda, ldb, s) : M == 2 ? launchFewRows<2>(A, Bt, epi, M, N, K, lda, ldb, s)
              : M <= 4 ? launchFewRows<4>(A, Bt, epi, M, N, K, lda, ldb, s) : launchFewRows<8>(A, Bt, epi, M, N, K, lda, ldb, s);
@@ -2276,6 +2301,78 @@ int bf_hip_matmul_bf16_shared_input_img(const float* a, const uint16_t* aImage, 
         if (st != BF_OK) return st;
     }
     return BF_OK;
+}
+
+// c[i] = bf16(rmsnorm(x)) b[i]: the projections of an attention block's normalised input (ops_transformer.cu:217-232) for
+// a caller that keeps nothing for a backward pass.  At most eight rows: the normalisation is made by the product's own
+// kernel while it stages the rows (one launch); otherwise the row kernel writes the image and the products follow.
+int bf_hip_rmsnorm_matmul_bf16_shared_input(const float* x, const float* const* b, float* const* c, size_t count, size_t m, size_t k, size_t n,
+                                            int cacheWeight, bf_stream_t stream) {
+    BF_REQUIRE(count >= 1 && count <= 3, "count must be 1, 2 or 3");
+    BF_REQUIRE(b && c, "NULL pointer array");
+    if (m == 0 || n == 0) return BF_OK;
+    BF_REQUIRE(k > 0 && x != nullptr, "NULL or empty input");
+    for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] != nullptr && c[i] != nullptr, "NULL operand");
+    hipStream_t s = asStream(stream);
+    const bool stacked = count == 1 || n % 256 == 0;
+    if (stacked && fewRowsServe(nullptr, nullptr, 0, m, k, k, k)) {
+        unsigned short* wImg = nullptr;
+        size_t wBytes = 0;
+        int st = count > 1 ? weightImage(b, count, k, n, 2, cacheWeight != 0, s, &wImg, &wBytes)
+                           : weightImage(b[0], k, n, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
+        if (st != BF_OK) return st;
+        Epilogue epi{{c[0], count > 1 ? c[1] : nullptr, count > 2 ? c[2] : nullptr}, int(n), nullptr, nullptr};
+        epi.normInput = x;
+        st = fewRowsServe(nullptr, wImg, 0, m, k, k, k) ? launchGemmNt(nullptr, wImg, epi, m, count * n, k, k, k, s)
+                                                        : failInvalid(__func__, "unaligned weight image");
+        if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+        return st;
+    }
+    const size_t kp = pad8(k);
+    Scratch image(m * kp * sizeof(unsigned short));
+    if (image.status != BF_OK) return image.status;
+    int st = bf_hip_rmsnorm_img(x, nullptr, image.as<uint16_t>(), m, k, stream);
+    if (st != BF_OK) return st;
+    return bf_hip_matmul_bf16_shared_input_img(nullptr, image.as<uint16_t>(), b, c, count, m, k, n, cacheWeight, stream);
+}
+
+// out = input + act(bf16(rmsnorm(input)) w1 + b1) w2 + b2: the feed-forward block (ops_transformer.cu:182-215) for a
+// caller that keeps nothing for a backward pass (incremental decoding).  At most eight rows: two launches, the
+// normalisation made while the first product stages its rows and the activation in its store.
+int bf_hip_rmsnorm_feedforward_bf16(const float* input, const float* w1, const float* b1, const float* w2, const float* b2, int act, float* out,
+                                    size_t m, size_t d, size_t hidden, int cacheWeight, bf_stream_t stream) {
+    if (m == 0) return BF_OK;
+    BF_REQUIRE(d > 0 && hidden > 0 && d % 8 == 0 && hidden % 8 == 0, "d and hidden must be positive multiples of 8");
+    BF_REQUIRE(act == BF_ACT_SILU || act == BF_ACT_GELU || act == BF_ACT_RELU, "unknown activation");
+    BF_REQUIRE(input && w1 && w2 && out, "NULL pointer");
+    hipStream_t s = asStream(stream);
+    Scratch z(m * hidden * sizeof(float)), hImage(m * hidden * sizeof(unsigned short));
+    if (z.status != BF_OK) return z.status;
+    if (hImage.status != BF_OK) return hImage.status;
+    if (fewRowsServe(nullptr, nullptr, 1, m, d, d, d) && fewRowsServe(nullptr, nullptr, 0, m, hidden, hidden, hidden) &&
+        (reinterpret_cast<uintptr_t>(b1) & 15u) == 0) {
+        unsigned short* wImg = nullptr;
+        size_t wBytes = 0;
+        int st = weightImage(w1, d, hidden, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
+        if (st != BF_OK) return st;
+        Epilogue first{{z.as<float>(), nullptr, nullptr}, int(hidden), b1, nullptr};
+        first.fuse = 1; first.act = act; first.image = hImage.as<unsigned short>();
+        first.normInput = input;
+        st = launchGemmNt(nullptr, wImg, first, m, hidden, d, d, d, s);
+        if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+        if (st != BF_OK) return st;
+        st = weightImage(w2, hidden, d, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
+        if (st != BF_OK) return st;
+        st = launchGemmNt(hImage.as<unsigned short>(), wImg, Epilogue{{out, nullptr, nullptr}, int(d), b2, input}, m, d, hidden, hidden, hidden, s);
+        if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+        return st;
+    }
+    Scratch xImage(m * d * sizeof(unsigned short));
+    if (xImage.status != BF_OK) return xImage.status;
+    int st = bf_hip_rmsnorm_img(input, nullptr, xImage.as<uint16_t>(), m, d, stream);
+    if (st != BF_OK) return st;
+    return bf_hip_feedforward_bf16(nullptr, w1, b1, w2, b2, input, act, z.as<float>(), hImage.as<uint16_t>(), xImage.as<uint16_t>(), out, m, d, hidden,
+                                   cacheWeight, stream);
 }
 
 int bf_hip_matmul_bf16_shared_input_backward(const float* a, const float* const* b, const float* const* g, float* dA,

@@ -11,7 +11,6 @@ namespace {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-constexpr float kRmsNormEps = 1e-6f;
 
 // Visits the row either from the register cache or (CACHED == false) from global memory.
 template <int G, int MAXE, int VEC, bool CACHED, bool NT = false>

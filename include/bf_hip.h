@@ -407,6 +407,17 @@ int bf_hip_attention_forward_img(const float* q, const float* k, const float* v,
 int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v, float* out, uint16_t* outImage, size_t imageLd, float* m,
                                   float* l, size_t batch, size_t heads, size_t newLen, size_t totalLen, size_t kvRows, size_t dim, float scale,
                                   size_t oldLen, bf_stream_t stream);
+/* Blocks of an incremental decoding step, which keeps nothing for a backward pass (no counterparts in the reference,
+ * which runs the training-time operators: ops_transformer.cu:133-180, 182-215).
+ * rmsnorm_matmul_bf16_shared_input: c[i] = bf16(rmsnorm(x)) b[i] for up to three weights [k, n] (an attention block's Q, K
+ * and V projections of its normalised input).  rmsnorm_feedforward_bf16: out = input + act(bf16(rmsnorm(input)) w1 + b1) w2
+ * + b2 (d and hidden multiples of 8).  For at most eight rows the normalisation is made by the first product's kernel
+ * while it stages its rows (double sum of squares, float division, as bf_hip_rmsnorm) and the activation in its store: one
+ * launch for the projections, two for the block; more rows run the row kernel and the products one after the other. */
+int bf_hip_rmsnorm_matmul_bf16_shared_input(const float* x, const float* const* b, float* const* c, size_t count, size_t m, size_t k, size_t n,
+                                            int cacheWeight, bf_stream_t stream);
+int bf_hip_rmsnorm_feedforward_bf16(const float* input, const float* w1, const float* b1, const float* w2, const float* b2, int act, float* out,
+                                    size_t m, size_t d, size_t hidden, int cacheWeight, bf_stream_t stream);
 /* ---- A decoding step whose position lives on the device (no counterparts in the reference, whose generation loop
  * reads the next token back and passes the position from the host at every step, main.cpp:594-617).  These entry points
  * read the number of cached positions from device memory instead, so that the host can launch step after step without

@@ -308,12 +308,10 @@ private:
                     throw std::invalid_argument("hip::Model::forwardIncremental: the pipeline contains 'bidirectional_attention', "
                                                 "which does not support incremental generation");
                 case LayerKind::FeedForward: {
-                    // the block as the training pass runs it (bias, activation and residual in the products' stores, cached
-                    // weight images); what it keeps for a backward pass is dropped
+                    // bias, activation and residual in the products' stores, cached weight images, nothing kept for a backward pass
                     Activation act = s.arg1 == 1 ? Activation::Gelu : Activation::Silu;
-                    FeedForwardCache unused;
-                    current = feedForwardForwardCached(in, layer.params[0].value, layer.params[1].value, layer.params[2].value,
-                                                       layer.params[3].value, useBf16_, unused, act);
+                    current = feedForwardIncremental(in, layer.params[0].value, layer.params[1].value, layer.params[2].value,
+                                                     layer.params[3].value, useBf16_, act);
                     break;
                 }
                 case LayerKind::Linear:

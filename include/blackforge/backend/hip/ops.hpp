@@ -280,6 +280,26 @@ inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const De
     return detail::projectionFused(cache.hidden, w2, &b2, &input, mode, input.shape());
 }
 
+// The feed-forward block of an incremental step: nothing is kept for a backward pass.  With bf16 projections whose
+// widths allow it (the condition of the fused training block) one library call makes the block, and for at most eight
+// rows that is two launches: the normalisation joins the first product's staging of its rows, the activation its store.
+inline DeviceTensor feedForwardIncremental(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1, const DeviceTensor& w2,
+                                            const DeviceTensor& b2, bool useBf16, Activation act = Activation::Silu) {
+    require(input.rank() >= 2 && w1.rank() == 2 && w2.rank() == 2 && detail::lastDim(input) == w1.dim(0) && w1.dim(1) == w2.dim(0),
+            "feedForward: incompatible shapes on the device");
+    if (!detail::feedForwardFuses(input, w1, useBf16)) {
+        FeedForwardCache unused;
+        return feedForwardForwardCached(input, w1, b1, w2, b2, useBf16, unused, act);
+    }
+    require(b1.rank() == 1 && b1.dim(0) == w1.dim(1), "addBiasSilu: expected input [..., features] and bias [features]");
+    require(b2.rank() == 1 && b2.dim(0) == w2.dim(1), "addBiasResidual: expected input [..., features] and bias [features]");
+    require(w2.dim(1) == detail::lastDim(input), "addBiasResidual: residual shape differs from the product");
+    DeviceTensor out(input.shape());
+    check(bf_hip_rmsnorm_feedforward_bf16(input.data(), w1.data(), b1.data(), w2.data(), b2.data(), static_cast<int>(act), out.data(),
+                                          detail::rowsOf(input), detail::lastDim(input), w1.dim(1), 1, nullptr));
+    return out;
+}
+
 namespace detail {
 inline DeviceTensor feedForwardImpl(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1,
                                      const DeviceTensor& w2, const DeviceTensor& b2, bool useBf16, Activation act) {
@@ -463,14 +483,11 @@ inline void incrementalProjections(const DeviceTensor& newInput, const DeviceTen
                                    float* const (&outs)[3], int mode) {
     const std::size_t dim = newInput.dim(2), rows = newInput.dim(0) * newInput.dim(1);
     if (mode != 0 && dim % 8 == 0 && rows > 0) {
-        // the normalised rows have no reader but the three projections: written as a bf16 image only, and the three
-        // products made by one call over that image
-        DeviceTensor normedImage({rows, dim / 2});
-        check(bf_hip_rmsnorm_img(newInput.data(), nullptr, reinterpret_cast<std::uint16_t*>(normedImage.data()), rows, dim, nullptr));
+        // the normalised rows have no reader but the three projections: one library call normalises and multiplies (for at
+        // most eight rows one launch: the product's kernel normalises the rows while it stages them)
         const float* weights[3] = {wq.data(), wk.data(), wv.data()};
         float* targets[3] = {outs[0], outs[1], outs[2]};
-        check(bf_hip_matmul_bf16_shared_input_img(nullptr, reinterpret_cast<const std::uint16_t*>(normedImage.data()), weights, targets, 3, rows, dim,
-                                                  dim, mode == 2, nullptr));
+        check(bf_hip_rmsnorm_matmul_bf16_shared_input(newInput.data(), weights, targets, 3, rows, dim, dim, mode == 2, nullptr));
     } else {
         DeviceTensor normedFlat = rmsnorm(newInput).reshaped({rows, dim});
         const DeviceTensor* w[3] = {&wq, &wk, &wv};

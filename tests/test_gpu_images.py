@@ -138,6 +138,39 @@ def test_few_queries_over_a_cache_with_room_to_grow(hip, oracle, rng, batch, hea
     assert_bits_equal(timg, oracle.roundToBf16(to), "O image of the tile kernels")
 
 
+@pytest.mark.parametrize("m,d,hidden,act", [(1, 768, 3072, 1), (3, 72, 264, 0), (8, 1032, 520, 2), (1, 8, 8, 1), (5, 256, 256, 0), (9, 64, 128, 1),
+                                            (8, 8200, 64, 0), (40, 128, 512, 1)])
+def test_blocks_of_a_decoding_step_normalise_inside_the_product(hip, oracle, rng, m, d, hidden, act):
+    """bf_hip_rmsnorm_matmul_bf16_shared_input and bf_hip_rmsnorm_feedforward_bf16 (the projections and the feed-forward
+    block of selfAttentionIncremental / forwardIncremental, ops_transformer.cu:133-215) against the separate operators
+    (rmsnorm, then the bf16 products): at most eight rows normalise inside the product's kernel, more rows (and rows too long
+    for that kernel's LDS) run the row kernel first.  Same arithmetic either way; the sum of squares is taken in another
+    order, so the agreement is to the last bits, not bit for bit."""
+    D, ops, call = hip.DeviceTensor, hip.ops, hip.capi.call
+    x = r(rng, m, d, scale=2.0)
+    normed = ops.rmsnorm(D.fromHost(x))
+    assert_close(normed.toHost(), oracle.rmsnorm(x), tol=1e-5, what="rmsnorm")
+    for count, n in ((3, 256), (3, hidden), (1, hidden), (2, 512)):
+        ws = [r(rng, d, n, scale=0.1) for _ in range(count)]
+        dws = [D.fromHost(w) for w in ws]
+        outs = [D((m, n)) for _ in range(count)]
+        barr = (ctypes.c_void_p * count)(*[w.ptr for w in dws])
+        carr = (ctypes.c_void_p * count)(*[o.ptr for o in outs])
+        dx = D.fromHost(x)
+        call("bf_hip_rmsnorm_matmul_bf16_shared_input", dx.ptr, barr, carr, count, m, d, n, 0, None)
+        for i in range(count):
+            assert_close(outs[i].toHost(), ops.matmulBf16(normed, dws[i]).toHost(), tol=2e-5, what=f"projection {i} of {count} of the normalised rows")
+    w1, b1, w2, b2 = r(rng, d, hidden, scale=0.1), r(rng, hidden, scale=0.5), r(rng, hidden, d, scale=0.1), r(rng, d)
+    dw1, db1, dw2, db2, dx = map(D.fromHost, (w1, b1, w2, b2, x))
+    out = D((m, d))
+    call("bf_hip_rmsnorm_feedforward_bf16", dx.ptr, dw1.ptr, db1.ptr, dw2.ptr, db2.ptr, act, out.ptr, m, d, hidden, 0, None)
+    expected, _, _, _ = ops.feedForwardBf16Fused(normed, dw1, db1, dw2, db2, dx, act)
+    assert_close(out.toHost(), expected.toHost(), tol=2e-5, what="feed-forward block of a decoding step")
+    again = D((m, d))
+    call("bf_hip_rmsnorm_feedforward_bf16", dx.ptr, dw1.ptr, db1.ptr, dw2.ptr, db2.ptr, act, again.ptr, m, d, hidden, 0, None)
+    assert_bits_equal(again.toHost(), out.toHost(), "the same block twice")
+
+
 @pytest.mark.parametrize("rows,classes", [(5, 16), (7, 1000), (300, 256), (3, 32000), (2, 40000)])
 def test_cross_entropy_gradient_image(hip, oracle, rng, rows, classes):
     D, call = hip.DeviceTensor, hip.capi.call
