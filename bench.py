@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X operator backend on the headline workload.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras] [--no-decode] [--train LIST]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras] [--no-decode | --decode] [--train LIST]
 
 Workload (BASELINE.json configs[2], the one the fused-attention TFLOP/s metric is quoted on):
 standalone causal fused attention in fp32, batch 8, heads 16, seq 2048, head_dim 64, Q/K/V/dOut
@@ -726,7 +726,8 @@ def main():
                     "steady clocks (3 warm-up steps read 6 %% slower than 20)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the bandwidth kernels and the bf16 GEMMs")
-    ap.add_argument("--no-decode", action="store_true", help="skip the incremental-decoding leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the incremental-decoding leg (--no-extras skips it too)")
+    ap.add_argument("--decode", action="store_true", help="run the incremental-decoding leg even with --no-extras")
     ap.add_argument("--no-graph", action="store_true", help="skip the recorded (HIP graph) variant of the tiny-LM step; for runs under a "
                     "profiler, whose kernel tracing does not survive a stream capture on this stack")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -815,7 +816,7 @@ def main():
         line["train_step"] = {name: (bench_mlp if name == "mlp" else lambda b, s_, w_: bench_train_step(b, name, s_, w_, not args.no_graph))(
                                   bf, max(3, args.steps // 2), max(1, args.warmup // 2))
                               for name in args.train.split(",")}
-    if not args.no_decode:
+    if args.decode or not (args.no_decode or args.no_extras):
         line["decode"] = bench_decode(bf)
     if not args.no_extras:
         line["extras"] = bench_extras(bf, min(10, max(5, args.steps // 2)))   # ten launches a kernel: what profiles/hbm_kernels_and_gemm.md describes
