@@ -1159,11 +1159,11 @@ __global__ void __launch_bounds__(kBlock) splitReduceKernel(const float* __restr
 // be all padding and six workgroups would walk a 768-wide weight alone; here the product is what it is by nature, a walk
 // over the weights: a wavefront owns COLS output columns (rows of Bt), each lane takes 16 bytes (eight bf16) of every
 // column per step, U steps loaded before any is used (a weight of a few MB is in flight all at once, which is what the
-// memory's latency asks for), and multiplies them with the same eight elements of the M rows of A, which the workgroup
-// holds in LDS.  The lanes' sums are added by a butterfly and lane r * COLS + j stores element (r, n0 + j) through the
+// memory's latency asks for), and multiplies them with the same eight elements of the M rows of A (one or two rows: held
+// in LDS by the workgroup; more: read where they lie).  The lanes' sums are added by a butterfly and lane r * COLS + j stores element (r, n0 + j) through the
 // epilogue (fuse 1 included: z and the image of act(z)).  Products in fp32 of the bf16 values, as on the MFMA; the order of
 // additions is fixed (even and odd elements of a lane's eight apart, then the butterfly), so results repeat bit for bit.
-// K, lda and ldb multiples of 8, operands 16-byte aligned, M * K bf16 within the LDS.
+// K, lda and ldb multiples of 8, operands 16-byte aligned, staged rows within the LDS.
 __device__ __forceinline__ void dot8(const uint4v& a, const uint4v& b, float& even, float& odd) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1198,29 +1198,45 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
     };
     int k0 = lane * 8;
     loadSteps(k0);                                           // in flight while A is staged
-    if (e.normInput == nullptr) {
+    // One or two rows are staged in LDS (and normalised on the way, if asked).  More rows are read where they lie: every
+    // wavefront reads the same few KB, which the caches serve, while staging them would cost each workgroup M * K * 2
+    // bytes of copying for the four columns it computes (eight rows of 3072: 48 KB of LDS, three workgroups a compute
+    // unit).  Four columns a wavefront instead of one, to read A less often, measured half again as slow at 4 and 8 rows.
+    constexpr bool STAGED = MR <= 2;
+    if constexpr (!STAGED) {
+    } else if (e.normInput == nullptr) {
         for (int at = int(threadIdx.x) * 8; at < M * K; at += 2048) {
             const int r = at / K, k = at - r * K;            // K is a multiple of 8: a group of eight lies in one row
             *reinterpret_cast<uint4v*>(aRows + at) = *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k);
         }
     } else {
         // x / sqrt(mean(x^2) + eps) with the sum of squares in double and the division in float, as the row kernel that
-        // this replaces forms it (ops.cpp:264-275), rounded to bf16; every workgroup normalises all M rows for itself
-        __shared__ double squares[4];
-        for (int r = 0; r < M; ++r) {
-            const float* row = e.normInput + size_t(r) * K;
-            double ss = 0.0;
-            for (int k = int(threadIdx.x); k < K; k += 256) ss += double(row[k]) * double(row[k]);
+        // this replaces forms it (ops.cpp:264-275), rounded to bf16; every workgroup normalises all M rows for itself, all
+        // rows in one pass (one barrier whatever M)
+        __shared__ double squares[4][MR];
+        double ss[MR];
 #pragma unroll
-            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-            if (lane == 0) squares[threadIdx.x >> 6] = ss;
-            __syncthreads();
-            const float rms = float(sqrt(((squares[0] + squares[1]) + (squares[2] + squares[3])) / double(K) + double(kRmsNormEps)));
-            for (int k = int(threadIdx.x); k < K; k += 256) aRows[r * K + k] = toBf16Bits(row[k] / rms);
-            __syncthreads();                                 // `squares` is free for the next row
+        for (int r = 0; r < MR; ++r) {
+            ss[r] = 0.0;
+            if (r < M)
+                for (int k = int(threadIdx.x); k < K; k += 256) {
+                    const double v = double(e.normInput[size_t(r) * K + k]);
+                    ss[r] += v * v;
+                }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) ss[r] += __shfl_xor(ss[r], o, 64);
+            if (lane == 0) squares[threadIdx.x >> 6][r] = ss[r];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+            if (r < M) {
+                const float rms = float(sqrt(((squares[0][r] + squares[1][r]) + (squares[2][r] + squares[3][r])) / double(K) + double(kRmsNormEps)));
+                for (int k = int(threadIdx.x); k < K; k += 256) aRows[r * K + k] = toBf16Bits(e.normInput[size_t(r) * K + k] / rms);
+            }
         }
     }
-    __syncthreads();
+    if constexpr (STAGED) __syncthreads();
     if (!owner) return;
     while (k0 < K) {
 #pragma unroll
@@ -1230,7 +1246,8 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
 #pragma unroll
                 for (int r = 0; r < MR; ++r) {
                     if (r < M) {
-                        const uint4v a = *reinterpret_cast<const uint4v*>(aRows + r * K + k);
+                        const uint4v a = STAGED ? *reinterpret_cast<const uint4v*>(aRows + r * K + k)
+                                                : *reinterpret_cast<const uint4v*>(A + size_t(r) * lda + k);
 #pragma unroll
                         for (int j = 0; j < COLS; ++j) dot8(a, b[u][j], even[r][j], odd[r][j]);
                     }
@@ -1261,7 +1278,7 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
 template <int MR>
 int launchFewRows(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K, size_t lda, size_t ldb,
                   hipStream_t s) {
-    const size_t smem = M * K * sizeof(unsigned short);
+    const size_t smem = MR <= 2 ? M * K * sizeof(unsigned short) : 0;   // rows of A in LDS: one or two rows only
     // one column a wavefront until that gives every SIMD several wavefronts; four from there on (fewer butterflies per byte)
     if (N <= 8192) {
         auto kernel = gemmBf16FewRowsKernel<MR, 1, 8>;
@@ -1690,12 +1707,14 @@ int launchGemmTn(const unsigned short* A, const unsigned short* B, const Epilogu
 // what the walk over the weights (gemmBf16FewRowsKernel) asks for; launchGemmNt sends every such product there
 bool fewRowsServe(const void* A, const void* Bt, int fuse, size_t M, size_t K, size_t lda, size_t ldb) {
     return g_ntRoute == BF_GEMM_ROUTE_AUTO && M <= 8 && fuse != 2 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
-           M * K * sizeof(unsigned short) <= kFewRowsLds && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) & 15u) == 0;
+           (M > 2 || M * K * sizeof(unsigned short) <= kFewRowsLds) && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) & 15u) == 0;
 }
+// ... and with the rows of A made from fp32 rows by rmsnorm while they are staged (Epilogue::normInput): staged rows only
+bool fewRowsNormalise(size_t M, size_t K) { return M <= 2 && fewRowsServe(nullptr, nullptr, 0, M, K, K, K); }
 bool fusedActivationFits(size_t M, size_t N, size_t K, int fuse) {
     if (g_ntRoute != BF_GEMM_ROUTE_AUTO || N % 8 != 0) return false;
     const size_t cus = size_t(computeUnits());
-    if (M <= 8) return fuse == 1 && K % 8 == 0 && M * K * sizeof(unsigned short) <= kFewRowsLds;   // the walk over the weights
+    if (M <= 8) return fuse == 1 && fewRowsServe(nullptr, nullptr, 1, M, K, K, K);   // the walk over the weights
     const size_t halfTiles = ((M + 127) / 128) * ((N + 255) / 256);   // the 256-row form needs no fewer
     return halfTiles >= cus * 3 / 4 || (N % 192 == 0 && ((M + 127) / 128) * (N / 192) >= cus * 3 / 4);
 }
@@ -2315,7 +2334,7 @@ int bf_hip_rmsnorm_matmul_bf16_shared_input(const float* x, const float* const* 
     for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] != nullptr && c[i] != nullptr, "NULL operand");
     hipStream_t s = asStream(stream);
     const bool stacked = count == 1 || n % 256 == 0;
-    if (stacked && fewRowsServe(nullptr, nullptr, 0, m, k, k, k)) {
+    if (stacked && fewRowsNormalise(m, k)) {
         unsigned short* wImg = nullptr;
         size_t wBytes = 0;
         int st = count > 1 ? weightImage(b, count, k, n, 2, cacheWeight != 0, s, &wImg, &wBytes)
@@ -2349,8 +2368,7 @@ int bf_hip_rmsnorm_feedforward_bf16(const float* input, const float* w1, const f
     Scratch z(m * hidden * sizeof(float)), hImage(m * hidden * sizeof(unsigned short));
     if (z.status != BF_OK) return z.status;
     if (hImage.status != BF_OK) return hImage.status;
-    if (fewRowsServe(nullptr, nullptr, 1, m, d, d, d) && fewRowsServe(nullptr, nullptr, 0, m, hidden, hidden, hidden) &&
-        (reinterpret_cast<uintptr_t>(b1) & 15u) == 0) {
+    if (fewRowsNormalise(m, d) && fewRowsServe(nullptr, nullptr, 0, m, hidden, hidden, hidden) && (reinterpret_cast<uintptr_t>(b1) & 15u) == 0) {
         unsigned short* wImg = nullptr;
         size_t wBytes = 0;
         int st = weightImage(w1, d, hidden, /*transposed=*/true, cacheWeight != 0, s, &wImg, &wBytes);
