@@ -2323,7 +2323,7 @@ int bf_hip_matmul_bf16_shared_input_img(const float* a, const uint16_t* aImage, 
 }
 
 // c[i] = bf16(rmsnorm(x)) b[i]: the projections of an attention block's normalised input (ops_transformer.cu:217-232) for
-// a caller that keeps nothing for a backward pass.  At most eight rows: the normalisation is made by the product's own
+// a caller that keeps nothing for a backward pass.  One or two rows: the normalisation is made by the product's own
 // kernel while it stages the rows (one launch); otherwise the row kernel writes the image and the products follow.
 int bf_hip_rmsnorm_matmul_bf16_shared_input(const float* x, const float* const* b, float* const* c, size_t count, size_t m, size_t k, size_t n,
                                             int cacheWeight, bf_stream_t stream) {
@@ -2356,7 +2356,7 @@ int bf_hip_rmsnorm_matmul_bf16_shared_input(const float* x, const float* const* 
 }
 
 // out = input + act(bf16(rmsnorm(input)) w1 + b1) w2 + b2: the feed-forward block (ops_transformer.cu:182-215) for a
-// caller that keeps nothing for a backward pass (incremental decoding).  At most eight rows: two launches, the
+// caller that keeps nothing for a backward pass (incremental decoding).  One or two rows: two launches, the
 // normalisation made while the first product stages its rows and the activation in its store.
 int bf_hip_rmsnorm_feedforward_bf16(const float* input, const float* w1, const float* b1, const float* w2, const float* b2, int act, float* out,
                                     size_t m, size_t d, size_t hidden, int cacheWeight, bf_stream_t stream) {

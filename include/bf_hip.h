@@ -411,7 +411,7 @@ int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v
  * which runs the training-time operators: ops_transformer.cu:133-180, 182-215).
  * rmsnorm_matmul_bf16_shared_input: c[i] = bf16(rmsnorm(x)) b[i] for up to three weights [k, n] (an attention block's Q, K
  * and V projections of its normalised input).  rmsnorm_feedforward_bf16: out = input + act(bf16(rmsnorm(input)) w1 + b1) w2
- * + b2 (d and hidden multiples of 8).  For at most eight rows the normalisation is made by the first product's kernel
+ * + b2 (d and hidden multiples of 8).  For one or two rows the normalisation is made by the first product's kernel
  * while it stages its rows (double sum of squares, float division, as bf_hip_rmsnorm) and the activation in its store: one
  * launch for the projections, two for the block; more rows run the row kernel and the products one after the other. */
 int bf_hip_rmsnorm_matmul_bf16_shared_input(const float* x, const float* const* b, float* const* c, size_t count, size_t m, size_t k, size_t n,

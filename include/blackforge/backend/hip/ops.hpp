@@ -281,7 +281,7 @@ inline DeviceTensor feedForwardForwardCached(const DeviceTensor& input, const De
 }
 
 // The feed-forward block of an incremental step: nothing is kept for a backward pass.  With bf16 projections whose
-// widths allow it (the condition of the fused training block) one library call makes the block, and for at most eight
+// widths allow it (the condition of the fused training block) one library call makes the block, and for one or two
 // rows that is two launches: the normalisation joins the first product's staging of its rows, the activation its store.
 inline DeviceTensor feedForwardIncremental(const DeviceTensor& input, const DeviceTensor& w1, const DeviceTensor& b1, const DeviceTensor& w2,
                                             const DeviceTensor& b2, bool useBf16, Activation act = Activation::Silu) {
@@ -483,8 +483,8 @@ inline void incrementalProjections(const DeviceTensor& newInput, const DeviceTen
                                    float* const (&outs)[3], int mode) {
     const std::size_t dim = newInput.dim(2), rows = newInput.dim(0) * newInput.dim(1);
     if (mode != 0 && dim % 8 == 0 && rows > 0) {
-        // the normalised rows have no reader but the three projections: one library call normalises and multiplies (for at
-        // most eight rows one launch: the product's kernel normalises the rows while it stages them)
+        // the normalised rows have no reader but the three projections: one library call normalises and multiplies (for
+        // one or two rows one launch: the product's kernel normalises the rows while it stages them)
         const float* weights[3] = {wq.data(), wk.data(), wv.data()};
         float* targets[3] = {outs[0], outs[1], outs[2]};
         check(bf_hip_rmsnorm_matmul_bf16_shared_input(newInput.data(), weights, targets, 3, rows, dim, dim, mode == 2, nullptr));

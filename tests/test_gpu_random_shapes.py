@@ -102,6 +102,52 @@ def test_attention_random_shape(hip, seed):
             assert_close(dV[bi, :, sl], dv, what="dV", scale=0.05)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_decoding_step_kernels_random_shape(hip, seed):
+    """The kernels of an incremental decoding step at random extents: products of one to eight rows in both precisions
+    (walks over the weights) with bias and residual, and attention of one to eight queries over a cache whose buffers are
+    longer than the cached positions (the walk over the cache), against float64."""
+    import ctypes
+    rng = np.random.default_rng(5000 + seed)
+    m, n, k = int(rng.integers(1, 9)), _extent(rng), _extent(rng)
+    if seed % 3 == 0:
+        k = 8 * int(rng.integers(1, 600))          # the bf16 walk asks for a multiple of eight; other lengths stay on the tiles
+    if seed % 4 == 0:
+        n = int(rng.integers(8000, 40000))         # wide enough for four columns a wavefront
+    print(f"few-row products m={m} n={n} k={k}", flush=True)
+    D, ops, call = hip.DeviceTensor, hip.ops, hip.capi.call
+    a, w, bias, res = _rnd(rng, m, k), _rnd(rng, k, n, scale=0.1), _rnd(rng, n), _rnd(rng, m, n)
+    da, dw, dbias, dres = map(D.fromHost, (a, w, bias, res))
+    y = ops.linearBf16Fused(da, dw, dbias, dres).toHost()
+    assert_close(y, _bf16(a).astype(np.float64) @ _bf16(w).astype(np.float64) + bias + res, tol=2e-4, what="bf16 few-row product", scale=0.1 * np.sqrt(k))
+    out = D((m, n))
+    call("bf_hip_gemm_f32_adds", 0, 0, da.ptr, dw.ptr, dbias.ptr, dres.ptr, out.ptr, m, n, k, None)
+    assert_close(out.toHost(), a.astype(np.float64) @ w.astype(np.float64) + bias + res, what="fp32 few-row product", scale=0.1 * np.sqrt(k))
+
+    b, h, new = int(rng.integers(1, 4)), int(rng.integers(1, 5)), int(rng.integers(1, 9))
+    hd = int(rng.choice([4, 8, 16, 32, 40, 64, 96, 128, 192, 256]))
+    old = int(rng.integers(0, 3000))
+    rows = old + new + int(rng.integers(0, 300))
+    print(f"few-query attention batch={b} heads={h} head_dim={hd} newLen={new} oldLen={old} rows={rows}", flush=True)
+    dim, scale = h * hd, 1.0 / np.sqrt(hd)
+    q = _rnd(rng, b, new, dim)
+    kc, vc = (np.full((b, rows, dim), np.nan, f32) for _ in range(2))
+    kc[:, :old + new], vc[:, :old + new] = _rnd(rng, b, old + new, dim), _rnd(rng, b, old + new, dim)
+    dq_, dk_, dv_ = map(D.fromHost, (q, kc, vc))
+    o, mm, ll = D((b, new, dim)), D((b, h, new)), D((b, h, new))
+    call("bf_hip_attention_forward_rows", dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, None, 0, mm.ptr, ll.ptr, b, h, new, old + new, rows, dim,
+         ctypes.c_float(scale), old, None)
+    O, M, L = o.toHost(), mm.toHost(), ll.toHost()
+    zero = np.zeros((new, hd))
+    for bi in range(b):
+        for hi in range(h):
+            sl = slice(hi * hd, (hi + 1) * hd)
+            eo, em, el, _, _, _ = attention_slice(q[bi, :, sl], kc[bi, :old + new, sl], vc[bi, :old + new, sl], zero, scale, old)
+            assert_close(O[bi, :, sl], eo, what="O")
+            assert_close(M[bi, hi], em, what="m", scale=1.0)
+            assert_close(L[bi, hi], el, what="l")
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_row_kernels_random_shape(hip, seed):
     rng = np.random.default_rng(4000 + seed)
