@@ -1296,6 +1296,96 @@ int launchFewRows(const unsigned short* A, const unsigned short* Bt, const Epilo
 }
 constexpr size_t kFewRowsLds = 128 * 1024;   // what the rows of A may take of a compute unit's 160 KB
 
+// Products of a few dozen rows (a decoding step of several sequences, a small batch): 32 x 32 output tiles on the MFMA
+// without LDS staging.  A workgroup owns one tile (blockIdx.x: 32 columns, blockIdx.y: 32 rows) and its eight wavefronts
+// share out the contraction: wavefront w takes K steps w, w + 8, ... of sixteen, and loads its operand fragments
+// straight from memory, which is how they lie there: lane (li, half) needs eight consecutive k of row li of A and of row
+// li of Bt, 16 bytes each.  Twelve steps are loaded before the first is multiplied (a wavefront's share of K = 1536),
+// longer contractions go round again.  The eight partial tiles are added in wavefront order through LDS and stored through
+// the epilogue (bias, residual, split outputs, fuse 1).  K, lda, ldb multiples of 8, operands 16-byte aligned.
+constexpr int kSkinnyWaves = 8, kSkinnyDepth = 12;
+__global__ void __launch_bounds__(64 * kSkinnyWaves) gemmBf16SkinnyKernel(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
+                                                                          Epilogue e, int M, int N, int K, int lda, int ldb, int kPer,
+                                                                          size_t sliceStride) {
+    __shared__ float partial[kSkinnyWaves][32][33];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, li = lane & 31, half = lane >> 5;
+    const int col0 = int(blockIdx.x) * 32, row0 = int(blockIdx.y) * 32;
+    const bool rowLive = row0 + li < M, colLive = col0 + li < N;
+    const unsigned short* aRow = A + size_t(rowLive ? row0 + li : 0) * lda + 8 * half;
+    const unsigned short* bRow = Bt + size_t(colLive ? col0 + li : 0) * ldb + 8 * half;
+    const uint4v none = {0u, 0u, 0u, 0u};
+    float16v acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    // blockIdx.z: the slice of K (kPer, a multiple of 16, each) when few tiles share a long contraction; slice z writes its
+    // sums sliceStride floats after the slice before it and splitReduceKernel adds them, with the epilogue's adds
+    const int kBegin = int(blockIdx.z) * kPer;
+    K = min(K, kBegin + kPer);
+    if (gridDim.z > 1) e.c[0] += size_t(blockIdx.z) * sliceStride;
+    for (int k0 = kBegin + wave * 16; k0 < K; k0 += 16 * kSkinnyWaves * kSkinnyDepth) {   // the same for all lanes of a wavefront
+        uint4v a[kSkinnyDepth], b[kSkinnyDepth];
+#pragma unroll
+        for (int u = 0; u < kSkinnyDepth; ++u) {
+            const int k = k0 + u * 16 * kSkinnyWaves;
+            const bool in = k + 8 * half < K;            // K is a multiple of 8: the second half of the last step may be past the end
+            b[u] = in && colLive ? __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(bRow + k)) : none;
+            a[u] = in && rowLive ? *reinterpret_cast<const uint4v*>(aRow + k) : none;
+        }
+#pragma unroll
+        for (int u = 0; u < kSkinnyDepth; ++u)
+            if (k0 + u * 16 * kSkinnyWaves < K)
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[u]), __builtin_bit_cast(bf16x8, b[u]), acc, 0, 0, 0);
+    }
+    // lane (li, half) holds column li of rows 8 g + 4 half + i
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) partial[wave][8 * g + 4 * half + i][li] = acc[4 * g + i];
+    __syncthreads();
+    for (int at = t; at < 32 * 32; at += 64 * kSkinnyWaves) {
+        const int r = at >> 5, c = at & 31, row = row0 + r, col = col0 + c;
+        if (row < M && col < N) {
+            float v = partial[0][r][c];
+#pragma unroll
+            for (int w = 1; w < kSkinnyWaves; ++w) v += partial[w][r][c];
+            const int which = col / e.splitN;
+            float* C = which == 0 ? e.c[0] : which == 1 ? e.c[1] : e.c[2];
+            if (e.bias) v += e.bias[col];
+            if (e.residual) v += e.residual[size_t(row) * N + col];
+            C[size_t(row) * e.splitN + (col - which * e.splitN)] = v;
+            if (e.fuse == 1) e.image[size_t(row) * N + col] = toBf16Bits(actF1(e.act, v));
+        }
+    }
+}
+int launchSkinny(const unsigned short* A, const unsigned short* Bt, const Epilogue& epi, size_t M, size_t N, size_t K, size_t lda, size_t ldb,
+                 hipStream_t s) {
+    const size_t tiles = ((N + 31) / 32) * ((M + 31) / 32);
+    // few tiles and a long contraction (a feed-forward block's second product): K in slices over more workgroups, at least
+    // four steps a wavefront each, summed in slice order by a second kernel
+    size_t slices = 1;
+    if (tiles < 64 && K >= 2048 && epi.fuse == 0) slices = std::min<size_t>(std::min<size_t>(8, K / 512), 128 / tiles);
+    if (slices > 1) {
+        const size_t kPer = ((K + slices - 1) / slices + 127) / 128 * 128;
+        slices = (K + kPer - 1) / kPer;
+        const size_t count = M * N, sliceStride = (count + 3) / 4 * 4;
+        Scratch partial(slices * sliceStride * sizeof(float));
+        if (partial.status != BF_OK) return partial.status;
+        Epilogue plain{{partial.as<float>(), nullptr, nullptr}, int(N), nullptr, nullptr};
+        const dim3 grid{unsigned((N + 31) / 32), unsigned((M + 31) / 32), unsigned(slices)};
+        gemmBf16SkinnyKernel<<<grid, 64 * kSkinnyWaves, 0, s>>>(A, Bt, plain, int(M), int(N), int(K), int(lda), int(ldb), int(kPer), sliceStride);
+        BF_LAUNCH_CHECK();
+        const int vec = ((reinterpret_cast<uintptr_t>(epi.c[0]) | reinterpret_cast<uintptr_t>(epi.c[1]) | reinterpret_cast<uintptr_t>(epi.c[2]) |
+                          reinterpret_cast<uintptr_t>(epi.residual) | reinterpret_cast<uintptr_t>(epi.bias)) & 15u) == 0 && N % 4 == 0 && epi.splitN % 4 == 0;
+        splitReduceKernel<<<gridFor(count / 4 + 1, kBlock), kBlock, 0, s>>>(partial.as<float>(), epi, count, sliceStride, int(slices), vec, N);
+        BF_LAUNCH_CHECK();
+        return BF_OK;
+    }
+    const dim3 grid{unsigned((N + 31) / 32), unsigned((M + 31) / 32), 1u};
+    gemmBf16SkinnyKernel<<<grid, 64 * kSkinnyWaves, 0, s>>>(A, Bt, epi, int(M), int(N), int(K), int(lda), int(ldb), int((K + 15) / 16 * 16), size_t(0));
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
 // The same kernel for operands that lie the other way round: C[M,N] = A^T * B with A [K, lda] and B [K, ldb], the
 // contraction index K running over ROWS (a weight gradient dW = X^T * G: both the activations X and the gradient G have
 // one row per token).  A K step is 64 rows of either operand, staged in LDS as they lie in memory ([k][m], rows padded
@@ -1709,11 +1799,18 @@ bool fewRowsServe(const void* A, const void* Bt, int fuse, size_t M, size_t K, s
     return g_ntRoute == BF_GEMM_ROUTE_AUTO && M <= 8 && fuse != 2 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
            (M > 2 || M * K * sizeof(unsigned short) <= kFewRowsLds) && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) & 15u) == 0;
 }
+// what the 32 x 32 tiles without LDS staging (gemmBf16SkinnyKernel) ask for: the products between the walk and the big tiles
+bool skinnyServes(const void* A, const void* Bt, int fuse, size_t M, size_t K, size_t lda, size_t ldb) {
+    // five rows and up: below, the walk measures the same or better; past 64 the 128-row tiles are within a few per cent
+    return g_ntRoute == BF_GEMM_ROUTE_AUTO && M >= 5 && M <= 64 && fuse != 2 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 &&
+           ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) & 15u) == 0;
+}
 // ... and with the rows of A made from fp32 rows by rmsnorm while they are staged (Epilogue::normInput): staged rows only
 bool fewRowsNormalise(size_t M, size_t K) { return M <= 2 && fewRowsServe(nullptr, nullptr, 0, M, K, K, K); }
 bool fusedActivationFits(size_t M, size_t N, size_t K, int fuse) {
     if (g_ntRoute != BF_GEMM_ROUTE_AUTO || N % 8 != 0) return false;
     const size_t cus = size_t(computeUnits());
+    if (skinnyServes(nullptr, nullptr, fuse, M, K, K, K)) return fuse == 1;
     if (M <= 8) return fuse == 1 && fewRowsServe(nullptr, nullptr, 1, M, K, K, K);   // the walk over the weights
     const size_t halfTiles = ((M + 127) / 128) * ((N + 255) / 256);   // the 256-row form needs no fewer
     return halfTiles >= cus * 3 / 4 || (N % 192 == 0 && ((M + 127) / 128) * (N / 192) >= cus * 3 / 4);
@@ -1744,6 +1841,7 @@ int launchGemmNt(const unsigned short* A, const unsigned short* Bt, const Epilog
             return launchWideWave<3>(A, Bt, epi, M, N, K, lda, ldb, s, g_ntRoute == BF_GEMM_ROUTE_WIDE_192_PERSISTENT);
         default: break;
     }
+    if (skinnyServes(A, Bt, epi.fuse, M, K, lda, ldb)) return N == 0 ? BF_OK : launchSkinny(A, Bt, epi, M, N, K, lda, ldb, s);
     if (fewRowsServe(A, Bt, epi.fuse, M, K, lda, ldb)) {   // a walk over the weights, no tiles
         if (M == 0 || N == 0) return BF_OK;
         return M == 1 ? launchFewRows<1>(A, Bt, epi, M, N, K, lda, ldb, s) : M == 2 ? launchFewRows<2>(A, Bt, epi, M, N, K, lda, ldb, s)
