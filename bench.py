@@ -647,7 +647,7 @@ def bench_decode(bf, tokens=32, prompt=1024):
     from blackforge_amd import hostlayer as hl
     c = TRAIN_CONFIGS["gpt_small"]
     out = {}
-    for mode, bf16 in (("bf16", True), ("fp32", False)):
+    for mode, bf16 in (("fp32", False), ("bf16", True)):
         model = hl.HostModel(lm_layers(hl, c["vocab"], c["dim"], 2 * prompt, c["heads"], c["ffn"], c["act"], c["blocks"]), use_bf16=bf16)
         rng = np.random.default_rng(42)
         for i, count in enumerate(model.counts):
