@@ -1179,6 +1179,11 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
     const int lane = threadIdx.x & 63;
     const int n0 = (int(blockIdx.x) * 4 + int(threadIdx.x >> 6)) * COLS;
     const bool owner = n0 < N;                               // a wavefront past the last column only helps to stage A
+    // lane r * COLS + j stores element (r, n0 + j): what the epilogue adds there is fetched now, not after the sums
+    const int storeRow = lane / COLS, storeCol = n0 + lane % COLS;
+    const bool stores = owner && lane < MR * COLS && storeRow < M && storeCol < N;
+    const float biasHere = stores && e.bias ? e.bias[storeCol] : 0.0f;
+    const float residualHere = stores && e.residual ? e.residual[size_t(storeRow) * N + storeCol] : 0.0f;
     float even[MR][COLS], odd[MR][COLS];
 #pragma unroll
     for (int r = 0; r < MR; ++r)
@@ -1268,8 +1273,8 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
             if (lane == r * COLS + j && r < M && col < N) {
                 const int which = col / e.splitN;
                 float* C = which == 0 ? e.c[0] : which == 1 ? e.c[1] : e.c[2];
-                if (e.bias) v += e.bias[col];
-                if (e.residual) v += e.residual[size_t(r) * N + col];
+                if (e.bias) v += biasHere;
+                if (e.residual) v += residualHere;
                 C[size_t(r) * e.splitN + (col - which * e.splitN)] = v;
                 if (e.fuse == 1) e.image[size_t(r) * N + col] = toBf16Bits(actF1(e.act, v));
             }
