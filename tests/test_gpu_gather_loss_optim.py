@@ -112,6 +112,58 @@ def test_concat_seq_and_argmax(hip, oracle, rng):
     assert ops.argmaxLastPosition(D.fromHost(logits)) == 0
 
 
+def test_position_on_the_device_entry_points(hip, oracle, rng):
+    """The entry points of a decoding step that read the position from device memory (bf_hip_positional_forward_indirect,
+    bf_hip_kv_append_indirect, bf_hip_argmax_last_position_device, bf_hip_counter_add) and the strided copy of the growing
+    cache (bf_hip_copy_pitched), each against the host-position operator it mirrors (addPositionalEmbeddingAt ops.hpp:391,
+    concatSeq ops_transformer.cu:22-58, argmaxLastPosition main.cpp:504-518) or numpy, bit for bit; a position that does
+    not fit writes nothing."""
+    import ctypes
+    D, ops, call = hip.DeviceTensor, hip.ops, hip.capi.call
+    counter = D.fromHost(np.array([5], np.int32).view(f32))
+    as_int = lambda: int(counter.toHost().view(np.int32)[0])
+    call("bf_hip_counter_add", counter.ptr, 3, None)
+    call("bf_hip_counter_add", counter.ptr, -1, None)
+    assert as_int() == 7
+    for dim in (12, 7):   # 16-byte rows and rows that are not
+        batch, seq, max_seq = 3, 2, 11
+        x, table = r(rng, batch, seq, dim), r(rng, max_seq, dim)
+        out, dx, dtable = D.fromHost(np.zeros_like(x)), D.fromHost(x), D.fromHost(table)   # named: a temporary's buffer goes back to the pool at once
+        call("bf_hip_positional_forward_indirect", dx.ptr, dtable.ptr, out.ptr, batch, seq, dim, max_seq, counter.ptr, None)
+        assert_bits_equal(out.toHost(), ops.addPositionalEmbeddingAt(D.fromHost(x), D.fromHost(table), 7).toHost(), "positions from the device")
+        too_far = D.fromHost(np.array([max_seq - 1], np.int32).view(f32))
+        untouched = D.fromHost(np.full_like(x, 3.0))
+        call("bf_hip_positional_forward_indirect", dx.ptr, dtable.ptr, untouched.ptr, batch, seq, dim, max_seq, too_far.ptr, None)
+        assert_bits_equal(untouched.toHost(), np.full_like(x, 3.0), "a position past the table writes nothing")
+        # append at row 7 of caches with 10 rows a sequence
+        capacity = 10
+        kc, vc = r(rng, batch, capacity, dim), r(rng, batch, capacity, dim)
+        kn, vn = r(rng, batch, seq, dim), r(rng, batch, seq, dim)
+        dk, dv, dkn, dvn = D.fromHost(kc), D.fromHost(vc), D.fromHost(kn), D.fromHost(vn)
+        call("bf_hip_kv_append_indirect", dk.ptr, dv.ptr, dkn.ptr, dvn.ptr, batch, seq, dim, capacity, counter.ptr, None)
+        ek, ev = kc.copy(), vc.copy()
+        ek[:, 7:9], ev[:, 7:9] = kn, vn
+        assert_bits_equal(dk.toHost(), ek, "keys appended at the device-side position")
+        assert_bits_equal(dv.toHost(), ev, "values appended at the device-side position")
+        full = D.fromHost(np.array([9], np.int32).view(f32))
+        call("bf_hip_kv_append_indirect", dk.ptr, dv.ptr, dkn.ptr, dvn.ptr, batch, seq, dim, capacity, full.ptr, None)
+        assert_bits_equal(dk.toHost(), ek, "rows that do not fit are not written")
+        # the dense [batch, length, dim] view of a cache and back
+        dense = D((batch, 9, dim))
+        call("bf_hip_copy_pitched", dense.ptr, 9 * dim, dk.ptr, capacity * dim, 9 * dim, batch, None)
+        assert_bits_equal(dense.toHost(), ek[:, :9], "dense view of the cache")
+    for vocab in (1, 5, 1000, 50257):
+        logits = r(rng, 1, 3, vocab)
+        logits[0, 2, vocab // 2] = logits[0, 2].max()   # a tie: the lower index must win
+        token, history, dlogits = D.fromHost(np.zeros((1, 1), f32)), D.fromHost(np.full(4, -1.0, f32)), D.fromHost(logits)
+        call("bf_hip_argmax_last_position_device", dlogits.ptr, 3, vocab, token.ptr, history.ptr, 4, counter.ptr, ctypes.c_longlong(-5), None)
+        expected = oracle.argmaxLastPosition(logits[0])
+        assert token.toHost()[0, 0] == expected
+        np.testing.assert_array_equal(history.toHost(), [-1, -1, expected, -1])   # slot 7 - 5
+        call("bf_hip_argmax_last_position_device", dlogits.ptr, 3, vocab, token.ptr, history.ptr, 4, counter.ptr, ctypes.c_longlong(0), None)
+        np.testing.assert_array_equal(history.toHost(), [-1, -1, expected, -1])   # slot 7 lies outside: left alone
+
+
 @pytest.mark.parametrize("rows,classes", [(1, 2), (2, 3), (7, 13), (512, 256), (5, 1000), (3, 32000), (2, 50257), (1, 70001), (3, 40000),
                                           (2, 50260)])
 def test_cross_entropy(hip, oracle, rng, rows, classes):
