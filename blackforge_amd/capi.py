@@ -130,6 +130,8 @@ SIGNATURES = {
     "bf_hip_argmax_last_position_device": [P, c_size, c_size, P, P, c_size, P, ctypes.c_longlong, S],
     "bf_hip_counter_add": [P, ctypes.c_int, S],
     "bf_hip_rmsnorm_matmul_bf16_shared_input": [P, ctypes.POINTER(P), ctypes.POINTER(P), c_size, c_size, c_size, c_size, ctypes.c_int, S],
+    "bf_hip_rmsnorm_matmul_f32_shared_input": [P, ctypes.POINTER(P), ctypes.POINTER(P), c_size, c_size, c_size, c_size, S],
+    "bf_hip_rmsnorm_feedforward_f32": [P, P, P, P, P, ctypes.c_int, P, c_size, c_size, c_size, S],
     "bf_hip_rmsnorm_feedforward_bf16": [P, P, P, P, P, ctypes.c_int, P, c_size, c_size, c_size, ctypes.c_int, S],
     "bf_hip_attention_backward_img": [P, P, P, P, P, P, P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, c_size, c_size, c_float,
                                       c_size, S],

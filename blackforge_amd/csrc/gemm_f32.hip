@@ -375,6 +375,43 @@ __global__ void __launch_bounds__(kBlock) sliceSumKernel(const float* __restrict
     C[i] = withAdds(sum, bias, residual, i, i % N);
 }
 
+// up to three products of one shape in one launch of the few-row kernel, and of the kernel that sums their K slices
+struct FewRowsProducts {
+    const float* A[3];
+    const float* B[3];
+    float* out[3];          // with K slices: the product's first slice in the scratch buffer
+    const float* bias[3];
+    const float* residual[3];
+    // one or two rows only: A[] is ignored and the rows are those of rmsnorm(normInput) ([M, K], dense), normalised while
+    // the kernel stages its slice of them (a decoding step's projections and feed-forward block)
+    const float* normInput;
+    int act;                // BF_ACT_* applied after the adds, or -1
+};
+__device__ __forceinline__ float actOrNot(int act, float v) {
+    return act < 0 ? v : act == BF_ACT_SILU ? siluF(v) : act == BF_ACT_GELU ? geluF(v) : reluF(v);
+}
+// sliceSumKernel for product blockIdx.y: partial sums at partial[y], `slices` of them `stride` floats apart, to C[y]
+__global__ void __launch_bounds__(kBlock) sliceSumProductsKernel(FewRowsProducts g, float* const C0, float* const C1, float* const C2, size_t count,
+                                                                 size_t stride, int slices, size_t N) {
+    const int which = blockIdx.y;
+    const float* partial = which == 0 ? g.out[0] : which == 1 ? g.out[1] : g.out[2];
+    float* C = which == 0 ? C0 : which == 1 ? C1 : C2;
+    const float* bias = which == 0 ? g.bias[0] : which == 1 ? g.bias[1] : g.bias[2];
+    const float* residual = which == 0 ? g.residual[0] : which == 1 ? g.residual[1] : g.residual[2];
+    const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float sum = partial[i];
+    for (int s0 = 1; s0 < slices; s0 += 8) {   // eight loads in flight, added in index order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = s0 + u < slices ? partial[size_t(s0 + u) * stride + i] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (s0 + u < slices) sum += v[u];
+    }
+    C[i] = actOrNot(g.act, withAdds(sum, bias, residual, i, i % N));
+}
+
 // Products of at most eight rows, C[M, N] = A[M, K] B[K, N] (a step of incremental decoding: one new token per sequence),
 // as a walk over B: a lane owns VEC adjacent columns, the WAVES wavefronts of a workgroup take every WAVES-th row of the
 // workgroup's K slice, eight rows loaded before any is used, and multiply them with the slice's elements of A, which the
@@ -382,9 +419,14 @@ __global__ void __launch_bounds__(kBlock) sliceSumKernel(const float* __restrict
 // slices (blockIdx.y) a slice writes its sums `sliceStride` floats after the slice before it and sliceSumKernel adds them,
 // with one slice the adds of the epilogue are made here.  VEC 4: N a multiple of 4 and B 16-byte aligned.
 template <int MR, int VEC, int WAVES>
-__global__ void __launch_bounds__(64 * WAVES) gemmF32FewRowsKernel(const float* __restrict__ A, const float* __restrict__ B, float* out,
-                                                            int M, int N, int K, int kPer, size_t sliceStride,
-                                                            const float* __restrict__ bias, const float* residual) {   // residual may be out
+__global__ void __launch_bounds__(64 * WAVES) gemmF32FewRowsKernel(FewRowsProducts g, int M, int N, int K, int kPer, size_t sliceStride) {
+    // blockIdx.z: which of up to three products of one shape (the Q, K and V projections of a decoding step)
+    const int which = blockIdx.z;
+    const float* __restrict__ A = which == 0 ? g.A[0] : which == 1 ? g.A[1] : g.A[2];
+    const float* __restrict__ B = which == 0 ? g.B[0] : which == 1 ? g.B[1] : g.B[2];
+    float* out = which == 0 ? g.out[0] : which == 1 ? g.out[1] : g.out[2];
+    const float* __restrict__ bias = which == 0 ? g.bias[0] : which == 1 ? g.bias[1] : g.bias[2];
+    const float* residual = which == 0 ? g.residual[0] : which == 1 ? g.residual[1] : g.residual[2];   // may be `out`
     extern __shared__ float fewRowsLds[];
     constexpr int U = 8, WIDTH = 64 * VEC;
     float* aRows = fewRowsLds;                      // [MR][kPer]
@@ -408,9 +450,36 @@ __global__ void __launch_bounds__(64 * WAVES) gemmF32FewRowsKernel(const float* 
     };
     int k0 = kBeg + wave;
     loadRows(k0);                                   // in flight while A is staged
-    for (int i = t; i < M * kLen; i += 64 * WAVES) {
-        const int r = i / kLen, k = i - r * kLen;
-        aRows[r * kPer + k] = A[size_t(r) * K + kBeg + k];
+    if (g.normInput == nullptr) {
+        for (int i = t; i < M * kLen; i += 64 * WAVES) {
+            const int r = i / kLen, k = i - r * kLen;
+            aRows[r * kPer + k] = A[size_t(r) * K + kBeg + k];
+        }
+    } else {
+        // x / sqrt(mean(x^2) + eps), sum of squares in double, division in float (the row kernel's arithmetic, ops.cpp:264-275);
+        // every workgroup sums whole rows for itself and stages its K slice of them
+        __shared__ double squares[WAVES][MR];
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+            double ss = 0.0;
+            if (r < M)
+                for (int k = t; k < K; k += 64 * WAVES) {
+                    const double v = double(g.normInput[size_t(r) * K + k]);
+                    ss += v * v;
+                }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            if (lane == 0) squares[wave][r] = ss;
+        }
+        __syncthreads();
+        for (int i = t; i < M * kLen; i += 64 * WAVES) {
+            const int r = i / kLen, k = i - r * kLen;
+            double ss = 0.0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) ss += squares[w][r];
+            const float rms = float(sqrt(ss / double(K) + double(kRmsNormEps)));
+            aRows[r * kPer + k] = g.normInput[size_t(r) * K + kBeg + k] / rms;
+        }
     }
     __syncthreads();
     float acc[MR][VEC];
@@ -449,19 +518,21 @@ __global__ void __launch_bounds__(64 * WAVES) gemmF32FewRowsKernel(const float* 
 #pragma unroll
             for (int w = 1; w < WAVES; ++w) total += sums[(w * MR + r) * WIDTH + c];
             const size_t at = size_t(r) * N + column;
-            dst[at] = withAdds(total, bias, residual, at, size_t(column));
+            dst[at] = gridDim.y > 1 ? total : actOrNot(g.act, withAdds(total, bias, residual, at, size_t(column)));
         }
     }
 }
+// `products` (1 to 3) of one shape: p.out = where each product goes, p.bias / p.residual its adds
 template <int MR>
-int launchFewRowsF32(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, const float* bias, const float* residual,
-                     hipStream_t s, bool* served) {
+int launchFewRowsF32(const FewRowsProducts& p, size_t products, size_t M, size_t N, size_t K, hipStream_t s, bool* served) {
     *served = false;
     constexpr int WAVES = MR <= 4 ? 8 : 4;          // WAVES * MR * 256 sums in LDS
-    const bool vec = N % 4 == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
+    bool vec = N % 4 == 0;
+    for (size_t i = 0; i < products; ++i) vec = vec && (reinterpret_cast<uintptr_t>(p.B[i]) & 15u) == 0;
     const size_t width = vec ? 256 : 64, colBlocks = (N + width - 1) / width;
     // K slices of at least one round of loads per wavefront (8 * WAVES rows), at most 32 of them, about two workgroups
-    // per compute unit; the slices are summed by a second kernel
+    // per compute unit and product (the same cut whatever the number of products, so that a product's bits do not depend on
+    // what it is launched with); the slices are summed by a second kernel
     const size_t cus = size_t(computeUnits()), round = size_t(8) * WAVES;
     size_t slices = std::max<size_t>(1, std::min<size_t>(std::min<size_t>((K + round - 1) / round, 32), 2 * cus / colBlocks));
     size_t kPer = ((K + slices - 1) / slices + 3) / 4 * 4;
@@ -469,31 +540,41 @@ int launchFewRowsF32(const float* A, const float* B, float* C, size_t M, size_t 
     const size_t smem = (size_t(MR) * kPer + size_t(WAVES) * MR * width) * sizeof(float);
     if (smem > 96 * 1024) return BF_OK;             // rows of A too long for the LDS: the tile kernels serve
     const size_t count = M * N;
-    Scratch partial(slices > 1 ? slices * count * sizeof(float) : 0);
+    Scratch partial(slices > 1 ? products * slices * count * sizeof(float) : 0);
     if (partial.status != BF_OK) return partial.status;
-    float* out = slices > 1 ? partial.as<float>() : C;
-    const dim3 grid{unsigned(colBlocks), unsigned(slices), 1u};
+    FewRowsProducts g = p;
+    if (slices > 1)
+        for (size_t i = 0; i < products; ++i) {
+            g.out[i] = partial.as<float>() + i * slices * count;
+            g.bias[i] = g.residual[i] = nullptr;    // added when the slices are summed
+        }
+    const dim3 grid{unsigned(colBlocks), unsigned(slices), unsigned(products)};
     int st;
     if (vec) {
         auto kernel = gemmF32FewRowsKernel<MR, 4, WAVES>;
         st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
         if (st != BF_OK) return st;
-        kernel<<<grid, 64 * WAVES, smem, s>>>(A, B, out, int(M), int(N), int(K), int(kPer), count, slices > 1 ? nullptr : bias,
-                                              slices > 1 ? nullptr : residual);
+        kernel<<<grid, 64 * WAVES, smem, s>>>(g, int(M), int(N), int(K), int(kPer), count);
     } else {
         auto kernel = gemmF32FewRowsKernel<MR, 1, WAVES>;
         st = allowDynamicSharedMemory(reinterpret_cast<const void*>(kernel), smem);
         if (st != BF_OK) return st;
-        kernel<<<grid, 64 * WAVES, smem, s>>>(A, B, out, int(M), int(N), int(K), int(kPer), count, slices > 1 ? nullptr : bias,
-                                              slices > 1 ? nullptr : residual);
+        kernel<<<grid, 64 * WAVES, smem, s>>>(g, int(M), int(N), int(K), int(kPer), count);
     }
     BF_LAUNCH_CHECK();
     if (slices > 1) {
-        sliceSumKernel<<<gridFor(count, kBlock), kBlock, 0, s>>>(partial.as<float>(), C, count, count, int(slices), N, bias, residual);
+        FewRowsProducts sums = g;                   // out[i]: the partial sums; bias, residual and activation from the caller
+        for (size_t i = 0; i < products; ++i) { sums.bias[i] = p.bias[i]; sums.residual[i] = p.residual[i]; }
+        const dim3 sumGrid{unsigned((count + kBlock - 1) / kBlock), unsigned(products), 1u};
+        sliceSumProductsKernel<<<sumGrid, kBlock, 0, s>>>(sums, p.out[0], p.out[1], p.out[2], count, count, int(slices), N);
         BF_LAUNCH_CHECK();
     }
     *served = true;
     return BF_OK;
+}
+inline int launchFewRowsF32Any(const FewRowsProducts& p, size_t products, size_t M, size_t N, size_t K, hipStream_t s, bool* served) {
+    return M == 1 ? launchFewRowsF32<1>(p, products, M, N, K, s, served) : M == 2 ? launchFewRowsF32<2>(p, products, M, N, K, s, served)
+         : M <= 4 ? launchFewRowsF32<4>(p, products, M, N, K, s, served) : launchFewRowsF32<8>(p, products, M, N, K, s, served);
 }
 
 template <int BM, int BN>
@@ -529,10 +610,8 @@ int gemmF32(int transA, int transB, const float* A, const float* B, float* C, si
     hipStream_t s = asStream(stream);
     if (!transA && !transB && M <= 8 && N < (size_t(1) << 31) && K < (size_t(1) << 31)) {   // a walk over B, no tiles
         bool served = false;
-        int st = M == 1 ? launchFewRowsF32<1>(A, B, C, M, N, K, bias, residual, s, &served)
-               : M == 2 ? launchFewRowsF32<2>(A, B, C, M, N, K, bias, residual, s, &served)
-               : M <= 4 ? launchFewRowsF32<4>(A, B, C, M, N, K, bias, residual, s, &served)
-                        : launchFewRowsF32<8>(A, B, C, M, N, K, bias, residual, s, &served);
+        const FewRowsProducts one{{A, nullptr, nullptr}, {B, nullptr, nullptr}, {C, nullptr, nullptr}, {bias, nullptr, nullptr}, {residual, nullptr, nullptr}, nullptr, -1};
+        int st = launchFewRowsF32Any(one, 1, M, N, K, s, &served);
         if (st != BF_OK || served) return st;
     }
     // Large tiles once they alone can fill the chip twice over; small tiles otherwise.
@@ -595,11 +674,88 @@ extern "C" int bf_hip_gemm_f32_adds(int transA, int transB, const float* A, cons
     return gemmF32(transA, transB, A, B, C, M, N, K, bias, residual, stream);
 }
 
+// c[i] = rmsnorm(x) b[i] in fp32 for up to three weights [k, n]: the projections of an attention block's normalised input
+// (ops_transformer.cu:107-111) for a caller that keeps nothing for a backward pass.  One or two rows: the normalisation is
+// made by the products' kernel while it stages the rows; otherwise the row kernel runs first.
+extern "C" int bf_hip_rmsnorm_matmul_f32_shared_input(const float* x, const float* const* b, float* const* c, size_t count, size_t m, size_t k,
+                                                      size_t n, bf_stream_t stream) {
+    BF_REQUIRE(count >= 1 && count <= 3, "count must be 1, 2 or 3");
+    BF_REQUIRE(b && c, "NULL pointer array");
+    if (m == 0 || n == 0) return BF_OK;
+    BF_REQUIRE(k > 0 && x != nullptr, "NULL or empty input");
+    for (size_t i = 0; i < count; ++i) BF_REQUIRE(b[i] != nullptr && c[i] != nullptr, "NULL operand");
+    if (m <= 2 && n < (size_t(1) << 31) && k < (size_t(1) << 31)) {
+        FewRowsProducts g = {};
+        g.act = -1;
+        g.normInput = x;
+        for (size_t i = 0; i < count; ++i) { g.B[i] = b[i]; g.out[i] = c[i]; }
+        bool served = false;
+        int st = launchFewRowsF32Any(g, count, m, n, k, asStream(stream), &served);
+        if (st != BF_OK || served) return st;
+    }
+    Scratch normed(m * k * sizeof(float));
+    if (normed.status != BF_OK) return normed.status;
+    int st = bf_hip_rmsnorm(x, normed.as<float>(), m, k, stream);
+    if (st != BF_OK) return st;
+    bf_gemm_f32_problem problems[3];
+    for (size_t i = 0; i < count; ++i) problems[i] = bf_gemm_f32_problem{normed.as<float>(), b[i], c[i], nullptr, nullptr, m, n, k, 0, 0};
+    return bf_hip_gemm_f32_group(problems, count, stream);
+}
+
+// out = input + act(rmsnorm(input) w1 + b1) w2 + b2 in fp32: the feed-forward block (ops_transformer.cu:182-215) for a caller
+// that keeps nothing for a backward pass.  One or two rows: the first product normalises while it stages its rows and the
+// activation is applied where its K slices are summed.
+extern "C" int bf_hip_rmsnorm_feedforward_f32(const float* input, const float* w1, const float* b1, const float* w2, const float* b2, int act,
+                                              float* out, size_t m, size_t d, size_t hidden, bf_stream_t stream) {
+    if (m == 0) return BF_OK;
+    BF_REQUIRE(d > 0 && hidden > 0, "d and hidden must be positive");
+    BF_REQUIRE(act == BF_ACT_SILU || act == BF_ACT_GELU || act == BF_ACT_RELU, "unknown activation");
+    BF_REQUIRE(input && w1 && b1 && w2 && b2 && out, "NULL pointer");
+    Scratch h(m * hidden * sizeof(float));
+    if (h.status != BF_OK) return h.status;
+    bool served = false;
+    if (m <= 2 && d < (size_t(1) << 31) && hidden < (size_t(1) << 31)) {
+        FewRowsProducts g = {};
+        g.act = act;
+        g.normInput = input;
+        g.B[0] = w1; g.out[0] = h.as<float>(); g.bias[0] = b1;
+        int st = launchFewRowsF32Any(g, 1, m, hidden, d, asStream(stream), &served);
+        if (st != BF_OK) return st;
+    }
+    if (!served) {
+        Scratch normed(m * d * sizeof(float)), z(m * hidden * sizeof(float));
+        if (normed.status != BF_OK) return normed.status;
+        if (z.status != BF_OK) return z.status;
+        int st = bf_hip_rmsnorm(input, normed.as<float>(), m, d, stream);
+        if (st == BF_OK) st = bf_hip_gemm_f32(0, 0, normed.as<float>(), w1, z.as<float>(), m, hidden, d, stream);
+        if (st == BF_OK) st = bf_hip_add_bias_act(z.as<float>(), b1, h.as<float>(), m, hidden, act, stream);
+        if (st != BF_OK) return st;
+    }
+    return bf_hip_gemm_f32_adds(0, 0, h.as<float>(), w2, b2, input, out, m, d, hidden, stream);
+}
+
 extern "C" int bf_hip_gemm_f32_group(const bf_gemm_f32_problem* problems, size_t count, bf_stream_t stream) {
     if (count == 0) return BF_OK;
     BF_REQUIRE(problems != nullptr, "NULL problem list");
     // one launch when every product is small enough for the 32 x 32 form without K slices (the form bf_hip_gemm_f32 itself
     // would pick); otherwise, or beyond eight products, the products are launched one after the other
+    // two or three products of at most eight rows and one shape (the Q, K and V projections of a decoding step): one walk
+    if (count >= 2 && count <= 3) {
+        const bf_gemm_f32_problem& f = problems[0];
+        bool alike = f.M >= 1 && f.M <= 8 && f.N >= 1 && f.K >= 1 && f.N < (size_t(1) << 31) && f.K < (size_t(1) << 31);
+        FewRowsProducts g = {};
+        g.act = -1;
+        for (size_t i = 0; i < count && alike; ++i) {
+            const bf_gemm_f32_problem& p = problems[i];
+            alike = !p.transA && !p.transB && p.M == f.M && p.N == f.N && p.K == f.K && p.A && p.B && p.C;
+            g.A[i] = p.A; g.B[i] = p.B; g.out[i] = p.C; g.bias[i] = p.bias; g.residual[i] = p.residual;
+        }
+        if (alike) {
+            bool served = false;
+            int st = launchFewRowsF32Any(g, count, f.M, f.N, f.K, asStream(stream), &served);
+            if (st != BF_OK || served) return st;
+        }
+    }
     const size_t cus = size_t(computeUnits());
     auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     bool together = count <= size_t(kMaxGroup) && count > 1, vec = true;
@@ -609,7 +765,8 @@ extern "C" int bf_hip_gemm_f32_group(const bf_gemm_f32_problem* problems, size_t
         if (p.M == 0 || p.N == 0) continue;
         BF_REQUIRE(p.C != nullptr, "NULL output");
         const size_t tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
-        together = p.K > 0 && p.K < size_t(16) * SBK && tiles * 2 <= cus && p.M < (size_t(1) << 31) && p.N < (size_t(1) << 31) && p.A && p.B;
+        together = p.K > 0 && p.K < size_t(16) * SBK && tiles * 2 <= cus && p.M < (size_t(1) << 31) && p.N < (size_t(1) << 31) && p.A && p.B &&
+                   (p.transA || p.transB || p.M > 8);   // a product of a few rows is a walk when launched alone: the same here
         vec = vec && aligned16(p.A) && aligned16(p.B) && (p.transA ? p.M : p.K) % 4 == 0 && (p.transB ? p.K : p.N) % 4 == 0;
         tilesM = std::max(tilesM, (p.M + SBT - 1) / SBT);
         tilesN = std::max(tilesN, (p.N + SBT - 1) / SBT);

@@ -414,6 +414,12 @@ int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v
  * + b2 (d and hidden multiples of 8).  For one or two rows the normalisation is made by the first product's kernel
  * while it stages its rows (double sum of squares, float division, as bf_hip_rmsnorm) and the activation in its store: one
  * launch for the projections, two for the block; more rows run the row kernel and the products one after the other. */
+/* The same two blocks in fp32 (products by bf_hip_gemm_f32's kernels): the normalisation inside the first product for one
+ * or two rows, the feed-forward's activation where that product's K slices are summed. */
+int bf_hip_rmsnorm_matmul_f32_shared_input(const float* x, const float* const* b, float* const* c, size_t count, size_t m, size_t k, size_t n,
+                                           bf_stream_t stream);
+int bf_hip_rmsnorm_feedforward_f32(const float* input, const float* w1, const float* b1, const float* w2, const float* b2, int act, float* out,
+                                   size_t m, size_t d, size_t hidden, bf_stream_t stream);
 int bf_hip_rmsnorm_matmul_bf16_shared_input(const float* x, const float* const* b, float* const* c, size_t count, size_t m, size_t k, size_t n,
                                             int cacheWeight, bf_stream_t stream);
 int bf_hip_rmsnorm_feedforward_bf16(const float* input, const float* w1, const float* b1, const float* w2, const float* b2, int act, float* out,

@@ -287,6 +287,15 @@ inline DeviceTensor feedForwardIncremental(const DeviceTensor& input, const Devi
                                             const DeviceTensor& b2, bool useBf16, Activation act = Activation::Silu) {
     require(input.rank() >= 2 && w1.rank() == 2 && w2.rank() == 2 && detail::lastDim(input) == w1.dim(0) && w1.dim(1) == w2.dim(0),
             "feedForward: incompatible shapes on the device");
+    if (!useBf16 && input.elementCount() > 0) {
+        require(b1.rank() == 1 && b1.dim(0) == w1.dim(1), "addBiasSilu: expected input [..., features] and bias [features]");
+        require(b2.rank() == 1 && b2.dim(0) == w2.dim(1), "addBiasResidual: expected input [..., features] and bias [features]");
+        require(w2.dim(1) == detail::lastDim(input), "addBiasResidual: residual shape differs from the product");
+        DeviceTensor out(input.shape());
+        check(bf_hip_rmsnorm_feedforward_f32(input.data(), w1.data(), b1.data(), w2.data(), b2.data(), static_cast<int>(act), out.data(),
+                                             detail::rowsOf(input), detail::lastDim(input), w1.dim(1), nullptr));
+        return out;
+    }
     if (!detail::feedForwardFuses(input, w1, useBf16)) {
         FeedForwardCache unused;
         return feedForwardForwardCached(input, w1, b1, w2, b2, useBf16, unused, act);
@@ -489,11 +498,14 @@ inline void incrementalProjections(const DeviceTensor& newInput, const DeviceTen
         float* targets[3] = {outs[0], outs[1], outs[2]};
         check(bf_hip_rmsnorm_matmul_bf16_shared_input(newInput.data(), weights, targets, 3, rows, dim, dim, mode == 2, nullptr));
     } else {
-        DeviceTensor normedFlat = rmsnorm(newInput).reshaped({rows, dim});
-        const DeviceTensor* w[3] = {&wq, &wk, &wv};
-        for (int i = 0; i < 3; ++i) {
-            if (mode == 0) check(bf_hip_gemm_f32_adds(0, 0, normedFlat.data(), w[i]->data(), nullptr, nullptr, outs[i], rows, dim, dim, nullptr));
-            else check(bf_hip_linear_bf16_img(normedFlat.data(), nullptr, w[i]->data(), nullptr, nullptr, outs[i], rows, dim, dim, mode == 2, nullptr));
+        const float* weights[3] = {wq.data(), wk.data(), wv.data()};
+        float* targets[3] = {outs[0], outs[1], outs[2]};
+        if (mode == 0) {   // fp32: one library call as well (one or two rows: the products' kernel normalises, all three in one launch)
+            check(bf_hip_rmsnorm_matmul_f32_shared_input(newInput.data(), weights, targets, 3, rows, dim, dim, nullptr));
+        } else {
+            DeviceTensor normedFlat = rmsnorm(newInput).reshaped({rows, dim});
+            for (int i = 0; i < 3; ++i)
+                check(bf_hip_linear_bf16_img(normedFlat.data(), nullptr, weights[i], nullptr, nullptr, outs[i], rows, dim, dim, mode == 2, nullptr));
         }
     }
 }

@@ -513,3 +513,7 @@ def test_fp32_gemm_group_matches_single_products(hip, rng):
     run([(0, 1, 70, 33, 45, True, False), (1, 1, 5, 7, 300, False, True), (1, 0, 130, 64, 513, True, True), (0, 0, 1, 1, 1, False, False)])
     run([(0, 0, 64, 64, 64, False, False), (0, 0, 2048, 4224, 300, True, False)])                       # one member needs the large tiles
     run([(0, 1, 96, 96, 4100, False, False), (1, 0, 96, 96, 96, False, False)])                         # one member needs K slices
+    run([(0, 0, 1, 768, 768, False, False)] * 3)                                                        # Q, K and V of one decoded token: one walk
+    run([(0, 0, 5, 300, 3000, True, True), (0, 0, 5, 300, 3000, False, False)])                         # few rows, adds after the slice sums
+    run([(0, 0, 3, 41, 20, True, False)] * 2 + [(0, 0, 3, 41, 20, False, True)])                        # few rows, one slice, odd width
+    run([(0, 0, 2, 64, 64, False, False), (0, 0, 2, 64, 72, False, False)])                             # few rows of different shapes: one by one

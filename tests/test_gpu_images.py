@@ -169,6 +169,23 @@ def test_blocks_of_a_decoding_step_normalise_inside_the_product(hip, oracle, rng
     again = D((m, d))
     call("bf_hip_rmsnorm_feedforward_bf16", dx.ptr, dw1.ptr, db1.ptr, dw2.ptr, db2.ptr, act, again.ptr, m, d, hidden, 0, None)
     assert_bits_equal(again.toHost(), out.toHost(), "the same block twice")
+    # the fp32 forms of the two blocks (bf_hip_rmsnorm_matmul_f32_shared_input, bf_hip_rmsnorm_feedforward_f32)
+    for count, n in ((3, hidden), (1, 41)):
+        ws = [r(rng, d, n, scale=0.1) for _ in range(count)]
+        dws = [D.fromHost(w) for w in ws]
+        outs = [D((m, n)) for _ in range(count)]
+        barr = (ctypes.c_void_p * count)(*[w.ptr for w in dws])
+        carr = (ctypes.c_void_p * count)(*[o.ptr for o in outs])
+        call("bf_hip_rmsnorm_matmul_f32_shared_input", dx.ptr, barr, carr, count, m, d, n, None)
+        for i in range(count):
+            assert_close(outs[i].toHost(), ops.matmul(normed, dws[i]).toHost(), tol=2e-5, what=f"fp32 projection {i} of {count} of the normalised rows")
+    out32 = D((m, d))
+    call("bf_hip_rmsnorm_feedforward_f32", dx.ptr, dw1.ptr, db1.ptr, dw2.ptr, db2.ptr, act, out32.ptr, m, d, hidden, None)
+    hidden32 = ops.addBiasAct(ops.matmul(normed, dw1), db1, act)
+    expected32 = ops.addBiasResidual(ops.matmul(hidden32, dw2), db2, dx)
+    assert_close(out32.toHost(), expected32.toHost(), tol=2e-5, what="fp32 feed-forward block of a decoding step")
+    if act != 2:   # the CPU backend's block knows silu and gelu
+        assert_close(out32.toHost(), oracle.feedForward(x, w1, b1, w2, b2, act), what="fp32 feed-forward block vs the CPU backend's")
 
 
 @pytest.mark.parametrize("rows,classes", [(5, 16), (7, 1000), (300, 256), (3, 32000), (2, 40000)])
