@@ -136,8 +136,9 @@ inline TrainRunResult trainOnDevice(const DeviceSpec& spec, const ast::Program& 
 
 // The GPU branch of runGenerate (main.cpp:594-617), from token ids to token ids: the model of the module's precision
 // policy loads the checkpoint, the prompt goes through forwardIncremental once and every further token alone, each
-// chosen as the first maximum of the last position's logits (main.cpp:504-518).  The choice is made on the device, so
-// one index per token crosses to the host instead of the logits.  Like the CLI, generation stops quietly when the model
+// chosen as the first maximum of the last position's logits (main.cpp:504-518).  The choice is made on the device; for a
+// pipeline from token ids to logits over the same vocabulary the token never leaves it (Model::generateGreedy: the ids
+// are read back once, at the end), otherwise one index per token crosses to the host instead of the logits.  Like the CLI, generation stops quietly when the model
 // refuses a further position (its positional table is exhausted); `stoppedAtCapacity` reports that.
 struct GenerateOutcome {
     std::vector<std::uint32_t> tokens;   // the prompt followed by the generated ids
@@ -155,6 +156,17 @@ inline GenerateOutcome generateOnDevice(const DeviceSpec& spec, const ir::Module
     GenerateOutcome outcome;
     outcome.tokens = promptIds;
     const std::vector<float> promptFloats(promptIds.begin(), promptIds.end());
+    const std::size_t promptLen = promptIds.size(), limit = loaded.maxPositions();
+    if (maxNewTokens > 0 && promptLen <= limit && loaded.supportsGenerateGreedy()) {
+        // the same loop with token and position kept on the device (Model::generateGreedy): the step that would feed a token
+        // at position `limit` is the one the loop below stops at
+        const std::size_t untilFull = limit - promptLen + 1;
+        const std::size_t count = std::min(maxNewTokens, untilFull);
+        outcome.stoppedAtCapacity = maxNewTokens >= untilFull;
+        for (std::size_t id : loaded.generateGreedy(DeviceTensor::fromHost(runtime::Tensor({1, promptLen}, promptFloats)), count))
+            outcome.tokens.push_back(static_cast<std::uint32_t>(id));
+        return outcome;
+    }
     DeviceTensor logits = loaded.forwardIncremental(DeviceTensor::fromHost(runtime::Tensor({1, promptIds.size()}, promptFloats)));
     for (std::size_t step = 0; step < maxNewTokens; ++step) {
         const auto best = static_cast<std::uint32_t>(argmaxLastPosition(logits));

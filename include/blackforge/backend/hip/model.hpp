@@ -5,6 +5,7 @@
 // A model is a list of layers; each layer kind corresponds to one ir::OpKind of the reference.  Inside a
 // BlackForge build the constructor taking ir::ModelIR is available as well and initialises the weights
 // from the project's own deterministic generator, exactly like the reference backends do.
+#include <algorithm>
 #include <cstddef>
 #include <optional>
 #include <string>
@@ -242,6 +243,25 @@ public:
         std::vector<std::size_t> result(count);
         for (std::size_t i = 0; i < count; ++i) result[i] = static_cast<std::size_t>(ids[i]);
         return result;
+    }
+
+    // Whether generateGreedy can run this pipeline (token ids in, logits over the same vocabulary out, no layer that
+    // refuses incremental generation), and how many positions its positional tables allow (SIZE_MAX: no table).
+    [[nodiscard]] bool supportsGenerateGreedy() const {
+        if (layers_.empty() || layers_.front().spec.kind != LayerKind::Embedding) return false;
+        std::size_t features = 0;
+        for (const LayerState& layer : layers_) {
+            if (layer.spec.kind == LayerKind::BidirectionalAttention) return false;
+            if (layer.spec.kind == LayerKind::Embedding) features = layer.spec.arg1;
+            if (layer.spec.kind == LayerKind::Linear) features = layer.spec.arg0;
+        }
+        return features == layers_.front().spec.arg0;
+    }
+    [[nodiscard]] std::size_t maxPositions() const {
+        std::size_t limit = static_cast<std::size_t>(-1);
+        for (const LayerState& layer : layers_)
+            if (layer.spec.kind == LayerKind::PositionalEmbedding) limit = std::min(limit, layer.params[0].value.dim(0));
+        return limit;
     }
 
     void resetGenerationState() {
