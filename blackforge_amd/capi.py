@@ -127,9 +127,11 @@ SIGNATURES = {
     "bf_hip_positional_forward_indirect": [P, P, P, c_size, c_size, c_size, c_size, P, S],
     "bf_hip_kv_append_indirect": [P, P, P, P, c_size, c_size, c_size, c_size, P, S],
     "bf_hip_attention_forward_rows_indirect": [P, P, P, P, P, c_size, P, P, c_size, c_size, c_size, c_size, c_size, c_float, P, S],
-    "bf_hip_argmax_last_position_device": [P, c_size, c_size, P, P, c_size, P, ctypes.c_longlong, S],
+    "bf_hip_argmax_last_position_device": [P, c_size, c_size, P, P, c_size, P, ctypes.c_int, ctypes.c_longlong, S],
     "bf_hip_counter_add": [P, ctypes.c_int, S],
     "bf_hip_rmsnorm_matmul_bf16_shared_input": [P, ctypes.POINTER(P), ctypes.POINTER(P), c_size, c_size, c_size, c_size, ctypes.c_int, S],
+    "bf_hip_decode_projections_bf16": [P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, P, ctypes.c_int, S],
+    "bf_hip_decode_projections_f32": [P, P, P, P, P, P, P, c_size, c_size, c_size, c_size, P, S],
     "bf_hip_rmsnorm_matmul_f32_shared_input": [P, ctypes.POINTER(P), ctypes.POINTER(P), c_size, c_size, c_size, c_size, S],
     "bf_hip_rmsnorm_feedforward_f32": [P, P, P, P, P, ctypes.c_int, P, c_size, c_size, c_size, S],
     "bf_hip_rmsnorm_feedforward_bf16": [P, P, P, P, P, ctypes.c_int, P, c_size, c_size, c_size, ctypes.c_int, S],

@@ -419,15 +419,21 @@ __global__ void __launch_bounds__(1024) argmaxRowKernel(const float* __restrict_
     if (threadIdx.x == 0) result[0] = (long long)best;
 }
 // The same index left on the device: as a float token id in token[0] (the next step's input) and, when `history` is
-// given, in history[*position + historyOffset] if that lies within historyLen.
+// given, in history[*position + historyOffset] if that lies within historyLen; *position is advanced by `advance` first
+// (the step that produced the logits has consumed that many positions).
 __global__ void __launch_bounds__(1024) argmaxToTokenKernel(const float* __restrict__ row, size_t n, float* __restrict__ token,
-                                                            float* __restrict__ history, size_t historyLen, const int* __restrict__ position,
-                                                            long long historyOffset) {
+                                                            float* __restrict__ history, size_t historyLen, int* __restrict__ position,
+                                                            int advance, long long historyOffset) {
     const unsigned long long best = argmaxOfRow(row, n);
     if (threadIdx.x == 0) {
         token[0] = float(best);
+        long long at = 0;
+        if (position) {
+            at = (long long)(*position) + advance;
+            if (advance != 0) *position = int(at);
+        }
         if (history) {
-            const long long slot = (position ? (long long)(*position) : 0) + historyOffset;
+            const long long slot = at + historyOffset;
             if (slot >= 0 && size_t(slot) < historyLen) history[slot] = float(best);
         }
     }
@@ -618,11 +624,11 @@ int bf_hip_argmax_last_position(const float* logits, size_t seq, size_t vocab, l
 }
 
 int bf_hip_argmax_last_position_device(const float* logits, size_t seq, size_t vocab, float* token, float* history, size_t historyLen,
-                                       const int* position, long long historyOffset, bf_stream_t stream) {
+                                       int* position, int advance, long long historyOffset, bf_stream_t stream) {
     BF_REQUIRE(seq > 0 && vocab > 0, "empty logits");
     BF_REQUIRE(vocab <= (size_t(1) << 24), "a token id beyond 2^24 has no exact float");
     BF_REQUIRE(logits && token, "NULL pointer");
-    argmaxToTokenKernel<<<1, 1024, 0, asStream(stream)>>>(logits + (seq - 1) * vocab, vocab, token, history, historyLen, position, historyOffset);
+    argmaxToTokenKernel<<<1, 1024, 0, asStream(stream)>>>(logits + (seq - 1) * vocab, vocab, token, history, historyLen, position, advance, historyOffset);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

@@ -232,6 +232,10 @@ struct Epilogue {
     // products of at most eight rows only (gemmBf16FewRowsKernel), A == NULL: the rows of A are those of rmsnorm(normInput)
     // ([M, K] fp32, dense) rounded to bf16, made while the kernel stages them
     const float* normInput;
+    // the same kernel only: outputs c[1] and c[2] are written *rowShift rows further down, as long as the row stays below
+    // rowLimit (a decoding step's new keys and values, placed at the cache's device-side length)
+    const int* rowShift;
+    int rowLimit;
 };
 
 // An accumulator tile of the 32x32 MFMA gives lane (li, half) column li of rows 8g + 4 half + 0..3 (g = 0..3).  Stored
@@ -1275,7 +1279,9 @@ __global__ void __launch_bounds__(256) gemmBf16FewRowsKernel(const unsigned shor
                 float* C = which == 0 ? e.c[0] : which == 1 ? e.c[1] : e.c[2];
                 if (e.bias) v += biasHere;
                 if (e.residual) v += residualHere;
-                C[size_t(r) * e.splitN + (col - which * e.splitN)] = v;
+                size_t row = size_t(r);
+                if (e.rowShift != nullptr && which >= 1) row += size_t(*e.rowShift);
+                if (e.rowShift == nullptr || which == 0 || row < size_t(e.rowLimit)) C[row * e.splitN + (col - which * e.splitN)] = v;
                 if (e.fuse == 1) e.image[size_t(r) * N + col] = toBf16Bits(actF1(e.act, v));
             }
         }
@@ -2456,6 +2462,41 @@ int bf_hip_rmsnorm_matmul_bf16_shared_input(const float* x, const float* const* 
     int st = bf_hip_rmsnorm_img(x, nullptr, image.as<uint16_t>(), m, k, stream);
     if (st != BF_OK) return st;
     return bf_hip_matmul_bf16_shared_input_img(nullptr, image.as<uint16_t>(), b, c, count, m, k, n, cacheWeight, stream);
+}
+
+// The projections of a decoding step whose position lives on the device: q = bf16(rmsnorm(x)) wq, and the rows of
+// bf16(rmsnorm(x)) wk and ... wv appended to caches of `capacity` rows a sequence at row *position.  One sequence of one or
+// two new rows, width a multiple of 256: one launch (the few-row kernel normalises, multiplies and stores the keys and
+// values where they belong); anything else: the products into scratch rows, then bf_hip_kv_append_indirect.
+int bf_hip_decode_projections_bf16(const float* x, const float* wq, const float* wk, const float* wv, float* q, float* kCache, float* vCache,
+                                   size_t batch, size_t newLen, size_t dim, size_t capacity, const int* position, int cacheWeight,
+                                   bf_stream_t stream) {
+    if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(x && wq && wk && wv && q && kCache && vCache && position, "NULL pointer");
+    BF_REQUIRE(newLen <= capacity && capacity < (size_t(1) << 31), "more new rows than the cache holds");
+    hipStream_t s = asStream(stream);
+    const size_t rows = batch * newLen;
+    const float* weights[3] = {wq, wk, wv};
+    if (batch == 1 && dim % 256 == 0 && fewRowsNormalise(rows, dim)) {
+        unsigned short* wImg = nullptr;
+        size_t wBytes = 0;
+        int st = weightImage(weights, 3, dim, dim, 2, cacheWeight != 0, s, &wImg, &wBytes);
+        if (st != BF_OK) return st;
+        Epilogue epi{{q, kCache, vCache}, int(dim), nullptr, nullptr};
+        epi.normInput = x;
+        epi.rowShift = position;
+        epi.rowLimit = int(capacity);
+        st = fewRowsServe(nullptr, wImg, 0, rows, dim, dim, dim) ? launchGemmNt(nullptr, wImg, epi, rows, 3 * dim, dim, dim, dim, s)
+                                                                 : failInvalid(__func__, "unaligned weight image");
+        if (!cacheWeight) bf_hip_pool_release(wImg, wBytes);
+        return st;
+    }
+    Scratch fresh(2 * rows * dim * sizeof(float));
+    if (fresh.status != BF_OK) return fresh.status;
+    float* outs[3] = {q, fresh.as<float>(), fresh.as<float>() + rows * dim};
+    int st = bf_hip_rmsnorm_matmul_bf16_shared_input(x, weights, outs, 3, rows, dim, dim, cacheWeight, stream);
+    if (st != BF_OK) return st;
+    return bf_hip_kv_append_indirect(kCache, vCache, outs[1], outs[2], batch, newLen, dim, capacity, position, stream);
 }
 
 // out = input + act(bf16(rmsnorm(input)) w1 + b1) w2 + b2: the feed-forward block (ops_transformer.cu:182-215) for a

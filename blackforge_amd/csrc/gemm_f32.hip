@@ -386,6 +386,10 @@ struct FewRowsProducts {
     // the kernel stages its slice of them (a decoding step's projections and feed-forward block)
     const float* normInput;
     int act;                // BF_ACT_* applied after the adds, or -1
+    // products 1 and 2 are stored *rowShift rows further down, as long as the row stays below rowLimit (a decoding step's
+    // new keys and values, placed at the cache's device-side length)
+    const int* rowShift;
+    int rowLimit;
 };
 __device__ __forceinline__ float actOrNot(int act, float v) {
     return act < 0 ? v : act == BF_ACT_SILU ? siluF(v) : act == BF_ACT_GELU ? geluF(v) : reluF(v);
@@ -409,7 +413,13 @@ __global__ void __launch_bounds__(kBlock) sliceSumProductsKernel(FewRowsProducts
         for (int u = 0; u < 8; ++u)
             if (s0 + u < slices) sum += v[u];
     }
-    C[i] = actOrNot(g.act, withAdds(sum, bias, residual, i, i % N));
+    const float value = actOrNot(g.act, withAdds(sum, bias, residual, i, i % N));
+    if (g.rowShift != nullptr && which >= 1) {
+        const size_t row = i / N + size_t(*g.rowShift);
+        if (row < size_t(g.rowLimit)) C[row * N + i % N] = value;
+    } else {
+        C[i] = value;
+    }
 }
 
 // Products of at most eight rows, C[M, N] = A[M, K] B[K, N] (a step of incremental decoding: one new token per sequence),
@@ -518,7 +528,14 @@ __global__ void __launch_bounds__(64 * WAVES) gemmF32FewRowsKernel(FewRowsProduc
 #pragma unroll
             for (int w = 1; w < WAVES; ++w) total += sums[(w * MR + r) * WIDTH + c];
             const size_t at = size_t(r) * N + column;
-            dst[at] = gridDim.y > 1 ? total : actOrNot(g.act, withAdds(total, bias, residual, at, size_t(column)));
+            if (gridDim.y > 1) {
+                dst[at] = total;
+            } else {
+                const float value = actOrNot(g.act, withAdds(total, bias, residual, at, size_t(column)));
+                size_t row = size_t(r);
+                if (g.rowShift != nullptr && which >= 1) row += size_t(*g.rowShift);
+                if (g.rowShift == nullptr || which == 0 || row < size_t(g.rowLimit)) dst[row * N + column] = value;
+            }
         }
     }
 }
@@ -700,6 +717,38 @@ extern "C" int bf_hip_rmsnorm_matmul_f32_shared_input(const float* x, const floa
     bf_gemm_f32_problem problems[3];
     for (size_t i = 0; i < count; ++i) problems[i] = bf_gemm_f32_problem{normed.as<float>(), b[i], c[i], nullptr, nullptr, m, n, k, 0, 0};
     return bf_hip_gemm_f32_group(problems, count, stream);
+}
+
+// The projections of a decoding step whose position lives on the device, in fp32: q = rmsnorm(x) wq, and the rows of
+// rmsnorm(x) wk and ... wv appended to caches of `capacity` rows a sequence at row *position.  One sequence of one or two new
+// rows: the three products in one walk that stores the keys and values where they belong; anything else: the products
+// into scratch rows, then bf_hip_kv_append_indirect.
+extern "C" int bf_hip_decode_projections_f32(const float* x, const float* wq, const float* wk, const float* wv, float* q, float* kCache,
+                                             float* vCache, size_t batch, size_t newLen, size_t dim, size_t capacity, const int* position,
+                                             bf_stream_t stream) {
+    if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(x && wq && wk && wv && q && kCache && vCache && position, "NULL pointer");
+    BF_REQUIRE(newLen <= capacity && capacity < (size_t(1) << 31), "more new rows than the cache holds");
+    const size_t rows = batch * newLen;
+    if (batch == 1 && rows <= 2 && dim < (size_t(1) << 31)) {
+        FewRowsProducts g = {};
+        g.act = -1;
+        g.normInput = x;
+        g.rowShift = position;
+        g.rowLimit = int(capacity);
+        g.B[0] = wq; g.B[1] = wk; g.B[2] = wv;
+        g.out[0] = q; g.out[1] = kCache; g.out[2] = vCache;
+        bool served = false;
+        int st = launchFewRowsF32Any(g, 3, rows, dim, dim, asStream(stream), &served);
+        if (st != BF_OK || served) return st;
+    }
+    Scratch fresh(2 * rows * dim * sizeof(float));
+    if (fresh.status != BF_OK) return fresh.status;
+    const float* weights[3] = {wq, wk, wv};
+    float* outs[3] = {q, fresh.as<float>(), fresh.as<float>() + rows * dim};
+    int st = bf_hip_rmsnorm_matmul_f32_shared_input(x, weights, outs, 3, rows, dim, dim, stream);
+    if (st != BF_OK) return st;
+    return bf_hip_kv_append_indirect(kCache, vCache, outs[1], outs[2], batch, newLen, dim, capacity, position, stream);
 }
 
 // out = input + act(rmsnorm(input) w1 + b1) w2 + b2 in fp32: the feed-forward block (ops_transformer.cu:182-215) for a caller

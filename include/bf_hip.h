@@ -431,10 +431,20 @@ int bf_hip_rmsnorm_feedforward_bf16(const float* input, const float* w1, const f
  * keys and values to rows *position.. of caches with `capacity` rows a sequence, attention_forward_rows_indirect attends
  * to the first *oldLen + newLen rows of k and v (the walk over the cache of bf_hip_attention_forward_rows, at most eight
  * queries per sequence; its chunks cover all kvRows and those past the current length do nothing),
- * argmax_last_position_device leaves the index on the device as a float token id (and in history[*position +
- * historyOffset] when that lies within historyLen), counter_add advances the counter.  The caller promises that the
+ * argmax_last_position_device first advances *position by `advance` (the positions the step that made the logits has
+ * consumed), then leaves the index on the device as a float token id (and in history[*position + historyOffset] when that
+ * lies within historyLen), counter_add advances a counter on its own.  The caller promises that the
  * positions fit (table rows, cache capacity): a kernel that finds otherwise writes nothing.  (They may also be recorded
  * in a graph, whose arguments are frozen; replaying a whole decoding step that way measured slower than launching it.) */
+/* decode_projections_{bf16,f32}: the attention block's three projections in that form: q = rmsnorm(x) wq (bf16: of the rows
+ * rounded to bf16), the rows of rmsnorm(x) wk and rmsnorm(x) wv appended to the caches at row *position.  One sequence of
+ * one or two new rows (bf16: width a multiple of 256) is one launch that stores the keys and values where they belong;
+ * anything else computes them into scratch rows and appends. */
+int bf_hip_decode_projections_bf16(const float* x, const float* wq, const float* wk, const float* wv, float* q, float* kCache, float* vCache,
+                                   size_t batch, size_t newLen, size_t dim, size_t capacity, const int* position, int cacheWeight,
+                                   bf_stream_t stream);
+int bf_hip_decode_projections_f32(const float* x, const float* wq, const float* wk, const float* wv, float* q, float* kCache, float* vCache,
+                                  size_t batch, size_t newLen, size_t dim, size_t capacity, const int* position, bf_stream_t stream);
 int bf_hip_positional_forward_indirect(const float* x, const float* table, float* out, size_t batch, size_t seq, size_t dim, size_t maxSeq,
                                        const int* offset, bf_stream_t stream);
 int bf_hip_kv_append_indirect(float* kCache, float* vCache, const float* kNew, const float* vNew, size_t batch, size_t newLen, size_t dim,
@@ -443,7 +453,7 @@ int bf_hip_attention_forward_rows_indirect(const float* q, const float* k, const
                                            float* m, float* l, size_t batch, size_t heads, size_t newLen, size_t kvRows, size_t dim, float scale,
                                            const int* oldLen, bf_stream_t stream);
 int bf_hip_argmax_last_position_device(const float* logits, size_t seq, size_t vocab, float* token, float* history, size_t historyLen,
-                                       const int* position, long long historyOffset, bf_stream_t stream);
+                                       int* position, int advance, long long historyOffset, bf_stream_t stream);
 int bf_hip_counter_add(int* counter, int by, bf_stream_t stream);
 /* computeDKernel: fused_attention.cu:166-190   D[b,h,i] = dot(out[b,i,h,:], dOut[b,i,h,:]) */
 int bf_hip_attention_dot_o_do(const float* out, const float* dOut, float* D, size_t batch, size_t heads,

@@ -226,14 +226,15 @@ public:
         DeviceTensor token({1, 1}), history({count}), position({1});   // position: one int, the number of positions processed
         const int start = static_cast<int>(promptLen);
         check(bf_hip_memcpy_h2d(position.data(), &start, sizeof(int)));
-        const int* devicePosition = reinterpret_cast<const int*>(position.data());
+        int* devicePosition = reinterpret_cast<int*>(position.data());
         const long long firstSlot = -static_cast<long long>(promptLen);    // a token goes to history[*position - promptLen]
-        check(bf_hip_argmax_last_position_device(logits.data(), promptLen, vocab, token.data(), history.data(), count, devicePosition, firstSlot,
-                                                 nullptr));
+        check(bf_hip_argmax_last_position_device(logits.data(), promptLen, vocab, token.data(), history.data(), count, devicePosition, 0,
+                                                 firstSlot, nullptr));
         for (std::size_t i = 1; i < count; ++i) {
             DeviceTensor next = incrementalStep(token, devicePosition);
-            check(bf_hip_counter_add(reinterpret_cast<int*>(position.data()), 1, nullptr));
-            check(bf_hip_argmax_last_position_device(next.data(), 1, vocab, token.data(), history.data(), count, devicePosition, firstSlot, nullptr));
+            // the step has consumed one position: the counter moves on in the same launch that picks the next token
+            check(bf_hip_argmax_last_position_device(next.data(), 1, vocab, token.data(), history.data(), count, devicePosition, 1, firstSlot,
+                                                     nullptr));
         }
         generationPosition_ += count - 1;
         for (LayerState& layer : layers_)

@@ -519,11 +519,20 @@ inline DeviceTensor selfAttentionIncrementalOnDevicePosition(const char* op, con
     const std::size_t batch = newInput.dim(0), newLen = newInput.dim(1), dim = newInput.dim(2);
     require(cache.capacity != 0 && cache.k.rank() == 3 && cache.k.dim(0) == batch && cache.k.dim(2) == dim,
             std::string(op) + ": a step on a device-side position needs a cache that already holds the prompt, for this batch size and width");
-    DeviceTensor qNew({batch, newLen, dim}), kNew({batch, newLen, dim}), vNew({batch, newLen, dim});
-    float* const outs[3] = {qNew.data(), kNew.data(), vNew.data()};
-    incrementalProjections(newInput, wq, wk, wv, outs, mode);
-    check(bf_hip_kv_append_indirect(cache.k.data(), cache.v.data(), kNew.data(), vNew.data(), batch, newLen, dim, cache.capacity, devicePosition,
-                                    nullptr));
+    DeviceTensor qNew({batch, newLen, dim});
+    if (mode == 0) {
+        check(bf_hip_decode_projections_f32(newInput.data(), wq.data(), wk.data(), wv.data(), qNew.data(), cache.k.data(), cache.v.data(), batch,
+                                            newLen, dim, cache.capacity, devicePosition, nullptr));
+    } else if (dim % 8 == 0) {
+        check(bf_hip_decode_projections_bf16(newInput.data(), wq.data(), wk.data(), wv.data(), qNew.data(), cache.k.data(), cache.v.data(), batch,
+                                             newLen, dim, cache.capacity, devicePosition, mode == 2, nullptr));
+    } else {
+        DeviceTensor kNew({batch, newLen, dim}), vNew({batch, newLen, dim});
+        float* const outs[3] = {qNew.data(), kNew.data(), vNew.data()};
+        incrementalProjections(newInput, wq, wk, wv, outs, mode);
+        check(bf_hip_kv_append_indirect(cache.k.data(), cache.v.data(), kNew.data(), vNew.data(), batch, newLen, dim, cache.capacity,
+                                        devicePosition, nullptr));
+    }
     const float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
     const bool imageOnly = mode != 0 && dim % 8 == 0;
     DeviceTensor attnOut = imageOnly ? DeviceTensor::imageOnly({batch, newLen, dim}) : DeviceTensor({batch, newLen, dim});

@@ -156,12 +156,16 @@ def test_position_on_the_device_entry_points(hip, oracle, rng):
         logits = r(rng, 1, 3, vocab)
         logits[0, 2, vocab // 2] = logits[0, 2].max()   # a tie: the lower index must win
         token, history, dlogits = D.fromHost(np.zeros((1, 1), f32)), D.fromHost(np.full(4, -1.0, f32)), D.fromHost(logits)
-        call("bf_hip_argmax_last_position_device", dlogits.ptr, 3, vocab, token.ptr, history.ptr, 4, counter.ptr, ctypes.c_longlong(-5), None)
+        call("bf_hip_argmax_last_position_device", dlogits.ptr, 3, vocab, token.ptr, history.ptr, 4, counter.ptr, 0, ctypes.c_longlong(-5), None)
         expected = oracle.argmaxLastPosition(logits[0])
         assert token.toHost()[0, 0] == expected
         np.testing.assert_array_equal(history.toHost(), [-1, -1, expected, -1])   # slot 7 - 5
-        call("bf_hip_argmax_last_position_device", dlogits.ptr, 3, vocab, token.ptr, history.ptr, 4, counter.ptr, ctypes.c_longlong(0), None)
+        call("bf_hip_argmax_last_position_device", dlogits.ptr, 3, vocab, token.ptr, history.ptr, 4, counter.ptr, 0, ctypes.c_longlong(0), None)
         np.testing.assert_array_equal(history.toHost(), [-1, -1, expected, -1])   # slot 7 lies outside: left alone
+        call("bf_hip_argmax_last_position_device", dlogits.ptr, 3, vocab, token.ptr, history.ptr, 4, counter.ptr, 1, ctypes.c_longlong(-5), None)
+        np.testing.assert_array_equal(history.toHost(), [-1, -1, expected, expected])   # the counter moves on first: slot 8 - 5
+        assert as_int() == 8
+        call("bf_hip_counter_add", counter.ptr, -1, None)
 
 
 @pytest.mark.parametrize("rows,classes", [(1, 2), (2, 3), (7, 13), (512, 256), (5, 1000), (3, 32000), (2, 50257), (1, 70001), (3, 40000),

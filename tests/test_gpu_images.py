@@ -188,6 +188,43 @@ def test_blocks_of_a_decoding_step_normalise_inside_the_product(hip, oracle, rng
         assert_close(out32.toHost(), oracle.feedForward(x, w1, b1, w2, b2, act), what="fp32 feed-forward block vs the CPU backend's")
 
 
+@pytest.mark.parametrize("batch,new_len,dim", [(1, 1, 768), (1, 2, 256), (1, 1, 72), (2, 1, 256), (1, 3, 512), (3, 2, 40)])
+def test_projections_of_a_decoding_step_at_a_position_on_the_device(hip, oracle, rng, batch, new_len, dim):
+    """bf_hip_decode_projections_{bf16,f32}: q, k and v of selfAttentionIncremental (ops_transformer.cu:133-160: rmsnorm,
+    three projections, the new keys and values joined to the cache) with the cache's length read from device memory.  One
+    sequence of one or two rows takes the single launch that stores keys and values in place, the other cases the scratch
+    rows and the append; both against the separate operators, the rest of the caches untouched, rows that would not fit
+    not written."""
+    D, ops, call = hip.DeviceTensor, hip.ops, hip.capi.call
+    capacity, at = 9, 4
+    x = r(rng, batch * new_len, dim, scale=2.0)
+    ws = [r(rng, dim, dim, scale=0.1) for _ in range(3)]
+    dx, dws = D.fromHost(x), [D.fromHost(w) for w in ws]
+    normed = ops.rmsnorm(dx)
+    position = D.fromHost(np.array([at], np.int32).view(f32))
+    for mode in ("bf16", "f32"):
+        kc, vc = r(rng, batch, capacity, dim), r(rng, batch, capacity, dim)
+        dk, dv, q = D.fromHost(kc), D.fromHost(vc), D((batch * new_len, dim))
+        args = [dx.ptr, dws[0].ptr, dws[1].ptr, dws[2].ptr, q.ptr, dk.ptr, dv.ptr, batch, new_len, dim, capacity, position.ptr]
+        call("bf_hip_decode_projections_" + mode, *(args + ([0] if mode == "bf16" else []) + [None]))
+        product = ops.matmulBf16 if mode == "bf16" else ops.matmul
+        eq, ek, ev = (product(normed, w).toHost() for w in dws)
+        assert_close(q.toHost(), eq, tol=2e-5, what=f"{mode} q")
+        gk, gv = dk.toHost(), dv.toHost()
+        assert_close(gk[:, at:at + new_len].reshape(-1, dim), ek, tol=2e-5, what=f"{mode} keys at the device-side position")
+        assert_close(gv[:, at:at + new_len].reshape(-1, dim), ev, tol=2e-5, what=f"{mode} values at the device-side position")
+        keep = np.ones(capacity, bool)
+        keep[at:at + new_len] = False
+        assert_bits_equal(gk[:, keep], kc[:, keep], f"{mode}: the other rows of the key cache")
+        assert_bits_equal(gv[:, keep], vc[:, keep], f"{mode}: the other rows of the value cache")
+        full = D.fromHost(np.array([capacity - new_len + 1], np.int32).view(f32))   # the last new row would not fit
+        before = dk.toHost()
+        args[-1] = full.ptr
+        call("bf_hip_decode_projections_" + mode, *(args + ([0] if mode == "bf16" else []) + [None]))
+        after = dk.toHost()
+        assert_bits_equal(after[:, :capacity - new_len + 1], before[:, :capacity - new_len + 1], f"{mode}: rows below a position that does not fit")
+
+
 @pytest.mark.parametrize("rows,classes", [(5, 16), (7, 1000), (300, 256), (3, 32000), (2, 40000)])
 def test_cross_entropy_gradient_image(hip, oracle, rng, rows, classes):
     D, call = hip.DeviceTensor, hip.capi.call
