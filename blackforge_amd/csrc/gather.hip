@@ -391,9 +391,21 @@ __device__ __forceinline__ unsigned long long argmaxOfRow(const float* __restric
     __shared__ unsigned long long idxs[16];
     float best = -INFINITY;
     unsigned long long bestIdx = ~0ull;  // "no candidate": loses against everything
-    for (size_t i = threadIdx.x; i < n; i += blockDim.x) {
-        float k = argmaxKey(row[i], i);
-        if (bestIdx == ~0ull || k > best) { best = k; bestIdx = i; }
+    for (size_t i0 = threadIdx.x; i0 < n; i0 += size_t(8) * blockDim.x) {   // eight loads in flight, compared in index order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const size_t i = i0 + size_t(u) * blockDim.x;
+            v[u] = i < n ? row[i] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const size_t i = i0 + size_t(u) * blockDim.x;
+            if (i < n) {
+                const float k = argmaxKey(v[u], i);
+                if (bestIdx == ~0ull || k > best) { best = k; bestIdx = i; }
+            }
+        }
     }
     // (value, index) pairs: larger value wins, equal values go to the lower index
     auto takeOther = [](float v, unsigned long long i, float ov, unsigned long long oi) {
