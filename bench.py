@@ -702,6 +702,37 @@ def bench_decode(bf, tokens=32, prompt=1024):
     return out
 
 
+def cpu_baseline_decode(prompt=1024):
+    """The reference CPU backend on one decoding step of the same model (fp32, one host core): ONE block's incremental
+    attention over a cache of `prompt` positions and its feed-forward block, timed and multiplied by the twelve blocks,
+    plus the head once (the embedding row and the positional add are negligible beside them)."""
+    from oracle import bfo
+    impl = bfo.reference() or bfo.oracle()
+    c = TRAIN_CONFIGS["gpt_small"]
+    rng = np.random.default_rng(12)
+    dim, ffn, vocab = c["dim"], c["ffn"], c["vocab"]
+    fill = lambda *shape: np.resize(rng.standard_normal(4099, dtype=np.float32) * np.float32(0.02), shape)
+    x = rng.standard_normal((1, 1, dim), dtype=np.float32)
+    wq, wk, wv, wo = (fill(dim, dim) for _ in range(4))
+    kc, vc = rng.standard_normal((1, prompt, dim), dtype=np.float32), rng.standard_normal((1, prompt, dim), dtype=np.float32)
+    w1, b1, w2, b2 = fill(dim, ffn), fill(ffn), fill(ffn, dim), fill(dim)
+    head_w, head_b = fill(dim, vocab), fill(vocab)
+    best_block, best_head = 1e30, 1e30
+    for _ in range(3):
+        t0 = time.perf_counter()
+        y, _, _ = impl.selfAttentionIncremental(x, wq, wk, wv, wo, c["heads"], kc, vc)
+        impl.feedForward(y, w1, b1, w2, b2, 0)
+        t1 = time.perf_counter()
+        impl.linear(y.reshape(1, dim), head_w, head_b)
+        t2 = time.perf_counter()
+        best_block, best_head = min(best_block, t1 - t0), min(best_head, t2 - t1)
+    token_s = c["blocks"] * best_block + best_head
+    return {"value": round(1.0 / token_s, 2), "unit": "tokens/s", "cores": 1, "kind": "reference" if impl.is_reference else "port",
+            "extrapolated": True,
+            "sample": f"one block (selfAttentionIncremental over {prompt} cached positions + feedForward, SiLU) {best_block * 1e3:.1f} ms x {c['blocks']} blocks + "
+                      f"the head {best_head * 1e3:.1f} ms = {token_s * 1e3:.0f} ms a token on one host core, best of 3"}
+
+
 def extras_summary(extras):
     """The north-star targets in three numbers: the bf16 projection at 4096^3 against the bf16 MFMA peak, and the worst and
     the median bandwidth kernel against the HBM peak."""
@@ -824,6 +855,8 @@ def main():
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_attention()
         line["cpu_baseline"]["host_cores"] = os.cpu_count()
+        if "decode" in line:
+            line["decode"]["cpu_baseline"] = cpu_baseline_decode()
         for name in line.get("train_step", {}):
             line["train_step"][name]["cpu_baseline"] = cpu_baseline_mlp() if name == "mlp" else cpu_baseline_train_step(name)
     print(json.dumps(line))
