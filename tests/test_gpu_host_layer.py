@@ -307,6 +307,51 @@ def test_greedy_generation_without_reading_back(hip, rng, use_bf16, heads, dim):
         model.generateGreedy(D.fromHost(prompt), seq)   # positions past the positional table
 
 
+@pytest.mark.parametrize("use_bf16", [False, True])
+def test_decoding_at_the_gpt_small_shape(hip, rng, use_bf16):
+    """The decoding path at the widths BASELINE.json's configs[3] names (d_model 768, 12 heads of 64, ffn 3072, vocab 32000,
+    12 blocks), where the small cases above do not reach: the walks over 768- and 3072-wide weights, the 32000-wide head
+    with four columns a wavefront, the cache of a 150-token prompt.  Size-independent properties: the logits of
+    forwardIncremental at each new position equal those of Model::forward over the whole prefix (model.cu:385-424 against
+    :174-239; the reference's own check, model_tests.cu:536-611), and generateGreedy returns the argmax tokens of that
+    loop."""
+    from blackforge_amd import hostlayer as hl
+    vocab, dim, seq, heads, hidden, blocks = 32000, 768, 256, 12, 3072, 12
+    D = hip.DeviceTensor
+    model = hl.HostModel(_lm_layers(hl, vocab, dim, seq, heads, hidden, 1, blocks), use_bf16=use_bf16)
+    for i, c in enumerate(model.counts):
+        model.set_value(i, rng.standard_normal(c, dtype=f32) * f32(0.02))   # N(0, 0.02), the configuration's initialisation
+    prompt = rng.integers(0, vocab, (1, 150)).astype(f32)
+    tokens = model.generateGreedy(D.fromHost(prompt), 4)
+    model.resetGenerationState()
+    ids = prompt
+    logits = model.forwardIncremental(D.fromHost(prompt)).reshape(-1, vocab)[-1]
+    # bf16 mode: the new position's products add in another order than the full pass's tiles, and one last-bit difference
+    # that flips the bf16 rounding of an operand moves the logits by a per cent of their size (measured with the SAME
+    # kernels on both sides: scaling one input row by 1 + 3e-7 changes the logits of a model like this one by 1.5e-2 of
+    # their rms); with the tile kernels forced on both sides the two agree bit for bit
+    tol = BF16_TOL if use_bf16 else 1e-4
+    for step, t in enumerate(tokens):
+        full = model.forward(D.fromHost(ids)).reshape(-1, vocab)[-1]
+        assert_close(logits, full, tol=tol, what=f"incremental logits at position {ids.shape[1] - 1} vs the full forward",
+                     scale=float(np.abs(full).max()) if use_bf16 else 0.0)
+        best = int(np.argmax(logits))
+        assert t == best or logits[best] - logits[t] <= tol * np.abs(logits).max(), f"token {step}: {t} against the loop's argmax {best}"
+        ids = np.concatenate([ids, np.array([[t]], f32)], axis=1)
+        logits = model.forwardIncremental(D.fromHost(np.array([[t]], f32))).reshape(vocab)
+    if use_bf16:   # the same comparison with every product and the attention on the tile kernels: the same additions in the same order
+        hip.capi.call("bf_hip_gemm_bf16_set_route", 1)
+        hip.capi.call("bf_hip_attention_set_route", 7 | 8)
+        try:
+            model.resetGenerationState()
+            model.forwardIncremental(D.fromHost(ids[:, :-1]))
+            last = model.forwardIncremental(D.fromHost(ids[:, -1:])).reshape(vocab)
+            assert_bits_equal(last, model.forward(D.fromHost(ids)).reshape(-1, vocab)[-1], "incremental vs full forward on one kernel family")
+        finally:
+            hip.capi.call("bf_hip_gemm_bf16_set_route", 0)
+            hip.capi.call("bf_hip_attention_set_route", 7)
+
+
 @pytest.mark.parametrize("act", [0, 1])
 def test_config1_tiny_lm_full_step_against_oracle(hip, oracle, rng, act):
     """BASELINE config 1 shape: vocab 256, d_model 128, 4 heads, 1 attention + 1 feedforward(512) block, seq 64,
