@@ -323,6 +323,24 @@ int main() {
             // positions continue without a reset: 6 + 3 > maxSeq rows of the positional table
             (void)model.forwardIncremental(dev({1, 6}, tokens));
             EXPECT_THROW_INVALID((void)model.forwardIncremental(dev({1, 3}, {1, 2, 3})));
+
+            // generateGreedy (token and position kept on the device) = the loop of the reference's generate command
+            // (main.cpp:594-617): argmax of the last logits, fed back
+            const std::vector<float> prompt = {3, 17, 5};
+            EXPECT_TRUE(model.supportsGenerateGreedy() && model.maxPositions() == maxSeq);
+            const std::vector<std::size_t> fast = model.generateGreedy(dev({1, 3}, prompt), 5);
+            model.resetGenerationState();
+            DeviceTensor logits = model.forwardIncremental(dev({1, 3}, prompt));
+            EXPECT_TRUE(fast.size() == 5);
+            for (std::size_t step = 0; step < fast.size(); ++step) {
+                const Tensor host = logits.toHost();
+                const std::size_t rows = host.elementCount() / vocab, best = hip::argmaxLastPosition(logits);
+                const float margin = host.data()[(rows - 1) * vocab + best] - host.data()[(rows - 1) * vocab + fast[step]];
+                EXPECT_TRUE(fast[step] == best || margin <= float(tol));   // a near tie may fall the other way: other kernels, other last bits
+                if (step + 1 < fast.size()) logits = model.forwardIncremental(dev({1, 1}, {static_cast<float>(fast[step])}));
+            }
+            EXPECT_THROW_INVALID((void)model.generateGreedy(dev({1, 3}, prompt), maxSeq));   // 3 + 8 - 1 positions > 8 table rows
+            EXPECT_TRUE(model.generateGreedy(dev({1, 3}, prompt), 6).size() == 6);         // the last token is not fed: 3 + 5 positions fit
         });
     }
 
