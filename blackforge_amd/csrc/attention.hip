@@ -90,6 +90,26 @@ __device__ __forceinline__ void applyKeyChunk(AttnParams& p) {
     p.l += size_t(c) * p.partStatStride;
 }
 
+// A chunk whose keys all lie after the last query of a workgroup's tile (a causal pass from position 0 whose keys are
+// taken in chunks: the upper right of the triangle): the tile's rows get zero output, maximum -inf and sum 0 for this
+// chunk, which attnCombineChunksKernel weighs with zero.  Chunk starts are multiples of 128 like the tiles' first
+// queries, so a chunk is either empty for a whole tile or holds a visible key for each of its rows.
+__device__ __forceinline__ bool chunkIsEmptyFor(const AttnParams& p, int qt) {
+    return p.numChunks > 1 && p.oldLen + min(p.newLen, qt * 128 + 128) <= 0;   // p.oldLen: already relative to the chunk's first key
+}
+__device__ __forceinline__ void writeEmptyChunk(const AttnParams& p, int b, int h, int qt) {
+    const int rows = min(128, p.newLen - qt * 128);
+    for (int e = threadIdx.x; e < rows * p.hd; e += 256) {
+        const int r = e / p.hd, d = e - r * p.hd;
+        p.out[(size_t(b) * p.newLen + qt * 128 + r) * p.dim + size_t(h) * p.hd + d] = 0.0f;
+    }
+    for (int r = threadIdx.x; r < rows; r += 256) {
+        const size_t at = (size_t(b) * p.heads + h) * p.newLen + qt * 128 + r;
+        p.m[at] = -INFINITY;
+        p.l[at] = 0.0f;
+    }
+}
+
 __device__ __forceinline__ float fastExp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Workgroup -> (batch*head, tile), heaviest tiles first over ALL (batch, head) pairs: causal tiles differ in
@@ -382,6 +402,10 @@ __global__ void __launch_bounds__(256, HDP <= 128 ? 2 : 1) attnForwardKernel(Att
     int bh, qt;
     decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
     const int b = bh / p.heads, h = bh - b * p.heads;
+    if (chunkIsEmptyFor(p, qt)) {                 // the same for the whole workgroup, before any barrier
+        writeEmptyChunk(p, b, h, qt);
+        return;
+    }
     const int hd = p.hd, dim = p.dim;
     const float* qb = p.q + size_t(b) * p.newLen * dim + size_t(h) * hd;
     const float* kb = p.k + size_t(b) * p.kvRows * dim + size_t(h) * hd;
@@ -2272,6 +2296,10 @@ __global__ void __launch_bounds__(256, HDP <= 64 ? 2 : 1) attnForwardPipedKernel
     int bh, qt;
     decodeBlock(p.numTiles, gridDim.x, true, bh, qt);
     const int b = bh / p.heads, h = bh - b * p.heads;
+    if (chunkIsEmptyFor(p, qt)) {                 // the same for the whole workgroup, before any barrier
+        writeEmptyChunk(p, b, h, qt);
+        return;
+    }
     const int hd = p.hd, dim = p.dim;
     const float* qb = p.q + size_t(b) * p.newLen * dim + size_t(h) * hd;
     const float* kb = p.k + size_t(b) * p.kvRows * dim + size_t(h) * hd;
@@ -2430,6 +2458,47 @@ __global__ void __launch_bounds__(256) attnCombineChunksKernel(const float* __re
 // wavefronts in order through LDS.  blockIdx.x is the chunk of keys, blockIdx.y the (batch, head, query).  Head dims that
 // are multiples of 4, 16-byte aligned operands.  Chunk c of numChunks > 1 writes its normalised output and statistics as
 // the tile kernels do (attnCombineChunksKernel joins them); a single chunk writes the results themselves.
+// The same for many rows of few chunks (a prompt's pass: thousands of (batch, query, head) rows, at most eight chunks): a
+// wavefront per row, every lane with the row's chunk weights, four head columns a lane.
+__global__ void __launch_bounds__(256) attnCombineRowsKernel(const float* __restrict__ partOut, const float* __restrict__ partM,
+                                                             const float* __restrict__ partL, float* __restrict__ out,
+                                                             unsigned short* __restrict__ outImg, size_t imgLd, float* __restrict__ m,
+                                                             float* __restrict__ l, size_t groups, int heads, int newLen, int dim, int hd,
+                                                             int numChunks, size_t partOutStride, size_t partStatStride) {
+    const int lane = threadIdx.x & 63;
+    const size_t group = size_t(blockIdx.x) * 4 + (threadIdx.x >> 6);   // (b, i, h), h fastest
+    if (group >= groups) return;
+    const int h = int(group % heads);
+    const size_t bi = group / heads;
+    const size_t b = bi / newLen, i = bi - b * newLen;
+    const size_t stat = (b * heads + h) * newLen + i;
+    float ms[8], ls[8];
+    float rowMax = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        ms[c] = c < numChunks ? partM[c * partStatStride + stat] : -INFINITY;
+        ls[c] = c < numChunks ? partL[c * partStatStride + stat] : 0.0f;
+        rowMax = fmaxf(rowMax, ms[c]);
+    }
+    float total = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        ls[c] = c < numChunks ? ls[c] * expf(ms[c] - rowMax) : 0.0f;   // the chunk's weight before the division
+        total += ls[c];
+    }
+    const size_t at = bi * dim + size_t(h) * hd;
+    for (int d = lane; d < hd; d += 64) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            if (c < numChunks && ls[c] != 0.0f) acc += ls[c] * partOut[c * partOutStride + at + d];
+        const float value = acc / total;
+        if (out) out[at + d] = value;
+        if (outImg) outImg[bi * imgLd + size_t(h) * hd + d] = toBf16Bits(value);
+    }
+    if (lane == 0) { m[stat] = rowMax; l[stat] = total; }
+}
+
 // exp(x) for x <= 0 as the hardware's 2^(x log2 e): the walk below is a chain of a few dozen dependent steps on one
 // wavefront, where the library routine's forty instructions apiece are a large part of the kernel's time
 __device__ __forceinline__ float expFast(float x) { return fastExp2(x * kLog2e); }
@@ -2726,36 +2795,53 @@ int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v
         const size_t numChunks = std::max<size_t>(1, std::min((totalLen + chunkKeys - 1) / chunkKeys, oldLen / chunkKeys + 1));
         return launchFewQueries(p, batch, heads, newLen, chunkKeys, numChunks, s);
     }
-    // Few queries against many keys (a step of incremental decoding: one workgroup per head would walk all the keys alone):
-    // the keys go to the workgroups in chunks, each with its own statistics, and a second kernel puts the chunks together.
-    // A chunk must start at or before the first query's own position, so that every query sees a key in every chunk: the
-    // last chunk takes everything from the last such start.
-    if (size_t(grid) * 2 <= cus && totalLen >= 1024) {
+    // Keys in chunks over the workgroups, each chunk with its own statistics, a second kernel putting the chunks together.
+    //  * Cached positions (oldLen > 0) and so few (batch, head, tile) triples that half the compute units would idle: one
+    //    workgroup per head would walk all the keys alone.  A chunk starts at or before the first query's own position,
+    //    so that every query sees a key in every chunk; the last chunk takes everything from the last such start.
+    //  * A causal pass from position 0 (a prompt, a small batch) whose heaviest tile, all T key tiles of the last query
+    //    tile in a row, is at least twice what a workgroup slot would get if the triangle's work were dealt evenly: the
+    //    chunks cut that row; those that lie wholly after a tile's queries are skipped by that tile's workgroup
+    //    (chunkIsEmptyFor).  The GPT-small training pass (ratio 1.2) and the headline shape (0.5) stay whole.
+    size_t chunkKeys = 0, numChunks = 1;
+    if (oldLen > 0 && size_t(grid) * 2 <= cus && totalLen >= 1024) {
         const size_t wanted = (4 * cus + grid - 1) / grid;   // about four workgroups per compute unit
-        size_t chunkKeys = ((totalLen + wanted - 1) / wanted + 127) / 128 * 128;
-        if (chunkKeys < 128) chunkKeys = 128;
-        const size_t numChunks = std::min((totalLen + chunkKeys - 1) / chunkKeys, oldLen / chunkKeys + 1);
-        if (numChunks > 1) {
-            const size_t outFloats = batch * newLen * dim, statFloats = batch * heads * newLen;
-            Scratch part(numChunks * (outFloats + 2 * statFloats) * sizeof(float));
-            if (part.status != BF_OK) return part.status;
-            AttnParams c = p;
-            c.chunkKeys = int(chunkKeys);
-            c.numChunks = int(numChunks);
-            c.partOutStride = outFloats;
-            c.partStatStride = statFloats;
-            c.out = part.as<float>();
-            c.m = c.out + numChunks * outFloats;
-            c.l = c.m + numChunks * statFloats;
-            c.outImg = nullptr;
-            st = dispatch<0>(c, vec4Ok(c, {q, k, v, c.out}), grid, s);
-            if (st != BF_OK) return st;
-            const size_t groups = batch * newLen * heads;
-            attnCombineChunksKernel<<<unsigned(groups), 256, 0, s>>>(c.out, c.m, c.l, out, outImage, imageLd, m, l, int(heads), int(newLen), int(dim),
-                                                                  p.hd, int(numChunks), outFloats, statFloats);
-            BF_LAUNCH_CHECK();
-            return BF_OK;
+        chunkKeys = std::max<size_t>(128, ((totalLen + wanted - 1) / wanted + 127) / 128 * 128);
+        numChunks = std::min((totalLen + chunkKeys - 1) / chunkKeys, oldLen / chunkKeys + 1);
+    } else if (oldLen == 0 && totalLen >= 1024 && newLen == totalLen) {
+        const double tiles = double(p.numTiles);
+        const double even = std::max(1.0, double(batch * heads) * tiles * (tiles + 1.0) / 2.0 / double(2 * cus));
+        if (tiles >= 2.0 * even) {
+            const size_t cuts = std::min<size_t>(8, size_t(std::ceil(tiles / even)));
+            chunkKeys = std::max<size_t>(128, ((totalLen + cuts - 1) / cuts + 127) / 128 * 128);
+            numChunks = (totalLen + chunkKeys - 1) / chunkKeys;
         }
+    }
+    if (numChunks > 1) {
+        const size_t outFloats = batch * newLen * dim, statFloats = batch * heads * newLen;
+        Scratch part(numChunks * (outFloats + 2 * statFloats) * sizeof(float));
+        if (part.status != BF_OK) return part.status;
+        AttnParams c = p;
+        c.chunkKeys = int(chunkKeys);
+        c.numChunks = int(numChunks);
+        c.partOutStride = outFloats;
+        c.partStatStride = statFloats;
+        c.out = part.as<float>();
+        c.m = c.out + numChunks * outFloats;
+        c.l = c.m + numChunks * statFloats;
+        c.outImg = nullptr;
+        st = dispatch<0>(c, vec4Ok(c, {q, k, v, c.out}), grid, s);
+        if (st != BF_OK) return st;
+        const size_t groups = batch * newLen * heads;
+        if (groups >= 2048 && numChunks <= 8) {   // many rows, few chunks: a wavefront per row
+            attnCombineRowsKernel<<<unsigned((groups + 3) / 4), 256, 0, s>>>(c.out, c.m, c.l, out, outImage, imageLd, m, l, groups, int(heads), int(newLen),
+                                                                          int(dim), p.hd, int(numChunks), outFloats, statFloats);
+        } else {
+            attnCombineChunksKernel<<<unsigned(groups), 256, 0, s>>>(c.out, c.m, c.l, out, outImage, imageLd, m, l, int(heads), int(newLen), int(dim), p.hd,
+                                                                  int(numChunks), outFloats, statFloats);
+        }
+        BF_LAUNCH_CHECK();
+        return BF_OK;
     }
     return dispatch<0>(p, vec4Ok(p, {q, k, v, out}), grid, s);
 }

@@ -442,7 +442,7 @@ int bfh_model_forward_incremental(void* h, const float* input, int rank, const s
         Borrowed in(input, std::vector<std::size_t>(shape, shape + rank));
         if (!handle->weightImagesCurrent) hip::invalidateBf16WeightCache();   // weights set or trained since the images were made
         handle->weightImagesCurrent = true;
-        handle->output = handle->model->forwardIncremental(in.tensor);
+        handle->output = handle->model->forwardIncremental(in.tensor, /*weightImagesCurrent=*/true);
         if (output) *output = handle->output.data();
         if (outCount) *outCount = handle->output.elementCount();
     });
@@ -454,7 +454,7 @@ int bfh_model_generate_greedy(void* h, const float* promptIds, size_t n, size_t 
         Borrowed in(promptIds, {1, n});
         if (!handle->weightImagesCurrent) hip::invalidateBf16WeightCache();
         handle->weightImagesCurrent = true;
-        std::vector<std::size_t> ids = handle->model->generateGreedy(in.tensor, count);
+        std::vector<std::size_t> ids = handle->model->generateGreedy(in.tensor, count, /*weightImagesCurrent=*/true);
         for (std::size_t i = 0; i < ids.size(); ++i) tokens[i] = static_cast<long long>(ids[i]);
     });
 }

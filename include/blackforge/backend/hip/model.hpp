@@ -192,8 +192,10 @@ public:
     // The weights must not change while a generation runs (the cached keys and values were made with them): in bf16
     // mode their images are converted at the first call after resetGenerationState() (or after anything else that
     // invalidated them) and kept for the calls that follow, where the reference converts them in every call.
-    DeviceTensor forwardIncremental(const DeviceTensor& newTokenIds) {
-        if (useBf16_ && generationPosition_ == 0) invalidateBf16WeightCache();
+    // weightImagesCurrent: the caller's word that no weight has changed since its images were last made (as for forward()):
+    // a new generation then starts without converting them again.
+    DeviceTensor forwardIncremental(const DeviceTensor& newTokenIds, bool weightImagesCurrent = false) {
+        if (useBf16_ && generationPosition_ == 0 && !weightImagesCurrent) invalidateBf16WeightCache();
         std::size_t newLen = newTokenIds.rank() >= 2 ? newTokenIds.dim(1) : 0;
         DeviceTensor output = incrementalStep(newTokenIds, nullptr);
         generationPosition_ += newLen;
@@ -210,7 +212,7 @@ public:
     // Starts a new generation (resetGenerationState) and leaves the model as count - 1 further calls of
     // forwardIncremental would: the last token returned has not been fed.  Needs a pipeline that starts with an
     // embedding; the ids are returned in order.  Not part of the reference's interface.
-    [[nodiscard]] std::vector<std::size_t> generateGreedy(const DeviceTensor& promptIds, std::size_t count) {
+    [[nodiscard]] std::vector<std::size_t> generateGreedy(const DeviceTensor& promptIds, std::size_t count, bool weightImagesCurrent = false) {
         require(promptIds.rank() == 2 && promptIds.dim(0) == 1 && promptIds.dim(1) >= 1, "generateGreedy: the prompt must be [1, n] token ids, n >= 1");
         require(!layers_.empty() && layers_.front().spec.kind == LayerKind::Embedding, "generateGreedy: the pipeline must start with an embedding");
         const std::size_t promptLen = promptIds.dim(1), vocab = layers_.front().spec.arg0;
@@ -219,7 +221,7 @@ public:
                 require(promptLen + count - 1 <= layer.params[0].value.dim(0), "generateGreedy: the positions exceed the positional table");
         resetGenerationState();
         if (count == 0) return {};
-        DeviceTensor logits = forwardIncremental(promptIds);
+        DeviceTensor logits = forwardIncremental(promptIds, weightImagesCurrent);
         require(logits.rank() == 3 && logits.dim(2) == vocab, "generateGreedy: the pipeline must end in logits over the embedding's vocabulary");
         for (LayerState& layer : layers_)
             if (layer.spec.kind == LayerKind::Attention) layer.kvCache.reserve(1, promptLen + count, layer.kvCache.k.dim(2));

@@ -49,7 +49,10 @@ CASES = [(1, 1, 1, 0, 2), (1, 2, 3, 0, 2), (2, 2, 5, 0, 4), (2, 3, 33, 0, 32), (
          # a few queries against a long cache (a step of incremental decoding): the forward pass takes the keys in chunks
          # and puts the chunks together (chunk ends inside and outside the new tokens, every head-dim class, ragged ends)
          (1, 2, 1, 2047, 64), (2, 3, 5, 3000, 32), (1, 1, 1, 4500, 128), (1, 2, 16, 1500, 256), (1, 2, 3, 1100, 100), (1, 1, 130, 1024, 64),
-         (1, 1, 1, 1023, 192)]
+         (1, 1, 1, 1023, 192),
+         # a causal pass from position 0 over few (batch, head) pairs (a prompt, a small batch): the keys go to the workgroups
+         # in chunks as well, and a chunk that lies wholly after a tile's queries is skipped by that tile
+         (1, 2, 1100, 0, 64), (2, 1, 1024, 0, 32), (1, 1, 1300, 0, 128), (1, 1, 1030, 0, 256), (1, 1, 1100, 0, 62), (1, 3, 2050, 0, 16)]
 
 
 @pytest.mark.parametrize("batch,heads,new_len,old_len,hd", CASES)
