@@ -321,13 +321,14 @@ def test_bf16_linear_with_adds_in_the_store(hip, oracle, rng, m, k, n, with_bias
 
 @pytest.mark.parametrize("m,k,n", [(1, 768, 768), (1, 3072, 768), (1, 768, 32003), (2, 72, 9000), (3, 520, 41), (5, 1032, 8200), (8, 768, 2304),
                                    (7, 8, 1), (1, 4100, 16), (4, 44, 300), (4, 3072, 768),
-                                   (16, 3072, 768), (33, 2504, 40), (64, 768, 2304), (9, 72, 100), (40, 4104, 96), (32, 776, 33), (6, 20000, 8)])
+                                   (16, 3072, 768), (33, 2504, 40), (64, 768, 2304), (9, 72, 100), (40, 4104, 96), (32, 776, 33), (6, 20000, 8), (128, 768, 768),
+                                   (100, 3080, 136)])
 @pytest.mark.parametrize("with_bias,with_residual", [(True, True), (False, False)])
 def test_bf16_products_of_a_few_rows(hip, oracle, rng, m, k, n, with_bias, with_residual):
     """matmulBf16 / linearBf16 (ops.hpp:14,30,8) with a few rows, the shape of a step of incremental decoding (model.cpp:169,
     one new token per sequence).  Up to four rows are served by a walk over the weights instead of MFMA tiles: widths on
     both sides of the switch from one to four columns a wavefront, odd widths, a contraction of several steps a lane, and
-    one that is not a multiple of eight (which stays on the tiles).  Five to 64 rows take 32 x 32 MFMA tiles whose
+    one that is not a multiple of eight (which stays on the tiles).  Five to 128 rows take 32 x 32 MFMA tiles whose
     wavefronts share out the contraction: one and two row tiles, ragged tiles, contractions that end in half a step, that go
     round the load loop again, and that are cut into slices over several workgroups."""
     D, ops = hip.DeviceTensor, hip.ops
