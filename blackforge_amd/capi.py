@@ -125,6 +125,7 @@ SIGNATURES = {
     "bf_hip_attention_forward_rows": [P, P, P, P, P, c_size, P, P, c_size, c_size, c_size, c_size, c_size, c_size, c_float, c_size, S],
     "bf_hip_copy_pitched": [P, c_size, P, c_size, c_size, c_size, S],
     "bf_hip_positional_forward_indirect": [P, P, P, c_size, c_size, c_size, c_size, P, S],
+    "bf_hip_kv_append": [P, P, P, P, c_size, c_size, c_size, c_size, c_size, S],
     "bf_hip_kv_append_indirect": [P, P, P, P, c_size, c_size, c_size, c_size, P, S],
     "bf_hip_attention_forward_rows_indirect": [P, P, P, P, P, c_size, P, P, c_size, c_size, c_size, c_size, c_size, c_float, P, S],
     "bf_hip_argmax_last_position_device": [P, c_size, c_size, P, P, c_size, P, ctypes.c_int, ctypes.c_longlong, S],

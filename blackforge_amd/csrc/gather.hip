@@ -360,8 +360,8 @@ __global__ void __launch_bounds__(256) copyPitchedKernel(float* __restrict__ dst
 template <int VEC>
 __global__ void __launch_bounds__(256) kvAppendKernel(float* __restrict__ kCache, float* __restrict__ vCache, const float* __restrict__ kNew,
                                                       const float* __restrict__ vNew, size_t batch, size_t newLen, size_t dim, size_t capacity,
-                                                      const int* __restrict__ position) {
-    const size_t at = size_t(*position);
+                                                      const int* __restrict__ position, size_t hostPosition) {
+    const size_t at = position ? size_t(*position) : hostPosition;   // the caller's position when it knows it
     if (at + newLen > capacity) return;
     float* cache = blockIdx.z == 0 ? kCache : vCache;
     const float* rows = blockIdx.z == 0 ? kNew : vNew;
@@ -652,8 +652,21 @@ int bf_hip_kv_append_indirect(float* kCache, float* vCache, const float* kNew, c
     BF_REQUIRE(newLen <= capacity, "more new rows than the cache holds");
     Geom2D g = geometry2D(batch * newLen, dim, aligned16(kCache) && aligned16(vCache) && aligned16(kNew) && aligned16(vNew));
     g.grid.z = 2;
-    if (g.vec == 4) kvAppendKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(kCache, vCache, kNew, vNew, batch, newLen, dim, capacity, position);
-    else kvAppendKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(kCache, vCache, kNew, vNew, batch, newLen, dim, capacity, position);
+    if (g.vec == 4) kvAppendKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(kCache, vCache, kNew, vNew, batch, newLen, dim, capacity, position, 0);
+    else kvAppendKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(kCache, vCache, kNew, vNew, batch, newLen, dim, capacity, position, 0);
+    BF_LAUNCH_CHECK();
+    return BF_OK;
+}
+
+int bf_hip_kv_append(float* kCache, float* vCache, const float* kNew, const float* vNew, size_t batch, size_t newLen, size_t dim, size_t capacity,
+                     size_t position, bf_stream_t stream) {
+    if (batch == 0 || newLen == 0 || dim == 0) return BF_OK;
+    BF_REQUIRE(kCache && vCache && kNew && vNew, "NULL pointer");
+    BF_REQUIRE(position + newLen <= capacity, "the new rows do not fit the cache");
+    Geom2D g = geometry2D(batch * newLen, dim, aligned16(kCache) && aligned16(vCache) && aligned16(kNew) && aligned16(vNew));
+    g.grid.z = 2;
+    if (g.vec == 4) kvAppendKernel<4><<<g.grid, g.block, 0, asStream(stream)>>>(kCache, vCache, kNew, vNew, batch, newLen, dim, capacity, nullptr, position);
+    else kvAppendKernel<1><<<g.grid, g.block, 0, asStream(stream)>>>(kCache, vCache, kNew, vNew, batch, newLen, dim, capacity, nullptr, position);
     BF_LAUNCH_CHECK();
     return BF_OK;
 }

@@ -222,6 +222,11 @@ int bf_hip_concat_seq(const float* a, const float* b, float* out, size_t batch, 
  * new keys and values to a cache with room to grow (hip::KVCache), where the reference concatenates into a new tensor at
  * every step (ops_transformer.cu:22-58). */
 int bf_hip_copy_pitched(float* dst, size_t dstPitch, const float* src, size_t srcPitch, size_t width, size_t rows, bf_stream_t stream);
+/* New keys and values, [batch, newLen, dim] each, to rows position.. of every sequence of caches with `capacity` rows a
+ * sequence, both in one launch: the append of selfAttentionIncremental for several sequences (ops_transformer.cu:147-160,
+ * where the reference concatenates). */
+int bf_hip_kv_append(float* kCache, float* vCache, const float* kNew, const float* vNew, size_t batch, size_t newLen, size_t dim, size_t capacity,
+                     size_t position, bf_stream_t stream);
 /* argmaxLastPosition: main.cpp:504-518, moved to the device.  logits: [seq, vocab]; *index (HOST) gets
  * the lowest index of the maximum of the last row.  Synchronous. */
 int bf_hip_argmax_last_position(const float* logits, size_t seq, size_t vocab, long long* index, bf_stream_t stream);

@@ -555,7 +555,7 @@ inline DeviceTensor selfAttentionIncrementalImpl(const char* op, const DeviceTen
     if (cache.length != 0) require(cache.k.rank() == 3 && cache.k.dim(0) == batch && cache.k.dim(2) == dim, std::string(op) + ": the cache was filled with another batch size or width");
     cache.reserve(batch, oldLen + newLen, dim);
     // one sequence: its new keys and values are rows oldLen.. of the cache, and the projections write them there;
-    // several: the projections' rows lie batch by batch and a copy spreads them over the sequences
+    // several: the projections' rows lie batch by batch and one launch spreads both over the sequences
     const bool inPlace = batch == 1;
     DeviceTensor qNew({batch, newLen, dim}), kNew, vNew;
     if (!inPlace) {
@@ -566,10 +566,7 @@ inline DeviceTensor selfAttentionIncrementalImpl(const char* op, const DeviceTen
     float* vRows = inPlace ? cache.v.data() + oldLen * dim : vNew.data();
     float* const outs[3] = {qNew.data(), kRows, vRows};
     incrementalProjections(newInput, wq, wk, wv, outs, mode);
-    if (!inPlace) {
-        check(bf_hip_copy_pitched(cache.k.data() + oldLen * dim, cache.capacity * dim, kNew.data(), newLen * dim, newLen * dim, batch, nullptr));
-        check(bf_hip_copy_pitched(cache.v.data() + oldLen * dim, cache.capacity * dim, vNew.data(), newLen * dim, newLen * dim, batch, nullptr));
-    }
+    if (!inPlace) check(bf_hip_kv_append(cache.k.data(), cache.v.data(), kNew.data(), vNew.data(), batch, newLen, dim, cache.capacity, oldLen, nullptr));
     cache.length = oldLen + newLen;
     const float scaleFactor = 1.0F / std::sqrt(static_cast<float>(dim / numHeads));
     // the attention output has one reader, the output projection: in bf16 mode it is written as that product's operand image only

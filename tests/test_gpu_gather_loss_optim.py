@@ -145,6 +145,12 @@ def test_position_on_the_device_entry_points(hip, oracle, rng):
         ek[:, 7:9], ev[:, 7:9] = kn, vn
         assert_bits_equal(dk.toHost(), ek, "keys appended at the device-side position")
         assert_bits_equal(dv.toHost(), ev, "values appended at the device-side position")
+        dk2, dv2 = D.fromHost(kc), D.fromHost(vc)
+        call("bf_hip_kv_append", dk2.ptr, dv2.ptr, dkn.ptr, dvn.ptr, batch, seq, dim, capacity, 7, None)   # the position from the host
+        assert_bits_equal(dk2.toHost(), ek, "keys appended at the caller's position")
+        assert_bits_equal(dv2.toHost(), ev, "values appended at the caller's position")
+        with pytest.raises(ValueError):
+            call("bf_hip_kv_append", dk2.ptr, dv2.ptr, dkn.ptr, dvn.ptr, batch, seq, dim, capacity, 9, None)
         full = D.fromHost(np.array([9], np.int32).view(f32))
         call("bf_hip_kv_append_indirect", dk.ptr, dv.ptr, dkn.ptr, dvn.ptr, batch, seq, dim, capacity, full.ptr, None)
         assert_bits_equal(dk.toHost(), ek, "rows that do not fit are not written")
