@@ -2800,9 +2800,11 @@ int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v
     //    workgroup per head would walk all the keys alone.  A chunk starts at or before the first query's own position,
     //    so that every query sees a key in every chunk; the last chunk takes everything from the last such start.
     //  * A causal pass from position 0 (a prompt, a small batch) whose heaviest tile, all T key tiles of the last query
-    //    tile in a row, is at least twice what a workgroup slot would get if the triangle's work were dealt evenly: the
-    //    chunks cut that row; those that lie wholly after a tile's queries are skipped by that tile's workgroup
-    //    (chunkIsEmptyFor).  The GPT-small training pass (ratio 1.2) and the headline shape (0.5) stay whole.
+    //    tile in a row, is at least two and a half times what a workgroup slot would get if the triangle's work were dealt
+    //    evenly: the chunks cut that row; those that lie wholly after a tile's queries are skipped by that tile's
+    //    workgroup (chunkIsEmptyFor).  Measured, 12 heads of 64: batch 1 at 1024 / 2048 / 4000 positions (ratios 9.5, 5, 2.6)
+    //    66 -> 52, 126 -> 89, 257 -> 226 us; batch 4 at 1024 (2.4) would lose, 74 -> 90 us, and stays whole, like the
+    //    GPT-small training pass (1.2) and the headline shape (0.5).
     size_t chunkKeys = 0, numChunks = 1;
     if (oldLen > 0 && size_t(grid) * 2 <= cus && totalLen >= 1024) {
         const size_t wanted = (4 * cus + grid - 1) / grid;   // about four workgroups per compute unit
@@ -2811,7 +2813,7 @@ int bf_hip_attention_forward_rows(const float* q, const float* k, const float* v
     } else if (oldLen == 0 && totalLen >= 1024 && newLen == totalLen) {
         const double tiles = double(p.numTiles);
         const double even = std::max(1.0, double(batch * heads) * tiles * (tiles + 1.0) / 2.0 / double(2 * cus));
-        if (tiles >= 2.0 * even) {
+        if (tiles >= 2.5 * even) {
             const size_t cuts = std::min<size_t>(8, size_t(std::ceil(tiles / even)));
             chunkKeys = std::max<size_t>(128, ((totalLen + cuts - 1) / cuts + 127) / 128 * 128);
             numChunks = (totalLen + chunkKeys - 1) / chunkKeys;

@@ -392,7 +392,8 @@ int bf_hip_bf16_weight_cache_refresh(const float* const* changed, size_t count, 
  * (head, chunk), and puts the chunks together in a second kernel: batch 1, 12 heads of 64, 4096 cached positions 244 ->
  * 38 us; the results are the unchunked ones up to the order of the additions.  So does a causal pass from position 0
  * (oldLen = 0, newLen = totalLen >= 1024) over so few (batch, head) pairs that the last query tile's row of key tiles is
- * at least twice an even share of the work (a prompt: batch 1, 12 heads, 1024 positions 158 -> 42 us).
+ * at least two and a half times an even share of the work (a prompt: batch 1, 12 heads, 1024 positions 158 -> 42 us
+ * inside the model's pass).
  * ------------------------------------------------------------------------------------------- */
 /* fusedAttentionForward: out:[batch,newLen,dim]; m,l:[batch,heads,newLen] = row max of the scaled
  * scores and sum of exp(score - m) (the statistics the backward reuses). */
